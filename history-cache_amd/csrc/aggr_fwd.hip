@@ -1,0 +1,305 @@
+// History-aware CSR gather-reduce, forward.
+//
+// One wavefront owns one destination row.  The row's neighbour ids are staged
+// 64 at a time with one coalesced load (one id per lane); each id is then
+// broadcast with v_readlane so the neighbour row's base address is
+// wave-uniform and the 64 lanes read one contiguous span of the row with
+// vector loads (16 bytes per lane when the row length allows).  Up to UNROLL
+// neighbour rows are in flight per wave before the first add; the adds run in
+// CSR order in fp32, so every output element is summed in exactly the order a
+// sequential CPU loop would use.
+//
+// Semantics follow the reference kernels gen_fwd_history_v2,
+// gen_fwd_history_v2_edge_value and gen_fwd_history_v2_edge_value_multi_head
+// (/root/reference/src/cpp/src/history_aggr.cu:7-125); offsets are 64-bit
+// (the reference truncates neighbour ids and offsets to 32-bit int, :19,34-35).
+#include "hc_common.h"
+
+namespace {
+
+// Wave-cooperative copy of one row of a history buffer into an fp32 output row.
+template <typename TH>
+__device__ __forceinline__ void copy_row_typed(const TH *__restrict__ src, float *__restrict__ dst,
+                                               int64_t F, int lane) {
+  constexpr int V = 4;
+  const bool vec_ok = (F % V == 0) && ((reinterpret_cast<uintptr_t>(src) % (sizeof(TH) * V)) == 0) &&
+                      ((reinterpret_cast<uintptr_t>(dst) % 16) == 0);
+  if (vec_ok) {
+    for (int64_t c = (int64_t)lane * V; c < F; c += HC_WAVE * V) {
+      float v[V];
+      hc_vec<TH, V>::load(src + c, v);
+      *reinterpret_cast<float4 *>(dst + c) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+  } else {
+    for (int64_t c = lane; c < F; c += HC_WAVE) dst[c] = hc_to_f32<TH>(src[c]);
+  }
+}
+
+__device__ __forceinline__ void copy_row_any(const void *hbuf, int hist_dtype, int64_t elem_off,
+                                             float *dst, int64_t F, int lane) {
+  if (hist_dtype == HC_F32) {
+    copy_row_typed<float>(static_cast<const float *>(hbuf) + elem_off, dst, F, lane);
+  } else if (hist_dtype == HC_F16) {
+    copy_row_typed<__half>(static_cast<const __half *>(hbuf) + elem_off, dst, F, lane);
+  } else {
+    copy_row_typed<__hip_bfloat16>(static_cast<const __hip_bfloat16 *>(hbuf) + elem_off, dst, F, lane);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Fast path: mean aggregation, row length F == 64 * VEC * CHUNKS elements exactly.
+// src_mode == 0: per-destination-row substitution (hbuf row-aligned, any dtype).
+// src_mode == 1: per-source substitution (hbuf is a table of the same dtype as vin).
+// ---------------------------------------------------------------------------------------
+template <typename T, int VEC, int CHUNKS, int UNROLL>
+__global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
+    const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const T *__restrict__ vin,
+    const int64_t *__restrict__ hmap, const void *__restrict__ hbuf, int hist_dtype, int64_t hsize,
+    int src_mode, float *__restrict__ vout, int64_t R) {
+  constexpr int F = HC_WAVE * VEC * CHUNKS;
+  const int lane = hc_lane();
+  const int64_t row = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (row >= R) return;
+  float *__restrict__ orow = vout + row * F;
+
+  if (!src_mode && hmap != nullptr) {
+    if (hmap[row] != -1) {
+      copy_row_any(hbuf, hist_dtype, row * hsize, orow, F, lane);
+      return;
+    }
+  }
+
+  const int64_t begin = ptr[row];
+  const int64_t end = ptr[row + 1];
+  float acc[CHUNKS][VEC];
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
+
+  const T *__restrict__ htab = static_cast<const T *>(hbuf);
+  for (int64_t base = begin; base < end; base += HC_WAVE) {
+    const int64_t left = end - base;
+    const int n = left < HC_WAVE ? (int)left : HC_WAVE;
+    // Stage: lane l resolves the address of neighbour base+l.
+    int64_t my_addr = 0;
+    if (lane < n) {
+      const int64_t id = idx[base + lane];
+      const T *p = vin + id * F;
+      if (src_mode && hmap != nullptr) {
+        const int64_t slot = hmap[id];
+        if (slot != -1) p = htab + slot * hsize;
+      }
+      my_addr = reinterpret_cast<int64_t>(p);
+    }
+    for (int j = 0; j < n; j += UNROLL) {
+      float v[UNROLL][CHUNKS][VEC];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        if (j + u < n) {
+          const T *p = reinterpret_cast<const T *>(hc_readlane64(my_addr, j + u)) + lane * VEC;
+#pragma unroll
+          for (int k = 0; k < CHUNKS; ++k) hc_vec<T, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
+        } else {
+#pragma unroll
+          for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) v[u][k][i] = 0.0f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) acc[k][i] += v[u][k][i];
+    }
+  }
+
+  const int64_t deg = end - begin;
+  const float fdeg = (float)(int)deg;
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    float o[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) o[i] = deg > 0 ? acc[k][i] / fdeg : 0.0f;
+    hc_store_f32<VEC>(orow + k * HC_WAVE * VEC + lane * VEC, o);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Generic path: any F, optional per-edge weights, optional heads.  One wave per
+// (row, head); columns are walked in tiles of 256; the neighbour list is re-read per tile.
+// ---------------------------------------------------------------------------------------
+template <typename T, bool WEIGHTED>
+__global__ __launch_bounds__(HC_BLOCK) void fwd_generic(
+    const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const T *__restrict__ vin,
+    const int64_t *__restrict__ hmap, const void *__restrict__ hbuf, int hist_dtype, int64_t hsize,
+    int src_mode, const float *__restrict__ ev, int64_t H, float *__restrict__ vout, int64_t R,
+    int64_t F) {
+  constexpr int TILE_K = 4;
+  const int lane = hc_lane();
+  const int64_t vrow = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (vrow >= R * H) return;
+  const int64_t row = vrow / H;
+  const int64_t head = vrow - row * H;
+  float *__restrict__ orow = vout + vrow * F;
+
+  if (!src_mode && hmap != nullptr) {
+    if (hmap[row] != -1) {
+      const int64_t off = row * hsize + (hsize == F ? 0 : head * F);
+      copy_row_any(hbuf, hist_dtype, off, orow, F, lane);
+      return;
+    }
+  }
+  const int64_t begin = ptr[row];
+  const int64_t end = ptr[row + 1];
+  const int64_t deg = end - begin;
+  const float fdeg = (float)(int)deg;
+  const T *__restrict__ htab = static_cast<const T *>(hbuf);
+
+  for (int64_t c0 = 0; c0 < F; c0 += HC_WAVE * TILE_K) {
+    float acc[TILE_K];
+#pragma unroll
+    for (int k = 0; k < TILE_K; ++k) acc[k] = 0.0f;
+    for (int64_t base = begin; base < end; base += HC_WAVE) {
+      const int64_t left = end - base;
+      const int n = left < HC_WAVE ? (int)left : HC_WAVE;
+      int64_t my_addr = 0;
+      float my_w = 0.0f;
+      if (lane < n) {
+        const int64_t id = idx[base + lane];
+        const T *p = vin + (id * H + head) * F;
+        if (src_mode && hmap != nullptr) {
+          const int64_t slot = hmap[id];
+          if (slot != -1) p = htab + slot * hsize;
+        }
+        my_addr = reinterpret_cast<int64_t>(p);
+        if (WEIGHTED) my_w = ev[(base + lane) * H + head];
+      }
+      for (int j = 0; j < n; ++j) {
+        const T *p = reinterpret_cast<const T *>(hc_readlane64(my_addr, j));
+        const float w = WEIGHTED ? hc_readlane_f(my_w, j) : 1.0f;
+#pragma unroll
+        for (int k = 0; k < TILE_K; ++k) {
+          const int64_t c = c0 + k * HC_WAVE + lane;
+          if (c < F) {
+            const float x = hc_to_f32<T>(p[c]);
+            acc[k] = WEIGHTED ? __fmaf_rn(x, w, acc[k]) : acc[k] + x;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < TILE_K; ++k) {
+      const int64_t c = c0 + k * HC_WAVE + lane;
+      if (c < F) orow[c] = WEIGHTED ? acc[k] : (deg > 0 ? acc[k] / fdeg : 0.0f);
+    }
+  }
+}
+
+template <typename T, int VEC, int CHUNKS>
+int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const int64_t *hmap,
+                const void *hbuf, int hist_dtype, int64_t hsize, int src_mode, float *vout, int64_t R,
+                hipStream_t st) {
+  constexpr int per = VEC * CHUNKS;
+  constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
+  const int64_t blocks = (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  if (!hc_grid_ok(blocks)) return HC_EUNSUPPORTED;
+  fwd_mean_fast<T, VEC, CHUNKS, UNROLL><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(
+      ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, vout, R);
+  return hc_launch_status();
+}
+
+// Pick (VEC, CHUNKS) with F == 64*VEC*CHUNKS, VEC as wide as 16 bytes allows, CHUNKS <= 4.
+template <typename T>
+int dispatch_fast(int64_t F, const int64_t *ptr, const int64_t *idx, const void *vin,
+                  const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize, int src_mode,
+                  float *vout, int64_t R, hipStream_t st, bool *handled) {
+  *handled = true;
+#define HC_FAST(V, C)                                                                              \
+  if (F == 64 * (V) * (C))                                                                         \
+    return launch_fast<T, V, C>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, vout, R, st);
+  constexpr int VMAX = 16 / (int)sizeof(T);
+  if constexpr (VMAX == 8) {
+    HC_FAST(8, 1) HC_FAST(8, 2) HC_FAST(8, 3) HC_FAST(8, 4)
+  }
+  HC_FAST(4, 1) HC_FAST(4, 3)
+  if constexpr (VMAX == 4) { HC_FAST(4, 2) HC_FAST(4, 4) }
+  HC_FAST(2, 1) HC_FAST(2, 3)
+  HC_FAST(1, 1) HC_FAST(1, 3)
+#undef HC_FAST
+  *handled = false;
+  return HC_OK;
+}
+
+template <typename T>
+int launch_generic(const int64_t *ptr, const int64_t *idx, const void *vin, const int64_t *hmap,
+                   const void *hbuf, int hist_dtype, int64_t hsize, int src_mode, const float *ev,
+                   int64_t H, float *vout, int64_t R, int64_t F, hipStream_t st) {
+  const int64_t blocks = (R * H + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  if (!hc_grid_ok(blocks)) return HC_EUNSUPPORTED;
+  dim3 g((unsigned)blocks), b(HC_BLOCK);
+  if (ev)
+    fwd_generic<T, true><<<g, b, 0, st>>>(ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype,
+                                          hsize, src_mode, ev, H, vout, R, F);
+  else
+    fwd_generic<T, false><<<g, b, 0, st>>>(ptr, idx, static_cast<const T *>(vin), hmap, hbuf,
+                                           hist_dtype, hsize, src_mode, ev, H, vout, R, F);
+  return hc_launch_status();
+}
+
+}  // namespace
+
+extern "C" int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, const void *vin,
+                           int in_dtype, const int64_t *hmap, const void *hbuf, int hist_dtype,
+                           int64_t hsize, const float *edge_value, int64_t n_head, float *vout,
+                           int64_t R, int64_t F, int64_t n_src, void *stream) {
+  HC_REQUIRE(R >= 0 && F > 0 && n_src >= 0 && n_head >= 1);
+  if (R == 0) return HC_OK;
+  HC_REQUIRE(ptr && vout);
+  HC_REQUIRE(mode == HC_SUBST_ROW || mode == HC_SUBST_SRC);
+  if (in_dtype < HC_F32 || in_dtype > HC_BF16) return HC_EDTYPE;
+  if (hmap && (hist_dtype < HC_F32 || hist_dtype > HC_BF16)) return HC_EDTYPE;
+  if (hmap) HC_REQUIRE(hbuf != nullptr && hsize > 0);
+  if (n_head > 1) HC_REQUIRE(edge_value != nullptr);
+  const int src_mode = (mode == HC_SUBST_SRC) ? 1 : 0;
+  if (src_mode) {
+    if (edge_value) return HC_EUNSUPPORTED;
+    if (hmap) {
+      HC_REQUIRE(hsize >= F);
+      if (hist_dtype != in_dtype) return HC_EUNSUPPORTED;
+    }
+  } else if (hmap) {
+    HC_REQUIRE(hsize == F * n_head || (hsize >= F && n_head == 1) || hsize == F);
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+
+  const size_t esz = in_dtype == HC_F32 ? 4 : 2;
+  const bool aligned = (reinterpret_cast<uintptr_t>(vin) % 16 == 0) &&
+                       (reinterpret_cast<uintptr_t>(vout) % 16 == 0) &&
+                       (!src_mode || !hmap ||
+                        ((reinterpret_cast<uintptr_t>(hbuf) % 16 == 0) && ((hsize * esz) % 16 == 0)));
+  if (!edge_value && n_head == 1 && aligned && vin != nullptr) {
+    bool handled = false;
+    int rc;
+    if (in_dtype == HC_F32)
+      rc = dispatch_fast<float>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, vout, R, st,
+                                &handled);
+    else if (in_dtype == HC_F16)
+      rc = dispatch_fast<__half>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, vout, R, st,
+                                 &handled);
+    else
+      rc = dispatch_fast<__hip_bfloat16>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode,
+                                         vout, R, st, &handled);
+    if (handled) return rc;
+  }
+  if (in_dtype == HC_F32)
+    return launch_generic<float>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value,
+                                 n_head, vout, R, F, st);
+  if (in_dtype == HC_F16)
+    return launch_generic<__half>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value,
+                                  n_head, vout, R, F, st);
+  return launch_generic<__hip_bfloat16>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode,
+                                        edge_value, n_head, vout, R, F, st);
+}

@@ -1,0 +1,497 @@
+// Gradient-based cache admission ("grad_check"): row scores, the threshold /
+// staleness test, the admission mask, ring-slot assignment in row order and the
+// history-table scatter-update.
+//
+// Reference semantics: record_history_kernel_used_mask
+// (/root/reference/src/cpp/src/grad_check.cu:6-46) for the ring insert and the
+// predicate on precomputed scores; HistoryCache.update_history
+// (/root/reference/hiscache/history_cache.py:205-254) for the L2 score, the
+// strict "<" test and the append-only variant; HistoryTable.record_history
+// (/root/reference/hiscache/history_table.py:161) for the L1 score.
+//
+// The reference takes ring slots with atomicInc in arrival order
+// (grad_check.cu:25), so its slot numbering changes from run to run.  Here the
+// k-th admitted row (in row order) gets slot (header + k) mod capacity:
+//   pass 1  score + predicate per row, mask byte, admitted count per 64-row tile
+//   pass 2  one block scans the tile counts (exclusive), advances the header
+//   pass 3  per tile: ballot-rank the mask, un-map old owners, copy rows, map
+// Pass 1 is the only pass that touches the gradient matrix; pass 3 only touches
+// admitted rows, so HBM traffic is the algorithmic minimum.
+#include "hc_common.h"
+
+namespace {
+
+constexpr int GC_TILE = 64;                                   // rows per block (= one ballot)
+constexpr int GC_ROWS_PER_WAVE = GC_TILE / HC_WAVES_PER_BLOCK;  // 16
+
+// Scalars shared between the passes (workspace prefix).
+struct GcScalars {
+  int64_t header_old;  // header before this call
+  int64_t admitted;    // number of admitted rows
+  int64_t written;     // append mode: rows that fit below capacity
+  int64_t pad[5];
+};
+
+__device__ __forceinline__ float fold(float acc, float x, int norm_kind) {
+  return norm_kind == HC_NORM_L2 ? __fmaf_rn(x, x, acc) : acc + fabsf(x);
+}
+
+// Partial score of one row held by this lane: elements e with (e/4)%64 == lane, increasing e.
+__device__ __forceinline__ float row_partial_generic(const float *__restrict__ row, int64_t F,
+                                                     int lane, int norm_kind) {
+  float acc = 0.0f;
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(row) % 16) == 0;
+  for (int64_t b = (int64_t)lane * 4; b < F; b += HC_WAVE * 4) {
+    if (vec_ok && b + 3 < F) {
+      const float4 v = *reinterpret_cast<const float4 *>(row + b);
+      acc = fold(acc, v.x, norm_kind);
+      acc = fold(acc, v.y, norm_kind);
+      acc = fold(acc, v.z, norm_kind);
+      acc = fold(acc, v.w, norm_kind);
+    } else {
+      for (int i = 0; i < 4; ++i)
+        if (b + i < F) acc = fold(acc, row[b + i], norm_kind);
+    }
+  }
+  return acc;
+}
+
+__device__ __forceinline__ float finish_score(float partial, int norm_kind) {
+  const float tot = hc_wave_sum_butterfly(partial);
+  return norm_kind == HC_NORM_L2 ? __fsqrt_rn(tot) : tot;
+}
+
+// Scores of the GC_ROWS_PER_WAVE rows owned by this wave; lane i ends up holding row i's score.
+// CH > 0: F == 256*CH, 16-byte aligned rows, 8 rows of loads in flight.  CH == 0: any F.
+template <int CH>
+__device__ __forceinline__ float wave_scores(const float *__restrict__ grad, int64_t row0, int64_t M,
+                                             int64_t F, int lane, int norm_kind) {
+  float mine = 0.0f;
+  if constexpr (CH > 0) {
+    constexpr int RB = (CH <= 2) ? 8 : 4;
+    for (int i0 = 0; i0 < GC_ROWS_PER_WAVE; i0 += RB) {
+      float4 v[RB][CH];
+#pragma unroll
+      for (int i = 0; i < RB; ++i) {
+        const int64_t r = row0 + i0 + i;
+        if (r < M) {
+          const float4 *p = reinterpret_cast<const float4 *>(grad + r * (256 * CH)) + lane;
+#pragma unroll
+          for (int k = 0; k < CH; ++k) v[i][k] = p[k * HC_WAVE];
+        } else {
+#pragma unroll
+          for (int k = 0; k < CH; ++k) v[i][k] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < RB; ++i) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int k = 0; k < CH; ++k) {
+          acc = fold(acc, v[i][k].x, norm_kind);
+          acc = fold(acc, v[i][k].y, norm_kind);
+          acc = fold(acc, v[i][k].z, norm_kind);
+          acc = fold(acc, v[i][k].w, norm_kind);
+        }
+        const float s = finish_score(acc, norm_kind);
+        if (lane == i0 + i) mine = s;
+      }
+    }
+  } else {
+    for (int i = 0; i < GC_ROWS_PER_WAVE; ++i) {
+      const int64_t r = row0 + i;
+      float acc = 0.0f;
+      if (r < M) acc = row_partial_generic(grad + r * F, F, lane, norm_kind);
+      const float s = finish_score(acc, norm_kind);
+      if (lane == i) mine = s;
+    }
+  }
+  return mine;
+}
+
+// ---------------------------------------------------------------------------------------
+// Pass 1.  PRED == false: scores only (counts untouched).
+// ---------------------------------------------------------------------------------------
+template <int CH, bool PRED>
+__global__ __launch_bounds__(HC_BLOCK) void gc_pass1(
+    const float *__restrict__ grad, const float *__restrict__ score_in, const int64_t *__restrict__ slot,
+    const int32_t *__restrict__ age, const uint8_t *__restrict__ used, const float *__restrict__ thres_p,
+    int32_t age_limit, int norm_kind, int cmp_kind, uint8_t *__restrict__ mask_out,
+    float *__restrict__ score_out, int64_t *__restrict__ tile_counts, int64_t M, int64_t F) {
+  __shared__ int wave_cnt[HC_WAVES_PER_BLOCK];
+  const int lane = hc_lane();
+  const int wave = hc_wave_in_block();
+  const int64_t row0 = (int64_t)blockIdx.x * GC_TILE + wave * GC_ROWS_PER_WAVE;
+  const int64_t r = row0 + lane;
+  const bool owner = lane < GC_ROWS_PER_WAVE && r < M;
+
+  float sc = 0.0f;
+  if (grad != nullptr) sc = wave_scores<CH>(grad, row0, M, F, lane, norm_kind);
+  else if (owner) sc = score_in[r];
+  if (owner && score_out != nullptr) score_out[r] = sc;
+  if (!PRED) return;
+
+  bool admit = false;
+  if (owner) {
+    const float thres = thres_p[0];
+    const bool pass = (cmp_kind == HC_CMP_LT) ? (sc < thres) : !(thres != 0.0f && sc > thres);
+    const bool fresh = (slot[r] == -1) || (age != nullptr && age[r] >= age_limit);
+    const bool use = (used == nullptr) || (used[r] != 0);
+    admit = pass && fresh && use;
+    mask_out[r] = admit ? 1 : 0;
+  }
+  const unsigned long long bal = __ballot(admit);
+  if (lane == 0) wave_cnt[wave] = __popcll(bal);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int t = 0;
+#pragma unroll
+    for (int w = 0; w < HC_WAVES_PER_BLOCK; ++w) t += wave_cnt[w];
+    tile_counts[blockIdx.x] = t;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Pass 2: exclusive scan of the tile counts by one block; header bookkeeping.
+// ring != 0: header = (header + A) mod capacity.   ring == 0 (append): rows beyond capacity
+// are dropped, header += written, *overflow = dropped.
+// ---------------------------------------------------------------------------------------
+constexpr int GC_SCAN_THREADS = 1024;
+__global__ __launch_bounds__(GC_SCAN_THREADS) void gc_pass2(int64_t *__restrict__ tile_counts,
+                                                             int64_t n_tiles, GcScalars *__restrict__ sc,
+                                                             int64_t *__restrict__ header,
+                                                             int64_t capacity, int ring,
+                                                             int64_t *__restrict__ overflow) {
+  __shared__ int64_t wave_tot[GC_SCAN_THREADS / HC_WAVE];
+  __shared__ int64_t carry_s;
+  const int lane = hc_lane();
+  const int wave = (int)(threadIdx.x >> 6);
+  if (threadIdx.x == 0) carry_s = 0;
+  __syncthreads();
+  for (int64_t base = 0; base < n_tiles; base += GC_SCAN_THREADS) {
+    const int64_t i = base + threadIdx.x;
+    const int64_t v = i < n_tiles ? tile_counts[i] : 0;
+    // inclusive scan inside the wave
+    int64_t x = v;
+#pragma unroll
+    for (int d = 1; d < HC_WAVE; d <<= 1) {
+      const int lo = __shfl_up((int)(uint32_t)(uint64_t)x, d, HC_WAVE);
+      const int hi = __shfl_up((int)(uint32_t)((uint64_t)x >> 32), d, HC_WAVE);
+      const int64_t y = (int64_t)(((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo);
+      if (lane >= d) x += y;
+    }
+    if (lane == HC_WAVE - 1) wave_tot[wave] = x;
+    __syncthreads();
+    int64_t wave_off = 0;
+    for (int w = 0; w < wave; ++w) wave_off += wave_tot[w];
+    const int64_t carry = carry_s;
+    if (i < n_tiles) tile_counts[i] = carry + wave_off + x - v;  // exclusive
+    __syncthreads();
+    if (threadIdx.x == GC_SCAN_THREADS - 1) carry_s = carry + wave_off + x;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const int64_t A = carry_s;
+    const int64_t h = header[0];
+    sc->header_old = h;
+    sc->admitted = A;
+    if (ring) {
+      sc->written = A;
+      header[0] = capacity > 0 ? (h + A) % capacity : 0;
+    } else {
+      int64_t room = capacity - h;
+      if (room < 0) room = 0;
+      const int64_t w = A < room ? A : room;
+      sc->written = w;
+      header[0] = h + w;
+      if (overflow != nullptr) overflow[0] = A - w;
+    }
+  }
+}
+
+// Wave-cooperative row store with conversion to the table dtype.
+template <typename TT>
+__device__ __forceinline__ void store_row(const float *__restrict__ src, TT *__restrict__ dst, int64_t F,
+                                          int lane) {
+  const bool vec_ok = (F % 4 == 0) && (reinterpret_cast<uintptr_t>(src) % 16 == 0) &&
+                      (reinterpret_cast<uintptr_t>(dst) % (4 * sizeof(TT)) == 0);
+  if (vec_ok) {
+    for (int64_t c = (int64_t)lane * 4; c < F; c += HC_WAVE * 4) {
+      float v[4];
+      hc_vec<float, 4>::load(src + c, v);
+      hc_vec<TT, 4>::store(dst + c, v);
+    }
+  } else {
+    for (int64_t c = lane; c < F; c += HC_WAVE) dst[c] = hc_from_f32<TT>(src[c]);
+  }
+}
+
+__device__ __forceinline__ void store_row_any(const float *src, void *table, int table_dtype,
+                                              int64_t elem_off, int64_t F, int lane) {
+  if (table_dtype == HC_F32) store_row<float>(src, static_cast<float *>(table) + elem_off, F, lane);
+  else if (table_dtype == HC_F16) store_row<__half>(src, static_cast<__half *>(table) + elem_off, F, lane);
+  else store_row<__hip_bfloat16>(src, static_cast<__hip_bfloat16 *>(table) + elem_off, F, lane);
+}
+
+__device__ __forceinline__ void store_relaxed(int64_t *p, int64_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---------------------------------------------------------------------------------------
+// Pass 3 (ring): per tile, rank the admitted rows, un-map old owners, copy, map.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(HC_BLOCK) void gc_pass3_ring(
+    const uint8_t *__restrict__ mask, const int64_t *__restrict__ tile_offsets,
+    const GcScalars *__restrict__ sc, const float *__restrict__ emb,
+    const int64_t *__restrict__ sub_to_full, void *__restrict__ table, int table_dtype, int64_t capacity,
+    int64_t *__restrict__ full2slot, int64_t *__restrict__ slot2full, int64_t *__restrict__ checkin,
+    int64_t *__restrict__ slot_out, int64_t glb_iter, int64_t M, int64_t F) {
+  __shared__ int local_rows[GC_TILE];
+  __shared__ int n_admitted_s;
+  const int lane = hc_lane();
+  const int wave = hc_wave_in_block();
+  const int64_t tile0 = (int64_t)blockIdx.x * GC_TILE;
+  const int64_t header_old = sc->header_old;
+  const int64_t A = sc->admitted;
+  const int64_t tile_off = tile_offsets[blockIdx.x];
+  if (wave == 0) {
+    const int64_t r = tile0 + lane;
+    const bool m = r < M && mask[r] != 0;
+    const unsigned long long bal = __ballot(m);
+    const int rank = __popcll(bal & ((1ull << lane) - 1ull));
+    if (m) local_rows[rank] = lane;
+    if (lane == 0) n_admitted_s = __popcll(bal);
+    if (slot_out != nullptr && r < M)
+      slot_out[r] = m ? (header_old + tile_off + rank) % capacity : -1;
+  }
+  __syncthreads();
+  const int n_adm = n_admitted_s;
+  const int64_t first_live = A > capacity ? A - capacity : 0;  // ranks below are overwritten later
+  for (int q = wave; q < n_adm; q += HC_WAVES_PER_BLOCK) {
+    const int64_t r = tile0 + local_rows[q];
+    const int64_t k = tile_off + q;
+    const int64_t full = sub_to_full[r];
+    if (k < first_live) {
+      // Inserted and evicted again within this call: net effect is "not cached".
+      if (lane == 0) store_relaxed(full2slot + full, -1);
+      continue;
+    }
+    const int64_t s = (header_old + k) % capacity;
+    if (lane == 0) {
+      const int64_t old = slot2full[s];
+      if (old != -1) {
+        unsigned long long expect = (unsigned long long)s;
+        __hip_atomic_compare_exchange_strong(reinterpret_cast<unsigned long long *>(full2slot + old),
+                                             &expect, (unsigned long long)(int64_t)-1, __ATOMIC_RELAXED,
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    store_row_any(emb + r * F, table, table_dtype, s * F, F, lane);
+    if (lane == 0) {
+      store_relaxed(full2slot + full, s);
+      slot2full[s] = full;
+      if (checkin != nullptr) checkin[s] = glb_iter;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Append mode (HistoryCache.update_history): invalidation, then copy + map.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(HC_BLOCK) void gc_append_invalidate(
+    const GcScalars *__restrict__ sc, int64_t H, int64_t F_in, int64_t *__restrict__ full2embed,
+    const int64_t *__restrict__ embed2full, const int64_t *__restrict__ feat2full, int64_t n_feat,
+    int64_t max_feat_span, int64_t M) {
+  const int64_t h = sc->header_old;
+  const int64_t w = sc->written;
+  const int64_t t = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  // (a) feature slots overlapped by [h, h+w) embedding rows (history_cache.py:223-226)
+  if (t < max_feat_span && feat2full != nullptr && w >= 0) {
+    const int64_t b = h * H / F_in;
+    int64_t e = ((h + w) * H + F_in - 1) / F_in;
+    if (e > n_feat) e = n_feat;
+    const int64_t i = b + t;
+    if (i < e) {
+      const int64_t f = feat2full[i];
+      if (f >= 0) full2embed[f] = -1;
+    }
+  }
+  // (b) previous owners of the overwritten embedding slots (history_cache.py:230-240)
+  if (t < M && t < w) {
+    const int64_t f = embed2full[h + t];
+    if (f >= 0) {
+      const int64_t v = full2embed[f];
+      if (v >= h && v < h + w) full2embed[f] = -1;
+    }
+  }
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void gc_pass3_append(
+    const uint8_t *__restrict__ mask, const int64_t *__restrict__ tile_offsets,
+    const GcScalars *__restrict__ sc, const float *__restrict__ emb,
+    const int64_t *__restrict__ sub_to_full, float *__restrict__ buffer, int64_t H,
+    int64_t *__restrict__ full2embed, int64_t *__restrict__ embed2full, int64_t M) {
+  __shared__ int local_rows[GC_TILE];
+  __shared__ int n_admitted_s;
+  const int lane = hc_lane();
+  const int wave = hc_wave_in_block();
+  const int64_t tile0 = (int64_t)blockIdx.x * GC_TILE;
+  const int64_t header_old = sc->header_old;
+  const int64_t written = sc->written;
+  const int64_t tile_off = tile_offsets[blockIdx.x];
+  if (wave == 0) {
+    const int64_t r = tile0 + lane;
+    const bool m = r < M && mask[r] != 0;
+    const unsigned long long bal = __ballot(m);
+    const int rank = __popcll(bal & ((1ull << lane) - 1ull));
+    if (m) local_rows[rank] = lane;
+    if (lane == 0) n_admitted_s = __popcll(bal);
+  }
+  __syncthreads();
+  const int n_adm = n_admitted_s;
+  for (int q = wave; q < n_adm; q += HC_WAVES_PER_BLOCK) {
+    const int64_t k = tile_off + q;
+    if (k >= written) continue;  // would land beyond the buffer
+    const int64_t r = tile0 + local_rows[q];
+    const int64_t s = header_old + k;
+    store_row<float>(emb + r * H, buffer + s * H, H, lane);
+    if (lane == 0) {
+      const int64_t full = sub_to_full[r];
+      full2embed[full] = s;
+      embed2full[s] = full;
+    }
+  }
+}
+
+size_t ws_bytes(int64_t M) {
+  const int64_t tiles = (M + GC_TILE - 1) / GC_TILE;
+  return hc_align_up(sizeof(GcScalars) + (size_t)(tiles > 0 ? tiles : 1) * sizeof(int64_t), 256);
+}
+
+template <bool PRED>
+int launch_pass1(const float *grad, const float *score_in, const int64_t *slot, const int32_t *age,
+                 const uint8_t *used, const float *thres, int32_t age_limit, int norm_kind, int cmp_kind,
+                 uint8_t *mask_out, float *score_out, int64_t *tile_counts, int64_t M, int64_t F,
+                 hipStream_t st) {
+  const int64_t tiles = (M + GC_TILE - 1) / GC_TILE;
+  if (!hc_grid_ok(tiles)) return HC_EUNSUPPORTED;
+  dim3 g((unsigned)tiles), b(HC_BLOCK);
+  const bool fast = grad != nullptr && (F % 256 == 0) && (F / 256 <= 4) &&
+                    (reinterpret_cast<uintptr_t>(grad) % 16 == 0);
+#define HC_P1(CH)                                                                                    \
+  gc_pass1<CH, PRED><<<g, b, 0, st>>>(grad, score_in, slot, age, used, thres, age_limit, norm_kind,  \
+                                      cmp_kind, mask_out, score_out, tile_counts, M, F)
+  if (fast && F == 256) HC_P1(1);
+  else if (fast && F == 512) HC_P1(2);
+  else if (fast && F == 768) HC_P1(3);
+  else if (fast && F == 1024) HC_P1(4);
+  else HC_P1(0);
+#undef HC_P1
+  return hc_launch_status();
+}
+
+}  // namespace
+
+extern "C" size_t hc_grad_check_workspace_bytes(int64_t M) { return M < 0 ? 0 : ws_bytes(M); }
+
+extern "C" int hc_row_scores(const float *grad, float *score, int64_t M, int64_t F, int norm_kind,
+                             void *stream) {
+  HC_REQUIRE(M >= 0 && F > 0);
+  HC_REQUIRE(norm_kind == HC_NORM_L2 || norm_kind == HC_NORM_L1);
+  if (M == 0) return HC_OK;
+  HC_REQUIRE(grad && score);
+  return launch_pass1<false>(grad, nullptr, nullptr, nullptr, nullptr, nullptr, 0, norm_kind, 0, nullptr,
+                             score, nullptr, M, F, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int hc_grad_check(const float *grad, const float *score_in, const float *emb,
+                             const int64_t *slot, const int32_t *age, const uint8_t *used,
+                             const int64_t *sub_to_full, const float *thres, int32_t age_limit,
+                             int norm_kind, int cmp_kind, uint8_t *mask_out, float *score_out,
+                             int64_t *slot_out, void *table, int table_dtype, int64_t capacity,
+                             int64_t *full2slot, int64_t *slot2full, int64_t *checkin, int64_t *header,
+                             int64_t glb_iter, int64_t M, int64_t F, void *workspace,
+                             size_t workspace_bytes, void *stream) {
+  HC_REQUIRE(M >= 0 && F > 0 && capacity > 0);
+  HC_REQUIRE(norm_kind == HC_NORM_L2 || norm_kind == HC_NORM_L1);
+  HC_REQUIRE(cmp_kind == HC_CMP_LT || cmp_kind == HC_CMP_NOT_GT);
+  if (table_dtype < HC_F32 || table_dtype > HC_BF16) return HC_EDTYPE;
+  HC_REQUIRE(header != nullptr);
+  if (M == 0) return HC_OK;
+  HC_REQUIRE((grad || score_in) && emb && slot && sub_to_full && thres && mask_out && table &&
+             full2slot && slot2full);
+  if (!workspace || workspace_bytes < ws_bytes(M) || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+    return HC_EWORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  GcScalars *sc = static_cast<GcScalars *>(workspace);
+  int64_t *tiles_buf = reinterpret_cast<int64_t *>(sc + 1);
+  const int64_t tiles = (M + GC_TILE - 1) / GC_TILE;
+
+  int rc = launch_pass1<true>(grad, score_in, slot, age, used, thres, age_limit, norm_kind, cmp_kind,
+                              mask_out, score_out, tiles_buf, M, F, st);
+  if (rc != HC_OK) return rc;
+  gc_pass2<<<dim3(1), dim3(GC_SCAN_THREADS), 0, st>>>(tiles_buf, tiles, sc, header, capacity, 1, nullptr);
+  if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
+  gc_pass3_ring<<<dim3((unsigned)tiles), dim3(HC_BLOCK), 0, st>>>(
+      mask_out, tiles_buf, sc, emb, sub_to_full, table, table_dtype, capacity, full2slot, slot2full,
+      checkin, slot_out, glb_iter, M, F);
+  return hc_launch_status();
+}
+
+extern "C" int hc_record_history(const float *buffer_new, float *buffer_all, const uint8_t *used_mask,
+                                 const int64_t *sub_to_full, const int64_t *sub_to_history,
+                                 int64_t *history_to_full, int64_t *full_to_history, int64_t *header,
+                                 const float *score, const float *thres, int64_t *checkin_iter,
+                                 int64_t glb_iter, int64_t M, int64_t history_num, int64_t history_size,
+                                 void *workspace, size_t workspace_bytes, void *stream) {
+  HC_REQUIRE(M >= 0 && history_size > 0 && history_num >= 0);
+  if (M == 0 || history_num == 0) return HC_OK;
+  HC_REQUIRE(score != nullptr);
+  // mask lives behind the tile array in the workspace: the reference has no mask output
+  const size_t base = ws_bytes(M);
+  const size_t need = base + hc_align_up((size_t)M, 256);
+  if (!workspace || workspace_bytes < need) return HC_EWORKSPACE;
+  uint8_t *mask = static_cast<uint8_t *>(workspace) + base;
+  return hc_grad_check(nullptr, score, buffer_new, sub_to_history, nullptr, used_mask, sub_to_full, thres,
+                       0, HC_NORM_L2, HC_CMP_NOT_GT, mask, nullptr, nullptr, buffer_all, HC_F32,
+                       history_num, full_to_history, history_to_full, checkin_iter, header, glb_iter, M,
+                       history_size, workspace, base, stream);
+}
+
+extern "C" int hc_cache_append(const float *score, const float *thres, const float *emb,
+                               const int64_t *sub2embed, const int64_t *sub_to_full, uint8_t *mask_out,
+                               float *buffer, int64_t capacity, int64_t H, int64_t F_in,
+                               int64_t *full2embed, int64_t *embed2full, const int64_t *feat2full,
+                               int64_t n_feat, int64_t *header, int64_t *overflow, int64_t M,
+                               void *workspace, size_t workspace_bytes, void *stream) {
+  HC_REQUIRE(M >= 0 && H > 0 && F_in > 0 && capacity >= 0 && n_feat >= 0);
+  HC_REQUIRE(header != nullptr);
+  if (M == 0) return HC_OK;
+  HC_REQUIRE(score && thres && emb && sub2embed && sub_to_full && mask_out && buffer && full2embed &&
+             embed2full);
+  HC_REQUIRE(feat2full != nullptr || n_feat == 0);
+  if (!workspace || workspace_bytes < ws_bytes(M) || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+    return HC_EWORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  GcScalars *sc = static_cast<GcScalars *>(workspace);
+  int64_t *tiles_buf = reinterpret_cast<int64_t *>(sc + 1);
+  const int64_t tiles = (M + GC_TILE - 1) / GC_TILE;
+
+  int rc = launch_pass1<true>(nullptr, score, sub2embed, nullptr, nullptr, thres, 0, HC_NORM_L2,
+                              HC_CMP_LT, mask_out, nullptr, tiles_buf, M, H, st);
+  if (rc != HC_OK) return rc;
+  gc_pass2<<<dim3(1), dim3(GC_SCAN_THREADS), 0, st>>>(tiles_buf, tiles, sc, header, capacity, 0, overflow);
+  if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
+  // worst-case span of feature slots covered by M embedding rows
+  const int64_t max_feat_span = (M * H + F_in - 1) / F_in + 2;
+  const int64_t span = max_feat_span > M ? max_feat_span : M;
+  const int64_t iblocks = (span + HC_BLOCK - 1) / HC_BLOCK;
+  if (!hc_grid_ok(iblocks)) return HC_EUNSUPPORTED;
+  gc_append_invalidate<<<dim3((unsigned)iblocks), dim3(HC_BLOCK), 0, st>>>(
+      sc, H, F_in, full2embed, embed2full, feat2full, n_feat, max_feat_span, M);
+  if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
+  gc_pass3_append<<<dim3((unsigned)tiles), dim3(HC_BLOCK), 0, st>>>(mask_out, tiles_buf, sc, emb,
+                                                                    sub_to_full, buffer, H, full2embed,
+                                                                    embed2full, M);
+  return hc_launch_status();
+}

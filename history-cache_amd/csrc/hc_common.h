@@ -1,0 +1,137 @@
+// Shared device/host helpers for the gfx950 kernels (wave64 only).
+#pragma once
+
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "hiscache_hip.h"
+
+#define HC_WAVE 64
+#define HC_BLOCK 256
+#define HC_WAVES_PER_BLOCK (HC_BLOCK / HC_WAVE)
+
+#define HC_REQUIRE(cond) \
+  do {                   \
+    if (!(cond)) return HC_EINVAL; \
+  } while (0)
+
+static inline int hc_launch_status() {
+  return hipGetLastError() == hipSuccess ? HC_OK : HC_ELAUNCH;
+}
+
+static inline size_t hc_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Grid limit for a 1-D launch: gridDim.x * blockDim.x must stay below 2^32 (blocks of up to
+// 1024 threads are used by the scan kernel, so the bound is taken for those).
+static inline bool hc_grid_ok(int64_t blocks) { return blocks > 0 && blocks <= 0xffffffffLL / HC_BLOCK; }
+
+#ifdef __HIPCC__
+
+__device__ __forceinline__ int hc_lane() { return (int)(threadIdx.x & (HC_WAVE - 1)); }
+
+// Index of this wave inside its block, forced into a scalar register so that
+// everything derived from it (row id, row bounds) is wave-uniform.
+__device__ __forceinline__ int hc_wave_in_block() {
+  return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+}
+
+__device__ __forceinline__ int64_t hc_readlane64(int64_t v, int lane) {
+  int lo = __builtin_amdgcn_readlane((int)(uint32_t)(uint64_t)v, lane);
+  int hi = __builtin_amdgcn_readlane((int)(uint32_t)((uint64_t)v >> 32), lane);
+  return (int64_t)(((uint64_t)(uint32_t)hi << 32) | (uint64_t)(uint32_t)lo);
+}
+
+__device__ __forceinline__ int64_t hc_uniform64(int64_t v) {
+  int lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)(uint64_t)v);
+  int hi = __builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)v >> 32));
+  return (int64_t)(((uint64_t)(uint32_t)hi << 32) | (uint64_t)(uint32_t)lo);
+}
+
+__device__ __forceinline__ float hc_readlane_f(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// Butterfly sum over the 64 lanes, partner distance 32,16,8,4,2,1.  Every lane
+// ends with the same bits (fp add is commutative), and the order is the one
+// the CPU checker reproduces.
+__device__ __forceinline__ float hc_wave_sum_butterfly(float v) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) v = v + __shfl_xor(v, d, HC_WAVE);
+  return v;
+}
+
+// ---- element conversion ----------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float hc_to_f32(T v);
+template <>
+__device__ __forceinline__ float hc_to_f32<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ float hc_to_f32<__half>(__half v) { return __half2float(v); }
+template <>
+__device__ __forceinline__ float hc_to_f32<__hip_bfloat16>(__hip_bfloat16 v) {
+  return __bfloat162float(v);
+}
+
+template <typename T>
+__device__ __forceinline__ T hc_from_f32(float v);
+template <>
+__device__ __forceinline__ float hc_from_f32<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ __half hc_from_f32<__half>(float v) { return __float2half_rn(v); }
+template <>
+__device__ __forceinline__ __hip_bfloat16 hc_from_f32<__hip_bfloat16>(float v) {
+  return __float2bfloat16(v);
+}
+
+// ---- vector load of VEC consecutive elements, widened to fp32 ---------------
+template <int BYTES>
+struct hc_raw;
+template <>
+struct hc_raw<2> { typedef uint16_t type; };
+template <>
+struct hc_raw<4> { typedef uint32_t type; };
+template <>
+struct hc_raw<8> { typedef uint2 type; };
+template <>
+struct hc_raw<16> { typedef uint4 type; };
+
+template <typename T, int VEC>
+struct hc_vec {
+  typedef typename hc_raw<sizeof(T) * VEC>::type raw_t;
+  union U {
+    raw_t raw;
+    T e[VEC];
+    __device__ U() {}
+  };
+  // p must be aligned to sizeof(T) * VEC
+  __device__ __forceinline__ static void load(const T *p, float (&out)[VEC]) {
+    U u;
+    u.raw = *reinterpret_cast<const raw_t *>(p);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) out[i] = hc_to_f32<T>(u.e[i]);
+  }
+  __device__ __forceinline__ static void store(T *p, const float (&in)[VEC]) {
+    U u;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) u.e[i] = hc_from_f32<T>(in[i]);
+    *reinterpret_cast<raw_t *>(p) = u.raw;
+  }
+};
+
+// Store VEC consecutive fp32 values (VEC may exceed one 16-byte store).
+template <int VEC>
+__device__ __forceinline__ void hc_store_f32(float *p, const float (&in)[VEC]) {
+  if constexpr (VEC <= 4) {
+    hc_vec<float, VEC>::store(p, in);
+  } else {
+#pragma unroll
+    for (int q = 0; q < VEC / 4; ++q) {
+      const float t[4] = {in[4 * q], in[4 * q + 1], in[4 * q + 2], in[4 * q + 3]};
+      hc_vec<float, 4>::store(p + 4 * q, t);
+    }
+  }
+}
+
+#endif  // __HIPCC__

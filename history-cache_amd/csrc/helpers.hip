@@ -1,0 +1,294 @@
+// Used-mask reconstruction, small graph helpers, row gathers and library metadata.
+#include "hc_common.h"
+
+namespace {
+
+__global__ __launch_bounds__(HC_BLOCK) void fill_u8(uint8_t *__restrict__ p, int64_t n, uint8_t v) {
+  // 16 bytes per thread where possible
+  const int64_t i = ((int64_t)blockIdx.x * HC_BLOCK + threadIdx.x) * 16;
+  if (i + 16 <= n && (reinterpret_cast<uintptr_t>(p) % 16) == 0) {
+    const uint32_t w = 0x01010101u * v;
+    *reinterpret_cast<uint4 *>(p + i) = make_uint4(w, w, w, w);
+  } else {
+    for (int64_t k = i; k < n && k < i + 16; ++k) p[k] = v;
+  }
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void fill_i64(int64_t *__restrict__ p, int64_t n, int64_t v) {
+  const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void fill_i32(int32_t *__restrict__ p, int64_t n, int32_t v) {
+  const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// One pass of the used-mask rule (/root/reference/src/cpp/src/grad_check.cu:70-101).
+// Wave per row.  A row is active if it is a seed on the first pass (:79-82) or use_in[row]
+// is set (:83-84); an active row with history stops (:87-90); otherwise it marks itself
+// (:92-94) and its neighbours (:97-100).  Every store writes the constant 1.
+__global__ __launch_bounds__(HC_BLOCK) void count_history_pass(
+    const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const int64_t *__restrict__ hmap,
+    int64_t hmap_len, uint8_t *__restrict__ use_in, uint8_t *__restrict__ use_out, int64_t ptr_rows,
+    int64_t n_all, int64_t n_seed, int first_pass) {
+  const int lane = hc_lane();
+  const int64_t row = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (row >= ptr_rows || row >= n_all) return;
+  if (first_pass && row < n_seed) {
+    if (lane == 0) use_in[row] = 1;
+  } else if (use_in[row] != 1) {
+    return;
+  }
+  if (hmap != nullptr && row < hmap_len && hmap[row] != -1) return;
+  if (lane == 0) use_out[row] = 1;
+  const int64_t begin = ptr[row];
+  const int64_t end = ptr[row + 1];
+  for (int64_t e = begin + lane; e < end; e += HC_WAVE) {
+    const int64_t n = idx[e];
+    if (n >= 0 && n < n_all) use_out[n] = 1;
+  }
+}
+
+// Histogram that skips value 0 (/root/reference/src/cpp/src/grad_check.cu:165-172).
+__global__ __launch_bounds__(HC_BLOCK) void count_num_kernel(const int64_t *__restrict__ arr,
+                                                              int32_t *__restrict__ out, int64_t n,
+                                                              int64_t mmax) {
+  const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (i >= n) return;
+  const int64_t a = arr[i];
+  if (a > 0 && a <= mmax) atomicAdd(out + a, 1);
+}
+
+// One level-synchronous pass of the structure score: rows with prev != 0 offer prev*deg to
+// neighbours whose prev is 0; the smallest offer wins (unsigned min over a 0 = "unset" encoding).
+__global__ __launch_bounds__(HC_BLOCK) void structure_pass(const int64_t *__restrict__ ptr,
+                                                            const int64_t *__restrict__ idx,
+                                                            const int64_t *__restrict__ prev,
+                                                            unsigned long long *__restrict__ next,
+                                                            int64_t ptr_rows, int64_t n_all) {
+  const int lane = hc_lane();
+  const int64_t row = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (row >= ptr_rows || row >= n_all) return;
+  const int64_t pv = prev[row];
+  if (pv == 0) return;
+  const int64_t begin = ptr[row];
+  const int64_t end = ptr[row + 1];
+  const int64_t offer = pv * (end - begin);
+  for (int64_t e = begin + lane; e < end; e += HC_WAVE) {
+    const int64_t n = idx[e];
+    if (n < 0 || n >= n_all || prev[n] != 0) continue;
+    // "unset" is stored as 0; offer-1 in unsigned space keeps 0 (from deg 0 rows) representable
+    atomicMin(next + n, (unsigned long long)offer - 1ull);
+  }
+}
+
+// Reset the offer array to "unset" (all ones) before a pass.
+__global__ __launch_bounds__(HC_BLOCK) void structure_stage(unsigned long long *__restrict__ next,
+                                                             int64_t n_all) {
+  const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (i < n_all) next[i] = ~0ull;
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void structure_commit(int64_t *__restrict__ out,
+                                                              const unsigned long long *__restrict__ next,
+                                                              int64_t n_all) {
+  const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (i >= n_all) return;
+  const unsigned long long v = next[i];
+  if (out[i] == 0 && v != ~0ull) out[i] = (int64_t)(v + 1ull);
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void structure_seed(int64_t *__restrict__ out, int64_t n_seed,
+                                                            int64_t n_all) {
+  const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (i < n_seed && i < n_all) out[i] = 1;
+}
+
+// dst[i,:] = (mask == NULL || mask[i]) ? src[ids[i],:] : 0  (optionally accumulated).
+// Wave per output row; 16-byte loads when the row allows.  src may be mapped host memory.
+template <typename T>
+__global__ __launch_bounds__(HC_BLOCK) void gather_rows_kernel(const T *__restrict__ src, int64_t n_rows,
+                                                                const int64_t *__restrict__ ids,
+                                                                const uint8_t *__restrict__ mask,
+                                                                float *__restrict__ dst, int accumulate,
+                                                                int64_t n, int64_t F) {
+  constexpr int V = 16 / (int)sizeof(T) > 4 ? 4 : 16 / (int)sizeof(T);  // 4 elements per lane
+  const int lane = hc_lane();
+  const int64_t i = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (i >= n) return;
+  float *__restrict__ o = dst + i * F;
+  bool take = mask == nullptr || mask[i] != 0;
+  int64_t id = 0;
+  if (take) {
+    id = ids[i];
+    if (id < 0) id += n_rows;
+    if (id < 0 || id >= n_rows) take = false;
+  }
+  const T *__restrict__ s = src + id * F;
+  const bool vec_ok = (F % V == 0) && (reinterpret_cast<uintptr_t>(s) % (sizeof(T) * V) == 0) &&
+                      (reinterpret_cast<uintptr_t>(o) % 16 == 0);
+  if (vec_ok) {
+    for (int64_t c = (int64_t)lane * V; c < F; c += HC_WAVE * V) {
+      float v[V];
+      if (take) {
+        hc_vec<T, V>::load(s + c, v);
+      } else {
+#pragma unroll
+        for (int k = 0; k < V; ++k) v[k] = 0.0f;
+      }
+      if (accumulate) {
+        float old[V];
+        hc_vec<float, V>::load(o + c, old);
+#pragma unroll
+        for (int k = 0; k < V; ++k) v[k] = old[k] + v[k];
+      }
+      hc_vec<float, V>::store(o + c, v);
+    }
+  } else {
+    for (int64_t c = lane; c < F; c += HC_WAVE) {
+      float v = take ? hc_to_f32<T>(s[c]) : 0.0f;
+      if (accumulate) v = o[c] + v;
+      o[c] = v;
+    }
+  }
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void lookup_kernel(const int64_t *__restrict__ map,
+                                                           int64_t map_len,
+                                                           const int64_t *__restrict__ ids,
+                                                           int64_t offset, int64_t *__restrict__ out,
+                                                           int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (i >= n) return;
+  int64_t k = ids[i] + offset;
+  if (k < 0) k += map_len;  // -1 addresses the last entry, as Python indexing does
+  out[i] = (k >= 0 && k < map_len) ? map[k] : -1;
+}
+
+inline unsigned blocks_for(int64_t n) { return (unsigned)((n + HC_BLOCK - 1) / HC_BLOCK); }
+
+}  // namespace
+
+extern "C" const char *hc_version(void) { return "hiscache_hip 0.1 (gfx950)"; }
+
+extern "C" const char *hc_strerror(int status) {
+  switch (status) {
+    case HC_OK: return "ok";
+    case HC_EINVAL: return "invalid argument (null pointer, negative size or inconsistent shapes)";
+    case HC_EDTYPE: return "unknown dtype";
+    case HC_ELAUNCH: return "HIP launch error";
+    case HC_EWORKSPACE: return "workspace missing, misaligned or too small";
+    case HC_EUNSUPPORTED: return "request outside what the kernels cover";
+    case HC_ENODEVICE: return "no usable GPU";
+    default: return "unknown status";
+  }
+}
+
+extern "C" int hc_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n;
+}
+
+extern "C" int hc_count_history(const int64_t *ptr, const int64_t *idx, const int64_t *hmap,
+                                int64_t hmap_len, uint8_t *masks, int64_t ptr_rows, int64_t n_all,
+                                int64_t n_seed, int num_layer, void *stream) {
+  HC_REQUIRE(ptr_rows >= 0 && n_all >= 0 && n_seed >= 0 && num_layer >= 0 && hmap_len >= 0);
+  if (n_all == 0) return HC_OK;
+  HC_REQUIRE(masks != nullptr);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t total = (int64_t)(num_layer + 1) * n_all;
+  const int64_t fb = (total + HC_BLOCK * 16 - 1) / (HC_BLOCK * 16);
+  if (!hc_grid_ok(fb)) return HC_EUNSUPPORTED;
+  fill_u8<<<dim3((unsigned)fb), dim3(HC_BLOCK), 0, st>>>(masks, total, 0);
+  if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
+  if (ptr_rows == 0 || num_layer == 0) return HC_OK;
+  HC_REQUIRE(ptr != nullptr);
+  const int64_t rb = (ptr_rows + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  if (!hc_grid_ok(rb)) return HC_EUNSUPPORTED;
+  const int L = num_layer;
+  for (int i = 0; i < L; ++i) {
+    // history prunes on the second pass only (grad_check.cu:122-124)
+    const int64_t *hm = (i == 1) ? hmap : nullptr;
+    count_history_pass<<<dim3((unsigned)rb), dim3(HC_BLOCK), 0, st>>>(
+        ptr, idx, hm, hmap_len, masks + (int64_t)(L - i) * n_all, masks + (int64_t)(L - 1 - i) * n_all,
+        ptr_rows, n_all, n_seed, i == 0 ? 1 : 0);
+    if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
+  }
+  return HC_OK;
+}
+
+extern "C" int hc_count_num(const int64_t *arr, int64_t n, int64_t mmax, int32_t *out, void *stream) {
+  HC_REQUIRE(n >= 0 && mmax >= 0 && out);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  fill_i32<<<dim3(blocks_for(mmax + 1)), dim3(HC_BLOCK), 0, st>>>(out, mmax + 1, 0);
+  if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
+  if (n == 0) return HC_OK;
+  HC_REQUIRE(arr);
+  if (!hc_grid_ok((n + HC_BLOCK - 1) / HC_BLOCK)) return HC_EUNSUPPORTED;
+  count_num_kernel<<<dim3(blocks_for(n)), dim3(HC_BLOCK), 0, st>>>(arr, out, n, mmax);
+  return hc_launch_status();
+}
+
+extern "C" int hc_structure_score(const int64_t *ptr, const int64_t *idx, int64_t ptr_rows,
+                                  int64_t n_all, int64_t n_seed, int num_layer, int64_t *out,
+                                  int64_t *scratch, void *stream) {
+  HC_REQUIRE(ptr_rows >= 0 && n_all >= 0 && n_seed >= 0 && num_layer >= 0);
+  if (n_all == 0) return HC_OK;
+  HC_REQUIRE(out && scratch);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!hc_grid_ok((n_all + HC_BLOCK - 1) / HC_BLOCK)) return HC_EUNSUPPORTED;
+  fill_i64<<<dim3(blocks_for(n_all)), dim3(HC_BLOCK), 0, st>>>(out, n_all, 0);
+  unsigned long long *next = reinterpret_cast<unsigned long long *>(scratch);
+  const int64_t rb = (ptr_rows + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  for (int p = 0; p < num_layer; ++p) {
+    structure_seed<<<dim3(blocks_for(n_all)), dim3(HC_BLOCK), 0, st>>>(out, n_seed, n_all);
+    structure_stage<<<dim3(blocks_for(n_all)), dim3(HC_BLOCK), 0, st>>>(next, n_all);
+    if (rb > 0) {
+      HC_REQUIRE(ptr != nullptr);
+      if (!hc_grid_ok(rb)) return HC_EUNSUPPORTED;
+      structure_pass<<<dim3((unsigned)rb), dim3(HC_BLOCK), 0, st>>>(ptr, idx, out, next, ptr_rows, n_all);
+    }
+    structure_commit<<<dim3(blocks_for(n_all)), dim3(HC_BLOCK), 0, st>>>(out, next, n_all);
+    if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
+  }
+  return HC_OK;
+}
+
+extern "C" int hc_gather_rows(const void *src, int src_dtype, int64_t n_rows, const int64_t *ids,
+                              const uint8_t *mask, float *dst, int accumulate, int64_t n, int64_t F,
+                              void *stream) {
+  HC_REQUIRE(n >= 0 && F > 0 && n_rows >= 0);
+  if (src_dtype < HC_F32 || src_dtype > HC_BF16) return HC_EDTYPE;
+  if (n == 0) return HC_OK;
+  HC_REQUIRE(ids && dst && (src || n_rows == 0));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t b = (n + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  if (!hc_grid_ok(b)) return HC_EUNSUPPORTED;
+  dim3 g((unsigned)b), bl(HC_BLOCK);
+  if (src_dtype == HC_F32)
+    gather_rows_kernel<float><<<g, bl, 0, st>>>(static_cast<const float *>(src), n_rows, ids, mask, dst,
+                                                accumulate, n, F);
+  else if (src_dtype == HC_F16)
+    gather_rows_kernel<__half><<<g, bl, 0, st>>>(static_cast<const __half *>(src), n_rows, ids, mask,
+                                                 dst, accumulate, n, F);
+  else
+    gather_rows_kernel<__hip_bfloat16><<<g, bl, 0, st>>>(static_cast<const __hip_bfloat16 *>(src),
+                                                         n_rows, ids, mask, dst, accumulate, n, F);
+  return hc_launch_status();
+}
+
+extern "C" int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset,
+                         int64_t *out, int64_t n, void *stream) {
+  HC_REQUIRE(n >= 0 && map_len >= 0);
+  if (n == 0) return HC_OK;
+  HC_REQUIRE(map && ids && out);
+  if (!hc_grid_ok((n + HC_BLOCK - 1) / HC_BLOCK)) return HC_EUNSUPPORTED;
+  lookup_kernel<<<dim3(blocks_for(n)), dim3(HC_BLOCK), 0, static_cast<hipStream_t>(stream)>>>(
+      map, map_len, ids, offset, out, n);
+  return hc_launch_status();
+}

@@ -1,0 +1,173 @@
+// Transposed (CSC) view of a CSR block, built with a stable sort so that the
+// backward pass can gather instead of scattering with float atomics.
+//
+// The reference has no such step: its backward pushes gradients with
+// atomicAdd (/root/reference/src/cpp/src/history_aggr.cu:164), which makes the
+// sums depend on scheduling.  Here every source's incoming edges end up in
+// ascending destination-row order, so the backward sums have one fixed order.
+//
+// Pipeline (all on the caller's stream):
+//   1. fill      keys[e] = n_src (sentinel) for every edge slot
+//   2. expand    wave per row: keys[e] = idx[e], rows[e] = r for the row's edges
+//                (rows flagged by hmap_row are skipped and keep the sentinel)
+//   3. sort      rocPRIM LSD radix sort of (key, edge slot) pairs -- stable
+//   4. finalize  rowT/edgeT from the sorted pairs; ptrT[s] = lower_bound(keys, s)
+#include <cstring>
+
+#include <rocprim/rocprim.hpp>
+
+#include "hc_common.h"
+
+namespace {
+
+__global__ __launch_bounds__(HC_BLOCK) void tr_fill(uint32_t *__restrict__ keys,
+                                                     uint32_t *__restrict__ vals, int64_t E,
+                                                     uint32_t sentinel) {
+  const int64_t e = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (e < E) {
+    keys[e] = sentinel;
+    vals[e] = (uint32_t)e;
+  }
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void tr_expand(const int64_t *__restrict__ ptr,
+                                                       const int64_t *__restrict__ idx,
+                                                       const int64_t *__restrict__ hmap_row,
+                                                       uint32_t *__restrict__ keys,
+                                                       uint32_t *__restrict__ rows, int64_t R,
+                                                       int64_t E, int64_t n_src) {
+  const int lane = hc_lane();
+  const int64_t row = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (row >= R) return;
+  if (hmap_row != nullptr && hmap_row[row] != -1) return;
+  const int64_t begin = ptr[row];
+  int64_t end = ptr[row + 1];
+  if (end > E) end = E;
+  for (int64_t e = begin + lane; e < end; e += HC_WAVE) {
+    const int64_t s = idx[e];
+    // ids outside [0, n_src) keep the sentinel and drop out of the view
+    if (s >= 0 && s < n_src) keys[e] = (uint32_t)s;
+    rows[e] = (uint32_t)row;
+  }
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void tr_finalize_edges(const uint32_t *__restrict__ skeys,
+                                                               const uint32_t *__restrict__ svals,
+                                                               const uint32_t *__restrict__ rows,
+                                                               int32_t *__restrict__ rowT,
+                                                               int32_t *__restrict__ edgeT, int64_t E,
+                                                               uint32_t sentinel) {
+  const int64_t p = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (p >= E) return;
+  const uint32_t k = skeys[p];
+  const uint32_t e = svals[p];
+  if (k != sentinel) {
+    rowT[p] = (int32_t)rows[e];
+    edgeT[p] = (int32_t)e;
+  } else {
+    rowT[p] = -1;
+    edgeT[p] = -1;
+  }
+}
+
+// ptrT[s] = number of sorted keys strictly below s, for s in [0, n_src].
+__global__ __launch_bounds__(HC_BLOCK) void tr_finalize_ptr(const uint32_t *__restrict__ skeys,
+                                                             int64_t *__restrict__ ptrT, int64_t E,
+                                                             int64_t n_src) {
+  const int64_t s = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (s > n_src) return;
+  int64_t lo = 0, hi = E;
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    if ((int64_t)skeys[mid] < s) lo = mid + 1;
+    else hi = mid;
+  }
+  ptrT[s] = lo;
+}
+
+int key_bits(int64_t n_src) {
+  int b = 1;
+  while (b < 32 && ((int64_t)1 << b) <= n_src) ++b;
+  return b;
+}
+
+struct Layout {
+  size_t keys0, keys1, vals0, vals1, rows, temp, total;
+};
+
+hipError_t sort_temp_bytes(int64_t E, int bits, size_t *bytes) {
+  rocprim::double_buffer<uint32_t> k(nullptr, nullptr), v(nullptr, nullptr);
+  *bytes = 0;
+  return rocprim::radix_sort_pairs(nullptr, *bytes, k, v, (size_t)E, 0u, (unsigned)bits,
+                                   (hipStream_t)0, false);
+}
+
+bool make_layout(int64_t E, int64_t n_src, Layout *L) {
+  size_t temp = 0;
+  if (E > 0 && sort_temp_bytes(E, key_bits(n_src), &temp) != hipSuccess) return false;
+  const size_t arr = hc_align_up((size_t)(E > 0 ? E : 1) * sizeof(uint32_t), 256);
+  L->keys0 = 0;
+  L->keys1 = arr;
+  L->vals0 = 2 * arr;
+  L->vals1 = 3 * arr;
+  L->rows = 4 * arr;
+  L->temp = 5 * arr;
+  L->total = 5 * arr + hc_align_up(temp > 0 ? temp : 1, 256);
+  return true;
+}
+
+}  // namespace
+
+extern "C" size_t hc_transpose_workspace_bytes(int64_t R, int64_t E, int64_t n_src) {
+  (void)R;
+  if (E < 0 || n_src < 0) return 0;
+  Layout L;
+  if (!make_layout(E, n_src, &L)) return 0;
+  return L.total;
+}
+
+extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row,
+                                  int64_t R, int64_t E, int64_t n_src, int64_t *ptrT, int32_t *rowT,
+                                  int32_t *edgeT, void *workspace, size_t workspace_bytes,
+                                  void *stream) {
+  HC_REQUIRE(R >= 0 && E >= 0 && n_src >= 0 && ptrT);
+  const int64_t lim = 0x7ffffffeLL;
+  if (R > lim || E > lim || n_src > lim) return HC_EUNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t pblocks = (n_src + 1 + HC_BLOCK - 1) / HC_BLOCK;
+  if (E == 0 || R == 0) {
+    // no edges: every segment is empty (binary search over zero keys writes 0)
+    tr_finalize_ptr<<<dim3((unsigned)pblocks), dim3(HC_BLOCK), 0, st>>>(nullptr, ptrT, 0, n_src);
+    return hc_launch_status();
+  }
+  HC_REQUIRE(ptr && idx && rowT && edgeT);
+  Layout L;
+  if (!make_layout(E, n_src, &L)) return HC_ELAUNCH;
+  if (!workspace || workspace_bytes < L.total) return HC_EWORKSPACE;
+  char *ws = static_cast<char *>(workspace);
+  if (reinterpret_cast<uintptr_t>(ws) % 256 != 0) return HC_EWORKSPACE;
+  uint32_t *keys0 = reinterpret_cast<uint32_t *>(ws + L.keys0);
+  uint32_t *keys1 = reinterpret_cast<uint32_t *>(ws + L.keys1);
+  uint32_t *vals0 = reinterpret_cast<uint32_t *>(ws + L.vals0);
+  uint32_t *vals1 = reinterpret_cast<uint32_t *>(ws + L.vals1);
+  uint32_t *rows = reinterpret_cast<uint32_t *>(ws + L.rows);
+  void *temp = ws + L.temp;
+  size_t temp_bytes = L.total - L.temp;
+  const uint32_t sentinel = (uint32_t)n_src;
+
+  const int64_t eblocks = (E + HC_BLOCK - 1) / HC_BLOCK;
+  const int64_t rblocks = (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  if (!hc_grid_ok(eblocks) || !hc_grid_ok(rblocks) || !hc_grid_ok(pblocks)) return HC_EUNSUPPORTED;
+
+  tr_fill<<<dim3((unsigned)eblocks), dim3(HC_BLOCK), 0, st>>>(keys0, vals0, E, sentinel);
+  tr_expand<<<dim3((unsigned)rblocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, rows, R, E,
+                                                                n_src);
+  rocprim::double_buffer<uint32_t> dk(keys0, keys1), dv(vals0, vals1);
+  if (rocprim::radix_sort_pairs(temp, temp_bytes, dk, dv, (size_t)E, 0u, (unsigned)key_bits(n_src), st,
+                                false) != hipSuccess)
+    return HC_ELAUNCH;
+  tr_finalize_edges<<<dim3((unsigned)eblocks), dim3(HC_BLOCK), 0, st>>>(dk.current(), dv.current(),
+                                                                        rows, rowT, edgeT, E, sentinel);
+  tr_finalize_ptr<<<dim3((unsigned)pblocks), dim3(HC_BLOCK), 0, st>>>(dk.current(), ptrT, E, n_src);
+  return hc_launch_status();
+}

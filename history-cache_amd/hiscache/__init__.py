@@ -1,0 +1,19 @@
+"""HisCache for MI355X: the package a user of the reference's ``hiscache`` imports.
+
+Exports follow /root/reference/hiscache/__init__.py:1-6 for the single-GPU hot path, plus
+``HistoryCache`` (which the reference README imports from the package but its ``__init__`` omits).
+The trainers and the multi-GPU communication helpers are not part of this package.
+"""
+from hiscache_backend import count_history_reconstruct, get_graph_structure_score, record_history
+
+from .feature_store import PinnedFeatureStore
+from .history_cache import HistoryCache
+from .history_model import HistorySAGE, MySageConvHistory, get_model
+from .history_table import HistoryTable
+from .util import Config, make_config, quantile_threshold
+
+__all__ = [
+    "HistoryCache", "HistoryTable", "HistorySAGE", "MySageConvHistory", "get_model",
+    "PinnedFeatureStore", "Config", "make_config", "quantile_threshold",
+    "count_history_reconstruct", "get_graph_structure_score", "record_history",
+]

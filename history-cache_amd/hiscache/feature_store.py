@@ -1,0 +1,57 @@
+"""Zero-copy node-feature store: features stay in pinned host memory and the GPU reads the
+requested rows directly over the host link with a gather kernel.
+
+It offers the three members of ``cxgnndl.UVM`` that the cache uses -- ``buffer``, ``get(ids)``,
+``masked_get(ids, mask)`` (call sites: /root/reference/hiscache/history_cache.py:161,283,301,345).
+``masked_get`` returns zeros for rows whose mask is false: the caller adds cached features on top
+(history_cache.py:345-349)."""
+import torch
+
+import hiscache_backend as _be
+
+
+class PinnedFeatureStore:
+
+    def __init__(self, features, device="cuda:0"):
+        if features.dim() != 2:
+            raise ValueError("features must be [num_nodes, feature_dim]")
+        if features.is_cuda:
+            self.buffer = features.contiguous()
+        else:
+            buf = features.contiguous()
+            if not buf.is_pinned():
+                pinned = torch.empty(buf.shape, dtype=buf.dtype, pin_memory=True)
+                pinned.copy_(buf)
+                buf = pinned
+            self.buffer = buf
+        self.device = torch.device(device)
+        self._side = None
+        self._done = None
+
+    def _side_stream(self):
+        if self._side is None:
+            self._side = torch.cuda.Stream(device=self.device)
+            self._done = torch.cuda.Event()
+        return self._side
+
+    def get(self, ids):
+        return _be.gather_rows(self.buffer, ids)
+
+    def masked_get(self, ids, mask):
+        return _be.gather_rows(self.buffer, ids, mask=mask)
+
+    def masked_get_async(self, ids, mask):
+        """Start the gather on a side stream (default priority) that first waits for the work
+        queued so far on the current stream.  Returns (tensor, event); wait on the event (or call
+        ``join``) before reading the tensor on another stream."""
+        cur = torch.cuda.current_stream(self.device)
+        side = self._side_stream()
+        side.wait_stream(cur)
+        with torch.cuda.stream(side):
+            out = _be.gather_rows(self.buffer, ids, mask=mask)
+            self._done.record(side)
+        out.record_stream(cur)
+        return out, self._done
+
+    def join(self, event):
+        torch.cuda.current_stream(self.device).wait_event(event)

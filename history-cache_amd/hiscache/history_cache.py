@@ -1,0 +1,248 @@
+"""HistoryCache: one flat GPU buffer holding hot raw features (filled from the end) and
+historical embeddings (appended from the front), with the id maps and the admission policy.
+
+Same public surface as the reference class (/root/reference/hiscache/history_cache.py):
+``lookup_and_load(batch, num_layer, feature_cache_only=False)``, ``update_history(batch, glb_iter)``
+and the attributes the model and trainers read (``sub2embed``, ``cached_embedding``,
+``produced_embedding``, ``used_masks``, ``method``, ``buffer``, ``full2embed``, ``embed2full``,
+``feat2full``, ``header``, ``glb_iter``).  The hot steps run as gfx950 kernels through
+``hiscache_backend``; nothing on the per-iteration path synchronises with the host.
+
+Differences that a caller can see:
+  * sizes and the hot-node list may be passed as arguments instead of being read from
+    ``processed/num_nodes.txt`` / ``processed/sorted_indices.dat`` (both still work);
+  * ``header`` lives on the device; reading the attribute synchronises;
+  * rows that would be appended beyond the buffer are dropped and counted in ``overflow``
+    (the reference raises a shape error there, history_cache.py:219-221);
+  * ``num_layer`` of ``lookup_and_load`` may be omitted (taken from the config).
+"""
+import math
+import time
+from os import path
+
+import numpy as np
+import torch
+
+import hiscache_backend as _be
+
+from .util import log, quantile_threshold
+
+
+class HistoryCache:
+
+    def __init__(self, uvm, config, mode, device_id=-1, total_num_node=None, buffer_bytes=None,
+                 hot_ids=None):
+        self.in_channels = config.dl.dataset.feature_dim
+        self.out_channels = config.dl.dataset.num_classes
+        self.hidden_channels = config.train.model.hidden_dim
+        self.num_layers_all = config.train.model.num_layers
+        if total_num_node is None:
+            total_num_node = int(
+                open(path.join(str(config["dl"]["dataset"]["path"]), "processed",
+                               "num_nodes.txt")).readline())
+        self.total_num_node = int(total_num_node)
+        self.num_device = 1
+        self.device_id = device_id
+        self.start_history = config.history.start_history
+        if config["dl"]["num_device"] > 1:
+            raise NotImplementedError("one GPU per cache; the multi-GPU trainer is out of scope")
+        self.device = torch.device(config["dl"]["device"])
+        self.method = config.history["method"]
+        self.rate = float(config.history["rate"])
+        assert self.method in ["random", "grad", "staleness"]
+        self.staleness_thres = int(config.history.staleness_thres)
+        self.limit = float(config.history.limit)
+
+        self.full2embed = torch.full((self.total_num_node * 2 + 1,), -1, dtype=torch.int64,
+                                     device=self.device)
+        self._header = torch.zeros(1, dtype=torch.int64, device=self.device)
+        self._overflow = torch.zeros(1, dtype=torch.int64, device=self.device)
+        self._num_stored = torch.zeros(1, dtype=torch.int64, device=self.device)
+        self.produced_embedding = None
+        self.feat_mode = mode
+        self.uvm = uvm
+        self.glb_iter = 0
+        self.used_masks = None
+        self.sub2embed = None
+        self.sub2feat = None
+        self.cached_embedding = None
+        self.last_record_mask = None
+        self.distributed_store = False
+        self.feat2full = torch.empty(0, dtype=torch.int64, device=self.device)
+        if "history" in self.feat_mode:
+            self.allocate(buffer_bytes)
+            self.fill(config, hot_ids)
+
+    # ------------------------------------------------------------------ attributes kept on device
+    @property
+    def header(self):
+        return int(self._header.item())
+
+    @header.setter
+    def header(self, v):
+        self._header.fill_(int(v))
+
+    @property
+    def overflow(self):
+        return int(self._overflow.item())
+
+    @property
+    def num_stored_history(self):
+        return int(self._num_stored.item())
+
+    # ------------------------------------------------------------------ sizing and pre-fill
+    def allocate(self, buffer_bytes=None):
+        """Size the flat buffer (/root/reference/hiscache/history_cache.py:95-119): free device
+        memory minus 4 GiB, capped by ``limit`` GiB, rounded up to a multiple of
+        lcm(hidden, in_channels) floats.  ``buffer_bytes`` overrides the free-memory probe."""
+        t0 = time.time()
+        if buffer_bytes is None:
+            max_byte = torch.cuda.mem_get_info(self.device)[0] - 4 * 1024 * 1024 * 1024
+        else:
+            max_byte = int(buffer_bytes)
+        lcm = self.hidden_channels * self.in_channels // math.gcd(self.hidden_channels,
+                                                                  self.in_channels)
+        max_buffer_byte = max_byte
+        if self.limit > 0 and max_buffer_byte > self.limit * 1024 * 1024 * 1024:
+            max_buffer_byte = int(self.limit * 1024 * 1024 * 1024)
+        max_buffer_byte = (max_buffer_byte + 4 * lcm - 1) // (4 * lcm) * (4 * lcm)
+        n_float = max_buffer_byte // 4
+        self.buffer = torch.empty([n_float], dtype=torch.float32, device=self.device)
+        self.embed2full = torch.full((n_float // self.hidden_channels,), -1, dtype=torch.int64,
+                                     device=self.device)
+        self.overall_feat_num = n_float // self.in_channels
+        self.overall_embed_num = n_float // self.hidden_channels
+        self.max_buffer_byte = max_buffer_byte
+        log.info(f"allocating buffer of {n_float} floats: {time.time() - t0:.3f}s")
+
+    def fill(self, config, hot_ids=None):
+        """Pre-fill the tail of the buffer with the raw features of the hottest nodes
+        (/root/reference/hiscache/history_cache.py:121-178).  ``hot_ids`` (int64, hottest last)
+        replaces ``processed/sorted_indices.dat``."""
+        t0 = time.time()
+        if hot_ids is None:
+            p = path.join(str(config["dl"]["dataset"]["path"]), "processed", "sorted_indices.dat")
+            indice = torch.from_numpy(np.fromfile(p, dtype=np.int64))
+        else:
+            indice = torch.as_tensor(hot_ids, dtype=torch.int64).cpu()
+        if self.overall_feat_num > self.total_num_node:
+            cache_indice = indice
+        else:
+            cache_indice = indice[-self.overall_feat_num:] if self.overall_feat_num > 0 else indice[:0]
+        n_cached = cache_indice.shape[0]
+        # Feature slot i of the buffer (viewed as [overall_feat_num, in_channels]) holds node
+        # feat2full[i] - total_num_node; the cached block sits at the end of the view and empty
+        # slots hold -1.  (The reference keeps only the cached block in feat2full, which shifts
+        # its slot arithmetic when the buffer could hold more than all features,
+        # history_cache.py:136-137 against :223-226.)
+        first = self.overall_feat_num - n_cached
+        new_id = torch.arange(first, first + n_cached, device=self.device)
+        self.feat2full = torch.full((self.overall_feat_num,), -1, dtype=torch.int64,
+                                    device=self.device)
+        cached_full = cache_indice.to(self.device) + self.total_num_node
+        self.feat2full[first:] = cached_full
+        self.full2embed[cached_full] = new_id
+        if n_cached > 0:
+            rows = _be.gather_rows(self.uvm.buffer, cache_indice.to(self.device))
+            self.buffer.view(-1, self.in_channels)[first:self.overall_feat_num] = rows
+        log.info(f"filling buffer with {n_cached} raw feature rows: {time.time() - t0:.3f}s")
+
+    # ------------------------------------------------------------------ admission
+    @torch.no_grad()
+    def update_history(self, batch, glb_iter):
+        """Gradient-based admission (/root/reference/hiscache/history_cache.py:180-255):
+        score = ||dL/d embedding||_2 per row, thres = quantile(score, rate), rows with
+        score < thres that are not cached are appended at ``header``; overlapped feature slots
+        and overwritten embedding slots are invalidated; maps and header advance."""
+        if "history" not in self.feat_mode or self.staleness_thres == 0:
+            return
+        if glb_iter < self.start_history:
+            return
+        if (glb_iter % self.staleness_thres) == 0:
+            torch.maximum(self._num_stored, self._header, out=self._num_stored)
+            self._header.zero_()
+        if self.produced_embedding is None:
+            raise AssertionError("produced embedding is None")
+        emb = self.produced_embedding
+        num_node = emb.shape[0]
+        if emb.grad is not None and self.method == "grad":
+            g = emb.grad
+            assert g.shape[0] == num_node, "grad shape: {}, num_node: {}".format(g.shape, num_node)
+            score = _be.row_scores(g.contiguous(), _be.NORM_L2)
+        else:
+            score = torch.randn([num_node], device=self.device)
+        emb.grad = None
+        thres = quantile_threshold(score, self.rate)
+        mask = _be.cache_append(score, thres, emb.detach().contiguous(), self.sub2embed,
+                                batch.sub_to_full[:num_node].contiguous(), self.buffer,
+                                self.hidden_channels, self.in_channels, self.full2embed,
+                                self.embed2full, self.feat2full, self._header, self._overflow)
+        self.last_record_mask = mask
+        self.last_score = score
+        self.produced_embedding = None
+
+    # ------------------------------------------------------------------ lookup
+    def lookup_and_load(self, batch, num_layer=None, feature_cache_only=False):
+        """Translate the batch's node ids to cache slots, gather cached embeddings, compute which
+        nodes are still needed, load their raw features (zero-copy from host memory, merged with
+        the feature cache) into ``batch.x``
+        (/root/reference/hiscache/history_cache.py:275-356)."""
+        if num_layer is None:
+            num_layer = self.num_layers_all
+        sub_to_full = batch.sub_to_full
+        if feature_cache_only:
+            self.sub2feat = _be.lookup(self.full2embed, sub_to_full, self.total_num_node)
+            hit = self.sub2feat != -1
+            x = self.uvm.masked_get(sub_to_full, ~hit)
+            _be.gather_rows(self.buffer.view(-1, self.in_channels), self.sub2feat, mask=hit, out=x,
+                            accumulate=True)
+            batch.x = x
+            return None
+
+        n1 = int(batch.num_node_in_layer[1])
+        if "history" not in self.feat_mode:
+            self.sub2embed = torch.full((n1,), -1, dtype=torch.int64, device=self.device)
+            self.cached_embedding = torch.empty(0, device=self.device)
+            if self.feat_mode in ["uvm", "mmap"]:
+                batch.x = self.uvm.get(sub_to_full)
+            else:
+                raise AssertionError("unsupported feat_mode " + str(self.feat_mode))
+            return None
+
+        layer1_nodes = sub_to_full[:n1]
+        self.sub2embed = _be.lookup(self.full2embed, layer1_nodes, 0)
+        self.sub2feat = _be.lookup(self.full2embed, sub_to_full, self.total_num_node)
+        self.used_masks = _be.count_history_reconstruct(batch.ptr, batch.idx, self.sub2embed,
+                                                        sub_to_full.shape[0], batch.y.shape[0],
+                                                        num_layer)
+        hit_feat_mask = self.sub2feat != -1
+        load_mask = torch.logical_and(self.used_masks[0], ~hit_feat_mask)
+        self.glb_iter += 1
+        # host-link read on a side stream, overlapped with the two HBM gathers below
+        async_get = getattr(self.uvm, "masked_get_async", None)
+        if async_get is not None:
+            x, done = async_get(sub_to_full, load_mask)
+        else:
+            x, done = self.uvm.masked_get(sub_to_full, load_mask), None
+        # slot -1 reads the last row of the view, as the reference's indexing does; such rows
+        # are ignored by the aggregation
+        self.cached_embedding = _be.gather_rows(self.buffer.view(-1, self.hidden_channels),
+                                                self.sub2embed)
+        if done is not None:
+            self.uvm.join(done)
+        _be.gather_rows(self.buffer.view(-1, self.in_channels), self.sub2feat, mask=hit_feat_mask,
+                        out=x, accumulate=True)
+        batch.x = x
+        self.load_mask = load_mask
+        return None
+
+    def stats(self):
+        """Cache occupancy (synchronises)."""
+        n = self.total_num_node
+        return {
+            "header": self.header,
+            "overflow": self.overflow,
+            "embed_cached": int((self.full2embed[:n] != -1).sum().item()),
+            "feat_cached": int((self.full2embed[n:2 * n] != -1).sum().item()),
+            "glb_iter": self.glb_iter,
+        }

@@ -1,0 +1,521 @@
+"""``hiscache_backend`` -- the operator module of HisCache, for MI355X.
+
+Drop-in for the reference's pybind11 module of the same name
+(/root/reference/src/cpp/python_bindings/binding.cpp:9-24): the six in-scope
+callables keep their names and positional signatures
+
+    aggr_forward_history, aggr_forward_history_edge_value, record_history,
+    count_history_reconstruct, get_graph_structure_score, count_num
+
+but run hand-written gfx950 kernels from ``libhiscache_hip.so`` through its C
+ABI (ctypes; raw device pointers, sizes, dtype enums, the current HIP stream).
+``p2psend`` / ``p2psend_gentensor`` (multi-GPU) are not provided.
+
+There is no CPU or PyTorch fallback: if the shared library is missing or a
+tensor is not on a GPU, the call raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhiscache_hip.so")
+
+# enums of include/hiscache_hip.h
+HC_F32, HC_F16, HC_BF16 = 0, 1, 2
+SUBST_ROW, SUBST_SRC = 0, 1
+NORM_L2, NORM_L1 = 0, 1
+CMP_LT, CMP_NOT_GT = 0, 1
+
+_DTYPES = {torch.float32: HC_F32, torch.float16: HC_F16, torch.bfloat16: HC_BF16}
+
+_c_i64 = ctypes.c_int64
+_c_p = ctypes.c_void_p
+_c_int = ctypes.c_int
+_c_sz = ctypes.c_size_t
+
+# name -> (restype, argtypes): the full export list of include/hiscache_hip.h
+_SIGNATURES = {
+    "hc_version": (ctypes.c_char_p, []),
+    "hc_strerror": (ctypes.c_char_p, [_c_int]),
+    "hc_device_count": (_c_int, []),
+    "hc_aggr_fwd": (_c_int, [_c_int, _c_p, _c_p, _c_p, _c_int, _c_p, _c_p, _c_int, _c_i64, _c_p, _c_i64,
+                             _c_p, _c_i64, _c_i64, _c_i64, _c_p]),
+    "hc_transpose_workspace_bytes": (_c_sz, [_c_i64, _c_i64, _c_i64]),
+    "hc_build_transpose": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p,
+                                    _c_sz, _c_p]),
+    "hc_aggr_bwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_p,
+                             _c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_p]),
+    "hc_count_history": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p]),
+    "hc_row_scores": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_int, _c_p]),
+    "hc_grad_check_workspace_bytes": (_c_sz, [_c_i64]),
+    "hc_grad_check": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, ctypes.c_int32, _c_int,
+                               _c_int, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_p,
+                               _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]),
+    "hc_record_history": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,
+                                   _c_i64, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]),
+    "hc_cache_append": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p,
+                                 _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_sz, _c_p]),
+    "hc_count_num": (_c_int, [_c_p, _c_i64, _c_i64, _c_p, _c_p]),
+    "hc_structure_score": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p]),
+    "hc_gather_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_i64, _c_p]),
+    "hc_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p]),
+}
+
+_lib_handle = None
+
+
+def load_library():
+    """Load ``libhiscache_hip.so`` and bind every export.  Raises if it is not built."""
+    global _lib_handle
+    if _lib_handle is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is not built; run `make -C {os.path.join(_HERE, 'csrc')}` "
+                "(there is no fallback path)")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib_handle = lib
+    return _lib_handle
+
+
+def exported_symbols():
+    return sorted(_SIGNATURES)
+
+
+def _check(rc, what):
+    if rc != 0:
+        msg = load_library().hc_strerror(rc).decode()
+        if rc in (1, 2, 4, 5):
+            raise ValueError(f"{what}: {msg}")
+        raise RuntimeError(f"{what}: {msg}")
+
+
+def _stream():
+    return _c_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    if t is None:
+        return _c_p(None)
+    return _c_p(t.data_ptr())
+
+
+def _dev(t, name, dtype=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU (got {t.device}); this module has no CPU path")
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    return t
+
+
+def _float_dtype(t, name):
+    if t.dtype not in _DTYPES:
+        raise ValueError(f"{name} must be float32, float16 or bfloat16, got {t.dtype}")
+    return _DTYPES[t.dtype]
+
+
+def _empty(t):
+    return t is None or t.numel() == 0
+
+
+def _workspace(nbytes, device):
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+# ----------------------------------------------------------------------------- raw launchers
+def _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, num_node):
+    lib = load_library()
+    _dev(ptr, "ptr", torch.int64)
+    _dev(idx, "idx", torch.int64)
+    _dev(x, "input")
+    R = int(num_node) if num_node else ptr.numel() - 1
+    if R < 0 or R > ptr.numel() - 1:
+        raise ValueError("num_node exceeds the rows of ptr")
+    n_head = 1
+    if edge_value is not None:
+        _dev(edge_value, "edge_value", torch.float32)
+        if edge_value.dim() == 2:
+            n_head = edge_value.shape[1]
+            if x.dim() != 3 or x.shape[1] != n_head:
+                raise ValueError("multi-head edge_value needs input of shape [N, H, F] with the same H")
+        elif edge_value.dim() != 1:
+            raise ValueError("edge_value must be [E] or [E, H]")
+    F = x.shape[-1]
+    n_src = x.shape[0]
+    if hmap is not None:
+        _dev(hmap, "history_map", torch.int64)
+        _dev(hbuf, "history_buffer")
+        need = R if mode == SUBST_ROW else n_src
+        if hmap.numel() < need:
+            raise ValueError(f"history_map has {hmap.numel()} entries, needs {need}")
+        if mode == SUBST_ROW and hbuf.numel() < R * hsize:
+            raise ValueError("history_buffer is smaller than num_node x history_size")
+    out_shape = (R, F) if n_head == 1 and x.dim() == 2 else (R, n_head, F)
+    out = torch.empty(out_shape, dtype=torch.float32, device=x.device)
+    rc = lib.hc_aggr_fwd(mode, _ptr(ptr), _ptr(idx), _ptr(x), _float_dtype(x, "input"),
+                         _ptr(hmap), _ptr(hbuf), _float_dtype(hbuf, "history_buffer") if hmap is not None else 0,
+                         int(hsize), _ptr(edge_value), n_head, _ptr(out), R, F, n_src, _stream())
+    _check(rc, "hc_aggr_fwd")
+    return out
+
+
+def build_transpose(ptr, idx, history_map_row, num_node, n_src, num_edge=None):
+    """Stable CSC view of the first ``num_node`` rows: returns (ptrT, rowT, edgeT).
+
+    ``num_edge`` bounds the edge slots that are sorted (default: all of ``idx``)."""
+    lib = load_library()
+    _dev(ptr, "ptr", torch.int64)
+    _dev(idx, "idx", torch.int64)
+    R = int(num_node) if num_node else ptr.numel() - 1
+    E = int(num_edge) if num_edge is not None else idx.numel()
+    E = min(E, idx.numel())
+    dev = ptr.device
+    ptrT = torch.empty(n_src + 1, dtype=torch.int64, device=dev)
+    rowT = torch.empty(max(E, 1), dtype=torch.int32, device=dev)
+    edgeT = torch.empty(max(E, 1), dtype=torch.int32, device=dev)
+    nbytes = lib.hc_transpose_workspace_bytes(R, E, n_src)
+    if nbytes == 0:
+        raise RuntimeError("hc_transpose_workspace_bytes failed (no usable GPU?)")
+    ws = _workspace(nbytes, dev)
+    hm = None if _empty(history_map_row) else _dev(history_map_row, "history_map", torch.int64)
+    rc = lib.hc_build_transpose(_ptr(ptr), _ptr(idx), _ptr(hm), R, E, n_src, _ptr(ptrT), _ptr(rowT),
+                                _ptr(edgeT), _ptr(ws), ws.numel(), _stream())
+    _check(rc, "hc_build_transpose")
+    return ptrT, rowT, edgeT
+
+
+def _aggr_bwd(ptr, idx, tr, g, hmap, edge_value, x, want_edge_grad, hbuf_shape, hsize, num_node, n_src):
+    lib = load_library()
+    ptrT, rowT, edgeT = tr
+    g = _dev(g.contiguous(), "grad_output", torch.float32)
+    R = int(num_node)
+    F = g.shape[-1]
+    n_head = g.shape[1] if g.dim() == 3 else 1
+    dev = g.device
+    gshape = (n_src, F) if g.dim() == 2 else (n_src, n_head, F)
+    grad_x = torch.empty(gshape, dtype=torch.float32, device=dev)
+    grad_h = None
+    if hmap is not None:
+        grad_h = torch.empty(hbuf_shape, dtype=torch.float32, device=dev)
+        if grad_h.numel() != R * hsize:
+            # history buffers longer than num_node rows: only the first num_node rows get gradient
+            grad_h.zero_()
+    edge_grad = None
+    if want_edge_grad:
+        edge_grad = torch.empty_like(edge_value)
+    E_total = edge_value.shape[0] if edge_value is not None else 0
+    rc = lib.hc_aggr_bwd(_ptr(ptr), _ptr(idx), _ptr(ptrT), _ptr(rowT), _ptr(edgeT), _ptr(g), _ptr(hmap),
+                         _ptr(edge_value), _ptr(x) if want_edge_grad else _c_p(None),
+                         _float_dtype(x, "input") if want_edge_grad else 0, n_head, _ptr(grad_x),
+                         _ptr(grad_h), int(hsize), _ptr(edge_grad), E_total, R, F, n_src, _stream())
+    _check(rc, "hc_aggr_bwd")
+    return grad_x, grad_h, edge_grad
+
+
+class _AggrHistory(torch.autograd.Function):
+    """Counterpart of AggrHistoryFunction / AggrHistoryEdgeValueFunction
+    (/root/reference/src/cpp/src/history_aggr.cu:475-596).  Tensor references are kept on the
+    context (the reference keeps raw addresses, :406-408)."""
+
+    @staticmethod
+    def forward(ctx, x, ptr, idx, edge_value, hmap, hbuf, hsize, num_node, mode):
+        R = int(num_node) if num_node else ptr.numel() - 1
+        out = _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, R)
+        ctx.hc = (ptr, idx, hmap, hsize, R, mode, None if hbuf is None else tuple(hbuf.shape))
+        ctx.save_for_backward(x, edge_value if edge_value is not None else x.new_empty(0))
+        ctx.has_ev = edge_value is not None
+        ctx.mark_non_differentiable()
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        ptr, idx, hmap, hsize, R, mode, hshape = ctx.hc
+        x, ev = ctx.saved_tensors
+        ev = ev if ctx.has_ev else None
+        n_src = x.shape[0]
+        row_map = hmap if mode == SUBST_ROW else None
+        tr = build_transpose(ptr, idx, row_map, R, n_src)
+        want_eg = ev is not None and ctx.needs_input_grad[3]
+        grad_x, grad_h, edge_grad = _aggr_bwd(ptr, idx, tr, g, row_map, ev, x, want_eg, hshape, hsize, R,
+                                              n_src)
+        if grad_x.dtype != x.dtype:
+            grad_x = grad_x.to(x.dtype)
+        if mode == SUBST_SRC:
+            grad_h = None
+        return grad_x, None, None, edge_grad, None, grad_h, None, None, None
+
+
+def _norm_history(history_map, history_buffer, history_size):
+    if history_size == 0 or _empty(history_map):
+        return None, None, 0
+    return history_map, history_buffer, int(history_size)
+
+
+# ----------------------------------------------------------------------------- reference API
+def aggr_forward_history(input, ptr, idx, history_map, history_buffer, history_size, num_node):
+    """Mean aggregation with history substitution; same signature as the reference
+    (/root/reference/src/cpp/include/history_aggr.h:34-37).  ``history_size == 0`` or an
+    empty ``history_map`` gives the plain mean (the reference exits there, history_aggr.cu:440-441).
+    The result always requires grad (history_aggr.cu:604)."""
+    hmap, hbuf, hsize = _norm_history(history_map, history_buffer, history_size)
+    out = _AggrHistory.apply(input, ptr, idx, None, hmap, hbuf, hsize, num_node, SUBST_ROW)
+    if not out.requires_grad:
+        out.requires_grad_(True)
+    return out
+
+
+def aggr_forward_history_edge_value(input, ptr, idx, edge_value, history_map, history_buffer,
+                                    history_size, num_node):
+    """Weighted (and multi-head) aggregation; same signature as the reference
+    (/root/reference/src/cpp/include/history_aggr.h:39-42).  An empty ``edge_value`` falls
+    back to the mean op, as the reference's dispatch does (history_aggr.cu:439)."""
+    if _empty(edge_value):
+        return aggr_forward_history(input, ptr, idx, history_map, history_buffer, history_size, num_node)
+    hmap, hbuf, hsize = _norm_history(history_map, history_buffer, history_size)
+    out = _AggrHistory.apply(input, ptr, idx, edge_value, hmap, hbuf, hsize, num_node, SUBST_ROW)
+    if not out.requires_grad:
+        out.requires_grad_(True)
+    return out
+
+
+def aggr_forward_source_history(input, ptr, idx, source_history_map, history_table, num_node=0):
+    """Extension: per-SOURCE substitution.  Neighbour j is read from
+    ``history_table[source_history_map[idx[j]]]`` when the map entry is not -1, else from
+    ``input[idx[j]]``.  Backward returns the gradient of the substituted source rows."""
+    hsize = 0 if _empty(source_history_map) else history_table.shape[-1]
+    hmap, hbuf, hsize = _norm_history(source_history_map, history_table, hsize)
+    return _AggrHistory.apply(input, ptr, idx, None, hmap, hbuf, hsize, num_node, SUBST_SRC)
+
+
+def count_history_reconstruct(ptr, idx, history_maps, num_node, num_seed, num_layer):
+    """Per-level "still needed" masks; same signature and result layout as the reference
+    (/root/reference/src/cpp/include/grad_check.h:18-20): a list of num_layer+1 bool tensors
+    of size num_node, [0] = raw-feature level, [num_layer] = seed level."""
+    lib = load_library()
+    _dev(ptr, "ptr", torch.int64)
+    _dev(idx, "idx", torch.int64)
+    hm = None if _empty(history_maps) else _dev(history_maps, "history_maps", torch.int64)
+    L = int(num_layer)
+    masks = torch.empty((L + 1, int(num_node)), dtype=torch.uint8, device=ptr.device)
+    rc = lib.hc_count_history(_ptr(ptr), _ptr(idx), _ptr(hm), 0 if hm is None else hm.numel(), _ptr(masks),
+                              ptr.numel() - 1, int(num_node), int(num_seed), L, _stream())
+    _check(rc, "hc_count_history")
+    masks = masks.view(torch.bool)
+    return [masks[i] for i in range(L + 1)]
+
+
+def record_history(buffer_new, buffer_all, used_mask, sub_to_full, sub_to_history, history_to_full,
+                   full_to_history, header, score, thres, checkin_iter, glb_iter):
+    """Ring-buffer admission on precomputed scores; same signature as the reference
+    (/root/reference/src/cpp/include/grad_check.h:12-16).  In place on ``buffer_all``,
+    ``history_to_full``, ``full_to_history``, ``header`` and ``checkin_iter``.  Slots are handed
+    out in row order (the reference: atomic arrival order)."""
+    lib = load_library()
+    _dev(buffer_new, "buffer_new", torch.float32)
+    _dev(buffer_all, "buffer_all", torch.float32)
+    M = buffer_new.shape[0]
+    hs = buffer_all.shape[1] if buffer_all.dim() == 2 else buffer_new.shape[1]
+    if buffer_new.dim() != 2 or buffer_new.shape[1] != hs:
+        raise ValueError("buffer_new must be [M, history_size]")
+    um = _dev(used_mask, "used_mask")
+    if um.dtype not in (torch.bool, torch.uint8):
+        raise ValueError("used_mask must be bool")
+    for t, n in ((sub_to_full, "sub_to_full"), (sub_to_history, "sub_to_history"),
+                 (history_to_full, "history_to_full"), (full_to_history, "full_to_history"),
+                 (header, "header"), (checkin_iter, "checkin_iter")):
+        _dev(t, n, torch.int64)
+    _dev(score, "score", torch.float32)
+    thres = _dev(thres.reshape(1).contiguous(), "thres", torch.float32)
+    if min(um.numel(), sub_to_full.numel(), sub_to_history.numel(), score.numel()) < M:
+        raise ValueError("per-row arguments are shorter than buffer_new")
+    nbytes = lib.hc_grad_check_workspace_bytes(M) + (M + 255) // 256 * 256
+    ws = _workspace(nbytes, buffer_new.device)
+    rc = lib.hc_record_history(_ptr(buffer_new), _ptr(buffer_all), _ptr(um), _ptr(sub_to_full),
+                               _ptr(sub_to_history), _ptr(history_to_full), _ptr(full_to_history),
+                               _ptr(header), _ptr(score), _ptr(thres), _ptr(checkin_iter), int(glb_iter), M,
+                               buffer_all.shape[0], hs, _ptr(ws), ws.numel(), _stream())
+    _check(rc, "hc_record_history")
+
+
+def get_graph_structure_score(ptr, idx, num_node, num_seed, num_layer):
+    """Same signature as the reference (/root/reference/src/cpp/include/grad_check.h:22-24);
+    level-synchronous and deterministic (the reference result depends on scheduling)."""
+    lib = load_library()
+    _dev(ptr, "ptr", torch.int64)
+    _dev(idx, "idx", torch.int64)
+    out = torch.empty(int(num_node), dtype=torch.int64, device=ptr.device)
+    scratch = torch.empty(int(num_node), dtype=torch.int64, device=ptr.device)
+    rc = lib.hc_structure_score(_ptr(ptr), _ptr(idx), ptr.numel() - 1, int(num_node), int(num_seed),
+                                int(num_layer), _ptr(out), _ptr(scratch), _stream())
+    _check(rc, "hc_structure_score")
+    return out
+
+
+def count_num(arr, mmax):
+    """Histogram into int32[mmax+1] that skips value 0; same signature as the reference
+    (/root/reference/src/cpp/include/grad_check.h:26)."""
+    lib = load_library()
+    _dev(arr, "arr", torch.int64)
+    out = torch.empty(int(mmax) + 1, dtype=torch.int32, device=arr.device)
+    rc = lib.hc_count_num(_ptr(arr), arr.numel(), int(mmax), _ptr(out), _stream())
+    _check(rc, "hc_count_num")
+    return out
+
+
+# ----------------------------------------------------------------------------- extensions
+def row_scores(grad, norm_kind=NORM_L2):
+    """score[r] = ||grad[r]||_2 (or the L1 norm) in the library's fixed summation order."""
+    lib = load_library()
+    _dev(grad, "grad", torch.float32)
+    if grad.dim() != 2:
+        raise ValueError("grad must be [M, F]")
+    M, F = grad.shape
+    out = torch.empty(M, dtype=torch.float32, device=grad.device)
+    _check(lib.hc_row_scores(_ptr(grad), _ptr(out), M, F, int(norm_kind), _stream()), "hc_row_scores")
+    return out
+
+
+def grad_check(grad, emb, slot, sub_to_full, thres, table, full2slot, slot2full, header, glb_iter,
+               age=None, age_limit=0, used=None, checkin=None, norm_kind=NORM_L2, cmp_kind=CMP_LT,
+               score=None, want_slots=False):
+    """Fused admission pass (scores, predicate, mask, row-order ring slots, table scatter, maps).
+
+    ``grad`` [M,F] fp32 (or None with ``score`` given), ``emb`` [M,F] fp32, ``slot`` [M] int64
+    (-1 = not cached), ``thres`` 1-element fp32 device tensor, ``table`` [capacity,F]
+    fp32/fp16/bf16, maps int64, ``header`` 1-element int64 device tensor (advanced in place).
+    Returns (mask[bool], score[f32]) and the per-row slot when ``want_slots``."""
+    lib = load_library()
+    _dev(emb, "emb", torch.float32)
+    M, F = emb.shape
+    dev = emb.device
+    if grad is not None:
+        _dev(grad, "grad", torch.float32)
+        if tuple(grad.shape) != (M, F):
+            raise ValueError("grad and emb must have the same shape")
+    elif score is None:
+        raise ValueError("either grad or score is required")
+    else:
+        _dev(score, "score", torch.float32)
+    _dev(slot, "slot", torch.int64)
+    _dev(sub_to_full, "sub_to_full", torch.int64)
+    thres = _dev(thres.reshape(1), "thres", torch.float32)
+    _dev(table, "table")
+    if table.dim() != 2 or table.shape[1] != F:
+        raise ValueError("table must be [capacity, F]")
+    for t, n in ((full2slot, "full2slot"), (slot2full, "slot2full"), (header, "header")):
+        _dev(t, n, torch.int64)
+    if slot2full.numel() < table.shape[0]:
+        raise ValueError("slot2full is shorter than the table")
+    if age is not None:
+        _dev(age, "age", torch.int32)
+    if used is not None:
+        _dev(used, "used")
+        if used.dtype not in (torch.bool, torch.uint8):
+            raise ValueError("used must be bool")
+    if checkin is not None:
+        _dev(checkin, "checkin", torch.int64)
+    mask = torch.empty(M, dtype=torch.uint8, device=dev)
+    score_out = torch.empty(M, dtype=torch.float32, device=dev)
+    slot_out = torch.empty(M, dtype=torch.int64, device=dev) if want_slots else None
+    ws = _workspace(lib.hc_grad_check_workspace_bytes(M), dev)
+    rc = lib.hc_grad_check(_ptr(grad), _ptr(score), _ptr(emb), _ptr(slot), _ptr(age), _ptr(used),
+                           _ptr(sub_to_full), _ptr(thres), int(age_limit), int(norm_kind), int(cmp_kind),
+                           _ptr(mask), _ptr(score_out), _ptr(slot_out), _ptr(table),
+                           _float_dtype(table, "table"), table.shape[0], _ptr(full2slot), _ptr(slot2full),
+                           _ptr(checkin), _ptr(header), int(glb_iter), M, F, _ptr(ws), ws.numel(), _stream())
+    _check(rc, "hc_grad_check")
+    if want_slots:
+        return mask.view(torch.bool), score_out, slot_out
+    return mask.view(torch.bool), score_out
+
+
+def cache_append(score, thres, emb, sub2embed, sub_to_full, buffer, hidden, in_channels, full2embed,
+                 embed2full, feat2full, header, overflow=None):
+    """Append-only admission of HistoryCache.update_history
+    (/root/reference/hiscache/history_cache.py:215-254) as one launch sequence.
+    ``buffer`` is the flat fp32 cache; ``header`` / ``overflow`` are 1-element int64 device tensors.
+    Returns the admission mask."""
+    lib = load_library()
+    _dev(score, "score", torch.float32)
+    _dev(emb, "emb", torch.float32)
+    M = emb.shape[0]
+    H = int(hidden)
+    if emb.dim() != 2 or emb.shape[1] != H:
+        raise ValueError("emb must be [M, hidden]")
+    thres = _dev(thres.reshape(1), "thres", torch.float32)
+    _dev(buffer, "buffer", torch.float32)
+    capacity = buffer.numel() // H
+    for t, n in ((sub2embed, "sub2embed"), (sub_to_full, "sub_to_full"), (full2embed, "full2embed"),
+                 (embed2full, "embed2full"), (header, "header")):
+        _dev(t, n, torch.int64)
+    if embed2full.numel() < capacity:
+        capacity = embed2full.numel()
+    n_feat = 0
+    if feat2full is not None and feat2full.numel() > 0:
+        _dev(feat2full, "feat2full", torch.int64)
+        n_feat = feat2full.numel()
+    else:
+        feat2full = None
+    if overflow is not None:
+        _dev(overflow, "overflow", torch.int64)
+    mask = torch.empty(M, dtype=torch.uint8, device=emb.device)
+    ws = _workspace(lib.hc_grad_check_workspace_bytes(M), emb.device)
+    rc = lib.hc_cache_append(_ptr(score), _ptr(thres), _ptr(emb), _ptr(sub2embed), _ptr(sub_to_full),
+                             _ptr(mask), _ptr(buffer), capacity, H, int(in_channels), _ptr(full2embed),
+                             _ptr(embed2full), _ptr(feat2full), n_feat, _ptr(header), _ptr(overflow), M,
+                             _ptr(ws), ws.numel(), _stream())
+    _check(rc, "hc_cache_append")
+    return mask.view(torch.bool)
+
+
+def gather_rows(src, ids, mask=None, out=None, accumulate=False):
+    """out[i] = src[ids[i]] where mask[i] (else 0), as fp32.  ``src`` may be a GPU tensor or a
+    pinned host tensor (read zero-copy over the host link).  Negative ids index from the end."""
+    lib = load_library()
+    if not isinstance(src, torch.Tensor) or src.dim() != 2 or not src.is_contiguous():
+        raise ValueError("src must be a contiguous 2-D tensor")
+    if not src.is_cuda and not src.is_pinned():
+        raise RuntimeError("src must be on the GPU or in pinned host memory")
+    _dev(ids, "ids", torch.int64)
+    n, F = ids.numel(), src.shape[1]
+    if mask is not None:
+        _dev(mask, "mask")
+        if mask.dtype not in (torch.bool, torch.uint8) or mask.numel() < n:
+            raise ValueError("mask must be a bool tensor with one entry per id")
+    if out is None:
+        if accumulate:
+            raise ValueError("accumulate needs an existing out tensor")
+        out = torch.empty((n, F), dtype=torch.float32, device=ids.device)
+    else:
+        _dev(out, "out", torch.float32)
+        if tuple(out.shape) != (n, F):
+            raise ValueError("out must be [len(ids), F]")
+    rc = lib.hc_gather_rows(_ptr(src), _float_dtype(src, "src"), src.shape[0], _ptr(ids), _ptr(mask),
+                            _ptr(out), 1 if accumulate else 0, n, F, _stream())
+    _check(rc, "hc_gather_rows")
+    return out
+
+
+def lookup(map_tensor, ids, offset=0):
+    """out[i] = map[ids[i] + offset] (int64 gather; negative positions index from the end)."""
+    lib = load_library()
+    _dev(map_tensor, "map", torch.int64)
+    _dev(ids, "ids", torch.int64)
+    out = torch.empty(ids.numel(), dtype=torch.int64, device=ids.device)
+    rc = lib.hc_lookup(_ptr(map_tensor), map_tensor.numel(), _ptr(ids), int(offset), _ptr(out), ids.numel(),
+                       _stream())
+    _check(rc, "hc_lookup")
+    return out
+
+
+def version():
+    return load_library().hc_version().decode()

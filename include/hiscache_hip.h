@@ -1,0 +1,236 @@
+/*
+ * hiscache_hip.h -- C ABI of libhiscache_hip.so, the MI355X (gfx950) kernel
+ * library for HisCache's history-aware aggregation and cache admission.
+ *
+ * It replaces the reference's pybind11 operator module `hiscache_backend`
+ * (/root/reference: src/cpp/python_bindings/binding.cpp:9-24).  The reference
+ * passes torch::Tensor handles; this ABI passes raw DEVICE pointers, sizes,
+ * dtype enums and a hipStream_t (as void*).  Conventions:
+ *
+ *   - every function returns an hc_status (0 = ok); nothing aborts the process
+ *     (the reference exits on ASSERT, src/cpp/include/common.h:13-34);
+ *   - the library never allocates or frees device memory: outputs and
+ *     workspaces are caller-owned; hc_*_workspace_bytes() sizes them;
+ *   - all launches are asynchronous on the given stream; nothing synchronises;
+ *   - indices are int64 (reference: common.h:12) unless a name says otherwise;
+ *   - feature/history data may be fp32, fp16 or bf16 (hc_dtype); accumulation
+ *     and all outputs of the aggregation are fp32;
+ *   - row-major, densely packed 2-D arrays; a NULL optional pointer means
+ *     "absent" as documented per argument.
+ */
+#ifndef HISCACHE_HIP_H
+#define HISCACHE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  HC_OK = 0,
+  HC_EINVAL = 1,       /* null pointer, negative size, inconsistent shapes */
+  HC_EDTYPE = 2,       /* unknown dtype enum */
+  HC_ELAUNCH = 3,      /* the HIP runtime reported a launch error */
+  HC_EWORKSPACE = 4,   /* workspace missing or too small */
+  HC_EUNSUPPORTED = 5, /* valid request outside what the kernels cover */
+  HC_ENODEVICE = 6     /* no usable GPU */
+} hc_status;
+
+typedef enum { HC_F32 = 0, HC_F16 = 1, HC_BF16 = 2 } hc_dtype;
+
+/* Which rows a history map substitutes. */
+typedef enum {
+  HC_SUBST_ROW = 0, /* reference rule: hmap[R] flags DESTINATION rows, hbuf[R,hsize] is row-aligned */
+  HC_SUBST_SRC = 1  /* extension: hmap[n_src] maps SOURCE ids to rows of a history table hbuf[Hn,hsize] */
+} hc_subst_mode;
+
+typedef enum { HC_NORM_L2 = 0, HC_NORM_L1 = 1 } hc_norm_kind;
+typedef enum {
+  HC_CMP_LT = 0,    /* admit when score <  thres            (hiscache/history_cache.py:215) */
+  HC_CMP_NOT_GT = 1 /* admit unless thres != 0 && score > thres (src/cpp/src/grad_check.cu:18) */
+} hc_cmp_kind;
+
+const char *hc_version(void);
+const char *hc_strerror(int status);
+/* Number of visible GPUs; 0 when there is none (never fails). */
+int hc_device_count(void);
+
+/* ---------------------------------------------------------------- aggregation forward
+ * Replaces aggr_forward_history (src/cpp/include/history_aggr.h:34-37, kernels
+ * src/cpp/src/history_aggr.cu:7-40) and aggr_forward_history_edge_value
+ * (history_aggr.h:39-42, kernels history_aggr.cu:42-125).
+ *
+ *   edge_value == NULL : mean aggregation.  Row r with hmap[r] != -1 copies
+ *       hbuf[r, :F]; otherwise vout[r,:] = (sum_j vin[idx[j],:]) / deg(r); a
+ *       zero-degree row is written as 0.
+ *   edge_value != NULL : vout[r,h,:] = sum_j edge_value[j,h] * vin[idx[j],h,:]
+ *       (fused multiply-add, no division); history rows copy hbuf[r,:F]
+ *       (hsize == F) or hbuf[r, h*F:(h+1)*F] (hsize == F*n_head).
+ *   mode == HC_SUBST_SRC (mean only): every neighbour row is read from
+ *       hbuf[hmap[idx[j]], :F] when hmap[idx[j]] != -1, else from vin.
+ *
+ * ptr[R+1], idx[>= ptr[R]], vin[n_src, n_head, F] (in_dtype), hmap NULL = no
+ * history, hbuf (hist_dtype), vout[R, n_head, F] fp32.  Sums run in CSR order
+ * in fp32, so results are bit-reproducible.  n_head >= 1; n_head > 1 requires
+ * edge_value. */
+int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, const void *vin, int in_dtype,
+                const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize,
+                const float *edge_value, int64_t n_head, float *vout, int64_t R, int64_t F,
+                int64_t n_src, void *stream);
+
+/* ---------------------------------------------------------------- transpose (CSC view)
+ * No reference counterpart: the reference backward scatters with float
+ * atomicAdd (history_aggr.cu:164); this library gathers over a transposed view
+ * instead, which makes the sums deterministic.
+ *
+ * Stable sort of the first E edge slots by source id.  Edge slots >= ptr[R]
+ * and, when hmap_row != NULL, edges of rows with hmap_row[r] != -1 are
+ * dropped.  Outputs: ptrT[n_src+1] (int64), rowT[E] (destination row per
+ * transposed edge, ascending inside a source), edgeT[E] (original edge slot);
+ * only the first ptrT[n_src] entries of rowT/edgeT are meaningful.
+ * Requires R, E, n_src < 2^31 - 1. */
+size_t hc_transpose_workspace_bytes(int64_t R, int64_t E, int64_t n_src);
+int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row, int64_t R,
+                       int64_t E, int64_t n_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT,
+                       void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------- aggregation backward
+ * Replaces AggrHistoryFunction::backward / AggrHistoryEdgeValueFunction::backward
+ * (history_aggr.cu:493-596; kernels :127-397).
+ *
+ *   grad_vin[n_src, n_head, F] : for every source s, the sum over its incoming
+ *       edges (ascending destination row) of g[r,h,:]/deg(r) (mean) or
+ *       g[r,h,:]*edge_value[j,h] (weighted); rows without edges are written 0.
+ *   grad_hbuf[R, hsize] (nullable; HC_SUBST_ROW with hmap only): g[r,:] for
+ *       history rows, 0 elsewhere.  With n_head > 1 and hsize == F the heads
+ *       are summed in head order; with hsize == F*n_head they are concatenated.
+ *   edge_grad[E_total, n_head] (nullable; needs edge_value and vin):
+ *       edge_grad[j,h] = <g[r,h,:], vin[idx[j],h,:]> for edges of non-history
+ *       rows, 0 for the others.  E_total = number of edge slots to fill.
+ *
+ * ptrT/rowT/edgeT come from hc_build_transpose called with the same hmap_row
+ * (so edges of history rows are already gone).  In HC_SUBST_SRC mode pass
+ * hmap = NULL: the result is the gradient with respect to the substituted
+ * source row, whichever table it came from. */
+int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t *ptrT, const int32_t *rowT,
+                const int32_t *edgeT, const float *g, const int64_t *hmap, const float *edge_value,
+                const void *vin, int in_dtype, int64_t n_head, float *grad_vin, float *grad_hbuf,
+                int64_t hsize, float *edge_grad, int64_t E_total, int64_t R, int64_t F,
+                int64_t n_src, void *stream);
+
+/* ---------------------------------------------------------------- used masks
+ * Replaces count_history_reconstruct (src/cpp/include/grad_check.h:18-20,
+ * src/cpp/src/grad_check.cu:70-130).  masks is (num_layer+1) x n_all bytes
+ * (0/1), written in full: masks[num_layer] is the seed level, masks[0] the
+ * raw-feature level.  hmap (nullable) covers rows [0, hmap_len); rows beyond
+ * it count as "no history". */
+int hc_count_history(const int64_t *ptr, const int64_t *idx, const int64_t *hmap, int64_t hmap_len,
+                     uint8_t *masks, int64_t ptr_rows, int64_t n_all, int64_t n_seed, int num_layer,
+                     void *stream);
+
+/* ---------------------------------------------------------------- admission
+ * hc_row_scores: score[r] = ||grad[r,:]||_2 (hiscache/history_cache.py:205) or
+ * sum|grad[r,:]| (hiscache/history_table.py:161).  Summation order: element e
+ * of a row belongs to lane (e/4)%64; a lane folds its elements in increasing e
+ * (L2: acc = fma(x,x,acc)); the 64 partials are combined by a butterfly with
+ * partner distance 32,16,8,4,2,1; L2 takes sqrtf (correctly rounded). */
+int hc_row_scores(const float *grad, float *score, int64_t M, int64_t F, int norm_kind, void *stream);
+
+/* hc_grad_check: the fused admission pass.  Replaces record_history
+ * (grad_check.h:12-16, grad_check.cu:6-68) and the torch sequence of
+ * HistoryCache.update_history (hiscache/history_cache.py:205-221,243-254).
+ *
+ *   score[r] = row score of grad (grad != NULL) or score_in[r] (grad == NULL)
+ *   pass[r]  = cmp(score[r], *thres)                 (thres: 1 fp32 on device)
+ *   admit[r] = (used == NULL || used[r]) && pass[r] &&
+ *              (slot[r] == -1 || (age != NULL && age[r] >= age_limit))
+ *   mask_out[r] = admit[r]; score_out[r] = score[r] (nullable)
+ *
+ * Admitted rows take ring slots in ROW ORDER: the k-th admitted row gets
+ * (header + k) mod capacity; header advances by the admitted count (the
+ * reference hands slots out in atomic arrival order, grad_check.cu:25).  Per
+ * admitted row: the slot's previous owner is un-mapped if it still points at
+ * the slot (grad_check.cu:26-30), emb[r,:F] is stored into table[slot,:F]
+ * (converted to table_dtype, round to nearest even), full2slot[sub_to_full[r]]
+ * = slot, slot2full[slot] = sub_to_full[r], checkin[slot] = glb_iter
+ * (:40-45; checkin nullable).  slot_out[r] (nullable) = slot or -1.
+ * If more rows are admitted than the ring holds, the result equals inserting
+ * them one by one in row order.  sub_to_full[0:M) must not repeat an id.
+ * header is 1 int64 on the device, updated in place. */
+size_t hc_grad_check_workspace_bytes(int64_t M);
+int hc_grad_check(const float *grad, const float *score_in, const float *emb, const int64_t *slot,
+                  const int32_t *age, const uint8_t *used, const int64_t *sub_to_full,
+                  const float *thres, int32_t age_limit, int norm_kind, int cmp_kind,
+                  uint8_t *mask_out, float *score_out, int64_t *slot_out, void *table,
+                  int table_dtype, int64_t capacity, int64_t *full2slot, int64_t *slot2full,
+                  int64_t *checkin, int64_t *header, int64_t glb_iter, int64_t M, int64_t F,
+                  void *workspace, size_t workspace_bytes, void *stream);
+
+/* hc_record_history: the reference's argument set, in its order
+ * (grad_check.h:12-16): precomputed score, device threshold, used mask,
+ * "not greater" comparison, fp32 table buffer_all[history_num, history_size].
+ * Same row-order slot rule as hc_grad_check. */
+int hc_record_history(const float *buffer_new, float *buffer_all, const uint8_t *used_mask,
+                      const int64_t *sub_to_full, const int64_t *sub_to_history,
+                      int64_t *history_to_full, int64_t *full_to_history, int64_t *header,
+                      const float *score, const float *thres, int64_t *checkin_iter,
+                      int64_t glb_iter, int64_t M, int64_t history_num, int64_t history_size,
+                      void *workspace, size_t workspace_bytes, void *stream);
+
+/* hc_cache_append: the append-only admission of HistoryCache.update_history
+ * (hiscache/history_cache.py:215-254) as one sequence of launches.
+ *   mask[r] = (score[r] < *thres) && (sub2embed[r] == -1)                    (:215)
+ *   the k-th admitted row is written to embedding slot header + k            (:216-221)
+ *   feature slots overlapped by [header, header+A) are invalidated:
+ *     full2embed[feat2full[b:e]] = -1, b = header*H/F_in,
+ *     e = ceil((header+A)*H/F_in), clipped to n_feat                         (:223-226)
+ *   previous owners of the overwritten slots are un-mapped when they point
+ *     into [header, header+A)                                                (:230-240)
+ *   full2embed[sub_to_full[r]] = slot, embed2full[slot] = sub_to_full[r]     (:243-253)
+ *   header += A                                                              (:254)
+ * buffer is the flat fp32 cache viewed as [capacity, H]; rows that would land
+ * at or beyond `capacity` are dropped and *overflow (1 int64, nullable) is set
+ * to their count (the reference raises a shape error there).  header is 1
+ * int64 on the device. */
+int hc_cache_append(const float *score, const float *thres, const float *emb,
+                    const int64_t *sub2embed, const int64_t *sub_to_full, uint8_t *mask_out,
+                    float *buffer, int64_t capacity, int64_t H, int64_t F_in, int64_t *full2embed,
+                    int64_t *embed2full, const int64_t *feat2full, int64_t n_feat, int64_t *header,
+                    int64_t *overflow, int64_t M, void *workspace, size_t workspace_bytes,
+                    void *stream);
+
+/* ---------------------------------------------------------------- helpers
+ * hc_count_num replaces count_num (grad_check.h:26, grad_check.cu:165-182):
+ * histogram of arr into out[mmax+1] (int32, zeroed here) that skips value 0.
+ * Values outside [0, mmax] are ignored. */
+int hc_count_num(const int64_t *arr, int64_t n, int64_t mmax, int32_t *out, void *stream);
+
+/* hc_structure_score replaces get_graph_structure_score (grad_check.h:22-24,
+ * grad_check.cu:132-163) with a level-synchronous, deterministic reading of
+ * the same rule: per pass, seeds hold 1; a row with a non-zero value offers
+ * value*deg to each neighbour that was 0 before the pass; the smallest offer
+ * wins.  out[n_all] int64; scratch[n_all] int64 is caller-provided. */
+int hc_structure_score(const int64_t *ptr, const int64_t *idx, int64_t ptr_rows, int64_t n_all,
+                       int64_t n_seed, int num_layer, int64_t *out, int64_t *scratch, void *stream);
+
+/* hc_gather_rows: dst[i,:] = (mask == NULL || mask[i]) ? src[ids[i],:] : 0,
+ * optionally accumulated (dst += ...) when accumulate != 0.  A negative id
+ * addresses from the end (-1 = last row), as the torch indexing it replaces
+ * does (hiscache/history_cache.py:312-313,345-350).  src may be device memory
+ * or pinned, mapped host memory (zero-copy read over the host link); dst is
+ * fp32 [n, F]; src is [n_rows, F] of src_dtype. */
+int hc_gather_rows(const void *src, int src_dtype, int64_t n_rows, const int64_t *ids,
+                   const uint8_t *mask, float *dst, int accumulate, int64_t n, int64_t F,
+                   void *stream);
+
+/* hc_lookup: out[i] = map[ids[i] + offset]  (int64 gather; the id translation
+ * of lookup_and_load, hiscache/history_cache.py:310,315). */
+int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset, int64_t *out,
+              int64_t n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HISCACHE_HIP_H */

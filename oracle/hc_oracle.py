@@ -1,0 +1,298 @@
+"""NumPy front end of the CPU oracle (``hc_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: tests, the smoke check and the benchmark's CPU
+baseline leg may import this module; the product package never does.
+
+Every function takes and returns NumPy arrays (int64 indices, fp32 data) and
+calls the plain-C restatement of the reference semantics.  The C file cites the
+reference lines each routine follows.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liborc.so")
+
+NORM_L2, NORM_L1 = 0, 1
+CMP_LT, CMP_NOT_GT = 0, 1
+DT_F32, DT_F16, DT_BF16 = 0, 1, 2
+
+
+def build(force=False):
+    """Compile ``hc_oracle.c`` with gcc (a one-file build, about a second)."""
+    src = os.path.join(_HERE, "hc_oracle.c")
+    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liborc.so"], stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.orc_row_score.restype = ctypes.c_float
+        _lib.orc_f16_to_f32.restype = ctypes.c_float
+        _lib.orc_bf16_to_f32.restype = ctypes.c_float
+        _lib.orc_f32_to_f16.restype = ctypes.c_uint16
+        _lib.orc_f32_to_bf16.restype = ctypes.c_uint16
+    return _lib
+
+
+def _p(a):
+    if a is None:
+        return ctypes.c_void_p(None)
+    assert a.flags["C_CONTIGUOUS"], "oracle arrays must be C-contiguous"
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def _i64(a):
+    return np.ascontiguousarray(a, dtype=np.int64)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _u8(a):
+    return None if a is None else np.ascontiguousarray(a).astype(np.uint8)
+
+
+def _I(v):
+    return ctypes.c_int64(int(v))
+
+
+def _check(rc, name):
+    if rc != 0:
+        raise ValueError(f"oracle {name} rejected its input (code {rc})")
+
+
+# --------------------------------------------------------------------------- aggregation
+def fwd_mean_row(ptr, idx, vin, hmap, hbuf, num_node=None):
+    ptr, idx, vin = _i64(ptr), _i64(idx), _f32(vin)
+    R = len(ptr) - 1 if not num_node else int(num_node)
+    F = vin.shape[-1]
+    hsize = 0
+    if hmap is not None:
+        hmap, hbuf = _i64(hmap), _f32(hbuf)
+        hsize = hbuf.shape[-1] if hbuf.ndim == 2 else F
+    out = np.zeros((R, F), np.float32)
+    _check(lib().orc_fwd_mean_row(_p(ptr), _p(idx), _p(vin), _p(hmap), _p(hbuf), _p(out),
+                                  _I(R), _I(F), _I(hsize)), "fwd_mean_row")
+    return out
+
+
+def fwd_edge_value(ptr, idx, ev, vin, hmap, hbuf, num_node=None):
+    ptr, idx, vin, ev = _i64(ptr), _i64(idx), _f32(vin), _f32(ev)
+    R = len(ptr) - 1 if not num_node else int(num_node)
+    if ev.ndim == 2:
+        H, F = vin.shape[1], vin.shape[2]
+        hsize = 0
+        if hmap is not None:
+            hmap, hbuf = _i64(hmap), _f32(hbuf)
+            hsize = hbuf.shape[-1]
+        out = np.zeros((R, H, F), np.float32)
+        _check(lib().orc_fwd_edge_value_multi_head(_p(ptr), _p(idx), _p(ev), _p(vin), _p(hmap),
+                                                   _p(hbuf), _p(out), _I(R), _I(F), _I(hsize), _I(H)),
+               "fwd_edge_value_multi_head")
+        return out
+    F = vin.shape[-1]
+    hsize = 0
+    if hmap is not None:
+        hmap, hbuf = _i64(hmap), _f32(hbuf)
+        hsize = hbuf.shape[-1]
+    out = np.zeros((R, F), np.float32)
+    _check(lib().orc_fwd_edge_value(_p(ptr), _p(idx), _p(ev), _p(vin), _p(hmap), _p(hbuf), _p(out),
+                                    _I(R), _I(F), _I(hsize)), "fwd_edge_value")
+    return out
+
+
+def fwd_mean_src(ptr, idx, feat, hmap_src, hist, num_node=None):
+    ptr, idx, feat = _i64(ptr), _i64(idx), _f32(feat)
+    R = len(ptr) - 1 if not num_node else int(num_node)
+    F = feat.shape[-1]
+    hsize = 0
+    if hmap_src is not None:
+        hmap_src, hist = _i64(hmap_src), _f32(hist)
+        hsize = hist.shape[-1]
+    out = np.zeros((R, F), np.float32)
+    _check(lib().orc_fwd_mean_src(_p(ptr), _p(idx), _p(feat), _p(hmap_src), _p(hist), _p(out),
+                                  _I(R), _I(F), _I(hsize)), "fwd_mean_src")
+    return out
+
+
+def bwd_mean_row(ptr, idx, g, hmap, n_src, hbuf_shape=None):
+    """Returns (grad_input[n_src,F], grad_history[R,hsize] or None)."""
+    ptr, idx, g = _i64(ptr), _i64(idx), _f32(g)
+    R, F = g.shape
+    gout = np.zeros((n_src, F), np.float32)
+    ghist = None
+    hsize = 0
+    if hmap is not None:
+        hmap = _i64(hmap)
+        hsize = hbuf_shape[-1] if hbuf_shape is not None else F
+        ghist = np.zeros((R, hsize), np.float32)
+    _check(lib().orc_bwd_mean_row(_p(ptr), _p(idx), _p(g), _p(hmap), _p(gout), _p(ghist),
+                                  _I(R), _I(F), _I(hsize), _I(n_src)), "bwd_mean_row")
+    return gout, ghist
+
+
+def bwd_mean_src(ptr, idx, g, n_src):
+    return bwd_mean_row(ptr, idx, g, None, n_src)[0]
+
+
+def bwd_edge_value(ptr, idx, ev, g, hmap, vin, n_src, hsize=None, want_edge_grad=False):
+    """Returns (grad_input, grad_history or None, edge_grad or None)."""
+    ptr, idx, ev, g = _i64(ptr), _i64(idx), _f32(ev), _f32(g)
+    E = len(idx)
+    vin = _f32(vin) if vin is not None else None
+    if ev.ndim == 2:
+        R, H, F = g.shape
+        hs = 0
+        ghist = None
+        if hmap is not None:
+            hmap = _i64(hmap)
+            hs = int(hsize)
+            ghist = np.zeros((R, hs), np.float32)
+        gout = np.zeros((n_src, H, F), np.float32)
+        eg = np.zeros((E, H), np.float32) if want_edge_grad else None
+        _check(lib().orc_bwd_edge_value_multi_head(_p(ptr), _p(idx), _p(ev), _p(g), _p(hmap), _p(vin),
+                                                   _p(gout), _p(ghist), _p(eg), _I(R), _I(F), _I(hs),
+                                                   _I(H), _I(n_src), _I(E)), "bwd_edge_value_multi_head")
+        return gout, ghist, eg
+    R, F = g.shape
+    hs = 0
+    ghist = None
+    if hmap is not None:
+        hmap = _i64(hmap)
+        hs = int(hsize) if hsize else F
+        ghist = np.zeros((R, hs), np.float32)
+    gout = np.zeros((n_src, F), np.float32)
+    eg = np.zeros((E,), np.float32) if want_edge_grad else None
+    _check(lib().orc_bwd_edge_value(_p(ptr), _p(idx), _p(ev), _p(g), _p(hmap), _p(vin), _p(gout),
+                                    _p(ghist), _p(eg), _I(R), _I(F), _I(hs), _I(n_src), _I(E)),
+           "bwd_edge_value")
+    return gout, ghist, eg
+
+
+def build_transpose(ptr, idx, hmap_row, n_src, num_node=None):
+    """Stable CSC view: (ptrT[n_src+1], rowT[E_kept], edgeT[E_kept])."""
+    ptr, idx = _i64(ptr), _i64(idx)
+    R = len(ptr) - 1 if not num_node else int(num_node)
+    hm = _i64(hmap_row) if hmap_row is not None else None
+    E = int(ptr[R])
+    ptrT = np.zeros(n_src + 1, np.int64)
+    rowT = np.zeros(max(E, 1), np.int32)
+    edgeT = np.zeros(max(E, 1), np.int32)
+    _check(lib().orc_build_transpose(_p(ptr), _p(idx), _p(hm), _I(R), _I(n_src), _p(ptrT), _p(rowT),
+                                     _p(edgeT)), "build_transpose")
+    k = int(ptrT[n_src])
+    return ptrT, rowT[:k].copy(), edgeT[:k].copy()
+
+
+# --------------------------------------------------------------------------- used masks
+def count_history_reconstruct(ptr, idx, history_map, num_node, num_seed, num_layer):
+    """Returns a list of num_layer+1 bool arrays of size num_node (reference order)."""
+    ptr, idx = _i64(ptr), _i64(idx)
+    hm = _i64(history_map) if history_map is not None else None
+    L = int(num_layer)
+    masks = np.zeros((L + 1, int(num_node)), np.uint8)
+    _check(lib().orc_count_history(_p(ptr), _p(idx), _p(hm), _I(0 if hm is None else len(hm)),
+                                   _p(masks), _I(len(ptr) - 1), _I(num_node), _I(num_seed),
+                                   ctypes.c_int(L)), "count_history")
+    return [masks[i].astype(bool) for i in range(L + 1)]
+
+
+# --------------------------------------------------------------------------- admission
+def row_scores(grad, norm_kind=NORM_L2):
+    grad = _f32(grad)
+    M, F = grad.shape
+    out = np.zeros(M, np.float32)
+    lib().orc_row_scores(_p(grad), _p(out), _I(M), _I(F), ctypes.c_int(norm_kind))
+    return out
+
+
+def record_history(buffer_new, buffer_all, used_mask, sub_to_full, sub_to_history, history_to_full,
+                   full_to_history, header, score, thres, checkin_iter, glb_iter):
+    """In-place on buffer_all / history_to_full / full_to_history / header / checkin_iter
+    (all NumPy arrays of the reference dtypes).  Returns the admitted mask."""
+    for a, dt in ((buffer_all, np.float32), (history_to_full, np.int64), (full_to_history, np.int64),
+                  (header, np.int64), (checkin_iter, np.int64)):
+        assert a.dtype == dt and a.flags["C_CONTIGUOUS"]
+    buffer_new = _f32(buffer_new)
+    M = buffer_new.shape[0]
+    mask = np.zeros(M, np.uint8)
+    thres = np.asarray(thres, np.float32).reshape(1)
+    _check(lib().orc_record_history(_p(buffer_new), _p(buffer_all), _p(_u8(used_mask)),
+                                    _p(_i64(sub_to_full)), _p(_i64(sub_to_history)),
+                                    _p(history_to_full), _p(full_to_history), _p(header),
+                                    _p(_f32(score)), _p(thres), _p(checkin_iter), _I(glb_iter), _I(M),
+                                    _I(buffer_all.shape[0]), _I(buffer_all.shape[1]), _p(mask)),
+           "record_history")
+    return mask.astype(bool)
+
+
+def grad_check(grad, emb, slot, age, used, sub_to_full, thres, age_limit, norm_kind, cmp_kind, table,
+               table_dtype, full2slot, slot2full, checkin, header, glb_iter, score_in=None):
+    """Fused admission.  `table` is a NumPy array viewed as fp32 or uint16 (fp16/bf16 bits);
+    maps/header are int64 arrays updated in place.
+    Returns (mask[bool], score[f32], slot_of_row[int64, -1 when not admitted])."""
+    emb = _f32(emb)
+    M, F = emb.shape
+    grad = _f32(grad) if grad is not None else None
+    score_in = _f32(score_in) if score_in is not None else None
+    mask = np.zeros(M, np.uint8)
+    score = np.zeros(M, np.float32)
+    slot_out = np.zeros(M, np.int64)
+    age = np.ascontiguousarray(age, np.int32) if age is not None else None
+    assert table.flags["C_CONTIGUOUS"]
+    _check(lib().orc_grad_check(_p(grad), _p(score_in), _p(emb), _p(_i64(slot)), _p(age), _p(_u8(used)),
+                                _p(_i64(sub_to_full)), ctypes.c_float(float(thres)),
+                                ctypes.c_int32(int(age_limit)), ctypes.c_int(norm_kind),
+                                ctypes.c_int(cmp_kind), _p(mask), _p(score), _p(table),
+                                ctypes.c_int(table_dtype), _I(table.shape[0]), _p(full2slot),
+                                _p(slot2full), _p(checkin), _p(header), _I(glb_iter), _I(M), _I(F),
+                                _p(slot_out)), "grad_check")
+    return mask.astype(bool), score, slot_out
+
+
+# --------------------------------------------------------------------------- helpers
+def count_num(arr, mmax):
+    arr = _i64(arr)
+    out = np.zeros(int(mmax) + 1, np.int32)
+    _check(lib().orc_count_num(_p(arr), _I(len(arr)), _I(mmax), _p(out)), "count_num")
+    return out
+
+
+def get_graph_structure_score(ptr, idx, num_node, num_seed, num_layer):
+    ptr, idx = _i64(ptr), _i64(idx)
+    out = np.zeros(int(num_node), np.int64)
+    _check(lib().orc_structure_score(_p(ptr), _p(idx), _I(len(ptr) - 1), _I(num_node), _I(num_seed),
+                                     ctypes.c_int(int(num_layer)), _p(out)), "structure_score")
+    return out
+
+
+def gather_rows(table, ids, mask=None):
+    table = _f32(table)
+    ids = _i64(ids)
+    out = np.zeros((len(ids), table.shape[1]), np.float32)
+    _check(lib().orc_gather_rows(_p(table), _I(table.shape[0]), _p(ids), _p(_u8(mask)), _p(out),
+                                 _I(len(ids)), _I(table.shape[1])), "gather_rows")
+    return out
+
+
+def f32_to_f16_bits(x):
+    x = _f32(x).ravel()
+    return np.array([lib().orc_f32_to_f16(ctypes.c_float(v)) for v in x], np.uint16)
+
+
+def f32_to_bf16_bits(x):
+    x = _f32(x).ravel()
+    return np.array([lib().orc_f32_to_bf16(ctypes.c_float(v)) for v in x], np.uint16)

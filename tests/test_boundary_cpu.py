@@ -1,0 +1,102 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header declares, and its
+argument checks return status codes (no kernel is launched here)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hiscache_hip.h")
+
+
+def header_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hc_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    import hiscache_backend as be
+    assert header_functions() == be.exported_symbols()
+
+
+def test_library_exports_every_declared_symbol():
+    import hiscache_backend as be
+    lib = be.load_library()
+    for name in header_functions():
+        assert hasattr(lib, name), name
+    assert b"gfx950" in lib.hc_version()
+    assert lib.hc_strerror(0) == b"ok"
+    assert lib.hc_device_count() >= 0
+
+
+def test_argument_errors_are_status_codes():
+    import hiscache_backend as be
+    lib = be.load_library()
+    null = ctypes.c_void_p(None)
+    # negative row count, zero feature width
+    assert lib.hc_aggr_fwd(0, null, null, null, 0, null, null, 0, 0, null, 1, null, -1, 4, 0, null) == 1
+    assert lib.hc_aggr_fwd(0, null, null, null, 0, null, null, 0, 0, null, 1, null, 4, 0, 0, null) == 1
+    # missing pointers
+    assert lib.hc_aggr_fwd(0, null, null, null, 0, null, null, 0, 0, null, 1, null, 4, 4, 4, null) == 1
+    buf = np.zeros(64, np.int64)
+    p = ctypes.c_void_p(buf.ctypes.data)
+    # unknown dtype / substitution mode
+    assert lib.hc_aggr_fwd(0, p, p, p, 7, null, null, 0, 0, null, 1, p, 4, 4, 4, null) == 2
+    assert lib.hc_aggr_fwd(9, p, p, p, 0, null, null, 0, 0, null, 1, p, 4, 4, 4, null) == 1
+    # heads need edge values; history map needs a buffer
+    assert lib.hc_aggr_fwd(0, p, p, p, 0, null, null, 0, 0, null, 2, p, 4, 4, 4, null) == 1
+    assert lib.hc_aggr_fwd(0, p, p, p, 0, p, null, 0, 4, null, 1, p, 4, 4, 4, null) == 1
+    # grad_check: bad enums, missing workspace
+    args = [p, null, p, p, null, null, p, p, 0, 0, 0, p, null, null, p, 0, 8, p, p, null, p, 0, 4, 4]
+    assert lib.hc_grad_check(*args, null, 0, null) == 4
+    bad = list(args); bad[9] = 5
+    assert lib.hc_grad_check(*bad, p, 512, null) == 1
+    bad = list(args); bad[15] = 9
+    assert lib.hc_grad_check(*bad, p, 512, null) == 2
+    assert lib.hc_grad_check_workspace_bytes(2_000_000) >= 8 * (2_000_000 // 64)
+    assert lib.hc_row_scores(null, null, 4, 4, 0, null) == 1
+    assert lib.hc_gather_rows(p, 5, 4, p, null, p, 0, 2, 4, null) == 2
+    assert lib.hc_count_history(null, null, null, 0, null, 4, 4, 1, 2, null) == 1
+    for code in range(0, 8):
+        assert lib.hc_strerror(code)
+
+
+def test_python_shim_refuses_cpu_tensors():
+    import torch
+    import hiscache_backend as be
+    x = torch.zeros(4, 4)
+    ptr = torch.zeros(5, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="GPU"):
+        be.aggr_forward_history(x, ptr, ptr, torch.tensor([]), torch.tensor([]), 0, 4)
+    with pytest.raises(RuntimeError, match="GPU"):
+        be.count_history_reconstruct(ptr, ptr, ptr, 4, 1, 2)
+    with pytest.raises(RuntimeError):
+        be.gather_rows(torch.zeros(4, 4), ptr)          # neither on the GPU nor pinned
+
+
+def test_config_and_synthetic_batch_layout():
+    from hiscache import make_config
+    from hiscache.synthetic import direct_power_law_batch, sample_layered_batch, uniform_graph, zipf_degrees
+    cfg = make_config(128, 10, 128, 2)
+    assert cfg.dl.dataset.feature_dim == cfg["dl"]["dataset"]["feature_dim"] == 128
+    assert cfg.history.get("store_last_layer", False) is False
+    rng = np.random.default_rng(0)
+    indptr, indices = uniform_graph(2000, 15, 1)
+    s = sample_layered_batch(indptr, indices, rng.choice(2000, 50, replace=False), [10, 5], rng)
+    nnl = s["num_node_in_layer"]
+    assert len(s["ptr"]) - 1 == nnl[1] and nnl[0] == 50 and nnl[2] == len(s["sub_to_full"])
+    assert len(np.unique(s["sub_to_full"])) == len(s["sub_to_full"])
+    assert s["idx"][: s["ptr"][nnl[0]]].max() < nnl[1]             # seeds' neighbours are within 1 hop
+    for r in range(len(s["ptr"]) - 1):                              # sampled edges exist in the graph
+        full = s["sub_to_full"][r]
+        nb = s["sub_to_full"][s["idx"][s["ptr"][r]:s["ptr"][r + 1]]]
+        assert np.isin(nb, indices[indptr[full]:indptr[full + 1]]).all()
+    d = direct_power_law_batch(10**7, 100, [15, 10, 5], 2.0, 3)
+    nnl = d["num_node_in_layer"]
+    assert len(d["ptr"]) - 1 == nnl[2] and d["idx"].max() < nnl[3]
+    assert len(np.unique(d["sub_to_full"])) == len(d["sub_to_full"])
+    deg = zipf_degrees(10000, 200000, 2.1, 5000, rng)
+    assert deg.sum() == 200000 and deg.min() >= 1 and deg.max() <= 5000

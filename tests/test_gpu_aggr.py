@@ -1,0 +1,264 @@
+"""GPU parity of the aggregation kernels (forward, transpose, backward) against the CPU oracle,
+through the C ABI (``hiscache_backend`` is a ctypes shim over ``libhiscache_hip.so``).
+
+Bars: index outputs bit-exact; fp32 aggregates bit-exact against the oracle (same summation
+order) and within 1e-5 relative of an fp64 closed form; fp16/bf16 inputs within 1e-2."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import random_csr, random_hmap
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def T(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+    return t.to(dtype) if dtype is not None else t
+
+
+def none():
+    return torch.empty(0, device=DEV)
+
+
+@pytest.fixture(scope="module")
+def be():
+    import hiscache_backend
+    hiscache_backend.load_library()
+    assert torch.cuda.is_available()
+    return hiscache_backend
+
+
+CASES = [  # (R, N, F, maxdeg, hub, dtype)
+    (300, 200, 256, 12, 300, torch.float32),   # fast path 16-byte loads, a row longer than one staging batch
+    (300, 200, 128, 12, 130, torch.float32),   # 8-byte loads
+    (257, 100, 64, 9, None, torch.float32),    # 4-byte loads
+    (200, 150, 512, 20, 70, torch.float32),    # two chunks per lane
+    (120, 90, 768, 6, None, torch.float32),    # three chunks
+    (120, 90, 1024, 6, 65, torch.float32),     # four chunks
+    (150, 120, 100, 10, 100, torch.float32),   # generic path (F not a multiple of 64)
+    (90, 70, 172, 5, None, torch.float32),     # generic path
+    (90, 70, 300, 5, None, torch.float32),     # generic path, more than one column tile
+    (200, 150, 256, 12, 80, torch.float16),
+    (200, 150, 768, 12, 80, torch.float16),    # mag240M-shaped rows
+    (200, 150, 512, 12, None, torch.bfloat16),
+    (64, 50, 1, 4, None, torch.float32),
+]
+
+
+@pytest.mark.parametrize("R,N,F,maxdeg,hub,dtype", CASES)
+@pytest.mark.parametrize("with_hist", [False, True])
+def test_fwd_mean_row_mode(be, orc, R, N, F, maxdeg, hub, dtype, with_hist):
+    rng = np.random.default_rng(R * 7 + F)
+    ptr, idx = random_csr(rng, R, N, maxdeg, hub=hub)
+    x = T(rng.standard_normal((N, F)).astype(np.float32), dtype)
+    x32 = x.float().cpu().numpy()
+    if with_hist:
+        hmap = random_hmap(rng, R, 0.35)
+        hbuf = T(rng.standard_normal((R, F)).astype(np.float32), dtype)
+        out = be.aggr_forward_history(x, T(ptr), T(idx), T(hmap), hbuf, F, R)
+        ref = orc.fwd_mean_row(ptr, idx, x32, hmap, hbuf.float().cpu().numpy())
+    else:
+        out = be.aggr_forward_history(x, T(ptr), T(idx), none(), none(), 0, R)
+        ref = orc.fwd_mean_row(ptr, idx, x32, None, None)
+    assert out.dtype == torch.float32 and out.requires_grad
+    np.testing.assert_array_equal(out.detach().cpu().numpy(), ref)
+
+
+def test_fwd_mean_closed_form_tolerance(be):
+    """Against an fp64 closed form (independent of the oracle): 1e-5 relative."""
+    rng = np.random.default_rng(1)
+    R, N, F = 500, 400, 256
+    ptr, idx = random_csr(rng, R, N, 40, hub=900)
+    x = rng.standard_normal((N, F)).astype(np.float32)
+    out = be.aggr_forward_history(T(x), T(ptr), T(idx), none(), none(), 0, 0).detach().cpu().numpy()
+    deg = np.diff(ptr)
+    ref = np.add.reduceat(x[idx].astype(np.float64), np.minimum(ptr[:-1], len(idx) - 1), axis=0)
+    ref[deg == 0] = 0
+    ref /= np.maximum(deg, 1)[:, None]
+    np.testing.assert_allclose(out, ref, rtol=1e-5, atol=1e-6)
+
+
+def test_fwd_history_wider_than_features_and_num_node(be, orc):
+    rng = np.random.default_rng(2)
+    R, N, F, hs = 100, 80, 128, 160
+    ptr, idx = random_csr(rng, R, N, 8)
+    x = rng.standard_normal((N, F)).astype(np.float32)
+    hmap = random_hmap(rng, R, 0.5)
+    hbuf = rng.standard_normal((R, hs)).astype(np.float32)
+    out = be.aggr_forward_history(T(x), T(ptr), T(idx), T(hmap), T(hbuf), hs, 61)
+    ref = orc.fwd_mean_row(ptr, idx, x, hmap[:61], hbuf[:61], num_node=61)
+    np.testing.assert_array_equal(out.detach().cpu().numpy(), ref)
+    # mixed dtypes: fp32 features, fp16 row-aligned history
+    h16 = T(hbuf[:, :F]).half()
+    out = be.aggr_forward_history(T(x), T(ptr), T(idx), T(hmap), h16, F, R)
+    ref = orc.fwd_mean_row(ptr, idx, x, hmap, h16.float().cpu().numpy())
+    np.testing.assert_array_equal(out.detach().cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("F,dtype", [(256, torch.float32), (128, torch.float32), (100, torch.float32),
+                                     (256, torch.float16)])
+def test_fwd_src_mode(be, orc, F, dtype):
+    rng = np.random.default_rng(3)
+    R, N, Hn = 400, 300, 120
+    ptr, idx = random_csr(rng, R, N, 15, hub=200)
+    feat = T(rng.standard_normal((N, F)).astype(np.float32), dtype)
+    hist = T(0.5 * rng.standard_normal((Hn, F)).astype(np.float32), dtype)
+    hmap = np.full(N, -1, np.int64)
+    hit = rng.random(N) < 0.4
+    hmap[hit] = rng.integers(0, Hn, size=int(hit.sum()))
+    out = be.aggr_forward_source_history(feat, T(ptr), T(idx), T(hmap), hist)
+    ref = orc.fwd_mean_src(ptr, idx, feat.float().cpu().numpy(), hmap, hist.float().cpu().numpy())
+    np.testing.assert_array_equal(out.detach().cpu().numpy(), ref)
+    # an all-miss map is the plain mean
+    out2 = be.aggr_forward_source_history(feat, T(ptr), T(idx), T(np.full(N, -1, np.int64)), hist)
+    out3 = be.aggr_forward_history(feat, T(ptr), T(idx), none(), none(), 0, 0)
+    assert torch.equal(out2, out3)
+
+
+@pytest.mark.parametrize("R,N,E_extra", [(200, 150, 0), (200, 150, 77), (1, 5, 0), (50, 3, 10)])
+def test_build_transpose_bit_exact(be, orc, R, N, E_extra):
+    rng = np.random.default_rng(4 + R)
+    ptr, idx = random_csr(rng, R, N, 9, hub=150)
+    idx_all = np.concatenate([idx, rng.integers(0, N, size=E_extra)]).astype(np.int64)  # edges of deeper layers
+    hmap = random_hmap(rng, R, 0.3)
+    for hm in (None, hmap):
+        ptrT, rowT, edgeT = be.build_transpose(T(ptr), T(idx_all), None if hm is None else T(hm), R, N)
+        rp, rr, re = orc.build_transpose(ptr, idx_all, hm, N, num_node=R)
+        np.testing.assert_array_equal(ptrT.cpu().numpy(), rp)
+        k = int(rp[-1])
+        np.testing.assert_array_equal(rowT.cpu().numpy()[:k], rr)
+        np.testing.assert_array_equal(edgeT.cpu().numpy()[:k], re)
+
+
+def test_build_transpose_no_edges(be):
+    ptr = torch.zeros(11, dtype=torch.int64, device=DEV)
+    idx = torch.zeros(0, dtype=torch.int64, device=DEV)
+    ptrT, _, _ = be.build_transpose(ptr, idx, None, 10, 7)
+    assert ptrT.cpu().tolist() == [0] * 8
+
+
+@pytest.mark.parametrize("R,N,F,maxdeg,hub", [(300, 200, 256, 12, 300), (300, 250, 128, 12, 130),
+                                               (200, 150, 64, 9, None), (150, 120, 512, 10, 70),
+                                               (150, 120, 100, 10, 100), (90, 70, 300, 5, None)])
+@pytest.mark.parametrize("with_hist", [False, True])
+def test_bwd_mean_bit_exact_and_deterministic(be, orc, R, N, F, maxdeg, hub, with_hist):
+    rng = np.random.default_rng(R + F)
+    ptr, idx = random_csr(rng, R, N, maxdeg, hub=hub)
+    x = T(rng.standard_normal((N, F)).astype(np.float32)).requires_grad_(True)
+    g = rng.standard_normal((R, F)).astype(np.float32)
+    if with_hist:
+        hmap = random_hmap(rng, R, 0.35)
+        hbuf = T(rng.standard_normal((R, F)).astype(np.float32)).requires_grad_(True)
+        out = be.aggr_forward_history(x, T(ptr), T(idx), T(hmap), hbuf, F, R)
+    else:
+        hmap, hbuf = None, None
+        out = be.aggr_forward_history(x, T(ptr), T(idx), none(), none(), 0, R)
+    out.backward(T(g))
+    gx, gh = orc.bwd_mean_row(ptr, idx, g, hmap, N, hbuf_shape=(R, F))
+    np.testing.assert_array_equal(x.grad.cpu().numpy(), gx)
+    if with_hist:
+        np.testing.assert_array_equal(hbuf.grad.cpu().numpy(), gh)
+    # run-to-run bit equality (no float atomics)
+    first = x.grad.clone()
+    x.grad = None
+    out2 = be.aggr_forward_history(x, T(ptr), T(idx), none() if hmap is None else T(hmap),
+                                   none() if hbuf is None else hbuf.detach(), 0 if hmap is None else F, R)
+    out2.backward(T(g))
+    assert torch.equal(first, x.grad)
+
+
+def test_bwd_retain_grad_on_output_and_raw_feature_input(be, orc):
+    """The op's output always requires grad so that the produced embedding can collect dL/d(out)
+    even when the input is a raw feature tensor (history_aggr.cu:604)."""
+    rng = np.random.default_rng(6)
+    R, N, F = 60, 50, 128
+    ptr, idx = random_csr(rng, R, N, 6)
+    x = T(rng.standard_normal((N, F)).astype(np.float32))           # no grad
+    out = be.aggr_forward_history(x, T(ptr), T(idx), none(), none(), 0, R)
+    assert out.requires_grad
+    out.retain_grad()
+    w = T(rng.standard_normal((F, 3)).astype(np.float32)).requires_grad_(True)
+    (out @ w).sum().backward()
+    assert out.grad is not None and out.grad.shape == out.shape
+
+
+def test_src_mode_backward(be, orc):
+    rng = np.random.default_rng(7)
+    R, N, F = 300, 200, 256
+    ptr, idx = random_csr(rng, R, N, 10, hub=90)
+    feat = T(rng.standard_normal((N, F)).astype(np.float32)).requires_grad_(True)
+    hist = T(rng.standard_normal((N, F)).astype(np.float32))
+    hmap = np.where(rng.random(N) < 0.4, np.arange(N), -1).astype(np.int64)
+    g = rng.standard_normal((R, F)).astype(np.float32)
+    out = be.aggr_forward_source_history(feat, T(ptr), T(idx), T(hmap), hist)
+    out.backward(T(g))
+    np.testing.assert_array_equal(feat.grad.cpu().numpy(), orc.bwd_mean_src(ptr, idx, g, N))
+
+
+@pytest.mark.parametrize("F,H", [(64, 1), (96, 1), (32, 3), (256, 2)])
+@pytest.mark.parametrize("hist_kind", ["none", "shared", "concat"])
+def test_edge_value_variants(be, orc, F, H, hist_kind):
+    rng = np.random.default_rng(F + H)
+    R, N = 120, 90
+    ptr, idx = random_csr(rng, R, N, 8, hub=70)
+    E = len(idx)
+    multi = H > 1
+    vin = rng.standard_normal((N, H, F) if multi else (N, F)).astype(np.float32)
+    ev = rng.standard_normal((E, H) if multi else (E,)).astype(np.float32)
+    g = rng.standard_normal((R, H, F) if multi else (R, F)).astype(np.float32)
+    if hist_kind == "none":
+        hmap, hbuf, hs = None, None, 0
+    else:
+        hs = F * H if (hist_kind == "concat" and multi) else F
+        hmap = random_hmap(rng, R, 0.3)
+        hbuf = rng.standard_normal((R, hs)).astype(np.float32)
+    x = T(vin).requires_grad_(True)
+    evt = T(ev).requires_grad_(True)
+    hb = None if hbuf is None else T(hbuf).requires_grad_(True)
+    out = be.aggr_forward_history_edge_value(x, T(ptr), T(idx), evt, none() if hmap is None else T(hmap),
+                                             none() if hb is None else hb, hs, R)
+    ref = orc.fwd_edge_value(ptr, idx, ev, vin, hmap, hbuf)
+    np.testing.assert_array_equal(out.detach().cpu().numpy(), ref)
+    out.backward(T(g))
+    gx, gh, eg = orc.bwd_edge_value(ptr, idx, ev, g, hmap, vin, N, hsize=hs, want_edge_grad=True)
+    np.testing.assert_array_equal(x.grad.cpu().numpy(), gx)
+    if hb is not None:
+        np.testing.assert_array_equal(hb.grad.cpu().numpy(), gh)
+    # edge_grad: dot products, summation order differs from the oracle's fp64 -> tolerance scaled by sum |terms|
+    deg = np.diff(ptr)
+    dst = np.repeat(np.arange(R), deg)
+    scale = (np.abs(g[dst]) * np.abs(vin[idx])).sum(-1)
+    err = np.abs(evt.grad.cpu().numpy() - eg)
+    assert (err <= 1e-5 * scale + 1e-7).all()
+
+
+def test_empty_inputs(be):
+    ptr = torch.zeros(1, dtype=torch.int64, device=DEV)
+    idx = torch.zeros(0, dtype=torch.int64, device=DEV)
+    x = torch.zeros((5, 128), device=DEV)
+    out = be.aggr_forward_history(x, ptr, idx, none(), none(), 0, 0)
+    assert out.shape == (0, 128)
+    # rows without any edge
+    ptr = torch.zeros(9, dtype=torch.int64, device=DEV)
+    out = be.aggr_forward_history(x, ptr, idx, none(), none(), 0, 8)
+    assert out.shape == (8, 128) and (out == 0).all()
+    out.sum().backward()
+
+
+def test_shim_rejects_bad_arguments(be):
+    x = torch.zeros((4, 128), device=DEV)
+    ptr = torch.zeros(5, dtype=torch.int64, device=DEV)
+    idx = torch.zeros(0, dtype=torch.int64, device=DEV)
+    with pytest.raises(ValueError):
+        be.aggr_forward_history(x, ptr.int(), idx, none(), none(), 0, 4)        # wrong index dtype
+    with pytest.raises(ValueError):
+        be.aggr_forward_history(x, ptr, idx, none(), none(), 0, 9)              # more rows than ptr has
+    with pytest.raises(ValueError):
+        be.aggr_forward_history(x.double(), ptr, idx, none(), none(), 0, 4)     # unsupported dtype
+    with pytest.raises(ValueError):
+        be.aggr_forward_history(x.t(), ptr, idx, none(), none(), 0, 4)          # not contiguous
+    with pytest.raises(ValueError):
+        be.aggr_forward_history(x, ptr, idx, torch.full((2,), -1, device=DEV), x, 128, 4)  # short map
