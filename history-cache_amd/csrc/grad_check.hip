@@ -58,7 +58,7 @@ __device__ __forceinline__ float row_partial_generic(const float *__restrict__ r
 
 __device__ __forceinline__ float finish_score(float partial, int norm_kind) {
   const float tot = hc_wave_sum_butterfly(partial);
-  return norm_kind == HC_NORM_L2 ? __fsqrt_rn(tot) : tot;
+  return norm_kind == HC_NORM_L2 ? sqrtf(tot) : tot;  // correctly rounded (-fhip-fp32-correctly-rounded-divide-sqrt)
 }
 
 // Scores of the GC_ROWS_PER_WAVE rows owned by this wave; lane i ends up holding row i's score.
