@@ -1,0 +1,290 @@
+#!/usr/bin/env python3
+"""Benchmark of the HisCache hot path on one MI355X.
+
+Default workload ("c2", the aggregation microbenchmark the metric is quoted on):
+  CSR block with 1M destination rows and 20M edges (Zipf alpha=2.1 degrees, max 5000), source ids
+  uniform over 10M nodes, 40% of which hit a 10M x 256 fp32 history table (the rest read a
+  10M x 256 fp32 feature matrix); mean aggregation forward, then backward with upstream ~N(0,1).
+A step = forward + transposed-view build + backward over that block, inputs resident in HBM.
+
+Prints ONE JSON line: edges/s over the whole step, the roofline of the dominant kernel (the forward
+gather, timed with HIP events on the launch stream) and a CPU baseline (the same semantics written
+with PyTorch CPU index_add, timed on this machine's host cores on a 1/10-size sample).
+
+Other workloads (--workload c4 | c2row | c3) print their own line and are not the headline.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "history-cache_amd"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c4", "c3"])
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+def sync():
+    import torch
+    torch.cuda.synchronize()
+
+
+def timed_steps(step, steps, warmup):
+    """W untimed steps, then exactly K steps between two synchronisations."""
+    for _ in range(warmup):
+        step()
+    sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    sync()
+    return (time.perf_counter() - t0) / steps
+
+
+class KernelClock:
+    """HIP-event timing of one launch site on the current stream, accumulated over the timed region."""
+
+    def __init__(self):
+        self.pairs = []
+
+    def __call__(self, fn):
+        import torch
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        out = fn()
+        b.record()
+        self.pairs.append((a, b))
+        return out
+
+    def reset(self):
+        self.pairs = []
+
+    def mean_ms(self):
+        return sum(a.elapsed_time(b) for a, b in self.pairs) / max(1, len(self.pairs))
+
+
+# ----------------------------------------------------------------------------------------- C2
+def c2_bytes_fwd(R, E, F, s_row=4, mode="src"):
+    # (R+1) ptr + E idx + E map lookups + E rows + R output rows  (int64 indices, fp32 data)
+    return (R + 1) * 8 + 2 * E * 8 + E * F * s_row + R * F * 4
+
+
+def c2_bytes_bwd(R, E, F, n_src):
+    # E g-rows + E transposed-edge ids + (n_src+1) ptrT + R degrees + n_src output rows
+    return E * F * 4 + E * 8 + (n_src + 1) * 8 + R * 4 + n_src * F * 4
+
+
+def run_c2(args, row_mode=False):
+    import torch
+
+    import hiscache_backend as be
+    from hiscache.synthetic import power_law_block
+
+    dev = "cuda:0"
+    s = args.scale
+    R, E, N, F = int(1_000_000 * s), int(20_000_000 * s), int(10_000_000 * s), 256
+    ptr, idx = power_law_block(R, E, N, alpha=2.1, max_degree=5000, seed=2)
+    ptr, idx = ptr.to(dev), idx.to(dev)
+    gen = torch.Generator(device=dev).manual_seed(2)
+    feat = torch.randn(N, F, device=dev, generator=gen)
+    g = torch.randn(R, F, device=dev, generator=gen)
+    if row_mode:
+        # reference-exact substitution: 40% of the destination rows carry a cached embedding
+        hbuf = 0.5 * torch.randn(R, F, device=dev, generator=gen)
+        hmap = torch.where(torch.rand(R, device=dev, generator=gen) < 0.4,
+                           torch.arange(R, device=dev), torch.full((R,), -1, device=dev))
+    else:
+        hist = 0.5 * torch.randn(N, F, device=dev, generator=gen)
+        hmap = torch.where(torch.rand(N, device=dev, generator=gen) < 0.4,
+                           torch.arange(N, device=dev), torch.full((N,), -1, device=dev))
+    feat.requires_grad_(True)
+    clk_f, clk_t, clk_b = KernelClock(), KernelClock(), KernelClock()
+
+    def step():
+        # the same three launches the autograd Function issues, with a clock on each
+        if row_mode:
+            out = clk_f(lambda: be._aggr_fwd(be.SUBST_ROW, ptr, idx, feat.detach(), hmap, hbuf, F, None, R))
+            tr = clk_t(lambda: be.build_transpose(ptr, idx, hmap, R, N))
+            clk_b(lambda: be._aggr_bwd(ptr, idx, tr, g, hmap, None, feat, False, tuple(hbuf.shape), F, R, N))
+        else:
+            out = clk_f(lambda: be._aggr_fwd(be.SUBST_SRC, ptr, idx, feat.detach(), hmap, hist, F, None, R))
+            tr = clk_t(lambda: be.build_transpose(ptr, idx, None, R, N))
+            clk_b(lambda: be._aggr_bwd(ptr, idx, tr, g, None, None, feat, False, None, 0, R, N))
+        return out
+
+    for _ in range(args.warmup):
+        step()
+    sync()
+    for c in (clk_f, clk_t, clk_b):
+        c.reset()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    sync()
+    sec = (time.perf_counter() - t0) / args.steps
+
+    # autograd round trip once, to show the user-level path runs the same kernels
+    if row_mode:
+        out = be.aggr_forward_history(feat, ptr, idx, hmap, hbuf, F, R)
+    else:
+        out = be.aggr_forward_source_history(feat, ptr, idx, hmap, hist)
+    out.backward(g)
+    sync()
+    feat.grad = None
+
+    t_f, t_t, t_b = clk_f.mean_ms(), clk_t.mean_ms(), clk_b.mean_ms()
+    if row_mode:
+        n_hist = int((hmap != -1).sum())
+        deg = (ptr[1:] - ptr[:-1])
+        e_nh = int(deg[hmap == -1].sum())
+        bytes_f = (R + 1) * 8 + R * 8 + e_nh * 8 + e_nh * F * 4 + n_hist * F * 4 + R * F * 4
+        bytes_b = e_nh * F * 4 + e_nh * 8 + (N + 1) * 8 + R * 4 + N * F * 4 + 2 * n_hist * F * 4
+    else:
+        bytes_f = c2_bytes_fwd(R, E, F)
+        bytes_b = c2_bytes_bwd(R, E, F, N)
+    res = {
+        "metric": "aggregated edges/sec (fwd+bwd)",
+        "value": E / sec,
+        "unit": "edges/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": ("c2row" if row_mode else "c2") +
+                   ": history_aggr microbench, R=%d rows, E=%d edges (Zipf 2.1, max deg 5000), %d sources x %d fp32, "
+                   "40%% history hits (%s substitution), mean fwd + transpose build + bwd"
+                   % (R, E, N, F, "per-row" if row_mode else "per-source")},
+        "roofline": {"bound": "hbm", "kernel": "fwd_mean_fast<float,4,1>", "achieved": bytes_f / (t_f * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_f / (t_f * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes": bytes_f, "launch_ms": t_f},
+        "kernels": {
+            "fwd_ms": t_f, "fwd_GBps": bytes_f / t_f / 1e6, "fwd_edges_per_s": E / (t_f * 1e-3),
+            "transpose_ms": t_t,
+            "bwd_ms": t_b, "bwd_GBps": bytes_b / t_b / 1e6, "bwd_edges_per_s": E / (t_b * 1e-3),
+            "fwd_plus_bwd_edges_per_s": E / ((t_f + t_b) * 1e-3),
+            "fwd_plus_bwd_GBps": (bytes_f + bytes_b) / (t_f + t_b) / 1e6,
+        },
+    }
+    return res, dict(R=R, E=E, N=N, F=F)
+
+
+def cpu_baseline_c2(shape):
+    """The same semantics with PyTorch CPU operators (index_add), on a 1/10-size sample."""
+    import torch
+
+    from hiscache.synthetic import power_law_block
+    from oracle import torch_cpu_path as tp
+
+    R, E, N, F = shape["R"] // 10, shape["E"] // 10, shape["N"] // 10, shape["F"]
+    torch.set_num_threads(os.cpu_count())
+    ptr, idx = power_law_block(R, E, N, alpha=2.1, max_degree=5000, seed=2)
+    gen = torch.Generator().manual_seed(2)
+    feat = torch.randn(N, F, generator=gen)
+    hist = 0.5 * torch.randn(N, F, generator=gen)
+    hmap = torch.where(torch.rand(N, generator=gen) < 0.4, torch.arange(N), torch.full((N,), -1))
+    g = torch.randn(R, F, generator=gen)
+
+    def one():
+        tp.aggr_fwd_src(feat, hist, hmap, ptr, idx, R)
+        tp.aggr_bwd_row(g, ptr, idx, None, N, R)
+
+    one()
+    times = []
+    t_end = time.perf_counter() + 20.0
+    while len(times) < 5 and (len(times) < 2 or time.perf_counter() < t_end):
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": E / med, "unit": "edges/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "1/10-size c2 block (R=%d, E=%d, %d sources x %d fp32), fwd+bwd with torch CPU index_add, "
+                      "median of %d runs" % (R, E, N, F, len(times))}
+
+
+# ----------------------------------------------------------------------------------------- C4
+def run_c4(args):
+    import torch
+
+    import hiscache_backend as be
+    from hiscache.synthetic import lognormal_grads
+
+    dev = "cuda:0"
+    s = args.scale
+    M, F, cap = int(2_000_000 * s), 256, int(50_000_000 * s)
+    gen = torch.Generator(device=dev).manual_seed(4)
+    grad = lognormal_grads(M, F, -3.0, 1.5, device=dev, generator=gen)
+    emb = torch.randn(M, F, device=dev, generator=gen)
+    age = torch.randint(0, 21, (M,), device=dev, generator=gen, dtype=torch.int32)
+    Nfull = max(4 * M, cap)
+    sub_to_full = torch.randperm(Nfull, device=dev, generator=gen)[:M].contiguous()
+    cached = torch.rand(M, device=dev, generator=gen) < 0.35
+    slot0 = torch.where(cached, torch.randperm(cap, device=dev, generator=gen)[:M], torch.full((M,), -1, device=dev))
+    table = torch.zeros(cap, F, dtype=torch.float16, device=dev)
+    full2slot = torch.full((Nfull,), -1, dtype=torch.int64, device=dev)
+    slot2full = torch.full((cap,), -1, dtype=torch.int64, device=dev)
+    checkin = torch.full((cap,), -1, dtype=torch.int64, device=dev)
+    header = torch.zeros(1, dtype=torch.int64, device=dev)
+    thres = torch.tensor([0.05], device=dev)
+    state = {"A": 0}
+
+    def step():
+        header.zero_()
+        mask, _ = be.grad_check(grad, emb, slot0, sub_to_full, thres, table, full2slot, slot2full, header, 1,
+                                age=age, age_limit=10, checkin=checkin)
+        state["mask"] = mask
+
+    sec = timed_steps(step, args.steps, args.warmup)
+    A = int(state["mask"].sum())
+    bytes_ = M * F * 4 + M * 13 + M + A * (F * 4 + F * 2 + 32)
+    return {
+        "metric": "grad_check admission rows/sec", "value": M / sec, "unit": "rows/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "c4: grad_check microbench, %d rows x %d fp32 grads (lognormal norms), ages in [0,20], "
+                               "thres 0.05, age limit 10, fp16 table %d x %d; admitted %d" % (M, F, cap, F, A)},
+        "roofline": {"bound": "hbm", "kernel": "gc_pass1+gc_pass2+gc_pass3_ring", "achieved": bytes_ / sec / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_ / sec / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes": bytes_},
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the reference's multi-GPU trainer "
+              "and comm.cu are out of scope); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    import hiscache_backend as be
+    be.load_library()
+    if args.workload in ("c2", "c2row"):
+        res, shape = run_c2(args, row_mode=(args.workload == "c2row"))
+        if not args.no_cpu_baseline:
+            torch.cuda.empty_cache()
+            res["cpu_baseline"] = cpu_baseline_c2(shape)
+    elif args.workload == "c4":
+        res = run_c4(args)
+    else:
+        raise SystemExit("workload c3 is not wired yet")
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

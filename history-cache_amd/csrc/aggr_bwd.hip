@@ -1,10 +1,10 @@
 // History-aware aggregation, backward, as a gather over the transposed view.
 //
-// One wavefront owns one SOURCE row s and sums, in ascending destination-row
-// order, g[r,:]/deg(r) (mean) or g[r,:]*edge_value[j] (weighted) over the
-// edges that point at s.  No float atomics: each output element has exactly
-// one writer and a fixed summation order, the same order a sequential walk of
-// the CSR block in row/edge order produces.
+// Every SOURCE row s is summed by exactly one wavefront, in ascending
+// destination-row order: g[r,:]/deg(r) (mean) or g[r,:]*edge_value[j]
+// (weighted) over the edges that point at s.  No float atomics: each output
+// element has one writer and a fixed summation order, the same order a
+// sequential walk of the CSR block in row/edge order produces.
 //
 // Semantics follow the reference kernels gen_bwd_history_grad_v2*
 // (/root/reference/src/cpp/src/history_aggr.cu:127-397): history rows route
@@ -17,14 +17,26 @@ namespace {
 
 // ---------------------------------------------------------------------------------------
 // Fast path: mean, fp32 upstream gradient, F == 64 * VEC * CHUNKS.
+//
+// A wave owns BWD_SRC_PER_WAVE consecutive source rows.  Their incoming edges are one
+// contiguous span of the transposed arrays, so the wave streams that span 64 edges at a time
+// (one coalesced load of destination rows, one gather of their degrees) and walks it with a
+// wave-uniform cursor: when the cursor passes the end of a source's segment the accumulator
+// is stored (zeros for sources without edges) and reset.  Up to UNROLL gradient rows are in
+// flight before the first add; adds stay in transposed-edge order.  Compared with one wave
+// per source this amortises the dependent loads (segment bounds -> rows -> degrees) over
+// many sources, which matters when most sources have only one or two incoming edges.
 // Blocks [0, src_blocks) own source rows; blocks beyond own rows of grad_hbuf.
 // ---------------------------------------------------------------------------------------
+constexpr int BWD_SRC_PER_WAVE = 32;
+
 template <int VEC, int CHUNKS, int UNROLL>
 __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ ptrT, const int32_t *__restrict__ rowT,
     const float *__restrict__ g, const int64_t *__restrict__ hmap, float *__restrict__ grad_vin,
     float *__restrict__ grad_hbuf, int64_t hsize, int64_t R, int64_t n_src, int64_t src_blocks) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
+  constexpr int S = BWD_SRC_PER_WAVE;
   const int lane = hc_lane();
   const int wave = hc_wave_in_block();
   if ((int64_t)blockIdx.x >= src_blocks) {
@@ -37,18 +49,26 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     for (int64_t c = lane; c < hsize; c += HC_WAVE) d[c] = (hit && c < F) ? s[c] : 0.0f;
     return;
   }
-  const int64_t src = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + wave;
-  if (src >= n_src) return;
-  const int64_t begin = ptrT[src];
-  const int64_t end = ptrT[src + 1];
+  const int64_t s0 = ((int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + wave) * S;
+  if (s0 >= n_src) return;
+  const int64_t rest = n_src - s0;
+  const int ns = rest < S ? (int)rest : S;
+  // lane l holds the segment bound ptrT[s0 + l], l = 0..ns
+  const int64_t my_p = ptrT[s0 + (lane < ns ? lane : ns)];
+  const int64_t e_begin = hc_readlane64(my_p, 0);
+  const int64_t e_end = hc_readlane64(my_p, ns);
+
   float acc[CHUNKS][VEC];
 #pragma unroll
   for (int k = 0; k < CHUNKS; ++k)
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
+  int cur = 0;                                   // source (relative to s0) being accumulated
+  int64_t cur_end = hc_readlane64(my_p, 1);      // end of its segment
+  float *__restrict__ obase = grad_vin + s0 * F + lane * VEC;
 
-  for (int64_t base = begin; base < end; base += HC_WAVE) {
-    const int64_t left = end - base;
+  for (int64_t base = e_begin; base < e_end; base += HC_WAVE) {
+    const int64_t left = e_end - base;
     const int n = left < HC_WAVE ? (int)left : HC_WAVE;
     int my_row = 0;
     float my_deg = 1.0f;
@@ -67,25 +87,39 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
           const float *p = g + (int64_t)r * F + lane * VEC;
 #pragma unroll
           for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
-        } else {
-          d[u] = 1.0f;
-#pragma unroll
-          for (int k = 0; k < CHUNKS; ++k)
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) v[u][k][i] = 0.0f;
         }
       }
 #pragma unroll
-      for (int u = 0; u < UNROLL; ++u)
+      for (int u = 0; u < UNROLL; ++u) {
+        if (j + u < n) {
+          const int64_t e = base + j + u;
+          while (e >= cur_end) {  // wave-uniform: close finished (possibly empty) segments
 #pragma unroll
-        for (int k = 0; k < CHUNKS; ++k)
+            for (int k = 0; k < CHUNKS; ++k) {
+              hc_vec<float, VEC>::store(obase + (int64_t)cur * F + k * HC_WAVE * VEC, acc[k]);
 #pragma unroll
-          for (int i = 0; i < VEC; ++i) acc[k][i] += v[u][k][i] / d[u];
+              for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
+            }
+            ++cur;
+            cur_end = hc_readlane64(my_p, cur + 1);
+          }
+#pragma unroll
+          for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[k][i] += v[u][k][i] / d[u];
+        }
+      }
     }
   }
-  float *__restrict__ o = grad_vin + src * F + lane * VEC;
+  // flush the open segment and the trailing sources without edges
+  for (; cur < ns; ++cur) {
 #pragma unroll
-  for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store(o + k * HC_WAVE * VEC, acc[k]);
+    for (int k = 0; k < CHUNKS; ++k) {
+      hc_vec<float, VEC>::store(obase + (int64_t)cur * F + k * HC_WAVE * VEC, acc[k]);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -221,7 +255,8 @@ int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, co
                 int64_t n_src, hipStream_t st) {
   constexpr int per = VEC * CHUNKS;
   constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
-  const int64_t sb = (n_src + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  const int64_t per_block = (int64_t)HC_WAVES_PER_BLOCK * BWD_SRC_PER_WAVE;
+  const int64_t sb = (n_src + per_block - 1) / per_block;
   const int64_t hb = (grad_hbuf && hmap) ? (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK : 0;
   if (sb + hb == 0) return HC_OK;
   if (!hc_grid_ok(sb + hb)) return HC_EUNSUPPORTED;
