@@ -31,7 +31,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c4", "c3"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c4", "c3", "copy"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
@@ -262,6 +262,18 @@ def run_c4(args):
     }
 
 
+def run_copy(args):
+    """Plain device copy of known size: the calibration point for the HBM traffic counters."""
+    import torch
+    n = 1 << 30  # 4 GiB of fp32 read, 4 GiB written
+    x = torch.ones(n, device="cuda:0")
+    y = torch.empty_like(x)
+    sec = timed_steps(lambda: y.copy_(x), args.steps, args.warmup)
+    return {"metric": "copy GB/s (read+write)", "value": 2 * n * 4 / sec / 1e9, "unit": "GB/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": True,
+            "config": {"workload": "copy: 4 GiB fp32 device-to-device copy (4 GiB read + 4 GiB written)"}}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -281,6 +293,8 @@ def main():
             res["cpu_baseline"] = cpu_baseline_c2(shape)
     elif args.workload == "c4":
         res = run_c4(args)
+    elif args.workload == "copy":
+        res = run_copy(args)
     else:
         raise SystemExit("workload c3 is not wired yet")
     print(json.dumps(res))

@@ -6,8 +6,10 @@
 // wave-uniform and the 64 lanes read one contiguous span of the row with
 // vector loads (16 bytes per lane when the row length allows).  Up to UNROLL
 // neighbour rows are in flight per wave before the first add; the adds run in
-// CSR order in fp32, so every output element is summed in exactly the order a
-// sequential CPU loop would use.
+// CSR order in fp32.  Rows of up to 256 edges are therefore summed in exactly
+// the order a sequential CPU loop would use; longer rows (fast path only) are
+// summed as four contiguous quarters combined left to right -- a fixed order,
+// so results stay bit-reproducible.
 //
 // Semantics follow the reference kernels gen_fwd_history_v2,
 // gen_fwd_history_v2_edge_value and gen_fwd_history_v2_edge_value_multi_head
@@ -16,6 +18,10 @@
 #include "hc_common.h"
 
 namespace {
+
+// Rows with more edges than this are summed by the four waves of their block (quarter split).
+// The CPU checker applies the same rule; the header documents it.
+constexpr int64_t HC_LONG_ROW_EDGES = 256;
 
 // Wave-cooperative copy of one row of a history buffer into an fp32 output row.
 template <typename TH>
@@ -51,33 +57,13 @@ __device__ __forceinline__ void copy_row_any(const void *hbuf, int hist_dtype, i
 // src_mode == 0: per-destination-row substitution (hbuf row-aligned, any dtype).
 // src_mode == 1: per-source substitution (hbuf is a table of the same dtype as vin).
 // ---------------------------------------------------------------------------------------
+// Sum of the neighbour rows of edges [begin, end), added to acc in edge order by the calling wave.
 template <typename T, int VEC, int CHUNKS, int UNROLL>
-__global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
-    const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const T *__restrict__ vin,
-    const int64_t *__restrict__ hmap, const void *__restrict__ hbuf, int hist_dtype, int64_t hsize,
-    int src_mode, float *__restrict__ vout, int64_t R) {
+__device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, const T *__restrict__ vin,
+                                               const int64_t *__restrict__ hmap, const T *__restrict__ htab,
+                                               int64_t hsize, int src_mode, int64_t begin, int64_t end,
+                                               int lane, float (&acc)[CHUNKS][VEC]) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
-  const int lane = hc_lane();
-  const int64_t row = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
-  if (row >= R) return;
-  float *__restrict__ orow = vout + row * F;
-
-  if (!src_mode && hmap != nullptr) {
-    if (hmap[row] != -1) {
-      copy_row_any(hbuf, hist_dtype, row * hsize, orow, F, lane);
-      return;
-    }
-  }
-
-  const int64_t begin = ptr[row];
-  const int64_t end = ptr[row + 1];
-  float acc[CHUNKS][VEC];
-#pragma unroll
-  for (int k = 0; k < CHUNKS; ++k)
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
-
-  const T *__restrict__ htab = static_cast<const T *>(hbuf);
   for (int64_t base = begin; base < end; base += HC_WAVE) {
     const int64_t left = end - base;
     const int n = left < HC_WAVE ? (int)left : HC_WAVE;
@@ -115,15 +101,113 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
           for (int i = 0; i < VEC; ++i) acc[k][i] += v[u][k][i];
     }
   }
+}
 
-  const int64_t deg = end - begin;
-  const float fdeg = (float)(int)deg;
+// A block owns four consecutive destination rows, one per wave.  Rows of up to `long_thres`
+// edges are summed by their wave, in CSR order.  Longer rows are then summed by the whole block:
+// wave w takes the w-th contiguous quarter of the row's edges (quarter length ceil(deg/4)), sums
+// it in CSR order, and wave 0 combines the four partial sums left to right,
+// ((q0 + q1) + q2) + q3, before the division.  Without this a power-law block ends with a few
+// waves grinding through multi-thousand-edge rows at one wave's memory parallelism.
+// long_thres == 0 disables the split (every row is then summed strictly in CSR order).
+constexpr int FWD_ROWS_PER_BLOCK = HC_WAVES_PER_BLOCK;
+
+template <typename T, int VEC, int CHUNKS, int UNROLL>
+__global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
+    const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const T *__restrict__ vin,
+    const int64_t *__restrict__ hmap, const void *__restrict__ hbuf, int hist_dtype, int64_t hsize,
+    int src_mode, float *__restrict__ vout, int64_t R, int64_t long_thres) {
+  constexpr int F = HC_WAVE * VEC * CHUNKS;
+  __shared__ float part[HC_WAVES_PER_BLOCK - 1][F];
+  __shared__ int long_rows[FWD_ROWS_PER_BLOCK];
+  __shared__ int n_long_s;
+  const int lane = hc_lane();
+  const int wave = hc_wave_in_block();
+  const T *__restrict__ htab = static_cast<const T *>(hbuf);
+  const int64_t row0 = (int64_t)blockIdx.x * FWD_ROWS_PER_BLOCK;
+  const int64_t rest = R - row0;
+  const int nrows = rest < FWD_ROWS_PER_BLOCK ? (int)rest : FWD_ROWS_PER_BLOCK;
+
+  if (long_thres > 0) {
+    if (threadIdx.x == 0) n_long_s = 0;
+    __syncthreads();
+  }
+
+  float acc[CHUNKS][VEC];
+  const int k = wave;
+  if (k < nrows) {
+    const int64_t row = row0 + k;
+    float *__restrict__ orow = vout + row * F;
+    bool hist = false;
+    if (!src_mode && hmap != nullptr) hist = hmap[row] != -1;
+    if (hist) {
+      copy_row_any(hbuf, hist_dtype, row * hsize, orow, F, lane);
+    } else {
+      const int64_t begin = ptr[row];
+      const int64_t end = ptr[row + 1];
+      const int64_t deg = end - begin;
+      if (long_thres > 0 && deg > long_thres) {
+        if (lane == 0) long_rows[atomicAdd(&n_long_s, 1)] = k;
+      } else {
 #pragma unroll
-  for (int k = 0; k < CHUNKS; ++k) {
-    float o[VEC];
+        for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) o[i] = deg > 0 ? acc[k][i] / fdeg : 0.0f;
-    hc_store_f32<VEC>(orow + k * HC_WAVE * VEC + lane * VEC, o);
+          for (int i = 0; i < VEC; ++i) acc[c][i] = 0.0f;
+        fwd_accumulate<T, VEC, CHUNKS, UNROLL>(idx, vin, hmap, htab, hsize, src_mode, begin, end, lane, acc);
+        const float fdeg = (float)(int)deg;
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) {
+          float o[VEC];
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) o[i] = deg > 0 ? acc[c][i] / fdeg : 0.0f;
+          hc_store_f32<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
+        }
+      }
+    }
+  }
+  if (long_thres <= 0) return;  // kernel argument: the whole grid takes the same branch
+  __syncthreads();
+  const int n_long = n_long_s;
+  // The order in which long rows were noted does not matter: each is summed on its own.
+  for (int t = 0; t < n_long; ++t) {
+    const int64_t lrow = row0 + long_rows[t];
+    const int64_t lb = ptr[lrow];
+    const int64_t le = ptr[lrow + 1];
+    const int64_t deg = le - lb;
+    const int64_t q = (deg + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+    int64_t sb = lb + wave * q;
+    int64_t se = sb + q;
+    if (sb > le) sb = le;
+    if (se > le) se = le;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) acc[c][i] = 0.0f;
+    fwd_accumulate<T, VEC, CHUNKS, UNROLL>(idx, vin, hmap, htab, hsize, src_mode, sb, se, lane, acc);
+    if (wave > 0) {
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) part[wave - 1][(c * HC_WAVE + lane) * VEC + i] = acc[c][i];
+    }
+    __syncthreads();
+    if (wave == 0) {
+      const float fdeg = (float)(int)deg;
+      float *__restrict__ orow = vout + lrow * F;
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c) {
+        float o[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          float t2 = acc[c][i];
+#pragma unroll
+          for (int pw = 0; pw < HC_WAVES_PER_BLOCK - 1; ++pw) t2 += part[pw][(c * HC_WAVE + lane) * VEC + i];
+          o[i] = t2 / fdeg;
+        }
+        hc_store_f32<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -204,10 +288,11 @@ int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const i
                 hipStream_t st) {
   constexpr int per = VEC * CHUNKS;
   constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
-  const int64_t blocks = (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  const int64_t blocks = (R + FWD_ROWS_PER_BLOCK - 1) / FWD_ROWS_PER_BLOCK;
   if (!hc_grid_ok(blocks)) return HC_EUNSUPPORTED;
   fwd_mean_fast<T, VEC, CHUNKS, UNROLL><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(
-      ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, vout, R);
+      ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, vout, R,
+      (int64_t)HC_LONG_ROW_EDGES);
   return hc_launch_status();
 }
 
@@ -250,6 +335,25 @@ int launch_generic(const int64_t *ptr, const int64_t *idx, const void *vin, cons
 }
 
 }  // namespace
+
+namespace {
+bool fast_shape(int64_t F, int in_dtype) {
+  if (F <= 0 || F % 64 != 0) return false;
+  const int vmax = in_dtype == HC_F32 ? 4 : 8;
+  for (int v = vmax; v >= 1; v /= 2) {
+    if (F % (64 * v) != 0) continue;
+    const int64_t c = F / (64 * v);
+    if (v == vmax) return c >= 1 && c <= 4;
+    return c == 1 || c == 3;
+  }
+  return false;
+}
+}  // namespace
+
+extern "C" int64_t hc_aggr_fwd_long_row_edges(int64_t F, int in_dtype) {
+  if (in_dtype < HC_F32 || in_dtype > HC_BF16) return 0;
+  return fast_shape(F, in_dtype) ? HC_LONG_ROW_EDGES : 0;
+}
 
 extern "C" int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, const void *vin,
                            int in_dtype, const int64_t *hmap, const void *hbuf, int hist_dtype,

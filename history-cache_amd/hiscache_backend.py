@@ -42,6 +42,7 @@ _SIGNATURES = {
     "hc_device_count": (_c_int, []),
     "hc_aggr_fwd": (_c_int, [_c_int, _c_p, _c_p, _c_p, _c_int, _c_p, _c_p, _c_int, _c_i64, _c_p, _c_i64,
                              _c_p, _c_i64, _c_i64, _c_i64, _c_p]),
+    "hc_aggr_fwd_long_row_edges": (_c_i64, [_c_i64, _c_int]),
     "hc_transpose_workspace_bytes": (_c_sz, [_c_i64, _c_i64, _c_i64]),
     "hc_build_transpose": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p,
                                     _c_sz, _c_p]),
@@ -515,6 +516,11 @@ def lookup(map_tensor, ids, offset=0):
                        _stream())
     _check(rc, "hc_lookup")
     return out
+
+
+def long_row_edges(feature_width, dtype=torch.float32):
+    """Rows with more edges than this are summed as four quarters by the mean forward (0: never)."""
+    return int(load_library().hc_aggr_fwd_long_row_edges(int(feature_width), _DTYPES[dtype]))
 
 
 def version():

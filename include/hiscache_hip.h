@@ -72,13 +72,23 @@ int hc_device_count(void);
  *       hbuf[hmap[idx[j]], :F] when hmap[idx[j]] != -1, else from vin.
  *
  * ptr[R+1], idx[>= ptr[R]], vin[n_src, n_head, F] (in_dtype), hmap NULL = no
- * history, hbuf (hist_dtype), vout[R, n_head, F] fp32.  Sums run in CSR order
- * in fp32, so results are bit-reproducible.  n_head >= 1; n_head > 1 requires
- * edge_value. */
+ * history, hbuf (hist_dtype), vout[R, n_head, F] fp32.  n_head >= 1; n_head > 1
+ * requires edge_value.
+ * Summation order (fp32, fixed, so results are bit-reproducible): a row is
+ * summed in CSR order; when hc_aggr_fwd_long_row_edges() reports a threshold
+ * T > 0 for the shape, a row with more than T edges is summed as four
+ * contiguous quarters of ceil(deg/4) edges, each in CSR order, combined left to
+ * right ((q0+q1)+q2)+q3, then divided. */
 int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, const void *vin, int in_dtype,
                 const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize,
                 const float *edge_value, int64_t n_head, float *vout, int64_t R, int64_t F,
                 int64_t n_src, void *stream);
+
+/* The long-row threshold T that hc_aggr_fwd applies to a mean aggregation with
+ * rows of F elements of in_dtype; 0 when every row is summed strictly in CSR
+ * order.  No reference counterpart (the reference sums every row with one
+ * warp per 32 columns, history_aggr.cu:27-37). */
+int64_t hc_aggr_fwd_long_row_edges(int64_t F, int in_dtype);
 
 /* ---------------------------------------------------------------- transpose (CSC view)
  * No reference counterpart: the reference backward scatters with float

@@ -94,9 +94,22 @@ float orc_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
  *   else            -> vout[row,:] = (sum_j vin[idx[j],:]) / deg   (:27-39)
  *   deg == 0        -> row is left as the caller's zero fill (:38, :425)
  * hmap may be NULL (no history at all). */
+static void sum_rows_seq(const Index *idx, const float *vin, Index F, Index b, Index e, float *o) {
+  for (Index j = b; j < e; ++j) {
+    const float *x = vin + idx[j] * F;
+    for (Index c = 0; c < F; ++c) o[c] += x[c];
+  }
+}
+
+/* split_above == 0: every row is summed strictly in CSR order (the order a sequential reader of
+ * the reference kernel produces).  split_above > 0 restates the device library's documented order
+ * for long rows: a row with more than split_above edges is summed as four contiguous quarters of
+ * ceil(deg/4) edges, each in CSR order, combined left to right ((q0+q1)+q2)+q3. */
 int orc_fwd_mean_row(const Index *ptr, const Index *idx, const float *vin,
                      const Index *hmap, const float *hbuf, float *vout,
-                     Index R, Index F, Index hsize) {
+                     Index R, Index F, Index hsize, Index split_above) {
+  float *part = (float *)malloc((size_t)F * sizeof(float));
+  if (!part) return ORC_EINVAL;
   for (Index row = 0; row < R; ++row) {
     float *o = vout + row * F;
     memset(o, 0, (size_t)F * sizeof(float));
@@ -107,12 +120,26 @@ int orc_fwd_mean_row(const Index *ptr, const Index *idx, const float *vin,
     Index b = ptr[row], e = ptr[row + 1];
     int n = (int)(e - b);
     if (n == 0) continue;
-    for (Index j = b; j < e; ++j) {
-      const float *x = vin + idx[j] * F;
-      for (Index c = 0; c < F; ++c) o[c] += x[c];
+    if (split_above > 0 && n > split_above) {
+      Index q = (n + 3) / 4;
+      for (int w = 0; w < 4; ++w) {
+        Index sb = b + w * q, se = sb + q;
+        if (sb > e) sb = e;
+        if (se > e) se = e;
+        if (w == 0) {
+          sum_rows_seq(idx, vin, F, sb, se, o);
+        } else {
+          memset(part, 0, (size_t)F * sizeof(float));
+          sum_rows_seq(idx, vin, F, sb, se, part);
+          for (Index c = 0; c < F; ++c) o[c] += part[c];
+        }
+      }
+    } else {
+      sum_rows_seq(idx, vin, F, b, e, o);
     }
     for (Index c = 0; c < F; ++c) o[c] = o[c] / (float)n;
   }
+  free(part);
   return ORC_OK;
 }
 
@@ -171,22 +198,46 @@ int orc_fwd_edge_value_multi_head(const Index *ptr, const Index *idx,
 /* Mean aggregation with per-SOURCE substitution (build extension, not in the
  * reference): x_j = hmap[idx[j]] != -1 ? hist[hmap[idx[j]], :F] : feat[idx[j], :F].
  * With an all -1 map it is orc_fwd_mean_row without history. */
+static void sum_rows_src(const Index *idx, const float *feat, const Index *hmap_src, const float *hist,
+                         Index F, Index hsize, Index b, Index e, float *o) {
+  for (Index j = b; j < e; ++j) {
+    Index s = idx[j];
+    const float *x = (hmap_src && hmap_src[s] != -1) ? hist + hmap_src[s] * hsize : feat + s * F;
+    for (Index c = 0; c < F; ++c) o[c] += x[c];
+  }
+}
+
 int orc_fwd_mean_src(const Index *ptr, const Index *idx, const float *feat,
                      const Index *hmap_src, const float *hist, float *vout,
-                     Index R, Index F, Index hsize) {
+                     Index R, Index F, Index hsize, Index split_above) {
+  float *part = (float *)malloc((size_t)F * sizeof(float));
+  if (!part) return ORC_EINVAL;
   for (Index row = 0; row < R; ++row) {
     float *o = vout + row * F;
     memset(o, 0, (size_t)F * sizeof(float));
     Index b = ptr[row], e = ptr[row + 1];
     int n = (int)(e - b);
     if (n == 0) continue;
-    for (Index j = b; j < e; ++j) {
-      Index s = idx[j];
-      const float *x = (hmap_src && hmap_src[s] != -1) ? hist + hmap_src[s] * hsize : feat + s * F;
-      for (Index c = 0; c < F; ++c) o[c] += x[c];
+    if (split_above > 0 && n > split_above) {   /* same quarter rule as orc_fwd_mean_row */
+      Index q = (n + 3) / 4;
+      for (int w = 0; w < 4; ++w) {
+        Index sb = b + w * q, se = sb + q;
+        if (sb > e) sb = e;
+        if (se > e) se = e;
+        if (w == 0) {
+          sum_rows_src(idx, feat, hmap_src, hist, F, hsize, sb, se, o);
+        } else {
+          memset(part, 0, (size_t)F * sizeof(float));
+          sum_rows_src(idx, feat, hmap_src, hist, F, hsize, sb, se, part);
+          for (Index c = 0; c < F; ++c) o[c] += part[c];
+        }
+      }
+    } else {
+      sum_rows_src(idx, feat, hmap_src, hist, F, hsize, b, e, o);
     }
     for (Index c = 0; c < F; ++c) o[c] = o[c] / (float)n;
   }
+  free(part);
   return ORC_OK;
 }
 

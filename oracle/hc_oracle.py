@@ -75,7 +75,7 @@ def _check(rc, name):
 
 
 # --------------------------------------------------------------------------- aggregation
-def fwd_mean_row(ptr, idx, vin, hmap, hbuf, num_node=None):
+def fwd_mean_row(ptr, idx, vin, hmap, hbuf, num_node=None, split_above=0):
     ptr, idx, vin = _i64(ptr), _i64(idx), _f32(vin)
     R = len(ptr) - 1 if not num_node else int(num_node)
     F = vin.shape[-1]
@@ -85,7 +85,7 @@ def fwd_mean_row(ptr, idx, vin, hmap, hbuf, num_node=None):
         hsize = hbuf.shape[-1] if hbuf.ndim == 2 else F
     out = np.zeros((R, F), np.float32)
     _check(lib().orc_fwd_mean_row(_p(ptr), _p(idx), _p(vin), _p(hmap), _p(hbuf), _p(out),
-                                  _I(R), _I(F), _I(hsize)), "fwd_mean_row")
+                                  _I(R), _I(F), _I(hsize), _I(split_above)), "fwd_mean_row")
     return out
 
 
@@ -114,7 +114,7 @@ def fwd_edge_value(ptr, idx, ev, vin, hmap, hbuf, num_node=None):
     return out
 
 
-def fwd_mean_src(ptr, idx, feat, hmap_src, hist, num_node=None):
+def fwd_mean_src(ptr, idx, feat, hmap_src, hist, num_node=None, split_above=0):
     ptr, idx, feat = _i64(ptr), _i64(idx), _f32(feat)
     R = len(ptr) - 1 if not num_node else int(num_node)
     F = feat.shape[-1]
@@ -124,7 +124,7 @@ def fwd_mean_src(ptr, idx, feat, hmap_src, hist, num_node=None):
         hsize = hist.shape[-1]
     out = np.zeros((R, F), np.float32)
     _check(lib().orc_fwd_mean_src(_p(ptr), _p(idx), _p(feat), _p(hmap_src), _p(hist), _p(out),
-                                  _I(R), _I(F), _I(hsize)), "fwd_mean_src")
+                                  _I(R), _I(F), _I(hsize), _I(split_above)), "fwd_mean_src")
     return out
 
 

@@ -59,11 +59,46 @@ def test_fwd_mean_row_mode(be, orc, R, N, F, maxdeg, hub, dtype, with_hist):
         hmap = random_hmap(rng, R, 0.35)
         hbuf = T(rng.standard_normal((R, F)).astype(np.float32), dtype)
         out = be.aggr_forward_history(x, T(ptr), T(idx), T(hmap), hbuf, F, R)
-        ref = orc.fwd_mean_row(ptr, idx, x32, hmap, hbuf.float().cpu().numpy())
+        ref = orc.fwd_mean_row(ptr, idx, x32, hmap, hbuf.float().cpu().numpy(), split_above=be.long_row_edges(F, dtype))
     else:
         out = be.aggr_forward_history(x, T(ptr), T(idx), none(), none(), 0, R)
-        ref = orc.fwd_mean_row(ptr, idx, x32, None, None)
+        ref = orc.fwd_mean_row(ptr, idx, x32, None, None, split_above=be.long_row_edges(F, dtype))
     assert out.dtype == torch.float32 and out.requires_grad
+    np.testing.assert_array_equal(out.detach().cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("mode", ["plain", "row", "src"])
+def test_fwd_long_rows_started_first(be, orc, mode):
+    """Rows above the long-row threshold are summed as four quarters by their block: same bits as the
+    oracle applying the documented quarter rule, and within 1e-5 of the strictly sequential sum."""
+    rng = np.random.default_rng(42)
+    R, N, F = 9000, 3000, 128
+    ptr, idx = random_csr(rng, R, N, 6)
+    deg = np.diff(ptr)
+    for r in rng.choice(R, size=12, replace=False):           # a dozen long rows, one of them empty-adjacent
+        deg[r] = int(rng.integers(257, 900))
+    deg[R - 1] = 1500                                          # the very last row is long
+    ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    idx = rng.integers(0, N, size=int(ptr[-1]), dtype=np.int64)
+    x = rng.standard_normal((N, F)).astype(np.float32)
+    if mode == "plain":
+        out = be.aggr_forward_history(T(x), T(ptr), T(idx), none(), none(), 0, R)
+        ref = orc.fwd_mean_row(ptr, idx, x, None, None, split_above=be.long_row_edges(F))
+        seq = orc.fwd_mean_row(ptr, idx, x, None, None)
+        assert (ref != seq).any()                              # the two orders really differ in rounding
+        np.testing.assert_allclose(ref, seq, rtol=1e-5, atol=1e-6)
+    elif mode == "row":
+        hmap = random_hmap(rng, R, 0.4)
+        hmap[R - 1] = -1
+        hmap[np.flatnonzero(deg > 256)[:3]] = 7                # long rows that are history rows
+        hbuf = rng.standard_normal((R, F)).astype(np.float32)
+        out = be.aggr_forward_history(T(x), T(ptr), T(idx), T(hmap), T(hbuf), F, R)
+        ref = orc.fwd_mean_row(ptr, idx, x, hmap, hbuf, split_above=be.long_row_edges(F))
+    else:
+        hist = rng.standard_normal((500, F)).astype(np.float32)
+        hmap = np.where(rng.random(N) < 0.4, rng.integers(0, 500, size=N), -1).astype(np.int64)
+        out = be.aggr_forward_source_history(T(x), T(ptr), T(idx), T(hmap), T(hist))
+        ref = orc.fwd_mean_src(ptr, idx, x, hmap, hist, split_above=be.long_row_edges(F))
     np.testing.assert_array_equal(out.detach().cpu().numpy(), ref)
 
 
@@ -110,7 +145,8 @@ def test_fwd_src_mode(be, orc, F, dtype):
     hit = rng.random(N) < 0.4
     hmap[hit] = rng.integers(0, Hn, size=int(hit.sum()))
     out = be.aggr_forward_source_history(feat, T(ptr), T(idx), T(hmap), hist)
-    ref = orc.fwd_mean_src(ptr, idx, feat.float().cpu().numpy(), hmap, hist.float().cpu().numpy())
+    ref = orc.fwd_mean_src(ptr, idx, feat.float().cpu().numpy(), hmap, hist.float().cpu().numpy(),
+                           split_above=be.long_row_edges(F, dtype))
     np.testing.assert_array_equal(out.detach().cpu().numpy(), ref)
     # an all-miss map is the plain mean
     out2 = be.aggr_forward_source_history(feat, T(ptr), T(idx), T(np.full(N, -1, np.int64)), hist)

@@ -212,3 +212,37 @@ def test_build_transpose_is_stable_sort(orc):
     np.testing.assert_array_equal(edgeT, order)
     np.testing.assert_array_equal(rowT, dst[order])
     np.testing.assert_array_equal(ptrT, np.concatenate([[0], np.cumsum(np.bincount(idx[keep], minlength=N))]))
+
+
+def test_quarter_split_order(orc):
+    """split_above restates the device library's long-row order: four contiguous quarters summed
+    separately, combined left to right.  Written out independently with NumPy float32."""
+    rng = np.random.default_rng(11)
+    N, F = 50, 9
+    deg = np.array([3, 0, 23, 8, 41])
+    ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    idx = rng.integers(0, N, size=int(ptr[-1]), dtype=np.int64)
+    vin = rng.standard_normal((N, F)).astype(np.float32)
+    got = orc.fwd_mean_row(ptr, idx, vin, None, None, split_above=8)
+    seq = orc.fwd_mean_row(ptr, idx, vin, None, None)
+    for r, d in enumerate(deg):
+        nb = idx[ptr[r]:ptr[r + 1]]
+        if d <= 8:
+            np.testing.assert_array_equal(got[r], seq[r])
+            continue
+        q = -(-d // 4)
+        parts = []
+        for w in range(4):
+            acc = np.zeros(F, np.float32)
+            for j in nb[w * q:(w + 1) * q]:
+                acc = acc + vin[j]
+            parts.append(acc)
+        tot = ((parts[0] + parts[1]) + parts[2]) + parts[3]
+        np.testing.assert_array_equal(got[r], tot / np.float32(d))
+    np.testing.assert_allclose(got, seq, rtol=1e-5, atol=1e-6)
+    hist = rng.standard_normal((7, F)).astype(np.float32)
+    hm = np.where(rng.random(N) < 0.5, rng.integers(0, 7, size=N), -1).astype(np.int64)
+    sub = vin.copy()
+    sub[hm != -1] = hist[hm[hm != -1]]
+    np.testing.assert_array_equal(orc.fwd_mean_src(ptr, idx, vin, hm, hist, split_above=8),
+                                  orc.fwd_mean_row(ptr, idx, sub, None, None, split_above=8))
