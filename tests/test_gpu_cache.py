@@ -1,0 +1,293 @@
+"""GPU parity of the host-side cache policy (HistoryCache, HistoryTable, the SAGE wiring) against the
+torch-CPU restatement of the reference.  Index outputs, masks and cached-id sets bit-exact; embeddings
+and gradients of the full model within 1e-5 relative of the same model evaluated on the CPU."""
+import copy
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import layered_batch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def make_world(seed, N=3000, Fin=32, H=48, buffer_rows=400):
+    from hiscache import HistoryCache, PinnedFeatureStore, make_config
+    from oracle import host_model
+    rng = np.random.default_rng(seed)
+    feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32))
+    hot = rng.permutation(N).astype(np.int64)
+    lcm = np.lcm(Fin, H)
+    buffer_floats = int(buffer_rows * lcm)
+    cfg = make_config(Fin, 7, H, 3, method="grad", rate=0.6, staleness_thres=4, device=DEV)
+    store = PinnedFeatureStore(feats, device=DEV)
+    cache = HistoryCache(store, cfg, "history_uvm", total_num_node=N, buffer_bytes=buffer_floats * 4, hot_ids=hot)
+    st = host_model.new_cache_state(N, Fin, H, buffer_floats, hot, feats)
+    return rng, feats, cfg, cache, st
+
+
+def batch_pair(rng, N, n_seed, fanout):
+    from hiscache.synthetic import make_batch
+    b = layered_batch(rng, N, n_seed, fanout)
+    labels = rng.integers(0, 7, size=N)
+    gpu = make_batch(b, labels, DEV)
+    cpu = make_batch(b, labels, "cpu")
+    return gpu, cpu
+
+
+def assert_state_equal(cache, st):
+    np.testing.assert_array_equal(cache.full2embed.cpu().numpy(), st.full2embed.numpy())
+    np.testing.assert_array_equal(cache.embed2full.cpu().numpy(), st.embed2full.numpy())
+    np.testing.assert_array_equal(cache.feat2full.cpu().numpy(), st.feat2full.numpy())
+    assert cache.header == st.header
+
+
+def test_fill_matches_model():
+    rng, feats, cfg, cache, st = make_world(0)
+    assert_state_equal(cache, st)
+    n_feat = st.feat2full.numel()
+    live = st.feat2full >= 0
+    np.testing.assert_array_equal(cache.buffer.view(-1, st.Fin)[:n_feat][live.to(DEV)].cpu().numpy(),
+                                  st.buffer.view(-1, st.Fin)[:n_feat][live].numpy())
+
+
+def test_lookup_update_cycles_match_model():
+    """Several iterations of lookup_and_load -> (synthetic gradients) -> update_history, including a
+    staleness refresh, compared tensor by tensor with the CPU model."""
+    from oracle import hc_oracle as orc
+    from oracle import host_model
+    rng, feats, cfg, cache, st = make_world(1)
+    N, H = st.N, st.H
+    for it in range(1, 10):
+        gpu, cpu = batch_pair(rng, N, 40, [6, 4, 3])
+        cache.lookup_and_load(gpu, 3)
+        ref = host_model.lookup_and_load(st, cpu, 3, feats)
+        np.testing.assert_array_equal(cache.sub2embed.cpu().numpy(), ref.sub2embed.numpy())
+        np.testing.assert_array_equal(cache.sub2feat.cpu().numpy(), ref.sub2feat.numpy())
+        for a, b in zip(cache.used_masks, ref.used_masks):
+            np.testing.assert_array_equal(a.cpu().numpy(), b.numpy())
+        np.testing.assert_array_equal(cache.load_mask.cpu().numpy(), ref.load_mask.numpy())
+        np.testing.assert_array_equal(gpu.x.cpu().numpy(), ref.x.numpy())
+        np.testing.assert_array_equal(cache.cached_embedding.cpu().numpy(), ref.cached_embedding.numpy())
+        # produced embeddings and their gradients for the 1-hop nodes
+        n1 = int(cpu.num_node_in_layer[1])
+        emb = rng.standard_normal((n1, H)).astype(np.float32)
+        grad = (rng.standard_normal((n1, H)) * np.exp(rng.normal(-3, 1.5, size=(n1, 1)))).astype(np.float32)
+        pe = torch.from_numpy(emb).to(DEV).requires_grad_(True)
+        pe.grad = torch.from_numpy(grad).to(DEV)
+        cache.produced_embedding = pe
+        cache.update_history(gpu, it)
+        score = torch.from_numpy(orc.row_scores(grad))
+        mask, _ = host_model.update_history(st, cpu.sub_to_full, ref.sub2embed, torch.from_numpy(emb), score,
+                                            0.6, 4, it)
+        np.testing.assert_array_equal(cache.last_record_mask.cpu().numpy(), mask.numpy())
+        assert_state_equal(cache, st)
+        n_emb = st.header
+        np.testing.assert_array_equal(cache.buffer.view(-1, H)[:n_emb].cpu().numpy(),
+                                      st.buffer.view(-1, H)[:n_emb].numpy())
+        assert cache.produced_embedding is None and cache.overflow == 0
+    s = cache.stats()
+    assert s["embed_cached"] == int((st.full2embed[:N] != -1).sum())
+    assert s["feat_cached"] == int((st.full2embed[N:2 * N] != -1).sum())
+
+
+def test_update_history_overflow_is_counted():
+    from oracle import hc_oracle as orc
+    from oracle import host_model
+    rng, feats, cfg, cache, st = make_world(2, buffer_rows=2)       # room for very few embedding rows
+    N, H = st.N, st.H
+    cap = st.embed2full.numel()
+    gpu, cpu = batch_pair(rng, N, 60, [8, 4, 2])
+    cache.lookup_and_load(gpu, 3)
+    ref = host_model.lookup_and_load(st, cpu, 3, feats)
+    n1 = int(cpu.num_node_in_layer[1])
+    emb = rng.standard_normal((n1, H)).astype(np.float32)
+    grad = rng.standard_normal((n1, H)).astype(np.float32)
+    pe = torch.from_numpy(emb).to(DEV).requires_grad_(True)
+    pe.grad = torch.from_numpy(grad).to(DEV)
+    cache.produced_embedding = pe
+    cache.update_history(gpu, 1)
+    mask, _ = host_model.update_history(st, cpu.sub_to_full, ref.sub2embed, torch.from_numpy(emb),
+                                        torch.from_numpy(orc.row_scores(grad)), 0.6, 4, 1)
+    assert int(mask.sum()) > cap
+    assert cache.header == cap == st.header and cache.overflow == int(mask.sum()) - cap
+    assert_state_equal(cache, st)
+
+
+def test_feature_cache_only_and_no_cache_modes():
+    from hiscache import HistoryCache, PinnedFeatureStore, make_config
+    rng, feats, cfg, cache, st = make_world(3)
+    gpu, cpu = batch_pair(rng, st.N, 30, [5, 3, 2])
+    cache.lookup_and_load(gpu, 3, feature_cache_only=True)
+    np.testing.assert_array_equal(gpu.x.cpu().numpy(), feats[cpu.sub_to_full].numpy())
+    plain = HistoryCache(PinnedFeatureStore(feats, device=DEV), cfg, "uvm", total_num_node=st.N)
+    plain.lookup_and_load(gpu, 3)
+    np.testing.assert_array_equal(gpu.x.cpu().numpy(), feats[cpu.sub_to_full].numpy())
+    assert (plain.sub2embed == -1).all() and plain.cached_embedding.numel() == 0
+    plain.update_history(gpu, 1)            # a no-op without a history buffer
+
+
+class CpuSage(torch.nn.Module):
+    """The same network evaluated with dense CPU operators (mean aggregation by index_add)."""
+
+    def __init__(self, model):
+        super().__init__()
+        self.m = copy.deepcopy(model).cpu()
+
+    def forward(self, batch, x, sub2embed, cached_embedding):
+        from oracle import torch_cpu_path as tp
+        m = self.m
+        L = m.num_layers
+        his_out = None
+        for i, conv in enumerate(m.convs):
+            n = int(batch.num_node_in_layer[L - 1 - i])
+            if m.training and i == L - 2:
+                # differentiable statement of the history layer
+                agg = mean_rows(x, batch.ptr, batch.idx, n)
+                hit = (sub2embed != -1)[:, None]
+                agg = torch.where(hit, cached_embedding, agg)
+                agg.retain_grad()
+                his_out = agg
+            else:
+                agg = mean_rows(x, batch.ptr, batch.idx, n)
+            x = conv.lin_l(agg) + conv.lin_r(x[:n])
+            if i < L - 1:
+                x = m.bns[i](x)
+                x = torch.relu(x)
+        return x.log_softmax(dim=-1), his_out
+
+
+def mean_rows(x, ptr, idx, n):
+    deg = (ptr[1:n + 1] - ptr[:n])
+    dst = torch.repeat_interleave(torch.arange(n), deg)
+    out = torch.zeros(n, x.shape[1], dtype=x.dtype)
+    out = out.index_add(0, dst, x[idx[: int(ptr[n])]])
+    return out / deg.clamp(min=1).to(x.dtype)[:, None]
+
+
+def test_sage_training_iteration_matches_cpu():
+    """lookup_and_load -> HistorySAGE forward -> loss.backward -> update_history on the GPU, against the
+    same network on the CPU: logits, the gradient reaching the produced embedding, parameter gradients
+    (1e-5 relative, fp32) and the admitted id set (exact, thresholds kept away from knife edges)."""
+    from hiscache import get_model
+    from oracle import hc_oracle as orc
+    from oracle import host_model
+    torch.manual_seed(0)
+    rng, feats, cfg, cache, st = make_world(4, N=4000, Fin=64, H=128, buffer_rows=300)
+    N, H = st.N, st.H
+    model = get_model(cfg, cache).to(DEV)
+    model.train()
+    cpu_model = CpuSage(model)
+    cpu_model.m.train()
+    for it in range(1, 4):
+        gpu, cpu = batch_pair(rng, N, 50, [6, 4, 3])
+        cache.lookup_and_load(gpu, 3)
+        ref = host_model.lookup_and_load(st, cpu, 3, feats)
+        out = model(gpu)
+        loss = torch.nn.functional.nll_loss(out, gpu.y)
+        model.zero_grad()
+        loss.backward()
+        out_c, his_c = cpu_model(cpu, ref.x, ref.sub2embed, ref.cached_embedding)
+        loss_c = torch.nn.functional.nll_loss(out_c, cpu.y)
+        cpu_model.m.zero_grad()
+        loss_c.backward()
+        np.testing.assert_allclose(out.detach().cpu().numpy(), out_c.detach().numpy(), rtol=1e-4, atol=1e-5)
+        pe = cache.produced_embedding
+        assert pe is not None and pe.grad is not None
+        np.testing.assert_allclose(pe.detach().cpu().numpy(), his_c.detach().numpy(), rtol=1e-5, atol=1e-6)
+        scale = float(his_c.grad.abs().max())
+        np.testing.assert_allclose(pe.grad.cpu().numpy(), his_c.grad.numpy(), rtol=1e-3, atol=1e-5 * scale)
+        # biases in front of a batch norm have a mathematically zero gradient (pure rounding noise), so
+        # the absolute floor is taken from the largest parameter gradient of the network
+        gscale = max(float(q.grad.abs().max()) for q in cpu_model.m.parameters() if q.grad is not None)
+        for (n_, p), (_, q) in zip(model.named_parameters(), cpu_model.m.named_parameters()):
+            if p.grad is None:
+                continue
+            np.testing.assert_allclose(p.grad.cpu().numpy(), q.grad.numpy(), rtol=1e-3, atol=2e-5 * gscale,
+                                       err_msg=n_)
+        # admission on the GPU gradient itself, mirrored on the CPU model state
+        grad_gpu = pe.grad.cpu().numpy()
+        emb_gpu = pe.detach().cpu().numpy()
+        cache.update_history(gpu, it)
+        score = torch.from_numpy(orc.row_scores(grad_gpu))
+        mask, _ = host_model.update_history(st, cpu.sub_to_full, ref.sub2embed, torch.from_numpy(emb_gpu), score,
+                                            0.6, 4, it)
+        np.testing.assert_array_equal(cache.last_record_mask.cpu().numpy(), mask.numpy())
+        assert_state_equal(cache, st)
+    model.eval()
+    gpu, cpu = batch_pair(rng, N, 20, [4, 3, 2])
+    cache.lookup_and_load(gpu, 3, feature_cache_only=True)
+    with torch.no_grad():
+        ev = model(gpu)
+    assert ev.shape == (20, 7) and torch.isfinite(ev).all()
+
+
+def test_history_table_record_and_evict():
+    from hiscache import HistoryTable, make_config
+    from oracle import hc_oracle as orc
+    from oracle import host_model
+    rng = np.random.default_rng(5)
+    N, Fin, H = 2000, 16, 24
+    cfg = make_config(Fin, 5, H, 3, method="grad", rate=0.7, staleness_thres=3, device=DEV, model_type="SAGE",
+                      buffer_size=150)
+    table = HistoryTable(cfg, total_num_node=N)
+    assert table.num_layers == 2 and table.history_size_layered == [Fin, H]
+    ref = [dict(buf=np.zeros((150, w), np.float32), h2f=np.full(150, -1, np.int64), f2h=np.full(N, -1, np.int64),
+                checkin=np.full(150, -1, np.int64), header=np.zeros(1, np.int64)) for w in (Fin, H)]
+    for it in range(1, 7):
+        b = layered_batch(rng, N, 25, [5, 4, 3])
+        nnl = b["num_node_in_layer"]
+        from hiscache.synthetic import make_batch
+        batch = make_batch(b, rng.integers(0, 5, size=N), DEV)
+        batch.x = torch.zeros((int(nnl[-1]), Fin), device=DEV)
+        table.lookup(batch.sub_to_full, nnl)
+        used = orc.count_history_reconstruct(b["ptr"], b["idx"], None, int(nnl[-1]), 25, 3)
+        used_dev = [torch.from_numpy(u).to(DEV) for u in used]
+        table.history_out = []
+        outs = []
+        for layer_id, w in enumerate((Fin, H)):
+            n = int(nnl[3 - 1 - layer_id])
+            his = torch.from_numpy(rng.standard_normal((n, w)).astype(np.float32)).to(DEV).requires_grad_(True)
+            his.grad = torch.from_numpy((rng.standard_normal((n, w)) * np.exp(rng.normal(-3, 1, size=(n, 1)))
+                                         ).astype(np.float32)).to(DEV)
+            table.history_out.append(his)
+            outs.append(his)
+            s2h = table.sub_to_history[layer_id].cpu().numpy()
+            expect = ref[layer_id]["f2h"][b["sub_to_full"][:n]].copy()
+            expect[:25] = -1
+            np.testing.assert_array_equal(s2h, expect)
+            # compact ids and compact buffer
+            comp = table.sub_to_history_layered[layer_id].cpu().numpy()
+            hit = expect != -1
+            np.testing.assert_array_equal(comp[hit], np.arange(hit.sum()))
+            assert (comp[~hit] == -1).all()
+            np.testing.assert_array_equal(table.tmp_history_buffer_layered[layer_id].detach().cpu().numpy(),
+                                          ref[layer_id]["buf"][expect[hit]])
+        table.record_history(batch.sub_to_full, batch, it, used_dev)
+        for layer_id, w in enumerate((Fin, H)):
+            n = int(nnl[3 - 1 - layer_id])
+            r = ref[layer_id]
+            score = orc.row_scores(outs[layer_id].grad.cpu().numpy(), orc.NORM_L1)
+            thres = host_model.quantile_threshold(score, 0.7)
+            s2h = r["f2h"][b["sub_to_full"][:n]].copy()
+            s2h[:25] = -1
+            orc.record_history(outs[layer_id].detach().cpu().numpy(), r["buf"], used[layer_id + 1][:n],
+                               b["sub_to_full"], s2h, r["h2f"], r["f2h"], r["header"], score, thres, r["checkin"], it)
+            np.testing.assert_array_equal(table.history_to_full_layered[layer_id].cpu().numpy(), r["h2f"])
+            np.testing.assert_array_equal(table.full_to_history_layered[layer_id].cpu().numpy(), r["f2h"])
+            np.testing.assert_array_equal(table.checkin_iter[layer_id].cpu().numpy(), r["checkin"])
+            np.testing.assert_array_equal(table.cuda_header_layered[layer_id].cpu().numpy(), r["header"])
+            live = r["h2f"] != -1
+            np.testing.assert_array_equal(table.history_buffer_layered[layer_id].cpu().numpy()[live], r["buf"][live])
+        if it % 2 == 0:
+            table.evict_by_staleness(it, 3)
+            for layer_id in range(2):
+                r = ref[layer_id]
+                c, h, f = (torch.from_numpy(r[k]) for k in ("checkin", "h2f", "f2h"))
+                host_model.evict_by_staleness(c, h, f, it, 3)
+                np.testing.assert_array_equal(table.history_to_full_layered[layer_id].cpu().numpy(), r["h2f"])
+                np.testing.assert_array_equal(table.full_to_history_layered[layer_id].cpu().numpy(), r["f2h"])
+    assert sum(table.show()) > 0
