@@ -24,6 +24,9 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "history-cache_amd"))
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel at full size, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs of this file (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000: factors from a 4 GiB device copy).
+MEASURED_TRAFFIC = {"c2": 24.30e9, "c2row": 13.98e9, "c4": 3.50e9}
 
 
 def parse():
@@ -169,7 +172,8 @@ def run_c2(args, row_mode=False):
                    % (R, E, N, F, "per-row" if row_mode else "per-source")},
         "roofline": {"bound": "hbm", "kernel": "fwd_mean_fast<float,4,1>", "achieved": bytes_f / (t_f * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_f / (t_f * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": None, "algorithmic_bytes": bytes_f, "launch_ms": t_f},
+                     "traffic": MEASURED_TRAFFIC["c2row" if row_mode else "c2"] if s == 1.0 else None,
+                     "algorithmic_bytes": bytes_f, "launch_ms": t_f},
         "kernels": {
             "fwd_ms": t_f, "fwd_GBps": bytes_f / t_f / 1e6, "fwd_edges_per_s": E / (t_f * 1e-3),
             "transpose_ms": t_t,
@@ -258,7 +262,7 @@ def run_c4(args):
                                "thres 0.05, age limit 10, fp16 table %d x %d; admitted %d" % (M, F, cap, F, A)},
         "roofline": {"bound": "hbm", "kernel": "gc_pass1+gc_pass2+gc_pass3_ring", "achieved": bytes_ / sec / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_ / sec / 1e9 / HBM_PEAK_GBS,
-                     "traffic": None, "algorithmic_bytes": bytes_},
+                     "traffic": MEASURED_TRAFFIC["c4"] if s == 1.0 else None, "algorithmic_bytes": bytes_},
     }
 
 
