@@ -10,10 +10,11 @@ from .feature_store import PinnedFeatureStore
 from .history_cache import HistoryCache
 from .history_model import HistorySAGE, MySageConvHistory, get_model
 from .history_table import HistoryTable
+from .ring_cache import RingHistoryCache
 from .util import Config, make_config, quantile_threshold
 
 __all__ = [
-    "HistoryCache", "HistoryTable", "HistorySAGE", "MySageConvHistory", "get_model",
+    "HistoryCache", "HistoryTable", "RingHistoryCache", "HistorySAGE", "MySageConvHistory", "get_model",
     "PinnedFeatureStore", "Config", "make_config", "quantile_threshold",
     "count_history_reconstruct", "get_graph_structure_score", "record_history",
 ]

@@ -1,0 +1,123 @@
+"""RingHistoryCache: historical-embedding cache as one ring table in fp32 / fp16 / bf16 with the
+admission pass fused on the device.
+
+A build extension for the large synthetic configurations (a 111M x 256 fp16 table does not fit the
+reference's flat fp32 buffer design).  It plays the role of ``HistoryCache`` for the model
+(/root/reference/hiscache/history_model.py:123-134 reads ``sub2embed``, ``cached_embedding``,
+``method`` and sets ``produced_embedding``) and keeps its two entry points,
+``lookup_and_load(batch, num_layer)`` and ``update_history(batch, glb_iter)``.  The policy is the
+ring of ``HistoryTable`` (/root/reference/hiscache/history_table.py:127-200, kernel
+/root/reference/src/cpp/src/grad_check.cu:6-46): a row is admitted when its gradient norm is below
+the threshold and it is either not cached or its entry is at least ``age_limit`` iterations old;
+admitted rows overwrite the ring in row order.  Norms, test, mask, slot assignment, the
+fp32 -> table-dtype row copy and the map updates are one ``hiscache_backend.grad_check`` call.
+"""
+import torch
+
+import hiscache_backend as _be
+
+from .util import quantile_threshold
+
+
+class RingHistoryCache:
+
+    def __init__(self, uvm, total_num_node, in_channels, hidden_channels, capacity, num_layers,
+                 table_dtype=torch.float16, rate=0.5, thres=None, age_limit=1 << 30, method="grad",
+                 device="cuda:0"):
+        self.uvm = uvm
+        self.total_num_node = int(total_num_node)
+        self.in_channels = in_channels
+        self.hidden_channels = hidden_channels
+        self.num_layers_all = num_layers
+        self.device = torch.device(device)
+        self.method = method
+        self.rate = rate
+        self.age_limit = int(age_limit)
+        self.table = torch.zeros((capacity, hidden_channels), dtype=table_dtype, device=self.device)
+        self.full2slot = torch.full((self.total_num_node,), -1, dtype=torch.int64, device=self.device)
+        self.slot2full = torch.full((capacity,), -1, dtype=torch.int64, device=self.device)
+        self.checkin = torch.full((capacity,), -1, dtype=torch.int64, device=self.device)
+        self._header = torch.zeros(1, dtype=torch.int64, device=self.device)
+        # a fixed threshold (1-element tensor) skips the quantile; otherwise quantile(score, rate)
+        self.thres = None if thres is None else torch.tensor([float(thres)], dtype=torch.float32,
+                                                             device=self.device)
+        self.glb_iter = 0
+        self.produced_embedding = None
+        self.sub2embed = None
+        self.cached_embedding = None
+        self.used_masks = None
+        self.last_record_mask = None
+
+    @property
+    def header(self):
+        return int(self._header.item())
+
+    def lookup_and_load(self, batch, num_layer=None):
+        if num_layer is None:
+            num_layer = self.num_layers_all
+        sub_to_full = batch.sub_to_full
+        n1 = int(batch.num_node_in_layer[1])
+        self.sub2embed = _be.lookup(self.full2slot, sub_to_full[:n1], 0)
+        self.used_masks = _be.count_history_reconstruct(batch.ptr, batch.idx, self.sub2embed,
+                                                        sub_to_full.shape[0], batch.y.shape[0], num_layer)
+        self.glb_iter += 1
+        async_get = getattr(self.uvm, "masked_get_async", None)
+        if async_get is not None:
+            x, done = async_get(sub_to_full, self.used_masks[0])
+        else:
+            x, done = self.uvm.masked_get(sub_to_full, self.used_masks[0]), None
+        # rows without a slot (-1) read the last table row and are ignored by the aggregation
+        self.cached_embedding = _be.gather_rows(self.table, self.sub2embed)
+        if done is not None:
+            self.uvm.join(done)
+        batch.x = x
+        return None
+
+    @torch.no_grad()
+    def update_history(self, batch, glb_iter):
+        emb = self.produced_embedding
+        if emb is None:
+            raise AssertionError("produced embedding is None")
+        n1 = emb.shape[0]
+        slot = self.sub2embed
+        # age of the cached entry, in iterations (0 for rows without an entry)
+        age = (glb_iter - self.checkin[slot.clamp(min=0)]).to(torch.int32)
+        sub_to_full = batch.sub_to_full[:n1].contiguous()
+        if self.method == "grad" and emb.grad is not None:
+            grad = emb.grad.contiguous()
+            if self.thres is not None:
+                mask, score = _be.grad_check(grad, emb.detach().contiguous(), slot, sub_to_full, self.thres,
+                                             self.table, self.full2slot, self.slot2full, self._header, glb_iter,
+                                             age=age, age_limit=self.age_limit, checkin=self.checkin)
+            else:
+                score = _be.row_scores(grad)
+                thres = quantile_threshold(score, self.rate)
+                mask, _ = _be.grad_check(None, emb.detach().contiguous(), slot, sub_to_full, thres, self.table,
+                                         self.full2slot, self.slot2full, self._header, glb_iter, age=age,
+                                         age_limit=self.age_limit, checkin=self.checkin, score=score)
+        else:
+            score = torch.randn([n1], device=self.device)
+            thres = quantile_threshold(score, self.rate)
+            mask, _ = _be.grad_check(None, emb.detach().contiguous(), slot, sub_to_full, thres, self.table,
+                                     self.full2slot, self.slot2full, self._header, glb_iter, age=age,
+                                     age_limit=self.age_limit, checkin=self.checkin, score=score)
+        emb.grad = None
+        self.last_record_mask = mask
+        self.last_score = score
+        self.produced_embedding = None
+
+    def preload(self, node_ids, rows=None):
+        """Mark ``node_ids`` (unique int64 on the device) as cached in slots header.. (benchmark /
+        warm-start helper).  ``rows`` [len, hidden] fills the table rows, else they stay as they are."""
+        n = node_ids.numel()
+        h = self.header
+        cap = self.table.shape[0]
+        if h + n > cap:
+            raise ValueError("preload does not wrap the ring")
+        slots = torch.arange(h, h + n, device=self.device)
+        self.full2slot[node_ids] = slots
+        self.slot2full[h:h + n] = node_ids
+        self.checkin[h:h + n] = 0
+        if rows is not None:
+            self.table[h:h + n] = rows.to(self.table.dtype)
+        self._header.fill_((h + n) % cap)

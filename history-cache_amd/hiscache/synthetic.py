@@ -111,10 +111,12 @@ def make_batch(sample, labels, device):
     )
 
 
-def direct_power_law_batch(total_num_node, n_seed, fanout, alpha, seed, popularity_alpha=None):
+def direct_power_law_batch(total_num_node, n_seed, fanout, alpha, seed, popularity_alpha=None,
+                           degree_scale=1.0):
     """A sampled batch drawn directly (no full graph is materialised): every node reached at hop k
-    gets min(Zipf(alpha), fanout[k]) neighbours whose full ids are uniform (or Zipf-popular) over
-    ``total_num_node``.  For graphs too large to build on the host (hundreds of millions of nodes)."""
+    gets min(max(1, floor(Zipf(alpha) * degree_scale)), fanout[k]) neighbours whose full ids are
+    uniform (or Zipf-popular) over ``total_num_node``.  For graphs too large to build on the host
+    (hundreds of millions of nodes); ``degree_scale`` sets the mean degree of the underlying graph."""
     rng = np.random.default_rng(seed)
     seeds = rng.choice(total_num_node, size=n_seed, replace=False).astype(np.int64)
     sub_to_full = seeds.copy()
@@ -125,7 +127,8 @@ def direct_power_law_batch(total_num_node, n_seed, fanout, alpha, seed, populari
     n_edges = 0
     for f in fanout:
         n_front = hi - lo
-        deg = np.minimum(rng.zipf(alpha, size=n_front), f).astype(np.int64)
+        raw = np.minimum(rng.zipf(alpha, size=n_front), 1 << 20).astype(np.float64)
+        deg = np.minimum(np.maximum(1, np.floor(raw * degree_scale)), f).astype(np.int64)
         e = int(deg.sum())
         if popularity_alpha is None:
             nb_full = rng.integers(0, total_num_node, size=e, dtype=np.int64)
