@@ -244,15 +244,30 @@ class _AggrHistory(torch.autograd.Function):
         ev = ev if ctx.has_ev else None
         n_src = x.shape[0]
         row_map = hmap if mode == SUBST_ROW else None
-        tr = build_transpose(ptr, idx, row_map, R, n_src)
+        want_x = ctx.needs_input_grad[0]
         want_eg = ev is not None and ctx.needs_input_grad[3]
+        want_h = row_map is not None and ctx.needs_input_grad[5]
+        if not want_x and not want_eg:
+            # raw features at the input layer: nothing flows further back, so the transposed view
+            # and the gather are skipped; the history buffer's gradient is a masked copy of g
+            grad_h = None
+            if want_h:
+                g2 = g.contiguous()
+                if g2.dim() == 3 and hsize == g2.shape[-1]:
+                    g2 = g2.sum(1)
+                grad_h = torch.zeros(hshape, dtype=torch.float32, device=g.device)
+                flat = g2.reshape(R, -1)
+                hit = (row_map[:R] != -1).unsqueeze(1)
+                grad_h.view(-1, hsize)[:R, :flat.shape[1]] = torch.where(hit, flat, torch.zeros_like(flat))
+            return None, None, None, None, None, grad_h, None, None, None
+        tr = build_transpose(ptr, idx, row_map, R, n_src)
         grad_x, grad_h, edge_grad = _aggr_bwd(ptr, idx, tr, g, row_map, ev, x, want_eg, hshape, hsize, R,
                                               n_src)
         if grad_x.dtype != x.dtype:
             grad_x = grad_x.to(x.dtype)
-        if mode == SUBST_SRC:
+        if mode == SUBST_SRC or not want_h:
             grad_h = None
-        return grad_x, None, None, edge_grad, None, grad_h, None, None, None
+        return (grad_x if want_x else None), None, None, edge_grad, None, grad_h, None, None, None
 
 
 def _norm_history(history_map, history_buffer, history_size):

@@ -291,3 +291,75 @@ def test_history_table_record_and_evict():
                 np.testing.assert_array_equal(table.history_to_full_layered[layer_id].cpu().numpy(), r["h2f"])
                 np.testing.assert_array_equal(table.full_to_history_layered[layer_id].cpu().numpy(), r["f2h"])
     assert sum(table.show()) > 0
+
+
+def test_ring_cache_cycles_match_oracle():
+    """RingHistoryCache (fp16 ring table, fused admission with staleness ages, fixed threshold and
+    quantile threshold) against the CPU oracle's grad_check over several iterations."""
+    from hiscache import PinnedFeatureStore, RingHistoryCache
+    from oracle import hc_oracle as orc
+    from oracle import host_model
+    from hiscache.synthetic import make_batch
+    rng = np.random.default_rng(6)
+    N, Fin, H, cap = 3000, 32, 64, 500
+    feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32))
+    for fixed in (True, False):
+        cache = RingHistoryCache(PinnedFeatureStore(feats, device=DEV), N, Fin, H, capacity=cap, num_layers=3,
+                                 table_dtype=torch.float16, thres=0.05 if fixed else None, rate=0.6, age_limit=3,
+                                 device=DEV)
+        ref = dict(table=np.zeros((cap, H), np.uint16), f2s=np.full(N, -1, np.int64), s2f=np.full(cap, -1, np.int64),
+                   checkin=np.full(cap, -1, np.int64), header=np.zeros(1, np.int64))
+        for it in range(1, 9):
+            b = layered_batch(rng, N, 40, [6, 4, 3])
+            batch = make_batch(b, rng.integers(0, 5, size=N), DEV)
+            cache.lookup_and_load(batch, 3)
+            n1 = int(b["num_node_in_layer"][1])
+            nodes = b["sub_to_full"][:n1]
+            slot = ref["f2s"][nodes].copy()
+            np.testing.assert_array_equal(cache.sub2embed.cpu().numpy(), slot)
+            used = orc.count_history_reconstruct(b["ptr"], b["idx"], slot, len(b["sub_to_full"]), 40, 3)
+            np.testing.assert_array_equal(cache.used_masks[0].cpu().numpy(), used[0])
+            x_ref = feats[torch.from_numpy(b["sub_to_full"])].numpy() * used[0][:, None]
+            np.testing.assert_array_equal(batch.x.cpu().numpy(), x_ref)
+            hit = slot != -1
+            tab16 = ref["table"].view(np.float16)
+            np.testing.assert_array_equal(cache.cached_embedding.cpu().numpy()[hit], tab16[slot[hit]].astype(np.float32))
+            emb = rng.standard_normal((n1, H)).astype(np.float32)
+            grad = (rng.standard_normal((n1, H)) * np.exp(rng.normal(-3, 1.5, size=(n1, 1)))).astype(np.float32)
+            pe = torch.from_numpy(emb).to(DEV).requires_grad_(True)
+            pe.grad = torch.from_numpy(grad).to(DEV)
+            cache.produced_embedding = pe
+            cache.update_history(batch, it)
+            age = (it - ref["checkin"][np.maximum(slot, 0)]).astype(np.int32)
+            score = orc.row_scores(grad)
+            thres = 0.05 if fixed else float(host_model.quantile_threshold(score, 0.6))
+            rmask, _, _ = orc.grad_check(grad, emb, slot, age, None, nodes, thres, 3, orc.NORM_L2, orc.CMP_LT,
+                                         ref["table"], orc.DT_F16, ref["f2s"], ref["s2f"], ref["checkin"],
+                                         ref["header"], it)
+            np.testing.assert_array_equal(cache.last_record_mask.cpu().numpy(), rmask)
+            np.testing.assert_array_equal(cache.full2slot.cpu().numpy(), ref["f2s"])
+            np.testing.assert_array_equal(cache.slot2full.cpu().numpy(), ref["s2f"])
+            np.testing.assert_array_equal(cache.checkin.cpu().numpy(), ref["checkin"])
+            assert cache.header == int(ref["header"][0])
+            live = ref["s2f"] != -1
+            np.testing.assert_array_equal(cache.table.view(torch.int16).cpu().numpy().view(np.uint16)[live],
+                                          ref["table"][live])
+        assert (ref["s2f"] != -1).sum() > 0
+
+
+def test_input_layer_backward_is_skipped_but_history_grad_is_kept():
+    import hiscache_backend as be
+    from helpers import random_csr, random_hmap
+    from oracle import hc_oracle as orc
+    rng = np.random.default_rng(7)
+    R, N, F = 80, 60, 128
+    ptr, idx = random_csr(rng, R, N, 6)
+    hmap = random_hmap(rng, R, 0.4)
+    x = torch.from_numpy(rng.standard_normal((N, F)).astype(np.float32)).to(DEV)        # raw features: no grad
+    hb = torch.from_numpy(rng.standard_normal((R, F)).astype(np.float32)).to(DEV).requires_grad_(True)
+    g = rng.standard_normal((R, F)).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    out = be.aggr_forward_history(x, t(ptr), t(idx), t(hmap), hb, F, R)
+    out.backward(t(g))
+    assert x.grad is None
+    np.testing.assert_array_equal(hb.grad.cpu().numpy(), orc.bwd_mean_row(ptr, idx, g, hmap, N, (R, F))[1])
