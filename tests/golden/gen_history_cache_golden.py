@@ -1,0 +1,137 @@
+"""Generates tests/golden/history_cache_golden.npz by running the reference's own
+``HistoryCache.update_history`` and ``HistoryCache.lookup_and_load``
+(/root/reference/hiscache/history_cache.py:180-356) on CPU tensors.
+
+Run in the build container only (the reference tree is not available elsewhere):
+
+    python tests/golden/gen_history_cache_golden.py
+
+The reference module is loaded from /root/reference as text-and-exec by importlib; its package
+``__init__`` (which imports CUDA-only extensions) is not executed.  Two collaborators that do not
+exist here are supplied as small stand-ins, and the fixture records which outputs depend on them:
+  * ``hiscache.count_history_reconstruct`` -> this repo's CPU oracle (so ``used_masks`` and everything
+    derived from it in lookup_and_load is NOT independent evidence; the id translation, the
+    cached-embedding gather with -1 slots and the feature-cache merge are);
+  * ``uvm.masked_get(ids, mask)`` -> rows of the feature matrix where the mask is set, zeros elsewhere
+    (semantics inferred from history_cache.py:345-349).
+``update_history`` needs neither: its golden vectors are produced by the reference code alone.
+Only inputs and outputs are stored; no reference source text is copied.
+"""
+import importlib.util
+import logging
+import os
+import sys
+import types
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+sys.path.insert(0, os.path.join(ROOT, "history-cache_amd"))  # synthetic batch generator only
+REF = "/root/reference/hiscache/history_cache.py"
+
+
+def load_reference_class():
+    from oracle import hc_oracle as orc
+
+    def count_history_reconstruct(ptr, idx, hmap, num_node, num_seed, num_layer):
+        out = orc.count_history_reconstruct(ptr.numpy(), idx.numpy(), hmap.numpy(), num_node, num_seed, num_layer)
+        return [torch.from_numpy(m) for m in out]
+
+    pkg = types.ModuleType("hiscache")
+    pkg.__path__ = []
+    pkg.count_history_reconstruct = count_history_reconstruct
+    util = types.ModuleType("hiscache.util")
+    util.log = logging.getLogger("reference")
+    saved = {k: sys.modules.get(k) for k in ("hiscache", "hiscache.util", "hiscache.history_cache")}
+    sys.modules["hiscache"] = pkg
+    sys.modules["hiscache.util"] = util
+    spec = importlib.util.spec_from_file_location("hiscache.history_cache", REF)
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules["hiscache.history_cache"] = mod
+    spec.loader.exec_module(mod)
+    for k, v in saved.items():
+        if v is None:
+            sys.modules.pop(k, None)
+        else:
+            sys.modules[k] = v
+    return mod.HistoryCache
+
+
+class Store:
+    def __init__(self, feats):
+        self.buffer = feats
+
+    def masked_get(self, ids, mask):
+        out = torch.zeros((ids.shape[0], self.buffer.shape[1]), dtype=torch.float32)
+        out[mask] = self.buffer[ids[mask]]
+        return out
+
+
+def main():
+    from helpers import layered_batch
+    HistoryCache = load_reference_class()
+    rng = np.random.default_rng(2024)
+    N, Fin, H, n_iter = 1500, 8, 12, 7
+    buffer_floats = 24 * 400                      # 1200 feature slots, 800 embedding slots
+    feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32))
+    hot = torch.from_numpy(rng.permutation(N).astype(np.int64))
+
+    c = HistoryCache.__new__(HistoryCache)         # __init__ needs a GPU and dataset files
+    c.in_channels, c.hidden_channels, c.total_num_node = Fin, H, N
+    c.device = torch.device("cpu")
+    c.method, c.rate, c.staleness_thres, c.start_history = "grad", 0.6, 4, 0
+    c.feat_mode, c.distributed_store = "history_uvm", False
+    c.uvm = Store(feats)
+    c.header, c.glb_iter, c.num_stored_history = 0, 0, 0
+    c.produced_embedding, c.used_masks = None, None
+    # the state HistoryCache.allocate/fill build (history_cache.py:42-46, 110-116, 134-139, 156-167)
+    c.full2embed = torch.ones([2 * N + 1], dtype=torch.int64) * -1
+    c.buffer = torch.zeros(buffer_floats)
+    c.embed2full = torch.ones(buffer_floats // H, dtype=torch.int64) * -1
+    n_feat = buffer_floats // Fin
+    cache_ids = hot[-n_feat:]
+    c.feat2full = cache_ids + N
+    c.full2embed[c.feat2full] = torch.arange(0, n_feat)
+    c.buffer.view(-1, Fin)[-n_feat:] = feats[cache_ids]
+
+    out = {"N": N, "Fin": Fin, "H": H, "buffer_floats": buffer_floats, "features": feats.numpy(), "hot": hot.numpy(),
+           "rate": 0.6, "staleness_thres": 4, "n_iter": n_iter}
+    high = 0
+    for it in range(1, n_iter + 1):
+        b = layered_batch(rng, N, 20, [5, 4])
+        batch = types.SimpleNamespace(ptr=torch.from_numpy(b["ptr"]), idx=torch.from_numpy(b["idx"]),
+                                      sub_to_full=torch.from_numpy(b["sub_to_full"]),
+                                      num_node_in_layer=torch.from_numpy(b["num_node_in_layer"]),
+                                      y=torch.zeros(20, dtype=torch.int64), x=None)
+        c.lookup_and_load(batch, 2)
+        n1 = int(b["num_node_in_layer"][1])
+        emb = rng.standard_normal((n1, H)).astype(np.float32)
+        grad = (rng.standard_normal((n1, H)) * np.exp(rng.normal(-3, 1.5, size=(n1, 1)))).astype(np.float32)
+        pe = torch.from_numpy(emb.copy()).requires_grad_(True)
+        pe.grad = torch.from_numpy(grad.copy())
+        c.produced_embedding = pe
+        pre = f"it{it}_"
+        for k in ("ptr", "idx", "sub_to_full", "num_node_in_layer"):
+            out[pre + k] = b[k]
+        out[pre + "emb"], out[pre + "grad"] = emb, grad
+        out[pre + "sub2embed"] = c.sub2embed.numpy().copy()
+        out[pre + "sub2feat"] = c.sub2feat.numpy().copy()
+        out[pre + "cached_embedding"] = c.cached_embedding.numpy().copy()
+        out[pre + "x"] = batch.x.numpy().copy()
+        c.update_history(batch, it)
+        out[pre + "full2embed"] = c.full2embed.numpy().copy()
+        out[pre + "embed2full"] = c.embed2full.numpy().copy()
+        out[pre + "header"] = np.int64(c.header)
+        high = max(high, c.header)
+        out[pre + "buffer_front"] = c.buffer.numpy()[: high * H].copy()   # every embedding row written so far
+    np.savez_compressed(os.path.join(HERE, "history_cache_golden.npz"), **out)
+    print("wrote", os.path.join(HERE, "history_cache_golden.npz"), "headers:",
+          [int(out[f"it{i}_header"]) for i in range(1, n_iter + 1)])
+
+
+if __name__ == "__main__":
+    main()
