@@ -120,11 +120,11 @@ def run_c2(args, row_mode=False):
         # the same three launches the autograd Function issues, with a clock on each
         if row_mode:
             out = clk_f(lambda: be._aggr_fwd(be.SUBST_ROW, ptr, idx, feat.detach(), hmap, hbuf, F, None, R))
-            tr = clk_t(lambda: be.build_transpose(ptr, idx, hmap, R, N))
+            tr = clk_t(lambda: be.build_transpose(ptr, idx, hmap, R, N, want_edges=False))
             clk_b(lambda: be._aggr_bwd(ptr, idx, tr, g, hmap, None, feat, False, tuple(hbuf.shape), F, R, N))
         else:
             out = clk_f(lambda: be._aggr_fwd(be.SUBST_SRC, ptr, idx, feat.detach(), hmap, hist, F, None, R))
-            tr = clk_t(lambda: be.build_transpose(ptr, idx, None, R, N))
+            tr = clk_t(lambda: be.build_transpose(ptr, idx, None, R, N, want_edges=False))
             clk_b(lambda: be._aggr_bwd(ptr, idx, tr, g, None, None, feat, False, None, 0, R, N))
         return out
 
@@ -394,7 +394,7 @@ def run_c3(args):
 
     def kstep():
         cf(lambda: be._aggr_fwd(be.SUBST_ROW, ptr, idx, x, hmap, hbuf, H, None, R))
-        tr = ct(lambda: be.build_transpose(ptr, idx, hmap, R, Nsrc))
+        tr = ct(lambda: be.build_transpose(ptr, idx, hmap, R, Nsrc, want_edges=False))
         cb(lambda: be._aggr_bwd(ptr, idx, tr, g, hmap, None, x, False, (R, H), H, R, Nsrc))
         hdr.zero_()
         st["mask"] = cg(lambda: be.grad_check(grad, emb, hmap, sub_to_full, thr, table, f2s, s2f, hdr, 1,

@@ -10,8 +10,10 @@
 //   1. fill      keys[e] = n_src (sentinel) for every edge slot
 //   2. expand    wave per row: keys[e] = idx[e], rows[e] = r for the row's edges
 //                (rows flagged by hmap_row are skipped and keep the sentinel)
-//   3. sort      rocPRIM LSD radix sort of (key, edge slot) pairs -- stable
-//   4. finalize  rowT/edgeT from the sorted pairs; ptrT[s] = lower_bound(keys, s)
+//   3. sort      rocPRIM LSD radix sort of (key, value) pairs -- stable.  When the caller wants
+//                edgeT the value is the edge slot and rowT is gathered afterwards; when it does not
+//                (mean aggregation) the value is the destination row and the sort writes rowT itself
+//   4. finalize  ptrT[s] = first sorted position whose key is >= s
 #include <cstring>
 
 #include <rocprim/rocprim.hpp>
@@ -36,6 +38,8 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_expand(const int64_t *__restrict_
                                                        uint32_t *__restrict__ keys,
                                                        uint32_t *__restrict__ rows, int64_t R,
                                                        int64_t E, int64_t n_src) {
+  // `rows` is indexed by edge slot: either the side array for the later gather, or the sort's
+  // value array itself (mean aggregation)
   const int lane = hc_lane();
   const int64_t row = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
   if (row >= R) return;
@@ -70,7 +74,23 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_finalize_edges(const uint32_t *__
   }
 }
 
-// ptrT[s] = number of sorted keys strictly below s, for s in [0, n_src].
+// ptrT from the sorted keys by boundary detection: position p owns the sources in
+// (key[p-1], key[p]] and writes ptrT[s] = p for them; the last position also closes the tail.
+// Used when sources are not much more numerous than edges, so the per-thread fill loops are short.
+__global__ __launch_bounds__(HC_BLOCK) void tr_ptr_from_boundaries(const uint32_t *__restrict__ skeys,
+                                                                    int64_t *__restrict__ ptrT, int64_t E,
+                                                                    int64_t n_src) {
+  const int64_t p = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (p >= E) return;
+  const int64_t cur = skeys[p];
+  const int64_t prev = p == 0 ? -1 : (int64_t)skeys[p - 1];
+  for (int64_t s = prev + 1; s <= cur; ++s) ptrT[s] = p;
+  if (p == E - 1)
+    for (int64_t s = cur + 1; s <= n_src; ++s) ptrT[s] = E;
+}
+
+// ptrT[s] = number of sorted keys strictly below s, for s in [0, n_src] (binary search; used
+// when there are many more sources than edges).
 __global__ __launch_bounds__(HC_BLOCK) void tr_finalize_ptr(const uint32_t *__restrict__ skeys,
                                                              int64_t *__restrict__ ptrT, int64_t E,
                                                              int64_t n_src) {
@@ -140,7 +160,7 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
     tr_finalize_ptr<<<dim3((unsigned)pblocks), dim3(HC_BLOCK), 0, st>>>(nullptr, ptrT, 0, n_src);
     return hc_launch_status();
   }
-  HC_REQUIRE(ptr && idx && rowT && edgeT);
+  HC_REQUIRE(ptr && idx && rowT);
   Layout L;
   if (!make_layout(E, n_src, &L)) return HC_ELAUNCH;
   if (!workspace || workspace_bytes < L.total) return HC_EWORKSPACE;
@@ -159,15 +179,35 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
   const int64_t rblocks = (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
   if (!hc_grid_ok(eblocks) || !hc_grid_ok(rblocks) || !hc_grid_ok(pblocks)) return HC_EUNSUPPORTED;
 
+  const bool want_edges = edgeT != nullptr;
+  const unsigned bits = (unsigned)key_bits(n_src);
+  const uint32_t *skeys = nullptr;
   tr_fill<<<dim3((unsigned)eblocks), dim3(HC_BLOCK), 0, st>>>(keys0, vals0, E, sentinel);
-  tr_expand<<<dim3((unsigned)rblocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, rows, R, E,
-                                                                n_src);
-  rocprim::double_buffer<uint32_t> dk(keys0, keys1), dv(vals0, vals1);
-  if (rocprim::radix_sort_pairs(temp, temp_bytes, dk, dv, (size_t)E, 0u, (unsigned)key_bits(n_src), st,
-                                false) != hipSuccess)
-    return HC_ELAUNCH;
-  tr_finalize_edges<<<dim3((unsigned)eblocks), dim3(HC_BLOCK), 0, st>>>(dk.current(), dv.current(),
-                                                                        rows, rowT, edgeT, E, sentinel);
-  tr_finalize_ptr<<<dim3((unsigned)pblocks), dim3(HC_BLOCK), 0, st>>>(dk.current(), ptrT, E, n_src);
+  if (want_edges) {
+    tr_expand<<<dim3((unsigned)rblocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, rows, R, E, n_src);
+    rocprim::double_buffer<uint32_t> dk(keys0, keys1), dv(vals0, vals1);
+    if (rocprim::radix_sort_pairs(temp, temp_bytes, dk, dv, (size_t)E, 0u, bits, st, false) != hipSuccess)
+      return HC_ELAUNCH;
+    tr_finalize_edges<<<dim3((unsigned)eblocks), dim3(HC_BLOCK), 0, st>>>(dk.current(), dv.current(), rows,
+                                                                          rowT, edgeT, E, sentinel);
+    skeys = dk.current();
+  } else {
+    // value = destination row; dropped edge slots keep the fill value and sort behind the sentinel
+    tr_expand<<<dim3((unsigned)rblocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, R, E, n_src);
+    // rowT doubles as the sort's second value buffer; copy only if the result landed in the first
+    uint32_t *rowT_u = reinterpret_cast<uint32_t *>(rowT);
+    rocprim::double_buffer<uint32_t> dk(keys0, keys1), dv(vals0, rowT_u);
+    if (rocprim::radix_sort_pairs(temp, temp_bytes, dk, dv, (size_t)E, 0u, bits, st, false) != hipSuccess)
+      return HC_ELAUNCH;
+    if (dv.current() != rowT_u &&
+        hipMemcpyAsync(rowT, dv.current(), (size_t)E * sizeof(uint32_t), hipMemcpyDeviceToDevice, st) != hipSuccess)
+      return HC_ELAUNCH;
+    skeys = dk.current();
+  }
+  if (n_src <= 4 * E) {
+    tr_ptr_from_boundaries<<<dim3((unsigned)eblocks), dim3(HC_BLOCK), 0, st>>>(skeys, ptrT, E, n_src);
+  } else {
+    tr_finalize_ptr<<<dim3((unsigned)pblocks), dim3(HC_BLOCK), 0, st>>>(skeys, ptrT, E, n_src);
+  }
   return hc_launch_status();
 }

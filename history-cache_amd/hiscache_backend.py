@@ -169,10 +169,11 @@ def _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, num_node):
     return out
 
 
-def build_transpose(ptr, idx, history_map_row, num_node, n_src, num_edge=None):
+def build_transpose(ptr, idx, history_map_row, num_node, n_src, num_edge=None, want_edges=True):
     """Stable CSC view of the first ``num_node`` rows: returns (ptrT, rowT, edgeT).
 
-    ``num_edge`` bounds the edge slots that are sorted (default: all of ``idx``)."""
+    ``num_edge`` bounds the edge slots that are sorted (default: all of ``idx``).  With
+    ``want_edges=False`` (enough for the mean aggregation) edgeT is None and the build is cheaper."""
     lib = load_library()
     _dev(ptr, "ptr", torch.int64)
     _dev(idx, "idx", torch.int64)
@@ -182,7 +183,7 @@ def build_transpose(ptr, idx, history_map_row, num_node, n_src, num_edge=None):
     dev = ptr.device
     ptrT = torch.empty(n_src + 1, dtype=torch.int64, device=dev)
     rowT = torch.empty(max(E, 1), dtype=torch.int32, device=dev)
-    edgeT = torch.empty(max(E, 1), dtype=torch.int32, device=dev)
+    edgeT = torch.empty(max(E, 1), dtype=torch.int32, device=dev) if want_edges else None
     nbytes = lib.hc_transpose_workspace_bytes(R, E, n_src)
     if nbytes == 0:
         raise RuntimeError("hc_transpose_workspace_bytes failed (no usable GPU?)")
@@ -260,7 +261,7 @@ class _AggrHistory(torch.autograd.Function):
                 hit = (row_map[:R] != -1).unsqueeze(1)
                 grad_h.view(-1, hsize)[:R, :flat.shape[1]] = torch.where(hit, flat, torch.zeros_like(flat))
             return None, None, None, None, None, grad_h, None, None, None
-        tr = build_transpose(ptr, idx, row_map, R, n_src)
+        tr = build_transpose(ptr, idx, row_map, R, n_src, want_edges=ev is not None)
         grad_x, grad_h, edge_grad = _aggr_bwd(ptr, idx, tr, g, row_map, ev, x, want_eg, hshape, hsize, R,
                                               n_src)
         if grad_x.dtype != x.dtype:

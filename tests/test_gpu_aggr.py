@@ -167,6 +167,23 @@ def test_build_transpose_bit_exact(be, orc, R, N, E_extra):
         k = int(rp[-1])
         np.testing.assert_array_equal(rowT.cpu().numpy()[:k], rr)
         np.testing.assert_array_equal(edgeT.cpu().numpy()[:k], re)
+        # the cheaper build without edge slots gives the same segments and rows
+        ptrT2, rowT2, none_ = be.build_transpose(T(ptr), T(idx_all), None if hm is None else T(hm), R, N,
+                                                 want_edges=False)
+        assert none_ is None
+        np.testing.assert_array_equal(ptrT2.cpu().numpy(), rp)
+        np.testing.assert_array_equal(rowT2.cpu().numpy()[:k], rr)
+
+
+def test_build_transpose_many_more_sources_than_edges(be, orc):
+    rng = np.random.default_rng(9)
+    R, N = 40, 5000                                   # sparse: the segment bounds come from a binary search
+    ptr, idx = random_csr(rng, R, N, 5)
+    for want in (True, False):
+        ptrT, rowT, _ = be.build_transpose(T(ptr), T(idx), None, R, N, want_edges=want)
+        rp, rr, _ = orc.build_transpose(ptr, idx, None, N)
+        np.testing.assert_array_equal(ptrT.cpu().numpy(), rp)
+        np.testing.assert_array_equal(rowT.cpu().numpy()[: int(rp[-1])], rr)
 
 
 def test_build_transpose_no_edges(be):
