@@ -157,6 +157,7 @@ __global__ __launch_bounds__(HC_BLOCK) void gc_pass1(
 // are dropped, header += written, *overflow = dropped.
 // ---------------------------------------------------------------------------------------
 constexpr int GC_SCAN_THREADS = 1024;
+constexpr int GC_SCAN_ITEMS = 8;  // consecutive counts per thread per sweep
 __global__ __launch_bounds__(GC_SCAN_THREADS) void gc_pass2(int64_t *__restrict__ tile_counts,
                                                              int64_t n_tiles, GcScalars *__restrict__ sc,
                                                              int64_t *__restrict__ header,
@@ -168,11 +169,18 @@ __global__ __launch_bounds__(GC_SCAN_THREADS) void gc_pass2(int64_t *__restrict_
   const int wave = (int)(threadIdx.x >> 6);
   if (threadIdx.x == 0) carry_s = 0;
   __syncthreads();
-  for (int64_t base = 0; base < n_tiles; base += GC_SCAN_THREADS) {
-    const int64_t i = base + threadIdx.x;
-    const int64_t v = i < n_tiles ? tile_counts[i] : 0;
-    // inclusive scan inside the wave
-    int64_t x = v;
+  constexpr int64_t SWEEP = (int64_t)GC_SCAN_THREADS * GC_SCAN_ITEMS;
+  for (int64_t base = 0; base < n_tiles; base += SWEEP) {
+    const int64_t i0 = base + (int64_t)threadIdx.x * GC_SCAN_ITEMS;
+    int64_t v[GC_SCAN_ITEMS];
+    int64_t mine = 0;
+#pragma unroll
+    for (int k = 0; k < GC_SCAN_ITEMS; ++k) {
+      v[k] = i0 + k < n_tiles ? tile_counts[i0 + k] : 0;
+      mine += v[k];
+    }
+    // inclusive scan of the per-thread sums inside the wave
+    int64_t x = mine;
 #pragma unroll
     for (int d = 1; d < HC_WAVE; d <<= 1) {
       const int lo = __shfl_up((int)(uint32_t)(uint64_t)x, d, HC_WAVE);
@@ -182,12 +190,21 @@ __global__ __launch_bounds__(GC_SCAN_THREADS) void gc_pass2(int64_t *__restrict_
     }
     if (lane == HC_WAVE - 1) wave_tot[wave] = x;
     __syncthreads();
-    int64_t wave_off = 0;
-    for (int w = 0; w < wave; ++w) wave_off += wave_tot[w];
+    int64_t wave_off = 0, sweep_total = 0;
+    for (int w = 0; w < GC_SCAN_THREADS / HC_WAVE; ++w) {
+      const int64_t t = wave_tot[w];
+      if (w < wave) wave_off += t;
+      sweep_total += t;
+    }
     const int64_t carry = carry_s;
-    if (i < n_tiles) tile_counts[i] = carry + wave_off + x - v;  // exclusive
+    int64_t run = carry + wave_off + x - mine;  // exclusive prefix of this thread's first item
+#pragma unroll
+    for (int k = 0; k < GC_SCAN_ITEMS; ++k) {
+      if (i0 + k < n_tiles) tile_counts[i0 + k] = run;
+      run += v[k];
+    }
     __syncthreads();
-    if (threadIdx.x == GC_SCAN_THREADS - 1) carry_s = carry + wave_off + x;
+    if (threadIdx.x == 0) carry_s = carry + sweep_total;
     __syncthreads();
   }
   if (threadIdx.x == 0) {
