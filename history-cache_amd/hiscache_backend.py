@@ -66,6 +66,18 @@ _SIGNATURES = {
 
 _lib_handle = None
 
+# Build the transposed view of a block on a side stream during the forward pass (it only depends
+# on the graph), so that backward finds it ready.  Set to False to build it inside backward.
+PREFETCH_TRANSPOSE = True
+_side_streams = {}
+
+
+def _side_stream(device):
+    key = torch.device(device).index or 0
+    if key not in _side_streams:
+        _side_streams[key] = torch.cuda.Stream(device=device)  # default priority
+    return _side_streams[key]
+
 
 def load_library():
     """Load ``libhiscache_hip.so`` and bind every export.  Raises if it is not built."""
@@ -231,11 +243,24 @@ class _AggrHistory(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, ptr, idx, edge_value, hmap, hbuf, hsize, num_node, mode):
         R = int(num_node) if num_node else ptr.numel() - 1
+        ctx.tr = None
+        needs = ctx.needs_input_grad
+        if PREFETCH_TRANSPOSE and (needs[0] or (edge_value is not None and needs[3])):
+            # The transposed view depends on the graph only: build it on a side stream while the
+            # forward gather runs, and hand it to backward.
+            cur = torch.cuda.current_stream(x.device)
+            side = _side_stream(x.device)
+            side.wait_stream(cur)
+            with torch.cuda.stream(side):
+                tr = build_transpose(ptr, idx, hmap if mode == SUBST_ROW else None, R, x.shape[0],
+                                     want_edges=edge_value is not None)
+                done = torch.cuda.Event()
+                done.record(side)
+            ctx.tr = (tr, done)
         out = _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, R)
         ctx.hc = (ptr, idx, hmap, hsize, R, mode, None if hbuf is None else tuple(hbuf.shape))
         ctx.save_for_backward(x, edge_value if edge_value is not None else x.new_empty(0))
         ctx.has_ev = edge_value is not None
-        ctx.mark_non_differentiable()
         return out
 
     @staticmethod
@@ -261,7 +286,15 @@ class _AggrHistory(torch.autograd.Function):
                 hit = (row_map[:R] != -1).unsqueeze(1)
                 grad_h.view(-1, hsize)[:R, :flat.shape[1]] = torch.where(hit, flat, torch.zeros_like(flat))
             return None, None, None, None, None, grad_h, None, None, None
-        tr = build_transpose(ptr, idx, row_map, R, n_src, want_edges=ev is not None)
+        if ctx.tr is not None:
+            tr, done = ctx.tr
+            cur = torch.cuda.current_stream(g.device)
+            cur.wait_event(done)
+            for t in tr:
+                if t is not None:
+                    t.record_stream(cur)
+        else:
+            tr = build_transpose(ptr, idx, row_map, R, n_src, want_edges=ev is not None)
         grad_x, grad_h, edge_grad = _aggr_bwd(ptr, idx, tr, g, row_map, ev, x, want_eg, hshape, hsize, R,
                                               n_src)
         if grad_x.dtype != x.dtype:
