@@ -29,12 +29,184 @@ namespace {
 // Blocks [0, src_blocks) own source rows; blocks beyond own rows of grad_hbuf.
 // ---------------------------------------------------------------------------------------
 constexpr int BWD_SRC_PER_WAVE = 32;
+// With a workspace, a source with more than BWD_CHUNK incoming edges ("hub") is summed in chunks
+// of BWD_CHUNK edges by independent waves; the chunk sums are then combined left to right.
+constexpr int BWD_CHUNK = 512;
+
+// Workspace of the hub path.
+struct BwdHubHeader {
+  int n_hubs;
+  int n_chunks;
+  int pad[62];
+};
+struct BwdHubLayout {
+  size_t hub_src, hub_chunk0, chunk_hub, partial, total;
+  int64_t max_hubs, max_chunks;
+};
+inline BwdHubLayout bwd_hub_layout(int64_t E, int64_t F) {
+  BwdHubLayout L;
+  L.max_hubs = E / BWD_CHUNK + 1;          // a hub has more than BWD_CHUNK edges
+  L.max_chunks = E / BWD_CHUNK + L.max_hubs + 1;  // sum of ceil(len/BWD_CHUNK) over hubs
+  size_t off = sizeof(BwdHubHeader);
+  L.hub_src = off;
+  off += hc_align_up((size_t)L.max_hubs * sizeof(int32_t), 256);
+  L.hub_chunk0 = off;
+  off += hc_align_up((size_t)L.max_hubs * sizeof(int32_t), 256);
+  L.chunk_hub = off;
+  off += hc_align_up((size_t)L.max_chunks * sizeof(int32_t), 256);
+  L.partial = off;
+  off += hc_align_up((size_t)L.max_chunks * (size_t)F * sizeof(float), 256);
+  L.total = off;
+  return L;
+}
+
+__global__ void bwd_hub_clear(BwdHubHeader *h) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    h->n_hubs = 0;
+    h->n_chunks = 0;
+  }
+}
+
+// One thread per source: sources with more than BWD_CHUNK incoming edges take a run of chunk slots.
+// The order in which hubs take their slots only decides where scratch data lives.
+__global__ __launch_bounds__(HC_BLOCK) void bwd_hub_find(const int64_t *__restrict__ ptrT, int64_t n_src,
+                                                          BwdHubHeader *__restrict__ h,
+                                                          int32_t *__restrict__ hub_src,
+                                                          int32_t *__restrict__ hub_chunk0,
+                                                          int32_t *__restrict__ chunk_hub, int64_t max_hubs,
+                                                          int64_t max_chunks) {
+  const int64_t s = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (s >= n_src) return;
+  const int64_t len = ptrT[s + 1] - ptrT[s];
+  if (len <= BWD_CHUNK) return;
+  const int nch = (int)((len + BWD_CHUNK - 1) / BWD_CHUNK);
+  const int hub = atomicAdd(&h->n_hubs, 1);
+  const int c0 = atomicAdd(&h->n_chunks, nch);
+  // The bounds hold whenever ptrT[n_src] <= E_total (the caller's contract); the guard only keeps
+  // a violated contract from writing outside the workspace.
+  if (hub >= max_hubs || (int64_t)c0 + nch > max_chunks) {
+    if (hub < max_hubs) hub_src[hub] = -1;
+    for (int i = 0; i < nch && (int64_t)c0 + i < max_chunks; ++i) chunk_hub[c0 + i] = -1;
+    return;
+  }
+  hub_src[hub] = (int32_t)s;
+  hub_chunk0[hub] = c0;
+  for (int i = 0; i < nch; ++i) chunk_hub[c0 + i] = hub;
+}
+
+// Sum of g[r,:]/deg(r) over transposed edges [begin, end), added to acc in order by the calling wave.
+template <int VEC, int CHUNKS, int UNROLL>
+__device__ __forceinline__ void bwd_accumulate(const int64_t *__restrict__ ptr, const int32_t *__restrict__ rowT,
+                                               const float *__restrict__ g, int64_t begin, int64_t end,
+                                               int lane, float (&acc)[CHUNKS][VEC]) {
+  constexpr int F = HC_WAVE * VEC * CHUNKS;
+  for (int64_t base = begin; base < end; base += HC_WAVE) {
+    const int64_t left = end - base;
+    const int n = left < HC_WAVE ? (int)left : HC_WAVE;
+    int my_row = 0;
+    float my_deg = 1.0f;
+    if (lane < n) {
+      my_row = rowT[base + lane];
+      my_deg = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
+    }
+    for (int j = 0; j < n; j += UNROLL) {
+      float v[UNROLL][CHUNKS][VEC];
+      float d[UNROLL];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        d[u] = 1.0f;
+        if (j + u < n) {
+          const int r = __builtin_amdgcn_readlane(my_row, j + u);
+          d[u] = hc_readlane_f(my_deg, j + u);
+          const float *p = g + (int64_t)r * F + lane * VEC;
+#pragma unroll
+          for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        if (j + u < n) {
+#pragma unroll
+          for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[k][i] += v[u][k][i] / d[u];
+        }
+      }
+    }
+  }
+}
+
+// One wave per chunk slot: the chunk's edges are summed in transposed order into partial[slot].
+template <int VEC, int CHUNKS, int UNROLL>
+__global__ __launch_bounds__(HC_BLOCK) void bwd_hub_partial(
+    const int64_t *__restrict__ ptr, const int64_t *__restrict__ ptrT, const int32_t *__restrict__ rowT,
+    const float *__restrict__ g, const BwdHubHeader *__restrict__ h, const int32_t *__restrict__ hub_src,
+    const int32_t *__restrict__ hub_chunk0, const int32_t *__restrict__ chunk_hub,
+    float *__restrict__ partial, int64_t max_chunks) {
+  constexpr int F = HC_WAVE * VEC * CHUNKS;
+  const int lane = hc_lane();
+  const int64_t c = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (c >= h->n_chunks || c >= max_chunks) return;
+  const int hub = chunk_hub[c];
+  if (hub < 0) return;
+  const int64_t s = hub_src[hub];
+  if (s < 0) return;
+  const int64_t local = c - hub_chunk0[hub];
+  const int64_t begin = ptrT[s] + local * BWD_CHUNK;
+  int64_t end = begin + BWD_CHUNK;
+  const int64_t seg_end = ptrT[s + 1];
+  if (end > seg_end) end = seg_end;
+  float acc[CHUNKS][VEC];
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
+  bwd_accumulate<VEC, CHUNKS, UNROLL>(ptr, rowT, g, begin, end, lane, acc);
+  float *__restrict__ o = partial + c * F + lane * VEC;
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store(o + k * HC_WAVE * VEC, acc[k]);
+}
+
+// One wave per hub: chunk sums combined left to right into the hub's output row.
+template <int VEC, int CHUNKS>
+__global__ __launch_bounds__(HC_BLOCK) void bwd_hub_final(const int64_t *__restrict__ ptrT,
+                                                           const BwdHubHeader *__restrict__ h,
+                                                           const int32_t *__restrict__ hub_src,
+                                                           const int32_t *__restrict__ hub_chunk0,
+                                                           const float *__restrict__ partial,
+                                                           float *__restrict__ grad_vin, int64_t max_hubs) {
+  constexpr int F = HC_WAVE * VEC * CHUNKS;
+  const int lane = hc_lane();
+  const int64_t hub = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (hub >= h->n_hubs || hub >= max_hubs) return;
+  const int64_t s = hub_src[hub];
+  if (s < 0) return;
+  const int64_t len = ptrT[s + 1] - ptrT[s];
+  const int nch = (int)((len + BWD_CHUNK - 1) / BWD_CHUNK);
+  const float *__restrict__ p = partial + (int64_t)hub_chunk0[hub] * F + lane * VEC;
+  float acc[CHUNKS][VEC];
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, acc[k]);
+  for (int c = 1; c < nch; ++c) {
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k) {
+      float v[VEC];
+      hc_vec<float, VEC>::load(p + (int64_t)c * F + k * HC_WAVE * VEC, v);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) acc[k][i] += v[i];
+    }
+  }
+  float *__restrict__ o = grad_vin + s * F + lane * VEC;
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store(o + k * HC_WAVE * VEC, acc[k]);
+}
 
 template <int VEC, int CHUNKS, int UNROLL>
 __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ ptrT, const int32_t *__restrict__ rowT,
     const float *__restrict__ g, const int64_t *__restrict__ hmap, float *__restrict__ grad_vin,
-    float *__restrict__ grad_hbuf, int64_t hsize, int64_t R, int64_t n_src, int64_t src_blocks) {
+    float *__restrict__ grad_hbuf, int64_t hsize, int64_t R, int64_t n_src, int64_t src_blocks,
+    int64_t hub_thres) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   constexpr int S = BWD_SRC_PER_WAVE;
   const int lane = hc_lane();
@@ -55,8 +227,11 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
   const int ns = rest < S ? (int)rest : S;
   // lane l holds the segment bound ptrT[s0 + l], l = 0..ns
   const int64_t my_p = ptrT[s0 + (lane < ns ? lane : ns)];
-  const int64_t e_begin = hc_readlane64(my_p, 0);
+  const int64_t my_p1 = ptrT[s0 + (lane + 1 < ns ? lane + 1 : ns)];
   const int64_t e_end = hc_readlane64(my_p, ns);
+  // sources summed elsewhere (hub path): their segments are stepped over and not stored here
+  const unsigned long long hub_mask =
+      hub_thres > 0 ? __ballot(lane < ns && (my_p1 - my_p) > hub_thres) : 0ull;
 
   float acc[CHUNKS][VEC];
 #pragma unroll
@@ -66,9 +241,32 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
   int cur = 0;                                   // source (relative to s0) being accumulated
   int64_t cur_end = hc_readlane64(my_p, 1);      // end of its segment
   float *__restrict__ obase = grad_vin + s0 * F + lane * VEC;
+  int64_t base = hc_readlane64(my_p, 0);
 
-  for (int64_t base = e_begin; base < e_end; base += HC_WAVE) {
-    const int64_t left = e_end - base;
+  while (true) {  // every branch below advances `cur` or `base`; all of it is wave-uniform
+    // close the sources whose segment ends at or before `base` (zeros for sources without edges)
+    while (cur < ns && base >= cur_end) {
+      if (((hub_mask >> cur) & 1ull) == 0ull) {
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store(obase + (int64_t)cur * F + k * HC_WAVE * VEC, acc[k]);
+      }
+#pragma unroll
+      for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
+      ++cur;
+      cur_end = hc_readlane64(my_p, cur + 1 <= ns ? cur + 1 : ns);
+    }
+    if (cur >= ns) break;
+    if ((hub_mask >> cur) & 1ull) {  // step over a hub's segment
+      base = cur_end;
+      continue;
+    }
+    // stage up to 64 edges, stopping in front of the next hub's segment
+    const unsigned long long ahead = hub_mask >> cur;
+    const int nh = ahead != 0ull ? cur + __builtin_ctzll(ahead) : ns;
+    const int64_t stop = hc_readlane64(my_p, nh);
+    const int64_t left = stop - base;
     const int n = left < HC_WAVE ? (int)left : HC_WAVE;
     int my_row = 0;
     float my_deg = 1.0f;
@@ -81,6 +279,7 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
       float d[UNROLL];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
+        d[u] = 1.0f;
         if (j + u < n) {
           const int r = __builtin_amdgcn_readlane(my_row, j + u);
           d[u] = hc_readlane_f(my_deg, j + u);
@@ -93,7 +292,7 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
       for (int u = 0; u < UNROLL; ++u) {
         if (j + u < n) {
           const int64_t e = base + j + u;
-          while (e >= cur_end) {  // wave-uniform: close finished (possibly empty) segments
+          while (e >= cur_end) {  // close finished (possibly empty) segments; none of them is a hub
 #pragma unroll
             for (int k = 0; k < CHUNKS; ++k) {
               hc_vec<float, VEC>::store(obase + (int64_t)cur * F + k * HC_WAVE * VEC, acc[k]);
@@ -110,16 +309,9 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
         }
       }
     }
+    base += n;
   }
-  // flush the open segment and the trailing sources without edges
-  for (; cur < ns; ++cur) {
-#pragma unroll
-    for (int k = 0; k < CHUNKS; ++k) {
-      hc_vec<float, VEC>::store(obase + (int64_t)cur * F + k * HC_WAVE * VEC, acc[k]);
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
-    }
-  }
+  (void)e_end;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -252,27 +444,69 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_edge_grad(
 template <int VEC, int CHUNKS>
 int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, const float *g,
                 const int64_t *hmap, float *grad_vin, float *grad_hbuf, int64_t hsize, int64_t R,
-                int64_t n_src, hipStream_t st) {
+                int64_t n_src, int64_t E_slots, void *workspace, size_t workspace_bytes, hipStream_t st) {
   constexpr int per = VEC * CHUNKS;
   constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
+  constexpr int F = HC_WAVE * VEC * CHUNKS;
   const int64_t per_block = (int64_t)HC_WAVES_PER_BLOCK * BWD_SRC_PER_WAVE;
   const int64_t sb = (n_src + per_block - 1) / per_block;
   const int64_t hb = (grad_hbuf && hmap) ? (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK : 0;
   if (sb + hb == 0) return HC_OK;
   if (!hc_grid_ok(sb + hb)) return HC_EUNSUPPORTED;
+  int64_t hub_thres = 0;
+  BwdHubLayout L = bwd_hub_layout(E_slots, F);
+  char *ws = static_cast<char *>(workspace);
+  const bool hubs = workspace != nullptr && E_slots > BWD_CHUNK && n_src > 0 && workspace_bytes >= L.total &&
+                    reinterpret_cast<uintptr_t>(ws) % 256 == 0;
+  BwdHubHeader *hh = reinterpret_cast<BwdHubHeader *>(ws);
+  int32_t *hub_src = reinterpret_cast<int32_t *>(ws + L.hub_src);
+  int32_t *hub_chunk0 = reinterpret_cast<int32_t *>(ws + L.hub_chunk0);
+  int32_t *chunk_hub = reinterpret_cast<int32_t *>(ws + L.chunk_hub);
+  float *partial = reinterpret_cast<float *>(ws + L.partial);
+  if (hubs) {
+    hub_thres = BWD_CHUNK;
+    const int64_t fb = (n_src + HC_BLOCK - 1) / HC_BLOCK;
+    const int64_t cb = (L.max_chunks + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+    if (!hc_grid_ok(fb) || !hc_grid_ok(cb)) return HC_EUNSUPPORTED;
+    bwd_hub_clear<<<dim3(1), dim3(64), 0, st>>>(hh);
+    bwd_hub_find<<<dim3((unsigned)fb), dim3(HC_BLOCK), 0, st>>>(ptrT, n_src, hh, hub_src, hub_chunk0, chunk_hub,
+                                                                L.max_hubs, L.max_chunks);
+    bwd_hub_partial<VEC, CHUNKS, UNROLL><<<dim3((unsigned)cb), dim3(HC_BLOCK), 0, st>>>(
+        ptr, ptrT, rowT, g, hh, hub_src, hub_chunk0, chunk_hub, partial, L.max_chunks);
+    if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
+  }
   bwd_mean_fast<VEC, CHUNKS, UNROLL><<<dim3((unsigned)(sb + hb)), dim3(HC_BLOCK), 0, st>>>(
-      ptr, ptrT, rowT, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb);
+      ptr, ptrT, rowT, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hub_thres);
+  if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
+  if (hubs) {
+    const int64_t hbk = (L.max_hubs + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+    if (!hc_grid_ok(hbk)) return HC_EUNSUPPORTED;
+    bwd_hub_final<VEC, CHUNKS><<<dim3((unsigned)hbk), dim3(HC_BLOCK), 0, st>>>(ptrT, hh, hub_src, hub_chunk0,
+                                                                            partial, grad_vin, L.max_hubs);
+  }
   return hc_launch_status();
 }
 
+bool bwd_fast_shape(int64_t F) {
+  return F == 64 || F == 128 || F == 192 || F == 256 || F == 384 || F == 512 || F == 768 || F == 1024;
+}
+
 }  // namespace
+
+extern "C" size_t hc_aggr_bwd_workspace_bytes(int64_t E_total, int64_t F) {
+  if (E_total < 0 || F <= 0) return 0;
+  if (!bwd_fast_shape(F) || E_total <= BWD_CHUNK) return 0;
+  return bwd_hub_layout(E_total, F).total;
+}
+
+extern "C" int64_t hc_aggr_bwd_chunk_edges(int64_t F) { return bwd_fast_shape(F) ? BWD_CHUNK : 0; }
 
 extern "C" int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t *ptrT,
                            const int32_t *rowT, const int32_t *edgeT, const float *g,
                            const int64_t *hmap, const float *edge_value, const void *vin, int in_dtype,
                            int64_t n_head, float *grad_vin, float *grad_hbuf, int64_t hsize,
                            float *edge_grad, int64_t E_total, int64_t R, int64_t F, int64_t n_src,
-                           void *stream) {
+                           void *workspace, size_t workspace_bytes, void *stream) {
   HC_REQUIRE(R >= 0 && F > 0 && n_src >= 0 && n_head >= 1 && E_total >= 0);
   HC_REQUIRE(ptr && ptrT && g);
   HC_REQUIRE(grad_vin || n_src == 0);
@@ -297,7 +531,8 @@ extern "C" int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t
     done = true;
 #define HC_FAST(V, C)                                                                             \
   if (F == 64 * (V) * (C))                                                                        \
-    rc = launch_fast<V, C>(ptr, ptrT, rowT, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, st);   \
+    rc = launch_fast<V, C>(ptr, ptrT, rowT, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, E_total,  \
+                           workspace, workspace_bytes, st);                                      \
   else
     HC_FAST(4, 1) HC_FAST(4, 2) HC_FAST(4, 3) HC_FAST(4, 4) HC_FAST(2, 1) HC_FAST(2, 3) HC_FAST(1, 1)
     HC_FAST(1, 3) done = false;

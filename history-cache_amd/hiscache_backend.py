@@ -46,8 +46,10 @@ _SIGNATURES = {
     "hc_transpose_workspace_bytes": (_c_sz, [_c_i64, _c_i64, _c_i64]),
     "hc_build_transpose": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p,
                                     _c_sz, _c_p]),
+    "hc_aggr_bwd_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
+    "hc_aggr_bwd_chunk_edges": (_c_i64, [_c_i64]),
     "hc_aggr_bwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_p,
-                             _c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_p]),
+                             _c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]),
     "hc_count_history": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p]),
     "hc_row_scores": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_int, _c_p]),
     "hc_grad_check_workspace_bytes": (_c_sz, [_c_i64]),
@@ -226,11 +228,16 @@ def _aggr_bwd(ptr, idx, tr, g, hmap, edge_value, x, want_edge_grad, hbuf_shape, 
     edge_grad = None
     if want_edge_grad:
         edge_grad = torch.empty_like(edge_value)
-    E_total = edge_value.shape[0] if edge_value is not None else 0
+    E_total = rowT.numel()
+    if edge_value is not None:
+        E_total = max(E_total, edge_value.shape[0]) if edge_grad is None else edge_value.shape[0]
+    nbytes = lib.hc_aggr_bwd_workspace_bytes(rowT.numel(), F) if edge_value is None and n_head == 1 else 0
+    ws = _workspace(nbytes, dev) if nbytes else None
     rc = lib.hc_aggr_bwd(_ptr(ptr), _ptr(idx), _ptr(ptrT), _ptr(rowT), _ptr(edgeT), _ptr(g), _ptr(hmap),
                          _ptr(edge_value), _ptr(x) if want_edge_grad else _c_p(None),
                          _float_dtype(x, "input") if want_edge_grad else 0, n_head, _ptr(grad_x),
-                         _ptr(grad_h), int(hsize), _ptr(edge_grad), E_total, R, F, n_src, _stream())
+                         _ptr(grad_h), int(hsize), _ptr(edge_grad), E_total, R, F, n_src, _ptr(ws),
+                         ws.numel() if ws is not None else 0, _stream())
     _check(rc, "hc_aggr_bwd")
     return grad_x, grad_h, edge_grad
 
@@ -570,6 +577,11 @@ def lookup(map_tensor, ids, offset=0):
 def long_row_edges(feature_width, dtype=torch.float32):
     """Rows with more edges than this are summed as four quarters by the mean forward (0: never)."""
     return int(load_library().hc_aggr_fwd_long_row_edges(int(feature_width), _DTYPES[dtype]))
+
+
+def bwd_chunk_edges(feature_width):
+    """Sources with more incoming edges than this are summed in chunks by the mean backward (0: never)."""
+    return int(load_library().hc_aggr_bwd_chunk_edges(int(feature_width)))
 
 
 def version():

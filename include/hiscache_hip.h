@@ -121,14 +121,23 @@ int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hm
  *       rows, 0 for the others.  E_total = number of edge slots to fill.
  *
  * ptrT/rowT/edgeT come from hc_build_transpose called with the same hmap_row
- * (so edges of history rows are already gone).  In HC_SUBST_SRC mode pass
- * hmap = NULL: the result is the gradient with respect to the substituted
- * source row, whichever table it came from. */
+ * (so edges of history rows are already gone); ptrT[n_src] <= E_total.  In
+ * HC_SUBST_SRC mode pass hmap = NULL: the result is the gradient with respect
+ * to the substituted source row, whichever table it came from.
+ * Summation order (fp32, fixed): ascending destination row.  When a workspace
+ * of hc_aggr_bwd_workspace_bytes() is given and hc_aggr_bwd_chunk_edges(F)
+ * reports C > 0, a source with more than C incoming edges is summed in chunks
+ * of C consecutive edges (each chunk in order, by its own wave) and the chunk
+ * sums are combined left to right; without a workspace (NULL) every source is
+ * summed strictly in order by one wave.  The workspace must be 256-byte
+ * aligned. */
+size_t hc_aggr_bwd_workspace_bytes(int64_t E_total, int64_t F);
+int64_t hc_aggr_bwd_chunk_edges(int64_t F);
 int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t *ptrT, const int32_t *rowT,
                 const int32_t *edgeT, const float *g, const int64_t *hmap, const float *edge_value,
                 const void *vin, int in_dtype, int64_t n_head, float *grad_vin, float *grad_hbuf,
                 int64_t hsize, float *edge_grad, int64_t E_total, int64_t R, int64_t F,
-                int64_t n_src, void *stream);
+                int64_t n_src, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---------------------------------------------------------------- used masks
  * Replaces count_history_reconstruct (src/cpp/include/grad_check.h:18-20,

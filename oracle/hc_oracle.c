@@ -252,9 +252,29 @@ int orc_fwd_mean_src(const Index *ptr, const Index *idx, const float *feat,
  * grads_out[n_src,F] and grads_history[R,hsize] are zero-filled first (:503-504). */
 int orc_bwd_mean_row(const Index *ptr, const Index *idx, const float *g,
                      const Index *hmap, float *grads_out, float *grads_history,
-                     Index R, Index F, Index hsize, Index n_src) {
+                     Index R, Index F, Index hsize, Index n_src, Index chunk) {
+  /* chunk == 0: every source row is summed strictly in (row, edge) order.  chunk > 0 restates the
+   * device library's documented order for hubs: a source with more than `chunk` incoming edges is
+   * summed in chunks of `chunk` consecutive incoming edges, each chunk from zero in order, and the
+   * chunk sums are combined left to right. */
   memset(grads_out, 0, (size_t)(n_src * F) * sizeof(float));
   if (grads_history) memset(grads_history, 0, (size_t)(R * hsize) * sizeof(float));
+  Index *indeg = NULL, *seen = NULL, *hub_of = NULL;
+  float *part = NULL;
+  Index n_hubs = 0;
+  if (chunk > 0) {
+    indeg = (Index *)calloc((size_t)(n_src > 0 ? n_src : 1), sizeof(Index));
+    seen = (Index *)calloc((size_t)(n_src > 0 ? n_src : 1), sizeof(Index));
+    hub_of = (Index *)malloc((size_t)(n_src > 0 ? n_src : 1) * sizeof(Index));
+    if (!indeg || !seen || !hub_of) return ORC_EINVAL;
+    for (Index row = 0; row < R; ++row) {
+      if (hmap && hmap[row] != -1) continue;
+      for (Index j = ptr[row]; j < ptr[row + 1]; ++j) indeg[idx[j]]++;
+    }
+    for (Index s = 0; s < n_src; ++s) hub_of[s] = indeg[s] > chunk ? n_hubs++ : -1;
+    part = (float *)calloc((size_t)((n_hubs > 0 ? n_hubs : 1) * F), sizeof(float));
+    if (!part) return ORC_EINVAL;
+  }
   for (Index row = 0; row < R; ++row) {
     const float *gr = g + row * F;
     if (hmap && hmap[row] != -1) {
@@ -265,10 +285,21 @@ int orc_bwd_mean_row(const Index *ptr, const Index *idx, const float *g,
     int n = (int)(e - b);
     if (n == 0) continue;
     for (Index j = b; j < e; ++j) {
-      float *o = grads_out + idx[j] * F;
-      for (Index c = 0; c < F; ++c) o[c] += gr[c] / (float)n;
+      Index s = idx[j];
+      float *o = grads_out + s * F;
+      if (chunk > 0 && hub_of[s] >= 0) {
+        float *p = part + hub_of[s] * F;
+        for (Index c = 0; c < F; ++c) p[c] += gr[c] / (float)n;
+        seen[s]++;
+        if (seen[s] % chunk == 0 || seen[s] == indeg[s]) { /* chunk complete: fold it in */
+          for (Index c = 0; c < F; ++c) { o[c] += p[c]; p[c] = 0.0f; }
+        }
+      } else {
+        for (Index c = 0; c < F; ++c) o[c] += gr[c] / (float)n;
+      }
     }
   }
+  free(indeg); free(seen); free(hub_of); free(part);
   return ORC_OK;
 }
 
@@ -276,7 +307,7 @@ int orc_bwd_mean_row(const Index *ptr, const Index *idx, const float *g,
  * with respect to the substituted source row, whichever table it came from. */
 int orc_bwd_mean_src(const Index *ptr, const Index *idx, const float *g,
                      float *grad_src, Index R, Index F, Index n_src) {
-  return orc_bwd_mean_row(ptr, idx, g, NULL, grad_src, NULL, R, F, 0, n_src);
+  return orc_bwd_mean_row(ptr, idx, g, NULL, grad_src, NULL, R, F, 0, n_src, 0);
 }
 
 /* Follows gen_bwd_history_grad_v2_edge_value (:170-213) and its _edge_grad

@@ -128,7 +128,7 @@ def fwd_mean_src(ptr, idx, feat, hmap_src, hist, num_node=None, split_above=0):
     return out
 
 
-def bwd_mean_row(ptr, idx, g, hmap, n_src, hbuf_shape=None):
+def bwd_mean_row(ptr, idx, g, hmap, n_src, hbuf_shape=None, chunk=0):
     """Returns (grad_input[n_src,F], grad_history[R,hsize] or None)."""
     ptr, idx, g = _i64(ptr), _i64(idx), _f32(g)
     R, F = g.shape
@@ -140,12 +140,12 @@ def bwd_mean_row(ptr, idx, g, hmap, n_src, hbuf_shape=None):
         hsize = hbuf_shape[-1] if hbuf_shape is not None else F
         ghist = np.zeros((R, hsize), np.float32)
     _check(lib().orc_bwd_mean_row(_p(ptr), _p(idx), _p(g), _p(hmap), _p(gout), _p(ghist),
-                                  _I(R), _I(F), _I(hsize), _I(n_src)), "bwd_mean_row")
+                                  _I(R), _I(F), _I(hsize), _I(n_src), _I(chunk)), "bwd_mean_row")
     return gout, ghist
 
 
-def bwd_mean_src(ptr, idx, g, n_src):
-    return bwd_mean_row(ptr, idx, g, None, n_src)[0]
+def bwd_mean_src(ptr, idx, g, n_src, chunk=0):
+    return bwd_mean_row(ptr, idx, g, None, n_src, chunk=chunk)[0]
 
 
 def bwd_edge_value(ptr, idx, ev, g, hmap, vin, n_src, hsize=None, want_edge_grad=False):

@@ -210,7 +210,7 @@ def test_bwd_mean_bit_exact_and_deterministic(be, orc, R, N, F, maxdeg, hub, wit
         hmap, hbuf = None, None
         out = be.aggr_forward_history(x, T(ptr), T(idx), none(), none(), 0, R)
     out.backward(T(g))
-    gx, gh = orc.bwd_mean_row(ptr, idx, g, hmap, N, hbuf_shape=(R, F))
+    gx, gh = orc.bwd_mean_row(ptr, idx, g, hmap, N, hbuf_shape=(R, F), chunk=be.bwd_chunk_edges(F))
     np.testing.assert_array_equal(x.grad.cpu().numpy(), gx)
     if with_hist:
         np.testing.assert_array_equal(hbuf.grad.cpu().numpy(), gh)
@@ -221,6 +221,45 @@ def test_bwd_mean_bit_exact_and_deterministic(be, orc, R, N, F, maxdeg, hub, wit
                                    none() if hbuf is None else hbuf.detach(), 0 if hmap is None else F, R)
     out2.backward(T(g))
     assert torch.equal(first, x.grad)
+
+
+@pytest.mark.parametrize("with_hist", [False, True])
+def test_bwd_hub_sources_are_chunked(be, orc, with_hist):
+    """Sources with more than 512 incoming edges (hubs of a sampled batch) are summed in chunks by
+    independent waves: same bits as the oracle applying the documented chunk rule, 1e-5 from the
+    strictly ordered sum.  Includes a hub at the first and at the last source id, hubs next to each
+    other, sources without edges and a hub whose size is a multiple of the chunk."""
+    rng = np.random.default_rng(77)
+    R, N, F = 6000, 500, 128
+    deg = rng.integers(0, 8, size=R)
+    ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    E = int(ptr[-1])
+    idx = rng.integers(0, N, size=E, dtype=np.int64)
+    hubs = {0: 1700, 1: 513, 2: 1024, 250: 3000, N - 1: 2200}
+    pos = rng.permutation(E)
+    o = 0
+    for s_, k in hubs.items():
+        idx[pos[o:o + k]] = s_
+        o += k
+    idx[idx == 7] = 8                                            # source 7 has no edges at all
+    x = T(rng.standard_normal((N, F)).astype(np.float32)).requires_grad_(True)
+    g = rng.standard_normal((R, F)).astype(np.float32)
+    hmap = random_hmap(rng, R, 0.2) if with_hist else None
+    if with_hist:
+        hbuf = T(rng.standard_normal((R, F)).astype(np.float32)).requires_grad_(True)
+        out = be.aggr_forward_history(x, T(ptr), T(idx), T(hmap), hbuf, F, R)
+    else:
+        out = be.aggr_forward_history(x, T(ptr), T(idx), none(), none(), 0, R)
+    out.backward(T(g))
+    C = be.bwd_chunk_edges(F)
+    assert C == 512
+    ref, _ = orc.bwd_mean_row(ptr, idx, g, hmap, N, hbuf_shape=(R, F), chunk=C)
+    seq, _ = orc.bwd_mean_row(ptr, idx, g, hmap, N, hbuf_shape=(R, F))
+    got = x.grad.cpu().numpy()
+    np.testing.assert_array_equal(got, ref)
+    assert (ref != seq).any()
+    np.testing.assert_allclose(ref, seq, rtol=1e-4, atol=1e-5)
+    assert (got[7] == 0).all()
 
 
 def test_bwd_retain_grad_on_output_and_raw_feature_input(be, orc):
@@ -248,7 +287,7 @@ def test_src_mode_backward(be, orc):
     g = rng.standard_normal((R, F)).astype(np.float32)
     out = be.aggr_forward_source_history(feat, T(ptr), T(idx), T(hmap), hist)
     out.backward(T(g))
-    np.testing.assert_array_equal(feat.grad.cpu().numpy(), orc.bwd_mean_src(ptr, idx, g, N))
+    np.testing.assert_array_equal(feat.grad.cpu().numpy(), orc.bwd_mean_src(ptr, idx, g, N, chunk=be.bwd_chunk_edges(F)))
 
 
 @pytest.mark.parametrize("F,H", [(64, 1), (96, 1), (32, 3), (256, 2)])

@@ -246,3 +246,33 @@ def test_quarter_split_order(orc):
     sub[hm != -1] = hist[hm[hm != -1]]
     np.testing.assert_array_equal(orc.fwd_mean_src(ptr, idx, vin, hm, hist, split_above=8),
                                   orc.fwd_mean_row(ptr, idx, sub, None, None, split_above=8))
+
+
+def test_chunked_backward_order(orc):
+    """chunk > 0 restates the device order for hub sources: chunks of `chunk` incoming edges summed
+    from zero, chunk sums combined left to right.  Written out independently with NumPy float32."""
+    rng = np.random.default_rng(12)
+    R, N, F, C = 60, 6, 5, 8
+    deg = rng.integers(1, 5, size=R)
+    ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    idx = rng.integers(0, N, size=int(ptr[-1]), dtype=np.int64)
+    idx[idx == 4] = 5                                   # source 4 has no edges
+    g = rng.standard_normal((R, F)).astype(np.float32)
+    hmap = np.where(rng.random(R) < 0.2, 3, -1).astype(np.int64)
+    got, _ = orc.bwd_mean_row(ptr, idx, g, hmap, N, hbuf_shape=(R, F), chunk=C)
+    seq, _ = orc.bwd_mean_row(ptr, idx, g, hmap, N, hbuf_shape=(R, F))
+    dst = np.repeat(np.arange(R), deg)
+    for s in range(N):
+        es = [e for e in range(len(idx)) if idx[e] == s and hmap[dst[e]] == -1]
+        terms = [g[dst[e]] / np.float32(deg[dst[e]]) for e in es]
+        if len(es) <= C:
+            np.testing.assert_array_equal(got[s], seq[s])
+            continue
+        tot = None
+        for c0 in range(0, len(terms), C):
+            acc = np.zeros(F, np.float32)
+            for t in terms[c0:c0 + C]:
+                acc = acc + t
+            tot = acc if tot is None else tot + acc
+        np.testing.assert_array_equal(got[s], tot)
+    np.testing.assert_allclose(got, seq, rtol=1e-5, atol=1e-6)
