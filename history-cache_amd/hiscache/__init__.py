@@ -8,13 +8,14 @@ from hiscache_backend import count_history_reconstruct, get_graph_structure_scor
 
 from .feature_store import PinnedFeatureStore
 from .history_cache import HistoryCache
-from .history_model import HistorySAGE, MySageConvHistory, get_model
+from .history_model import (HistoryRGCN, HistorySAGE, MyRGCNConvHistory2, MySageConvHistory, get_model,
+                            typed_csr)
 from .history_table import HistoryTable
 from .ring_cache import RingHistoryCache
 from .util import Config, make_config, quantile_threshold
 
 __all__ = [
-    "HistoryCache", "HistoryTable", "RingHistoryCache", "HistorySAGE", "MySageConvHistory", "get_model",
+    "HistoryCache", "HistoryTable", "RingHistoryCache", "HistorySAGE", "HistoryRGCN", "MySageConvHistory", "MyRGCNConvHistory2", "typed_csr", "get_model",
     "PinnedFeatureStore", "Config", "make_config", "quantile_threshold",
     "count_history_reconstruct", "get_graph_structure_score", "record_history",
 ]

@@ -1,11 +1,13 @@
-"""GraphSAGE with a history-aware aggregation layer.
+"""GraphSAGE and RGCN with a history-aware aggregation layer.
 
-Same classes and forward wiring as the reference's SAGE path
-(/root/reference/hiscache/history_model.py:54-184): ``MySageConvHistory``, ``HistorySAGE`` and
-``get_model``.  Aggregation (with and without history) runs through ``hiscache_backend``; the
-dense layers are stock PyTorch.  The plain mean that the reference takes from
-``cxgnncomp.sage_mean_forward`` (history_model.py:90) is the same kernel with no history map.
-The RGCN / DGL wrappers depend on external operator libraries and are not part of this module.
+Same classes and forward wiring as the reference (/root/reference/hiscache/history_model.py):
+``MySageConvHistory`` / ``HistorySAGE`` (:54-184), ``MyRGCNConvHistory2`` / ``HistoryRGCN``
+(:220-431) and ``get_model`` (:446-470).  Aggregation (with and without history) runs through
+``hiscache_backend``; the dense layers are stock PyTorch.  The plain mean that the reference takes
+from ``cxgnncomp.sage_mean_forward`` (history_model.py:90) is the same kernel with no history map.
+The relational layer replaces ``cxgnncomp.RGCNOP_sorted`` (:266) by a typed gather-reduce -- the
+mean kernel over (row, relation) virtual rows -- followed by one GEMM; the result is the same
+quantity, sum_j x[src_j] @ W[rel_j] / deg.  The DGL wrapper is not part of this module.
 """
 import torch
 import torch.nn.functional as F
@@ -110,7 +112,165 @@ class HistorySAGE(torch.nn.Module):
             bn.reset_parameters()
 
 
-model_dict = {"sage": HistorySAGE}
+def typed_csr(ptr, idx, edge_types, num_rel, num_node, used_mask=None):
+    """Group the edges of the first ``num_node`` rows by (row, relation): returns (ptr2, idx2, cnt)
+    where ptr2 has num_node*num_rel+1 entries (virtual row r*num_rel+k holds row r's edges of relation
+    k, in their original order) and cnt[num_node, num_rel] the group sizes.  Edges whose source is
+    not in ``used_mask`` are dropped, as the reference drops them by giving them an extra relation
+    (/root/reference/hiscache/history_model.py:248-250)."""
+    num_edge = int(ptr[num_node])
+    deg = ptr[1:num_node + 1] - ptr[:num_node]
+    dst = torch.repeat_interleave(torch.arange(num_node, device=ptr.device), deg)
+    src = idx[:num_edge]
+    rel = edge_types[:num_edge].to(torch.int64)
+    key = dst * num_rel + rel
+    if used_mask is not None:
+        keep = used_mask[src]
+        key, src = key[keep], src[keep]
+    perm = torch.argsort(key, stable=True)
+    idx2 = src[perm].contiguous()
+    cnt = torch.bincount(key, minlength=num_node * num_rel)
+    ptr2 = torch.zeros(num_node * num_rel + 1, dtype=torch.int64, device=ptr.device)
+    torch.cumsum(cnt, 0, out=ptr2[1:])
+    return ptr2, idx2, cnt.view(num_node, num_rel), deg
+
+
+def edge_types_by_node_ranges(ptr, idx, sub_to_full, num_node, type_bounds, pair_to_rel):
+    """Relation of every edge of the first ``num_node`` rows from the node types of its ends; a node's
+    type is the range of ``type_bounds`` its full id falls into (mag240M stores papers, authors and
+    institutions in consecutive id ranges).  ``pair_to_rel[type(dst), type(src)]`` gives the relation.
+    Stands in for ``cxgnncomp_backend.gen_edge_type_mag240m``
+    (/root/reference/hiscache/history_model.py:356), whose exact numbering is not available here."""
+    num_edge = int(ptr[num_node])
+    deg = ptr[1:num_node + 1] - ptr[:num_node]
+    dst = torch.repeat_interleave(torch.arange(num_node, device=ptr.device), deg)
+    bounds = torch.as_tensor(type_bounds, dtype=torch.int64, device=ptr.device)
+    t_dst = torch.bucketize(sub_to_full[dst], bounds, right=True)
+    t_src = torch.bucketize(sub_to_full[idx[:num_edge]], bounds, right=True)
+    table = torch.as_tensor(pair_to_rel, dtype=torch.int64, device=ptr.device)
+    return table[t_dst, t_src]
+
+
+class MyRGCNConvHistory2(torch.nn.Module):
+    """Relational convolution with history substitution: out[r] = sum_j x[src_j] @ W[rel_j] / deg(r),
+    rows with a cached embedding take it instead
+    (/root/reference/hiscache/history_model.py:220-278)."""
+
+    def __init__(self, in_channels, hidden_channels, num_rel, need_grad):
+        super().__init__()
+        self.in_channels = in_channels
+        self.hidden_channels = hidden_channels
+        self.num_rel = num_rel
+        self.linear = torch.nn.Parameter(torch.empty(num_rel, in_channels, hidden_channels))
+        self.reset_parameters()
+        self.need_grad = need_grad
+
+    def reset_parameters(self):
+        # glorot, as torch_geometric.nn.inits.glorot does for a [K, in, out] weight
+        bound = (6.0 / (self.linear.size(-2) + self.linear.size(-1))) ** 0.5
+        torch.nn.init.uniform_(self.linear, -bound, bound)
+
+    def forward(self, x, ptr, idx, edge_types, count, history_map, history_buffer, used_mask, history_size,
+                num_node):
+        num_node = int(num_node)
+        K = self.num_rel
+        ptr2, idx2, cnt, deg = typed_csr(ptr, idx, edge_types, K, num_node, used_mask)
+        # per-relation edge counts, as the reference takes them (history_model.py:260)
+        self.last_count = hiscache_backend.count_num(edge_types[: int(ptr[num_node])].to(torch.int64).contiguous(), K)
+        none = torch.empty(0, device=x.device)
+        # mean over every (row, relation) group; cnt/deg turns the group means into the row's share
+        agg = hiscache_backend.aggr_forward_history(x, ptr2, idx2, none, none, 0, num_node * K)
+        scale = cnt.to(torch.float32) / deg.clamp(min=1).to(torch.float32)[:, None]
+        agg = agg.view(num_node, K, -1) * scale[:, :, None]
+        out = agg.reshape(num_node, -1) @ self.linear.reshape(K * self.in_channels, self.hidden_channels)
+        if history_size > 0:
+            hit = (history_map[:num_node] != -1)[:, None]
+            out = torch.where(hit, history_buffer[:num_node].to(out.dtype), out)
+        his = out
+        if self.need_grad and self.training and history_size > 0:
+            his.retain_grad()
+        return out, his
+
+
+MyRGCNConvHistory = MyRGCNConvHistory2
+
+
+class HistoryRGCN(torch.nn.Module):
+    """Forward wiring of /root/reference/hiscache/history_model.py:329-431."""
+
+    def __init__(self, in_channels, hidden_channels, out_channels, num_layers, dropout, graph_type, config,
+                 table, **kwargs):
+        super().__init__()
+        self.in_channels = in_channels
+        self.hidden_channels = hidden_channels
+        self.out_channels = out_channels
+        self.graph_type = graph_type
+        self.bns = torch.nn.ModuleList()
+        self.num_layers = num_layers
+        for _ in range(self.num_layers - 1):
+            self.bns.append(torch.nn.BatchNorm1d(hidden_channels))
+        self.dropout = dropout
+        self.table = table
+        self.num_rel = kwargs["num_rel"]
+        self.dataset_name = kwargs.get("dataset_name", "")
+        self.gen_rel = self.dataset_name == "rmag240m"
+        if self.gen_rel:
+            self.num_rel = 5
+        # node-type id ranges and the (dst type, src type) -> relation table used when gen_rel
+        self.type_bounds = kwargs.get("type_bounds")
+        self.pair_to_rel = kwargs.get("pair_to_rel")
+        need_grad = self.table.method == "grad"
+        self.convs = torch.nn.ModuleList()
+        self.convs.append(MyRGCNConvHistory2(in_channels, hidden_channels, self.num_rel, need_grad))
+        for _ in range(self.num_layers - 2):
+            self.convs.append(MyRGCNConvHistory2(hidden_channels, hidden_channels, self.num_rel, need_grad))
+        if self.num_layers > 1:
+            self.last_layer_history = False
+            self.convs.append(MyRGCNConvHistory2(hidden_channels, out_channels, self.num_rel, need_grad))
+
+    def edge_types(self, batch):
+        L = self.num_layers
+        if getattr(batch, "edge_type", None) is not None:
+            return batch.edge_type
+        if self.gen_rel and self.type_bounds is not None:
+            return edge_types_by_node_ranges(batch.ptr, batch.idx, batch.sub_to_full,
+                                             int(batch.num_node_in_layer[L - 1]), self.type_bounds,
+                                             self.pair_to_rel)
+        return torch.randint(0, self.num_rel, (batch.num_edge_in_layer[L - 1],), device=batch.ptr.device)
+
+    def forward(self, batch):
+        x = batch.x
+        L = self.num_layers
+        etypes = self.edge_types(batch)
+        none = torch.empty(0, device=x.device)
+        masks = self.table.used_masks
+        for i, conv in enumerate(self.convs[:-1]):
+            n = batch.num_node_in_layer[L - 1 - i]
+            et = etypes[: batch.num_edge_in_layer[L - 1 - i]]
+            um = masks[i] if masks is not None else None
+            if self.training and i == L - 2:
+                x, his = conv(x, batch.ptr, batch.idx, et, None, self.table.sub2embed,
+                              self.table.cached_embedding, um, self.hidden_channels, n)
+                self.table.produced_embedding = his
+                self.table.produced_embedding.retain_grad()
+            else:
+                x, his = conv(x, batch.ptr, batch.idx, et, None, none, none, um, 0, n)
+            x = self.bns[i](x)
+            x = F.relu(x)
+            x = F.dropout(x, p=self.dropout, training=self.training)
+        um = masks[-2] if masks is not None else None
+        x, his = self.convs[-1](x, batch.ptr, batch.idx, etypes[: batch.num_edge_in_layer[0]], None, none, none,
+                                um, 0, batch.num_node_in_layer[0])
+        return x.log_softmax(dim=-1)
+
+    def reset_parameters(self):
+        for conv in self.convs:
+            conv.reset_parameters()
+        for bn in self.bns:
+            bn.reset_parameters()
+
+
+model_dict = {"sage": HistorySAGE, "rgcn": HistoryRGCN}
 graph_type_dict = {"cxg": "CSR_Layer", "dgl": "DGL"}
 
 
@@ -118,7 +278,13 @@ def get_model(config, table):
     """Model factory with the reference's signature (/root/reference/hiscache/history_model.py:446-470)."""
     mtype = config.train.model.type.lower()
     if mtype not in model_dict:
-        raise NotImplementedError(f"model type {mtype!r}: only the SAGE path is provided")
+        raise NotImplementedError(f"model type {mtype!r}: sage and rgcn are provided")
+    if mtype == "rgcn":
+        return HistoryRGCN(config.dl.dataset.feature_dim, config.train.model.hidden_dim,
+                           config.dl.dataset.num_classes, config.train.model.num_layers,
+                           config.train.model.dropout, graph_type_dict[config.train.type.lower()], config,
+                           table, num_rel=config.train.model.num_rel,
+                           dataset_name=config.dl.dataset.name.lower())
     return model_dict[mtype](config.dl.dataset.feature_dim, config.train.model.hidden_dim,
                              config.dl.dataset.num_classes, config.train.model.num_layers,
                              config.train.model.dropout, graph_type_dict[config.train.type.lower()],

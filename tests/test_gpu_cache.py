@@ -363,3 +363,95 @@ def test_input_layer_backward_is_skipped_but_history_grad_is_kept():
     out.backward(t(g))
     assert x.grad is None
     np.testing.assert_array_equal(hb.grad.cpu().numpy(), orc.bwd_mean_row(ptr, idx, g, hmap, N, (R, F))[1])
+
+
+def rgcn_layer_cpu(x, W, ptr, idx, rel, used, n, hit=None, hbuf=None):
+    """sum_j x[src_j] @ W[rel_j] / deg over the first n rows, unused sources dropped, in fp64."""
+    deg = (ptr[1:n + 1] - ptr[:n])
+    E = int(ptr[n])
+    dst = torch.repeat_interleave(torch.arange(n), deg)
+    src = idx[:E]
+    msg = torch.einsum("ef,efh->eh", x[src].double(), W.double()[rel[:E]])
+    if used is not None:
+        msg = msg * used[src][:, None]
+    out = torch.zeros(n, W.shape[2], dtype=torch.float64).index_add(0, dst, msg)
+    out = out / deg.clamp(min=1)[:, None]
+    if hit is not None:
+        out = torch.where(hit[:, None], hbuf.double(), out)
+    return out
+
+
+@pytest.mark.parametrize("feat_dtype", [torch.float32, torch.float16])
+def test_rgcn_typed_aggregation_matches_dense_cpu(feat_dtype):
+    """HistoryRGCN (typed gather-reduce over (row, relation) groups + one GEMM) against a dense fp64
+    statement of sum_j x[src_j] @ W[rel_j] / deg with history substitution; gradients too."""
+    from hiscache import HistoryRGCN, PinnedFeatureStore, RingHistoryCache, make_config
+    from hiscache.synthetic import make_batch
+    rng = np.random.default_rng(8)
+    torch.manual_seed(1)
+    N, Fin, H, C, K, L = 3000, 128, 64, 6, 5, 2
+    feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32)).to(feat_dtype)
+    cache = RingHistoryCache(PinnedFeatureStore(feats, device=DEV), N, Fin, H, capacity=800, num_layers=L,
+                             table_dtype=torch.float32, thres=0.5, device=DEV)
+    pre = torch.from_numpy(rng.choice(N, size=700, replace=False)).to(DEV)
+    cache.preload(pre, torch.randn(700, H, device=DEV))
+    cfg = make_config(Fin, C, H, L, device=DEV, model_type="rgcn", num_rel=K)
+    model = HistoryRGCN(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache, num_rel=K).to(DEV)
+    model.train()
+    b = layered_batch(rng, N, 40, [6, 4])
+    batch = make_batch(b, rng.integers(0, C, size=N), DEV)
+    batch.edge_type = torch.from_numpy(rng.integers(0, K, size=len(b["idx"]))).to(DEV)
+    cache.lookup_and_load(batch, L)
+    out = model(batch)
+    loss = torch.nn.functional.nll_loss(out, batch.y)
+    loss.backward()
+    # the same network in fp64 on the CPU
+    nnl = b["num_node_in_layer"]
+    ptr, idx = torch.from_numpy(b["ptr"]), torch.from_numpy(b["idx"])
+    rel = batch.edge_type.cpu()
+    used = [m.cpu() for m in cache.used_masks]
+    x0 = batch.x.cpu()
+    W0 = model.convs[0].linear.detach().cpu().double().requires_grad_(True)
+    W1 = model.convs[1].linear.detach().cpu().double().requires_grad_(True)
+    n1, n0 = int(nnl[1]), int(nnl[0])
+    hit = cache.sub2embed.cpu() != -1
+    assert hit.any() and (~hit).any() and (~used[0]).any()
+    h1 = rgcn_layer_cpu(x0, W0, ptr, idx, rel, used[0].double(), n1, hit, cache.cached_embedding.cpu())
+    h1.retain_grad()
+    bn = model.bns[0]
+    mu, var = h1.mean(0), h1.var(0, unbiased=False)
+    z = (h1 - mu) / torch.sqrt(var + bn.eps) * bn.weight.detach().cpu().double() + bn.bias.detach().cpu().double()
+    z = torch.relu(z)
+    o = rgcn_layer_cpu(z, W1, ptr, idx, rel, used[-2].double(), n0).log_softmax(dim=-1)
+    loss_c = torch.nn.functional.nll_loss(o, batch.y.cpu())
+    loss_c.backward()
+    tol = 2e-3 if feat_dtype == torch.float16 else 2e-4
+    np.testing.assert_allclose(out.detach().cpu().numpy(), o.detach().numpy(), rtol=tol, atol=tol)
+    pe = cache.produced_embedding
+    gs = float(h1.grad.abs().max())
+    np.testing.assert_allclose(pe.grad.cpu().numpy(), h1.grad.numpy(), rtol=1e-2, atol=tol * gs)
+    for got, ref in ((model.convs[0].linear.grad, W0.grad), (model.convs[1].linear.grad, W1.grad)):
+        s = float(ref.abs().max())
+        np.testing.assert_allclose(got.cpu().numpy(), ref.numpy(), rtol=1e-2, atol=tol * s)
+    cache.update_history(batch, 1)
+    assert cache.last_record_mask.shape[0] == n1
+
+
+def test_typed_csr_groups_edges_by_row_and_relation():
+    from hiscache import typed_csr
+    from helpers import random_csr
+    rng = np.random.default_rng(9)
+    R, N, K = 50, 40, 4
+    ptr, idx = random_csr(rng, R + 10, N, 7)           # deeper-layer rows beyond the first R
+    rel = rng.integers(0, K, size=len(idx))
+    used = rng.random(N) < 0.8
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    ptr2, idx2, cnt, deg = typed_csr(t(ptr), t(idx), t(rel), K, R, t(used))
+    ptr2, idx2, cnt = ptr2.cpu().numpy(), idx2.cpu().numpy(), cnt.cpu().numpy()
+    np.testing.assert_array_equal(deg.cpu().numpy(), np.diff(ptr)[:R])
+    for r in range(R):
+        for k in range(K):
+            e = [j for j in range(ptr[r], ptr[r + 1]) if rel[j] == k and used[idx[j]]]
+            v = r * K + k
+            np.testing.assert_array_equal(idx2[ptr2[v]:ptr2[v + 1]], idx[e])
+            assert cnt[r, k] == len(e)
