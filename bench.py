@@ -11,7 +11,7 @@ Prints ONE JSON line: edges/s over the whole step, the roofline of the dominant 
 gather, timed with HIP events on the launch stream) and a CPU baseline (the same semantics written
 with PyTorch CPU index_add, timed on this machine's host cores on a 1/10-size sample).
 
-Other workloads (--workload c4 | c2row | c3) print their own line and are not the headline.
+Other workloads (--workload c4 | c2row | c3 | c5) print their own line and are not the headline.
 """
 import argparse
 import json
@@ -34,7 +34,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c4", "c3", "copy"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c4", "c3", "c5", "copy"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
@@ -437,6 +437,102 @@ def run_c3(args):
     }
 
 
+# ----------------------------------------------------------------------------------------- C5
+def run_c5(args):
+    """mag240M-shaped heterogeneous RGCN iteration: one GPU's share at its real batch shape."""
+    import numpy as np
+    import torch
+
+    from hiscache import HistoryRGCN, PinnedFeatureStore, RingHistoryCache, make_config
+    from hiscache.synthetic import direct_power_law_batch, make_batch
+
+    dev = "cuda:0"
+    s = args.scale
+    n_paper, n_author, n_inst = int(122_000_000 * s), int(122_000_000 * s), max(1, int(26_000 * s))
+    N = n_paper + n_author + n_inst
+    Fin, H, C, K, L = 768, 256, 153, 5, 2
+    fanout, n_seed = [25, 15], 1000
+    pool_rows = min(N, 4_000_000)
+
+    class PooledStore(PinnedFeatureStore):
+        def get(self, ids):
+            return super().get(ids % pool_rows)
+
+        def masked_get(self, ids, mask):
+            return super().masked_get(ids % pool_rows, mask)
+
+        def masked_get_async(self, ids, mask):
+            return super().masked_get_async(ids % pool_rows, mask)
+
+    gen = torch.Generator(device=dev).manual_seed(5)
+    pinned = torch.empty((pool_rows, Fin), dtype=torch.float16, pin_memory=True)
+    chunk = 500_000
+    for lo in range(0, pool_rows, chunk):
+        hi = min(pool_rows, lo + chunk)
+        pinned[lo:hi].copy_(torch.randn(hi - lo, Fin, device=dev, generator=gen).half())
+    store = PooledStore(pinned, device=dev, out_dtype=torch.float16)
+    cache = RingHistoryCache(store, N, Fin, H, capacity=N, num_layers=L, table_dtype=torch.float16, thres=0.05,
+                             age_limit=200, device=dev)
+    hit = torch.nonzero(torch.rand(N, device=dev, generator=gen) < 0.35).view(-1)
+    cache.preload(hit)
+    del hit
+    cfg = make_config(Fin, C, H, L, device=dev, model_type="rgcn", num_rel=K, name="rmag240m")
+    torch.manual_seed(5)
+    # relation of an edge from the node types of (destination, source): paper-cites-paper,
+    # paper<-author, author<-paper, author<-institution, institution<-author
+    pair_to_rel = [[0, 1, 0], [2, 0, 3], [0, 4, 0]]
+    model = HistoryRGCN(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache, num_rel=K, dataset_name="rmag240m",
+                        type_bounds=[n_paper, n_paper + n_author], pair_to_rel=pair_to_rel).to(dev)
+    model.train()
+    opt = torch.optim.Adam(model.parameters(), lr=1e-3)
+
+    class FoldedLabels:
+        base = np.random.default_rng(5).integers(0, C, size=1 << 20)
+
+        def __getitem__(self, ids):
+            return self.base[np.asarray(ids) % self.base.size]
+
+    n_pre = 8
+    samples = [direct_power_law_batch(N, n_seed, fanout, 2.0, 50 + i, degree_scale=1.25) for i in range(n_pre)]
+    batches = [make_batch(smp, FoldedLabels(), dev) for smp in samples]
+    ev = {k: KernelClock() for k in ("load", "forward", "backward", "step", "update")}
+    state = {"it": 0}
+
+    def step():
+        b = batches[state["it"] % n_pre]
+        state["it"] += 1
+        ev["load"](lambda: cache.lookup_and_load(b, L))
+        out = ev["forward"](lambda: model(b))
+        loss = torch.nn.functional.nll_loss(out, b.y)
+        opt.zero_grad(set_to_none=True)
+        ev["backward"](lambda: loss.backward())
+        ev["step"](lambda: opt.step())
+        ev["update"](lambda: cache.update_history(b, state["it"]))
+
+    for _ in range(args.warmup):
+        step()
+    sync()
+    for c in ev.values():
+        c.reset()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    sync()
+    sec = (time.perf_counter() - t0) / args.steps
+    shape = {k: int(np.mean([int(x["num_node_in_layer"][i]) for x in samples])) for i, k in enumerate(("n0", "n1", "n2"))}
+    shape["edges"] = int(np.mean([x["idx"].size for x in samples]))
+    return {
+        "metric": "mag240M-shaped RGCN iteration ms (1 GPU)", "value": sec * 1e3, "unit": "ms", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "c5: mag240M-shaped, %d nodes of 3 types, 5 relations from node-type pairs, 2-layer RGCN "
+                               "hidden 256, fanout [25,15], batch 1000, fp16 history table %d x 256 (about 35%% cached), "
+                               "features 768-dim fp16 in a pinned host pool of %d rows read zero-copy; mean batch %s"
+                               % (N, N, pool_rows, shape)},
+        "phases_ms": {k: c.mean_ms() for k, c in ev.items()},
+    }
+
+
 def run_copy(args):
     """Plain device copy of known size: the calibration point for the HBM traffic counters."""
     import torch
@@ -470,6 +566,8 @@ def main():
         res = run_c4(args)
     elif args.workload == "copy":
         res = run_copy(args)
+    elif args.workload == "c5":
+        res = run_c5(args)
     else:
         res = run_c3(args)
     print(json.dumps(res))

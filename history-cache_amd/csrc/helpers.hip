@@ -106,18 +106,19 @@ __global__ __launch_bounds__(HC_BLOCK) void structure_seed(int64_t *__restrict__
 }
 
 // dst[i,:] = (mask == NULL || mask[i]) ? src[ids[i],:] : 0  (optionally accumulated).
-// Wave per output row; 16-byte loads when the row allows.  src may be mapped host memory.
-template <typename T>
-__global__ __launch_bounds__(HC_BLOCK) void gather_rows_kernel(const T *__restrict__ src, int64_t n_rows,
+// Wave per output row; 4 elements per lane per step when the row allows.  src may be mapped host
+// memory.  TS / TD are the element types of the source table and of the destination.
+template <typename TS, typename TD>
+__global__ __launch_bounds__(HC_BLOCK) void gather_rows_kernel(const TS *__restrict__ src, int64_t n_rows,
                                                                 const int64_t *__restrict__ ids,
                                                                 const uint8_t *__restrict__ mask,
-                                                                float *__restrict__ dst, int accumulate,
+                                                                TD *__restrict__ dst, int accumulate,
                                                                 int64_t n, int64_t F) {
-  constexpr int V = 16 / (int)sizeof(T) > 4 ? 4 : 16 / (int)sizeof(T);  // 4 elements per lane
+  constexpr int V = 4;
   const int lane = hc_lane();
   const int64_t i = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
   if (i >= n) return;
-  float *__restrict__ o = dst + i * F;
+  TD *__restrict__ o = dst + i * F;
   bool take = mask == nullptr || mask[i] != 0;
   int64_t id = 0;
   if (take) {
@@ -125,31 +126,31 @@ __global__ __launch_bounds__(HC_BLOCK) void gather_rows_kernel(const T *__restri
     if (id < 0) id += n_rows;
     if (id < 0 || id >= n_rows) take = false;
   }
-  const T *__restrict__ s = src + id * F;
-  const bool vec_ok = (F % V == 0) && (reinterpret_cast<uintptr_t>(s) % (sizeof(T) * V) == 0) &&
-                      (reinterpret_cast<uintptr_t>(o) % 16 == 0);
+  const TS *__restrict__ s = src + id * F;
+  const bool vec_ok = (F % V == 0) && (reinterpret_cast<uintptr_t>(s) % (sizeof(TS) * V) == 0) &&
+                      (reinterpret_cast<uintptr_t>(o) % (sizeof(TD) * V) == 0);
   if (vec_ok) {
     for (int64_t c = (int64_t)lane * V; c < F; c += HC_WAVE * V) {
       float v[V];
       if (take) {
-        hc_vec<T, V>::load(s + c, v);
+        hc_vec<TS, V>::load(s + c, v);
       } else {
 #pragma unroll
         for (int k = 0; k < V; ++k) v[k] = 0.0f;
       }
       if (accumulate) {
         float old[V];
-        hc_vec<float, V>::load(o + c, old);
+        hc_vec<TD, V>::load(o + c, old);
 #pragma unroll
         for (int k = 0; k < V; ++k) v[k] = old[k] + v[k];
       }
-      hc_vec<float, V>::store(o + c, v);
+      hc_vec<TD, V>::store(o + c, v);
     }
   } else {
     for (int64_t c = lane; c < F; c += HC_WAVE) {
-      float v = take ? hc_to_f32<T>(s[c]) : 0.0f;
-      if (accumulate) v = o[c] + v;
-      o[c] = v;
+      float v = take ? hc_to_f32<TS>(s[c]) : 0.0f;
+      if (accumulate) v = hc_to_f32<TD>(o[c]) + v;
+      o[c] = hc_from_f32<TD>(v);
     }
   }
 }
@@ -259,27 +260,34 @@ extern "C" int hc_structure_score(const int64_t *ptr, const int64_t *idx, int64_
   return HC_OK;
 }
 
+template <typename TS>
+int launch_gather(const void *src, int64_t n_rows, const int64_t *ids, const uint8_t *mask, void *dst,
+                  int dst_dtype, int accumulate, int64_t n, int64_t F, dim3 g, dim3 bl, hipStream_t st) {
+  const TS *s = static_cast<const TS *>(src);
+  if (dst_dtype == HC_F32)
+    gather_rows_kernel<TS, float><<<g, bl, 0, st>>>(s, n_rows, ids, mask, static_cast<float *>(dst), accumulate, n, F);
+  else if (dst_dtype == HC_F16)
+    gather_rows_kernel<TS, __half><<<g, bl, 0, st>>>(s, n_rows, ids, mask, static_cast<__half *>(dst), accumulate, n, F);
+  else
+    gather_rows_kernel<TS, __hip_bfloat16><<<g, bl, 0, st>>>(s, n_rows, ids, mask, static_cast<__hip_bfloat16 *>(dst),
+                                                             accumulate, n, F);
+  return hc_launch_status();
+}
+
 extern "C" int hc_gather_rows(const void *src, int src_dtype, int64_t n_rows, const int64_t *ids,
-                              const uint8_t *mask, float *dst, int accumulate, int64_t n, int64_t F,
-                              void *stream) {
+                              const uint8_t *mask, void *dst, int dst_dtype, int accumulate, int64_t n,
+                              int64_t F, void *stream) {
   HC_REQUIRE(n >= 0 && F > 0 && n_rows >= 0);
-  if (src_dtype < HC_F32 || src_dtype > HC_BF16) return HC_EDTYPE;
+  if (src_dtype < HC_F32 || src_dtype > HC_BF16 || dst_dtype < HC_F32 || dst_dtype > HC_BF16) return HC_EDTYPE;
   if (n == 0) return HC_OK;
   HC_REQUIRE(ids && dst && (src || n_rows == 0));
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int64_t b = (n + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
   if (!hc_grid_ok(b)) return HC_EUNSUPPORTED;
   dim3 g((unsigned)b), bl(HC_BLOCK);
-  if (src_dtype == HC_F32)
-    gather_rows_kernel<float><<<g, bl, 0, st>>>(static_cast<const float *>(src), n_rows, ids, mask, dst,
-                                                accumulate, n, F);
-  else if (src_dtype == HC_F16)
-    gather_rows_kernel<__half><<<g, bl, 0, st>>>(static_cast<const __half *>(src), n_rows, ids, mask,
-                                                 dst, accumulate, n, F);
-  else
-    gather_rows_kernel<__hip_bfloat16><<<g, bl, 0, st>>>(static_cast<const __hip_bfloat16 *>(src),
-                                                         n_rows, ids, mask, dst, accumulate, n, F);
-  return hc_launch_status();
+  if (src_dtype == HC_F32) return launch_gather<float>(src, n_rows, ids, mask, dst, dst_dtype, accumulate, n, F, g, bl, st);
+  if (src_dtype == HC_F16) return launch_gather<__half>(src, n_rows, ids, mask, dst, dst_dtype, accumulate, n, F, g, bl, st);
+  return launch_gather<__hip_bfloat16>(src, n_rows, ids, mask, dst, dst_dtype, accumulate, n, F, g, bl, st);
 }
 
 extern "C" int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset,

@@ -12,7 +12,10 @@ import hiscache_backend as _be
 
 class PinnedFeatureStore:
 
-    def __init__(self, features, device="cuda:0"):
+    def __init__(self, features, device="cuda:0", out_dtype=torch.float32):
+        # out_dtype: element type of the gathered rows (keep torch.float16 for fp16 feature files to
+        # halve the traffic of the first aggregation layer)
+        self.out_dtype = out_dtype
         if features.dim() != 2:
             raise ValueError("features must be [num_nodes, feature_dim]")
         if features.is_cuda:
@@ -35,10 +38,10 @@ class PinnedFeatureStore:
         return self._side
 
     def get(self, ids):
-        return _be.gather_rows(self.buffer, ids)
+        return _be.gather_rows(self.buffer, ids, out_dtype=self.out_dtype)
 
     def masked_get(self, ids, mask):
-        return _be.gather_rows(self.buffer, ids, mask=mask)
+        return _be.gather_rows(self.buffer, ids, mask=mask, out_dtype=self.out_dtype)
 
     def masked_get_async(self, ids, mask):
         """Start the gather on a side stream (default priority) that first waits for the work
@@ -48,7 +51,7 @@ class PinnedFeatureStore:
         side = self._side_stream()
         side.wait_stream(cur)
         with torch.cuda.stream(side):
-            out = _be.gather_rows(self.buffer, ids, mask=mask)
+            out = _be.gather_rows(self.buffer, ids, mask=mask, out_dtype=self.out_dtype)
             self._done.record(side)
         out.record_stream(cur)
         return out, self._done

@@ -113,26 +113,32 @@ class HistorySAGE(torch.nn.Module):
 
 
 def typed_csr(ptr, idx, edge_types, num_rel, num_node, used_mask=None):
-    """Group the edges of the first ``num_node`` rows by (row, relation): returns (ptr2, idx2, cnt)
-    where ptr2 has num_node*num_rel+1 entries (virtual row r*num_rel+k holds row r's edges of relation
-    k, in their original order) and cnt[num_node, num_rel] the group sizes.  Edges whose source is
+    """Group the edges of the first ``num_node`` rows by (row, relation): returns (ptr2, idx2, cnt, deg)
+    where virtual row r*num_rel+k of (ptr2, idx2) holds row r's edges of relation k in their original
+    order, cnt[num_node, num_rel] are the group sizes and deg[num_node] the full row degrees.
+    ``edge_types`` covers at least the edges of those rows (it may be longer).  Edges whose source is
     not in ``used_mask`` are dropped, as the reference drops them by giving them an extra relation
-    (/root/reference/hiscache/history_model.py:248-250)."""
-    num_edge = int(ptr[num_node])
+    (/root/reference/hiscache/history_model.py:248-250).  Dropped and surplus edges are parked in one
+    extra group behind the last virtual row, so nothing is compacted and no device value is read
+    back; ptr2 therefore has num_node*num_rel+2 entries and callers aggregate num_node*num_rel rows."""
+    num_edge = min(int(edge_types.shape[0]), int(idx.shape[0]))
+    dev = ptr.device
     deg = ptr[1:num_node + 1] - ptr[:num_node]
-    dst = torch.repeat_interleave(torch.arange(num_node, device=ptr.device), deg)
+    e = torch.arange(num_edge, device=dev)
+    dst = torch.searchsorted(ptr[1:num_node + 1].contiguous(), e, right=True)   # row of every edge slot
     src = idx[:num_edge]
     rel = edge_types[:num_edge].to(torch.int64)
-    key = dst * num_rel + rel
+    ok = (dst < num_node) & (rel >= 0) & (rel < num_rel)
     if used_mask is not None:
-        keep = used_mask[src]
-        key, src = key[keep], src[keep]
+        ok = ok & used_mask[src]
+    trash = num_node * num_rel
+    key = torch.where(ok, dst * num_rel + rel, torch.full_like(dst, trash))
     perm = torch.argsort(key, stable=True)
     idx2 = src[perm].contiguous()
-    cnt = torch.bincount(key, minlength=num_node * num_rel)
-    ptr2 = torch.zeros(num_node * num_rel + 1, dtype=torch.int64, device=ptr.device)
+    cnt = torch.zeros(trash + 1, dtype=torch.int64, device=dev).index_add_(0, key, torch.ones_like(key))
+    ptr2 = torch.zeros(trash + 2, dtype=torch.int64, device=dev)
     torch.cumsum(cnt, 0, out=ptr2[1:])
-    return ptr2, idx2, cnt.view(num_node, num_rel), deg
+    return ptr2, idx2, cnt[:trash].view(num_node, num_rel), deg
 
 
 def edge_types_by_node_ranges(ptr, idx, sub_to_full, num_node, type_bounds, pair_to_rel):
@@ -141,9 +147,9 @@ def edge_types_by_node_ranges(ptr, idx, sub_to_full, num_node, type_bounds, pair
     institutions in consecutive id ranges).  ``pair_to_rel[type(dst), type(src)]`` gives the relation.
     Stands in for ``cxgnncomp_backend.gen_edge_type_mag240m``
     (/root/reference/hiscache/history_model.py:356), whose exact numbering is not available here."""
-    num_edge = int(ptr[num_node])
-    deg = ptr[1:num_node + 1] - ptr[:num_node]
-    dst = torch.repeat_interleave(torch.arange(num_node, device=ptr.device), deg)
+    num_edge = int(idx.shape[0])
+    e = torch.arange(num_edge, device=ptr.device)
+    dst = torch.searchsorted(ptr[1:num_node + 1].contiguous(), e, right=True).clamp(max=num_node - 1)
     bounds = torch.as_tensor(type_bounds, dtype=torch.int64, device=ptr.device)
     t_dst = torch.bucketize(sub_to_full[dst], bounds, right=True)
     t_src = torch.bucketize(sub_to_full[idx[:num_edge]], bounds, right=True)
@@ -176,7 +182,7 @@ class MyRGCNConvHistory2(torch.nn.Module):
         K = self.num_rel
         ptr2, idx2, cnt, deg = typed_csr(ptr, idx, edge_types, K, num_node, used_mask)
         # per-relation edge counts, as the reference takes them (history_model.py:260)
-        self.last_count = hiscache_backend.count_num(edge_types[: int(ptr[num_node])].to(torch.int64).contiguous(), K)
+        self.last_count = hiscache_backend.count_num(edge_types.to(torch.int64).contiguous(), K)
         none = torch.empty(0, device=x.device)
         # mean over every (row, relation) group; cnt/deg turns the group means into the row's share
         agg = hiscache_backend.aggr_forward_history(x, ptr2, idx2, none, none, 0, num_node * K)

@@ -62,7 +62,7 @@ _SIGNATURES = {
                                  _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_sz, _c_p]),
     "hc_count_num": (_c_int, [_c_p, _c_i64, _c_i64, _c_p, _c_p]),
     "hc_structure_score": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p]),
-    "hc_gather_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_i64, _c_p]),
+    "hc_gather_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p]),
 }
 
@@ -534,9 +534,10 @@ def cache_append(score, thres, emb, sub2embed, sub_to_full, buffer, hidden, in_c
     return mask.view(torch.bool)
 
 
-def gather_rows(src, ids, mask=None, out=None, accumulate=False):
-    """out[i] = src[ids[i]] where mask[i] (else 0), as fp32.  ``src`` may be a GPU tensor or a
-    pinned host tensor (read zero-copy over the host link).  Negative ids index from the end."""
+def gather_rows(src, ids, mask=None, out=None, accumulate=False, out_dtype=torch.float32):
+    """out[i] = src[ids[i]] where mask[i] (else 0), as ``out_dtype`` (fp32 by default).  ``src`` may be
+    a GPU tensor or a pinned host tensor (read zero-copy over the host link).  Negative ids index
+    from the end."""
     lib = load_library()
     if not isinstance(src, torch.Tensor) or src.dim() != 2 or not src.is_contiguous():
         raise ValueError("src must be a contiguous 2-D tensor")
@@ -551,13 +552,13 @@ def gather_rows(src, ids, mask=None, out=None, accumulate=False):
     if out is None:
         if accumulate:
             raise ValueError("accumulate needs an existing out tensor")
-        out = torch.empty((n, F), dtype=torch.float32, device=ids.device)
+        out = torch.empty((n, F), dtype=out_dtype, device=ids.device)
     else:
-        _dev(out, "out", torch.float32)
+        _dev(out, "out")
         if tuple(out.shape) != (n, F):
             raise ValueError("out must be [len(ids), F]")
     rc = lib.hc_gather_rows(_ptr(src), _float_dtype(src, "src"), src.shape[0], _ptr(ids), _ptr(mask),
-                            _ptr(out), 1 if accumulate else 0, n, F, _stream())
+                            _ptr(out), _float_dtype(out, "out"), 1 if accumulate else 0, n, F, _stream())
     _check(rc, "hc_gather_rows")
     return out
 

@@ -239,10 +239,10 @@ int hc_structure_score(const int64_t *ptr, const int64_t *idx, int64_t ptr_rows,
  * addresses from the end (-1 = last row), as the torch indexing it replaces
  * does (hiscache/history_cache.py:312-313,345-350).  src may be device memory
  * or pinned, mapped host memory (zero-copy read over the host link); dst is
- * fp32 [n, F]; src is [n_rows, F] of src_dtype. */
+ * [n, F] of dst_dtype; src is [n_rows, F] of src_dtype. */
 int hc_gather_rows(const void *src, int src_dtype, int64_t n_rows, const int64_t *ids,
-                   const uint8_t *mask, float *dst, int accumulate, int64_t n, int64_t F,
-                   void *stream);
+                   const uint8_t *mask, void *dst, int dst_dtype, int accumulate, int64_t n,
+                   int64_t F, void *stream);
 
 /* hc_lookup: out[i] = map[ids[i] + offset]  (int64 gather; the id translation
  * of lookup_and_load, hiscache/history_cache.py:310,315). */

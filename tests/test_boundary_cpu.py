@@ -58,7 +58,8 @@ def test_argument_errors_are_status_codes():
     assert lib.hc_grad_check(*bad, p, 512, null) == 2
     assert lib.hc_grad_check_workspace_bytes(2_000_000) >= 8 * (2_000_000 // 64)
     assert lib.hc_row_scores(null, null, 4, 4, 0, null) == 1
-    assert lib.hc_gather_rows(p, 5, 4, p, null, p, 0, 2, 4, null) == 2
+    assert lib.hc_gather_rows(p, 5, 4, p, null, p, 0, 0, 2, 4, null) == 2
+    assert lib.hc_gather_rows(p, 0, 4, p, null, p, 9, 0, 2, 4, null) == 2
     assert lib.hc_count_history(null, null, null, 0, null, 4, 4, 1, 2, null) == 1
     for code in range(0, 8):
         assert lib.hc_strerror(code)

@@ -169,5 +169,9 @@ def test_small_helpers(be, orc):
     be.gather_rows(host, T(ids), T(mask), out=out, accumulate=True)
     np.testing.assert_array_equal(out.cpu().numpy(),
                                   1 + orc.gather_rows(host.float().numpy(), ids, mask))
+    # destination in the source's own precision (fp16 feature files stay fp16)
+    got16 = be.gather_rows(host, T(ids), T(mask), out_dtype=torch.float16)
+    assert got16.dtype == torch.float16
+    np.testing.assert_array_equal(got16.float().cpu().numpy(), orc.gather_rows(host.float().numpy(), ids, mask))
     m = rng.integers(-1, 99, size=1000)
     np.testing.assert_array_equal(be.lookup(T(m), T(ids), 3).cpu().numpy(), m[ids + 3])
