@@ -76,17 +76,48 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_finalize_edges(const uint32_t *__
 
 // ptrT from the sorted keys by boundary detection: position p owns the sources in
 // (key[p-1], key[p]] and writes ptrT[s] = p for them; the last position also closes the tail.
-// Used when sources are not much more numerous than edges, so the per-thread fill loops are short.
+// Short runs are written by the owning lane; a long run (many consecutive sources without edges)
+// is written by the whole wave, 64 entries per step, so no single lane loops for long.
 __global__ __launch_bounds__(HC_BLOCK) void tr_ptr_from_boundaries(const uint32_t *__restrict__ skeys,
                                                                     int64_t *__restrict__ ptrT, int64_t E,
                                                                     int64_t n_src) {
+  const int lane = hc_lane();
   const int64_t p = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
-  if (p >= E) return;
-  const int64_t cur = skeys[p];
-  const int64_t prev = p == 0 ? -1 : (int64_t)skeys[p - 1];
-  for (int64_t s = prev + 1; s <= cur; ++s) ptrT[s] = p;
-  if (p == E - 1)
-    for (int64_t s = cur + 1; s <= n_src; ++s) ptrT[s] = E;
+  int64_t first = 0, last = -1;  // sources [first, last] get ptrT = p
+  int64_t tail_first = 0, tail_last = -1;
+  if (p < E) {
+    const int64_t cur = skeys[p];
+    const int64_t prev = p == 0 ? -1 : (int64_t)skeys[p - 1];
+    first = prev + 1;
+    last = cur;
+    if (p == E - 1) {
+      tail_first = cur + 1;
+      tail_last = n_src;
+    }
+  }
+  constexpr int64_t SHORT_RUN = 4;
+  const int64_t run = last - first + 1;
+  if (run > 0 && run <= SHORT_RUN)
+    for (int64_t s = first; s <= last; ++s) ptrT[s] = p;
+  // long runs: one at a time, by the whole wave
+  unsigned long long m = __ballot(run > SHORT_RUN);
+  while (m != 0ull) {
+    const int l = __builtin_ctzll(m);
+    m &= m - 1ull;
+    const int64_t f = hc_readlane64(first, l);
+    const int64_t t = hc_readlane64(last, l);
+    const int64_t v = hc_readlane64(p, l);
+    for (int64_t s = f + lane; s <= t; s += HC_WAVE) ptrT[s] = v;
+  }
+  // the tail behind the last key (at most one lane of the grid has one)
+  unsigned long long mt = __ballot(tail_last >= tail_first);
+  while (mt != 0ull) {
+    const int l = __builtin_ctzll(mt);
+    mt &= mt - 1ull;
+    const int64_t f = hc_readlane64(tail_first, l);
+    const int64_t t = hc_readlane64(tail_last, l);
+    for (int64_t s = f + lane; s <= t; s += HC_WAVE) ptrT[s] = E;
+  }
 }
 
 // ptrT[s] = number of sorted keys strictly below s, for s in [0, n_src] (binary search; used
