@@ -60,6 +60,29 @@ __global__ __launch_bounds__(HC_BLOCK) void count_num_kernel(const int64_t *__re
   if (a > 0 && a <= mmax) atomicAdd(out + a, 1);
 }
 
+// Same histogram for few bins (relation ids): every block counts its slice in LDS and adds its
+// non-zero bins to the result once, instead of one contended global atomic per element.
+constexpr int CN_LDS_BINS = 4096;
+__global__ __launch_bounds__(HC_BLOCK) void count_num_lds_kernel(const int64_t *__restrict__ arr,
+                                                                  int32_t *__restrict__ out, int64_t n,
+                                                                  int mmax, int64_t per_block) {
+  __shared__ int hist[CN_LDS_BINS];
+  const int bins = mmax + 1;
+  for (int b = threadIdx.x; b < bins; b += HC_BLOCK) hist[b] = 0;
+  __syncthreads();
+  const int64_t begin = (int64_t)blockIdx.x * per_block;
+  const int64_t end = begin + per_block < n ? begin + per_block : n;
+  for (int64_t i = begin + threadIdx.x; i < end; i += HC_BLOCK) {
+    const int64_t a = arr[i];
+    if (a > 0 && a <= mmax) atomicAdd(&hist[(int)a], 1);
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < bins; b += HC_BLOCK) {
+    const int c = hist[b];
+    if (c != 0) atomicAdd(out + b, c);
+  }
+}
+
 // One level-synchronous pass of the structure score: rows with prev != 0 offer prev*deg to
 // neighbours whose prev is 0; the smallest offer wins (unsigned min over a 0 = "unset" encoding).
 __global__ __launch_bounds__(HC_BLOCK) void structure_pass(const int64_t *__restrict__ ptr,
@@ -231,7 +254,15 @@ extern "C" int hc_count_num(const int64_t *arr, int64_t n, int64_t mmax, int32_t
   if (n == 0) return HC_OK;
   HC_REQUIRE(arr);
   if (!hc_grid_ok((n + HC_BLOCK - 1) / HC_BLOCK)) return HC_EUNSUPPORTED;
-  count_num_kernel<<<dim3(blocks_for(n)), dim3(HC_BLOCK), 0, st>>>(arr, out, n, mmax);
+  if (mmax < CN_LDS_BINS) {
+    // at most 2048 blocks, at least 16 elements per thread
+    int64_t per_block = (n + 2047) / 2048;
+    if (per_block < 16 * HC_BLOCK) per_block = 16 * HC_BLOCK;
+    const int64_t blocks = (n + per_block - 1) / per_block;
+    count_num_lds_kernel<<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(arr, out, n, (int)mmax, per_block);
+  } else {
+    count_num_kernel<<<dim3(blocks_for(n)), dim3(HC_BLOCK), 0, st>>>(arr, out, n, mmax);
+  }
   return hc_launch_status();
 }
 

@@ -1,0 +1,150 @@
+// Typed CSR: the edges of every row regrouped by relation, so that one mean-aggregation launch
+// over (row, relation) groups feeds the relational convolution
+// (/root/reference/hiscache/history_model.py:248-270 does the grouping with a per-call sort inside
+// cxgnncomp's RGCNOP_sorted; here it is two wave-per-row passes and one scan, no sort).
+//
+//   1. count   wave per row: lane k counts the row's kept edges of relation k
+//   2. scan    rocPRIM inclusive scan of the counts -> group offsets
+//   3. place   wave per row: every kept edge goes to its group's next slot, in edge order
+//
+// An edge is kept when its relation is in [0, K), its source id is in [0, n_src) and, when a used
+// mask is given, the mask holds for its source.
+#include <cstring>
+
+#include <rocprim/rocprim.hpp>
+
+#include "hc_common.h"
+
+namespace {
+
+constexpr int TC_MAX_REL = HC_WAVE;  // one lane per relation
+
+struct TcEdge {
+  int64_t src;
+  int rel;
+  bool ok;
+};
+
+__device__ __forceinline__ TcEdge tc_load(const int64_t *__restrict__ idx, const int64_t *__restrict__ et,
+                                          const uint8_t *__restrict__ used, int64_t e, int64_t end, int K,
+                                          int64_t n_src) {
+  TcEdge r;
+  r.src = -1;
+  r.rel = -1;
+  r.ok = false;
+  if (e < end) {
+    r.src = idx[e];
+    const int64_t t = et[e];
+    if (t >= 0 && t < K && r.src >= 0 && r.src < n_src) {
+      r.rel = (int)t;
+      r.ok = used == nullptr || used[r.src] != 0;
+    }
+  }
+  return r;
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void tc_count(const int64_t *__restrict__ ptr,
+                                                      const int64_t *__restrict__ idx,
+                                                      const int64_t *__restrict__ et,
+                                                      const uint8_t *__restrict__ used,
+                                                      int64_t *__restrict__ cnt, int64_t *__restrict__ deg,
+                                                      int64_t *__restrict__ ptr2, int64_t R, int64_t E, int K,
+                                                      int64_t n_src) {
+  const int lane = hc_lane();
+  const int64_t row = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (row == 0 && lane == 0) ptr2[0] = 0;
+  if (row >= R) return;
+  const int64_t begin = ptr[row];
+  const int64_t full_end = ptr[row + 1];
+  const int64_t end = full_end < E ? full_end : E;
+  int c = 0;
+  for (int64_t base = begin; base < end; base += HC_WAVE) {
+    const TcEdge ed = tc_load(idx, et, used, base + lane, end, K, n_src);
+    for (int k = 0; k < K; ++k) {
+      const unsigned long long b = __ballot(ed.ok && ed.rel == k);
+      if (lane == k) c += __popcll(b);
+    }
+  }
+  if (lane < K) cnt[row * K + lane] = c;
+  if (lane == 0) deg[row] = full_end - begin;
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void tc_place(const int64_t *__restrict__ ptr,
+                                                      const int64_t *__restrict__ idx,
+                                                      const int64_t *__restrict__ et,
+                                                      const uint8_t *__restrict__ used,
+                                                      const int64_t *__restrict__ ptr2,
+                                                      int64_t *__restrict__ idx2, int64_t R, int64_t E, int K,
+                                                      int64_t n_src) {
+  const int lane = hc_lane();
+  const int64_t row = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (row >= R) return;
+  const int64_t begin = ptr[row];
+  const int64_t full_end = ptr[row + 1];
+  const int64_t end = full_end < E ? full_end : E;
+  // lane k: next free slot of group (row, k)
+  int64_t next = lane < K ? ptr2[row * K + lane] : 0;
+  const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (HC_WAVE - lane));
+  for (int64_t base = begin; base < end; base += HC_WAVE) {
+    const TcEdge ed = tc_load(idx, et, used, base + lane, end, K, n_src);
+    int rank = 0, add = 0;
+    for (int k = 0; k < K; ++k) {
+      const unsigned long long b = __ballot(ed.ok && ed.rel == k);
+      if (ed.ok && ed.rel == k) rank = __popcll(b & below);
+      if (lane == k) add = __popcll(b);
+    }
+    const int from = ed.ok ? ed.rel : 0;
+    const uint32_t lo = (uint32_t)__shfl((int)(uint32_t)(uint64_t)next, from, HC_WAVE);
+    const uint32_t hi = (uint32_t)__shfl((int)(uint32_t)((uint64_t)next >> 32), from, HC_WAVE);
+    const int64_t start = (int64_t)(((uint64_t)hi << 32) | lo);
+    if (ed.ok && start + rank < E) idx2[start + rank] = ed.src;
+    next += add;
+  }
+}
+
+__global__ void tc_zero_first(int64_t *ptr2) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) ptr2[0] = 0;
+}
+
+size_t tc_scan_bytes(int64_t n) {
+  size_t bytes = 0;
+  int64_t *none = nullptr;
+  if (rocprim::inclusive_scan(nullptr, bytes, none, none, (size_t)n, rocprim::plus<int64_t>()) != hipSuccess)
+    return 0;
+  return bytes;
+}
+
+}  // namespace
+
+extern "C" size_t hc_typed_csr_workspace_bytes(int64_t R, int num_rel) {
+  if (R <= 0 || num_rel <= 0) return 256;
+  return hc_align_up(tc_scan_bytes(R * (int64_t)num_rel), 256) + 256;
+}
+
+extern "C" int hc_typed_csr(const int64_t *ptr, const int64_t *idx, const int64_t *edge_types,
+                            const uint8_t *used_mask, int64_t R, int64_t E, int64_t n_src, int num_rel,
+                            int64_t *ptr2, int64_t *idx2, int64_t *cnt, int64_t *deg, void *workspace,
+                            size_t workspace_bytes, void *stream) {
+  HC_REQUIRE(R >= 0 && E >= 0 && n_src >= 0 && num_rel > 0 && ptr2);
+  if (num_rel > TC_MAX_REL) return HC_EUNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (R == 0) {
+    tc_zero_first<<<dim3(1), dim3(HC_WAVE), 0, st>>>(ptr2);
+    return hc_launch_status();
+  }
+  HC_REQUIRE(ptr && cnt && deg && (E == 0 || (idx && edge_types && idx2)));
+  const int64_t groups = R * (int64_t)num_rel;
+  if (workspace_bytes < hc_typed_csr_workspace_bytes(R, num_rel) || !workspace) return HC_EWORKSPACE;
+  const int64_t blocks = (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  if (!hc_grid_ok(blocks)) return HC_EUNSUPPORTED;
+  tc_count<<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, edge_types, used_mask, cnt, deg, ptr2,
+                                                             R, E, num_rel, n_src);
+  if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
+  size_t scan_bytes = tc_scan_bytes(groups);
+  if (rocprim::inclusive_scan(workspace, scan_bytes, cnt, ptr2 + 1, (size_t)groups, rocprim::plus<int64_t>(),
+                              st) != hipSuccess)
+    return HC_ELAUNCH;
+  tc_place<<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, edge_types, used_mask, ptr2, idx2, R, E,
+                                                             num_rel, n_src);
+  return hc_launch_status();
+}

@@ -112,33 +112,18 @@ class HistorySAGE(torch.nn.Module):
             bn.reset_parameters()
 
 
-def typed_csr(ptr, idx, edge_types, num_rel, num_node, used_mask=None):
+def typed_csr(ptr, idx, edge_types, num_rel, num_node, used_mask=None, n_src=None):
     """Group the edges of the first ``num_node`` rows by (row, relation): returns (ptr2, idx2, cnt, deg)
     where virtual row r*num_rel+k of (ptr2, idx2) holds row r's edges of relation k in their original
     order, cnt[num_node, num_rel] are the group sizes and deg[num_node] the full row degrees.
     ``edge_types`` covers at least the edges of those rows (it may be longer).  Edges whose source is
     not in ``used_mask`` are dropped, as the reference drops them by giving them an extra relation
-    (/root/reference/hiscache/history_model.py:248-250).  Dropped and surplus edges are parked in one
-    extra group behind the last virtual row, so nothing is compacted and no device value is read
-    back; ptr2 therefore has num_node*num_rel+2 entries and callers aggregate num_node*num_rel rows."""
-    num_edge = min(int(edge_types.shape[0]), int(idx.shape[0]))
-    dev = ptr.device
-    deg = ptr[1:num_node + 1] - ptr[:num_node]
-    e = torch.arange(num_edge, device=dev)
-    dst = torch.searchsorted(ptr[1:num_node + 1].contiguous(), e, right=True)   # row of every edge slot
-    src = idx[:num_edge]
-    rel = edge_types[:num_edge].to(torch.int64)
-    ok = (dst < num_node) & (rel >= 0) & (rel < num_rel)
-    if used_mask is not None:
-        ok = ok & used_mask[src]
-    trash = num_node * num_rel
-    key = torch.where(ok, dst * num_rel + rel, torch.full_like(dst, trash))
-    perm = torch.argsort(key, stable=True)
-    idx2 = src[perm].contiguous()
-    cnt = torch.zeros(trash + 1, dtype=torch.int64, device=dev).index_add_(0, key, torch.ones_like(key))
-    ptr2 = torch.zeros(trash + 2, dtype=torch.int64, device=dev)
-    torch.cumsum(cnt, 0, out=ptr2[1:])
-    return ptr2, idx2, cnt[:trash].view(num_node, num_rel), deg
+    (/root/reference/hiscache/history_model.py:248-250).  One library call: nothing is sorted and no
+    device value is read back."""
+    if n_src is None:
+        n_src = int(used_mask.shape[0]) if used_mask is not None else (1 << 62)
+    return hiscache_backend.typed_csr(ptr, idx, edge_types.to(torch.int64).contiguous(), num_rel, num_node,
+                                      n_src, used_mask)
 
 
 def edge_types_by_node_ranges(ptr, idx, sub_to_full, num_node, type_bounds, pair_to_rel):
@@ -180,7 +165,7 @@ class MyRGCNConvHistory2(torch.nn.Module):
                 num_node):
         num_node = int(num_node)
         K = self.num_rel
-        ptr2, idx2, cnt, deg = typed_csr(ptr, idx, edge_types, K, num_node, used_mask)
+        ptr2, idx2, cnt, deg = typed_csr(ptr, idx, edge_types, K, num_node, used_mask, n_src=x.shape[0])
         # per-relation edge counts, as the reference takes them (history_model.py:260)
         self.last_count = hiscache_backend.count_num(edge_types.to(torch.int64).contiguous(), K)
         none = torch.empty(0, device=x.device)

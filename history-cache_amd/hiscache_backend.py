@@ -64,6 +64,9 @@ _SIGNATURES = {
     "hc_structure_score": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p]),
     "hc_gather_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p]),
+    "hc_typed_csr_workspace_bytes": (_c_sz, [_c_i64, _c_int]),
+    "hc_typed_csr": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_p,
+                              _c_p, _c_sz, _c_p]),
 }
 
 _lib_handle = None
@@ -573,6 +576,45 @@ def lookup(map_tensor, ids, offset=0):
                        _stream())
     _check(rc, "hc_lookup")
     return out
+
+
+MAX_TYPED_RELATIONS = 64
+
+
+def typed_csr(ptr, idx, edge_types, num_rel, num_node, n_src, used_mask=None):
+    """Regroup the edges of the first ``num_node`` rows by (row, relation), keeping the edge order
+    inside every group.  Returns (ptr2[num_node*num_rel+1], idx2, cnt[num_node, num_rel], deg[num_node]);
+    edges with a relation outside [0, num_rel), a source outside [0, n_src) or a source that
+    ``used_mask`` (bool[n_src]) rules out are dropped.  Only the first ptr2[-1] entries of idx2 are
+    defined.  The grouping the reference obtains from a per-call sort by relation
+    (/root/reference/hiscache/history_model.py:248-270)."""
+    lib = load_library()
+    _dev(ptr, "ptr", torch.int64)
+    _dev(idx, "idx", torch.int64)
+    _dev(edge_types, "edge_types", torch.int64)
+    R, K = int(num_node), int(num_rel)
+    if K < 1 or K > MAX_TYPED_RELATIONS:
+        raise ValueError("num_rel must be in [1, %d]" % MAX_TYPED_RELATIONS)
+    if ptr.numel() < R + 1:
+        raise ValueError("ptr is shorter than num_node + 1")
+    E = min(int(edge_types.numel()), int(idx.numel()))
+    if used_mask is not None:
+        _dev(used_mask, "used_mask")
+        if used_mask.dtype not in (torch.bool, torch.uint8):
+            raise ValueError("used_mask must be bool or uint8")
+        if used_mask.numel() < int(n_src):
+            raise ValueError("used_mask is shorter than n_src")
+    dev = ptr.device
+    ptr2 = torch.empty(R * K + 1, dtype=torch.int64, device=dev)
+    idx2 = torch.empty(max(E, 1), dtype=torch.int64, device=dev)
+    cnt = torch.empty(R * K, dtype=torch.int64, device=dev)
+    deg = torch.empty(R, dtype=torch.int64, device=dev)
+    ws_bytes = int(lib.hc_typed_csr_workspace_bytes(R, K))
+    ws = _workspace(ws_bytes, dev)
+    rc = lib.hc_typed_csr(_ptr(ptr), _ptr(idx), _ptr(edge_types), _ptr(used_mask), R, E, int(n_src), K,
+                          _ptr(ptr2), _ptr(idx2), _ptr(cnt), _ptr(deg), _ptr(ws), ws_bytes, _stream())
+    _check(rc, "hc_typed_csr")
+    return ptr2, idx2, cnt.view(R, K), deg
 
 
 def long_row_edges(feature_width, dtype=torch.float32):

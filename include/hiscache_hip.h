@@ -226,6 +226,25 @@ int hc_cache_append(const float *score, const float *thres, const float *emb,
  * Values outside [0, mmax] are ignored. */
 int hc_count_num(const int64_t *arr, int64_t n, int64_t mmax, int32_t *out, void *stream);
 
+/* hc_typed_csr regroups the edges of the first R rows by (row, relation) for
+ * the relational convolution (hiscache/history_model.py:248-270, where the
+ * reference marks unused edges with an extra relation and lets cxgnncomp's
+ * RGCNOP_sorted sort the edges by relation on every call).  Group
+ * v = r*num_rel + k of (ptr2, idx2) holds, in their original order, the source
+ * ids of row r's edges e with edge_types[e] == k whose source is in
+ * [0, n_src) and, when used_mask (n_src bytes, nullable) is given, has
+ * used_mask[src] != 0.  Only edge slots below E are read (E = entries
+ * available in idx and in edge_types).  Outputs: ptr2[R*num_rel + 1],
+ * idx2[E] (only the first ptr2[R*num_rel] entries are written),
+ * cnt[R*num_rel] = group sizes, deg[R] = full row degrees ptr[r+1]-ptr[r].
+ * num_rel <= 64 (HC_EUNSUPPORTED above).  Integer work only: results are
+ * exact and independent of scheduling. */
+size_t hc_typed_csr_workspace_bytes(int64_t R, int num_rel);
+int hc_typed_csr(const int64_t *ptr, const int64_t *idx, const int64_t *edge_types,
+                 const uint8_t *used_mask, int64_t R, int64_t E, int64_t n_src, int num_rel,
+                 int64_t *ptr2, int64_t *idx2, int64_t *cnt, int64_t *deg, void *workspace,
+                 size_t workspace_bytes, void *stream);
+
 /* hc_structure_score replaces get_graph_structure_score (grad_check.h:22-24,
  * grad_check.cu:132-163) with a level-synchronous, deterministic reading of
  * the same rule: per pass, seeds hold 1; a row with a non-zero value offers

@@ -612,6 +612,37 @@ int orc_count_num(const Index *arr, Index n, Index mmax, int32_t *out) {
   return ORC_OK;
 }
 
+/* Typed CSR for the relational convolution (hiscache/history_model.py:248-270:
+ * edges whose source is unused get an extra relation and are ignored; the rest
+ * are grouped by relation).  Group r*K+k of (ptr2, idx2) lists, in edge order,
+ * the sources of row r's edges of relation k that are kept.  cnt = group
+ * sizes, deg = full row degrees.  Pinned by the tests against a stable sort by
+ * (row, relation) written with numpy. */
+int orc_typed_csr(const Index *ptr, const Index *idx, const Index *et, const uint8_t *used,
+                  Index R, Index E, Index n_src, int K, Index *ptr2, Index *idx2, Index *cnt,
+                  Index *deg) {
+  if (K < 1 || R < 0) return ORC_EINVAL;
+  Index pos = 0;
+  ptr2[0] = 0;
+  for (Index r = 0; r < R; ++r) {
+    Index begin = ptr[r], end = ptr[r + 1] < E ? ptr[r + 1] : E;
+    deg[r] = ptr[r + 1] - ptr[r];
+    for (int k = 0; k < K; ++k) {
+      Index c = 0;
+      for (Index e = begin; e < end; ++e) {
+        Index s = idx[e];
+        if (et[e] != k || s < 0 || s >= n_src) continue;
+        if (used && !used[s]) continue;
+        idx2[pos++] = s;
+        ++c;
+      }
+      cnt[r * K + k] = c;
+      ptr2[r * K + k + 1] = pos;
+    }
+  }
+  return ORC_OK;
+}
+
 /* get_graph_structure_score, grad_check.cu:132-163.  The reference reads and
  * writes `output` across warps inside one pass, so its result depends on
  * scheduling.  This is the level-synchronous reading of the same rule: pass

@@ -271,6 +271,21 @@ def count_num(arr, mmax):
     return out
 
 
+def typed_csr(ptr, idx, edge_types, num_rel, num_node, n_src, used_mask=None):
+    """(ptr2, idx2[:ptr2[-1]], cnt[num_node, num_rel], deg) of the (row, relation) grouping."""
+    ptr, idx, et = _i64(ptr), _i64(idx), _i64(edge_types)
+    R, K = int(num_node), int(num_rel)
+    E = min(len(idx), len(et))
+    used = None if used_mask is None else np.ascontiguousarray(used_mask, dtype=np.uint8)
+    ptr2 = np.zeros(R * K + 1, np.int64)
+    idx2 = np.zeros(max(E, 1), np.int64)
+    cnt = np.zeros(R * K, np.int64)
+    deg = np.zeros(R, np.int64)
+    _check(lib().orc_typed_csr(_p(ptr), _p(idx), _p(et), _p(used) if used is not None else None, _I(R), _I(E),
+                               _I(n_src), ctypes.c_int(K), _p(ptr2), _p(idx2), _p(cnt), _p(deg)), "typed_csr")
+    return ptr2, idx2[:ptr2[-1]], cnt.reshape(R, K), deg
+
+
 def get_graph_structure_score(ptr, idx, num_node, num_seed, num_layer):
     ptr, idx = _i64(ptr), _i64(idx)
     out = np.zeros(int(num_node), np.int64)

@@ -455,3 +455,41 @@ def test_typed_csr_groups_edges_by_row_and_relation():
             v = r * K + k
             np.testing.assert_array_equal(idx2[ptr2[v]:ptr2[v + 1]], idx[e])
             assert cnt[r, k] == len(e)
+
+
+@pytest.mark.parametrize("K,with_mask,short_types", [(5, True, False), (1, False, False), (64, True, True),
+                                                      (7, False, True)])
+def test_typed_csr_matches_oracle(orc, K, with_mask, short_types):
+    """hc_typed_csr against the CPU checker: rows longer than one wave, relations and sources outside
+    their ranges, relation arrays shorter than the edge list, with and without a used mask."""
+    from helpers import random_csr
+    rng = np.random.default_rng(50 + K)
+    R, N = 700, 400
+    ptr, idx = random_csr(rng, R + 50, N, 200, hub=5)
+    idx = idx.copy()
+    idx[rng.random(len(idx)) < 0.02] = N + 5
+    rel = rng.integers(-1, K + 1, size=len(idx))
+    if short_types:
+        rel = rel[: int(ptr[R - 20])]
+    used = (rng.random(N) < 0.7) if with_mask else None
+    import hiscache_backend as be
+    t = lambda a: None if a is None else torch.from_numpy(a).to(DEV)
+    ptr2, idx2, cnt, deg = be.typed_csr(t(ptr), t(idx), t(rel), K, R, N, t(used))
+    w_ptr2, w_idx2, w_cnt, w_deg = orc.typed_csr(ptr, idx, rel, K, R, N, used)
+    np.testing.assert_array_equal(ptr2.cpu().numpy(), w_ptr2)
+    np.testing.assert_array_equal(idx2.cpu().numpy()[: w_ptr2[-1]], w_idx2)
+    np.testing.assert_array_equal(cnt.cpu().numpy(), w_cnt)
+    np.testing.assert_array_equal(deg.cpu().numpy(), w_deg)
+    p0 = be.typed_csr(t(ptr), t(idx), t(rel), K, 0, N, t(used))[0]
+    assert p0.cpu().tolist() == [0]
+    with pytest.raises(ValueError):
+        be.typed_csr(t(ptr), t(idx), t(rel), 65, R, N, t(used))
+
+
+def test_count_num_few_and_many_bins(orc):
+    import hiscache_backend as be
+    rng = np.random.default_rng(61)
+    for n, mmax in ((0, 3), (5, 1), (300_000, 5), (300_000, 4095), (100_000, 6000)):
+        arr = rng.integers(0, mmax + 1, size=n)
+        got = be.count_num(torch.from_numpy(arr).to(DEV), mmax).cpu().numpy()
+        np.testing.assert_array_equal(got, orc.count_num(arr, mmax))

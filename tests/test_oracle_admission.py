@@ -412,3 +412,39 @@ def test_small_helpers(orc):
     t = rng.standard_normal((7, 3)).astype(np.float32)
     got = orc.gather_rows(t, np.array([0, -1, 3]), np.array([True, True, False]))
     np.testing.assert_array_equal(got, np.stack([t[0], t[6], np.zeros(3, np.float32)]))
+
+
+def typed_csr_by_stable_sort(ptr, idx, rel, K, R, n_src, used=None):
+    """(row, relation) grouping stated with numpy: keep-filter, then a stable sort by row*K + relation."""
+    E = min(len(idx), len(rel))
+    row_of = np.searchsorted(ptr[1:R + 1], np.arange(E), side="right")
+    keep = (row_of < R) & (rel[:E] >= 0) & (rel[:E] < K) & (idx[:E] >= 0) & (idx[:E] < n_src)
+    if used is not None:
+        keep &= used[np.clip(idx[:E], 0, n_src - 1)]
+    key = row_of[keep] * K + rel[:E][keep]
+    order = np.argsort(key, kind="stable")
+    cnt = np.bincount(key, minlength=R * K)[:R * K]
+    ptr2 = np.concatenate([[0], np.cumsum(cnt)])
+    return ptr2, idx[:E][keep][order], cnt.reshape(R, K), np.diff(ptr)[:R]
+
+
+@pytest.mark.parametrize("K,with_mask,short_types", [(5, True, False), (1, False, False), (64, True, True),
+                                                      (7, False, True)])
+def test_typed_csr_equals_stable_sort(orc, K, with_mask, short_types):
+    from helpers import random_csr
+    rng = np.random.default_rng(40 + K)
+    R, N = 120, 90
+    ptr, idx = random_csr(rng, R + 30, N, 150, hub=3)          # some rows longer than 64 edges
+    idx = idx.copy()
+    idx[rng.random(len(idx)) < 0.02] = N + 5                    # sources outside the range are dropped
+    rel = rng.integers(-1, K + 1, size=len(idx))                # -1 and K are dropped
+    if short_types:
+        rel = rel[: int(ptr[R - 10])]                           # the last rows have no relation entries
+    used = (rng.random(N) < 0.7) if with_mask else None
+    want = typed_csr_by_stable_sort(ptr, idx, rel, K, R, N, used)
+    got = orc.typed_csr(ptr, idx, rel, K, R, N, used)
+    for g, w in zip(got, want):
+        np.testing.assert_array_equal(g, w)
+    # no rows: a single zero offset
+    p2, i2, c, d = orc.typed_csr(ptr, idx, rel, K, 0, N, used)
+    assert p2.tolist() == [0] and i2.size == 0 and c.size == 0 and d.size == 0
