@@ -148,3 +148,57 @@ extern "C" int hc_typed_csr(const int64_t *ptr, const int64_t *idx, const int64_
                                                              num_rel, n_src);
   return hc_launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Relation of every edge from the node types of its two ends; a node's type is the number of
+// bounds its full id has reached (bounds ascending).  Wave per row: the row's type is found once,
+// every lane classifies one source.
+namespace {
+
+constexpr int TC_MAX_BOUNDS = 64;
+
+__device__ __forceinline__ int tc_type_of(int64_t full, const int64_t *__restrict__ bounds, int n_bounds) {
+  int t = 0;
+  for (int b = 0; b < n_bounds; ++b) t += full >= bounds[b] ? 1 : 0;
+  return t;
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void tc_edge_types(const int64_t *__restrict__ ptr,
+                                                           const int64_t *__restrict__ idx,
+                                                           const int64_t *__restrict__ sub_to_full,
+                                                           const int64_t *__restrict__ bounds, int n_bounds,
+                                                           const int64_t *__restrict__ pair_to_rel,
+                                                           int64_t *__restrict__ out, int64_t R, int64_t E,
+                                                           int64_t n_all) {
+  const int lane = hc_lane();
+  const int64_t row = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (row >= R) return;
+  const int64_t begin = ptr[row];
+  const int64_t full_end = ptr[row + 1];
+  const int64_t end = full_end < E ? full_end : E;
+  const int n_types = n_bounds + 1;
+  const int t_dst = row < n_all ? tc_type_of(sub_to_full[row], bounds, n_bounds) : 0;
+  for (int64_t e = begin + lane; e < end; e += HC_WAVE) {
+    const int64_t s = idx[e];
+    int64_t rel = -1;
+    if (s >= 0 && s < n_all) rel = pair_to_rel[t_dst * n_types + tc_type_of(sub_to_full[s], bounds, n_bounds)];
+    out[e] = rel;
+  }
+}
+
+}  // namespace
+
+extern "C" int hc_edge_types_by_ranges(const int64_t *ptr, const int64_t *idx, const int64_t *sub_to_full,
+                                       int64_t n_all, const int64_t *bounds, int n_bounds,
+                                       const int64_t *pair_to_rel, int64_t *out, int64_t R, int64_t E,
+                                       void *stream) {
+  HC_REQUIRE(R >= 0 && E >= 0 && n_all >= 0 && n_bounds >= 0);
+  if (n_bounds > TC_MAX_BOUNDS) return HC_EUNSUPPORTED;
+  if (R == 0 || E == 0) return HC_OK;
+  HC_REQUIRE(ptr && idx && sub_to_full && pair_to_rel && out && (n_bounds == 0 || bounds));
+  const int64_t blocks = (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  if (!hc_grid_ok(blocks)) return HC_EUNSUPPORTED;
+  tc_edge_types<<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, static_cast<hipStream_t>(stream)>>>(
+      ptr, idx, sub_to_full, bounds, n_bounds, pair_to_rel, out, R, E, n_all);
+  return hc_launch_status();
+}

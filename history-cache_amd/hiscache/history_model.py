@@ -131,15 +131,15 @@ def edge_types_by_node_ranges(ptr, idx, sub_to_full, num_node, type_bounds, pair
     type is the range of ``type_bounds`` its full id falls into (mag240M stores papers, authors and
     institutions in consecutive id ranges).  ``pair_to_rel[type(dst), type(src)]`` gives the relation.
     Stands in for ``cxgnncomp_backend.gen_edge_type_mag240m``
-    (/root/reference/hiscache/history_model.py:356), whose exact numbering is not available here."""
-    num_edge = int(idx.shape[0])
-    e = torch.arange(num_edge, device=ptr.device)
-    dst = torch.searchsorted(ptr[1:num_node + 1].contiguous(), e, right=True).clamp(max=num_node - 1)
-    bounds = torch.as_tensor(type_bounds, dtype=torch.int64, device=ptr.device)
-    t_dst = torch.bucketize(sub_to_full[dst], bounds, right=True)
-    t_src = torch.bucketize(sub_to_full[idx[:num_edge]], bounds, right=True)
-    table = torch.as_tensor(pair_to_rel, dtype=torch.int64, device=ptr.device)
-    return table[t_dst, t_src]
+    (/root/reference/hiscache/history_model.py:356), whose exact numbering is not available here.
+    ``type_bounds`` and ``pair_to_rel`` may be device tensors (no copy) or host sequences."""
+    dev = ptr.device
+    bounds = type_bounds if isinstance(type_bounds, torch.Tensor) else torch.as_tensor(
+        type_bounds, dtype=torch.int64, device=dev)
+    table = pair_to_rel if isinstance(pair_to_rel, torch.Tensor) else torch.as_tensor(
+        pair_to_rel, dtype=torch.int64, device=dev)
+    return hiscache_backend.edge_types_by_ranges(ptr, idx, sub_to_full, num_node, bounds.contiguous(),
+                                                 table.contiguous())
 
 
 class MyRGCNConvHistory2(torch.nn.Module):
@@ -224,6 +224,10 @@ class HistoryRGCN(torch.nn.Module):
         if getattr(batch, "edge_type", None) is not None:
             return batch.edge_type
         if self.gen_rel and self.type_bounds is not None:
+            if not isinstance(self.type_bounds, torch.Tensor):     # moved to the device once
+                dev = batch.ptr.device
+                self.type_bounds = torch.as_tensor(self.type_bounds, dtype=torch.int64, device=dev)
+                self.pair_to_rel = torch.as_tensor(self.pair_to_rel, dtype=torch.int64, device=dev)
             return edge_types_by_node_ranges(batch.ptr, batch.idx, batch.sub_to_full,
                                              int(batch.num_node_in_layer[L - 1]), self.type_bounds,
                                              self.pair_to_rel)

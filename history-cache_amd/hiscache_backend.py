@@ -65,6 +65,7 @@ _SIGNATURES = {
     "hc_gather_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p]),
     "hc_typed_csr_workspace_bytes": (_c_sz, [_c_i64, _c_int]),
+    "hc_edge_types_by_ranges": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_p, _c_p, _c_i64, _c_i64, _c_p]),
     "hc_typed_csr": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_p,
                               _c_p, _c_sz, _c_p]),
 }
@@ -615,6 +616,29 @@ def typed_csr(ptr, idx, edge_types, num_rel, num_node, n_src, used_mask=None):
                           _ptr(ptr2), _ptr(idx2), _ptr(cnt), _ptr(deg), _ptr(ws), ws_bytes, _stream())
     _check(rc, "hc_typed_csr")
     return ptr2, idx2, cnt.view(R, K), deg
+
+
+def edge_types_by_ranges(ptr, idx, sub_to_full, num_node, bounds, pair_to_rel):
+    """out[e] = pair_to_rel[type(row of e), type(idx[e])] for the edges of the first ``num_node`` rows,
+    where a node's type is the number of entries of ``bounds`` (ascending int64 tensor) its full id
+    has reached; other entries of the result are -1."""
+    lib = load_library()
+    _dev(ptr, "ptr", torch.int64)
+    _dev(idx, "idx", torch.int64)
+    _dev(sub_to_full, "sub_to_full", torch.int64)
+    _dev(bounds, "bounds", torch.int64)
+    _dev(pair_to_rel, "pair_to_rel", torch.int64)
+    T = bounds.numel() + 1
+    if pair_to_rel.numel() != T * T:
+        raise ValueError("pair_to_rel must be [T, T] with T = len(bounds) + 1")
+    R = int(num_node)
+    if ptr.numel() < R + 1:
+        raise ValueError("ptr is shorter than num_node + 1")
+    out = torch.full((idx.numel(),), -1, dtype=torch.int64, device=idx.device)
+    rc = lib.hc_edge_types_by_ranges(_ptr(ptr), _ptr(idx), _ptr(sub_to_full), sub_to_full.numel(), _ptr(bounds),
+                                     int(bounds.numel()), _ptr(pair_to_rel), _ptr(out), R, idx.numel(), _stream())
+    _check(rc, "hc_edge_types_by_ranges")
+    return out
 
 
 def long_row_edges(feature_width, dtype=torch.float32):

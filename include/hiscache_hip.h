@@ -245,6 +245,19 @@ int hc_typed_csr(const int64_t *ptr, const int64_t *idx, const int64_t *edge_typ
                  int64_t *ptr2, int64_t *idx2, int64_t *cnt, int64_t *deg, void *workspace,
                  size_t workspace_bytes, void *stream);
 
+/* hc_edge_types_by_ranges: relation of every edge of the first R rows from the
+ * node types of its ends, out[e] = pair_to_rel[type(row) * T + type(idx[e])]
+ * with T = n_bounds + 1 and type(v) = number of bounds[b] <= sub_to_full[v]
+ * (node types stored as consecutive full-id ranges, as mag240M stores papers,
+ * authors and institutions).  Stands in for cxgnncomp_backend.gen_edge_type_mag240m
+ * (called at hiscache/history_model.py:356), which is not part of the
+ * reference repository.  Edge slots at or beyond ptr[R] (or E) are left as
+ * they are; a source outside [0, n_all) gets -1.  n_bounds <= 64. */
+int hc_edge_types_by_ranges(const int64_t *ptr, const int64_t *idx, const int64_t *sub_to_full,
+                            int64_t n_all, const int64_t *bounds, int n_bounds,
+                            const int64_t *pair_to_rel, int64_t *out, int64_t R, int64_t E,
+                            void *stream);
+
 /* hc_structure_score replaces get_graph_structure_score (grad_check.h:22-24,
  * grad_check.cu:132-163) with a level-synchronous, deterministic reading of
  * the same rule: per pass, seeds hold 1; a row with a non-zero value offers

@@ -286,6 +286,27 @@ def typed_csr(ptr, idx, edge_types, num_rel, num_node, n_src, used_mask=None):
     return ptr2, idx2[:ptr2[-1]], cnt.reshape(R, K), deg
 
 
+def edge_types_by_ranges(ptr, idx, sub_to_full, num_node, bounds, pair_to_rel):
+    """Relation per edge from the node types of its ends (numpy statement; type = number of bounds
+    the full id has reached).  -1 outside the first ``num_node`` rows and for sources out of range.
+    Stand-in for cxgnncomp_backend.gen_edge_type_mag240m (history_model.py:356): PARITY UNPINNED
+    against that library, which is not part of the reference repository."""
+    ptr, idx, s2f = _i64(ptr), _i64(idx), _i64(sub_to_full)
+    bounds = _i64(bounds)
+    table = np.asarray(pair_to_rel, np.int64).reshape(len(bounds) + 1, len(bounds) + 1)
+    R = int(num_node)
+    out = np.full(len(idx), -1, np.int64)
+    end = min(int(ptr[R]), len(idx))
+    e = np.arange(end)
+    row = np.searchsorted(ptr[1:R + 1], e, side="right")
+    src = idx[:end]
+    ok = (src >= 0) & (src < len(s2f))
+    t_dst = np.searchsorted(bounds, s2f[row], side="right")
+    t_src = np.searchsorted(bounds, s2f[np.where(ok, src, 0)], side="right")
+    out[:end] = np.where(ok, table[t_dst, t_src], -1)
+    return out
+
+
 def get_graph_structure_score(ptr, idx, num_node, num_seed, num_layer):
     ptr, idx = _i64(ptr), _i64(idx)
     out = np.zeros(int(num_node), np.int64)

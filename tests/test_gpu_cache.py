@@ -493,3 +493,21 @@ def test_count_num_few_and_many_bins(orc):
         arr = rng.integers(0, mmax + 1, size=n)
         got = be.count_num(torch.from_numpy(arr).to(DEV), mmax).cpu().numpy()
         np.testing.assert_array_equal(got, orc.count_num(arr, mmax))
+
+
+def test_edge_types_by_ranges_matches_oracle(orc):
+    import hiscache_backend as be
+    from helpers import random_csr
+    rng = np.random.default_rng(72)
+    R, n_all = 900, 1500
+    ptr, idx = random_csr(rng, R + 100, n_all, 150, hub=4)
+    idx = idx.copy()
+    idx[rng.random(len(idx)) < 0.01] = n_all + 3
+    s2f = rng.permutation(100_000)[:n_all]
+    bounds = np.array([30_000, 65_000])
+    table = np.array([[0, 1, -1], [2, -1, 3], [-1, 4, -1]])
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.int64)).to(DEV)
+    got = be.edge_types_by_ranges(t(ptr), t(idx), t(s2f), R, t(bounds), t(table)).cpu().numpy()
+    np.testing.assert_array_equal(got, orc.edge_types_by_ranges(ptr, idx, s2f, R, bounds, table))
+    none = be.edge_types_by_ranges(t(ptr), t(idx), t(s2f), R, t(np.zeros(0)), t(np.array([[7]]))).cpu().numpy()
+    assert set(np.unique(none[: ptr[R]])) <= {7, -1}

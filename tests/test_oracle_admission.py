@@ -448,3 +448,19 @@ def test_typed_csr_equals_stable_sort(orc, K, with_mask, short_types):
     # no rows: a single zero offset
     p2, i2, c, d = orc.typed_csr(ptr, idx, rel, K, 0, N, used)
     assert p2.tolist() == [0] and i2.size == 0 and c.size == 0 and d.size == 0
+
+
+def test_edge_types_by_ranges_brute_force(orc):
+    from helpers import random_csr
+    rng = np.random.default_rng(71)
+    R, n_all = 40, 60
+    ptr, idx = random_csr(rng, R + 5, n_all, 9)
+    s2f = rng.permutation(1000)[:n_all]
+    bounds = np.array([300, 650])
+    table = np.array([[0, 1, -1], [2, -1, 3], [-1, 4, -1]])
+    got = orc.edge_types_by_ranges(ptr, idx, s2f, R, bounds, table)
+    typ = lambda v: int(v >= 300) + int(v >= 650)
+    for r in range(R + 5):
+        for e in range(ptr[r], ptr[r + 1]):
+            want = table[typ(s2f[r]), typ(s2f[idx[e]])] if r < R else -1
+            assert got[e] == want
