@@ -12,10 +12,11 @@ from .history_model import (HistoryRGCN, HistorySAGE, MyRGCNConvHistory2, MySage
                             typed_csr)
 from .history_table import HistoryTable
 from .ring_cache import RingHistoryCache
+from .sampler import NeighborSampler
 from .util import Config, make_config, quantile_threshold
 
 __all__ = [
     "HistoryCache", "HistoryTable", "RingHistoryCache", "HistorySAGE", "HistoryRGCN", "MySageConvHistory", "MyRGCNConvHistory2", "typed_csr", "get_model",
-    "PinnedFeatureStore", "Config", "make_config", "quantile_threshold",
+    "PinnedFeatureStore", "NeighborSampler", "Config", "make_config", "quantile_threshold",
     "count_history_reconstruct", "get_graph_structure_score", "record_history",
 ]

@@ -64,6 +64,11 @@ _SIGNATURES = {
     "hc_structure_score": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p]),
     "hc_gather_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p]),
+    "hc_sample_capacity": (_c_int, [_c_i64, _c_p, _c_int, _c_i64, _c_p, _c_p, _c_p]),
+    "hc_sample_workspace_bytes": (_c_sz, [_c_i64, _c_p, _c_int, _c_i64]),
+    "hc_sample_map_init": (_c_int, [_c_p, _c_i64, _c_p]),
+    "hc_sample_layers": (_c_int, [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_int, ctypes.c_uint64, _c_p, _c_p,
+                                  _c_p, _c_p, _c_p, _c_p, _c_sz, _c_p]),
     "hc_typed_csr_workspace_bytes": (_c_sz, [_c_i64, _c_int]),
     "hc_edge_types_by_ranges": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_p, _c_p, _c_i64, _c_i64, _c_p]),
     "hc_typed_csr": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_p,
@@ -639,6 +644,64 @@ def edge_types_by_ranges(ptr, idx, sub_to_full, num_node, bounds, pair_to_rel):
                                      int(bounds.numel()), _ptr(pair_to_rel), _ptr(out), R, idx.numel(), _stream())
     _check(rc, "hc_edge_types_by_ranges")
     return out
+
+
+def sample_map(num_nodes, device):
+    """The sampler's persistent node map (int32[num_nodes], every entry "unseen")."""
+    lib = load_library()
+    m = torch.empty(int(num_nodes), dtype=torch.int32, device=device)
+    with torch.cuda.device(m.device):
+        _check(lib.hc_sample_map_init(_ptr(m), m.numel(), _stream()), "hc_sample_map_init")
+    return m
+
+
+def sample_capacity(n_seed, fanout, num_nodes):
+    """(max_rows, max_edges, max_nodes) a batch of ``n_seed`` seeds can reach."""
+    lib = load_library()
+    fan = (ctypes.c_int64 * len(fanout))(*[int(f) for f in fanout])
+    out = [ctypes.c_int64(0) for _ in range(3)]
+    rc = lib.hc_sample_capacity(int(n_seed), ctypes.cast(fan, _c_p), len(fanout), int(num_nodes),
+                                *[ctypes.cast(ctypes.pointer(o), _c_p) for o in out])
+    _check(rc, "hc_sample_capacity")
+    return tuple(int(o.value) for o in out)
+
+
+def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map):
+    """Layered neighbour sampling without replacement.  Returns (ptr, idx, sub_to_full, counts) as
+    device tensors at their capacity; ``counts`` (int64[2L+1] on the device) holds the node count
+    within k hops for k = 0..L and then the cumulative edge count after every hop, so the caller
+    slices ptr[:counts[L-1]+1], idx[:counts[2L]], sub_to_full[:counts[L]] once it has read them.
+    ``seeds`` must be distinct valid node ids; ``node_map`` comes from ``sample_map`` and is left
+    all-unseen again.  Stands where the reference's external loader does
+    (/root/reference/hiscache/history_trainer.py:19,26)."""
+    lib = load_library()
+    _dev(indptr, "indptr", torch.int64)
+    _dev(indices, "indices", torch.int64)
+    _dev(seeds, "seeds", torch.int64)
+    _dev(node_map, "node_map", torch.int32)
+    N = indptr.numel() - 1
+    if node_map.numel() < N:
+        raise ValueError("node_map is shorter than the graph")
+    L = len(fanout)
+    n_seed = seeds.numel()
+    if n_seed == 0:
+        raise ValueError("no seeds")
+    fan = (ctypes.c_int64 * L)(*[int(f) for f in fanout])
+    rows, edges, nodes = sample_capacity(n_seed, fanout, N)
+    dev = seeds.device
+    ptr = torch.empty(rows + 1, dtype=torch.int64, device=dev)
+    idx = torch.empty(max(edges, 1), dtype=torch.int64, device=dev)
+    s2f = torch.empty(max(nodes, 1), dtype=torch.int64, device=dev)
+    counts = torch.empty(2 * L + 1, dtype=torch.int64, device=dev)
+    ws_bytes = int(lib.hc_sample_workspace_bytes(n_seed, ctypes.cast(fan, _c_p), L, N))
+    if ws_bytes == 0:
+        raise ValueError("unsupported fanout / batch size")
+    ws = _workspace(ws_bytes, dev)
+    rc = lib.hc_sample_layers(_ptr(indptr), _ptr(indices), N, _ptr(seeds), n_seed, ctypes.cast(fan, _c_p), L,
+                              ctypes.c_uint64(int(rng_seed) & 0xFFFFFFFFFFFFFFFF), _ptr(node_map), _ptr(ptr),
+                              _ptr(idx), _ptr(s2f), _ptr(counts), _ptr(ws), ws_bytes, _stream())
+    _check(rc, "hc_sample_layers")
+    return ptr, idx, s2f, counts
 
 
 def long_row_edges(feature_width, dtype=torch.float32):

@@ -220,6 +220,42 @@ int hc_cache_append(const float *score, const float *thres, const float *emb,
                     int64_t *overflow, int64_t M, void *workspace, size_t workspace_bytes,
                     void *stream);
 
+/* ---------------------------------------------------------------- sampler
+ * Layered neighbour sampling on the device.  The reference takes its batches
+ * from the external cxgnndl loader (hiscache/history_trainer.py:19,26); these
+ * entry points produce the same wire format the model and the cache read
+ * (hiscache/history_model.py:120-153, hiscache/history_cache.py:307-324):
+ * sub-graph nodes numbered seeds first, then each hop's new nodes in
+ * first-seen order; counts[k] = nodes within k hops; one shared CSR
+ * (ptr, idx) with the sampled neighbours of the first counts[L-1] nodes.
+ *
+ * Rule for row u (full id f, degree d) at hop k: if d <= fanout[k] all
+ * neighbours in list order, else neighbour j (j < fanout[k]) is list position
+ * perm(j), a bijection of [0, d) keyed by (rng_seed, k, f): four Feistel
+ * rounds over the next even power of two, round function splitmix64, with
+ * cycle walking.  The picks of a row are therefore distinct list positions.
+ *
+ * node_map is int32[num_nodes], persistent between calls, all "unseen" on
+ * entry and on return (hc_sample_map_init fills it once).  seeds must be
+ * distinct valid ids.  fanout is a HOST array of num_hops entries
+ * (<= HC_SAMPLE_MAX_HOPS).  Outputs are sized by hc_sample_capacity: ptr
+ * [max_rows + 1], idx [max_edges], sub_to_full [max_nodes]; counts is
+ * int64[2*num_hops + 1] on the device: counts[0..L] node counts, then the
+ * cumulative edge count after every hop.  Nothing is read back: the caller
+ * copies counts to the host when it needs the sizes.  Calls that share a
+ * node_map must not overlap. */
+#define HC_SAMPLE_MAX_HOPS 8
+int hc_sample_capacity(int64_t n_seed, const int64_t *fanout, int num_hops, int64_t num_nodes,
+                       int64_t *max_rows, int64_t *max_edges, int64_t *max_nodes);
+size_t hc_sample_workspace_bytes(int64_t n_seed, const int64_t *fanout, int num_hops,
+                                 int64_t num_nodes);
+int hc_sample_map_init(int32_t *node_map, int64_t num_nodes, void *stream);
+int hc_sample_layers(const int64_t *indptr, const int64_t *indices, int64_t num_nodes,
+                     const int64_t *seeds, int64_t n_seed, const int64_t *fanout, int num_hops,
+                     uint64_t rng_seed, int32_t *node_map, int64_t *ptr, int64_t *idx,
+                     int64_t *sub_to_full, int64_t *counts, void *workspace, size_t workspace_bytes,
+                     void *stream);
+
 /* ---------------------------------------------------------------- helpers
  * hc_count_num replaces count_num (grad_check.h:26, grad_check.cu:165-182):
  * histogram of arr into out[mmax+1] (int32, zeroed here) that skips value 0.

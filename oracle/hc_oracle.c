@@ -689,3 +689,84 @@ int orc_gather_rows(const float *table, Index n_rows, const Index *ids,
   }
   return ORC_OK;
 }
+
+/* ------------------------------------------------------------------ sampler
+ * Layered neighbour sampling, stated sequentially.  The reference has no
+ * sampler of its own (batches come from the external cxgnndl loader,
+ * hiscache/history_trainer.py:19,26), so this restates the library's published
+ * rule, not reference code: PARITY UNPINNED against cxgnndl; the batch layout
+ * is the one hiscache/history_model.py:120-153 reads.  Pinned by the tests
+ * through what the rule implies: perm is a bijection of [0, d) (brute force),
+ * rows hold min(d, fanout) distinct list positions, local ids are first-seen
+ * order, and the pick frequencies are uniform (chi-square). */
+uint64_t orc_mix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+/* Keyed bijection of [0, d), d >= 2: 4 Feistel rounds on 2h bits (h = half of
+ * the bit length of d-1, rounded up), cycle walking back into [0, d). */
+uint64_t orc_sample_perm(uint64_t j, uint64_t d, uint64_t key) {
+  int bits = 0;
+  for (uint64_t t = d - 1; t; t >>= 1) ++bits;
+  int h = (bits + 1) / 2;
+  uint64_t mask = (1ull << h) - 1ull;
+  uint64_t x = j;
+  do {
+    uint64_t l = x >> h, r = x & mask;
+    for (int round = 0; round < 4; ++round) {
+      uint64_t f = orc_mix64(r ^ key ^ ((uint64_t)round << 56)) & mask;
+      uint64_t t = l ^ f;
+      l = r;
+      r = t;
+    }
+    x = (l << h) | r;
+  } while (x >= d);
+  return x;
+}
+
+int orc_sample_layers(const Index *indptr, const Index *indices, Index num_nodes,
+                      const Index *seeds, Index n_seed, const Index *fanout, int L,
+                      uint64_t rng_seed, Index *ptr, Index *idx, Index *sub_to_full,
+                      Index *counts) {
+  Index *loc = (Index *)malloc((size_t)num_nodes * sizeof(Index));
+  if (!loc) return ORC_EINVAL;
+  for (Index i = 0; i < num_nodes; ++i) loc[i] = -1;
+  for (Index i = 0; i < n_seed; ++i) {
+    sub_to_full[i] = seeds[i];
+    loc[seeds[i]] = i;
+  }
+  Index lo = 0, hi = n_seed, E = 0;
+  ptr[0] = 0;
+  counts[0] = n_seed;
+  for (int k = 0; k < L; ++k) {
+    Index next = hi;
+    uint64_t hop_key = orc_mix64(rng_seed + (uint64_t)k);
+    for (Index u = lo; u < hi; ++u) {
+      Index f = sub_to_full[u];
+      Index first = indptr[f];
+      Index d = indptr[f + 1] - first;
+      Index c = d < fanout[k] ? d : fanout[k];
+      uint64_t key = orc_mix64(hop_key ^ (uint64_t)f);
+      for (Index j = 0; j < c; ++j) {
+        Index pos = d > fanout[k] ? (Index)orc_sample_perm((uint64_t)j, (uint64_t)d, key) : j;
+        Index v = indices[first + pos];
+        if (loc[v] < 0) {
+          loc[v] = next;
+          sub_to_full[next++] = v;
+        }
+        idx[E++] = loc[v];
+      }
+      ptr[u + 1] = E;
+    }
+    lo = hi;
+    hi = next;
+    counts[k + 1] = hi;
+    counts[L + 1 + k] = E;
+  }
+  free(loc);
+  return ORC_OK;
+}
+

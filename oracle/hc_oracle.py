@@ -332,3 +332,45 @@ def f32_to_f16_bits(x):
 def f32_to_bf16_bits(x):
     x = _f32(x).ravel()
     return np.array([lib().orc_f32_to_bf16(ctypes.c_float(v)) for v in x], np.uint16)
+
+
+# --------------------------------------------------------------------------- sampler
+def mix64(z):
+    f = lib().orc_mix64
+    f.restype = ctypes.c_uint64
+    return int(f(ctypes.c_uint64(int(z) & 0xFFFFFFFFFFFFFFFF)))
+
+
+def sample_perm(j, d, key):
+    f = lib().orc_sample_perm
+    f.restype = ctypes.c_uint64
+    return int(f(ctypes.c_uint64(int(j)), ctypes.c_uint64(int(d)), ctypes.c_uint64(int(key) & 0xFFFFFFFFFFFFFFFF)))
+
+
+def sample_layers(indptr, indices, seeds, fanout, rng_seed):
+    """Sequential statement of the layered sampler.  Returns a dict with ptr, idx, sub_to_full,
+    num_node_in_layer, num_edge_in_layer (NumPy int64), trimmed to their real sizes."""
+    indptr, indices, seeds = _i64(indptr), _i64(indices), _i64(seeds)
+    fan = _i64(np.asarray(fanout))
+    L, n0 = len(fan), len(seeds)
+    rows, edges, nodes = 0, 0, n0
+    r = n0
+    for f in fan:
+        rows += r
+        edges += r * int(f)
+        r = r * int(f)
+        nodes += r
+    N = len(indptr) - 1
+    nodes = min(nodes, max(N, n0))
+    ptr = np.zeros(rows + 1, np.int64)
+    idx = np.zeros(max(edges, 1), np.int64)
+    s2f = np.zeros(nodes, np.int64)
+    counts = np.zeros(2 * L + 1, np.int64)
+    _check(lib().orc_sample_layers(_p(indptr), _p(indices), _I(N), _p(seeds), _I(n0), _p(fan), ctypes.c_int(L),
+                                   ctypes.c_uint64(int(rng_seed) & 0xFFFFFFFFFFFFFFFF), _p(ptr), _p(idx), _p(s2f),
+                                   _p(counts)), "sample_layers")
+    nnl = counts[:L + 1].copy()
+    nel = counts[L + 1:].copy()
+    return {"ptr": ptr[: nnl[L - 1] + 1].copy(), "idx": idx[: nel[-1]].copy(), "sub_to_full": s2f[: nnl[L]].copy(),
+            "num_node_in_layer": nnl, "num_edge_in_layer": nel}
+

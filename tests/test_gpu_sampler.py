@@ -1,0 +1,91 @@
+"""hc_sample_layers through the C ABI against the sequential CPU statement: ptr, idx, sub_to_full
+and the layer sizes bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from test_oracle_sampler import check_batch, simple_graph
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def to_np(batch):
+    return {"ptr": batch.ptr.cpu().numpy(), "idx": batch.idx.cpu().numpy(),
+            "sub_to_full": batch.sub_to_full.cpu().numpy(),
+            "num_node_in_layer": batch.num_node_in_layer.numpy(),
+            "num_edge_in_layer": np.asarray(batch.num_edge_in_layer)}
+
+
+@pytest.mark.parametrize("fanout,n_seed", [([4], 50), ([5, 3], 64), ([15, 10, 5], 200), ([20, 20], 1)])
+def test_sampler_matches_oracle(orc, fanout, n_seed):
+    from hiscache import NeighborSampler
+    rng = np.random.default_rng(200 + len(fanout))
+    indptr, indices = simple_graph(rng, 5000, 30, hubs=5)
+    labels = rng.integers(0, 7, size=5000)
+    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=3, device=DEV)
+    for it in range(4):                         # consecutive batches share the node map
+        seeds = rng.choice(5000, size=n_seed, replace=False).astype(np.int64)
+        print("sampler case", fanout, n_seed, it, flush=True)
+        batch = sampler.sample(torch.from_numpy(seeds).to(DEV))
+        want = orc.sample_layers(indptr, indices, seeds, fanout, sampler.batch_seed(it))
+        got = to_np(batch)
+        for k in want:
+            np.testing.assert_array_equal(got[k], want[k], err_msg=k)
+        np.testing.assert_array_equal(batch.y.cpu().numpy(), labels[seeds])
+        check_batch(got, indptr, indices, seeds, fanout)
+    # the node map is left clean
+    assert int((sampler.node_map != 0x7fffffff).sum()) == 0
+
+
+def test_sampler_multi_edges_and_isolated_nodes(orc):
+    """Adjacency lists with repeated neighbours and nodes without neighbours."""
+    from hiscache import NeighborSampler
+    rng = np.random.default_rng(210)
+    n = 300
+    deg = rng.integers(0, 40, size=n)
+    deg[:20] = 0
+    indptr = np.zeros(n + 1, np.int64)
+    np.cumsum(deg, out=indptr[1:])
+    indices = rng.integers(0, 25, size=int(indptr[-1])).astype(np.int64)     # few targets: many repeats
+    sampler = NeighborSampler(indptr, indices, [6, 6], seed=9, device=DEV)
+    seeds = np.arange(0, 60, dtype=np.int64)
+    batch = sampler.sample(torch.from_numpy(seeds).to(DEV))
+    want = orc.sample_layers(indptr, indices, seeds, [6, 6], sampler.batch_seed(0))
+    got = to_np(batch)
+    for k in want:
+        np.testing.assert_array_equal(got[k], want[k], err_msg=k)
+
+
+def test_sampled_batch_trains(orc):
+    """A batch from the sampler runs through lookup_and_load, the model and update_history."""
+    from hiscache import HistoryCache, HistorySAGE, NeighborSampler, PinnedFeatureStore, make_config
+    rng = np.random.default_rng(220)
+    N, Fin, H, C, L = 4000, 32, 48, 5, 3
+    indptr, indices = simple_graph(rng, N, 12)
+    feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32))
+    labels = rng.integers(0, C, size=N)
+    sampler = NeighborSampler(indptr, indices, [5, 4, 3], labels=labels, seed=1, device=DEV)
+    cfg = make_config(Fin, C, H, L, method="grad", rate=0.6, device=DEV)
+    lcm = int(np.lcm(Fin, H))
+    cache = HistoryCache(PinnedFeatureStore(feats, device=DEV), cfg, "history_uvm", total_num_node=N,
+                         buffer_bytes=600 * lcm * 4, hot_ids=rng.permutation(N).astype(np.int64))
+    model = HistorySAGE(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache).to(DEV)
+    model.train()
+    opt = torch.optim.Adam(model.parameters(), lr=1e-2)
+    losses = []
+    for it in range(6):
+        seeds = torch.from_numpy(rng.choice(N, size=100, replace=False)).to(DEV)
+        batch = sampler.sample(seeds)
+        cache.lookup_and_load(batch, L)
+        np.testing.assert_array_equal(batch.x.cpu().numpy()[cache.used_masks[0].cpu().numpy()],
+                                      feats.numpy()[batch.sub_to_full.cpu().numpy()[cache.used_masks[0].cpu().numpy()]])
+        out = model(batch)
+        loss = torch.nn.functional.nll_loss(out, batch.y)
+        opt.zero_grad()
+        loss.backward()
+        opt.step()
+        cache.update_history(batch, it)
+        losses.append(float(loss.detach()))
+    assert all(np.isfinite(losses))
+    assert cache.header > 0                                   # embeddings were admitted
