@@ -34,7 +34,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c4", "c3", "c5", "copy"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c4", "c3", "c5", "sample", "copy"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
@@ -545,6 +545,94 @@ def run_copy(args):
             "config": {"workload": "copy: 4 GiB fp32 device-to-device copy (4 GiB read + 4 GiB written)"}}
 
 
+def device_power_law_graph(N, mean_degree, dev, gen, max_degree=100_000):
+    """CSR of a directed graph generated on the device: log-normal out-degrees (sigma 1.2) with the
+    given mean, neighbour ids skewed towards popular nodes (u^3 over the id range, scattered by a
+    multiplicative hash).  Multi-edges are possible, as in raw edge lists."""
+    import math
+
+    import torch
+    sigma = 1.2
+    mu = math.log(mean_degree) - sigma * sigma / 2
+    deg = torch.exp(mu + sigma * torch.randn(N, device=dev, generator=gen)).floor_().clamp_(0, max_degree).long()
+    indptr = torch.zeros(N + 1, dtype=torch.int64, device=dev)
+    torch.cumsum(deg, 0, out=indptr[1:])
+    del deg
+    E = int(indptr[-1])
+    indices = torch.empty(E, dtype=torch.int64, device=dev)
+    chunk = 100_000_000
+    for lo in range(0, E, chunk):
+        hi = min(E, lo + chunk)
+        u = torch.rand(hi - lo, device=dev, generator=gen, dtype=torch.float64)
+        v = (u * u * u * N).long().clamp_(0, N - 1)
+        indices[lo:hi] = (v * 2654435761) % N
+        del u, v
+    return indptr, indices
+
+
+def run_sample(args):
+    """Layered neighbour sampling on a papers100M-sized graph resident in HBM: time per batch when
+    the caller waits for it, and what is left on the training thread when the next batch is
+    sampled on the side stream while the current one trains."""
+    import numpy as np
+    import torch
+
+    from hiscache import NeighborSampler
+
+    dev = "cuda:0"
+    s = args.scale
+    N = int(111_000_000 * s)
+    fanout, n_seed = [15, 10, 5], 1000
+    gen = torch.Generator(device=dev).manual_seed(6)
+    indptr, indices = device_power_law_graph(N, 14.5, dev, gen)
+    E_graph = indices.numel()
+    sampler = NeighborSampler(indptr, indices, fanout, seed=6, device=dev, validate=False)
+    seed_sets = [torch.randperm(N, device=dev, generator=gen)[:n_seed].contiguous() for _ in range(16)]
+    clock = KernelClock()
+    shapes = []
+
+    def step(i):
+        b = clock(lambda: sampler.sample(seed_sets[i % len(seed_sets)]))
+        return b
+
+    for i in range(args.warmup):
+        step(i)
+    sync()
+    clock.reset()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        b = step(i)
+        shapes.append(list(b.num_node_in_layer.tolist()) + [b.idx.numel()])
+    sync()
+    sec = (time.perf_counter() - t0) / args.steps
+    # prefetched: batch i+1 is launched before batch i is consumed; the consumer does 1 ms of other work
+    filler = torch.empty(64 << 20, dtype=torch.float32, device=dev)
+    pending = sampler.sample_async(seed_sets[0])
+    waits = []
+    for i in range(args.steps):
+        nxt = sampler.sample_async(seed_sets[(i + 1) % len(seed_sets)])
+        for _ in range(4):
+            filler.add_(1.0)                       # stands for the training iteration
+        torch.cuda.current_stream().synchronize()
+        t1 = time.perf_counter()
+        pending.get()
+        waits.append(time.perf_counter() - t1)
+        pending = nxt
+    pending.get()
+    sync()
+    mean = np.mean(np.asarray(shapes, dtype=np.float64), axis=0)
+    edges = float(mean[-1])
+    return {
+        "metric": "sampled edges per second (1 GPU, layered neighbour sampling)", "value": edges / sec,
+        "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int64", "data": "synthetic",
+        "config": {"workload": "sample: graph of %d nodes / %d edges in HBM, fanout %s, %d seeds; mean batch nodes "
+                               "%s, edges %d" % (N, E_graph, fanout, n_seed, [int(x) for x in mean[:-1]], int(edges))},
+        "device_ms_per_batch": clock.mean_ms(),
+        "wait_ms_when_prefetched": float(np.mean(waits) * 1e3),
+    }
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -568,6 +656,8 @@ def main():
         res = run_copy(args)
     elif args.workload == "c5":
         res = run_c5(args)
+    elif args.workload == "sample":
+        res = run_sample(args)
     else:
         res = run_c3(args)
     print(json.dumps(res))

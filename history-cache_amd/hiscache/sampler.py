@@ -35,7 +35,8 @@ class NeighborSampler:
             if int(self.indptr[-1]) != self.indices.numel() or int(self.indptr[0]) != 0:
                 raise ValueError("indptr does not span indices")
         self.node_map = _be.sample_map(self.num_nodes, self.device)
-        self._counts_host = torch.empty(2 * len(self.fanout) + 1, dtype=torch.int64, pin_memory=True)
+        self._host_pool = []          # pinned read-back buffers for the layer sizes
+        self._stream = None
 
     def batch_seed(self, batch_no):
         """The 64-bit key of batch ``batch_no`` (the sampler's seed and the batch number, mixed)."""
@@ -43,25 +44,68 @@ class NeighborSampler:
 
     def sample(self, seeds, rng_seed=None):
         """Sample the layered sub-graph of ``seeds`` (distinct int64 ids on the device)."""
+        return self.sample_async(seeds, rng_seed, stream=torch.cuda.current_stream(self.device)).get()
+
+    def sample_async(self, seeds, rng_seed=None, stream=None):
+        """Launch the sampling of one batch on the sampler's side stream (or ``stream``) and return a
+        handle; ``handle.get()`` waits for it and returns the batch.  Launching batch i+1 before
+        training on batch i keeps the sampling and its size read-back off the training stream.
+        Batches of one sampler are sampled one after another (they share the node map)."""
         seeds = torch.as_tensor(seeds, dtype=torch.int64).to(self.device).contiguous()
         if rng_seed is None:
             rng_seed = self.batch_seed(self.batches)
         self.batches += 1
+        cur = torch.cuda.current_stream(self.device)
+        if stream is None:
+            if self._stream is None:
+                self._stream = torch.cuda.Stream(device=self.device)   # default priority
+            stream = self._stream
+        if stream != cur:
+            stream.wait_stream(cur)                                    # seeds may have been produced there
+        with torch.cuda.stream(stream):
+            out = _be.sample_layers(self.indptr, self.indices, seeds, self.fanout, rng_seed, self.node_map)
+            counts_host = self._host_pool.pop() if self._host_pool else torch.empty(
+                2 * len(self.fanout) + 1, dtype=torch.int64, pin_memory=True)
+            counts_host.copy_(out[3], non_blocking=True)
+            done = torch.cuda.Event()
+            done.record(stream)
+            y = None if self.labels is None else self.labels[seeds]
+        return _PendingBatch(self, out, counts_host, done, seeds, y, stream)
+
+    def _finish(self, out, counts_host, seeds, y, stream):
+        ptr, idx, s2f, _ = out
         L = len(self.fanout)
-        ptr, idx, s2f, counts = _be.sample_layers(self.indptr, self.indices, seeds, self.fanout, rng_seed,
-                                                  self.node_map)
-        self._counts_host.copy_(counts, non_blocking=True)
-        torch.cuda.current_stream(self.device).synchronize()
-        c = self._counts_host.tolist()
+        c = counts_host.tolist()
+        self._host_pool.append(counts_host)
         nnl, nel = c[: L + 1], c[L + 1:]
+        cur = torch.cuda.current_stream(self.device)
+        if stream != cur:
+            for t in (ptr, idx, s2f, seeds) + (() if y is None else (y,)):
+                t.record_stream(cur)
         return SimpleNamespace(
             ptr=ptr[: nnl[L - 1] + 1],
             idx=idx[: nel[-1]],
             sub_to_full=s2f[: nnl[L]],
             num_node_in_layer=torch.tensor(nnl, dtype=torch.int64),   # on the host, as the model reads it
             num_edge_in_layer=list(nel),
-            y=None if self.labels is None else self.labels[seeds],
+            y=y,
             x=None,
             edge_type=None,
             typed_num_node_in_layer=None,
         )
+
+
+class _PendingBatch:
+    """A batch being sampled; ``get()`` returns it once the device has finished."""
+
+    def __init__(self, sampler, out, counts_host, done, seeds, y, stream):
+        self._args = (sampler, out, counts_host, done, seeds, y, stream)
+        self._batch = None
+
+    def get(self):
+        if self._batch is None:
+            sampler, out, counts_host, done, seeds, y, stream = self._args
+            done.synchronize()
+            self._batch = sampler._finish(out, counts_host, seeds, y, stream)
+            self._args = None
+        return self._batch
