@@ -6,6 +6,7 @@ The trainers and the multi-GPU communication helpers are not part of this packag
 """
 from hiscache_backend import count_history_reconstruct, get_graph_structure_score, record_history
 
+from .dataset import ProcessedDataset, write_processed
 from .feature_store import PinnedFeatureStore
 from .history_cache import HistoryCache
 from .history_model import (HistoryRGCN, HistorySAGE, MyRGCNConvHistory2, MySageConvHistory, get_model,
@@ -17,6 +18,6 @@ from .util import Config, make_config, quantile_threshold
 
 __all__ = [
     "HistoryCache", "HistoryTable", "RingHistoryCache", "HistorySAGE", "HistoryRGCN", "MySageConvHistory", "MyRGCNConvHistory2", "typed_csr", "get_model",
-    "PinnedFeatureStore", "NeighborSampler", "Config", "make_config", "quantile_threshold",
+    "PinnedFeatureStore", "NeighborSampler", "ProcessedDataset", "write_processed", "Config", "make_config", "quantile_threshold",
     "count_history_reconstruct", "get_graph_structure_score", "record_history",
 ]

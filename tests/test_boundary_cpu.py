@@ -101,3 +101,32 @@ def test_config_and_synthetic_batch_layout():
     assert len(np.unique(d["sub_to_full"])) == len(d["sub_to_full"])
     deg = zipf_degrees(10000, 200000, 2.1, 5000, rng)
     assert deg.sum() == 200000 and deg.min() >= 1 and deg.max() <= 5000
+
+
+def test_processed_dataset_files_round_trip(tmp_path):
+    """The on-disk layout of /root/reference/hiscache/history_cache.py:17-20,124-142 and
+    test/test_cache.py:19-56: raw int64 / float arrays plus num_nodes.txt."""
+    from hiscache import ProcessedDataset, write_processed
+    from hiscache.synthetic import uniform_graph
+    rng = np.random.default_rng(5)
+    indptr, indices = uniform_graph(200, 6, 5)
+    feats = rng.standard_normal((200, 12)).astype(np.float16)
+    hot = rng.permutation(200)
+    labels = rng.integers(0, 4, size=200)
+    train = rng.choice(200, size=50, replace=False)
+    d = write_processed(tmp_path, indptr, indices, feats, hot, labels, train)
+    assert open(os.path.join(d, "num_nodes.txt")).read().strip() == "200"
+    assert os.path.getsize(os.path.join(d, "node_features.dat")) == 200 * 12 * 2
+    ds = ProcessedDataset(tmp_path, 12, np.float16)
+    assert ds.num_nodes == 200
+    p, i = ds.graph()
+    np.testing.assert_array_equal(p, indptr)
+    np.testing.assert_array_equal(i, indices)
+    np.testing.assert_array_equal(ds.hot_ids(), hot)
+    np.testing.assert_array_equal(ds.labels(), labels)
+    np.testing.assert_array_equal(ds.train_idx(), train)
+    np.testing.assert_array_equal(np.fromfile(os.path.join(d, "sorted_indices.dat"), dtype=np.int64), hot)
+    # a truncated CSR file is refused
+    np.asarray(indices[:-3], np.int64).tofile(os.path.join(d, "csr_idx_undirected.dat"))
+    with pytest.raises(ValueError):
+        ds.graph()

@@ -89,3 +89,42 @@ def test_sampled_batch_trains(orc):
         losses.append(float(loss.detach()))
     assert all(np.isfinite(losses))
     assert cache.header > 0                                   # embeddings were admitted
+
+
+def test_training_from_processed_files(tmp_path):
+    """Dataset directory -> feature store, sampler and cache (which reads num_nodes.txt and
+    sorted_indices.dat itself) -> a few training iterations."""
+    from hiscache import HistoryCache, HistorySAGE, ProcessedDataset, make_config, write_processed
+    rng = np.random.default_rng(230)
+    N, Fin, H, C, L = 3000, 16, 32, 4, 3
+    indptr, indices = simple_graph(rng, N, 10)
+    feats = rng.standard_normal((N, Fin)).astype(np.float32)
+    write_processed(tmp_path, indptr, indices, feats, hot_ids=rng.permutation(N), labels=rng.integers(0, C, size=N),
+                    train_idx=rng.choice(N, size=600, replace=False))
+    ds = ProcessedDataset(tmp_path, Fin)
+    store = ds.feature_store(device=DEV)
+    np.testing.assert_array_equal(store.get(torch.tensor([0, 5, N - 1], device=DEV)).cpu().numpy(),
+                                  feats[[0, 5, N - 1]])
+    sampler = ds.sampler([4, 3, 2], device=DEV, seed=2)
+    cfg = make_config(Fin, C, H, L, method="grad", rate=0.6, device=DEV, path=str(tmp_path))
+    cache = HistoryCache(store, cfg, "history_uvm", buffer_bytes=500 * int(np.lcm(Fin, H)) * 4)
+    assert cache.total_num_node == N
+    model = HistorySAGE(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache).to(DEV)
+    model.train()
+    opt = torch.optim.Adam(model.parameters(), lr=1e-2)
+    train = torch.from_numpy(ds.train_idx()).to(DEV)
+    pending = sampler.sample_async(train[:100])
+    for it in range(5):
+        batch = pending.get()
+        pending = sampler.sample_async(train[100 * (it + 1): 100 * (it + 2)])     # next batch in flight
+        cache.lookup_and_load(batch, L)
+        um = cache.used_masks[0].cpu().numpy()
+        np.testing.assert_array_equal(batch.x.cpu().numpy()[um], feats[batch.sub_to_full.cpu().numpy()[um]])
+        loss = torch.nn.functional.nll_loss(model(batch), batch.y)
+        opt.zero_grad()
+        loss.backward()
+        opt.step()
+        cache.update_history(batch, it)
+        assert np.isfinite(float(loss.detach()))
+    pending.get()
+    assert cache.header > 0
