@@ -135,7 +135,11 @@ class CpuSage(torch.nn.Module):
 
     def __init__(self, model):
         super().__init__()
-        self.m = copy.deepcopy(model).cpu()
+        table, model.table = model.table, None          # the cache (streams, device buffers) is not copied
+        try:
+            self.m = copy.deepcopy(model).cpu()
+        finally:
+            model.table = table
 
     def forward(self, batch, x, sub2embed, cached_embedding):
         from oracle import torch_cpu_path as tp
@@ -149,6 +153,8 @@ class CpuSage(torch.nn.Module):
                 agg = mean_rows(x, batch.ptr, batch.idx, n)
                 hit = (sub2embed != -1)[:, None]
                 agg = torch.where(hit, cached_embedding, agg)
+                if not agg.requires_grad:               # history layer on raw features (2-layer models)
+                    agg.requires_grad_(True)
                 agg.retain_grad()
                 his_out = agg
             else:
