@@ -221,7 +221,7 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     for (int64_t c = lane; c < hsize; c += HC_WAVE) d[c] = (hit && c < F) ? s[c] : 0.0f;
     return;
   }
-  const int64_t s0 = ((int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + wave) * S;
+  const int64_t s0 = (hc_xcd_block((int64_t)blockIdx.x, src_blocks) * HC_WAVES_PER_BLOCK + wave) * S;
   if (s0 >= n_src) return;
   const int64_t rest = n_src - s0;
   const int ns = rest < S ? (int)rest : S;
@@ -248,7 +248,7 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     while (cur < ns && base >= cur_end) {
       if (((hub_mask >> cur) & 1ull) == 0ull) {
 #pragma unroll
-        for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store(obase + (int64_t)cur * F + k * HC_WAVE * VEC, acc[k]);
+        for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store_nt(obase + (int64_t)cur * F + k * HC_WAVE * VEC, acc[k]);
       }
 #pragma unroll
       for (int k = 0; k < CHUNKS; ++k)
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
           while (e >= cur_end) {  // close finished (possibly empty) segments; none of them is a hub
 #pragma unroll
             for (int k = 0; k < CHUNKS; ++k) {
-              hc_vec<float, VEC>::store(obase + (int64_t)cur * F + k * HC_WAVE * VEC, acc[k]);
+              hc_vec<float, VEC>::store_nt(obase + (int64_t)cur * F + k * HC_WAVE * VEC, acc[k]);
 #pragma unroll
               for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
             }

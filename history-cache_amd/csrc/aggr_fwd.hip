@@ -58,7 +58,10 @@ __device__ __forceinline__ void copy_row_any(const void *hbuf, int hist_dtype, i
 // src_mode == 1: per-source substitution (hbuf is a table of the same dtype as vin).
 // ---------------------------------------------------------------------------------------
 // Sum of the neighbour rows of edges [begin, end), added to acc in edge order by the calling wave.
-template <typename T, int VEC, int CHUNKS, int UNROLL>
+// STREAM: neighbour rows and ids are loaded with the non-temporal hint.  With per-source
+// substitution every edge also looks its source up in the map, and the map (not the rows, which
+// are too many to be reused) is what is worth keeping in the caches.
+template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM>
 __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, const T *__restrict__ vin,
                                                const int64_t *__restrict__ hmap, const T *__restrict__ htab,
                                                int64_t hsize, int src_mode, int64_t begin, int64_t end,
@@ -70,7 +73,7 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
     // Stage: lane l resolves the address of neighbour base+l.
     int64_t my_addr = 0;
     if (lane < n) {
-      const int64_t id = idx[base + lane];
+      const int64_t id = STREAM ? __builtin_nontemporal_load(idx + base + lane) : idx[base + lane];
       const T *p = vin + id * F;
       if (src_mode && hmap != nullptr) {
         const int64_t slot = hmap[id];
@@ -85,7 +88,10 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
         if (j + u < n) {
           const T *p = reinterpret_cast<const T *>(hc_readlane64(my_addr, j + u)) + lane * VEC;
 #pragma unroll
-          for (int k = 0; k < CHUNKS; ++k) hc_vec<T, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
+          for (int k = 0; k < CHUNKS; ++k) {
+            if constexpr (STREAM) hc_vec<T, VEC>::load_nt(p + k * HC_WAVE * VEC, v[u][k]);
+            else hc_vec<T, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
+          }
         } else {
 #pragma unroll
           for (int k = 0; k < CHUNKS; ++k)
@@ -112,7 +118,7 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
 // long_thres == 0 disables the split (every row is then summed strictly in CSR order).
 constexpr int FWD_ROWS_PER_BLOCK = HC_WAVES_PER_BLOCK;
 
-template <typename T, int VEC, int CHUNKS, int UNROLL>
+template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM>
 __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const T *__restrict__ vin,
     const int64_t *__restrict__ hmap, const void *__restrict__ hbuf, int hist_dtype, int64_t hsize,
@@ -124,7 +130,7 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
   const int lane = hc_lane();
   const int wave = hc_wave_in_block();
   const T *__restrict__ htab = static_cast<const T *>(hbuf);
-  const int64_t row0 = (int64_t)blockIdx.x * FWD_ROWS_PER_BLOCK;
+  const int64_t row0 = hc_xcd_block((int64_t)blockIdx.x, (int64_t)gridDim.x) * FWD_ROWS_PER_BLOCK;
   const int64_t rest = R - row0;
   const int nrows = rest < FWD_ROWS_PER_BLOCK ? (int)rest : FWD_ROWS_PER_BLOCK;
 
@@ -153,14 +159,15 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
         for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
           for (int i = 0; i < VEC; ++i) acc[c][i] = 0.0f;
-        fwd_accumulate<T, VEC, CHUNKS, UNROLL>(idx, vin, hmap, htab, hsize, src_mode, begin, end, lane, acc);
+        fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM>(idx, vin, hmap, htab, hsize, src_mode, begin, end, lane, acc);
         const float fdeg = (float)(int)deg;
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) {
           float o[VEC];
 #pragma unroll
           for (int i = 0; i < VEC; ++i) o[i] = deg > 0 ? acc[c][i] / fdeg : 0.0f;
-          hc_store_f32<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
+          if constexpr (STREAM) hc_store_f32_nt<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
+          else hc_store_f32<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
         }
       }
     }
@@ -183,7 +190,7 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
     for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
       for (int i = 0; i < VEC; ++i) acc[c][i] = 0.0f;
-    fwd_accumulate<T, VEC, CHUNKS, UNROLL>(idx, vin, hmap, htab, hsize, src_mode, sb, se, lane, acc);
+    fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM>(idx, vin, hmap, htab, hsize, src_mode, sb, se, lane, acc);
     if (wave > 0) {
 #pragma unroll
       for (int c = 0; c < CHUNKS; ++c)
@@ -204,7 +211,8 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
           for (int pw = 0; pw < HC_WAVES_PER_BLOCK - 1; ++pw) t2 += part[pw][(c * HC_WAVE + lane) * VEC + i];
           o[i] = t2 / fdeg;
         }
-        hc_store_f32<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
+        if constexpr (STREAM) hc_store_f32_nt<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
+        else hc_store_f32<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
       }
     }
     __syncthreads();
@@ -290,9 +298,14 @@ int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const i
   constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
   const int64_t blocks = (R + FWD_ROWS_PER_BLOCK - 1) / FWD_ROWS_PER_BLOCK;
   if (!hc_grid_ok(blocks)) return HC_EUNSUPPORTED;
-  fwd_mean_fast<T, VEC, CHUNKS, UNROLL><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(
-      ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, vout, R,
-      (int64_t)HC_LONG_ROW_EDGES);
+  if (src_mode && hmap != nullptr)
+    fwd_mean_fast<T, VEC, CHUNKS, UNROLL, true><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(
+        ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, vout, R,
+        (int64_t)HC_LONG_ROW_EDGES);
+  else
+    fwd_mean_fast<T, VEC, CHUNKS, UNROLL, false><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(
+        ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, vout, R,
+        (int64_t)HC_LONG_ROW_EDGES);
   return hc_launch_status();
 }
 

@@ -77,7 +77,11 @@ __device__ __forceinline__ float wave_scores(const float *__restrict__ grad, int
         if (r < M) {
           const float4 *p = reinterpret_cast<const float4 *>(grad + r * (256 * CH)) + lane;
 #pragma unroll
-          for (int k = 0; k < CH; ++k) v[i][k] = p[k * HC_WAVE];
+          for (int k = 0; k < CH; ++k) {
+            float t[4];
+            hc_vec<float, 4>::load_nt(reinterpret_cast<const float *>(p + k * HC_WAVE), t);
+            v[i][k] = make_float4(t[0], t[1], t[2], t[3]);
+          }
         } else {
 #pragma unroll
           for (int k = 0; k < CH; ++k) v[i][k] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -235,8 +239,8 @@ __device__ __forceinline__ void store_row(const float *__restrict__ src, TT *__r
   if (vec_ok) {
     for (int64_t c = (int64_t)lane * 4; c < F; c += HC_WAVE * 4) {
       float v[4];
-      hc_vec<float, 4>::load(src + c, v);
-      hc_vec<TT, 4>::store(dst + c, v);
+      hc_vec<float, 4>::load_nt(src + c, v);
+      hc_vec<TT, 4>::store_nt(dst + c, v);
     }
   } else {
     for (int64_t c = lane; c < F; c += HC_WAVE) dst[c] = hc_from_f32<TT>(src[c]);

@@ -53,6 +53,18 @@ __device__ __forceinline__ float hc_readlane_f(float v, int lane) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
 
+// Workgroups are handed to the 8 XCDs round-robin (workgroup i runs on XCD i % 8) and every XCD
+// has its own L2.  This maps the hardware block index to a logical one so that each XCD works
+// through one contiguous eighth of the logical range: neighbouring rows or sources, which tend to
+// touch the same data, then share an L2.  A bijection of [0, n).
+#define HC_NUM_XCD 8
+__device__ __forceinline__ int64_t hc_xcd_block(int64_t bid, int64_t n) {
+  const int64_t per = n / HC_NUM_XCD;
+  const int64_t body = per * HC_NUM_XCD;
+  if (bid >= body) return bid;
+  return (bid % HC_NUM_XCD) * per + bid / HC_NUM_XCD;
+}
+
 // Butterfly sum over the 64 lanes, partner distance 32,16,8,4,2,1.  Every lane
 // ends with the same bits (fp add is commutative), and the order is the one
 // the CPU checker reproduces.
@@ -118,6 +130,37 @@ struct hc_vec {
     for (int i = 0; i < VEC; ++i) u.e[i] = hc_from_f32<T>(in[i]);
     *reinterpret_cast<raw_t *>(p) = u.raw;
   }
+  // Same load / store with the non-temporal hint: rows that are read or written once should not
+  // displace the index and map lines that are reused.
+  typedef uint32_t nt_t __attribute__((ext_vector_type(sizeof(T) * VEC >= 4 ? sizeof(T) * VEC / 4 : 1)));
+  __device__ __forceinline__ static void load_nt(const T *p, float (&out)[VEC]) {
+    if constexpr (sizeof(T) * VEC >= 4) {
+      union N {
+        nt_t raw;
+        T e[VEC];
+        __device__ N() {}
+      } u;
+      u.raw = __builtin_nontemporal_load(reinterpret_cast<const nt_t *>(p));
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) out[i] = hc_to_f32<T>(u.e[i]);
+    } else {
+      load(p, out);
+    }
+  }
+  __device__ __forceinline__ static void store_nt(T *p, const float (&in)[VEC]) {
+    if constexpr (sizeof(T) * VEC >= 4) {
+      union N {
+        nt_t raw;
+        T e[VEC];
+        __device__ N() {}
+      } u;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) u.e[i] = hc_from_f32<T>(in[i]);
+      __builtin_nontemporal_store(u.raw, reinterpret_cast<nt_t *>(p));
+    } else {
+      store(p, in);
+    }
+  }
 };
 
 // Store VEC consecutive fp32 values (VEC may exceed one 16-byte store).
@@ -130,6 +173,20 @@ __device__ __forceinline__ void hc_store_f32(float *p, const float (&in)[VEC]) {
     for (int q = 0; q < VEC / 4; ++q) {
       const float t[4] = {in[4 * q], in[4 * q + 1], in[4 * q + 2], in[4 * q + 3]};
       hc_vec<float, 4>::store(p + 4 * q, t);
+    }
+  }
+}
+
+// Same with the non-temporal hint (output rows that this launch does not read again).
+template <int VEC>
+__device__ __forceinline__ void hc_store_f32_nt(float *p, const float (&in)[VEC]) {
+  if constexpr (VEC <= 4) {
+    hc_vec<float, VEC>::store_nt(p, in);
+  } else {
+#pragma unroll
+    for (int q = 0; q < VEC / 4; ++q) {
+      const float t[4] = {in[4 * q], in[4 * q + 1], in[4 * q + 2], in[4 * q + 3]};
+      hc_vec<float, 4>::store_nt(p + 4 * q, t);
     }
   }
 }

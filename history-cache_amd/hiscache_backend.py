@@ -20,7 +20,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libhiscache_hip.so")
+# HISCACHE_HIP_LIB overrides the location of the built library (default: next to this file)
+LIB_PATH = os.environ.get("HISCACHE_HIP_LIB") or os.path.join(_HERE, "libhiscache_hip.so")
 
 # enums of include/hiscache_hip.h
 HC_F32, HC_F16, HC_BF16 = 0, 1, 2
