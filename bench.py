@@ -26,7 +26,7 @@ sys.path.insert(0, os.path.join(ROOT, "history-cache_amd"))
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel at full size, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of this file (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000: factors from a 4 GiB device copy).
-MEASURED_TRAFFIC = {"c2": 24.30e9, "c2row": 13.98e9, "c4": 3.50e9}
+MEASURED_TRAFFIC = {"c2": 24.21e9, "c2row": 13.93e9, "c4": 3.50e9}
 
 
 def parse():
@@ -170,7 +170,7 @@ def run_c2(args, row_mode=False):
                    ": history_aggr microbench, R=%d rows, E=%d edges (Zipf 2.1, max deg 5000), %d sources x %d fp32, "
                    "40%% history hits (%s substitution), mean fwd + transpose build + bwd"
                    % (R, E, N, F, "per-row" if row_mode else "per-source")},
-        "roofline": {"bound": "hbm", "kernel": "fwd_mean_fast<float,4,1>", "achieved": bytes_f / (t_f * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "kernel": "fwd_mean_fast<float,4,1,8,%s>" % ("false" if row_mode else "true"), "achieved": bytes_f / (t_f * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_f / (t_f * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC["c2row" if row_mode else "c2"] if s == 1.0 else None,
                      "algorithmic_bytes": bytes_f, "launch_ms": t_f},
