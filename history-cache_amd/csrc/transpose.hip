@@ -7,13 +7,13 @@
 // ascending destination-row order, so the backward sums have one fixed order.
 //
 // Pipeline (all on the caller's stream):
-//   1. fill      keys[e] = n_src (sentinel) for every edge slot
-//   2. expand    wave per row: keys[e] = idx[e], rows[e] = r for the row's edges
-//                (rows flagged by hmap_row are skipped and keep the sentinel)
-//   3. sort      rocPRIM LSD radix sort of (key, value) pairs -- stable.  When the caller wants
+//   1. expand    thread per edge slot: keys[e] = idx[e] and the slot's destination row (found by
+//                binary search over the row offsets of the block's tile); slots outside the first R
+//                rows and rows flagged by hmap_row get the sentinel key n_src
+//   2. sort      rocPRIM LSD radix sort of (key, value) pairs -- stable.  When the caller wants
 //                edgeT the value is the edge slot and rowT is gathered afterwards; when it does not
 //                (mean aggregation) the value is the destination row and the sort writes rowT itself
-//   4. finalize  ptrT[s] = first sorted position whose key is >= s
+//   3. finalize  ptrT[s] = first sorted position whose key is >= s
 #include <cstring>
 
 #include <rocprim/rocprim.hpp>
@@ -22,36 +22,68 @@
 
 namespace {
 
-__global__ __launch_bounds__(HC_BLOCK) void tr_fill(uint32_t *__restrict__ keys,
-                                                     uint32_t *__restrict__ vals, int64_t E,
-                                                     uint32_t sentinel) {
-  const int64_t e = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
-  if (e < E) {
-    keys[e] = sentinel;
-    vals[e] = (uint32_t)e;
+// Sort input for every edge slot, one thread per slot: key = source id, or the sentinel for slots
+// outside the first R rows, rows flagged by hmap_row and ids outside [0, n_src); value = edge slot
+// (VAL_IS_ROW false; `rows[e]` then gets the destination row) or the destination row itself (mean
+// aggregation; dropped slots carry their slot number, they sort behind every real key).
+// A block covers TR_TILE consecutive slots.  The rows that overlap the tile are found with two
+// binary searches; their offsets are staged in LDS when they fit, and every thread then finds the
+// row of its slot with a short search.  Reads and writes are coalesced whatever the degrees are.
+constexpr int TR_ITEMS = 8;
+constexpr int TR_TILE = HC_BLOCK * TR_ITEMS;
+constexpr int TR_LDS_ROWS = 2048;
+
+// largest r in [lo, hi] with ptr[r] <= e (ptr[lo] <= e is the caller's business)
+template <typename P>
+__device__ __forceinline__ int64_t tr_row_of(P ptr, int64_t lo, int64_t hi, int64_t e) {
+  while (lo < hi) {
+    const int64_t mid = (lo + hi + 1) >> 1;
+    if (ptr[mid] <= e) lo = mid;
+    else hi = mid - 1;
   }
+  return lo;
 }
 
-__global__ __launch_bounds__(HC_BLOCK) void tr_expand(const int64_t *__restrict__ ptr,
-                                                       const int64_t *__restrict__ idx,
-                                                       const int64_t *__restrict__ hmap_row,
-                                                       uint32_t *__restrict__ keys,
-                                                       uint32_t *__restrict__ rows, int64_t R,
-                                                       int64_t E, int64_t n_src) {
-  // `rows` is indexed by edge slot: either the side array for the later gather, or the sort's
-  // value array itself (mean aggregation)
-  const int lane = hc_lane();
-  const int64_t row = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
-  if (row >= R) return;
-  if (hmap_row != nullptr && hmap_row[row] != -1) return;
-  const int64_t begin = ptr[row];
-  int64_t end = ptr[row + 1];
-  if (end > E) end = E;
-  for (int64_t e = begin + lane; e < end; e += HC_WAVE) {
-    const int64_t s = idx[e];
-    // ids outside [0, n_src) keep the sentinel and drop out of the view
-    if (s >= 0 && s < n_src) keys[e] = (uint32_t)s;
-    rows[e] = (uint32_t)row;
+template <bool VAL_IS_ROW>
+__global__ __launch_bounds__(HC_BLOCK) void tr_expand_edges(const int64_t *__restrict__ ptr,
+                                                             const int64_t *__restrict__ idx,
+                                                             const int64_t *__restrict__ hmap_row,
+                                                             uint32_t *__restrict__ keys,
+                                                             uint32_t *__restrict__ vals,
+                                                             uint32_t *__restrict__ rows, int64_t R, int64_t E,
+                                                             int64_t n_src) {
+  __shared__ int64_t s_ptr[TR_LDS_ROWS];
+  __shared__ int64_t s_range[2];
+  const int64_t e0 = (int64_t)blockIdx.x * TR_TILE;
+  const int64_t e1 = e0 + TR_TILE < E ? e0 + TR_TILE : E;
+  if (threadIdx.x < 2) s_range[threadIdx.x] = tr_row_of(ptr, (int64_t)0, R, threadIdx.x == 0 ? e0 : e1 - 1);
+  __syncthreads();
+  const int64_t r_lo = s_range[0], r_hi = s_range[1];
+  const int64_t span = r_hi - r_lo + 1;  // rows r_lo..r_hi (r_hi may be R: slots behind the last row)
+  const bool staged = span <= TR_LDS_ROWS;
+  if (staged)
+    for (int64_t i = threadIdx.x; i < span; i += HC_BLOCK) s_ptr[i] = ptr[r_lo + i];
+  __syncthreads();
+  const uint32_t sentinel = (uint32_t)n_src;
+#pragma unroll
+  for (int it = 0; it < TR_ITEMS; ++it) {
+    const int64_t e = e0 + (int64_t)it * HC_BLOCK + threadIdx.x;
+    if (e >= e1) break;
+    const int64_t row = staged ? r_lo + tr_row_of(s_ptr, (int64_t)0, span - 1, e) : tr_row_of(ptr, r_lo, r_hi, e);
+    uint32_t key = sentinel;
+    bool live = row < R && ptr[row] <= e;  // ptr[row + 1] > e by construction when row < R
+    if (live && hmap_row != nullptr && hmap_row[row] != -1) live = false;
+    if (live) {
+      const int64_t s = idx[e];
+      if (s >= 0 && s < n_src) key = (uint32_t)s;
+    }
+    keys[e] = key;
+    if (VAL_IS_ROW) {
+      vals[e] = live ? (uint32_t)row : (uint32_t)e;
+    } else {
+      vals[e] = (uint32_t)e;
+      if (live) rows[e] = (uint32_t)row;
+    }
   }
 }
 
@@ -213,9 +245,10 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
   const bool want_edges = edgeT != nullptr;
   const unsigned bits = (unsigned)key_bits(n_src);
   const uint32_t *skeys = nullptr;
-  tr_fill<<<dim3((unsigned)eblocks), dim3(HC_BLOCK), 0, st>>>(keys0, vals0, E, sentinel);
+  const int64_t tblocks = (E + TR_TILE - 1) / TR_TILE;
   if (want_edges) {
-    tr_expand<<<dim3((unsigned)rblocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, rows, R, E, n_src);
+    tr_expand_edges<false><<<dim3((unsigned)tblocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, rows,
+                                                                              R, E, n_src);
     rocprim::double_buffer<uint32_t> dk(keys0, keys1), dv(vals0, vals1);
     if (rocprim::radix_sort_pairs(temp, temp_bytes, dk, dv, (size_t)E, 0u, bits, st, false) != hipSuccess)
       return HC_ELAUNCH;
@@ -224,7 +257,8 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
     skeys = dk.current();
   } else {
     // value = destination row; dropped edge slots keep the fill value and sort behind the sentinel
-    tr_expand<<<dim3((unsigned)rblocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, R, E, n_src);
+    tr_expand_edges<true><<<dim3((unsigned)tblocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, nullptr,
+                                                                             R, E, n_src);
     // rowT doubles as the sort's second value buffer; copy only if the result landed in the first
     uint32_t *rowT_u = reinterpret_cast<uint32_t *>(rowT);
     rocprim::double_buffer<uint32_t> dk(keys0, keys1), dv(vals0, rowT_u);
