@@ -253,13 +253,17 @@ def run_c4(args):
 
     sec = timed_steps(step, args.steps, args.warmup)
     A = int(state["mask"].sum())
+    # rows whose score sits within 4 ulp of the threshold (a differently ordered sum could flip them)
+    score = be.row_scores(grad)
+    guard = int(((score.view(torch.int32) - thres.view(torch.int32)).abs() <= 4).sum())
     bytes_ = M * F * 4 + M * 13 + M + A * (F * 4 + F * 2 + 32)
     return {
         "metric": "grad_check admission rows/sec", "value": M / sec, "unit": "rows/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "c4: grad_check microbench, %d rows x %d fp32 grads (lognormal norms), ages in [0,20], "
-                               "thres 0.05, age limit 10, fp16 table %d x %d; admitted %d" % (M, F, cap, F, A)},
+                               "thres 0.05, age limit 10, fp16 table %d x %d; admitted %d; %d rows within 4 ulp of the "
+                               "threshold" % (M, F, cap, F, A, guard)},
         "roofline": {"bound": "hbm", "kernel": "gc_pass1+gc_pass2+gc_pass3_ring", "achieved": bytes_ / sec / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_ / sec / 1e9 / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC["c4"] if s == 1.0 else None, "algorithmic_bytes": bytes_},

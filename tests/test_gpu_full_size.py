@@ -1,0 +1,174 @@
+"""The microbenchmark configurations at their full sizes, checked through properties that do not need a
+CPU pass over 20 M edges: closed forms on a random sample of rows, weighted column sums (a checksum of
+the whole output), the adjoint identity between forward and backward, sortedness and permutation
+checksums of the transposed view, the prefix-sum slot rule of the admission pass, and run-to-run
+bit-identity.  Reference values are computed with torch ops in fp64 on the device, a path that
+shares nothing with the library.  Tolerance: 1e-5 relative for fp32 sums; integer results exact."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+R, E, N, F = 1_000_000, 20_000_000, 10_000_000, 256
+
+
+@pytest.fixture(scope="module")
+def c2():
+    import hiscache_backend as be
+    from hiscache.synthetic import power_law_block
+    ptr, idx = power_law_block(R, E, N, alpha=2.1, max_degree=5000, seed=2)
+    ptr, idx = ptr.to(DEV), idx.to(DEV)
+    gen = torch.Generator(device=DEV).manual_seed(2)
+    feat = torch.randn(N, F, device=DEV, generator=gen)
+    g = torch.randn(R, F, device=DEV, generator=gen)
+    hist = 0.5 * torch.randn(N, F, device=DEV, generator=gen)
+    hmap = torch.where(torch.rand(N, device=DEV, generator=gen) < 0.4, torch.arange(N, device=DEV),
+                       torch.full((N,), -1, device=DEV))
+    print("full-size c2 block built", flush=True)
+    out = be._aggr_fwd(be.SUBST_SRC, ptr, idx, feat, hmap, hist, F, None, R)
+    tr = be.build_transpose(ptr, idx, None, R, N, want_edges=False)
+    grad_x, _, _ = be._aggr_bwd(ptr, idx, tr, g, None, None, feat, False, None, 0, R, N)
+    torch.cuda.synchronize()
+    yield dict(ptr=ptr, idx=idx, feat=feat, g=g, hist=hist, hmap=hmap, out=out, tr=tr, grad_x=grad_x)
+    torch.cuda.empty_cache()
+
+
+def substituted_rows(c, ids):
+    """fp64 rows the per-source rule reads for source ids ``ids``."""
+    slot = c["hmap"][ids]
+    hit = slot != -1
+    rows = c["feat"][ids].double()
+    rows[hit] = c["hist"][slot[hit]].double()
+    return rows
+
+
+def test_c2_forward_sample_rows_closed_form(c2):
+    gen = torch.Generator(device=DEV).manual_seed(11)
+    deg = c2["ptr"][1:] - c2["ptr"][:-1]
+    sample = torch.randint(0, R, (3000,), device=DEV, generator=gen)
+    sample = torch.cat([sample, torch.topk(deg, 8).indices])         # and the longest rows (quarter split)
+    starts, ends = c2["ptr"][sample], c2["ptr"][sample + 1]
+    worst = 0.0
+    for r, b, e in zip(sample.tolist(), starts.tolist(), ends.tolist()):
+        want = substituted_rows(c2, c2["idx"][b:e]).sum(0) / max(e - b, 1)
+        got = c2["out"][r].double()
+        err = float((got - want).abs().max() / want.abs().max().clamp(min=1e-30))
+        worst = max(worst, err)
+    assert worst < 1e-5, worst
+
+
+def test_c2_forward_weighted_column_sums(c2):
+    """sum_r deg(r) * out[r, :] == sum over all edges of the substituted source row."""
+    deg = (c2["ptr"][1:] - c2["ptr"][:-1]).double()
+    lhs = (c2["out"].double() * deg[:, None]).sum(0)
+    rhs = torch.zeros(F, dtype=torch.float64, device=DEV)
+    for lo in range(0, E, 2_000_000):
+        rhs += substituted_rows(c2, c2["idx"][lo:lo + 2_000_000]).sum(0)
+    scale = float(rhs.abs().max())
+    assert float((lhs - rhs).abs().max()) < 1e-5 * scale + 1e-3
+
+
+def test_c2_adjoint_identity(c2):
+    """<fwd(x), g> == <x, bwd(g)> over the substituted source rows (the forward is linear in them)."""
+    lhs = float((c2["out"].double() * c2["g"].double()).sum())
+    rhs = 0.0
+    for lo in range(0, N, 1_000_000):
+        ids = torch.arange(lo, min(N, lo + 1_000_000), device=DEV)
+        rhs += float((substituted_rows(c2, ids) * c2["grad_x"][ids].double()).sum())
+    assert abs(lhs - rhs) < 1e-5 * max(abs(lhs), abs(rhs)) + 1e-2, (lhs, rhs)
+
+
+def test_c2_backward_sample_sources_closed_form(c2):
+    ptrT, rowT, _ = c2["tr"]
+    gen = torch.Generator(device=DEV).manual_seed(12)
+    deg = (c2["ptr"][1:] - c2["ptr"][:-1]).double()
+    sample = torch.randint(0, N, (3000,), device=DEV, generator=gen)
+    worst = 0.0
+    for s, b, e in zip(sample.tolist(), ptrT[sample].tolist(), ptrT[sample + 1].tolist()):
+        rows = rowT[b:e].long()
+        want = (c2["g"][rows].double() / deg[rows][:, None]).sum(0)
+        got = c2["grad_x"][s].double()
+        worst = max(worst, float((got - want).abs().max() / want.abs().max().clamp(min=1e-30)) if e > b
+                    else float(got.abs().max()))
+    assert worst < 1e-5, worst
+
+
+def test_c2_transposed_view_is_a_sorted_stable_permutation(c2):
+    ptrT, rowT, _ = c2["tr"]
+    ptr, idx = c2["ptr"], c2["idx"]
+    assert int(ptrT[0]) == 0 and int(ptrT[N]) == E
+    seg = ptrT[1:] - ptrT[:-1]
+    assert int(seg.min()) >= 0
+    # segment sizes are the in-degrees
+    assert torch.equal(seg, torch.bincount(idx, minlength=N))
+    # inside a segment destination rows ascend (stable sort of a row-major edge list)
+    src_of = torch.repeat_interleave(torch.arange(N, device=DEV), seg)
+    same = src_of[1:] == src_of[:-1]
+    assert bool((rowT[1:][same] >= rowT[:-1][same]).all())
+    # the view is a permutation of the edge list: two independent checksums over (source, row) pairs
+    row_of = torch.repeat_interleave(torch.arange(R, device=DEV), ptr[1:] - ptr[:-1])
+    for a, b in ((1_000_003, 998_244_353), (7, 1_000_000_007)):
+        want = int(((idx * a + row_of * b) % 2_147_483_647).sum())
+        got = int(((src_of * a + rowT.long() * b) % 2_147_483_647).sum())
+        assert want == got
+
+
+def test_c2_results_are_bit_identical_run_to_run(c2):
+    import hiscache_backend as be
+    out = be._aggr_fwd(be.SUBST_SRC, c2["ptr"], c2["idx"], c2["feat"], c2["hmap"], c2["hist"], F, None, R)
+    assert torch.equal(out, c2["out"])
+    tr = be.build_transpose(c2["ptr"], c2["idx"], None, R, N, want_edges=False)
+    assert torch.equal(tr[0], c2["tr"][0]) and torch.equal(tr[1], c2["tr"][1])
+    grad_x, _, _ = be._aggr_bwd(c2["ptr"], c2["idx"], tr, c2["g"], None, None, c2["feat"], False, None, 0, R, N)
+    assert torch.equal(grad_x, c2["grad_x"])
+
+
+def test_c4_admission_full_size():
+    """2 M rows x 256, fp16 table 50 M x 256: mask == predicate on the kernel's own scores, slots ==
+    header + exclusive prefix sum of the mask, table rows == fp16(embedding), maps consistent."""
+    import hiscache_backend as be
+    from hiscache.synthetic import lognormal_grads
+    M, cap = 2_000_000, 50_000_000
+    gen = torch.Generator(device=DEV).manual_seed(4)
+    grad = lognormal_grads(M, F, -3.0, 1.5, device=DEV, generator=gen)
+    emb = torch.randn(M, F, device=DEV, generator=gen)
+    age = torch.randint(0, 21, (M,), device=DEV, generator=gen, dtype=torch.int32)
+    Nfull = cap
+    sub_to_full = torch.randperm(Nfull, device=DEV, generator=gen)[:M].contiguous()
+    cached = torch.rand(M, device=DEV, generator=gen) < 0.35
+    slot0 = torch.where(cached, torch.randperm(cap, device=DEV, generator=gen)[:M], torch.full((M,), -1, device=DEV))
+    table = torch.zeros(cap, F, dtype=torch.float16, device=DEV)
+    full2slot = torch.full((Nfull,), -1, dtype=torch.int64, device=DEV)
+    slot2full = torch.full((cap,), -1, dtype=torch.int64, device=DEV)
+    checkin = torch.full((cap,), -1, dtype=torch.int64, device=DEV)
+    header = torch.full((1,), cap - 300_000, dtype=torch.int64, device=DEV)     # the ring wraps inside the call
+    thres = torch.tensor([0.05], device=DEV)
+    print("full-size c4 block built", flush=True)
+    mask, score, slot_out = be.grad_check(grad, emb, slot0, sub_to_full, thres, table, full2slot, slot2full, header,
+                                          7, age=age, age_limit=10, checkin=checkin, want_slots=True)
+    # scores: the library's summation order against an fp64 norm
+    ref = grad.double().norm(dim=1)
+    assert float(((score.double() - ref).abs() / ref).max()) < 1e-6
+    band = ((score.view(torch.int32) - thres.view(torch.int32)).abs() <= 4).sum()
+    print("rows within 4 ulp of the threshold:", int(band), flush=True)
+    want = (score < thres) & ((slot0 == -1) | (age >= 10))
+    assert torch.equal(mask, want)
+    A = int(mask.sum())
+    assert 700_000 < A < 950_000
+    rank = torch.cumsum(mask.long(), 0) - mask.long()
+    want_slot = torch.where(mask, (cap - 300_000 + rank) % cap, torch.full_like(rank, -1))
+    assert torch.equal(slot_out, want_slot)
+    assert int(header) == (cap - 300_000 + A) % cap
+    s = slot_out[mask]
+    assert torch.equal(table[s], emb[mask].half())
+    assert torch.equal(slot2full[s], sub_to_full[mask]) and torch.equal(full2slot[sub_to_full[mask]], s)
+    assert bool((checkin[s] == 7).all()) and int((checkin != -1).sum()) == A
+    assert int((slot2full != -1).sum()) == A and int((full2slot != -1).sum()) == A
+    # a second identical call admits the same rows into the next slots and un-maps nothing it should not
+    mask2, _, slot2 = be.grad_check(grad, emb, slot0, sub_to_full, thres, table, full2slot, slot2full, header,
+                                    8, age=age, age_limit=10, checkin=checkin, want_slots=True)
+    assert torch.equal(mask2, mask)
+    assert torch.equal(slot2[mask], (s + A) % cap)
+    assert int((full2slot != -1).sum()) == A                 # same nodes, moved to their new slots
+    assert torch.equal(full2slot[sub_to_full[mask]], slot2[mask])
