@@ -29,6 +29,7 @@ namespace {
 // Blocks [0, src_blocks) own source rows; blocks beyond own rows of grad_hbuf.
 // ---------------------------------------------------------------------------------------
 constexpr int BWD_SRC_PER_WAVE = 32;
+constexpr int BWD_XCD_CHUNK = 64;  // consecutive blocks (8192 sources) that share an XCD
 // With a workspace, a source with more than BWD_CHUNK incoming edges ("hub") is summed in chunks
 // of BWD_CHUNK edges by independent waves; the chunk sums are then combined left to right.
 constexpr int BWD_CHUNK = 512;
@@ -221,7 +222,7 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     for (int64_t c = lane; c < hsize; c += HC_WAVE) d[c] = (hit && c < F) ? s[c] : 0.0f;
     return;
   }
-  const int64_t s0 = (hc_xcd_block((int64_t)blockIdx.x, src_blocks) * HC_WAVES_PER_BLOCK + wave) * S;
+  const int64_t s0 = (hc_xcd_block<BWD_XCD_CHUNK>((int64_t)blockIdx.x, src_blocks) * HC_WAVES_PER_BLOCK + wave) * S;
   if (s0 >= n_src) return;
   const int64_t rest = n_src - s0;
   const int ns = rest < S ? (int)rest : S;

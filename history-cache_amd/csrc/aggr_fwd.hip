@@ -117,6 +117,7 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
 // waves grinding through multi-thousand-edge rows at one wave's memory parallelism.
 // long_thres == 0 disables the split (every row is then summed strictly in CSR order).
 constexpr int FWD_ROWS_PER_BLOCK = HC_WAVES_PER_BLOCK;
+constexpr int FWD_XCD_CHUNK = 256;  // consecutive blocks (1024 rows) that share an XCD
 
 template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM>
 __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
   const int lane = hc_lane();
   const int wave = hc_wave_in_block();
   const T *__restrict__ htab = static_cast<const T *>(hbuf);
-  const int64_t row0 = hc_xcd_block((int64_t)blockIdx.x, (int64_t)gridDim.x) * FWD_ROWS_PER_BLOCK;
+  const int64_t row0 = hc_xcd_block<FWD_XCD_CHUNK>((int64_t)blockIdx.x, (int64_t)gridDim.x) * FWD_ROWS_PER_BLOCK;
   const int64_t rest = R - row0;
   const int nrows = rest < FWD_ROWS_PER_BLOCK ? (int)rest : FWD_ROWS_PER_BLOCK;
 

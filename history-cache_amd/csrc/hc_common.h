@@ -54,15 +54,20 @@ __device__ __forceinline__ float hc_readlane_f(float v, int lane) {
 }
 
 // Workgroups are handed to the 8 XCDs round-robin (workgroup i runs on XCD i % 8) and every XCD
-// has its own L2.  This maps the hardware block index to a logical one so that each XCD works
-// through one contiguous eighth of the logical range: neighbouring rows or sources, which tend to
-// touch the same data, then share an L2.  A bijection of [0, n).
+// has its own L2.  This maps the hardware block index to a logical one so that an XCD works on
+// runs of CHUNK consecutive logical blocks: neighbouring rows or sources, which tend to touch the
+// same index lines and the same data, then share an L2.  The runs of the 8 XCDs are interleaved
+// (XCD x takes run x of every group of 8 runs), so that work whose cost drifts along the block
+// range -- rows sorted by degree, layers with different fan-outs -- stays balanced over the XCDs.
+// A bijection of [0, n); blocks behind the last full group keep their index.
 #define HC_NUM_XCD 8
+template <int CHUNK>
 __device__ __forceinline__ int64_t hc_xcd_block(int64_t bid, int64_t n) {
-  const int64_t per = n / HC_NUM_XCD;
-  const int64_t body = per * HC_NUM_XCD;
-  if (bid >= body) return bid;
-  return (bid % HC_NUM_XCD) * per + bid / HC_NUM_XCD;
+  constexpr int64_t GROUP = (int64_t)HC_NUM_XCD * CHUNK;
+  const int64_t g = bid / GROUP;
+  if ((g + 1) * GROUP > n) return bid;
+  const int64_t in = bid - g * GROUP;
+  return g * GROUP + (in % HC_NUM_XCD) * CHUNK + in / HC_NUM_XCD;
 }
 
 // Butterfly sum over the 64 lanes, partner distance 32,16,8,4,2,1.  Every lane
