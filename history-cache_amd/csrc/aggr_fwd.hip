@@ -119,11 +119,96 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
 constexpr int FWD_ROWS_PER_BLOCK = HC_WAVES_PER_BLOCK;
 constexpr int FWD_XCD_CHUNK = 256;  // consecutive blocks (1024 rows) that share an XCD
 
+// List of the long rows of a launch (optional, in caller-provided scratch): a pre-pass notes every
+// row with more than `long_thres` edges, and the first `front` blocks of the grid sum those rows
+// before anything else is scheduled, so that a multi-thousand-edge row overlaps with the bulk of
+// the launch instead of finishing alone at its end.  Each listed row is summed exactly as an
+// unlisted long row would be (same quarters, same order); the order of the list does not matter.
+struct FwdLongList {
+  int count;  // rows noted (may exceed cap: then the list is ignored)
+  int cap;
+  int pad[62];
+};
+
+struct FwdSched {
+  FwdLongList *head;  // nullptr: no list
+  int *rows;
+  int front;          // blocks at the start of the grid that work through the list
+};
+
+__global__ void fwd_long_clear(FwdLongList *h, int cap) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    h->count = 0;
+    h->cap = cap;
+  }
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void fwd_long_find(const int64_t *__restrict__ ptr,
+                                                           const int64_t *__restrict__ hmap_row, int64_t R,
+                                                           int64_t long_thres, FwdLongList *__restrict__ h,
+                                                           int *__restrict__ rows) {
+  const int64_t r = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (r >= R) return;
+  if (ptr[r + 1] - ptr[r] <= long_thres) return;
+  if (hmap_row != nullptr && hmap_row[r] != -1) return;
+  const int pos = atomicAdd(&h->count, 1);
+  if (pos < h->cap) rows[pos] = (int)r;
+}
+
+// One long row summed by the four waves of the calling block (all of them must call this).
+template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM>
+__device__ __forceinline__ void fwd_long_row(const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx,
+                                             const T *__restrict__ vin, const int64_t *__restrict__ hmap,
+                                             const T *__restrict__ htab, int64_t hsize, int src_mode,
+                                             float *__restrict__ vout, int64_t lrow, int lane, int wave,
+                                             float (*part)[HC_WAVE * VEC * CHUNKS]) {
+  constexpr int F = HC_WAVE * VEC * CHUNKS;
+  const int64_t lb = ptr[lrow];
+  const int64_t le = ptr[lrow + 1];
+  const int64_t deg = le - lb;
+  const int64_t q = (deg + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  int64_t sb = lb + wave * q;
+  int64_t se = sb + q;
+  if (sb > le) sb = le;
+  if (se > le) se = le;
+  float acc[CHUNKS][VEC];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[c][i] = 0.0f;
+  fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM>(idx, vin, hmap, htab, hsize, src_mode, sb, se, lane, acc);
+  if (wave > 0) {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) part[wave - 1][(c * HC_WAVE + lane) * VEC + i] = acc[c][i];
+  }
+  __syncthreads();
+  if (wave == 0) {
+    const float fdeg = (float)(int)deg;
+    float *__restrict__ orow = vout + lrow * F;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      float o[VEC];
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        float t2 = acc[c][i];
+#pragma unroll
+        for (int pw = 0; pw < HC_WAVES_PER_BLOCK - 1; ++pw) t2 += part[pw][(c * HC_WAVE + lane) * VEC + i];
+        o[i] = deg > 0 ? t2 / fdeg : 0.0f;
+      }
+      if constexpr (STREAM) hc_store_f32_nt<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
+      else hc_store_f32<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
+    }
+  }
+  __syncthreads();
+}
+
 template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM>
 __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const T *__restrict__ vin,
     const int64_t *__restrict__ hmap, const void *__restrict__ hbuf, int hist_dtype, int64_t hsize,
-    int src_mode, float *__restrict__ vout, int64_t R, int64_t long_thres) {
+    int src_mode, float *__restrict__ vout, int64_t R, int64_t long_thres, FwdSched sched) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   __shared__ float part[HC_WAVES_PER_BLOCK - 1][F];
   __shared__ int long_rows[FWD_ROWS_PER_BLOCK];
@@ -131,7 +216,18 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
   const int lane = hc_lane();
   const int wave = hc_wave_in_block();
   const T *__restrict__ htab = static_cast<const T *>(hbuf);
-  const int64_t row0 = hc_xcd_block<FWD_XCD_CHUNK>((int64_t)blockIdx.x, (int64_t)gridDim.x) * FWD_ROWS_PER_BLOCK;
+  // every thread of the grid reads the same two words, so the decision is uniform
+  const int n_listed = sched.head != nullptr ? sched.head->count : 0;
+  const bool listed = sched.head != nullptr && n_listed <= sched.head->cap;
+  if ((int)blockIdx.x < sched.front) {
+    if (!listed) return;
+    for (int t = (int)blockIdx.x; t < n_listed; t += sched.front)
+      fwd_long_row<T, VEC, CHUNKS, UNROLL, STREAM>(ptr, idx, vin, hmap, htab, hsize, src_mode, vout,
+                                                   (int64_t)sched.rows[t], lane, wave, part);
+    return;
+  }
+  const int64_t row0 = hc_xcd_block<FWD_XCD_CHUNK>((int64_t)blockIdx.x - sched.front,
+                                                   (int64_t)gridDim.x - sched.front) * FWD_ROWS_PER_BLOCK;
   const int64_t rest = R - row0;
   const int nrows = rest < FWD_ROWS_PER_BLOCK ? (int)rest : FWD_ROWS_PER_BLOCK;
 
@@ -154,7 +250,8 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
       const int64_t end = ptr[row + 1];
       const int64_t deg = end - begin;
       if (long_thres > 0 && deg > long_thres) {
-        if (lane == 0) long_rows[atomicAdd(&n_long_s, 1)] = k;
+        // a listed row is summed by the front blocks
+        if (!listed && lane == 0) long_rows[atomicAdd(&n_long_s, 1)] = k;
       } else {
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c)
@@ -173,51 +270,13 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
       }
     }
   }
-  if (long_thres <= 0) return;  // kernel argument: the whole grid takes the same branch
+  if (long_thres <= 0 || listed) return;  // the whole grid takes the same branch
   __syncthreads();
   const int n_long = n_long_s;
   // The order in which long rows were noted does not matter: each is summed on its own.
-  for (int t = 0; t < n_long; ++t) {
-    const int64_t lrow = row0 + long_rows[t];
-    const int64_t lb = ptr[lrow];
-    const int64_t le = ptr[lrow + 1];
-    const int64_t deg = le - lb;
-    const int64_t q = (deg + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
-    int64_t sb = lb + wave * q;
-    int64_t se = sb + q;
-    if (sb > le) sb = le;
-    if (se > le) se = le;
-#pragma unroll
-    for (int c = 0; c < CHUNKS; ++c)
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) acc[c][i] = 0.0f;
-    fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM>(idx, vin, hmap, htab, hsize, src_mode, sb, se, lane, acc);
-    if (wave > 0) {
-#pragma unroll
-      for (int c = 0; c < CHUNKS; ++c)
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) part[wave - 1][(c * HC_WAVE + lane) * VEC + i] = acc[c][i];
-    }
-    __syncthreads();
-    if (wave == 0) {
-      const float fdeg = (float)(int)deg;
-      float *__restrict__ orow = vout + lrow * F;
-#pragma unroll
-      for (int c = 0; c < CHUNKS; ++c) {
-        float o[VEC];
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-          float t2 = acc[c][i];
-#pragma unroll
-          for (int pw = 0; pw < HC_WAVES_PER_BLOCK - 1; ++pw) t2 += part[pw][(c * HC_WAVE + lane) * VEC + i];
-          o[i] = t2 / fdeg;
-        }
-        if constexpr (STREAM) hc_store_f32_nt<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
-        else hc_store_f32<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
-      }
-    }
-    __syncthreads();
-  }
+  for (int t = 0; t < n_long; ++t)
+    fwd_long_row<T, VEC, CHUNKS, UNROLL, STREAM>(ptr, idx, vin, hmap, htab, hsize, src_mode, vout,
+                                                 row0 + long_rows[t], lane, wave, part);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -291,22 +350,48 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_generic(
   }
 }
 
+// Rows below this count are launched without the long-row list even when scratch is given: the two
+// extra launches cost more than the list saves.
+constexpr int64_t FWD_LIST_MIN_ROWS = 65536;
+constexpr int FWD_FRONT_BLOCKS = 2048;
+
+struct FwdScratch {
+  void *ptr;
+  size_t bytes;
+};
+
 template <typename T, int VEC, int CHUNKS>
 int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const int64_t *hmap,
                 const void *hbuf, int hist_dtype, int64_t hsize, int src_mode, float *vout, int64_t R,
-                hipStream_t st) {
+                FwdScratch ws, hipStream_t st) {
   constexpr int per = VEC * CHUNKS;
   constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
-  const int64_t blocks = (R + FWD_ROWS_PER_BLOCK - 1) / FWD_ROWS_PER_BLOCK;
+  int64_t blocks = (R + FWD_ROWS_PER_BLOCK - 1) / FWD_ROWS_PER_BLOCK;
+  FwdSched sched{nullptr, nullptr, 0};
+  int64_t cap = 0;
+  if (ws.ptr != nullptr && ws.bytes >= sizeof(FwdLongList) + sizeof(int) && R >= FWD_LIST_MIN_ROWS &&
+      R <= 0x7fffffffLL && reinterpret_cast<uintptr_t>(ws.ptr) % 256 == 0) {
+    cap = (int64_t)((ws.bytes - sizeof(FwdLongList)) / sizeof(int));
+    if (cap > R) cap = R;
+    sched.head = static_cast<FwdLongList *>(ws.ptr);
+    sched.rows = reinterpret_cast<int *>(static_cast<char *>(ws.ptr) + sizeof(FwdLongList));
+    sched.front = (int)(cap < FWD_FRONT_BLOCKS ? cap : FWD_FRONT_BLOCKS);
+    blocks += sched.front;
+  }
   if (!hc_grid_ok(blocks)) return HC_EUNSUPPORTED;
+  if (sched.head != nullptr) {
+    fwd_long_clear<<<dim3(1), dim3(HC_WAVE), 0, st>>>(sched.head, (int)cap);
+    fwd_long_find<<<dim3((unsigned)((R + HC_BLOCK - 1) / HC_BLOCK)), dim3(HC_BLOCK), 0, st>>>(
+        ptr, src_mode ? nullptr : hmap, R, (int64_t)HC_LONG_ROW_EDGES, sched.head, sched.rows);
+  }
   if (src_mode && hmap != nullptr)
     fwd_mean_fast<T, VEC, CHUNKS, UNROLL, true><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(
         ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, vout, R,
-        (int64_t)HC_LONG_ROW_EDGES);
+        (int64_t)HC_LONG_ROW_EDGES, sched);
   else
     fwd_mean_fast<T, VEC, CHUNKS, UNROLL, false><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(
         ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, vout, R,
-        (int64_t)HC_LONG_ROW_EDGES);
+        (int64_t)HC_LONG_ROW_EDGES, sched);
   return hc_launch_status();
 }
 
@@ -314,11 +399,11 @@ int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const i
 template <typename T>
 int dispatch_fast(int64_t F, const int64_t *ptr, const int64_t *idx, const void *vin,
                   const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize, int src_mode,
-                  float *vout, int64_t R, hipStream_t st, bool *handled) {
+                  float *vout, int64_t R, FwdScratch ws, hipStream_t st, bool *handled) {
   *handled = true;
 #define HC_FAST(V, C)                                                                              \
   if (F == 64 * (V) * (C))                                                                         \
-    return launch_fast<T, V, C>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, vout, R, st);
+    return launch_fast<T, V, C>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, vout, R, ws, st);
   constexpr int VMAX = 16 / (int)sizeof(T);
   if constexpr (VMAX == 8) {
     HC_FAST(8, 1) HC_FAST(8, 2) HC_FAST(8, 3) HC_FAST(8, 4)
@@ -369,10 +454,20 @@ extern "C" int64_t hc_aggr_fwd_long_row_edges(int64_t F, int in_dtype) {
   return fast_shape(F, in_dtype) ? HC_LONG_ROW_EDGES : 0;
 }
 
+extern "C" size_t hc_aggr_fwd_workspace_bytes(int64_t R, int64_t E) {
+  if (R < FWD_LIST_MIN_ROWS || E <= HC_LONG_ROW_EDGES) return 0;
+  // at most E / (HC_LONG_ROW_EDGES + 1) rows can be long
+  int64_t cap = E / (HC_LONG_ROW_EDGES + 1) + 1;
+  if (cap > R) cap = R;
+  return hc_align_up(sizeof(FwdLongList) + (size_t)cap * sizeof(int), 256);
+}
+
 extern "C" int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, const void *vin,
                            int in_dtype, const int64_t *hmap, const void *hbuf, int hist_dtype,
                            int64_t hsize, const float *edge_value, int64_t n_head, float *vout,
-                           int64_t R, int64_t F, int64_t n_src, void *stream) {
+                           int64_t R, int64_t F, int64_t n_src, void *workspace,
+                           size_t workspace_bytes, void *stream) {
+  const FwdScratch ws{workspace, workspace ? workspace_bytes : 0};
   HC_REQUIRE(R >= 0 && F > 0 && n_src >= 0 && n_head >= 1);
   if (R == 0) return HC_OK;
   HC_REQUIRE(ptr && vout);
@@ -402,14 +497,14 @@ extern "C" int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, con
     bool handled = false;
     int rc;
     if (in_dtype == HC_F32)
-      rc = dispatch_fast<float>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, vout, R, st,
+      rc = dispatch_fast<float>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, vout, R, ws, st,
                                 &handled);
     else if (in_dtype == HC_F16)
-      rc = dispatch_fast<__half>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, vout, R, st,
+      rc = dispatch_fast<__half>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, vout, R, ws, st,
                                  &handled);
     else
       rc = dispatch_fast<__hip_bfloat16>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode,
-                                         vout, R, st, &handled);
+                                         vout, R, ws, st, &handled);
     if (handled) return rc;
   }
   if (in_dtype == HC_F32)

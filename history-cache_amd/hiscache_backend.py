@@ -41,8 +41,9 @@ _SIGNATURES = {
     "hc_version": (ctypes.c_char_p, []),
     "hc_strerror": (ctypes.c_char_p, [_c_int]),
     "hc_device_count": (_c_int, []),
+    "hc_aggr_fwd_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
     "hc_aggr_fwd": (_c_int, [_c_int, _c_p, _c_p, _c_p, _c_int, _c_p, _c_p, _c_int, _c_i64, _c_p, _c_i64,
-                             _c_p, _c_i64, _c_i64, _c_i64, _c_p]),
+                             _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]),
     "hc_aggr_fwd_long_row_edges": (_c_i64, [_c_i64, _c_int]),
     "hc_transpose_workspace_bytes": (_c_sz, [_c_i64, _c_i64, _c_i64]),
     "hc_build_transpose": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p,
@@ -186,9 +187,13 @@ def _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, num_node):
             raise ValueError("history_buffer is smaller than num_node x history_size")
     out_shape = (R, F) if n_head == 1 and x.dim() == 2 else (R, n_head, F)
     out = torch.empty(out_shape, dtype=torch.float32, device=x.device)
+    # scratch for the long-row list (large blocks only: the library reports 0 bytes otherwise)
+    ws_bytes = int(lib.hc_aggr_fwd_workspace_bytes(R, idx.numel())) if edge_value is None else 0
+    ws = _workspace(ws_bytes, x.device) if ws_bytes > 0 else None
     rc = lib.hc_aggr_fwd(mode, _ptr(ptr), _ptr(idx), _ptr(x), _float_dtype(x, "input"),
                          _ptr(hmap), _ptr(hbuf), _float_dtype(hbuf, "history_buffer") if hmap is not None else 0,
-                         int(hsize), _ptr(edge_value), n_head, _ptr(out), R, F, n_src, _stream())
+                         int(hsize), _ptr(edge_value), n_head, _ptr(out), R, F, n_src, _ptr(ws), ws_bytes,
+                         _stream())
     _check(rc, "hc_aggr_fwd")
     return out
 

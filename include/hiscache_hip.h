@@ -78,11 +78,16 @@ int hc_device_count(void);
  * summed in CSR order; when hc_aggr_fwd_long_row_edges() reports a threshold
  * T > 0 for the shape, a row with more than T edges is summed as four
  * contiguous quarters of ceil(deg/4) edges, each in CSR order, combined left to
- * right ((q0+q1)+q2)+q3, then divided. */
+ * right ((q0+q1)+q2)+q3, then divided.
+ * workspace (optional, NULL allowed; 256-byte aligned, of
+ * hc_aggr_fwd_workspace_bytes(R, E) bytes, E = an upper bound of ptr[R]): on
+ * large blocks the long rows are listed first and scheduled at the start of
+ * the launch, which shortens its tail; results do not depend on it. */
+size_t hc_aggr_fwd_workspace_bytes(int64_t R, int64_t E);
 int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, const void *vin, int in_dtype,
                 const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize,
                 const float *edge_value, int64_t n_head, float *vout, int64_t R, int64_t F,
-                int64_t n_src, void *stream);
+                int64_t n_src, void *workspace, size_t workspace_bytes, void *stream);
 
 /* The long-row threshold T that hc_aggr_fwd applies to a mean aggregation with
  * rows of F elements of in_dtype; 0 when every row is summed strictly in CSR

@@ -37,18 +37,18 @@ def test_argument_errors_are_status_codes():
     lib = be.load_library()
     null = ctypes.c_void_p(None)
     # negative row count, zero feature width
-    assert lib.hc_aggr_fwd(0, null, null, null, 0, null, null, 0, 0, null, 1, null, -1, 4, 0, null) == 1
-    assert lib.hc_aggr_fwd(0, null, null, null, 0, null, null, 0, 0, null, 1, null, 4, 0, 0, null) == 1
+    assert lib.hc_aggr_fwd(0, null, null, null, 0, null, null, 0, 0, null, 1, null, -1, 4, 0, null, 0, null) == 1
+    assert lib.hc_aggr_fwd(0, null, null, null, 0, null, null, 0, 0, null, 1, null, 4, 0, 0, null, 0, null) == 1
     # missing pointers
-    assert lib.hc_aggr_fwd(0, null, null, null, 0, null, null, 0, 0, null, 1, null, 4, 4, 4, null) == 1
+    assert lib.hc_aggr_fwd(0, null, null, null, 0, null, null, 0, 0, null, 1, null, 4, 4, 4, null, 0, null) == 1
     buf = np.zeros(64, np.int64)
     p = ctypes.c_void_p(buf.ctypes.data)
     # unknown dtype / substitution mode
-    assert lib.hc_aggr_fwd(0, p, p, p, 7, null, null, 0, 0, null, 1, p, 4, 4, 4, null) == 2
-    assert lib.hc_aggr_fwd(9, p, p, p, 0, null, null, 0, 0, null, 1, p, 4, 4, 4, null) == 1
+    assert lib.hc_aggr_fwd(0, p, p, p, 7, null, null, 0, 0, null, 1, p, 4, 4, 4, null, 0, null) == 2
+    assert lib.hc_aggr_fwd(9, p, p, p, 0, null, null, 0, 0, null, 1, p, 4, 4, 4, null, 0, null) == 1
     # heads need edge values; history map needs a buffer
-    assert lib.hc_aggr_fwd(0, p, p, p, 0, null, null, 0, 0, null, 2, p, 4, 4, 4, null) == 1
-    assert lib.hc_aggr_fwd(0, p, p, p, 0, p, null, 0, 4, null, 1, p, 4, 4, 4, null) == 1
+    assert lib.hc_aggr_fwd(0, p, p, p, 0, null, null, 0, 0, null, 2, p, 4, 4, 4, null, 0, null) == 1
+    assert lib.hc_aggr_fwd(0, p, p, p, 0, p, null, 0, 4, null, 1, p, 4, 4, 4, null, 0, null) == 1
     # grad_check: bad enums, missing workspace
     args = [p, null, p, p, null, null, p, p, 0, 0, 0, p, null, null, p, 0, 8, p, p, null, p, 0, 4, 4]
     assert lib.hc_grad_check(*args, null, 0, null) == 4

@@ -67,12 +67,14 @@ def test_fwd_mean_row_mode(be, orc, R, N, F, maxdeg, hub, dtype, with_hist):
     np.testing.assert_array_equal(out.detach().cpu().numpy(), ref)
 
 
+@pytest.mark.parametrize("R", [9000, 70000])
 @pytest.mark.parametrize("mode", ["plain", "row", "src"])
-def test_fwd_long_rows_started_first(be, orc, mode):
-    """Rows above the long-row threshold are summed as four quarters by their block: same bits as the
-    oracle applying the documented quarter rule, and within 1e-5 of the strictly sequential sum."""
+def test_fwd_long_rows_quarter_rule(be, orc, mode, R):
+    """Rows above the long-row threshold are summed as four quarters by a whole block: same bits as the
+    oracle applying the documented quarter rule, and within 1e-5 of the strictly sequential sum.  With
+    70000 rows the shim passes scratch and the long rows are listed and scheduled first."""
     rng = np.random.default_rng(42)
-    R, N, F = 9000, 3000, 128
+    N, F = 3000, 128
     ptr, idx = random_csr(rng, R, N, 6)
     deg = np.diff(ptr)
     for r in rng.choice(R, size=12, replace=False):           # a dozen long rows, one of them empty-adjacent
@@ -354,3 +356,28 @@ def test_shim_rejects_bad_arguments(be):
         be.aggr_forward_history(x.t(), ptr, idx, none(), none(), 0, 4)          # not contiguous
     with pytest.raises(ValueError):
         be.aggr_forward_history(x, ptr, idx, torch.full((2,), -1, device=DEV), x, 128, 4)  # short map
+
+
+def test_fwd_long_row_list_overflow_falls_back(be, orc):
+    """Scratch that cannot hold every long row: the list is ignored and the rows are summed in place,
+    with the same bits."""
+    import ctypes
+    rng = np.random.default_rng(43)
+    R, N, F = 70000, 2000, 64
+    ptr, idx = random_csr(rng, R, N, 4)
+    deg = np.diff(ptr)
+    deg[rng.choice(R, size=9, replace=False)] = 300
+    ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    idx = rng.integers(0, N, size=int(ptr[-1]), dtype=np.int64)
+    x = rng.standard_normal((N, F)).astype(np.float32)
+    ref = orc.fwd_mean_row(ptr, idx, x, None, None, split_above=be.long_row_edges(F))
+    lib = be.load_library()
+    tp, ti, tx = T(ptr), T(idx), T(x)
+    for ws_ints in (4, 64):                                    # room for 4 rows (overflow) and for 64
+        out = torch.full((R, F), float("nan"), device=DEV)
+        ws = torch.empty(256 + 4 * ws_ints, dtype=torch.uint8, device=DEV)
+        rc = lib.hc_aggr_fwd(0, tp.data_ptr(), ti.data_ptr(), tx.data_ptr(), 0, None, None, 0, 0, None, 1,
+                             out.data_ptr(), R, F, N, ws.data_ptr(), ws.numel(),
+                             torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        np.testing.assert_array_equal(out.cpu().numpy(), ref)
