@@ -143,16 +143,35 @@ __global__ void fwd_long_clear(FwdLongList *h, int cap) {
   }
 }
 
+// A block scans FWD_FIND_TILE rows, collects its long rows in LDS and takes one run of list slots
+// with a single global atomic (one atomic per long row would serialise on the counter).
+constexpr int FWD_FIND_ITEMS = 8;
+constexpr int FWD_FIND_TILE = HC_BLOCK * FWD_FIND_ITEMS;
+
 __global__ __launch_bounds__(HC_BLOCK) void fwd_long_find(const int64_t *__restrict__ ptr,
                                                            const int64_t *__restrict__ hmap_row, int64_t R,
                                                            int64_t long_thres, FwdLongList *__restrict__ h,
                                                            int *__restrict__ rows) {
-  const int64_t r = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
-  if (r >= R) return;
-  if (ptr[r + 1] - ptr[r] <= long_thres) return;
-  if (hmap_row != nullptr && hmap_row[r] != -1) return;
-  const int pos = atomicAdd(&h->count, 1);
-  if (pos < h->cap) rows[pos] = (int)r;
+  __shared__ int found[FWD_FIND_TILE];
+  __shared__ int n_found;
+  __shared__ int base;
+  if (threadIdx.x == 0) n_found = 0;
+  __syncthreads();
+  const int64_t r0 = (int64_t)blockIdx.x * FWD_FIND_TILE;
+#pragma unroll
+  for (int it = 0; it < FWD_FIND_ITEMS; ++it) {
+    const int64_t r = r0 + (int64_t)it * HC_BLOCK + threadIdx.x;
+    if (r < R && ptr[r + 1] - ptr[r] > long_thres && (hmap_row == nullptr || hmap_row[r] == -1))
+      found[atomicAdd(&n_found, 1)] = (int)r;
+  }
+  __syncthreads();
+  const int n = n_found;
+  if (n == 0) return;
+  if (threadIdx.x == 0) base = atomicAdd(&h->count, n);
+  __syncthreads();
+  const int cap = h->cap;
+  for (int i = threadIdx.x; i < n; i += HC_BLOCK)
+    if (base + i < cap) rows[base + i] = found[i];
 }
 
 // One long row summed by the four waves of the calling block (all of them must call this).
@@ -381,7 +400,7 @@ int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const i
   if (!hc_grid_ok(blocks)) return HC_EUNSUPPORTED;
   if (sched.head != nullptr) {
     fwd_long_clear<<<dim3(1), dim3(HC_WAVE), 0, st>>>(sched.head, (int)cap);
-    fwd_long_find<<<dim3((unsigned)((R + HC_BLOCK - 1) / HC_BLOCK)), dim3(HC_BLOCK), 0, st>>>(
+    fwd_long_find<<<dim3((unsigned)((R + FWD_FIND_TILE - 1) / FWD_FIND_TILE)), dim3(HC_BLOCK), 0, st>>>(
         ptr, src_mode ? nullptr : hmap, R, (int64_t)HC_LONG_ROW_EDGES, sched.head, sched.rows);
   }
   if (src_mode && hmap != nullptr)
