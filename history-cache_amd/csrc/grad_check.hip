@@ -516,3 +516,58 @@ extern "C" int hc_cache_append(const float *score, const float *thres, const flo
                                                                     embed2full, M);
   return hc_launch_status();
 }
+
+// ---------------------------------------------------------------------------------------
+// Eviction (HistoryTable.evict_by_staleness / evict_by_both,
+// /root/reference/hiscache/history_table.py:189-251) as one launch.  Threads [0, M) handle the
+// batch rows: a row with a slot and score >= *thres gives its slot up.  Threads [M, M + capacity)
+// handle the slots: a slot with -1 < checkin <= stale_iter is given up.  Giving a slot up writes
+// -1 into the owner's map entry, the slot's owner and its check-in; a slot reached from both
+// sides gets the same three stores twice, so the result does not depend on the interleaving.
+// ---------------------------------------------------------------------------------------
+namespace {
+
+__device__ __forceinline__ void evict_slot(int64_t s, int64_t *__restrict__ checkin,
+                                           int64_t *__restrict__ slot2full, int64_t *__restrict__ full2slot,
+                                           int64_t n_full) {
+  const int64_t owner = slot2full[s];
+  if (owner >= 0 && owner < n_full) full2slot[owner] = -1;
+  slot2full[s] = -1;
+  checkin[s] = -1;
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void evict_kernel(const int64_t *__restrict__ sub2slot,
+                                                          const float *__restrict__ score,
+                                                          const float *__restrict__ thres, int64_t M,
+                                                          int64_t stale_iter, int64_t *__restrict__ checkin,
+                                                          int64_t *__restrict__ slot2full,
+                                                          int64_t *__restrict__ full2slot, int64_t capacity,
+                                                          int64_t n_full) {
+  const int64_t t = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (t < M) {
+    const int64_t s = sub2slot[t];
+    if (s >= 0 && s < capacity && score[t] >= *thres) evict_slot(s, checkin, slot2full, full2slot, n_full);
+    return;
+  }
+  const int64_t s = t - M;
+  if (s >= capacity) return;
+  const int64_t c = checkin[s];
+  if (c > -1 && c <= stale_iter) evict_slot(s, checkin, slot2full, full2slot, n_full);
+}
+
+}  // namespace
+
+extern "C" int hc_evict(const int64_t *sub2slot, const float *score, const float *thres, int64_t M,
+                        int64_t stale_iter, int64_t *checkin, int64_t *slot2full, int64_t *full2slot,
+                        int64_t capacity, int64_t n_full, void *stream) {
+  HC_REQUIRE(M >= 0 && capacity >= 0 && n_full >= 0);
+  if (M > 0) HC_REQUIRE(sub2slot && score && thres);
+  if (M + capacity == 0) return HC_OK;
+  HC_REQUIRE(checkin && slot2full && full2slot);
+  const int64_t blocks = (M + capacity + HC_BLOCK - 1) / HC_BLOCK;
+  if (!hc_grid_ok(blocks)) return HC_EUNSUPPORTED;
+  evict_kernel<<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, static_cast<hipStream_t>(stream)>>>(
+      sub2slot, score, thres, M, stale_iter, checkin, slot2full, full2slot, capacity, n_full);
+  return hc_launch_status();
+}
+

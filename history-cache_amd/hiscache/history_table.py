@@ -150,25 +150,18 @@ class HistoryTable:
                                self.cuda_header_layered[layer_id], record_sum, thres,
                                self.checkin_iter[layer_id], glb_iter)
 
-    def _evict_stale(self, layer_id, stale_iter):
-        checkin = self.checkin_iter[layer_id]
-        hist_id = torch.logical_and(-1 < checkin, checkin <= stale_iter).nonzero().view(-1)
-        full_id = self.history_to_full_layered[layer_id][hist_id]
-        self.checkin_iter[layer_id][hist_id] = -1
-        self.history_to_full_layered[layer_id][hist_id] = -1
-        self.full_to_history_layered[layer_id][full_id] = -1
-
     def evict_by_staleness(self, glb_iter, staleness_thres):
         """Un-map slots with -1 < checkin <= glb_iter - limit
         (/root/reference/hiscache/history_table.py:189-200)."""
         if isinstance(staleness_thres, int):
             staleness_thres = [staleness_thres] * self.num_layers
         for layer_id in range(self.num_layers):
-            self._evict_stale(layer_id, glb_iter - staleness_thres[layer_id])
+            _be.evict(self.checkin_iter[layer_id], self.history_to_full_layered[layer_id],
+                      self.full_to_history_layered[layer_id], glb_iter - staleness_thres[layer_id])
 
     def evict_by_both(self, batch, glb_iter, staleness_thres):
         """Evict cached rows whose score is in the top ``rate`` quantile, then by staleness
-        (/root/reference/hiscache/history_table.py:202-251)."""
+        (/root/reference/hiscache/history_table.py:202-251); one launch per table."""
         if self.method == "staleness":
             self.evict_by_staleness(glb_iter, staleness_thres)
             return
@@ -181,13 +174,9 @@ class HistoryTable:
             grad = (self.history_out[layer_id].grad)[:num_node]
             evict_sum = self._score(grad, batch)
             thres = quantile_threshold(evict_sum, 1 - self.rate)
-            to_evict_id = torch.masked_select(self.sub_to_history[layer_id], evict_sum >= thres)
-            to_evict_id = to_evict_id[to_evict_id != -1]
-            owners = self.history_to_full_layered[layer_id][to_evict_id]
-            self.full_to_history_layered[layer_id][owners] = -1
-            self.history_to_full_layered[layer_id][to_evict_id] = -1
-            self.checkin_iter[layer_id][to_evict_id] = -1
-            self._evict_stale(layer_id, glb_iter - staleness_thres[layer_id])
+            _be.evict(self.checkin_iter[layer_id], self.history_to_full_layered[layer_id],
+                      self.full_to_history_layered[layer_id], glb_iter - staleness_thres[layer_id],
+                      sub2slot=self.sub_to_history[layer_id][:num_node].contiguous(), score=evict_sum, thres=thres)
 
     def evict_history(self, batch, glb_iter):
         self.evict_by_both(batch, glb_iter, self.staleness_thres)

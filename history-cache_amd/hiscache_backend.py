@@ -66,6 +66,7 @@ _SIGNATURES = {
     "hc_structure_score": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p]),
     "hc_gather_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p]),
+    "hc_evict": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p]),
     "hc_sample_capacity": (_c_int, [_c_i64, _c_p, _c_int, _c_i64, _c_p, _c_p, _c_p]),
     "hc_sample_workspace_bytes": (_c_sz, [_c_i64, _c_p, _c_int, _c_i64]),
     "hc_sample_map_init": (_c_int, [_c_p, _c_i64, _c_p]),
@@ -650,6 +651,30 @@ def edge_types_by_ranges(ptr, idx, sub_to_full, num_node, bounds, pair_to_rel):
                                      int(bounds.numel()), _ptr(pair_to_rel), _ptr(out), R, idx.numel(), _stream())
     _check(rc, "hc_edge_types_by_ranges")
     return out
+
+
+def evict(checkin, slot2full, full2slot, stale_iter, sub2slot=None, score=None, thres=None):
+    """Give up table slots in place: every slot with -1 < checkin <= ``stale_iter`` and, when
+    ``sub2slot`` / ``score`` / ``thres`` (1-element fp32 device tensor) are given, the slot of every
+    batch row whose score is >= thres (/root/reference/hiscache/history_table.py:189-251)."""
+    lib = load_library()
+    _dev(checkin, "checkin", torch.int64)
+    _dev(slot2full, "slot2full", torch.int64)
+    _dev(full2slot, "full2slot", torch.int64)
+    M = 0
+    if sub2slot is not None:
+        _dev(sub2slot, "sub2slot", torch.int64)
+        _dev(score, "score", torch.float32)
+        _dev(thres, "thres", torch.float32)
+        M = sub2slot.numel()
+        if score.numel() < M:
+            raise ValueError("score is shorter than sub2slot")
+    cap = slot2full.numel()
+    if checkin.numel() < cap:
+        raise ValueError("checkin is shorter than slot2full")
+    rc = lib.hc_evict(_ptr(sub2slot), _ptr(score), _ptr(thres), M, int(stale_iter), _ptr(checkin), _ptr(slot2full),
+                      _ptr(full2slot), cap, full2slot.numel(), _stream())
+    _check(rc, "hc_evict")
 
 
 def sample_map(num_nodes, device):

@@ -225,6 +225,19 @@ int hc_cache_append(const float *score, const float *thres, const float *emb,
                     int64_t *overflow, int64_t M, void *workspace, size_t workspace_bytes,
                     void *stream);
 
+/* hc_evict replaces the torch sequences of HistoryTable.evict_by_staleness and
+ * evict_by_both (hiscache/history_table.py:189-251) for one table.  Gradient
+ * rule (M > 0): batch row r with sub2slot[r] != -1 and score[r] >= *thres
+ * gives up its slot (:234-244).  Staleness rule: every slot with
+ * -1 < checkin <= stale_iter is given up (:193-200, :246-251); pass
+ * stale_iter < 0 to skip it.  Giving up slot s: full2slot[slot2full[s]] = -1,
+ * slot2full[s] = -1, checkin[s] = -1.  The final state is the one the
+ * reference reaches by applying the gradient rule first and the staleness rule
+ * second. */
+int hc_evict(const int64_t *sub2slot, const float *score, const float *thres, int64_t M,
+             int64_t stale_iter, int64_t *checkin, int64_t *slot2full, int64_t *full2slot,
+             int64_t capacity, int64_t n_full, void *stream);
+
 /* ---------------------------------------------------------------- sampler
  * Layered neighbour sampling on the device.  The reference takes its batches
  * from the external cxgnndl loader (hiscache/history_trainer.py:19,26); these

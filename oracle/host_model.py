@@ -125,3 +125,18 @@ def evict_by_staleness(checkin, history_to_full, full_to_history, glb_iter, stal
     checkin[hist_id] = -1
     history_to_full[hist_id] = -1
     full_to_history[full_id] = -1
+
+
+def evict_by_both(checkin, history_to_full, full_to_history, sub_to_history, score, rate, glb_iter,
+                  staleness_thres):
+    """history_table.py:230-251 for one layer, in place: rows of the batch whose score reaches
+    quantile(score, 1 - rate) give up their slot, then the staleness rule runs."""
+    thres = quantile_threshold(score, 1 - rate)
+    to_evict = torch.masked_select(sub_to_history, score >= thres)
+    to_evict = to_evict[to_evict != -1]
+    full_to_history[history_to_full[to_evict]] = -1
+    history_to_full[to_evict] = -1
+    checkin[to_evict] = -1
+    evict_by_staleness(checkin, history_to_full, full_to_history, glb_iter, staleness_thres)
+    return thres
+

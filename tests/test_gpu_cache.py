@@ -288,7 +288,20 @@ def test_history_table_record_and_evict():
             np.testing.assert_array_equal(table.cuda_header_layered[layer_id].cpu().numpy(), r["header"])
             live = r["h2f"] != -1
             np.testing.assert_array_equal(table.history_buffer_layered[layer_id].cpu().numpy()[live], r["buf"][live])
-        if it % 2 == 0:
+        if it == 5:
+            # gradient eviction + staleness eviction (HistoryTable.evict_by_both)
+            table.evict_by_both(batch, it, 3)
+            for layer_id in range(2):
+                n = int(nnl[3 - 1 - layer_id])
+                r = ref[layer_id]
+                score = torch.from_numpy(orc.row_scores(outs[layer_id].grad.cpu().numpy(), orc.NORM_L1))
+                s2h = table.sub_to_history[layer_id][:n].cpu()
+                c, h, f = (torch.from_numpy(r[k]) for k in ("checkin", "h2f", "f2h"))
+                host_model.evict_by_both(c, h, f, s2h, score, 0.7, it, 3)
+                np.testing.assert_array_equal(table.history_to_full_layered[layer_id].cpu().numpy(), r["h2f"])
+                np.testing.assert_array_equal(table.full_to_history_layered[layer_id].cpu().numpy(), r["f2h"])
+                np.testing.assert_array_equal(table.checkin_iter[layer_id].cpu().numpy(), r["checkin"])
+        elif it % 2 == 0:
             table.evict_by_staleness(it, 3)
             for layer_id in range(2):
                 r = ref[layer_id]
@@ -517,3 +530,36 @@ def test_edge_types_by_ranges_matches_oracle(orc):
     np.testing.assert_array_equal(got, orc.edge_types_by_ranges(ptr, idx, s2f, R, bounds, table))
     none = be.edge_types_by_ranges(t(ptr), t(idx), t(s2f), R, t(np.zeros(0)), t(np.array([[7]]))).cpu().numpy()
     assert set(np.unique(none[: ptr[R]])) <= {7, -1}
+
+
+def test_evict_matches_oracle(orc):
+    """hc_evict (gradient rule + staleness rule in one launch) against the CPU statement of
+    HistoryTable.evict_by_both, and the staleness rule alone."""
+    import hiscache_backend as be
+    from oracle import host_model
+    rng = np.random.default_rng(81)
+    cap, N, M = 5000, 20000, 3000
+    for trial in range(4):
+        owners = rng.choice(N, size=4000, replace=False)
+        slots = rng.choice(cap, size=4000, replace=False)
+        h2f = np.full(cap, -1, np.int64); f2h = np.full(N, -1, np.int64); chk = np.full(cap, -1, np.int64)
+        h2f[slots] = owners; f2h[owners] = slots; chk[slots] = rng.integers(0, 30, size=4000)
+        nodes = rng.choice(N, size=M, replace=False)
+        s2h = f2h[nodes].copy()
+        s2h[:100] = -1
+        score = rng.random(M).astype(np.float32)
+        score[5:9] = score[4]                                      # ties around the threshold side
+        dev = [torch.from_numpy(a.copy()).to(DEV) for a in (chk, h2f, f2h)]
+        cpu = [torch.from_numpy(a.copy()) for a in (chk, h2f, f2h)]
+        if trial % 2 == 0:
+            thres = host_model.evict_by_both(cpu[0], cpu[1], cpu[2], torch.from_numpy(s2h), torch.from_numpy(score),
+                                             rate=0.25, glb_iter=30, staleness_thres=12)
+            be.evict(dev[0], dev[1], dev[2], 30 - 12, sub2slot=torch.from_numpy(s2h).to(DEV),
+                     score=torch.from_numpy(score).to(DEV),
+                     thres=torch.tensor([float(thres)], dtype=torch.float32, device=DEV))
+        else:
+            host_model.evict_by_staleness(cpu[0], cpu[1], cpu[2], 30, 12)
+            be.evict(dev[0], dev[1], dev[2], 30 - 12)
+        for d, c in zip(dev, cpu):
+            np.testing.assert_array_equal(d.cpu().numpy(), c.numpy())
+        assert (cpu[1] != -1).sum() < 4000

@@ -464,3 +464,35 @@ def test_edge_types_by_ranges_brute_force(orc):
         for e in range(ptr[r], ptr[r + 1]):
             want = table[typ(s2f[r]), typ(s2f[idx[e]])] if r < R else -1
             assert got[e] == want
+
+
+def test_evict_by_both_brute_force():
+    """Gradient rule then staleness rule against a dictionary model of the table."""
+    from oracle import host_model
+    rng = np.random.default_rng(77)
+    cap, N, M = 60, 200, 40
+    for trial in range(5):
+        owners = rng.choice(N, size=45, replace=False)
+        slots = rng.choice(cap, size=45, replace=False)
+        h2f = np.full(cap, -1, np.int64); f2h = np.full(N, -1, np.int64); chk = np.full(cap, -1, np.int64)
+        h2f[slots] = owners; f2h[owners] = slots; chk[slots] = rng.integers(0, 12, size=45)
+        batch_nodes = rng.choice(N, size=M, replace=False)
+        s2h = f2h[batch_nodes].copy()
+        s2h[:5] = -1                                              # seeds never use history
+        score = rng.random(M).astype(np.float32)
+        model = {int(s): (int(o), int(c)) for s, o, c in zip(slots, owners, chk[slots])}
+        t = [torch.from_numpy(a) for a in (chk, h2f, f2h, s2h, score)]
+        thres = host_model.evict_by_both(t[0], t[1], t[2], t[3], t[4], rate=0.3, glb_iter=12, staleness_thres=6)
+        thr = float(thres)
+        for r in range(M):
+            if s2h[r] != -1 and score[r] >= thr:
+                model.pop(int(s2h[r]), None)
+        for s in [s for s, (o, c) in model.items() if -1 < c <= 6]:
+            model.pop(s)
+        want_h2f = np.full(cap, -1, np.int64); want_f2h = np.full(N, -1, np.int64); want_chk = np.full(cap, -1, np.int64)
+        for s, (o, c) in model.items():
+            want_h2f[s] = o; want_f2h[o] = s; want_chk[s] = c
+        np.testing.assert_array_equal(t[1].numpy(), want_h2f)
+        np.testing.assert_array_equal(t[2].numpy(), want_f2h)
+        np.testing.assert_array_equal(t[0].numpy(), want_chk)
+        assert 0 < len(model) < 45
