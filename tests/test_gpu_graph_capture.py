@@ -1,0 +1,79 @@
+"""The entry points under HIP graph capture: nothing in them allocates or synchronises, so a caller
+may record them.  Every replay is checked against the eager result, with eager work and
+synchronisations between the replays and fresh input values for each of them."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import random_csr, random_hmap
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def be():
+    import hiscache_backend
+    hiscache_backend.load_library()
+    return hiscache_backend
+
+
+def test_aggregation_and_admission_replay_like_eager(be):
+    rng = np.random.default_rng(90)
+    R, N, F, cap = 3000, 2500, 128, 4096
+    ptr, idx = random_csr(rng, R, N, 9, hub=700)
+    hmap = random_hmap(rng, R, 0.3)
+    T = lambda a: torch.from_numpy(a).to(DEV)
+    ptr_d, idx_d, hmap_d = T(ptr), T(idx), T(hmap)
+    x = torch.zeros(N, F, device=DEV)
+    hbuf = torch.zeros(R, F, device=DEV)
+    g = torch.zeros(R, F, device=DEV)
+    emb = torch.zeros(R, F, device=DEV)
+    slot = torch.full((R,), -1, dtype=torch.int64, device=DEV)
+    sub_to_full = T(rng.permutation(3 * R)[:R].astype(np.int64))
+    thres = torch.tensor([11.3], device=DEV)          # about the median norm of a 128-dim N(0,1) row
+
+    def fresh_state():
+        return dict(table=torch.zeros(cap, F, dtype=torch.float16, device=DEV),
+                    full2slot=torch.full((3 * R,), -1, dtype=torch.int64, device=DEV),
+                    slot2full=torch.full((cap,), -1, dtype=torch.int64, device=DEV),
+                    header=torch.zeros(1, dtype=torch.int64, device=DEV))
+
+    def work(st):
+        out = be._aggr_fwd(be.SUBST_ROW, ptr_d, idx_d, x, hmap_d, hbuf, F, None, R)
+        tr = be.build_transpose(ptr_d, idx_d, hmap_d, R, N, want_edges=False)
+        gx, gh, _ = be._aggr_bwd(ptr_d, idx_d, tr, g, hmap_d, None, x, False, (R, F), F, R, N)
+        mask, score = be.grad_check(g, emb, slot, sub_to_full, thres, st["table"], st["full2slot"], st["slot2full"],
+                                    st["header"], 3)
+        return out, tr[0], tr[1], gx, gh, mask, score
+
+    def load_inputs(seed):
+        gen = torch.Generator(device=DEV).manual_seed(seed)
+        for t in (x, hbuf, g, emb):
+            t.copy_(torch.randn(t.shape, device=DEV, generator=gen))
+
+    load_inputs(0)
+    st_graph = fresh_state()
+    work(st_graph)                                   # warm-up outside capture (library handles, allocator pools)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            captured = work(st_graph)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(1, 5):
+        load_inputs(rep)
+        for k, v in fresh_state().items():
+            st_graph[k].copy_(v)
+        st_eager = fresh_state()
+        eager = work(st_eager)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("out", "ptrT", "rowT", "grad_x", "grad_h", "mask", "score"), captured, eager):
+            assert torch.equal(a, b), (rep, name)
+        for k in st_eager:
+            assert torch.equal(st_graph[k], st_eager[k]), (rep, k)
+        assert 0 < int(st_eager["header"]) < R
