@@ -246,6 +246,47 @@ extern "C" int hc_count_history(const int64_t *ptr, const int64_t *idx, const in
   return HC_OK;
 }
 
+// Input check for a CSR block: thread t < R looks at row t's bounds, thread R + e at edge slot e.
+// report[0] rows whose end lies before their start, report[1] offsets outside [0, E],
+// report[2] neighbour ids outside [0, n_src) among the slots the rows cover.
+namespace {
+__global__ __launch_bounds__(HC_BLOCK) void check_csr_kernel(const int64_t *__restrict__ ptr,
+                                                              const int64_t *__restrict__ idx, int64_t R,
+                                                              int64_t E, int64_t n_src,
+                                                              unsigned long long *__restrict__ report) {
+  const int64_t t = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (t < R) {
+    const int64_t b = ptr[t], e = ptr[t + 1];
+    if (e < b) atomicAdd(report + 0, 1ull);
+    if (b < 0 || b > E || e < 0 || e > E) atomicAdd(report + 1, 1ull);
+    return;
+  }
+  const int64_t slot = t - R;
+  if (slot >= E) return;
+  const int64_t first = ptr[0], last = ptr[R];
+  if (slot < first || slot >= last) return;
+  const int64_t s = idx[slot];
+  if (s < 0 || s >= n_src) atomicAdd(report + 2, 1ull);
+}
+
+__global__ void clear_report(unsigned long long *report) {
+  if (threadIdx.x < 4 && blockIdx.x == 0) report[threadIdx.x] = 0ull;
+}
+}  // namespace
+
+extern "C" int hc_check_csr(const int64_t *ptr, const int64_t *idx, int64_t R, int64_t E, int64_t n_src,
+                            int64_t *report, void *stream) {
+  HC_REQUIRE(R >= 0 && E >= 0 && n_src >= 0 && report);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  unsigned long long *rep = reinterpret_cast<unsigned long long *>(report);
+  clear_report<<<dim3(1), dim3(HC_WAVE), 0, st>>>(rep);
+  if (R == 0) return hc_launch_status();
+  HC_REQUIRE(ptr && (E == 0 || idx));
+  if (!hc_grid_ok((R + E + HC_BLOCK - 1) / HC_BLOCK)) return HC_EUNSUPPORTED;
+  check_csr_kernel<<<dim3(blocks_for(R + E)), dim3(HC_BLOCK), 0, st>>>(ptr, idx, R, E, n_src, rep);
+  return hc_launch_status();
+}
+
 extern "C" int hc_count_num(const int64_t *arr, int64_t n, int64_t mmax, int32_t *out, void *stream) {
   HC_REQUIRE(n >= 0 && mmax >= 0 && out);
   hipStream_t st = static_cast<hipStream_t>(stream);

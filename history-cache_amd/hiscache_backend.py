@@ -66,6 +66,7 @@ _SIGNATURES = {
     "hc_structure_score": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p]),
     "hc_gather_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p]),
+    "hc_check_csr": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p]),
     "hc_evict": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p]),
     "hc_sample_capacity": (_c_int, [_c_i64, _c_p, _c_int, _c_i64, _c_p, _c_p, _c_p]),
     "hc_sample_workspace_bytes": (_c_sz, [_c_i64, _c_p, _c_int, _c_i64]),
@@ -158,6 +159,29 @@ def _workspace(nbytes, device):
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
 
 
+# With HISCACHE_CHECK_INPUTS=1 every aggregation call first checks its CSR block on the device
+# (one extra launch and a synchronisation: for debugging, the kernels themselves trust their indices).
+CHECK_INPUTS = os.environ.get("HISCACHE_CHECK_INPUTS", "0") not in ("", "0")
+
+
+def check_csr(ptr, idx, num_node, n_src):
+    """Raise ValueError if the first ``num_node`` rows of (ptr, idx) are not a valid CSR block over
+    ``n_src`` sources: offsets must not decrease and must stay inside ``idx``, ids inside [0, n_src)."""
+    lib = load_library()
+    _dev(ptr, "ptr", torch.int64)
+    _dev(idx, "idx", torch.int64)
+    R = int(num_node)
+    if R < 0 or R > ptr.numel() - 1:
+        raise ValueError("num_node exceeds the rows of ptr")
+    report = torch.empty(4, dtype=torch.int64, device=ptr.device)
+    _check(lib.hc_check_csr(_ptr(ptr), _ptr(idx), R, idx.numel(), int(n_src), _ptr(report), _stream()),
+           "hc_check_csr")
+    bad = report.tolist()
+    if any(bad[:3]):
+        raise ValueError(f"invalid CSR block: {bad[0]} rows end before they start, {bad[1]} offsets outside "
+                         f"[0, {idx.numel()}], {bad[2]} neighbour ids outside [0, {int(n_src)})")
+
+
 # ----------------------------------------------------------------------------- raw launchers
 def _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, num_node):
     lib = load_library()
@@ -186,6 +210,8 @@ def _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, num_node):
             raise ValueError(f"history_map has {hmap.numel()} entries, needs {need}")
         if mode == SUBST_ROW and hbuf.numel() < R * hsize:
             raise ValueError("history_buffer is smaller than num_node x history_size")
+    if CHECK_INPUTS:
+        check_csr(ptr, idx, R, n_src)
     out_shape = (R, F) if n_head == 1 and x.dim() == 2 else (R, n_head, F)
     out = torch.empty(out_shape, dtype=torch.float32, device=x.device)
     # scratch for the long-row list (large blocks only: the library reports 0 bytes otherwise)

@@ -312,6 +312,15 @@ int hc_edge_types_by_ranges(const int64_t *ptr, const int64_t *idx, const int64_
                             const int64_t *pair_to_rel, int64_t *out, int64_t R, int64_t E,
                             void *stream);
 
+/* hc_check_csr: input check a caller can run before handing a block to the
+ * aggregation entry points, which (like the reference kernels) trust their
+ * indices.  report is int64[4] on the device: [0] rows whose end offset lies
+ * before their start, [1] offsets outside [0, E], [2] neighbour ids outside
+ * [0, n_src) among the slots [ptr[0], ptr[R]), [3] zero.  No reference
+ * counterpart. */
+int hc_check_csr(const int64_t *ptr, const int64_t *idx, int64_t R, int64_t E, int64_t n_src,
+                 int64_t *report, void *stream);
+
 /* hc_structure_score replaces get_graph_structure_score (grad_check.h:22-24,
  * grad_check.cu:132-163) with a level-synchronous, deterministic reading of
  * the same rule: per pass, seeds hold 1; a row with a non-zero value offers

@@ -381,3 +381,22 @@ def test_fwd_long_row_list_overflow_falls_back(be, orc):
                              torch.cuda.current_stream().cuda_stream)
         assert rc == 0
         np.testing.assert_array_equal(out.cpu().numpy(), ref)
+
+
+def test_check_csr_reports_bad_blocks(be):
+    rng = np.random.default_rng(44)
+    R, N = 500, 300
+    ptr, idx = random_csr(rng, R, N, 7)
+    be.check_csr(T(ptr), T(idx), R, N)                          # a valid block passes
+    bad_idx = idx.copy(); bad_idx[[3, 10]] = [N, -1]
+    with pytest.raises(ValueError, match="2 neighbour ids"):
+        be.check_csr(T(ptr), T(bad_idx), R, N)
+    bad_ptr = ptr.copy(); bad_ptr[100] = bad_ptr[101] + 5       # row 99 overshoots, row 100 runs backwards
+    with pytest.raises(ValueError, match="1 rows end before"):
+        be.check_csr(T(bad_ptr), T(idx), R, N)
+    long_ptr = ptr.copy(); long_ptr[-1] += 4                    # the last row reaches past idx
+    with pytest.raises(ValueError, match="offsets outside"):
+        be.check_csr(T(long_ptr), T(idx), R, N)
+    # ids behind ptr[R] are nobody's business
+    tail = np.concatenate([idx, np.array([10**9], np.int64)])
+    be.check_csr(T(ptr), T(tail), R, N)
