@@ -10,6 +10,15 @@
  * of the reference kernel would produce.
  *
  * Index type is int64 everywhere (reference: src/cpp/include/common.h:12).
+ *
+ * Every function here is pinned by the tests against closed forms, brute
+ * force or library routines, except (PARITY UNPINNED against the reference):
+ *   orc_structure_score   the reference result depends on thread scheduling;
+ *                         only the level-synchronous reading is pinned;
+ *   orc_sample_layers     the reference has no sampler (external loader); the
+ *                         rule is pinned through its consequences only;
+ *   edge_types_by_ranges  (hc_oracle.py) stands in for an external library
+ *                         routine whose numbering is not available.
  */
 #include <math.h>
 #include <stdint.h>
