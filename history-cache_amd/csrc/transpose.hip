@@ -65,24 +65,48 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_expand_edges(const int64_t *__res
     for (int64_t i = threadIdx.x; i < span; i += HC_BLOCK) s_ptr[i] = ptr[r_lo + i];
   __syncthreads();
   const uint32_t sentinel = (uint32_t)n_src;
+  // three sweeps over the thread's slots, so that the loads of each sweep are all in flight together
+  int64_t row[TR_ITEMS];
+  bool live[TR_ITEMS];
 #pragma unroll
   for (int it = 0; it < TR_ITEMS; ++it) {
     const int64_t e = e0 + (int64_t)it * HC_BLOCK + threadIdx.x;
-    if (e >= e1) break;
-    const int64_t row = staged ? r_lo + tr_row_of(s_ptr, (int64_t)0, span - 1, e) : tr_row_of(ptr, r_lo, r_hi, e);
-    uint32_t key = sentinel;
-    bool live = row < R && ptr[row] <= e;  // ptr[row + 1] > e by construction when row < R
-    if (live && hmap_row != nullptr && hmap_row[row] != -1) live = false;
-    if (live) {
-      const int64_t s = idx[e];
-      if (s >= 0 && s < n_src) key = (uint32_t)s;
+    live[it] = false;
+    row[it] = 0;
+    if (e < e1) {
+      if (staged) {
+        const int64_t l = tr_row_of(s_ptr, (int64_t)0, span - 1, e);
+        row[it] = r_lo + l;
+        live[it] = row[it] < R && s_ptr[l] <= e;  // ptr[row + 1] > e by construction when row < R
+      } else {
+        row[it] = tr_row_of(ptr, r_lo, r_hi, e);
+        live[it] = row[it] < R && ptr[row[it]] <= e;
+      }
     }
-    keys[e] = key;
+  }
+  if (hmap_row != nullptr) {
+    int64_t h[TR_ITEMS];
+#pragma unroll
+    for (int it = 0; it < TR_ITEMS; ++it) h[it] = live[it] ? hmap_row[row[it]] : -1;
+#pragma unroll
+    for (int it = 0; it < TR_ITEMS; ++it) live[it] = live[it] && h[it] == -1;
+  }
+  int64_t src[TR_ITEMS];
+#pragma unroll
+  for (int it = 0; it < TR_ITEMS; ++it) {
+    const int64_t e = e0 + (int64_t)it * HC_BLOCK + threadIdx.x;
+    src[it] = live[it] ? idx[e] : -1;
+  }
+#pragma unroll
+  for (int it = 0; it < TR_ITEMS; ++it) {
+    const int64_t e = e0 + (int64_t)it * HC_BLOCK + threadIdx.x;
+    if (e >= e1) continue;
+    keys[e] = (src[it] >= 0 && src[it] < n_src) ? (uint32_t)src[it] : sentinel;
     if (VAL_IS_ROW) {
-      vals[e] = live ? (uint32_t)row : (uint32_t)e;
+      vals[e] = live[it] ? (uint32_t)row[it] : (uint32_t)e;
     } else {
       vals[e] = (uint32_t)e;
-      if (live) rows[e] = (uint32_t)row;
+      if (live[it]) rows[e] = (uint32_t)row[it];
     }
   }
 }
