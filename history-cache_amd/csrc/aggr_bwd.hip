@@ -219,6 +219,23 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     const bool hit = hmap[row] != -1;
     float *__restrict__ d = grad_hbuf + row * hsize;
     const float *__restrict__ s = g + row * F;
+    if (hsize == F && (reinterpret_cast<uintptr_t>(grad_hbuf) % 16) == 0) {
+      // the usual shape: one 16-byte store per lane and chunk (F is a multiple of 256 bytes here)
+      float *__restrict__ dv = d + lane * VEC;
+      const float *__restrict__ sv = s + lane * VEC;
+#pragma unroll
+      for (int k = 0; k < CHUNKS; ++k) {
+        float v[VEC];
+        if (hit) {
+          hc_vec<float, VEC>::load(sv + k * HC_WAVE * VEC, v);
+        } else {
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) v[i] = 0.0f;
+        }
+        hc_vec<float, VEC>::store_nt(dv + k * HC_WAVE * VEC, v);
+      }
+      return;
+    }
     for (int64_t c = lane; c < hsize; c += HC_WAVE) d[c] = (hit && c < F) ? s[c] : 0.0f;
     return;
   }

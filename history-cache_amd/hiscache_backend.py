@@ -251,7 +251,11 @@ def build_transpose(ptr, idx, history_map_row, num_node, n_src, num_edge=None, w
     return ptrT, rowT, edgeT
 
 
-def _aggr_bwd(ptr, idx, tr, g, hmap, edge_value, x, want_edge_grad, hbuf_shape, hsize, num_node, n_src):
+def _aggr_bwd(ptr, idx, tr, g, hmap, edge_value, x, want_edge_grad, hbuf_shape, hsize, num_node, n_src,
+              want_hist_grad=True):
+    """Gradient of the aggregation: (grad_input, grad_history_buffer or None, edge_grad or None).
+    ``want_hist_grad=False`` skips the history buffer's gradient (a full-size write that a cached
+    embedding without ``requires_grad`` has no use for)."""
     lib = load_library()
     ptrT, rowT, edgeT = tr
     g = _dev(g.contiguous(), "grad_output", torch.float32)
@@ -262,7 +266,7 @@ def _aggr_bwd(ptr, idx, tr, g, hmap, edge_value, x, want_edge_grad, hbuf_shape, 
     gshape = (n_src, F) if g.dim() == 2 else (n_src, n_head, F)
     grad_x = torch.empty(gshape, dtype=torch.float32, device=dev)
     grad_h = None
-    if hmap is not None:
+    if hmap is not None and want_hist_grad:
         grad_h = torch.empty(hbuf_shape, dtype=torch.float32, device=dev)
         if grad_h.numel() != R * hsize:
             # history buffers longer than num_node rows: only the first num_node rows get gradient
@@ -345,7 +349,7 @@ class _AggrHistory(torch.autograd.Function):
         else:
             tr = build_transpose(ptr, idx, row_map, R, n_src, want_edges=ev is not None)
         grad_x, grad_h, edge_grad = _aggr_bwd(ptr, idx, tr, g, row_map, ev, x, want_eg, hshape, hsize, R,
-                                              n_src)
+                                              n_src, want_hist_grad=want_h)
         if grad_x.dtype != x.dtype:
             grad_x = grad_x.to(x.dtype)
         if mode == SUBST_SRC or not want_h:
