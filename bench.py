@@ -219,6 +219,34 @@ def cpu_baseline_c2(shape):
                       "median of %d runs" % (R, E, N, F, len(times))}
 
 
+def cpu_baseline_c4(M, F):
+    """Admission with PyTorch CPU operators (norm, predicate, masked row copy into an fp16 table) on a
+    1/4-size sample."""
+    import torch
+
+    from hiscache.synthetic import lognormal_grads
+    from oracle import torch_cpu_path as tp
+
+    M = M // 4
+    torch.set_num_threads(os.cpu_count())
+    gen = torch.Generator().manual_seed(4)
+    grad = lognormal_grads(M, F, -3.0, 1.5, device="cpu", generator=gen)
+    emb = torch.randn(M, F, generator=gen)
+    slot = torch.where(torch.rand(M, generator=gen) < 0.35, torch.zeros(M, dtype=torch.int64),
+                       torch.full((M,), -1))
+    table = torch.zeros(M, F, dtype=torch.float16)
+    tp.admission(grad, emb, slot, 0.05, table, 0)
+    times = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        tp.admission(grad, emb, slot, 0.05, table, 0)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return {"value": M / times[2], "unit": "rows/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "%d rows x %d fp32 (1/4 of c4): torch CPU norm, predicate, masked copy into an fp16 table, "
+                      "median of 5 runs" % (M, F)}
+
+
 # ----------------------------------------------------------------------------------------- C4
 def run_c4(args):
     import torch
@@ -656,6 +684,8 @@ def main():
             res["cpu_baseline"] = cpu_baseline_c2(shape)
     elif args.workload == "c4":
         res = run_c4(args)
+        if not args.no_cpu_baseline:
+            res["cpu_baseline"] = cpu_baseline_c4(int(2_000_000 * args.scale), 256)
     elif args.workload == "copy":
         res = run_copy(args)
     elif args.workload == "c5":
