@@ -11,6 +11,11 @@ but run hand-written gfx950 kernels from ``libhiscache_hip.so`` through its C
 ABI (ctypes; raw device pointers, sizes, dtype enums, the current HIP stream).
 ``p2psend`` / ``p2psend_gentensor`` (multi-GPU) are not provided.
 
+Beyond the reference's set: ``aggr_forward_source_history`` (per-source substitution),
+``build_transpose``, ``row_scores``, ``grad_check`` / ``cache_append`` (fused admission), ``evict``,
+``gather_rows`` / ``lookup``, ``typed_csr`` / ``edge_types_by_ranges`` (relational blocks),
+``sample_layers`` (device sampler) and ``check_csr`` (input validation).
+
 There is no CPU or PyTorch fallback: if the shared library is missing or a
 tensor is not on a GPU, the call raises.
 """
