@@ -61,17 +61,20 @@ __device__ __forceinline__ void copy_row_any(const void *hbuf, int hist_dtype, i
 // STREAM: neighbour rows and ids are loaded with the non-temporal hint.  With per-source
 // substitution every edge also looks its source up in the map, and the map (not the rows, which
 // are too many to be reused) is what is worth keeping in the caches.
-template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM>
+// WEIGHTED: acc = fma(row, edge_value[edge], acc) instead of acc += row.
+template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM, bool WEIGHTED>
 __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, const T *__restrict__ vin,
                                                const int64_t *__restrict__ hmap, const T *__restrict__ htab,
-                                               int64_t hsize, int src_mode, int64_t begin, int64_t end,
-                                               int lane, float (&acc)[CHUNKS][VEC]) {
+                                               int64_t hsize, int src_mode, const float *__restrict__ ev,
+                                               int64_t begin, int64_t end, int lane,
+                                               float (&acc)[CHUNKS][VEC]) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   for (int64_t base = begin; base < end; base += HC_WAVE) {
     const int64_t left = end - base;
     const int n = left < HC_WAVE ? (int)left : HC_WAVE;
     // Stage: lane l resolves the address of neighbour base+l.
     int64_t my_addr = 0;
+    float my_w = 0.0f;
     if (lane < n) {
       const int64_t id = STREAM ? __builtin_nontemporal_load(idx + base + lane) : idx[base + lane];
       const T *p = vin + id * F;
@@ -80,6 +83,7 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
         if (slot != -1) p = htab + slot * hsize;
       }
       my_addr = reinterpret_cast<int64_t>(p);
+      if constexpr (WEIGHTED) my_w = ev[base + lane];
     }
     for (int j = 0; j < n; j += UNROLL) {
       float v[UNROLL][CHUNKS][VEC];
@@ -100,11 +104,23 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
         }
       }
 #pragma unroll
-      for (int u = 0; u < UNROLL; ++u)
+      for (int u = 0; u < UNROLL; ++u) {
+        if constexpr (WEIGHTED) {
+          // lanes past the row's end hold zero rows and a zero weight: fma(0, 0, acc) == acc
+          const float w = j + u < n ? hc_readlane_f(my_w, j + u) : 0.0f;
+          if (j + u < n) {
 #pragma unroll
-        for (int k = 0; k < CHUNKS; ++k)
+            for (int k = 0; k < CHUNKS; ++k)
 #pragma unroll
-          for (int i = 0; i < VEC; ++i) acc[k][i] += v[u][k][i];
+              for (int i = 0; i < VEC; ++i) acc[k][i] = __fmaf_rn(v[u][k][i], w, acc[k][i]);
+          }
+        } else {
+#pragma unroll
+          for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[k][i] += v[u][k][i];
+        }
+      }
     }
   }
 }
@@ -175,11 +191,12 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_long_find(const int64_t *__restr
 }
 
 // One long row summed by the four waves of the calling block (all of them must call this).
-template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM>
+template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM, bool WEIGHTED>
 __device__ __forceinline__ void fwd_long_row(const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx,
                                              const T *__restrict__ vin, const int64_t *__restrict__ hmap,
                                              const T *__restrict__ htab, int64_t hsize, int src_mode,
-                                             float *__restrict__ vout, int64_t lrow, int lane, int wave,
+                                             const float *__restrict__ ev, float *__restrict__ vout,
+                                             int64_t lrow, int lane, int wave,
                                              float (*part)[HC_WAVE * VEC * CHUNKS]) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   const int64_t lb = ptr[lrow];
@@ -195,7 +212,8 @@ __device__ __forceinline__ void fwd_long_row(const int64_t *__restrict__ ptr, co
   for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[c][i] = 0.0f;
-  fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM>(idx, vin, hmap, htab, hsize, src_mode, sb, se, lane, acc);
+  fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM, WEIGHTED>(idx, vin, hmap, htab, hsize, src_mode, ev, sb, se, lane,
+                                                           acc);
   if (wave > 0) {
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c)
@@ -214,7 +232,7 @@ __device__ __forceinline__ void fwd_long_row(const int64_t *__restrict__ ptr, co
         float t2 = acc[c][i];
 #pragma unroll
         for (int pw = 0; pw < HC_WAVES_PER_BLOCK - 1; ++pw) t2 += part[pw][(c * HC_WAVE + lane) * VEC + i];
-        o[i] = deg > 0 ? t2 / fdeg : 0.0f;
+        o[i] = WEIGHTED ? t2 : (deg > 0 ? t2 / fdeg : 0.0f);
       }
       if constexpr (STREAM) hc_store_f32_nt<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
       else hc_store_f32<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
@@ -223,11 +241,12 @@ __device__ __forceinline__ void fwd_long_row(const int64_t *__restrict__ ptr, co
   __syncthreads();
 }
 
-template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM>
+template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM, bool WEIGHTED>
 __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const T *__restrict__ vin,
     const int64_t *__restrict__ hmap, const void *__restrict__ hbuf, int hist_dtype, int64_t hsize,
-    int src_mode, float *__restrict__ vout, int64_t R, int64_t long_thres, FwdSched sched) {
+    int src_mode, const float *__restrict__ ev, float *__restrict__ vout, int64_t R, int64_t long_thres,
+    FwdSched sched) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   __shared__ float part[HC_WAVES_PER_BLOCK - 1][F];
   __shared__ int long_rows[FWD_ROWS_PER_BLOCK];
@@ -241,8 +260,8 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
   if ((int)blockIdx.x < sched.front) {
     if (!listed) return;
     for (int t = (int)blockIdx.x; t < n_listed; t += sched.front)
-      fwd_long_row<T, VEC, CHUNKS, UNROLL, STREAM>(ptr, idx, vin, hmap, htab, hsize, src_mode, vout,
-                                                   (int64_t)sched.rows[t], lane, wave, part);
+      fwd_long_row<T, VEC, CHUNKS, UNROLL, STREAM, WEIGHTED>(ptr, idx, vin, hmap, htab, hsize, src_mode, ev, vout,
+                                                             (int64_t)sched.rows[t], lane, wave, part);
     return;
   }
   const int64_t row0 = hc_xcd_block<FWD_XCD_CHUNK>((int64_t)blockIdx.x - sched.front,
@@ -276,13 +295,14 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
         for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
           for (int i = 0; i < VEC; ++i) acc[c][i] = 0.0f;
-        fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM>(idx, vin, hmap, htab, hsize, src_mode, begin, end, lane, acc);
+        fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM, WEIGHTED>(idx, vin, hmap, htab, hsize, src_mode, ev, begin,
+                                                                 end, lane, acc);
         const float fdeg = (float)(int)deg;
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) {
           float o[VEC];
 #pragma unroll
-          for (int i = 0; i < VEC; ++i) o[i] = deg > 0 ? acc[c][i] / fdeg : 0.0f;
+          for (int i = 0; i < VEC; ++i) o[i] = WEIGHTED ? acc[c][i] : (deg > 0 ? acc[c][i] / fdeg : 0.0f);
           if constexpr (STREAM) hc_store_f32_nt<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
           else hc_store_f32<VEC>(orow + c * HC_WAVE * VEC + lane * VEC, o);
         }
@@ -294,8 +314,8 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
   const int n_long = n_long_s;
   // The order in which long rows were noted does not matter: each is summed on its own.
   for (int t = 0; t < n_long; ++t)
-    fwd_long_row<T, VEC, CHUNKS, UNROLL, STREAM>(ptr, idx, vin, hmap, htab, hsize, src_mode, vout,
-                                                 row0 + long_rows[t], lane, wave, part);
+    fwd_long_row<T, VEC, CHUNKS, UNROLL, STREAM, WEIGHTED>(ptr, idx, vin, hmap, htab, hsize, src_mode, ev, vout,
+                                                           row0 + long_rows[t], lane, wave, part);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -381,8 +401,8 @@ struct FwdScratch {
 
 template <typename T, int VEC, int CHUNKS>
 int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const int64_t *hmap,
-                const void *hbuf, int hist_dtype, int64_t hsize, int src_mode, float *vout, int64_t R,
-                FwdScratch ws, hipStream_t st) {
+                const void *hbuf, int hist_dtype, int64_t hsize, int src_mode, const float *ev, float *vout,
+                int64_t R, FwdScratch ws, hipStream_t st) {
   constexpr int per = VEC * CHUNKS;
   constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
   int64_t blocks = (R + FWD_ROWS_PER_BLOCK - 1) / FWD_ROWS_PER_BLOCK;
@@ -403,14 +423,14 @@ int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const i
     fwd_long_find<<<dim3((unsigned)((R + FWD_FIND_TILE - 1) / FWD_FIND_TILE)), dim3(HC_BLOCK), 0, st>>>(
         ptr, src_mode ? nullptr : hmap, R, (int64_t)HC_LONG_ROW_EDGES, sched.head, sched.rows);
   }
-  if (src_mode && hmap != nullptr)
-    fwd_mean_fast<T, VEC, CHUNKS, UNROLL, true><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(
-        ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, vout, R,
-        (int64_t)HC_LONG_ROW_EDGES, sched);
-  else
-    fwd_mean_fast<T, VEC, CHUNKS, UNROLL, false><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(
-        ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, vout, R,
-        (int64_t)HC_LONG_ROW_EDGES, sched);
+#define HC_FWD_LAUNCH(STREAM, WEIGHTED)                                                                \
+  fwd_mean_fast<T, VEC, CHUNKS, UNROLL, STREAM, WEIGHTED><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>( \
+      ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, ev, vout, R,     \
+      (int64_t)HC_LONG_ROW_EDGES, sched)
+  if (ev != nullptr) HC_FWD_LAUNCH(false, true);
+  else if (src_mode && hmap != nullptr) HC_FWD_LAUNCH(true, false);
+  else HC_FWD_LAUNCH(false, false);
+#undef HC_FWD_LAUNCH
   return hc_launch_status();
 }
 
@@ -418,11 +438,11 @@ int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const i
 template <typename T>
 int dispatch_fast(int64_t F, const int64_t *ptr, const int64_t *idx, const void *vin,
                   const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize, int src_mode,
-                  float *vout, int64_t R, FwdScratch ws, hipStream_t st, bool *handled) {
+                  const float *ev, float *vout, int64_t R, FwdScratch ws, hipStream_t st, bool *handled) {
   *handled = true;
 #define HC_FAST(V, C)                                                                              \
   if (F == 64 * (V) * (C))                                                                         \
-    return launch_fast<T, V, C>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, vout, R, ws, st);
+    return launch_fast<T, V, C>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, ev, vout, R, ws, st);
   constexpr int VMAX = 16 / (int)sizeof(T);
   if constexpr (VMAX == 8) {
     HC_FAST(8, 1) HC_FAST(8, 2) HC_FAST(8, 3) HC_FAST(8, 4)
@@ -512,18 +532,20 @@ extern "C" int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, con
                        (reinterpret_cast<uintptr_t>(vout) % 16 == 0) &&
                        (!src_mode || !hmap ||
                         ((reinterpret_cast<uintptr_t>(hbuf) % 16 == 0) && ((hsize * esz) % 16 == 0)));
-  if (!edge_value && n_head == 1 && aligned && vin != nullptr) {
+  // single-head weighted sums share the fast path; a history row of a weighted block copies hbuf[r, :F]
+  const bool weighted_ok = !edge_value || (!src_mode && (!hmap || hsize >= F));
+  if (n_head == 1 && weighted_ok && aligned && vin != nullptr) {
     bool handled = false;
     int rc;
     if (in_dtype == HC_F32)
-      rc = dispatch_fast<float>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, vout, R, ws, st,
-                                &handled);
+      rc = dispatch_fast<float>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value, vout, R, ws,
+                                st, &handled);
     else if (in_dtype == HC_F16)
-      rc = dispatch_fast<__half>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, vout, R, ws, st,
-                                 &handled);
+      rc = dispatch_fast<__half>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value, vout, R, ws,
+                                 st, &handled);
     else
       rc = dispatch_fast<__hip_bfloat16>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode,
-                                         vout, R, ws, st, &handled);
+                                         edge_value, vout, R, ws, st, &handled);
     if (handled) return rc;
   }
   if (in_dtype == HC_F32)

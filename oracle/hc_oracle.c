@@ -155,9 +155,22 @@ int orc_fwd_mean_row(const Index *ptr, const Index *idx, const float *vin,
 /* Weighted-sum aggregation, follows gen_fwd_history_v2_edge_value,
  * history_aggr.cu:42-78: no division, every non-history row is written
  * (0 for empty rows, :77).  `rs += vin * val` is one fused multiply-add. */
+static void wsum_rows_seq(const Index *idx, const float *ev, const float *vin, Index F, Index b,
+                          Index e, float *o) {
+  for (Index j = b; j < e; ++j) {
+    const float *x = vin + idx[j] * F;
+    float w = ev[j];
+    for (Index c = 0; c < F; ++c) o[c] = fmaf(x[c], w, o[c]);
+  }
+}
+
+/* split_above as in orc_fwd_mean_row: the device library's quarter rule for rows with more than
+ * split_above edges (four contiguous quarters, each from zero in CSR order, combined left to right). */
 int orc_fwd_edge_value(const Index *ptr, const Index *idx, const float *ev,
                        const float *vin, const Index *hmap, const float *hbuf,
-                       float *vout, Index R, Index F, Index hsize) {
+                       float *vout, Index R, Index F, Index hsize, Index split_above) {
+  float *part = (float *)malloc((size_t)F * sizeof(float));
+  if (!part) return ORC_EINVAL;
   for (Index row = 0; row < R; ++row) {
     float *o = vout + row * F;
     if (hmap && hmap[row] != -1) {
@@ -165,12 +178,27 @@ int orc_fwd_edge_value(const Index *ptr, const Index *idx, const float *ev,
       continue;
     }
     for (Index c = 0; c < F; ++c) o[c] = 0.0f;
-    for (Index j = ptr[row]; j < ptr[row + 1]; ++j) {
-      const float *x = vin + idx[j] * F;
-      float w = ev[j];
-      for (Index c = 0; c < F; ++c) o[c] = fmaf(x[c], w, o[c]);
+    Index b = ptr[row], e = ptr[row + 1];
+    Index n = e - b;
+    if (split_above > 0 && n > split_above) {
+      Index q = (n + 3) / 4;
+      for (int w = 0; w < 4; ++w) {
+        Index sb = b + w * q, se = sb + q;
+        if (sb > e) sb = e;
+        if (se > e) se = e;
+        if (w == 0) {
+          wsum_rows_seq(idx, ev, vin, F, sb, se, o);
+        } else {
+          memset(part, 0, (size_t)F * sizeof(float));
+          wsum_rows_seq(idx, ev, vin, F, sb, se, part);
+          for (Index c = 0; c < F; ++c) o[c] += part[c];
+        }
+      }
+    } else {
+      wsum_rows_seq(idx, ev, vin, F, b, e, o);
     }
   }
+  free(part);
   return ORC_OK;
 }
 

@@ -89,7 +89,7 @@ def fwd_mean_row(ptr, idx, vin, hmap, hbuf, num_node=None, split_above=0):
     return out
 
 
-def fwd_edge_value(ptr, idx, ev, vin, hmap, hbuf, num_node=None):
+def fwd_edge_value(ptr, idx, ev, vin, hmap, hbuf, num_node=None, split_above=0):
     ptr, idx, vin, ev = _i64(ptr), _i64(idx), _f32(vin), _f32(ev)
     R = len(ptr) - 1 if not num_node else int(num_node)
     if ev.ndim == 2:
@@ -110,7 +110,7 @@ def fwd_edge_value(ptr, idx, ev, vin, hmap, hbuf, num_node=None):
         hsize = hbuf.shape[-1]
     out = np.zeros((R, F), np.float32)
     _check(lib().orc_fwd_edge_value(_p(ptr), _p(idx), _p(ev), _p(vin), _p(hmap), _p(hbuf), _p(out),
-                                    _I(R), _I(F), _I(hsize)), "fwd_edge_value")
+                                    _I(R), _I(F), _I(hsize), _I(split_above)), "fwd_edge_value")
     return out
 
 
