@@ -34,7 +34,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c4", "c3", "c5", "sample", "copy"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c2w", "c4", "c3", "c5", "sample", "copy"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
@@ -183,6 +183,60 @@ def run_c2(args, row_mode=False):
         },
     }
     return res, dict(R=R, E=E, N=N, F=F)
+
+
+def run_c2w(args):
+    """Weighted (edge_value) aggregation on the C2 block: forward, transposed view with edge slots,
+    backward of the input and the SDDMM gradient of the edge values."""
+    import torch
+
+    import hiscache_backend as be
+    from hiscache.synthetic import power_law_block
+
+    dev = "cuda:0"
+    s = args.scale
+    R, E, N, F = int(1_000_000 * s), int(20_000_000 * s), int(10_000_000 * s), 256
+    ptr, idx = power_law_block(R, E, N, alpha=2.1, max_degree=5000, seed=2)
+    ptr, idx = ptr.to(dev), idx.to(dev)
+    gen = torch.Generator(device=dev).manual_seed(2)
+    feat = torch.randn(N, F, device=dev, generator=gen)
+    g = torch.randn(R, F, device=dev, generator=gen)
+    ev = torch.rand(E, device=dev, generator=gen)
+    clk_f, clk_t, clk_b = KernelClock(), KernelClock(), KernelClock()
+
+    def step():
+        clk_f(lambda: be._aggr_fwd(be.SUBST_ROW, ptr, idx, feat, None, None, 0, ev, R))
+        tr = clk_t(lambda: be.build_transpose(ptr, idx, None, R, N, want_edges=True))
+        clk_b(lambda: be._aggr_bwd(ptr, idx, tr, g, None, ev, feat, True, None, 0, R, N))
+
+    for _ in range(args.warmup):
+        step()
+    sync()
+    for c in (clk_f, clk_t, clk_b):
+        c.reset()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    sync()
+    sec = (time.perf_counter() - t0) / args.steps
+    t_f, t_t, t_b = clk_f.mean_ms(), clk_t.mean_ms(), clk_b.mean_ms()
+    bytes_f = (R + 1) * 8 + E * (8 + 4) + E * F * 4 + R * F * 4
+    bytes_b = E * F * 4 + E * (4 + 4 + 4) + (N + 1) * 8 + N * F * 4      # input gradient
+    bytes_eg = E * (2 * F * 4 + 8 + 4)                                    # edge gradient: two rows per edge
+    return {
+        "metric": "aggregated edges/sec (weighted fwd+bwd+edge_grad)", "value": E / sec, "unit": "edges/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "c2w: weighted aggregation (edge_value) on the c2 block, R=%d, E=%d, %d sources x %d "
+                               "fp32: fwd + transposed view with edge slots + bwd (input gradient and edge gradient)"
+                               % (R, E, N, F)},
+        "roofline": {"bound": "hbm", "kernel": "fwd_mean_fast<float,4,1,8,false,true>",
+                     "achieved": bytes_f / (t_f * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": bytes_f / (t_f * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes": bytes_f, "launch_ms": t_f},
+        "kernels": {"fwd_ms": t_f, "fwd_GBps": bytes_f / (t_f * 1e-3) / 1e9, "transpose_ms": t_t, "bwd_ms": t_b,
+                    "bwd_GBps": (bytes_b + bytes_eg) / (t_b * 1e-3) / 1e9},
+    }
 
 
 def cpu_baseline_c2(shape):
@@ -682,6 +736,8 @@ def main():
         if not args.no_cpu_baseline:
             torch.cuda.empty_cache()
             res["cpu_baseline"] = cpu_baseline_c2(shape)
+    elif args.workload == "c2w":
+        res = run_c2w(args)
     elif args.workload == "c4":
         res = run_c4(args)
         if not args.no_cpu_baseline:

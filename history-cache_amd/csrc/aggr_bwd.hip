@@ -202,12 +202,14 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_hub_final(const int64_t *__restr
   for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store(o + k * HC_WAVE * VEC, acc[k]);
 }
 
-template <int VEC, int CHUNKS, int UNROLL>
+// WEIGHTED: every transposed edge contributes g[row] * edge_value[edge] (product rounded, then
+// added) instead of g[row] / deg(row); edgeT gives the edge slot of a transposed edge.
+template <int VEC, int CHUNKS, int UNROLL, bool WEIGHTED>
 __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ ptrT, const int32_t *__restrict__ rowT,
-    const float *__restrict__ g, const int64_t *__restrict__ hmap, float *__restrict__ grad_vin,
-    float *__restrict__ grad_hbuf, int64_t hsize, int64_t R, int64_t n_src, int64_t src_blocks,
-    int64_t hub_thres) {
+    const int32_t *__restrict__ edgeT, const float *__restrict__ ev, const float *__restrict__ g,
+    const int64_t *__restrict__ hmap, float *__restrict__ grad_vin, float *__restrict__ grad_hbuf,
+    int64_t hsize, int64_t R, int64_t n_src, int64_t src_blocks, int64_t hub_thres) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   constexpr int S = BWD_SRC_PER_WAVE;
   const int lane = hc_lane();
@@ -290,7 +292,8 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     float my_deg = 1.0f;
     if (lane < n) {
       my_row = rowT[base + lane];
-      my_deg = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
+      if constexpr (WEIGHTED) my_deg = ev[edgeT[base + lane]];   // the weight takes the divisor's place
+      else my_deg = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
     }
     for (int j = 0; j < n; j += UNROLL) {
       float v[UNROLL][CHUNKS][VEC];
@@ -323,7 +326,8 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
 #pragma unroll
           for (int k = 0; k < CHUNKS; ++k)
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) acc[k][i] += v[u][k][i] / d[u];
+            for (int i = 0; i < VEC; ++i)
+              acc[k][i] += WEIGHTED ? __fmul_rn(v[u][k][i], d[u]) : v[u][k][i] / d[u];
         }
       }
     }
@@ -459,10 +463,89 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_edge_grad(
   }
 }
 
+// edge_grad on the fast widths, single head: one wave per 64 consecutive edge slots, whatever rows
+// they belong to (a row of thousands of edges is shared by many waves).  Lane l finds the row of
+// slot base + l by binary search over the row offsets between the rows of the wave's first and last
+// slot; then, UNROLL edges at a time, the wave loads g[row] and vin[idx] (consecutive edges of one
+// row re-read the same g row from L1), forms the 64 per-lane partial dot products with fused
+// multiply-adds and sums them with the butterfly.  Slots of history rows and slots behind the last
+// row get 0.
+template <typename T, int VEC, int CHUNKS, int UNROLL>
+__global__ __launch_bounds__(HC_BLOCK) void bwd_edge_grad_fast(
+    const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const float *__restrict__ g,
+    const int64_t *__restrict__ hmap, const T *__restrict__ vin, float *__restrict__ edge_grad,
+    int64_t E_total, int64_t R) {
+  constexpr int F = HC_WAVE * VEC * CHUNKS;
+  const int lane = hc_lane();
+  const int64_t base = ((int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block()) * HC_WAVE;
+  if (base >= E_total) return;
+  const int64_t left = E_total - base;
+  const int n = left < HC_WAVE ? (int)left : HC_WAVE;
+  // rows of the first and the last slot: largest r in [0, R] with ptr[r] <= slot
+  int64_t lo = 0, hi = R;
+  const int64_t probe = lane == 0 ? base : base + n - 1;
+  while (lo < hi) {
+    const int64_t mid = (lo + hi + 1) >> 1;
+    if (ptr[mid] <= probe) lo = mid;
+    else hi = mid - 1;
+  }
+  // lanes 0 and 1 searched for the first and the last slot (every other lane repeated the last)
+  int64_t a = hc_readlane64(lo, 0), b = hc_readlane64(lo, 1);
+  int64_t my_row = -1, my_id = 0;
+  if (lane < n) {
+    const int64_t e = base + lane;
+    while (a < b) {
+      const int64_t mid = (a + b + 1) >> 1;
+      if (ptr[mid] <= e) a = mid;
+      else b = mid - 1;
+    }
+    if (a < R && ptr[a] <= e && (hmap == nullptr || hmap[a] == -1)) {
+      my_row = a;
+      my_id = idx[e];
+    }
+  }
+  float my_out = 0.0f;
+  for (int j = 0; j < n; j += UNROLL) {
+    float x[UNROLL][CHUNKS][VEC], gr[UNROLL][CHUNKS][VEC];
+    bool live[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      live[u] = false;
+      if (j + u < n) {
+        const int64_t r = hc_readlane64(my_row, j + u);
+        if (r >= 0) {
+          live[u] = true;
+          const T *px = vin + hc_readlane64(my_id, j + u) * F + lane * VEC;
+          const float *pg = g + r * F + lane * VEC;
+#pragma unroll
+          for (int k = 0; k < CHUNKS; ++k) {
+            hc_vec<T, VEC>::load(px + k * HC_WAVE * VEC, x[u][k]);
+            hc_vec<float, VEC>::load(pg + k * HC_WAVE * VEC, gr[u][k]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      if (live[u]) {  // wave-uniform
+        float part = 0.0f;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) part = __fmaf_rn(gr[u][k][i], x[u][k][i], part);
+        part = hc_wave_sum_butterfly(part);
+        if (lane == j + u) my_out = part;
+      }
+    }
+  }
+  if (lane < n) edge_grad[base + lane] = my_out;
+}
+
 template <int VEC, int CHUNKS>
-int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, const float *g,
-                const int64_t *hmap, float *grad_vin, float *grad_hbuf, int64_t hsize, int64_t R,
-                int64_t n_src, int64_t E_slots, void *workspace, size_t workspace_bytes, hipStream_t st) {
+int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, const int32_t *edgeT,
+                const float *ev, const float *g, const int64_t *hmap, float *grad_vin, float *grad_hbuf,
+                int64_t hsize, int64_t R, int64_t n_src, int64_t E_slots, void *workspace,
+                size_t workspace_bytes, hipStream_t st) {
   constexpr int per = VEC * CHUNKS;
   constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
   constexpr int F = HC_WAVE * VEC * CHUNKS;
@@ -474,8 +557,9 @@ int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, co
   int64_t hub_thres = 0;
   BwdHubLayout L = bwd_hub_layout(E_slots, F);
   char *ws = static_cast<char *>(workspace);
-  const bool hubs = workspace != nullptr && E_slots > BWD_CHUNK && n_src > 0 && workspace_bytes >= L.total &&
-                    reinterpret_cast<uintptr_t>(ws) % 256 == 0;
+  // weighted sums keep the strictly sequential order (no hub chunks)
+  const bool hubs = ev == nullptr && workspace != nullptr && E_slots > BWD_CHUNK && n_src > 0 &&
+                    workspace_bytes >= L.total && reinterpret_cast<uintptr_t>(ws) % 256 == 0;
   BwdHubHeader *hh = reinterpret_cast<BwdHubHeader *>(ws);
   int32_t *hub_src = reinterpret_cast<int32_t *>(ws + L.hub_src);
   int32_t *hub_chunk0 = reinterpret_cast<int32_t *>(ws + L.hub_chunk0);
@@ -493,8 +577,12 @@ int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, co
         ptr, ptrT, rowT, g, hh, hub_src, hub_chunk0, chunk_hub, partial, L.max_chunks);
     if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
   }
-  bwd_mean_fast<VEC, CHUNKS, UNROLL><<<dim3((unsigned)(sb + hb)), dim3(HC_BLOCK), 0, st>>>(
-      ptr, ptrT, rowT, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hub_thres);
+  if (ev != nullptr)
+    bwd_mean_fast<VEC, CHUNKS, UNROLL, true><<<dim3((unsigned)(sb + hb)), dim3(HC_BLOCK), 0, st>>>(
+        ptr, ptrT, rowT, edgeT, ev, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hub_thres);
+  else
+    bwd_mean_fast<VEC, CHUNKS, UNROLL, false><<<dim3((unsigned)(sb + hb)), dim3(HC_BLOCK), 0, st>>>(
+        ptr, ptrT, rowT, edgeT, ev, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hub_thres);
   if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
   if (hubs) {
     const int64_t hbk = (L.max_hubs + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
@@ -544,13 +632,14 @@ extern "C" int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t
   bool done = false;
   const bool aligned = (reinterpret_cast<uintptr_t>(g) % 16 == 0) &&
                        (reinterpret_cast<uintptr_t>(grad_vin) % 16 == 0);
-  if (!edge_value && n_head == 1 && aligned) {
+  // single-head weighted sums share the fast kernel when the history buffer has the plain width
+  if (n_head == 1 && aligned && (!edge_value || !grad_hbuf || hsize == F)) {
     int rc = HC_OK;
     done = true;
 #define HC_FAST(V, C)                                                                             \
   if (F == 64 * (V) * (C))                                                                        \
-    rc = launch_fast<V, C>(ptr, ptrT, rowT, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, E_total,  \
-                           workspace, workspace_bytes, st);                                      \
+    rc = launch_fast<V, C>(ptr, ptrT, rowT, edgeT, edge_value, g, hmap, grad_vin, grad_hbuf, hsize, R, \
+                           n_src, E_total, workspace, workspace_bytes, st);                         \
   else
     HC_FAST(4, 1) HC_FAST(4, 2) HC_FAST(4, 3) HC_FAST(4, 4) HC_FAST(2, 1) HC_FAST(2, 3) HC_FAST(1, 1)
     HC_FAST(1, 3) done = false;
@@ -579,7 +668,32 @@ extern "C" int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t
       if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
     }
   }
-  if (edge_grad && E_total > 0) {
+  bool eg_done = false;
+  if (edge_grad && E_total > 0 && n_head == 1 && (reinterpret_cast<uintptr_t>(vin) % 16 == 0) &&
+      (reinterpret_cast<uintptr_t>(g) % 16 == 0)) {
+    const int64_t wb = ((E_total + HC_WAVE - 1) / HC_WAVE + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+    if (!hc_grid_ok(wb)) return HC_EUNSUPPORTED;
+    dim3 gr((unsigned)wb), bl(HC_BLOCK);
+    eg_done = true;
+#define HC_EG(T, V, C)                                                                                 \
+  if (F == 64 * (V) * (C))                                                                             \
+    bwd_edge_grad_fast<T, V, C, ((V) * (C) >= 16 ? 2 : ((V) * (C) >= 8 ? 4 : 8))><<<gr, bl, 0, st>>>(     \
+        ptr, idx, g, hmap, static_cast<const T *>(vin), edge_grad, E_total, R);                         \
+  else
+    if (in_dtype == HC_F32) {
+      HC_EG(float, 4, 1) HC_EG(float, 4, 2) HC_EG(float, 4, 3) HC_EG(float, 4, 4) HC_EG(float, 2, 1)
+      HC_EG(float, 1, 1) eg_done = false;
+    } else if (in_dtype == HC_F16) {
+      HC_EG(__half, 4, 1) HC_EG(__half, 4, 2) HC_EG(__half, 4, 3) HC_EG(__half, 4, 4) HC_EG(__half, 2, 1)
+      HC_EG(__half, 1, 1) eg_done = false;
+    } else {
+      HC_EG(__hip_bfloat16, 4, 1) HC_EG(__hip_bfloat16, 4, 2) HC_EG(__hip_bfloat16, 4, 3)
+      HC_EG(__hip_bfloat16, 4, 4) HC_EG(__hip_bfloat16, 2, 1) HC_EG(__hip_bfloat16, 1, 1) eg_done = false;
+    }
+#undef HC_EG
+    if (eg_done && hc_launch_status() != HC_OK) return HC_ELAUNCH;
+  }
+  if (edge_grad && E_total > 0 && !eg_done) {
     const int64_t rb = (R * n_head + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
     const int64_t tail_blocks = 64;
     if (!hc_grid_ok(rb + tail_blocks)) return HC_EUNSUPPORTED;

@@ -220,7 +220,7 @@ def _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, num_node):
     out_shape = (R, F) if n_head == 1 and x.dim() == 2 else (R, n_head, F)
     out = torch.empty(out_shape, dtype=torch.float32, device=x.device)
     # scratch for the long-row list (large blocks only: the library reports 0 bytes otherwise)
-    ws_bytes = int(lib.hc_aggr_fwd_workspace_bytes(R, idx.numel())) if edge_value is None else 0
+    ws_bytes = int(lib.hc_aggr_fwd_workspace_bytes(R, idx.numel())) if n_head == 1 else 0
     ws = _workspace(ws_bytes, x.device) if ws_bytes > 0 else None
     rc = lib.hc_aggr_fwd(mode, _ptr(ptr), _ptr(idx), _ptr(x), _float_dtype(x, "input"),
                          _ptr(hmap), _ptr(hbuf), _float_dtype(hbuf, "history_buffer") if hmap is not None else 0,

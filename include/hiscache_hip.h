@@ -76,7 +76,8 @@ int hc_device_count(void);
  * requires edge_value.
  * Summation order (fp32, fixed, so results are bit-reproducible): a row is
  * summed in CSR order; when hc_aggr_fwd_long_row_edges() reports a threshold
- * T > 0 for the shape, a row with more than T edges is summed as four
+ * T > 0 for the shape (mean and single-head weighted aggregation on widths
+ * that are a multiple of 64), a row with more than T edges is summed as four
  * contiguous quarters of ceil(deg/4) edges, each in CSR order, combined left to
  * right ((q0+q1)+q2)+q3, then divided.
  * workspace (optional, NULL allowed; 256-byte aligned, of
@@ -133,8 +134,8 @@ int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hm
  * of hc_aggr_bwd_workspace_bytes() is given and hc_aggr_bwd_chunk_edges(F)
  * reports C > 0, a source with more than C incoming edges is summed in chunks
  * of C consecutive edges (each chunk in order, by its own wave) and the chunk
- * sums are combined left to right; without a workspace (NULL) every source is
- * summed strictly in order by one wave.  The workspace must be 256-byte
+ * sums are combined left to right; without a workspace (NULL), and always for
+ * weighted sums, every source is summed strictly in order by one wave.  The workspace must be 256-byte
  * aligned. */
 size_t hc_aggr_bwd_workspace_bytes(int64_t E_total, int64_t F);
 int64_t hc_aggr_bwd_chunk_edges(int64_t F);

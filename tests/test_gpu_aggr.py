@@ -401,3 +401,39 @@ def test_check_csr_reports_bad_blocks(be):
     # ids behind ptr[R] are nobody's business
     tail = np.concatenate([idx, np.array([10**9], np.int64)])
     be.check_csr(T(ptr), T(tail), R, N)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_weighted_fast_path_prefix_rows_and_dtypes(be, orc, dtype):
+    """Single-head weighted aggregation on a fast width over a row prefix: edge slots behind the last
+    used row get a zero edge gradient, history rows too; fp16 inputs accumulate in fp32."""
+    rng = np.random.default_rng(46)
+    R_all, R, N, F = 500, 380, 300, 128
+    ptr, idx = random_csr(rng, R_all, N, 9, hub=900)
+    E = len(idx)
+    vin = T(rng.standard_normal((N, F)).astype(np.float32), dtype)
+    v32 = vin.float().cpu().numpy()
+    ev = rng.standard_normal(E).astype(np.float32)
+    g = rng.standard_normal((R, F)).astype(np.float32)
+    hmap = random_hmap(rng, R, 0.3)
+    hbuf = rng.standard_normal((R, F)).astype(np.float32)
+    x = vin.clone().requires_grad_(True)
+    evt = T(ev).requires_grad_(True)
+    out = be.aggr_forward_history_edge_value(x, T(ptr), T(idx), evt, T(hmap), T(hbuf), F, R)
+    ref = orc.fwd_edge_value(ptr[: R + 1], idx, ev, v32, hmap, hbuf, split_above=be.long_row_edges(F, dtype))
+    np.testing.assert_array_equal(out.detach().cpu().numpy(), ref)
+    out.backward(T(g))
+    gx, _, eg = orc.bwd_edge_value(ptr[: R + 1], idx, ev, g, hmap, v32, N, hsize=F, want_edge_grad=True)
+    got_gx = x.grad.float().cpu().numpy()
+    if dtype == torch.float32:
+        np.testing.assert_array_equal(got_gx, gx)
+    else:
+        np.testing.assert_allclose(got_gx, gx, rtol=1e-2, atol=1e-2 * np.abs(gx).max())
+    got = evt.grad.cpu().numpy()
+    used = int(ptr[R])
+    assert (got[used:] == 0).all() and used < E
+    dst = np.repeat(np.arange(R), np.diff(ptr[: R + 1]))
+    hist_edge = hmap[dst] != -1
+    assert (got[:used][hist_edge] == 0).all() and hist_edge.any()
+    scale = (np.abs(g[dst]) * np.abs(v32[idx[:used]])).sum(-1)
+    assert (np.abs(got[:used] - eg[:used]) <= 1e-5 * scale + 1e-7).all()
