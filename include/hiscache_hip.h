@@ -79,7 +79,7 @@ int hc_device_count(void);
  * T > 0 for the shape (mean and single-head weighted aggregation on widths
  * that are a multiple of 64), a row with more than T edges is summed as four
  * contiguous quarters of ceil(deg/4) edges, each in CSR order, combined left to
- * right ((q0+q1)+q2)+q3, then divided.
+ * right ((q0+q1)+q2)+q3, then divided (mean only).
  * workspace (optional, NULL allowed; 256-byte aligned, of
  * hc_aggr_fwd_workspace_bytes(R, E) bytes, E = an upper bound of ptr[R]): on
  * large blocks the long rows are listed first and scheduled at the start of
