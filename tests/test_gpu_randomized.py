@@ -87,3 +87,20 @@ def test_random_block_forward_backward(be, orc, seed, R, N, F, mean_deg, n_long,
     out_s = be.aggr_forward_source_history(T(x), T(ptr), T(idx), T(smap), T(hist))
     np.testing.assert_array_equal(out_s.cpu().numpy(),
                                   orc.fwd_mean_src(ptr, idx, x, smap, hist, split_above=be.long_row_edges(F)))
+    # single-head weighted sums over the same block (fast widths take the gather kernels too)
+    ev = rng.standard_normal(len(idx)).astype(np.float32)
+    xw = T(x).requires_grad_(True)
+    evt = T(ev).requires_grad_(True)
+    if hmap is not None:
+        out_w = be.aggr_forward_history_edge_value(xw, T(ptr), T(idx), evt, T(hmap), T(hbuf), F, R)
+    else:
+        out_w = be.aggr_forward_history_edge_value(xw, T(ptr), T(idx), evt, none, none, 0, R)
+    np.testing.assert_array_equal(out_w.detach().cpu().numpy(),
+                                  orc.fwd_edge_value(ptr, idx, ev, x, hmap, hbuf, split_above=be.long_row_edges(F)))
+    out_w.backward(T(g))
+    gxw, _, egw = orc.bwd_edge_value(ptr, idx, ev, g, hmap, x, N, hsize=F, want_edge_grad=True)
+    np.testing.assert_array_equal(xw.grad.cpu().numpy(), gxw)
+    dst = np.repeat(np.arange(R), np.diff(ptr))
+    scale = (np.abs(g[dst]) * np.abs(x[idx])).sum(-1)
+    assert (np.abs(evt.grad.cpu().numpy() - egw) <= 1e-5 * scale + 1e-7).all()
+
