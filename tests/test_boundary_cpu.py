@@ -130,3 +130,12 @@ def test_processed_dataset_files_round_trip(tmp_path):
     np.asarray(indices[:-3], np.int64).tofile(os.path.join(d, "csr_idx_undirected.dat"))
     with pytest.raises(ValueError):
         ds.graph()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True,
+                       text=True, timeout=120)
+    assert p.returncode == 2 and "one GPU" in p.stderr and p.stdout.strip() == ""
