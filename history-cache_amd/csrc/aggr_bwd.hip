@@ -367,16 +367,34 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_generic(
         if (WEIGHTED) my_s = ev[(int64_t)edgeT[base + lane] * H + head];
         else my_s = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
       }
-      for (int j = 0; j < n; ++j) {
-        const int r = __builtin_amdgcn_readlane(my_row, j);
-        const float s = hc_readlane_f(my_s, j);
-        const float *p = g + ((int64_t)r * H + head) * F;
+      constexpr int GEN_UNROLL = 4;  // gradient rows in flight before the first add (order kept)
+      for (int j = 0; j < n; j += GEN_UNROLL) {
+        float x[GEN_UNROLL][TILE_K];
+        float sc[GEN_UNROLL];
 #pragma unroll
-        for (int k = 0; k < TILE_K; ++k) {
-          const int64_t c = c0 + k * HC_WAVE + lane;
-          if (c < F) {
-            const float x = p[c];
-            acc[k] += WEIGHTED ? __fmul_rn(x, s) : x / s;
+        for (int u = 0; u < GEN_UNROLL; ++u) {
+          sc[u] = 1.0f;
+#pragma unroll
+          for (int k = 0; k < TILE_K; ++k) x[u][k] = 0.0f;
+          if (j + u < n) {
+            const int r = __builtin_amdgcn_readlane(my_row, j + u);
+            sc[u] = hc_readlane_f(my_s, j + u);
+            const float *p = g + ((int64_t)r * H + head) * F;
+#pragma unroll
+            for (int k = 0; k < TILE_K; ++k) {
+              const int64_t c = c0 + k * HC_WAVE + lane;
+              if (c < F) x[u][k] = p[c];
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < GEN_UNROLL; ++u) {
+          if (j + u < n) {
+#pragma unroll
+            for (int k = 0; k < TILE_K; ++k) {
+              const int64_t c = c0 + k * HC_WAVE + lane;
+              if (c < F) acc[k] += WEIGHTED ? __fmul_rn(x[u][k], sc[u]) : x[u][k] / sc[u];
+            }
           }
         }
       }

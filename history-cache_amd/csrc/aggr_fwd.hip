@@ -368,15 +368,31 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_generic(
         my_addr = reinterpret_cast<int64_t>(p);
         if (WEIGHTED) my_w = ev[(base + lane) * H + head];
       }
-      for (int j = 0; j < n; ++j) {
-        const T *p = reinterpret_cast<const T *>(hc_readlane64(my_addr, j));
-        const float w = WEIGHTED ? hc_readlane_f(my_w, j) : 1.0f;
+      // GEN_UNROLL neighbour rows are loaded before the first add; the adds keep the edge order
+      constexpr int GEN_UNROLL = 4;
+      for (int j = 0; j < n; j += GEN_UNROLL) {
+        float x[GEN_UNROLL][TILE_K];
+        float w[GEN_UNROLL];
 #pragma unroll
-        for (int k = 0; k < TILE_K; ++k) {
-          const int64_t c = c0 + k * HC_WAVE + lane;
-          if (c < F) {
-            const float x = hc_to_f32<T>(p[c]);
-            acc[k] = WEIGHTED ? __fmaf_rn(x, w, acc[k]) : acc[k] + x;
+        for (int u = 0; u < GEN_UNROLL; ++u) {
+          w[u] = 0.0f;
+#pragma unroll
+          for (int k = 0; k < TILE_K; ++k) x[u][k] = 0.0f;
+          if (j + u < n) {
+            const T *p = reinterpret_cast<const T *>(hc_readlane64(my_addr, j + u));
+            w[u] = WEIGHTED ? hc_readlane_f(my_w, j + u) : 1.0f;
+#pragma unroll
+            for (int k = 0; k < TILE_K; ++k) {
+              const int64_t c = c0 + k * HC_WAVE + lane;
+              if (c < F) x[u][k] = hc_to_f32<T>(p[c]);
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < GEN_UNROLL; ++u) {
+          if (j + u < n) {
+#pragma unroll
+            for (int k = 0; k < TILE_K; ++k) acc[k] = WEIGHTED ? __fmaf_rn(x[u][k], w[u], acc[k]) : acc[k] + x[u][k];
           }
         }
       }
