@@ -139,3 +139,23 @@ def test_bench_refuses_more_than_one_gpu():
     p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True,
                        text=True, timeout=120)
     assert p.returncode == 2 and "one GPU" in p.stderr and p.stdout.strip() == ""
+
+
+def test_header_is_plain_c_and_links(tmp_path):
+    """include/hiscache_hip.h compiles as C11 and a C program linked against the library can call it
+    (no GPU is touched: hc_version / hc_strerror / hc_device_count only)."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib_dir = os.path.join(root, "history-cache_amd")
+    if not os.path.exists(os.path.join(lib_dir, "libhiscache_hip.so")):
+        pytest.skip("library not built")
+    src = tmp_path / "abi_check.c"
+    src.write_text('#include <stdio.h>\n#include "hiscache_hip.h"\n'
+                   'int main(void) { printf("%s|%s|%d\\n", hc_version(), hc_strerror(HC_EWORKSPACE), '
+                   'hc_device_count() >= 0); return 0; }\n')
+    exe = tmp_path / "abi_check"
+    subprocess.run(["gcc", "-std=c11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(root, "include"),
+                    str(src), "-o", str(exe), "-L", lib_dir, "-lhiscache_hip", "-Wl,-rpath," + lib_dir],
+                   check=True, capture_output=True, text=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True, timeout=60).stdout
+    assert out.startswith("hiscache_hip") and out.strip().endswith("|1")
