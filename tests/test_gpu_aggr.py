@@ -437,3 +437,15 @@ def test_weighted_fast_path_prefix_rows_and_dtypes(be, orc, dtype):
     assert (got[:used][hist_edge] == 0).all() and hist_edge.any()
     scale = (np.abs(g[dst]) * np.abs(v32[idx[:used]])).sum(-1)
     assert (np.abs(got[:used] - eg[:used]) <= 1e-5 * scale + 1e-7).all()
+
+
+def test_c_abi_from_a_program_without_python():
+    """history-cache_amd/abi_demo (built with the library): hipMalloc'd buffers, raw pointers, status
+    codes; it checks forward, transposed view and backward of a 4-row block against hand-worked values."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "history-cache_amd", "abi_demo")
+    assert os.path.exists(exe), "abi_demo is built by make -C history-cache_amd/csrc"
+    p = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0 and p.stdout.startswith("abi_demo: ok"), (p.returncode, p.stdout, p.stderr)
