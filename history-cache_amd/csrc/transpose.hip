@@ -29,9 +29,11 @@ namespace {
 // A block covers TR_TILE consecutive slots.  The rows that overlap the tile are found with two
 // binary searches; their offsets are staged in LDS when they fit, and every thread then finds the
 // row of its slot with a short search.  Reads and writes are coalesced whatever the degrees are.
-constexpr int TR_ITEMS = 8;
-constexpr int TR_TILE = HC_BLOCK * TR_ITEMS;
 constexpr int TR_LDS_ROWS = 2048;
+// slots per thread: 8 on large blocks; 1 on small ones (sampled batches), where more, shorter blocks
+// matter more than the amortised tile search
+constexpr int TR_ITEMS_LARGE = 8;
+constexpr int64_t TR_SMALL_EDGES = 1 << 18;
 
 // largest r in [lo, hi] with ptr[r] <= e (ptr[lo] <= e is the caller's business)
 template <typename P>
@@ -44,7 +46,7 @@ __device__ __forceinline__ int64_t tr_row_of(P ptr, int64_t lo, int64_t hi, int6
   return lo;
 }
 
-template <bool VAL_IS_ROW>
+template <bool VAL_IS_ROW, int TR_ITEMS>
 __global__ __launch_bounds__(HC_BLOCK) void tr_expand_edges(const int64_t *__restrict__ ptr,
                                                              const int64_t *__restrict__ idx,
                                                              const int64_t *__restrict__ hmap_row,
@@ -52,6 +54,7 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_expand_edges(const int64_t *__res
                                                              uint32_t *__restrict__ vals,
                                                              uint32_t *__restrict__ rows, int64_t R, int64_t E,
                                                              int64_t n_src) {
+  constexpr int TR_TILE = HC_BLOCK * TR_ITEMS;
   __shared__ int64_t s_ptr[TR_LDS_ROWS];
   __shared__ int64_t s_range[2];
   const int64_t e0 = (int64_t)blockIdx.x * TR_TILE;
@@ -269,10 +272,15 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
   const bool want_edges = edgeT != nullptr;
   const unsigned bits = (unsigned)key_bits(n_src);
   const uint32_t *skeys = nullptr;
-  const int64_t tblocks = (E + TR_TILE - 1) / TR_TILE;
+  const int items = E <= TR_SMALL_EDGES ? 1 : TR_ITEMS_LARGE;
+  const int64_t tile = (int64_t)HC_BLOCK * items;
+  const dim3 tgrid((unsigned)((E + tile - 1) / tile));
   if (want_edges) {
-    tr_expand_edges<false><<<dim3((unsigned)tblocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, rows,
-                                                                              R, E, n_src);
+    if (items == 1)
+      tr_expand_edges<false, 1><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, rows, R, E, n_src);
+    else
+      tr_expand_edges<false, TR_ITEMS_LARGE><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, rows,
+                                                                               R, E, n_src);
     rocprim::double_buffer<uint32_t> dk(keys0, keys1), dv(vals0, vals1);
     if (rocprim::radix_sort_pairs(temp, temp_bytes, dk, dv, (size_t)E, 0u, bits, st, false) != hipSuccess)
       return HC_ELAUNCH;
@@ -281,8 +289,11 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
     skeys = dk.current();
   } else {
     // value = destination row; dropped edge slots keep the fill value and sort behind the sentinel
-    tr_expand_edges<true><<<dim3((unsigned)tblocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, nullptr,
-                                                                             R, E, n_src);
+    if (items == 1)
+      tr_expand_edges<true, 1><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, nullptr, R, E, n_src);
+    else
+      tr_expand_edges<true, TR_ITEMS_LARGE><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, nullptr,
+                                                                              R, E, n_src);
     // rowT doubles as the sort's second value buffer; copy only if the result landed in the first
     uint32_t *rowT_u = reinterpret_cast<uint32_t *>(rowT);
     rocprim::double_buffer<uint32_t> dk(keys0, keys1), dv(vals0, rowT_u);
