@@ -50,7 +50,9 @@ def _p(a):
     if a is None:
         return ctypes.c_void_p(None)
     assert a.flags["C_CONTIGUOUS"], "oracle arrays must be C-contiguous"
-    return ctypes.c_void_p(a.ctypes.data)
+    # data_as keeps a reference to the array, so a converted temporary (``_p(_u8(mask))``) stays
+    # alive until the C call that receives the pointer has returned
+    return a.ctypes.data_as(ctypes.c_void_p)
 
 
 def _i64(a):

@@ -277,6 +277,29 @@ def test_grad_check_more_admitted_than_capacity(orc):
     assert (f2s != -1).sum() == cap
 
 
+def test_grad_check_large_block_with_used_mask(orc):
+    """A block large enough that a converted copy of the used mask would be recycled by the allocator
+    if the wrapper let go of it before the C call: the mask equals the numpy predicate."""
+    rng = np.random.default_rng(13)
+    N, F, cap, M = 40000, 16, 700, 8000
+    table = np.zeros((cap, F), np.float32)
+    f2s, s2f = np.full(N, -1, np.int64), np.full(cap, -1, np.int64)
+    checkin, header = np.full(cap, -1, np.int64), np.array([5], np.int64)
+    for it in range(3):
+        sub_to_full = rng.choice(N, size=M, replace=False).astype(np.int32)     # converted by the wrapper
+        grad = (rng.standard_normal((M, F)) * np.exp(rng.normal(-3, 1.5, size=(M, 1)))).astype(np.float32)
+        emb = rng.standard_normal((M, F)).astype(np.float32)
+        slot = f2s[sub_to_full].astype(np.int32)                               # converted by the wrapper
+        age = rng.integers(0, 21, size=M).astype(np.int32)
+        used = rng.random(M) < 0.9
+        score = orc.row_scores(grad)
+        thres = float(np.sort(score)[M // 3])
+        mask, _, _ = orc.grad_check(grad, emb, slot, age, used, sub_to_full, thres, 10, orc.NORM_L2, orc.CMP_LT,
+                                    table, orc.DT_F32, f2s, s2f, checkin, header, it)
+        expect = used & (score < np.float32(thres)) & ((slot == -1) | (age >= 10))
+        np.testing.assert_array_equal(mask, expect)
+
+
 # ----------------------------------------------------------------------------- thresholds
 def test_quantile_threshold_matches_torch_quantile():
     from oracle import host_model
