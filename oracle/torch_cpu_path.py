@@ -2,8 +2,9 @@
 
 TEST INFRASTRUCTURE ONLY.  The reference has no CPU implementation; this is its semantics
 (/root/reference/src/cpp/src/history_aggr.cu:7-40,127-168; /root/reference/hiscache/history_cache.py:205-221)
-written the way a PyTorch user would on a CPU.  The benchmark times it on the host cores as the
-reported CPU baseline; tests use it as a second, independently written checker of the C oracle.
+written the way a PyTorch user would on a CPU.  Tests use it as a second, independently written
+checker of the C oracle; the benchmark times its admission pass as the CPU baseline of that workload
+(the aggregation step's baseline is the OpenMP statement in ``hc_cpu_mt.c``).
 """
 import torch
 

@@ -276,3 +276,31 @@ def test_chunked_backward_order(orc):
             tot = acc if tot is None else tot + acc
         np.testing.assert_array_equal(got[s], tot)
     np.testing.assert_allclose(got, seq, rtol=1e-5, atol=1e-6)
+
+
+def test_multithreaded_cpu_statement_equals_the_sequential_one(orc):
+    """The OpenMP statement that the benchmark times as its CPU baseline gives the sequential statement's
+    bits: forward with per-source substitution (long rows as quarters), transposed view, backward gather
+    (hub sources in chunks)."""
+    from oracle import hc_cpu_mt as mt
+    assert mt.num_threads() >= 1
+    rng = np.random.default_rng(77)
+    for R, N, F, hub in [(3000, 2000, 64, 1500), (500, 40, 17, None), (1, 1, 8, None), (257, 5000, 256, 300)]:
+        ptr, idx = random_csr(rng, R, N, 12, hub=hub)
+        idx[rng.random(len(idx)) < 0.2] = N // 3                    # one very popular source
+        feat = rng.standard_normal((N, F)).astype(np.float32)
+        hist = rng.standard_normal((50, F)).astype(np.float32)
+        smap = np.where(rng.random(N) < 0.4, rng.integers(0, 50, size=N), -1).astype(np.int64)
+        for m, h in ((smap, hist), (None, None)):
+            np.testing.assert_array_equal(mt.fwd_mean_src(ptr, idx, feat, m, h, split_above=256),
+                                          orc.fwd_mean_src(ptr, idx, feat, m, h, split_above=256))
+        ptrT, rowT = mt.build_transpose(ptr, idx, N)
+        wp, wr, _ = orc.build_transpose(ptr, idx, None, N)
+        np.testing.assert_array_equal(ptrT, wp)
+        np.testing.assert_array_equal(rowT[: len(wr)], wr)
+        g = rng.standard_normal((R, F)).astype(np.float32)
+        for chunk in (0, 512):
+            np.testing.assert_array_equal(mt.bwd_mean(ptr, ptrT, rowT, g, N, chunk=chunk),
+                                          orc.bwd_mean_src(ptr, idx, g, N, chunk=chunk))
+    with pytest.raises(ValueError):
+        mt.build_transpose(np.array([0, 1]), np.array([5]), 3)
