@@ -156,3 +156,150 @@ int mt_bwd_mean(const Index *ptr, const Index *ptrT, const int32_t *rowT, const 
   }
   return bad ? ORC_EINVAL : ORC_OK;
 }
+
+/* ---------------------------------------------------------------------------------------------- */
+/* Fused admission (orc_grad_check's rule) for all host cores: scores and predicate per row in
+ * parallel, ring slots in row order from a two-level prefix sum of the mask, then previous owners
+ * un-mapped, then the new owners written and the rows copied (fp32 -> fp16, round to nearest even).
+ * Un-mapping before mapping gives the sequential result as long as no slot is handed out twice in
+ * one call; a call that admits more rows than the table holds is refused (ORC_EINVAL) and left to
+ * the sequential statement.  Scores use the 64-lane order of orc_row_score.                         */
+/* ---------------------------------------------------------------------------------------------- */
+#include <math.h>
+
+static uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+
+static uint16_t f32_to_f16(float f) {
+  const uint32_t x = f2u(f), sign = (x >> 16) & 0x8000u, mag = x & 0x7fffffffu;
+  if (mag >= 0x7f800000u) return (uint16_t)(sign | 0x7c00u | (mag > 0x7f800000u ? 0x200u | ((mag >> 13) & 0x3ffu) : 0));
+  if (mag >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);          /* rounds to infinity */
+  if (mag < 0x33000001u) return (uint16_t)sign;                        /* rounds to zero */
+  int32_t e = (int32_t)(mag >> 23) - 127;
+  uint32_t m = (mag & 0x7fffffu) | 0x800000u;
+  int shift = e < -14 ? 13 + (-14 - e) : 13;
+  uint32_t half = m >> shift, rem = m & ((1u << shift) - 1), mid = 1u << (shift - 1);
+  if (rem > mid || (rem == mid && (half & 1))) half++;
+  if (e < -14) return (uint16_t)(sign | half);                         /* subnormal (may carry into normal) */
+  return (uint16_t)(sign | ((uint32_t)((e + 15) << 10) + (half - 0x400u)));
+}
+
+uint16_t mt_f32_to_f16(float f) { return f32_to_f16(f); }
+
+/* acc[l] folds the elements of lane l in increasing index (fma), the 64 partials meet in a butterfly with
+ * partner distance 32 ... 1: orc_row_score's order, laid out so that a 256-element block is one pass. */
+static inline __attribute__((always_inline)) float row_score_l2(const float *row, Index F) {
+  float acc[64];
+  for (int l = 0; l < 64; ++l) acc[l] = 0.0f;
+  Index e = 0;
+  for (; e + 256 <= F; e += 256) {
+    for (int l = 0; l < 64; ++l) {
+      const float *x = row + e + 4 * l;
+      float a = acc[l];
+      a = fmaf(x[0], x[0], a);
+      a = fmaf(x[1], x[1], a);
+      a = fmaf(x[2], x[2], a);
+      a = fmaf(x[3], x[3], a);
+      acc[l] = a;
+    }
+  }
+  for (; e < F; ++e) {
+    const int l = (int)((e / 4) % 64);
+    acc[l] = fmaf(row[e], row[e], acc[l]);
+  }
+  for (int d = 32; d >= 1; d >>= 1) {
+    float nxt[64];
+    for (int l = 0; l < 64; ++l) nxt[l] = acc[l] + acc[l ^ d];
+    memcpy(acc, nxt, sizeof(acc));
+  }
+  return sqrtf(acc[0]);
+}
+
+/* Two builds of the two hot loops: plain C for any x86-64, and one for cores with FMA and F16C (a fused
+ * multiply-add instruction instead of the library call, eight conversions per instruction; both round
+ * exactly like the portable code).  Chosen once per call from the CPU's feature bits. */
+#include <immintrin.h>
+
+static void score_rows_any(const float *grad, Index lo, Index hi, Index F, float *score) {
+  for (Index r = lo; r < hi; ++r) score[r] = row_score_l2(grad + r * F, F);
+}
+__attribute__((target("avx2,fma"))) static void score_rows_fma(const float *grad, Index lo, Index hi, Index F,
+                                                               float *score) {
+  for (Index r = lo; r < hi; ++r) score[r] = row_score_l2(grad + r * F, F);
+}
+static void convert_row_any(const float *src, uint16_t *d, Index F) {
+  for (Index c = 0; c < F; ++c) d[c] = f32_to_f16(src[c]);
+}
+__attribute__((target("avx2,f16c"))) static void convert_row_f16c(const float *src, uint16_t *d, Index F) {
+  Index c = 0;
+  for (; c + 8 <= F; c += 8)
+    _mm_storeu_si128((__m128i *)(d + c),
+                     _mm256_cvtps_ph(_mm256_loadu_ps(src + c), _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC));
+  for (; c < F; ++c) d[c] = f32_to_f16(src[c]);
+}
+void mt_convert_row(const float *src, uint16_t *d, Index F, int hw) {
+  if (hw && __builtin_cpu_supports("f16c") && __builtin_cpu_supports("avx2")) convert_row_f16c(src, d, F);
+  else convert_row_any(src, d, F);
+}
+void mt_score_rows(const float *grad, Index M, Index F, float *score, int hw) {
+  if (hw && __builtin_cpu_supports("fma") && __builtin_cpu_supports("avx2")) score_rows_fma(grad, 0, M, F, score);
+  else score_rows_any(grad, 0, M, F, score);
+}
+
+int mt_grad_check_f16(const float *grad, const float *emb, const Index *slot, const int32_t *age,
+                      const Index *sub_to_full, float thres, int32_t age_limit, uint8_t *mask_out,
+                      float *score_out, uint16_t *table, Index capacity, Index *full2slot, Index *slot2full,
+                      Index *checkin, Index *header, Index glb_iter, Index M, Index F, Index *rank /* [M] scratch */) {
+  const int T = omp_get_max_threads();
+  Index *part = (Index *)calloc((size_t)T + 1, sizeof(Index));
+  if (!part) return ORC_EINVAL;
+  int bad = 0;
+  const Index h0 = *header;
+  const int hw_fma = __builtin_cpu_supports("fma") && __builtin_cpu_supports("avx2");
+  const int hw_f16c = __builtin_cpu_supports("f16c") && __builtin_cpu_supports("avx2");
+#pragma omp parallel num_threads(T)
+  {
+    const int t = omp_get_thread_num();
+    const Index lo = M * t / T, hi = M * (t + 1) / T;
+    Index n = 0;
+    if (hw_fma) score_rows_fma(grad, lo, hi, F, score_out);
+    else score_rows_any(grad, lo, hi, F, score_out);
+    for (Index r = lo; r < hi; ++r) {
+      const float sc = score_out[r];
+      const int admit = (sc < thres) && (slot[r] == -1 || (age && age[r] >= age_limit));
+      mask_out[r] = (uint8_t)admit;
+      rank[r] = n;
+      n += admit;
+    }
+    part[t + 1] = n;
+#pragma omp barrier
+#pragma omp single
+    {
+      for (int k = 0; k < T; ++k) part[k + 1] += part[k];
+      if (part[T] > capacity) bad = 1;
+      else *header = (h0 + part[T]) % capacity;
+    }
+    if (!bad) {
+      for (Index r = lo; r < hi; ++r) {                 /* un-map the previous owners of the slots taken */
+        if (!mask_out[r]) continue;
+        const Index s = (h0 + part[t] + rank[r]) % capacity;
+        rank[r] = s;
+        const Index old = slot2full[s];
+        /* two slots can name the same previous owner (a stale entry); at most one of them matches */
+        if (old != -1 && __atomic_load_n(&full2slot[old], __ATOMIC_RELAXED) == s)
+          __atomic_store_n(&full2slot[old], (Index)-1, __ATOMIC_RELAXED);
+      }
+#pragma omp barrier
+      for (Index r = lo; r < hi; ++r) {
+        if (!mask_out[r]) continue;
+        const Index s = rank[r];
+        full2slot[sub_to_full[r]] = s;
+        slot2full[s] = sub_to_full[r];
+        if (checkin) checkin[s] = glb_iter;
+        if (hw_f16c) convert_row_f16c(emb + r * F, table + s * F, F);
+        else convert_row_any(emb + r * F, table + s * F, F);
+      }
+    }
+  }
+  free(part);
+  return bad ? ORC_EINVAL : ORC_OK;
+}

@@ -85,3 +85,49 @@ def bwd_mean(ptr, ptrT, rowT, g, n_src, chunk=0, out=None):
     if rc != 0:
         raise RuntimeError("mt_bwd_mean failed")
     return out
+
+
+def f32_to_f16_bits(x):
+    f = lib().mt_f32_to_f16
+    f.restype = ctypes.c_uint16
+    return np.array([f(ctypes.c_float(float(v))) for v in np.asarray(x, np.float32).ravel()], np.uint16)
+
+
+def grad_check_f16(grad, emb, slot, age, sub_to_full, thres, age_limit, table, full2slot, slot2full, checkin,
+                   header, glb_iter):
+    """Fused admission into an fp16 table (uint16 bits), L2 scores, strict ``<``; maps, header and table are
+    updated in place.  Returns (mask[bool], score[f32]).  Raises when more rows are admitted than the table
+    holds (the sequential statement covers that case)."""
+    grad, emb = _arr(grad, np.float32), _arr(emb, np.float32)
+    M, F = emb.shape
+    slot, sub_to_full = _arr(slot, np.int64), _arr(sub_to_full, np.int64)
+    age = None if age is None else _arr(age, np.int32)
+    assert table.dtype == np.uint16 and table.flags["C_CONTIGUOUS"] and table.shape[1] == F
+    for a in (full2slot, slot2full, header):
+        assert a.dtype == np.int64 and a.flags["C_CONTIGUOUS"]
+    mask = np.zeros(M, np.uint8)
+    score = np.zeros(M, np.float32)
+    rank = np.zeros(M, np.int64)
+    rc = lib().mt_grad_check_f16(_p(grad), _p(emb), _p(slot), _p(age), _p(sub_to_full), ctypes.c_float(float(thres)),
+                                 ctypes.c_int32(int(age_limit)), _p(mask), _p(score), _p(table), _I(table.shape[0]),
+                                 _p(full2slot), _p(slot2full), _p(checkin), _p(header), _I(glb_iter), _I(M), _I(F),
+                                 _p(rank))
+    if rc != 0:
+        raise ValueError("mt_grad_check_f16: more admitted rows than table slots")
+    return mask.astype(bool), score
+
+
+def score_rows(grad, hw=True):
+    """L2 row scores; ``hw`` selects the build that uses the FMA instruction when the CPU has it."""
+    grad = _arr(grad, np.float32)
+    out = np.zeros(grad.shape[0], np.float32)
+    lib().mt_score_rows(_p(grad), _I(grad.shape[0]), _I(grad.shape[1]), _p(out), ctypes.c_int(int(hw)))
+    return out
+
+
+def convert_row(x, hw=True):
+    """fp32 -> fp16 bits of one row; ``hw`` selects the F16C build when the CPU has it."""
+    x = _arr(x, np.float32).ravel()
+    out = np.zeros(x.size, np.uint16)
+    lib().mt_convert_row(_p(x), _p(out), _I(x.size), ctypes.c_int(int(hw)))
+    return out

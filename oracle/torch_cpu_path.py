@@ -3,8 +3,8 @@
 TEST INFRASTRUCTURE ONLY.  The reference has no CPU implementation; this is its semantics
 (/root/reference/src/cpp/src/history_aggr.cu:7-40,127-168; /root/reference/hiscache/history_cache.py:205-221)
 written the way a PyTorch user would on a CPU.  Tests use it as a second, independently written
-checker of the C oracle; the benchmark times its admission pass as the CPU baseline of that workload
-(the aggregation step's baseline is the OpenMP statement in ``hc_cpu_mt.c``).
+checker of the C oracle.  (The benchmark's CPU baselines are the OpenMP statements in ``hc_cpu_mt.c``,
+which run several times faster than this spelling.)
 """
 import torch
 

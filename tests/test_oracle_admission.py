@@ -300,6 +300,52 @@ def test_grad_check_large_block_with_used_mask(orc):
         np.testing.assert_array_equal(mask, expect)
 
 
+def test_multithreaded_admission_equals_the_sequential_one(orc):
+    """The OpenMP admission that the benchmark times as its CPU baseline: scores, mask, maps, header and
+    fp16 table bit for bit equal to the sequential statement, across a ring wrap and with stale rows
+    re-admitted; its fp32 -> fp16 rounding equals NumPy's."""
+    from oracle import hc_cpu_mt as mt
+    rng = np.random.default_rng(14)
+    v = np.concatenate([rng.standard_normal(3000).astype(np.float32) * np.float32(10) ** rng.integers(-9, 5, size=3000).astype(np.float32),
+                        np.array([0, -0.0, 65504, 65519.99, 65520, np.inf, -np.inf, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0001,
+                                  2.0 ** -14, 2.0 ** -14 * 0.9999, 5.96e-8, 3e-8], np.float32)])
+    with np.errstate(over="ignore"):
+        np.testing.assert_array_equal(mt.f32_to_f16_bits(v), v.astype(np.float16).view(np.uint16))
+        for hw in (False, True):                       # portable build and the FMA / F16C build
+            np.testing.assert_array_equal(mt.convert_row(v, hw), v.astype(np.float16).view(np.uint16))
+    for width in (1, 5, 64, 255, 256, 300, 768):
+        g = (rng.standard_normal((50, width)) * np.exp(rng.normal(-3, 1.5, size=(50, 1)))).astype(np.float32)
+        for hw in (False, True):
+            np.testing.assert_array_equal(mt.score_rows(g, hw), orc.row_scores(g))
+    N, F, cap, M = 40000, 64, 9000, 8000
+    ref = dict(table=np.zeros((cap, F), np.uint16), f2s=np.full(N, -1, np.int64), s2f=np.full(cap, -1, np.int64),
+               checkin=np.full(cap, -1, np.int64), header=np.array([cap - 100], np.int64))
+    got = {k: a.copy() for k, a in ref.items()}
+    readmitted = 0
+    for it in range(5):
+        nodes = rng.choice(N, size=M, replace=False).astype(np.int64)
+        grad = (rng.standard_normal((M, F)) * np.exp(rng.normal(-3, 1.5, size=(M, 1)))).astype(np.float32)
+        emb = rng.standard_normal((M, F)).astype(np.float32)
+        slot = ref["f2s"][nodes].copy()
+        age = rng.integers(0, 21, size=M).astype(np.int32)
+        thres = float(np.sort(orc.row_scores(grad))[M // 4])
+        rmask, rscore, _ = orc.grad_check(grad, emb, slot, age, None, nodes, thres, 10, orc.NORM_L2, orc.CMP_LT,
+                                          ref["table"], orc.DT_F16, ref["f2s"], ref["s2f"], ref["checkin"],
+                                          ref["header"], it)
+        mask, score = mt.grad_check_f16(grad, emb, slot, age, nodes, thres, 10, got["table"], got["f2s"], got["s2f"],
+                                        got["checkin"], got["header"], it)
+        np.testing.assert_array_equal(mask, rmask)
+        np.testing.assert_array_equal(score, rscore)
+        for k in ref:
+            np.testing.assert_array_equal(got[k], ref[k], err_msg=k)
+        readmitted += int(((slot != -1) & rmask).sum())
+    assert readmitted > 100 and ref["header"][0] < cap - 100          # stale rows came back, the ring wrapped
+    small = np.zeros((10, F), np.uint16)
+    with pytest.raises(ValueError):                                    # more admitted rows than slots
+        mt.grad_check_f16(grad, emb, np.full(M, -1), None, nodes, 1e9, 10, small, got["f2s"], np.full(10, -1, np.int64),
+                          None, np.zeros(1, np.int64), 9)
+
+
 # ----------------------------------------------------------------------------- thresholds
 def test_quantile_threshold_matches_torch_quantile():
     from oracle import host_model
