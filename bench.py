@@ -276,7 +276,34 @@ def cpu_baseline_c2(shape):
     return {"value": E / med, "unit": "edges/s", "cores": mt.num_threads(), "kind": "port",
             "sample": "1/10-size c2 block (R=%d, E=%d, %d sources x %d fp32), fwd + transposed view + bwd in C with "
                       "OpenMP over rows and sources (same sums, same order), median of %d runs"
-                      % (R, E, N, F, len(times))}
+                      % (R, E, N, F, len(times)),
+            "torch_index_add": torch_spelling_c2(ptr, idx, feat, hist, hmap, g, R, E, N)}
+
+
+def torch_spelling_c2(ptr, idx, feat, hist, hmap, g, R, E, N):
+    """The same sample through stock PyTorch CPU operators (index_add), the way a PyTorch user would spell
+    the step on a CPU: edges/s, median of up to 3 runs."""
+    import torch
+
+    from oracle import torch_cpu_path as tp
+
+    torch.set_num_threads(os.cpu_count())
+    t = [torch.from_numpy(a) for a in (ptr, idx, feat, hist, hmap, g)]
+    ptr, idx, feat, hist, hmap, g = t
+
+    def one():
+        tp.aggr_fwd_src(feat, hist, hmap, ptr, idx, R)
+        tp.aggr_bwd_row(g, ptr, idx, None, N, R)
+
+    one()
+    times = []
+    t_end = time.perf_counter() + 8.0
+    while len(times) < 3 and (not times or time.perf_counter() < t_end):
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return {"value": E / times[len(times) // 2], "unit": "edges/s", "threads": torch.get_num_threads()}
 
 
 def cpu_baseline_c4(M, F):
