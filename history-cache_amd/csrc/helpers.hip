@@ -139,8 +139,8 @@ __global__ __launch_bounds__(HC_BLOCK) void gather_rows_kernel(const TS *__restr
                                                                 int64_t n, int64_t F) {
   constexpr int V = 4;
   const int lane = hc_lane();
-  const int64_t i = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
-  if (i >= n) return;
+  const int64_t stride = (int64_t)gridDim.x * HC_WAVES_PER_BLOCK;
+  for (int64_t i = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block(); i < n; i += stride) {
   TD *__restrict__ o = dst + i * F;
   bool take = mask == nullptr || mask[i] != 0;
   int64_t id = 0;
@@ -175,6 +175,7 @@ __global__ __launch_bounds__(HC_BLOCK) void gather_rows_kernel(const TS *__restr
       if (accumulate) v = hc_to_f32<TD>(o[c]) + v;
       o[c] = hc_from_f32<TD>(v);
     }
+  }
   }
 }
 
@@ -354,8 +355,21 @@ extern "C" int hc_gather_rows(const void *src, int src_dtype, int64_t n_rows, co
   if (n == 0) return HC_OK;
   HC_REQUIRE(ids && dst && (src || n_rows == 0));
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const int64_t b = (n + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  int64_t b = (n + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
   if (!hc_grid_ok(b)) return HC_EUNSUPPORTED;
+  // A table in host memory is read over the host link: a few hundred waves keep the link busy, and a
+  // launch of one wave per row would park tens of thousands of waiting waves on the compute units,
+  // in the way of whatever runs beside it on other streams.
+  // (256 blocks = 1 024 waves read 56 - 57 GB/s, the same as 22 000 blocks).
+  constexpr int64_t HOST_GATHER_BLOCKS = 256;
+  if (b > HOST_GATHER_BLOCKS) {
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, src) == hipSuccess) {
+      if (attr.type == hipMemoryTypeHost) b = HOST_GATHER_BLOCKS;
+    } else {
+      (void)hipGetLastError();   // an address the runtime does not know: treat it as device memory
+    }
+  }
   dim3 g((unsigned)b), bl(HC_BLOCK);
   if (src_dtype == HC_F32) return launch_gather<float>(src, n_rows, ids, mask, dst, dst_dtype, accumulate, n, F, g, bl, st);
   if (src_dtype == HC_F16) return launch_gather<__half>(src, n_rows, ids, mask, dst, dst_dtype, accumulate, n, F, g, bl, st);

@@ -30,6 +30,7 @@ class PinnedFeatureStore:
         self.device = torch.device(device)
         self._side = None
         self._done = None
+        self._prefetch_side = None
 
     def _side_stream(self):
         if self._side is None:
@@ -54,7 +55,40 @@ class PinnedFeatureStore:
             out = _be.gather_rows(self.buffer, ids, mask=mask, out_dtype=self.out_dtype)
             self._done.record(side)
         out.record_stream(cur)
+        ids.record_stream(side)          # the caller may drop its last reference before the read is done
+        mask.record_stream(side)
         return out, self._done
 
     def join(self, event):
         torch.cuda.current_stream(self.device).wait_event(event)
+
+    def prefetch(self, ids):
+        """Start reading the rows of ALL ``ids`` on a side stream (default priority) now, so that the
+        host-link read overlaps whatever the caller queues next -- typically the previous batch's
+        forward and backward.  No mask: which rows the cache makes unnecessary is not known before that
+        batch's update.  Returns a handle for ``take``."""
+        cur = torch.cuda.current_stream(self.device)
+        if self._prefetch_side is None:
+            self._prefetch_side = torch.cuda.Stream(device=self.device)
+        side = self._prefetch_side
+        side.wait_stream(cur)                      # the ids are produced on the current stream
+        with torch.cuda.stream(side):
+            rows = _be.gather_rows(self.buffer, ids, out_dtype=self.out_dtype)
+            done = torch.cuda.Event()
+            done.record(side)
+        ids.record_stream(side)
+        return PrefetchedRows(ids, rows, done)
+
+    def take(self, handle):
+        """The rows of a ``prefetch``; the current stream waits for the read to finish."""
+        cur = torch.cuda.current_stream(self.device)
+        cur.wait_event(handle.done)
+        handle.rows.record_stream(cur)
+        return handle.rows
+
+
+class PrefetchedRows:
+    __slots__ = ("ids", "rows", "done")
+
+    def __init__(self, ids, rows, done):
+        self.ids, self.rows, self.done = ids, rows, done

@@ -218,23 +218,45 @@ class HistoryCache:
         hit_feat_mask = self.sub2feat != -1
         load_mask = torch.logical_and(self.used_masks[0], ~hit_feat_mask)
         self.glb_iter += 1
-        # host-link read on a side stream, overlapped with the two HBM gathers below
-        async_get = getattr(self.uvm, "masked_get_async", None)
-        if async_get is not None:
-            x, done = async_get(sub_to_full, load_mask)
-        else:
-            x, done = self.uvm.masked_get(sub_to_full, load_mask), None
+        pre = self._take_prefetched(batch)
+        if pre is not None:
+            # every row was read ahead of time: keep what masked_get + the feature-cache merge would have
+            # produced (needed rows and feature-cache hits), zero the rest
+            self.cached_embedding = _be.gather_rows(self.buffer.view(-1, self.hidden_channels),
+                                                    self.sub2embed)
+            keep = torch.logical_or(self.used_masks[0], hit_feat_mask)
+            pre.masked_fill_(~keep[:, None], 0)
+            batch.x = pre
+            self.load_mask = load_mask
+            return None
+        # Host-link read of the needed rows.  (Reading it on a side stream here would only overlap
+        # the small gather below and costs the host more than that saves; ``prefetch`` is the way to
+        # overlap the read with compute.)
+        x = self.uvm.masked_get(sub_to_full, load_mask)
         # slot -1 reads the last row of the view, as the reference's indexing does; such rows
         # are ignored by the aggregation
         self.cached_embedding = _be.gather_rows(self.buffer.view(-1, self.hidden_channels),
                                                 self.sub2embed)
-        if done is not None:
-            self.uvm.join(done)
         _be.gather_rows(self.buffer.view(-1, self.in_channels), self.sub2feat, mask=hit_feat_mask,
                         out=x, accumulate=True)
         batch.x = x
         self.load_mask = load_mask
         return None
+
+    def prefetch(self, batch):
+        """Start the host-link read of ``batch``'s feature rows now (all of them), to overlap it with the
+        work queued before that batch's ``lookup_and_load``, which then only masks the rows.  Optional:
+        without it ``lookup_and_load`` reads the needed rows itself.  ``batch.x`` comes out the same."""
+        start = getattr(self.uvm, "prefetch", None)
+        if start is not None and "history" in self.feat_mode:
+            batch.prefetched_x = start(batch.sub_to_full)
+
+    def _take_prefetched(self, batch):
+        handle = getattr(batch, "prefetched_x", None)
+        if handle is None or handle.ids is not batch.sub_to_full:
+            return None
+        batch.prefetched_x = None
+        return self.uvm.take(handle)
 
     def stats(self):
         """Cache occupancy (synchronises)."""

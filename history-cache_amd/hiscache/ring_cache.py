@@ -61,17 +61,27 @@ class RingHistoryCache:
         self.used_masks = _be.count_history_reconstruct(batch.ptr, batch.idx, self.sub2embed,
                                                         sub_to_full.shape[0], batch.y.shape[0], num_layer)
         self.glb_iter += 1
-        async_get = getattr(self.uvm, "masked_get_async", None)
-        if async_get is not None:
-            x, done = async_get(sub_to_full, self.used_masks[0])
-        else:
-            x, done = self.uvm.masked_get(sub_to_full, self.used_masks[0]), None
+        handle = getattr(batch, "prefetched_x", None)
+        if handle is not None and handle.ids is sub_to_full:
+            # every row was read ahead of time (``prefetch``): zero the rows the cache makes unnecessary
+            batch.prefetched_x = None
+            x = self.uvm.take(handle)
+            x.masked_fill_(~self.used_masks[0][:, None], 0)
+            self.cached_embedding = _be.gather_rows(self.table, self.sub2embed)
+            batch.x = x
+            return None
+        x = self.uvm.masked_get(sub_to_full, self.used_masks[0])
         # rows without a slot (-1) read the last table row and are ignored by the aggregation
         self.cached_embedding = _be.gather_rows(self.table, self.sub2embed)
-        if done is not None:
-            self.uvm.join(done)
         batch.x = x
         return None
+
+    def prefetch(self, batch):
+        """Start the host-link read of ``batch``'s feature rows now (all of them), to overlap it with the
+        work queued before that batch's ``lookup_and_load``, which then only masks the rows."""
+        start = getattr(self.uvm, "prefetch", None)
+        if start is not None:
+            batch.prefetched_x = start(batch.sub_to_full)
 
     @torch.no_grad()
     def update_history(self, batch, glb_iter):

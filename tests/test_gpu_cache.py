@@ -94,6 +94,81 @@ def test_lookup_update_cycles_match_model():
     assert s["feat_cached"] == int((st.full2embed[N:2 * N] != -1).sum())
 
 
+def test_prefetched_features_give_the_same_batch():
+    """``prefetch`` issued one batch ahead (before the previous batch's update changes the cache) leaves
+    ``batch.x``, the slots, the masks and the cache state exactly as the unpipelined path does, for the
+    buffer cache and the ring cache."""
+    from oracle import hc_oracle as orc
+    from oracle import host_model
+    from hiscache import PinnedFeatureStore, RingHistoryCache
+    rng, feats, cfg, cache, st = make_world(5)
+    N, H = st.N, st.H
+    pairs = [batch_pair(rng, N, 40, [6, 4, 3]) for _ in range(6)]
+    cache.prefetch(pairs[0][0])
+    for it, (gpu, cpu) in enumerate(pairs, start=1):
+        assert gpu.prefetched_x is not None
+        cache.lookup_and_load(gpu, 3)
+        assert gpu.prefetched_x is None                      # consumed
+        if it < len(pairs):
+            cache.prefetch(pairs[it][0])                     # next batch, before this batch's update
+        ref = host_model.lookup_and_load(st, cpu, 3, feats)
+        np.testing.assert_array_equal(gpu.x.cpu().numpy(), ref.x.numpy())
+        np.testing.assert_array_equal(cache.sub2embed.cpu().numpy(), ref.sub2embed.numpy())
+        np.testing.assert_array_equal(cache.load_mask.cpu().numpy(), ref.load_mask.numpy())
+        np.testing.assert_array_equal(cache.cached_embedding.cpu().numpy(), ref.cached_embedding.numpy())
+        n1 = int(cpu.num_node_in_layer[1])
+        emb = rng.standard_normal((n1, H)).astype(np.float32)
+        grad = (rng.standard_normal((n1, H)) * np.exp(rng.normal(-3, 1.5, size=(n1, 1)))).astype(np.float32)
+        pe = torch.from_numpy(emb).to(DEV).requires_grad_(True)
+        pe.grad = torch.from_numpy(grad).to(DEV)
+        cache.produced_embedding = pe
+        cache.update_history(gpu, it)
+        host_model.update_history(st, cpu.sub_to_full, ref.sub2embed, torch.from_numpy(emb),
+                                  torch.from_numpy(orc.row_scores(grad)), 0.6, 4, it)
+        assert_state_equal(cache, st)
+    # a handle made for other ids is ignored
+    gpu, cpu = batch_pair(rng, N, 30, [5, 3, 2])
+    cache.prefetch(gpu)
+    gpu.sub_to_full = gpu.sub_to_full.clone()
+    cache.lookup_and_load(gpu, 3)
+    np.testing.assert_array_equal(gpu.x.cpu().numpy(), host_model.lookup_and_load(st, cpu, 3, feats).x.numpy())
+
+    # the store's side-stream read of a masked subset equals the plain one
+    store = cache.uvm
+    m = torch.from_numpy(rng.random(gpu.sub_to_full.numel()) < 0.5).to(DEV)
+    rows, done = store.masked_get_async(gpu.sub_to_full, m)
+    store.join(done)
+    np.testing.assert_array_equal(rows.cpu().numpy(), store.masked_get(gpu.sub_to_full, m).cpu().numpy())
+
+    # ring cache: two caches in the same state, one pipelined
+    from hiscache.synthetic import make_batch
+    ring = [RingHistoryCache(PinnedFeatureStore(feats, device=DEV), N, st.Fin, 64, capacity=500, num_layers=3,
+                             table_dtype=torch.float16, thres=0.05, age_limit=3, device=DEV) for _ in range(2)]
+    bs = [layered_batch(rng, N, 40, [6, 4, 3]) for _ in range(5)]
+    mk = lambda b: make_batch(b, np.zeros(N, np.int64), DEV)
+    nxt = mk(bs[0])
+    ring[1].prefetch(nxt)
+    for it, b in enumerate(bs, start=1):
+        plain, piped = mk(b), nxt
+        ring[0].lookup_and_load(plain, 3)
+        ring[1].lookup_and_load(piped, 3)
+        if it < len(bs):
+            nxt = mk(bs[it])
+            ring[1].prefetch(nxt)
+        np.testing.assert_array_equal(piped.x.cpu().numpy(), plain.x.cpu().numpy())
+        np.testing.assert_array_equal(ring[1].cached_embedding.cpu().numpy(), ring[0].cached_embedding.cpu().numpy())
+        n1 = int(b["num_node_in_layer"][1])
+        emb = torch.from_numpy(rng.standard_normal((n1, 64)).astype(np.float32)).to(DEV)
+        grad = torch.from_numpy((rng.standard_normal((n1, 64)) * np.exp(rng.normal(-3, 1.5, size=(n1, 1)))).astype(np.float32)).to(DEV)
+        for c, bb in zip(ring, (plain, piped)):
+            pe = emb.clone().requires_grad_(True)
+            pe.grad = grad.clone()
+            c.produced_embedding = pe
+            c.update_history(bb, it)
+        np.testing.assert_array_equal(ring[1].full2slot.cpu().numpy(), ring[0].full2slot.cpu().numpy())
+    assert ring[0].header > 0
+
+
 def test_update_history_overflow_is_counted():
     from oracle import hc_oracle as orc
     from oracle import host_model
