@@ -32,6 +32,7 @@ namespace {
 constexpr int TR_LDS_ROWS = 2048;
 // slots per thread: 8 on large blocks; 1 on small ones (sampled batches), where more, shorter blocks
 // matter more than the amortised tile search
+constexpr int64_t TR_SORT_MEMSET_EDGES = 1 << 20;  // rocPRIM sorts up to this many pairs by merging (kernels only)
 constexpr int TR_ITEMS_LARGE = 8;
 constexpr int64_t TR_SMALL_EDGES = 1 << 18;
 
@@ -251,6 +252,16 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
     return hc_launch_status();
   }
   HC_REQUIRE(ptr && idx && rowT);
+  if (E > TR_SORT_MEMSET_EDGES) {
+    // Above this size the sort library takes its one-sweep path, which clears its counters with
+    // hipMemsetAsync; a captured graph would replay those as memset nodes.  Refuse instead.
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess) {
+      (void)hipGetLastError();
+    } else if (cs != hipStreamCaptureStatusNone) {
+      return HC_EUNSUPPORTED;
+    }
+  }
   Layout L;
   if (!make_layout(E, n_src, &L)) return HC_ELAUNCH;
   if (!workspace || workspace_bytes < L.total) return HC_EWORKSPACE;

@@ -107,10 +107,10 @@ int64_t hc_aggr_fwd_long_row_edges(int64_t F, int in_dtype);
  * transposed edge, ascending inside a source), edgeT[E] (original edge slot);
  * only the first ptrT[n_src] entries of rowT/edgeT are meaningful.
  * Requires R, E, n_src < 2^31 - 1.
- * Stream capture: with E above 2^20 the sort library underneath clears its
- * counters with hipMemsetAsync, which then becomes part of a captured graph;
- * keep such a call outside the capture if memset nodes are unwelcome.  Below
- * that size the call records kernels only. */
+ * Stream capture: up to 2^20 edge slots the call records kernels only.  Above,
+ * the sort library underneath clears its counters with hipMemsetAsync, which a
+ * captured graph would replay as memset nodes: on a capturing stream such a
+ * call returns HC_EUNSUPPORTED and records nothing. */
 size_t hc_transpose_workspace_bytes(int64_t R, int64_t E, int64_t n_src);
 int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row, int64_t R,
                        int64_t E, int64_t n_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT,

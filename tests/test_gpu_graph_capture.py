@@ -77,3 +77,28 @@ def test_aggregation_and_admission_replay_like_eager(be):
         for k in st_eager:
             assert torch.equal(st_graph[k], st_eager[k]), (rep, k)
         assert 0 < int(st_eager["header"]) < R
+
+
+def test_large_transposed_build_is_refused_on_a_capturing_stream(be):
+    """Above 2^20 edge slots the sort library would record memset nodes: the call returns an error on a
+    capturing stream, records nothing, and works again once the capture is over."""
+    R, N, deg = 300_000, 50_000, 4
+    E = R * deg
+    assert E > 1 << 20
+    gen = torch.Generator(device=DEV).manual_seed(7)
+    ptr = torch.arange(R + 1, device=DEV, dtype=torch.int64) * deg
+    idx = torch.randint(0, N, (E,), device=DEV, generator=gen)
+    eager = be.build_transpose(ptr, idx, None, R, N, want_edges=False)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(ValueError):
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                kept = idx + 1                          # the capture is not empty
+                be.build_transpose(ptr, idx, None, R, N, want_edges=False)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    again = be.build_transpose(ptr, idx, None, R, N, want_edges=False)
+    assert torch.equal(again[0], eager[0]) and torch.equal(again[1][:E], eager[1][:E])
