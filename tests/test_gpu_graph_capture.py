@@ -32,6 +32,8 @@ def test_aggregation_and_admission_replay_like_eager(be):
     slot = torch.full((R,), -1, dtype=torch.int64, device=DEV)
     sub_to_full = T(rng.permutation(3 * R)[:R].astype(np.int64))
     thres = torch.tensor([11.3], device=DEV)          # about the median norm of a 128-dim N(0,1) row
+    gather_ids = T(rng.integers(0, N, size=2000).astype(np.int64))
+    N_all = max(R, N)
 
     def fresh_state():
         return dict(table=torch.zeros(cap, F, dtype=torch.float16, device=DEV),
@@ -45,7 +47,10 @@ def test_aggregation_and_admission_replay_like_eager(be):
         gx, gh, _ = be._aggr_bwd(ptr_d, idx_d, tr, g, hmap_d, None, x, False, (R, F), F, R, N)
         mask, score = be.grad_check(g, emb, slot, sub_to_full, thres, st["table"], st["full2slot"], st["slot2full"],
                                     st["header"], 3)
-        return out, tr[0], tr[1], gx, gh, mask, score
+        rows = be.gather_rows(x, gather_ids)             # more rows than the capped grid of a host-memory table
+        found = be.lookup(st["full2slot"], sub_to_full, 0)
+        used = torch.stack(be.count_history_reconstruct(ptr_d, idx_d, hmap_d[:R], N_all, 64, 2))
+        return out, tr[0], tr[1], gx, gh, mask, score, rows, found, used
 
     def load_inputs(seed):
         gen = torch.Generator(device=DEV).manual_seed(seed)
@@ -72,7 +77,8 @@ def test_aggregation_and_admission_replay_like_eager(be):
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        for name, a, b in zip(("out", "ptrT", "rowT", "grad_x", "grad_h", "mask", "score"), captured, eager):
+        for name, a, b in zip(("out", "ptrT", "rowT", "grad_x", "grad_h", "mask", "score", "rows", "found", "used"),
+                              captured, eager):
             assert torch.equal(a, b), (rep, name)
         for k in st_eager:
             assert torch.equal(st_graph[k], st_eager[k]), (rep, k)
