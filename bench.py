@@ -37,6 +37,7 @@ def parse():
     ap.add_argument("--prefetch", action="store_true",
                     help="c3/c5: start each batch's host-link feature read one batch ahead, on a side stream")
     ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c2w", "c4", "c3", "c5", "sample", "copy", "ceilings"])
+    ap.add_argument("--heads", type=int, default=1, help="c2w: heads of the weighted aggregation (divides 256)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
@@ -208,9 +209,15 @@ def run_c2w(args):
     ptr, idx = power_law_block(R, E, N, alpha=2.1, max_degree=5000, seed=2)
     ptr, idx = ptr.to(dev), idx.to(dev)
     gen = torch.Generator(device=dev).manual_seed(2)
+    H = max(1, int(args.heads))
+    if F % H != 0:
+        raise SystemExit("--heads must divide %d" % F)
     feat = torch.randn(N, F, device=dev, generator=gen)
     g = torch.randn(R, F, device=dev, generator=gen)
     ev = torch.rand(E, device=dev, generator=gen)
+    if H > 1:        # the same bytes seen as H heads of F / H elements with a weight per edge and head
+        feat, g = feat.view(N, H, F // H), g.view(R, H, F // H)
+        ev = torch.rand(E, H, device=dev, generator=gen)
     clk_f, clk_t, clk_b = KernelClock(), KernelClock(), KernelClock()
 
     def step():
@@ -229,17 +236,17 @@ def run_c2w(args):
     sync()
     sec = (time.perf_counter() - t0) / args.steps
     t_f, t_t, t_b = clk_f.mean_ms(), clk_t.mean_ms(), clk_b.mean_ms()
-    bytes_f = (R + 1) * 8 + E * (8 + 4) + E * F * 4 + R * F * 4
-    bytes_b = E * F * 4 + E * (4 + 4 + 4) + (N + 1) * 8 + N * F * 4      # input gradient
-    bytes_eg = E * (2 * F * 4 + 8 + 4)                                    # edge gradient: two rows per edge
+    bytes_f = (R + 1) * 8 + E * (8 + 4 * H) + E * F * 4 + R * F * 4
+    bytes_b = E * F * 4 + E * (4 + 4 + 4 * H) + (N + 1) * 8 + N * F * 4  # input gradient
+    bytes_eg = E * (2 * F * 4 + 8 + 4 * H)                                # edge gradient: two rows per edge
     return {
         "metric": "aggregated edges/sec (weighted fwd+bwd+edge_grad)", "value": E / sec, "unit": "edges/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "c2w: weighted aggregation (edge_value) on the c2 block, R=%d, E=%d, %d sources x %d "
-                               "fp32: fwd + transposed view with edge slots + bwd (input gradient and edge gradient)"
-                               % (R, E, N, F)},
-        "roofline": {"bound": "hbm", "kernel": "fwd_mean_fast<float,4,1,8,false,true>",
+                               "fp32 in %d head(s): fwd + transposed view with edge slots + bwd (input gradient and "
+                               "edge gradient)" % (R, E, N, F, H)},
+        "roofline": {"bound": "hbm", "kernel": "fwd_mean_fast<float,4,1,8,false,%d>" % (2 if H > 1 else 1),
                      "achieved": bytes_f / (t_f * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bytes_f / (t_f * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes": bytes_f, "launch_ms": t_f},

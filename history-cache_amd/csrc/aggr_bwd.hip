@@ -202,15 +202,20 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_hub_final(const int64_t *__restr
   for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store(o + k * HC_WAVE * VEC, acc[k]);
 }
 
-// WEIGHTED: every transposed edge contributes g[row] * edge_value[edge] (product rounded, then
+// WMODE W_EDGE: every transposed edge contributes g[row] * edge_value[edge] (product rounded, then
 // added) instead of g[row] / deg(row); edgeT gives the edge slot of a transposed edge.
-template <int VEC, int CHUNKS, int UNROLL, bool WEIGHTED>
+// WMODE W_EDGE_HEAD: a row is n_head heads side by side and the weight is edge_value[edge, head]; a
+// lane's VEC elements of a chunk lie inside one head, whose weight the lane loads itself.  (grad_hbuf
+// of such blocks is written by bwd_hist_generic.)
+constexpr int W_NONE = 0, W_EDGE = 1, W_EDGE_HEAD = 2;
+template <int VEC, int CHUNKS, int UNROLL, int WMODE>
 __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ ptrT, const int32_t *__restrict__ rowT,
-    const int32_t *__restrict__ edgeT, const float *__restrict__ ev, const float *__restrict__ g,
+    const int32_t *__restrict__ edgeT, const float *__restrict__ ev, int n_head, const float *__restrict__ g,
     const int64_t *__restrict__ hmap, float *__restrict__ grad_vin, float *__restrict__ grad_hbuf,
     int64_t hsize, int64_t R, int64_t n_src, int64_t src_blocks, int64_t hub_thres) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
+  constexpr bool WEIGHTED = WMODE != W_NONE;
   constexpr int S = BWD_SRC_PER_WAVE;
   const int lane = hc_lane();
   const int wave = hc_wave_in_block();
@@ -262,6 +267,9 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
   int64_t cur_end = hc_readlane64(my_p, 1);      // end of its segment
   float *__restrict__ obase = grad_vin + s0 * F + lane * VEC;
   int64_t base = hc_readlane64(my_p, 0);
+  int hd[CHUNKS];
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) hd[k] = WMODE == W_EDGE_HEAD ? ((k * HC_WAVE + lane) * VEC) / (F / n_head) : 0;
 
   while (true) {  // every branch below advances `cur` or `base`; all of it is wave-uniform
     // close the sources whose segment ends at or before `base` (zeros for sources without edges)
@@ -289,15 +297,18 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     const int64_t left = stop - base;
     const int n = left < HC_WAVE ? (int)left : HC_WAVE;
     int my_row = 0;
+    int my_edge = 0;
     float my_deg = 1.0f;
     if (lane < n) {
       my_row = rowT[base + lane];
-      if constexpr (WEIGHTED) my_deg = ev[edgeT[base + lane]];   // the weight takes the divisor's place
+      if constexpr (WMODE == W_EDGE_HEAD) my_edge = edgeT[base + lane];
+      else if constexpr (WMODE == W_EDGE) my_deg = ev[edgeT[base + lane]];   // the weight takes the divisor's place
       else my_deg = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
     }
     for (int j = 0; j < n; j += UNROLL) {
       float v[UNROLL][CHUNKS][VEC];
       float d[UNROLL];
+      float wh[WMODE == W_EDGE_HEAD ? UNROLL : 1][CHUNKS];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         d[u] = 1.0f;
@@ -307,6 +318,11 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
           const float *p = g + (int64_t)r * F + lane * VEC;
 #pragma unroll
           for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
+          if constexpr (WMODE == W_EDGE_HEAD) {
+            const int64_t e = (int64_t)__builtin_amdgcn_readlane(my_edge, j + u) * n_head;
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) wh[u][k] = ev[e + hd[k]];
+          }
         }
       }
 #pragma unroll
@@ -326,8 +342,10 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
 #pragma unroll
           for (int k = 0; k < CHUNKS; ++k)
 #pragma unroll
-            for (int i = 0; i < VEC; ++i)
-              acc[k][i] += WEIGHTED ? __fmul_rn(v[u][k][i], d[u]) : v[u][k][i] / d[u];
+            for (int i = 0; i < VEC; ++i) {
+              if constexpr (WMODE == W_EDGE_HEAD) acc[k][i] += __fmul_rn(v[u][k][i], wh[u][k]);
+              else acc[k][i] += WEIGHTED ? __fmul_rn(v[u][k][i], d[u]) : v[u][k][i] / d[u];
+            }
         }
       }
     }
@@ -559,17 +577,119 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_edge_grad_fast(
   if (lane < n) edge_grad[base + lane] = my_out;
 }
 
+// The same for rows of n_head heads side by side (F = n_head * fh elements): edge_grad[e, h] is the dot
+// product over head h only.  A head is either a whole number of 64-lane chunks (one butterfly over the
+// wave per head) or a power-of-two group of lanes inside a chunk (a butterfly inside each group); the
+// first lane of a group stores its head's value.  Slots of history rows and behind the last row get 0.
+template <typename T, int VEC, int CHUNKS, int UNROLL>
+__global__ __launch_bounds__(HC_BLOCK) void bwd_edge_grad_fast_heads(
+    const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const float *__restrict__ g,
+    const int64_t *__restrict__ hmap, const T *__restrict__ vin, float *__restrict__ edge_grad,
+    int64_t E_total, int64_t R, int n_head) {
+  constexpr int F = HC_WAVE * VEC * CHUNKS;
+  const int lane = hc_lane();
+  const int64_t base = ((int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block()) * HC_WAVE;
+  if (base >= E_total) return;
+  const int64_t left = E_total - base;
+  const int n = left < HC_WAVE ? (int)left : HC_WAVE;
+  const int lanes_per_head = (F / n_head) / VEC;
+  int64_t lo = 0, hi = R;
+  const int64_t probe = lane == 0 ? base : base + n - 1;
+  while (lo < hi) {
+    const int64_t mid = (lo + hi + 1) >> 1;
+    if (ptr[mid] <= probe) lo = mid;
+    else hi = mid - 1;
+  }
+  int64_t a = hc_readlane64(lo, 0), b = hc_readlane64(lo, 1);
+  int64_t my_row = -1, my_id = 0;
+  if (lane < n) {
+    const int64_t e = base + lane;
+    while (a < b) {
+      const int64_t mid = (a + b + 1) >> 1;
+      if (ptr[mid] <= e) a = mid;
+      else b = mid - 1;
+    }
+    if (a < R && ptr[a] <= e && (hmap == nullptr || hmap[a] == -1)) {
+      my_row = a;
+      my_id = idx[e];
+    }
+  }
+  for (int j = 0; j < n; j += UNROLL) {
+    float x[UNROLL][CHUNKS][VEC], gr[UNROLL][CHUNKS][VEC];
+    bool live[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      live[u] = false;
+      if (j + u < n) {
+        const int64_t r = hc_readlane64(my_row, j + u);
+        if (r >= 0) {
+          live[u] = true;
+          const T *px = vin + hc_readlane64(my_id, j + u) * F + lane * VEC;
+          const float *pg = g + r * F + lane * VEC;
+#pragma unroll
+          for (int k = 0; k < CHUNKS; ++k) {
+            hc_vec<T, VEC>::load(px + k * HC_WAVE * VEC, x[u][k]);
+            hc_vec<float, VEC>::load(pg + k * HC_WAVE * VEC, gr[u][k]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      if (!live[u]) continue;  // wave-uniform
+      float *__restrict__ o = edge_grad + (base + j + u) * n_head;
+      if (lanes_per_head >= HC_WAVE) {
+        const int chunks_per_head = lanes_per_head / HC_WAVE;
+        for (int h = 0; h < n_head; ++h) {
+          float part = 0.0f;
+#pragma unroll
+          for (int k = 0; k < CHUNKS; ++k)
+            if (k / chunks_per_head == h) {
+#pragma unroll
+              for (int i = 0; i < VEC; ++i) part = __fmaf_rn(gr[u][k][i], x[u][k][i], part);
+            }
+          part = hc_wave_sum_butterfly(part);
+          if (lane == 0) o[h] = part;
+        }
+      } else {
+        const int heads_per_chunk = HC_WAVE / lanes_per_head;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+          float part = 0.0f;
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) part = __fmaf_rn(gr[u][k][i], x[u][k][i], part);
+          for (int d = lanes_per_head >> 1; d >= 1; d >>= 1) part += __shfl_xor(part, d, HC_WAVE);
+          if (lane % lanes_per_head == 0) o[k * heads_per_chunk + lane / lanes_per_head] = part;
+        }
+      }
+    }
+  }
+  if (lane < n && my_row < 0) {
+    float *__restrict__ o = edge_grad + (base + lane) * n_head;
+    for (int h = 0; h < n_head; ++h) o[h] = 0.0f;
+  }
+}
+
+// Can bwd_edge_grad_fast_heads<.., VEC, ..> take rows of n_head heads of fh elements?
+inline bool edge_grad_heads_ok(int64_t fh, int vec) {
+  if (fh % vec != 0) return false;
+  const int64_t lanes = fh / vec;
+  if (lanes >= HC_WAVE) return lanes % HC_WAVE == 0;
+  return lanes >= 1 && (lanes & (lanes - 1)) == 0;
+}
+
 template <int VEC, int CHUNKS>
 int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, const int32_t *edgeT,
-                const float *ev, const float *g, const int64_t *hmap, float *grad_vin, float *grad_hbuf,
-                int64_t hsize, int64_t R, int64_t n_src, int64_t E_slots, void *workspace,
+                const float *ev, int n_head, const float *g, const int64_t *hmap, float *grad_vin,
+                float *grad_hbuf, int64_t hsize, int64_t R, int64_t n_src, int64_t E_slots, void *workspace,
                 size_t workspace_bytes, hipStream_t st) {
   constexpr int per = VEC * CHUNKS;
   constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   const int64_t per_block = (int64_t)HC_WAVES_PER_BLOCK * BWD_SRC_PER_WAVE;
   const int64_t sb = (n_src + per_block - 1) / per_block;
-  const int64_t hb = (grad_hbuf && hmap) ? (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK : 0;
+  // rows of several heads: grad_hbuf is written by bwd_hist_generic (the caller launches it)
+  const int64_t hb = (grad_hbuf && hmap && n_head == 1) ? (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK : 0;
   if (sb + hb == 0) return HC_OK;
   if (!hc_grid_ok(sb + hb)) return HC_EUNSUPPORTED;
   int64_t hub_thres = 0;
@@ -595,12 +715,15 @@ int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, co
         ptr, ptrT, rowT, g, hh, hub_src, hub_chunk0, chunk_hub, partial, L.max_chunks);
     if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
   }
-  if (ev != nullptr)
-    bwd_mean_fast<VEC, CHUNKS, UNROLL, true><<<dim3((unsigned)(sb + hb)), dim3(HC_BLOCK), 0, st>>>(
-        ptr, ptrT, rowT, edgeT, ev, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hub_thres);
+  if (ev != nullptr && n_head > 1)
+    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_EDGE_HEAD><<<dim3((unsigned)(sb + hb)), dim3(HC_BLOCK), 0, st>>>(
+        ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hub_thres);
+  else if (ev != nullptr)
+    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_EDGE><<<dim3((unsigned)(sb + hb)), dim3(HC_BLOCK), 0, st>>>(
+        ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hub_thres);
   else
-    bwd_mean_fast<VEC, CHUNKS, UNROLL, false><<<dim3((unsigned)(sb + hb)), dim3(HC_BLOCK), 0, st>>>(
-        ptr, ptrT, rowT, edgeT, ev, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hub_thres);
+    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_NONE><<<dim3((unsigned)(sb + hb)), dim3(HC_BLOCK), 0, st>>>(
+        ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hub_thres);
   if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
   if (hubs) {
     const int64_t hbk = (L.max_hubs + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
@@ -650,19 +773,30 @@ extern "C" int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t
   bool done = false;
   const bool aligned = (reinterpret_cast<uintptr_t>(g) % 16 == 0) &&
                        (reinterpret_cast<uintptr_t>(grad_vin) % 16 == 0);
-  // single-head weighted sums share the fast kernel when the history buffer has the plain width
-  if (n_head == 1 && aligned && (!edge_value || !grad_hbuf || hsize == F)) {
+  // Weighted sums share the fast kernel: a single head when the history buffer has the plain width, several
+  // heads as one row of F * n_head elements whose lanes fetch their own head's weight.
+  const int64_t Frow = F * n_head;
+  bool fast_hist_pending = false;
+  if (n_head <= 64 && aligned && (n_head > 1 || !edge_value || !grad_hbuf || hsize == F)) {
     int rc = HC_OK;
     done = true;
+    const int nh = (int)n_head;
 #define HC_FAST(V, C)                                                                             \
-  if (F == 64 * (V) * (C))                                                                        \
-    rc = launch_fast<V, C>(ptr, ptrT, rowT, edgeT, edge_value, g, hmap, grad_vin, grad_hbuf, hsize, R, \
+  if (Frow == 64 * (V) * (C) && F % (V) == 0)                                                     \
+    rc = launch_fast<V, C>(ptr, ptrT, rowT, edgeT, edge_value, nh, g, hmap, grad_vin, grad_hbuf, hsize, R, \
                            n_src, E_total, workspace, workspace_bytes, st);                         \
   else
     HC_FAST(4, 1) HC_FAST(4, 2) HC_FAST(4, 3) HC_FAST(4, 4) HC_FAST(2, 1) HC_FAST(2, 3) HC_FAST(1, 1)
     HC_FAST(1, 3) done = false;
 #undef HC_FAST
     if (done && rc != HC_OK) return rc;
+    fast_hist_pending = done && n_head > 1;
+  }
+  if (fast_hist_pending && grad_hbuf && R > 0) {
+    const int64_t hb = (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+    if (!hc_grid_ok(hb)) return HC_EUNSUPPORTED;
+    bwd_hist_generic<<<dim3((unsigned)hb), dim3(HC_BLOCK), 0, st>>>(g, hmap, grad_hbuf, hsize, R, F, n_head);
+    if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
   }
   if (!done) {
     const int64_t sb = (n_src * n_head + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
@@ -709,6 +843,32 @@ extern "C" int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t
       HC_EG(__hip_bfloat16, 4, 4) HC_EG(__hip_bfloat16, 2, 1) HC_EG(__hip_bfloat16, 1, 1) eg_done = false;
     }
 #undef HC_EG
+    if (eg_done && hc_launch_status() != HC_OK) return HC_ELAUNCH;
+  }
+  if (edge_grad && E_total > 0 && !eg_done && n_head > 1 && n_head <= 64 &&
+      (reinterpret_cast<uintptr_t>(vin) % 16 == 0) && (reinterpret_cast<uintptr_t>(g) % 16 == 0)) {
+    const int64_t wb = ((E_total + HC_WAVE - 1) / HC_WAVE + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+    if (!hc_grid_ok(wb)) return HC_EUNSUPPORTED;
+    dim3 gr((unsigned)wb), bl(HC_BLOCK);
+    const int64_t Fall = F * n_head;
+    const int nh = (int)n_head;
+    eg_done = true;
+#define HC_EGH(T, V, C)                                                                                  \
+  if (Fall == 64 * (V) * (C) && edge_grad_heads_ok(F, V))                                                \
+    bwd_edge_grad_fast_heads<T, V, C, ((V) * (C) >= 16 ? 2 : ((V) * (C) >= 8 ? 4 : 8))><<<gr, bl, 0, st>>>( \
+        ptr, idx, g, hmap, static_cast<const T *>(vin), edge_grad, E_total, R, nh);                       \
+  else
+    if (in_dtype == HC_F32) {
+      HC_EGH(float, 4, 1) HC_EGH(float, 4, 2) HC_EGH(float, 4, 3) HC_EGH(float, 4, 4) HC_EGH(float, 2, 1)
+      HC_EGH(float, 1, 1) eg_done = false;
+    } else if (in_dtype == HC_F16) {
+      HC_EGH(__half, 4, 1) HC_EGH(__half, 4, 2) HC_EGH(__half, 4, 3) HC_EGH(__half, 4, 4) HC_EGH(__half, 2, 1)
+      HC_EGH(__half, 1, 1) eg_done = false;
+    } else {
+      HC_EGH(__hip_bfloat16, 4, 1) HC_EGH(__hip_bfloat16, 4, 2) HC_EGH(__hip_bfloat16, 4, 3)
+      HC_EGH(__hip_bfloat16, 4, 4) HC_EGH(__hip_bfloat16, 2, 1) HC_EGH(__hip_bfloat16, 1, 1) eg_done = false;
+    }
+#undef HC_EGH
     if (eg_done && hc_launch_status() != HC_OK) return HC_ELAUNCH;
   }
   if (edge_grad && E_total > 0 && !eg_done) {

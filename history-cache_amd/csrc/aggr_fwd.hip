@@ -61,14 +61,19 @@ __device__ __forceinline__ void copy_row_any(const void *hbuf, int hist_dtype, i
 // STREAM: neighbour rows and ids are loaded with the non-temporal hint.  With per-source
 // substitution every edge also looks its source up in the map, and the map (not the rows, which
 // are too many to be reused) is what is worth keeping in the caches.
-// WEIGHTED: acc = fma(row, edge_value[edge], acc) instead of acc += row.
-template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM, bool WEIGHTED>
+// WMODE 0: acc += row.  WMODE 1: acc = fma(row, edge_value[edge], acc).  WMODE 2: the row holds
+// n_head heads side by side and every head has its own weight, edge_value[edge, head]; a lane's VEC
+// elements of a chunk lie inside one head (hd[chunk]), whose weight the lane loads itself.
+constexpr int W_NONE = 0, W_EDGE = 1, W_EDGE_HEAD = 2;
+template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM, int WMODE>
 __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, const T *__restrict__ vin,
                                                const int64_t *__restrict__ hmap, const T *__restrict__ htab,
                                                int64_t hsize, int src_mode, const float *__restrict__ ev,
+                                               int n_head, const int (&hd)[CHUNKS],
                                                int64_t begin, int64_t end, int lane,
                                                float (&acc)[CHUNKS][VEC]) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
+  constexpr bool WEIGHTED = WMODE != W_NONE;
   for (int64_t base = begin; base < end; base += HC_WAVE) {
     const int64_t left = end - base;
     const int n = left < HC_WAVE ? (int)left : HC_WAVE;
@@ -83,10 +88,11 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
         if (slot != -1) p = htab + slot * hsize;
       }
       my_addr = reinterpret_cast<int64_t>(p);
-      if constexpr (WEIGHTED) my_w = ev[base + lane];
+      if constexpr (WMODE == W_EDGE) my_w = ev[base + lane];
     }
     for (int j = 0; j < n; j += UNROLL) {
       float v[UNROLL][CHUNKS][VEC];
+      float wh[WMODE == W_EDGE_HEAD ? UNROLL : 1][CHUNKS];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         if (j + u < n) {
@@ -95,6 +101,7 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
           for (int k = 0; k < CHUNKS; ++k) {
             if constexpr (STREAM) hc_vec<T, VEC>::load_nt(p + k * HC_WAVE * VEC, v[u][k]);
             else hc_vec<T, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
+            if constexpr (WMODE == W_EDGE_HEAD) wh[u][k] = ev[(base + j + u) * n_head + hd[k]];
           }
         } else {
 #pragma unroll
@@ -105,7 +112,14 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
       }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
-        if constexpr (WEIGHTED) {
+        if constexpr (WMODE == W_EDGE_HEAD) {
+          if (j + u < n) {
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+              for (int i = 0; i < VEC; ++i) acc[k][i] = __fmaf_rn(v[u][k][i], wh[u][k], acc[k][i]);
+          }
+        } else if constexpr (WEIGHTED) {
           // lanes past the row's end hold zero rows and a zero weight: fma(0, 0, acc) == acc
           const float w = j + u < n ? hc_readlane_f(my_w, j + u) : 0.0f;
           if (j + u < n) {
@@ -191,7 +205,7 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_long_find(const int64_t *__restr
 }
 
 // One long row summed by the four waves of the calling block (all of them must call this).
-template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM, bool WEIGHTED>
+template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM, int WMODE>
 __device__ __forceinline__ void fwd_long_row(const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx,
                                              const T *__restrict__ vin, const int64_t *__restrict__ hmap,
                                              const T *__restrict__ htab, int64_t hsize, int src_mode,
@@ -199,6 +213,9 @@ __device__ __forceinline__ void fwd_long_row(const int64_t *__restrict__ ptr, co
                                              int64_t lrow, int lane, int wave,
                                              float (*part)[HC_WAVE * VEC * CHUNKS]) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
+  constexpr bool WEIGHTED = WMODE != W_NONE;
+  static_assert(WMODE != W_EDGE_HEAD, "rows of several heads are never split");
+  const int no_heads[CHUNKS] = {};
   const int64_t lb = ptr[lrow];
   const int64_t le = ptr[lrow + 1];
   const int64_t deg = le - lb;
@@ -212,8 +229,8 @@ __device__ __forceinline__ void fwd_long_row(const int64_t *__restrict__ ptr, co
   for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[c][i] = 0.0f;
-  fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM, WEIGHTED>(idx, vin, hmap, htab, hsize, src_mode, ev, sb, se, lane,
-                                                           acc);
+  fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM, WMODE>(idx, vin, hmap, htab, hsize, src_mode, ev, 1, no_heads, sb,
+                                                        se, lane, acc);
   if (wave > 0) {
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c)
@@ -241,13 +258,20 @@ __device__ __forceinline__ void fwd_long_row(const int64_t *__restrict__ ptr, co
   __syncthreads();
 }
 
-template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM, bool WEIGHTED>
+// WMODE == W_EDGE_HEAD: a row is n_head heads of F / n_head elements side by side (vin[n_src, n_head, F/n_head],
+// edge_value[E, n_head]); such launches come with long_thres == 0 and no list, so every row is summed
+// strictly in CSR order by its wave, and a history row copies hbuf[r, :hsize] once (hsize == F) or once
+// per head (hsize == F / n_head).
+template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM, int WMODE>
 __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const T *__restrict__ vin,
     const int64_t *__restrict__ hmap, const void *__restrict__ hbuf, int hist_dtype, int64_t hsize,
-    int src_mode, const float *__restrict__ ev, float *__restrict__ vout, int64_t R, int64_t long_thres,
-    FwdSched sched) {
+    int src_mode, const float *__restrict__ ev, int n_head, float *__restrict__ vout, int64_t R,
+    int64_t long_thres, FwdSched sched) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
+  constexpr bool WEIGHTED = WMODE != W_NONE;
+  // without heads the rows may be split: the split code is compiled for those modes only
+  constexpr int LMODE = WMODE == W_EDGE_HEAD ? W_EDGE : WMODE;
   __shared__ float part[HC_WAVES_PER_BLOCK - 1][F];
   __shared__ int long_rows[FWD_ROWS_PER_BLOCK];
   __shared__ int n_long_s;
@@ -260,8 +284,8 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
   if ((int)blockIdx.x < sched.front) {
     if (!listed) return;
     for (int t = (int)blockIdx.x; t < n_listed; t += sched.front)
-      fwd_long_row<T, VEC, CHUNKS, UNROLL, STREAM, WEIGHTED>(ptr, idx, vin, hmap, htab, hsize, src_mode, ev, vout,
-                                                             (int64_t)sched.rows[t], lane, wave, part);
+      fwd_long_row<T, VEC, CHUNKS, UNROLL, STREAM, LMODE>(ptr, idx, vin, hmap, htab, hsize, src_mode, ev, vout,
+                                                          (int64_t)sched.rows[t], lane, wave, part);
     return;
   }
   const int64_t row0 = hc_xcd_block<FWD_XCD_CHUNK>((int64_t)blockIdx.x - sched.front,
@@ -282,7 +306,12 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
     bool hist = false;
     if (!src_mode && hmap != nullptr) hist = hmap[row] != -1;
     if (hist) {
-      copy_row_any(hbuf, hist_dtype, row * hsize, orow, F, lane);
+      if (WMODE == W_EDGE_HEAD && hsize != F) {      // one history row shared by the heads
+        const int64_t fh = F / n_head;
+        for (int h = 0; h < n_head; ++h) copy_row_any(hbuf, hist_dtype, row * hsize, orow + h * fh, fh, lane);
+      } else {
+        copy_row_any(hbuf, hist_dtype, row * hsize, orow, F, lane);
+      }
     } else {
       const int64_t begin = ptr[row];
       const int64_t end = ptr[row + 1];
@@ -295,8 +324,11 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
         for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
           for (int i = 0; i < VEC; ++i) acc[c][i] = 0.0f;
-        fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM, WEIGHTED>(idx, vin, hmap, htab, hsize, src_mode, ev, begin,
-                                                                 end, lane, acc);
+        int hd[CHUNKS];
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) hd[c] = WMODE == W_EDGE_HEAD ? ((c * HC_WAVE + lane) * VEC) / (F / n_head) : 0;
+        fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM, WMODE>(idx, vin, hmap, htab, hsize, src_mode, ev, n_head, hd,
+                                                              begin, end, lane, acc);
         const float fdeg = (float)(int)deg;
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) {
@@ -314,8 +346,8 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
   const int n_long = n_long_s;
   // The order in which long rows were noted does not matter: each is summed on its own.
   for (int t = 0; t < n_long; ++t)
-    fwd_long_row<T, VEC, CHUNKS, UNROLL, STREAM, WEIGHTED>(ptr, idx, vin, hmap, htab, hsize, src_mode, ev, vout,
-                                                           row0 + long_rows[t], lane, wave, part);
+    fwd_long_row<T, VEC, CHUNKS, UNROLL, STREAM, LMODE>(ptr, idx, vin, hmap, htab, hsize, src_mode, ev, vout,
+                                                        row0 + long_rows[t], lane, wave, part);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -417,14 +449,15 @@ struct FwdScratch {
 
 template <typename T, int VEC, int CHUNKS>
 int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const int64_t *hmap,
-                const void *hbuf, int hist_dtype, int64_t hsize, int src_mode, const float *ev, float *vout,
-                int64_t R, FwdScratch ws, hipStream_t st) {
+                const void *hbuf, int hist_dtype, int64_t hsize, int src_mode, const float *ev, int n_head,
+                float *vout, int64_t R, FwdScratch ws, hipStream_t st) {
   constexpr int per = VEC * CHUNKS;
   constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
   int64_t blocks = (R + FWD_ROWS_PER_BLOCK - 1) / FWD_ROWS_PER_BLOCK;
   FwdSched sched{nullptr, nullptr, 0};
   int64_t cap = 0;
-  if (ws.ptr != nullptr && ws.bytes >= sizeof(FwdLongList) + sizeof(int) && R >= FWD_LIST_MIN_ROWS &&
+  const int64_t long_thres = n_head > 1 ? 0 : (int64_t)HC_LONG_ROW_EDGES;   // rows of several heads are never split
+  if (n_head == 1 && ws.ptr != nullptr && ws.bytes >= sizeof(FwdLongList) + sizeof(int) && R >= FWD_LIST_MIN_ROWS &&
       R <= 0x7fffffffLL && reinterpret_cast<uintptr_t>(ws.ptr) % 256 == 0) {
     cap = (int64_t)((ws.bytes - sizeof(FwdLongList)) / sizeof(int));
     if (cap > R) cap = R;
@@ -439,13 +472,14 @@ int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const i
     fwd_long_find<<<dim3((unsigned)((R + FWD_FIND_TILE - 1) / FWD_FIND_TILE)), dim3(HC_BLOCK), 0, st>>>(
         ptr, src_mode ? nullptr : hmap, R, (int64_t)HC_LONG_ROW_EDGES, sched.head, sched.rows);
   }
-#define HC_FWD_LAUNCH(STREAM, WEIGHTED)                                                                \
-  fwd_mean_fast<T, VEC, CHUNKS, UNROLL, STREAM, WEIGHTED><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>( \
-      ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, ev, vout, R,     \
-      (int64_t)HC_LONG_ROW_EDGES, sched)
-  if (ev != nullptr) HC_FWD_LAUNCH(false, true);
-  else if (src_mode && hmap != nullptr) HC_FWD_LAUNCH(true, false);
-  else HC_FWD_LAUNCH(false, false);
+#define HC_FWD_LAUNCH(STREAM, WMODE)                                                                   \
+  fwd_mean_fast<T, VEC, CHUNKS, UNROLL, STREAM, WMODE><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>( \
+      ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, ev, n_head, vout, R, \
+      long_thres, sched)
+  if (ev != nullptr && n_head > 1) HC_FWD_LAUNCH(false, W_EDGE_HEAD);
+  else if (ev != nullptr) HC_FWD_LAUNCH(false, W_EDGE);
+  else if (src_mode && hmap != nullptr) HC_FWD_LAUNCH(true, W_NONE);
+  else HC_FWD_LAUNCH(false, W_NONE);
 #undef HC_FWD_LAUNCH
   return hc_launch_status();
 }
@@ -454,11 +488,14 @@ int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const i
 template <typename T>
 int dispatch_fast(int64_t F, const int64_t *ptr, const int64_t *idx, const void *vin,
                   const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize, int src_mode,
-                  const float *ev, float *vout, int64_t R, FwdScratch ws, hipStream_t st, bool *handled) {
+                  const float *ev, int n_head, float *vout, int64_t R, FwdScratch ws, hipStream_t st,
+                  bool *handled) {
+  // F is the whole row (all heads); with several heads a lane's vector must not straddle two of them
   *handled = true;
 #define HC_FAST(V, C)                                                                              \
-  if (F == 64 * (V) * (C))                                                                         \
-    return launch_fast<T, V, C>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, ev, vout, R, ws, st);
+  if (F == 64 * (V) * (C) && (F / n_head) % (V) == 0)                                              \
+    return launch_fast<T, V, C>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, ev, n_head, vout, R, ws, \
+                                st);
   constexpr int VMAX = 16 / (int)sizeof(T);
   if constexpr (VMAX == 8) {
     HC_FAST(8, 1) HC_FAST(8, 2) HC_FAST(8, 3) HC_FAST(8, 4)
@@ -548,20 +585,23 @@ extern "C" int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, con
                        (reinterpret_cast<uintptr_t>(vout) % 16 == 0) &&
                        (!src_mode || !hmap ||
                         ((reinterpret_cast<uintptr_t>(hbuf) % 16 == 0) && ((hsize * esz) % 16 == 0)));
-  // single-head weighted sums share the fast path; a history row of a weighted block copies hbuf[r, :F]
+  // weighted sums share the fast path; a history row of a weighted block copies hbuf[r, :F].  With several
+  // heads the row of the fast path is all heads side by side (F * n_head elements).
   const bool weighted_ok = !edge_value || (!src_mode && (!hmap || hsize >= F));
-  if (n_head == 1 && weighted_ok && aligned && vin != nullptr) {
+  const int64_t Frow = F * n_head;
+  if (n_head <= 64 && weighted_ok && aligned && vin != nullptr) {
     bool handled = false;
     int rc;
+    const int nh = (int)n_head;
     if (in_dtype == HC_F32)
-      rc = dispatch_fast<float>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value, vout, R, ws,
-                                st, &handled);
+      rc = dispatch_fast<float>(Frow, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value, nh, vout, R,
+                                ws, st, &handled);
     else if (in_dtype == HC_F16)
-      rc = dispatch_fast<__half>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value, vout, R, ws,
-                                 st, &handled);
+      rc = dispatch_fast<__half>(Frow, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value, nh, vout,
+                                 R, ws, st, &handled);
     else
-      rc = dispatch_fast<__hip_bfloat16>(F, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode,
-                                         edge_value, vout, R, ws, st, &handled);
+      rc = dispatch_fast<__hip_bfloat16>(Frow, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode,
+                                         edge_value, nh, vout, R, ws, st, &handled);
     if (handled) return rc;
   }
   if (in_dtype == HC_F32)

@@ -292,12 +292,14 @@ def test_src_mode_backward(be, orc):
     np.testing.assert_array_equal(feat.grad.cpu().numpy(), orc.bwd_mean_src(ptr, idx, g, N, chunk=be.bwd_chunk_edges(F)))
 
 
-@pytest.mark.parametrize("F,H", [(64, 1), (256, 1), (96, 1), (32, 3), (256, 2)])
+@pytest.mark.parametrize("F,H", [(64, 1), (256, 1), (96, 1), (32, 3), (256, 2),
+                                 # several heads on the fast widths: heads of 8, 16, 32 lanes and of 2 chunks
+                                 (32, 8), (64, 4), (128, 2), (512, 2), (64, 3)])
 @pytest.mark.parametrize("hist_kind", ["none", "shared", "concat"])
 def test_edge_value_variants(be, orc, F, H, hist_kind):
     rng = np.random.default_rng(F + H)
     R, N = 120, 90
-    ptr, idx = random_csr(rng, R, N, 8, hub=70 if H > 1 else 700)     # one row above the long-row threshold
+    ptr, idx = random_csr(rng, R, N, 8, hub=700)     # one row above the long-row threshold (never split with heads)
     E = len(idx)
     multi = H > 1
     vin = rng.standard_normal((N, H, F) if multi else (N, F)).astype(np.float32)
