@@ -13,7 +13,7 @@
 // (grad_check.cu:25), so its slot numbering changes from run to run.  Here the
 // k-th admitted row (in row order) gets slot (header + k) mod capacity:
 //   pass 1  score + predicate per row, mask byte, admitted count per 64-row tile
-//   pass 2  one block scans the tile counts (exclusive), advances the header
+//   pass 2  one block scans the counts of 32-tile chunks (exclusive), advances the header
 //   pass 3  per tile: ballot-rank the mask, un-map old owners, copy rows, map
 // Pass 1 is the only pass that touches the gradient matrix; pass 3 only touches
 // admitted rows, so HBM traffic is the algorithmic minimum.
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(HC_BLOCK) void gc_pass1(
     const float *__restrict__ grad, const float *__restrict__ score_in, const int64_t *__restrict__ slot,
     const int32_t *__restrict__ age, const uint8_t *__restrict__ used, const float *__restrict__ thres_p,
     int32_t age_limit, int norm_kind, int cmp_kind, uint8_t *__restrict__ mask_out,
-    float *__restrict__ score_out, int64_t *__restrict__ tile_counts, int64_t M, int64_t F) {
+    float *__restrict__ score_out, uint8_t *__restrict__ tile_counts, int64_t M, int64_t F) {
   __shared__ int wave_cnt[HC_WAVES_PER_BLOCK];
   const int lane = hc_lane();
   const int wave = hc_wave_in_block();
@@ -151,62 +151,74 @@ __global__ __launch_bounds__(HC_BLOCK) void gc_pass1(
     int t = 0;
 #pragma unroll
     for (int w = 0; w < HC_WAVES_PER_BLOCK; ++w) t += wave_cnt[w];
-    tile_counts[blockIdx.x] = t;
+    tile_counts[blockIdx.x] = (uint8_t)t;   // at most GC_TILE = 64
   }
 }
 
 // ---------------------------------------------------------------------------------------
-// Pass 2: exclusive scan of the tile counts by one block; header bookkeeping.
+// Pass 2: header bookkeeping and the exclusive scan of the admitted counts, by one block.  Pass 1
+// leaves one BYTE per tile (a count is at most 64); a thread takes a chunk of GC_CHUNK = 32
+// consecutive tiles with two 16-byte loads and the block scans the chunk sums.  Pass 3 adds the
+// counts of the tiles before its own inside the chunk (the same two loads, masked).  Scanning 32
+// times fewer values than one 8-byte count per tile takes the pass from 27 to a few microseconds
+// for 2 M rows; writing one offset per tile from this single block would cost most of that again.
 // ring != 0: header = (header + A) mod capacity.   ring == 0 (append): rows beyond capacity
 // are dropped, header += written, *overflow = dropped.
 // ---------------------------------------------------------------------------------------
 constexpr int GC_SCAN_THREADS = 1024;
-constexpr int GC_SCAN_ITEMS = 8;  // consecutive counts per thread per sweep
-__global__ __launch_bounds__(GC_SCAN_THREADS) void gc_pass2(int64_t *__restrict__ tile_counts,
-                                                             int64_t n_tiles, GcScalars *__restrict__ sc,
+constexpr int GC_CHUNK = 32;  // tiles per thread and sweep
+
+__global__ __launch_bounds__(GC_SCAN_THREADS) void gc_pass2(const uint8_t *__restrict__ tile_counts,
+                                                             int64_t n_tiles, int64_t *__restrict__ chunk_prefix,
+                                                             GcScalars *__restrict__ sc,
                                                              int64_t *__restrict__ header,
                                                              int64_t capacity, int ring,
                                                              int64_t *__restrict__ overflow) {
-  __shared__ int64_t wave_tot[GC_SCAN_THREADS / HC_WAVE];
+  __shared__ int wave_tot[GC_SCAN_THREADS / HC_WAVE];
   __shared__ int64_t carry_s;
   const int lane = hc_lane();
   const int wave = (int)(threadIdx.x >> 6);
   if (threadIdx.x == 0) carry_s = 0;
   __syncthreads();
-  constexpr int64_t SWEEP = (int64_t)GC_SCAN_THREADS * GC_SCAN_ITEMS;
-  for (int64_t base = 0; base < n_tiles; base += SWEEP) {
-    const int64_t i0 = base + (int64_t)threadIdx.x * GC_SCAN_ITEMS;
-    int64_t v[GC_SCAN_ITEMS];
-    int64_t mine = 0;
+  const int64_t n_chunks = (n_tiles + GC_CHUNK - 1) / GC_CHUNK;
+  for (int64_t base = 0; base < n_chunks; base += GC_SCAN_THREADS) {
+    const int64_t t0 = (base + threadIdx.x) * GC_CHUNK;
+    uint32_t w[GC_CHUNK / 4];
 #pragma unroll
-    for (int k = 0; k < GC_SCAN_ITEMS; ++k) {
-      v[k] = i0 + k < n_tiles ? tile_counts[i0 + k] : 0;
-      mine += v[k];
+    for (int k = 0; k < GC_CHUNK / 4; ++k) w[k] = 0u;
+    if (t0 + GC_CHUNK <= n_tiles) {        // tile_counts is 16-byte aligned
+      const uint4 a = *reinterpret_cast<const uint4 *>(tile_counts + t0);
+      const uint4 b = *reinterpret_cast<const uint4 *>(tile_counts + t0 + 16);
+      w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w;
+      w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
+    } else {
+#pragma unroll
+      for (int k = 0; k < GC_CHUNK; ++k)
+        if (t0 + k < n_tiles) w[k / 4] |= (uint32_t)tile_counts[t0 + k] << (8 * (k % 4));
     }
-    // inclusive scan of the per-thread sums inside the wave
-    int64_t x = mine;
+    int mine = 0;
+#pragma unroll
+    for (int k = 0; k < GC_CHUNK / 4; ++k) {
+      const uint32_t s2 = (w[k] & 0x00ff00ffu) + ((w[k] >> 8) & 0x00ff00ffu);
+      mine += (int)((s2 & 0xffffu) + (s2 >> 16));
+    }
+    // inclusive scan of the per-thread sums inside the wave (a sweep's total is below 2^22)
+    int x = mine;
 #pragma unroll
     for (int d = 1; d < HC_WAVE; d <<= 1) {
-      const int lo = __shfl_up((int)(uint32_t)(uint64_t)x, d, HC_WAVE);
-      const int hi = __shfl_up((int)(uint32_t)((uint64_t)x >> 32), d, HC_WAVE);
-      const int64_t y = (int64_t)(((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo);
+      const int y = __shfl_up(x, d, HC_WAVE);
       if (lane >= d) x += y;
     }
     if (lane == HC_WAVE - 1) wave_tot[wave] = x;
     __syncthreads();
-    int64_t wave_off = 0, sweep_total = 0;
-    for (int w = 0; w < GC_SCAN_THREADS / HC_WAVE; ++w) {
-      const int64_t t = wave_tot[w];
-      if (w < wave) wave_off += t;
+    int wave_off = 0, sweep_total = 0;
+    for (int wv = 0; wv < GC_SCAN_THREADS / HC_WAVE; ++wv) {
+      const int t = wave_tot[wv];
+      if (wv < wave) wave_off += t;
       sweep_total += t;
     }
     const int64_t carry = carry_s;
-    int64_t run = carry + wave_off + x - mine;  // exclusive prefix of this thread's first item
-#pragma unroll
-    for (int k = 0; k < GC_SCAN_ITEMS; ++k) {
-      if (i0 + k < n_tiles) tile_counts[i0 + k] = run;
-      run += v[k];
-    }
+    if (base + threadIdx.x < n_chunks) chunk_prefix[base + threadIdx.x] = carry + wave_off + x - mine;
     __syncthreads();
     if (threadIdx.x == 0) carry_s = carry + sweep_total;
     __syncthreads();
@@ -258,12 +270,35 @@ __device__ __forceinline__ void store_relaxed(int64_t *p, int64_t v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Rank of a tile's first admitted row among all admitted rows: its chunk's prefix plus the counts of
+// the tiles before it inside the chunk.  Every thread of the block computes the same value from the
+// same 40 bytes.  (The count array is padded to whole chunks; bytes of tiles that do not exist are
+// never added, because they lie behind every existing tile of their chunk.)
+__device__ __forceinline__ int64_t tile_offset(const uint8_t *__restrict__ tile_counts,
+                                               const int64_t *__restrict__ chunk_prefix, int64_t tile) {
+  const int64_t chunk = tile / GC_CHUNK;
+  const int within = (int)(tile - chunk * GC_CHUNK);
+  const uint4 a = *reinterpret_cast<const uint4 *>(tile_counts + chunk * GC_CHUNK);
+  const uint4 b = *reinterpret_cast<const uint4 *>(tile_counts + chunk * GC_CHUNK + 16);
+  const uint32_t w[GC_CHUNK / 4] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  int sum = 0;
+#pragma unroll
+  for (int k = 0; k < GC_CHUNK / 4; ++k) {
+    const int nb = within - 4 * k;   // bytes of this word that belong to earlier tiles
+    const uint32_t m = nb >= 4 ? 0xffffffffu : (nb <= 0 ? 0u : ((1u << (8 * nb)) - 1u));
+    const uint32_t v = w[k] & m;
+    const uint32_t s2 = (v & 0x00ff00ffu) + ((v >> 8) & 0x00ff00ffu);
+    sum += (int)((s2 & 0xffffu) + (s2 >> 16));
+  }
+  return chunk_prefix[chunk] + sum;
+}
+
 // ---------------------------------------------------------------------------------------
 // Pass 3 (ring): per tile, rank the admitted rows, un-map old owners, copy, map.
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(HC_BLOCK) void gc_pass3_ring(
-    const uint8_t *__restrict__ mask, const int64_t *__restrict__ tile_offsets,
-    const GcScalars *__restrict__ sc, const float *__restrict__ emb,
+    const uint8_t *__restrict__ mask, const uint8_t *__restrict__ tile_counts,
+    const int64_t *__restrict__ chunk_prefix, const GcScalars *__restrict__ sc, const float *__restrict__ emb,
     const int64_t *__restrict__ sub_to_full, void *__restrict__ table, int table_dtype, int64_t capacity,
     int64_t *__restrict__ full2slot, int64_t *__restrict__ slot2full, int64_t *__restrict__ checkin,
     int64_t *__restrict__ slot_out, int64_t glb_iter, int64_t M, int64_t F) {
@@ -274,7 +309,7 @@ __global__ __launch_bounds__(HC_BLOCK) void gc_pass3_ring(
   const int64_t tile0 = (int64_t)blockIdx.x * GC_TILE;
   const int64_t header_old = sc->header_old;
   const int64_t A = sc->admitted;
-  const int64_t tile_off = tile_offsets[blockIdx.x];
+  const int64_t tile_off = tile_offset(tile_counts, chunk_prefix, (int64_t)blockIdx.x);
   if (wave == 0) {
     const int64_t r = tile0 + lane;
     const bool m = r < M && mask[r] != 0;
@@ -348,8 +383,8 @@ __global__ __launch_bounds__(HC_BLOCK) void gc_append_invalidate(
 }
 
 __global__ __launch_bounds__(HC_BLOCK) void gc_pass3_append(
-    const uint8_t *__restrict__ mask, const int64_t *__restrict__ tile_offsets,
-    const GcScalars *__restrict__ sc, const float *__restrict__ emb,
+    const uint8_t *__restrict__ mask, const uint8_t *__restrict__ tile_counts,
+    const int64_t *__restrict__ chunk_prefix, const GcScalars *__restrict__ sc, const float *__restrict__ emb,
     const int64_t *__restrict__ sub_to_full, float *__restrict__ buffer, int64_t H,
     int64_t *__restrict__ full2embed, int64_t *__restrict__ embed2full, int64_t M) {
   __shared__ int local_rows[GC_TILE];
@@ -359,7 +394,7 @@ __global__ __launch_bounds__(HC_BLOCK) void gc_pass3_append(
   const int64_t tile0 = (int64_t)blockIdx.x * GC_TILE;
   const int64_t header_old = sc->header_old;
   const int64_t written = sc->written;
-  const int64_t tile_off = tile_offsets[blockIdx.x];
+  const int64_t tile_off = tile_offset(tile_counts, chunk_prefix, (int64_t)blockIdx.x);
   if (wave == 0) {
     const int64_t r = tile0 + lane;
     const bool m = r < M && mask[r] != 0;
@@ -384,15 +419,25 @@ __global__ __launch_bounds__(HC_BLOCK) void gc_pass3_append(
   }
 }
 
-size_t ws_bytes(int64_t M) {
-  const int64_t tiles = (M + GC_TILE - 1) / GC_TILE;
-  return hc_align_up(sizeof(GcScalars) + (size_t)(tiles > 0 ? tiles : 1) * sizeof(int64_t), 256);
+// Workspace: GcScalars | chunk_prefix[chunks] int64 | tile_counts[chunks * 32] uint8 (16-byte aligned).
+struct GcLayout {
+  size_t prefix, counts, total;
+};
+GcLayout gc_layout(int64_t M) {
+  const int64_t tiles = M > 0 ? (M + GC_TILE - 1) / GC_TILE : 1;
+  const int64_t chunks = (tiles + GC_CHUNK - 1) / GC_CHUNK;
+  GcLayout L;
+  L.prefix = sizeof(GcScalars);
+  L.counts = hc_align_up(L.prefix + (size_t)chunks * sizeof(int64_t), 16);
+  L.total = hc_align_up(L.counts + (size_t)chunks * GC_CHUNK, 256);
+  return L;
 }
+size_t ws_bytes(int64_t M) { return gc_layout(M).total; }
 
 template <bool PRED>
 int launch_pass1(const float *grad, const float *score_in, const int64_t *slot, const int32_t *age,
                  const uint8_t *used, const float *thres, int32_t age_limit, int norm_kind, int cmp_kind,
-                 uint8_t *mask_out, float *score_out, int64_t *tile_counts, int64_t M, int64_t F,
+                 uint8_t *mask_out, float *score_out, uint8_t *tile_counts, int64_t M, int64_t F,
                  hipStream_t st) {
   const int64_t tiles = (M + GC_TILE - 1) / GC_TILE;
   if (!hc_grid_ok(tiles)) return HC_EUNSUPPORTED;
@@ -445,16 +490,19 @@ extern "C" int hc_grad_check(const float *grad, const float *score_in, const flo
     return HC_EWORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
   GcScalars *sc = static_cast<GcScalars *>(workspace);
-  int64_t *tiles_buf = reinterpret_cast<int64_t *>(sc + 1);
+  const GcLayout L = gc_layout(M);
+  int64_t *chunk_prefix = reinterpret_cast<int64_t *>(static_cast<char *>(workspace) + L.prefix);
+  uint8_t *tiles_buf = reinterpret_cast<uint8_t *>(workspace) + L.counts;
   const int64_t tiles = (M + GC_TILE - 1) / GC_TILE;
 
   int rc = launch_pass1<true>(grad, score_in, slot, age, used, thres, age_limit, norm_kind, cmp_kind,
                               mask_out, score_out, tiles_buf, M, F, st);
   if (rc != HC_OK) return rc;
-  gc_pass2<<<dim3(1), dim3(GC_SCAN_THREADS), 0, st>>>(tiles_buf, tiles, sc, header, capacity, 1, nullptr);
+  gc_pass2<<<dim3(1), dim3(GC_SCAN_THREADS), 0, st>>>(tiles_buf, tiles, chunk_prefix, sc, header, capacity, 1,
+                                                      nullptr);
   if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
   gc_pass3_ring<<<dim3((unsigned)tiles), dim3(HC_BLOCK), 0, st>>>(
-      mask_out, tiles_buf, sc, emb, sub_to_full, table, table_dtype, capacity, full2slot, slot2full,
+      mask_out, tiles_buf, chunk_prefix, sc, emb, sub_to_full, table, table_dtype, capacity, full2slot, slot2full,
       checkin, slot_out, glb_iter, M, F);
   return hc_launch_status();
 }
@@ -495,13 +543,16 @@ extern "C" int hc_cache_append(const float *score, const float *thres, const flo
     return HC_EWORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
   GcScalars *sc = static_cast<GcScalars *>(workspace);
-  int64_t *tiles_buf = reinterpret_cast<int64_t *>(sc + 1);
+  const GcLayout L = gc_layout(M);
+  int64_t *chunk_prefix = reinterpret_cast<int64_t *>(static_cast<char *>(workspace) + L.prefix);
+  uint8_t *tiles_buf = reinterpret_cast<uint8_t *>(workspace) + L.counts;
   const int64_t tiles = (M + GC_TILE - 1) / GC_TILE;
 
   int rc = launch_pass1<true>(nullptr, score, sub2embed, nullptr, nullptr, thres, 0, HC_NORM_L2,
                               HC_CMP_LT, mask_out, nullptr, tiles_buf, M, H, st);
   if (rc != HC_OK) return rc;
-  gc_pass2<<<dim3(1), dim3(GC_SCAN_THREADS), 0, st>>>(tiles_buf, tiles, sc, header, capacity, 0, overflow);
+  gc_pass2<<<dim3(1), dim3(GC_SCAN_THREADS), 0, st>>>(tiles_buf, tiles, chunk_prefix, sc, header, capacity, 0,
+                                                      overflow);
   if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
   // worst-case span of feature slots covered by M embedding rows
   const int64_t max_feat_span = (M * H + F_in - 1) / F_in + 2;
@@ -511,7 +562,7 @@ extern "C" int hc_cache_append(const float *score, const float *thres, const flo
   gc_append_invalidate<<<dim3((unsigned)iblocks), dim3(HC_BLOCK), 0, st>>>(
       sc, H, F_in, full2embed, embed2full, feat2full, n_feat, max_feat_span, M);
   if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
-  gc_pass3_append<<<dim3((unsigned)tiles), dim3(HC_BLOCK), 0, st>>>(mask_out, tiles_buf, sc, emb,
+  gc_pass3_append<<<dim3((unsigned)tiles), dim3(HC_BLOCK), 0, st>>>(mask_out, tiles_buf, chunk_prefix, sc, emb,
                                                                     sub_to_full, buffer, H, full2embed,
                                                                     embed2full, M);
   return hc_launch_status();
