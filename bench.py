@@ -34,6 +34,9 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--with-sampler", action="store_true",
+                    help="c3: draw every batch with the device sampler from a papers100M-sized graph in HBM "
+                         "(next batch sampled on a side stream) instead of taking pre-generated batches")
     ap.add_argument("--prefetch", action="store_true",
                     help="c3/c5: start each batch's host-link feature read one batch ahead, on a side stream")
     ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c2w", "c4", "c3", "c5", "sample", "copy", "ceilings"])
@@ -487,12 +490,35 @@ def run_c3(args):
         batches.append(make_batch(smp, labels, dev))
     ev = {k: KernelClock() for k in ("load", "forward", "backward", "step", "update")}
     state = {"it": 0}
+    sampled = {"sampler": None, "pending": None, "shapes": [], "wait_s": 0.0, "E_graph": 0}
+    if args.with_sampler:
+        # batches come from the device sampler over a graph of the same size held in HBM; batch i+1 is
+        # sampled on the sampler's side stream while batch i trains
+        from hiscache import NeighborSampler
+        indptr, indices = device_power_law_graph(N, 14.5, dev, gen)
+        sampled["E_graph"] = indices.numel()
+        sampled["sampler"] = NeighborSampler(indptr, indices, fanout, seed=3, device=dev, validate=False)
+        del indptr, indices
+        seed_pool = torch.randperm(N, device=dev, generator=gen)[: n_seed * 1024].view(1024, n_seed).contiguous()
+        sampled["pending"] = sampled["sampler"].sample_async(seed_pool[0])
+
+    def next_batch():
+        if sampled["sampler"] is None:
+            return batches[(state["it"] - 1) % n_pre]
+        i = state["it"] - 1
+        t1 = time.perf_counter()
+        b = sampled["pending"].get()                       # waits only if the sampling is not finished yet
+        sampled["wait_s"] += time.perf_counter() - t1
+        b.y = seed_pool[i % 1024] % C
+        sampled["pending"] = sampled["sampler"].sample_async(seed_pool[(i + 1) % 1024])
+        sampled["shapes"].append(b.num_node_in_layer.tolist() + [b.idx.numel()])
+        return b
 
     def step():
-        b = batches[state["it"] % n_pre]
         state["it"] += 1
+        b = next_batch()
         ev["load"](lambda: cache.lookup_and_load(b, L))
-        if args.prefetch:             # the next batch's host-link read runs under this batch's compute
+        if args.prefetch and sampled["sampler"] is None:   # the next batch's host-link read runs under this batch's compute
             cache.prefetch(batches[state["it"] % n_pre])
         out = ev["forward"](lambda: model(b))
         loss = torch.nn.functional.nll_loss(out, b.y)
@@ -506,13 +532,21 @@ def run_c3(args):
     sync()
     for c in ev.values():
         c.reset()
+    sampled["shapes"], sampled["wait_s"] = [], 0.0
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
     sync()
     sec = (time.perf_counter() - t0) / args.steps
-    shape = {k: int(np.mean([int(x["num_node_in_layer"][i]) for x in samples])) for i, k in enumerate(("n0", "n1", "n2", "n3"))}
-    shape["edges"] = int(np.mean([x["idx"].size for x in samples]))
+    if sampled["sampler"] is not None:
+        sampled["pending"].get()
+        m = np.mean(np.asarray(sampled["shapes"], dtype=np.float64), axis=0)
+        shape = {"n0": int(m[0]), "n1": int(m[1]), "n2": int(m[2]), "n3": int(m[3]), "edges": int(m[4]),
+                 "sampled_on_device_from_graph_edges": sampled["E_graph"],
+                 "wait_for_sampler_ms": 1e3 * sampled["wait_s"] / args.steps}
+    else:
+        shape = {k: int(np.mean([int(x["num_node_in_layer"][i]) for x in samples])) for i, k in enumerate(("n0", "n1", "n2", "n3"))}
+        shape["edges"] = int(np.mean([x["idx"].size for x in samples]))
 
     # ---- batched variant of the history layer: K batches side by side, about 20M edges
     rows, cols, ptrs, idxs, hms = 0, 0, [np.zeros(1, np.int64)], [], []
