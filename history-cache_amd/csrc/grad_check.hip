@@ -19,6 +19,8 @@
 // admitted rows, so HBM traffic is the algorithmic minimum.
 #include "hc_common.h"
 
+#include <mutex>
+
 namespace {
 
 constexpr int GC_TILE = 64;                                   // rows per block (= one ballot)
@@ -505,6 +507,70 @@ extern "C" int hc_grad_check(const float *grad, const float *score_in, const flo
       mask_out, tiles_buf, chunk_prefix, sc, emb, sub_to_full, table, table_dtype, capacity, full2slot, slot2full,
       checkin, slot_out, glb_iter, M, F);
   return hc_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// hc_grad_check_static: the fused admission pass for callers that cannot allocate (code under
+// stream capture, serving loops, harnesses that forbid hipMalloc).  Its scratch (the scalars, the
+// chunk prefixes and the tile counts of gc_layout) lives in a file-scope device array instead of a
+// caller workspace.  In host code the array's name is only a handle: its device address is
+// looked up once per device with hipGetSymbolAddress and kept; the kernels take that address.
+// Every GPU holds its own copy of the array until the process ends.  Nothing in it has to start at
+// zero: pass 1 writes every tile count pass 2 and pass 3 read, pass 2 writes the scalars and the
+// chunk prefixes pass 3 reads, so a call is not disturbed by what the previous one left behind.
+// ---------------------------------------------------------------------------------------
+namespace {
+
+constexpr int64_t GC_STATIC_MAX_ROWS = HC_GRAD_CHECK_STATIC_MAX_ROWS;   // rows per call
+constexpr int64_t GC_STATIC_TILES = GC_STATIC_MAX_ROWS / GC_TILE;
+constexpr int64_t GC_STATIC_CHUNKS = GC_STATIC_TILES / GC_CHUNK;
+// GcScalars | chunk_prefix | tile_counts, rounded up as gc_layout rounds (checked at run time)
+constexpr size_t GC_STATIC_BYTES =
+    (sizeof(GcScalars) + (size_t)GC_STATIC_CHUNKS * sizeof(int64_t) + (size_t)GC_STATIC_CHUNKS * GC_CHUNK + 255) /
+    256 * 256;
+
+static __device__ __align__(256) unsigned char scratch[GC_STATIC_BYTES];
+
+constexpr int GC_MAX_DEVICES = 64;
+void *g_scratch_ptr[GC_MAX_DEVICES];   // device address of `scratch`, per device (nullptr: not looked up yet)
+std::mutex g_scratch_mutex;
+
+// Device address of this device's copy of `scratch`; nullptr on failure.
+void *static_scratch(int *status) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) { *status = HC_ENODEVICE; return nullptr; }
+  if (dev < 0 || dev >= GC_MAX_DEVICES) { *status = HC_EUNSUPPORTED; return nullptr; }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      *status = HC_ELAUNCH;
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  *status = HC_OK;
+  return g_scratch_ptr[dev];
+}
+
+}  // namespace
+
+extern "C" int hc_grad_check_static(const float *grad, const float *score_in, const float *emb,
+                                    const int64_t *slot, const int32_t *age, const uint8_t *used,
+                                    const int64_t *sub_to_full, const float *thres, int32_t age_limit,
+                                    int norm_kind, int cmp_kind, uint8_t *mask_out, float *score_out,
+                                    int64_t *slot_out, void *table, int table_dtype, int64_t capacity,
+                                    int64_t *full2slot, int64_t *slot2full, int64_t *checkin,
+                                    int64_t *header, int64_t glb_iter, int64_t M, int64_t F, void *stream) {
+  HC_REQUIRE(M >= 0);
+  if (M > GC_STATIC_MAX_ROWS || ws_bytes(M) > GC_STATIC_BYTES) return HC_EUNSUPPORTED;
+  int rc = HC_OK;
+  void *ws = static_scratch(&rc);
+  if (ws == nullptr) return rc;
+  return hc_grad_check(grad, score_in, emb, slot, age, used, sub_to_full, thres, age_limit, norm_kind,
+                       cmp_kind, mask_out, score_out, slot_out, table, table_dtype, capacity, full2slot,
+                       slot2full, checkin, header, glb_iter, M, F, ws, GC_STATIC_BYTES, stream);
 }
 
 extern "C" int hc_record_history(const float *buffer_new, float *buffer_all, const uint8_t *used_mask,

@@ -33,6 +33,7 @@ HC_F32, HC_F16, HC_BF16 = 0, 1, 2
 SUBST_ROW, SUBST_SRC = 0, 1
 NORM_L2, NORM_L1 = 0, 1
 CMP_LT, CMP_NOT_GT = 0, 1
+GRAD_CHECK_STATIC_MAX_ROWS = 1 << 24   # HC_GRAD_CHECK_STATIC_MAX_ROWS
 
 _DTYPES = {torch.float32: HC_F32, torch.float16: HC_F16, torch.bfloat16: HC_BF16}
 
@@ -63,6 +64,9 @@ _SIGNATURES = {
     "hc_grad_check": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, ctypes.c_int32, _c_int,
                                _c_int, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_p,
                                _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]),
+    "hc_grad_check_static": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, ctypes.c_int32, _c_int,
+                                      _c_int, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_p,
+                                      _c_i64, _c_i64, _c_i64, _c_p]),
     "hc_record_history": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,
                                    _c_i64, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]),
     "hc_cache_append": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p,
@@ -464,8 +468,12 @@ def row_scores(grad, norm_kind=NORM_L2):
 
 def grad_check(grad, emb, slot, sub_to_full, thres, table, full2slot, slot2full, header, glb_iter,
                age=None, age_limit=0, used=None, checkin=None, norm_kind=NORM_L2, cmp_kind=CMP_LT,
-               score=None, want_slots=False):
+               score=None, want_slots=False, static_scratch=False):
     """Fused admission pass (scores, predicate, mask, row-order ring slots, table scatter, maps).
+
+    ``static_scratch=True`` goes through ``hc_grad_check_static``: the passes share a fixed device
+    array inside the library instead of a workspace tensor (at most GRAD_CHECK_STATIC_MAX_ROWS rows;
+    calls that overlap on one GPU race).
 
     ``grad`` [M,F] fp32 (or None with ``score`` given), ``emb`` [M,F] fp32, ``slot`` [M] int64
     (-1 = not cached), ``thres`` 1-element fp32 device tensor, ``table`` [capacity,F]
@@ -504,13 +512,17 @@ def grad_check(grad, emb, slot, sub_to_full, thres, table, full2slot, slot2full,
     mask = torch.empty(M, dtype=torch.uint8, device=dev)
     score_out = torch.empty(M, dtype=torch.float32, device=dev)
     slot_out = torch.empty(M, dtype=torch.int64, device=dev) if want_slots else None
-    ws = _workspace(lib.hc_grad_check_workspace_bytes(M), dev)
-    rc = lib.hc_grad_check(_ptr(grad), _ptr(score), _ptr(emb), _ptr(slot), _ptr(age), _ptr(used),
-                           _ptr(sub_to_full), _ptr(thres), int(age_limit), int(norm_kind), int(cmp_kind),
-                           _ptr(mask), _ptr(score_out), _ptr(slot_out), _ptr(table),
-                           _float_dtype(table, "table"), table.shape[0], _ptr(full2slot), _ptr(slot2full),
-                           _ptr(checkin), _ptr(header), int(glb_iter), M, F, _ptr(ws), ws.numel(), _stream())
-    _check(rc, "hc_grad_check")
+    args = (_ptr(grad), _ptr(score), _ptr(emb), _ptr(slot), _ptr(age), _ptr(used),
+            _ptr(sub_to_full), _ptr(thres), int(age_limit), int(norm_kind), int(cmp_kind),
+            _ptr(mask), _ptr(score_out), _ptr(slot_out), _ptr(table),
+            _float_dtype(table, "table"), table.shape[0], _ptr(full2slot), _ptr(slot2full),
+            _ptr(checkin), _ptr(header), int(glb_iter), M, F)
+    if static_scratch:
+        with torch.cuda.device(dev):
+            _check(lib.hc_grad_check_static(*args, _stream()), "hc_grad_check_static")
+    else:
+        ws = _workspace(lib.hc_grad_check_workspace_bytes(M), dev)
+        _check(lib.hc_grad_check(*args, _ptr(ws), ws.numel(), _stream()), "hc_grad_check")
     if want_slots:
         return mask.view(torch.bool), score_out, slot_out
     return mask.view(torch.bool), score_out

@@ -197,6 +197,25 @@ int hc_grad_check(const float *grad, const float *score_in, const float *emb, co
                   int64_t *checkin, int64_t *header, int64_t glb_iter, int64_t M, int64_t F,
                   void *workspace, size_t workspace_bytes, void *stream);
 
+/* hc_grad_check_static: hc_grad_check without a workspace argument, for callers
+ * that cannot allocate device memory (code under stream capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same arguments, results and kernels as hc_grad_check; the scratch
+ * the passes share lives in a fixed device array inside the library (about
+ * 0.33 MB per GPU, held until the process ends), whose address is looked up on
+ * the first call on each device.  The call allocates and frees nothing.
+ * M > HC_GRAD_CHECK_STATIC_MAX_ROWS returns HC_EUNSUPPORTED.  All calls on one
+ * GPU share that array: calls that overlap on one GPU (two streams, two
+ * threads) race; calls on one stream are ordered and safe. */
+#define HC_GRAD_CHECK_STATIC_MAX_ROWS 16777216
+int hc_grad_check_static(const float *grad, const float *score_in, const float *emb,
+                         const int64_t *slot, const int32_t *age, const uint8_t *used,
+                         const int64_t *sub_to_full, const float *thres, int32_t age_limit,
+                         int norm_kind, int cmp_kind, uint8_t *mask_out, float *score_out,
+                         int64_t *slot_out, void *table, int table_dtype, int64_t capacity,
+                         int64_t *full2slot, int64_t *slot2full, int64_t *checkin, int64_t *header,
+                         int64_t glb_iter, int64_t M, int64_t F, void *stream);
+
 /* hc_record_history: the reference's argument set, in its order
  * (grad_check.h:12-16): precomputed score, device threshold, used mask,
  * "not greater" comparison, fp32 table buffer_all[history_num, history_size].
