@@ -68,7 +68,7 @@ int main() {
 
   HC_OK_(hc_aggr_fwd(HC_SUBST_ROW, d_ptr, d_idx, d_x, HC_F32, d_hmap, d_h, HC_F32, F, nullptr, 1, d_out, R, F, N,
                      nullptr, 0, st));
-  HC_OK_(hc_build_transpose(d_ptr, d_idx, d_hmap, R, E, N, d_ptrT, d_rowT, nullptr, d_ws, ws_bytes, st));
+  HC_OK_(hc_build_transpose(d_ptr, d_idx, d_hmap, nullptr, R, E, N, d_ptrT, d_rowT, nullptr, d_ws, ws_bytes, st));
   HC_OK_(hc_aggr_bwd(d_ptr, d_idx, d_ptrT, d_rowT, nullptr, d_g, d_hmap, nullptr, nullptr, HC_F32, 1, d_gx, d_gh, F,
                      nullptr, E, R, F, N, nullptr, 0, st));
   HIP_OK(hipStreamSynchronize(st));

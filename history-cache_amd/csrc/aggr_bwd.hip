@@ -33,66 +33,30 @@ constexpr int BWD_XCD_CHUNK = 64;  // consecutive blocks (8192 sources) that sha
 // With a workspace, a source with more than BWD_CHUNK incoming edges ("hub") is summed in chunks
 // of BWD_CHUNK edges by independent waves; the chunk sums are then combined left to right.
 constexpr int BWD_CHUNK = 512;
+constexpr int W_NONE = 0, W_EDGE = 1, W_EDGE_HEAD = 2;
 
-// Workspace of the hub path.
-struct BwdHubHeader {
-  int n_hubs;
-  int n_chunks;
-  int pad[62];
-};
-struct BwdHubLayout {
-  size_t hub_src, hub_chunk0, chunk_hub, partial, total;
-  int64_t max_hubs, max_chunks;
-};
-inline BwdHubLayout bwd_hub_layout(int64_t E, int64_t F) {
-  BwdHubLayout L;
-  L.max_hubs = E / BWD_CHUNK + 1;          // a hub has more than BWD_CHUNK edges
-  L.max_chunks = E / BWD_CHUNK + L.max_hubs + 1;  // sum of ceil(len/BWD_CHUNK) over hubs
-  size_t off = sizeof(BwdHubHeader);
-  L.hub_src = off;
-  off += hc_align_up((size_t)L.max_hubs * sizeof(int32_t), 256);
-  L.hub_chunk0 = off;
-  off += hc_align_up((size_t)L.max_hubs * sizeof(int32_t), 256);
-  L.chunk_hub = off;
-  off += hc_align_up((size_t)L.max_chunks * sizeof(int32_t), 256);
-  L.partial = off;
-  off += hc_align_up((size_t)L.max_chunks * (size_t)F * sizeof(float), 256);
-  L.total = off;
-  return L;
+// Hubs need no list.  The transposed edge positions are cut into windows of BWD_CHUNK positions and
+// one wave looks at each window.  A hub's chunks start at ptrT[s] + k * BWD_CHUNK, so a window holds at
+// most two chunk starts: one of the hub that covers the window's first position from before (found by
+// a binary search over ptrT) and the first chunk of a hub that starts inside the window (the last
+// source that starts before the window's end, because a hub is longer than a window).  The wave sums
+// those chunks into partial[2 * window] and partial[2 * window + 1].  A second launch, again one wave
+// per window, combines the chunk sums of the hub that starts in its window, left to right.
+inline int64_t bwd_windows(int64_t E) { return (E + BWD_CHUNK - 1) / BWD_CHUNK; }
+inline size_t bwd_partial_bytes(int64_t E, int64_t F) {
+  return hc_align_up((size_t)(2 * bwd_windows(E)) * (size_t)F * sizeof(float), 256);
 }
 
-__global__ void bwd_hub_clear(BwdHubHeader *h) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) {
-    h->n_hubs = 0;
-    h->n_chunks = 0;
+// last s in [0, n_src) with ptrT[s] <= target (ptrT[0] == 0 <= target)
+__device__ __forceinline__ int64_t bwd_last_source_at(const int64_t *__restrict__ ptrT, int64_t n_src,
+                                                      int64_t target) {
+  int64_t lo = 0, hi = n_src - 1;
+  while (lo < hi) {
+    const int64_t mid = (lo + hi + 1) >> 1;
+    if (ptrT[mid] <= target) lo = mid;
+    else hi = mid - 1;
   }
-}
-
-// One thread per source: sources with more than BWD_CHUNK incoming edges take a run of chunk slots.
-// The order in which hubs take their slots only decides where scratch data lives.
-__global__ __launch_bounds__(HC_BLOCK) void bwd_hub_find(const int64_t *__restrict__ ptrT, int64_t n_src,
-                                                          BwdHubHeader *__restrict__ h,
-                                                          int32_t *__restrict__ hub_src,
-                                                          int32_t *__restrict__ hub_chunk0,
-                                                          int32_t *__restrict__ chunk_hub, int64_t max_hubs,
-                                                          int64_t max_chunks) {
-  const int64_t s = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
-  if (s >= n_src) return;
-  const int64_t len = ptrT[s + 1] - ptrT[s];
-  if (len <= BWD_CHUNK) return;
-  const int nch = (int)((len + BWD_CHUNK - 1) / BWD_CHUNK);
-  const int hub = atomicAdd(&h->n_hubs, 1);
-  const int c0 = atomicAdd(&h->n_chunks, nch);
-  // The bounds hold whenever ptrT[n_src] <= E_total (the caller's contract); the guard only keeps
-  // a violated contract from writing outside the workspace.
-  if (hub >= max_hubs || (int64_t)c0 + nch > max_chunks) {
-    if (hub < max_hubs) hub_src[hub] = -1;
-    for (int i = 0; i < nch && (int64_t)c0 + i < max_chunks; ++i) chunk_hub[c0 + i] = -1;
-    return;
-  }
-  hub_src[hub] = (int32_t)s;
-  hub_chunk0[hub] = c0;
-  for (int i = 0; i < nch; ++i) chunk_hub[c0 + i] = hub;
+  return lo;
 }
 
 // Sum of g[r,:]/deg(r) over transposed edges [begin, end), added to acc in order by the calling wave.
@@ -137,62 +101,76 @@ __device__ __forceinline__ void bwd_accumulate(const int64_t *__restrict__ ptr, 
   }
 }
 
-// One wave per chunk slot: the chunk's edges are summed in transposed order into partial[slot].
+// The chunk sums of the window owned by the calling wave (see the note above bwd_windows).
 template <int VEC, int CHUNKS, int UNROLL>
-__global__ __launch_bounds__(HC_BLOCK) void bwd_hub_partial(
-    const int64_t *__restrict__ ptr, const int64_t *__restrict__ ptrT, const int32_t *__restrict__ rowT,
-    const float *__restrict__ g, const BwdHubHeader *__restrict__ h, const int32_t *__restrict__ hub_src,
-    const int32_t *__restrict__ hub_chunk0, const int32_t *__restrict__ chunk_hub,
-    float *__restrict__ partial, int64_t max_chunks) {
+__device__ __forceinline__ void bwd_window_partials(const int64_t *__restrict__ ptr,
+                                                    const int64_t *__restrict__ ptrT,
+                                                    const int32_t *__restrict__ rowT,
+                                                    const float *__restrict__ g, float *__restrict__ partial,
+                                                    int64_t n_src, int64_t window, int lane) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
-  const int lane = hc_lane();
-  const int64_t c = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
-  if (c >= h->n_chunks || c >= max_chunks) return;
-  const int hub = chunk_hub[c];
-  if (hub < 0) return;
-  const int64_t s = hub_src[hub];
-  if (s < 0) return;
-  const int64_t local = c - hub_chunk0[hub];
-  const int64_t begin = ptrT[s] + local * BWD_CHUNK;
-  int64_t end = begin + BWD_CHUNK;
-  const int64_t seg_end = ptrT[s + 1];
-  if (end > seg_end) end = seg_end;
-  float acc[CHUNKS][VEC];
+  const int64_t wstart = window * BWD_CHUNK;
+  const int64_t wend = wstart + BWD_CHUNK;
+  if (wstart >= ptrT[n_src]) return;
+  // lane 0 looks for the source that covers the window's first position, lane 1 for the last source that
+  // starts inside the window; the other lanes repeat lane 1's search
+  const int64_t found = bwd_last_source_at(ptrT, n_src, lane == 0 ? wstart : wend - 1);
+  for (int which = 0; which < 2; ++which) {
+    const int64_t s = hc_readlane64(found, which);
+    const int64_t seg_b = ptrT[s];
+    const int64_t seg_e = ptrT[s + 1];
+    if (seg_e - seg_b <= BWD_CHUNK) continue;
+    int64_t begin;
+    if (which == 0) {
+      if (seg_b >= wstart) continue;                 // it starts inside the window: handled as `which == 1`
+      begin = seg_b + (wstart - seg_b + BWD_CHUNK - 1) / BWD_CHUNK * BWD_CHUNK;
+      if (begin >= wend || begin >= seg_e) continue;
+    } else {
+      if (seg_b < wstart) continue;
+      begin = seg_b;
+    }
+    const int64_t end = begin + BWD_CHUNK < seg_e ? begin + BWD_CHUNK : seg_e;
+    float acc[CHUNKS][VEC];
 #pragma unroll
-  for (int k = 0; k < CHUNKS; ++k)
+    for (int k = 0; k < CHUNKS; ++k)
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
-  bwd_accumulate<VEC, CHUNKS, UNROLL>(ptr, rowT, g, begin, end, lane, acc);
-  float *__restrict__ o = partial + c * F + lane * VEC;
+      for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
+    bwd_accumulate<VEC, CHUNKS, UNROLL>(ptr, rowT, g, begin, end, lane, acc);
+    float *__restrict__ o = partial + (2 * window + which) * F + lane * VEC;
 #pragma unroll
-  for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store(o + k * HC_WAVE * VEC, acc[k]);
+    for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store(o + k * HC_WAVE * VEC, acc[k]);
+  }
 }
 
-// One wave per hub: chunk sums combined left to right into the hub's output row.
+// One wave per window: if a hub starts in the window, its chunk sums are combined left to right into
+// its output row.
 template <int VEC, int CHUNKS>
 __global__ __launch_bounds__(HC_BLOCK) void bwd_hub_final(const int64_t *__restrict__ ptrT,
-                                                           const BwdHubHeader *__restrict__ h,
-                                                           const int32_t *__restrict__ hub_src,
-                                                           const int32_t *__restrict__ hub_chunk0,
                                                            const float *__restrict__ partial,
-                                                           float *__restrict__ grad_vin, int64_t max_hubs) {
+                                                           float *__restrict__ grad_vin, int64_t n_src,
+                                                           int64_t windows) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   const int lane = hc_lane();
-  const int64_t hub = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
-  if (hub >= h->n_hubs || hub >= max_hubs) return;
-  const int64_t s = hub_src[hub];
-  if (s < 0) return;
-  const int64_t len = ptrT[s + 1] - ptrT[s];
+  const int64_t window = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (window >= windows) return;
+  const int64_t wstart = window * BWD_CHUNK;
+  if (wstart >= ptrT[n_src]) return;
+  const int64_t s = hc_uniform64(bwd_last_source_at(ptrT, n_src, wstart + BWD_CHUNK - 1));
+  const int64_t seg_b = ptrT[s];
+  const int64_t len = ptrT[s + 1] - seg_b;
+  if (len <= BWD_CHUNK || seg_b < wstart) return;
   const int nch = (int)((len + BWD_CHUNK - 1) / BWD_CHUNK);
-  const float *__restrict__ p = partial + (int64_t)hub_chunk0[hub] * F + lane * VEC;
   float acc[CHUNKS][VEC];
+  const float *__restrict__ p0 = partial + (2 * window + 1) * F + lane * VEC;
 #pragma unroll
-  for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, acc[k]);
+  for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p0 + k * HC_WAVE * VEC, acc[k]);
   for (int c = 1; c < nch; ++c) {
+    const int64_t w = (seg_b + (int64_t)c * BWD_CHUNK) / BWD_CHUNK;
+    const float *__restrict__ p = partial + (2 * w) * F + lane * VEC;
 #pragma unroll
     for (int k = 0; k < CHUNKS; ++k) {
       float v[VEC];
-      hc_vec<float, VEC>::load(p + (int64_t)c * F + k * HC_WAVE * VEC, v);
+      hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v);
 #pragma unroll
       for (int i = 0; i < VEC; ++i) acc[k][i] += v[i];
     }
@@ -207,18 +185,26 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_hub_final(const int64_t *__restr
 // WMODE W_EDGE_HEAD: a row is n_head heads side by side and the weight is edge_value[edge, head]; a
 // lane's VEC elements of a chunk lie inside one head, whose weight the lane loads itself.  (grad_hbuf
 // of such blocks is written by bwd_hist_generic.)
-constexpr int W_NONE = 0, W_EDGE = 1, W_EDGE_HEAD = 2;
 template <int VEC, int CHUNKS, int UNROLL, int WMODE>
 __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ ptrT, const int32_t *__restrict__ rowT,
     const int32_t *__restrict__ edgeT, const float *__restrict__ ev, int n_head, const float *__restrict__ g,
     const int64_t *__restrict__ hmap, float *__restrict__ grad_vin, float *__restrict__ grad_hbuf,
-    int64_t hsize, int64_t R, int64_t n_src, int64_t src_blocks, int64_t hub_thres) {
+    int64_t hsize, int64_t R, int64_t n_src, int64_t src_blocks, int64_t hist_blocks, int64_t hub_thres,
+    float *__restrict__ partial, int64_t windows) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   constexpr bool WEIGHTED = WMODE != W_NONE;
   constexpr int S = BWD_SRC_PER_WAVE;
   const int lane = hc_lane();
   const int wave = hc_wave_in_block();
+  if ((int64_t)blockIdx.x >= src_blocks + hist_blocks) {
+    // blocks behind the source and history blocks: the hubs' chunk sums, one window per wave
+    if constexpr (WMODE == W_NONE) {
+      const int64_t window = ((int64_t)blockIdx.x - src_blocks - hist_blocks) * HC_WAVES_PER_BLOCK + wave;
+      if (window < windows) bwd_window_partials<VEC, CHUNKS, UNROLL>(ptr, ptrT, rowT, g, partial, n_src, window, lane);
+    }
+    return;
+  }
   if ((int64_t)blockIdx.x >= src_blocks) {
     // grad_hbuf rows: copy g for history rows, zero otherwise
     const int64_t row = ((int64_t)blockIdx.x - src_blocks) * HC_WAVES_PER_BLOCK + wave;
@@ -691,45 +677,33 @@ int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, co
   // rows of several heads: grad_hbuf is written by bwd_hist_generic (the caller launches it)
   const int64_t hb = (grad_hbuf && hmap && n_head == 1) ? (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK : 0;
   if (sb + hb == 0) return HC_OK;
-  if (!hc_grid_ok(sb + hb)) return HC_EUNSUPPORTED;
   int64_t hub_thres = 0;
-  BwdHubLayout L = bwd_hub_layout(E_slots, F);
   char *ws = static_cast<char *>(workspace);
-  // weighted sums keep the strictly sequential order (no hub chunks)
+  // weighted sums keep the strictly sequential order (no hub chunks); a block of up to BWD_CHUNK edge
+  // slots cannot hold a hub
   const bool hubs = ev == nullptr && workspace != nullptr && E_slots > BWD_CHUNK && n_src > 0 &&
-                    workspace_bytes >= L.total && reinterpret_cast<uintptr_t>(ws) % 256 == 0;
-  BwdHubHeader *hh = reinterpret_cast<BwdHubHeader *>(ws);
-  int32_t *hub_src = reinterpret_cast<int32_t *>(ws + L.hub_src);
-  int32_t *hub_chunk0 = reinterpret_cast<int32_t *>(ws + L.hub_chunk0);
-  int32_t *chunk_hub = reinterpret_cast<int32_t *>(ws + L.chunk_hub);
-  float *partial = reinterpret_cast<float *>(ws + L.partial);
-  if (hubs) {
-    hub_thres = BWD_CHUNK;
-    const int64_t fb = (n_src + HC_BLOCK - 1) / HC_BLOCK;
-    const int64_t cb = (L.max_chunks + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
-    if (!hc_grid_ok(fb) || !hc_grid_ok(cb)) return HC_EUNSUPPORTED;
-    bwd_hub_clear<<<dim3(1), dim3(64), 0, st>>>(hh);
-    bwd_hub_find<<<dim3((unsigned)fb), dim3(HC_BLOCK), 0, st>>>(ptrT, n_src, hh, hub_src, hub_chunk0, chunk_hub,
-                                                                L.max_hubs, L.max_chunks);
-    bwd_hub_partial<VEC, CHUNKS, UNROLL><<<dim3((unsigned)cb), dim3(HC_BLOCK), 0, st>>>(
-        ptr, ptrT, rowT, g, hh, hub_src, hub_chunk0, chunk_hub, partial, L.max_chunks);
-    if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
-  }
+                    workspace_bytes >= bwd_partial_bytes(E_slots, F) && reinterpret_cast<uintptr_t>(ws) % 256 == 0;
+  float *partial = reinterpret_cast<float *>(ws);
+  const int64_t windows = hubs ? bwd_windows(E_slots) : 0;
+  const int64_t wb = (windows + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  if (hubs) hub_thres = BWD_CHUNK;
+  if (!hc_grid_ok(sb + hb + wb)) return HC_EUNSUPPORTED;
+  const dim3 grid((unsigned)(sb + hb + wb)), block(HC_BLOCK);
   if (ev != nullptr && n_head > 1)
-    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_EDGE_HEAD><<<dim3((unsigned)(sb + hb)), dim3(HC_BLOCK), 0, st>>>(
-        ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hub_thres);
+    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_EDGE_HEAD><<<grid, block, 0, st>>>(
+        ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hb, hub_thres, partial,
+        windows);
   else if (ev != nullptr)
-    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_EDGE><<<dim3((unsigned)(sb + hb)), dim3(HC_BLOCK), 0, st>>>(
-        ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hub_thres);
+    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_EDGE><<<grid, block, 0, st>>>(
+        ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hb, hub_thres, partial,
+        windows);
   else
-    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_NONE><<<dim3((unsigned)(sb + hb)), dim3(HC_BLOCK), 0, st>>>(
-        ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hub_thres);
+    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_NONE><<<grid, block, 0, st>>>(
+        ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hb, hub_thres, partial,
+        windows);
   if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
   if (hubs) {
-    const int64_t hbk = (L.max_hubs + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
-    if (!hc_grid_ok(hbk)) return HC_EUNSUPPORTED;
-    bwd_hub_final<VEC, CHUNKS><<<dim3((unsigned)hbk), dim3(HC_BLOCK), 0, st>>>(ptrT, hh, hub_src, hub_chunk0,
-                                                                            partial, grad_vin, L.max_hubs);
+    bwd_hub_final<VEC, CHUNKS><<<dim3((unsigned)wb), block, 0, st>>>(ptrT, partial, grad_vin, n_src, windows);
   }
   return hc_launch_status();
 }
@@ -743,7 +717,7 @@ bool bwd_fast_shape(int64_t F) {
 extern "C" size_t hc_aggr_bwd_workspace_bytes(int64_t E_total, int64_t F) {
   if (E_total < 0 || F <= 0) return 0;
   if (!bwd_fast_shape(F) || E_total <= BWD_CHUNK) return 0;
-  return bwd_hub_layout(E_total, F).total;
+  return bwd_partial_bytes(E_total, F);
 }
 
 extern "C" int64_t hc_aggr_bwd_chunk_edges(int64_t F) { return bwd_fast_shape(F) ? BWD_CHUNK : 0; }

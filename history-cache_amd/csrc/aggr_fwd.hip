@@ -17,6 +17,8 @@
 // (the reference truncates neighbour ids and offsets to 32-bit int, :19,34-35).
 #include "hc_common.h"
 
+#include <type_traits>
+
 namespace {
 
 // Rows with more edges than this are summed by the four waves of their block (quarter split).
@@ -65,15 +67,27 @@ __device__ __forceinline__ void copy_row_any(const void *hbuf, int hist_dtype, i
 // n_head heads side by side and every head has its own weight, edge_value[edge, head]; a lane's VEC
 // elements of a chunk lie inside one head (hd[chunk]), whose weight the lane loads itself.
 constexpr int W_NONE = 0, W_EDGE = 1, W_EDGE_HEAD = 2;
-template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM, int WMODE>
+// Per-source substitution.  `bits` (nullable) holds one bit per source, set when the source has an entry in
+// the map: a source whose bit is clear never touches the map, which costs a whole cache line per lookup.
+// TH is the element type of the history table; when it differs from T the staged address carries a tag in
+// its lowest bit (rows are at least 8-byte aligned) and the load of a neighbour row picks the element type
+// from it -- the branch is wave-uniform, as the row address is.
+struct FwdSrc {
+  const int64_t *hmap;    // nullptr: no substitution
+  const void *htab;
+  int64_t hsize;
+  const uint32_t *bits;
+};
+template <typename T, typename TH, int VEC, int CHUNKS, int UNROLL, bool STREAM, int WMODE>
 __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, const T *__restrict__ vin,
-                                               const int64_t *__restrict__ hmap, const T *__restrict__ htab,
-                                               int64_t hsize, int src_mode, const float *__restrict__ ev,
+                                               const FwdSrc src, const float *__restrict__ ev,
                                                int n_head, const int (&hd)[CHUNKS],
                                                int64_t begin, int64_t end, int lane,
                                                float (&acc)[CHUNKS][VEC]) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   constexpr bool WEIGHTED = WMODE != W_NONE;
+  constexpr bool MIXED = !std::is_same<T, TH>::value;
+  const TH *__restrict__ htab = static_cast<const TH *>(src.htab);
   for (int64_t base = begin; base < end; base += HC_WAVE) {
     const int64_t left = end - base;
     const int n = left < HC_WAVE ? (int)left : HC_WAVE;
@@ -82,12 +96,14 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
     float my_w = 0.0f;
     if (lane < n) {
       const int64_t id = STREAM ? __builtin_nontemporal_load(idx + base + lane) : idx[base + lane];
-      const T *p = vin + id * F;
-      if (src_mode && hmap != nullptr) {
-        const int64_t slot = hmap[id];
-        if (slot != -1) p = htab + slot * hsize;
+      my_addr = reinterpret_cast<int64_t>(vin + id * F);
+      if (src.hmap != nullptr) {
+        const bool maybe = src.bits == nullptr || ((src.bits[id >> 5] >> (id & 31)) & 1u) != 0u;
+        if (maybe) {
+          const int64_t slot = src.hmap[id];
+          if (slot != -1) my_addr = reinterpret_cast<int64_t>(htab + slot * src.hsize) | (MIXED ? 1 : 0);
+        }
       }
-      my_addr = reinterpret_cast<int64_t>(p);
       if constexpr (WMODE == W_EDGE) my_w = ev[base + lane];
     }
     for (int j = 0; j < n; j += UNROLL) {
@@ -96,12 +112,22 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         if (j + u < n) {
-          const T *p = reinterpret_cast<const T *>(hc_readlane64(my_addr, j + u)) + lane * VEC;
+          const int64_t a = hc_readlane64(my_addr, j + u);
+          if (MIXED && (a & 1) != 0) {      // a row of the history table, in its own element type
+            const TH *p = reinterpret_cast<const TH *>(a - 1) + lane * VEC;
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) {
+              if constexpr (STREAM) hc_vec<TH, VEC>::load_nt(p + k * HC_WAVE * VEC, v[u][k]);
+              else hc_vec<TH, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
+            }
+          } else {
+          const T *p = reinterpret_cast<const T *>(a) + lane * VEC;
 #pragma unroll
           for (int k = 0; k < CHUNKS; ++k) {
             if constexpr (STREAM) hc_vec<T, VEC>::load_nt(p + k * HC_WAVE * VEC, v[u][k]);
             else hc_vec<T, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
             if constexpr (WMODE == W_EDGE_HEAD) wh[u][k] = ev[(base + j + u) * n_head + hd[k]];
+          }
           }
         } else {
 #pragma unroll
@@ -205,10 +231,9 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_long_find(const int64_t *__restr
 }
 
 // One long row summed by the four waves of the calling block (all of them must call this).
-template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM, int WMODE>
+template <typename T, typename TH, int VEC, int CHUNKS, int UNROLL, bool STREAM, int WMODE>
 __device__ __forceinline__ void fwd_long_row(const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx,
-                                             const T *__restrict__ vin, const int64_t *__restrict__ hmap,
-                                             const T *__restrict__ htab, int64_t hsize, int src_mode,
+                                             const T *__restrict__ vin, const FwdSrc src,
                                              const float *__restrict__ ev, float *__restrict__ vout,
                                              int64_t lrow, int lane, int wave,
                                              float (*part)[HC_WAVE * VEC * CHUNKS]) {
@@ -229,8 +254,7 @@ __device__ __forceinline__ void fwd_long_row(const int64_t *__restrict__ ptr, co
   for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[c][i] = 0.0f;
-  fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM, WMODE>(idx, vin, hmap, htab, hsize, src_mode, ev, 1, no_heads, sb,
-                                                        se, lane, acc);
+  fwd_accumulate<T, TH, VEC, CHUNKS, UNROLL, STREAM, WMODE>(idx, vin, src, ev, 1, no_heads, sb, se, lane, acc);
   if (wave > 0) {
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c)
@@ -262,12 +286,12 @@ __device__ __forceinline__ void fwd_long_row(const int64_t *__restrict__ ptr, co
 // edge_value[E, n_head]); such launches come with long_thres == 0 and no list, so every row is summed
 // strictly in CSR order by its wave, and a history row copies hbuf[r, :hsize] once (hsize == F) or once
 // per head (hsize == F / n_head).
-template <typename T, int VEC, int CHUNKS, int UNROLL, bool STREAM, int WMODE>
+template <typename T, typename TH, int VEC, int CHUNKS, int UNROLL, bool STREAM, int WMODE>
 __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const T *__restrict__ vin,
     const int64_t *__restrict__ hmap, const void *__restrict__ hbuf, int hist_dtype, int64_t hsize,
-    int src_mode, const float *__restrict__ ev, int n_head, float *__restrict__ vout, int64_t R,
-    int64_t long_thres, FwdSched sched) {
+    int src_mode, const uint32_t *__restrict__ src_bits, const float *__restrict__ ev, int n_head,
+    float *__restrict__ vout, int64_t R, int64_t long_thres, FwdSched sched) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   constexpr bool WEIGHTED = WMODE != W_NONE;
   // without heads the rows may be split: the split code is compiled for those modes only
@@ -277,15 +301,15 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
   __shared__ int n_long_s;
   const int lane = hc_lane();
   const int wave = hc_wave_in_block();
-  const T *__restrict__ htab = static_cast<const T *>(hbuf);
+  const FwdSrc src{src_mode ? hmap : nullptr, hbuf, hsize, src_bits};
   // every thread of the grid reads the same two words, so the decision is uniform
   const int n_listed = sched.head != nullptr ? sched.head->count : 0;
   const bool listed = sched.head != nullptr && n_listed <= sched.head->cap;
   if ((int)blockIdx.x < sched.front) {
     if (!listed) return;
     for (int t = (int)blockIdx.x; t < n_listed; t += sched.front)
-      fwd_long_row<T, VEC, CHUNKS, UNROLL, STREAM, LMODE>(ptr, idx, vin, hmap, htab, hsize, src_mode, ev, vout,
-                                                          (int64_t)sched.rows[t], lane, wave, part);
+      fwd_long_row<T, TH, VEC, CHUNKS, UNROLL, STREAM, LMODE>(ptr, idx, vin, src, ev, vout,
+                                                              (int64_t)sched.rows[t], lane, wave, part);
     return;
   }
   const int64_t row0 = hc_xcd_block<FWD_XCD_CHUNK>((int64_t)blockIdx.x - sched.front,
@@ -327,8 +351,8 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
         int hd[CHUNKS];
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) hd[c] = WMODE == W_EDGE_HEAD ? ((c * HC_WAVE + lane) * VEC) / (F / n_head) : 0;
-        fwd_accumulate<T, VEC, CHUNKS, UNROLL, STREAM, WMODE>(idx, vin, hmap, htab, hsize, src_mode, ev, n_head, hd,
-                                                              begin, end, lane, acc);
+        fwd_accumulate<T, TH, VEC, CHUNKS, UNROLL, STREAM, WMODE>(idx, vin, src, ev, n_head, hd, begin, end, lane,
+                                                                  acc);
         const float fdeg = (float)(int)deg;
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) {
@@ -346,8 +370,8 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
   const int n_long = n_long_s;
   // The order in which long rows were noted does not matter: each is summed on its own.
   for (int t = 0; t < n_long; ++t)
-    fwd_long_row<T, VEC, CHUNKS, UNROLL, STREAM, LMODE>(ptr, idx, vin, hmap, htab, hsize, src_mode, ev, vout,
-                                                        row0 + long_rows[t], lane, wave, part);
+    fwd_long_row<T, TH, VEC, CHUNKS, UNROLL, STREAM, LMODE>(ptr, idx, vin, src, ev, vout, row0 + long_rows[t], lane,
+                                                            wave, part);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -379,7 +403,9 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_generic(
   const int64_t end = ptr[row + 1];
   const int64_t deg = end - begin;
   const float fdeg = (float)(int)deg;
-  const T *__restrict__ htab = static_cast<const T *>(hbuf);
+  // per-source substitution may read a table of another element type than vin (hist_dtype)
+  const bool same_type = hist_dtype == (std::is_same<T, float>::value ? HC_F32 : (std::is_same<T, __half>::value ? HC_F16 : HC_BF16));
+  const size_t hesz = hist_dtype == HC_F32 ? 4 : 2;
 
   for (int64_t c0 = 0; c0 < F; c0 += HC_WAVE * TILE_K) {
     float acc[TILE_K];
@@ -389,15 +415,18 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_generic(
       const int64_t left = end - base;
       const int n = left < HC_WAVE ? (int)left : HC_WAVE;
       int64_t my_addr = 0;
+      int my_hist = 0;   // 1: the address is a row of the history table in another element type
       float my_w = 0.0f;
       if (lane < n) {
         const int64_t id = idx[base + lane];
-        const T *p = vin + (id * H + head) * F;
+        my_addr = reinterpret_cast<int64_t>(vin + (id * H + head) * F);
         if (src_mode && hmap != nullptr) {
           const int64_t slot = hmap[id];
-          if (slot != -1) p = htab + slot * hsize;
+          if (slot != -1) {
+            my_addr = reinterpret_cast<int64_t>(static_cast<const char *>(hbuf) + slot * hsize * hesz);
+            my_hist = same_type ? 0 : 1;
+          }
         }
-        my_addr = reinterpret_cast<int64_t>(p);
         if (WEIGHTED) my_w = ev[(base + lane) * H + head];
       }
       // GEN_UNROLL neighbour rows are loaded before the first add; the adds keep the edge order
@@ -411,12 +440,17 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_generic(
 #pragma unroll
           for (int k = 0; k < TILE_K; ++k) x[u][k] = 0.0f;
           if (j + u < n) {
-            const T *p = reinterpret_cast<const T *>(hc_readlane64(my_addr, j + u));
+            const int64_t a = hc_readlane64(my_addr, j + u);
+            const int other = __builtin_amdgcn_readlane(my_hist, j + u);
             w[u] = WEIGHTED ? hc_readlane_f(my_w, j + u) : 1.0f;
 #pragma unroll
             for (int k = 0; k < TILE_K; ++k) {
               const int64_t c = c0 + k * HC_WAVE + lane;
-              if (c < F) x[u][k] = hc_to_f32<T>(p[c]);
+              if (c >= F) continue;
+              if (!other) x[u][k] = hc_to_f32<T>(reinterpret_cast<const T *>(a)[c]);
+              else if (hist_dtype == HC_F32) x[u][k] = reinterpret_cast<const float *>(a)[c];
+              else if (hist_dtype == HC_F16) x[u][k] = __half2float(reinterpret_cast<const __half *>(a)[c]);
+              else x[u][k] = __bfloat162float(reinterpret_cast<const __hip_bfloat16 *>(a)[c]);
             }
           }
         }
@@ -441,25 +475,75 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_generic(
 // extra launches cost more than the list saves.
 constexpr int64_t FWD_LIST_MIN_ROWS = 65536;
 constexpr int FWD_FRONT_BLOCKS = 2048;
+// Source tables below this size go without the one-bit-per-source filter in front of the map lookup:
+// their map (8 bytes per source) stays in the L2s anyway.
+constexpr int64_t FWD_BITS_MIN_SRC = (int64_t)1 << 20;
 
 struct FwdScratch {
   void *ptr;
   size_t bytes;
 };
 
+// Workspace of a forward launch: the long-row list (large blocks), then one bit per source (per-source
+// substitution over many sources).  Either part may be absent (0 bytes).
+struct FwdWsLayout {
+  size_t list_bytes, bits_off, bits_bytes, total;
+};
+FwdWsLayout fwd_ws_layout(int mode, int64_t R, int64_t E, int64_t n_src) {
+  FwdWsLayout L{0, 0, 0, 0};
+  if (R >= FWD_LIST_MIN_ROWS && E > HC_LONG_ROW_EDGES) {
+    // at most E / (HC_LONG_ROW_EDGES + 1) rows can be long
+    int64_t cap = E / (HC_LONG_ROW_EDGES + 1) + 1;
+    if (cap > R) cap = R;
+    L.list_bytes = hc_align_up(sizeof(FwdLongList) + (size_t)cap * sizeof(int), 256);
+  }
+  L.bits_off = L.list_bytes;
+  if (mode == HC_SUBST_SRC && n_src >= FWD_BITS_MIN_SRC) L.bits_bytes = hc_align_up((size_t)((n_src + 63) / 64) * 8, 256);
+  L.total = L.bits_off + L.bits_bytes;
+  return L;
+}
+
+// bits[s] = (hmap[s] != -1), 64 sources per ballot.  The map is read with ordinary loads: this pass also
+// brings it into the last-level cache in front of the launch that looks sources up in it.
+__global__ __launch_bounds__(HC_BLOCK) void fwd_src_bits(const int64_t *__restrict__ hmap, int64_t n_src,
+                                                          unsigned long long *__restrict__ bits) {
+  const int lane = hc_lane();
+  const int64_t stride = (int64_t)gridDim.x * HC_WAVES_PER_BLOCK * HC_WAVE;
+  for (int64_t base = ((int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block()) * HC_WAVE; base < n_src;
+       base += stride) {
+    const bool has = base + lane < n_src && hmap[base + lane] != -1;
+    const unsigned long long b = __ballot(has);
+    if (lane == 0) bits[base / HC_WAVE] = b;
+  }
+}
+
 template <typename T, int VEC, int CHUNKS>
 int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const int64_t *hmap,
                 const void *hbuf, int hist_dtype, int64_t hsize, int src_mode, const float *ev, int n_head,
-                float *vout, int64_t R, FwdScratch ws, hipStream_t st) {
+                float *vout, int64_t R, int64_t n_src, FwdScratch ws, hipStream_t st) {
   constexpr int per = VEC * CHUNKS;
   constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
   int64_t blocks = (R + FWD_ROWS_PER_BLOCK - 1) / FWD_ROWS_PER_BLOCK;
   FwdSched sched{nullptr, nullptr, 0};
   int64_t cap = 0;
   const int64_t long_thres = n_head > 1 ? 0 : (int64_t)HC_LONG_ROW_EDGES;   // rows of several heads are never split
-  if (n_head == 1 && ws.ptr != nullptr && ws.bytes >= sizeof(FwdLongList) + sizeof(int) && R >= FWD_LIST_MIN_ROWS &&
-      R <= 0x7fffffffLL && reinterpret_cast<uintptr_t>(ws.ptr) % 256 == 0) {
-    cap = (int64_t)((ws.bytes - sizeof(FwdLongList)) / sizeof(int));
+  // the caller sized the workspace with hc_aggr_fwd_workspace_bytes(mode, R, E, n_src): the bitmap, when
+  // there is one, takes the last bits_bytes bytes and the list what lies in front of it
+  const uint32_t *src_bits = nullptr;
+  const bool ws_ok = ws.ptr != nullptr && reinterpret_cast<uintptr_t>(ws.ptr) % 256 == 0;
+  size_t list_room = ws_ok ? ws.bytes : 0;
+  if (ws_ok && src_mode && hmap != nullptr && n_src >= FWD_BITS_MIN_SRC) {
+    const size_t bb = hc_align_up((size_t)((n_src + 63) / 64) * 8, 256);
+    if (ws.bytes >= bb) {
+      list_room = (ws.bytes - bb) / 256 * 256;
+      unsigned long long *bits = reinterpret_cast<unsigned long long *>(static_cast<char *>(ws.ptr) + list_room);
+      fwd_src_bits<<<dim3(2048), dim3(HC_BLOCK), 0, st>>>(hmap, n_src, bits);
+      src_bits = reinterpret_cast<const uint32_t *>(bits);
+    }
+  }
+  if (n_head == 1 && list_room >= sizeof(FwdLongList) + sizeof(int) && R >= FWD_LIST_MIN_ROWS &&
+      R <= 0x7fffffffLL) {
+    cap = (int64_t)((list_room - sizeof(FwdLongList)) / sizeof(int));
     if (cap > R) cap = R;
     sched.head = static_cast<FwdLongList *>(ws.ptr);
     sched.rows = reinterpret_cast<int *>(static_cast<char *>(ws.ptr) + sizeof(FwdLongList));
@@ -472,14 +556,18 @@ int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const i
     fwd_long_find<<<dim3((unsigned)((R + FWD_FIND_TILE - 1) / FWD_FIND_TILE)), dim3(HC_BLOCK), 0, st>>>(
         ptr, src_mode ? nullptr : hmap, R, (int64_t)HC_LONG_ROW_EDGES, sched.head, sched.rows);
   }
-#define HC_FWD_LAUNCH(STREAM, WMODE)                                                                   \
-  fwd_mean_fast<T, VEC, CHUNKS, UNROLL, STREAM, WMODE><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>( \
-      ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, ev, n_head, vout, R, \
+#define HC_FWD_LAUNCH(TH, STREAM, WMODE)                                                                   \
+  fwd_mean_fast<T, TH, VEC, CHUNKS, UNROLL, STREAM, WMODE><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>( \
+      ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, src_bits, ev, n_head, vout, R, \
       long_thres, sched)
-  if (ev != nullptr && n_head > 1) HC_FWD_LAUNCH(false, W_EDGE_HEAD);
-  else if (ev != nullptr) HC_FWD_LAUNCH(false, W_EDGE);
-  else if (src_mode && hmap != nullptr) HC_FWD_LAUNCH(true, W_NONE);
-  else HC_FWD_LAUNCH(false, W_NONE);
+  if (ev != nullptr && n_head > 1) HC_FWD_LAUNCH(T, false, W_EDGE_HEAD);
+  else if (ev != nullptr) HC_FWD_LAUNCH(T, false, W_EDGE);
+  else if (src_mode && hmap != nullptr) {
+    // the table of a per-source substitution may be narrower than fp32 features
+    if (std::is_same<T, float>::value && hist_dtype == HC_F16) HC_FWD_LAUNCH(__half, true, W_NONE);
+    else if (std::is_same<T, float>::value && hist_dtype == HC_BF16) HC_FWD_LAUNCH(__hip_bfloat16, true, W_NONE);
+    else HC_FWD_LAUNCH(T, true, W_NONE);
+  } else HC_FWD_LAUNCH(T, false, W_NONE);
 #undef HC_FWD_LAUNCH
   return hc_launch_status();
 }
@@ -488,14 +576,14 @@ int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const i
 template <typename T>
 int dispatch_fast(int64_t F, const int64_t *ptr, const int64_t *idx, const void *vin,
                   const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize, int src_mode,
-                  const float *ev, int n_head, float *vout, int64_t R, FwdScratch ws, hipStream_t st,
-                  bool *handled) {
+                  const float *ev, int n_head, float *vout, int64_t R, int64_t n_src, FwdScratch ws,
+                  hipStream_t st, bool *handled) {
   // F is the whole row (all heads); with several heads a lane's vector must not straddle two of them
   *handled = true;
 #define HC_FAST(V, C)                                                                              \
   if (F == 64 * (V) * (C) && (F / n_head) % (V) == 0)                                              \
-    return launch_fast<T, V, C>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, ev, n_head, vout, R, ws, \
-                                st);
+    return launch_fast<T, V, C>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, ev, n_head, vout, R, n_src, \
+                                ws, st);
   constexpr int VMAX = 16 / (int)sizeof(T);
   if constexpr (VMAX == 8) {
     HC_FAST(8, 1) HC_FAST(8, 2) HC_FAST(8, 3) HC_FAST(8, 4)
@@ -546,12 +634,9 @@ extern "C" int64_t hc_aggr_fwd_long_row_edges(int64_t F, int in_dtype) {
   return fast_shape(F, in_dtype) ? HC_LONG_ROW_EDGES : 0;
 }
 
-extern "C" size_t hc_aggr_fwd_workspace_bytes(int64_t R, int64_t E) {
-  if (R < FWD_LIST_MIN_ROWS || E <= HC_LONG_ROW_EDGES) return 0;
-  // at most E / (HC_LONG_ROW_EDGES + 1) rows can be long
-  int64_t cap = E / (HC_LONG_ROW_EDGES + 1) + 1;
-  if (cap > R) cap = R;
-  return hc_align_up(sizeof(FwdLongList) + (size_t)cap * sizeof(int), 256);
+extern "C" size_t hc_aggr_fwd_workspace_bytes(int mode, int64_t R, int64_t E, int64_t n_src) {
+  if (R < 0 || E < 0 || n_src < 0) return 0;
+  return fwd_ws_layout(mode, R, E, n_src).total;
 }
 
 extern "C" int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, const void *vin,
@@ -573,18 +658,19 @@ extern "C" int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, con
     if (edge_value) return HC_EUNSUPPORTED;
     if (hmap) {
       HC_REQUIRE(hsize >= F);
-      if (hist_dtype != in_dtype) return HC_EUNSUPPORTED;
+      // the table has the features' element type, or the features are fp32 and the table is narrower
+      if (hist_dtype != in_dtype && in_dtype != HC_F32) return HC_EUNSUPPORTED;
     }
   } else if (hmap) {
     HC_REQUIRE(hsize == F * n_head || (hsize >= F && n_head == 1) || hsize == F);
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
 
-  const size_t esz = in_dtype == HC_F32 ? 4 : 2;
+  const size_t hesz = hist_dtype == HC_F32 ? 4 : 2;
   const bool aligned = (reinterpret_cast<uintptr_t>(vin) % 16 == 0) &&
                        (reinterpret_cast<uintptr_t>(vout) % 16 == 0) &&
                        (!src_mode || !hmap ||
-                        ((reinterpret_cast<uintptr_t>(hbuf) % 16 == 0) && ((hsize * esz) % 16 == 0)));
+                        ((reinterpret_cast<uintptr_t>(hbuf) % 16 == 0) && ((hsize * hesz) % 16 == 0)));
   // weighted sums share the fast path; a history row of a weighted block copies hbuf[r, :F].  With several
   // heads the row of the fast path is all heads side by side (F * n_head elements).
   const bool weighted_ok = !edge_value || (!src_mode && (!hmap || hsize >= F));
@@ -595,13 +681,13 @@ extern "C" int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, con
     const int nh = (int)n_head;
     if (in_dtype == HC_F32)
       rc = dispatch_fast<float>(Frow, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value, nh, vout, R,
-                                ws, st, &handled);
+                                n_src, ws, st, &handled);
     else if (in_dtype == HC_F16)
       rc = dispatch_fast<__half>(Frow, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value, nh, vout,
-                                 R, ws, st, &handled);
+                                 R, n_src, ws, st, &handled);
     else
       rc = dispatch_fast<__hip_bfloat16>(Frow, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode,
-                                         edge_value, nh, vout, R, ws, st, &handled);
+                                         edge_value, nh, vout, R, n_src, ws, st, &handled);
     if (handled) return rc;
   }
   if (in_dtype == HC_F32)

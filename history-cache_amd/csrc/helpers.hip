@@ -191,6 +191,38 @@ __global__ __launch_bounds__(HC_BLOCK) void lookup_kernel(const int64_t *__restr
   out[i] = (k >= 0 && k < map_len) ? map[k] : -1;
 }
 
+// Ring-table lookup: slot of every id, entries at least age_limit iterations old count as absent,
+// and the table row of every hit widened to fp32 (zeros for the others).  Wave per id.
+template <typename TT>
+__global__ __launch_bounds__(HC_BLOCK) void ring_lookup_kernel(
+    const int64_t *__restrict__ full2slot, int64_t n_full, const int64_t *__restrict__ ids,
+    const int64_t *__restrict__ checkin, int64_t now, int64_t age_limit, const TT *__restrict__ table,
+    int64_t capacity, int64_t F, int64_t *__restrict__ slot_out, float *__restrict__ rows_out, int64_t n) {
+  constexpr int V = 4;
+  const int lane = hc_lane();
+  const int64_t i = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (i >= n) return;
+  const int64_t id = ids[i];
+  int64_t slot = (id >= 0 && id < n_full) ? full2slot[id] : -1;
+  if (slot < 0 || slot >= capacity) slot = -1;
+  if (slot >= 0 && checkin != nullptr && now - checkin[slot] >= age_limit) slot = -1;
+  if (lane == 0) slot_out[i] = slot;
+  if (rows_out == nullptr) return;
+  float *__restrict__ o = rows_out + i * F;
+  const TT *__restrict__ s = table + (slot >= 0 ? slot : 0) * F;
+  const bool vec_ok = (F % V == 0) && (reinterpret_cast<uintptr_t>(table) % (sizeof(TT) * V) == 0) &&
+                      (reinterpret_cast<uintptr_t>(rows_out) % 16 == 0);
+  if (vec_ok) {
+    for (int64_t c = (int64_t)lane * V; c < F; c += HC_WAVE * V) {
+      float v[V] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (slot >= 0) hc_vec<TT, V>::load(s + c, v);
+      hc_vec<float, V>::store(o + c, v);
+    }
+  } else {
+    for (int64_t c = lane; c < F; c += HC_WAVE) o[c] = slot >= 0 ? hc_to_f32<TT>(s[c]) : 0.0f;
+  }
+}
+
 inline unsigned blocks_for(int64_t n) { return (unsigned)((n + HC_BLOCK - 1) / HC_BLOCK); }
 
 }  // namespace
@@ -384,5 +416,31 @@ extern "C" int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids
   if (!hc_grid_ok((n + HC_BLOCK - 1) / HC_BLOCK)) return HC_EUNSUPPORTED;
   lookup_kernel<<<dim3(blocks_for(n)), dim3(HC_BLOCK), 0, static_cast<hipStream_t>(stream)>>>(
       map, map_len, ids, offset, out, n);
+  return hc_launch_status();
+}
+
+extern "C" int hc_ring_lookup(const int64_t *full2slot, int64_t n_full, const int64_t *ids,
+                              const int64_t *checkin, int64_t now, int64_t age_limit, const void *table,
+                              int table_dtype, int64_t capacity, int64_t F, int64_t *slot_out,
+                              float *rows_out, int64_t n, void *stream) {
+  HC_REQUIRE(n >= 0 && n_full >= 0 && capacity >= 0 && F > 0);
+  if (table_dtype < HC_F32 || table_dtype > HC_BF16) return HC_EDTYPE;
+  if (n == 0) return HC_OK;
+  HC_REQUIRE(full2slot && ids && slot_out);
+  HC_REQUIRE(rows_out == nullptr || table != nullptr);
+  const int64_t b = (n + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  if (!hc_grid_ok(b)) return HC_EUNSUPPORTED;
+  dim3 g((unsigned)b), bl(HC_BLOCK);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (table_dtype == HC_F32)
+    ring_lookup_kernel<float><<<g, bl, 0, st>>>(full2slot, n_full, ids, checkin, now, age_limit,
+                                                static_cast<const float *>(table), capacity, F, slot_out, rows_out, n);
+  else if (table_dtype == HC_F16)
+    ring_lookup_kernel<__half><<<g, bl, 0, st>>>(full2slot, n_full, ids, checkin, now, age_limit,
+                                                 static_cast<const __half *>(table), capacity, F, slot_out, rows_out, n);
+  else
+    ring_lookup_kernel<__hip_bfloat16><<<g, bl, 0, st>>>(full2slot, n_full, ids, checkin, now, age_limit,
+                                                         static_cast<const __hip_bfloat16 *>(table), capacity, F,
+                                                         slot_out, rows_out, n);
   return hc_launch_status();
 }

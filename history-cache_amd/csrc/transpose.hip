@@ -51,6 +51,8 @@ template <bool VAL_IS_ROW, int TR_ITEMS>
 __global__ __launch_bounds__(HC_BLOCK) void tr_expand_edges(const int64_t *__restrict__ ptr,
                                                              const int64_t *__restrict__ idx,
                                                              const int64_t *__restrict__ hmap_row,
+                                                             const int64_t *__restrict__ hmap_src,
+                                                             const uint32_t *__restrict__ src_bits,
                                                              uint32_t *__restrict__ keys,
                                                              uint32_t *__restrict__ vals,
                                                              uint32_t *__restrict__ rows, int64_t R, int64_t E,
@@ -100,6 +102,24 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_expand_edges(const int64_t *__res
   for (int it = 0; it < TR_ITEMS; ++it) {
     const int64_t e = e0 + (int64_t)it * HC_BLOCK + threadIdx.x;
     src[it] = live[it] ? idx[e] : -1;
+  }
+  if (hmap_src != nullptr) {   // sources that were substituted in the forward pass receive no gradient
+    // src_bits (one bit per source, derived from the map by tr_src_bits) answers the question without
+    // touching the map, which costs a cache line per lookup when the sources are many
+    bool sub[TR_ITEMS];
+#pragma unroll
+    for (int it = 0; it < TR_ITEMS; ++it) {
+      sub[it] = false;
+      if (src[it] >= 0 && src[it] < n_src)
+        sub[it] = src_bits != nullptr ? ((src_bits[src[it] >> 5] >> (src[it] & 31)) & 1u) != 0u
+                                      : hmap_src[src[it]] != -1;
+    }
+#pragma unroll
+    for (int it = 0; it < TR_ITEMS; ++it)
+      if (sub[it]) {
+        src[it] = -1;
+        live[it] = false;
+      }
   }
 #pragma unroll
   for (int it = 0; it < TR_ITEMS; ++it) {
@@ -196,6 +216,260 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_finalize_ptr(const uint32_t *__re
   ptrT[s] = lo;
 }
 
+// ---------------------------------------------------------------------------------------
+// Small blocks (sampled mini-batches: at most TR_SMALL_EDGES edge slots and TR_SMALL_SOURCES sources):
+// a counting sort in four launches of this file's own kernels instead of the library sort's dozen.
+//   tr_small_clear  zero the per-source counters and the ticket
+//   tr_small_count  thread per edge slot: the slot's key (source id, or the sentinel for a dropped
+//                   slot) and destination row are saved and the source's counter is bumped (integer
+//                   atomics: the final counts do not depend on their order); the block that finishes
+//                   last turns the counters into ptrT (exclusive scan) and into per-source cursors
+//   tr_small_place  thread per edge slot: takes the next free position of its source's segment
+//                   (atomic: WHICH slots a segment holds is fixed, their order inside it is not yet)
+//                   and writes (row, slot) there, into temporary arrays
+//   tr_small_order  copies every segment to its final place in ascending slot order -- the order a
+//                   stable sort gives: one-edge segments as they are, segments of up to 64 edges
+//                   ranked inside a wave, longer ones by the whole block through a bitmap of the
+//                   segment's slots in LDS (rank = number of set bits below the slot)
+// The result is bit-identical to the sorted view of the large-block path.
+// ---------------------------------------------------------------------------------------
+constexpr int TRS_BLOCK = 1024;
+constexpr int64_t TR_SMALL_SOURCES = 1 << 20;
+constexpr int TRS_BITMAP_WORDS = (int)(TR_SMALL_EDGES / 32);   // one bit per edge slot
+constexpr int TRS_ORDER_SOURCES = HC_BLOCK;                     // sources per block of tr_small_order
+
+struct TrSmallHeader {
+  unsigned ticket;
+  unsigned pad[63];
+};
+
+__global__ __launch_bounds__(HC_BLOCK) void tr_small_clear(uint32_t *__restrict__ p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+__device__ __forceinline__ int trs_load(const int *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
+    const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const int64_t *__restrict__ hmap_row,
+    const int64_t *__restrict__ hmap_src, uint32_t *__restrict__ keys, int32_t *__restrict__ rows,
+    int *__restrict__ count, TrSmallHeader *__restrict__ header, int64_t *__restrict__ ptrT, int64_t R,
+    int64_t E, int64_t n_src) {
+  __shared__ int64_t s_ptr[TR_LDS_ROWS];
+  __shared__ int64_t s_range[2];
+  __shared__ int s_wave[TRS_BLOCK / HC_WAVE];
+  __shared__ int s_last;
+  const int64_t e0 = (int64_t)blockIdx.x * TRS_BLOCK;
+  const int64_t e1 = e0 + TRS_BLOCK < E ? e0 + TRS_BLOCK : E;
+  if (threadIdx.x < 2) s_range[threadIdx.x] = tr_row_of(ptr, (int64_t)0, R, threadIdx.x == 0 ? e0 : e1 - 1);
+  __syncthreads();
+  const int64_t r_lo = s_range[0], r_hi = s_range[1];
+  const int64_t span = r_hi - r_lo + 1;
+  const bool staged = span <= TR_LDS_ROWS;
+  if (staged)
+    for (int64_t i = threadIdx.x; i < span; i += TRS_BLOCK) s_ptr[i] = ptr[r_lo + i];
+  __syncthreads();
+  const int64_t e = e0 + threadIdx.x;
+  if (e < e1) {
+    int64_t row;
+    bool live;
+    if (staged) {
+      const int64_t l = tr_row_of(s_ptr, (int64_t)0, span - 1, e);
+      row = r_lo + l;
+      live = row < R && s_ptr[l] <= e;
+    } else {
+      row = tr_row_of(ptr, r_lo, r_hi, e);
+      live = row < R && ptr[row] <= e;
+    }
+    if (live && hmap_row != nullptr) live = hmap_row[row] == -1;
+    int64_t src = live ? idx[e] : -1;
+    if (src < 0 || src >= n_src) live = false;
+    if (live && hmap_src != nullptr) live = hmap_src[src] == -1;
+    keys[e] = live ? (uint32_t)src : (uint32_t)n_src;
+    rows[e] = live ? (int32_t)row : -1;
+    if (live) atomicAdd(count + src, 1);
+  }
+  // the block that takes the last ticket sees every block's counts
+  __threadfence();
+  __syncthreads();
+  if (threadIdx.x == 0) s_last = atomicAdd(&header->ticket, 1u) == gridDim.x - 1 ? 1 : 0;
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
+  // exclusive scan of count[0, n_src): thread t owns a contiguous run of sources
+  const int64_t per = (n_src + TRS_BLOCK - 1) / TRS_BLOCK;
+  int64_t lo = (int64_t)threadIdx.x * per;
+  int64_t hi = lo + per;
+  if (lo > n_src) lo = n_src;
+  if (hi > n_src) hi = n_src;
+  int sum = 0;
+  for (int64_t q = lo; q < hi; ++q) sum += trs_load(count + q);
+  const int lane = hc_lane();
+  const int wave = (int)(threadIdx.x >> 6);
+  int x = sum;
+#pragma unroll
+  for (int d = 1; d < HC_WAVE; d <<= 1) {
+    const int y = __shfl_up(x, d, HC_WAVE);
+    if (lane >= d) x += y;
+  }
+  if (lane == HC_WAVE - 1) s_wave[wave] = x;
+  __syncthreads();
+  int off = x - sum;
+  for (int w = 0; w < wave; ++w) off += s_wave[w];
+  int run = off;
+  for (int64_t q = lo; q < hi; ++q) {
+    const int c = trs_load(count + q);
+    ptrT[q] = run;
+    count[q] = run;   // the segment's cursor for tr_small_place
+    run += c;
+  }
+  if (threadIdx.x == TRS_BLOCK - 1) ptrT[n_src] = run;
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void tr_small_place(const uint32_t *__restrict__ keys,
+                                                            const int32_t *__restrict__ rows,
+                                                            int *__restrict__ cursor,
+                                                            int32_t *__restrict__ tmp_row,
+                                                            int32_t *__restrict__ tmp_edge, int64_t E,
+                                                            uint32_t sentinel) {
+  const int64_t e = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  if (e >= E) return;
+  const uint32_t k = keys[e];
+  if (k == sentinel) return;
+  const int p = atomicAdd(cursor + k, 1);
+  tmp_row[p] = rows[e];
+  tmp_edge[p] = (int32_t)e;
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void tr_small_order(const int64_t *__restrict__ ptrT,
+                                                            const int32_t *__restrict__ tmp_row,
+                                                            const int32_t *__restrict__ tmp_edge,
+                                                            int32_t *__restrict__ rowT,
+                                                            int32_t *__restrict__ edgeT, int64_t n_src,
+                                                            int64_t E) {
+  __shared__ uint32_t bits[TRS_BITMAP_WORDS];
+  __shared__ int pre8[TRS_BITMAP_WORDS / 8];
+  __shared__ int long_src[TRS_ORDER_SOURCES];
+  __shared__ int n_long_s;
+  __shared__ int s_wave[HC_WAVES_PER_BLOCK];
+  const int lane = hc_lane();
+  const int wave = hc_wave_in_block();
+  if (threadIdx.x == 0) n_long_s = 0;
+  __syncthreads();
+  const int64_t s = (int64_t)blockIdx.x * TRS_ORDER_SOURCES + threadIdx.x;
+  int64_t b = 0;
+  int len = 0;
+  if (s < n_src) {
+    b = ptrT[s];
+    len = (int)(ptrT[s + 1] - b);
+  }
+  if (len == 1) {
+    rowT[b] = tmp_row[b];
+    if (edgeT != nullptr) edgeT[b] = tmp_edge[b];
+  }
+  if (len > HC_WAVE) long_src[atomicAdd(&n_long_s, 1)] = (int)threadIdx.x;
+  // segments of 2..64 edges: ranked inside the wave, one segment at a time
+  unsigned long long m = __ballot(len >= 2 && len <= HC_WAVE);
+  while (m != 0ull) {
+    const int l = __builtin_ctzll(m);
+    m &= m - 1ull;
+    const int64_t sb = hc_readlane64(b, l);
+    const int sl = __builtin_amdgcn_readlane(len, l);
+    const bool have = lane < sl;
+    const int ve = have ? tmp_edge[sb + lane] : 0x7fffffff;
+    const int vr = have ? tmp_row[sb + lane] : 0;
+    int rank = 0;
+    for (int j = 0; j < sl; ++j) rank += __builtin_amdgcn_readlane(ve, j) < ve ? 1 : 0;   // slots are distinct
+    if (have) {
+      rowT[sb + rank] = vr;
+      if (edgeT != nullptr) edgeT[sb + rank] = ve;
+    }
+  }
+  __syncthreads();
+  // longer segments: the whole block, one segment at a time.  The segment's slots set their bits in an
+  // LDS bitmap over all edge slots; a slot's rank is the number of set bits below it.
+  const int n_long = n_long_s;
+  const int words = (int)((E + 31) / 32);
+  for (int t = 0; t < n_long; ++t) {
+    const int64_t src = (int64_t)blockIdx.x * TRS_ORDER_SOURCES + long_src[t];
+    const int64_t sb = ptrT[src];
+    const int sl = (int)(ptrT[src + 1] - sb);
+    for (int w = threadIdx.x; w < words; w += HC_BLOCK) bits[w] = 0u;
+    __syncthreads();
+    for (int i = threadIdx.x; i < sl; i += HC_BLOCK) {
+      const int e = tmp_edge[sb + i];
+      atomicOr(&bits[e >> 5], 1u << (e & 31));
+    }
+    __syncthreads();
+    // pre8[g] = set bits in front of word group g (8 words): per-thread run of groups, block scan
+    const int groups = (words + 7) / 8;
+    const int per = (groups + HC_BLOCK - 1) / HC_BLOCK;
+    int glo = (int)threadIdx.x * per, ghi = glo + per;
+    if (glo > groups) glo = groups;
+    if (ghi > groups) ghi = groups;
+    int sum = 0;
+    for (int g = glo; g < ghi; ++g)
+      for (int w = g * 8; w < g * 8 + 8 && w < words; ++w) sum += __popc(bits[w]);
+    int x = sum;
+#pragma unroll
+    for (int d = 1; d < HC_WAVE; d <<= 1) {
+      const int y = __shfl_up(x, d, HC_WAVE);
+      if (lane >= d) x += y;
+    }
+    if (lane == HC_WAVE - 1) s_wave[wave] = x;
+    __syncthreads();
+    int run = x - sum;
+    for (int w = 0; w < wave; ++w) run += s_wave[w];
+    for (int g = glo; g < ghi; ++g) {
+      pre8[g] = run;
+      for (int w = g * 8; w < g * 8 + 8 && w < words; ++w) run += __popc(bits[w]);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < sl; i += HC_BLOCK) {
+      const int e = tmp_edge[sb + i];
+      const int r = tmp_row[sb + i];
+      const int w = e >> 5;
+      int rank = pre8[w >> 3];
+      for (int q = (w >> 3) * 8; q < w; ++q) rank += __popc(bits[q]);
+      rank += __popc(bits[w] & ((1u << (e & 31)) - 1u));
+      rowT[sb + rank] = r;
+      if (edgeT != nullptr) edgeT[sb + rank] = e;
+    }
+    __syncthreads();
+  }
+}
+
+struct SmallLayout {
+  size_t count, keys, rows, tmp_row, tmp_edge, total;
+};
+SmallLayout small_layout(int64_t E, int64_t n_src) {
+  SmallLayout L;
+  const size_t arr = hc_align_up((size_t)(E > 0 ? E : 1) * sizeof(uint32_t), 256);
+  L.count = sizeof(TrSmallHeader);
+  L.keys = L.count + hc_align_up((size_t)(n_src + 1) * sizeof(int), 256);
+  L.rows = L.keys + arr;
+  L.tmp_row = L.rows + arr;
+  L.tmp_edge = L.tmp_row + arr;
+  L.total = L.tmp_edge + arr;
+  return L;
+}
+inline bool small_block(int64_t E, int64_t n_src) { return E <= TR_SMALL_EDGES && n_src <= TR_SMALL_SOURCES; }
+
+// bits[s] = (hmap_src[s] != -1), 64 sources per ballot
+__global__ __launch_bounds__(HC_BLOCK) void tr_src_bits(const int64_t *__restrict__ hmap, int64_t n_src,
+                                                         unsigned long long *__restrict__ bits) {
+  const int lane = hc_lane();
+  const int64_t stride = (int64_t)gridDim.x * HC_WAVES_PER_BLOCK * HC_WAVE;
+  for (int64_t base = ((int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block()) * HC_WAVE; base < n_src;
+       base += stride) {
+    const bool has = base + lane < n_src && hmap[base + lane] != -1;
+    const unsigned long long bal = __ballot(has);
+    if (lane == 0) bits[base / HC_WAVE] = bal;
+  }
+}
+
 int key_bits(int64_t n_src) {
   int b = 1;
   while (b < 32 && ((int64_t)1 << b) <= n_src) ++b;
@@ -203,7 +477,7 @@ int key_bits(int64_t n_src) {
 }
 
 struct Layout {
-  size_t keys0, keys1, vals0, vals1, rows, temp, total;
+  size_t keys0, keys1, vals0, vals1, rows, bits, temp, total;
 };
 
 hipError_t sort_temp_bytes(int64_t E, int bits, size_t *bytes) {
@@ -222,8 +496,9 @@ bool make_layout(int64_t E, int64_t n_src, Layout *L) {
   L->vals0 = 2 * arr;
   L->vals1 = 3 * arr;
   L->rows = 4 * arr;
-  L->temp = 5 * arr;
-  L->total = 5 * arr + hc_align_up(temp > 0 ? temp : 1, 256);
+  L->bits = 5 * arr;   // one bit per source (used when a source map is given)
+  L->temp = L->bits + hc_align_up((size_t)((n_src + 63) / 64) * 8 + 8, 256);
+  L->total = L->temp + hc_align_up(temp > 0 ? temp : 1, 256);
   return true;
 }
 
@@ -232,13 +507,15 @@ bool make_layout(int64_t E, int64_t n_src, Layout *L) {
 extern "C" size_t hc_transpose_workspace_bytes(int64_t R, int64_t E, int64_t n_src) {
   (void)R;
   if (E < 0 || n_src < 0) return 0;
+  if (small_block(E, n_src)) return small_layout(E, n_src).total;   // no library query on this path
   Layout L;
   if (!make_layout(E, n_src, &L)) return 0;
   return L.total;
 }
 
 extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row,
-                                  int64_t R, int64_t E, int64_t n_src, int64_t *ptrT, int32_t *rowT,
+                                  const int64_t *hmap_src, int64_t R, int64_t E, int64_t n_src, int64_t *ptrT,
+                                  int32_t *rowT,
                                   int32_t *edgeT, void *workspace, size_t workspace_bytes,
                                   void *stream) {
   HC_REQUIRE(R >= 0 && E >= 0 && n_src >= 0 && ptrT);
@@ -252,6 +529,29 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
     return hc_launch_status();
   }
   HC_REQUIRE(ptr && idx && rowT);
+  if (small_block(E, n_src)) {
+    const SmallLayout S = small_layout(E, n_src);
+    if (!workspace || workspace_bytes < S.total) return HC_EWORKSPACE;
+    char *w = static_cast<char *>(workspace);
+    if (reinterpret_cast<uintptr_t>(w) % 256 != 0) return HC_EWORKSPACE;
+    TrSmallHeader *header = reinterpret_cast<TrSmallHeader *>(w);
+    int *count = reinterpret_cast<int *>(w + S.count);
+    uint32_t *keys = reinterpret_cast<uint32_t *>(w + S.keys);
+    int32_t *rows = reinterpret_cast<int32_t *>(w + S.rows);
+    int32_t *tmp_row = reinterpret_cast<int32_t *>(w + S.tmp_row);
+    int32_t *tmp_edge = reinterpret_cast<int32_t *>(w + S.tmp_edge);
+    const int64_t clear_words = (int64_t)(S.keys / sizeof(uint32_t));   // header + counters
+    tr_small_clear<<<dim3((unsigned)((clear_words + HC_BLOCK - 1) / HC_BLOCK)), dim3(HC_BLOCK), 0, st>>>(
+        reinterpret_cast<uint32_t *>(w), clear_words);
+    tr_small_count<<<dim3((unsigned)((E + TRS_BLOCK - 1) / TRS_BLOCK)), dim3(TRS_BLOCK), 0, st>>>(
+        ptr, idx, hmap_row, hmap_src, keys, rows, count, header, ptrT, R, E, n_src);
+    tr_small_place<<<dim3((unsigned)((E + HC_BLOCK - 1) / HC_BLOCK)), dim3(HC_BLOCK), 0, st>>>(
+        keys, rows, count, tmp_row, tmp_edge, E, (uint32_t)n_src);
+    if (n_src > 0)
+      tr_small_order<<<dim3((unsigned)((n_src + TRS_ORDER_SOURCES - 1) / TRS_ORDER_SOURCES)), dim3(HC_BLOCK), 0, st>>>(
+          ptrT, tmp_row, tmp_edge, rowT, edgeT, n_src, E);
+    return hc_launch_status();
+  }
   if (E > TR_SORT_MEMSET_EDGES) {
     // Above this size the sort library takes its one-sweep path, which clears its counters with
     // hipMemsetAsync; a captured graph would replay those as memset nodes.  Refuse instead.
@@ -275,6 +575,12 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
   void *temp = ws + L.temp;
   size_t temp_bytes = L.total - L.temp;
   const uint32_t sentinel = (uint32_t)n_src;
+  const uint32_t *src_bits = nullptr;
+  if (hmap_src != nullptr && n_src >= ((int64_t)1 << 20)) {
+    unsigned long long *bits = reinterpret_cast<unsigned long long *>(ws + L.bits);
+    tr_src_bits<<<dim3(2048), dim3(HC_BLOCK), 0, st>>>(hmap_src, n_src, bits);
+    src_bits = reinterpret_cast<const uint32_t *>(bits);
+  }
 
   const int64_t eblocks = (E + HC_BLOCK - 1) / HC_BLOCK;
   const int64_t rblocks = (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
@@ -288,10 +594,10 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
   const dim3 tgrid((unsigned)((E + tile - 1) / tile));
   if (want_edges) {
     if (items == 1)
-      tr_expand_edges<false, 1><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, rows, R, E, n_src);
+      tr_expand_edges<false, 1><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, src_bits, keys0, vals0, rows, R, E, n_src);
     else
-      tr_expand_edges<false, TR_ITEMS_LARGE><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, rows,
-                                                                               R, E, n_src);
+      tr_expand_edges<false, TR_ITEMS_LARGE><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, src_bits, keys0,
+                                                                               vals0, rows, R, E, n_src);
     rocprim::double_buffer<uint32_t> dk(keys0, keys1), dv(vals0, vals1);
     if (rocprim::radix_sort_pairs(temp, temp_bytes, dk, dv, (size_t)E, 0u, bits, st, false) != hipSuccess)
       return HC_ELAUNCH;
@@ -301,10 +607,10 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
   } else {
     // value = destination row; dropped edge slots keep the fill value and sort behind the sentinel
     if (items == 1)
-      tr_expand_edges<true, 1><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, nullptr, R, E, n_src);
+      tr_expand_edges<true, 1><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, src_bits, keys0, vals0, nullptr, R, E, n_src);
     else
-      tr_expand_edges<true, TR_ITEMS_LARGE><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, keys0, vals0, nullptr,
-                                                                              R, E, n_src);
+      tr_expand_edges<true, TR_ITEMS_LARGE><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, src_bits, keys0,
+                                                                              vals0, nullptr, R, E, n_src);
     // rowT doubles as the sort's second value buffer; copy only if the result landed in the first
     uint32_t *rowT_u = reinterpret_cast<uint32_t *>(rowT);
     rocprim::double_buffer<uint32_t> dk(keys0, keys1), dv(vals0, rowT_u);

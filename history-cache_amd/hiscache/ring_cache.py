@@ -11,6 +11,12 @@ ring of ``HistoryTable`` (/root/reference/hiscache/history_table.py:127-200, ker
 the threshold and it is either not cached or its entry is at least ``age_limit`` iterations old;
 admitted rows overwrite the ring in row order.  Norms, test, mask, slot assignment, the
 fp32 -> table-dtype row copy and the map updates are one ``hiscache_backend.grad_check`` call.
+
+The age bound is applied at LOOKUP: an entry that is ``age_limit`` iterations old is reported as
+absent, so the model recomputes that row from its neighbours and the admission pass may then store
+the fresh value (the reference un-maps old slots for the same effect,
+/root/reference/hiscache/history_table.py:189-200).  A row that was served from the table is never
+re-admitted: what it would store is the cached value itself.
 """
 import torch
 
@@ -57,23 +63,22 @@ class RingHistoryCache:
             num_layer = self.num_layers_all
         sub_to_full = batch.sub_to_full
         n1 = int(batch.num_node_in_layer[1])
-        self.sub2embed = _be.lookup(self.full2slot, sub_to_full[:n1], 0)
+        self.glb_iter += 1
+        # slots (stale entries count as absent) and the cached rows of the hits, one launch
+        self.sub2embed, self.cached_embedding = _be.ring_lookup(
+            self.full2slot, sub_to_full[:n1], self.table, checkin=self.checkin, now=self.glb_iter,
+            age_limit=self.age_limit)
         self.used_masks = _be.count_history_reconstruct(batch.ptr, batch.idx, self.sub2embed,
                                                         sub_to_full.shape[0], batch.y.shape[0], num_layer)
-        self.glb_iter += 1
         handle = getattr(batch, "prefetched_x", None)
         if handle is not None and handle.ids is sub_to_full:
             # every row was read ahead of time (``prefetch``): zero the rows the cache makes unnecessary
             batch.prefetched_x = None
             x = self.uvm.take(handle)
             x.masked_fill_(~self.used_masks[0][:, None], 0)
-            self.cached_embedding = _be.gather_rows(self.table, self.sub2embed)
             batch.x = x
             return None
-        x = self.uvm.masked_get(sub_to_full, self.used_masks[0])
-        # rows without a slot (-1) read the last table row and are ignored by the aggregation
-        self.cached_embedding = _be.gather_rows(self.table, self.sub2embed)
-        batch.x = x
+        batch.x = self.uvm.masked_get(sub_to_full, self.used_masks[0])
         return None
 
     def prefetch(self, batch):
@@ -90,27 +95,31 @@ class RingHistoryCache:
             raise AssertionError("produced embedding is None")
         n1 = emb.shape[0]
         slot = self.sub2embed
-        # age of the cached entry, in iterations (0 for rows without an entry)
-        age = (glb_iter - self.checkin[slot.clamp(min=0)]).to(torch.int32)
+        if slot is None or slot.numel() != n1:
+            raise ValueError("produced_embedding has %d rows but the last lookup covered %d 1-hop nodes"
+                             % (n1, -1 if slot is None else slot.numel()))
         sub_to_full = batch.sub_to_full[:n1].contiguous()
+        # rows with a slot were served from the table (stale entries were reported absent at lookup):
+        # only rows that were computed in this iteration can be admitted, so no age is passed
+        common = dict(checkin=self.checkin)
         if self.method == "grad" and emb.grad is not None:
             grad = emb.grad.contiguous()
             if self.thres is not None:
                 mask, score = _be.grad_check(grad, emb.detach().contiguous(), slot, sub_to_full, self.thres,
                                              self.table, self.full2slot, self.slot2full, self._header, glb_iter,
-                                             age=age, age_limit=self.age_limit, checkin=self.checkin)
+                                             **common)
             else:
                 score = _be.row_scores(grad)
                 thres = quantile_threshold(score, self.rate)
                 mask, _ = _be.grad_check(None, emb.detach().contiguous(), slot, sub_to_full, thres, self.table,
-                                         self.full2slot, self.slot2full, self._header, glb_iter, age=age,
-                                         age_limit=self.age_limit, checkin=self.checkin, score=score)
+                                         self.full2slot, self.slot2full, self._header, glb_iter, score=score,
+                                         **common)
         else:
             score = torch.randn([n1], device=self.device)
             thres = quantile_threshold(score, self.rate)
             mask, _ = _be.grad_check(None, emb.detach().contiguous(), slot, sub_to_full, thres, self.table,
-                                     self.full2slot, self.slot2full, self._header, glb_iter, age=age,
-                                     age_limit=self.age_limit, checkin=self.checkin, score=score)
+                                     self.full2slot, self.slot2full, self._header, glb_iter, score=score,
+                                     **common)
         emb.grad = None
         self.last_record_mask = mask
         self.last_score = score

@@ -47,12 +47,12 @@ _SIGNATURES = {
     "hc_version": (ctypes.c_char_p, []),
     "hc_strerror": (ctypes.c_char_p, [_c_int]),
     "hc_device_count": (_c_int, []),
-    "hc_aggr_fwd_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
+    "hc_aggr_fwd_workspace_bytes": (_c_sz, [_c_int, _c_i64, _c_i64, _c_i64]),
     "hc_aggr_fwd": (_c_int, [_c_int, _c_p, _c_p, _c_p, _c_int, _c_p, _c_p, _c_int, _c_i64, _c_p, _c_i64,
                              _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]),
     "hc_aggr_fwd_long_row_edges": (_c_i64, [_c_i64, _c_int]),
     "hc_transpose_workspace_bytes": (_c_sz, [_c_i64, _c_i64, _c_i64]),
-    "hc_build_transpose": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p,
+    "hc_build_transpose": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p,
                                     _c_sz, _c_p]),
     "hc_aggr_bwd_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
     "hc_aggr_bwd_chunk_edges": (_c_i64, [_c_i64]),
@@ -75,6 +75,8 @@ _SIGNATURES = {
     "hc_structure_score": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p]),
     "hc_gather_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p]),
+    "hc_ring_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_int, _c_i64, _c_i64, _c_p, _c_p,
+                                _c_i64, _c_p]),
     "hc_check_csr": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p]),
     "hc_evict": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p]),
     "hc_sample_capacity": (_c_int, [_c_i64, _c_p, _c_int, _c_i64, _c_p, _c_p, _c_p]),
@@ -211,7 +213,7 @@ def _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, num_node):
     out_shape = (R, F) if n_head == 1 and x.dim() == 2 else (R, n_head, F)
     out = torch.empty(out_shape, dtype=torch.float32, device=x.device)
     # scratch for the long-row list (large blocks only: the library reports 0 bytes otherwise)
-    ws_bytes = int(lib.hc_aggr_fwd_workspace_bytes(R, idx.numel())) if n_head == 1 else 0
+    ws_bytes = int(lib.hc_aggr_fwd_workspace_bytes(mode, R, idx.numel(), n_src)) if n_head == 1 else 0
     ws = _workspace(ws_bytes, x.device) if ws_bytes > 0 else None
     rc = lib.hc_aggr_fwd(mode, _ptr(ptr), _ptr(idx), _ptr(x), _float_dtype(x, "input"),
                          _ptr(hmap), _ptr(hbuf), _float_dtype(hbuf, "history_buffer") if hmap is not None else 0,
@@ -221,11 +223,14 @@ def _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, num_node):
     return out
 
 
-def build_transpose(ptr, idx, history_map_row, num_node, n_src, num_edge=None, want_edges=True):
+def build_transpose(ptr, idx, history_map_row, num_node, n_src, num_edge=None, want_edges=True,
+                    history_map_src=None):
     """Stable CSC view of the first ``num_node`` rows: returns (ptrT, rowT, edgeT).
 
     ``num_edge`` bounds the edge slots that are sorted (default: all of ``idx``).  With
-    ``want_edges=False`` (enough for the mean aggregation) edgeT is None and the build is cheaper."""
+    ``want_edges=False`` (enough for the mean aggregation) edgeT is None and the build is cheaper.
+    Edges of rows flagged by ``history_map_row`` and edges whose source is flagged by
+    ``history_map_src`` (per-source substitution) are left out."""
     lib = load_library()
     _dev(ptr, "ptr", torch.int64)
     _dev(idx, "idx", torch.int64)
@@ -241,7 +246,12 @@ def build_transpose(ptr, idx, history_map_row, num_node, n_src, num_edge=None, w
         raise RuntimeError("hc_transpose_workspace_bytes failed (no usable GPU?)")
     ws = _workspace(nbytes, dev)
     hm = None if _empty(history_map_row) else _dev(history_map_row, "history_map", torch.int64)
-    rc = lib.hc_build_transpose(_ptr(ptr), _ptr(idx), _ptr(hm), R, E, n_src, _ptr(ptrT), _ptr(rowT),
+    hs = None if _empty(history_map_src) else _dev(history_map_src, "source_history_map", torch.int64)
+    if hs is not None and hs.numel() < n_src:
+        raise ValueError("source_history_map is shorter than n_src")
+    if hm is not None and hm.numel() < R:
+        raise ValueError("history_map is shorter than num_node")
+    rc = lib.hc_build_transpose(_ptr(ptr), _ptr(idx), _ptr(hm), _ptr(hs), R, E, n_src, _ptr(ptrT), _ptr(rowT),
                                 _ptr(edgeT), _ptr(ws), ws.numel(), _stream())
     _check(rc, "hc_build_transpose")
     return ptrT, rowT, edgeT
@@ -290,10 +300,14 @@ class _AggrHistory(torch.autograd.Function):
     context (the reference keeps raw addresses, :406-408)."""
 
     @staticmethod
-    def forward(ctx, x, ptr, idx, edge_value, hmap, hbuf, hsize, num_node, mode):
+    def forward(ctx, x, ptr, idx, edge_value, hmap, hbuf, hsize, num_node, mode, num_edge=None):
         R = int(num_node) if num_node else ptr.numel() - 1
         out = _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, R)
         ctx.hc = (ptr, idx, hmap, hsize, R, mode, None if hbuf is None else tuple(hbuf.shape))
+        # edge slots the first R rows can reach, when the caller knows it (a layer of a shared CSR owns a
+        # prefix of idx): the transposed view then sorts that prefix only
+        ctx.num_edge = num_edge
+        ctx.hdtype = None if hbuf is None else hbuf.dtype
         ctx.save_for_backward(x, edge_value if edge_value is not None else x.new_empty(0))
         ctx.has_ev = edge_value is not None
         return out
@@ -320,20 +334,34 @@ class _AggrHistory(torch.autograd.Function):
                 flat = g2.reshape(R, -1)
                 hit = (row_map[:R] != -1).unsqueeze(1)
                 grad_h.view(-1, hsize)[:R, :flat.shape[1]] = torch.where(hit, flat, torch.zeros_like(flat))
-            return None, None, None, None, None, grad_h, None, None, None
+            return None, None, None, None, None, grad_h, None, None, None, None
         # The transposed view is built here, on the stream backward runs on.  Building it during the
         # forward pass on a side stream was measured and dropped: concurrent with the bandwidth-bound
         # forward it finishes no earlier (9.15 against 9.09 ms for forward + backward on a 20 M-edge
         # block), and on sampled mini-batches the stream switch costs the host more than the build
         # costs the GPU.
-        tr = build_transpose(ptr, idx, row_map, R, n_src, want_edges=ev is not None)
+        src_map = hmap if mode == SUBST_SRC else None
+        want_table = src_map is not None and ctx.needs_input_grad[5]
+        # Per-source substitution: a substituted source passes nothing to input[s] (that row was never
+        # read).  When the table needs no gradient those edges are left out of the view; when it does,
+        # every source is summed and the rows of substituted sources are moved to the table's gradient.
+        num_edge = ctx.num_edge
+        tr = build_transpose(ptr, idx, row_map, R, n_src, num_edge=num_edge, want_edges=ev is not None,
+                             history_map_src=None if want_table else src_map)
         grad_x, grad_h, edge_grad = _aggr_bwd(ptr, idx, tr, g, row_map, ev, x, want_eg, hshape, hsize, R,
                                               n_src, want_hist_grad=want_h)
+        if want_table:
+            sub = src_map[:n_src] != -1
+            grad_h = torch.zeros(hshape, dtype=torch.float32, device=g.device)
+            grad_h.view(-1, hsize)[:, :grad_x.shape[-1]].index_add_(0, src_map[:n_src][sub], grad_x[sub])
+            grad_x = grad_x.masked_fill(sub.unsqueeze(1), 0.0)
+        elif mode == SUBST_SRC or not want_h:
+            grad_h = None
         if grad_x.dtype != x.dtype:
             grad_x = grad_x.to(x.dtype)
-        if mode == SUBST_SRC or not want_h:
-            grad_h = None
-        return (grad_x if want_x else None), None, None, edge_grad, None, grad_h, None, None, None
+        if grad_h is not None and grad_h.dtype != ctx.hdtype:
+            grad_h = grad_h.to(ctx.hdtype)
+        return (grad_x if want_x else None), None, None, edge_grad, None, grad_h, None, None, None, None
 
 
 def _norm_history(history_map, history_buffer, history_size):
@@ -343,13 +371,15 @@ def _norm_history(history_map, history_buffer, history_size):
 
 
 # ----------------------------------------------------------------------------- reference API
-def aggr_forward_history(input, ptr, idx, history_map, history_buffer, history_size, num_node):
-    """Mean aggregation with history substitution; same signature as the reference
+def aggr_forward_history(input, ptr, idx, history_map, history_buffer, history_size, num_node, num_edge=None):
+    """Mean aggregation with history substitution; same positional signature as the reference
     (/root/reference/src/cpp/include/history_aggr.h:34-37).  ``history_size == 0`` or an
     empty ``history_map`` gives the plain mean (the reference exits there, history_aggr.cu:440-441).
-    The result always requires grad (history_aggr.cu:604)."""
+    The result always requires grad (history_aggr.cu:604).  ``num_edge`` (optional, beyond the
+    reference) is an upper bound of ptr[num_node] for callers that know it -- a layer of a shared
+    mini-batch CSR owns a prefix of ``idx`` -- so that backward looks at that prefix only."""
     hmap, hbuf, hsize = _norm_history(history_map, history_buffer, history_size)
-    out = _AggrHistory.apply(input, ptr, idx, None, hmap, hbuf, hsize, num_node, SUBST_ROW)
+    out = _AggrHistory.apply(input, ptr, idx, None, hmap, hbuf, hsize, num_node, SUBST_ROW, num_edge)
     if not out.requires_grad:
         out.requires_grad_(True)
     return out
@@ -372,7 +402,8 @@ def aggr_forward_history_edge_value(input, ptr, idx, edge_value, history_map, hi
 def aggr_forward_source_history(input, ptr, idx, source_history_map, history_table, num_node=0):
     """Extension: per-SOURCE substitution.  Neighbour j is read from
     ``history_table[source_history_map[idx[j]]]`` when the map entry is not -1, else from
-    ``input[idx[j]]``.  Backward returns the gradient of the substituted source rows."""
+    ``input[idx[j]]``.  Backward: ``input`` rows of substituted sources get a zero gradient (they
+    were not read); their share goes to ``history_table``'s gradient when it requires one."""
     hsize = 0 if _empty(source_history_map) else history_table.shape[-1]
     hmap, hbuf, hsize = _norm_history(source_history_map, history_table, hsize)
     return _AggrHistory.apply(input, ptr, idx, None, hmap, hbuf, hsize, num_node, SUBST_SRC)
@@ -606,6 +637,30 @@ def lookup(map_tensor, ids, offset=0):
                        _stream())
     _check(rc, "hc_lookup")
     return out
+
+
+def ring_lookup(full2slot, ids, table, checkin=None, now=0, age_limit=1 << 62, want_rows=True):
+    """Slots of ``ids`` in a ring table and the table rows of the hits, in one launch.  An entry with
+    ``now - checkin[slot] >= age_limit`` counts as absent (-1).  Returns (slot[int64], rows[fp32] or
+    None); rows of absent ids are zero."""
+    lib = load_library()
+    _dev(full2slot, "full2slot", torch.int64)
+    _dev(ids, "ids", torch.int64)
+    _dev(table, "table")
+    if table.dim() != 2:
+        raise ValueError("table must be [capacity, F]")
+    if checkin is not None:
+        _dev(checkin, "checkin", torch.int64)
+        if checkin.numel() < table.shape[0]:
+            raise ValueError("checkin is shorter than the table")
+    n = ids.numel()
+    slot = torch.empty(n, dtype=torch.int64, device=ids.device)
+    rows = torch.empty((n, table.shape[1]), dtype=torch.float32, device=ids.device) if want_rows else None
+    rc = lib.hc_ring_lookup(_ptr(full2slot), full2slot.numel(), _ptr(ids), _ptr(checkin), int(now), int(age_limit),
+                            _ptr(table), _float_dtype(table, "table"), table.shape[0], table.shape[1], _ptr(slot),
+                            _ptr(rows), n, _stream())
+    _check(rc, "hc_ring_lookup")
+    return slot, rows
 
 
 MAX_TYPED_RELATIONS = 64

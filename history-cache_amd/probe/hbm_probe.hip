@@ -14,6 +14,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <string>
 #include <vector>
 
 #define CK(x)                                                                      \
@@ -134,12 +135,61 @@ static double gather_gbps(const f4 *tab, const int *ids, f4 *out, int K, int64_t
   return (double)n_out * K * (1024.0 * VPR) / ms / 1e6;
 }
 
+// `hbm_probe <GB> gather <pattern>`: only the 1 KiB row gather (8 rows in flight, ordinary loads), with the
+// row ids drawn by one of these patterns -- short enough for a counter pass of its own:
+//   uniform     every row id uniform over the table (the pattern of the table above)
+//   page        the 20 rows of one output row lie in one 2 MiB-aligned window (windows uniform): random DRAM
+//               rows, but one address translation per wave
+//   block       the same with one window per block of 4 waves
+//   sequential  row id = position: the gather kernel reading the table front to back
+static int gather_only(double table_gb, const char *pattern) {
+  const int K = 20;
+  const int64_t table_bytes = (int64_t)(table_gb * 1e9) / (2 << 20) * (2 << 20);
+  const int64_t rows = table_bytes / 1024, E = 20000000, n_out = E / K;
+  const int64_t win_rows = (2 << 20) / 1024, n_win = rows / win_rows;
+  if (n_win < 1) return 2;
+  f4 *tab = nullptr, *dst = nullptr;
+  int *ids = nullptr;
+  CK(hipMalloc(&tab, (size_t)table_bytes));
+  CK(hipMalloc(&dst, (size_t)n_out * 1024));
+  CK(hipMalloc(&ids, (size_t)E * sizeof(int)));
+  CK(hipMemset(tab, 0, (size_t)table_bytes));
+  std::vector<int> h((size_t)E);
+  uint64_t s = 0x9E3779B97F4A7C15ull;
+  auto next = [&](uint64_t m) {
+    s = s * 6364136223846793005ull + 1442695040888963407ull;
+    return (int64_t)((s >> 33) % m);
+  };
+  const std::string pat(pattern);
+  int64_t win = 0;
+  for (int64_t i = 0; i < E; ++i) {
+    if (pat == "uniform") h[(size_t)i] = (int)next((uint64_t)rows);
+    else if (pat == "sequential") h[(size_t)i] = (int)(i % rows);
+    else if (pat == "page" || pat == "block") {
+      const int64_t group = pat == "page" ? K : 4 * K;
+      if (i % group == 0) win = next((uint64_t)n_win);
+      h[(size_t)i] = (int)(win * win_rows + next((uint64_t)win_rows));
+    } else {
+      std::printf("unknown pattern %s\n", pattern);
+      return 2;
+    }
+  }
+  CK(hipMemcpy(ids, h.data(), (size_t)E * sizeof(int), hipMemcpyHostToDevice));
+  const double gbps = gather_gbps<8, 1, false>(tab, ids, dst, K, n_out);
+  std::printf("row gather 1 KiB, pattern %-10s over %6.2f GB: %6.0f GB/s\n", pattern, table_bytes / 1e9, gbps);
+  CK(hipFree(ids));
+  CK(hipFree(dst));
+  CK(hipFree(tab));
+  return 0;
+}
+
 int main(int argc, char **argv) {
   const double table_gb = argc > 1 ? std::atof(argv[1]) : 20.0;   // footprint of the gathered table
   if (!(table_gb >= 0.01 && table_gb <= 64.0)) {
-    std::printf("usage: hbm_probe [table GB in 0.01..64]\n");
+    std::printf("usage: hbm_probe [table GB in 0.01..64] [gather uniform|page|block|sequential]\n");
     return 2;
   }
+  if (argc > 3 && std::string(argv[2]) == "gather") return gather_only(table_gb, argv[3]);
   const int K = 20;                                               // rows summed per output row
   const int64_t table_bytes = (int64_t)(table_gb * 1e9) / 4096 * 4096;
   const int64_t n16 = table_bytes / 16;

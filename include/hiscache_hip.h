@@ -69,7 +69,9 @@ int hc_device_count(void);
  *       (fused multiply-add, no division); history rows copy hbuf[r,:F]
  *       (hsize == F) or hbuf[r, h*F:(h+1)*F] (hsize == F*n_head).
  *   mode == HC_SUBST_SRC (mean only): every neighbour row is read from
- *       hbuf[hmap[idx[j]], :F] when hmap[idx[j]] != -1, else from vin.
+ *       hbuf[hmap[idx[j]], :F] when hmap[idx[j]] != -1, else from vin; hmap has
+ *       n_src entries; the table has vin's element type, or vin is fp32 and
+ *       the table fp16 / bf16 (other pairs return HC_EUNSUPPORTED).
  *
  * ptr[R+1], idx[>= ptr[R]], vin[n_src, n_head, F] (in_dtype), hmap NULL = no
  * history, hbuf (hist_dtype), vout[R, n_head, F] fp32.  n_head >= 1; n_head > 1
@@ -81,10 +83,13 @@ int hc_device_count(void);
  * contiguous quarters of ceil(deg/4) edges, each in CSR order, combined left to
  * right ((q0+q1)+q2)+q3, then divided (mean only).
  * workspace (optional, NULL allowed; 256-byte aligned, of
- * hc_aggr_fwd_workspace_bytes(R, E) bytes, E = an upper bound of ptr[R]): on
- * large blocks the long rows are listed first and scheduled at the start of
- * the launch, which shortens its tail; results do not depend on it. */
-size_t hc_aggr_fwd_workspace_bytes(int64_t R, int64_t E);
+ * hc_aggr_fwd_workspace_bytes(mode, R, E, n_src) bytes, E = an upper bound of
+ * ptr[R]): on large blocks the long rows are listed first and scheduled at the
+ * start of the launch, which shortens its tail; with HC_SUBST_SRC over a
+ * million sources or more, one bit per source ("has an entry") is derived from
+ * hmap first, so that sources without an entry never touch the map.  Results
+ * do not depend on the workspace. */
+size_t hc_aggr_fwd_workspace_bytes(int mode, int64_t R, int64_t E, int64_t n_src);
 int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, const void *vin, int in_dtype,
                 const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize,
                 const float *edge_value, int64_t n_head, float *vout, int64_t R, int64_t F,
@@ -101,9 +106,12 @@ int64_t hc_aggr_fwd_long_row_edges(int64_t F, int in_dtype);
  * atomicAdd (history_aggr.cu:164); this library gathers over a transposed view
  * instead, which makes the sums deterministic.
  *
- * Stable sort of the first E edge slots by source id.  Edge slots >= ptr[R]
- * and, when hmap_row != NULL, edges of rows with hmap_row[r] != -1 are
- * dropped.  Outputs: ptrT[n_src+1] (int64), rowT[E] (destination row per
+ * Stable sort of the first E edge slots by source id.  Edge slots >= ptr[R],
+ * when hmap_row != NULL the edges of rows with hmap_row[r] != -1, and when
+ * hmap_src != NULL (n_src entries) the edges whose source s has
+ * hmap_src[s] != -1 are dropped: a row that took its history row, and a source
+ * that was substituted by a history-table row, pass no gradient to vin.
+ * Outputs: ptrT[n_src+1] (int64), rowT[E] (destination row per
  * transposed edge, ascending inside a source), edgeT[E] (original edge slot);
  * only the first ptrT[n_src] entries of rowT/edgeT are meaningful.
  * Requires R, E, n_src < 2^31 - 1.
@@ -112,9 +120,10 @@ int64_t hc_aggr_fwd_long_row_edges(int64_t F, int in_dtype);
  * captured graph would replay as memset nodes: on a capturing stream such a
  * call returns HC_EUNSUPPORTED and records nothing. */
 size_t hc_transpose_workspace_bytes(int64_t R, int64_t E, int64_t n_src);
-int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row, int64_t R,
-                       int64_t E, int64_t n_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT,
-                       void *workspace, size_t workspace_bytes, void *stream);
+int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row,
+                       const int64_t *hmap_src, int64_t R, int64_t E, int64_t n_src, int64_t *ptrT,
+                       int32_t *rowT, int32_t *edgeT, void *workspace, size_t workspace_bytes,
+                       void *stream);
 
 /* ---------------------------------------------------------------- aggregation backward
  * Replaces AggrHistoryFunction::backward / AggrHistoryEdgeValueFunction::backward
@@ -131,9 +140,13 @@ int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hm
  *       rows, 0 for the others.  E_total = number of edge slots to fill.
  *
  * ptrT/rowT/edgeT come from hc_build_transpose called with the same hmap_row
- * (so edges of history rows are already gone); ptrT[n_src] <= E_total.  In
- * HC_SUBST_SRC mode pass hmap = NULL: the result is the gradient with respect
- * to the substituted source row, whichever table it came from.
+ * (so edges of history rows are already gone); ptrT[n_src] <= E_total.  After
+ * a forward pass in HC_SUBST_SRC mode pass hmap = NULL here and build the view
+ * with hmap_src: substituted sources then have no incoming edges and their
+ * rows of grad_vin are written 0 (vin[s] was never read for them).  A view
+ * built without hmap_src gives every source the gradient of the row that was
+ * read for it, whichever table it came from; the caller routes the rows of
+ * substituted sources to the history table's gradient if it wants one.
  * Summation order (fp32, fixed): ascending destination row.  When a workspace
  * of hc_aggr_bwd_workspace_bytes() is given and hc_aggr_bwd_chunk_edges(F)
  * reports C > 0, a source with more than C incoming edges is summed in chunks
@@ -367,6 +380,21 @@ int hc_gather_rows(const void *src, int src_dtype, int64_t n_rows, const int64_t
  * of lookup_and_load, hiscache/history_cache.py:310,315). */
 int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset, int64_t *out,
               int64_t n, void *stream);
+
+/* hc_ring_lookup: lookup of a ring table (full2slot / checkin / table as
+ * hc_grad_check maintains them) for one batch, in one launch:
+ *   slot_out[i] = full2slot[ids[i]], or -1 when the id has no entry or its entry
+ *                 is stale: now - checkin[slot] >= age_limit (checkin nullable:
+ *                 then no entry is stale);
+ *   rows_out[i,:F] (fp32, nullable) = table[slot_out[i], :F], zeros for -1.
+ * A stale entry is reported as absent so that the caller recomputes the row and
+ * may admit the fresh value; the reference bounds the age of an entry the same
+ * way by un-mapping old slots (hiscache/history_table.py:189-200) and looks
+ * slots up with torch indexing (hiscache/history_cache.py:307-313). */
+int hc_ring_lookup(const int64_t *full2slot, int64_t n_full, const int64_t *ids,
+                   const int64_t *checkin, int64_t now, int64_t age_limit, const void *table,
+                   int table_dtype, int64_t capacity, int64_t F, int64_t *slot_out, float *rows_out,
+                   int64_t n, void *stream);
 
 #ifdef __cplusplus
 }

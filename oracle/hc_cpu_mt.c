@@ -80,7 +80,10 @@ int mt_fwd_mean_src(const Index *ptr, const Index *idx, const float *feat, const
 /* Transposed view (stable by destination row): ptrT[n_src+1], rowT[E].  Every thread owns a range of
  * sources and walks all edges twice (count, place); no atomics, the order inside a source is the walk
  * order, i.e. ascending (row, edge). */
-int mt_build_transpose(const Index *ptr, const Index *idx, Index R, Index n_src, Index *ptrT, int32_t *rowT) {
+/* hmap_src (nullable, n_src entries): edges whose source has hmap_src[s] != -1 are left out (a source that
+ * was substituted by a history-table row in the forward pass passes no gradient to its feature row). */
+int mt_build_transpose(const Index *ptr, const Index *idx, Index R, Index n_src, Index *ptrT, int32_t *rowT,
+                       const Index *hmap_src) {
   const Index E = ptr[R];
   for (Index j = 0; j < E; ++j)
     if (idx[j] < 0 || idx[j] >= n_src) return ORC_EINVAL;
@@ -93,7 +96,7 @@ int mt_build_transpose(const Index *ptr, const Index *idx, Index R, Index n_src,
     const Index lo = n_src * t / T, hi = n_src * (t + 1) / T;
     for (Index j = 0; j < E; ++j) {
       const Index s = idx[j];
-      if (s >= lo && s < hi) ptrT[s + 1]++;
+      if (s >= lo && s < hi && (!hmap_src || hmap_src[s] == -1)) ptrT[s + 1]++;
     }
 #pragma omp barrier
 #pragma omp single
@@ -104,7 +107,7 @@ int mt_build_transpose(const Index *ptr, const Index *idx, Index R, Index n_src,
     for (Index row = 0; row < R; ++row) {
       for (Index j = ptr[row]; j < ptr[row + 1]; ++j) {
         const Index s = idx[j];
-        if (s >= lo && s < hi) rowT[cur[s]++] = (int32_t)row;
+        if (s >= lo && s < hi && (!hmap_src || hmap_src[s] == -1)) rowT[cur[s]++] = (int32_t)row;
       }
     }
   }

@@ -63,14 +63,15 @@ def fwd_mean_src(ptr, idx, feat, hmap_src, hist, split_above=0, out=None):
     return out
 
 
-def build_transpose(ptr, idx, n_src, ptrT=None, rowT=None):
+def build_transpose(ptr, idx, n_src, ptrT=None, rowT=None, hmap_src=None):
     ptr, idx = _arr(ptr, np.int64), _arr(idx, np.int64)
+    hmap_src = None if hmap_src is None else _arr(hmap_src, np.int64)
     R = len(ptr) - 1
     if ptrT is None:
         ptrT = np.empty(n_src + 1, np.int64)
     if rowT is None:
         rowT = np.empty(max(int(ptr[R]), 1), np.int32)
-    rc = lib().mt_build_transpose(_p(ptr), _p(idx), _I(R), _I(n_src), _p(ptrT), _p(rowT))
+    rc = lib().mt_build_transpose(_p(ptr), _p(idx), _I(R), _I(n_src), _p(ptrT), _p(rowT), _p(hmap_src))
     if rc != 0:
         raise ValueError("mt_build_transpose: a source id is out of range")
     return ptrT, rowT

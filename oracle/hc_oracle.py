@@ -146,8 +146,26 @@ def bwd_mean_row(ptr, idx, g, hmap, n_src, hbuf_shape=None, chunk=0):
     return gout, ghist
 
 
-def bwd_mean_src(ptr, idx, g, n_src, chunk=0):
-    return bwd_mean_row(ptr, idx, g, None, n_src, chunk=chunk)[0]
+def bwd_mean_src(ptr, idx, g, n_src, chunk=0, hmap_src=None, hist_shape=None):
+    """Backward of the mean with per-source substitution.  Without ``hmap_src``: the gradient of the
+    row that was read for every source, whichever table it came from.  With ``hmap_src``: returns
+    (grad_feat, grad_hist) -- a substituted source s leaves grad_feat[s] = 0 (feat[s] was not read) and
+    adds its sum to grad_hist[hmap_src[s]] (sources that share a table row are added in ascending
+    source order); ``hist_shape`` None skips grad_hist."""
+    all_src = bwd_mean_row(ptr, idx, g, None, n_src, chunk=chunk)[0]
+    if hmap_src is None:
+        return all_src
+    hmap_src = _i64(hmap_src)[:n_src]
+    sub = hmap_src != -1
+    grad_feat = all_src.copy()
+    grad_feat[sub] = 0.0
+    grad_hist = None
+    if hist_shape is not None:
+        grad_hist = np.zeros(hist_shape, np.float32)
+        F = all_src.shape[1]
+        for s in np.nonzero(sub)[0]:
+            grad_hist[hmap_src[s], :F] += all_src[s]
+    return grad_feat, grad_hist
 
 
 def bwd_edge_value(ptr, idx, ev, g, hmap, vin, n_src, hsize=None, want_edge_grad=False):

@@ -140,3 +140,21 @@ def evict_by_both(checkin, history_to_full, full_to_history, sub_to_history, sco
     evict_by_staleness(checkin, history_to_full, full_to_history, glb_iter, staleness_thres)
     return thres
 
+
+
+def ring_lookup(full2slot, checkin, ids, now, age_limit, table_f32=None):
+    """Lookup of a ring table with the age bound applied at lookup time: the slot of every id, -1
+    when the id has no entry or the entry is at least ``age_limit`` iterations old
+    (now - checkin[slot] >= age_limit); the reference bounds the age of an entry by un-mapping old
+    slots (history_table.py:189-200).  With ``table_f32`` also the rows of the hits (zeros elsewhere)."""
+    full2slot, checkin, ids = (np.asarray(a, np.int64) for a in (full2slot, checkin, ids))
+    slot = full2slot[ids].copy()
+    held = slot >= 0
+    stale = held & ((int(now) - checkin[np.maximum(slot, 0)]) >= int(age_limit))
+    slot[stale] = -1
+    if table_f32 is None:
+        return slot
+    rows = np.zeros((len(ids), table_f32.shape[1]), np.float32)
+    hit = slot >= 0
+    rows[hit] = table_f32[slot[hit]]
+    return slot, rows

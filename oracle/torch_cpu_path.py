@@ -54,6 +54,19 @@ def aggr_fwd_src(feat, hist, hmap_src, ptr, idx, num_node):
     return out / deg.clamp(min=1).to(torch.float32)[:, None]
 
 
+def aggr_bwd_src(g, ptr, idx, hmap_src, n_src, num_node):
+    """Backward of aggr_fwd_src with respect to ``feat``: substituted sources get a zero row."""
+    dst, deg = edge_rows(ptr, num_node)
+    E = int(ptr[num_node])
+    src = idx[:E]
+    scaled = (g / deg.clamp(min=1).to(torch.float32)[:, None])[dst]
+    if hmap_src is not None:
+        scaled = scaled * (hmap_src[src] == -1)[:, None]
+    gx = torch.zeros(n_src, g.shape[1], dtype=torch.float32)
+    gx.index_add_(0, src, scaled)
+    return gx
+
+
 def admission(grad, emb, slot, thres, table, header):
     """norm -> mask -> append (history_cache.py:205-221), no ring wrap."""
     norm = grad.norm(dim=1)

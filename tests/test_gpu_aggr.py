@@ -188,6 +188,46 @@ def test_build_transpose_many_more_sources_than_edges(be, orc):
         np.testing.assert_array_equal(rowT.cpu().numpy()[: int(rp[-1])], rr)
 
 
+@pytest.mark.parametrize("R,N,deg,popular", [
+    (3000, 40, 30, None),        # 90 k edges onto 40 sources: every segment is ranked through the LDS bitmap
+    (20000, 5000, 12, 0.3),      # one source with ~70 k incoming edges beside short segments
+    (4000, 900_000, 6, None),    # many sources without edges (still the counting-sort path)
+    (262_144 // 4, 300, 4, None),  # exactly the largest block of the counting-sort path
+    (70_000, 3000, 5, 0.2),      # above it: the library-sort path
+    (5000, (1 << 20) + 5, 5, None),  # few edges but more sources than the counting sort takes
+])
+def test_build_transpose_paths_agree_with_a_stable_argsort(be, R, N, deg, popular):
+    """The counting-sort path of small blocks and the library-sort path of large ones against NumPy's
+    stable argsort: segment bounds, rows and edge slots, with long segments, dropped rows and dropped
+    sources."""
+    rng = np.random.default_rng(R + N)
+    ptr = (np.arange(R + 1) * deg).astype(np.int64)
+    idx = rng.integers(0, N, size=R * deg, dtype=np.int64)
+    if popular:
+        idx[rng.random(len(idx)) < popular] = N // 3
+    hrow = random_hmap(rng, R, 0.2)
+    hsrc = np.where(rng.random(N) < 0.3, 1, -1).astype(np.int64)
+    hsrc[N // 3] = -1
+    e = np.arange(len(idx))
+    row = e // deg
+    for use_row, use_src in ((False, False), (True, True)):
+        keep = np.ones(len(idx), bool)
+        if use_row:
+            keep &= hrow[row] == -1
+        if use_src:
+            keep &= hsrc[idx] == -1
+        order = e[keep][np.argsort(idx[keep], kind="stable")]
+        want_ptrT = np.searchsorted(idx[order], np.arange(N + 1), side="left")
+        for want_edges in (True, False):
+            ptrT, rowT, edgeT = be.build_transpose(T(ptr), T(idx), T(hrow) if use_row else None, R, N,
+                                                   want_edges=want_edges,
+                                                   history_map_src=T(hsrc) if use_src else None)
+            np.testing.assert_array_equal(ptrT.cpu().numpy(), want_ptrT)
+            np.testing.assert_array_equal(rowT.cpu().numpy()[: len(order)], row[order])
+            if want_edges:
+                np.testing.assert_array_equal(edgeT.cpu().numpy()[: len(order)], order)
+
+
 def test_build_transpose_no_edges(be):
     ptr = torch.zeros(11, dtype=torch.int64, device=DEV)
     idx = torch.zeros(0, dtype=torch.int64, device=DEV)
@@ -279,17 +319,83 @@ def test_bwd_retain_grad_on_output_and_raw_feature_input(be, orc):
     assert out.grad is not None and out.grad.shape == out.shape
 
 
-def test_src_mode_backward(be, orc):
+@pytest.mark.parametrize("table_grad", [False, True])
+def test_src_mode_backward(be, orc, table_grad):
+    """Backward of the per-source substitution: a substituted source gets no gradient in ``feat`` (its
+    row was not read); its share goes to the table's gradient when the table requires one."""
     rng = np.random.default_rng(7)
-    R, N, F = 300, 200, 256
+    R, N, F, Hn = 300, 200, 256, 150
     ptr, idx = random_csr(rng, R, N, 10, hub=90)
     feat = T(rng.standard_normal((N, F)).astype(np.float32)).requires_grad_(True)
-    hist = T(rng.standard_normal((N, F)).astype(np.float32))
-    hmap = np.where(rng.random(N) < 0.4, np.arange(N), -1).astype(np.int64)
+    hist = T(rng.standard_normal((Hn, F)).astype(np.float32)).requires_grad_(table_grad)
+    hmap = np.where(rng.random(N) < 0.4, rng.integers(0, Hn, size=N), -1).astype(np.int64)
     g = rng.standard_normal((R, F)).astype(np.float32)
     out = be.aggr_forward_source_history(feat, T(ptr), T(idx), T(hmap), hist)
     out.backward(T(g))
-    np.testing.assert_array_equal(feat.grad.cpu().numpy(), orc.bwd_mean_src(ptr, idx, g, N, chunk=be.bwd_chunk_edges(F)))
+    gf, gh = orc.bwd_mean_src(ptr, idx, g, N, chunk=be.bwd_chunk_edges(F), hmap_src=hmap, hist_shape=(Hn, F))
+    np.testing.assert_array_equal(feat.grad.cpu().numpy(), gf)
+    assert (feat.grad.cpu().numpy()[hmap != -1] == 0).all()
+    if table_grad:
+        # rows shared by several sources are added by index_add_ (any order): compare with a tolerance
+        np.testing.assert_allclose(hist.grad.cpu().numpy(), gh, rtol=1e-5, atol=1e-6)
+    else:
+        assert hist.grad is None
+
+
+def test_transposed_view_drops_substituted_sources(be, orc):
+    rng = np.random.default_rng(71)
+    R, N = 500, 300
+    ptr, idx = random_csr(rng, R + 20, N, 12, hub=200)
+    hrow = random_hmap(rng, R, 0.3)
+    hsrc = np.where(rng.random(N) < 0.4, 5, -1).astype(np.int64)
+    ptrT, rowT, edgeT = be.build_transpose(T(ptr), T(idx), T(hrow), R, N, history_map_src=T(hsrc))
+    e = np.arange(int(ptr[R]))
+    row = np.searchsorted(ptr[1:R + 1], e, side="right")
+    keep = (hrow[row] == -1) & (hsrc[idx[e]] == -1)
+    order = e[keep][np.argsort(idx[e[keep]], kind="stable")]
+    n = len(order)
+    np.testing.assert_array_equal(edgeT.cpu().numpy()[:n], order)
+    np.testing.assert_array_equal(rowT.cpu().numpy()[:n], row[order])
+    want_ptrT = np.searchsorted(idx[order], np.arange(N + 1), side="left")
+    np.testing.assert_array_equal(ptrT.cpu().numpy(), want_ptrT)
+
+
+@pytest.mark.parametrize("table_dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("F,R", [(256, 300), (128, 300), (64, 70_000), (100, 200)])
+def test_src_mode_table_narrower_than_features(be, orc, table_dtype, F, R):
+    """Per-source substitution with fp32 features and an fp16 / bf16 table (the papers100M-shaped
+    combination), fast widths and a generic width, long rows, a block above the long-row-list
+    threshold: bit-exact against the checker on the table widened to fp32."""
+    rng = np.random.default_rng(F + R)
+    N, Hn = 5000, 3000
+    ptr, idx = random_csr(rng, R, N, 12, hub=700)
+    feat = rng.standard_normal((N, F)).astype(np.float32)
+    hist = T(rng.standard_normal((Hn, F)).astype(np.float32)).to(table_dtype)
+    hmap = np.where(rng.random(N) < 0.4, rng.integers(0, Hn, size=N), -1).astype(np.int64)
+    out = be.aggr_forward_source_history(T(feat), T(ptr), T(idx), T(hmap), hist)
+    ref = orc.fwd_mean_src(ptr, idx, feat, hmap, hist.float().cpu().numpy(), split_above=be.long_row_edges(F))
+    np.testing.assert_array_equal(out.detach().cpu().numpy(), ref)
+    # narrower features than the table: refused
+    with pytest.raises(ValueError):
+        be.aggr_forward_source_history(T(feat).half(), T(ptr), T(idx), T(hmap), hist.float())
+
+
+def test_src_mode_bitmap_over_many_sources(be, orc):
+    """Above 2^20 sources the forward derives one bit per source from the map and consults it before
+    the map: same bits out, with maps that are empty, full, and that end inside a 64-source group."""
+    rng = np.random.default_rng(72)
+    R, F = 3000, 64
+    for N in ((1 << 20) + 37, (1 << 20) + 64):
+        ptr, idx = random_csr(rng, R, N, 20, hub=900)
+        idx[:50] = N - 1 - np.arange(50)              # the last sources, in the bitmap's last word
+        feat = T(rng.standard_normal((N, F)).astype(np.float32))
+        Hn = 1000
+        hist = rng.standard_normal((Hn, F)).astype(np.float32)
+        for frac in (0.4, 0.0, 1.0):
+            hmap = np.where(rng.random(N) < frac, rng.integers(0, Hn, size=N), -1).astype(np.int64)
+            out = be.aggr_forward_source_history(feat, T(ptr), T(idx), T(hmap), T(hist))
+            ref = orc.fwd_mean_src(ptr, idx, feat.cpu().numpy(), hmap, hist, split_above=be.long_row_edges(F))
+            np.testing.assert_array_equal(out.detach().cpu().numpy(), ref)
 
 
 @pytest.mark.parametrize("F,H", [(64, 1), (256, 1), (96, 1), (32, 3), (256, 2),

@@ -403,31 +403,32 @@ def test_ring_cache_cycles_match_oracle():
                                  device=DEV)
         ref = dict(table=np.zeros((cap, H), np.uint16), f2s=np.full(N, -1, np.int64), s2f=np.full(cap, -1, np.int64),
                    checkin=np.full(cap, -1, np.int64), header=np.zeros(1, np.int64))
+        n_stale = 0
         for it in range(1, 9):
             b = layered_batch(rng, N, 40, [6, 4, 3])
             batch = make_batch(b, rng.integers(0, 5, size=N), DEV)
             cache.lookup_and_load(batch, 3)
             n1 = int(b["num_node_in_layer"][1])
             nodes = b["sub_to_full"][:n1]
-            slot = ref["f2s"][nodes].copy()
+            # entries that are 3 iterations old count as absent at lookup (the cache's counter equals `it`)
+            tab32 = ref["table"].view(np.float16).astype(np.float32)
+            slot, rows = host_model.ring_lookup(ref["f2s"], ref["checkin"], nodes, it, 3, tab32)
+            n_stale += int(((ref["f2s"][nodes] != -1) & (slot == -1)).sum())
             np.testing.assert_array_equal(cache.sub2embed.cpu().numpy(), slot)
+            np.testing.assert_array_equal(cache.cached_embedding.cpu().numpy(), rows)
             used = orc.count_history_reconstruct(b["ptr"], b["idx"], slot, len(b["sub_to_full"]), 40, 3)
             np.testing.assert_array_equal(cache.used_masks[0].cpu().numpy(), used[0])
             x_ref = feats[torch.from_numpy(b["sub_to_full"])].numpy() * used[0][:, None]
             np.testing.assert_array_equal(batch.x.cpu().numpy(), x_ref)
-            hit = slot != -1
-            tab16 = ref["table"].view(np.float16)
-            np.testing.assert_array_equal(cache.cached_embedding.cpu().numpy()[hit], tab16[slot[hit]].astype(np.float32))
             emb = rng.standard_normal((n1, H)).astype(np.float32)
             grad = (rng.standard_normal((n1, H)) * np.exp(rng.normal(-3, 1.5, size=(n1, 1)))).astype(np.float32)
             pe = torch.from_numpy(emb).to(DEV).requires_grad_(True)
             pe.grad = torch.from_numpy(grad).to(DEV)
             cache.produced_embedding = pe
             cache.update_history(batch, it)
-            age = (it - ref["checkin"][np.maximum(slot, 0)]).astype(np.int32)
             score = orc.row_scores(grad)
             thres = 0.05 if fixed else float(host_model.quantile_threshold(score, 0.6))
-            rmask, _, _ = orc.grad_check(grad, emb, slot, age, None, nodes, thres, 3, orc.NORM_L2, orc.CMP_LT,
+            rmask, _, _ = orc.grad_check(grad, emb, slot, None, None, nodes, thres, 0, orc.NORM_L2, orc.CMP_LT,
                                          ref["table"], orc.DT_F16, ref["f2s"], ref["s2f"], ref["checkin"],
                                          ref["header"], it)
             np.testing.assert_array_equal(cache.last_record_mask.cpu().numpy(), rmask)
@@ -438,7 +439,54 @@ def test_ring_cache_cycles_match_oracle():
             live = ref["s2f"] != -1
             np.testing.assert_array_equal(cache.table.view(torch.int16).cpu().numpy().view(np.uint16)[live],
                                           ref["table"][live])
-        assert (ref["s2f"] != -1).sum() > 0
+        assert (ref["s2f"] != -1).sum() > 0 and n_stale > 0
+
+
+def test_ring_cache_refreshes_stale_entries_with_recomputed_values():
+    """An entry that reaches the age limit is reported absent at lookup, so the model recomputes the
+    row and the admission stores the NEW value in a new slot; an entry below the limit is served from
+    the table and is not re-admitted.  Driven with the model's own history-layer output."""
+    from hiscache import HistorySAGE, PinnedFeatureStore, RingHistoryCache, make_config
+    from hiscache.synthetic import make_batch
+    rng = np.random.default_rng(66)
+    torch.manual_seed(66)
+    N, Fin, H, C, L = 2000, 64, 64, 4, 3       # 3 layers: the history layer's input depends on weights
+    feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32))
+    cache = RingHistoryCache(PinnedFeatureStore(feats, device=DEV), N, Fin, H, capacity=4000, num_layers=L,
+                             table_dtype=torch.float32, thres=1e9, age_limit=2, device=DEV)   # every row passes
+    model = HistorySAGE(Fin, H, C, L, 0.0, "CSR_Layer", make_config(Fin, C, H, L, device=DEV), cache).to(DEV)
+    model.train()
+    opt = torch.optim.SGD(model.parameters(), lr=0.5)
+    b = layered_batch(rng, N, 30, [5, 4, 3])
+    batch = make_batch(b, rng.integers(0, C, size=N), DEV)
+    n1 = int(b["num_node_in_layer"][1])
+    stored, slots = [], []
+    for it in range(1, 5):
+        cache.lookup_and_load(batch, L)
+        hit = (cache.sub2embed != -1).cpu().numpy()
+        out = model(batch)
+        loss = torch.nn.functional.nll_loss(out, batch.y)
+        opt.zero_grad()
+        loss.backward()
+        opt.step()
+        pe = cache.produced_embedding.detach().clone()
+        cache.update_history(batch, it)
+        mask = cache.last_record_mask.cpu().numpy()
+        f2s = cache.full2slot[batch.sub_to_full[:n1]].cpu().numpy()
+        tab = cache.table[torch.from_numpy(np.maximum(f2s, 0)).to(DEV)].cpu().numpy()
+        if it == 1:                       # nothing cached: everything is computed and admitted
+            assert not hit.any() and mask.all()
+        elif it == 2:                     # age 1 < 2: served from the table, nothing re-admitted
+            assert hit.all() and not mask.any()
+            np.testing.assert_array_equal(pe.cpu().numpy(), stored[0])
+            np.testing.assert_array_equal(f2s, slots[0])
+        elif it == 3:                     # age 2: stale -> recomputed with the trained weights, re-admitted
+            assert not hit.any() and mask.all()
+            assert (f2s != slots[0]).all()
+            assert np.abs(pe.cpu().numpy() - stored[0]).max() > 1e-4     # the fresh value differs
+        np.testing.assert_array_equal(tab, pe.cpu().numpy() if mask.all() else stored[-1])
+        stored.append(tab.copy())
+        slots.append(f2s.copy())
 
 
 def test_input_layer_backward_is_skipped_but_history_grad_is_kept():

@@ -79,6 +79,9 @@ def test_aggregation_and_admission_replay_like_eager(be):
         torch.cuda.synchronize()
         for name, a, b in zip(("out", "ptrT", "rowT", "grad_x", "grad_h", "mask", "score", "rows", "found", "used"),
                               captured, eager):
+            if name == "rowT":                     # only the first ptrT[-1] entries are defined
+                n_tr = int(eager[1][-1])
+                a, b = a[:n_tr], b[:n_tr]
             assert torch.equal(a, b), (rep, name)
         for k in st_eager:
             assert torch.equal(st_graph[k], st_eager[k]), (rep, k)

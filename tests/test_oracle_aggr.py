@@ -82,6 +82,36 @@ def test_fwd_src_mode(orc):
     np.testing.assert_allclose(out, t.numpy(), rtol=1e-5, atol=1e-6)
 
 
+def test_bwd_src_mode_routes_gradients_like_autograd(orc):
+    """Per-source substitution, backward: pinned by torch autograd of the dense fp64 statement
+    out = D^-1 A where(hit, hist[hmap], feat).  A substituted source leaves feat.grad[s] = 0 and sends
+    its share to hist.grad[hmap[s]]; table rows shared by several sources add up."""
+    rng = np.random.default_rng(41)
+    R, N, F, Hn = 30, 40, 8, 9
+    ptr, idx = random_csr(rng, R, N, 7)
+    hmap = np.full(N, -1, np.int64)
+    hit = rng.random(N) < 0.5
+    hmap[hit] = rng.integers(0, Hn, size=int(hit.sum()))        # 20 sources onto 9 rows: rows are shared
+    g = rng.standard_normal((R, F)).astype(np.float32)
+    feat = torch.from_numpy(rng.standard_normal((N, F))).requires_grad_(True)
+    hist = torch.from_numpy(rng.standard_normal((Hn, F))).requires_grad_(True)
+    hm = torch.from_numpy(hmap)
+    rows = torch.where((hm != -1)[:, None], hist[hm.clamp(min=0)], feat)
+    deg = np.diff(ptr)
+    A = torch.zeros(R, N, dtype=torch.float64)
+    for r in range(R):
+        for j in range(ptr[r], ptr[r + 1]):
+            A[r, idx[j]] += 1.0 / deg[r]
+    (A @ rows).backward(torch.from_numpy(g).double())
+    gf, gh = orc.bwd_mean_src(ptr, idx, g, N, hmap_src=hmap, hist_shape=(Hn, F))
+    np.testing.assert_allclose(gf, feat.grad.numpy(), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(gh, hist.grad.numpy(), rtol=1e-5, atol=1e-6)
+    assert (gf[hit] == 0).all() and np.abs(gh).sum() > 0
+    # without a map: the gradient of whichever row was read
+    np.testing.assert_allclose(orc.bwd_mean_src(ptr, idx, g, N), (A.T @ torch.from_numpy(g).double()).numpy(),
+                               rtol=1e-5, atol=1e-6)
+
+
 @pytest.mark.parametrize("seed", [5, 6])
 def test_bwd_mean_closed_form_and_adjoint(orc, seed):
     rng = np.random.default_rng(seed)
@@ -302,5 +332,10 @@ def test_multithreaded_cpu_statement_equals_the_sequential_one(orc):
         for chunk in (0, 512):
             np.testing.assert_array_equal(mt.bwd_mean(ptr, ptrT, rowT, g, N, chunk=chunk),
                                           orc.bwd_mean_src(ptr, idx, g, N, chunk=chunk))
+        # the view without the substituted sources: their gradient rows are zero, the others keep their bits
+        ptrS, rowS = mt.build_transpose(ptr, idx, N, hmap_src=smap)
+        np.testing.assert_array_equal(np.diff(ptrS), np.where(smap == -1, np.diff(ptrT), 0))
+        np.testing.assert_array_equal(mt.bwd_mean(ptr, ptrS, rowS, g, N, chunk=512),
+                                      orc.bwd_mean_src(ptr, idx, g, N, chunk=512, hmap_src=smap)[0])
     with pytest.raises(ValueError):
         mt.build_transpose(np.array([0, 1]), np.array([5]), 3)
