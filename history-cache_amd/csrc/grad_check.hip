@@ -14,7 +14,8 @@
 // k-th admitted row (in row order) gets slot (header + k) mod capacity:
 //   pass 1  score + predicate per row, mask byte, admitted count per 64-row tile
 //   pass 2  one block scans the counts of 32-tile chunks (exclusive), advances the header
-//   pass 3  per tile: ballot-rank the mask, un-map old owners, copy rows, map
+//           (calls of up to 65 536 rows go without it: pass 3 adds the tile counts up itself)
+//   pass 3  per tile: ballot-rank the mask, un-map old owners, map, copy rows
 // Pass 1 is the only pass that touches the gradient matrix; pass 3 only touches
 // admitted rows, so HBM traffic is the algorithmic minimum.
 #include "hc_common.h"
@@ -123,8 +124,11 @@ __global__ __launch_bounds__(HC_BLOCK) void gc_pass1(
     const float *__restrict__ grad, const float *__restrict__ score_in, const int64_t *__restrict__ slot,
     const int32_t *__restrict__ age, const uint8_t *__restrict__ used, const float *__restrict__ thres_p,
     int32_t age_limit, int norm_kind, int cmp_kind, uint8_t *__restrict__ mask_out,
-    float *__restrict__ score_out, uint8_t *__restrict__ tile_counts, int64_t M, int64_t F) {
+    float *__restrict__ score_out, uint8_t *__restrict__ tile_counts, int64_t M, int64_t F,
+    const int64_t *__restrict__ header, GcScalars *__restrict__ scalars) {
   __shared__ int wave_cnt[HC_WAVES_PER_BLOCK];
+  // without a pass 2 (small calls) pass 3 takes the header from here: nothing changes it in between
+  if (PRED && scalars != nullptr && blockIdx.x == 0 && threadIdx.x == 0) scalars->header_old = header[0];
   const int lane = hc_lane();
   const int wave = hc_wave_in_block();
   const int64_t row0 = (int64_t)blockIdx.x * GC_TILE + wave * GC_ROWS_PER_WAVE;
@@ -296,60 +300,183 @@ __device__ __forceinline__ int64_t tile_offset(const uint8_t *__restrict__ tile_
 }
 
 // ---------------------------------------------------------------------------------------
-// Pass 3 (ring): per tile, rank the admitted rows, un-map old owners, copy, map.
+// Pass 3 (ring): per tile, rank the admitted rows, un-map old owners, map, copy.
+// The map work of a tile is done by the lanes of wave 0 side by side (one row per lane): the
+// slots of a tile's admitted rows are consecutive, so their previous owners are one coalesced
+// read, and the un-map compare-and-swaps of the whole tile are in flight together instead of
+// one dependent chain per row in front of its copy.  The four waves then copy the admitted
+// rows, GC_COPY_ROWS rows in flight per wave.
+// SMALL: there was no pass 2 (at most GC_SMALL_TILES tiles): every block adds up the tile counts in
+// front of its own tile itself, and block 0 advances the header.
 // ---------------------------------------------------------------------------------------
+constexpr int GC_COPY_ROWS = 4;
+constexpr int GC_SMALL_TILES = 1024;   // 65 536 rows
+
+// Sum of the four bytes of every word of v.
+__device__ __forceinline__ int byte_sum4(uint4 v) {
+  int t = 0;
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint32_t s2 = (w[k] & 0x00ff00ffu) + ((w[k] >> 8) & 0x00ff00ffu);
+    t += (int)((s2 & 0xffffu) + (s2 >> 16));
+  }
+  return t;
+}
+
+// Rows of the tile copied by the calling wave: admitted rows of rank q0, q0+1, ... (GC_COPY_ROWS at a
+// time, all loads in front of the stores); src_lane[j] (held by lane j) is the tile row of rank j.
+template <typename TT, int CH>
+__device__ __forceinline__ void copy_rows_fast(const float *__restrict__ emb, TT *__restrict__ table,
+                                               int src_lane, int64_t tile0, int64_t slot0, int64_t capacity,
+                                               int first_rank, int n_adm, int wave, int lane) {
+  constexpr int F = 256 * CH;
+  for (int q0 = first_rank + wave * GC_COPY_ROWS; q0 < n_adm; q0 += HC_WAVES_PER_BLOCK * GC_COPY_ROWS) {
+    float v[GC_COPY_ROWS][CH][4];
+#pragma unroll
+    for (int u = 0; u < GC_COPY_ROWS; ++u) {
+      if (q0 + u < n_adm) {
+        const int rl = __builtin_amdgcn_readlane(src_lane, q0 + u);
+        const float *p = emb + (tile0 + rl) * F + lane * 4;
+#pragma unroll
+        for (int k = 0; k < CH; ++k) hc_vec<float, 4>::load_nt(p + k * 256, v[u][k]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < GC_COPY_ROWS; ++u) {
+      if (q0 + u < n_adm) {
+        const int64_t s = (slot0 + q0 + u) % capacity;
+        TT *d = table + s * F + lane * 4;
+#pragma unroll
+        for (int k = 0; k < CH; ++k) hc_vec<TT, 4>::store_nt(d + k * 256, v[u][k]);
+      }
+    }
+  }
+}
+
+// No barrier and no LDS: every wave of the block reads the tile's 64 mask bytes and offsets itself, so
+// its first row loads are issued one memory round trip after the wave starts.
+template <bool SMALL>
 __global__ __launch_bounds__(HC_BLOCK) void gc_pass3_ring(
     const uint8_t *__restrict__ mask, const uint8_t *__restrict__ tile_counts,
     const int64_t *__restrict__ chunk_prefix, const GcScalars *__restrict__ sc, const float *__restrict__ emb,
     const int64_t *__restrict__ sub_to_full, void *__restrict__ table, int table_dtype, int64_t capacity,
     int64_t *__restrict__ full2slot, int64_t *__restrict__ slot2full, int64_t *__restrict__ checkin,
-    int64_t *__restrict__ slot_out, int64_t glb_iter, int64_t M, int64_t F) {
-  __shared__ int local_rows[GC_TILE];
-  __shared__ int n_admitted_s;
+    int64_t *__restrict__ slot_out, int64_t *__restrict__ header, int64_t glb_iter, int64_t M, int64_t F,
+    int64_t n_tiles) {
   const int lane = hc_lane();
   const int wave = hc_wave_in_block();
   const int64_t tile0 = (int64_t)blockIdx.x * GC_TILE;
+  const int64_t r = tile0 + lane;
+  // everything that does not depend on anything else is requested first
+  const bool m = r < M && mask[r] != 0;
+  const int64_t full = (wave == 0 && r < M) ? sub_to_full[r] : 0;
   const int64_t header_old = sc->header_old;
-  const int64_t A = sc->admitted;
-  const int64_t tile_off = tile_offset(tile_counts, chunk_prefix, (int64_t)blockIdx.x);
-  if (wave == 0) {
-    const int64_t r = tile0 + lane;
-    const bool m = r < M && mask[r] != 0;
-    const unsigned long long bal = __ballot(m);
-    const int rank = __popcll(bal & ((1ull << lane) - 1ull));
-    if (m) local_rows[rank] = lane;
-    if (lane == 0) n_admitted_s = __popcll(bal);
-    if (slot_out != nullptr && r < M)
-      slot_out[r] = m ? (header_old + tile_off + rank) % capacity : -1;
-  }
-  __syncthreads();
-  const int n_adm = n_admitted_s;
-  const int64_t first_live = A > capacity ? A - capacity : 0;  // ranks below are overwritten later
-  for (int q = wave; q < n_adm; q += HC_WAVES_PER_BLOCK) {
-    const int64_t r = tile0 + local_rows[q];
-    const int64_t k = tile_off + q;
-    const int64_t full = sub_to_full[r];
-    if (k < first_live) {
-      // Inserted and evicted again within this call: net effect is "not cached".
-      if (lane == 0) store_relaxed(full2slot + full, -1);
-      continue;
+  int64_t A, tile_off;
+  if constexpr (SMALL) {
+    // at most 1 024 tile counts of one byte: 16 per lane, summed over the wave
+    const int64_t t0 = (int64_t)lane * 16;
+    uint4 c = make_uint4(0u, 0u, 0u, 0u);
+    if (t0 + 16 <= n_tiles) {
+      c = *reinterpret_cast<const uint4 *>(tile_counts + t0);   // the count array is 16-byte aligned and padded
+    } else {
+      uint32_t w[4] = {0u, 0u, 0u, 0u};
+      for (int k = 0; k < 16; ++k)
+        if (t0 + k < n_tiles) w[k / 4] |= (uint32_t)tile_counts[t0 + k] << (8 * (k % 4));
+      c = make_uint4(w[0], w[1], w[2], w[3]);
     }
-    const int64_t s = (header_old + k) % capacity;
-    if (lane == 0) {
-      const int64_t old = slot2full[s];
-      if (old != -1) {
-        unsigned long long expect = (unsigned long long)s;
-        __hip_atomic_compare_exchange_strong(reinterpret_cast<unsigned long long *>(full2slot + old),
-                                             &expect, (unsigned long long)(int64_t)-1, __ATOMIC_RELAXED,
-                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    int all = byte_sum4(c);
+    // counts of the tiles in front of this block's tile
+    const int64_t mine = (int64_t)blockIdx.x;
+    int before = 0;
+    if (t0 + 16 <= mine) {
+      before = all;
+    } else if (t0 < mine) {
+      const int nb = (int)(mine - t0);   // 1..15 leading bytes
+      const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+      for (int k = 0; k < 4; ++k) {
+        const int n = nb - 4 * k;
+        const uint32_t msk = n >= 4 ? 0xffffffffu : (n <= 0 ? 0u : ((1u << (8 * n)) - 1u));
+        const uint32_t v = w[k] & msk;
+        const uint32_t s2 = (v & 0x00ff00ffu) + ((v >> 8) & 0x00ff00ffu);
+        before += (int)((s2 & 0xffffu) + (s2 >> 16));
       }
     }
-    store_row_any(emb + r * F, table, table_dtype, s * F, F, lane);
-    if (lane == 0) {
-      store_relaxed(full2slot + full, s);
-      slot2full[s] = full;
-      if (checkin != nullptr) checkin[s] = glb_iter;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+      before += __shfl_xor(before, d, HC_WAVE);
+      all += __shfl_xor(all, d, HC_WAVE);
     }
+    tile_off = before;
+    A = all;
+    // nobody reads the header in this launch (pass 1 left its value in sc->header_old)
+    if (blockIdx.x == 0 && threadIdx.x == 0) header[0] = (header_old + A) % capacity;
+  } else {
+    A = sc->admitted;
+    tile_off = tile_offset(tile_counts, chunk_prefix, (int64_t)blockIdx.x);
+  }
+  const unsigned long long bal = __ballot(m);
+  const int n_adm = __popcll(bal);
+  if (n_adm == 0 && slot_out == nullptr) return;
+  const unsigned long long below = (1ull << lane) - 1ull;
+  const int rank = __popcll(bal & below);
+  const int64_t first_live = A > capacity ? A - capacity : 0;   // ranks below are overwritten later in this call
+  // ranks of this tile that are dead on arrival: a prefix of the tile's ranks
+  const int64_t dead64 = first_live - tile_off;
+  const int first_rank = dead64 <= 0 ? 0 : (dead64 >= n_adm ? n_adm : (int)dead64);
+  const int64_t slot0 = header_old + tile_off;                   // slot of rank q is (slot0 + q) % capacity
+
+  if (wave == 0) {
+    // the tile's map work, one row per lane: consecutive slots, so the previous owners are one
+    // coalesced read and the un-map compare-and-swaps of the whole tile are in flight together
+    if (m) {
+      if (rank < first_rank) {
+        // inserted and evicted again within this call: net effect is "not cached"
+        store_relaxed(full2slot + full, -1);
+      } else {
+        const int64_t s = (slot0 + rank) % capacity;
+        const int64_t old = slot2full[s];
+        if (old != -1) {
+          unsigned long long expect = (unsigned long long)s;
+          __hip_atomic_compare_exchange_strong(reinterpret_cast<unsigned long long *>(full2slot + old),
+                                               &expect, (unsigned long long)(int64_t)-1, __ATOMIC_RELAXED,
+                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // The un-map above and this store may land in either order when `old` is this call's own node of
+        // another row: the compare-and-swap only clears an entry that still names the slot, so the new
+        // mapping survives both orders.  This row's own node and slot are touched by this lane only.
+        store_relaxed(full2slot + full, s);
+        slot2full[s] = full;
+        if (checkin != nullptr) checkin[s] = glb_iter;
+      }
+    }
+    if (slot_out != nullptr && r < M) slot_out[r] = m ? (slot0 + rank) % capacity : -1;
+  }
+  if (n_adm == 0) return;
+  // lane j learns which tile row has rank j: admitted lanes push their lane number to lane `rank`,
+  // the others to the lanes behind the admitted ones (a permutation of the 64 lanes)
+  const int target = m ? rank : n_adm + (lane - rank);
+  const int src_lane = __builtin_amdgcn_ds_permute(target << 2, lane);
+  const bool fast = (F % 256 == 0) && (F / 256 <= 4) && (reinterpret_cast<uintptr_t>(emb) % 16 == 0) &&
+                    (reinterpret_cast<uintptr_t>(table) % 16 == 0);
+  if (fast) {
+#define HC_COPY(TT)                                                                                              \
+  switch (F / 256) {                                                                                             \
+    case 1: copy_rows_fast<TT, 1>(emb, static_cast<TT *>(table), src_lane, tile0, slot0, capacity, first_rank, n_adm, wave, lane); break; \
+    case 2: copy_rows_fast<TT, 2>(emb, static_cast<TT *>(table), src_lane, tile0, slot0, capacity, first_rank, n_adm, wave, lane); break; \
+    case 3: copy_rows_fast<TT, 3>(emb, static_cast<TT *>(table), src_lane, tile0, slot0, capacity, first_rank, n_adm, wave, lane); break; \
+    default: copy_rows_fast<TT, 4>(emb, static_cast<TT *>(table), src_lane, tile0, slot0, capacity, first_rank, n_adm, wave, lane); break; \
+  }
+    if (table_dtype == HC_F32) { HC_COPY(float) }
+    else if (table_dtype == HC_F16) { HC_COPY(__half) }
+    else { HC_COPY(__hip_bfloat16) }
+#undef HC_COPY
+    return;
+  }
+  for (int q = first_rank + wave; q < n_adm; q += HC_WAVES_PER_BLOCK) {
+    const int rl = __builtin_amdgcn_readlane(src_lane, q);
+    const int64_t s = (slot0 + q) % capacity;
+    store_row_any(emb + (tile0 + rl) * F, table, table_dtype, s * F, F, lane);
   }
 }
 
@@ -440,7 +567,7 @@ template <bool PRED>
 int launch_pass1(const float *grad, const float *score_in, const int64_t *slot, const int32_t *age,
                  const uint8_t *used, const float *thres, int32_t age_limit, int norm_kind, int cmp_kind,
                  uint8_t *mask_out, float *score_out, uint8_t *tile_counts, int64_t M, int64_t F,
-                 hipStream_t st) {
+                 hipStream_t st, const int64_t *header = nullptr, GcScalars *sc = nullptr) {
   const int64_t tiles = (M + GC_TILE - 1) / GC_TILE;
   if (!hc_grid_ok(tiles)) return HC_EUNSUPPORTED;
   dim3 g((unsigned)tiles), b(HC_BLOCK);
@@ -448,7 +575,7 @@ int launch_pass1(const float *grad, const float *score_in, const int64_t *slot, 
                     (reinterpret_cast<uintptr_t>(grad) % 16 == 0);
 #define HC_P1(CH)                                                                                    \
   gc_pass1<CH, PRED><<<g, b, 0, st>>>(grad, score_in, slot, age, used, thres, age_limit, norm_kind,  \
-                                      cmp_kind, mask_out, score_out, tile_counts, M, F)
+                                      cmp_kind, mask_out, score_out, tile_counts, M, F, header, sc)
   if (fast && F == 256) HC_P1(1);
   else if (fast && F == 512) HC_P1(2);
   else if (fast && F == 768) HC_P1(3);
@@ -497,15 +624,23 @@ extern "C" int hc_grad_check(const float *grad, const float *score_in, const flo
   uint8_t *tiles_buf = reinterpret_cast<uint8_t *>(workspace) + L.counts;
   const int64_t tiles = (M + GC_TILE - 1) / GC_TILE;
 
+  const bool small = tiles <= GC_SMALL_TILES;
   int rc = launch_pass1<true>(grad, score_in, slot, age, used, thres, age_limit, norm_kind, cmp_kind,
-                              mask_out, score_out, tiles_buf, M, F, st);
+                              mask_out, score_out, tiles_buf, M, F, st, header, small ? sc : nullptr);
   if (rc != HC_OK) return rc;
+  if (small) {
+    // two launches: every pass-3 block adds up the (at most 1 024) tile counts in front of it itself
+    gc_pass3_ring<true><<<dim3((unsigned)tiles), dim3(HC_BLOCK), 0, st>>>(
+        mask_out, tiles_buf, chunk_prefix, sc, emb, sub_to_full, table, table_dtype, capacity, full2slot, slot2full,
+        checkin, slot_out, header, glb_iter, M, F, tiles);
+    return hc_launch_status();
+  }
   gc_pass2<<<dim3(1), dim3(GC_SCAN_THREADS), 0, st>>>(tiles_buf, tiles, chunk_prefix, sc, header, capacity, 1,
                                                       nullptr);
   if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
-  gc_pass3_ring<<<dim3((unsigned)tiles), dim3(HC_BLOCK), 0, st>>>(
+  gc_pass3_ring<false><<<dim3((unsigned)tiles), dim3(HC_BLOCK), 0, st>>>(
       mask_out, tiles_buf, chunk_prefix, sc, emb, sub_to_full, table, table_dtype, capacity, full2slot, slot2full,
-      checkin, slot_out, glb_iter, M, F);
+      checkin, slot_out, header, glb_iter, M, F, tiles);
   return hc_launch_status();
 }
 
