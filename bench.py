@@ -47,6 +47,8 @@ def parse():
     ap.add_argument("--heads", type=int, default=1, help="c2w: heads of the weighted aggregation (divides 256)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="c2: skip the c4 and batched-c3 kernel figures that the default run adds to its line")
     return ap.parse_args()
 
 
@@ -436,6 +438,99 @@ def run_c4(args):
 
 
 # ----------------------------------------------------------------------------------------- C3
+def c3_batched_layer(args, samples=None):
+    """The papers100M-shaped history layer for about 800 batches side by side (about 20 M edges): forward with
+    per-row substitution from an fp16 row-aligned buffer, transposed-view build, backward, fused admission of the
+    produced rows into an fp16 ring.  The roofline fraction counts the algorithmic bytes of forward, backward and
+    admission over the time of all four steps (the transposed-view build is in the time, not in the bytes)."""
+    import numpy as np
+    import torch
+
+    import hiscache_backend as be
+    from hiscache.synthetic import direct_power_law_batch, lognormal_grads
+
+    dev = "cuda:0"
+    s = args.scale
+    N, H = int(111_000_000 * s), 256
+    if samples is None:
+        samples = [direct_power_law_batch(N, 1000, [15, 10, 5], 2.0, 30 + i, degree_scale=2.6) for i in range(8)]
+    n_pre = len(samples)
+    gen = torch.Generator(device=dev).manual_seed(33)
+    rows, cols, ptrs, idxs, hms = 0, 0, [np.zeros(1, np.int64)], [], []
+    k = 0
+    e_tot = 0
+    target = int(20_000_000 * s)
+    while e_tot < target:
+        smp = samples[k % min(8, n_pre)]
+        n1, n2 = int(smp["num_node_in_layer"][1]), int(smp["num_node_in_layer"][2])
+        p = smp["ptr"][: n1 + 1]
+        e = int(p[-1])
+        ptrs.append(p[1:] + e_tot)
+        idxs.append(smp["idx"][:e] + cols)
+        e_tot += e
+        rows += n1
+        cols += n2
+        k += 1
+    ptr = torch.from_numpy(np.concatenate(ptrs)).to(dev)
+    idx = torch.from_numpy(np.concatenate(idxs)).to(dev)
+    R, E, Nsrc = rows, e_tot, cols
+    x = torch.randn(Nsrc, H, device=dev, generator=gen)
+    hbuf = (0.5 * torch.randn(R, H, device=dev, generator=gen)).half()
+    hmap = torch.where(torch.rand(R, device=dev, generator=gen) < 0.35, torch.arange(R, device=dev),
+                       torch.full((R,), -1, device=dev))
+    g = torch.randn(R, H, device=dev, generator=gen)
+    grad = lognormal_grads(R, H, -3.0, 1.5, device=dev, generator=gen)
+    emb = torch.randn(R, H, device=dev, generator=gen)
+    cap = max(R, 1 << 20)
+    table = torch.zeros(cap, H, dtype=torch.float16, device=dev)
+    f2s = torch.full((2 * R,), -1, dtype=torch.int64, device=dev)
+    s2f = torch.full((cap,), -1, dtype=torch.int64, device=dev)
+    chk = torch.full((cap,), -1, dtype=torch.int64, device=dev)
+    hdr = torch.zeros(1, dtype=torch.int64, device=dev)
+    sub_to_full = torch.randperm(2 * R, device=dev, generator=gen)[:R].contiguous()
+    thr = torch.tensor([0.05], device=dev)
+    cf, ct, cb, cg = KernelClock(), KernelClock(), KernelClock(), KernelClock()
+    st = {}
+
+    def kstep():
+        cf(lambda: be._aggr_fwd(be.SUBST_ROW, ptr, idx, x, hmap, hbuf, H, None, R))
+        tr = ct(lambda: be.build_transpose(ptr, idx, hmap, R, Nsrc, want_edges=False))
+        cb(lambda: be._aggr_bwd(ptr, idx, tr, g, hmap, None, x, False, (R, H), H, R, Nsrc))
+        hdr.zero_()
+        st["mask"] = cg(lambda: be.grad_check(grad, emb, hmap, sub_to_full, thr, table, f2s, s2f, hdr, 1,
+                                              checkin=chk))[0]
+
+    for _ in range(args.warmup):
+        kstep()
+    sync()
+    for c in (cf, ct, cb, cg):
+        c.reset()
+    for _ in range(args.steps):
+        kstep()
+    sync()
+    t_f, t_t, t_b, t_g = cf.mean_ms(), ct.mean_ms(), cb.mean_ms(), cg.mean_ms()
+    n_hist = int((hmap != -1).sum())
+    deg = ptr[1:] - ptr[:-1]
+    e_nh = int(deg[hmap == -1].sum())
+    A = int(st["mask"].sum())
+    bytes_f = (R + 1) * 8 + R * 8 + e_nh * 8 + e_nh * H * 4 + n_hist * H * 2 + R * H * 4
+    bytes_b = e_nh * H * 4 + e_nh * 8 + (Nsrc + 1) * 8 + R * 4 + Nsrc * H * 4 + 2 * n_hist * H * 4
+    bytes_g = R * H * 4 + R * 13 + R + A * (H * 4 + H * 2 + 32)
+    tot_b, tot_t = bytes_f + bytes_b + bytes_g, (t_f + t_t + t_b + t_g) * 1e-3
+    detail = {
+        "rows": R, "edges": E, "sources": Nsrc, "history_rows": n_hist, "admitted": A,
+        "fwd_ms": t_f, "transpose_ms": t_t, "bwd_ms": t_b, "grad_check_ms": t_g,
+        "fwd_GBps": bytes_f / t_f / 1e6, "bwd_GBps": bytes_b / t_b / 1e6, "grad_check_GBps": bytes_g / t_g / 1e6,
+        "edges_per_s_fwd_bwd": E / ((t_f + t_t + t_b) * 1e-3),
+        "algorithmic_bytes": tot_b, "ms": tot_t * 1e3, "frac": tot_b / tot_t / 1e9 / HBM_PEAK_GBS,
+    }
+    roofline = {"bound": "hbm",
+                "kernel": "fwd_mean_fast + transposed view + bwd_mean_fast + gc_pass1..3 (batched history layer)",
+                "achieved": tot_b / tot_t / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": tot_b / tot_t / 1e9 / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": tot_b}
+    return {"detail": detail, "roofline": roofline}
+
+
 def run_c3(args):
     """papers100M-shaped training iteration (one GPU's share at its real batch shape) and a batched
     variant of its history layer (many batches side by side) for the kernels' asymptotic rate."""
@@ -568,69 +663,7 @@ def run_c3(args):
         shape = {k: int(np.mean([int(x["num_node_in_layer"][i]) for x in samples])) for i, k in enumerate(("n0", "n1", "n2", "n3"))}
         shape["edges"] = int(np.mean([x["idx"].size for x in samples]))
 
-    # ---- batched variant of the history layer: K batches side by side, about 20M edges
-    rows, cols, ptrs, idxs, hms = 0, 0, [np.zeros(1, np.int64)], [], []
-    k = 0
-    e_tot = 0
-    target = int(20_000_000 * s)
-    while e_tot < target:
-        smp = samples[k % min(8, n_pre)]
-        n1, n2 = int(smp["num_node_in_layer"][1]), int(smp["num_node_in_layer"][2])
-        p = smp["ptr"][: n1 + 1]
-        e = int(p[-1])
-        ptrs.append(p[1:] + e_tot)
-        idxs.append(smp["idx"][:e] + cols)
-        e_tot += e
-        rows += n1
-        cols += n2
-        k += 1
-    ptr = torch.from_numpy(np.concatenate(ptrs)).to(dev)
-    idx = torch.from_numpy(np.concatenate(idxs)).to(dev)
-    R, E, Nsrc = rows, e_tot, cols
-    x = torch.randn(Nsrc, H, device=dev, generator=gen)
-    hbuf = (0.5 * torch.randn(R, H, device=dev, generator=gen)).half()
-    hmap = torch.where(torch.rand(R, device=dev, generator=gen) < 0.35, torch.arange(R, device=dev),
-                       torch.full((R,), -1, device=dev))
-    g = torch.randn(R, H, device=dev, generator=gen)
-    from hiscache.synthetic import lognormal_grads
-    grad = lognormal_grads(R, H, -3.0, 1.5, device=dev, generator=gen)
-    emb = torch.randn(R, H, device=dev, generator=gen)
-    cap = max(R, 1 << 20)
-    table = torch.zeros(cap, H, dtype=torch.float16, device=dev)
-    f2s = torch.full((2 * R,), -1, dtype=torch.int64, device=dev)
-    s2f = torch.full((cap,), -1, dtype=torch.int64, device=dev)
-    chk = torch.full((cap,), -1, dtype=torch.int64, device=dev)
-    hdr = torch.zeros(1, dtype=torch.int64, device=dev)
-    sub_to_full = torch.randperm(2 * R, device=dev, generator=gen)[:R].contiguous()
-    thr = torch.tensor([0.05], device=dev)
-    cf, ct, cb, cg = KernelClock(), KernelClock(), KernelClock(), KernelClock()
-    st = {}
-
-    def kstep():
-        cf(lambda: be._aggr_fwd(be.SUBST_ROW, ptr, idx, x, hmap, hbuf, H, None, R))
-        tr = ct(lambda: be.build_transpose(ptr, idx, hmap, R, Nsrc, want_edges=False))
-        cb(lambda: be._aggr_bwd(ptr, idx, tr, g, hmap, None, x, False, (R, H), H, R, Nsrc))
-        hdr.zero_()
-        st["mask"] = cg(lambda: be.grad_check(grad, emb, hmap, sub_to_full, thr, table, f2s, s2f, hdr, 1,
-                                              checkin=chk))[0]
-
-    for _ in range(args.warmup):
-        kstep()
-    sync()
-    for c in (cf, ct, cb, cg):
-        c.reset()
-    for _ in range(args.steps):
-        kstep()
-    sync()
-    t_f, t_t, t_b, t_g = cf.mean_ms(), ct.mean_ms(), cb.mean_ms(), cg.mean_ms()
-    n_hist = int((hmap != -1).sum())
-    deg = ptr[1:] - ptr[:-1]
-    e_nh = int(deg[hmap == -1].sum())
-    A = int(st["mask"].sum())
-    bytes_f = (R + 1) * 8 + R * 8 + e_nh * 8 + e_nh * H * 4 + n_hist * H * 2 + R * H * 4
-    bytes_b = e_nh * H * 4 + e_nh * 8 + (Nsrc + 1) * 8 + R * 4 + Nsrc * H * 4 + 2 * n_hist * H * 4
-    bytes_g = R * H * 4 + R * 13 + R + A * (H * 4 + H * 2 + 32)
-    tot_b, tot_t = bytes_f + bytes_b + bytes_g, (t_f + t_b + t_g) * 1e-3
+    batched = c3_batched_layer(args, samples)
     return {
         "metric": "papers100M-shaped iteration ms (1 GPU)", "value": sec * 1e3, "unit": "ms", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": False,
@@ -642,15 +675,8 @@ def run_c3(args):
         "phases_host_enqueue_ms": {k: c.mean_cpu_ms() for k, c in ev.items()},
         "feature_rows_read_last_batch": int(cache.used_masks[0].sum()),
         "cached_1hop_fraction_last_batch": float((cache.sub2embed != -1).float().mean()),
-        "batched_history_layer": {
-            "rows": R, "edges": E, "sources": Nsrc, "history_rows": n_hist, "admitted": A,
-            "fwd_ms": t_f, "transpose_ms": t_t, "bwd_ms": t_b, "grad_check_ms": t_g,
-            "fwd_GBps": bytes_f / t_f / 1e6, "bwd_GBps": bytes_b / t_b / 1e6, "grad_check_GBps": bytes_g / t_g / 1e6,
-            "edges_per_s_fwd_bwd": E / ((t_f + t_b) * 1e-3),
-        },
-        "roofline": {"bound": "hbm", "kernel": "fwd_mean_fast + bwd_mean_fast + gc_pass1..3 (batched history layer)",
-                     "achieved": tot_b / tot_t / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": tot_b / tot_t / 1e9 / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": tot_b},
+        "batched_history_layer": batched["detail"],
+        "roofline": batched["roofline"],
     }
 
 
@@ -912,8 +938,21 @@ def main():
     be.load_library()
     if args.workload in ("c2", "c2row"):
         res, shape = run_c2(args, row_mode=(args.workload == "c2row"))
-        if not args.no_cpu_baseline:
+        torch.cuda.empty_cache()
+        if args.workload == "c2" and not args.headline_only:
+            # the two other kernel figures of the path, in the same line: the fused admission microbenchmark
+            # and the papers100M-shaped history layer batched to 20 M edges
+            c4 = run_c4(args)
             torch.cuda.empty_cache()
+            res["kernels"]["c4"] = {"workload": c4["config"]["workload"], "ms": c4["ms_per_step"],
+                                    "rows_per_s": c4["value"],
+                                    "algorithmic_bytes": c4["roofline"]["algorithmic_bytes"],
+                                    "GBps": c4["roofline"]["achieved"], "frac": c4["roofline"]["frac"],
+                                    "traffic": c4["roofline"]["traffic"]}
+            c3b = c3_batched_layer(args)["detail"]
+            torch.cuda.empty_cache()
+            res["kernels"]["c3_batched"] = c3b
+        if not args.no_cpu_baseline:
             res["cpu_baseline"] = cpu_baseline_c2(shape)
     elif args.workload == "c2w":
         res = run_c2w(args)

@@ -304,8 +304,16 @@ __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
   int64_t hi = lo + per;
   if (lo > n_src) lo = n_src;
   if (hi > n_src) hi = n_src;
+  // the loads of a run are issued eight at a time (one after the other they would cost a memory round
+  // trip each, and this block runs alone at the end of the launch)
   int sum = 0;
-  for (int64_t q = lo; q < hi; ++q) sum += trs_load(count + q);
+  for (int64_t q = lo; q < hi; q += 8) {
+    int c[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) c[k] = q + k < hi ? trs_load(count + q + k) : 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) sum += c[k];
+  }
   const int lane = hc_lane();
   const int wave = (int)(threadIdx.x >> 6);
   int x = sum;
@@ -319,11 +327,18 @@ __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
   int off = x - sum;
   for (int w = 0; w < wave; ++w) off += s_wave[w];
   int run = off;
-  for (int64_t q = lo; q < hi; ++q) {
-    const int c = trs_load(count + q);
-    ptrT[q] = run;
-    count[q] = run;   // the segment's cursor for tr_small_place
-    run += c;
+  for (int64_t q = lo; q < hi; q += 8) {
+    int c[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) c[k] = q + k < hi ? trs_load(count + q + k) : 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (q + k < hi) {
+        ptrT[q + k] = run;
+        count[q + k] = run;   // the segment's cursor for tr_small_place
+        run += c[k];
+      }
+    }
   }
   if (threadIdx.x == TRS_BLOCK - 1) ptrT[n_src] = run;
 }

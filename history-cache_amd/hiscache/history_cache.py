@@ -165,6 +165,11 @@ class HistoryCache:
             raise AssertionError("produced embedding is None")
         emb = self.produced_embedding
         num_node = emb.shape[0]
+        # the reference asserts the same against num_node_in_layer[1] (history_cache.py:200-204): an embedding
+        # produced by another layer must not reach the admission kernels
+        n1 = int(batch.num_node_in_layer[1])
+        if num_node != n1 or self.sub2embed is None or self.sub2embed.numel() < num_node:
+            raise ValueError("produced_embedding has {} rows, the batch has {} 1-hop nodes".format(num_node, n1))
         if emb.grad is not None and self.method == "grad":
             g = emb.grad
             assert g.shape[0] == num_node, "grad shape: {}, num_node: {}".format(g.shape, num_node)

@@ -34,11 +34,12 @@ class MySageConvHistory(torch.nn.Module):
         if self.root_weight:
             self.lin_r.reset_parameters()
 
-    def forward(self, x, ptr, idx, history_map, history_buffer, history_size, num_node):
+    def forward(self, x, ptr, idx, history_map, history_buffer, history_size, num_node, num_edge=None):
         num_node = int(num_node)
-        # history_size == 0 selects the plain mean inside the operator
+        # history_size == 0 selects the plain mean inside the operator; num_edge (optional, beyond the
+        # reference) bounds the edge slots of these rows inside the mini-batch's shared CSR
         out = hiscache_backend.aggr_forward_history(x, ptr, idx, history_map, history_buffer,
-                                                    history_size, num_node)
+                                                    history_size, num_node, num_edge)
         his = out
         if self.need_grad and self.training and history_size > 0:
             his.retain_grad()
@@ -71,19 +72,23 @@ class HistorySAGE(torch.nn.Module):
     def forward(self, batch):
         x = batch.x
         none = torch.empty(0, device=x.device)
+        nel = getattr(batch, "num_edge_in_layer", None)      # edges of the first num_node_in_layer[k] rows
         for i, conv in enumerate(self.convs[:-1]):
-            n = batch.num_node_in_layer[self.num_layers - 1 - i]
+            k = self.num_layers - 1 - i
+            n = batch.num_node_in_layer[k]
+            ne = None if nel is None else int(nel[k])
             if self.training and i == self.num_layers - 2:
                 # the layer whose output is one hop from the seeds uses (and produces) history
                 x, his = conv(x, batch.ptr, batch.idx, self.table.sub2embed,
-                              self.table.cached_embedding, self.hidden_channels, n)
+                              self.table.cached_embedding, self.hidden_channels, n, ne)
                 self.table.produced_embedding = his
             else:
-                x, his = conv(x, batch.ptr, batch.idx, none, none, 0, n)
+                x, his = conv(x, batch.ptr, batch.idx, none, none, 0, n, ne)
             x = self.bns[i](x)
             x = F.relu(x)
             x = F.dropout(x, p=self.dropout, training=self.training)
-        x, his = self.convs[-1](x, batch.ptr, batch.idx, none, none, 0, batch.num_node_in_layer[0])
+        x, his = self.convs[-1](x, batch.ptr, batch.idx, none, none, 0, batch.num_node_in_layer[0],
+                                None if nel is None else int(nel[0]))
         return x.log_softmax(dim=-1)
 
     def init_convs(self, **kwargs):
@@ -153,6 +158,9 @@ class MyRGCNConvHistory2(torch.nn.Module):
         self.hidden_channels = hidden_channels
         self.num_rel = num_rel
         self.linear = torch.nn.Parameter(torch.empty(num_rel, in_channels, hidden_channels))
+        # the reference registers the same tensor a second time under this name
+        # (/root/reference/hiscache/history_model.py:233-236), so its checkpoints hold both keys
+        self.register_parameter("rel_weight", self.linear)
         self.reset_parameters()
         self.need_grad = need_grad
 

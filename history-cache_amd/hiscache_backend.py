@@ -540,6 +540,10 @@ def grad_check(grad, emb, slot, sub_to_full, thres, table, full2slot, slot2full,
             raise ValueError("used must be bool")
     if checkin is not None:
         _dev(checkin, "checkin", torch.int64)
+    # every per-row argument must cover the M rows of emb: the kernels trust their lengths
+    for t, n in ((slot, "slot"), (sub_to_full, "sub_to_full"), (age, "age"), (used, "used"), (score, "score")):
+        if t is not None and t.numel() < M:
+            raise ValueError(f"{n} has {t.numel()} entries, emb has {M} rows")
     mask = torch.empty(M, dtype=torch.uint8, device=dev)
     score_out = torch.empty(M, dtype=torch.float32, device=dev)
     slot_out = torch.empty(M, dtype=torch.int64, device=dev) if want_slots else None
@@ -578,6 +582,9 @@ def cache_append(score, thres, emb, sub2embed, sub_to_full, buffer, hidden, in_c
     for t, n in ((sub2embed, "sub2embed"), (sub_to_full, "sub_to_full"), (full2embed, "full2embed"),
                  (embed2full, "embed2full"), (header, "header")):
         _dev(t, n, torch.int64)
+    for t, n in ((score, "score"), (sub2embed, "sub2embed"), (sub_to_full, "sub_to_full")):
+        if t.numel() < M:
+            raise ValueError(f"{n} has {t.numel()} entries, emb has {M} rows")
     if embed2full.numel() < capacity:
         capacity = embed2full.numel()
     n_feat = 0

@@ -6,8 +6,10 @@ Run in the build container only (the reference tree is not available elsewhere):
 
     python tests/golden/gen_history_cache_golden.py
 
-The reference module is loaded from /root/reference as text-and-exec by importlib; its package
-``__init__`` (which imports CUDA-only extensions) is not executed.  Two collaborators that do not
+The reference module's SOURCE TEXT is read from /root/reference, compiled and executed here (no
+importlib loader: a loader would prefer a ``__pycache__/*.pyc`` lying beside the source, and would
+write one if there was none); its package ``__init__`` (which imports CUDA-only extensions) is not
+executed.  Two collaborators that do not
 exist here are supplied as small stand-ins, and the fixture records which outputs depend on them:
   * ``hiscache.count_history_reconstruct`` -> this repo's CPU oracle (so ``used_masks`` and everything
     derived from it in lookup_and_load is NOT independent evidence; the id translation, the
@@ -17,7 +19,6 @@ exist here are supplied as small stand-ins, and the fixture records which output
 ``update_history`` needs neither: its golden vectors are produced by the reference code alone.
 Only inputs and outputs are stored; no reference source text is copied.
 """
-import importlib.util
 import logging
 import os
 import sys
@@ -49,10 +50,13 @@ def load_reference_class():
     saved = {k: sys.modules.get(k) for k in ("hiscache", "hiscache.util", "hiscache.history_cache")}
     sys.modules["hiscache"] = pkg
     sys.modules["hiscache.util"] = util
-    spec = importlib.util.spec_from_file_location("hiscache.history_cache", REF)
-    mod = importlib.util.module_from_spec(spec)
+    sys.dont_write_bytecode = True
+    mod = types.ModuleType("hiscache.history_cache")
+    mod.__file__ = REF
     sys.modules["hiscache.history_cache"] = mod
-    spec.loader.exec_module(mod)
+    with open(REF, "r", encoding="utf-8") as f:
+        code = compile(f.read(), REF, "exec")      # the source text itself, never cached bytecode
+    exec(code, mod.__dict__)
     for k, v in saved.items():
         if v is None:
             sys.modules.pop(k, None)

@@ -27,3 +27,20 @@ def layered_batch(rng, n_full, n_seed, fanout, avg_deg=8):
     indptr, indices = uniform_graph(n_full, avg_deg, int(rng.integers(1 << 30)))
     seeds = rng.choice(n_full, size=n_seed, replace=False)
     return sample_layered_batch(indptr, indices, seeds, fanout, rng)
+
+
+def power_law_graph(rng, num_nodes, degree_scale, alpha=2.0, max_degree=2000, popular=True):
+    """CSR of a directed graph with Zipf(alpha) out-degrees (scaled, capped) and neighbour ids skewed
+    towards popular nodes (a cubed uniform scattered by a multiplicative hash), multi-edges possible:
+    the shape of a citation graph, small enough to hold on the host."""
+    raw = np.minimum(rng.zipf(alpha, size=num_nodes), 1 << 20).astype(np.float64)
+    deg = np.minimum(np.floor(raw * degree_scale), max_degree).astype(np.int64)
+    indptr = np.zeros(num_nodes + 1, np.int64)
+    np.cumsum(deg, out=indptr[1:])
+    E = int(indptr[-1])
+    if popular:
+        u = rng.random(E)
+        indices = ((u * u * u * num_nodes).astype(np.int64) * 2654435761) % num_nodes
+    else:
+        indices = rng.integers(0, num_nodes, size=E, dtype=np.int64)
+    return indptr, indices.astype(np.int64)
