@@ -24,13 +24,14 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "history-cache_amd"))
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the dominant kernel at full size, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of this file (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000: factors from a 4 GiB device copy).
+# HBM bytes per launch at full size, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file (FETCH_SIZE
+# scaled by 2.000, WRITE_SIZE by 1.000: factors from a 4 GiB device copy; profiles/aggr_c2_hbm_traffic.md): the
+# forward gather of c2 / c2row, the three admission passes of c4, forward + backward + admission of the batched layer.
 # Age limit of the ring caches in the iteration workloads: entries preloaded at iteration 0 must stay valid
 # for the whole run so that the hit rate stays at the configuration's 35% (the age bound itself is exercised
 # by the c4 workload and by the tests).
 AGE_LIMIT_ITERS = 100_000
-MEASURED_TRAFFIC = {"c2": 24.21e9, "c2row": 13.93e9, "c4": 3.50e9}
+MEASURED_TRAFFIC = {"c2": 23.08e9, "c2row": 13.93e9, "c4": 3.48e9, "c3_batched": 51.94e9}
 
 
 def parse():
@@ -495,7 +496,8 @@ def c3_batched_layer(args, samples=None):
     def kstep():
         cf(lambda: be._aggr_fwd(be.SUBST_ROW, ptr, idx, x, hmap, hbuf, H, None, R))
         tr = ct(lambda: be.build_transpose(ptr, idx, hmap, R, Nsrc, want_edges=False))
-        cb(lambda: be._aggr_bwd(ptr, idx, tr, g, hmap, None, x, False, (R, H), H, R, Nsrc))
+        # as in the training iteration, the cached embeddings need no gradient: no grad_hbuf is written
+        cb(lambda: be._aggr_bwd(ptr, idx, tr, g, hmap, None, x, False, (R, H), H, R, Nsrc, want_hist_grad=False))
         hdr.zero_()
         st["mask"] = cg(lambda: be.grad_check(grad, emb, hmap, sub_to_full, thr, table, f2s, s2f, hdr, 1,
                                               checkin=chk))[0]
@@ -514,7 +516,7 @@ def c3_batched_layer(args, samples=None):
     e_nh = int(deg[hmap == -1].sum())
     A = int(st["mask"].sum())
     bytes_f = (R + 1) * 8 + R * 8 + e_nh * 8 + e_nh * H * 4 + n_hist * H * 2 + R * H * 4
-    bytes_b = e_nh * H * 4 + e_nh * 8 + (Nsrc + 1) * 8 + R * 4 + Nsrc * H * 4 + 2 * n_hist * H * 4
+    bytes_b = e_nh * H * 4 + e_nh * 8 + (Nsrc + 1) * 8 + R * 4 + Nsrc * H * 4
     bytes_g = R * H * 4 + R * 13 + R + A * (H * 4 + H * 2 + 32)
     tot_b, tot_t = bytes_f + bytes_b + bytes_g, (t_f + t_t + t_b + t_g) * 1e-3
     detail = {
@@ -523,6 +525,7 @@ def c3_batched_layer(args, samples=None):
         "fwd_GBps": bytes_f / t_f / 1e6, "bwd_GBps": bytes_b / t_b / 1e6, "grad_check_GBps": bytes_g / t_g / 1e6,
         "edges_per_s_fwd_bwd": E / ((t_f + t_t + t_b) * 1e-3),
         "algorithmic_bytes": tot_b, "ms": tot_t * 1e3, "frac": tot_b / tot_t / 1e9 / HBM_PEAK_GBS,
+        "traffic": MEASURED_TRAFFIC["c3_batched"] if s == 1.0 else None,
     }
     roofline = {"bound": "hbm",
                 "kernel": "fwd_mean_fast + transposed view + bwd_mean_fast + gc_pass1..3 (batched history layer)",

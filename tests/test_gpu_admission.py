@@ -150,6 +150,21 @@ def test_record_history_reference_signature(be, orc):
             np.testing.assert_array_equal(dev[k].cpu().numpy(), ref[k], err_msg=f"{k} iter {it}")
 
 
+@pytest.mark.parametrize("seed,n_seed,depth,kids", [(1, 5, 3, 4), (2, 400, 2, 7), (3, 1, 4, 3), (4, 300, 3, 6)])
+def test_structure_score_on_forests(be, seed, n_seed, depth, kids):
+    """On a forest of depth <= num_layer the reference's get_graph_structure_score
+    (src/cpp/src/grad_check.cu:132-163) has one possible result, the product of the ancestors'
+    degrees: the device kernel must give it."""
+    from test_oracle_admission import random_forest_batch
+    rng = np.random.default_rng(seed)
+    ptr, idx, n_nodes, want = random_forest_batch(rng, n_seed, depth, kids)
+    expect = np.zeros(n_nodes + 2, np.int64)
+    for v, prod in want.items():
+        expect[v] = prod
+    got = be.get_graph_structure_score(T(ptr), T(idx), n_nodes + 2, n_seed, depth)
+    np.testing.assert_array_equal(got.cpu().numpy(), expect)
+
+
 def test_small_helpers(be, orc):
     rng = np.random.default_rng(14)
     arr = rng.integers(0, 6, size=100000)

@@ -361,6 +361,89 @@ def test_quantile_threshold_matches_torch_quantile():
     assert worst <= 2, worst
 
 
+def test_quantile_threshold_gives_torch_quantiles_admission_mask():
+    """The reference thresholds with torch.quantile (hiscache/history_cache.py:211-215).  Over 1 200
+    seeded batches at the 1-hop sizes of the plumbing and papers100M-shaped configurations (scores
+    with the lognormal spread of gradient norms, rates 0.5 / 0.7 / 0.9) the mask ``score < threshold``
+    from the build's threshold (host statement and the package's own function) is compared with the
+    mask from torch.quantile on the same scores: a row may only differ when its score lies within
+    2 ulp of torch's threshold; such rows are counted and reported."""
+    from hiscache.util import quantile_threshold as pkg_quantile
+    from oracle import host_model
+    rng = np.random.default_rng(2111)
+    knife, differ, same_bits = 0, 0, 0
+    sizes = [11_000, 5_544, 10_873, 16_000, 7, 1_000]
+    n_batches = 1200
+    for it in range(n_batches):
+        n = sizes[it % len(sizes)] + int(rng.integers(0, 50))
+        rate = (0.5, 0.7, 0.9)[it % 3]
+        s = np.exp(rng.normal(-3, 1.5, size=n)).astype(np.float32)
+        if it % 7 == 0:
+            s[rng.integers(0, n, size=n // 4)] = s[0]            # many equal scores around the threshold
+        ref = torch.quantile(torch.from_numpy(s), rate).numpy().astype(np.float32)
+        mine = np.float32(host_model.quantile_threshold(s, rate))
+        pkg = pkg_quantile(torch.from_numpy(s), rate).numpy().astype(np.float32).reshape(())
+        assert pkg.view(np.int32) == mine.view(np.int32)          # host statement and package function agree
+        same_bits += int(mine.view(np.int32) == ref.view(np.int32))
+        # scores within 2 ulp of torch's threshold (positive floats: ordered like their bit patterns)
+        near = np.abs(s.view(np.int32).astype(np.int64) - int(ref.view(np.int32))) <= 2
+        knife += int(near.sum())
+        diff = (s < mine) != (s < ref)
+        differ += int(diff.sum())
+        assert not (diff & ~near).any(), "a row outside the 2-ulp band changed sides (batch %d)" % it
+    print("quantile masks: %d batches, threshold bit-identical to torch.quantile in %d; %d rows within 2 ulp of "
+          "the threshold, %d of them on the other side" % (n_batches, same_bits, knife, differ))
+    assert same_bits >= 0.9 * n_batches
+
+
+# ----------------------------------------------------------------------------- structure score
+def random_forest_batch(rng, n_seed, depth, max_children):
+    """A layered batch whose rows form a forest: every node is the neighbour of exactly one row, so
+    every node is reached along exactly one path from a seed, at most ``depth`` hops long."""
+    ptr, idx = [0], []
+    level = list(range(n_seed))
+    n_nodes = n_seed
+    parent_deg_product = {v: 1 for v in level}        # product of the degrees of a node's ancestors
+    for d in range(depth):
+        nxt = []
+        for u in level:                                # rows are numbered in node order, level by level
+            c = int(rng.integers(0, max_children + 1))
+            kids = list(range(n_nodes, n_nodes + c))
+            n_nodes += c
+            idx.extend(kids)
+            ptr.append(len(idx))
+            for k in kids:
+                parent_deg_product[k] = parent_deg_product[u] * c
+            nxt.extend(kids)
+        level = nxt
+    return np.asarray(ptr, np.int64), np.asarray(idx, np.int64), n_nodes, parent_deg_product
+
+
+@pytest.mark.parametrize("seed,n_seed,depth,kids", [(1, 5, 3, 4), (2, 40, 2, 7), (3, 1, 4, 3), (4, 30, 3, 6)])
+def test_structure_score_on_forests_has_the_references_only_possible_result(orc, seed, n_seed, depth, kids):
+    """get_graph_structure_score (src/cpp/src/grad_check.cu:132-163) reads and writes its output
+    across warps inside one pass, so in general its result depends on scheduling.  On a forest of
+    depth <= num_layer every node receives exactly one offer, whatever the interleaving: the product
+    of the degrees of its ancestors.  There the reference has one possible answer and the
+    level-synchronous statement must give it; seeds keep 1, unreached ids keep 0."""
+    rng = np.random.default_rng(seed)
+    ptr, idx, n_nodes, want = random_forest_batch(rng, n_seed, depth, kids)
+    # shuffle the neighbour ids' numbering beyond the rows so that node order is not level order
+    n_rows = len(ptr) - 1
+    perm = np.arange(n_nodes + 3)                     # three extra ids that nothing reaches
+    tail = perm[n_rows:].copy()
+    rng.shuffle(tail)
+    perm[n_rows:] = tail
+    idx2 = perm[idx]
+    got = orc.get_graph_structure_score(ptr, idx2, n_nodes + 3, n_seed, depth)
+    expect = np.zeros(n_nodes + 3, np.int64)
+    for v, prod in want.items():
+        expect[perm[v]] = prod
+    np.testing.assert_array_equal(got, expect)
+    # more passes than levels change nothing; fewer passes reach fewer levels
+    np.testing.assert_array_equal(orc.get_graph_structure_score(ptr, idx2, n_nodes + 3, n_seed, depth + 2), expect)
+
+
 # ----------------------------------------------------------------------------- cache policy
 class DictCache:
     """HistoryCache.update_history as a dictionary model: embeddings appended at `header`,
