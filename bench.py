@@ -589,7 +589,7 @@ def run_c3(args):
     torch.manual_seed(3)
     model = HistorySAGE(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache).to(dev)
     model.train()
-    opt = torch.optim.Adam(model.parameters(), lr=1e-3)
+    opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True)      # one multi-tensor launch per step
     class FoldedLabels:
         """Labels of a huge id space folded into a small table."""
         base = np.random.default_rng(3).integers(0, C, size=1 << 20)
@@ -739,7 +739,7 @@ def run_c5(args):
     model = HistoryRGCN(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache, num_rel=K, dataset_name="rmag240m",
                         type_bounds=[n_paper, n_paper + n_author], pair_to_rel=pair_to_rel).to(dev)
     model.train()
-    opt = torch.optim.Adam(model.parameters(), lr=1e-3)
+    opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True)      # one multi-tensor launch per step
 
     class FoldedLabels:
         base = np.random.default_rng(5).integers(0, C, size=1 << 20)

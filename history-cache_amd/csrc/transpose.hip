@@ -47,6 +47,32 @@ __device__ __forceinline__ int64_t tr_row_of(P ptr, int64_t lo, int64_t hi, int6
   return lo;
 }
 
+// The same search by a whole wave, 64 probes per memory round trip (three round trips for 2^18 rows
+// instead of eighteen): largest r in [0, R] with ptr[r] <= e, assuming ptr[0] <= e.  Every lane
+// returns the result.
+__device__ __forceinline__ int64_t tr_row_of_wave(const int64_t *__restrict__ ptr, int64_t R, int64_t e,
+                                                  int lane) {
+  int64_t lo = 0, hi = R;   // ptr[lo] <= e; the answer lies in [lo, hi]
+  while (hi > lo) {
+    const int64_t step = (hi - lo + HC_WAVE - 1) / HC_WAVE;
+    int64_t p = lo + (int64_t)(lane + 1) * step;
+    if (p > hi) p = hi;
+    const unsigned long long ok = __ballot(ptr[p] <= e);   // a prefix of the lanes: ptr does not decrease
+    const int k = __popcll(ok);
+    int64_t nlo = lo + (int64_t)k * step;                  // the last probe that held (lo itself when k == 0)
+    if (nlo > hi) nlo = hi;
+    int64_t nhi = hi;
+    if (k < HC_WAVE) {
+      nhi = lo + (int64_t)(k + 1) * step;                  // the first probe that failed, minus one
+      if (nhi > hi) nhi = hi;
+      nhi -= 1;
+    }
+    lo = nlo;
+    hi = nhi < nlo ? nlo : nhi;
+  }
+  return lo;
+}
+
 template <bool VAL_IS_ROW, int TR_ITEMS>
 __global__ __launch_bounds__(HC_BLOCK) void tr_expand_edges(const int64_t *__restrict__ ptr,
                                                              const int64_t *__restrict__ idx,
@@ -62,7 +88,15 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_expand_edges(const int64_t *__res
   __shared__ int64_t s_range[2];
   const int64_t e0 = (int64_t)blockIdx.x * TR_TILE;
   const int64_t e1 = e0 + TR_TILE < E ? e0 + TR_TILE : E;
-  if (threadIdx.x < 2) s_range[threadIdx.x] = tr_row_of(ptr, (int64_t)0, R, threadIdx.x == 0 ? e0 : e1 - 1);
+  if (threadIdx.x < HC_WAVE) {
+    const int lane0 = hc_lane();
+    const int64_t a = tr_row_of_wave(ptr, R, e0, lane0);
+    const int64_t b = tr_row_of_wave(ptr, R, e1 - 1, lane0);
+    if (lane0 == 0) {
+      s_range[0] = a;
+      s_range[1] = b;
+    }
+  }
   __syncthreads();
   const int64_t r_lo = s_range[0], r_hi = s_range[1];
   const int64_t span = r_hi - r_lo + 1;  // rows r_lo..r_hi (r_hi may be R: slots behind the last row)
@@ -228,15 +262,17 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_finalize_ptr(const uint32_t *__re
 //                   (atomic: WHICH slots a segment holds is fixed, their order inside it is not yet)
 //                   and writes (row, slot) there, into temporary arrays
 //   tr_small_order  copies every segment to its final place in ascending slot order -- the order a
-//                   stable sort gives: one-edge segments as they are, segments of up to 64 edges
-//                   ranked inside a wave, longer ones by the whole block through a bitmap of the
-//                   segment's slots in LDS (rank = number of set bits below the slot)
+//                   stable sort gives: one-edge segments as they are, segments of up to 8 edges
+//                   sorted by their lane in registers, of up to 64 edges ranked inside a wave, longer
+//                   ones by the whole block through a bitmap of the segment's slots in LDS (rank =
+//                   number of set bits below the slot)
 // The result is bit-identical to the sorted view of the large-block path.
 // ---------------------------------------------------------------------------------------
 constexpr int TRS_BLOCK = 1024;
 constexpr int64_t TR_SMALL_SOURCES = 1 << 20;
 constexpr int TRS_BITMAP_WORDS = (int)(TR_SMALL_EDGES / 32);   // one bit per edge slot
 constexpr int TRS_ORDER_SOURCES = HC_BLOCK;                     // sources per block of tr_small_order
+constexpr int TRS_LANE_SORT = 8;                                // longest segment a single lane sorts
 
 struct TrSmallHeader {
   unsigned ticket;
@@ -248,9 +284,10 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_small_clear(uint32_t *__restrict_
   if (i < n) p[i] = 0u;
 }
 
-__device__ __forceinline__ int trs_load(const int *p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
+// Read of a counter by the block that scans them.  The counters were only ever touched by atomics (which
+// work in the L2) and this block reads them behind its device-scope fence, so an ordinary load sees the
+// final values; ordinary loads, unlike atomic ones, are issued back to back.
+__device__ __forceinline__ int trs_load(const int *p) { return *p; }
 
 __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const int64_t *__restrict__ hmap_row,
@@ -263,7 +300,15 @@ __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
   __shared__ int s_last;
   const int64_t e0 = (int64_t)blockIdx.x * TRS_BLOCK;
   const int64_t e1 = e0 + TRS_BLOCK < E ? e0 + TRS_BLOCK : E;
-  if (threadIdx.x < 2) s_range[threadIdx.x] = tr_row_of(ptr, (int64_t)0, R, threadIdx.x == 0 ? e0 : e1 - 1);
+  if (threadIdx.x < HC_WAVE) {
+    const int lane0 = hc_lane();
+    const int64_t a = tr_row_of_wave(ptr, R, e0, lane0);
+    const int64_t b = tr_row_of_wave(ptr, R, e1 - 1, lane0);
+    if (lane0 == 0) {
+      s_range[0] = a;
+      s_range[1] = b;
+    }
+  }
   __syncthreads();
   const int64_t r_lo = s_range[0], r_hi = s_range[1];
   const int64_t span = r_hi - r_lo + 1;
@@ -291,56 +336,79 @@ __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
     rows[e] = live ? (int32_t)row : -1;
     if (live) atomicAdd(count + src, 1);
   }
-  // the block that takes the last ticket sees every block's counts
-  __threadfence();
+  // The block that takes the last ticket sees every block's counts.  One device-scope release per
+  // block, by the thread that takes the ticket, behind the block's barrier (which orders the other
+  // waves' atomics in front of it): on this multi-die part a device-scope release writes the die's L2
+  // back, and one per wave made this kernel several times longer.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
-  if (threadIdx.x == 0) s_last = atomicAdd(&header->ticket, 1u) == gridDim.x - 1 ? 1 : 0;
+  if (threadIdx.x == 0) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    s_last = atomicAdd(&header->ticket, 1u) == gridDim.x - 1 ? 1 : 0;
+  }
   __syncthreads();
   if (!s_last) return;
-  __threadfence();
-  // exclusive scan of count[0, n_src): thread t owns a contiguous run of sources
-  const int64_t per = (n_src + TRS_BLOCK - 1) / TRS_BLOCK;
-  int64_t lo = (int64_t)threadIdx.x * per;
-  int64_t hi = lo + per;
-  if (lo > n_src) lo = n_src;
-  if (hi > n_src) hi = n_src;
-  // the loads of a run are issued eight at a time (one after the other they would cost a memory round
-  // trip each, and this block runs alone at the end of the launch)
-  int sum = 0;
-  for (int64_t q = lo; q < hi; q += 8) {
-    int c[8];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) c[k] = q + k < hi ? trs_load(count + q + k) : 0;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) sum += c[k];
-  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  // Exclusive scan of count[0, n_src] by this one block, TRS_SUPER entries per sweep.  A thread loads
+  // its 8 x 4 entries of the sweep with eight 16-byte loads issued together (entry = (g * 1024 + t) * 4 + j:
+  // coalesced), keeps them in registers, and the block scans the eight slabs of 4 096 entries one after
+  // the other.  (One thread per contiguous run of entries would issue 64 scattered requests per
+  // instruction from a single compute unit: measured 60 us for 26 000 sources.)  Entries between n_src
+  // and the end of the counter array are zero.
+  constexpr int NW = TRS_BLOCK / HC_WAVE;
+  constexpr int G = 8;
+  constexpr int64_t TRS_SUPER = (int64_t)TRS_BLOCK * 4 * G;
   const int lane = hc_lane();
   const int wave = (int)(threadIdx.x >> 6);
-  int x = sum;
+  const int64_t n_entries = n_src + 1;                      // ptrT has n_src + 1 entries
+  const int64_t padded = (n_entries + 3) / 4 * 4;           // the counter array is zero-padded to 256 bytes
+  int carry = 0;
+  for (int64_t base = 0; base < n_entries; base += TRS_SUPER) {
+    int4 c[G];
 #pragma unroll
-  for (int d = 1; d < HC_WAVE; d <<= 1) {
-    const int y = __shfl_up(x, d, HC_WAVE);
-    if (lane >= d) x += y;
-  }
-  if (lane == HC_WAVE - 1) s_wave[wave] = x;
-  __syncthreads();
-  int off = x - sum;
-  for (int w = 0; w < wave; ++w) off += s_wave[w];
-  int run = off;
-  for (int64_t q = lo; q < hi; q += 8) {
-    int c[8];
+    for (int g = 0; g < G; ++g) {
+      const int64_t i = base + ((int64_t)g * TRS_BLOCK + threadIdx.x) * 4;
+      c[g] = i < padded ? *reinterpret_cast<const int4 *>(count + i) : make_int4(0, 0, 0, 0);
+    }
 #pragma unroll
-    for (int k = 0; k < 8; ++k) c[k] = q + k < hi ? trs_load(count + q + k) : 0;
+    for (int g = 0; g < G; ++g) {
+      const int64_t i = base + ((int64_t)g * TRS_BLOCK + threadIdx.x) * 4;
+      const int mine = (c[g].x + c[g].y) + (c[g].z + c[g].w);
+      int x = mine;                                         // inclusive scan over the block's 1 024 threads
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      if (q + k < hi) {
-        ptrT[q + k] = run;
-        count[q + k] = run;   // the segment's cursor for tr_small_place
-        run += c[k];
+      for (int d = 1; d < HC_WAVE; d <<= 1) {
+        const int y = __shfl_up(x, d, HC_WAVE);
+        if (lane >= d) x += y;
+      }
+      if (lane == HC_WAVE - 1) s_wave[wave] = x;
+      __syncthreads();
+      int off = carry + x - mine;
+      int slab = 0;
+      for (int w = 0; w < NW; ++w) {
+        const int t = s_wave[w];
+        if (w < wave) off += t;
+        slab += t;
+      }
+      __syncthreads();
+      carry += slab;
+      if (i < n_entries) {
+        const int p0 = off, p1 = p0 + c[g].x, p2 = p1 + c[g].y, p3 = p2 + c[g].z;
+        if (i + 3 < n_entries) {
+          *reinterpret_cast<int4 *>(count + i) = make_int4(p0, p1, p2, p3);   // the segments' cursors
+          ptrT[i] = p0;
+          ptrT[i + 1] = p1;
+          ptrT[i + 2] = p2;
+          ptrT[i + 3] = p3;
+        } else {
+          const int p[4] = {p0, p1, p2, p3};
+          for (int j = 0; j < 4 && i + j < n_entries; ++j) {
+            count[i + j] = p[j];
+            ptrT[i + j] = p[j];
+          }
+        }
       }
     }
   }
-  if (threadIdx.x == TRS_BLOCK - 1) ptrT[n_src] = run;
 }
 
 __global__ __launch_bounds__(HC_BLOCK) void tr_small_place(const uint32_t *__restrict__ keys,
@@ -385,8 +453,36 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_small_order(const int64_t *__rest
     if (edgeT != nullptr) edgeT[b] = tmp_edge[b];
   }
   if (len > HC_WAVE) long_src[atomicAdd(&n_long_s, 1)] = (int)threadIdx.x;
-  // segments of 2..64 edges: ranked inside the wave, one segment at a time
-  unsigned long long m = __ballot(len >= 2 && len <= HC_WAVE);
+  // segments of 2..TRS_LANE_SORT edges (most of what is not a single edge): every lane sorts its own
+  // segment in registers -- an odd-even transposition network on the slots, the rows ride along
+  if (len >= 2 && len <= TRS_LANE_SORT) {
+    int ve[TRS_LANE_SORT], vr[TRS_LANE_SORT];
+#pragma unroll
+    for (int k = 0; k < TRS_LANE_SORT; ++k) {
+      ve[k] = k < len ? tmp_edge[b + k] : 0x7fffffff;
+      vr[k] = k < len ? tmp_row[b + k] : 0;
+    }
+#pragma unroll
+    for (int round = 0; round < TRS_LANE_SORT; ++round) {
+#pragma unroll
+      for (int k = round & 1; k + 1 < TRS_LANE_SORT; k += 2) {
+        const bool sw = ve[k + 1] < ve[k];
+        const int e0 = sw ? ve[k + 1] : ve[k], e1 = sw ? ve[k] : ve[k + 1];
+        const int r0 = sw ? vr[k + 1] : vr[k], r1 = sw ? vr[k] : vr[k + 1];
+        ve[k] = e0; ve[k + 1] = e1;
+        vr[k] = r0; vr[k + 1] = r1;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < TRS_LANE_SORT; ++k) {
+      if (k < len) {
+        rowT[b + k] = vr[k];
+        if (edgeT != nullptr) edgeT[b + k] = ve[k];
+      }
+    }
+  }
+  // segments of up to 64 edges: ranked inside the wave, one segment at a time
+  unsigned long long m = __ballot(len > TRS_LANE_SORT && len <= HC_WAVE);
   while (m != 0ull) {
     const int l = __builtin_ctzll(m);
     m &= m - 1ull;

@@ -9,10 +9,77 @@ The relational layer replaces ``cxgnncomp.RGCNOP_sorted`` (:266) by a typed gath
 mean kernel over (row, relation) virtual rows -- followed by one GEMM; the result is the same
 quantity, sum_j x[src_j] @ W[rel_j] / deg.  The DGL wrapper is not part of this module.
 """
+import weakref
+
 import torch
 import torch.nn.functional as F
 
 import hiscache_backend
+
+
+class _GradSink:
+    """Where the fused convolution leaves the gradient that reached its aggregation output: the
+    tensor the model hands to the cache as ``produced_embedding`` (held weakly)."""
+    __slots__ = ("target",)
+
+    def __init__(self):
+        self.target = None
+
+
+class _SageConvFunction(torch.autograd.Function):
+    """``lin_l(aggregate(x)) + lin_r(x[:n])`` as ONE autograd node.
+
+    Spelled with separate operators (as /root/reference/hiscache/history_model.py:85-100 does) the
+    backward of a layer runs, besides its GEMMs, a zero fill and a copy for the gradient of the slice
+    ``x[:n]`` and an add that joins it with the aggregation's input gradient.  Here the aggregation's
+    input gradient is written first and the root term's gradient is accumulated into its first n rows
+    by the GEMM itself.  The aggregation output is returned as a second, non-differentiable result;
+    the gradient that reaches it (what ``retain_grad()`` keeps in the unfused spelling) is stored in
+    its ``.grad`` during backward when a sink is given."""
+
+    @staticmethod
+    def forward(ctx, x, w_l, b_l, w_r, ptr, idx, hmap, hbuf, hsize, num_node, num_edge, sink):
+        be = hiscache_backend
+        R = int(num_node) if num_node else ptr.numel() - 1
+        agg = be._aggr_fwd(be.SUBST_ROW, ptr, idx, x, hmap, hbuf, hsize, None, R)
+        out = torch.addmm(b_l, agg, w_l.t()) if b_l is not None else agg @ w_l.t()
+        if w_r is not None:
+            root = x[:R] if x.dtype == agg.dtype else x[:R].to(agg.dtype)
+            out.addmm_(root, w_r.t())
+        ctx.save_for_backward(x, agg, w_l, w_r if w_r is not None else w_l.new_empty(0))
+        ctx.hc = (ptr, idx, hmap, hsize, R, num_edge, b_l is not None, w_r is not None, sink)
+        ctx.mark_non_differentiable(agg)
+        return out, agg
+
+    @staticmethod
+    def backward(ctx, g_out, _g_agg_unused):
+        be = hiscache_backend
+        ptr, idx, hmap, hsize, R, num_edge, has_bias, has_root, sink = ctx.hc
+        x, agg, w_l, w_r = ctx.saved_tensors
+        g_out = g_out.contiguous()
+        need = ctx.needs_input_grad
+        g_agg = g_out @ w_l                                   # gradient reaching the aggregation output
+        if sink is not None and sink.target is not None:
+            his = sink.target()
+            if his is not None:
+                his.grad = g_agg
+        g_wl = g_out.t() @ agg if need[1] else None
+        g_bl = g_out.sum(0) if has_bias and need[2] else None
+        g_wr = None
+        if has_root and need[3]:
+            root = x[:R] if x.dtype == g_out.dtype else x[:R].to(g_out.dtype)
+            g_wr = g_out.t() @ root
+        g_x = None
+        if need[0]:
+            n_src = x.shape[0]
+            tr = be.build_transpose(ptr, idx, hmap, R, n_src, num_edge=num_edge, want_edges=False)
+            g_x, _, _ = be._aggr_bwd(ptr, idx, tr, g_agg, hmap, None, x, False, None, hsize, R, n_src,
+                                     want_hist_grad=False)
+            if has_root:
+                g_x[:R].addmm_(g_out, w_r)
+            if g_x.dtype != x.dtype:
+                g_x = g_x.to(x.dtype)
+        return g_x, g_wl, g_bl, g_wr, None, None, None, None, None, None, None, None
 
 
 class MySageConvHistory(torch.nn.Module):
@@ -34,8 +101,23 @@ class MySageConvHistory(torch.nn.Module):
         if self.root_weight:
             self.lin_r.reset_parameters()
 
+    # one autograd node per layer (see _SageConvFunction); False spells the layer operator by operator
+    fused = True
+
     def forward(self, x, ptr, idx, history_map, history_buffer, history_size, num_node, num_edge=None):
         num_node = int(num_node)
+        use_hist = history_size > 0 and history_map is not None and history_map.numel() > 0
+        if self.fused and x.is_cuda and not (use_hist and history_buffer.requires_grad):
+            sink = None
+            if self.need_grad and self.training and history_size > 0:
+                sink = _GradSink()
+            out, his = _SageConvFunction.apply(
+                x, self.lin_l.weight, self.lin_l.bias, self.lin_r.weight if self.root_weight else None, ptr, idx,
+                history_map if use_hist else None, history_buffer if use_hist else None,
+                int(history_size) if use_hist else 0, num_node, num_edge, sink)
+            if sink is not None:
+                sink.target = weakref.ref(his)
+            return out, his
         # history_size == 0 selects the plain mean inside the operator; num_edge (optional, beyond the
         # reference) bounds the edge slots of these rows inside the mini-batch's shared CSR
         out = hiscache_backend.aggr_forward_history(x, ptr, idx, history_map, history_buffer,

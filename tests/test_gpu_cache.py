@@ -306,6 +306,46 @@ def test_sage_training_iteration_matches_cpu():
     assert ev.shape == (20, 7) and torch.isfinite(ev).all()
 
 
+def test_fused_sage_layer_equals_the_operator_by_operator_spelling():
+    """MySageConvHistory as one autograd node (aggregation, both linear maps, the root term's gradient
+    accumulated into the aggregation's input gradient) against the same layer spelled operator by
+    operator: identical aggregation output and produced-embedding gradient, outputs and parameter
+    gradients to fp32 GEMM rounding."""
+    from hiscache import MySageConvHistory
+    from helpers import random_csr, random_hmap
+    rng = np.random.default_rng(31)
+    torch.manual_seed(31)
+    R, N, Fin, H = 700, 1500, 128, 64
+    ptr, idx = random_csr(rng, R, N, 9, hub=300)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+    hmap = t(random_hmap(rng, R, 0.3))
+    hbuf = t(rng.standard_normal((R, Fin)).astype(np.float32))
+    g = t(rng.standard_normal((R, H)).astype(np.float32))
+    conv = MySageConvHistory(Fin, H, need_grad=True).to(DEV)
+    conv.train()
+    res = {}
+    for fused in (True, False):
+        conv.fused = fused
+        conv.zero_grad()
+        x = t(rng.standard_normal((N, Fin)).astype(np.float32) * 0 + 1).requires_grad_(True)
+        x.data.copy_(t(np.random.default_rng(5).standard_normal((N, Fin)).astype(np.float32)))
+        out, his = conv(x, t(ptr), t(idx), hmap, hbuf, Fin, R, int(ptr[R]))
+        out.backward(g)
+        res[fused] = (out.detach(), his.detach(), his.grad.clone(), x.grad.clone(), conv.lin_l.weight.grad.clone(),
+                      conv.lin_l.bias.grad.clone(), conv.lin_r.weight.grad.clone())
+    a, b = res[True], res[False]
+    assert torch.equal(a[1], b[1])                                   # aggregation output, bit for bit
+    for i, name in ((0, "out"), (2, "his.grad"), (3, "x.grad"), (4, "lin_l.weight.grad"), (5, "lin_l.bias.grad"),
+                    (6, "lin_r.weight.grad")):
+        scale = float(b[i].abs().max())
+        np.testing.assert_allclose(a[i].cpu().numpy(), b[i].cpu().numpy(), rtol=1e-4, atol=1e-5 * scale, err_msg=name)
+    # without history and without a gradient sink the fused layer still returns the aggregation
+    conv.fused = True
+    none = torch.empty(0, device=DEV)
+    out2, his2 = conv(t(rng.standard_normal((N, Fin)).astype(np.float32)), t(ptr), t(idx), none, none, 0, R)
+    assert his2.grad is None and tuple(out2.shape) == (R, H)
+
+
 def test_history_table_record_and_evict():
     from hiscache import HistoryTable, make_config
     from oracle import hc_oracle as orc
