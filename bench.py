@@ -541,7 +541,7 @@ def run_c3(args):
     import torch
 
     import hiscache_backend as be
-    from hiscache import HistorySAGE, PinnedFeatureStore, RingHistoryCache, make_config
+    from hiscache import HistorySAGE, PinnedFeatureStore, RingHistoryCache, make_config, prefer_low_latency_gemm
     from hiscache.synthetic import direct_power_law_batch, make_batch
 
     dev = "cuda:0"
@@ -587,6 +587,7 @@ def run_c3(args):
     cache.table.normal_(0.0, 0.5, generator=gen) if N <= 20_000_000 else cache.table[:hit.numel()].normal_(0.0, 0.5)
     cfg = make_config(Fin, C, H, L, device=dev)
     torch.manual_seed(3)
+    prefer_low_latency_gemm()                                            # what get_model() does by default
     model = HistorySAGE(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache).to(dev)
     model.train()
     opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True)      # one multi-tensor launch per step
@@ -689,7 +690,7 @@ def run_c5(args):
     import numpy as np
     import torch
 
-    from hiscache import HistoryRGCN, PinnedFeatureStore, RingHistoryCache, make_config
+    from hiscache import HistoryRGCN, PinnedFeatureStore, RingHistoryCache, make_config, prefer_low_latency_gemm
     from hiscache.synthetic import direct_power_law_batch, make_batch
 
     dev = "cuda:0"
@@ -736,6 +737,7 @@ def run_c5(args):
     # relation of an edge from the node types of (destination, source): paper-cites-paper,
     # paper<-author, author<-paper, author<-institution, institution<-author
     pair_to_rel = [[0, 1, 0], [2, 0, 3], [0, 4, 0]]
+    prefer_low_latency_gemm()                                            # what get_model() does by default
     model = HistoryRGCN(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache, num_rel=K, dataset_name="rmag240m",
                         type_bounds=[n_paper, n_paper + n_author], pair_to_rel=pair_to_rel).to(dev)
     model.train()

@@ -10,14 +10,14 @@ from .dataset import ProcessedDataset, write_processed
 from .feature_store import PinnedFeatureStore
 from .history_cache import HistoryCache
 from .history_model import (HistoryRGCN, HistorySAGE, MyRGCNConvHistory2, MySageConvHistory, get_model,
-                            typed_csr)
+                            prefer_low_latency_gemm, typed_csr)
 from .history_table import HistoryTable
 from .ring_cache import RingHistoryCache
 from .sampler import NeighborSampler
 from .util import Config, make_config, quantile_threshold
 
 __all__ = [
-    "HistoryCache", "HistoryTable", "RingHistoryCache", "HistorySAGE", "HistoryRGCN", "MySageConvHistory", "MyRGCNConvHistory2", "typed_csr", "get_model",
+    "HistoryCache", "HistoryTable", "RingHistoryCache", "HistorySAGE", "HistoryRGCN", "MySageConvHistory", "MyRGCNConvHistory2", "typed_csr", "get_model", "prefer_low_latency_gemm",
     "PinnedFeatureStore", "NeighborSampler", "ProcessedDataset", "write_processed", "Config", "make_config", "quantile_threshold",
     "count_history_reconstruct", "get_graph_structure_score", "record_history",
 ]

@@ -42,10 +42,14 @@ class _SageConvFunction(torch.autograd.Function):
         be = hiscache_backend
         R = int(num_node) if num_node else ptr.numel() - 1
         agg = be._aggr_fwd(be.SUBST_ROW, ptr, idx, x, hmap, hbuf, hsize, None, R)
-        out = torch.addmm(b_l, agg, w_l.t()) if b_l is not None else agg @ w_l.t()
+        # plain GEMMs and a separate bias add: a GEMM with a bias epilogue goes to hipBLASLt whatever
+        # library is preferred, and its per-shape set-up costs the host more than the extra launch
+        out = agg @ w_l.t()
         if w_r is not None:
             root = x[:R] if x.dtype == agg.dtype else x[:R].to(agg.dtype)
             out.addmm_(root, w_r.t())
+        if b_l is not None:
+            out += b_l
         ctx.save_for_backward(x, agg, w_l, w_r if w_r is not None else w_l.new_empty(0))
         ctx.hc = (ptr, idx, hmap, hsize, R, num_edge, b_l is not None, w_r is not None, sink)
         ctx.mark_non_differentiable(agg)
@@ -82,6 +86,28 @@ class _SageConvFunction(torch.autograd.Function):
         return g_x, g_wl, g_bl, g_wr, None, None, None, None, None, None, None, None
 
 
+def bn_relu(x, bn, bias=None, fused=True):
+    """``F.relu(bn(x + bias))`` (/root/reference/hiscache/history_model.py:139-140).  In training mode on
+    the GPU this is one autograd node over the library's epilogue kernels (two launches forward, two
+    backward, against eight and four operator by operator); ``bias`` then must NOT have been added to
+    ``x`` yet.  Otherwise the torch operators run.  ``bn``'s running statistics and batch counter are
+    updated as ``torch.nn.BatchNorm1d.forward`` updates them."""
+    be = hiscache_backend
+    if not (fused and bn.training and x.dim() == 2 and be.bn_relu_supported(x, x.shape[1])
+            and x.shape[0] > 1):
+        if bias is not None:
+            x = x + bias
+        return F.relu(bn(x))
+    momentum = 0.0 if bn.momentum is None else bn.momentum
+    track = bn.track_running_stats and bn.running_mean is not None
+    if track and bn.num_batches_tracked is not None:
+        bn.num_batches_tracked.add_(1)
+        if bn.momentum is None:                       # cumulative moving average
+            momentum = 1.0 / float(bn.num_batches_tracked)
+    return be.bias_bn_relu(x, bias, bn.weight, bn.bias, bn.running_mean if track else None,
+                           bn.running_var if track else None, momentum, bn.eps)
+
+
 class MySageConvHistory(torch.nn.Module):
 
     def __init__(self, in_channels, hidden_channels, need_grad, root_weight: bool = True,
@@ -104,7 +130,10 @@ class MySageConvHistory(torch.nn.Module):
     # one autograd node per layer (see _SageConvFunction); False spells the layer operator by operator
     fused = True
 
-    def forward(self, x, ptr, idx, history_map, history_buffer, history_size, num_node, num_edge=None):
+    def forward(self, x, ptr, idx, history_map, history_buffer, history_size, num_node, num_edge=None,
+                add_bias=True):
+        """``add_bias=False`` (fused spelling only) leaves ``lin_l``'s bias to the caller, who hands it
+        to the normalisation that follows (see ``bn_relu``)."""
         num_node = int(num_node)
         use_hist = history_size > 0 and history_map is not None and history_map.numel() > 0
         if self.fused and x.is_cuda and not (use_hist and history_buffer.requires_grad):
@@ -112,12 +141,15 @@ class MySageConvHistory(torch.nn.Module):
             if self.need_grad and self.training and history_size > 0:
                 sink = _GradSink()
             out, his = _SageConvFunction.apply(
-                x, self.lin_l.weight, self.lin_l.bias, self.lin_r.weight if self.root_weight else None, ptr, idx,
+                x, self.lin_l.weight, self.lin_l.bias if add_bias else None,
+                self.lin_r.weight if self.root_weight else None, ptr, idx,
                 history_map if use_hist else None, history_buffer if use_hist else None,
                 int(history_size) if use_hist else 0, num_node, num_edge, sink)
             if sink is not None:
                 sink.target = weakref.ref(his)
             return out, his
+        if not add_bias:
+            raise ValueError("add_bias=False needs the fused spelling of the layer")
         # history_size == 0 selects the plain mean inside the operator; num_edge (optional, beyond the
         # reference) bounds the edge slots of these rows inside the mini-batch's shared CSR
         out = hiscache_backend.aggr_forward_history(x, ptr, idx, history_map, history_buffer,
@@ -151,6 +183,10 @@ class HistorySAGE(torch.nn.Module):
         self.table = table
         self.init_convs(**kwargs)
 
+    # bias + batch norm + ReLU of a hidden layer as one autograd node (see bn_relu); False spells them
+    # with torch operators
+    fused_epilogue = True
+
     def forward(self, batch):
         x = batch.x
         none = torch.empty(0, device=x.device)
@@ -159,15 +195,16 @@ class HistorySAGE(torch.nn.Module):
             k = self.num_layers - 1 - i
             n = batch.num_node_in_layer[k]
             ne = None if nel is None else int(nel[k])
+            # the bias of lin_l goes to the normalisation's kernels instead of a launch of its own
+            defer = self.fused_epilogue and conv.fused and self.training and x.is_cuda
             if self.training and i == self.num_layers - 2:
                 # the layer whose output is one hop from the seeds uses (and produces) history
                 x, his = conv(x, batch.ptr, batch.idx, self.table.sub2embed,
-                              self.table.cached_embedding, self.hidden_channels, n, ne)
+                              self.table.cached_embedding, self.hidden_channels, n, ne, add_bias=not defer)
                 self.table.produced_embedding = his
             else:
-                x, his = conv(x, batch.ptr, batch.idx, none, none, 0, n, ne)
-            x = self.bns[i](x)
-            x = F.relu(x)
+                x, his = conv(x, batch.ptr, batch.idx, none, none, 0, n, ne, add_bias=not defer)
+            x = bn_relu(x, self.bns[i], conv.lin_l.bias if defer else None, fused=self.fused_epilogue)
             x = F.dropout(x, p=self.dropout, training=self.training)
         x, his = self.convs[-1](x, batch.ptr, batch.idx, none, none, 0, batch.num_node_in_layer[0],
                                 None if nel is None else int(nel[0]))
@@ -309,6 +346,8 @@ class HistoryRGCN(torch.nn.Module):
             self.last_layer_history = False
             self.convs.append(MyRGCNConvHistory2(hidden_channels, out_channels, self.num_rel, need_grad))
 
+    fused_epilogue = True
+
     def edge_types(self, batch):
         L = self.num_layers
         if getattr(batch, "edge_type", None) is not None:
@@ -340,8 +379,7 @@ class HistoryRGCN(torch.nn.Module):
                 self.table.produced_embedding.retain_grad()
             else:
                 x, his = conv(x, batch.ptr, batch.idx, et, None, none, none, um, 0, n)
-            x = self.bns[i](x)
-            x = F.relu(x)
+            x = bn_relu(x, self.bns[i], None, fused=self.fused_epilogue)
             x = F.dropout(x, p=self.dropout, training=self.training)
         um = masks[-2] if masks is not None else None
         x, his = self.convs[-1](x, batch.ptr, batch.idx, etypes[: batch.num_edge_in_layer[0]], None, none, none,
@@ -355,6 +393,18 @@ class HistoryRGCN(torch.nn.Module):
             bn.reset_parameters()
 
 
+def prefer_low_latency_gemm(enable=True):
+    """Route torch's GEMMs to rocBLAS (``enable``) or back to torch's default choice.
+
+    Sampled batches give every GEMM of an iteration a row count that was never seen before.
+    hipBLASLt, torch's default on this GPU, selects a kernel per problem shape, which costs the host
+    about 80 us per call for a new shape (20 us for a repeated one); rocBLAS costs 11 - 17 us either
+    way and its kernels for these tall, narrow problems are no slower.  The setting is global to the
+    process (``torch.backends.cuda.preferred_blas_library``); ``get_model`` applies it unless
+    ``config.train.dense_blas`` says "default"."""
+    torch.backends.cuda.preferred_blas_library("hipblas" if enable else "default")
+
+
 model_dict = {"sage": HistorySAGE, "rgcn": HistoryRGCN}
 graph_type_dict = {"cxg": "CSR_Layer", "dgl": "DGL"}
 
@@ -362,6 +412,8 @@ graph_type_dict = {"cxg": "CSR_Layer", "dgl": "DGL"}
 def get_model(config, table):
     """Model factory with the reference's signature (/root/reference/hiscache/history_model.py:446-470)."""
     mtype = config.train.model.type.lower()
+    if str(getattr(config.train, "dense_blas", "rocblas")).lower() != "default":
+        prefer_low_latency_gemm()
     if mtype not in model_dict:
         raise NotImplementedError(f"model type {mtype!r}: sage and rgcn are provided")
     if mtype == "rgcn":

@@ -14,7 +14,8 @@ ABI (ctypes; raw device pointers, sizes, dtype enums, the current HIP stream).
 Beyond the reference's set: ``aggr_forward_source_history`` (per-source substitution),
 ``build_transpose``, ``row_scores``, ``grad_check`` / ``cache_append`` (fused admission), ``evict``,
 ``gather_rows`` / ``lookup``, ``typed_csr`` / ``edge_types_by_ranges`` (relational blocks),
-``sample_layers`` (device sampler) and ``check_csr`` (input validation).
+``sample_layers`` (device sampler), ``bias_bn_relu`` (a hidden layer's epilogue) and ``check_csr`` (input
+validation).
 
 There is no CPU or PyTorch fallback: if the shared library is missing or a
 tensor is not on a GPU, the call raises.
@@ -84,6 +85,11 @@ _SIGNATURES = {
     "hc_sample_map_init": (_c_int, [_c_p, _c_i64, _c_p]),
     "hc_sample_layers": (_c_int, [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_int, ctypes.c_uint64, _c_p, _c_p,
                                   _c_p, _c_p, _c_p, _c_p, _c_sz, _c_p]),
+    "hc_bn_relu_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
+    "hc_bn_relu_fwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, ctypes.c_float, ctypes.c_float, _c_p, _c_p,
+                                _c_p, _c_i64, _c_i64, _c_p, _c_sz, _c_p, _c_p]),
+    "hc_bn_relu_bwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64,
+                                _c_p, _c_sz, _c_p, _c_p]),
     "hc_typed_csr_workspace_bytes": (_c_sz, [_c_i64, _c_int]),
     "hc_edge_types_by_ranges": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_p, _c_p, _c_i64, _c_i64, _c_p]),
     "hc_typed_csr": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_p,
@@ -730,6 +736,85 @@ def edge_types_by_ranges(ptr, idx, sub_to_full, num_node, bounds, pair_to_rel):
                                      int(bounds.numel()), _ptr(pair_to_rel), _ptr(out), R, idx.numel(), _stream())
     _check(rc, "hc_edge_types_by_ranges")
     return out
+
+
+# ------------------------------------------------------------------ layer epilogue
+BN_RELU_MAX_CHANNELS = 1024
+_tickets = {}
+
+
+def _ticket(device):
+    """The zeroed word the epilogue kernels count their blocks in (one per device and stream; the
+    kernels leave it zero)."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    t = _tickets.get(key)
+    if t is None:
+        t = _tickets[key] = torch.zeros(64, dtype=torch.int32, device=device)
+    return t
+
+
+def bn_relu_supported(x, channels):
+    return x.is_cuda and x.dtype == torch.float32 and channels % 4 == 0 and 4 <= channels <= BN_RELU_MAX_CHANNELS
+
+
+class _BiasBnRelu(torch.autograd.Function):
+    """relu(batch_norm(x + bias)) in training mode as one autograd node over ``hc_bn_relu_fwd`` /
+    ``hc_bn_relu_bwd`` (/root/reference/hiscache/history_model.py:139-140).  ``x`` comes WITHOUT the
+    bias; the running statistics are updated in place."""
+
+    @staticmethod
+    def forward(ctx, x, bias, gamma, beta, running_mean, running_var, momentum, eps):
+        lib = load_library()
+        n, C = x.shape
+        y = torch.empty_like(x)
+        stats = torch.empty((2, C), dtype=torch.float32, device=x.device)      # mean, 1/sqrt(var + eps)
+        ws = _workspace(lib.hc_bn_relu_workspace_bytes(n, C), x.device)
+        sp = stats.data_ptr()
+        _check(lib.hc_bn_relu_fwd(_ptr(x), _ptr(bias), _ptr(gamma), _ptr(beta), _ptr(running_mean),
+                                  _ptr(running_var), float(momentum), float(eps), _ptr(y), _c_p(sp),
+                                  _c_p(sp + 4 * C), n, C, _ptr(ws), ws.numel(), _ptr(_ticket(x.device)),
+                                  _stream()), "hc_bn_relu_fwd")
+        ctx.save_for_backward(x, stats, gamma if gamma is not None else x.new_empty(0),
+                              beta if beta is not None else x.new_empty(0))
+        ctx.hc = (bias is not None, gamma is not None, beta is not None)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        lib = load_library()
+        x, stats, gamma, beta = ctx.saved_tensors
+        has_bias, has_gamma, has_beta = ctx.hc
+        dy = dy.contiguous()
+        n, C = x.shape
+        dx = torch.empty_like(x)
+        grads = torch.empty((3, C), dtype=torch.float32, device=x.device)     # dgamma, dbeta, dbias
+        ws = _workspace(lib.hc_bn_relu_workspace_bytes(n, C), x.device)
+        sp, gp = stats.data_ptr(), grads.data_ptr()
+        _check(lib.hc_bn_relu_bwd(_ptr(dy), _ptr(x), _ptr(gamma if has_gamma else None),
+                                  _ptr(beta if has_beta else None), _c_p(sp), _c_p(sp + 4 * C), _ptr(dx),
+                                  _c_p(gp), _c_p(gp + 4 * C), _c_p(gp + 8 * C if has_bias else None), n, C,
+                                  _ptr(ws), ws.numel(), _ptr(_ticket(x.device)), _stream()), "hc_bn_relu_bwd")
+        return (dx, grads[2] if has_bias else None, grads[0] if has_gamma else None,
+                grads[1] if has_beta else None, None, None, None, None)
+
+
+def bias_bn_relu(x, bias, gamma, beta, running_mean, running_var, momentum, eps):
+    """Training-mode ``relu(batch_norm(x + bias))``; x is [n, C] fp32 on the GPU, n >= 2."""
+    _dev(x, "x")
+    if x.dim() != 2:
+        raise ValueError("x must be [n, C]")
+    if x.shape[0] < 2:
+        raise ValueError("Expected more than 1 value per channel when training, got input size %s"
+                         % (tuple(x.shape),))
+    if not bn_relu_supported(x, x.shape[1]):
+        raise ValueError("hc_bn_relu: fp32 on the GPU with C % 4 == 0 and C <= 1024")
+    for name, t in (("bias", bias), ("gamma", gamma), ("beta", beta), ("running_mean", running_mean),
+                    ("running_var", running_var)):
+        if t is not None:
+            _dev(t, name, torch.float32)
+            if t.numel() != x.shape[1]:
+                raise ValueError(f"{name} must hold C = {x.shape[1]} values")
+    return _BiasBnRelu.apply(x, bias, gamma, beta, running_mean, running_var, momentum, eps)
 
 
 def evict(checkin, slot2full, full2slot, stale_iter, sub2slot=None, score=None, thres=None):

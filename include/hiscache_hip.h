@@ -396,6 +396,38 @@ int hc_ring_lookup(const int64_t *full2slot, int64_t n_full, const int64_t *ids,
                    int table_dtype, int64_t capacity, int64_t F, int64_t *slot_out, float *rows_out,
                    int64_t n, void *stream);
 
+/* ---------------------------------------------------------------- layer epilogue
+ * hc_bn_relu_fwd / hc_bn_relu_bwd: the training-mode epilogue of a hidden
+ * layer, `x = self.bns[i](x); x = F.relu(x)` (hiscache/history_model.py:139-140,
+ * 386-387) behind a convolution whose linear layer adds a bias
+ * (history_model.py:66,94), as two launches forward and two backward.
+ *   forward:  mean[c], var[c] (biased) over the n rows of x[n, C] (fp32);
+ *             save_mean = mean, save_invstd = 1/sqrt(var + eps);
+ *             y = max(0, (x - mean) * invstd * gamma + beta);
+ *             running_mean = (1 - momentum) * running_mean + momentum * (mean + bias),
+ *             running_var  = (1 - momentum) * running_var + momentum * var * n/(n-1)
+ *             (torch.nn.BatchNorm1d's rule; both nullable).
+ *   backward: dy' = dy where y > 0, else 0; dbeta = sum dy', dgamma = sum dy' * xhat,
+ *             dx = gamma * invstd * (dy' - dbeta/n - xhat * dgamma/n), dbias = 0.
+ * bias (nullable) is a per-column constant that the caller has NOT added to x:
+ * in front of a normalisation it cancels in y and has zero gradient; it only
+ * shifts the mean that the running statistics record.  gamma / beta nullable
+ * (1 / 0).  x is the forward's input in both calls.  C % 4 == 0, C <= 1024
+ * (HC_EUNSUPPORTED otherwise).  Column statistics are summed per slab of rows and
+ * the slabs merged in slab order: results do not depend on scheduling.
+ * ticket: one 32-bit word of device memory that is zero on entry and zero again
+ * when the call's kernels have run; calls that share a ticket must not overlap.
+ * workspace: hc_bn_relu_workspace_bytes(n, C), 16-byte aligned; not preserved. */
+size_t hc_bn_relu_workspace_bytes(int64_t n, int64_t C);
+int hc_bn_relu_fwd(const float *x, const float *bias, const float *gamma, const float *beta,
+                   float *running_mean, float *running_var, float momentum, float eps, float *y,
+                   float *save_mean, float *save_invstd, int64_t n, int64_t C, void *workspace,
+                   size_t workspace_bytes, unsigned *ticket, void *stream);
+int hc_bn_relu_bwd(const float *dy, const float *x, const float *gamma, const float *beta,
+                   const float *save_mean, const float *save_invstd, float *dx, float *dgamma,
+                   float *dbeta, float *dbias, int64_t n, int64_t C, void *workspace,
+                   size_t workspace_bytes, unsigned *ticket, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
