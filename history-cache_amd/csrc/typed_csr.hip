@@ -74,14 +74,17 @@ __global__ __launch_bounds__(HC_BLOCK) void tc_place(const int64_t *__restrict__
                                                       const int64_t *__restrict__ et,
                                                       const uint8_t *__restrict__ used,
                                                       const int64_t *__restrict__ ptr2,
-                                                      int64_t *__restrict__ idx2, int64_t R, int64_t E, int K,
-                                                      int64_t n_src) {
+                                                      int64_t *__restrict__ idx2,
+                                                      float *__restrict__ edge_weight, int64_t R, int64_t E,
+                                                      int K, int64_t n_src) {
   const int lane = hc_lane();
   const int64_t row = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
   if (row >= R) return;
   const int64_t begin = ptr[row];
   const int64_t full_end = ptr[row + 1];
   const int64_t end = full_end < E ? full_end : E;
+  // what an edge of this row weighs in the row's mean over ALL its edges (kept or dropped)
+  const float w = 1.0f / (float)(full_end - begin > 0 ? full_end - begin : 1);
   // lane k: next free slot of group (row, k)
   int64_t next = lane < K ? ptr2[row * K + lane] : 0;
   const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (HC_WAVE - lane));
@@ -97,7 +100,10 @@ __global__ __launch_bounds__(HC_BLOCK) void tc_place(const int64_t *__restrict__
     const uint32_t lo = (uint32_t)__shfl((int)(uint32_t)(uint64_t)next, from, HC_WAVE);
     const uint32_t hi = (uint32_t)__shfl((int)(uint32_t)((uint64_t)next >> 32), from, HC_WAVE);
     const int64_t start = (int64_t)(((uint64_t)hi << 32) | lo);
-    if (ed.ok && start + rank < E) idx2[start + rank] = ed.src;
+    if (ed.ok && start + rank < E) {
+      idx2[start + rank] = ed.src;
+      if (edge_weight != nullptr) edge_weight[start + rank] = w;
+    }
     next += add;
   }
 }
@@ -123,8 +129,8 @@ extern "C" size_t hc_typed_csr_workspace_bytes(int64_t R, int num_rel) {
 
 extern "C" int hc_typed_csr(const int64_t *ptr, const int64_t *idx, const int64_t *edge_types,
                             const uint8_t *used_mask, int64_t R, int64_t E, int64_t n_src, int num_rel,
-                            int64_t *ptr2, int64_t *idx2, int64_t *cnt, int64_t *deg, void *workspace,
-                            size_t workspace_bytes, void *stream) {
+                            int64_t *ptr2, int64_t *idx2, int64_t *cnt, int64_t *deg, float *edge_weight,
+                            void *workspace, size_t workspace_bytes, void *stream) {
   HC_REQUIRE(R >= 0 && E >= 0 && n_src >= 0 && num_rel > 0 && ptr2);
   if (num_rel > TC_MAX_REL) return HC_EUNSUPPORTED;
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -144,8 +150,8 @@ extern "C" int hc_typed_csr(const int64_t *ptr, const int64_t *idx, const int64_
   if (rocprim::inclusive_scan(workspace, scan_bytes, cnt, ptr2 + 1, (size_t)groups, rocprim::plus<int64_t>(),
                               st) != hipSuccess)
     return HC_ELAUNCH;
-  tc_place<<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, edge_types, used_mask, ptr2, idx2, R, E,
-                                                             num_rel, n_src);
+  tc_place<<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(ptr, idx, edge_types, used_mask, ptr2, idx2,
+                                                             edge_weight, R, E, num_rel, n_src);
   return hc_launch_status();
 }
 

@@ -93,7 +93,7 @@ _SIGNATURES = {
     "hc_typed_csr_workspace_bytes": (_c_sz, [_c_i64, _c_int]),
     "hc_edge_types_by_ranges": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_p, _c_p, _c_i64, _c_i64, _c_p]),
     "hc_typed_csr": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_p,
-                              _c_p, _c_sz, _c_p]),
+                              _c_p, _c_p, _c_sz, _c_p]),
 }
 
 _lib_handle = None
@@ -679,13 +679,15 @@ def ring_lookup(full2slot, ids, table, checkin=None, now=0, age_limit=1 << 62, w
 MAX_TYPED_RELATIONS = 64
 
 
-def typed_csr(ptr, idx, edge_types, num_rel, num_node, n_src, used_mask=None):
+def typed_csr(ptr, idx, edge_types, num_rel, num_node, n_src, used_mask=None, want_weights=False):
     """Regroup the edges of the first ``num_node`` rows by (row, relation), keeping the edge order
     inside every group.  Returns (ptr2[num_node*num_rel+1], idx2, cnt[num_node, num_rel], deg[num_node]);
     edges with a relation outside [0, num_rel), a source outside [0, n_src) or a source that
     ``used_mask`` (bool[n_src]) rules out are dropped.  Only the first ptr2[-1] entries of idx2 are
     defined.  The grouping the reference obtains from a per-call sort by relation
-    (/root/reference/hiscache/history_model.py:248-270)."""
+    (/root/reference/hiscache/history_model.py:248-270).  With ``want_weights`` a fifth result holds,
+    beside every entry of idx2, 1/deg of its row (fp32): the edge values that turn the weighted
+    aggregation over the groups into each group's share of the row's mean."""
     lib = load_library()
     _dev(ptr, "ptr", torch.int64)
     _dev(idx, "idx", torch.int64)
@@ -707,11 +709,15 @@ def typed_csr(ptr, idx, edge_types, num_rel, num_node, n_src, used_mask=None):
     idx2 = torch.empty(max(E, 1), dtype=torch.int64, device=dev)
     cnt = torch.empty(R * K, dtype=torch.int64, device=dev)
     deg = torch.empty(R, dtype=torch.int64, device=dev)
+    weights = torch.empty(max(E, 1), dtype=torch.float32, device=dev) if want_weights else None
     ws_bytes = int(lib.hc_typed_csr_workspace_bytes(R, K))
     ws = _workspace(ws_bytes, dev)
     rc = lib.hc_typed_csr(_ptr(ptr), _ptr(idx), _ptr(edge_types), _ptr(used_mask), R, E, int(n_src), K,
-                          _ptr(ptr2), _ptr(idx2), _ptr(cnt), _ptr(deg), _ptr(ws), ws_bytes, _stream())
+                          _ptr(ptr2), _ptr(idx2), _ptr(cnt), _ptr(deg), _ptr(weights), _ptr(ws), ws_bytes,
+                          _stream())
     _check(rc, "hc_typed_csr")
+    if want_weights:
+        return ptr2, idx2, cnt.view(R, K), deg, weights
     return ptr2, idx2, cnt.view(R, K), deg
 
 

@@ -327,14 +327,18 @@ int hc_count_num(const int64_t *arr, int64_t n, int64_t mmax, int32_t *out, void
  * used_mask[src] != 0.  Only edge slots below E are read (E = entries
  * available in idx and in edge_types).  Outputs: ptr2[R*num_rel + 1],
  * idx2[E] (only the first ptr2[R*num_rel] entries are written),
- * cnt[R*num_rel] = group sizes, deg[R] = full row degrees ptr[r+1]-ptr[r].
- * num_rel <= 64 (HC_EUNSUPPORTED above).  Integer work only: results are
- * exact and independent of scheduling. */
+ * cnt[R*num_rel] = group sizes, deg[R] = full row degrees ptr[r+1]-ptr[r],
+ * edge_weight[E] (fp32, nullable; written where idx2 is) = 1/deg of the edge's
+ * row: with these weights the weighted aggregation over the groups gives each
+ * group's share of the row's mean over all its edges directly
+ * (sum over the group / deg), without a pass that rescales group means.
+ * num_rel <= 64 (HC_EUNSUPPORTED above).  Results are exact and independent of
+ * scheduling. */
 size_t hc_typed_csr_workspace_bytes(int64_t R, int num_rel);
 int hc_typed_csr(const int64_t *ptr, const int64_t *idx, const int64_t *edge_types,
                  const uint8_t *used_mask, int64_t R, int64_t E, int64_t n_src, int num_rel,
-                 int64_t *ptr2, int64_t *idx2, int64_t *cnt, int64_t *deg, void *workspace,
-                 size_t workspace_bytes, void *stream);
+                 int64_t *ptr2, int64_t *idx2, int64_t *cnt, int64_t *deg, float *edge_weight,
+                 void *workspace, size_t workspace_bytes, void *stream);
 
 /* hc_edge_types_by_ranges: relation of every edge of the first R rows from the
  * node types of its ends, out[e] = pair_to_rel[type(row) * T + type(idx[e])]

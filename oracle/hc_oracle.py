@@ -306,6 +306,14 @@ def typed_csr(ptr, idx, edge_types, num_rel, num_node, n_src, used_mask=None):
     return ptr2, idx2[:ptr2[-1]], cnt.reshape(R, K), deg
 
 
+def typed_csr_weights(ptr2, deg, num_rel):
+    """The edge weights hc_typed_csr writes beside idx2: fp32 1/deg of the edge's row (deg counts every
+    edge of the row, kept or dropped)."""
+    ptr2, deg = _i64(ptr2), _i64(deg)
+    per_group = np.repeat(np.float32(1.0) / np.maximum(deg, 1).astype(np.float32), int(num_rel))
+    return np.repeat(per_group, np.diff(ptr2)).astype(np.float32)
+
+
 def edge_types_by_ranges(ptr, idx, sub_to_full, num_node, bounds, pair_to_rel):
     """Relation per edge from the node types of its ends (numpy statement; type = number of bounds
     the full id has reached).  -1 outside the first ``num_node`` rows and for sources out of range.

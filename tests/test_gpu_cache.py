@@ -619,6 +619,51 @@ def test_rgcn_typed_aggregation_matches_dense_cpu(feat_dtype):
     assert cache.last_record_mask.shape[0] == n1
 
 
+@pytest.mark.parametrize("feat_dtype", [torch.float32, torch.float16])
+def test_fused_rgcn_layer_equals_the_operator_by_operator_spelling(feat_dtype):
+    """_RgcnConvFunction (edge weights 1/deg, one node) against the spelling with group means rescaled by
+    cnt/deg and torch's autograd: outputs, weight gradient, input gradient, gradient kept on the history
+    layer's output; with and without history, at an inner size on either side of the split-GEMM switch."""
+    from hiscache.history_model import MyRGCNConvHistory2
+    from helpers import random_csr
+    rng = np.random.default_rng(21)
+    torch.manual_seed(4)
+    for (R, N, Fin, H, K, use_hist, x_grad) in ((300, 900, 64, 32, 5, True, True), (700, 2000, 512, 64, 5, True, False),
+                                                (41, 200, 448, 16, 5, False, True)):
+        ptr, idx = random_csr(rng, R + 30, N, 9)
+        rel = rng.integers(0, K, size=len(idx))
+        used = rng.random(N) < 0.8
+        t = lambda a: torch.from_numpy(a).to(DEV)
+        x = torch.randn(N, Fin, device=DEV).to(feat_dtype)
+        hmap = torch.where(torch.rand(R, device=DEV) < 0.4, torch.arange(R, device=DEV), torch.full((R,), -1, device=DEV))
+        hbuf = torch.randn(R, H, device=DEV)
+        g = torch.randn(R, H, device=DEV)
+        res = {}
+        for fused in (True, False):
+            conv = MyRGCNConvHistory2(Fin, H, K, need_grad=True).to(DEV).train()
+            with torch.no_grad():
+                conv.linear.copy_(torch.randn(K, Fin, H, generator=torch.Generator().manual_seed(9)) * 0.1)
+            conv.fused = fused
+            xi = x.clone().requires_grad_(x_grad and feat_dtype == torch.float32)
+            out, his = conv(xi, t(ptr), t(idx), t(rel), None, hmap if use_hist else None, hbuf if use_hist else None,
+                            t(used), H if use_hist else 0, R)
+            out.backward(g)
+            res[fused] = (out.detach(), conv.linear.grad.clone(), None if xi.grad is None else xi.grad.clone(),
+                          his.grad.clone() if his.retains_grad else None)
+            want_count = np.bincount(rel, minlength=K + 1)
+            want_count[0] = 0                                   # count_num skips value 0
+            np.testing.assert_array_equal(conv.last_count.cpu().numpy(), want_count)
+        tol = 2e-3 if feat_dtype == torch.float16 else 2e-5
+        for a, b, what in zip(res[True], res[False], ("out", "weight grad", "input grad", "kept grad")):
+            assert (a is None) == (b is None), what
+            if a is not None:
+                scale = float(b.abs().max()) or 1.0
+                assert float((a - b).abs().max()) <= tol * scale, (what, R, Fin)
+        if use_hist:
+            hit = (hmap != -1).cpu().numpy()
+            np.testing.assert_array_equal(res[True][0].cpu().numpy()[hit], hbuf.cpu().numpy()[hit])
+
+
 def test_typed_csr_groups_edges_by_row_and_relation():
     from hiscache import typed_csr
     from helpers import random_csr
@@ -656,12 +701,16 @@ def test_typed_csr_matches_oracle(orc, K, with_mask, short_types):
     used = (rng.random(N) < 0.7) if with_mask else None
     import hiscache_backend as be
     t = lambda a: None if a is None else torch.from_numpy(a).to(DEV)
-    ptr2, idx2, cnt, deg = be.typed_csr(t(ptr), t(idx), t(rel), K, R, N, t(used))
+    ptr2, idx2, cnt, deg, wts = be.typed_csr(t(ptr), t(idx), t(rel), K, R, N, t(used), want_weights=True)
     w_ptr2, w_idx2, w_cnt, w_deg = orc.typed_csr(ptr, idx, rel, K, R, N, used)
     np.testing.assert_array_equal(ptr2.cpu().numpy(), w_ptr2)
     np.testing.assert_array_equal(idx2.cpu().numpy()[: w_ptr2[-1]], w_idx2)
     np.testing.assert_array_equal(cnt.cpu().numpy(), w_cnt)
     np.testing.assert_array_equal(deg.cpu().numpy(), w_deg)
+    # edge weights: 1/deg of the edge's row, so that the weighted sum over a group is its share of the mean
+    np.testing.assert_array_equal(wts.cpu().numpy()[: w_ptr2[-1]], orc.typed_csr_weights(w_ptr2, w_deg, K))
+    again = be.typed_csr(t(ptr), t(idx), t(rel), K, R, N, t(used))
+    assert len(again) == 4 and torch.equal(again[1][: w_ptr2[-1]], idx2[: w_ptr2[-1]])
     p0 = be.typed_csr(t(ptr), t(idx), t(rel), K, 0, N, t(used))[0]
     assert p0.cpu().tolist() == [0]
     with pytest.raises(ValueError):
