@@ -34,12 +34,14 @@ def test_aggregation_and_admission_replay_like_eager(be):
     thres = torch.tensor([11.3], device=DEV)          # about the median norm of a 128-dim N(0,1) row
     gather_ids = T(rng.integers(0, N, size=2000).astype(np.int64))
     N_all = max(R, N)
+    bn_bias, bn_gamma, bn_beta = (torch.randn(F, device=DEV) for _ in range(3))
 
     def fresh_state():
         return dict(table=torch.zeros(cap, F, dtype=torch.float16, device=DEV),
                     full2slot=torch.full((3 * R,), -1, dtype=torch.int64, device=DEV),
                     slot2full=torch.full((cap,), -1, dtype=torch.int64, device=DEV),
-                    header=torch.zeros(1, dtype=torch.int64, device=DEV))
+                    header=torch.zeros(1, dtype=torch.int64, device=DEV),
+                    running_mean=torch.zeros(F, device=DEV), running_var=torch.ones(F, device=DEV))
 
     def work(st):
         out = be._aggr_fwd(be.SUBST_ROW, ptr_d, idx_d, x, hmap_d, hbuf, F, None, R)
@@ -50,7 +52,11 @@ def test_aggregation_and_admission_replay_like_eager(be):
         rows = be.gather_rows(x, gather_ids)             # more rows than the capped grid of a host-memory table
         found = be.lookup(st["full2slot"], sub_to_full, 0)
         used = torch.stack(be.count_history_reconstruct(ptr_d, idx_d, hmap_d[:R], N_all, 64, 2))
-        return out, tr[0], tr[1], gx, gh, mask, score, rows, found, used
+        # a hidden layer's epilogue (its block counter is left at zero by every launch) and its backward
+        zin = out.detach().requires_grad_(True)
+        act = be.bias_bn_relu(zin, bn_bias, bn_gamma, bn_beta, st["running_mean"], st["running_var"], 0.1, 1e-5)
+        (dz,) = torch.autograd.grad(act, zin, g)
+        return out, tr[0], tr[1], gx, gh, mask, score, rows, found, used, act.detach(), dz
 
     def load_inputs(seed):
         gen = torch.Generator(device=DEV).manual_seed(seed)
@@ -77,8 +83,8 @@ def test_aggregation_and_admission_replay_like_eager(be):
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        for name, a, b in zip(("out", "ptrT", "rowT", "grad_x", "grad_h", "mask", "score", "rows", "found", "used"),
-                              captured, eager):
+        for name, a, b in zip(("out", "ptrT", "rowT", "grad_x", "grad_h", "mask", "score", "rows", "found", "used",
+                               "epilogue", "epilogue gradient"), captured, eager):
             if name == "rowT":                     # only the first ptrT[-1] entries are defined
                 n_tr = int(eager[1][-1])
                 a, b = a[:n_tr], b[:n_tr]
