@@ -448,33 +448,16 @@ def c3_batched_layer(args, samples=None):
     import torch
 
     import hiscache_backend as be
-    from hiscache.synthetic import direct_power_law_batch, lognormal_grads
+    from hiscache.synthetic import batched_history_layer, direct_power_law_batch, lognormal_grads
 
     dev = "cuda:0"
     s = args.scale
     N, H = int(111_000_000 * s), 256
     if samples is None:
         samples = [direct_power_law_batch(N, 1000, [15, 10, 5], 2.0, 30 + i, degree_scale=2.6) for i in range(8)]
-    n_pre = len(samples)
     gen = torch.Generator(device=dev).manual_seed(33)
-    rows, cols, ptrs, idxs, hms = 0, 0, [np.zeros(1, np.int64)], [], []
-    k = 0
-    e_tot = 0
-    target = int(20_000_000 * s)
-    while e_tot < target:
-        smp = samples[k % min(8, n_pre)]
-        n1, n2 = int(smp["num_node_in_layer"][1]), int(smp["num_node_in_layer"][2])
-        p = smp["ptr"][: n1 + 1]
-        e = int(p[-1])
-        ptrs.append(p[1:] + e_tot)
-        idxs.append(smp["idx"][:e] + cols)
-        e_tot += e
-        rows += n1
-        cols += n2
-        k += 1
-    ptr = torch.from_numpy(np.concatenate(ptrs)).to(dev)
-    idx = torch.from_numpy(np.concatenate(idxs)).to(dev)
-    R, E, Nsrc = rows, e_tot, cols
+    ptr_h, idx_h, R, E, Nsrc = batched_history_layer(samples[:8], int(20_000_000 * s))
+    ptr, idx = torch.from_numpy(ptr_h).to(dev), torch.from_numpy(idx_h).to(dev)
     x = torch.randn(Nsrc, H, device=dev, generator=gen)
     hbuf = (0.5 * torch.randn(R, H, device=dev, generator=gen)).half()
     hmap = torch.where(torch.rand(R, device=dev, generator=gen) < 0.35, torch.arange(R, device=dev),

@@ -164,3 +164,26 @@ def lognormal_grads(n_rows, width, mu=-3.0, sigma=1.5, seed=4, device="cpu", gen
     norms = torch.exp(mu + sigma * torch.randn(n_rows, device=device, generator=g))
     d *= norms[:, None]
     return d
+
+
+def batched_history_layer(samples, target_edges):
+    """The history layer of many sampled batches side by side as one CSR block: for every batch its first
+    num_node_in_layer[1] rows (the 1-hop nodes) with their edges, source ids shifted so that the batches'
+    num_node_in_layer[2] sources do not overlap.  ``samples`` (results of direct_power_law_batch or of the
+    sampler) are repeated until the block holds ``target_edges`` edges.  Returns (ptr, idx, rows, edges,
+    sources) with numpy int64 arrays."""
+    rows, cols, e_tot, k = 0, 0, 0, 0
+    ptrs, idxs = [np.zeros(1, np.int64)], []
+    while e_tot < target_edges:
+        smp = samples[k % len(samples)]
+        n1, n2 = int(smp["num_node_in_layer"][1]), int(smp["num_node_in_layer"][2])
+        p = smp["ptr"][: n1 + 1]
+        e = int(p[-1])
+        ptrs.append(p[1:] + e_tot)
+        idxs.append(smp["idx"][:e] + cols)
+        e_tot += e
+        rows += n1
+        cols += n2
+        k += 1
+    return np.concatenate(ptrs), np.concatenate(idxs), rows, e_tot, cols
+

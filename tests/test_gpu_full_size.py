@@ -172,3 +172,161 @@ def test_c4_admission_full_size():
     assert torch.equal(slot2[mask], (s + A) % cap)
     assert int((full2slot != -1).sum()) == A                 # same nodes, moved to their new slots
     assert torch.equal(full2slot[sub_to_full[mask]], slot2[mask])
+
+
+def test_c2_view_without_substituted_sources(c2):
+    """The view the benchmark's step builds (edges of substituted sources left out) against the full one:
+    exactly the edges of unsubstituted sources, in the same order, hence the same bits in their gradient
+    rows; substituted sources get empty segments and zero rows."""
+    import hiscache_backend as be
+    ptrT_f, rowT_f, _ = c2["tr"]
+    tr = be.build_transpose(c2["ptr"], c2["idx"], None, R, N, want_edges=False, history_map_src=c2["hmap"])
+    ptrT, rowT, _ = tr
+    sub = c2["hmap"] != -1
+    seg_f, seg = ptrT_f[1:] - ptrT_f[:-1], ptrT[1:] - ptrT[:-1]
+    assert int(ptrT[0]) == 0
+    assert torch.equal(seg, torch.where(sub, torch.zeros_like(seg_f), seg_f))
+    live = int(ptrT[N])
+    assert live == int((~sub[c2["idx"]]).sum()) and 0.55 * E < live < 0.65 * E
+    keep = torch.repeat_interleave(~sub, seg_f)               # transposed edges of the full view that stay
+    assert torch.equal(rowT[:live], rowT_f[keep])
+    grad_x, _, _ = be._aggr_bwd(c2["ptr"], c2["idx"], tr, c2["g"], None, None, c2["feat"], False, None, 0, R, N)
+    assert float(grad_x[sub].abs().max()) == 0.0
+    assert torch.equal(grad_x[~sub], c2["grad_x"][~sub])
+
+
+# ------------------------------------------------------------------------------------------------
+# The papers100M-shaped history layer of about 800 sampled batches side by side (4.7 M rows, 20 M edges,
+# 20.8 M sources x 256, 35% of the rows taken from an fp16 row-aligned history buffer): the block whose
+# forward + view + backward + admission the benchmark reports as kernels.c3_batched.
+@pytest.fixture(scope="module")
+def c3b():
+    import hiscache_backend as be
+    from hiscache.synthetic import batched_history_layer, direct_power_law_batch
+    samples = [direct_power_law_batch(111_000_000, 1000, [15, 10, 5], 2.0, 30 + i, degree_scale=2.6) for i in range(8)]
+    ptr_h, idx_h, Rb, Eb, Nb = batched_history_layer(samples, 20_000_000)
+    ptr, idx = torch.from_numpy(ptr_h).to(DEV), torch.from_numpy(idx_h).to(DEV)
+    gen = torch.Generator(device=DEV).manual_seed(33)
+    x = torch.randn(Nb, F, device=DEV, generator=gen)
+    hbuf = (0.5 * torch.randn(Rb, F, device=DEV, generator=gen)).half()
+    hmap = torch.where(torch.rand(Rb, device=DEV, generator=gen) < 0.35, torch.arange(Rb, device=DEV),
+                       torch.full((Rb,), -1, device=DEV))
+    g = torch.randn(Rb, F, device=DEV, generator=gen)
+    print("full-size batched history layer built: %d rows, %d edges, %d sources" % (Rb, Eb, Nb), flush=True)
+    out = be._aggr_fwd(be.SUBST_ROW, ptr, idx, x, hmap, hbuf, F, None, Rb)
+    tr = be.build_transpose(ptr, idx, hmap, Rb, Nb, want_edges=False)
+    grad_x, _, _ = be._aggr_bwd(ptr, idx, tr, g, hmap, None, x, False, (Rb, F), F, Rb, Nb, want_hist_grad=False)
+    torch.cuda.synchronize()
+    yield dict(ptr=ptr, idx=idx, x=x, hbuf=hbuf, hmap=hmap, g=g, out=out, tr=tr, grad_x=grad_x, R=Rb, E=Eb, N=Nb)
+    torch.cuda.empty_cache()
+
+
+def test_c3_batched_forward(c3b):
+    c = c3b
+    hit = c["hmap"] != -1
+    assert 4_000_000 < c["R"] < 6_000_000 and c["E"] >= 20_000_000 and 0.33 < float(hit.float().mean()) < 0.37
+    # history rows carry the fp16 buffer row exactly
+    assert torch.equal(c["out"][hit], c["hbuf"][hit].float())
+    # computed rows: closed form on a sample, and the degree-weighted column sums of all of them
+    gen = torch.Generator(device=DEV).manual_seed(21)
+    deg = c["ptr"][1:] - c["ptr"][:-1]
+    cand = torch.nonzero(~hit).view(-1)
+    sample = cand[torch.randint(0, cand.numel(), (3000,), device=DEV, generator=gen)]
+    sample = torch.cat([sample, cand[torch.topk(deg[cand], 8).indices]])
+    worst = 0.0
+    for r, b, e in zip(sample.tolist(), c["ptr"][sample].tolist(), c["ptr"][sample + 1].tolist()):
+        want = c["x"][c["idx"][b:e]].double().sum(0) / max(e - b, 1)
+        got = c["out"][r].double()
+        worst = max(worst, float((got - want).abs().max() / want.abs().max().clamp(min=1e-30)) if e > b
+                    else float(got.abs().max()))
+    assert worst < 1e-5, worst
+    w = torch.where(hit, torch.zeros_like(deg), deg).double()
+    lhs = (c["out"].double() * w[:, None]).sum(0)
+    row_of = torch.repeat_interleave(torch.arange(c["R"], device=DEV), deg)
+    rhs = torch.zeros(F, dtype=torch.float64, device=DEV)
+    for lo in range(0, c["E"], 2_000_000):
+        sl = slice(lo, lo + 2_000_000)
+        keep = ~hit[row_of[sl]]
+        rhs += c["x"][c["idx"][sl][keep]].double().sum(0)
+    assert float((lhs - rhs).abs().max()) < 1e-5 * float(rhs.abs().max()) + 1e-3
+
+
+def test_c3_batched_view_and_backward(c3b):
+    c = c3b
+    ptrT, rowT, _ = c["tr"]
+    hit = c["hmap"] != -1
+    deg = c["ptr"][1:] - c["ptr"][:-1]
+    row_of = torch.repeat_interleave(torch.arange(c["R"], device=DEV), deg)
+    live = ~hit[row_of]
+    n_live = int(live.sum())
+    assert int(ptrT[0]) == 0 and int(ptrT[c["N"]]) == n_live
+    seg = ptrT[1:] - ptrT[:-1]
+    assert torch.equal(seg, torch.bincount(c["idx"][live], minlength=c["N"]))
+    src_of = torch.repeat_interleave(torch.arange(c["N"], device=DEV), seg)
+    same = src_of[1:] == src_of[:-1]
+    rt = rowT[:n_live]
+    assert bool((rt[1:][same] >= rt[:-1][same]).all())
+    assert not bool(hit[rt.long()].any())                      # no edge of a history row survives
+    for a, b in ((1_000_003, 998_244_353), (7, 1_000_000_007)):
+        want = int(((c["idx"][live] * a + row_of[live] * b) % 2_147_483_647).sum())
+        got = int(((src_of * a + rt.long() * b) % 2_147_483_647).sum())
+        assert want == got
+    # backward: closed form on sampled sources, then the adjoint identity over the computed rows
+    gen = torch.Generator(device=DEV).manual_seed(22)
+    sample = torch.randint(0, c["N"], (3000,), device=DEV, generator=gen)
+    sample = torch.cat([sample, torch.topk(seg, 8).indices])
+    degd = deg.double()
+    worst = 0.0
+    for s_, b, e in zip(sample.tolist(), ptrT[sample].tolist(), ptrT[sample + 1].tolist()):
+        rows = rowT[b:e].long()
+        got = c["grad_x"][s_].double()
+        if e > b:
+            want = (c["g"][rows].double() / degd[rows][:, None]).sum(0)
+            worst = max(worst, float((got - want).abs().max() / want.abs().max().clamp(min=1e-30)))
+        else:
+            worst = max(worst, float(got.abs().max()))
+    assert worst < 1e-5, worst
+    lhs = float((c["out"].double() * c["g"].double())[~hit].sum())
+    rhs = 0.0
+    for lo in range(0, c["N"], 2_000_000):
+        rhs += float((c["x"][lo:lo + 2_000_000].double() * c["grad_x"][lo:lo + 2_000_000].double()).sum())
+    assert abs(lhs - rhs) < 1e-5 * max(abs(lhs), abs(rhs)) + 1e-2, (lhs, rhs)
+
+
+def test_c3_batched_admission_and_bit_identity(c3b):
+    import hiscache_backend as be
+    from hiscache.synthetic import lognormal_grads
+    c = c3b
+    Rb = c["R"]
+    gen = torch.Generator(device=DEV).manual_seed(34)
+    grad = lognormal_grads(Rb, F, -3.0, 1.5, device=DEV, generator=gen)
+    cap = max(Rb, 1 << 20)
+    table = torch.zeros(cap, F, dtype=torch.float16, device=DEV)
+    f2s = torch.full((2 * Rb,), -1, dtype=torch.int64, device=DEV)
+    s2f = torch.full((cap,), -1, dtype=torch.int64, device=DEV)
+    chk = torch.full((cap,), -1, dtype=torch.int64, device=DEV)
+    hdr = torch.zeros(1, dtype=torch.int64, device=DEV)
+    sub_to_full = torch.randperm(2 * Rb, device=DEV, generator=gen)[:Rb].contiguous()
+    thr = torch.tensor([0.05], device=DEV)
+    # the layer's own output is what gets admitted, the rows' slots are the history map
+    mask, score, slots = be.grad_check(grad, c["out"], c["hmap"], sub_to_full, thr, table, f2s, s2f, hdr, 1,
+                                       checkin=chk, want_slots=True)
+    want = (score < thr) & (c["hmap"] == -1)
+    assert torch.equal(mask, want)
+    A = int(mask.sum())
+    assert 0.25 * Rb < A < 0.45 * Rb and int(hdr) == A % cap
+    rank = torch.cumsum(mask.long(), 0) - mask.long()
+    assert torch.equal(slots, torch.where(mask, rank % cap, torch.full_like(rank, -1)))
+    s_ = slots[mask]
+    assert torch.equal(table[s_], c["out"][mask].half())
+    assert torch.equal(s2f[s_], sub_to_full[mask]) and torch.equal(f2s[sub_to_full[mask]], s_)
+    assert int((f2s != -1).sum()) == A and bool((chk[s_] == 1).all())
+    # forward, view and backward give the same bits when run again
+    out = be._aggr_fwd(be.SUBST_ROW, c["ptr"], c["idx"], c["x"], c["hmap"], c["hbuf"], F, None, Rb)
+    assert torch.equal(out, c["out"])
+    tr = be.build_transpose(c["ptr"], c["idx"], c["hmap"], Rb, c["N"], want_edges=False)
+    n_live = int(tr[0][-1])
+    assert torch.equal(tr[0], c["tr"][0]) and torch.equal(tr[1][:n_live], c["tr"][1][:n_live])
+    grad_x, _, _ = be._aggr_bwd(c["ptr"], c["idx"], tr, c["g"], c["hmap"], None, c["x"], False, (Rb, F), F, Rb, c["N"],
+                                want_hist_grad=False)
+    assert torch.equal(grad_x, c["grad_x"])
