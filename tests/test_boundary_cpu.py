@@ -160,3 +160,56 @@ def test_header_is_plain_c_and_links(tmp_path):
                    check=True, capture_output=True, text=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True, timeout=60).stdout
     assert out.startswith("hiscache_hip") and out.strip().endswith("|1")
+
+
+def test_relational_gemm_spellings_equal_the_single_gemm():
+    """The split spellings of the relational layer's two large GEMMs (over relations forward, over row
+    slabs for the weight gradient) against the plain products, on both sides of the size switch and with
+    row counts that leave a remainder."""
+    import torch
+    from hiscache import history_model as hm
+    torch.manual_seed(0)
+    for n, K, Fin, H in ((37, 5, 16, 8), (101, 5, 512, 24), (8, 3, 700, 4), (7, 5, 512, 6), (64, 1, 4096, 8)):
+        agg = torch.randn(n, K, Fin, dtype=torch.float64)
+        w = torch.randn(K, Fin, H, dtype=torch.float64)
+        g = torch.randn(n, H, dtype=torch.float64)
+        want = agg.reshape(n, K * Fin) @ w.reshape(K * Fin, H)
+        assert torch.allclose(hm._rel_matmul(agg, w), want, rtol=1e-12, atol=1e-12)
+        want_g = (agg.reshape(n, K * Fin).t() @ g).view(K, Fin, H)
+        got_g = hm._rel_weight_grad(agg, g)
+        assert got_g.shape == (K, Fin, H) and torch.allclose(got_g, want_g, rtol=1e-12, atol=1e-12)
+
+
+def test_bn_relu_takes_the_torch_operators_off_the_gpu():
+    """Without a GPU tensor (or in evaluation mode) bn_relu is exactly relu(bn(x + bias)), module state
+    included."""
+    import torch
+    import torch.nn.functional as F
+    from hiscache.history_model import bn_relu
+    torch.manual_seed(1)
+    a, b = torch.nn.BatchNorm1d(12), torch.nn.BatchNorm1d(12)
+    b.load_state_dict(a.state_dict())
+    x, bias = torch.randn(9, 12), torch.randn(12)
+    for mode in ("train", "eval"):
+        getattr(a, mode)(), getattr(b, mode)()
+        assert torch.equal(bn_relu(x, a, bias), F.relu(b(x + bias)))
+        assert torch.equal(a.running_mean, b.running_mean) and torch.equal(a.running_var, b.running_var)
+        assert int(a.num_batches_tracked) == int(b.num_batches_tracked)
+
+
+def test_batched_history_layer_block_layout():
+    """Rows, edge offsets and source shifts of the block the benchmark and the full-size test build."""
+    from hiscache.synthetic import batched_history_layer, direct_power_law_batch
+    samples = [direct_power_law_batch(1_000_000, 50, [5, 4, 3], 2.0, 3 + i, degree_scale=2.0) for i in range(3)]
+    ptr, idx, R, E, N = batched_history_layer(samples, 4000)
+    assert ptr[0] == 0 and ptr[-1] == E == len(idx) and len(ptr) == R + 1 and E >= 4000
+    assert (np.diff(ptr) >= 0).all() and idx.min() >= 0 and idx.max() < N
+    row0, col0, k = 0, 0, 0
+    while row0 < R:
+        smp = samples[k % 3]
+        n1, n2 = int(smp["num_node_in_layer"][1]), int(smp["num_node_in_layer"][2])
+        e0, e1 = int(ptr[row0]), int(ptr[row0 + n1])
+        np.testing.assert_array_equal(ptr[row0:row0 + n1 + 1] - e0, smp["ptr"][: n1 + 1])
+        np.testing.assert_array_equal(idx[e0:e1] - col0, smp["idx"][: e1 - e0])
+        row0, col0, k = row0 + n1, col0 + n2, k + 1
+    assert row0 == R and col0 == N
