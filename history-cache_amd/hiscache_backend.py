@@ -159,8 +159,32 @@ def _empty(t):
     return t is None or t.numel() == 0
 
 
+# Scratch memory of the calls.  Every entry point's workspace is dead when its kernels have run, and calls
+# issued on one stream run in order, so the calls of a stream share one buffer that grows to the largest
+# request seen (up to _WS_KEEP_BYTES; larger requests, and calls on a capturing stream, whose buffer must
+# stay alive with the graph, get a buffer of their own).  Sampled batches change every size at every
+# iteration; without this each call paid an allocator look-up, and a device allocation when it missed.
+_WS_KEEP_BYTES = 64 << 20
+_ws_cache = {}
+
+
 def _workspace(nbytes, device):
-    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+    nbytes = max(int(nbytes), 256)
+    if nbytes > _WS_KEEP_BYTES or torch.cuda.is_current_stream_capturing():
+        return torch.empty(nbytes, dtype=torch.uint8, device=device)
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    buf = _ws_cache.get(key)
+    if buf is None or buf.numel() < nbytes:
+        size = 1 << 20
+        while size < nbytes:
+            size <<= 1
+        buf = _ws_cache[key] = torch.empty(size, dtype=torch.uint8, device=device)
+    return buf
+
+
+def release_workspaces():
+    """Drop the per-stream scratch buffers (they are allocated again on demand)."""
+    _ws_cache.clear()
 
 
 # With HISCACHE_CHECK_INPUTS=1 every aggregation call first checks its CSR block on the device
