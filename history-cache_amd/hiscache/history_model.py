@@ -26,6 +26,31 @@ class _GradSink:
         self.target = None
 
 
+# rocBLAS's kernel choice for a weight gradient g^T x ([H, n] x [n, F], n = rows of a sampled layer) is
+# erratic in n: measured on MI355X with H = 256, the single GEMM takes 52 us at n = 25 800 and F = 128,
+# 353 us at F = 256, 1.5 ms at n = 55 000 and 2.4 ms at n = 89 000 (one or two tiles walking the whole
+# inner dimension).  As a batched GEMM over slabs of 1 024 rows plus a sum over the slabs it takes 42, 69,
+# 72 - 131 and 107 - 193 us: linear in n.  Below this many rows the single GEMM is used (21 us at 5 800).
+_WGRAD_SLAB_ROWS = 1024
+_WGRAD_SPLIT_MIN_ROWS = 8192
+# The library's own kernel (hc_weight_grad: both operands of a SAGE layer in one pair of launches, 59 us at
+# n = 25 800 and F = 128, 102 us at n = 55 000) takes over from this many rows when the widths fit it.
+_WGRAD_KERNEL_MIN_ROWS = 2048
+
+
+def _weight_grad(g, x):
+    """g^T @ x for g [n, H], x [n, F] (both contiguous): the gradient of a linear layer's weight."""
+    n = g.shape[0]
+    if n < _WGRAD_SPLIT_MIN_ROWS:
+        return g.t() @ x
+    S = n // _WGRAD_SLAB_ROWS
+    m = n // S * S
+    out = torch.bmm(g[:m].view(S, m // S, -1).transpose(1, 2), x[:m].view(S, m // S, -1)).sum(0)
+    if m < n:
+        out.addmm_(g[m:].t(), x[m:])
+    return out
+
+
 class _SageConvFunction(torch.autograd.Function):
     """``lin_l(aggregate(x)) + lin_r(x[:n])`` as ONE autograd node.
 
@@ -67,12 +92,18 @@ class _SageConvFunction(torch.autograd.Function):
             his = sink.target()
             if his is not None:
                 his.grad = g_agg
-        g_wl = g_out.t() @ agg if need[1] else None
         g_bl = g_out.sum(0) if has_bias and need[2] else None
-        g_wr = None
+        g_wl = g_wr = None
+        root = None
         if has_root and need[3]:
             root = x[:R] if x.dtype == g_out.dtype else x[:R].to(g_out.dtype)
-            g_wr = g_out.t() @ root
+        if need[1] and root is not None and R >= _WGRAD_KERNEL_MIN_ROWS and be.weight_grad_supported(g_out, agg):
+            g_wl, g_wr = be.weight_grad(g_out, agg, root)          # both products in one pair of launches
+        else:
+            if need[1]:
+                g_wl = _weight_grad(g_out, agg)
+            if root is not None:
+                g_wr = _weight_grad(g_out, root)
         g_x = None
         if need[0]:
             n_src = x.shape[0]
@@ -287,7 +318,7 @@ def _rel_weight_grad(agg, g):
     """agg^T @ g in the weight's layout: agg [n, K, F], g [n, H] -> [K, F, H]."""
     n, K, Fin = agg.shape
     a2 = agg.reshape(n, K * Fin)
-    S = _REL_WGRAD_SLABS
+    S = max(_REL_WGRAD_SLABS, n // _WGRAD_SLAB_ROWS)
     m = n // S * S
     if K * Fin < _REL_SPLIT_MIN_INNER or m == 0:
         return (a2.t() @ g).view(K, Fin, -1)

@@ -90,6 +90,8 @@ _SIGNATURES = {
                                 _c_p, _c_i64, _c_i64, _c_p, _c_sz, _c_p, _c_p]),
     "hc_bn_relu_bwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64,
                                 _c_p, _c_sz, _c_p, _c_p]),
+    "hc_weight_grad_workspace_bytes": (_c_sz, [_c_i64, _c_i64, _c_i64, _c_int]),
+    "hc_weight_grad": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_sz, _c_p]),
     "hc_typed_csr_workspace_bytes": (_c_sz, [_c_i64, _c_int]),
     "hc_edge_types_by_ranges": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_p, _c_p, _c_i64, _c_i64, _c_p]),
     "hc_typed_csr": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_p,
@@ -826,6 +828,36 @@ class _BiasBnRelu(torch.autograd.Function):
                                   _ptr(ws), ws.numel(), _ptr(_ticket(x.device)), _stream()), "hc_bn_relu_bwd")
         return (dx, grads[2] if has_bias else None, grads[0] if has_gamma else None,
                 grads[1] if has_beta else None, None, None, None, None)
+
+
+def weight_grad_supported(g, x):
+    return (g.is_cuda and g.dtype == torch.float32 and x.dtype == torch.float32 and g.dim() == 2 and x.dim() == 2
+            and g.shape[1] % 64 == 0 and x.shape[1] % 64 == 0 and g.shape[1] <= 4096 and x.shape[1] <= 4096
+            and g.shape[0] >= 1)
+
+
+def weight_grad(g, x0, x1=None):
+    """``g.t() @ x0`` (and ``g.t() @ x1``): the weight gradients of a layer's linear maps on the matrix
+    cores, rows split into slabs that are added in a fixed order.  g [n, H], x [n, F], fp32."""
+    lib = load_library()
+    _dev(g, "g", torch.float32)
+    _dev(x0, "x0", torch.float32)
+    if x1 is not None:
+        _dev(x1, "x1", torch.float32)
+        if x1.shape != x0.shape:
+            raise ValueError("x1 must have x0's shape")
+    if g.dim() != 2 or x0.dim() != 2 or x0.shape[0] != g.shape[0]:
+        raise ValueError("g [n, H] and x [n, F] must have the same number of rows")
+    n, H = g.shape
+    F = x0.shape[1]
+    n_op = 1 if x1 is None else 2
+    dw = torch.empty((n_op, H, F), dtype=torch.float32, device=g.device)
+    ws = _workspace(lib.hc_weight_grad_workspace_bytes(n, H, F, n_op), g.device)
+    p = dw.data_ptr()
+    _check(lib.hc_weight_grad(_ptr(g), _ptr(x0), _ptr(x1), n, H, F, _c_p(p),
+                              _c_p(p + 4 * H * F) if x1 is not None else _c_p(None), _ptr(ws), ws.numel(),
+                              _stream()), "hc_weight_grad")
+    return (dw[0], dw[1]) if x1 is not None else dw[0]
 
 
 def bias_bn_relu(x, bias, gamma, beta, running_mean, running_var, momentum, eps):

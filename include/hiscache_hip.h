@@ -432,6 +432,22 @@ int hc_bn_relu_bwd(const float *dy, const float *x, const float *gamma, const fl
                    float *dbeta, float *dbias, int64_t n, int64_t C, void *workspace,
                    size_t workspace_bytes, unsigned *ticket, void *stream);
 
+/* hc_weight_grad: the gradient of a layer's linear maps, dw[H, F] = g^T x for
+ * g [n, H] and x [n, F] (fp32, row-major, contiguous) -- what autograd computes
+ * for `self.lin_l(out)` and `self.lin_r(x[:num_node])`
+ * (hiscache/history_model.py:94-98), whose weights are [H, F].  x1 / dw1
+ * (both or neither NULL) is a second operand that shares g: the aggregated rows
+ * and the root rows of a SAGE layer go through the same two launches.  The rows
+ * are split into slabs, every slab's product is computed on the matrix cores in
+ * fp32 and the slabs are added in slab order: no atomics, the result does not
+ * depend on scheduling (the slab partition is a function of n, H, F and the
+ * operand count).  H % 64 == 0, F % 64 == 0, both at most 4096
+ * (HC_EUNSUPPORTED otherwise); dw 16-byte aligned.
+ * workspace: hc_weight_grad_workspace_bytes(n, H, F, operands), 16-byte aligned. */
+size_t hc_weight_grad_workspace_bytes(int64_t n, int64_t H, int64_t F, int n_operands);
+int hc_weight_grad(const float *g, const float *x0, const float *x1, int64_t n, int64_t H, int64_t F,
+                   float *dw0, float *dw1, void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -180,6 +180,19 @@ def test_relational_gemm_spellings_equal_the_single_gemm():
         assert got_g.shape == (K, Fin, H) and torch.allclose(got_g, want_g, rtol=1e-12, atol=1e-12)
 
 
+def test_weight_gradient_slab_spelling_equals_the_single_gemm():
+    import torch
+    from hiscache import history_model as hm
+    torch.manual_seed(3)
+    for n in (5, 8191, 8192, 9000, 20_001):
+        g = torch.randn(n, 12, dtype=torch.float64)
+        x = torch.randn(n, 20, dtype=torch.float64)
+        assert torch.allclose(hm._weight_grad(g, x), g.t() @ x, rtol=1e-11, atol=1e-9)
+    x_view = torch.randn(9000, 40, dtype=torch.float64)[:, :20]      # rows of a wider matrix
+    g = torch.randn(9000, 12, dtype=torch.float64)
+    assert torch.allclose(hm._weight_grad(g, x_view), g.t() @ x_view, rtol=1e-11, atol=1e-9)
+
+
 def test_bn_relu_takes_the_torch_operators_off_the_gpu():
     """Without a GPU tensor (or in evaluation mode) bn_relu is exactly relu(bn(x + bias)), module state
     included."""

@@ -171,3 +171,27 @@ def test_sage_with_fused_epilogue_equals_the_operator_spelling():
         close(out[True]["grads"][k], v.double().cpu(), k, 1e-3)
     for k, v in out[False]["stats"].items():
         close(out[True]["stats"][k], v.double().cpu(), k, 1e-5)
+
+
+@pytest.mark.parametrize("n,H,F,two", [(1, 64, 64, False), (2, 64, 64, True), (63, 128, 64, True), (1000, 192, 128, False),
+                                       (5_801, 256, 256, True), (25_817, 256, 128, True), (70_001, 256, 256, True),
+                                       (4_096, 512, 320, False)])
+def test_weight_grad_matches_fp64_product(n, H, F, two):
+    """hc_weight_grad (matrix cores, slabs added in order) against g^T x in fp64; same bits on a second call."""
+    import hiscache_backend as be
+    gen = torch.Generator(device=DEV).manual_seed(n + H)
+    g = torch.randn(n, H, device=DEV, generator=gen)
+    x0 = torch.randn(n + 5, F, device=DEV, generator=gen)[:n]              # a row prefix, as the root rows are
+    x1 = torch.randn(n, F, device=DEV, generator=gen) if two else None
+    got = be.weight_grad(g, x0, x1)
+    got = got if two else (got,)
+    for d, x in zip(got, (x0, x1)):
+        want = g.double().t() @ x.double()
+        scale = float(want.abs().max())
+        assert tuple(d.shape) == (H, F)
+        assert float((d.double() - want).abs().max()) <= 1e-5 * scale + 1e-6 * (n ** 0.5)
+    again = be.weight_grad(g, x0, x1)
+    again = again if two else (again,)
+    assert all(torch.equal(a, b) for a, b in zip(got, again))
+    with pytest.raises(ValueError):
+        be.weight_grad(g, torch.randn(n, 48, device=DEV))
