@@ -19,8 +19,11 @@ typedef float wg_acc __attribute__((ext_vector_type(16)));
 
 constexpr int WG_TILE_H = 256;      // output rows per block: 64 per wave
 constexpr int WG_TILE_F = 64;       // output columns per block
-constexpr int WG_STAGE = 8;         // k-steps (pairs of rows) loaded ahead of the matrix instructions
-constexpr int WG_TARGET_BLOCKS = 512;
+constexpr int WG_STAGE = 16;        // k-steps (pairs of rows) whose loads are in flight ahead of the matrix instructions
+// One block per compute unit: with 512 or 1024 blocks the partial tiles' traffic grows faster than the
+// matrix pipes gain (n = 25 800, F = 128, two operands: 48 us with 256 blocks, 57 with 512, 70 with 1024);
+// 16 k-steps in flight against 8: 98 against 90 TFLOP/s at n = 89 000.
+constexpr int WG_TARGET_BLOCKS = 256;
 constexpr int WG_MIN_SLAB_ROWS = 64;
 
 struct WgShape {
@@ -62,15 +65,33 @@ __global__ __launch_bounds__(HC_BLOCK) void wg_partial(const float *__restrict__
   const float *gp = g + (lo + kk) * (int64_t)H + h0 + c;
   const float *xp = x + (lo + kk) * (int64_t)F + f0 + c;
   int64_t r = lo;
-  // full stages: WG_STAGE k-steps = 2 * WG_STAGE rows, all loads issued before the first instruction
-  for (; r + 2 * WG_STAGE <= hi; r += 2 * WG_STAGE) {
-    float a0[WG_STAGE], a1[WG_STAGE], b0[WG_STAGE], b1[WG_STAGE];
+  // Full stages of WG_STAGE k-steps (2 * WG_STAGE rows).  The loads of the next stage are issued before the
+  // matrix instructions of the current one, so that a wave keeps its matrix pipe busy while they are in flight.
+  float a0[WG_STAGE], a1[WG_STAGE], b0[WG_STAGE], b1[WG_STAGE];
+  bool have = r + 2 * WG_STAGE <= hi;
+  if (have) {
 #pragma unroll
     for (int s = 0; s < WG_STAGE; ++s) {
       a0[s] = gp[(int64_t)2 * s * H];
       a1[s] = gp[(int64_t)2 * s * H + 32];
       b0[s] = xp[(int64_t)2 * s * F];
       b1[s] = xp[(int64_t)2 * s * F + 32];
+    }
+  }
+  while (have) {
+    gp += (int64_t)2 * WG_STAGE * H;
+    xp += (int64_t)2 * WG_STAGE * F;
+    r += 2 * WG_STAGE;
+    const bool more = r + 2 * WG_STAGE <= hi;
+    float na0[WG_STAGE], na1[WG_STAGE], nb0[WG_STAGE], nb1[WG_STAGE];
+    if (more) {
+#pragma unroll
+      for (int s = 0; s < WG_STAGE; ++s) {
+        na0[s] = gp[(int64_t)2 * s * H];
+        na1[s] = gp[(int64_t)2 * s * H + 32];
+        nb0[s] = xp[(int64_t)2 * s * F];
+        nb1[s] = xp[(int64_t)2 * s * F + 32];
+      }
     }
 #pragma unroll
     for (int s = 0; s < WG_STAGE; ++s) {
@@ -79,8 +100,16 @@ __global__ __launch_bounds__(HC_BLOCK) void wg_partial(const float *__restrict__
       acc10 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], b0[s], acc10, 0, 0, 0);
       acc11 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], b1[s], acc11, 0, 0, 0);
     }
-    gp += (int64_t)2 * WG_STAGE * H;
-    xp += (int64_t)2 * WG_STAGE * F;
+    if (more) {
+#pragma unroll
+      for (int s = 0; s < WG_STAGE; ++s) {
+        a0[s] = na0[s];
+        a1[s] = na1[s];
+        b0[s] = nb0[s];
+        b1[s] = nb1[s];
+      }
+    }
+    have = more;
   }
   // tail: k-steps whose second row may lie behind the slab
   for (; r < hi; r += 2) {
