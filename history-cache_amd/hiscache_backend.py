@@ -95,7 +95,7 @@ _SIGNATURES = {
     "hc_typed_csr_workspace_bytes": (_c_sz, [_c_i64, _c_int]),
     "hc_edge_types_by_ranges": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_p, _c_p, _c_i64, _c_i64, _c_p]),
     "hc_typed_csr": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_p,
-                              _c_p, _c_p, _c_sz, _c_p]),
+                              _c_p, _c_p, _c_sz, _c_p, _c_p]),
 }
 
 _lib_handle = None
@@ -736,11 +736,17 @@ def typed_csr(ptr, idx, edge_types, num_rel, num_node, n_src, used_mask=None, wa
     cnt = torch.empty(R * K, dtype=torch.int64, device=dev)
     deg = torch.empty(R, dtype=torch.int64, device=dev)
     weights = torch.empty(max(E, 1), dtype=torch.float32, device=dev) if want_weights else None
-    ws_bytes = int(lib.hc_typed_csr_workspace_bytes(R, K))
-    ws = _workspace(ws_bytes, dev)
-    rc = lib.hc_typed_csr(_ptr(ptr), _ptr(idx), _ptr(edge_types), _ptr(used_mask), R, E, int(n_src), K,
-                          _ptr(ptr2), _ptr(idx2), _ptr(cnt), _ptr(deg), _ptr(weights), _ptr(ws), ws_bytes,
-                          _stream())
+    if R * K <= TYPED_CSR_SMALL_GROUPS:
+        # sampled batches: the count kernel's last block scans the group sizes (no workspace, no library call)
+        rc = lib.hc_typed_csr(_ptr(ptr), _ptr(idx), _ptr(edge_types), _ptr(used_mask), R, E, int(n_src), K,
+                              _ptr(ptr2), _ptr(idx2), _ptr(cnt), _ptr(deg), _ptr(weights), _c_p(None), 0,
+                              _ptr(_ticket(dev)), _stream())
+    else:
+        ws_bytes = int(lib.hc_typed_csr_workspace_bytes(R, K))
+        ws = _workspace(ws_bytes, dev)
+        rc = lib.hc_typed_csr(_ptr(ptr), _ptr(idx), _ptr(edge_types), _ptr(used_mask), R, E, int(n_src), K,
+                              _ptr(ptr2), _ptr(idx2), _ptr(cnt), _ptr(deg), _ptr(weights), _ptr(ws), ws_bytes,
+                              _c_p(None), _stream())
     _check(rc, "hc_typed_csr")
     if want_weights:
         return ptr2, idx2, cnt.view(R, K), deg, weights
@@ -772,6 +778,7 @@ def edge_types_by_ranges(ptr, idx, sub_to_full, num_node, bounds, pair_to_rel):
 
 # ------------------------------------------------------------------ layer epilogue
 BN_RELU_MAX_CHANNELS = 1024
+TYPED_CSR_SMALL_GROUPS = 1 << 20
 _tickets = {}
 
 

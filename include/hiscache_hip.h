@@ -333,12 +333,15 @@ int hc_count_num(const int64_t *arr, int64_t n, int64_t mmax, int32_t *out, void
  * group's share of the row's mean over all its edges directly
  * (sum over the group / deg), without a pass that rescales group means.
  * num_rel <= 64 (HC_EUNSUPPORTED above).  Results are exact and independent of
- * scheduling. */
+ * scheduling.  ticket (nullable): one 32-bit word of device memory that is zero
+ * on entry and zero again when the call's kernels have run; with it, blocks of
+ * up to 2^20 (row, relation) groups take two launches, need no workspace and
+ * make no library call (calls that share a ticket must not overlap). */
 size_t hc_typed_csr_workspace_bytes(int64_t R, int num_rel);
 int hc_typed_csr(const int64_t *ptr, const int64_t *idx, const int64_t *edge_types,
                  const uint8_t *used_mask, int64_t R, int64_t E, int64_t n_src, int num_rel,
                  int64_t *ptr2, int64_t *idx2, int64_t *cnt, int64_t *deg, float *edge_weight,
-                 void *workspace, size_t workspace_bytes, void *stream);
+                 void *workspace, size_t workspace_bytes, unsigned *ticket, void *stream);
 
 /* hc_edge_types_by_ranges: relation of every edge of the first R rows from the
  * node types of its ends, out[e] = pair_to_rel[type(row) * T + type(idx[e])]

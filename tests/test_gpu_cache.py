@@ -717,6 +717,32 @@ def test_typed_csr_matches_oracle(orc, K, with_mask, short_types):
         be.typed_csr(t(ptr), t(idx), t(rel), 65, R, N, t(used))
 
 
+def test_typed_csr_library_scan_path_agrees(orc):
+    """Above 2^20 (row, relation) groups the group offsets come from the library's scan instead of the count
+    kernel's last block: same result as the CPU checker, and as the small path on a prefix of the rows."""
+    from helpers import random_csr
+    import hiscache_backend as be
+    rng = np.random.default_rng(77)
+    R, N, K = 17_000, 5000, 64
+    assert R * K > be.TYPED_CSR_SMALL_GROUPS
+    ptr, idx = random_csr(rng, R, N, 6)
+    rel = rng.integers(0, K, size=len(idx))
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    got = be.typed_csr(t(ptr), t(idx), t(rel), K, R, N, None, want_weights=True)
+    w_ptr2, w_idx2, w_cnt, w_deg = orc.typed_csr(ptr, idx, rel, K, R, N, None)
+    np.testing.assert_array_equal(got[0].cpu().numpy(), w_ptr2)
+    np.testing.assert_array_equal(got[1].cpu().numpy()[: w_ptr2[-1]], w_idx2)
+    np.testing.assert_array_equal(got[2].cpu().numpy(), w_cnt)
+    np.testing.assert_array_equal(got[4].cpu().numpy()[: w_ptr2[-1]], orc.typed_csr_weights(w_ptr2, w_deg, K))
+    R2 = 12_000                                                   # 768 000 groups: scanned by the count kernel
+    small = be.typed_csr(t(ptr), t(idx), t(rel), K, R2, N, None)
+    assert torch.equal(small[0], got[0][: R2 * K + 1]) and torch.equal(small[2], got[2][:R2])
+    n_small = int(small[0][-1])
+    assert torch.equal(small[1][:n_small], got[1][:n_small])
+    torch.cuda.synchronize()
+    assert int(be._ticket(torch.device(DEV)).abs().sum()) == 0
+
+
 def test_count_num_few_and_many_bins(orc):
     import hiscache_backend as be
     rng = np.random.default_rng(61)
