@@ -88,14 +88,11 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_expand_edges(const int64_t *__res
   __shared__ int64_t s_range[2];
   const int64_t e0 = (int64_t)blockIdx.x * TR_TILE;
   const int64_t e1 = e0 + TR_TILE < E ? e0 + TR_TILE : E;
-  if (threadIdx.x < HC_WAVE) {
+  if (threadIdx.x < 2 * HC_WAVE) {       // the tile's first and last row, searched by two waves side by side
     const int lane0 = hc_lane();
-    const int64_t a = tr_row_of_wave(ptr, R, e0, lane0);
-    const int64_t b = tr_row_of_wave(ptr, R, e1 - 1, lane0);
-    if (lane0 == 0) {
-      s_range[0] = a;
-      s_range[1] = b;
-    }
+    const int which = (int)(threadIdx.x >> 6);
+    const int64_t r = tr_row_of_wave(ptr, R, which == 0 ? e0 : e1 - 1, lane0);
+    if (lane0 == 0) s_range[which] = r;
   }
   __syncthreads();
   const int64_t r_lo = s_range[0], r_hi = s_range[1];
@@ -300,14 +297,11 @@ __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
   __shared__ int s_last;
   const int64_t e0 = (int64_t)blockIdx.x * TRS_BLOCK;
   const int64_t e1 = e0 + TRS_BLOCK < E ? e0 + TRS_BLOCK : E;
-  if (threadIdx.x < HC_WAVE) {
+  if (threadIdx.x < 2 * HC_WAVE) {       // the tile's first and last row, searched by two waves side by side
     const int lane0 = hc_lane();
-    const int64_t a = tr_row_of_wave(ptr, R, e0, lane0);
-    const int64_t b = tr_row_of_wave(ptr, R, e1 - 1, lane0);
-    if (lane0 == 0) {
-      s_range[0] = a;
-      s_range[1] = b;
-    }
+    const int which = (int)(threadIdx.x >> 6);
+    const int64_t r = tr_row_of_wave(ptr, R, which == 0 ? e0 : e1 - 1, lane0);
+    if (lane0 == 0) s_range[which] = r;
   }
   __syncthreads();
   const int64_t r_lo = s_range[0], r_hi = s_range[1];

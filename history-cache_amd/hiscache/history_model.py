@@ -163,8 +163,8 @@ class MySageConvHistory(torch.nn.Module):
 
     def forward(self, x, ptr, idx, history_map, history_buffer, history_size, num_node, num_edge=None,
                 add_bias=True):
-        """``add_bias=False`` (fused spelling only) leaves ``lin_l``'s bias to the caller, who hands it
-        to the normalisation that follows (see ``bn_relu``)."""
+        """``add_bias=False`` leaves ``lin_l``'s bias to the caller, who hands it to the normalisation
+        that follows (see ``bn_relu``)."""
         num_node = int(num_node)
         use_hist = history_size > 0 and history_map is not None and history_map.numel() > 0
         if self.fused and x.is_cuda and not (use_hist and history_buffer.requires_grad):
@@ -179,8 +179,6 @@ class MySageConvHistory(torch.nn.Module):
             if sink is not None:
                 sink.target = weakref.ref(his)
             return out, his
-        if not add_bias:
-            raise ValueError("add_bias=False needs the fused spelling of the layer")
         # history_size == 0 selects the plain mean inside the operator; num_edge (optional, beyond the
         # reference) bounds the edge slots of these rows inside the mini-batch's shared CSR
         out = hiscache_backend.aggr_forward_history(x, ptr, idx, history_map, history_buffer,
@@ -188,7 +186,7 @@ class MySageConvHistory(torch.nn.Module):
         his = out
         if self.need_grad and self.training and history_size > 0:
             his.retain_grad()
-        out = self.lin_l(out)
+        out = self.lin_l(out) if add_bias else F.linear(out, self.lin_l.weight)
         if self.root_weight:
             if num_node != 0:
                 out = out + self.lin_r(x[:num_node])
