@@ -195,3 +195,32 @@ def test_weight_grad_matches_fp64_product(n, H, F, two):
     assert all(torch.equal(a, b) for a, b in zip(got, again))
     with pytest.raises(ValueError):
         be.weight_grad(g, torch.randn(n, 48, device=DEV))
+
+
+def test_history_buffer_that_requires_grad_takes_the_operator_spelling():
+    """A cached-embedding buffer that asks for a gradient makes the history layer run operator by operator
+    (the fused node does not differentiate the buffer); the epilogue still takes the bias and the buffer's
+    gradient is the output gradient on the rows that were served from it."""
+    from hiscache import HistorySAGE, PinnedFeatureStore, RingHistoryCache, make_config
+    from hiscache.synthetic import make_batch, direct_power_law_batch
+    N, Fin, H, C, L = 20_000, 64, 64, 8, 3
+    rng = np.random.default_rng(5)
+    feats = torch.from_numpy(rng.standard_normal((N, Fin), dtype=np.float32))
+    smp = direct_power_law_batch(N, 100, [5, 4, 3], 2.0, 9, degree_scale=2.0)
+    torch.manual_seed(6)
+    cache = RingHistoryCache(PinnedFeatureStore(feats, device=DEV), N, Fin, H, capacity=N, num_layers=L,
+                             table_dtype=torch.float32, rate=0.5, device=DEV)
+    cache.preload(torch.arange(0, N, 2, device=DEV))
+    cache.table.normal_(0.0, 0.5)
+    model = HistorySAGE(Fin, H, C, L, 0.0, "CSR_Layer", make_config(Fin, C, H, L, device=DEV), cache).to(DEV).train()
+    b = make_batch(smp, rng.integers(0, C, size=N), DEV)
+    cache.lookup_and_load(b, L)
+    cache.cached_embedding.requires_grad_(True)
+    F.nll_loss(model(b), b.y).backward()
+    hit = cache.sub2embed != -1
+    assert hit.any() and (~hit).any()
+    gh = cache.cached_embedding.grad
+    assert gh is not None and float(gh[~hit].abs().max()) == 0.0 and float(gh[hit].abs().max()) > 0.0
+    pe = cache.produced_embedding
+    assert torch.equal(gh[hit], pe.grad[hit])
+    assert all(p.grad is not None for p in model.parameters())
