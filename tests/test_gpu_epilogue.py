@@ -175,7 +175,7 @@ def test_sage_with_fused_epilogue_equals_the_operator_spelling():
 
 @pytest.mark.parametrize("n,H,F,two", [(1, 64, 64, False), (2, 64, 64, True), (63, 128, 64, True), (1000, 192, 128, False),
                                        (5_801, 256, 256, True), (25_817, 256, 128, True), (70_001, 256, 256, True),
-                                       (4_096, 512, 320, False)])
+                                       (4_096, 512, 320, False), (301, 4096, 4096, False), (129, 64, 4096, True)])
 def test_weight_grad_matches_fp64_product(n, H, F, two):
     """hc_weight_grad (matrix cores, slabs added in order) against g^T x in fp64; same bits on a second call."""
     import hiscache_backend as be
@@ -194,7 +194,11 @@ def test_weight_grad_matches_fp64_product(n, H, F, two):
     again = again if two else (again,)
     assert all(torch.equal(a, b) for a, b in zip(got, again))
     with pytest.raises(ValueError):
-        be.weight_grad(g, torch.randn(n, 48, device=DEV))
+        be.weight_grad(g, torch.randn(n, 48, device=DEV))                 # width off a multiple of 64
+    with pytest.raises(ValueError):
+        be.weight_grad(g, torch.randn(n, 4160, device=DEV))               # wider than the kernel's limit
+    with pytest.raises(ValueError):
+        be.weight_grad(g, torch.randn(n + 1, F, device=DEV))              # row counts differ
 
 
 def test_history_buffer_that_requires_grad_takes_the_operator_spelling():
