@@ -600,6 +600,20 @@ def test_typed_csr_equals_stable_sort(orc, K, with_mask, short_types):
     # no rows: a single zero offset
     p2, i2, c, d = orc.typed_csr(ptr, idx, rel, K, 0, N, used)
     assert p2.tolist() == [0] and i2.size == 0 and c.size == 0 and d.size == 0
+    # edge weights: one loop over the groups; the weighted sums of a row's groups add up to the row's mean
+    # over all its edges restricted to the kept ones
+    ptr2, idx2, cnt, deg = got
+    wts = orc.typed_csr_weights(ptr2, deg, K)
+    assert wts.dtype == np.float32 and len(wts) == ptr2[-1]
+    for v in range(R * K):
+        r = v // K
+        assert (wts[ptr2[v]:ptr2[v + 1]] == np.float32(1.0) / np.float32(max(int(deg[r]), 1))).all()
+    x = rng.standard_normal(N + 6)
+    for r in (0, R // 2, R - 1):
+        kept = idx2[ptr2[r * K]:ptr2[(r + 1) * K]]
+        want_mean = x[kept].sum() / max(int(deg[r]), 1)
+        got_mean = sum(float(wts[e]) * x[idx2[e]] for e in range(ptr2[r * K], ptr2[(r + 1) * K]))
+        assert abs(got_mean - want_mean) <= 1e-5 * (abs(want_mean) + 1.0)
 
 
 def test_edge_types_by_ranges_brute_force(orc):
