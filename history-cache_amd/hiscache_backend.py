@@ -129,8 +129,20 @@ def _check(rc, what):
         raise RuntimeError(f"{what}: {msg}")
 
 
+def _raw_stream(device_index=None):
+    """Handle of the current HIP stream of a device (default: the current device) as an integer.
+    torch's private accessor returns it directly (0.3 us); building a torch.cuda.Stream object for it costs
+    2.7 us, and every call of this module asks at least once."""
+    if device_index is None:
+        device_index = torch.cuda.current_device()
+    get = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if get is not None:
+        return int(get(device_index))
+    return int(torch.cuda.current_stream(device_index).cuda_stream)
+
+
 def _stream():
-    return _c_p(torch.cuda.current_stream().cuda_stream)
+    return _c_p(_raw_stream())
 
 
 def _ptr(t):
@@ -174,7 +186,7 @@ def _workspace(nbytes, device):
     nbytes = max(int(nbytes), 256)
     if nbytes > _WS_KEEP_BYTES or torch.cuda.is_current_stream_capturing():
         return torch.empty(nbytes, dtype=torch.uint8, device=device)
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    key = (device.index, _raw_stream(device.index))
     buf = _ws_cache.get(key)
     if buf is None or buf.numel() < nbytes:
         size = 1 << 20
@@ -785,7 +797,7 @@ _tickets = {}
 def _ticket(device):
     """The zeroed word the epilogue kernels count their blocks in (one per device and stream; the
     kernels leave it zero)."""
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    key = (device.index, _raw_stream(device.index))
     t = _tickets.get(key)
     if t is None:
         t = _tickets[key] = torch.zeros(64, dtype=torch.int32, device=device)
