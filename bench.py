@@ -45,7 +45,7 @@ def parse():
                          "(next batch sampled on a side stream) instead of taking pre-generated batches")
     ap.add_argument("--prefetch", action="store_true",
                     help="c3/c5: start each batch's host-link feature read one batch ahead, on a side stream")
-    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c2w", "c4", "c3", "c5", "sample", "copy", "ceilings"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c2w", "c4", "c3", "c5", "sample", "layer", "copy", "ceilings"])
     ap.add_argument("--heads", type=int, default=1, help="c2w: heads of the weighted aggregation (divides 256)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -787,6 +787,71 @@ def run_c5(args):
     }
 
 
+def run_layer(args):
+    """The dense side of a sampled layer: weight gradients (hc_weight_grad against the library GEMM and its
+    slab-batched spelling) and the bias + batch norm + ReLU epilogue (hc_bn_relu against torch's operators), at
+    the row counts of the papers100M-shaped layers and of the sampler-fed loop.  Kernel time by HIP events; every
+    call is long enough for the device, not the host, to set the pace."""
+    import torch
+    import torch.nn.functional as Fn
+
+    import hiscache_backend as be
+    from hiscache import history_model as hm, prefer_low_latency_gemm
+
+    prefer_low_latency_gemm()
+    dev = "cuda:0"
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(args.steps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / args.steps * 1e3
+
+    H = 256
+    wg, bn = [], []
+    for n, F in ((5_800, 256), (25_800, 128), (25_800, 256), (55_000, 128), (55_000, 256), (89_000, 128)):
+        g = torch.randn(n, H, device=dev)
+        x0, x1 = torch.randn(n, F, device=dev), torch.randn(n, F, device=dev)
+        t_k = timed(lambda: be.weight_grad(g, x0, x1))
+        t_mm = timed(lambda: (g.t() @ x0, g.t() @ x1))
+        t_sl = timed(lambda: (hm._weight_grad(g, x0), hm._weight_grad(g, x1)))
+        flop = 2 * 2.0 * n * H * F
+        wg.append({"rows": n, "H": H, "F": F, "hc_weight_grad_us": t_k, "hc_weight_grad_TFLOPs": flop / t_k / 1e6,
+                   "library_gemm_us": t_mm, "slab_batched_gemm_us": t_sl})
+    for n in (5_800, 25_800, 55_000):
+        z = torch.randn(n, H, device=dev)
+        bias, gamma, beta = (torch.randn(H, device=dev) for _ in range(3))
+        rm, rv = torch.zeros(H, device=dev), torch.ones(H, device=dev)
+        dy = torch.randn(n, H, device=dev)
+
+        def ours():
+            zi = z.requires_grad_(True)
+            y = be.bias_bn_relu(zi, bias, gamma, beta, rm, rv, 0.1, 1e-5)
+            torch.autograd.grad(y, zi, dy)
+
+        def torch_ops():
+            zi = z.requires_grad_(True)
+            y = Fn.relu(Fn.batch_norm(zi + bias, rm, rv, gamma, beta, True, 0.1, 1e-5))
+            torch.autograd.grad(y, zi, dy)
+
+        bn.append({"rows": n, "C": H, "hc_bn_relu_fwd_bwd_us": timed(ours), "torch_fwd_bwd_us": timed(torch_ops)})
+    big = wg[-1]
+    return {"metric": "weight-gradient TFLOP/s (fp32, two operands, 89 000 rows)", "value": big["hc_weight_grad_TFLOPs"],
+            "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": big["hc_weight_grad_us"] / 1e3, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "layer: weight gradients g^T x (g [n, 256], two operands [n, F]) and bias + batch "
+                                   "norm + ReLU forward/backward of [n, 256], n = rows of sampled layers"},
+            "roofline": {"bound": "mfma", "kernel": "wg_partial + wg_reduce", "achieved": big["hc_weight_grad_TFLOPs"],
+                         "peak": 157.3, "unit": "TFLOP/s", "frac": big["hc_weight_grad_TFLOPs"] / 157.3, "traffic": None},
+            "weight_grad": wg, "bn_relu": bn}
+
+
 def run_copy(args):
     """Plain device copy of known size: the calibration point for the HBM traffic counters."""
     import torch
@@ -957,6 +1022,8 @@ def main():
         res = run_c4(args)
         if not args.no_cpu_baseline:
             res["cpu_baseline"] = cpu_baseline_c4(int(2_000_000 * args.scale), 256)
+    elif args.workload == "layer":
+        res = run_layer(args)
     elif args.workload == "copy":
         res = run_copy(args)
     elif args.workload == "c5":
