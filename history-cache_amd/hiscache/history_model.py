@@ -51,6 +51,23 @@ def _weight_grad(g, x):
     return out
 
 
+_ones_cache = {}
+
+
+def _column_sums(g):
+    """g.sum(0) as a matrix-vector product with a cached vector of ones: torch's column reduction of a tall
+    [n, H] matrix takes 25 us at n = 1 000 (one block per few columns walks all rows), the GEMV 12 us."""
+    n = g.shape[0]
+    key = (g.device, g.dtype)
+    ones = _ones_cache.get(key)
+    if ones is None or ones.numel() < n:
+        size = 1024
+        while size < n:
+            size <<= 1
+        ones = _ones_cache[key] = torch.ones(size, dtype=g.dtype, device=g.device)
+    return torch.mv(g.t(), ones[:n])
+
+
 class _SageConvFunction(torch.autograd.Function):
     """``lin_l(aggregate(x)) + lin_r(x[:n])`` as ONE autograd node.
 
@@ -92,7 +109,7 @@ class _SageConvFunction(torch.autograd.Function):
             his = sink.target()
             if his is not None:
                 his.grad = g_agg
-        g_bl = g_out.sum(0) if has_bias and need[2] else None
+        g_bl = _column_sums(g_out) if has_bias and need[2] else None
         g_wl = g_wr = None
         root = None
         if has_root and need[3]:

@@ -226,3 +226,12 @@ def test_batched_history_layer_block_layout():
         np.testing.assert_array_equal(idx[e0:e1] - col0, smp["idx"][: e1 - e0])
         row0, col0, k = row0 + n1, col0 + n2, k + 1
     assert row0 == R and col0 == N
+
+
+def test_column_sums_by_matrix_vector_product():
+    import torch
+    from hiscache import history_model as hm
+    torch.manual_seed(2)
+    for n in (1, 7, 1024, 1025, 5000):
+        g = torch.randn(n, 9, dtype=torch.float64)
+        assert torch.allclose(hm._column_sums(g), g.sum(0), rtol=1e-12, atol=1e-12)
