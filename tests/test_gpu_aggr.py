@@ -195,6 +195,8 @@ def test_build_transpose_many_more_sources_than_edges(be, orc):
     (262_144 // 4, 300, 4, None),  # exactly the largest block of the counting-sort path
     (70_000, 3000, 5, 0.2),      # above it: the library-sort path
     (5000, (1 << 20) + 5, 5, None),  # few edges but more sources than the counting sort takes
+    (300_000, 50_000, 4, 0.1),   # 1.2 M edges: the library's radix passes (9-bit digits), 16-bit keys: two passes
+    (270_000, 600_000, 4, None),  # the same with 20-bit keys: three passes
 ])
 def test_build_transpose_paths_agree_with_a_stable_argsort(be, R, N, deg, popular):
     """The counting-sort path of small blocks and the library-sort path of large ones against NumPy's
