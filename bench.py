@@ -45,9 +45,10 @@ def parse():
                          "(next batch sampled on a side stream) instead of taking pre-generated batches")
     ap.add_argument("--prefetch", action="store_true",
                     help="c3/c5: start each batch's host-link feature read one batch ahead, on a side stream")
-    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c2w", "c4", "c3", "c5", "sample", "layer", "copy", "ceilings"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c2w", "c4", "c3", "c3b", "c5", "sample", "layer", "copy", "ceilings"])
     ap.add_argument("--heads", type=int, default=1, help="c2w: heads of the weighted aggregation (divides 256)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
+    ap.add_argument("--reps", type=int, default=8, help="c3b: measurements with freshly allocated tensors")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="c2: skip the c4 and batched-c3 kernel figures that the default run adds to its line")
@@ -852,6 +853,29 @@ def run_layer(args):
             "weight_grad": wg, "bn_relu": bn}
 
 
+def run_c3b(args):
+    """The batched papers100M-shaped history layer measured several times in one process, its tensors freed
+    and allocated again between the measurements: the spread of its figure with where the allocations land."""
+    import gc
+
+    import torch
+
+    reps = []
+    for _ in range(max(1, args.reps)):
+        d = c3_batched_layer(args)["detail"]
+        reps.append({k: d[k] for k in ("fwd_ms", "transpose_ms", "bwd_ms", "grad_check_ms", "ms", "frac")})
+        gc.collect()
+        torch.cuda.empty_cache()
+    fr = sorted(r["frac"] for r in reps)
+    return {"metric": "batched history layer, fraction of 8 TB/s (median over re-allocations)", "value": fr[len(fr) // 2],
+            "unit": "fraction of HBM peak", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": sorted(r["ms"] for r in reps)[len(reps) // 2], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "c3b: papers100M-shaped history layer batched to 20 M edges, %d measurements with "
+                                   "freshly allocated tensors" % len(reps)},
+            "min_frac": fr[0], "max_frac": fr[-1], "measurements": reps}
+
+
 def run_copy(args):
     """Plain device copy of known size: the calibration point for the HBM traffic counters."""
     import torch
@@ -1024,6 +1048,8 @@ def main():
             res["cpu_baseline"] = cpu_baseline_c4(int(2_000_000 * args.scale), 256)
     elif args.workload == "layer":
         res = run_layer(args)
+    elif args.workload == "c3b":
+        res = run_c3b(args)
     elif args.workload == "copy":
         res = run_copy(args)
     elif args.workload == "c5":
