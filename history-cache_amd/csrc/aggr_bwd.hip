@@ -59,11 +59,23 @@ __device__ __forceinline__ int64_t bwd_last_source_at(const int64_t *__restrict_
   return lo;
 }
 
+// MASKED: the view covers the whole mini-batch CSR; transposed edges whose destination row lies outside
+// the first R rows, or took its history row (hmap[row] != -1), are stepped over.
+template <bool MASKED>
+__device__ __forceinline__ int bwd_live_row(int row, const int64_t *__restrict__ hmap, int64_t R) {
+  if constexpr (MASKED) {
+    if (row >= R) return -1;
+    if (hmap != nullptr && hmap[row] != -1) return -1;
+  }
+  return row;
+}
+
 // Sum of g[r,:]/deg(r) over transposed edges [begin, end), added to acc in order by the calling wave.
-template <int VEC, int CHUNKS, int UNROLL>
+template <int VEC, int CHUNKS, int UNROLL, bool MASKED>
 __device__ __forceinline__ void bwd_accumulate(const int64_t *__restrict__ ptr, const int32_t *__restrict__ rowT,
-                                               const float *__restrict__ g, int64_t begin, int64_t end,
-                                               int lane, float (&acc)[CHUNKS][VEC]) {
+                                               const float *__restrict__ g, const int64_t *__restrict__ hmap,
+                                               int64_t R, int64_t begin, int64_t end, int lane,
+                                               float (&acc)[CHUNKS][VEC]) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   for (int64_t base = begin; base < end; base += HC_WAVE) {
     const int64_t left = end - base;
@@ -71,26 +83,31 @@ __device__ __forceinline__ void bwd_accumulate(const int64_t *__restrict__ ptr, 
     int my_row = 0;
     float my_deg = 1.0f;
     if (lane < n) {
-      my_row = rowT[base + lane];
-      my_deg = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
+      my_row = bwd_live_row<MASKED>(rowT[base + lane], hmap, R);
+      if (!MASKED || my_row >= 0) my_deg = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
     }
     for (int j = 0; j < n; j += UNROLL) {
       float v[UNROLL][CHUNKS][VEC];
       float d[UNROLL];
+      bool on[UNROLL];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         d[u] = 1.0f;
+        on[u] = false;
         if (j + u < n) {
           const int r = __builtin_amdgcn_readlane(my_row, j + u);
-          d[u] = hc_readlane_f(my_deg, j + u);
-          const float *p = g + (int64_t)r * F + lane * VEC;
+          on[u] = !MASKED || r >= 0;
+          if (on[u]) {
+            d[u] = hc_readlane_f(my_deg, j + u);
+            const float *p = g + (int64_t)r * F + lane * VEC;
 #pragma unroll
-          for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
+            for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
+          }
         }
       }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
-        if (j + u < n) {
+        if (on[u]) {
 #pragma unroll
           for (int k = 0; k < CHUNKS; ++k)
 #pragma unroll
@@ -102,11 +119,13 @@ __device__ __forceinline__ void bwd_accumulate(const int64_t *__restrict__ ptr, 
 }
 
 // The chunk sums of the window owned by the calling wave (see the note above bwd_windows).
-template <int VEC, int CHUNKS, int UNROLL>
+template <int VEC, int CHUNKS, int UNROLL, bool MASKED>
 __device__ __forceinline__ void bwd_window_partials(const int64_t *__restrict__ ptr,
                                                     const int64_t *__restrict__ ptrT,
                                                     const int32_t *__restrict__ rowT,
-                                                    const float *__restrict__ g, float *__restrict__ partial,
+                                                    const float *__restrict__ g,
+                                                    const int64_t *__restrict__ hmap, int64_t R,
+                                                    float *__restrict__ partial,
                                                     int64_t n_src, int64_t window, int lane) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   const int64_t wstart = window * BWD_CHUNK;
@@ -135,7 +154,7 @@ __device__ __forceinline__ void bwd_window_partials(const int64_t *__restrict__ 
     for (int k = 0; k < CHUNKS; ++k)
 #pragma unroll
       for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
-    bwd_accumulate<VEC, CHUNKS, UNROLL>(ptr, rowT, g, begin, end, lane, acc);
+    bwd_accumulate<VEC, CHUNKS, UNROLL, MASKED>(ptr, rowT, g, hmap, R, begin, end, lane, acc);
     float *__restrict__ o = partial + (2 * window + which) * F + lane * VEC;
 #pragma unroll
     for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store(o + k * HC_WAVE * VEC, acc[k]);
@@ -185,7 +204,9 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_hub_final(const int64_t *__restr
 // WMODE W_EDGE_HEAD: a row is n_head heads side by side and the weight is edge_value[edge, head]; a
 // lane's VEC elements of a chunk lie inside one head, whose weight the lane loads itself.  (grad_hbuf
 // of such blocks is written by bwd_hist_generic.)
-template <int VEC, int CHUNKS, int UNROLL, int WMODE>
+// MASKED (plain mean only): see bwd_live_row.  Chunks of a hub are then runs of BWD_CHUNK positions of the
+// whole-batch view, of which only the live edges are added.
+template <int VEC, int CHUNKS, int UNROLL, int WMODE, bool MASKED>
 __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ ptrT, const int32_t *__restrict__ rowT,
     const int32_t *__restrict__ edgeT, const float *__restrict__ ev, int n_head, const float *__restrict__ g,
@@ -201,7 +222,8 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     // blocks behind the source and history blocks: the hubs' chunk sums, one window per wave
     if constexpr (WMODE == W_NONE) {
       const int64_t window = ((int64_t)blockIdx.x - src_blocks - hist_blocks) * HC_WAVES_PER_BLOCK + wave;
-      if (window < windows) bwd_window_partials<VEC, CHUNKS, UNROLL>(ptr, ptrT, rowT, g, partial, n_src, window, lane);
+      if (window < windows)
+        bwd_window_partials<VEC, CHUNKS, UNROLL, MASKED>(ptr, ptrT, rowT, g, hmap, R, partial, n_src, window, lane);
     }
     return;
   }
@@ -286,28 +308,33 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     int my_edge = 0;
     float my_deg = 1.0f;
     if (lane < n) {
-      my_row = rowT[base + lane];
+      my_row = bwd_live_row<MASKED>(rowT[base + lane], hmap, R);
       if constexpr (WMODE == W_EDGE_HEAD) my_edge = edgeT[base + lane];
       else if constexpr (WMODE == W_EDGE) my_deg = ev[edgeT[base + lane]];   // the weight takes the divisor's place
-      else my_deg = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
+      else if (!MASKED || my_row >= 0) my_deg = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
     }
     for (int j = 0; j < n; j += UNROLL) {
       float v[UNROLL][CHUNKS][VEC];
       float d[UNROLL];
+      bool on[UNROLL];
       float wh[WMODE == W_EDGE_HEAD ? UNROLL : 1][CHUNKS];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         d[u] = 1.0f;
+        on[u] = false;
         if (j + u < n) {
           const int r = __builtin_amdgcn_readlane(my_row, j + u);
-          d[u] = hc_readlane_f(my_deg, j + u);
-          const float *p = g + (int64_t)r * F + lane * VEC;
+          on[u] = !MASKED || r >= 0;
+          if (on[u]) {
+            d[u] = hc_readlane_f(my_deg, j + u);
+            const float *p = g + (int64_t)r * F + lane * VEC;
 #pragma unroll
-          for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
-          if constexpr (WMODE == W_EDGE_HEAD) {
-            const int64_t e = (int64_t)__builtin_amdgcn_readlane(my_edge, j + u) * n_head;
+            for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
+            if constexpr (WMODE == W_EDGE_HEAD) {
+              const int64_t e = (int64_t)__builtin_amdgcn_readlane(my_edge, j + u) * n_head;
 #pragma unroll
-            for (int k = 0; k < CHUNKS; ++k) wh[u][k] = ev[e + hd[k]];
+              for (int k = 0; k < CHUNKS; ++k) wh[u][k] = ev[e + hd[k]];
+            }
           }
         }
       }
@@ -325,13 +352,15 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
             ++cur;
             cur_end = hc_readlane64(my_p, cur + 1);
           }
+          if (on[u]) {
 #pragma unroll
-          for (int k = 0; k < CHUNKS; ++k)
+            for (int k = 0; k < CHUNKS; ++k)
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-              if constexpr (WMODE == W_EDGE_HEAD) acc[k][i] += __fmul_rn(v[u][k][i], wh[u][k]);
-              else acc[k][i] += WEIGHTED ? __fmul_rn(v[u][k][i], d[u]) : v[u][k][i] / d[u];
-            }
+              for (int i = 0; i < VEC; ++i) {
+                if constexpr (WMODE == W_EDGE_HEAD) acc[k][i] += __fmul_rn(v[u][k][i], wh[u][k]);
+                else acc[k][i] += WEIGHTED ? __fmul_rn(v[u][k][i], d[u]) : v[u][k][i] / d[u];
+              }
+          }
         }
       }
     }
@@ -347,7 +376,10 @@ template <bool WEIGHTED>
 __global__ __launch_bounds__(HC_BLOCK) void bwd_generic(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ ptrT, const int32_t *__restrict__ rowT,
     const int32_t *__restrict__ edgeT, const float *__restrict__ g, const float *__restrict__ ev,
-    int64_t H, float *__restrict__ grad_vin, int64_t n_src, int64_t F) {
+    int64_t H, float *__restrict__ grad_vin, int64_t n_src, int64_t F, const int64_t *__restrict__ mask_hmap,
+    int64_t mask_rows) {
+  // mask_rows >= 0: the view covers the whole mini-batch CSR; edges of rows >= mask_rows and of rows with
+  // mask_hmap[row] != -1 are stepped over
   constexpr int TILE_K = 4;
   const int lane = hc_lane();
   const int64_t vsrc = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
@@ -368,19 +400,25 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_generic(
       float my_s = 1.0f;
       if (lane < n) {
         my_row = rowT[base + lane];
-        if (WEIGHTED) my_s = ev[(int64_t)edgeT[base + lane] * H + head];
+        if (mask_rows >= 0 && (my_row >= mask_rows || (mask_hmap != nullptr && mask_hmap[my_row] != -1)))
+          my_row = -1;
+        if (my_row < 0) my_s = 1.0f;
+        else if (WEIGHTED) my_s = ev[(int64_t)edgeT[base + lane] * H + head];
         else my_s = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
       }
       constexpr int GEN_UNROLL = 4;  // gradient rows in flight before the first add (order kept)
       for (int j = 0; j < n; j += GEN_UNROLL) {
         float x[GEN_UNROLL][TILE_K];
         float sc[GEN_UNROLL];
+        bool on[GEN_UNROLL];
 #pragma unroll
         for (int u = 0; u < GEN_UNROLL; ++u) {
           sc[u] = 1.0f;
+          on[u] = false;
 #pragma unroll
           for (int k = 0; k < TILE_K; ++k) x[u][k] = 0.0f;
-          if (j + u < n) {
+          if (j + u < n && __builtin_amdgcn_readlane(my_row, j + u) >= 0) {
+            on[u] = true;
             const int r = __builtin_amdgcn_readlane(my_row, j + u);
             sc[u] = hc_readlane_f(my_s, j + u);
             const float *p = g + ((int64_t)r * H + head) * F;
@@ -393,7 +431,7 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_generic(
         }
 #pragma unroll
         for (int u = 0; u < GEN_UNROLL; ++u) {
-          if (j + u < n) {
+          if (on[u]) {
 #pragma unroll
             for (int k = 0; k < TILE_K; ++k) {
               const int64_t c = c0 + k * HC_WAVE + lane;
@@ -668,7 +706,7 @@ template <int VEC, int CHUNKS>
 int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, const int32_t *edgeT,
                 const float *ev, int n_head, const float *g, const int64_t *hmap, float *grad_vin,
                 float *grad_hbuf, int64_t hsize, int64_t R, int64_t n_src, int64_t E_slots, void *workspace,
-                size_t workspace_bytes, hipStream_t st) {
+                size_t workspace_bytes, bool masked, hipStream_t st) {
   constexpr int per = VEC * CHUNKS;
   constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
   constexpr int F = HC_WAVE * VEC * CHUNKS;
@@ -689,16 +727,21 @@ int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, co
   if (hubs) hub_thres = BWD_CHUNK;
   if (!hc_grid_ok(sb + hb + wb)) return HC_EUNSUPPORTED;
   const dim3 grid((unsigned)(sb + hb + wb)), block(HC_BLOCK);
-  if (ev != nullptr && n_head > 1)
-    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_EDGE_HEAD><<<grid, block, 0, st>>>(
+  if (masked && ev != nullptr) return HC_EUNSUPPORTED;
+  if (masked)
+    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_NONE, true><<<grid, block, 0, st>>>(
+        ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hb, hub_thres, partial,
+        windows);
+  else if (ev != nullptr && n_head > 1)
+    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_EDGE_HEAD, false><<<grid, block, 0, st>>>(
         ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hb, hub_thres, partial,
         windows);
   else if (ev != nullptr)
-    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_EDGE><<<grid, block, 0, st>>>(
+    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_EDGE, false><<<grid, block, 0, st>>>(
         ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hb, hub_thres, partial,
         windows);
   else
-    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_NONE><<<grid, block, 0, st>>>(
+    bwd_mean_fast<VEC, CHUNKS, UNROLL, W_NONE, false><<<grid, block, 0, st>>>(
         ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hb, hub_thres, partial,
         windows);
   if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
@@ -722,12 +765,14 @@ extern "C" size_t hc_aggr_bwd_workspace_bytes(int64_t E_total, int64_t F) {
 
 extern "C" int64_t hc_aggr_bwd_chunk_edges(int64_t F) { return bwd_fast_shape(F) ? BWD_CHUNK : 0; }
 
-extern "C" int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t *ptrT,
-                           const int32_t *rowT, const int32_t *edgeT, const float *g,
-                           const int64_t *hmap, const float *edge_value, const void *vin, int in_dtype,
-                           int64_t n_head, float *grad_vin, float *grad_hbuf, int64_t hsize,
-                           float *edge_grad, int64_t E_total, int64_t R, int64_t F, int64_t n_src,
-                           void *workspace, size_t workspace_bytes, void *stream) {
+namespace {
+
+int aggr_bwd_impl(const int64_t *ptr, const int64_t *idx, const int64_t *ptrT,
+                  const int32_t *rowT, const int32_t *edgeT, const float *g,
+                  const int64_t *hmap, const float *edge_value, const void *vin, int in_dtype,
+                  int64_t n_head, float *grad_vin, float *grad_hbuf, int64_t hsize,
+                  float *edge_grad, int64_t E_total, int64_t R, int64_t F, int64_t n_src,
+                  void *workspace, size_t workspace_bytes, bool masked, void *stream) {
   HC_REQUIRE(R >= 0 && F > 0 && n_src >= 0 && n_head >= 1 && E_total >= 0);
   HC_REQUIRE(ptr && ptrT && g);
   HC_REQUIRE(grad_vin || n_src == 0);
@@ -758,7 +803,7 @@ extern "C" int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t
 #define HC_FAST(V, C)                                                                             \
   if (Frow == 64 * (V) * (C) && F % (V) == 0)                                                     \
     rc = launch_fast<V, C>(ptr, ptrT, rowT, edgeT, edge_value, nh, g, hmap, grad_vin, grad_hbuf, hsize, R, \
-                           n_src, E_total, workspace, workspace_bytes, st);                         \
+                           n_src, E_total, workspace, workspace_bytes, masked, st);                 \
   else
     HC_FAST(4, 1) HC_FAST(4, 2) HC_FAST(4, 3) HC_FAST(4, 4) HC_FAST(2, 1) HC_FAST(2, 3) HC_FAST(1, 1)
     HC_FAST(1, 3) done = false;
@@ -779,11 +824,11 @@ extern "C" int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t
       if (edge_value)
         bwd_generic<true><<<dim3((unsigned)sb), dim3(HC_BLOCK), 0, st>>>(ptr, ptrT, rowT, edgeT, g,
                                                                          edge_value, n_head, grad_vin,
-                                                                         n_src, F);
+                                                                         n_src, F, nullptr, -1);
       else
         bwd_generic<false><<<dim3((unsigned)sb), dim3(HC_BLOCK), 0, st>>>(ptr, ptrT, rowT, edgeT, g,
                                                                           edge_value, n_head, grad_vin,
-                                                                          n_src, F);
+                                                                          n_src, F, hmap, masked ? R : -1);
       if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
     }
     if (grad_hbuf && R > 0) {
@@ -863,4 +908,25 @@ extern "C" int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t
     if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
   }
   return HC_OK;
+}
+
+}  // namespace
+
+extern "C" int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t *ptrT,
+                           const int32_t *rowT, const int32_t *edgeT, const float *g,
+                           const int64_t *hmap, const float *edge_value, const void *vin, int in_dtype,
+                           int64_t n_head, float *grad_vin, float *grad_hbuf, int64_t hsize,
+                           float *edge_grad, int64_t E_total, int64_t R, int64_t F, int64_t n_src,
+                           void *workspace, size_t workspace_bytes, void *stream) {
+  return aggr_bwd_impl(ptr, idx, ptrT, rowT, edgeT, g, hmap, edge_value, vin, in_dtype, n_head, grad_vin,
+                       grad_hbuf, hsize, edge_grad, E_total, R, F, n_src, workspace, workspace_bytes, false,
+                       stream);
+}
+
+extern "C" int hc_aggr_bwd_batch_view(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT,
+                                      const float *g, const int64_t *hmap, float *grad_vin,
+                                      float *grad_hbuf, int64_t hsize, int64_t E_view, int64_t R, int64_t F,
+                                      int64_t n_src, void *workspace, size_t workspace_bytes, void *stream) {
+  return aggr_bwd_impl(ptr, nullptr, ptrT, rowT, nullptr, g, hmap, nullptr, nullptr, 0, 1, grad_vin, grad_hbuf,
+                       hsize, nullptr, E_view, R, F, n_src, workspace, workspace_bytes, true, stream);
 }

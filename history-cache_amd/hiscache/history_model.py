@@ -80,7 +80,7 @@ class _SageConvFunction(torch.autograd.Function):
     its ``.grad`` during backward when a sink is given."""
 
     @staticmethod
-    def forward(ctx, x, w_l, b_l, w_r, ptr, idx, hmap, hbuf, hsize, num_node, num_edge, sink):
+    def forward(ctx, x, w_l, b_l, w_r, ptr, idx, hmap, hbuf, hsize, num_node, num_edge, sink, view=None):
         be = hiscache_backend
         R = int(num_node) if num_node else ptr.numel() - 1
         agg = be._aggr_fwd(be.SUBST_ROW, ptr, idx, x, hmap, hbuf, hsize, None, R)
@@ -94,6 +94,7 @@ class _SageConvFunction(torch.autograd.Function):
             out += b_l
         ctx.save_for_backward(x, agg, w_l, w_r if w_r is not None else w_l.new_empty(0))
         ctx.hc = (ptr, idx, hmap, hsize, R, num_edge, b_l is not None, w_r is not None, sink)
+        ctx.view = view if view is not None and view.covers(R, x.shape[0]) else None
         ctx.mark_non_differentiable(agg)
         return out, agg
 
@@ -124,14 +125,18 @@ class _SageConvFunction(torch.autograd.Function):
         g_x = None
         if need[0]:
             n_src = x.shape[0]
-            tr = be.build_transpose(ptr, idx, hmap, R, n_src, num_edge=num_edge, want_edges=False)
-            g_x, _, _ = be._aggr_bwd(ptr, idx, tr, g_agg, hmap, None, x, False, None, hsize, R, n_src,
-                                     want_hist_grad=False)
+            if ctx.view is not None:          # the batch came with its transposed view: none is built here
+                g_x, _ = be._aggr_bwd_batch_view(ptr, ctx.view, g_agg, hmap, None, hsize, R, n_src,
+                                                 want_hist_grad=False)
+            else:
+                tr = be.build_transpose(ptr, idx, hmap, R, n_src, num_edge=num_edge, want_edges=False)
+                g_x, _, _ = be._aggr_bwd(ptr, idx, tr, g_agg, hmap, None, x, False, None, hsize, R, n_src,
+                                         want_hist_grad=False)
             if has_root:
                 g_x[:R].addmm_(g_out, w_r)
             if g_x.dtype != x.dtype:
                 g_x = g_x.to(x.dtype)
-        return g_x, g_wl, g_bl, g_wr, None, None, None, None, None, None, None, None
+        return g_x, g_wl, g_bl, g_wr, None, None, None, None, None, None, None, None, None
 
 
 def bn_relu(x, bn, bias=None, fused=True):
@@ -179,9 +184,10 @@ class MySageConvHistory(torch.nn.Module):
     fused = True
 
     def forward(self, x, ptr, idx, history_map, history_buffer, history_size, num_node, num_edge=None,
-                add_bias=True):
+                add_bias=True, view=None):
         """``add_bias=False`` leaves ``lin_l``'s bias to the caller, who hands it to the normalisation
-        that follows (see ``bn_relu``)."""
+        that follows (see ``bn_relu``).  ``view``: the batch's shared transposed view
+        (``hiscache_backend.BatchView``), when the loader emitted one."""
         num_node = int(num_node)
         use_hist = history_size > 0 and history_map is not None and history_map.numel() > 0
         if self.fused and x.is_cuda and not (use_hist and history_buffer.requires_grad):
@@ -192,14 +198,14 @@ class MySageConvHistory(torch.nn.Module):
                 x, self.lin_l.weight, self.lin_l.bias if add_bias else None,
                 self.lin_r.weight if self.root_weight else None, ptr, idx,
                 history_map if use_hist else None, history_buffer if use_hist else None,
-                int(history_size) if use_hist else 0, num_node, num_edge, sink)
+                int(history_size) if use_hist else 0, num_node, num_edge, sink, view)
             if sink is not None:
                 sink.target = weakref.ref(his)
             return out, his
         # history_size == 0 selects the plain mean inside the operator; num_edge (optional, beyond the
         # reference) bounds the edge slots of these rows inside the mini-batch's shared CSR
         out = hiscache_backend.aggr_forward_history(x, ptr, idx, history_map, history_buffer,
-                                                    history_size, num_node, num_edge)
+                                                    history_size, num_node, num_edge, view)
         his = out
         if self.need_grad and self.training and history_size > 0:
             his.retain_grad()
@@ -237,6 +243,7 @@ class HistorySAGE(torch.nn.Module):
         x = batch.x
         none = torch.empty(0, device=x.device)
         nel = getattr(batch, "num_edge_in_layer", None)      # edges of the first num_node_in_layer[k] rows
+        view = getattr(batch, "view", None)                  # shared transposed view, if the loader emitted it
         for i, conv in enumerate(self.convs[:-1]):
             k = self.num_layers - 1 - i
             n = batch.num_node_in_layer[k]
@@ -246,14 +253,15 @@ class HistorySAGE(torch.nn.Module):
             if self.training and i == self.num_layers - 2:
                 # the layer whose output is one hop from the seeds uses (and produces) history
                 x, his = conv(x, batch.ptr, batch.idx, self.table.sub2embed,
-                              self.table.cached_embedding, self.hidden_channels, n, ne, add_bias=not defer)
+                              self.table.cached_embedding, self.hidden_channels, n, ne, add_bias=not defer,
+                              view=view)
                 self.table.produced_embedding = his
             else:
-                x, his = conv(x, batch.ptr, batch.idx, none, none, 0, n, ne, add_bias=not defer)
+                x, his = conv(x, batch.ptr, batch.idx, none, none, 0, n, ne, add_bias=not defer, view=view)
             x = bn_relu(x, self.bns[i], conv.lin_l.bias if defer else None, fused=self.fused_epilogue)
             x = F.dropout(x, p=self.dropout, training=self.training)
         x, his = self.convs[-1](x, batch.ptr, batch.idx, none, none, 0, batch.num_node_in_layer[0],
-                                None if nel is None else int(nel[0]))
+                                None if nel is None else int(nel[0]), view=view)
         return x.log_softmax(dim=-1)
 
     def init_convs(self, **kwargs):

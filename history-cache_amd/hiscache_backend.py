@@ -59,6 +59,8 @@ _SIGNATURES = {
     "hc_aggr_bwd_chunk_edges": (_c_i64, [_c_i64]),
     "hc_aggr_bwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_p,
                              _c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]),
+    "hc_aggr_bwd_batch_view": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_i64,
+                                        _c_i64, _c_p, _c_sz, _c_p]),
     "hc_count_history": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p]),
     "hc_row_scores": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_int, _c_p]),
     "hc_grad_check_workspace_bytes": (_c_sz, [_c_i64]),
@@ -338,19 +340,82 @@ def _aggr_bwd(ptr, idx, tr, g, hmap, edge_value, x, want_edge_grad, hbuf_shape, 
     return grad_x, grad_h, edge_grad
 
 
+class BatchView:
+    """One transposed view of a whole mini-batch CSR, shared by the layers of the batch: ``ptrT`` over
+    all ``n_src`` nodes of the batch, ``rowT`` (and ``edgeT`` when built) over the edges of its first
+    ``rows`` rows.  A layer that owns the first R <= rows rows and the first n <= n_src sources uses a
+    prefix of ``ptrT``; edges of other rows are stepped over in backward.  ``num_edge`` bounds the
+    entries of ``rowT`` that hold edges."""
+    __slots__ = ("ptrT", "rowT", "edgeT", "rows", "n_src", "num_edge")
+
+    def __init__(self, ptrT, rowT, edgeT, rows, n_src, num_edge):
+        self.ptrT, self.rowT, self.edgeT = ptrT, rowT, edgeT
+        self.rows, self.n_src, self.num_edge = int(rows), int(n_src), int(num_edge)
+
+    def covers(self, num_node, n_src):
+        return int(num_node) <= self.rows and int(n_src) <= self.n_src
+
+    def record_stream(self, stream):
+        for t in (self.ptrT, self.rowT, self.edgeT):
+            if t is not None:
+                t.record_stream(stream)
+
+
+def build_batch_view(ptr, idx, num_node, n_src, num_edge=None, want_edges=False):
+    """The shared view of a mini-batch: the stable transposed view of the first ``num_node`` rows of
+    (ptr, idx) -- all rows of the batch's CSR -- over ``n_src`` nodes, with nothing left out.  A loader
+    builds it once per batch, ahead of the training step (the device sampler does, with
+    ``emit_view=True``)."""
+    R = int(num_node) if num_node else ptr.numel() - 1
+    E = idx.numel() if num_edge is None else min(int(num_edge), idx.numel())
+    ptrT, rowT, edgeT = build_transpose(ptr, idx, None, R, int(n_src), num_edge=E, want_edges=want_edges)
+    return BatchView(ptrT, rowT, edgeT, R, n_src, E)
+
+
+def _aggr_bwd_batch_view(ptr, view, g, hmap, hbuf_shape, hsize, num_node, n_src, want_hist_grad=True):
+    """Gradient of the mean aggregation over the batch's shared view: (grad_input, grad_history or None)."""
+    lib = load_library()
+    g = _dev(g.contiguous(), "grad_output", torch.float32)
+    if g.dim() != 2:
+        raise ValueError("the shared view serves the plain mean: grad_output must be [num_node, F]")
+    R, F = int(num_node), g.shape[1]
+    if not view.covers(R, n_src):
+        raise ValueError(f"the batch view covers {view.rows} rows / {view.n_src} sources, "
+                         f"the layer has {R} / {n_src}")
+    if g.shape[0] < R or (hmap is not None and hmap.numel() < R):
+        raise ValueError("grad_output or history_map is shorter than num_node")
+    dev = g.device
+    grad_x = torch.empty((n_src, F), dtype=torch.float32, device=dev)
+    grad_h = None
+    if hmap is not None and want_hist_grad:
+        grad_h = torch.empty(hbuf_shape, dtype=torch.float32, device=dev)
+        if grad_h.numel() != R * hsize:
+            grad_h.zero_()
+    nbytes = lib.hc_aggr_bwd_workspace_bytes(view.num_edge, F)
+    ws = _workspace(nbytes, dev) if nbytes else None
+    rc = lib.hc_aggr_bwd_batch_view(_ptr(ptr), _ptr(view.ptrT), _ptr(view.rowT), _ptr(g), _ptr(hmap),
+                                    _ptr(grad_x), _ptr(grad_h), int(hsize), view.num_edge, R, F, int(n_src),
+                                    _ptr(ws), ws.numel() if ws is not None else 0, _stream())
+    _check(rc, "hc_aggr_bwd_batch_view")
+    return grad_x, grad_h
+
+
 class _AggrHistory(torch.autograd.Function):
     """Counterpart of AggrHistoryFunction / AggrHistoryEdgeValueFunction
     (/root/reference/src/cpp/src/history_aggr.cu:475-596).  Tensor references are kept on the
     context (the reference keeps raw addresses, :406-408)."""
 
     @staticmethod
-    def forward(ctx, x, ptr, idx, edge_value, hmap, hbuf, hsize, num_node, mode, num_edge=None):
+    def forward(ctx, x, ptr, idx, edge_value, hmap, hbuf, hsize, num_node, mode, num_edge=None, view=None):
         R = int(num_node) if num_node else ptr.numel() - 1
         out = _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, R)
         ctx.hc = (ptr, idx, hmap, hsize, R, mode, None if hbuf is None else tuple(hbuf.shape))
         # edge slots the first R rows can reach, when the caller knows it (a layer of a shared CSR owns a
         # prefix of idx): the transposed view then sorts that prefix only
         ctx.num_edge = num_edge
+        # the batch's shared transposed view (plain mean with per-row substitution only)
+        ctx.view = view if (edge_value is None and mode == SUBST_ROW and view is not None
+                            and view.covers(R, x.shape[0]) and x.dim() == 2) else None
         ctx.hdtype = None if hbuf is None else hbuf.dtype
         ctx.save_for_backward(x, edge_value if edge_value is not None else x.new_empty(0))
         ctx.has_ev = edge_value is not None
@@ -378,7 +443,15 @@ class _AggrHistory(torch.autograd.Function):
                 flat = g2.reshape(R, -1)
                 hit = (row_map[:R] != -1).unsqueeze(1)
                 grad_h.view(-1, hsize)[:R, :flat.shape[1]] = torch.where(hit, flat, torch.zeros_like(flat))
-            return None, None, None, None, None, grad_h, None, None, None, None
+            return None, None, None, None, None, grad_h, None, None, None, None, None
+        if ctx.view is not None:
+            grad_x, grad_h = _aggr_bwd_batch_view(ptr, ctx.view, g, row_map, hshape, hsize, R, n_src,
+                                                  want_hist_grad=want_h)
+            if grad_x.dtype != x.dtype:
+                grad_x = grad_x.to(x.dtype)
+            if grad_h is not None and grad_h.dtype != ctx.hdtype:
+                grad_h = grad_h.to(ctx.hdtype)
+            return grad_x, None, None, None, None, grad_h, None, None, None, None, None
         # The transposed view is built here, on the stream backward runs on.  Building it during the
         # forward pass on a side stream was measured and dropped: concurrent with the bandwidth-bound
         # forward it finishes no earlier (9.15 against 9.09 ms for forward + backward on a 20 M-edge
@@ -405,7 +478,7 @@ class _AggrHistory(torch.autograd.Function):
             grad_x = grad_x.to(x.dtype)
         if grad_h is not None and grad_h.dtype != ctx.hdtype:
             grad_h = grad_h.to(ctx.hdtype)
-        return (grad_x if want_x else None), None, None, edge_grad, None, grad_h, None, None, None, None
+        return (grad_x if want_x else None), None, None, edge_grad, None, grad_h, None, None, None, None, None
 
 
 def _norm_history(history_map, history_buffer, history_size):
@@ -415,15 +488,17 @@ def _norm_history(history_map, history_buffer, history_size):
 
 
 # ----------------------------------------------------------------------------- reference API
-def aggr_forward_history(input, ptr, idx, history_map, history_buffer, history_size, num_node, num_edge=None):
+def aggr_forward_history(input, ptr, idx, history_map, history_buffer, history_size, num_node, num_edge=None,
+                         view=None):
     """Mean aggregation with history substitution; same positional signature as the reference
     (/root/reference/src/cpp/include/history_aggr.h:34-37).  ``history_size == 0`` or an
     empty ``history_map`` gives the plain mean (the reference exits there, history_aggr.cu:440-441).
     The result always requires grad (history_aggr.cu:604).  ``num_edge`` (optional, beyond the
     reference) is an upper bound of ptr[num_node] for callers that know it -- a layer of a shared
-    mini-batch CSR owns a prefix of ``idx`` -- so that backward looks at that prefix only."""
+    mini-batch CSR owns a prefix of ``idx`` -- so that backward looks at that prefix only.  ``view``
+    (optional, a ``BatchView``) is the batch's shared transposed view: backward then builds none."""
     hmap, hbuf, hsize = _norm_history(history_map, history_buffer, history_size)
-    out = _AggrHistory.apply(input, ptr, idx, None, hmap, hbuf, hsize, num_node, SUBST_ROW, num_edge)
+    out = _AggrHistory.apply(input, ptr, idx, None, hmap, hbuf, hsize, num_node, SUBST_ROW, num_edge, view)
     if not out.requires_grad:
         out.requires_grad_(True)
     return out

@@ -162,6 +162,34 @@ int hc_aggr_bwd(const int64_t *ptr, const int64_t *idx, const int64_t *ptrT, con
                 int64_t hsize, float *edge_grad, int64_t E_total, int64_t R, int64_t F,
                 int64_t n_src, void *workspace, size_t workspace_bytes, void *stream);
 
+/* hc_aggr_bwd_batch_view: the mean aggregation's backward over ONE transposed
+ * view of the whole mini-batch CSR, shared by every layer of the batch and
+ * built before the cache has been consulted (hc_build_transpose over all rows
+ * of the batch with hmap_row = hmap_src = NULL, or hc_build_transpose_dev
+ * behind the sampler), so that no view is built inside backward.  The
+ * reference's layers share one CSR per batch the same way
+ * (hiscache/history_model.py:124-128) and scatter with atomics
+ * (history_aggr.cu:127-168).
+ *
+ * A layer owns the first R rows of the batch CSR and the first n_src sources;
+ * ptrT[0..n_src] is a prefix of the batch view's offsets.  Transposed edges
+ * whose destination row is >= R, or has hmap[row] != -1 (hmap nullable), are
+ * stepped over here instead of being left out of the view.  grad_vin[n_src, F]
+ * and grad_hbuf (nullable) as in hc_aggr_bwd.  E_view bounds ptrT[n_src] (the
+ * entries of rowT that may be read; it sizes the workspace:
+ * hc_aggr_bwd_workspace_bytes(E_view, F)).
+ * Summation order: ascending destination row over the live edges.  With a
+ * workspace and C = hc_aggr_bwd_chunk_edges(F) > 0, a source with more than C
+ * edges IN THE BATCH VIEW is summed in chunks of C consecutive view positions
+ * (live edges only, each chunk from zero), combined left to right.  For a
+ * source with at most C edges in the batch view the result has the same bits
+ * as hc_aggr_bwd over a view built for the layer.
+ * Plain mean, one head, fp32 gradient; any F. */
+int hc_aggr_bwd_batch_view(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT,
+                           const float *g, const int64_t *hmap, float *grad_vin, float *grad_hbuf,
+                           int64_t hsize, int64_t E_view, int64_t R, int64_t F, int64_t n_src,
+                           void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------- used masks
  * Replaces count_history_reconstruct (src/cpp/include/grad_check.h:18-20,
  * src/cpp/src/grad_check.cu:70-130).  masks is (num_layer+1) x n_all bytes

@@ -287,57 +287,82 @@ int orc_fwd_mean_src(const Index *ptr, const Index *idx, const float *feat,
  *   history row -> grads_history[row,:F] += g[row,:]        (:144-149, no division)
  *   else        -> grads_out[idx[j],:] += g[row,:] / deg    (:140-142, :161-166)
  * grads_out[n_src,F] and grads_history[R,hsize] are zero-filled first (:503-504). */
-int orc_bwd_mean_row(const Index *ptr, const Index *idx, const float *g,
-                     const Index *hmap, float *grads_out, float *grads_history,
-                     Index R, Index F, Index hsize, Index n_src, Index chunk) {
+static int bwd_mean_row_impl(const Index *ptr, const Index *idx, const float *g,
+                             const Index *hmap, float *grads_out, float *grads_history,
+                             Index R, Index F, Index hsize, Index n_src, Index chunk, Index view_rows) {
   /* chunk == 0: every source row is summed strictly in (row, edge) order.  chunk > 0 restates the
    * device library's documented order for hubs: a source with more than `chunk` incoming edges is
    * summed in chunks of `chunk` consecutive incoming edges, each chunk from zero in order, and the
-   * chunk sums are combined left to right. */
+   * chunk sums are combined left to right.
+   * view_rows < 0: "incoming edges" are the live ones (rows below R that did not take their history
+   * row): the order over a transposed view built for this layer.  view_rows >= R: the order over one
+   * view of the first view_rows rows of the whole mini-batch CSR (hc_aggr_bwd_batch_view): positions
+   * are counted over every edge of those rows, a hub is a source with more than `chunk` of them, and
+   * only the live edges of a chunk are added. */
   memset(grads_out, 0, (size_t)(n_src * F) * sizeof(float));
   if (grads_history) memset(grads_history, 0, (size_t)(R * hsize) * sizeof(float));
   Index *indeg = NULL, *seen = NULL, *hub_of = NULL;
   float *part = NULL;
   Index n_hubs = 0;
+  const Index walk_rows = view_rows < 0 ? R : view_rows;
   if (chunk > 0) {
     indeg = (Index *)calloc((size_t)(n_src > 0 ? n_src : 1), sizeof(Index));
     seen = (Index *)calloc((size_t)(n_src > 0 ? n_src : 1), sizeof(Index));
     hub_of = (Index *)malloc((size_t)(n_src > 0 ? n_src : 1) * sizeof(Index));
     if (!indeg || !seen || !hub_of) return ORC_EINVAL;
-    for (Index row = 0; row < R; ++row) {
-      if (hmap && hmap[row] != -1) continue;
-      for (Index j = ptr[row]; j < ptr[row + 1]; ++j) indeg[idx[j]]++;
+    for (Index row = 0; row < walk_rows; ++row) {
+      if (view_rows < 0 && hmap && hmap[row] != -1) continue;
+      for (Index j = ptr[row]; j < ptr[row + 1]; ++j)
+        if (idx[j] >= 0 && idx[j] < n_src) indeg[idx[j]]++;
     }
     for (Index s = 0; s < n_src; ++s) hub_of[s] = indeg[s] > chunk ? n_hubs++ : -1;
     part = (float *)calloc((size_t)((n_hubs > 0 ? n_hubs : 1) * F), sizeof(float));
     if (!part) return ORC_EINVAL;
   }
-  for (Index row = 0; row < R; ++row) {
-    const float *gr = g + row * F;
-    if (hmap && hmap[row] != -1) {
+  for (Index row = 0; row < walk_rows; ++row) {
+    const int live = row < R && !(hmap && hmap[row] != -1);
+    const float *gr = row < R ? g + row * F : g;
+    if (row < R && !live && grads_history) {
       for (Index c = 0; c < F; ++c) grads_history[row * hsize + c] += gr[c];
-      continue;
     }
+    if (!live && (view_rows < 0 || chunk == 0)) continue;
     Index b = ptr[row], e = ptr[row + 1];
     int n = (int)(e - b);
     if (n == 0) continue;
     for (Index j = b; j < e; ++j) {
       Index s = idx[j];
+      if (s < 0 || s >= n_src) continue;   /* a source of deeper layers: only rows >= R reach it */
       float *o = grads_out + s * F;
       if (chunk > 0 && hub_of[s] >= 0) {
         float *p = part + hub_of[s] * F;
-        for (Index c = 0; c < F; ++c) p[c] += gr[c] / (float)n;
+        if (live)
+          for (Index c = 0; c < F; ++c) p[c] += gr[c] / (float)n;
         seen[s]++;
         if (seen[s] % chunk == 0 || seen[s] == indeg[s]) { /* chunk complete: fold it in */
           for (Index c = 0; c < F; ++c) { o[c] += p[c]; p[c] = 0.0f; }
         }
-      } else {
+      } else if (live) {
         for (Index c = 0; c < F; ++c) o[c] += gr[c] / (float)n;
       }
     }
   }
   free(indeg); free(seen); free(hub_of); free(part);
   return ORC_OK;
+}
+
+int orc_bwd_mean_row(const Index *ptr, const Index *idx, const float *g,
+                     const Index *hmap, float *grads_out, float *grads_history,
+                     Index R, Index F, Index hsize, Index n_src, Index chunk) {
+  return bwd_mean_row_impl(ptr, idx, g, hmap, grads_out, grads_history, R, F, hsize, n_src, chunk, -1);
+}
+
+/* The same gradient in the summation order of hc_aggr_bwd_batch_view: `ptr` / `idx` hold at least
+ * view_rows >= R rows (the whole mini-batch CSR), g and hmap the layer's first R rows. */
+int orc_bwd_mean_row_batch_view(const Index *ptr, const Index *idx, const float *g,
+                                const Index *hmap, float *grads_out, float *grads_history,
+                                Index R, Index F, Index hsize, Index n_src, Index chunk, Index view_rows) {
+  if (view_rows < R) return ORC_EINVAL;
+  return bwd_mean_row_impl(ptr, idx, g, hmap, grads_out, grads_history, R, F, hsize, n_src, chunk, view_rows);
 }
 
 /* Source-substitution backward (build extension): the gradient of the mean

@@ -146,6 +146,25 @@ def bwd_mean_row(ptr, idx, g, hmap, n_src, hbuf_shape=None, chunk=0):
     return gout, ghist
 
 
+def bwd_mean_row_batch_view(ptr, idx, g, hmap, n_src, view_rows, hbuf_shape=None, chunk=0):
+    """bwd_mean_row in the summation order of hc_aggr_bwd_batch_view: (ptr, idx) is the whole
+    mini-batch CSR (at least ``view_rows`` rows, over which the shared view was built), g [R, F] and
+    hmap belong to the layer's first R rows."""
+    ptr, idx, g = _i64(ptr), _i64(idx), _f32(g)
+    R, F = g.shape
+    gout = np.zeros((n_src, F), np.float32)
+    ghist = None
+    hsize = 0
+    if hmap is not None:
+        hmap = _i64(hmap)
+        hsize = hbuf_shape[-1] if hbuf_shape is not None else F
+        ghist = np.zeros((R, hsize), np.float32)
+    _check(lib().orc_bwd_mean_row_batch_view(_p(ptr), _p(idx), _p(g), _p(hmap), _p(gout), _p(ghist),
+                                             _I(R), _I(F), _I(hsize), _I(n_src), _I(chunk),
+                                             _I(view_rows)), "bwd_mean_row_batch_view")
+    return gout, ghist
+
+
 def bwd_mean_src(ptr, idx, g, n_src, chunk=0, hmap_src=None, hist_shape=None):
     """Backward of the mean with per-source substitution.  Without ``hmap_src``: the gradient of the
     row that was read for every source, whichever table it came from.  With ``hmap_src``: returns

@@ -308,6 +308,53 @@ def test_chunked_backward_order(orc):
     np.testing.assert_allclose(got, seq, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("seed,R_layer", [(21, 25), (22, 60), (23, 1), (24, 0)])
+def test_batch_view_backward_order(orc, seed, R_layer):
+    """The summation order over ONE view of the whole mini-batch CSR (hc_aggr_bwd_batch_view): positions
+    count every edge of the batch's rows, a hub is a source with more than `chunk` of them, a chunk is a
+    run of `chunk` positions of which only the live edges (rows of the layer that did not take their
+    history row) are added.  Written out independently with NumPy float32; equal, as a value, to the
+    dense product in fp64; the same bits as the per-layer statement wherever no hub is involved."""
+    rng = np.random.default_rng(seed)
+    R_all, N, F, C = 60, 9, 5, 8
+    deg = rng.integers(0, 5, size=R_all)
+    ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    idx = rng.integers(0, N, size=int(ptr[-1]), dtype=np.int64)
+    idx[idx == 4] = 5                                   # source 4 has no edges
+    n_src = 7                                           # the layer's sources; rows of the layer stay below
+    dst = np.repeat(np.arange(R_all), deg)
+    idx[(dst < R_layer) & (idx >= n_src)] = 1
+    g = rng.standard_normal((R_layer, F)).astype(np.float32)
+    hmap = np.where(rng.random(R_layer) < 0.3, 3, -1).astype(np.int64)
+    got, gh = orc.bwd_mean_row_batch_view(ptr, idx, g, hmap, n_src, R_all, hbuf_shape=(R_layer, F), chunk=C)
+    seq, gh_seq = orc.bwd_mean_row(ptr[:R_layer + 1], idx, g, hmap, n_src, hbuf_shape=(R_layer, F))
+    np.testing.assert_array_equal(gh, gh_seq)
+    unchunked, _ = orc.bwd_mean_row_batch_view(ptr, idx, g, hmap, n_src, R_all, hbuf_shape=(R_layer, F))
+    np.testing.assert_array_equal(unchunked, seq)       # without a chunk rule the view's extent is irrelevant
+    live = lambda e: dst[e] < R_layer and hmap[dst[e]] == -1
+    any_hub = False
+    for s in range(n_src):
+        es = [e for e in range(len(idx)) if idx[e] == s]            # view positions: (row, slot) ascending
+        if len(es) <= C:
+            np.testing.assert_array_equal(got[s], seq[s])
+            continue
+        any_hub = True
+        tot = None
+        for c0 in range(0, len(es), C):
+            acc = np.zeros(F, np.float32)
+            for e in es[c0:c0 + C]:
+                if live(e):
+                    acc = acc + g[dst[e]] / np.float32(deg[dst[e]])
+            tot = acc if tot is None else tot + acc
+        np.testing.assert_array_equal(got[s], tot)
+    assert any_hub
+    # value: (D^-1 A restricted to live rows)^T g in fp64
+    A = sp.csr_matrix((np.ones(int(ptr[R_layer])), idx[:ptr[R_layer]], ptr[:R_layer + 1]), shape=(R_layer, N))
+    scale = (hmap == -1) / np.maximum(deg[:R_layer], 1)
+    ref = (A.T @ (g.astype(np.float64) * scale[:, None]))[:n_src]
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-6)
+
+
 def test_multithreaded_cpu_statement_equals_the_sequential_one(orc):
     """The OpenMP statement that the benchmark times as its CPU baseline gives the sequential statement's
     bits: forward with per-source substitution (long rows as quarters), transposed view, backward gather
