@@ -276,7 +276,29 @@ struct TrSmallHeader {
   unsigned pad[63];
 };
 
-__global__ __launch_bounds__(HC_BLOCK) void tr_small_clear(uint32_t *__restrict__ p, int64_t n) {
+// Sizes of the block: given by value, or -- when the host does not know them yet (a batch that the
+// sampler has just drawn) -- read from device memory and clamped to the bounds the launch was sized for.
+struct TrDims {
+  int64_t R, E, n_src;               // by value (or the upper bounds when the pointers are set)
+  const int64_t *pR, *pE, *pS;       // nullable, all three or none
+};
+__device__ __forceinline__ void tr_dims(const TrDims &d, int64_t &R, int64_t &E, int64_t &n_src) {
+  R = d.R;
+  E = d.E;
+  n_src = d.n_src;
+  if (d.pE != nullptr) {
+    const int64_t r = *d.pR, e = *d.pE, s = *d.pS;
+    R = r < 0 ? 0 : r;               // rows are bounded by the caller's ptr array
+    E = e < 0 ? 0 : (e < d.E ? e : d.E);
+    n_src = s < 0 ? 0 : (s < d.n_src ? s : d.n_src);
+  }
+}
+
+// zero the ticket and the counters of sources [0, n_src] (rounded up to whole 16-byte groups)
+__global__ __launch_bounds__(HC_BLOCK) void tr_small_clear(uint32_t *__restrict__ p, TrDims dims) {
+  int64_t R, E, n_src;
+  tr_dims(dims, R, E, n_src);
+  const int64_t n = (int64_t)(sizeof(TrSmallHeader) / sizeof(uint32_t)) + (n_src + 1 + 3) / 4 * 4;
   const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
   if (i < n) p[i] = 0u;
 }
@@ -289,46 +311,49 @@ __device__ __forceinline__ int trs_load(const int *p) { return *p; }
 __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const int64_t *__restrict__ hmap_row,
     const int64_t *__restrict__ hmap_src, uint32_t *__restrict__ keys, int32_t *__restrict__ rows,
-    int *__restrict__ count, TrSmallHeader *__restrict__ header, int64_t *__restrict__ ptrT, int64_t R,
-    int64_t E, int64_t n_src) {
+    int *__restrict__ count, TrSmallHeader *__restrict__ header, int64_t *__restrict__ ptrT, TrDims dims) {
   __shared__ int64_t s_ptr[TR_LDS_ROWS];
   __shared__ int64_t s_range[2];
   __shared__ int s_wave[TRS_BLOCK / HC_WAVE];
   __shared__ int s_last;
+  int64_t R, E, n_src;
+  tr_dims(dims, R, E, n_src);
   const int64_t e0 = (int64_t)blockIdx.x * TRS_BLOCK;
   const int64_t e1 = e0 + TRS_BLOCK < E ? e0 + TRS_BLOCK : E;
-  if (threadIdx.x < 2 * HC_WAVE) {       // the tile's first and last row, searched by two waves side by side
-    const int lane0 = hc_lane();
-    const int which = (int)(threadIdx.x >> 6);
-    const int64_t r = tr_row_of_wave(ptr, R, which == 0 ? e0 : e1 - 1, lane0);
-    if (lane0 == 0) s_range[which] = r;
-  }
-  __syncthreads();
-  const int64_t r_lo = s_range[0], r_hi = s_range[1];
-  const int64_t span = r_hi - r_lo + 1;
-  const bool staged = span <= TR_LDS_ROWS;
-  if (staged)
-    for (int64_t i = threadIdx.x; i < span; i += TRS_BLOCK) s_ptr[i] = ptr[r_lo + i];
-  __syncthreads();
-  const int64_t e = e0 + threadIdx.x;
-  if (e < e1) {
-    int64_t row;
-    bool live;
-    if (staged) {
-      const int64_t l = tr_row_of(s_ptr, (int64_t)0, span - 1, e);
-      row = r_lo + l;
-      live = row < R && s_ptr[l] <= e;
-    } else {
-      row = tr_row_of(ptr, r_lo, r_hi, e);
-      live = row < R && ptr[row] <= e;
+  if (e0 < E && R > 0) {                 // block-uniform: blocks behind the last edge slot only take a ticket
+    if (threadIdx.x < 2 * HC_WAVE) {       // the tile's first and last row, searched by two waves side by side
+      const int lane0 = hc_lane();
+      const int which = (int)(threadIdx.x >> 6);
+      const int64_t r = tr_row_of_wave(ptr, R, which == 0 ? e0 : e1 - 1, lane0);
+      if (lane0 == 0) s_range[which] = r;
     }
-    if (live && hmap_row != nullptr) live = hmap_row[row] == -1;
-    int64_t src = live ? idx[e] : -1;
-    if (src < 0 || src >= n_src) live = false;
-    if (live && hmap_src != nullptr) live = hmap_src[src] == -1;
-    keys[e] = live ? (uint32_t)src : (uint32_t)n_src;
-    rows[e] = live ? (int32_t)row : -1;
-    if (live) atomicAdd(count + src, 1);
+    __syncthreads();
+    const int64_t r_lo = s_range[0], r_hi = s_range[1];
+    const int64_t span = r_hi - r_lo + 1;
+    const bool staged = span <= TR_LDS_ROWS;
+    if (staged)
+      for (int64_t i = threadIdx.x; i < span; i += TRS_BLOCK) s_ptr[i] = ptr[r_lo + i];
+    __syncthreads();
+    const int64_t e = e0 + threadIdx.x;
+    if (e < e1) {
+      int64_t row;
+      bool live;
+      if (staged) {
+        const int64_t l = tr_row_of(s_ptr, (int64_t)0, span - 1, e);
+        row = r_lo + l;
+        live = row < R && s_ptr[l] <= e;
+      } else {
+        row = tr_row_of(ptr, r_lo, r_hi, e);
+        live = row < R && ptr[row] <= e;
+      }
+      if (live && hmap_row != nullptr) live = hmap_row[row] == -1;
+      int64_t src = live ? idx[e] : -1;
+      if (src < 0 || src >= n_src) live = false;
+      if (live && hmap_src != nullptr) live = hmap_src[src] == -1;
+      keys[e] = live ? (uint32_t)src : (uint32_t)n_src;
+      rows[e] = live ? (int32_t)row : -1;
+      if (live) atomicAdd(count + src, 1);
+    }
   }
   // The block that takes the last ticket sees every block's counts.  One device-scope release per
   // block, by the thread that takes the ticket, behind the block's barrier (which orders the other
@@ -409,12 +434,13 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_small_place(const uint32_t *__res
                                                             const int32_t *__restrict__ rows,
                                                             int *__restrict__ cursor,
                                                             int32_t *__restrict__ tmp_row,
-                                                            int32_t *__restrict__ tmp_edge, int64_t E,
-                                                            uint32_t sentinel) {
+                                                            int32_t *__restrict__ tmp_edge, TrDims dims) {
+  int64_t R, E, n_src;
+  tr_dims(dims, R, E, n_src);
   const int64_t e = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
-  if (e >= E) return;
+  if (e >= E || R <= 0) return;
   const uint32_t k = keys[e];
-  if (k == sentinel) return;
+  if (k == (uint32_t)n_src) return;      // the sentinel of a dropped slot
   const int p = atomicAdd(cursor + k, 1);
   tmp_row[p] = rows[e];
   tmp_edge[p] = (int32_t)e;
@@ -424,8 +450,9 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_small_order(const int64_t *__rest
                                                             const int32_t *__restrict__ tmp_row,
                                                             const int32_t *__restrict__ tmp_edge,
                                                             int32_t *__restrict__ rowT,
-                                                            int32_t *__restrict__ edgeT, int64_t n_src,
-                                                            int64_t E) {
+                                                            int32_t *__restrict__ edgeT, TrDims dims) {
+  int64_t R_unused, E, n_src;
+  tr_dims(dims, R_unused, E, n_src);
   __shared__ uint32_t bits[TRS_BITMAP_WORDS];
   __shared__ int pre8[TRS_BITMAP_WORDS / 8];
   __shared__ int long_src[TRS_ORDER_SOURCES];
@@ -494,55 +521,68 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_small_order(const int64_t *__rest
   }
   __syncthreads();
   // longer segments: the whole block, one segment at a time.  The segment's slots set their bits in an
-  // LDS bitmap over all edge slots; a slot's rank is the number of set bits below it.
+  // LDS bitmap over a window of TR_SMALL_EDGES edge slots (one window covers a whole block of that size;
+  // larger blocks take several); a slot's rank is the number of the segment's slots in earlier windows
+  // plus the set bits below it in its own.
   const int n_long = n_long_s;
-  const int words = (int)((E + 31) / 32);
   for (int t = 0; t < n_long; ++t) {
     const int64_t src = (int64_t)blockIdx.x * TRS_ORDER_SOURCES + long_src[t];
     const int64_t sb = ptrT[src];
     const int sl = (int)(ptrT[src + 1] - sb);
-    for (int w = threadIdx.x; w < words; w += HC_BLOCK) bits[w] = 0u;
-    __syncthreads();
-    for (int i = threadIdx.x; i < sl; i += HC_BLOCK) {
-      const int e = tmp_edge[sb + i];
-      atomicOr(&bits[e >> 5], 1u << (e & 31));
-    }
-    __syncthreads();
-    // pre8[g] = set bits in front of word group g (8 words): per-thread run of groups, block scan
-    const int groups = (words + 7) / 8;
-    const int per = (groups + HC_BLOCK - 1) / HC_BLOCK;
-    int glo = (int)threadIdx.x * per, ghi = glo + per;
-    if (glo > groups) glo = groups;
-    if (ghi > groups) ghi = groups;
-    int sum = 0;
-    for (int g = glo; g < ghi; ++g)
-      for (int w = g * 8; w < g * 8 + 8 && w < words; ++w) sum += __popc(bits[w]);
-    int x = sum;
+    int before = 0;                                  // the segment's slots in the windows already done
+    for (int64_t w0 = 0; w0 < E; w0 += TR_SMALL_EDGES) {
+      const int64_t span = E - w0 < TR_SMALL_EDGES ? E - w0 : TR_SMALL_EDGES;
+      const int words = (int)((span + 31) / 32);
+      for (int w = threadIdx.x; w < words; w += HC_BLOCK) bits[w] = 0u;
+      __syncthreads();
+      for (int i = threadIdx.x; i < sl; i += HC_BLOCK) {
+        const int64_t e = (int64_t)tmp_edge[sb + i] - w0;
+        if (e >= 0 && e < span) atomicOr(&bits[e >> 5], 1u << (e & 31));
+      }
+      __syncthreads();
+      // pre8[g] = set bits in front of word group g (8 words): per-thread run of groups, block scan
+      const int groups = (words + 7) / 8;
+      const int per = (groups + HC_BLOCK - 1) / HC_BLOCK;
+      int glo = (int)threadIdx.x * per, ghi = glo + per;
+      if (glo > groups) glo = groups;
+      if (ghi > groups) ghi = groups;
+      int sum = 0;
+      for (int g = glo; g < ghi; ++g)
+        for (int w = g * 8; w < g * 8 + 8 && w < words; ++w) sum += __popc(bits[w]);
+      int x = sum;
 #pragma unroll
-    for (int d = 1; d < HC_WAVE; d <<= 1) {
-      const int y = __shfl_up(x, d, HC_WAVE);
-      if (lane >= d) x += y;
+      for (int d = 1; d < HC_WAVE; d <<= 1) {
+        const int y = __shfl_up(x, d, HC_WAVE);
+        if (lane >= d) x += y;
+      }
+      if (lane == HC_WAVE - 1) s_wave[wave] = x;
+      __syncthreads();
+      int run = before + x - sum;
+      int in_window = 0;
+      for (int w = 0; w < HC_WAVES_PER_BLOCK; ++w) {
+        if (w < wave) run += s_wave[w];
+        in_window += s_wave[w];
+      }
+      for (int g = glo; g < ghi; ++g) {
+        pre8[g] = run;
+        for (int w = g * 8; w < g * 8 + 8 && w < words; ++w) run += __popc(bits[w]);
+      }
+      __syncthreads();
+      for (int i = threadIdx.x; i < sl; i += HC_BLOCK) {
+        const int e_abs = tmp_edge[sb + i];
+        const int64_t e = (int64_t)e_abs - w0;
+        if (e < 0 || e >= span) continue;
+        const int r = tmp_row[sb + i];
+        const int w = (int)(e >> 5);
+        int rank = pre8[w >> 3];
+        for (int q = (w >> 3) * 8; q < w; ++q) rank += __popc(bits[q]);
+        rank += __popc(bits[w] & ((1u << (e & 31)) - 1u));
+        rowT[sb + rank] = r;
+        if (edgeT != nullptr) edgeT[sb + rank] = e_abs;
+      }
+      before += in_window;
+      __syncthreads();
     }
-    if (lane == HC_WAVE - 1) s_wave[wave] = x;
-    __syncthreads();
-    int run = x - sum;
-    for (int w = 0; w < wave; ++w) run += s_wave[w];
-    for (int g = glo; g < ghi; ++g) {
-      pre8[g] = run;
-      for (int w = g * 8; w < g * 8 + 8 && w < words; ++w) run += __popc(bits[w]);
-    }
-    __syncthreads();
-    for (int i = threadIdx.x; i < sl; i += HC_BLOCK) {
-      const int e = tmp_edge[sb + i];
-      const int r = tmp_row[sb + i];
-      const int w = e >> 5;
-      int rank = pre8[w >> 3];
-      for (int q = (w >> 3) * 8; q < w; ++q) rank += __popc(bits[q]);
-      rank += __popc(bits[w] & ((1u << (e & 31)) - 1u));
-      rowT[sb + rank] = r;
-      if (edgeT != nullptr) edgeT[sb + rank] = e;
-    }
-    __syncthreads();
   }
 }
 
@@ -561,6 +601,31 @@ SmallLayout small_layout(int64_t E, int64_t n_src) {
   return L;
 }
 inline bool small_block(int64_t E, int64_t n_src) { return E <= TR_SMALL_EDGES && n_src <= TR_SMALL_SOURCES; }
+
+// The four launches of the counting sort; dims.E / dims.n_src size the grids (upper bounds when the real
+// sizes are read on the device).
+int small_launch(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row, const int64_t *hmap_src,
+                 const TrDims &dims, int64_t *ptrT, int32_t *rowT, int32_t *edgeT, char *w, const SmallLayout &S,
+                 hipStream_t st) {
+  TrSmallHeader *header = reinterpret_cast<TrSmallHeader *>(w);
+  int *count = reinterpret_cast<int *>(w + S.count);
+  uint32_t *keys = reinterpret_cast<uint32_t *>(w + S.keys);
+  int32_t *rows = reinterpret_cast<int32_t *>(w + S.rows);
+  int32_t *tmp_row = reinterpret_cast<int32_t *>(w + S.tmp_row);
+  int32_t *tmp_edge = reinterpret_cast<int32_t *>(w + S.tmp_edge);
+  const int64_t E = dims.E > 0 ? dims.E : 1, n_src = dims.n_src;
+  const int64_t clear_words = (int64_t)(S.keys / sizeof(uint32_t));   // header + counters
+  const int64_t cb = (clear_words + HC_BLOCK - 1) / HC_BLOCK, eb = (E + TRS_BLOCK - 1) / TRS_BLOCK;
+  const int64_t pb = (E + HC_BLOCK - 1) / HC_BLOCK, ob = (n_src + TRS_ORDER_SOURCES - 1) / TRS_ORDER_SOURCES;
+  if (!hc_grid_ok(cb) || !hc_grid_ok(eb) || !hc_grid_ok(pb) || !hc_grid_ok(ob)) return HC_EUNSUPPORTED;
+  tr_small_clear<<<dim3((unsigned)cb), dim3(HC_BLOCK), 0, st>>>(reinterpret_cast<uint32_t *>(w), dims);
+  tr_small_count<<<dim3((unsigned)eb), dim3(TRS_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, keys, rows, count,
+                                                                 header, ptrT, dims);
+  tr_small_place<<<dim3((unsigned)pb), dim3(HC_BLOCK), 0, st>>>(keys, rows, count, tmp_row, tmp_edge, dims);
+  if (n_src > 0)
+    tr_small_order<<<dim3((unsigned)ob), dim3(HC_BLOCK), 0, st>>>(ptrT, tmp_row, tmp_edge, rowT, edgeT, dims);
+  return hc_launch_status();
+}
 
 // bits[s] = (hmap_src[s] != -1), 64 sources per ballot
 __global__ __launch_bounds__(HC_BLOCK) void tr_src_bits(const int64_t *__restrict__ hmap, int64_t n_src,
@@ -650,23 +715,8 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
     if (!workspace || workspace_bytes < S.total) return HC_EWORKSPACE;
     char *w = static_cast<char *>(workspace);
     if (reinterpret_cast<uintptr_t>(w) % 256 != 0) return HC_EWORKSPACE;
-    TrSmallHeader *header = reinterpret_cast<TrSmallHeader *>(w);
-    int *count = reinterpret_cast<int *>(w + S.count);
-    uint32_t *keys = reinterpret_cast<uint32_t *>(w + S.keys);
-    int32_t *rows = reinterpret_cast<int32_t *>(w + S.rows);
-    int32_t *tmp_row = reinterpret_cast<int32_t *>(w + S.tmp_row);
-    int32_t *tmp_edge = reinterpret_cast<int32_t *>(w + S.tmp_edge);
-    const int64_t clear_words = (int64_t)(S.keys / sizeof(uint32_t));   // header + counters
-    tr_small_clear<<<dim3((unsigned)((clear_words + HC_BLOCK - 1) / HC_BLOCK)), dim3(HC_BLOCK), 0, st>>>(
-        reinterpret_cast<uint32_t *>(w), clear_words);
-    tr_small_count<<<dim3((unsigned)((E + TRS_BLOCK - 1) / TRS_BLOCK)), dim3(TRS_BLOCK), 0, st>>>(
-        ptr, idx, hmap_row, hmap_src, keys, rows, count, header, ptrT, R, E, n_src);
-    tr_small_place<<<dim3((unsigned)((E + HC_BLOCK - 1) / HC_BLOCK)), dim3(HC_BLOCK), 0, st>>>(
-        keys, rows, count, tmp_row, tmp_edge, E, (uint32_t)n_src);
-    if (n_src > 0)
-      tr_small_order<<<dim3((unsigned)((n_src + TRS_ORDER_SOURCES - 1) / TRS_ORDER_SOURCES)), dim3(HC_BLOCK), 0, st>>>(
-          ptrT, tmp_row, tmp_edge, rowT, edgeT, n_src, E);
-    return hc_launch_status();
+    const TrDims dims{R, E, n_src, nullptr, nullptr, nullptr};
+    return small_launch(ptr, idx, hmap_row, hmap_src, dims, ptrT, rowT, edgeT, w, S, st);
   }
   if (E > TR_SORT_MEMSET_EDGES) {
     // Above this size the sort library takes its one-sweep path, which clears its counters with
@@ -743,4 +793,28 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
     tr_finalize_ptr<<<dim3((unsigned)pblocks), dim3(HC_BLOCK), 0, st>>>(skeys, ptrT, E, n_src);
   }
   return hc_launch_status();
+}
+
+// Limits of the variant with device-resident sizes: the counters are 32-bit and one block scans them.
+constexpr int64_t TR_DEV_MAX_EDGES = (int64_t)1 << 24;
+constexpr int64_t TR_DEV_MAX_SOURCES = (int64_t)1 << 24;
+
+extern "C" size_t hc_transpose_dev_workspace_bytes(int64_t max_E, int64_t max_src) {
+  if (max_E < 0 || max_src < 0 || max_E > TR_DEV_MAX_EDGES || max_src > TR_DEV_MAX_SOURCES) return 0;
+  return small_layout(max_E, max_src).total;
+}
+
+extern "C" int hc_build_transpose_dev(const int64_t *ptr, const int64_t *idx, const int64_t *R_dev,
+                                      const int64_t *E_dev, const int64_t *n_src_dev, int64_t max_E,
+                                      int64_t max_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT,
+                                      void *workspace, size_t workspace_bytes, void *stream) {
+  HC_REQUIRE(ptr && idx && R_dev && E_dev && n_src_dev && ptrT && max_E >= 0 && max_src >= 0);
+  HC_REQUIRE(rowT != nullptr || max_E == 0);
+  if (max_E > TR_DEV_MAX_EDGES || max_src > TR_DEV_MAX_SOURCES) return HC_EUNSUPPORTED;
+  const SmallLayout S = small_layout(max_E, max_src);
+  if (!workspace || workspace_bytes < S.total) return HC_EWORKSPACE;
+  char *w = static_cast<char *>(workspace);
+  if (reinterpret_cast<uintptr_t>(w) % 256 != 0) return HC_EWORKSPACE;
+  const TrDims dims{0, max_E, max_src, R_dev, E_dev, n_src_dev};
+  return small_launch(ptr, idx, nullptr, nullptr, dims, ptrT, rowT, edgeT, w, S, static_cast<hipStream_t>(stream));
 }

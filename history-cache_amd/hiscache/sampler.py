@@ -17,9 +17,14 @@ import hiscache_backend as _be
 
 class NeighborSampler:
 
-    def __init__(self, indptr, indices, fanout, labels=None, seed=0, device="cuda:0", validate=True):
+    def __init__(self, indptr, indices, fanout, labels=None, seed=0, device="cuda:0", validate=True,
+                 emit_view=False):
         """``indptr`` / ``indices``: CSR of the full graph (int64; moved to ``device``).  ``fanout[k]``
-        neighbours are drawn, without replacement, for nodes first reached at hop k."""
+        neighbours are drawn, without replacement, for nodes first reached at hop k.  ``emit_view``:
+        every batch also carries ``batch.view``, the transposed view of its CSR
+        (``hiscache_backend.BatchView``), built right behind the sampling on the sampler's stream, so
+        that the layers' backward builds none."""
+        self.emit_view = bool(emit_view)
         self.device = torch.device(device)
         self.indptr = torch.as_tensor(indptr, dtype=torch.int64).to(self.device).contiguous()
         self.indices = torch.as_tensor(indices, dtype=torch.int64).to(self.device).contiguous()
@@ -63,7 +68,8 @@ class NeighborSampler:
         if stream != cur:
             stream.wait_stream(cur)                                    # seeds may have been produced there
         with torch.cuda.stream(stream):
-            out = _be.sample_layers(self.indptr, self.indices, seeds, self.fanout, rng_seed, self.node_map)
+            out = _be.sample_layers(self.indptr, self.indices, seeds, self.fanout, rng_seed, self.node_map,
+                                    emit_view=self.emit_view)
             counts_host = self._host_pool.pop() if self._host_pool else torch.empty(
                 2 * len(self.fanout) + 1, dtype=torch.int64, pin_memory=True)
             counts_host.copy_(out[3], non_blocking=True)
@@ -73,15 +79,21 @@ class NeighborSampler:
         return _PendingBatch(self, out, counts_host, done, seeds, y, stream)
 
     def _finish(self, out, counts_host, seeds, y, stream):
-        ptr, idx, s2f, _ = out
+        ptr, idx, s2f = out[:3]
         L = len(self.fanout)
         c = counts_host.tolist()
         self._host_pool.append(counts_host)
         nnl, nel = c[: L + 1], c[L + 1:]
         cur = torch.cuda.current_stream(self.device)
+        view = None
+        if self.emit_view:
+            ptrT, rowT = out[4], out[5]
+            view = _be.BatchView(ptrT[: nnl[L] + 1], rowT[: max(nel[-1], 1)], None, nnl[L - 1], nnl[L], nel[-1])
         if stream != cur:
             for t in (ptr, idx, s2f, seeds) + (() if y is None else (y,)):
                 t.record_stream(cur)
+            if view is not None:
+                view.record_stream(cur)
         return SimpleNamespace(
             ptr=ptr[: nnl[L - 1] + 1],
             idx=idx[: nel[-1]],
@@ -92,6 +104,7 @@ class NeighborSampler:
             x=None,
             edge_type=None,
             typed_num_node_in_layer=None,
+            view=view,
         )
 
 

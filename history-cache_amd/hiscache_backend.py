@@ -55,6 +55,9 @@ _SIGNATURES = {
     "hc_transpose_workspace_bytes": (_c_sz, [_c_i64, _c_i64, _c_i64]),
     "hc_build_transpose": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p,
                                     _c_sz, _c_p]),
+    "hc_transpose_dev_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
+    "hc_build_transpose_dev": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_sz,
+                                        _c_p]),
     "hc_aggr_bwd_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
     "hc_aggr_bwd_chunk_edges": (_c_i64, [_c_i64]),
     "hc_aggr_bwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_p,
@@ -1017,14 +1020,45 @@ def sample_capacity(n_seed, fanout, num_nodes):
     return tuple(int(o.value) for o in out)
 
 
-def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map):
+def build_transpose_dev(ptr, idx, rows_dev, edges_dev, nodes_dev, max_edges, max_nodes, want_edges=False):
+    """The transposed view of a block whose sizes are still on the device (one-element int64 views
+    ``rows_dev``, ``edges_dev``, ``nodes_dev``, e.g. slices of the sampler's ``counts``): returns
+    (ptrT, rowT, edgeT) at the capacities ``max_nodes + 1`` / ``max_edges``; nothing is read back."""
+    lib = load_library()
+    _dev(ptr, "ptr", torch.int64)
+    _dev(idx, "idx", torch.int64)
+    for t, name in ((rows_dev, "rows_dev"), (edges_dev, "edges_dev"), (nodes_dev, "nodes_dev")):
+        _dev(t, name, torch.int64)
+        if t.numel() < 1:
+            raise ValueError(f"{name} is empty")
+    max_edges, max_nodes = int(max_edges), int(max_nodes)
+    if idx.numel() < max_edges:
+        raise ValueError("idx is shorter than max_edges")
+    dev = ptr.device
+    nbytes = int(lib.hc_transpose_dev_workspace_bytes(max_edges, max_nodes))
+    if nbytes == 0:
+        raise ValueError("block too large for the device-sized transposed view (2^24 edges / nodes)")
+    ptrT = torch.empty(max_nodes + 1, dtype=torch.int64, device=dev)
+    rowT = torch.empty(max(max_edges, 1), dtype=torch.int32, device=dev)
+    edgeT = torch.empty(max(max_edges, 1), dtype=torch.int32, device=dev) if want_edges else None
+    ws = _workspace(nbytes, dev)
+    rc = lib.hc_build_transpose_dev(_ptr(ptr), _ptr(idx), _ptr(rows_dev), _ptr(edges_dev), _ptr(nodes_dev),
+                                    max_edges, max_nodes, _ptr(ptrT), _ptr(rowT), _ptr(edgeT), _ptr(ws),
+                                    ws.numel(), _stream())
+    _check(rc, "hc_build_transpose_dev")
+    return ptrT, rowT, edgeT
+
+
+def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map, emit_view=False):
     """Layered neighbour sampling without replacement.  Returns (ptr, idx, sub_to_full, counts) as
     device tensors at their capacity; ``counts`` (int64[2L+1] on the device) holds the node count
     within k hops for k = 0..L and then the cumulative edge count after every hop, so the caller
     slices ptr[:counts[L-1]+1], idx[:counts[2L]], sub_to_full[:counts[L]] once it has read them.
     ``seeds`` must be distinct valid node ids; ``node_map`` comes from ``sample_map`` and is left
     all-unseen again.  Stands where the reference's external loader does
-    (/root/reference/hiscache/history_trainer.py:19,26)."""
+    (/root/reference/hiscache/history_trainer.py:19,26).  ``emit_view=True`` appends (ptrT, rowT): the
+    transposed view of the whole sampled CSR, built behind the sampling with the sizes still on the
+    device (``build_transpose_dev``), for ``BatchView`` once the caller has read ``counts``."""
     lib = load_library()
     _dev(indptr, "indptr", torch.int64)
     _dev(indices, "indices", torch.int64)
@@ -1052,6 +1086,10 @@ def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map):
                               ctypes.c_uint64(int(rng_seed) & 0xFFFFFFFFFFFFFFFF), _ptr(node_map), _ptr(ptr),
                               _ptr(idx), _ptr(s2f), _ptr(counts), _ptr(ws), ws_bytes, _stream())
     _check(rc, "hc_sample_layers")
+    if emit_view:
+        ptrT, rowT, _ = build_transpose_dev(ptr, idx, counts[L - 1:L], counts[2 * L:2 * L + 1], counts[L:L + 1],
+                                            edges, nodes)
+        return ptr, idx, s2f, counts, ptrT, rowT
     return ptr, idx, s2f, counts
 
 

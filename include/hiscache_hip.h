@@ -125,6 +125,25 @@ int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hm
                        int32_t *rowT, int32_t *edgeT, void *workspace, size_t workspace_bytes,
                        void *stream);
 
+/* hc_build_transpose_dev: the same view (no history maps: nothing is left out)
+ * for a block whose sizes the host does not know yet -- a mini-batch that
+ * hc_sample_layers has just drawn, whose layer sizes are still in its `counts`
+ * array on the device.  *R_dev, *E_dev, *n_src_dev are read by the kernels;
+ * max_E / max_src (the capacities of idx and of the node list, at most 2^24
+ * each) size the launches, the workspace and the outputs: ptrT[max_src+1],
+ * rowT[max_E], edgeT[max_E] (nullable).  Only ptrT[0..n_src] and the first
+ * ptrT[n_src] entries of rowT/edgeT are written.  Four launches, kernels only
+ * (safe under stream capture), nothing is read back: this is how the sampler
+ * emits the batch's transposed view together with the batch, so that backward
+ * (hc_aggr_bwd_batch_view) builds none.  The loader of the reference hands over
+ * one shared CSR per batch (hiscache/history_model.py:124-128); the CSC is this
+ * library's addition to that wire format. */
+size_t hc_transpose_dev_workspace_bytes(int64_t max_E, int64_t max_src);
+int hc_build_transpose_dev(const int64_t *ptr, const int64_t *idx, const int64_t *R_dev,
+                           const int64_t *E_dev, const int64_t *n_src_dev, int64_t max_E,
+                           int64_t max_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT,
+                           void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------- aggregation backward
  * Replaces AggrHistoryFunction::backward / AggrHistoryEdgeValueFunction::backward
  * (history_aggr.cu:493-596; kernels :127-397).

@@ -118,3 +118,78 @@ def test_batch_view_rejects_a_layer_it_does_not_cover(be):
     g = torch.zeros(200, 64, device=DEV)
     with pytest.raises(ValueError):
         be._aggr_bwd_batch_view(T(ptr), view, g, None, None, 0, 200, 400)
+
+
+def _stable_view(ptr, idx, R, n_src):
+    """NumPy statement of the view: edges of the first R rows in stable order of their source."""
+    E = int(ptr[R])
+    dst = np.repeat(np.arange(R), np.diff(ptr[:R + 1]))
+    order = np.argsort(idx[:E], kind="stable")
+    ptrT = np.zeros(n_src + 1, np.int64)
+    np.cumsum(np.bincount(idx[:E], minlength=n_src), out=ptrT[1:])
+    return ptrT, dst[order].astype(np.int32), order.astype(np.int32)
+
+
+@pytest.mark.parametrize("R,n_src,max_deg,hub_edges,slack", [
+    (3000, 2000, 9, 700, 0),             # one window of edge slots, capacities equal to the sizes
+    (9000, 3000, 12, 3000, 5000),        # capacities above the sizes
+    (120000, 50000, 9, 9000, 200000),    # more than 2^18 edge slots: hubs ranked over several windows
+    (10, 2000, 0, 0, 100),               # no edge at all
+])
+def test_view_with_sizes_on_the_device(be, R, n_src, max_deg, hub_edges, slack):
+    """hc_build_transpose_dev reads R, E and n_src from device memory (launches sized by capacities):
+    the same view as a stable NumPy sort, with and without edge slots."""
+    rng = np.random.default_rng(R + n_src)
+    deg = rng.integers(0, max_deg + 1, size=R)
+    ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    E = int(ptr[-1])
+    idx = rng.integers(0, n_src, size=E, dtype=np.int64)
+    if hub_edges:
+        pos = rng.permutation(E)
+        idx[pos[:hub_edges]] = 5                        # a hub whose slots are spread over the whole block
+        idx[pos[hub_edges:hub_edges + 65]] = n_src - 1   # just above a wave's worth
+        idx[pos[hub_edges + 65:hub_edges + 129]] = 0     # exactly a wave's worth
+    max_E, max_src = E + slack, n_src + (slack // 7)
+    idx_cap = np.concatenate([idx, np.full(max_E - E, -7, np.int64)])     # capacity beyond the block: never read
+    sizes = T(np.array([R, E, n_src], np.int64))
+    want_ptrT, want_rowT, want_edgeT = _stable_view(ptr, idx, R, n_src)
+    for want_edges in (False, True):
+        ptrT, rowT, edgeT = be.build_transpose_dev(T(ptr), T(idx_cap), sizes[0:1], sizes[1:2], sizes[2:3], max_E,
+                                                   max_src, want_edges=want_edges)
+        np.testing.assert_array_equal(ptrT[: n_src + 1].cpu().numpy(), want_ptrT)
+        np.testing.assert_array_equal(rowT[:E].cpu().numpy(), want_rowT)
+        if want_edges:
+            np.testing.assert_array_equal(edgeT[:E].cpu().numpy(), want_edgeT)
+
+
+@pytest.mark.parametrize("fanout,n_seed", [([5, 3], 64), ([15, 10, 5], 1200)])
+def test_sampler_emits_the_view_with_the_batch(be, orc, fanout, n_seed):
+    """NeighborSampler(emit_view=True): batch.view is the stable transposed view of batch.ptr / batch.idx,
+    for consecutive batches, also when sampled ahead on the sampler's stream; the batch itself is the one
+    the plain sampler draws."""
+    from helpers import power_law_graph
+    from hiscache import NeighborSampler
+    rng = np.random.default_rng(31 + n_seed)
+    n = 60000
+    indptr, indices = power_law_graph(rng, n, 6.0, max_degree=3000)
+    plain = NeighborSampler(indptr, indices, fanout, seed=4, device=DEV)
+    emitting = NeighborSampler(indptr, indices, fanout, seed=4, device=DEV, emit_view=True)
+    pending = None
+    for it in range(3):
+        seeds = torch.from_numpy(rng.choice(n, size=n_seed, replace=False).astype(np.int64)).to(DEV)
+        print("view case", fanout, n_seed, it, flush=True)
+        a = plain.sample(seeds)
+        b = emitting.sample_async(seeds).get() if it else emitting.sample(seeds)
+        assert torch.equal(a.ptr, b.ptr) and torch.equal(a.idx, b.idx) and torch.equal(a.sub_to_full, b.sub_to_full)
+        L = len(fanout)
+        R, n_all = int(b.num_node_in_layer[L - 1]), int(b.num_node_in_layer[L])
+        v = b.view
+        assert (v.rows, v.n_src, v.num_edge) == (R, n_all, b.idx.numel())
+        want_ptrT, want_rowT, _ = _stable_view(b.ptr.cpu().numpy(), b.idx.cpu().numpy(), R, n_all)
+        np.testing.assert_array_equal(v.ptrT.cpu().numpy(), want_ptrT)
+        np.testing.assert_array_equal(v.rowT[: v.num_edge].cpu().numpy(), want_rowT)
+        o_ptrT, o_rowT, _ = orc.build_transpose(b.ptr.cpu().numpy(), b.idx.cpu().numpy(), None, n_all, R)
+        np.testing.assert_array_equal(want_ptrT, o_ptrT)
+        np.testing.assert_array_equal(want_rowT, o_rowT)
+    assert int((emitting.node_map != 0x7fffffff).sum()) == 0
+    del pending
