@@ -45,6 +45,9 @@ def parse():
                          "(next batch sampled on a side stream) instead of taking pre-generated batches")
     ap.add_argument("--prefetch", action="store_true",
                     help="c3/c5: start each batch's host-link feature read one batch ahead, on a side stream")
+    ap.add_argument("--no-batch-view", action="store_true",
+                    help="c3: batches come without the transposed view of their CSR, so every layer's "
+                         "backward builds one (the default: the loader emits it with the batch)")
     ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c2w", "c4", "c3", "c3b", "c5", "sample", "layer", "copy", "ceilings"])
     ap.add_argument("--heads", type=int, default=1, help="c2w: heads of the weighted aggregation (divides 256)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
@@ -591,7 +594,9 @@ def run_c3(args):
     samples = [direct_power_law_batch(N, n_seed, fanout, 2.0, 30 + i, degree_scale=2.6) for i in range(n_pre)]
     batches = []
     for smp in samples:
-        batches.append(make_batch(smp, labels, dev))
+        # a batch comes with the transposed view of its CSR, as the loader emits it (--no-batch-view: every
+        # layer's backward builds its own)
+        batches.append(make_batch(smp, labels, dev, emit_view=not args.no_batch_view))
     ev = {k: KernelClock() for k in ("load", "forward", "backward", "step", "update")}
     state = {"it": 0}
     sampled = {"sampler": None, "pending": None, "shapes": [], "wait_s": 0.0, "E_graph": 0}
@@ -601,7 +606,8 @@ def run_c3(args):
         from hiscache import NeighborSampler
         indptr, indices = device_power_law_graph(N, 14.5, dev, gen)
         sampled["E_graph"] = indices.numel()
-        sampled["sampler"] = NeighborSampler(indptr, indices, fanout, seed=3, device=dev, validate=False)
+        sampled["sampler"] = NeighborSampler(indptr, indices, fanout, seed=3, device=dev, validate=False,
+                                             emit_view=not args.no_batch_view)
         del indptr, indices
         seed_pool = torch.randperm(N, device=dev, generator=gen)[: n_seed * 1024].view(1024, n_seed).contiguous()
         sampled["pending"] = sampled["sampler"].sample_async(seed_pool[0])
@@ -667,6 +673,7 @@ def run_c3(args):
                                "pinned host pool of %d rows read zero-copy; mean batch %s" % (N, N, pool_rows, shape)},
         "phases_ms": {k: c.mean_ms() for k, c in ev.items()},
         "phases_host_enqueue_ms": {k: c.mean_cpu_ms() for k, c in ev.items()},
+        "transposed_view": "built in backward" if args.no_batch_view else "emitted with the batch",
         "feature_rows_read_last_batch": int(cache.used_masks[0].sum()),
         "cached_1hop_fraction_last_batch": float((cache.sub2embed != -1).float().mean()),
         "batched_history_layer": batched["detail"],

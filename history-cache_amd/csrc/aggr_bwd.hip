@@ -86,23 +86,25 @@ __device__ __forceinline__ void bwd_accumulate(const int64_t *__restrict__ ptr, 
       my_row = bwd_live_row<MASKED>(rowT[base + lane], hmap, R);
       if (!MASKED || my_row >= 0) my_deg = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
     }
-    for (int j = 0; j < n; j += UNROLL) {
+    // the staged edges that count, lowest position first (all of them without a mask)
+    unsigned long long todo = MASKED ? __ballot(lane < n && my_row >= 0)
+                                     : (n == HC_WAVE ? ~0ull : ((1ull << n) - 1ull));
+    while (todo != 0ull) {
       float v[UNROLL][CHUNKS][VEC];
       float d[UNROLL];
       bool on[UNROLL];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         d[u] = 1.0f;
-        on[u] = false;
-        if (j + u < n) {
-          const int r = __builtin_amdgcn_readlane(my_row, j + u);
-          on[u] = !MASKED || r >= 0;
-          if (on[u]) {
-            d[u] = hc_readlane_f(my_deg, j + u);
-            const float *p = g + (int64_t)r * F + lane * VEC;
+        on[u] = todo != 0ull;
+        if (on[u]) {
+          const int j = __builtin_ctzll(todo);
+          todo &= todo - 1ull;
+          const int r = __builtin_amdgcn_readlane(my_row, j);
+          d[u] = hc_readlane_f(my_deg, j);
+          const float *p = g + (int64_t)r * F + lane * VEC;
 #pragma unroll
-            for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
-          }
+          for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
         }
       }
 #pragma unroll
@@ -313,35 +315,44 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
       else if constexpr (WMODE == W_EDGE) my_deg = ev[edgeT[base + lane]];   // the weight takes the divisor's place
       else if (!MASKED || my_row >= 0) my_deg = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
     }
-    for (int j = 0; j < n; j += UNROLL) {
+    // MASKED: only the live edges of the stage are visited (lowest position first), so that UNROLL rows are
+    // in flight however many edges of other layers lie between them
+    unsigned long long todo = 0ull;
+    if constexpr (MASKED) todo = __ballot(lane < n && my_row >= 0);
+    for (int j = 0; MASKED ? todo != 0ull : j < n; j += UNROLL) {
       float v[UNROLL][CHUNKS][VEC];
       float d[UNROLL];
       bool on[UNROLL];
+      int pos[UNROLL];
       float wh[WMODE == W_EDGE_HEAD ? UNROLL : 1][CHUNKS];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         d[u] = 1.0f;
-        on[u] = false;
-        if (j + u < n) {
-          const int r = __builtin_amdgcn_readlane(my_row, j + u);
-          on[u] = !MASKED || r >= 0;
-          if (on[u]) {
-            d[u] = hc_readlane_f(my_deg, j + u);
-            const float *p = g + (int64_t)r * F + lane * VEC;
+        if constexpr (MASKED) {
+          on[u] = todo != 0ull;
+          pos[u] = on[u] ? __builtin_ctzll(todo) : 0;
+          todo &= todo - 1ull;                     // 0 stays 0
+        } else {
+          on[u] = j + u < n;
+          pos[u] = j + u;
+        }
+        if (on[u]) {
+          const int r = __builtin_amdgcn_readlane(my_row, pos[u]);
+          d[u] = hc_readlane_f(my_deg, pos[u]);
+          const float *p = g + (int64_t)r * F + lane * VEC;
 #pragma unroll
-            for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
-            if constexpr (WMODE == W_EDGE_HEAD) {
-              const int64_t e = (int64_t)__builtin_amdgcn_readlane(my_edge, j + u) * n_head;
+          for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
+          if constexpr (WMODE == W_EDGE_HEAD) {
+            const int64_t e = (int64_t)__builtin_amdgcn_readlane(my_edge, pos[u]) * n_head;
 #pragma unroll
-              for (int k = 0; k < CHUNKS; ++k) wh[u][k] = ev[e + hd[k]];
-            }
+            for (int k = 0; k < CHUNKS; ++k) wh[u][k] = ev[e + hd[k]];
           }
         }
       }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
-        if (j + u < n) {
-          const int64_t e = base + j + u;
+        if (on[u]) {
+          const int64_t e = base + pos[u];
           while (e >= cur_end) {  // close finished (possibly empty) segments; none of them is a hub
 #pragma unroll
             for (int k = 0; k < CHUNKS; ++k) {
@@ -352,15 +363,13 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
             ++cur;
             cur_end = hc_readlane64(my_p, cur + 1);
           }
-          if (on[u]) {
 #pragma unroll
-            for (int k = 0; k < CHUNKS; ++k)
+          for (int k = 0; k < CHUNKS; ++k)
 #pragma unroll
-              for (int i = 0; i < VEC; ++i) {
-                if constexpr (WMODE == W_EDGE_HEAD) acc[k][i] += __fmul_rn(v[u][k][i], wh[u][k]);
-                else acc[k][i] += WEIGHTED ? __fmul_rn(v[u][k][i], d[u]) : v[u][k][i] / d[u];
-              }
-          }
+            for (int i = 0; i < VEC; ++i) {
+              if constexpr (WMODE == W_EDGE_HEAD) acc[k][i] += __fmul_rn(v[u][k][i], wh[u][k]);
+              else acc[k][i] += WEIGHTED ? __fmul_rn(v[u][k][i], d[u]) : v[u][k][i] / d[u];
+            }
         }
       }
     }

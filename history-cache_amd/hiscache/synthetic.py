@@ -91,8 +91,20 @@ def sample_layered_batch(indptr, indices, seeds, fanout, rng):
     }
 
 
-def make_batch(sample, labels, device):
-    """Wrap a sampled sub-graph as the batch object the cache and the model read."""
+def make_batch(sample, labels, device, emit_view=False):
+    """Wrap a sampled sub-graph as the batch object the cache and the model read.  ``emit_view``: the
+    batch also carries the transposed view of its CSR (``batch.view``), as a loader that prepares
+    batches ahead of the training step emits it (``NeighborSampler(emit_view=True)`` does)."""
+    batch = _make_batch(sample, labels, device)
+    if emit_view and torch.device(device).type == "cuda":
+        import hiscache_backend
+        L = len(sample["num_node_in_layer"]) - 1
+        nnl = sample["num_node_in_layer"]
+        batch.view = hiscache_backend.build_batch_view(batch.ptr, batch.idx, int(nnl[L - 1]), int(nnl[L]))
+    return batch
+
+
+def _make_batch(sample, labels, device):
     n_seed = int(sample["num_node_in_layer"][0])
     L = len(sample["num_node_in_layer"]) - 1
     ptr = sample["ptr"]
@@ -108,6 +120,7 @@ def make_batch(sample, labels, device):
         x=None,
         edge_type=None,
         typed_num_node_in_layer=None,
+        view=None,
     )
 
 

@@ -17,7 +17,10 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def test_c3_iteration_matches_cpu(orc):
+@pytest.mark.parametrize("emit_view", [False, True])
+def test_c3_iteration_matches_cpu(orc, emit_view, monkeypatch):
+    """``emit_view``: the sampler hands the batch over together with the transposed view of its CSR and
+    the layers' backward builds none (the call is made to fail inside backward)."""
     from hiscache import HistorySAGE, NeighborSampler, PinnedFeatureStore, RingHistoryCache, make_config
     from hiscache.synthetic import make_batch
     from oracle import host_model
@@ -41,7 +44,7 @@ def test_c3_iteration_matches_cpu(orc):
     ref["checkin"][: len(cached)] = 0
 
     # --- sampling: device sampler against the sequential statement
-    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=3, device=DEV)
+    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=3, device=DEV, emit_view=emit_view)
     seeds = rng.choice(N, size=n_seed, replace=False).astype(np.int64)
     batch = sampler.sample(torch.from_numpy(seeds).to(DEV))
     b = orc.sample_layers(indptr, indices, seeds, fanout, sampler.batch_seed(0))
@@ -79,7 +82,15 @@ def test_c3_iteration_matches_cpu(orc):
     out = model(batch)
     hook.remove()
     loss = torch.nn.functional.nll_loss(out, batch.y)
+    assert (batch.view is not None) == emit_view
+    if emit_view:
+        import hiscache_backend
+
+        def no_view_in_backward(*a, **k):
+            raise AssertionError("a transposed view was built inside backward")
+        monkeypatch.setattr(hiscache_backend, "build_transpose", no_view_in_backward)
     loss.backward()
+    monkeypatch.undo()
     pe = cache.produced_embedding
     assert tuple(pe.shape) == (n1, H)
     # the history layer's output from the GPU's own layer-1 activations, bit for bit

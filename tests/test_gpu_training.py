@@ -40,12 +40,15 @@ def test_training_reduces_the_loss(kind):
         model = HistoryRGCN(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache, num_rel=3).to(DEV)
     model.train()
     opt = torch.optim.Adam(model.parameters(), lr=0.01)
-    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=1, device=DEV)
+    # batches are sampled one ahead on the sampler's stream and come with the transposed view of their CSR
+    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=1, device=DEV, emit_view=True)
     gen = torch.Generator(device=DEV).manual_seed(3)
     losses, hits = [], []
+    pending = sampler.sample_async(torch.randperm(N, device=DEV, generator=gen)[:256])
     for it in range(1, 91):
-        seeds = torch.randperm(N, device=DEV, generator=gen)[:256]
-        batch = sampler.sample(seeds)
+        batch = pending.get()
+        pending = sampler.sample_async(torch.randperm(N, device=DEV, generator=gen)[:256])
+        assert batch.view is not None and batch.view.num_edge == batch.idx.numel()
         if kind == "rgcn":
             batch.edge_type = (batch.idx % 3).contiguous()
         cache.lookup_and_load(batch, L)
@@ -56,6 +59,7 @@ def test_training_reduces_the_loss(kind):
         opt.step()
         cache.update_history(batch, it)
         losses.append(float(loss.detach()))
+    pending.get()
     assert all(np.isfinite(losses))
     first, last = float(np.mean(losses[:10])), float(np.mean(losses[-10:]))
     assert last < 0.7 * first, (first, last)
