@@ -760,6 +760,82 @@ int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, co
   return hc_launch_status();
 }
 
+// ---------------------------------------------------------------------------------------
+// Relational layer over the mini-batch's shared view.  The layer's forward sums, for every (row, relation)
+// group, x[src] * (1 / deg(row)) over the group's kept edges; here source s collects
+// g[row * K + rel(e), :] * (1 / deg(row)) over its kept edges in ascending (row, edge slot) order: the order
+// of the batch view, so that no view of the regrouped block has to be built.  An edge is kept under
+// hc_typed_csr's rule: row < R, slot < E, relation in [0, K), source flagged in `used` (when given).
+// One wave per source; up to UNROLL gradient rows in flight; products rounded, then added in order.
+// ---------------------------------------------------------------------------------------
+template <int VEC, int CHUNKS, int UNROLL>
+__global__ __launch_bounds__(HC_BLOCK) void bwd_typed_batch_view(
+    const int64_t *__restrict__ ptr, const int64_t *__restrict__ ptrT, const int32_t *__restrict__ rowT,
+    const int32_t *__restrict__ edgeT, const int64_t *__restrict__ et, const uint8_t *__restrict__ used,
+    const float *__restrict__ g, float *__restrict__ grad_vin, int64_t R, int64_t E, int K, int64_t n_src) {
+  constexpr int F = HC_WAVE * VEC * CHUNKS;
+  const int lane = hc_lane();
+  const int64_t s = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
+  if (s >= n_src) return;
+  float acc[CHUNKS][VEC];
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[k][i] = 0.0f;
+  const bool src_kept = used == nullptr || used[s] != 0;
+  const int64_t begin = src_kept ? ptrT[s] : 0;
+  const int64_t end = src_kept ? ptrT[s + 1] : 0;
+  for (int64_t base = begin; base < end; base += HC_WAVE) {
+    const int64_t left = end - base;
+    const int n = left < HC_WAVE ? (int)left : HC_WAVE;
+    int64_t my_group = -1;
+    float my_w = 0.0f;
+    if (lane < n) {
+      const int64_t row = rowT[base + lane];
+      const int64_t e = edgeT[base + lane];
+      if (row < R && e < E) {
+        const int64_t rel = et[e];
+        if (rel >= 0 && rel < K) {
+          my_group = row * K + rel;
+          const int64_t d = ptr[row + 1] - ptr[row];
+          my_w = 1.0f / (float)(d > 0 ? d : 1);
+        }
+      }
+    }
+    unsigned long long todo = __ballot(my_group >= 0);
+    while (todo != 0ull) {
+      float v[UNROLL][CHUNKS][VEC];
+      float w[UNROLL];
+      bool on[UNROLL];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        w[u] = 0.0f;
+        on[u] = todo != 0ull;
+        if (on[u]) {
+          const int j = __builtin_ctzll(todo);
+          todo &= todo - 1ull;
+          w[u] = hc_readlane_f(my_w, j);
+          const float *p = g + hc_readlane64(my_group, j) * F + lane * VEC;
+#pragma unroll
+          for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::load(p + k * HC_WAVE * VEC, v[u][k]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        if (on[u]) {
+#pragma unroll
+          for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[k][i] += __fmul_rn(v[u][k][i], w[u]);
+        }
+      }
+    }
+  }
+  float *__restrict__ o = grad_vin + s * F + lane * VEC;
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store(o + k * HC_WAVE * VEC, acc[k]);
+}
+
 bool bwd_fast_shape(int64_t F) {
   return F == 64 || F == 128 || F == 192 || F == 256 || F == 384 || F == 512 || F == 768 || F == 1024;
 }
@@ -938,4 +1014,32 @@ extern "C" int hc_aggr_bwd_batch_view(const int64_t *ptr, const int64_t *ptrT, c
                                       int64_t n_src, void *workspace, size_t workspace_bytes, void *stream) {
   return aggr_bwd_impl(ptr, nullptr, ptrT, rowT, nullptr, g, hmap, nullptr, nullptr, 0, 1, grad_vin, grad_hbuf,
                        hsize, nullptr, E_view, R, F, n_src, workspace, workspace_bytes, true, stream);
+}
+
+extern "C" int hc_aggr_bwd_batch_view_typed(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT,
+                                            const int32_t *edgeT, const int64_t *edge_types, int64_t E,
+                                            int num_rel, const uint8_t *used_mask, const float *g,
+                                            float *grad_vin, int64_t R, int64_t F, int64_t n_src, void *stream) {
+  HC_REQUIRE(R >= 0 && F > 0 && n_src >= 0 && E >= 0 && num_rel >= 1);
+  HC_REQUIRE(ptr && ptrT && g && edge_types);
+  HC_REQUIRE(grad_vin || n_src == 0);
+  HC_REQUIRE((rowT && edgeT) || n_src == 0);
+  if (R > 0x7ffffffeLL / num_rel) return HC_EUNSUPPORTED;
+  if (!bwd_fast_shape(F)) return HC_EUNSUPPORTED;
+  if (reinterpret_cast<uintptr_t>(g) % 16 != 0 || reinterpret_cast<uintptr_t>(grad_vin) % 16 != 0)
+    return HC_EUNSUPPORTED;
+  if (n_src == 0) return HC_OK;
+  const int64_t nb = (n_src + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  if (!hc_grid_ok(nb)) return HC_EUNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)nb), block(HC_BLOCK);
+#define HC_TYPED(V, C)                                                                                  \
+  if (F == 64 * (V) * (C))                                                                              \
+    bwd_typed_batch_view<V, C, ((V) * (C) >= 16 ? 4 : 8)><<<grid, block, 0, st>>>(                      \
+        ptr, ptrT, rowT, edgeT, edge_types, used_mask, g, grad_vin, R, E, num_rel, n_src);              \
+  else
+  HC_TYPED(4, 1) HC_TYPED(4, 2) HC_TYPED(4, 3) HC_TYPED(4, 4) HC_TYPED(2, 1) HC_TYPED(2, 3) HC_TYPED(1, 1)
+  HC_TYPED(1, 3) return HC_EUNSUPPORTED;
+#undef HC_TYPED
+  return hc_launch_status();
 }

@@ -359,7 +359,7 @@ class _RgcnConvFunction(torch.autograd.Function):
     the weighted aggregation's transposed view."""
 
     @staticmethod
-    def forward(ctx, x, weight, ptr, idx, edge_types, used_mask, hmap, hbuf, num_node):
+    def forward(ctx, x, weight, ptr, idx, edge_types, used_mask, hmap, hbuf, num_node, view=None):
         be = hiscache_backend
         R = int(num_node)
         K, Fin, H = weight.shape
@@ -373,6 +373,9 @@ class _RgcnConvFunction(torch.autograd.Function):
             out = torch.where(hit, hbuf[:R].to(out.dtype), out)
         ctx.save_for_backward(x, agg, weight, ptr2, idx2, w2, hit if hit is not None else x.new_empty(0))
         ctx.hc = (R, hit is not None, min(int(edge_types.numel()), int(idx.numel())))
+        # the batch's shared transposed view (with edge slots) serves backward directly
+        ctx.shared = (ptr, edge_types, used_mask, view) if be.typed_batch_view_supported(
+            view, R, x.shape[0], Fin) else None
         return out
 
     @staticmethod
@@ -389,12 +392,16 @@ class _RgcnConvFunction(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             g_agg = (g @ weight.reshape(K * Fin, H).t()).view(R * K, Fin)
             n_src = x.shape[0]
-            tr = be.build_transpose(ptr2, idx2, None, R * K, n_src, num_edge=E, want_edges=True)
-            g_x, _, _ = be._aggr_bwd(ptr2, idx2, tr, g_agg, None, w2, x, False, None, 0, R * K, n_src,
-                                     want_hist_grad=False)
+            if ctx.shared is not None:
+                ptr, edge_types, used_mask, view = ctx.shared
+                g_x = be._aggr_bwd_typed_batch_view(ptr, view, edge_types, K, used_mask, g_agg, R, n_src)
+            else:
+                tr = be.build_transpose(ptr2, idx2, None, R * K, n_src, num_edge=E, want_edges=True)
+                g_x, _, _ = be._aggr_bwd(ptr2, idx2, tr, g_agg, None, w2, x, False, None, 0, R * K, n_src,
+                                         want_hist_grad=False)
             if g_x.dtype != x.dtype:
                 g_x = g_x.to(x.dtype)
-        return g_x, g_w, None, None, None, None, None, None, None
+        return g_x, g_w, None, None, None, None, None, None, None, None
 
 
 class MyRGCNConvHistory2(torch.nn.Module):
@@ -432,7 +439,7 @@ class MyRGCNConvHistory2(torch.nn.Module):
         return hiscache_backend.count_num(self._count_of, self.num_rel)
 
     def forward(self, x, ptr, idx, edge_types, count, history_map, history_buffer, used_mask, history_size,
-                num_node):
+                num_node, view=None):
         num_node = int(num_node)
         K = self.num_rel
         edge_types = edge_types.to(torch.int64).contiguous()
@@ -441,7 +448,7 @@ class MyRGCNConvHistory2(torch.nn.Module):
         if self.fused and x.is_cuda and not (use_hist and history_buffer.requires_grad):
             out = _RgcnConvFunction.apply(x, self.linear, ptr, idx, edge_types, used_mask,
                                           history_map if use_hist else None,
-                                          history_buffer if use_hist else None, num_node)
+                                          history_buffer if use_hist else None, num_node, view)
             his = out
             if self.need_grad and self.training and history_size > 0:
                 his.retain_grad()
@@ -520,22 +527,23 @@ class HistoryRGCN(torch.nn.Module):
         etypes = self.edge_types(batch)
         none = torch.empty(0, device=x.device)
         masks = self.table.used_masks
+        view = getattr(batch, "view", None)                  # shared transposed view, if the loader emitted it
         for i, conv in enumerate(self.convs[:-1]):
             n = batch.num_node_in_layer[L - 1 - i]
             et = etypes[: batch.num_edge_in_layer[L - 1 - i]]
             um = masks[i] if masks is not None else None
             if self.training and i == L - 2:
                 x, his = conv(x, batch.ptr, batch.idx, et, None, self.table.sub2embed,
-                              self.table.cached_embedding, um, self.hidden_channels, n)
+                              self.table.cached_embedding, um, self.hidden_channels, n, view=view)
                 self.table.produced_embedding = his
                 self.table.produced_embedding.retain_grad()
             else:
-                x, his = conv(x, batch.ptr, batch.idx, et, None, none, none, um, 0, n)
+                x, his = conv(x, batch.ptr, batch.idx, et, None, none, none, um, 0, n, view=view)
             x = bn_relu(x, self.bns[i], None, fused=self.fused_epilogue)
             x = F.dropout(x, p=self.dropout, training=self.training)
         um = masks[-2] if masks is not None else None
         x, his = self.convs[-1](x, batch.ptr, batch.idx, etypes[: batch.num_edge_in_layer[0]], None, none, none,
-                                um, 0, batch.num_node_in_layer[0])
+                                um, 0, batch.num_node_in_layer[0], view=view)
         return x.log_softmax(dim=-1)
 
     def reset_parameters(self):

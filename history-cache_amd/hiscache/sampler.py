@@ -18,13 +18,15 @@ import hiscache_backend as _be
 class NeighborSampler:
 
     def __init__(self, indptr, indices, fanout, labels=None, seed=0, device="cuda:0", validate=True,
-                 emit_view=False):
+                 emit_view=False, view_edges=False):
         """``indptr`` / ``indices``: CSR of the full graph (int64; moved to ``device``).  ``fanout[k]``
         neighbours are drawn, without replacement, for nodes first reached at hop k.  ``emit_view``:
         every batch also carries ``batch.view``, the transposed view of its CSR
         (``hiscache_backend.BatchView``), built right behind the sampling on the sampler's stream, so
-        that the layers' backward builds none."""
+        that the layers' backward builds none; ``view_edges`` adds the view's edge slots, which the
+        relational layer's backward reads."""
         self.emit_view = bool(emit_view)
+        self.view_edges = bool(view_edges)
         self.device = torch.device(device)
         self.indptr = torch.as_tensor(indptr, dtype=torch.int64).to(self.device).contiguous()
         self.indices = torch.as_tensor(indices, dtype=torch.int64).to(self.device).contiguous()
@@ -69,7 +71,7 @@ class NeighborSampler:
             stream.wait_stream(cur)                                    # seeds may have been produced there
         with torch.cuda.stream(stream):
             out = _be.sample_layers(self.indptr, self.indices, seeds, self.fanout, rng_seed, self.node_map,
-                                    emit_view=self.emit_view)
+                                    emit_view=self.emit_view, view_edges=self.view_edges)
             counts_host = self._host_pool.pop() if self._host_pool else torch.empty(
                 2 * len(self.fanout) + 1, dtype=torch.int64, pin_memory=True)
             counts_host.copy_(out[3], non_blocking=True)
@@ -87,8 +89,10 @@ class NeighborSampler:
         cur = torch.cuda.current_stream(self.device)
         view = None
         if self.emit_view:
-            ptrT, rowT = out[4], out[5]
-            view = _be.BatchView(ptrT[: nnl[L] + 1], rowT[: max(nel[-1], 1)], None, nnl[L - 1], nnl[L], nel[-1])
+            ptrT, rowT, edgeT = out[4], out[5], out[6]
+            n_e = max(nel[-1], 1)
+            view = _be.BatchView(ptrT[: nnl[L] + 1], rowT[:n_e], None if edgeT is None else edgeT[:n_e],
+                                 nnl[L - 1], nnl[L], nel[-1])
         if stream != cur:
             for t in (ptr, idx, s2f, seeds) + (() if y is None else (y,)):
                 t.record_stream(cur)

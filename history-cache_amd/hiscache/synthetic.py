@@ -91,16 +91,18 @@ def sample_layered_batch(indptr, indices, seeds, fanout, rng):
     }
 
 
-def make_batch(sample, labels, device, emit_view=False):
+def make_batch(sample, labels, device, emit_view=False, view_edges=False):
     """Wrap a sampled sub-graph as the batch object the cache and the model read.  ``emit_view``: the
     batch also carries the transposed view of its CSR (``batch.view``), as a loader that prepares
-    batches ahead of the training step emits it (``NeighborSampler(emit_view=True)`` does)."""
+    batches ahead of the training step emits it (``NeighborSampler(emit_view=True)`` does); ``view_edges``
+    adds the view's edge slots (read by the relational layer's backward)."""
     batch = _make_batch(sample, labels, device)
     if emit_view and torch.device(device).type == "cuda":
         import hiscache_backend
         L = len(sample["num_node_in_layer"]) - 1
         nnl = sample["num_node_in_layer"]
-        batch.view = hiscache_backend.build_batch_view(batch.ptr, batch.idx, int(nnl[L - 1]), int(nnl[L]))
+        batch.view = hiscache_backend.build_batch_view(batch.ptr, batch.idx, int(nnl[L - 1]), int(nnl[L]),
+                                                       want_edges=view_edges)
     return batch
 
 

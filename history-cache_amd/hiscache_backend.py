@@ -64,6 +64,8 @@ _SIGNATURES = {
                              _c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]),
     "hc_aggr_bwd_batch_view": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_i64,
                                         _c_i64, _c_p, _c_sz, _c_p]),
+    "hc_aggr_bwd_batch_view_typed": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_i64,
+                                              _c_i64, _c_i64, _c_p]),
     "hc_count_history": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p]),
     "hc_row_scores": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_int, _c_p]),
     "hc_grad_check_workspace_bytes": (_c_sz, [_c_i64]),
@@ -401,6 +403,36 @@ def _aggr_bwd_batch_view(ptr, view, g, hmap, hbuf_shape, hsize, num_node, n_src,
                                     _ptr(ws), ws.numel() if ws is not None else 0, _stream())
     _check(rc, "hc_aggr_bwd_batch_view")
     return grad_x, grad_h
+
+
+def typed_batch_view_supported(view, num_node, n_src, feature_width):
+    """Can ``_aggr_bwd_typed_batch_view`` serve this layer (view with edge slots that covers it, fast width)?"""
+    return (view is not None and view.edgeT is not None and view.covers(num_node, n_src)
+            and bwd_chunk_edges(feature_width) > 0)
+
+
+def _aggr_bwd_typed_batch_view(ptr, view, edge_types, num_rel, used_mask, g, num_node, n_src):
+    """Input gradient of the relational layer over the batch's shared view: g is the gradient of the
+    (row, relation) groups' sums, [num_node * num_rel, F]."""
+    lib = load_library()
+    g = _dev(g.contiguous(), "grad_output", torch.float32)
+    _dev(edge_types, "edge_types", torch.int64)
+    R, K, F = int(num_node), int(num_rel), g.shape[-1]
+    if g.dim() != 2 or g.shape[0] < R * K:
+        raise ValueError("grad_output must be [num_node * num_rel, F]")
+    if not view.covers(R, n_src) or view.edgeT is None:
+        raise ValueError("the batch view does not cover this layer, or was built without edge slots")
+    if used_mask is not None:
+        used_mask = _dev(used_mask, "used_mask")
+        if used_mask.element_size() != 1 or used_mask.numel() < n_src:
+            raise ValueError("used_mask must hold one byte per source")
+    E = min(int(edge_types.numel()), view.num_edge)
+    grad_x = torch.empty((int(n_src), F), dtype=torch.float32, device=g.device)
+    rc = lib.hc_aggr_bwd_batch_view_typed(_ptr(ptr), _ptr(view.ptrT), _ptr(view.rowT), _ptr(view.edgeT),
+                                          _ptr(edge_types), E, K, _ptr(used_mask), _ptr(g), _ptr(grad_x), R, F,
+                                          int(n_src), _stream())
+    _check(rc, "hc_aggr_bwd_batch_view_typed")
+    return grad_x
 
 
 class _AggrHistory(torch.autograd.Function):
@@ -1049,16 +1081,17 @@ def build_transpose_dev(ptr, idx, rows_dev, edges_dev, nodes_dev, max_edges, max
     return ptrT, rowT, edgeT
 
 
-def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map, emit_view=False):
+def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map, emit_view=False, view_edges=False):
     """Layered neighbour sampling without replacement.  Returns (ptr, idx, sub_to_full, counts) as
     device tensors at their capacity; ``counts`` (int64[2L+1] on the device) holds the node count
     within k hops for k = 0..L and then the cumulative edge count after every hop, so the caller
     slices ptr[:counts[L-1]+1], idx[:counts[2L]], sub_to_full[:counts[L]] once it has read them.
     ``seeds`` must be distinct valid node ids; ``node_map`` comes from ``sample_map`` and is left
     all-unseen again.  Stands where the reference's external loader does
-    (/root/reference/hiscache/history_trainer.py:19,26).  ``emit_view=True`` appends (ptrT, rowT): the
-    transposed view of the whole sampled CSR, built behind the sampling with the sizes still on the
-    device (``build_transpose_dev``), for ``BatchView`` once the caller has read ``counts``."""
+    (/root/reference/hiscache/history_trainer.py:19,26).  ``emit_view=True`` appends (ptrT, rowT, edgeT):
+    the transposed view of the whole sampled CSR, built behind the sampling with the sizes still on the
+    device (``build_transpose_dev``), for ``BatchView`` once the caller has read ``counts``; edgeT is
+    None unless ``view_edges`` (the relational layer's backward reads it)."""
     lib = load_library()
     _dev(indptr, "indptr", torch.int64)
     _dev(indices, "indices", torch.int64)
@@ -1087,9 +1120,9 @@ def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map, emit_view=
                               _ptr(idx), _ptr(s2f), _ptr(counts), _ptr(ws), ws_bytes, _stream())
     _check(rc, "hc_sample_layers")
     if emit_view:
-        ptrT, rowT, _ = build_transpose_dev(ptr, idx, counts[L - 1:L], counts[2 * L:2 * L + 1], counts[L:L + 1],
-                                            edges, nodes)
-        return ptr, idx, s2f, counts, ptrT, rowT
+        ptrT, rowT, edgeT = build_transpose_dev(ptr, idx, counts[L - 1:L], counts[2 * L:2 * L + 1],
+                                                counts[L:L + 1], edges, nodes, want_edges=view_edges)
+        return ptr, idx, s2f, counts, ptrT, rowT, edgeT
     return ptr, idx, s2f, counts
 
 

@@ -209,6 +209,25 @@ int hc_aggr_bwd_batch_view(const int64_t *ptr, const int64_t *ptrT, const int32_
                            int64_t hsize, int64_t E_view, int64_t R, int64_t F, int64_t n_src,
                            void *workspace, size_t workspace_bytes, void *stream);
 
+/* hc_aggr_bwd_batch_view_typed: the input gradient of the relational layer
+ * (hiscache/history_model.py:220-278; forward: hc_typed_csr, then hc_aggr_fwd
+ * with its 1/deg edge weights over the (row, relation) groups) over the batch's
+ * shared view, which must carry edgeT.  g is [R*num_rel, F]: the gradient of
+ * the groups' sums.  For every source s
+ *   grad_vin[s,:] = sum over its kept edges e (row r, relation k = edge_types[e])
+ *                   of g[r*num_rel + k, :] * (1 / deg(r))
+ * in ascending (row, edge slot) order, product rounded, then added.  Kept as in
+ * hc_typed_csr: r < R, e < E, k in [0, num_rel), used_mask (n_src bytes,
+ * nullable) != 0 for s; deg(r) = ptr[r+1] - ptr[r].  Sources without kept edges
+ * get 0.  F must be one of the fast widths (64, 128, 192, 256, 384, 512, 768,
+ * 1024), else HC_EUNSUPPORTED.  (The order differs from hc_aggr_bwd over a view
+ * of the regrouped block only where parallel edges of one (source, row) pair
+ * carry different relations.) */
+int hc_aggr_bwd_batch_view_typed(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT,
+                                 const int32_t *edgeT, const int64_t *edge_types, int64_t E,
+                                 int num_rel, const uint8_t *used_mask, const float *g,
+                                 float *grad_vin, int64_t R, int64_t F, int64_t n_src, void *stream);
+
 /* ---------------------------------------------------------------- used masks
  * Replaces count_history_reconstruct (src/cpp/include/grad_check.h:18-20,
  * src/cpp/src/grad_check.cu:70-130).  masks is (num_layer+1) x n_all bytes

@@ -705,6 +705,34 @@ int orc_typed_csr(const Index *ptr, const Index *idx, const Index *et, const uin
   return ORC_OK;
 }
 
+/* Input gradient of the relational layer in the order of hc_aggr_bwd_batch_view_typed: the forward
+ * (history_model.py:248-270 with the grouping of orc_typed_csr) gives edge e of row r the weight
+ * 1/deg(r) inside group r*K + et[e]; walking rows and edge slots in ascending order adds
+ * g[r*K + et[e], :] * (1/deg(r)) to the edge's source, product rounded first. */
+int orc_bwd_typed_batch_view(const Index *ptr, const Index *idx, const Index *et, const uint8_t *used,
+                             const float *g, float *grads_out, Index R, Index E, Index F, int K,
+                             Index n_src) {
+  if (K < 1 || R < 0) return ORC_EINVAL;
+  memset(grads_out, 0, (size_t)(n_src * F) * sizeof(float));
+  for (Index r = 0; r < R; ++r) {
+    Index begin = ptr[r], end = ptr[r + 1] < E ? ptr[r + 1] : E;
+    Index d = ptr[r + 1] - ptr[r];
+    float w = 1.0f / (float)(d > 0 ? d : 1);
+    for (Index e = begin; e < end; ++e) {
+      Index s = idx[e], k = et[e];
+      if (k < 0 || k >= K || s < 0 || s >= n_src) continue;
+      if (used && !used[s]) continue;
+      const float *gr = g + (r * K + k) * F;
+      float *o = grads_out + s * F;
+      for (Index c = 0; c < F; ++c) {
+        float prod = gr[c] * w;
+        o[c] += prod;
+      }
+    }
+  }
+  return ORC_OK;
+}
+
 /* get_graph_structure_score, grad_check.cu:132-163.  The reference reads and
  * writes `output` across warps inside one pass, so its result depends on
  * scheduling.  This is the level-synchronous reading of the same rule: pass

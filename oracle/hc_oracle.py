@@ -325,6 +325,21 @@ def typed_csr(ptr, idx, edge_types, num_rel, num_node, n_src, used_mask=None):
     return ptr2, idx2[:ptr2[-1]], cnt.reshape(R, K), deg
 
 
+def bwd_typed_batch_view(ptr, idx, edge_types, num_rel, g, n_src, used_mask=None):
+    """Input gradient of the relational layer, rows and edge slots walked in ascending order
+    (hc_aggr_bwd_batch_view_typed); g is [R * num_rel, F]."""
+    ptr, idx, et, g = _i64(ptr), _i64(idx), _i64(edge_types), _f32(g)
+    K = int(num_rel)
+    R, F = g.shape[0] // K, g.shape[1]
+    E = min(len(idx), len(et))
+    used = None if used_mask is None else np.ascontiguousarray(used_mask, dtype=np.uint8)
+    out = np.zeros((n_src, F), np.float32)
+    _check(lib().orc_bwd_typed_batch_view(_p(ptr), _p(idx), _p(et), _p(used) if used is not None else None,
+                                          _p(g), _p(out), _I(R), _I(E), _I(F), ctypes.c_int(K), _I(n_src)),
+           "bwd_typed_batch_view")
+    return out
+
+
 def typed_csr_weights(ptr2, deg, num_rel):
     """The edge weights hc_typed_csr writes beside idx2: fp32 1/deg of the edge's row (deg counts every
     edge of the row, kept or dropped)."""

@@ -193,3 +193,54 @@ def test_sampler_emits_the_view_with_the_batch(be, orc, fanout, n_seed):
         np.testing.assert_array_equal(want_rowT, o_rowT)
     assert int((emitting.node_map != 0x7fffffff).sum()) == 0
     del pending
+
+
+@pytest.mark.parametrize("F,K,with_mask", [(256, 5, True), (64, 3, False), (768, 2, True), (128, 1, False)])
+def test_relational_backward_over_the_batch_view_bit_exact(be, orc, F, K, with_mask):
+    """hc_aggr_bwd_batch_view_typed against the oracle: relations outside [0, K), a relation array shorter
+    than the edge list, sources ruled out by the used mask, a layer that owns a prefix of the view's rows,
+    a source with hundreds of edges."""
+    rng = np.random.default_rng(F + K)
+    rows, sources = [400, 3000], [3000, 5000]
+    ptr, idx = layered_csr(rng, rows, sources, 8, hubs={3: 700, 2999: 150})
+    R_all, n_all = rows[-1], sources[-1]
+    tptr, tidx = T(ptr), T(idx)
+    view = be.build_batch_view(tptr, tidx, R_all, n_all, want_edges=True)
+    for R, n_src in zip(rows, sources):
+        rel = rng.integers(-1, K + 1, size=int(ptr[R]) - 3).astype(np.int64)
+        used = (rng.random(n_src) < 0.8) if with_mask else None
+        g = rng.standard_normal((R * K, F)).astype(np.float32)
+        got = be._aggr_bwd_typed_batch_view(tptr, view, T(rel), K, None if used is None else T(used), T(g), R, n_src)
+        want = orc.bwd_typed_batch_view(ptr[:R + 1], idx, rel, K, g, n_src, used)
+        np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
+def test_relational_layer_with_and_without_the_batch_view(be):
+    """The fused relational layer gives the same bits whether backward reads the batch's view or builds the
+    view of its regrouped block (relations that follow from the edge's ends)."""
+    from hiscache.history_model import MyRGCNConvHistory2
+    rng = np.random.default_rng(8)
+    torch.manual_seed(8)
+    rows, sources = [300, 2500], [2500, 4000]
+    ptr, idx = layered_csr(rng, rows, sources, 9, hubs={1: 600})
+    K, Fin, H = 4, 256, 128
+    tptr, tidx = T(ptr), T(idx)
+    view = be.build_batch_view(tptr, tidx, rows[-1], sources[-1], want_edges=True)
+    conv = MyRGCNConvHistory2(Fin, H, K, need_grad=True).to(DEV)
+    R, n_src = rows[0], sources[0]
+    et = T(((idx * 5 + 1) % K)[: int(ptr[R])])
+    used = T(rng.random(n_src) < 0.85)
+    hmap = T(random_hmap(rng, R, 0.3))
+    hbuf = T(rng.standard_normal((R, H)).astype(np.float32))
+    x0 = rng.standard_normal((n_src, Fin)).astype(np.float32)
+    g = T(rng.standard_normal((R, H)).astype(np.float32))
+    res = []
+    for v in (None, view):
+        x = T(x0).requires_grad_(True)
+        conv.zero_grad()
+        out, _ = conv(x, tptr, tidx, et, None, hmap, hbuf, used, H, R, view=v)
+        out.backward(g)
+        res.append((out.detach(), x.grad, conv.linear.grad.clone()))
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+    assert float(res[1][1].abs().max()) > 0

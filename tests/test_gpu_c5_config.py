@@ -35,7 +35,10 @@ def rgcn_layer_fp64(x, W, ptr, idx, rel, used, n, hit=None, hbuf=None):
     return out
 
 
-def test_c5_iteration_matches_cpu(orc):
+@pytest.mark.parametrize("emit_view", [False, True])
+def test_c5_iteration_matches_cpu(orc, emit_view, monkeypatch):
+    """``emit_view``: the sampler hands the batch over together with the transposed view of its CSR (with
+    edge slots) and the relational layer's backward builds none (the call is made to fail inside backward)."""
     from hiscache import HistoryRGCN, NeighborSampler, PinnedFeatureStore, RingHistoryCache, make_config
     from oracle import host_model
     n_paper, n_author, n_inst = 150_000, 147_000, 3_000
@@ -61,7 +64,8 @@ def test_c5_iteration_matches_cpu(orc):
     ref["checkin"][: len(cached)] = 0
 
     # --- sampling
-    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=5, device=DEV)
+    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=5, device=DEV, emit_view=emit_view,
+                              view_edges=True)
     seeds = rng.choice(n_paper, size=n_seed, replace=False).astype(np.int64)        # seeds are papers
     batch = sampler.sample(torch.from_numpy(seeds).to(DEV))
     b = orc.sample_layers(indptr, indices, seeds, fanout, sampler.batch_seed(0))
@@ -110,7 +114,13 @@ def test_c5_iteration_matches_cpu(orc):
     # --- model forward / backward against the dense fp64 statement
     out = model(batch)
     loss = torch.nn.functional.nll_loss(out, batch.y)
+    assert (batch.view is not None) == emit_view
+    if emit_view:
+        def no_view_in_backward(*a, **k):
+            raise AssertionError("a transposed view was built inside backward")
+        monkeypatch.setattr(be, "build_transpose", no_view_in_backward)
     loss.backward()
+    monkeypatch.undo()
     np.testing.assert_array_equal(model.convs[0].last_count.cpu().numpy(), orc.count_num(want_et[:e1], K))
     ptr, idx = torch.from_numpy(b["ptr"]), torch.from_numpy(b["idx"])
     rel = torch.from_numpy(want_et)

@@ -41,7 +41,8 @@ def test_training_reduces_the_loss(kind):
     model.train()
     opt = torch.optim.Adam(model.parameters(), lr=0.01)
     # batches are sampled one ahead on the sampler's stream and come with the transposed view of their CSR
-    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=1, device=DEV, emit_view=True)
+    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=1, device=DEV, emit_view=True,
+                              view_edges=kind == "rgcn")
     gen = torch.Generator(device=DEV).manual_seed(3)
     losses, hits = [], []
     pending = sampler.sample_async(torch.randperm(N, device=DEV, generator=gen)[:256])

@@ -616,6 +616,44 @@ def test_typed_csr_equals_stable_sort(orc, K, with_mask, short_types):
         assert abs(got_mean - want_mean) <= 1e-5 * (abs(want_mean) + 1.0)
 
 
+@pytest.mark.parametrize("K,with_mask,by_source", [(5, True, True), (3, False, False), (1, False, True)])
+def test_relational_input_gradient_over_the_batch_view(orc, K, with_mask, by_source):
+    """bwd_typed_batch_view: the relational layer's input gradient with rows and edge slots walked in
+    ascending order.  Pinned by the dense closed form in fp64 and, where the relation is a function of the
+    edge's ends (parallel edges then share it), bit for bit by the weighted backward over the regrouped
+    block (orc.typed_csr + orc.bwd_edge_value), which is the per-layer path's order."""
+    from helpers import random_csr
+    rng = np.random.default_rng(90 + K)
+    R, N, F = 70, 40, 6
+    ptr, idx = random_csr(rng, R + 20, N, 30, hub=90)
+    idx = idx.copy()
+    idx[rng.random(len(idx)) < 0.03] = N + 2                    # sources outside the range are dropped
+    if by_source:
+        rel = (idx * 7 + 3) % (K + 1) - (1 if K > 1 else 0)      # -1 and, for K > 1, every value below K
+    else:
+        rel = rng.integers(-1, K + 1, size=len(idx))
+    rel = rel[: int(ptr[R]) - 4]                                # the last edges have no relation entry
+    used = (rng.random(N) < 0.7) if with_mask else None
+    g = rng.standard_normal((R * K, F)).astype(np.float32)
+    got = orc.bwd_typed_batch_view(ptr, idx, rel, K, g, N, used)
+    # closed form
+    want = np.zeros((N, F))
+    deg = np.diff(ptr)
+    for r in range(R):
+        for e in range(ptr[r], min(ptr[r + 1], len(rel))):
+            s, k = idx[e], rel[e]
+            if 0 <= k < K and 0 <= s < N and (used is None or used[s]):
+                want[s] += g[r * K + k].astype(np.float64) / deg[r]
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+    if used is not None:
+        assert (got[~used] == 0).all()
+    if by_source:
+        ptr2, idx2, cnt, d = orc.typed_csr(ptr, idx, rel, K, R, N, used)
+        w2 = orc.typed_csr_weights(ptr2, d, K)
+        ref, _, _ = orc.bwd_edge_value(ptr2, idx2, w2, g, None, None, N)
+        np.testing.assert_array_equal(got, ref)
+
+
 def test_edge_types_by_ranges_brute_force(orc):
     from helpers import random_csr
     rng = np.random.default_rng(71)
