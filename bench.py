@@ -46,7 +46,7 @@ def parse():
     ap.add_argument("--prefetch", action="store_true",
                     help="c3/c5: start each batch's host-link feature read one batch ahead, on a side stream")
     ap.add_argument("--no-batch-view", action="store_true",
-                    help="c3: batches come without the transposed view of their CSR, so every layer's "
+                    help="c3/c5: batches come without the transposed view of their CSR, so every layer's "
                          "backward builds one (the default: the loader emits it with the batch)")
     ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c2w", "c4", "c3", "c3b", "c5", "sample", "layer", "copy", "ceilings"])
     ap.add_argument("--heads", type=int, default=1, help="c2w: heads of the weighted aggregation (divides 256)")
@@ -748,7 +748,10 @@ def run_c5(args):
 
     n_pre = min(args.warmup + args.steps + 1, 512)       # one batch per iteration, none reused (see run_c3)
     samples = [direct_power_law_batch(N, n_seed, fanout, 2.0, 50 + i, degree_scale=1.25) for i in range(n_pre)]
-    batches = [make_batch(smp, FoldedLabels(), dev) for smp in samples]
+    # a batch comes with the transposed view of its CSR (and the view's edge slots, which the relational
+    # layer reads), as the loader emits it (--no-batch-view: backward builds the view of the regrouped block)
+    batches = [make_batch(smp, FoldedLabels(), dev, emit_view=not args.no_batch_view, view_edges=True)
+               for smp in samples]
     ev = {k: KernelClock() for k in ("load", "forward", "backward", "step", "update")}
     state = {"it": 0}
 
@@ -790,6 +793,7 @@ def run_c5(args):
                                % (N, N, pool_rows, shape)},
         "phases_ms": {k: c.mean_ms() for k, c in ev.items()},
         "phases_host_enqueue_ms": {k: c.mean_cpu_ms() for k, c in ev.items()},
+        "transposed_view": "built in backward" if args.no_batch_view else "emitted with the batch",
         "feature_rows_read_last_batch": int(cache.used_masks[0].sum()),
         "cached_1hop_fraction_last_batch": float((cache.sub2embed != -1).float().mean()),
     }

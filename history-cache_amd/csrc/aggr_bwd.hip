@@ -859,7 +859,8 @@ int aggr_bwd_impl(const int64_t *ptr, const int64_t *idx, const int64_t *ptrT,
                   float *edge_grad, int64_t E_total, int64_t R, int64_t F, int64_t n_src,
                   void *workspace, size_t workspace_bytes, bool masked, void *stream) {
   HC_REQUIRE(R >= 0 && F > 0 && n_src >= 0 && n_head >= 1 && E_total >= 0);
-  HC_REQUIRE(ptr && ptrT && g);
+  HC_REQUIRE(ptr && ptrT);
+  HC_REQUIRE(g || R == 0);   // a layer without rows has no gradient rows to read
   HC_REQUIRE(grad_vin || n_src == 0);
   if (n_head > 1) HC_REQUIRE(edge_value != nullptr);
   if (grad_hbuf) HC_REQUIRE(hmap != nullptr && hsize >= F);

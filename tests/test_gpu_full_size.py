@@ -124,6 +124,26 @@ def test_c2_results_are_bit_identical_run_to_run(c2):
     assert torch.equal(grad_x, c2["grad_x"])
 
 
+def test_c2_backward_over_the_whole_block_view_has_the_same_bits(c2):
+    """hc_aggr_bwd_batch_view at full size: the unfiltered view of the block serves the whole block and
+    its first half of the rows (edges of the other rows stepped over in the kernel) with the bits of the
+    path that builds a view per call (no source of this block has more than a chunk of incoming edges)."""
+    import hiscache_backend as be
+    ptrT, rowT, _ = c2["tr"]
+    assert int((ptrT[1:] - ptrT[:-1]).max()) <= be.bwd_chunk_edges(F)
+    view = be.BatchView(ptrT, rowT, None, R, N, E)
+    gx, _ = be._aggr_bwd_batch_view(c2["ptr"], view, c2["g"], None, None, 0, R, N, want_hist_grad=False)
+    assert torch.equal(gx, c2["grad_x"])
+    del gx
+    half = R // 2
+    e_half = int(c2["ptr"][half])
+    tr_h = be.build_transpose(c2["ptr"], c2["idx"], None, half, N, num_edge=e_half, want_edges=False)
+    want, _, _ = be._aggr_bwd(c2["ptr"], c2["idx"], tr_h, c2["g"][:half], None, None, c2["feat"], False, None, 0,
+                              half, N)
+    got, _ = be._aggr_bwd_batch_view(c2["ptr"], view, c2["g"][:half], None, None, 0, half, N, want_hist_grad=False)
+    assert torch.equal(got, want)
+
+
 def test_c4_admission_full_size():
     """2 M rows x 256, fp16 table 50 M x 256: mask == predicate on the kernel's own scores, slots ==
     header + exclusive prefix sum of the mask, table rows == fp16(embedding), maps consistent."""

@@ -45,6 +45,8 @@ CASES = [  # (seed, R, N, F, mean_deg, n_long, n_hub_src, hist_frac)
     (8, 70001, 4000, 100, 2, 4, 1, 0.4),              # generic width: no list, no quarter rule
     (9, 2048 * 9 + 1, 777, 192, 5, 6, 2, 0.2),
     (10, 300, 100000, 64, 6, 2, 0, 0.3),              # many more sources than edges
+    (11, 200_000, 9000, 256, 2, 20, 2, 0.3),          # well above the large-block threshold, widest fast loads
+    (12, 262_144, 20000, 128, 2, 7, 1, 0.0),
 ]
 
 
@@ -75,6 +77,18 @@ def test_random_block_forward_backward(be, orc, seed, R, N, F, mean_deg, n_long,
     np.testing.assert_array_equal(xt.grad.cpu().numpy(), gx)
     if hmap is not None:
         np.testing.assert_array_equal(ht.grad.cpu().numpy(), gh)
+    # the same gradient over a view of the whole block with nothing left out (history rows stepped over
+    # in the kernel), for the first two thirds of the rows as well
+    view = be.build_batch_view(T(ptr), T(idx), R, N)
+    for Rl in (R, (2 * R) // 3):
+        hm_l = None if hmap is None else hmap[:Rl]
+        gv, ghv = be._aggr_bwd_batch_view(T(ptr), view, T(g[:Rl]), None if hm_l is None else T(hm_l), (Rl, F), F,
+                                          Rl, N, want_hist_grad=hmap is not None)
+        wv, whv = orc.bwd_mean_row_batch_view(ptr, idx, g[:Rl], hm_l, N, R, hbuf_shape=(Rl, F),
+                                              chunk=be.bwd_chunk_edges(F))
+        np.testing.assert_array_equal(gv.cpu().numpy(), wv)
+        if hmap is not None:
+            np.testing.assert_array_equal(ghv.cpu().numpy(), whv)
     # transposed view with edge slots, against the stable-sort statement
     ptrT, rowT, edgeT = be.build_transpose(T(ptr), T(idx), None if hmap is None else T(hmap), R, N)
     wp, wr, we = orc.build_transpose(ptr, idx, hmap, N)
