@@ -318,9 +318,16 @@ __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
   __shared__ int s_last;
   int64_t R, E, n_src;
   tr_dims(dims, R, E, n_src);
+  // The launch may be sized for more edge slots than the block has (sizes read on the device): only the
+  // blocks that own edge slots take part, and block 0 always does, so that some block runs the scan.
+  // (Every ticket is an atomic on one address; hundreds of idle blocks queueing for it cost more than
+  // the work itself.)
+  const int64_t with_edges = R > 0 ? (E + TRS_BLOCK - 1) / TRS_BLOCK : 0;
+  const unsigned active = with_edges > 0 ? (unsigned)with_edges : 1u;
+  if (blockIdx.x >= active) return;
   const int64_t e0 = (int64_t)blockIdx.x * TRS_BLOCK;
   const int64_t e1 = e0 + TRS_BLOCK < E ? e0 + TRS_BLOCK : E;
-  if (e0 < E && R > 0) {                 // block-uniform: blocks behind the last edge slot only take a ticket
+  if (e0 < E && R > 0) {                 // block-uniform (false only for block 0 of a block without edges)
     if (threadIdx.x < 2 * HC_WAVE) {       // the tile's first and last row, searched by two waves side by side
       const int lane0 = hc_lane();
       const int which = (int)(threadIdx.x >> 6);
@@ -363,55 +370,66 @@ __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
   __syncthreads();
   if (threadIdx.x == 0) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    s_last = atomicAdd(&header->ticket, 1u) == gridDim.x - 1 ? 1 : 0;
+    s_last = atomicAdd(&header->ticket, 1u) == active - 1u ? 1 : 0;
   }
   __syncthreads();
   if (!s_last) return;
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-  // Exclusive scan of count[0, n_src] by this one block, TRS_SUPER entries per sweep.  A thread loads
-  // its 8 x 4 entries of the sweep with eight 16-byte loads issued together (entry = (g * 1024 + t) * 4 + j:
-  // coalesced), keeps them in registers, and the block scans the eight slabs of 4 096 entries one after
-  // the other.  (One thread per contiguous run of entries would issue 64 scattered requests per
-  // instruction from a single compute unit: measured 60 us for 26 000 sources.)  Entries between n_src
-  // and the end of the counter array are zero.
+  // Exclusive scan of count[0, n_src] by this one block, TRS_SUPER entries per sweep.  Every wave owns a
+  // contiguous run of 2 048 entries of the sweep and loads it with eight 16-byte loads per lane issued
+  // together (entry = run + (g * 64 + lane) * 4 + j: each load instruction covers 1 KiB), scans its run
+  // with shuffles alone, and the sixteen waves exchange their totals once per sweep (two barriers per
+  // 32 768 entries; a block-wide scan per slab of 4 096 entries took a barrier pair per slab and made the
+  // scan of 230 000 counters 80 us long).  (One thread per contiguous run of entries would issue 64
+  // scattered requests per instruction from a single compute unit: measured 60 us for 26 000 sources.)
+  // Entries between n_src and the end of the counter array are zero.
   constexpr int NW = TRS_BLOCK / HC_WAVE;
   constexpr int G = 8;
-  constexpr int64_t TRS_SUPER = (int64_t)TRS_BLOCK * 4 * G;
+  constexpr int64_t WAVE_SPAN = (int64_t)HC_WAVE * 4 * G;
+  constexpr int64_t TRS_SUPER = WAVE_SPAN * NW;
   const int lane = hc_lane();
   const int wave = (int)(threadIdx.x >> 6);
   const int64_t n_entries = n_src + 1;                      // ptrT has n_src + 1 entries
   const int64_t padded = (n_entries + 3) / 4 * 4;           // the counter array is zero-padded to 256 bytes
   int carry = 0;
   for (int64_t base = 0; base < n_entries; base += TRS_SUPER) {
+    const int64_t run0 = base + (int64_t)wave * WAVE_SPAN;
     int4 c[G];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      const int64_t i = base + ((int64_t)g * TRS_BLOCK + threadIdx.x) * 4;
+      const int64_t i = run0 + ((int64_t)g * HC_WAVE + lane) * 4;
       c[g] = i < padded ? *reinterpret_cast<const int4 *>(count + i) : make_int4(0, 0, 0, 0);
     }
+    int pre[G];                                             // entries of the run in front of the lane's four
+    int run = 0;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      const int64_t i = base + ((int64_t)g * TRS_BLOCK + threadIdx.x) * 4;
       const int mine = (c[g].x + c[g].y) + (c[g].z + c[g].w);
-      int x = mine;                                         // inclusive scan over the block's 1 024 threads
+      int x = mine;                                         // inclusive scan over the wave
 #pragma unroll
       for (int d = 1; d < HC_WAVE; d <<= 1) {
         const int y = __shfl_up(x, d, HC_WAVE);
         if (lane >= d) x += y;
       }
-      if (lane == HC_WAVE - 1) s_wave[wave] = x;
-      __syncthreads();
-      int off = carry + x - mine;
-      int slab = 0;
-      for (int w = 0; w < NW; ++w) {
-        const int t = s_wave[w];
-        if (w < wave) off += t;
-        slab += t;
-      }
-      __syncthreads();
-      carry += slab;
+      pre[g] = run + x - mine;
+      run += __builtin_amdgcn_readlane(x, HC_WAVE - 1);
+    }
+    if (lane == 0) s_wave[wave] = run;
+    __syncthreads();
+    int off = carry;
+    int sweep = 0;
+    for (int w = 0; w < NW; ++w) {
+      const int t = s_wave[w];
+      if (w < wave) off += t;
+      sweep += t;
+    }
+    __syncthreads();
+    carry += sweep;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int64_t i = run0 + ((int64_t)g * HC_WAVE + lane) * 4;
       if (i < n_entries) {
-        const int p0 = off, p1 = p0 + c[g].x, p2 = p1 + c[g].y, p3 = p2 + c[g].z;
+        const int p0 = off + pre[g], p1 = p0 + c[g].x, p2 = p1 + c[g].y, p3 = p2 + c[g].z;
         if (i + 3 < n_entries) {
           *reinterpret_cast<int4 *>(count + i) = make_int4(p0, p1, p2, p3);   // the segments' cursors
           ptrT[i] = p0;

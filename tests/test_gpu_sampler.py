@@ -105,7 +105,7 @@ def test_training_from_processed_files(tmp_path):
     store = ds.feature_store(device=DEV)
     np.testing.assert_array_equal(store.get(torch.tensor([0, 5, N - 1], device=DEV)).cpu().numpy(),
                                   feats[[0, 5, N - 1]])
-    sampler = ds.sampler([4, 3, 2], device=DEV, seed=2)
+    sampler = ds.sampler([4, 3, 2], device=DEV, seed=2, emit_view=True)
     cfg = make_config(Fin, C, H, L, method="grad", rate=0.6, device=DEV, path=str(tmp_path))
     cache = HistoryCache(store, cfg, "history_uvm", buffer_bytes=500 * int(np.lcm(Fin, H)) * 4)
     assert cache.total_num_node == N
