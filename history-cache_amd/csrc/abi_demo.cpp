@@ -1,6 +1,6 @@
 // A caller of the C ABI with no Python and no torch: device memory from hipMalloc, raw pointers in,
-// status codes out.  Builds a 4-row block, runs the forward, the transposed view and the backward,
-// and checks the numbers it can work out by hand.  Prints "abi_demo: ok" and returns 0 on success.
+// status codes out.  Builds a 4-row block, runs the forward, the transposed view and the backward (over a
+// view built for the call and over one shared view of the block), and checks the numbers it can work out by hand.  Prints "abi_demo: ok" and returns 0 on success.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -93,6 +93,27 @@ int main() {
     bad += gx[4 * F + c] != 3.0f / 3.0f;
     bad += gh[3 * F + c] != 4.0f;    // the history buffer takes the row's gradient undivided
     bad += gh[0 * F + c] != 0.0f;
+  }
+  // The same backward over ONE view of the whole block with nothing left out (what a loader emits with a
+  // batch): the history row is stepped over inside the kernel; a layer that owns only rows 0 and 1 reads
+  // the same view.
+  HC_OK_(hc_build_transpose(d_ptr, d_idx, nullptr, nullptr, R, E, N, d_ptrT, d_rowT, nullptr, d_ws, ws_bytes, st));
+  HC_OK_(hc_aggr_bwd_batch_view(d_ptr, d_ptrT, d_rowT, d_g, d_hmap, d_gx, d_gh, F, E, R, F, N, nullptr, 0, st));
+  HIP_OK(hipStreamSynchronize(st));
+  std::vector<float> gx2(N * F), gh2(R * F);
+  HIP_OK(hipMemcpy(gx2.data(), d_gx, gx2.size() * sizeof(float), hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(gh2.data(), d_gh, gh2.size() * sizeof(float), hipMemcpyDeviceToHost));
+  for (size_t i = 0; i < gx.size(); ++i) bad += gx2[i] != gx[i];
+  for (size_t i = 0; i < gh.size(); ++i) bad += gh2[i] != gh[i];
+  HC_OK_(hc_aggr_bwd_batch_view(d_ptr, d_ptrT, d_rowT, d_g, nullptr, d_gx, nullptr, 0, E, 2, F, N, nullptr, 0, st));
+  HIP_OK(hipStreamSynchronize(st));
+  HIP_OK(hipMemcpy(gx2.data(), d_gx, gx2.size() * sizeof(float), hipMemcpyDeviceToHost));
+  for (int64_t c = 0; c < F; ++c) {
+    bad += gx2[0 * F + c] != 0.0f;
+    bad += gx2[1 * F + c] != 1.0f / 2.0f;
+    bad += gx2[2 * F + c] != 1.0f / 2.0f;
+    bad += gx2[3 * F + c] != 0.0f;
+    bad += gx2[4 * F + c] != 0.0f;
   }
   if (bad) {
     std::printf("abi_demo: %d wrong values\n", bad);

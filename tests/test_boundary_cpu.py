@@ -62,6 +62,20 @@ def test_argument_errors_are_status_codes():
     assert lib.hc_gather_rows(p, 5, 4, p, null, p, 0, 0, 2, 4, null) == 2
     assert lib.hc_gather_rows(p, 0, 4, p, null, p, 9, 0, 2, 4, null) == 2
     assert lib.hc_count_history(null, null, null, 0, null, 4, 4, 1, 2, null) == 1
+    # the batch's shared view: missing pointers, capacities beyond the device-sized build, missing workspace,
+    # widths off the relational kernel's list -- all refused before anything is launched
+    assert lib.hc_aggr_bwd_batch_view(null, null, null, null, null, null, null, 0, 0, 4, 64, 4, null, 0, null) == 1
+    assert lib.hc_aggr_bwd_batch_view(p, p, p, p, null, p, p, 64, 8, 4, 64, 4, null, 0, null) == 1   # hbuf without map
+    big = (1 << 24) + 1
+    assert lib.hc_transpose_dev_workspace_bytes(big, 10) == 0 and lib.hc_transpose_dev_workspace_bytes(10, big) == 0
+    need = lib.hc_transpose_dev_workspace_bytes(1000, 100)
+    assert need >= 4 * 4 * 1000 + 4 * 101
+    assert lib.hc_build_transpose_dev(p, p, p, p, p, big, 10, p, p, null, p, 1 << 40, null) == 5
+    assert lib.hc_build_transpose_dev(p, p, p, p, p, 1000, 100, p, p, null, null, 0, null) == 4
+    assert lib.hc_build_transpose_dev(p, p, null, p, p, 1000, 100, p, p, null, p, need, null) == 1
+    assert lib.hc_aggr_bwd_batch_view_typed(p, p, p, p, p, 8, 3, null, p, p, 4, 100, 4, null) == 5
+    assert lib.hc_aggr_bwd_batch_view_typed(p, p, p, p, null, 8, 3, null, p, p, 4, 64, 4, null) == 1
+    assert lib.hc_aggr_bwd_batch_view_typed(p, p, p, p, p, 8, 0, null, p, p, 4, 64, 4, null) == 1
     for code in range(0, 8):
         assert lib.hc_strerror(code)
 
