@@ -11,7 +11,11 @@ Prints ONE JSON line: edges/s over the whole step, the roofline of the dominant 
 gather, timed with HIP events on the launch stream) and a CPU baseline (the same semantics written
 with PyTorch CPU index_add, timed on this machine's host cores on a 1/10-size sample).
 
-Other workloads (--workload c4 | c2row | c3 | c5) print their own line and are not the headline.
+The default line also carries the admission microbenchmark (c4), the papers100M-shaped history layer
+batched to 20 M edges (kernels.c3_batched) and the per-iteration time of the papers100M- and
+mag240M-shaped training iterations at their real batch shapes (iterations.c3, iterations.c5);
+--headline-only leaves them out.
+Other workloads (--workload c4 | c2row | c3 | c5 ...) print their own line and are not the headline.
 """
 import argparse
 import gc
@@ -32,6 +36,8 @@ HBM_PEAK_GBS = 8000.0
 # for the whole run so that the hit rate stays at the configuration's 35% (the age bound itself is exercised
 # by the c4 workload and by the tests).
 AGE_LIMIT_ITERS = 100_000
+# the c3 / c5 training iterations that the default line reports beside the kernels' figures
+ITERATION_STEPS, ITERATION_WARMUP = 200, 20
 MEASURED_TRAFFIC = {"c2": 23.08e9, "c2row": 13.93e9, "c4": 3.48e9, "c3_batched": 51.94e9}
 
 
@@ -54,7 +60,8 @@ def parse():
     ap.add_argument("--reps", type=int, default=8, help="c3b: measurements with freshly allocated tensors")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
-                    help="c2: skip the c4 and batched-c3 kernel figures that the default run adds to its line")
+                    help="c2: skip the c4 and batched-c3 kernel figures and the c3 / c5 iteration figures that "
+                         "the default run adds to its line")
     return ap.parse_args()
 
 
@@ -522,7 +529,7 @@ def c3_batched_layer(args, samples=None):
     return {"detail": detail, "roofline": roofline}
 
 
-def run_c3(args):
+def run_c3(args, with_batched=True):
     """papers100M-shaped training iteration (one GPU's share at its real batch shape) and a batched
     variant of its history layer (many batches side by side) for the kernels' asymptotic rate."""
     import numpy as np
@@ -663,7 +670,7 @@ def run_c3(args):
         shape = {k: int(np.mean([int(x["num_node_in_layer"][i]) for x in samples])) for i, k in enumerate(("n0", "n1", "n2", "n3"))}
         shape["edges"] = int(np.mean([x["idx"].size for x in samples]))
 
-    batched = c3_batched_layer(args, samples)
+    batched = c3_batched_layer(args, samples) if with_batched else {"detail": None, "roofline": None}
     return {
         "metric": "papers100M-shaped iteration ms (1 GPU)", "value": sec * 1e3, "unit": "ms", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": False,
@@ -1049,6 +1056,21 @@ def main():
             c3b = c3_batched_layer(args)["detail"]
             torch.cuda.empty_cache()
             res["kernels"]["c3_batched"] = c3b
+            # the other half of the metric, per-iteration ms at one GPU: the papers100M- and mag240M-shaped
+            # training iterations at their real batch shapes (a fresh batch every iteration)
+            it_args = argparse.Namespace(**vars(args))
+            it_args.steps, it_args.warmup = ITERATION_STEPS, ITERATION_WARMUP
+            res["iterations"] = {}
+            for name, fn in (("c3", lambda: run_c3(it_args, with_batched=False)), ("c5", lambda: run_c5(it_args))):
+                gc.collect()
+                torch.cuda.empty_cache()
+                r = fn()
+                res["iterations"][name] = {
+                    "workload": r["config"]["workload"], "ms": r["ms_per_step"], "steps": r["steps"],
+                    "warmup": r["warmup"], "transposed_view": r["transposed_view"],
+                    "phases_ms": r["phases_ms"], "phases_host_enqueue_ms": r["phases_host_enqueue_ms"]}
+            gc.collect()
+            torch.cuda.empty_cache()
         if not args.no_cpu_baseline:
             res["cpu_baseline"] = cpu_baseline_c2(shape)
     elif args.workload == "c2w":
