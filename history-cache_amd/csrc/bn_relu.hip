@@ -118,8 +118,8 @@ __device__ __forceinline__ void bn_sum_slabs(const float *__restrict__ part, int
 __global__ __launch_bounds__(BN_BLOCK) void bn_stats(
     const float *__restrict__ x, const float *__restrict__ bias, float *__restrict__ part,
     float *__restrict__ save_mean, float *__restrict__ save_invstd, float *__restrict__ running_mean,
-    float *__restrict__ running_var, float momentum, float eps, int64_t n, int C, BnShape sh,
-    unsigned *__restrict__ ticket) {
+    float *__restrict__ running_var, int64_t *__restrict__ batches_tracked, float momentum, float eps,
+    int64_t n, int C, BnShape sh, unsigned *__restrict__ ticket) {
   __shared__ float4 s_red[2][BN_BLOCK];
   __shared__ int s_flag;
   const int G = sh.groups, P = sh.rows_per_pass;
@@ -161,6 +161,7 @@ __global__ __launch_bounds__(BN_BLOCK) void bn_stats(
     *reinterpret_cast<float4 *>(o + C) = s2;
   }
   if (!bn_last_block(ticket, &s_flag)) return;
+  if (threadIdx.x == 0 && batches_tracked != nullptr) *batches_tracked += 1;   // BatchNorm1d's batch counter
   float4 t1, t2;
   bn_sum_slabs(part, sh.slabs, C, G, P, g, p, s_red, t1, t2);
   if (p != 0) return;
@@ -306,9 +307,10 @@ extern "C" size_t hc_bn_relu_workspace_bytes(int64_t n, int64_t C) {
 }
 
 extern "C" int hc_bn_relu_fwd(const float *x, const float *bias, const float *gamma, const float *beta,
-                              float *running_mean, float *running_var, float momentum, float eps, float *y,
-                              float *save_mean, float *save_invstd, int64_t n, int64_t C, void *workspace,
-                              size_t workspace_bytes, unsigned *ticket, void *stream) {
+                              float *running_mean, float *running_var, int64_t *num_batches_tracked,
+                              float momentum, float eps, float *y, float *save_mean, float *save_invstd,
+                              int64_t n, int64_t C, void *workspace, size_t workspace_bytes, unsigned *ticket,
+                              void *stream) {
   HC_REQUIRE(x && y && save_mean && save_invstd && ticket);
   BnShape sh;
   if (!bn_shape(n, C, &sh)) return n >= 1 && C >= 1 ? HC_EUNSUPPORTED : HC_EINVAL;
@@ -319,8 +321,8 @@ extern "C" int hc_bn_relu_fwd(const float *x, const float *bias, const float *ga
   if (!hc_grid_ok(blocks)) return HC_ELAUNCH;
   hipStream_t st = static_cast<hipStream_t>(stream);
   bn_stats<<<dim3((unsigned)sh.slabs), dim3(BN_BLOCK), 0, st>>>(
-      x, bias, static_cast<float *>(workspace), save_mean, save_invstd, running_mean, running_var, momentum,
-      eps, n, (int)C, sh, ticket);
+      x, bias, static_cast<float *>(workspace), save_mean, save_invstd, running_mean, running_var,
+      num_batches_tracked, momentum, eps, n, (int)C, sh, ticket);
   bn_apply<<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(x, save_mean, save_invstd, gamma, beta, y, n4,
                                                               sh.groups);
   return hc_launch_status();

@@ -96,6 +96,8 @@ class _SageConvFunction(torch.autograd.Function):
         ctx.hc = (ptr, idx, hmap, hsize, R, num_edge, b_l is not None, w_r is not None, sink)
         ctx.view = view if view is not None and view.covers(R, x.shape[0]) else None
         ctx.mark_non_differentiable(agg)
+        # no zero tensor for the gradient of `agg`, which never has one (a fill of [R, F] per layer otherwise)
+        ctx.set_materialize_grads(False)
         return out, agg
 
     @staticmethod
@@ -103,6 +105,8 @@ class _SageConvFunction(torch.autograd.Function):
         be = hiscache_backend
         ptr, idx, hmap, hsize, R, num_edge, has_bias, has_root, sink = ctx.hc
         x, agg, w_l, w_r = ctx.saved_tensors
+        if g_out is None:                                     # the layer's output did not reach the loss
+            return (None,) * 13
         g_out = g_out.contiguous()
         need = ctx.needs_input_grad
         g_agg = g_out @ w_l                                   # gradient reaching the aggregation output
@@ -153,12 +157,15 @@ def bn_relu(x, bn, bias=None, fused=True):
         return F.relu(bn(x))
     momentum = 0.0 if bn.momentum is None else bn.momentum
     track = bn.track_running_stats and bn.running_mean is not None
+    counter = None
     if track and bn.num_batches_tracked is not None:
-        bn.num_batches_tracked.add_(1)
-        if bn.momentum is None:                       # cumulative moving average
+        if bn.momentum is None:                       # cumulative moving average: the count is needed here
+            bn.num_batches_tracked.add_(1)
             momentum = 1.0 / float(bn.num_batches_tracked)
+        else:
+            counter = bn.num_batches_tracked          # incremented by the statistics kernel
     return be.bias_bn_relu(x, bias, bn.weight, bn.bias, bn.running_mean if track else None,
-                           bn.running_var if track else None, momentum, bn.eps)
+                           bn.running_var if track else None, momentum, bn.eps, counter)
 
 
 class MySageConvHistory(torch.nn.Module):

@@ -93,8 +93,8 @@ _SIGNATURES = {
     "hc_sample_layers": (_c_int, [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_int, ctypes.c_uint64, _c_p, _c_p,
                                   _c_p, _c_p, _c_p, _c_p, _c_sz, _c_p]),
     "hc_bn_relu_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
-    "hc_bn_relu_fwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, ctypes.c_float, ctypes.c_float, _c_p, _c_p,
-                                _c_p, _c_i64, _c_i64, _c_p, _c_sz, _c_p, _c_p]),
+    "hc_bn_relu_fwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, ctypes.c_float, ctypes.c_float, _c_p,
+                                _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_sz, _c_p, _c_p]),
     "hc_bn_relu_bwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64,
                                 _c_p, _c_sz, _c_p, _c_p]),
     "hc_weight_grad_workspace_bytes": (_c_sz, [_c_i64, _c_i64, _c_i64, _c_int]),
@@ -924,7 +924,7 @@ class _BiasBnRelu(torch.autograd.Function):
     bias; the running statistics are updated in place."""
 
     @staticmethod
-    def forward(ctx, x, bias, gamma, beta, running_mean, running_var, momentum, eps):
+    def forward(ctx, x, bias, gamma, beta, running_mean, running_var, momentum, eps, batches_tracked=None):
         lib = load_library()
         n, C = x.shape
         y = torch.empty_like(x)
@@ -932,7 +932,8 @@ class _BiasBnRelu(torch.autograd.Function):
         ws = _workspace(lib.hc_bn_relu_workspace_bytes(n, C), x.device)
         sp = stats.data_ptr()
         _check(lib.hc_bn_relu_fwd(_ptr(x), _ptr(bias), _ptr(gamma), _ptr(beta), _ptr(running_mean),
-                                  _ptr(running_var), float(momentum), float(eps), _ptr(y), _c_p(sp),
+                                  _ptr(running_var), _ptr(batches_tracked), float(momentum), float(eps), _ptr(y),
+                                  _c_p(sp),
                                   _c_p(sp + 4 * C), n, C, _ptr(ws), ws.numel(), _ptr(_ticket(x.device)),
                                   _stream()), "hc_bn_relu_fwd")
         ctx.save_for_backward(x, stats, gamma if gamma is not None else x.new_empty(0),
@@ -956,7 +957,7 @@ class _BiasBnRelu(torch.autograd.Function):
                                   _c_p(gp), _c_p(gp + 4 * C), _c_p(gp + 8 * C if has_bias else None), n, C,
                                   _ptr(ws), ws.numel(), _ptr(_ticket(x.device)), _stream()), "hc_bn_relu_bwd")
         return (dx, grads[2] if has_bias else None, grads[0] if has_gamma else None,
-                grads[1] if has_beta else None, None, None, None, None)
+                grads[1] if has_beta else None, None, None, None, None, None)
 
 
 def weight_grad_supported(g, x):
@@ -989,8 +990,9 @@ def weight_grad(g, x0, x1=None):
     return (dw[0], dw[1]) if x1 is not None else dw[0]
 
 
-def bias_bn_relu(x, bias, gamma, beta, running_mean, running_var, momentum, eps):
-    """Training-mode ``relu(batch_norm(x + bias))``; x is [n, C] fp32 on the GPU, n >= 2."""
+def bias_bn_relu(x, bias, gamma, beta, running_mean, running_var, momentum, eps, num_batches_tracked=None):
+    """Training-mode ``relu(batch_norm(x + bias))``; x is [n, C] fp32 on the GPU, n >= 2.
+    ``num_batches_tracked`` (one int64 on the device, optional) is incremented by the call's first kernel."""
     _dev(x, "x")
     if x.dim() != 2:
         raise ValueError("x must be [n, C]")
@@ -1005,7 +1007,11 @@ def bias_bn_relu(x, bias, gamma, beta, running_mean, running_var, momentum, eps)
             _dev(t, name, torch.float32)
             if t.numel() != x.shape[1]:
                 raise ValueError(f"{name} must hold C = {x.shape[1]} values")
-    return _BiasBnRelu.apply(x, bias, gamma, beta, running_mean, running_var, momentum, eps)
+    if num_batches_tracked is not None:
+        _dev(num_batches_tracked, "num_batches_tracked", torch.int64)
+        if num_batches_tracked.numel() != 1:
+            raise ValueError("num_batches_tracked must hold one value")
+    return _BiasBnRelu.apply(x, bias, gamma, beta, running_mean, running_var, momentum, eps, num_batches_tracked)
 
 
 def evict(checkin, slot2full, full2slot, stale_iter, sub2slot=None, score=None, thres=None):

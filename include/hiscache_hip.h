@@ -479,7 +479,9 @@ int hc_ring_lookup(const int64_t *full2slot, int64_t n_full, const int64_t *ids,
  *             y = max(0, (x - mean) * invstd * gamma + beta);
  *             running_mean = (1 - momentum) * running_mean + momentum * (mean + bias),
  *             running_var  = (1 - momentum) * running_var + momentum * var * n/(n-1)
- *             (torch.nn.BatchNorm1d's rule; both nullable).
+ *             (torch.nn.BatchNorm1d's rule; both nullable);
+ *             *num_batches_tracked += 1 (one int64 on the device, nullable:
+ *             the module's batch counter, which costs a launch of its own otherwise).
  *   backward: dy' = dy where y > 0, else 0; dbeta = sum dy', dgamma = sum dy' * xhat,
  *             dx = gamma * invstd * (dy' - dbeta/n - xhat * dgamma/n), dbias = 0.
  * bias (nullable) is a per-column constant that the caller has NOT added to x:
@@ -493,9 +495,10 @@ int hc_ring_lookup(const int64_t *full2slot, int64_t n_full, const int64_t *ids,
  * workspace: hc_bn_relu_workspace_bytes(n, C), 16-byte aligned; not preserved. */
 size_t hc_bn_relu_workspace_bytes(int64_t n, int64_t C);
 int hc_bn_relu_fwd(const float *x, const float *bias, const float *gamma, const float *beta,
-                   float *running_mean, float *running_var, float momentum, float eps, float *y,
-                   float *save_mean, float *save_invstd, int64_t n, int64_t C, void *workspace,
-                   size_t workspace_bytes, unsigned *ticket, void *stream);
+                   float *running_mean, float *running_var, int64_t *num_batches_tracked,
+                   float momentum, float eps, float *y, float *save_mean, float *save_invstd,
+                   int64_t n, int64_t C, void *workspace, size_t workspace_bytes, unsigned *ticket,
+                   void *stream);
 int hc_bn_relu_bwd(const float *dy, const float *x, const float *gamma, const float *beta,
                    const float *save_mean, const float *save_invstd, float *dx, float *dgamma,
                    float *dbeta, float *dbias, int64_t n, int64_t C, void *workspace,
