@@ -34,6 +34,8 @@ def test_aggregation_and_admission_replay_like_eager(be):
     thres = torch.tensor([11.3], device=DEV)          # about the median norm of a 128-dim N(0,1) row
     gather_ids = T(rng.integers(0, N, size=2000).astype(np.int64))
     N_all = max(R, N)
+    E = int(ptr[-1])
+    sizes = T(np.array([R, E, N], np.int64))          # the block's sizes as the sampler leaves them: on the device
     bn_bias, bn_gamma, bn_beta = (torch.randn(F, device=DEV) for _ in range(3))
 
     def fresh_state():
@@ -41,7 +43,8 @@ def test_aggregation_and_admission_replay_like_eager(be):
                     full2slot=torch.full((3 * R,), -1, dtype=torch.int64, device=DEV),
                     slot2full=torch.full((cap,), -1, dtype=torch.int64, device=DEV),
                     header=torch.zeros(1, dtype=torch.int64, device=DEV),
-                    running_mean=torch.zeros(F, device=DEV), running_var=torch.ones(F, device=DEV))
+                    running_mean=torch.zeros(F, device=DEV), running_var=torch.ones(F, device=DEV),
+                    batches=torch.zeros((), dtype=torch.int64, device=DEV))
 
     def work(st):
         out = be._aggr_fwd(be.SUBST_ROW, ptr_d, idx_d, x, hmap_d, hbuf, F, None, R)
@@ -54,9 +57,15 @@ def test_aggregation_and_admission_replay_like_eager(be):
         used = torch.stack(be.count_history_reconstruct(ptr_d, idx_d, hmap_d[:R], N_all, 64, 2))
         # a hidden layer's epilogue (its block counter is left at zero by every launch) and its backward
         zin = out.detach().requires_grad_(True)
-        act = be.bias_bn_relu(zin, bn_bias, bn_gamma, bn_beta, st["running_mean"], st["running_var"], 0.1, 1e-5)
+        act = be.bias_bn_relu(zin, bn_bias, bn_gamma, bn_beta, st["running_mean"], st["running_var"], 0.1, 1e-5,
+                              st["batches"])
         (dz,) = torch.autograd.grad(act, zin, g)
-        return out, tr[0], tr[1], gx, gh, mask, score, rows, found, used, act.detach(), dz
+        # the whole block's view built with the sizes read on the device (capacities above the sizes), and the
+        # backward over it with the history rows stepped over in the kernel
+        vp, vr, _ = be.build_transpose_dev(ptr_d, idx_d, sizes[0:1], sizes[1:2], sizes[2:3], E, N + 100)
+        view = be.BatchView(vp[: N + 1], vr, None, R, N, E)
+        gx_v, gh_v = be._aggr_bwd_batch_view(ptr_d, view, g, hmap_d, (R, F), F, R, N)
+        return out, tr[0], tr[1], gx, gh, mask, score, rows, found, used, act.detach(), dz, vp[: N + 1], gx_v, gh_v
 
     def load_inputs(seed):
         gen = torch.Generator(device=DEV).manual_seed(seed)
@@ -84,7 +93,8 @@ def test_aggregation_and_admission_replay_like_eager(be):
         graph.replay()
         torch.cuda.synchronize()
         for name, a, b in zip(("out", "ptrT", "rowT", "grad_x", "grad_h", "mask", "score", "rows", "found", "used",
-                               "epilogue", "epilogue gradient"), captured, eager):
+                               "epilogue", "epilogue gradient", "ptrT of the whole block", "grad_x over it",
+                               "grad_h over it"), captured, eager):
             if name == "rowT":                     # only the first ptrT[-1] entries are defined
                 n_tr = int(eager[1][-1])
                 a, b = a[:n_tr], b[:n_tr]
@@ -92,6 +102,8 @@ def test_aggregation_and_admission_replay_like_eager(be):
         for k in st_eager:
             assert torch.equal(st_graph[k], st_eager[k]), (rep, k)
         assert 0 < int(st_eager["header"]) < R
+        assert int(st_eager["batches"]) == 1
+        assert torch.equal(eager[4], eager[14])        # the history rows' gradient does not depend on the view
 
 
 def test_large_transposed_build_is_refused_on_a_capturing_stream(be):
