@@ -262,8 +262,10 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_finalize_ptr(const uint32_t *__re
 //                   stable sort gives: one-edge segments as they are, segments of up to 8 edges
 //                   sorted by their lane in registers, of up to 64 edges ranked inside a wave, longer
 //                   ones by the whole block through a bitmap of the segment's slots in LDS (rank =
-//                   number of set bits below the slot)
+//                   number of set bits below the slot), one window of TR_SMALL_EDGES slots at a time
 // The result is bit-identical to the sorted view of the large-block path.
+// The same four kernels serve hc_build_transpose_dev, where the block's sizes are read from device
+// memory (TrDims) and the launches are sized by capacities of up to 2^24 edge slots / sources.
 // ---------------------------------------------------------------------------------------
 constexpr int TRS_BLOCK = 1024;
 constexpr int64_t TR_SMALL_SOURCES = 1 << 20;
