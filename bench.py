@@ -50,7 +50,12 @@ def parse():
                     help="c3: draw every batch with the device sampler from a papers100M-sized graph in HBM "
                          "(next batch sampled on a side stream) instead of taking pre-generated batches")
     ap.add_argument("--prefetch", action="store_true",
-                    help="c3/c5: start each batch's host-link feature read one batch ahead, on a side stream")
+                    help="c3/c5: start each batch's host-link feature read one batch ahead, on a side stream, for "
+                         "the rows that the cache's state at that moment makes necessary (fixed up at the lookup)")
+    ap.add_argument("--prefetch-cus", type=int, default=16,
+                    help="with --prefetch: compute units the read-ahead's stream may use (0: an ordinary stream)")
+    ap.add_argument("--prefetch-all", action="store_true",
+                    help="with --prefetch: read every row of the next batch and mask at the lookup")
     ap.add_argument("--no-batch-view", action="store_true",
                     help="c3/c5: batches come without the transposed view of their CSR, so every layer's "
                          "backward builds one (the default: the loader emits it with the batch)")
@@ -562,8 +567,8 @@ def run_c3(args, with_batched=True):
         def masked_get(self, ids, mask):
             return super().masked_get(self.fold(ids), mask)
 
-        def prefetch(self, ids):
-            handle = super().prefetch(self.fold(ids))
+        def prefetch(self, ids, mask=None):
+            handle = super().prefetch(self.fold(ids), mask)
             handle.ids = ids
             return handle
 
@@ -573,7 +578,7 @@ def run_c3(args, with_batched=True):
     for lo in range(0, pool_rows, chunk):
         hi = min(pool_rows, lo + chunk)
         pinned[lo:hi].copy_(torch.randn(hi - lo, Fin, device=dev, generator=gen))
-    store = PooledStore(pinned, device=dev)
+    store = PooledStore(pinned, device=dev, prefetch_cus=args.prefetch_cus if args.prefetch else 0)
     cache = RingHistoryCache(store, N, Fin, H, capacity=N, num_layers=L, table_dtype=torch.float16,
                              thres=0.05, age_limit=AGE_LIMIT_ITERS, device=dev)
     # about 35% of the nodes start with a cached embedding
@@ -606,7 +611,7 @@ def run_c3(args, with_batched=True):
         batches.append(make_batch(smp, labels, dev, emit_view=not args.no_batch_view))
     ev = {k: KernelClock() for k in ("load", "forward", "backward", "step", "update")}
     state = {"it": 0}
-    sampled = {"sampler": None, "pending": None, "shapes": [], "wait_s": 0.0, "E_graph": 0}
+    sampled = {"sampler": None, "pending": None, "ahead": None, "shapes": [], "wait_s": 0.0, "E_graph": 0}
     if args.with_sampler:
         # batches come from the device sampler over a graph of the same size held in HBM; batch i+1 is
         # sampled on the sampler's side stream while batch i trains
@@ -619,24 +624,42 @@ def run_c3(args, with_batched=True):
         seed_pool = torch.randperm(N, device=dev, generator=gen)[: n_seed * 1024].view(1024, n_seed).contiguous()
         sampled["pending"] = sampled["sampler"].sample_async(seed_pool[0])
 
-    def next_batch():
-        if sampled["sampler"] is None:
-            return batches[(state["it"] - 1) % n_pre]
-        i = state["it"] - 1
+    def sampled_batch(i):
+        """Batch i from the sampler (waits only if its sampling is not finished yet); batch i + 1 is started."""
         t1 = time.perf_counter()
-        b = sampled["pending"].get()                       # waits only if the sampling is not finished yet
+        b = sampled["pending"].get()
         sampled["wait_s"] += time.perf_counter() - t1
         b.y = seed_pool[i % 1024] % C
         sampled["pending"] = sampled["sampler"].sample_async(seed_pool[(i + 1) % 1024])
         sampled["shapes"].append(b.num_node_in_layer.tolist() + [b.idx.numel()])
         return b
 
+    def next_batch():
+        i = state["it"] - 1
+        if sampled["sampler"] is None:
+            return batches[i % n_pre]
+        if not args.prefetch:
+            return sampled_batch(i)
+        # two batches deep: batch i was taken from the sampler one iteration ago, when its feature read started
+        if sampled["ahead"] is None:
+            sampled["ahead"] = sampled_batch(i)
+        return sampled["ahead"]
+
+    def start_prefetch():
+        """The next batch's host-link read, under the masks of the cache's present state (--prefetch-all: every
+        row), runs beside this batch's forward and backward."""
+        if sampled["sampler"] is None:
+            nxt = batches[state["it"] % n_pre]
+        else:
+            nxt = sampled["ahead"] = sampled_batch(state["it"])
+        cache.prefetch(nxt, speculative=not args.prefetch_all)
+
     def step():
         state["it"] += 1
         b = next_batch()
         ev["load"](lambda: cache.lookup_and_load(b, L))
-        if args.prefetch and sampled["sampler"] is None:   # the next batch's host-link read runs under this batch's compute
-            cache.prefetch(batches[state["it"] % n_pre])
+        if args.prefetch:
+            start_prefetch()
         out = ev["forward"](lambda: model(b))
         loss = torch.nn.functional.nll_loss(out, b.y)
         opt.zero_grad(set_to_none=True)
@@ -644,6 +667,12 @@ def run_c3(args, with_batched=True):
         ev["step"](lambda: opt.step())
         ev["update"](lambda: cache.update_history(b, state["it"]))
 
+    if args.prefetch:
+        # the read-ahead only runs beside the compute when the compute is on a stream of its own: the
+        # default stream and the read's CU-limited stream wait for each other
+        compute = torch.cuda.Stream()
+        compute.wait_stream(torch.cuda.current_stream())
+        torch.cuda.set_stream(compute)
     for _ in range(args.warmup):
         step()
     sync()
@@ -719,8 +748,8 @@ def run_c5(args):
         def masked_get(self, ids, mask):
             return super().masked_get(self.fold(ids), mask)
 
-        def prefetch(self, ids):
-            handle = super().prefetch(self.fold(ids))
+        def prefetch(self, ids, mask=None):
+            handle = super().prefetch(self.fold(ids), mask)
             handle.ids = ids
             return handle
 
@@ -730,7 +759,8 @@ def run_c5(args):
     for lo in range(0, pool_rows, chunk):
         hi = min(pool_rows, lo + chunk)
         pinned[lo:hi].copy_(torch.randn(hi - lo, Fin, device=dev, generator=gen).half())
-    store = PooledStore(pinned, device=dev, out_dtype=torch.float16)
+    store = PooledStore(pinned, device=dev, out_dtype=torch.float16,
+                        prefetch_cus=args.prefetch_cus if args.prefetch else 0)
     cache = RingHistoryCache(store, N, Fin, H, capacity=N, num_layers=L, table_dtype=torch.float16, thres=0.05,
                              age_limit=AGE_LIMIT_ITERS, device=dev)
     hit = torch.nonzero(torch.rand(N, device=dev, generator=gen) < 0.35).view(-1)
@@ -767,7 +797,7 @@ def run_c5(args):
         state["it"] += 1
         ev["load"](lambda: cache.lookup_and_load(b, L))
         if args.prefetch:             # the next batch's host-link read runs under this batch's compute
-            cache.prefetch(batches[state["it"] % n_pre])
+            cache.prefetch(batches[state["it"] % n_pre], speculative=not args.prefetch_all)
         out = ev["forward"](lambda: model(b))
         loss = torch.nn.functional.nll_loss(out, b.y)
         opt.zero_grad(set_to_none=True)
@@ -775,6 +805,10 @@ def run_c5(args):
         ev["step"](lambda: opt.step())
         ev["update"](lambda: cache.update_history(b, state["it"]))
 
+    if args.prefetch:                 # see run_c3: the read-ahead needs the compute on a stream of its own
+        compute = torch.cuda.Stream()
+        compute.wait_stream(torch.cuda.current_stream())
+        torch.cuda.set_stream(compute)
     for _ in range(args.warmup):
         step()
     sync()

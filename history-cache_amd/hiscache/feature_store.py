@@ -12,10 +12,14 @@ import hiscache_backend as _be
 
 class PinnedFeatureStore:
 
-    def __init__(self, features, device="cuda:0", out_dtype=torch.float32):
+    def __init__(self, features, device="cuda:0", out_dtype=torch.float32, prefetch_cus=0):
         # out_dtype: element type of the gathered rows (keep torch.float16 for fp16 feature files to
         # halve the traffic of the first aggregation layer)
+        # prefetch_cus > 0: ``prefetch`` reads on a stream that is kept to that many compute units, so that
+        # the read, which waits on the host link, does not slow the compute it runs beside (16 - 32 units
+        # still saturate the link; the compute must run on a non-default stream for the two to overlap)
         self.out_dtype = out_dtype
+        self.prefetch_cus = int(prefetch_cus)
         if features.dim() != 2:
             raise ValueError("features must be [num_nodes, feature_dim]")
         if features.is_cuda:
@@ -37,6 +41,11 @@ class PinnedFeatureStore:
             self._side = torch.cuda.Stream(device=self.device)
             self._done = torch.cuda.Event()
         return self._side
+
+    def _make_prefetch_stream(self):
+        if self.prefetch_cus > 0:
+            return _be.cu_limited_stream(self.prefetch_cus, self.device)
+        return torch.cuda.Stream(device=self.device)
 
     def get(self, ids):
         return _be.gather_rows(self.buffer, ids, out_dtype=self.out_dtype)
@@ -62,33 +71,41 @@ class PinnedFeatureStore:
     def join(self, event):
         torch.cuda.current_stream(self.device).wait_event(event)
 
-    def prefetch(self, ids):
-        """Start reading the rows of ALL ``ids`` on a side stream (default priority) now, so that the
-        host-link read overlaps whatever the caller queues next -- typically the previous batch's
-        forward and backward.  No mask: which rows the cache makes unnecessary is not known before that
-        batch's update.  Returns a handle for ``take``."""
+    def prefetch(self, ids, mask=None):
+        """Start reading the rows of ``ids`` (all of them, or those flagged by ``mask``: the caller's guess
+        of which will be needed) on a side stream (default priority) now, so that the host-link read
+        overlaps whatever the caller queues next -- typically the previous batch's forward and
+        backward.  Returns a handle for ``take``; ``handle.mask`` is the mask that was read under."""
         cur = torch.cuda.current_stream(self.device)
         if self._prefetch_side is None:
-            self._prefetch_side = torch.cuda.Stream(device=self.device)
+            self._prefetch_side = self._make_prefetch_stream()
         side = self._prefetch_side
         side.wait_stream(cur)                      # the ids are produced on the current stream
         with torch.cuda.stream(side):
-            rows = _be.gather_rows(self.buffer, ids, out_dtype=self.out_dtype)
+            rows = _be.gather_rows(self.buffer, ids, mask=mask, out_dtype=self.out_dtype)
             done = torch.cuda.Event()
             done.record(side)
         ids.record_stream(side)
-        return PrefetchedRows(ids, rows, done)
+        if mask is not None:
+            mask.record_stream(side)
+        return PrefetchedRows(ids, rows, done, mask)
 
-    def take(self, handle):
-        """The rows of a ``prefetch``; the current stream waits for the read to finish."""
+    def take(self, handle, need=None):
+        """The rows of a ``prefetch``; the current stream waits for the read to finish.  ``need`` (the
+        exact mask, for a read that was started under a guessed one): rows that have become necessary are
+        read now, rows that no longer are get cleared -- the result equals ``masked_get(ids, need)``."""
         cur = torch.cuda.current_stream(self.device)
         cur.wait_event(handle.done)
         handle.rows.record_stream(cur)
+        if need is not None and handle.mask is not None:
+            _be.fixup_rows(self.buffer, handle.src_ids, need, handle.mask, handle.rows)
         return handle.rows
 
 
 class PrefetchedRows:
-    __slots__ = ("ids", "rows", "done")
+    """``ids``: what the caller asked for (its identity tells the batch apart); ``src_ids``: the rows of
+    the store that were read for them."""
+    __slots__ = ("ids", "src_ids", "rows", "done", "mask")
 
-    def __init__(self, ids, rows, done):
-        self.ids, self.rows, self.done = ids, rows, done
+    def __init__(self, ids, rows, done, mask=None):
+        self.ids, self.src_ids, self.rows, self.done, self.mask = ids, ids, rows, done, mask

@@ -72,21 +72,42 @@ class RingHistoryCache:
                                                         sub_to_full.shape[0], batch.y.shape[0], num_layer)
         handle = getattr(batch, "prefetched_x", None)
         if handle is not None and handle.ids is sub_to_full:
-            # every row was read ahead of time (``prefetch``): zero the rows the cache makes unnecessary
             batch.prefetched_x = None
-            x = self.uvm.take(handle)
-            x.masked_fill_(~self.used_masks[0][:, None], 0)
+            if handle.mask is None:
+                # every row was read ahead of time: zero the rows the cache makes unnecessary
+                x = self.uvm.take(handle)
+                x.masked_fill_(~self.used_masks[0][:, None], 0)
+            else:
+                # the rows were read under the masks of an earlier cache state: the few that have become
+                # necessary since are read now, the few that no longer are get cleared
+                x = self.uvm.take(handle, self.used_masks[0])
             batch.x = x
             return None
         batch.x = self.uvm.masked_get(sub_to_full, self.used_masks[0])
         return None
 
-    def prefetch(self, batch):
-        """Start the host-link read of ``batch``'s feature rows now (all of them), to overlap it with the
-        work queued before that batch's ``lookup_and_load``, which then only masks the rows."""
+    def prefetch(self, batch, speculative=True, num_layer=None):
+        """Start the host-link read of ``batch``'s feature rows now, to overlap it with the work queued
+        before that batch's ``lookup_and_load``.  ``speculative``: only the rows that the cache's PRESENT
+        state makes necessary are read (a lookup and the used masks, as ``lookup_and_load`` computes
+        them, one admission pass early); ``lookup_and_load`` then reads the rows that an admission or an
+        overwritten slot has made necessary since and clears those that have become unnecessary, so that
+        ``batch.x`` is the same tensor either way.  Otherwise every row is read and masked later."""
         start = getattr(self.uvm, "prefetch", None)
-        if start is not None:
+        if start is None:
+            return
+        if not speculative:
             batch.prefetched_x = start(batch.sub_to_full)
+            return
+        if num_layer is None:
+            num_layer = self.num_layers_all
+        sub_to_full = batch.sub_to_full
+        n1 = int(batch.num_node_in_layer[1])
+        slot, _ = _be.ring_lookup(self.full2slot, sub_to_full[:n1], self.table, checkin=self.checkin,
+                                  now=self.glb_iter + 1, age_limit=self.age_limit, want_rows=False)
+        masks = _be.count_history_reconstruct(batch.ptr, batch.idx, slot, sub_to_full.shape[0],
+                                              batch.y.shape[0], num_layer)
+        batch.prefetched_x = start(sub_to_full, masks[0])
 
     @torch.no_grad()
     def update_history(self, batch, glb_iter):

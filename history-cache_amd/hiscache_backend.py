@@ -82,6 +82,9 @@ _SIGNATURES = {
     "hc_count_num": (_c_int, [_c_p, _c_i64, _c_i64, _c_p, _c_p]),
     "hc_structure_score": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p]),
     "hc_gather_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_int, _c_i64, _c_i64, _c_p]),
+    "hc_stream_create_cu_limited": (_c_int, [_c_int, _c_p]),
+    "hc_stream_destroy": (_c_int, [_c_p]),
+    "hc_fixup_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p]),
     "hc_ring_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_int, _c_i64, _c_i64, _c_p, _c_p,
                                 _c_i64, _c_p]),
@@ -785,6 +788,43 @@ def gather_rows(src, ids, mask=None, out=None, accumulate=False, out_dtype=torch
     rc = lib.hc_gather_rows(_ptr(src), _float_dtype(src, "src"), src.shape[0], _ptr(ids), _ptr(mask),
                             _ptr(out), _float_dtype(out, "out"), 1 if accumulate else 0, n, F, _stream())
     _check(rc, "hc_gather_rows")
+    return out
+
+
+def cu_limited_stream(n_cus, device):
+    """A torch stream (default priority) whose kernels run on ``n_cus`` compute units only, spread over the
+    chip: for work that waits on the host link beside compute (``PinnedFeatureStore.prefetch``).  The
+    stream lives until the process ends."""
+    lib = load_library()
+    device = torch.device(device)
+    handle = ctypes.c_void_p()
+    with torch.cuda.device(device):
+        _check(lib.hc_stream_create_cu_limited(int(n_cus), ctypes.cast(ctypes.pointer(handle), _c_p)),
+               "hc_stream_create_cu_limited")
+    return torch.cuda.ExternalStream(handle.value, device=device)
+
+
+def fixup_rows(src, ids, need, have, out):
+    """``out`` holds ``gather_rows(src, ids, mask=have)`` (rows read ahead of time under a guess); bring it
+    to ``gather_rows(src, ids, mask=need)`` in place: rows that are needed but were not read are read,
+    rows that were read but are not needed are cleared, the others are not touched."""
+    lib = load_library()
+    if not isinstance(src, torch.Tensor) or src.dim() != 2 or not src.is_contiguous():
+        raise ValueError("src must be a contiguous 2-D tensor")
+    if not src.is_cuda and not src.is_pinned():
+        raise RuntimeError("src must be on the GPU or in pinned host memory")
+    _dev(ids, "ids", torch.int64)
+    _dev(out, "out")
+    n, F = ids.numel(), src.shape[1]
+    if tuple(out.shape) != (n, F):
+        raise ValueError("out must be [len(ids), F]")
+    for name, m in (("need", need), ("have", have)):
+        _dev(m, name)
+        if m.dtype not in (torch.bool, torch.uint8) or m.numel() < n:
+            raise ValueError(f"{name} must be a bool tensor with one entry per id")
+    rc = lib.hc_fixup_rows(_ptr(src), _float_dtype(src, "src"), src.shape[0], _ptr(ids), _ptr(need), _ptr(have),
+                           _ptr(out), _float_dtype(out, "out"), n, F, _stream())
+    _check(rc, "hc_fixup_rows")
     return out
 
 

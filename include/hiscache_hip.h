@@ -449,6 +449,29 @@ int hc_gather_rows(const void *src, int src_dtype, int64_t n_rows, const int64_t
                    const uint8_t *mask, void *dst, int dst_dtype, int accumulate, int64_t n,
                    int64_t F, void *stream);
 
+/* hc_stream_create_cu_limited: a HIP stream (non-default, default priority)
+ * whose kernels run on n_cus compute units only, spread over the chip; for the
+ * zero-copy feature read that runs beside the previous batch's forward and
+ * backward (the side stream of cxgnndl.UVM's role, hiscache/history_cache.py:
+ * 283,301,345): a kernel that waits on the host link slows the kernels beside
+ * it unless it is kept to a few compute units (16 - 32 still saturate the
+ * link), and the overlap only pays when the compute itself runs on a
+ * non-default stream.  The handle is a hipStream_t; release it with
+ * hc_stream_destroy once its work has finished. */
+int hc_stream_create_cu_limited(int n_cus, void **stream);
+int hc_stream_destroy(void *stream);
+
+/* hc_fixup_rows: rows that were gathered ahead of time under a guess of which
+ * are needed -- the zero-copy read of a batch's features started one batch
+ * early, under the cache state of that moment (uvm.masked_get of
+ * hiscache/history_cache.py:345 moved off the critical path) -- brought to the
+ * exact answer: dst[i,:] = src[ids[i],:] where need[i] && !have[i]; dst[i,:] = 0
+ * where !need[i] && have[i]; other rows are left untouched.  need / have: one
+ * byte per row.  Afterwards dst equals hc_gather_rows with mask = need. */
+int hc_fixup_rows(const void *src, int src_dtype, int64_t n_rows, const int64_t *ids,
+                  const uint8_t *need, const uint8_t *have, void *dst, int dst_dtype, int64_t n,
+                  int64_t F, void *stream);
+
 /* hc_lookup: out[i] = map[ids[i] + offset]  (int64 gather; the id translation
  * of lookup_and_load, hiscache/history_cache.py:310,315). */
 int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset, int64_t *out,

@@ -76,6 +76,10 @@ def test_argument_errors_are_status_codes():
     assert lib.hc_aggr_bwd_batch_view_typed(p, p, p, p, p, 8, 3, null, p, p, 4, 100, 4, null) == 5
     assert lib.hc_aggr_bwd_batch_view_typed(p, p, p, p, null, 8, 3, null, p, p, 4, 64, 4, null) == 1
     assert lib.hc_aggr_bwd_batch_view_typed(p, p, p, p, p, 8, 0, null, p, p, 4, 64, 4, null) == 1
+    assert lib.hc_fixup_rows(p, 0, 4, p, p, null, p, 0, 2, 4, null) == 1       # the guessed mask is missing
+    assert lib.hc_fixup_rows(p, 7, 4, p, p, p, p, 0, 2, 4, null) == 2
+    assert lib.hc_stream_create_cu_limited(0, p) == 1 and lib.hc_stream_create_cu_limited(8, null) == 1
+    assert lib.hc_stream_destroy(null) == 0
     for code in range(0, 8):
         assert lib.hc_strerror(code)
 

@@ -169,6 +169,75 @@ def test_prefetched_features_give_the_same_batch():
     assert ring[0].header > 0
 
 
+@pytest.mark.parametrize("src_dtype,out_dtype", [(torch.float32, torch.float32), (torch.float16, torch.float16),
+                                                 (torch.float16, torch.float32)])
+def test_fixup_rows_turns_a_guessed_gather_into_the_exact_one(src_dtype, out_dtype):
+    """hc_fixup_rows: rows read under a guessed mask become the rows of the exact mask -- missing rows are
+    read (from pinned host memory, zero-copy), surplus rows cleared, the others not touched."""
+    import hiscache_backend as be
+    rng = np.random.default_rng(21)
+    n_rows, F, n = 5000, 96, 3000
+    table = torch.from_numpy(rng.standard_normal((n_rows, F)).astype(np.float32)).to(src_dtype).pin_memory()
+    ids = torch.from_numpy(rng.integers(-5, n_rows, size=n)).to(DEV)           # a few negative ids: from the end
+    have = torch.from_numpy(rng.random(n) < 0.6).to(DEV)
+    need = torch.from_numpy(rng.random(n) < 0.6).to(DEV)
+    out = be.gather_rows(table, ids, mask=have, out_dtype=out_dtype)
+    same = (have == need)
+    marker = out[same].clone()
+    be.fixup_rows(table, ids, need, have, out)
+    want = be.gather_rows(table, ids, mask=need, out_dtype=out_dtype)
+    assert torch.equal(out, want)
+    assert torch.equal(out[same], marker)
+    assert int((need & ~have).sum()) > 100 and int((have & ~need).sum()) > 100
+    # nothing to fix: the call leaves the rows alone
+    before = out.clone()
+    be.fixup_rows(table, ids, need, need, out)
+    assert torch.equal(out, before)
+
+
+@pytest.mark.parametrize("prefetch_cus", [0, 16])
+def test_speculative_prefetch_is_fixed_up_at_the_lookup(prefetch_cus):
+    """The ring cache's read-ahead runs under the masks of the cache state at that moment; entries that are
+    admitted, or whose slot is given up, between the read-ahead and the lookup change which rows are needed.
+    ``batch.x`` still equals the unpipelined result, and the test makes sure rows moved in both directions.
+    With ``prefetch_cus`` the read runs on a stream kept to that many compute units."""
+    from hiscache import PinnedFeatureStore, RingHistoryCache
+    from hiscache.synthetic import make_batch
+    rng = np.random.default_rng(33)
+    N, Fin, H = 4000, 32, 64
+    feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32))
+    caches = [RingHistoryCache(PinnedFeatureStore(feats, device=DEV, prefetch_cus=cus), N, Fin, H, capacity=2000,
+                               num_layers=3, table_dtype=torch.float16, thres=0.05, age_limit=1000, device=DEV)
+              for cus in (0, prefetch_cus)]
+    b = layered_batch(rng, N, 60, [6, 5, 4])
+    n1 = int(b["num_node_in_layer"][1])
+    hop1 = b["sub_to_full"][:n1]
+    first = torch.from_numpy(hop1[: n1 // 3].copy()).to(DEV)        # cached when the read-ahead starts
+    later = torch.from_numpy(hop1[n1 // 3: 2 * n1 // 3].copy()).to(DEV)  # admitted in between
+    rows = torch.from_numpy(rng.standard_normal((n1, H)).astype(np.float32)).to(DEV)
+    for c in caches:
+        c.preload(first, rows[: first.numel()])
+    plain, piped = (make_batch(b, np.zeros(N, np.int64), DEV) for _ in range(2))
+    compute = torch.cuda.Stream()                                  # the read-ahead overlaps a non-default stream
+    compute.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(compute):
+        caches[1].prefetch(piped)
+        have = piped.prefetched_x.mask.clone()
+        for c in caches:                                            # the cache changes before the lookup
+            c.preload(later, rows[first.numel(): first.numel() + later.numel()])
+            c.full2slot[first[::2]] = -1                            # every other early entry gives up its slot
+        caches[0].lookup_and_load(plain, 3)
+        caches[1].lookup_and_load(piped, 3)
+        need = caches[1].used_masks[0]
+        assert int((need & ~have).sum()) > 0 and int((have & ~need).sum()) > 0
+        assert torch.equal(piped.x, plain.x)
+        assert torch.equal(caches[1].sub2embed, caches[0].sub2embed)
+        ref = feats.to(DEV)[piped.sub_to_full] * need[:, None]
+        assert torch.equal(piped.x, ref)
+    torch.cuda.current_stream().wait_stream(compute)
+    torch.cuda.synchronize()
+
+
 def test_update_history_overflow_is_counted():
     from oracle import hc_oracle as orc
     from oracle import host_model
