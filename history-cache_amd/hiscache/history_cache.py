@@ -223,8 +223,8 @@ class HistoryCache:
         hit_feat_mask = self.sub2feat != -1
         load_mask = torch.logical_and(self.used_masks[0], ~hit_feat_mask)
         self.glb_iter += 1
-        pre = self._take_prefetched(batch)
-        if pre is not None:
+        pre, exact = self._take_prefetched(batch, load_mask)
+        if pre is not None and not exact:
             # every row was read ahead of time: keep what masked_get + the feature-cache merge would have
             # produced (needed rows and feature-cache hits), zero the rest
             self.cached_embedding = _be.gather_rows(self.buffer.view(-1, self.hidden_channels),
@@ -237,7 +237,8 @@ class HistoryCache:
         # Host-link read of the needed rows.  (Reading it on a side stream here would only overlap
         # the small gather below and costs the host more than that saves; ``prefetch`` is the way to
         # overlap the read with compute.)
-        x = self.uvm.masked_get(sub_to_full, load_mask)
+        # (a read-ahead under the masks of an earlier cache state was brought to ``load_mask`` when it was taken)
+        x = pre if pre is not None else self.uvm.masked_get(sub_to_full, load_mask)
         # slot -1 reads the last row of the view, as the reference's indexing does; such rows
         # are ignored by the aggregation
         self.cached_embedding = _be.gather_rows(self.buffer.view(-1, self.hidden_channels),
@@ -248,20 +249,39 @@ class HistoryCache:
         self.load_mask = load_mask
         return None
 
-    def prefetch(self, batch):
-        """Start the host-link read of ``batch``'s feature rows now (all of them), to overlap it with the
-        work queued before that batch's ``lookup_and_load``, which then only masks the rows.  Optional:
-        without it ``lookup_and_load`` reads the needed rows itself.  ``batch.x`` comes out the same."""
+    def prefetch(self, batch, speculative=True, num_layer=None):
+        """Start the host-link read of ``batch``'s feature rows now, to overlap it with the work queued
+        before that batch's ``lookup_and_load``.  ``speculative``: the rows that the cache's PRESENT state
+        makes necessary (slots, used masks and feature-cache hits as ``lookup_and_load`` computes them, one
+        update early); ``lookup_and_load`` then reads the rows that have become necessary since and clears
+        those that no longer are.  Otherwise every row is read and masked later.  Optional: without it
+        ``lookup_and_load`` reads the needed rows itself.  ``batch.x`` comes out the same."""
         start = getattr(self.uvm, "prefetch", None)
-        if start is not None and "history" in self.feat_mode:
+        if start is None or "history" not in self.feat_mode:
+            return
+        if not speculative:
             batch.prefetched_x = start(batch.sub_to_full)
+            return
+        if num_layer is None:
+            num_layer = self.num_layers_all
+        sub_to_full = batch.sub_to_full
+        n1 = int(batch.num_node_in_layer[1])
+        sub2embed = _be.lookup(self.full2embed, sub_to_full[:n1], 0)
+        sub2feat = _be.lookup(self.full2embed, sub_to_full, self.total_num_node)
+        used = _be.count_history_reconstruct(batch.ptr, batch.idx, sub2embed, sub_to_full.shape[0],
+                                             batch.y.shape[0], num_layer)
+        batch.prefetched_x = start(sub_to_full, torch.logical_and(used[0], sub2feat == -1))
 
-    def _take_prefetched(self, batch):
+    def _take_prefetched(self, batch, need):
+        """(rows, exact): the rows of a read-ahead of this batch, or (None, False).  ``exact``: they were
+        read under a mask and have been brought to ``need``, i.e. they equal ``masked_get(ids, need)``."""
         handle = getattr(batch, "prefetched_x", None)
         if handle is None or handle.ids is not batch.sub_to_full:
-            return None
+            return None, False
         batch.prefetched_x = None
-        return self.uvm.take(handle)
+        if handle.mask is None:
+            return self.uvm.take(handle), False
+        return self.uvm.take(handle, need), True
 
     def stats(self):
         """Cache occupancy (synchronises)."""

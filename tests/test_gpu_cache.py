@@ -94,23 +94,25 @@ def test_lookup_update_cycles_match_model():
     assert s["feat_cached"] == int((st.full2embed[N:2 * N] != -1).sum())
 
 
-def test_prefetched_features_give_the_same_batch():
+@pytest.mark.parametrize("speculative", [True, False])
+def test_prefetched_features_give_the_same_batch(speculative):
     """``prefetch`` issued one batch ahead (before the previous batch's update changes the cache) leaves
     ``batch.x``, the slots, the masks and the cache state exactly as the unpipelined path does, for the
-    buffer cache and the ring cache."""
+    buffer cache and the ring cache; reading the rows that the cache's state at that moment makes necessary
+    (``speculative``) or every row."""
     from oracle import hc_oracle as orc
     from oracle import host_model
     from hiscache import PinnedFeatureStore, RingHistoryCache
     rng, feats, cfg, cache, st = make_world(5)
     N, H = st.N, st.H
     pairs = [batch_pair(rng, N, 40, [6, 4, 3]) for _ in range(6)]
-    cache.prefetch(pairs[0][0])
+    cache.prefetch(pairs[0][0], speculative=speculative)
     for it, (gpu, cpu) in enumerate(pairs, start=1):
         assert gpu.prefetched_x is not None
         cache.lookup_and_load(gpu, 3)
         assert gpu.prefetched_x is None                      # consumed
         if it < len(pairs):
-            cache.prefetch(pairs[it][0])                     # next batch, before this batch's update
+            cache.prefetch(pairs[it][0], speculative=speculative)   # next batch, before this batch's update
         ref = host_model.lookup_and_load(st, cpu, 3, feats)
         np.testing.assert_array_equal(gpu.x.cpu().numpy(), ref.x.numpy())
         np.testing.assert_array_equal(cache.sub2embed.cpu().numpy(), ref.sub2embed.numpy())
@@ -128,7 +130,7 @@ def test_prefetched_features_give_the_same_batch():
         assert_state_equal(cache, st)
     # a handle made for other ids is ignored
     gpu, cpu = batch_pair(rng, N, 30, [5, 3, 2])
-    cache.prefetch(gpu)
+    cache.prefetch(gpu, speculative=speculative)
     gpu.sub_to_full = gpu.sub_to_full.clone()
     cache.lookup_and_load(gpu, 3)
     np.testing.assert_array_equal(gpu.x.cpu().numpy(), host_model.lookup_and_load(st, cpu, 3, feats).x.numpy())
@@ -147,14 +149,14 @@ def test_prefetched_features_give_the_same_batch():
     bs = [layered_batch(rng, N, 40, [6, 4, 3]) for _ in range(5)]
     mk = lambda b: make_batch(b, np.zeros(N, np.int64), DEV)
     nxt = mk(bs[0])
-    ring[1].prefetch(nxt)
+    ring[1].prefetch(nxt, speculative=speculative)
     for it, b in enumerate(bs, start=1):
         plain, piped = mk(b), nxt
         ring[0].lookup_and_load(plain, 3)
         ring[1].lookup_and_load(piped, 3)
         if it < len(bs):
             nxt = mk(bs[it])
-            ring[1].prefetch(nxt)
+            ring[1].prefetch(nxt, speculative=speculative)
         np.testing.assert_array_equal(piped.x.cpu().numpy(), plain.x.cpu().numpy())
         np.testing.assert_array_equal(ring[1].cached_embedding.cpu().numpy(), ring[0].cached_embedding.cpu().numpy())
         n1 = int(b["num_node_in_layer"][1])
