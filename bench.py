@@ -13,7 +13,8 @@ with PyTorch CPU index_add, timed on this machine's host cores on a 1/10-size sa
 
 The default line also carries the admission microbenchmark (c4), the papers100M-shaped history layer
 batched to 20 M edges (kernels.c3_batched) and the per-iteration time of the papers100M- and
-mag240M-shaped training iterations at their real batch shapes (iterations.c3, iterations.c5);
+mag240M-shaped training iterations at their real batch shapes (iterations.c3, iterations.c5) and of the
+papers100M-shaped one fed by the device sampler with the features read one batch ahead (iterations.c3_sampled);
 --headline-only leaves them out.
 Other workloads (--workload c4 | c2row | c3 | c5 ...) print their own line and are not the headline.
 """
@@ -689,6 +690,7 @@ def run_c3(args, with_batched=True):
     sync()
     sec = (time.perf_counter() - t0) / args.steps
     gc.unfreeze()
+    torch.cuda.set_stream(torch.cuda.default_stream())
     if sampled["sampler"] is not None:
         sampled["pending"].get()
         m = np.mean(np.asarray(sampled["shapes"], dtype=np.float64), axis=0)
@@ -822,6 +824,7 @@ def run_c5(args):
     sync()
     sec = (time.perf_counter() - t0) / args.steps
     gc.unfreeze()
+    torch.cuda.set_stream(torch.cuda.default_stream())
     shape = {k: int(np.mean([int(x["num_node_in_layer"][i]) for x in samples])) for i, k in enumerate(("n0", "n1", "n2"))}
     shape["edges"] = int(np.mean([x["idx"].size for x in samples]))
     return {
@@ -1095,13 +1098,19 @@ def main():
             it_args = argparse.Namespace(**vars(args))
             it_args.steps, it_args.warmup = ITERATION_STEPS, ITERATION_WARMUP
             res["iterations"] = {}
-            for name, fn in (("c3", lambda: run_c3(it_args, with_batched=False)), ("c5", lambda: run_c5(it_args))):
+            # c3_sampled: the same iteration fed by the device sampler from a papers100M-sized graph in HBM
+            # (batches of about 236 k edges), features read one batch ahead on a CU-limited stream
+            sm_args = argparse.Namespace(**vars(it_args))
+            sm_args.with_sampler, sm_args.prefetch = True, True
+            for name, fn in (("c3", lambda: run_c3(it_args, with_batched=False)), ("c5", lambda: run_c5(it_args)),
+                             ("c3_sampled", lambda: run_c3(sm_args, with_batched=False))):
                 gc.collect()
                 torch.cuda.empty_cache()
                 r = fn()
                 res["iterations"][name] = {
                     "workload": r["config"]["workload"], "ms": r["ms_per_step"], "steps": r["steps"],
                     "warmup": r["warmup"], "transposed_view": r["transposed_view"],
+                    "feature_read_ahead": bool(getattr(sm_args if name == "c3_sampled" else it_args, "prefetch")),
                     "phases_ms": r["phases_ms"], "phases_host_enqueue_ms": r["phases_host_enqueue_ms"]}
             gc.collect()
             torch.cuda.empty_cache()
