@@ -791,16 +791,37 @@ def gather_rows(src, ids, mask=None, out=None, accumulate=False, out_dtype=torch
     return out
 
 
+_cu_stream_handles = []
+
+
+def _destroy_cu_streams():
+    """At interpreter exit: wait for the device and give the CU-limited streams back while the HIP runtime is
+    still up (a stream of this kind left to the runtime's own teardown crashed a profiled run at exit)."""
+    if not _cu_stream_handles:
+        return
+    try:
+        torch.cuda.synchronize()
+    except Exception:
+        pass
+    lib = load_library()
+    while _cu_stream_handles:
+        lib.hc_stream_destroy(_c_p(_cu_stream_handles.pop()))
+
+
 def cu_limited_stream(n_cus, device):
     """A torch stream (default priority) whose kernels run on ``n_cus`` compute units only, spread over the
     chip: for work that waits on the host link beside compute (``PinnedFeatureStore.prefetch``).  The
-    stream lives until the process ends."""
+    stream lives until the interpreter exits."""
     lib = load_library()
     device = torch.device(device)
     handle = ctypes.c_void_p()
     with torch.cuda.device(device):
         _check(lib.hc_stream_create_cu_limited(int(n_cus), ctypes.cast(ctypes.pointer(handle), _c_p)),
                "hc_stream_create_cu_limited")
+    if not _cu_stream_handles:
+        import atexit
+        atexit.register(_destroy_cu_streams)
+    _cu_stream_handles.append(handle.value)
     return torch.cuda.ExternalStream(handle.value, device=device)
 
 
