@@ -24,7 +24,9 @@ class NeighborSampler:
         every batch also carries ``batch.view``, the transposed view of its CSR
         (``hiscache_backend.BatchView``), built right behind the sampling on the sampler's stream, so
         that the layers' backward builds none; ``view_edges`` adds the view's edge slots, which the
-        relational layer's backward reads."""
+        relational layer's backward reads.  (The view is built with the batch's sizes still on the device,
+        for batches whose capacity -- seeds x the fanouts' products -- stays below 2^24 edges and nodes;
+        beyond that the sampling call raises and the batch must come without a view.)"""
         self.emit_view = bool(emit_view)
         self.view_edges = bool(view_edges)
         self.device = torch.device(device)
