@@ -305,8 +305,16 @@ __global__ __launch_bounds__(HC_BLOCK) void tc_edge_types(const int64_t *__restr
                                                            const int64_t *__restrict__ bounds, int n_bounds,
                                                            const int64_t *__restrict__ pair_to_rel,
                                                            int64_t *__restrict__ out, int64_t R, int64_t E,
-                                                           int64_t n_all) {
+                                                           int64_t n_all, int64_t row_blocks) {
   const int lane = hc_lane();
+  if ((int64_t)blockIdx.x >= row_blocks) {
+    // the blocks behind the rows' blocks: edge slots that no row of the block owns get -1
+    const int64_t nb = (int64_t)gridDim.x - row_blocks;
+    const int64_t start = R > 0 ? ptr[R] : 0;
+    for (int64_t e = start + ((int64_t)blockIdx.x - row_blocks) * HC_BLOCK + threadIdx.x; e < E; e += nb * HC_BLOCK)
+      out[e] = -1;
+    return;
+  }
   const int64_t row = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
   if (row >= R) return;
   const int64_t begin = ptr[row];
@@ -330,11 +338,13 @@ extern "C" int hc_edge_types_by_ranges(const int64_t *ptr, const int64_t *idx, c
                                        void *stream) {
   HC_REQUIRE(R >= 0 && E >= 0 && n_all >= 0 && n_bounds >= 0);
   if (n_bounds > TC_MAX_BOUNDS) return HC_EUNSUPPORTED;
-  if (R == 0 || E == 0) return HC_OK;
-  HC_REQUIRE(ptr && idx && sub_to_full && pair_to_rel && out && (n_bounds == 0 || bounds));
+  if (E == 0) return HC_OK;
+  HC_REQUIRE(out != nullptr);
+  if (R > 0) HC_REQUIRE(ptr && idx && sub_to_full && pair_to_rel && (n_bounds == 0 || bounds));
   const int64_t blocks = (R + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
-  if (!hc_grid_ok(blocks)) return HC_EUNSUPPORTED;
-  tc_edge_types<<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, static_cast<hipStream_t>(stream)>>>(
-      ptr, idx, sub_to_full, bounds, n_bounds, pair_to_rel, out, R, E, n_all);
+  const int64_t tail_blocks = 32;   // grid-stride over the slots behind the last row (usually none)
+  if (!hc_grid_ok(blocks + tail_blocks)) return HC_EUNSUPPORTED;
+  tc_edge_types<<<dim3((unsigned)(blocks + tail_blocks)), dim3(HC_BLOCK), 0, static_cast<hipStream_t>(stream)>>>(
+      ptr, idx, sub_to_full, bounds, n_bounds, pair_to_rel, out, R, E, n_all, blocks);
   return hc_launch_status();
 }

@@ -366,8 +366,9 @@ class _RgcnConvFunction(torch.autograd.Function):
     the weighted aggregation's transposed view."""
 
     @staticmethod
-    def forward(ctx, x, weight, ptr, idx, edge_types, used_mask, hmap, hbuf, num_node, view=None):
+    def forward(ctx, x, weight, ptr, idx, edge_types, used_mask, hmap, hbuf, num_node, view=None, sink=None):
         be = hiscache_backend
+        ctx.sink = sink
         R = int(num_node)
         K, Fin, H = weight.shape
         ptr2, idx2, _cnt, _deg, w2 = be.typed_csr(ptr, idx, edge_types, K, R, x.shape[0], used_mask,
@@ -392,6 +393,10 @@ class _RgcnConvFunction(torch.autograd.Function):
         R, has_hit, E = ctx.hc
         K, Fin, H = weight.shape
         g = g.contiguous()
+        if ctx.sink is not None and ctx.sink.target is not None:
+            his = ctx.sink.target()
+            if his is not None:
+                his.grad = g                          # what retain_grad() would keep, without its copy
         if has_hit:                                   # rows taken from the history pass nothing back
             g = g.masked_fill(hit, 0.0)
         g_w = _rel_weight_grad(agg, g) if ctx.needs_input_grad[1] else None
@@ -408,7 +413,7 @@ class _RgcnConvFunction(torch.autograd.Function):
                                          want_hist_grad=False)
             if g_x.dtype != x.dtype:
                 g_x = g_x.to(x.dtype)
-        return g_x, g_w, None, None, None, None, None, None, None, None
+        return g_x, g_w, None, None, None, None, None, None, None, None, None
 
 
 class MyRGCNConvHistory2(torch.nn.Module):
@@ -453,12 +458,15 @@ class MyRGCNConvHistory2(torch.nn.Module):
         self._count_of = edge_types
         use_hist = history_size > 0 and history_map is not None and history_map.numel() > 0
         if self.fused and x.is_cuda and not (use_hist and history_buffer.requires_grad):
+            # the gradient that reaches the layer's output is handed to ``his.grad`` by the node's backward
+            sink = _GradSink() if (self.need_grad and self.training and history_size > 0) else None
             out = _RgcnConvFunction.apply(x, self.linear, ptr, idx, edge_types, used_mask,
                                           history_map if use_hist else None,
-                                          history_buffer if use_hist else None, num_node, view)
+                                          history_buffer if use_hist else None, num_node, view, sink)
             his = out
-            if self.need_grad and self.training and history_size > 0:
-                his.retain_grad()
+            if sink is not None:
+                sink.target = weakref.ref(his)
+                his._hc_grad_sink = True
             return out, his
         ptr2, idx2, cnt, deg = typed_csr(ptr, idx, edge_types, K, num_node, used_mask, n_src=x.shape[0])
         none = torch.empty(0, device=x.device)
@@ -543,7 +551,8 @@ class HistoryRGCN(torch.nn.Module):
                 x, his = conv(x, batch.ptr, batch.idx, et, None, self.table.sub2embed,
                               self.table.cached_embedding, um, self.hidden_channels, n, view=view)
                 self.table.produced_embedding = his
-                self.table.produced_embedding.retain_grad()
+                if not getattr(his, "_hc_grad_sink", False):
+                    self.table.produced_embedding.retain_grad()
             else:
                 x, his = conv(x, batch.ptr, batch.idx, et, None, none, none, um, 0, n, view=view)
             x = bn_relu(x, self.bns[i], None, fused=self.fused_epilogue)

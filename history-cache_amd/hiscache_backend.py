@@ -952,7 +952,7 @@ def edge_types_by_ranges(ptr, idx, sub_to_full, num_node, bounds, pair_to_rel):
     R = int(num_node)
     if ptr.numel() < R + 1:
         raise ValueError("ptr is shorter than num_node + 1")
-    out = torch.full((idx.numel(),), -1, dtype=torch.int64, device=idx.device)
+    out = torch.empty(idx.numel(), dtype=torch.int64, device=idx.device)      # the call writes every entry
     rc = lib.hc_edge_types_by_ranges(_ptr(ptr), _ptr(idx), _ptr(sub_to_full), sub_to_full.numel(), _ptr(bounds),
                                      int(bounds.numel()), _ptr(pair_to_rel), _ptr(out), R, idx.numel(), _stream())
     _check(rc, "hc_edge_types_by_ranges")

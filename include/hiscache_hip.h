@@ -415,8 +415,8 @@ int hc_typed_csr(const int64_t *ptr, const int64_t *idx, const int64_t *edge_typ
  * (node types stored as consecutive full-id ranges, as mag240M stores papers,
  * authors and institutions).  Stands in for cxgnncomp_backend.gen_edge_type_mag240m
  * (called at hiscache/history_model.py:356), which is not part of the
- * reference repository.  Edge slots at or beyond ptr[R] (or E) are left as
- * they are; a source outside [0, n_all) gets -1.  n_bounds <= 64. */
+ * reference repository.  Edge slots in [ptr[R], E) are set to -1 (out needs no
+ * initialisation); a source outside [0, n_all) gets -1.  n_bounds <= 64. */
 int hc_edge_types_by_ranges(const int64_t *ptr, const int64_t *idx, const int64_t *sub_to_full,
                             int64_t n_all, const int64_t *bounds, int n_bounds,
                             const int64_t *pair_to_rel, int64_t *out, int64_t R, int64_t E,
