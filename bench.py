@@ -491,8 +491,12 @@ def c3_batched_layer(args, samples=None):
     hdr = torch.zeros(1, dtype=torch.int64, device=dev)
     sub_to_full = torch.randperm(2 * R, device=dev, generator=gen)[:R].contiguous()
     thr = torch.tensor([0.05], device=dev)
-    cf, ct, cb, cg = KernelClock(), KernelClock(), KernelClock(), KernelClock()
+    cf, ct, cb, cg, cv = KernelClock(), KernelClock(), KernelClock(), KernelClock(), KernelClock()
     st = {}
+    # the view of the whole block with nothing left out, as a loader emits it with a batch (built once, outside
+    # the time): the backward over it steps over the history rows' edges in the kernel; reported beside the figures
+    # of the step above, whose time includes the view it builds
+    shared_view = be.build_batch_view(ptr, idx, R, Nsrc)
 
     def kstep():
         cf(lambda: be._aggr_fwd(be.SUBST_ROW, ptr, idx, x, hmap, hbuf, H, None, R))
@@ -502,11 +506,12 @@ def c3_batched_layer(args, samples=None):
         hdr.zero_()
         st["mask"] = cg(lambda: be.grad_check(grad, emb, hmap, sub_to_full, thr, table, f2s, s2f, hdr, 1,
                                               checkin=chk))[0]
+        cv(lambda: be._aggr_bwd_batch_view(ptr, shared_view, g, hmap, None, H, R, Nsrc, want_hist_grad=False))
 
     for _ in range(args.warmup):
         kstep()
     sync()
-    for c in (cf, ct, cb, cg):
+    for c in (cf, ct, cb, cg, cv):
         c.reset()
     for _ in range(args.steps):
         kstep()
@@ -527,6 +532,10 @@ def c3_batched_layer(args, samples=None):
         "edges_per_s_fwd_bwd": E / ((t_f + t_t + t_b) * 1e-3),
         "algorithmic_bytes": tot_b, "ms": tot_t * 1e3, "frac": tot_b / tot_t / 1e9 / HBM_PEAK_GBS,
         "traffic": MEASURED_TRAFFIC["c3_batched"] if s == 1.0 else None,
+        # beside it: the same layer when the batch comes with its view (no build in the step; backward over the
+        # whole block's view)
+        "bwd_over_emitted_view_ms": cv.mean_ms(),
+        "frac_with_emitted_view": tot_b / ((t_f + cv.mean_ms() + t_g) * 1e-3) / 1e9 / HBM_PEAK_GBS,
     }
     roofline = {"bound": "hbm",
                 "kernel": "fwd_mean_fast + transposed view + bwd_mean_fast + gc_pass1..3 (batched history layer)",
