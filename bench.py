@@ -55,6 +55,8 @@ def parse():
                          "the rows that the cache's state at that moment makes necessary (fixed up at the lookup)")
     ap.add_argument("--prefetch-cus", type=int, default=16,
                     help="with --prefetch: compute units the read-ahead's stream may use (0: an ordinary stream)")
+    ap.add_argument("--prefetch-depth", type=int, default=1,
+                    help="with --prefetch and --with-sampler: batches whose feature read is under way")
     ap.add_argument("--prefetch-all", action="store_true",
                     help="with --prefetch: read every row of the next batch and mask at the lookup")
     ap.add_argument("--no-batch-view", action="store_true",
@@ -642,7 +644,7 @@ def run_c3(args, with_batched=True):
     store.prefold(batches)
     ev = {k: KernelClock() for k in ("load", "forward", "backward", "step", "update")}
     state = {"it": 0}
-    sampled = {"sampler": None, "pending": None, "ahead": None, "shapes": [], "wait_s": 0.0, "E_graph": 0}
+    sampled = {"sampler": None, "pending": None, "ahead": [], "shapes": [], "wait_s": 0.0, "E_graph": 0}
     if args.with_sampler:
         # batches come from the device sampler over a graph of the same size held in HBM; batch i+1 is
         # sampled on the sampler's side stream while batch i trains
@@ -671,19 +673,21 @@ def run_c3(args, with_batched=True):
             return batches[i % n_pre]
         if not args.prefetch:
             return sampled_batch(i)
-        # two batches deep: batch i was taken from the sampler one iteration ago, when its feature read started
-        if sampled["ahead"] is None:
-            sampled["ahead"] = sampled_batch(i)
-        return sampled["ahead"]
+        # batch i was taken from the sampler --prefetch-depth iterations ago, when its feature read started
+        if not sampled["ahead"]:
+            return sampled_batch(i)
+        return sampled["ahead"].pop(0)
 
     def start_prefetch():
-        """The next batch's host-link read, under the masks of the cache's present state (--prefetch-all: every
-        row), runs beside this batch's forward and backward."""
+        """The host-link read of the next batch (of the next --prefetch-depth batches), under the masks of the
+        cache's present state (--prefetch-all: every row), runs beside this batch's forward and backward."""
         if sampled["sampler"] is None:
-            nxt = batches[state["it"] % n_pre]
-        else:
-            nxt = sampled["ahead"] = sampled_batch(state["it"])
-        cache.prefetch(nxt, speculative=not args.prefetch_all)
+            cache.prefetch(batches[state["it"] % n_pre], speculative=not args.prefetch_all)
+            return
+        while len(sampled["ahead"]) < args.prefetch_depth:
+            nxt = sampled_batch(state["it"] + len(sampled["ahead"]))
+            cache.prefetch(nxt, speculative=not args.prefetch_all)
+            sampled["ahead"].append(nxt)
 
     def step():
         state["it"] += 1
