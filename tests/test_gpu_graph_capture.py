@@ -19,6 +19,8 @@ def be():
 
 
 def test_aggregation_and_admission_replay_like_eager(be):
+    if be.CHECK_INPUTS:
+        pytest.skip("HISCACHE_CHECK_INPUTS=1 validates every block with a read-back, which cannot be captured")
     rng = np.random.default_rng(90)
     R, N, F, cap = 3000, 2500, 128, 4096
     ptr, idx = random_csr(rng, R, N, 9, hub=700)
