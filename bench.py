@@ -13,7 +13,8 @@ with PyTorch CPU index_add, timed on this machine's host cores on a 1/10-size sa
 
 The default line also carries the admission microbenchmark (c4), the papers100M-shaped history layer
 batched to 20 M edges (kernels.c3_batched) and the per-iteration time of the papers100M- and
-mag240M-shaped training iterations at their real batch shapes (iterations.c3, iterations.c5) and of the
+mag240M-shaped training iterations at their real batch shapes (iterations.c3, iterations.c5), of the
+CPU-runnable plumbing configuration beside its PyTorch CPU spelling (iterations.c1) and of the
 papers100M-shaped one fed by the device sampler with the features read one batch ahead (iterations.c3_sampled);
 --headline-only leaves them out.
 Other workloads (--workload c4 | c2row | c3 | c5 ...) print their own line and are not the headline.
@@ -62,7 +63,7 @@ def parse():
     ap.add_argument("--no-batch-view", action="store_true",
                     help="c3/c5: batches come without the transposed view of their CSR, so every layer's "
                          "backward builds one (the default: the loader emits it with the batch)")
-    ap.add_argument("--workload", default="c2", choices=["c2", "c2row", "c2w", "c4", "c3", "c3b", "c5", "sample", "layer", "copy", "ceilings"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c2row", "c2w", "c4", "c3", "c3b", "c5", "sample", "layer", "copy", "ceilings"])
     ap.add_argument("--heads", type=int, default=1, help="c2w: heads of the weighted aggregation (divides 256)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--reps", type=int, default=8, help="c3b: measurements with freshly allocated tensors")
@@ -861,6 +862,117 @@ def run_c5(args):
     }
 
 
+def run_c1(args):
+    """The CPU-runnable plumbing configuration (`configs[0]`): uniform graph of 100 k nodes, mean out-degree 15,
+    128-dim fp32 features, 10 classes, 2-layer SAGE hidden 128, 1000 seeds, fanout [10, 5], fp32 history table
+    100 k x 128 with a random 30% of the nodes cached.  Per-iteration time of sampling (one batch ahead, view
+    emitted) -> lookup_and_load -> forward / backward -> optimizer -> admission on the GPU, and of the same
+    iteration with stock PyTorch CPU operators over the same batches (`oracle/torch_cpu_path.py`)."""
+    import copy
+
+    import numpy as np
+    import torch
+
+    from hiscache import HistorySAGE, NeighborSampler, PinnedFeatureStore, RingHistoryCache, make_config, prefer_low_latency_gemm
+    from hiscache.synthetic import uniform_graph
+
+    dev = "cuda:0"
+    N, Fin, H, C, L, n_seed, fanout, rate = 100_000, 128, 128, 10, 2, 1000, [10, 5], 0.5
+    rng = np.random.default_rng(1)
+    torch.manual_seed(1)
+    indptr, indices = uniform_graph(N, 15, 1)
+    feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32))
+    labels = torch.from_numpy(rng.integers(0, C, size=N))
+    cached = torch.from_numpy(rng.permutation(N)[: int(0.3 * N)].copy())
+    rows = torch.from_numpy(rng.standard_normal((cached.numel(), H)).astype(np.float32))
+    cache = RingHistoryCache(PinnedFeatureStore(feats, device=dev), N, Fin, H, capacity=N, num_layers=L,
+                             table_dtype=torch.float32, rate=rate, age_limit=AGE_LIMIT_ITERS, device=dev)
+    cache.preload(cached.to(dev), rows.to(dev))
+    prefer_low_latency_gemm()
+    model = HistorySAGE(Fin, H, C, L, 0.0, "CSR_Layer", make_config(Fin, C, H, L, device=dev), cache).to(dev)
+    model.train()
+    cpu_model = None
+    if not args.no_cpu_baseline:
+        table, model.table = model.table, None
+        cpu_model = copy.deepcopy(model).cpu()
+        model.table = table
+    opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True)
+    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=1, device=dev, validate=False,
+                              emit_view=not args.no_batch_view)
+    gen = torch.Generator(device=dev).manual_seed(1)
+    seed_pool = torch.randperm(N, device=dev, generator=gen)[: n_seed * 64].view(64, n_seed).contiguous()
+    ev = {k: KernelClock() for k in ("load", "forward", "backward", "step", "update")}
+    state = {"it": 0, "pending": sampler.sample_async(seed_pool[0]), "shapes": [], "kept": []}
+
+    def step():
+        state["it"] += 1
+        b = state["pending"].get()
+        state["pending"] = sampler.sample_async(seed_pool[state["it"] % 64])
+        state["shapes"].append(b.num_node_in_layer.tolist() + [b.idx.numel()])
+        if len(state["kept"]) < 8:
+            state["kept"].append(b)
+        ev["load"](lambda: cache.lookup_and_load(b, L))
+        out = ev["forward"](lambda: model(b))
+        loss = torch.nn.functional.nll_loss(out, b.y)
+        opt.zero_grad(set_to_none=True)
+        ev["backward"](lambda: loss.backward())
+        ev["step"](lambda: opt.step())
+        ev["update"](lambda: cache.update_history(b, state["it"]))
+
+    for _ in range(args.warmup):
+        step()
+    sync()
+    for c in ev.values():
+        c.reset()
+    state["shapes"] = []
+    gc.collect()
+    gc.freeze()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    sync()
+    sec = (time.perf_counter() - t0) / args.steps
+    gc.unfreeze()
+    state["pending"].get()
+    m = np.mean(np.asarray(state["shapes"], dtype=np.float64), axis=0)
+    res = {
+        "metric": "plumbing-configuration iteration ms (1 GPU)", "value": sec * 1e3, "unit": "ms", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "c1: 100000 nodes, mean out-degree 15, 2-layer SAGE hidden 128, fanout [10,5], batch 1000, "
+                               "fp32 history table 100000 x 128 (30%% of the nodes cached), features 128-dim fp32 in pinned "
+                               "host memory read zero-copy, batches from the device sampler; mean batch n0 %d, n1 %d, "
+                               "n2 %d, %d edges" % tuple(int(v) for v in m)},
+        "phases_ms": {k: c.mean_ms() for k, c in ev.items()},
+        "phases_host_enqueue_ms": {k: c.mean_cpu_ms() for k, c in ev.items()},
+        "transposed_view": "built in backward" if args.no_batch_view else "emitted with the batch",
+    }
+    if cpu_model is not None:
+        # the same iteration with stock PyTorch CPU operators, over batches the GPU loop trained on
+        from oracle import torch_cpu_path as tp
+        cpu_model.train()
+        cpu_opt = torch.optim.Adam(cpu_model.parameters(), lr=1e-3)
+        ring = tp.ring_state(N, N, H)
+        ring["table"][: cached.numel()] = rows
+        ring["f2s"][cached] = torch.arange(cached.numel())
+        ring["s2f"][: cached.numel()] = cached
+        ring["checkin"][: cached.numel()] = 0
+        ring["header"] = cached.numel() % N
+        cpu_batches = [dict(ptr=b.ptr.cpu().numpy(), idx=b.idx.cpu().numpy(), sub_to_full=b.sub_to_full.cpu().numpy(),
+                            num_node_in_layer=b.num_node_in_layer.numpy(), y=b.y.cpu()) for b in state["kept"]]
+        torch.set_num_threads(os.cpu_count() or 1)
+        tp.sage_iteration(cpu_model, cpu_opt, cpu_batches[0], feats, ring, 1, rate)          # warm-up
+        t0 = time.perf_counter()
+        for k, cb in enumerate(cpu_batches[1:], start=2):
+            tp.sage_iteration(cpu_model, cpu_opt, cb, feats, ring, k, rate)
+        cpu_ms = (time.perf_counter() - t0) / max(len(cpu_batches) - 1, 1) * 1e3
+        res["cpu_baseline"] = {"value": cpu_ms, "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": "%d iterations of the same configuration over batches the GPU loop trained on, "
+                                         "stock PyTorch CPU operators (index_add aggregation, torch.quantile admission; "
+                                         "used masks by the sequential C statement)" % max(len(cpu_batches) - 1, 1)}
+    return res
+
+
 def run_layer(args):
     """The dense side of a sampled layer: weight gradients (hc_weight_grad against the library GEMM and its
     slab-batched spelling) and the bias + batch norm + ReLU epilogue (hc_bn_relu against torch's operators), at
@@ -1120,8 +1232,8 @@ def main():
             # (batches of about 236 k edges), features read one batch ahead on a CU-limited stream
             sm_args = argparse.Namespace(**vars(it_args))
             sm_args.with_sampler, sm_args.prefetch = True, True
-            for name, fn in (("c3", lambda: run_c3(it_args, with_batched=False)), ("c5", lambda: run_c5(it_args)),
-                             ("c3_sampled", lambda: run_c3(sm_args, with_batched=False))):
+            for name, fn in (("c1", lambda: run_c1(it_args)), ("c3", lambda: run_c3(it_args, with_batched=False)),
+                             ("c5", lambda: run_c5(it_args)), ("c3_sampled", lambda: run_c3(sm_args, with_batched=False))):
                 gc.collect()
                 torch.cuda.empty_cache()
                 r = fn()
@@ -1130,6 +1242,9 @@ def main():
                     "warmup": r["warmup"], "transposed_view": r["transposed_view"],
                     "feature_read_ahead": bool(getattr(sm_args if name == "c3_sampled" else it_args, "prefetch")),
                     "phases_ms": r["phases_ms"], "phases_host_enqueue_ms": r["phases_host_enqueue_ms"]}
+                if "cpu_baseline" in r:          # c1, the CPU-runnable configuration: the same iteration on the host
+                    res["iterations"][name]["cpu_ms"] = r["cpu_baseline"]["value"]
+                    res["iterations"][name]["cpu_cores"] = r["cpu_baseline"]["cores"]
             gc.collect()
             torch.cuda.empty_cache()
         if not args.no_cpu_baseline:
@@ -1148,6 +1263,8 @@ def main():
         res = run_copy(args)
     elif args.workload == "c5":
         res = run_c5(args)
+    elif args.workload == "c1":
+        res = run_c1(args)
     elif args.workload == "sample":
         res = run_sample(args)
     else:

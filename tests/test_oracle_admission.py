@@ -700,3 +700,43 @@ def test_evict_by_both_brute_force():
         np.testing.assert_array_equal(t[2].numpy(), want_f2h)
         np.testing.assert_array_equal(t[0].numpy(), want_chk)
         assert 0 < len(model) < 45
+
+
+def test_cpu_iteration_of_the_plumbing_configuration(orc):
+    """oracle/torch_cpu_path.sage_iteration (the CPU side of `bench.py --workload c1`): the ring it maintains
+    stays consistent over iterations that wrap it, admitted rows hold the layer's output, and its admission of
+    cached rows are never admitted again."""
+    import copy
+    from types import SimpleNamespace
+
+    from helpers import layered_batch
+    from hiscache import HistorySAGE, make_config       # the model classes need torch only; no GPU is touched
+    from oracle import torch_cpu_path as tp
+    rng = np.random.default_rng(3)
+    torch.manual_seed(3)
+    N, Fin, H, C, L = 600, 16, 16, 4, 2                 # in a 2-layer model the cached rows have the input width
+    feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32))
+    table = SimpleNamespace(method="grad")
+    model = HistorySAGE(Fin, H, C, L, 0.0, "CSR_Layer", make_config(Fin, C, H, L, device="cpu"), table)
+    model.table = None
+    model = copy.deepcopy(model).train()
+    opt = torch.optim.Adam(model.parameters(), lr=1e-2)
+    cap = 150                                            # small ring: it wraps
+    ring = tp.ring_state(N, cap, H)
+    losses = []
+    for it in range(1, 9):
+        b = layered_batch(rng, N, 30, [5, 4])
+        b["y"] = torch.from_numpy(rng.integers(0, C, size=30))
+        n1 = int(b["num_node_in_layer"][1])
+        before = {k: (v.clone() if torch.is_tensor(v) else v) for k, v in ring.items()}
+        losses.append(tp.sage_iteration(model, opt, b, feats, ring, it, 0.5))
+        # every mapped node points at a slot that points back; slots written now carry this iteration
+        live = torch.nonzero(ring["f2s"] != -1).view(-1)
+        assert torch.equal(ring["s2f"][ring["f2s"][live]], live)
+        new = torch.nonzero(ring["checkin"] == it).view(-1)
+        assert new.numel() > 0 and (ring["header"] - before["header"]) % cap == new.numel() % cap
+        ids1 = torch.from_numpy(b["sub_to_full"][:n1])
+        assert bool(torch.isin(ring["s2f"][new], ids1).all())
+        assert not bool((before["f2s"][ring["s2f"][new]] != -1).any())     # cached rows are not admitted again
+    assert all(np.isfinite(losses))
+    assert int((ring["checkin"] != -1).sum()) == cap                       # the ring filled up and wrapped
