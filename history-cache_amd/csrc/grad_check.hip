@@ -823,3 +823,93 @@ extern "C" int hc_evict(const int64_t *sub2slot, const float *score, const float
   return hc_launch_status();
 }
 
+
+// ---------------------------------------------------------------------------------------
+// Admission threshold as a quantile of the scores: the two order statistics that
+// torch.quantile's linear interpolation reads (/root/reference/hiscache/history_cache.py:211,
+// history_table.py:173), found by a radix select instead of a sort, and the interpolation in
+// separately rounded fp32 steps.  One block; four 8-bit passes per order statistic over keys
+// that order like the floats (sign flipped for non-negative values, all bits for negative
+// ones).  Up to QT_MAX_N scores (a sampled batch's 1-hop nodes are a few thousand).
+// ---------------------------------------------------------------------------------------
+namespace {
+
+constexpr int QT_BLOCK = 1024;
+constexpr int64_t QT_MAX_N = 1 << 17;
+
+__device__ __forceinline__ uint32_t qt_key(float v) {
+  const uint32_t b = __float_as_uint(v);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float qt_value(uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+// the key of rank k (0-based) among score[0, n); every thread returns it
+__device__ uint32_t qt_select(const float *__restrict__ score, int64_t n, int64_t k, int *hist, int *s_pick) {
+  uint32_t prefix = 0u, mask = 0u;
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    for (int b = threadIdx.x; b < 256; b += QT_BLOCK) hist[b] = 0;
+    __syncthreads();
+    for (int64_t i = threadIdx.x; i < n; i += QT_BLOCK) {
+      const uint32_t key = qt_key(score[i]);
+      if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 0xffu], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x < HC_WAVE) {
+      // the bin that holds rank k: the first wave scans the 256 counts, four bins per lane
+      const int l = (int)threadIdx.x;
+      const int c[4] = {hist[4 * l], hist[4 * l + 1], hist[4 * l + 2], hist[4 * l + 3]};
+      const int mine = (c[0] + c[1]) + (c[2] + c[3]);
+      int x = mine;
+#pragma unroll
+      for (int d = 1; d < HC_WAVE; d <<= 1) {
+        const int y = __shfl_up(x, d, HC_WAVE);
+        if (l >= d) x += y;
+      }
+      const unsigned long long reached = __ballot((int64_t)x > k);
+      const int owner = reached != 0ull ? __builtin_ctzll(reached) : HC_WAVE - 1;
+      if (l == owner) {
+        int before = x - mine, b = 0;
+        for (; b < 3; ++b) {
+          if ((int64_t)before + c[b] > k) break;
+          before += c[b];
+        }
+        s_pick[0] = 4 * l + b;
+        s_pick[1] = before;           // at most n < 2^31
+      }
+    }
+    __syncthreads();
+    prefix |= (uint32_t)s_pick[0] << shift;
+    mask |= 0xffu << shift;
+    k -= s_pick[1];
+    __syncthreads();
+  }
+  return prefix;
+}
+
+__global__ __launch_bounds__(QT_BLOCK) void quantile_kernel(const float *__restrict__ score, int64_t n, int64_t lo,
+                                                             int64_t hi, float w, float one_minus_w,
+                                                             float *__restrict__ out) {
+  __shared__ int hist[256];
+  __shared__ int s_pick[2];
+  const float a = qt_value(qt_select(score, n, lo, hist, s_pick));
+  const float b = hi == lo ? a : qt_value(qt_select(score, n, hi, hist, s_pick));
+  if (threadIdx.x == 0) {
+    const float d = __fsub_rn(b, a);
+    out[0] = w < 0.5f ? __fadd_rn(a, __fmul_rn(d, w)) : __fsub_rn(b, __fmul_rn(d, one_minus_w));
+  }
+}
+
+}  // namespace
+
+extern "C" int64_t hc_quantile_max_scores(void) { return QT_MAX_N; }
+
+extern "C" int hc_quantile_threshold(const float *score, int64_t n, int64_t lo, int64_t hi, float w,
+                                     float one_minus_w, float *out, void *stream) {
+  HC_REQUIRE(score && out && n >= 1 && lo >= 0 && hi >= lo && hi < n && hi <= lo + 1);
+  if (n > QT_MAX_N) return HC_EUNSUPPORTED;
+  quantile_kernel<<<dim3(1), dim3(QT_BLOCK), 0, static_cast<hipStream_t>(stream)>>>(score, n, lo, hi, w,
+                                                                                   one_minus_w, out);
+  return hc_launch_status();
+}

@@ -246,6 +246,20 @@ int hc_count_history(const int64_t *ptr, const int64_t *idx, const int64_t *hmap
  * partner distance 32,16,8,4,2,1; L2 takes sqrtf (correctly rounded). */
 int hc_row_scores(const float *grad, float *score, int64_t M, int64_t F, int norm_kind, void *stream);
 
+/* hc_quantile_threshold: the admission threshold `torch.quantile(score, rate)`
+ * (hiscache/history_cache.py:211, hiscache/history_table.py:173) without a
+ * sort: out[0] = a + w*(b - a) for w < 0.5, else b - (b - a)*one_minus_w, where
+ * a and b are the order statistics of rank lo and hi (0-based, hi = lo or
+ * lo + 1) of score[0, n) and every step is rounded to fp32 on its own -- the
+ * caller works out lo, hi and w from rate and n the way torch.quantile does
+ * (pos = fp32(rate) * fp32(n - 1), lo = floor(pos), w = pos - lo).  One launch
+ * (a radix select by one block); n <= hc_quantile_max_scores(), else
+ * HC_EUNSUPPORTED (sort instead).  NaN scores rank behind +inf, as in a sort;
+ * -0 ranks in front of +0. */
+int64_t hc_quantile_max_scores(void);
+int hc_quantile_threshold(const float *score, int64_t n, int64_t lo, int64_t hi, float w,
+                          float one_minus_w, float *out, void *stream);
+
 /* hc_grad_check: the fused admission pass.  Replaces record_history
  * (grad_check.h:12-16, grad_check.cu:6-68) and the torch sequence of
  * HistoryCache.update_history (hiscache/history_cache.py:205-221,243-254).

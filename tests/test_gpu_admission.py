@@ -190,3 +190,27 @@ def test_small_helpers(be, orc):
     np.testing.assert_array_equal(got16.float().cpu().numpy(), orc.gather_rows(host.float().numpy(), ids, mask))
     m = rng.integers(-1, 99, size=1000)
     np.testing.assert_array_equal(be.lookup(T(m), T(ids), 3).cpu().numpy(), m[ids + 3])
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 257, 5800, 1 << 17, (1 << 17) + 1])
+def test_quantile_threshold_by_selection_equals_the_sort(n):
+    """hc_quantile_threshold (radix select of the two order statistics + the interpolation, one launch) gives
+    the bits of the sorted spelling -- which is torch.quantile's rule, pinned on the CPU side -- for rates
+    over [0, 1], negative scores, ties, infinities; above the kernel's size limit the sort runs instead."""
+    from hiscache.util import quantile_threshold
+    rng = np.random.default_rng(n)
+    cases = [rng.standard_normal(n), np.abs(rng.standard_normal(n)) * np.exp(rng.normal(-3, 1.5, size=n)),
+             rng.integers(0, 4, size=n).astype(np.float64), np.full(n, 0.25)]
+    if n > 3:
+        wild = rng.standard_normal(n)
+        wild[:2] = [np.inf, -np.inf]
+        cases.append(wild)
+    for s in cases:
+        s32 = s.astype(np.float32)
+        dev = torch.from_numpy(s32).to(DEV)
+        for rate in (0.0, 0.1, 0.5, 0.7, 0.9, 0.999, 1.0):
+            got = quantile_threshold(dev, rate)
+            want = quantile_threshold(torch.from_numpy(s32), rate)
+            assert got.is_cuda and got.shape == (1,)
+            np.testing.assert_array_equal(got.cpu().numpy().view(np.uint32), want.numpy().view(np.uint32),
+                                          err_msg=f"n={n} rate={rate}")
