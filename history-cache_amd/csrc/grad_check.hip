@@ -839,6 +839,7 @@ constexpr int64_t QT_MAX_N = 1 << 17;
 
 __device__ __forceinline__ uint32_t qt_key(float v) {
   const uint32_t b = __float_as_uint(v);
+  if (v != v) return 0xffffffffu;        // NaN of either sign ranks last, as a sort places it
   return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
 __device__ __forceinline__ float qt_value(uint32_t k) {

@@ -144,6 +144,30 @@ def test_c2_backward_over_the_whole_block_view_has_the_same_bits(c2):
     assert torch.equal(got, want)
 
 
+def test_c2_every_row_has_the_bits_of_the_cpu_statement(c2):
+    """All 1 M output rows, the whole transposed view and all 10 M gradient rows of the full-size block against
+    the OpenMP CPU statement (which tests/test_oracle_aggr.py holds to the sequential oracle's bits at small
+    sizes): bit for bit.  About 35 GB of host memory at the peak."""
+    import hiscache_backend as be
+    from oracle import hc_cpu_mt as mt
+    ptr, idx = c2["ptr"].cpu().numpy(), c2["idx"].cpu().numpy()
+    feat, hist, hmap = c2["feat"].cpu().numpy(), c2["hist"].cpu().numpy(), c2["hmap"].cpu().numpy()
+    print("c2 block on the host,", mt.num_threads(), "threads", flush=True)
+    want = mt.fwd_mean_src(ptr, idx, feat, hmap, hist, split_above=be.long_row_edges(F))
+    got = c2["out"].cpu().numpy()
+    bad = int((got.view(np.uint32) != want.view(np.uint32)).any(axis=1).sum())
+    assert bad == 0, f"{bad} forward rows differ"
+    del feat, hist, want, got
+    ptrT, rowT = mt.build_transpose(ptr, idx, N)
+    assert np.array_equal(c2["tr"][0].cpu().numpy(), ptrT)
+    assert np.array_equal(c2["tr"][1].cpu().numpy()[:E], rowT[:E])
+    print("c2 view equal", flush=True)
+    want = mt.bwd_mean(ptr, ptrT, rowT, c2["g"].cpu().numpy(), N, chunk=be.bwd_chunk_edges(F))
+    got = c2["grad_x"].cpu().numpy()
+    bad = int((got.view(np.uint32) != want.view(np.uint32)).any(axis=1).sum())
+    assert bad == 0, f"{bad} gradient rows differ"
+
+
 def test_c4_admission_full_size():
     """2 M rows x 256, fp16 table 50 M x 256: mask == predicate on the kernel's own scores, slots ==
     header + exclusive prefix sum of the mask, table rows == fp16(embedding), maps consistent."""
@@ -176,6 +200,11 @@ def test_c4_admission_full_size():
     assert torch.equal(mask, want)
     A = int(mask.sum())
     assert 700_000 < A < 950_000
+    # all 2 M scores have the bits of the CPU statement's summation order (portable build: separately rounded
+    # multiplies and adds, which tests/test_oracle_admission.py holds to the sequential oracle)
+    from oracle import hc_cpu_mt as mt
+    cpu_score = mt.score_rows(grad.cpu().numpy(), hw=False)
+    assert np.array_equal(score.cpu().numpy().view(np.uint32), cpu_score.view(np.uint32))
     rank = torch.cumsum(mask.long(), 0) - mask.long()
     want_slot = torch.where(mask, (cap - 300_000 + rank) % cap, torch.full_like(rank, -1))
     assert torch.equal(slot_out, want_slot)
