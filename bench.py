@@ -25,6 +25,7 @@ import json
 import os
 import sys
 import time
+import types
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
@@ -60,6 +61,13 @@ def parse():
                     help="with --prefetch and --with-sampler: batches whose feature read is under way")
     ap.add_argument("--prefetch-all", action="store_true",
                     help="with --prefetch: read every row of the next batch and mask at the lookup")
+    ap.add_argument("--features-in-hbm", action="store_true",
+                    help="c3: the node features live in device memory instead of pinned host memory (a variant beside "
+                         "the configuration's own placement: 288 GB hold the papers100M-sized matrix, 57 GB, next to "
+                         "the 57 GB history table; the mag240M-sized one, 187 GB beside a 125 GB table, does not fit)")
+    ap.add_argument("--sampler-replay", type=int, default=4,
+                    help="c1 / c3 --with-sampler: slots of the device sampler whose launches are recorded in HIP graphs "
+                         "and replayed, one launch per batch (0: every batch is launched kernel by kernel)")
     ap.add_argument("--no-batch-view", action="store_true",
                     help="c3/c5: batches come without the transposed view of their CSR, so every layer's "
                          "backward builds one (the default: the loader emits it with the batch)")
@@ -94,11 +102,15 @@ def timed_steps(step, steps, warmup):
 class KernelClock:
     """HIP-event timing of one launch site on the current stream, accumulated over the timed region."""
 
+    enabled = True                  # off: the wrapped call runs bare (its events cost the host 5 - 10 us a pair)
+
     def __init__(self):
         self.pairs = []
         self.cpu_s = 0.0            # host time spent inside fn (enqueueing; nothing here waits for the GPU)
 
     def __call__(self, fn):
+        if not KernelClock.enabled:
+            return fn()
         import torch
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
@@ -118,6 +130,37 @@ class KernelClock:
 
     def mean_ms(self):
         return sum(a.elapsed_time(b) for a, b in self.pairs) / max(1, len(self.pairs))
+
+
+def time_iterations(step, steps, clocks, reset=None):
+    """``steps`` iterations timed bare (sync, clock, sync), then up to 100 more with the per-phase event clocks
+    switched on for the phase figures: the events of five phases cost a host-bound loop 5 - 10% of its time.
+    ``reset()`` runs in front of each of the two passes.  Returns seconds per iteration of the bare pass."""
+    sync()
+    # the interpreter's full collections walk every object torch's import left behind (70 - 80 ms each, once
+    # every few hundred iterations): park what exists now in the permanent generation, as training loops do
+    gc.collect()
+    gc.freeze()
+    KernelClock.enabled = False
+    try:
+        if reset:
+            reset()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        sync()
+        sec = (time.perf_counter() - t0) / steps
+    finally:
+        KernelClock.enabled = True
+    for c in clocks.values():
+        c.reset()
+    if reset:
+        reset()
+    for _ in range(min(steps, 100)):
+        step()
+    sync()
+    gc.unfreeze()
+    return sec
 
 
 # ----------------------------------------------------------------------------------------- C2
@@ -611,6 +654,8 @@ def run_c3(args, with_batched=True):
     for lo in range(0, pool_rows, chunk):
         hi = min(pool_rows, lo + chunk)
         pinned[lo:hi].copy_(torch.randn(hi - lo, Fin, device=dev, generator=gen))
+    if args.features_in_hbm:
+        pinned = pinned.to(dev)
     store = PooledStore(pinned, device=dev, prefetch_cus=args.prefetch_cus if args.prefetch else 0)
     cache = RingHistoryCache(store, N, Fin, H, capacity=N, num_layers=L, table_dtype=torch.float16,
                              thres=0.05, age_limit=AGE_LIMIT_ITERS, device=dev)
@@ -653,7 +698,9 @@ def run_c3(args, with_batched=True):
         indptr, indices = device_power_law_graph(N, 14.5, dev, gen)
         sampled["E_graph"] = indices.numel()
         sampled["sampler"] = NeighborSampler(indptr, indices, fanout, seed=3, device=dev, validate=False,
-                                             emit_view=not args.no_batch_view)
+                                             emit_view=not args.no_batch_view,
+                                             replay_slots=max(args.sampler_replay, args.prefetch_depth + 2)
+                                             if args.sampler_replay else 0)
         del indptr, indices
         seed_pool = torch.randperm(N, device=dev, generator=gen)[: n_seed * 1024].view(1024, n_seed).contiguous()
         sampled["pending"] = sampled["sampler"].sample_async(seed_pool[0])
@@ -711,27 +758,18 @@ def run_c3(args, with_batched=True):
         torch.cuda.set_stream(compute)
     for _ in range(args.warmup):
         step()
-    sync()
-    for c in ev.values():
-        c.reset()
-    sampled["shapes"], sampled["wait_s"] = [], 0.0
-    # the interpreter's full collections walk every object torch's import left behind (70 - 80 ms each, once
-    # every few hundred iterations): park what exists now in the permanent generation, as training loops do
-    gc.collect()
-    gc.freeze()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    sync()
-    sec = (time.perf_counter() - t0) / args.steps
-    gc.unfreeze()
+
+    def reset():
+        sampled["shapes"], sampled["wait_s"] = [], 0.0
+
+    sec = time_iterations(step, args.steps, ev, reset)
     torch.cuda.set_stream(torch.cuda.default_stream())
     if sampled["sampler"] is not None:
         sampled["pending"].get()
         m = np.mean(np.asarray(sampled["shapes"], dtype=np.float64), axis=0)
         shape = {"n0": int(m[0]), "n1": int(m[1]), "n2": int(m[2]), "n3": int(m[3]), "edges": int(m[4]),
                  "sampled_on_device_from_graph_edges": sampled["E_graph"],
-                 "wait_for_sampler_ms": 1e3 * sampled["wait_s"] / args.steps}
+                 "wait_for_sampler_ms": 1e3 * sampled["wait_s"] / max(1, len(sampled["shapes"]))}
     else:
         shape = {k: int(np.mean([int(x["num_node_in_layer"][i]) for x in samples])) for i, k in enumerate(("n0", "n1", "n2", "n3"))}
         shape["edges"] = int(np.mean([x["idx"].size for x in samples]))
@@ -743,9 +781,12 @@ def run_c3(args, with_batched=True):
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "c3: papers100M-shaped, %d nodes, 3-layer SAGE hidden 256, fanout [15,10,5], batch 1000, "
                                "fp16 history table %d x 256 (about 35%% of nodes cached), features 128-dim fp32 in a "
-                               "pinned host pool of %d rows read zero-copy; mean batch %s" % (N, N, pool_rows, shape)},
+                               "%s of %d rows; mean batch %s"
+                               % (N, N, "device-memory pool" if args.features_in_hbm else "pinned host pool read zero-copy",
+                                  pool_rows, shape)},
         "phases_ms": {k: c.mean_ms() for k, c in ev.items()},
         "phases_host_enqueue_ms": {k: c.mean_cpu_ms() for k, c in ev.items()},
+        "feature_store": "device memory" if args.features_in_hbm else "pinned host memory, read zero-copy",
         "transposed_view": "built in backward" if args.no_batch_view else "emitted with the batch",
         "feature_rows_read_last_batch": int(cache.used_masks[0].sum()),
         "cached_1hop_fraction_last_batch": float((cache.sub2embed != -1).float().mean()),
@@ -832,17 +873,7 @@ def run_c5(args):
         torch.cuda.set_stream(compute)
     for _ in range(args.warmup):
         step()
-    sync()
-    for c in ev.values():
-        c.reset()
-    gc.collect()                # as in run_c3: no full collection of the interpreter inside the timed region
-    gc.freeze()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    sync()
-    sec = (time.perf_counter() - t0) / args.steps
-    gc.unfreeze()
+    sec = time_iterations(step, args.steps, ev)
     torch.cuda.set_stream(torch.cuda.default_stream())
     shape = {k: int(np.mean([int(x["num_node_in_layer"][i]) for x in samples])) for i, k in enumerate(("n0", "n1", "n2"))}
     shape["edges"] = int(np.mean([x["idx"].size for x in samples]))
@@ -898,7 +929,7 @@ def run_c1(args):
         model.table = table
     opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True)
     sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=1, device=dev, validate=False,
-                              emit_view=not args.no_batch_view)
+                              emit_view=not args.no_batch_view, replay_slots=args.sampler_replay)
     gen = torch.Generator(device=dev).manual_seed(1)
     seed_pool = torch.randperm(N, device=dev, generator=gen)[: n_seed * 64].view(64, n_seed).contiguous()
     ev = {k: KernelClock() for k in ("load", "forward", "backward", "step", "update")}
@@ -909,8 +940,10 @@ def run_c1(args):
         b = state["pending"].get()
         state["pending"] = sampler.sample_async(seed_pool[state["it"] % 64])
         state["shapes"].append(b.num_node_in_layer.tolist() + [b.idx.numel()])
-        if len(state["kept"]) < 8:
-            state["kept"].append(b)
+        if len(state["kept"]) < 8:                  # copies: a replayed sampler overwrites a batch's arrays later
+            state["kept"].append(types.SimpleNamespace(ptr=b.ptr.clone(), idx=b.idx.clone(), y=b.y.clone(),
+                                                       sub_to_full=b.sub_to_full.clone(),
+                                                       num_node_in_layer=b.num_node_in_layer.clone()))
         ev["load"](lambda: cache.lookup_and_load(b, L))
         out = ev["forward"](lambda: model(b))
         loss = torch.nn.functional.nll_loss(out, b.y)
@@ -921,18 +954,11 @@ def run_c1(args):
 
     for _ in range(args.warmup):
         step()
-    sync()
-    for c in ev.values():
-        c.reset()
-    state["shapes"] = []
-    gc.collect()
-    gc.freeze()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    sync()
-    sec = (time.perf_counter() - t0) / args.steps
-    gc.unfreeze()
+
+    def reset():
+        state["shapes"] = []
+
+    sec = time_iterations(step, args.steps, ev, reset)
     state["pending"].get()
     m = np.mean(np.asarray(state["shapes"], dtype=np.float64), axis=0)
     res = {

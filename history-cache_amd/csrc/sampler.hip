@@ -32,7 +32,7 @@ constexpr int SP_GROUP = 16;             // lanes that share one row in the pick
 struct SpState {
   int64_t lo, hi;   // frontier rows of the current hop
   int64_t edges;    // edges written by earlier hops
-  int64_t pad;
+  uint64_t key;     // the batch's sampling key
 };
 
 __host__ __device__ __forceinline__ uint64_t sp_mix64(uint64_t z) {
@@ -70,12 +70,14 @@ __global__ __launch_bounds__(HC_BLOCK) void sp_fill_map(int32_t *__restrict__ lo
 __global__ __launch_bounds__(HC_BLOCK) void sp_init(const int64_t *__restrict__ seeds, int64_t n_seed,
                                                      int64_t num_nodes, int32_t *__restrict__ loc,
                                                      int64_t *__restrict__ sub_to_full, int64_t *__restrict__ ptr,
-                                                     int64_t *__restrict__ counts, SpState *__restrict__ st) {
+                                                     int64_t *__restrict__ counts, SpState *__restrict__ st,
+                                                     uint64_t rng_seed, const uint64_t *__restrict__ rng_seed_at) {
   const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
   if (i == 0) {
     st->lo = 0;
     st->hi = n_seed;
     st->edges = 0;
+    st->key = rng_seed_at ? *rng_seed_at : rng_seed;
     ptr[0] = 0;
     counts[0] = n_seed;
   }
@@ -107,7 +109,7 @@ __global__ __launch_bounds__(HC_BLOCK) void sp_pick(const int64_t *__restrict__ 
                                                      const int64_t *__restrict__ indices,
                                                      const int64_t *__restrict__ sub_to_full,
                                                      const SpState *__restrict__ st, int64_t fanout,
-                                                     int64_t num_nodes, uint64_t hop_key,
+                                                     int64_t num_nodes, int hop,
                                                      const int32_t *__restrict__ cnt,
                                                      const int32_t *__restrict__ incl, int32_t *__restrict__ loc,
                                                      int64_t *__restrict__ ptr, int64_t *__restrict__ idx,
@@ -126,7 +128,7 @@ __global__ __launch_bounds__(HC_BLOCK) void sp_pick(const int64_t *__restrict__ 
   const int64_t full = sub_to_full[u];
   const int64_t first = indptr[full];
   const uint64_t d = (uint64_t)(indptr[full + 1] - first);
-  const uint64_t key = sp_mix64(hop_key ^ (uint64_t)full);
+  const uint64_t key = sp_mix64(sp_mix64(st->key + (uint64_t)hop) ^ (uint64_t)full);
   for (int64_t j = sub; j < c; j += SP_GROUP) {
     const uint64_t pos = d > (uint64_t)fanout ? sp_perm((uint64_t)j, d, key) : (uint64_t)j;
     const int64_t v = indices[first + (int64_t)pos];
@@ -316,11 +318,13 @@ extern "C" int hc_sample_map_init(int32_t *node_map, int64_t num_nodes, void *st
   return hc_launch_status();
 }
 
-extern "C" int hc_sample_layers(const int64_t *indptr, const int64_t *indices, int64_t num_nodes,
-                                const int64_t *seeds, int64_t n_seed, const int64_t *fanout, int num_hops,
-                                uint64_t rng_seed, int32_t *node_map, int64_t *ptr, int64_t *idx,
-                                int64_t *sub_to_full, int64_t *counts, void *workspace, size_t workspace_bytes,
-                                void *stream) {
+namespace {
+
+int sample_layers_impl(const int64_t *indptr, const int64_t *indices, int64_t num_nodes, const int64_t *seeds,
+                       int64_t n_seed, const int64_t *fanout, int num_hops, uint64_t rng_seed,
+                       const uint64_t *rng_seed_at, int32_t *node_map, int64_t *ptr, int64_t *idx,
+                       int64_t *sub_to_full, int64_t *counts, void *workspace, size_t workspace_bytes,
+                       void *stream) {
   HC_REQUIRE(num_nodes > 0 && n_seed > 0);
   HC_REQUIRE(indptr && indices && seeds && node_map && ptr && idx && sub_to_full && counts);
   const SpCaps c = sp_caps(n_seed, fanout, num_hops, num_nodes);
@@ -340,16 +344,16 @@ extern "C" int hc_sample_layers(const int64_t *indptr, const int64_t *indices, i
   void *scan_ws = w + l.scan;
   const dim3 bl(HC_BLOCK);
 
-  sp_init<<<dim3(sp_blocks(n_seed)), bl, 0, s>>>(seeds, n_seed, num_nodes, node_map, sub_to_full, ptr, counts, st);
+  sp_init<<<dim3(sp_blocks(n_seed)), bl, 0, s>>>(seeds, n_seed, num_nodes, node_map, sub_to_full, ptr, counts, st,
+                                                 rng_seed, rng_seed_at);
   for (int k = 0; k < num_hops; ++k) {
     const int64_t cap = c.rows[k], ecap = c.edges[k];
-    const uint64_t hop_key = sp_mix64(rng_seed + (uint64_t)k);
     sp_count<<<dim3(sp_blocks(cap)), bl, 0, s>>>(indptr, sub_to_full, st, fanout[k], num_nodes, cnt, cap);
     size_t bytes = sp_scan_bytes(cap);
     if (rocprim::inclusive_scan(scan_ws, bytes, cnt, incl, (size_t)cap, rocprim::plus<int32_t>(), s) != hipSuccess)
       return HC_ELAUNCH;
     sp_pick<<<dim3(sp_blocks(cap * SP_GROUP)), bl, 0, s>>>(indptr, indices, sub_to_full, st, fanout[k], num_nodes,
-                                                          hop_key, cnt, incl, node_map, ptr, idx, cap);
+                                                          k, cnt, incl, node_map, ptr, idx, cap);
     sp_flag<<<dim3(sp_blocks(ecap)), bl, 0, s>>>(idx, node_map, st, incl, cap, num_nodes, flag, ecap);
     bytes = sp_scan_bytes(ecap);
     if (rocprim::inclusive_scan(scan_ws, bytes, flag, rank, (size_t)ecap, rocprim::plus<int32_t>(), s) !=
@@ -363,4 +367,25 @@ extern "C" int hc_sample_layers(const int64_t *indptr, const int64_t *indices, i
   }
   sp_reset<<<dim3(sp_blocks(c.total_nodes)), bl, 0, s>>>(sub_to_full, st, num_nodes, node_map, c.total_nodes);
   return hc_launch_status();
+}
+
+}  // namespace
+
+extern "C" int hc_sample_layers(const int64_t *indptr, const int64_t *indices, int64_t num_nodes,
+                                const int64_t *seeds, int64_t n_seed, const int64_t *fanout, int num_hops,
+                                uint64_t rng_seed, int32_t *node_map, int64_t *ptr, int64_t *idx,
+                                int64_t *sub_to_full, int64_t *counts, void *workspace, size_t workspace_bytes,
+                                void *stream) {
+  return sample_layers_impl(indptr, indices, num_nodes, seeds, n_seed, fanout, num_hops, rng_seed, nullptr, node_map,
+                            ptr, idx, sub_to_full, counts, workspace, workspace_bytes, stream);
+}
+
+extern "C" int hc_sample_layers_seed_at(const int64_t *indptr, const int64_t *indices, int64_t num_nodes,
+                                        const int64_t *seeds, int64_t n_seed, const int64_t *fanout, int num_hops,
+                                        const uint64_t *rng_seed_at, int32_t *node_map, int64_t *ptr,
+                                        int64_t *idx, int64_t *sub_to_full, int64_t *counts, void *workspace,
+                                        size_t workspace_bytes, void *stream) {
+  HC_REQUIRE(rng_seed_at != nullptr);
+  return sample_layers_impl(indptr, indices, num_nodes, seeds, n_seed, fanout, num_hops, 0, rng_seed_at, node_map,
+                            ptr, idx, sub_to_full, counts, workspace, workspace_bytes, stream);
 }

@@ -18,7 +18,7 @@ import hiscache_backend as _be
 class NeighborSampler:
 
     def __init__(self, indptr, indices, fanout, labels=None, seed=0, device="cuda:0", validate=True,
-                 emit_view=False, view_edges=False):
+                 emit_view=False, view_edges=False, replay_slots=0):
         """``indptr`` / ``indices``: CSR of the full graph (int64; moved to ``device``).  ``fanout[k]``
         neighbours are drawn, without replacement, for nodes first reached at hop k.  ``emit_view``:
         every batch also carries ``batch.view``, the transposed view of its CSR
@@ -26,7 +26,16 @@ class NeighborSampler:
         that the layers' backward builds none; ``view_edges`` adds the view's edge slots, which the
         relational layer's backward reads.  (The view is built with the batch's sizes still on the device,
         for batches whose capacity -- seeds x the fanouts' products -- stays below 2^24 edges and nodes;
-        beyond that the sampling call raises and the batch must come without a view.)"""
+        beyond that the sampling call raises and the batch must come without a view.)
+        ``replay_slots`` = K > 0: the launches of one batch (about forty: every one has the same shape for
+        the same number of seeds, the sizes stay on the device) are recorded once per slot in a HIP graph and
+        replayed as one launch per batch; the batch's arrays then live in the slot's own memory and are
+        OVERWRITTEN when the slot comes round again, K batches later -- choose K above the number of batches
+        that are alive at once (in flight, being trained on, kept).  Batches with another number of seeds
+        (the last one of an epoch) take the ordinary path."""
+        self.replay_slots = int(replay_slots)
+        self._slots = [None] * self.replay_slots
+        self._next_slot = 0
         self.emit_view = bool(emit_view)
         self.view_edges = bool(view_edges)
         self.device = torch.device(device)
@@ -71,18 +80,37 @@ class NeighborSampler:
             stream = self._stream
         if stream != cur:
             stream.wait_stream(cur)                                    # seeds may have been produced there
+        slot = self._replay_slot(seeds)
         with torch.cuda.stream(stream):
-            out = _be.sample_layers(self.indptr, self.indices, seeds, self.fanout, rng_seed, self.node_map,
-                                    emit_view=self.emit_view, view_edges=self.view_edges)
+            if slot is not None:
+                out = slot.run(self, seeds, rng_seed, stream)
+            else:
+                out = _be.sample_layers(self.indptr, self.indices, seeds, self.fanout, rng_seed, self.node_map,
+                                        emit_view=self.emit_view, view_edges=self.view_edges)
             counts_host = self._host_pool.pop() if self._host_pool else torch.empty(
                 2 * len(self.fanout) + 1, dtype=torch.int64, pin_memory=True)
             counts_host.copy_(out[3], non_blocking=True)
             done = torch.cuda.Event()
             done.record(stream)
             y = None if self.labels is None else self.labels[seeds]
-        return _PendingBatch(self, out, counts_host, done, seeds, y, stream)
+        if slot is not None:
+            slot.done = done
+        return _PendingBatch(self, out, counts_host, done, seeds, y, stream, pooled=slot is not None)
 
-    def _finish(self, out, counts_host, seeds, y, stream):
+    def _replay_slot(self, seeds):
+        if not self.replay_slots:
+            return None
+        slot = self._slots[self._next_slot]
+        if slot is None:
+            slot = self._slots[self._next_slot] = _ReplaySlot(seeds.numel(), self.device)
+        if slot.n_seed != seeds.numel():
+            return None
+        self._next_slot = (self._next_slot + 1) % self.replay_slots
+        if slot.done is not None:
+            slot.done.synchronize()          # the slot's previous batch has been sampled (its seed has been read)
+        return slot
+
+    def _finish(self, out, counts_host, seeds, y, stream, pooled=False):
         ptr, idx, s2f = out[:3]
         L = len(self.fanout)
         c = counts_host.tolist()
@@ -96,9 +124,10 @@ class NeighborSampler:
             view = _be.BatchView(ptrT[: nnl[L] + 1], rowT[:n_e], None if edgeT is None else edgeT[:n_e],
                                  nnl[L - 1], nnl[L], nel[-1])
         if stream != cur:
-            for t in (ptr, idx, s2f, seeds) + (() if y is None else (y,)):
+            # arrays of a replay slot belong to its graph and are never handed back to the allocator
+            for t in ((seeds,) if pooled else (ptr, idx, s2f, seeds)) + (() if y is None else (y,)):
                 t.record_stream(cur)
-            if view is not None:
+            if view is not None and not pooled:
                 view.record_stream(cur)
         return SimpleNamespace(
             ptr=ptr[: nnl[L - 1] + 1],
@@ -117,14 +146,41 @@ class NeighborSampler:
 class _PendingBatch:
     """A batch being sampled; ``get()`` returns it once the device has finished."""
 
-    def __init__(self, sampler, out, counts_host, done, seeds, y, stream):
-        self._args = (sampler, out, counts_host, done, seeds, y, stream)
+    def __init__(self, sampler, out, counts_host, done, seeds, y, stream, pooled=False):
+        self._args = (sampler, out, counts_host, done, seeds, y, stream, pooled)
         self._batch = None
 
     def get(self):
         if self._batch is None:
-            sampler, out, counts_host, done, seeds, y, stream = self._args
+            sampler, out, counts_host, done, seeds, y, stream, pooled = self._args
             done.synchronize()
-            self._batch = sampler._finish(out, counts_host, seeds, y, stream)
+            self._batch = sampler._finish(out, counts_host, seeds, y, stream, pooled)
             self._args = None
         return self._batch
+
+
+class _ReplaySlot:
+    """One recorded sampling call: its seeds and its seed key are read from fixed places (a device array, a
+    pinned host word), its outputs live in the graph's own memory."""
+
+    def __init__(self, n_seed, device):
+        self.n_seed = int(n_seed)
+        self.seeds = torch.empty(self.n_seed, dtype=torch.int64, device=device)
+        self.key = torch.zeros(1, dtype=torch.int64, pin_memory=True)
+        self.graph = None
+        self.out = None
+        self.done = None
+
+    def run(self, sampler, seeds, rng_seed, stream):
+        self.seeds.copy_(seeds)
+        k = int(rng_seed) & 0xFFFFFFFFFFFFFFFF
+        self.key[0] = k - (1 << 64) if k >= (1 << 63) else k
+        if self.graph is None:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                self.out = _be.sample_layers(sampler.indptr, sampler.indices, self.seeds, sampler.fanout, 0,
+                                             sampler.node_map, emit_view=sampler.emit_view,
+                                             view_edges=sampler.view_edges, rng_seed_at=self.key)
+            self.graph = graph
+        self.graph.replay()
+        return self.out

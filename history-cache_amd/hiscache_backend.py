@@ -97,6 +97,8 @@ _SIGNATURES = {
     "hc_sample_map_init": (_c_int, [_c_p, _c_i64, _c_p]),
     "hc_sample_layers": (_c_int, [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_int, ctypes.c_uint64, _c_p, _c_p,
                                   _c_p, _c_p, _c_p, _c_p, _c_sz, _c_p]),
+    "hc_sample_layers_seed_at": (_c_int, [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_int, _c_p, _c_p, _c_p,
+                                          _c_p, _c_p, _c_p, _c_p, _c_sz, _c_p]),
     "hc_bn_relu_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
     "hc_bn_relu_fwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, ctypes.c_float, ctypes.c_float, _c_p,
                                 _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_sz, _c_p, _c_p]),
@@ -1171,7 +1173,8 @@ def build_transpose_dev(ptr, idx, rows_dev, edges_dev, nodes_dev, max_edges, max
     return ptrT, rowT, edgeT
 
 
-def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map, emit_view=False, view_edges=False):
+def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map, emit_view=False, view_edges=False,
+                  rng_seed_at=None):
     """Layered neighbour sampling without replacement.  Returns (ptr, idx, sub_to_full, counts) as
     device tensors at their capacity; ``counts`` (int64[2L+1] on the device) holds the node count
     within k hops for k = 0..L and then the cumulative edge count after every hop, so the caller
@@ -1181,7 +1184,9 @@ def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map, emit_view=
     (/root/reference/hiscache/history_trainer.py:19,26).  ``emit_view=True`` appends (ptrT, rowT, edgeT):
     the transposed view of the whole sampled CSR, built behind the sampling with the sizes still on the
     device (``build_transpose_dev``), for ``BatchView`` once the caller has read ``counts``; edgeT is
-    None unless ``view_edges`` (the relational layer's backward reads it)."""
+    None unless ``view_edges`` (the relational layer's backward reads it).  ``rng_seed_at`` (a one-element
+    int64 tensor in device or pinned host memory) replaces ``rng_seed``: the seed is read from it when the
+    first kernel runs, which lets a call recorded in a HIP graph be replayed with a new seed."""
     lib = load_library()
     _dev(indptr, "indptr", torch.int64)
     _dev(indices, "indices", torch.int64)
@@ -1205,9 +1210,17 @@ def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map, emit_view=
     if ws_bytes == 0:
         raise ValueError("unsupported fanout / batch size")
     ws = _workspace(ws_bytes, dev)
-    rc = lib.hc_sample_layers(_ptr(indptr), _ptr(indices), N, _ptr(seeds), n_seed, ctypes.cast(fan, _c_p), L,
-                              ctypes.c_uint64(int(rng_seed) & 0xFFFFFFFFFFFFFFFF), _ptr(node_map), _ptr(ptr),
-                              _ptr(idx), _ptr(s2f), _ptr(counts), _ptr(ws), ws_bytes, _stream())
+    if rng_seed_at is not None:
+        if rng_seed_at.dtype != torch.int64 or rng_seed_at.numel() < 1 or not (
+                rng_seed_at.is_cuda or rng_seed_at.is_pinned()):
+            raise ValueError("rng_seed_at must be an int64 tensor in device or pinned host memory")
+        rc = lib.hc_sample_layers_seed_at(_ptr(indptr), _ptr(indices), N, _ptr(seeds), n_seed,
+                                          ctypes.cast(fan, _c_p), L, _ptr(rng_seed_at), _ptr(node_map), _ptr(ptr),
+                                          _ptr(idx), _ptr(s2f), _ptr(counts), _ptr(ws), ws_bytes, _stream())
+    else:
+        rc = lib.hc_sample_layers(_ptr(indptr), _ptr(indices), N, _ptr(seeds), n_seed, ctypes.cast(fan, _c_p), L,
+                                  ctypes.c_uint64(int(rng_seed) & 0xFFFFFFFFFFFFFFFF), _ptr(node_map), _ptr(ptr),
+                                  _ptr(idx), _ptr(s2f), _ptr(counts), _ptr(ws), ws_bytes, _stream())
     _check(rc, "hc_sample_layers")
     if emit_view:
         ptrT, rowT, edgeT = build_transpose_dev(ptr, idx, counts[L - 1:L], counts[2 * L:2 * L + 1],

@@ -390,6 +390,17 @@ int hc_sample_layers(const int64_t *indptr, const int64_t *indices, int64_t num_
                      uint64_t rng_seed, int32_t *node_map, int64_t *ptr, int64_t *idx,
                      int64_t *sub_to_full, int64_t *counts, void *workspace, size_t workspace_bytes,
                      void *stream);
+/* hc_sample_layers_seed_at: the same call with the seed read from *rng_seed_at
+ * (memory the device can read: device memory or pinned host memory) when its
+ * first kernel runs, not when the call is made -- so that a call recorded in a
+ * HIP graph (every launch of it has the same shape for the same n_seed and
+ * fanout, the sizes stay on the device) can be replayed for the next batch
+ * after the host has stored a new seed there and new ids in `seeds`. */
+int hc_sample_layers_seed_at(const int64_t *indptr, const int64_t *indices, int64_t num_nodes,
+                             const int64_t *seeds, int64_t n_seed, const int64_t *fanout, int num_hops,
+                             const uint64_t *rng_seed_at, int32_t *node_map, int64_t *ptr, int64_t *idx,
+                             int64_t *sub_to_full, int64_t *counts, void *workspace,
+                             size_t workspace_bytes, void *stream);
 
 /* ---------------------------------------------------------------- helpers
  * hc_count_num replaces count_num (grad_check.h:26, grad_check.cu:165-182):

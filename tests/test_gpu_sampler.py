@@ -128,3 +128,50 @@ def test_training_from_processed_files(tmp_path):
         assert np.isfinite(float(loss.detach()))
     pending.get()
     assert cache.header > 0
+
+
+@pytest.mark.parametrize("view_edges", [False, True])
+def test_replayed_sampling_equals_the_launched_one(orc, view_edges):
+    """NeighborSampler(replay_slots=K): the launches of a batch recorded once per slot in a HIP graph and
+    replayed for the later batches (new seeds in the slot's array, a new seed key in its pinned word) give the
+    sequential statement's batch every time -- ten batches over three slots, with the program's own work and
+    synchronisations between the replays --, the emitted view included; a batch with another number of seeds
+    takes the ordinary path; a slot's arrays are overwritten when it comes round again."""
+    import hiscache_backend as be
+    from hiscache import NeighborSampler
+    rng = np.random.default_rng(77)
+    fanout, n_seed, N = [6, 4], 120, 6000
+    indptr, indices = simple_graph(rng, N, 25, hubs=4)
+    labels = rng.integers(0, 5, size=N)
+    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=9, device=DEV, emit_view=True,
+                              view_edges=view_edges, replay_slots=3)
+    first = None
+    for it in range(10):
+        n = 37 if it == 6 else n_seed
+        seeds = rng.choice(N, size=n, replace=False).astype(np.int64)
+        print("replayed sampler batch", it, n, flush=True)
+        pending = sampler.sample_async(torch.from_numpy(seeds).to(DEV))
+        x = torch.randn(256, 256, device=DEV)
+        (x @ x).sum().item()                                          # eager work and a synchronisation between
+        batch = pending.get()
+        want = orc.sample_layers(indptr, indices, seeds, fanout, sampler.batch_seed(it))
+        got = to_np(batch)
+        for k in want:
+            np.testing.assert_array_equal(got[k], want[k], err_msg=f"{k} of batch {it}")
+        np.testing.assert_array_equal(batch.y.cpu().numpy(), labels[seeds])
+        L = len(fanout)
+        n_rows, n_src, n_e = int(want["num_node_in_layer"][L - 1]), int(want["num_node_in_layer"][L]), len(want["idx"])
+        wp, wr, we = orc.build_transpose(want["ptr"], want["idx"], None, n_src)
+        assert batch.view.covers(n_rows, n_src) and batch.view.num_edge == n_e
+        np.testing.assert_array_equal(batch.view.ptrT.cpu().numpy(), wp)
+        np.testing.assert_array_equal(batch.view.rowT.cpu().numpy()[:n_e], wr)
+        if view_edges:
+            np.testing.assert_array_equal(batch.view.edgeT.cpu().numpy()[:n_e], we)
+        else:
+            assert batch.view.edgeT is None
+        if it == 0:
+            first = (batch, got["idx"].copy())
+        if it == 3:                                                   # slot 0 again: the first batch's memory
+            assert first[0].idx.data_ptr() == batch.idx.data_ptr()
+    assert sum(s is not None and s.graph is not None for s in sampler._slots) == 3
+    assert int((sampler.node_map != 0x7fffffff).sum()) == 0
