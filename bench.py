@@ -1205,6 +1205,28 @@ def run_sample(args):
         pending = nxt
     pending.get()
     sync()
+    # host time of one sample_async (the view emitted with the batch), launched kernel by kernel and replayed
+    # from the slots' HIP graphs; the device is idle when each call starts
+    host_us, latency_ms = {}, {}
+    del sampler
+    for name, slots in (("launched", 0), ("replayed", 4)):
+        sm = NeighborSampler(indptr, indices, fanout, seed=6, device=dev, validate=False, emit_view=True,
+                             replay_slots=slots)
+        t_host = t_done = 0.0
+        n_rep = max(args.steps, 20)
+        for i in range(8 + n_rep):
+            sync()
+            t0 = time.perf_counter()
+            p = sm.sample_async(seed_sets[i % len(seed_sets)])
+            t1 = time.perf_counter()
+            sync()
+            t2 = time.perf_counter()
+            p.get()
+            if i >= 8:
+                t_host += t1 - t0
+                t_done += t2 - t0
+        host_us[name], latency_ms[name] = 1e6 * t_host / n_rep, 1e3 * t_done / n_rep
+        del sm
     mean = np.mean(np.asarray(shapes, dtype=np.float64), axis=0)
     edges = float(mean[-1])
     return {
@@ -1215,6 +1237,8 @@ def run_sample(args):
                                "%s, edges %d" % (N, E_graph, fanout, n_seed, [int(x) for x in mean[:-1]], int(edges))},
         "device_ms_per_batch": clock.mean_ms(),
         "wait_ms_when_prefetched": float(np.mean(waits) * 1e3),
+        "with_view_host_us_per_batch": host_us,
+        "with_view_ms_until_batch_is_ready": latency_ms,
     }
 
 
