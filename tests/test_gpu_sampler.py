@@ -57,26 +57,41 @@ def test_sampler_multi_edges_and_isolated_nodes(orc):
         np.testing.assert_array_equal(got[k], want[k], err_msg=k)
 
 
-def test_sampled_batch_trains(orc):
-    """A batch from the sampler runs through lookup_and_load, the model and update_history."""
+@pytest.mark.parametrize("mode", ["launched", "view", "replayed"])
+def test_sampled_batch_trains(orc, mode):
+    """A batch from the sampler runs through lookup_and_load, the model and update_history; with the view emitted
+    with the batch, and with the sampling replayed from HIP graphs (batches pipelined one ahead), the losses
+    are the ones of the plain path bit for bit."""
+    losses = _train_on_sampled_batches(mode)
+    assert all(np.isfinite(losses))
+    if mode != "launched":
+        assert losses == _train_on_sampled_batches("launched")
+
+
+def _train_on_sampled_batches(mode):
     from hiscache import HistoryCache, HistorySAGE, NeighborSampler, PinnedFeatureStore, make_config
     rng = np.random.default_rng(220)
     N, Fin, H, C, L = 4000, 32, 48, 5, 3
     indptr, indices = simple_graph(rng, N, 12)
     feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32))
     labels = rng.integers(0, C, size=N)
-    sampler = NeighborSampler(indptr, indices, [5, 4, 3], labels=labels, seed=1, device=DEV)
+    sampler = NeighborSampler(indptr, indices, [5, 4, 3], labels=labels, seed=1, device=DEV,
+                              emit_view=mode != "launched", replay_slots=3 if mode == "replayed" else 0)
     cfg = make_config(Fin, C, H, L, method="grad", rate=0.6, device=DEV)
     lcm = int(np.lcm(Fin, H))
     cache = HistoryCache(PinnedFeatureStore(feats, device=DEV), cfg, "history_uvm", total_num_node=N,
                          buffer_bytes=600 * lcm * 4, hot_ids=rng.permutation(N).astype(np.int64))
+    torch.manual_seed(220)
     model = HistorySAGE(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache).to(DEV)
     model.train()
     opt = torch.optim.Adam(model.parameters(), lr=1e-2)
     losses = []
+    all_seeds = [torch.from_numpy(rng.choice(N, size=100, replace=False)).to(DEV) for _ in range(7)]
+    pending = sampler.sample_async(all_seeds[0])
     for it in range(6):
-        seeds = torch.from_numpy(rng.choice(N, size=100, replace=False)).to(DEV)
-        batch = sampler.sample(seeds)
+        batch = pending.get()
+        pending = sampler.sample_async(all_seeds[it + 1])         # the next batch is drawn while this one trains
+        assert (batch.view is None) == (mode == "launched")
         cache.lookup_and_load(batch, L)
         np.testing.assert_array_equal(batch.x.cpu().numpy()[cache.used_masks[0].cpu().numpy()],
                                       feats.numpy()[batch.sub_to_full.cpu().numpy()[cache.used_masks[0].cpu().numpy()]])
@@ -87,8 +102,9 @@ def test_sampled_batch_trains(orc):
         opt.step()
         cache.update_history(batch, it)
         losses.append(float(loss.detach()))
-    assert all(np.isfinite(losses))
+    pending.get()
     assert cache.header > 0                                   # embeddings were admitted
+    return losses
 
 
 def test_training_from_processed_files(tmp_path):
