@@ -300,6 +300,29 @@ def test_c3_batched_forward(c3b):
     assert float((lhs - rhs).abs().max()) < 1e-5 * float(rhs.abs().max()) + 1e-3
 
 
+def test_c3_batched_every_row_has_the_oracles_bits(c3b):
+    """All 4.7 M output rows (history rows from the fp16 buffer included) and all 20.8 M gradient rows of the
+    batched layer against the sequential CPU oracle, bit for bit.  About 60 GB of host memory at the peak."""
+    import hiscache_backend as be
+    from oracle import hc_oracle as orc
+    c = c3b
+    ptr, idx, hmap = c["ptr"].cpu().numpy(), c["idx"].cpu().numpy(), c["hmap"].cpu().numpy()
+    x = c["x"].cpu().numpy()
+    hbuf = c["hbuf"].float().cpu().numpy()
+    print("batched layer on the host", flush=True)
+    want = orc.fwd_mean_row(ptr, idx, x, hmap, hbuf, split_above=be.long_row_edges(F))
+    got = c["out"].cpu().numpy()
+    bad = int((got.view(np.uint32) != want.view(np.uint32)).any(axis=1).sum())
+    assert bad == 0, f"{bad} forward rows differ"
+    del x, hbuf, want, got
+    print("batched layer: forward equal", flush=True)
+    want, _ = orc.bwd_mean_row(ptr, idx, c["g"].cpu().numpy(), hmap, c["N"], (c["R"], F),
+                               chunk=be.bwd_chunk_edges(F))
+    got = c["grad_x"].cpu().numpy()
+    bad = int((got.view(np.uint32) != want.view(np.uint32)).any(axis=1).sum())
+    assert bad == 0, f"{bad} gradient rows differ"
+
+
 def test_c3_batched_view_and_backward(c3b):
     c = c3b
     ptrT, rowT, _ = c["tr"]
