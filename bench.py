@@ -1282,15 +1282,23 @@ def main():
             # (batches of about 236 k edges), features read one batch ahead on a CU-limited stream
             sm_args = argparse.Namespace(**vars(it_args))
             sm_args.with_sampler, sm_args.prefetch = True, True
-            for name, fn in (("c1", lambda: run_c1(it_args)), ("c3", lambda: run_c3(it_args, with_batched=False)),
-                             ("c5", lambda: run_c5(it_args)), ("c3_sampled", lambda: run_c3(sm_args, with_batched=False))):
+            # c3_sampled_features_in_hbm: a variant beside the configuration's own placement -- the feature matrix
+            # in device memory next to the table (288 GB hold both for papers100M), no read-ahead needed
+            hb_args = argparse.Namespace(**vars(it_args))
+            hb_args.with_sampler, hb_args.features_in_hbm = True, True
+            runs = (("c1", it_args, lambda: run_c1(it_args)),
+                    ("c3", it_args, lambda: run_c3(it_args, with_batched=False)),
+                    ("c5", it_args, lambda: run_c5(it_args)),
+                    ("c3_sampled", sm_args, lambda: run_c3(sm_args, with_batched=False)),
+                    ("c3_sampled_features_in_hbm", hb_args, lambda: run_c3(hb_args, with_batched=False)))
+            for name, used_args, fn in runs:
                 gc.collect()
                 torch.cuda.empty_cache()
                 r = fn()
                 res["iterations"][name] = {
                     "workload": r["config"]["workload"], "ms": r["ms_per_step"], "steps": r["steps"],
                     "warmup": r["warmup"], "transposed_view": r["transposed_view"],
-                    "feature_read_ahead": bool(getattr(sm_args if name == "c3_sampled" else it_args, "prefetch")),
+                    "feature_read_ahead": bool(used_args.prefetch),
                     "phases_ms": r["phases_ms"], "phases_host_enqueue_ms": r["phases_host_enqueue_ms"]}
                 if "cpu_baseline" in r:          # c1, the CPU-runnable configuration: the same iteration on the host
                     res["iterations"][name]["cpu_ms"] = r["cpu_baseline"]["value"]
