@@ -176,8 +176,10 @@ class _ReplaySlot:
         k = int(rng_seed) & 0xFFFFFFFFFFFFFFFF
         self.key[0] = k - (1 << 64) if k >= (1 << 63) else k
         if self.graph is None:
+            # recorded on a stream of its own (the caller's may be the default stream, which cannot record);
+            # the replays run on the caller's
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
+            with torch.cuda.graph(graph, stream=torch.cuda.Stream(device=self.seeds.device)):
                 self.out = _be.sample_layers(sampler.indptr, sampler.indices, self.seeds, sampler.fanout, 0,
                                              sampler.node_map, emit_view=sampler.emit_view,
                                              view_edges=sampler.view_edges, rng_seed_at=self.key)

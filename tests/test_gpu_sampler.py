@@ -166,10 +166,13 @@ def test_replayed_sampling_equals_the_launched_one(orc, view_edges):
         n = 37 if it == 6 else n_seed
         seeds = rng.choice(N, size=n, replace=False).astype(np.int64)
         print("replayed sampler batch", it, n, flush=True)
-        pending = sampler.sample_async(torch.from_numpy(seeds).to(DEV))
-        x = torch.randn(256, 256, device=DEV)
-        (x @ x).sum().item()                                          # eager work and a synchronisation between
-        batch = pending.get()
+        if it % 4 == 1:                                               # on the caller's (default) stream
+            batch = sampler.sample(torch.from_numpy(seeds).to(DEV))
+        else:
+            pending = sampler.sample_async(torch.from_numpy(seeds).to(DEV))
+            x = torch.randn(256, 256, device=DEV)
+            (x @ x).sum().item()                                      # eager work and a synchronisation between
+            batch = pending.get()
         want = orc.sample_layers(indptr, indices, seeds, fanout, sampler.batch_seed(it))
         got = to_np(batch)
         for k in want:
