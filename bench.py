@@ -132,6 +132,16 @@ class KernelClock:
         return sum(a.elapsed_time(b) for a, b in self.pairs) / max(1, len(self.pairs))
 
 
+def backward_on_this_thread(loss):
+    """``loss.backward()`` without the hand-over to autograd's device thread (``hiscache.backward_on_this_thread``);
+    HISCACHE_BENCH_AUTOGRAD_THREAD=1 keeps the hand-over, for comparison."""
+    if os.environ.get("HISCACHE_BENCH_AUTOGRAD_THREAD", "0") not in ("", "0"):
+        loss.backward()
+        return
+    from hiscache import backward_on_this_thread as run
+    run(loss)
+
+
 def time_iterations(step, steps, clocks, reset=None):
     """``steps`` iterations timed bare (sync, clock, sync), then up to 100 more with the per-phase event clocks
     switched on for the phase figures: the events of five phases cost a host-bound loop 5 - 10% of its time.
@@ -746,7 +756,7 @@ def run_c3(args, with_batched=True):
         out = ev["forward"](lambda: model(b))
         loss = torch.nn.functional.nll_loss(out, b.y)
         opt.zero_grad(set_to_none=True)
-        ev["backward"](lambda: loss.backward())
+        ev["backward"](lambda: backward_on_this_thread(loss))
         ev["step"](lambda: opt.step())
         ev["update"](lambda: cache.update_history(b, state["it"]))
 
@@ -863,7 +873,7 @@ def run_c5(args):
         out = ev["forward"](lambda: model(b))
         loss = torch.nn.functional.nll_loss(out, b.y)
         opt.zero_grad(set_to_none=True)
-        ev["backward"](lambda: loss.backward())
+        ev["backward"](lambda: backward_on_this_thread(loss))
         ev["step"](lambda: opt.step())
         ev["update"](lambda: cache.update_history(b, state["it"]))
 
@@ -948,7 +958,7 @@ def run_c1(args):
         out = ev["forward"](lambda: model(b))
         loss = torch.nn.functional.nll_loss(out, b.y)
         opt.zero_grad(set_to_none=True)
-        ev["backward"](lambda: loss.backward())
+        ev["backward"](lambda: backward_on_this_thread(loss))
         ev["step"](lambda: opt.step())
         ev["update"](lambda: cache.update_history(b, state["it"]))
 

@@ -13,6 +13,35 @@ DEV = "cuda:0"
 
 @pytest.mark.parametrize("kind", ["sage", "rgcn"])
 def test_training_reduces_the_loss(kind):
+    losses, hits, model, cache = _train(kind, 90, lambda loss: loss.backward())
+    assert all(np.isfinite(losses))
+    first, last = float(np.mean(losses[:10])), float(np.mean(losses[-10:]))
+    assert last < 0.7 * first, (first, last)
+    assert max(hits[30:]) > 0.02                      # admitted rows come back as hits
+    assert cache.header > 0
+    for p in model.parameters():
+        assert bool(torch.isfinite(p).all())
+    for name, buf in model.named_buffers():
+        if "running" in name:
+            assert bool(torch.isfinite(buf).all())
+        if "num_batches_tracked" in name:
+            assert int(buf) == 90
+
+
+@pytest.mark.parametrize("kind", ["sage", "rgcn"])
+def test_backward_on_the_calling_thread_changes_nothing(kind):
+    """hiscache.backward_on_this_thread(loss) (no hand-over to autograd's device thread) against loss.backward():
+    the same losses, parameters and cache state after twelve iterations, bit for bit."""
+    from hiscache import backward_on_this_thread
+    la, _, ma, ca = _train(kind, 12, lambda loss: loss.backward())
+    lb, _, mb, cb = _train(kind, 12, backward_on_this_thread)
+    assert la == lb
+    for (na, pa), (nb, pb) in zip(ma.named_parameters(), mb.named_parameters()):
+        assert na == nb and torch.equal(pa, pb), na
+    assert int(ca.header) == int(cb.header) and torch.equal(ca.table[: int(ca.header)], cb.table[: int(cb.header)])
+
+
+def _train(kind, iters, backward):
     from hiscache import (HistoryRGCN, HistorySAGE, NeighborSampler, PinnedFeatureStore, RingHistoryCache, make_config,
                           prefer_low_latency_gemm)
     prefer_low_latency_gemm()
@@ -46,7 +75,7 @@ def test_training_reduces_the_loss(kind):
     gen = torch.Generator(device=DEV).manual_seed(3)
     losses, hits = [], []
     pending = sampler.sample_async(torch.randperm(N, device=DEV, generator=gen)[:256])
-    for it in range(1, 91):
+    for it in range(1, iters + 1):
         batch = pending.get()
         pending = sampler.sample_async(torch.randperm(N, device=DEV, generator=gen)[:256])
         assert batch.view is not None and batch.view.num_edge == batch.idx.numel()
@@ -56,20 +85,9 @@ def test_training_reduces_the_loss(kind):
         hits.append(float((cache.sub2embed != -1).float().mean()))
         loss = F.nll_loss(model(batch), batch.y)
         opt.zero_grad(set_to_none=True)
-        loss.backward()
+        backward(loss)
         opt.step()
         cache.update_history(batch, it)
         losses.append(float(loss.detach()))
     pending.get()
-    assert all(np.isfinite(losses))
-    first, last = float(np.mean(losses[:10])), float(np.mean(losses[-10:]))
-    assert last < 0.7 * first, (first, last)
-    assert max(hits[30:]) > 0.02                      # admitted rows come back as hits
-    assert cache.header > 0
-    for p in model.parameters():
-        assert bool(torch.isfinite(p).all())
-    for name, buf in model.named_buffers():
-        if "running" in name:
-            assert bool(torch.isfinite(buf).all())
-        if "num_batches_tracked" in name:
-            assert int(buf) == 90
+    return losses, hits, model, cache
