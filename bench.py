@@ -142,8 +142,11 @@ def backward_on_this_thread(loss):
     run(loss)
 
 
+PHASE_STEPS = 100
+
+
 def time_iterations(step, steps, clocks, reset=None):
-    """``steps`` iterations timed bare (sync, clock, sync), then up to 100 more with the per-phase event clocks
+    """``steps`` iterations timed bare (sync, clock, sync), then up to PHASE_STEPS more with the per-phase event clocks
     switched on for the phase figures: the events of five phases cost a host-bound loop 5 - 10% of its time.
     ``reset()`` runs in front of each of the two passes.  Returns seconds per iteration of the bare pass."""
     sync()
@@ -166,7 +169,7 @@ def time_iterations(step, steps, clocks, reset=None):
         c.reset()
     if reset:
         reset()
-    for _ in range(min(steps, 100)):
+    for _ in range(min(steps, PHASE_STEPS)):
         step()
     sync()
     gc.unfreeze()
@@ -690,7 +693,7 @@ def run_c3(args, with_batched=True):
 
     # One batch per iteration, none reused: a batch that comes back finds the 1-hop nodes it admitted last
     # time in the cache, the used masks prune everything below them and no feature row is read at all.
-    n_pre = min(args.warmup + args.steps + 1, 512)
+    n_pre = min(args.warmup + args.steps + min(args.steps, PHASE_STEPS) + 1, 640)   # none reused, see time_iterations
     samples = [direct_power_law_batch(N, n_seed, fanout, 2.0, 30 + i, degree_scale=2.6) for i in range(n_pre)]
     batches = []
     for smp in samples:
@@ -854,7 +857,7 @@ def run_c5(args):
         def __getitem__(self, ids):
             return self.base[np.asarray(ids) % self.base.size]
 
-    n_pre = min(args.warmup + args.steps + 1, 512)       # one batch per iteration, none reused (see run_c3)
+    n_pre = min(args.warmup + args.steps + min(args.steps, PHASE_STEPS) + 1, 640)   # one batch per iteration, none reused
     samples = [direct_power_law_batch(N, n_seed, fanout, 2.0, 50 + i, degree_scale=1.25) for i in range(n_pre)]
     # a batch comes with the transposed view of its CSR (and the view's edge slots, which the relational
     # layer reads), as the loader emits it (--no-batch-view: backward builds the view of the regrouped block)
@@ -1296,8 +1299,12 @@ def main():
             # in device memory next to the table (288 GB hold both for papers100M), no read-ahead needed
             hb_args = argparse.Namespace(**vars(it_args))
             hb_args.with_sampler, hb_args.features_in_hbm = True, True
+            # c3: the features of the next batch are read ahead on the CU-limited stream (it pays since the loop
+            # became bound by the GPU; the mag240M-shaped loop is bound by the host and goes without)
+            c3_args = argparse.Namespace(**vars(it_args))
+            c3_args.prefetch = True
             runs = (("c1", it_args, lambda: run_c1(it_args)),
-                    ("c3", it_args, lambda: run_c3(it_args, with_batched=False)),
+                    ("c3", c3_args, lambda: run_c3(c3_args, with_batched=False)),
                     ("c5", it_args, lambda: run_c5(it_args)),
                     ("c3_sampled", sm_args, lambda: run_c3(sm_args, with_batched=False)),
                     ("c3_sampled_features_in_hbm", hb_args, lambda: run_c3(hb_args, with_batched=False)))
