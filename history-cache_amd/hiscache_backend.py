@@ -787,10 +787,12 @@ def cache_append(score, thres, emb, sub2embed, sub_to_full, buffer, hidden, in_c
     return mask.view(torch.bool)
 
 
-def gather_rows(src, ids, mask=None, out=None, accumulate=False, out_dtype=torch.float32):
+def gather_rows(src, ids, mask=None, out=None, accumulate=False, out_dtype=torch.float32, stream=None):
     """out[i] = src[ids[i]] where mask[i] (else 0), as ``out_dtype`` (fp32 by default).  ``src`` may be
     a GPU tensor or a pinned host tensor (read zero-copy over the host link).  Negative ids index
-    from the end."""
+    from the end.  ``stream`` (a torch stream; default: the current one): where the kernel is enqueued --
+    a new ``out`` still comes from the current stream's memory, so a caller that names another stream
+    records it on ``out`` (``out.record_stream(stream)``) and orders the two streams itself."""
     lib = load_library()
     if not isinstance(src, torch.Tensor) or src.dim() != 2 or not src.is_contiguous():
         raise ValueError("src must be a contiguous 2-D tensor")
@@ -811,7 +813,8 @@ def gather_rows(src, ids, mask=None, out=None, accumulate=False, out_dtype=torch
         if tuple(out.shape) != (n, F):
             raise ValueError("out must be [len(ids), F]")
     rc = lib.hc_gather_rows(_ptr(src), _float_dtype(src, "src"), src.shape[0], _ptr(ids), _ptr(mask),
-                            _ptr(out), _float_dtype(out, "out"), 1 if accumulate else 0, n, F, _stream())
+                            _ptr(out), _float_dtype(out, "out"), 1 if accumulate else 0, n, F,
+                            _stream() if stream is None else _c_p(stream.cuda_stream))
     _check(rc, "hc_gather_rows")
     return out
 
