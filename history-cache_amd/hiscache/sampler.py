@@ -83,7 +83,7 @@ class NeighborSampler:
         slot = self._replay_slot(seeds)
         with torch.cuda.stream(stream):
             if slot is not None:
-                out = slot.run(self, seeds, rng_seed, stream)
+                out = slot.run(self, seeds, rng_seed)
             else:
                 out = _be.sample_layers(self.indptr, self.indices, seeds, self.fanout, rng_seed, self.node_map,
                                         emit_view=self.emit_view, view_edges=self.view_edges)
@@ -101,7 +101,7 @@ class NeighborSampler:
         if not self.replay_slots:
             return None
         slot = self._slots[self._next_slot]
-        if slot is None:
+        if slot is None or (slot.graph is None and slot.n_seed != seeds.numel()):
             slot = self._slots[self._next_slot] = _ReplaySlot(seeds.numel(), self.device)
         if slot.n_seed != seeds.numel():
             return None
@@ -171,7 +171,7 @@ class _ReplaySlot:
         self.out = None
         self.done = None
 
-    def run(self, sampler, seeds, rng_seed, stream):
+    def run(self, sampler, seeds, rng_seed):
         self.seeds.copy_(seeds)
         k = int(rng_seed) & 0xFFFFFFFFFFFFFFFF
         self.key[0] = k - (1 << 64) if k >= (1 << 63) else k

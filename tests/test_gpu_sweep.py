@@ -7,6 +7,8 @@ single- and multi-head weights, ring wrap-around with capacity 1 upwards, relati
 cache buffers from two rows upwards, graphs with multi-edges and isolated nodes.  Bars as elsewhere:
 bit-exact except the edge gradient (dot products in another order: 1e-5 of the sum of magnitudes)
 and the reduced-precision input gradients (1e-2)."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -39,7 +41,9 @@ def be():
 
 
 def case_seeds(master_seed, n):
-    return [int(s) for s in np.random.default_rng(master_seed).integers(1 << 30, size=n)]
+    # HISCACHE_SWEEP_SHIFT=k draws another fixed set of cases (for a longer sweep on demand)
+    shift = int(os.environ.get("HISCACHE_SWEEP_SHIFT", "0"))
+    return [int(s) for s in np.random.default_rng(master_seed + 1000 * shift).integers(1 << 30, size=n)]
 
 
 # ------------------------------------------------------------------------------ aggregation
