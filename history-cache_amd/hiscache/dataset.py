@@ -62,22 +62,30 @@ class ProcessedDataset:
     def train_idx(self):
         return self._array("train")
 
-    def feature_store(self, device="cuda:0", out_dtype=None, chunk_rows=1 << 20):
+    def feature_store(self, device="cuda:0", out_dtype=None, chunk_rows=1 << 20, in_device_memory=False):
         """Pinned, GPU-mapped copy of ``node_features.dat``, read from disk in chunks (the file is
-        never held twice in memory)."""
+        never held twice in memory).  ``in_device_memory``: the matrix goes to the GPU's own memory
+        instead (288 GB hold the papers100M matrix, 57 GB, beside its history table), and the store's
+        gathers read it there."""
         p = path.join(self.dir, "node_features.dat")
         want = self.num_nodes * self.feature_dim * self.feature_dtype.itemsize
         if os.path.getsize(p) != want:
             raise ValueError(f"{p}: {os.path.getsize(p)} bytes, expected {want}")
         src = np.memmap(p, dtype=self.feature_dtype, mode="r", shape=(self.num_nodes, self.feature_dim))
         tdtype = {np.dtype(np.float32): torch.float32, np.dtype(np.float16): torch.float16}[self.feature_dtype]
-        pinned = torch.empty((self.num_nodes, self.feature_dim), dtype=tdtype, pin_memory=True)
-        dst = pinned.numpy()
-        for lo in range(0, self.num_nodes, chunk_rows):
-            hi = min(self.num_nodes, lo + chunk_rows)
-            dst[lo:hi] = src[lo:hi]
+        if in_device_memory:
+            buf = torch.empty((self.num_nodes, self.feature_dim), dtype=tdtype, device=device)
+            for lo in range(0, self.num_nodes, chunk_rows):
+                hi = min(self.num_nodes, lo + chunk_rows)
+                buf[lo:hi].copy_(torch.from_numpy(np.array(src[lo:hi])))       # a writable copy of the chunk
+        else:
+            buf = torch.empty((self.num_nodes, self.feature_dim), dtype=tdtype, pin_memory=True)
+            dst = buf.numpy()
+            for lo in range(0, self.num_nodes, chunk_rows):
+                hi = min(self.num_nodes, lo + chunk_rows)
+                dst[lo:hi] = src[lo:hi]
         del src
-        return PinnedFeatureStore(pinned, device=device, out_dtype=out_dtype or torch.float32)
+        return PinnedFeatureStore(buf, device=device, out_dtype=out_dtype or torch.float32)
 
     def sampler(self, fanout, device="cuda:0", seed=0, emit_view=False, view_edges=False):
         """``emit_view``: every batch carries the transposed view of its CSR (``batch.view``), so that the

@@ -107,9 +107,10 @@ def _train_on_sampled_batches(mode):
     return losses
 
 
-def test_training_from_processed_files(tmp_path):
-    """Dataset directory -> feature store, sampler and cache (which reads num_nodes.txt and
-    sorted_indices.dat itself) -> a few training iterations."""
+@pytest.mark.parametrize("in_device_memory", [False, True])
+def test_training_from_processed_files(tmp_path, in_device_memory):
+    """Dataset directory -> feature store (pinned host memory, or the GPU's own), sampler and cache (which reads
+    num_nodes.txt and sorted_indices.dat itself) -> a few training iterations."""
     from hiscache import HistoryCache, HistorySAGE, ProcessedDataset, make_config, write_processed
     rng = np.random.default_rng(230)
     N, Fin, H, C, L = 3000, 16, 32, 4, 3
@@ -118,7 +119,8 @@ def test_training_from_processed_files(tmp_path):
     write_processed(tmp_path, indptr, indices, feats, hot_ids=rng.permutation(N), labels=rng.integers(0, C, size=N),
                     train_idx=rng.choice(N, size=600, replace=False))
     ds = ProcessedDataset(tmp_path, Fin)
-    store = ds.feature_store(device=DEV)
+    store = ds.feature_store(device=DEV, in_device_memory=in_device_memory)
+    assert store.buffer.is_cuda == in_device_memory
     np.testing.assert_array_equal(store.get(torch.tensor([0, 5, N - 1], device=DEV)).cpu().numpy(),
                                   feats[[0, 5, N - 1]])
     sampler = ds.sampler([4, 3, 2], device=DEV, seed=2, emit_view=True)
