@@ -143,6 +143,16 @@ def backward_on_this_thread(loss):
 
 
 PHASE_STEPS = 100
+LAST_CHUNKS = []          # ms per iteration of every chunk (an eighth of the steps) of the last bare pass
+
+
+def chunk_figures():
+    """Median and range of the per-chunk figures of the last ``time_iterations`` pass (device timeline)."""
+    c = sorted(LAST_CHUNKS)
+    if not c:
+        return None
+    return {"median": c[len(c) // 2] if len(c) % 2 else 0.5 * (c[len(c) // 2 - 1] + c[len(c) // 2]),
+            "min": c[0], "max": c[-1], "chunks": len(c)}
 
 
 def time_iterations(step, steps, clocks, reset=None):
@@ -154,17 +164,27 @@ def time_iterations(step, steps, clocks, reset=None):
     # every few hundred iterations): park what exists now in the permanent generation, as training loops do
     gc.collect()
     gc.freeze()
+    import torch
     KernelClock.enabled = False
+    chunk = max(1, steps // 8)
+    marks = []
     try:
         if reset:
             reset()
         t0 = time.perf_counter()
-        for _ in range(steps):
+        for i in range(steps):
+            if i % chunk == 0:                      # one event per chunk: where a one-off stall fell shows afterwards
+                marks.append(torch.cuda.Event(enable_timing=True))
+                marks[-1].record()
             step()
+        marks.append(torch.cuda.Event(enable_timing=True))
+        marks[-1].record()
         sync()
         sec = (time.perf_counter() - t0) / steps
     finally:
         KernelClock.enabled = True
+    spans = [(a.elapsed_time(b), min(chunk, steps - k * chunk)) for k, (a, b) in enumerate(zip(marks[:-1], marks[1:]))]
+    LAST_CHUNKS[:] = [ms / n for ms, n in spans if n == chunk]
     for c in clocks.values():
         c.reset()
     if reset:
@@ -799,6 +819,7 @@ def run_c3(args, with_batched=True):
                                   pool_rows, shape)},
         "phases_ms": {k: c.mean_ms() for k, c in ev.items()},
         "phases_host_enqueue_ms": {k: c.mean_cpu_ms() for k, c in ev.items()},
+        "ms_per_chunk_of_steps": chunk_figures(),
         "feature_store": "device memory" if args.features_in_hbm else "pinned host memory, read zero-copy",
         "transposed_view": "built in backward" if args.no_batch_view else "emitted with the batch",
         "feature_rows_read_last_batch": int(cache.used_masks[0].sum()),
@@ -900,6 +921,7 @@ def run_c5(args):
                                % (N, N, pool_rows, shape)},
         "phases_ms": {k: c.mean_ms() for k, c in ev.items()},
         "phases_host_enqueue_ms": {k: c.mean_cpu_ms() for k, c in ev.items()},
+        "ms_per_chunk_of_steps": chunk_figures(),
         "transposed_view": "built in backward" if args.no_batch_view else "emitted with the batch",
         "feature_rows_read_last_batch": int(cache.used_masks[0].sum()),
         "cached_1hop_fraction_last_batch": float((cache.sub2embed != -1).float().mean()),
@@ -984,6 +1006,7 @@ def run_c1(args):
                                "n2 %d, %d edges" % tuple(int(v) for v in m)},
         "phases_ms": {k: c.mean_ms() for k, c in ev.items()},
         "phases_host_enqueue_ms": {k: c.mean_cpu_ms() for k, c in ev.items()},
+        "ms_per_chunk_of_steps": chunk_figures(),
         "transposed_view": "built in backward" if args.no_batch_view else "emitted with the batch",
     }
     if cpu_model is not None:
@@ -1316,6 +1339,7 @@ def main():
                     "workload": r["config"]["workload"], "ms": r["ms_per_step"], "steps": r["steps"],
                     "warmup": r["warmup"], "transposed_view": r["transposed_view"],
                     "feature_read_ahead": bool(used_args.prefetch),
+                    "ms_per_chunk_of_steps": r.get("ms_per_chunk_of_steps"),
                     "phases_ms": r["phases_ms"], "phases_host_enqueue_ms": r["phases_host_enqueue_ms"]}
                 if "cpu_baseline" in r:          # c1, the CPU-runnable configuration: the same iteration on the host
                     res["iterations"][name]["cpu_ms"] = r["cpu_baseline"]["value"]
