@@ -87,13 +87,15 @@ class ProcessedDataset:
         del src
         return PinnedFeatureStore(buf, device=device, out_dtype=out_dtype or torch.float32)
 
-    def sampler(self, fanout, device="cuda:0", seed=0, emit_view=False, view_edges=False):
+    def sampler(self, fanout, device="cuda:0", seed=0, emit_view=False, view_edges=False, replay_slots=0):
         """``emit_view``: every batch carries the transposed view of its CSR (``batch.view``), so that the
-        layers' backward builds none; ``view_edges`` adds the edge slots the relational layer reads."""
+        layers' backward builds none; ``view_edges`` adds the edge slots the relational layer reads;
+        ``replay_slots``: see ``NeighborSampler`` (one HIP-graph launch per batch; a batch's arrays are
+        overwritten that many batches later)."""
         indptr, indices = self.graph()
         labels = self.labels() if self.has("labels") else None
         return NeighborSampler(indptr, indices, fanout, labels=labels, seed=seed, device=device,
-                               emit_view=emit_view, view_edges=view_edges)
+                               emit_view=emit_view, view_edges=view_edges, replay_slots=replay_slots)
 
 
 def write_processed(root, indptr, indices, features, hot_ids=None, labels=None, train_idx=None):
