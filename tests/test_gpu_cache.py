@@ -197,6 +197,25 @@ def test_fixup_rows_turns_a_guessed_gather_into_the_exact_one(src_dtype, out_dty
     assert torch.equal(out, before)
 
 
+def test_gather_rows_on_a_named_stream():
+    """gather_rows(stream=side) enqueues on that stream without switching torch's current one: the rows are
+    those of the call on the current stream once the streams have been ordered."""
+    import hiscache_backend as be
+    rng = np.random.default_rng(22)
+    table = torch.from_numpy(rng.standard_normal((4000, 64)).astype(np.float32)).pin_memory()
+    ids = torch.from_numpy(rng.integers(0, 4000, size=2500)).to(DEV)
+    mask = torch.from_numpy(rng.random(2500) < 0.7).to(DEV)
+    want = be.gather_rows(table, ids, mask=mask)
+    side = torch.cuda.Stream()
+    cur = torch.cuda.current_stream()
+    side.wait_stream(cur)
+    got = be.gather_rows(table, ids, mask=mask, stream=side)
+    got.record_stream(side)
+    assert torch.cuda.current_stream() == cur
+    cur.wait_stream(side)
+    assert torch.equal(got, want)
+
+
 @pytest.mark.parametrize("prefetch_cus", [0, 16])
 def test_speculative_prefetch_is_fixed_up_at_the_lookup(prefetch_cus):
     """The ring cache's read-ahead runs under the masks of the cache state at that moment; entries that are
