@@ -828,9 +828,11 @@ extern "C" int hc_evict(const int64_t *sub2slot, const float *score, const float
 // Admission threshold as a quantile of the scores: the two order statistics that
 // torch.quantile's linear interpolation reads (/root/reference/hiscache/history_cache.py:211,
 // history_table.py:173), found by a radix select instead of a sort, and the interpolation in
-// separately rounded fp32 steps.  One block; four 8-bit passes per order statistic over keys
-// that order like the floats (sign flipped for non-negative values, all bits for negative
-// ones).  Up to QT_MAX_N scores (a sampled batch's 1-hop nodes are a few thousand).
+// separately rounded fp32 steps.  One block; four 8-bit passes over keys that order like the
+// floats (sign flipped for non-negative values, all bits for negative ones) find the lower
+// statistic, one more pass the upper one where it is another key.  Up to 16 384 scores are
+// read once and kept in registers (a sampled batch's 1-hop nodes are a few thousand); up to
+// QT_MAX_N are read again in every pass.
 // ---------------------------------------------------------------------------------------
 namespace {
 
@@ -846,21 +848,49 @@ __device__ __forceinline__ float qt_value(uint32_t k) {
   return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
 
-// the key of rank k (0-based) among score[0, n); every thread returns it
-__device__ uint32_t qt_select(const float *__restrict__ score, int64_t n, int64_t k, int *hist, int *s_pick) {
+constexpr int QT_WAVES = QT_BLOCK / HC_WAVE;
+constexpr int QT_REG = 16;   // keys a thread keeps in registers: up to QT_BLOCK * QT_REG scores are read once
+
+struct QtShared {
+  int hist[QT_WAVES][256];   // one histogram per wave: lanes of different waves never meet on a counter
+  int total[256];
+  int pick[3];               // the bin that holds the rank, the keys in front of it, the keys inside it
+  uint32_t next;             // smallest key above the selected one
+};
+
+// The key of rank k (0-based) among the n scores; every thread returns it.  REG: the keys sit in the
+// thread's registers (rk[0, nk)), otherwise they are read from `score` in every pass.  *k_in_bin and *n_equal
+// return the rank's position among the keys equal to the result and how many those are.
+template <bool REG>
+__device__ uint32_t qt_select(const float *__restrict__ score, int64_t n, const uint32_t (&rk)[QT_REG], int nk,
+                              int64_t k, QtShared &sh, int64_t *k_in_bin, int *n_equal) {
   uint32_t prefix = 0u, mask = 0u;
+  const int wave = (int)(threadIdx.x / HC_WAVE);
   for (int shift = 24; shift >= 0; shift -= 8) {
-    for (int b = threadIdx.x; b < 256; b += QT_BLOCK) hist[b] = 0;
+    for (int b = threadIdx.x; b < QT_WAVES * 256; b += QT_BLOCK) (&sh.hist[0][0])[b] = 0;
     __syncthreads();
-    for (int64_t i = threadIdx.x; i < n; i += QT_BLOCK) {
-      const uint32_t key = qt_key(score[i]);
-      if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 0xffu], 1);
+    if constexpr (REG) {
+#pragma unroll
+      for (int j = 0; j < QT_REG; ++j)
+        if (j < nk && (rk[j] & mask) == prefix) atomicAdd(&sh.hist[wave][(rk[j] >> shift) & 0xffu], 1);
+    } else {
+      for (int64_t i = threadIdx.x; i < n; i += QT_BLOCK) {
+        const uint32_t key = qt_key(score[i]);
+        if ((key & mask) == prefix) atomicAdd(&sh.hist[wave][(key >> shift) & 0xffu], 1);
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < 256) {
+      int t = 0;
+#pragma unroll
+      for (int w = 0; w < QT_WAVES; ++w) t += sh.hist[w][threadIdx.x];
+      sh.total[threadIdx.x] = t;
     }
     __syncthreads();
     if (threadIdx.x < HC_WAVE) {
       // the bin that holds rank k: the first wave scans the 256 counts, four bins per lane
       const int l = (int)threadIdx.x;
-      const int c[4] = {hist[4 * l], hist[4 * l + 1], hist[4 * l + 2], hist[4 * l + 3]};
+      const int c[4] = {sh.total[4 * l], sh.total[4 * l + 1], sh.total[4 * l + 2], sh.total[4 * l + 3]};
       const int mine = (c[0] + c[1]) + (c[2] + c[3]);
       int x = mine;
 #pragma unroll
@@ -876,27 +906,76 @@ __device__ uint32_t qt_select(const float *__restrict__ score, int64_t n, int64_
           if ((int64_t)before + c[b] > k) break;
           before += c[b];
         }
-        s_pick[0] = 4 * l + b;
-        s_pick[1] = before;           // at most n < 2^31
+        sh.pick[0] = 4 * l + b;
+        sh.pick[1] = before;           // at most n < 2^31
+        sh.pick[2] = c[b];
       }
     }
     __syncthreads();
-    prefix |= (uint32_t)s_pick[0] << shift;
+    prefix |= (uint32_t)sh.pick[0] << shift;
     mask |= 0xffu << shift;
-    k -= s_pick[1];
+    k -= sh.pick[1];
+    *n_equal = sh.pick[2];
     __syncthreads();
   }
+  *k_in_bin = k;
   return prefix;
 }
 
+// The smallest key above `key`; every thread returns it (0xffffffff when there is none).
+template <bool REG>
+__device__ uint32_t qt_next_above(const float *__restrict__ score, int64_t n, const uint32_t (&rk)[QT_REG], int nk,
+                                  uint32_t key, QtShared &sh) {
+  if (threadIdx.x == 0) sh.next = 0xffffffffu;
+  __syncthreads();
+  uint32_t m = 0xffffffffu;
+  if constexpr (REG) {
+#pragma unroll
+    for (int j = 0; j < QT_REG; ++j)
+      if (j < nk && rk[j] > key && rk[j] < m) m = rk[j];
+  } else {
+    for (int64_t i = threadIdx.x; i < n; i += QT_BLOCK) {
+      const uint32_t x = qt_key(score[i]);
+      if (x > key && x < m) m = x;
+    }
+  }
+#pragma unroll
+  for (int d = HC_WAVE / 2; d > 0; d >>= 1) {
+    const uint32_t y = (uint32_t)__shfl_xor((int)m, d, HC_WAVE);
+    m = y < m ? y : m;
+  }
+  if (hc_lane() == 0 && m != 0xffffffffu) atomicMin(&sh.next, m);
+  __syncthreads();
+  return sh.next;
+}
+
+// One block.  The order statistic of rank lo by four 8-bit passes; the one of rank hi = lo + 1 is the same key
+// when the rank stays among the keys equal to it, else the smallest key above it (one more pass).
+template <bool REG>
 __global__ __launch_bounds__(QT_BLOCK) void quantile_kernel(const float *__restrict__ score, int64_t n, int64_t lo,
                                                              int64_t hi, float w, float one_minus_w,
                                                              float *__restrict__ out) {
-  __shared__ int hist[256];
-  __shared__ int s_pick[2];
-  const float a = qt_value(qt_select(score, n, lo, hist, s_pick));
-  const float b = hi == lo ? a : qt_value(qt_select(score, n, hi, hist, s_pick));
+  __shared__ QtShared sh;
+  uint32_t rk[QT_REG];
+  int nk = 0;
+  if constexpr (REG) {
+#pragma unroll
+    for (int j = 0; j < QT_REG; ++j) {
+      const int64_t i = (int64_t)j * QT_BLOCK + threadIdx.x;
+      rk[j] = 0u;
+      if (i < n) {
+        rk[j] = qt_key(score[i]);
+        nk = j + 1;
+      }
+    }
+  }
+  int64_t k_in_bin = 0;
+  int n_equal = 0;
+  const uint32_t ka = qt_select<REG>(score, n, rk, nk, lo, sh, &k_in_bin, &n_equal);
+  uint32_t kb = ka;
+  if (hi != lo && k_in_bin + 1 >= (int64_t)n_equal) kb = qt_next_above<REG>(score, n, rk, nk, ka, sh);
   if (threadIdx.x == 0) {
+    const float a = qt_value(ka), b = qt_value(kb);
     const float d = __fsub_rn(b, a);
     out[0] = w < 0.5f ? __fadd_rn(a, __fmul_rn(d, w)) : __fsub_rn(b, __fmul_rn(d, one_minus_w));
   }
@@ -910,7 +989,10 @@ extern "C" int hc_quantile_threshold(const float *score, int64_t n, int64_t lo, 
                                      float one_minus_w, float *out, void *stream) {
   HC_REQUIRE(score && out && n >= 1 && lo >= 0 && hi >= lo && hi < n && hi <= lo + 1);
   if (n > QT_MAX_N) return HC_EUNSUPPORTED;
-  quantile_kernel<<<dim3(1), dim3(QT_BLOCK), 0, static_cast<hipStream_t>(stream)>>>(score, n, lo, hi, w,
-                                                                                   one_minus_w, out);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (n <= (int64_t)QT_BLOCK * QT_REG)
+    quantile_kernel<true><<<dim3(1), dim3(QT_BLOCK), 0, st>>>(score, n, lo, hi, w, one_minus_w, out);
+  else
+    quantile_kernel<false><<<dim3(1), dim3(QT_BLOCK), 0, st>>>(score, n, lo, hi, w, one_minus_w, out);
   return hc_launch_status();
 }
