@@ -43,8 +43,12 @@ constexpr int W_NONE = 0, W_EDGE = 1, W_EDGE_HEAD = 2;
 // those chunks into partial[2 * window] and partial[2 * window + 1].  A second launch, again one wave
 // per window, combines the chunk sums of the hub that starts in its window, left to right.
 inline int64_t bwd_windows(int64_t E) { return (E + BWD_CHUNK - 1) / BWD_CHUNK; }
-inline size_t bwd_partial_bytes(int64_t E, int64_t F) {
+inline size_t bwd_partial_sums_bytes(int64_t E, int64_t F) {
   return hc_align_up((size_t)(2 * bwd_windows(E)) * (size_t)F * sizeof(float), 256);
+}
+// the chunk sums, then one word per window: the hub that starts in the window, or -1
+inline size_t bwd_partial_bytes(int64_t E, int64_t F) {
+  return bwd_partial_sums_bytes(E, F) + hc_align_up((size_t)bwd_windows(E) * sizeof(int64_t), 256);
 }
 
 // last s in [0, n_src) with ptrT[s] <= target (ptrT[0] == 0 <= target)
@@ -128,11 +132,18 @@ __device__ __forceinline__ void bwd_window_partials(const int64_t *__restrict__ 
                                                     const float *__restrict__ g,
                                                     const int64_t *__restrict__ hmap, int64_t R,
                                                     float *__restrict__ partial,
+                                                    int64_t *__restrict__ hub_of,
                                                     int64_t n_src, int64_t window, int lane) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   const int64_t wstart = window * BWD_CHUNK;
   const int64_t wend = wstart + BWD_CHUNK;
-  if (wstart >= ptrT[n_src]) return;
+  // hub_of[window]: the hub that starts in this window (bwd_hub_final combines its chunk sums), else -1;
+  // written for every window at every call, so that the final pass needs no search of its own
+  int64_t hub = -1;
+  if (wstart >= ptrT[n_src]) {
+    if (lane == 0) hub_of[window] = hub;
+    return;
+  }
   // lane 0 looks for the source that covers the window's first position, lane 1 for the last source that
   // starts inside the window; the other lanes repeat lane 1's search
   const int64_t found = bwd_last_source_at(ptrT, n_src, lane == 0 ? wstart : wend - 1);
@@ -149,6 +160,7 @@ __device__ __forceinline__ void bwd_window_partials(const int64_t *__restrict__ 
     } else {
       if (seg_b < wstart) continue;
       begin = seg_b;
+      hub = s;
     }
     const int64_t end = begin + BWD_CHUNK < seg_e ? begin + BWD_CHUNK : seg_e;
     float acc[CHUNKS][VEC];
@@ -161,6 +173,7 @@ __device__ __forceinline__ void bwd_window_partials(const int64_t *__restrict__ 
 #pragma unroll
     for (int k = 0; k < CHUNKS; ++k) hc_vec<float, VEC>::store(o + k * HC_WAVE * VEC, acc[k]);
   }
+  if (lane == 0) hub_of[window] = hub;
 }
 
 // One wave per window: if a hub starts in the window, its chunk sums are combined left to right into
@@ -168,18 +181,17 @@ __device__ __forceinline__ void bwd_window_partials(const int64_t *__restrict__ 
 template <int VEC, int CHUNKS>
 __global__ __launch_bounds__(HC_BLOCK) void bwd_hub_final(const int64_t *__restrict__ ptrT,
                                                            const float *__restrict__ partial,
+                                                           const int64_t *__restrict__ hub_of,
                                                            float *__restrict__ grad_vin, int64_t n_src,
                                                            int64_t windows) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   const int lane = hc_lane();
   const int64_t window = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
   if (window >= windows) return;
-  const int64_t wstart = window * BWD_CHUNK;
-  if (wstart >= ptrT[n_src]) return;
-  const int64_t s = hc_uniform64(bwd_last_source_at(ptrT, n_src, wstart + BWD_CHUNK - 1));
+  const int64_t s = hc_uniform64(hub_of[window]);      // left by the window's wave of bwd_mean_fast
+  if (s < 0 || s >= n_src) return;
   const int64_t seg_b = ptrT[s];
   const int64_t len = ptrT[s + 1] - seg_b;
-  if (len <= BWD_CHUNK || seg_b < wstart) return;
   const int nch = (int)((len + BWD_CHUNK - 1) / BWD_CHUNK);
   float acc[CHUNKS][VEC];
   const float *__restrict__ p0 = partial + (2 * window + 1) * F + lane * VEC;
@@ -214,7 +226,7 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     const int32_t *__restrict__ edgeT, const float *__restrict__ ev, int n_head, const float *__restrict__ g,
     const int64_t *__restrict__ hmap, float *__restrict__ grad_vin, float *__restrict__ grad_hbuf,
     int64_t hsize, int64_t R, int64_t n_src, int64_t src_blocks, int64_t hist_blocks, int64_t hub_thres,
-    float *__restrict__ partial, int64_t windows) {
+    float *__restrict__ partial, int64_t *__restrict__ hub_of, int64_t windows) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   constexpr bool WEIGHTED = WMODE != W_NONE;
   constexpr int S = BWD_SRC_PER_WAVE;
@@ -225,7 +237,8 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
     if constexpr (WMODE == W_NONE) {
       const int64_t window = ((int64_t)blockIdx.x - src_blocks - hist_blocks) * HC_WAVES_PER_BLOCK + wave;
       if (window < windows)
-        bwd_window_partials<VEC, CHUNKS, UNROLL, MASKED>(ptr, ptrT, rowT, g, hmap, R, partial, n_src, window, lane);
+        bwd_window_partials<VEC, CHUNKS, UNROLL, MASKED>(ptr, ptrT, rowT, g, hmap, R, partial, hub_of, n_src, window,
+                                                         lane);
     }
     return;
   }
@@ -731,6 +744,7 @@ int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, co
   const bool hubs = ev == nullptr && workspace != nullptr && E_slots > BWD_CHUNK && n_src > 0 &&
                     workspace_bytes >= bwd_partial_bytes(E_slots, F) && reinterpret_cast<uintptr_t>(ws) % 256 == 0;
   float *partial = reinterpret_cast<float *>(ws);
+  int64_t *hub_of = hubs ? reinterpret_cast<int64_t *>(ws + bwd_partial_sums_bytes(E_slots, F)) : nullptr;
   const int64_t windows = hubs ? bwd_windows(E_slots) : 0;
   const int64_t wb = (windows + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
   if (hubs) hub_thres = BWD_CHUNK;
@@ -740,22 +754,22 @@ int launch_fast(const int64_t *ptr, const int64_t *ptrT, const int32_t *rowT, co
   if (masked)
     bwd_mean_fast<VEC, CHUNKS, UNROLL, W_NONE, true><<<grid, block, 0, st>>>(
         ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hb, hub_thres, partial,
-        windows);
+        hub_of, windows);
   else if (ev != nullptr && n_head > 1)
     bwd_mean_fast<VEC, CHUNKS, UNROLL, W_EDGE_HEAD, false><<<grid, block, 0, st>>>(
         ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hb, hub_thres, partial,
-        windows);
+        hub_of, windows);
   else if (ev != nullptr)
     bwd_mean_fast<VEC, CHUNKS, UNROLL, W_EDGE, false><<<grid, block, 0, st>>>(
         ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hb, hub_thres, partial,
-        windows);
+        hub_of, windows);
   else
     bwd_mean_fast<VEC, CHUNKS, UNROLL, W_NONE, false><<<grid, block, 0, st>>>(
         ptr, ptrT, rowT, edgeT, ev, n_head, g, hmap, grad_vin, grad_hbuf, hsize, R, n_src, sb, hb, hub_thres, partial,
-        windows);
+        hub_of, windows);
   if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
   if (hubs) {
-    bwd_hub_final<VEC, CHUNKS><<<dim3((unsigned)wb), block, 0, st>>>(ptrT, partial, grad_vin, n_src, windows);
+    bwd_hub_final<VEC, CHUNKS><<<dim3((unsigned)wb), block, 0, st>>>(ptrT, partial, hub_of, grad_vin, n_src, windows);
   }
   return hc_launch_status();
 }
