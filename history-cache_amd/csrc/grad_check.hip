@@ -104,6 +104,32 @@ __device__ __forceinline__ float wave_scores(const float *__restrict__ grad, int
         if (lane == i0 + i) mine = s;
       }
     }
+  } else if (F <= 256 && F % 4 == 0 && (reinterpret_cast<uintptr_t>(grad) % 16) == 0) {
+    // narrow rows (one 16-byte piece per lane at most): the loads of 8 rows are in flight before the first
+    // reduction, instead of a load and a reduction per row one after the other; same sums in the same order
+    constexpr int RB = 8;
+    const bool has = (int64_t)lane * 4 < F;
+    for (int i0 = 0; i0 < GC_ROWS_PER_WAVE; i0 += RB) {
+      float4 v[RB];
+#pragma unroll
+      for (int i = 0; i < RB; ++i) {
+        const int64_t r = row0 + i0 + i;
+        v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (r < M && has) v[i] = *(reinterpret_cast<const float4 *>(grad + r * F) + lane);
+      }
+#pragma unroll
+      for (int i = 0; i < RB; ++i) {
+        float acc = 0.0f;
+        if (has) {
+          acc = fold(acc, v[i].x, norm_kind);
+          acc = fold(acc, v[i].y, norm_kind);
+          acc = fold(acc, v[i].z, norm_kind);
+          acc = fold(acc, v[i].w, norm_kind);
+        }
+        const float s = finish_score(acc, norm_kind);
+        if (lane == i0 + i) mine = s;
+      }
+    }
   } else {
     for (int i = 0; i < GC_ROWS_PER_WAVE; ++i) {
       const int64_t r = row0 + i;
