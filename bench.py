@@ -71,7 +71,7 @@ def parse():
     ap.add_argument("--no-batch-view", action="store_true",
                     help="c3/c5: batches come without the transposed view of their CSR, so every layer's "
                          "backward builds one (the default: the loader emits it with the batch)")
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c2row", "c2w", "c4", "c3", "c3b", "c5", "sample", "layer", "copy", "ceilings"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c2row", "c2w", "c4", "c3", "c3b", "c5", "sample", "layer", "copy"])
     ap.add_argument("--heads", type=int, default=1, help="c2w: heads of the weighted aggregation (divides 256)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--reps", type=int, default=8, help="c3b: measurements with freshly allocated tensors")
@@ -1135,37 +1135,6 @@ def run_copy(args):
             "config": {"workload": "copy: 4 GiB fp32 device-to-device copy (4 GiB read + 4 GiB written)"}}
 
 
-def run_ceilings(args):
-    """What the memory system delivers to bare kernels (stream read, fill, copy, random row gathers): runs
-    the ``hbm_probe`` program (history-cache_amd/probe, built on demand) as a child process and returns its
-    table."""
-    import subprocess
-    probe_dir = os.path.join(ROOT, "history-cache_amd", "probe")
-    exe = os.path.join(probe_dir, "hbm_probe")
-    if not os.path.exists(exe):
-        subprocess.check_call(["make", "-C", probe_dir])
-    gb = 20.0 * args.scale
-    out = subprocess.run([exe, "%.3f" % gb], check=True, capture_output=True, text=True, timeout=300).stdout
-    lines = [ln.rstrip() for ln in out.splitlines() if ln.strip()]
-    for ln in lines:
-        print(ln, file=sys.stderr)
-    rates = {}
-    for ln in lines:
-        if ln.startswith(("stream read", "fill", "stream copy")):
-            name = ln[:14].strip()
-            rates[name] = float(ln.split("ms")[1].split()[0])
-        elif "ordinary loads" in ln or "non-temporal loads" in ln:
-            t = ln.split()
-            kind = "gather 1 KiB " + ("nt" if "non-temporal" in ln else "ordinary")
-            rates[kind] = {t[i].rstrip("="): float(t[i + 1]) for i in range(len(t) - 1) if t[i].startswith("U=")}
-        elif ln.startswith("row gather") and "GB/s" in ln and ":" in ln and "rows per launch" not in ln:
-            rates["gather " + " ".join(ln.split()[2:4]).rstrip(",")] = float(ln.split(":")[1].split()[0])
-    best = max(rates.get("gather 1 KiB ordinary", {"U": 0.0}).values())
-    return {"metric": "random 1 KiB row gather GB/s (bare kernel)", "value": best, "unit": "GB/s", "n_gpus": 1,
-            "steps": 5, "warmup": 2, "higher_is_better": True,
-            "config": {"workload": "ceilings: hbm_probe over a %.1f GB table" % gb}, "rates_GBps": rates}
-
-
 def device_power_law_graph(N, mean_degree, dev, gen, max_degree=100_000):
     """CSR of a directed graph generated on the device: log-normal out-degrees (sigma 1.2) with the
     given mean, neighbour ids skewed towards popular nodes (u^3 over the id range, scattered by a
@@ -1284,9 +1253,6 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path (the reference's multi-GPU trainer "
               "and comm.cu are out of scope); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
-    if args.workload == "ceilings":          # a child process does the measuring; nothing here touches the GPU
-        print(json.dumps(run_ceilings(args)))
-        return
     import torch
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)

@@ -19,6 +19,7 @@
 #include <rocprim/rocprim.hpp>
 
 #include "hc_common.h"
+#include "tr_shared.h"
 
 namespace {
 
@@ -35,43 +36,6 @@ constexpr int TR_LDS_ROWS = 2048;
 constexpr int64_t TR_SORT_MEMSET_EDGES = 1 << 20;  // rocPRIM sorts up to this many pairs by merging (kernels only)
 constexpr int TR_ITEMS_LARGE = 8;
 constexpr int64_t TR_SMALL_EDGES = 1 << 18;
-
-// largest r in [lo, hi] with ptr[r] <= e (ptr[lo] <= e is the caller's business)
-template <typename P>
-__device__ __forceinline__ int64_t tr_row_of(P ptr, int64_t lo, int64_t hi, int64_t e) {
-  while (lo < hi) {
-    const int64_t mid = (lo + hi + 1) >> 1;
-    if (ptr[mid] <= e) lo = mid;
-    else hi = mid - 1;
-  }
-  return lo;
-}
-
-// The same search by a whole wave, 64 probes per memory round trip (three round trips for 2^18 rows
-// instead of eighteen): largest r in [0, R] with ptr[r] <= e, assuming ptr[0] <= e.  Every lane
-// returns the result.
-__device__ __forceinline__ int64_t tr_row_of_wave(const int64_t *__restrict__ ptr, int64_t R, int64_t e,
-                                                  int lane) {
-  int64_t lo = 0, hi = R;   // ptr[lo] <= e; the answer lies in [lo, hi]
-  while (hi > lo) {
-    const int64_t step = (hi - lo + HC_WAVE - 1) / HC_WAVE;
-    int64_t p = lo + (int64_t)(lane + 1) * step;
-    if (p > hi) p = hi;
-    const unsigned long long ok = __ballot(ptr[p] <= e);   // a prefix of the lanes: ptr does not decrease
-    const int k = __popcll(ok);
-    int64_t nlo = lo + (int64_t)k * step;                  // the last probe that held (lo itself when k == 0)
-    if (nlo > hi) nlo = hi;
-    int64_t nhi = hi;
-    if (k < HC_WAVE) {
-      nhi = lo + (int64_t)(k + 1) * step;                  // the first probe that failed, minus one
-      if (nhi > hi) nhi = hi;
-      nhi -= 1;
-    }
-    lo = nlo;
-    hi = nhi < nlo ? nlo : nhi;
-  }
-  return lo;
-}
 
 template <bool VAL_IS_ROW, int TR_ITEMS>
 __global__ __launch_bounds__(HC_BLOCK) void tr_expand_edges(const int64_t *__restrict__ ptr,
@@ -621,6 +585,10 @@ SmallLayout small_layout(int64_t E, int64_t n_src) {
   return L;
 }
 inline bool small_block(int64_t E, int64_t n_src) { return E <= TR_SMALL_EDGES && n_src <= TR_SMALL_SOURCES; }
+// Large blocks go to the bucket sort of view_sort.hip; what it does not cover (more than 2^28 edge slots or
+// about 44 M sources) and the blocks between the two sizes stay with the library sort below.
+constexpr int64_t TR_BUCKET_SORT_EDGES = (int64_t)1 << 20;
+inline bool bucket_sorted(int64_t E, int64_t n_src) { return E > TR_BUCKET_SORT_EDGES && vs_supported(E, n_src); }
 
 // The four launches of the counting sort; dims.E / dims.n_src size the grids (upper bounds when the real
 // sizes are read on the device).
@@ -709,6 +677,7 @@ extern "C" size_t hc_transpose_workspace_bytes(int64_t R, int64_t E, int64_t n_s
   (void)R;
   if (E < 0 || n_src < 0) return 0;
   if (small_block(E, n_src)) return small_layout(E, n_src).total;   // no library query on this path
+  if (bucket_sorted(E, n_src)) return vs_workspace_bytes(E, n_src);
   Layout L;
   if (!make_layout(E, n_src, &L)) return 0;
   return L.total;
@@ -737,6 +706,11 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
     if (reinterpret_cast<uintptr_t>(w) % 256 != 0) return HC_EWORKSPACE;
     const TrDims dims{R, E, n_src, nullptr, nullptr, nullptr};
     return small_launch(ptr, idx, hmap_row, hmap_src, dims, ptrT, rowT, edgeT, w, S, st);
+  }
+  if (bucket_sorted(E, n_src)) {
+    char *w = static_cast<char *>(workspace);
+    if (!workspace || reinterpret_cast<uintptr_t>(w) % 256 != 0) return HC_EWORKSPACE;
+    return vs_launch(ptr, idx, hmap_row, hmap_src, R, E, n_src, ptrT, rowT, edgeT, w, workspace_bytes, st);
   }
   if (E > TR_SORT_MEMSET_EDGES) {
     // Above this size the sort library takes its one-sweep path, which clears its counters with

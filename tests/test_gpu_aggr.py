@@ -550,12 +550,12 @@ def test_weighted_fast_path_prefix_rows_and_dtypes(be, orc, dtype):
 
 
 def test_c_abi_from_a_program_without_python():
-    """history-cache_amd/abi_demo (built with the library): hipMalloc'd buffers, raw pointers, status
+    """tests/abi_demo/abi_demo (built against the library): hipMalloc'd buffers, raw pointers, status
     codes; it checks forward, transposed view and backward of a 4-row block against hand-worked values."""
     import os
     import subprocess
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    exe = os.path.join(root, "history-cache_amd", "abi_demo")
-    assert os.path.exists(exe), "abi_demo is built by make -C history-cache_amd/csrc"
+    exe = os.path.join(root, "tests", "abi_demo", "abi_demo")
+    assert os.path.exists(exe), "abi_demo is built by make -C tests/abi_demo"
     p = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert p.returncode == 0 and p.stdout.startswith("abi_demo: ok"), (p.returncode, p.stdout, p.stderr)
