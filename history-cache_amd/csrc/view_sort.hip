@@ -13,30 +13,40 @@
 //               exclusive offsets of every (tile, bucket) pair inside its bucket, in tile order
 //               (groups of 8 tiles; a wave scans one bucket's groups), and the buckets' offsets
 //   vs_scatter  block per tile again: every live slot is ranked among the slots of its bucket in the
-//               tile, in slot order (the four waves of the block own consecutive quarters of the
-//               tile; inside a wave 64 consecutive slots are ranked at a time by matching bucket
-//               ids bit by bit with ballots, the running per-wave count of a bucket lives in LDS),
-//               and (local id, value) goes to its final place inside the bucket: the partition is
-//               stable.  value = destination row (mean aggregation) or the edge slot
-//   vs_bucket   one wave per bucket: counts the local ids (LDS), scans them -- which IS this bucket's
-//               stretch of ptrT --, then ranks the bucket's pairs in order, 64 at a time with the same
-//               ballot matching, and writes rowT (and edgeT) at segment start + rank
-// Every (source, slot) pair therefore lands where a stable sort by source puts it; the passes move
-// 8 bytes per live slot twice instead of three to four radix passes over all slots.
+//               tile, in slot order, and (local id, value) goes to its final place inside the bucket:
+//               the partition is stable.  The eight waves of the block own consecutive eighths of the
+//               tile and keep a running count per bucket in LDS; a wave ranks 64 consecutive slots
+//               at a time (see vs_rank_among_equal).  value = destination row (mean aggregation)
+//               or the edge slot
+//   vs_bucket   block per bucket: counts the local ids per wave (the four waves own consecutive
+//               quarters of the bucket's pairs), scans them -- which IS this bucket's stretch of
+//               ptrT --, ranks the pairs in order the same way and writes rowT (and edgeT) at segment
+//               start + rank, through LDS so that the stores are whole lines
+// Every (source, slot) pair therefore lands where a stable sort by source puts it.  The cost is set
+// by the number of memory requests rather than by bytes: the scattered 8-byte stores of vs_scatter
+// are one request per live slot, which is why there are two levels and not three, and why everything
+// else is staged so that its requests are whole lines.
+#include <cstdlib>
+
 #include "tr_shared.h"
 
 namespace {
 
-constexpr int VS_WAVES = 4;
+constexpr int VS_WAVES = 8;                              // waves per block of vs_count / vs_scatter
 constexpr int VS_THREADS = VS_WAVES * HC_WAVE;
-constexpr int VS_ITERS = 32;                             // edge slots per lane
-constexpr int VS_WAVE_SLOTS = HC_WAVE * VS_ITERS;        // 2048 consecutive slots per wave
+constexpr int VS_ITERS = 16;                             // edge slots per lane
+constexpr int VS_WAVE_SLOTS = HC_WAVE * VS_ITERS;        // 1024 consecutive slots per wave
 constexpr int VS_TILE = VS_WAVES * VS_WAVE_SLOTS;        // 8192 slots per block
 constexpr int VS_GROUP = 8;                              // tiles per group of the offset scan
-constexpr int VS_MAX_BUCKETS = 5376;                     // 12 bytes of LDS per bucket in vs_scatter: 63 KB
-constexpr int VS_MAX_LOCAL_BITS = 13;                    // 4 bytes of LDS per local id in vs_bucket: 32 KB
+constexpr int VS_MAX_BUCKETS = 5376;                     // 20 bytes of LDS per bucket in vs_scatter: 105 KB
+constexpr int VS_MAX_LOCAL_BITS = 13;                    // 16 bytes of LDS per local id in vs_bucket: 128 KB
 constexpr int64_t VS_MAX_EDGES = (int64_t)1 << 28;       // the per-tile counts stay a few hundred MB
 constexpr uint32_t VS_DEAD = 0xffffffffu;
+
+constexpr int VB_WAVES = 4;                              // waves per block of vs_bucket
+constexpr int VB_THREADS = VB_WAVES * HC_WAVE;
+constexpr int VB_ITERS = 32;                             // pairs per lane on the register path
+constexpr uint32_t VB_STAGED = VB_THREADS * VB_ITERS;    // 8192: largest bucket that takes the register path
 
 // Tile of a block: workgroup i runs on XCD i % 8, and every XCD gets one contiguous eighth of the
 // tiles, so that the partial lines at the write front of every bucket (runs of a few pairs per tile)
@@ -56,16 +66,22 @@ __device__ __forceinline__ uint32_t vs_wave_incl_scan(uint32_t v, int lane) {
   return v;
 }
 
-// The lanes of the wave whose `id` equals this lane's, among the lanes of `live` (bits [0, nbits) of id
-// are compared).  A lane outside `live` gets a meaningless mask.
-__device__ __forceinline__ unsigned long long vs_match(uint32_t id, int nbits, unsigned long long live) {
-  unsigned long long peers = live;
-  for (int bit = 0; bit < nbits; ++bit) {
-    const bool one = ((id >> bit) & 1u) != 0u;
-    const unsigned long long bal = __ballot(one);
-    peers &= one ? bal : ~bal;
+// Rank of this lane among the live lanes of the wave that hold the same id, in lane order.  `same` is
+// the number of such lanes (this one included), which the caller reads off the id's counter: its value
+// behind the wave's adds minus its value in front of them.  A lane that is alone with its id (most are)
+// needs no matching; the others are matched one distinct id per round.
+__device__ __forceinline__ uint32_t vs_rank_among_equal(uint32_t id, bool live, uint32_t same,
+                                                        unsigned long long below) {
+  uint32_t rank = 0u;
+  unsigned long long dups = __ballot(live && same > 1u);
+  while (dups != 0ull) {                                   // wave-uniform
+    const int l = __builtin_ctzll(dups);
+    const uint32_t v = (uint32_t)__builtin_amdgcn_readlane((int)id, l);
+    const unsigned long long grp = __ballot(live && id == v);
+    if (live && id == v) rank = (uint32_t)__popcll(grp & below);
+    dups &= ~grp;
   }
-  return peers;
+  return rank;
 }
 
 // ---- destination row of an edge slot, for the slots of one tile -------------------------------
@@ -156,10 +172,10 @@ struct VsShape {
   int64_t R, E, n_src;
   int64_t ntiles, ngroups;
   int lb;          // bits of a local id
-  int bbits;       // bits of a bucket id
   int nb;          // buckets: ids 0 .. n_src (ptrT has an entry for n_src too)
   int nbp;         // row pitch of the per-tile and per-group count matrices
-  int nbc;         // pitch of a wave's 16-bit counters in vs_scatter's LDS
+  int nbc;         // pitch of a wave's 16-bit counters in vs_scatter's LDS (even)
+  int dbg;
 };
 
 template <bool ROWMAP>
@@ -167,6 +183,7 @@ __global__ __launch_bounds__(VS_THREADS) void vs_count(const int64_t *__restrict
                                                         const int64_t *__restrict__ idx,
                                                         const int64_t *__restrict__ hmap_row,
                                                         const uint32_t *__restrict__ src_bits,
+                                                        const uint8_t *__restrict__ edge_drop,
                                                         uint32_t *__restrict__ key32,
                                                         uint16_t *__restrict__ tile_count, VsShape S) {
   __shared__ uint32_t hist[VS_MAX_BUCKETS];
@@ -181,8 +198,6 @@ __global__ __launch_bounds__(VS_THREADS) void vs_count(const int64_t *__restrict
   const int64_t first = ptr[0], last = ptr[S.R];
   const int64_t a = e0 > first ? e0 : first;             // the tile's slots inside the first R rows: [a, bnd)
   const int64_t bnd = e1 < last ? e1 : last;
-  if (ROWMAP && a < bnd) vs_rows_setup(rf, ptr, S.R, e0, a, bnd);   // block-uniform condition
-  else __syncthreads();
   const int64_t base = e0 + (int64_t)wave * VS_WAVE_SLOTS + lane;
   int64_t src[VS_ITERS];
 #pragma unroll
@@ -190,6 +205,19 @@ __global__ __launch_bounds__(VS_THREADS) void vs_count(const int64_t *__restrict
     const int64_t e = base + (int64_t)j * HC_WAVE;
     src[j] = (e >= a && e < bnd) ? __builtin_nontemporal_load(idx + e) : -1;
   }
+  if (edge_drop != nullptr) {
+    uint8_t d[VS_ITERS];
+#pragma unroll
+    for (int j = 0; j < VS_ITERS; ++j) {
+      const int64_t e = base + (int64_t)j * HC_WAVE;
+      d[j] = (e >= a && e < bnd) ? __builtin_nontemporal_load(edge_drop + e) : (uint8_t)0;
+    }
+#pragma unroll
+    for (int j = 0; j < VS_ITERS; ++j)
+      if (d[j] != 0) src[j] = -1;
+  }
+  if (ROWMAP && a < bnd) vs_rows_setup(rf, ptr, S.R, e0, a, bnd);   // block-uniform condition
+  else __syncthreads();
 #pragma unroll
   for (int j = 0; j < VS_ITERS; ++j)
     if (src[j] >= S.n_src) src[j] = -1;
@@ -216,7 +244,7 @@ __global__ __launch_bounds__(VS_THREADS) void vs_count(const int64_t *__restrict
   for (int j = 0; j < VS_ITERS; ++j) {
     const int64_t e = base + (int64_t)j * HC_WAVE;
     const uint32_t key = src[j] >= 0 ? (uint32_t)src[j] : VS_DEAD;
-    if (e < e1) key32[e] = key;
+    if (e < e1) __builtin_nontemporal_store(key, key32 + e);
     if (src[j] >= 0) atomicAdd(&hist[key >> S.lb], 1u);
   }
   __syncthreads();
@@ -224,17 +252,25 @@ __global__ __launch_bounds__(VS_THREADS) void vs_count(const int64_t *__restrict
   for (int b = tid; b < S.nb; b += VS_THREADS) row[b] = (uint16_t)hist[b];   // at most VS_TILE
 }
 
-// group_count[g][b] = live slots of bucket b in the tiles of group g
-__global__ __launch_bounds__(HC_BLOCK) void vs_group_sum(const uint16_t *__restrict__ tile_count,
+// group_count[g][b] = live slots of bucket b in the tiles of group g; the tiles' own counts become
+// exclusive offsets inside their group (at most 7 * VS_TILE: 16 bits hold them).
+__global__ __launch_bounds__(HC_BLOCK) void vs_group_sum(uint16_t *__restrict__ tile_count,
                                                           uint32_t *__restrict__ group_count, VsShape S) {
   const int b = (int)(blockIdx.x * HC_BLOCK + threadIdx.x);
   const int64_t g = blockIdx.y;
   if (b >= S.nb) return;
+  uint32_t c[VS_GROUP];
+#pragma unroll
+  for (int i = 0; i < VS_GROUP; ++i) {
+    const int64_t t = g * VS_GROUP + i;
+    c[i] = t < S.ntiles ? tile_count[t * S.nbp + b] : 0u;
+  }
   uint32_t sum = 0u;
 #pragma unroll
   for (int i = 0; i < VS_GROUP; ++i) {
     const int64_t t = g * VS_GROUP + i;
-    if (t < S.ntiles) sum += tile_count[t * S.nbp + b];
+    if (t < S.ntiles) tile_count[t * S.nbp + b] = (uint16_t)sum;
+    sum += c[i];
   }
   group_count[g * S.nbp + b] = sum;
 }
@@ -287,11 +323,12 @@ __global__ __launch_bounds__(VS_OFF_THREADS) void vs_bucket_offsets(const uint32
   }
 }
 
-// Dynamic LDS: uint32 base[nb] (the tile's first position in every bucket), then uint16 cnt[4][nbc].
+// Dynamic LDS: uint32 base[nbc] (the tile's first position in every bucket), then the waves'
+// 16-bit counters, cnt[VS_WAVES][nbc], two to a 32-bit word.
 template <bool VAL_IS_ROW>
 __global__ __launch_bounds__(VS_THREADS) void vs_scatter(const int64_t *__restrict__ ptr,
                                                           const uint32_t *__restrict__ key32,
-                                                          const uint16_t *__restrict__ tile_count,
+                                                          const uint16_t *__restrict__ tile_off,
                                                           const uint32_t *__restrict__ group_off,
                                                           const uint32_t *__restrict__ bucket_off,
                                                           uint2 *__restrict__ pairs, uint32_t *__restrict__ rows,
@@ -299,60 +336,82 @@ __global__ __launch_bounds__(VS_THREADS) void vs_scatter(const int64_t *__restri
   extern __shared__ uint32_t vs_lds[];
   __shared__ VsRowFinder rf;
   uint32_t *gbase = vs_lds;
-  uint16_t *cnt = reinterpret_cast<uint16_t *>(vs_lds + S.nbc);
+  uint32_t *cnt32 = vs_lds + S.nbc;
+  uint16_t *cnt = reinterpret_cast<uint16_t *>(cnt32);
   const int tid = (int)threadIdx.x;
   const int lane = hc_lane();
   const int wave = tid >> 6;
   const int64_t tile = vs_tile_of_block(blockIdx.x, S.ntiles);
   const int64_t e0 = tile * VS_TILE;
   const int64_t e1 = e0 + VS_TILE < S.E ? e0 + VS_TILE : S.E;
-  {
-    uint32_t *c32 = reinterpret_cast<uint32_t *>(cnt);
-    for (int i = tid; i < VS_WAVES * S.nbc / 2; i += VS_THREADS) c32[i] = 0u;
-  }
-  const int64_t first = ptr[0], last = ptr[S.R];
-  const int64_t a = e0 > first ? e0 : first;
-  const int64_t bnd = e1 < last ? e1 : last;
-  if (a < bnd) vs_rows_setup(rf, ptr, S.R, e0, a, bnd);   // block-uniform condition
-  else __syncthreads();
   const int64_t base = e0 + (int64_t)wave * VS_WAVE_SLOTS + lane;
-  uint32_t key[VS_ITERS];
+  uint32_t key[VS_ITERS];                                 // in flight while the rows are set up
 #pragma unroll
   for (int j = 0; j < VS_ITERS; ++j) {
     const int64_t e = base + (int64_t)j * HC_WAVE;
     key[j] = e < e1 ? __builtin_nontemporal_load(key32 + e) : VS_DEAD;
   }
-  // rank of every live slot among the slots of its bucket in this wave's quarter, in slot order
-  uint16_t *mine = cnt + wave * S.nbc;
+  for (int i = tid; i < VS_WAVES * S.nbc / 2; i += VS_THREADS) cnt32[i] = 0u;
+  const int64_t first = ptr[0], last = ptr[S.R];
+  const int64_t a = e0 > first ? e0 : first;
+  const int64_t bnd = e1 < last ? e1 : last;
+  if (a < bnd) vs_rows_setup(rf, ptr, S.R, e0, a, bnd);   // block-uniform condition
+  else __syncthreads();
+  if (S.dbg == 3) { if (key[S.dbg] == 12345u) rows[0] = 1u; return; }
+  // Rank of every live slot among the slots of its bucket in this wave's eighth of the tile, in slot
+  // order: the bucket's running count in front of these 64 slots plus the rank among them.
+  uint32_t *mine32 = cnt32 + wave * (S.nbc / 2);
   const unsigned long long below = (1ull << lane) - 1ull;
   uint32_t rk[VS_ITERS];
 #pragma unroll
   for (int j = 0; j < VS_ITERS; ++j) {
     const bool live = key[j] != VS_DEAD;
     const uint32_t b = key[j] >> S.lb;
-    const unsigned long long peers = vs_match(b, S.bbits, __ballot(live));
-    uint32_t pre = 0u;
-    if (live) pre = mine[b];
-    if (live && (peers >> lane) == 1ull) mine[b] = (uint16_t)(pre + (uint32_t)__popcll(peers));   // the group's last lane
-    rk[j] = pre + (uint32_t)__popcll(peers & below);
+    uint32_t before = 0u, same = 0u;
+    if (live) {
+      const uint32_t sh = (b & 1u) * 16u;
+      const uint32_t w0 = mine32[b >> 1];
+      atomicAdd(&mine32[b >> 1], 1u << sh);
+      const uint32_t w1 = mine32[b >> 1];
+      before = (w0 >> sh) & 0xffffu;
+      same = ((w1 >> sh) & 0xffffu) - before;
+    }
+    rk[j] = before + vs_rank_among_equal(b, live, same, below);
   }
   __syncthreads();
-  // the waves' counts become offsets of the quarters; base = the tile's first position in the bucket
+  if (S.dbg == 4) { if (rk[S.dbg] == 12345u) rows[0] = 1u; return; }
+  // the waves' counts become the eighths' offsets; base = the tile's first position in the bucket
   {
     const int64_t g = tile / VS_GROUP;
-    const int t_in = (int)(tile - g * VS_GROUP);
-    for (int b = tid; b < S.nb; b += VS_THREADS) {
-      uint32_t p = bucket_off[b] + group_off[g * S.nbp + b];
-      for (int i = 0; i < t_in; ++i) p += tile_count[(g * VS_GROUP + i) * S.nbp + b];
-      const uint32_t c0 = cnt[b], c1 = cnt[S.nbc + b], c2 = cnt[2 * S.nbc + b];
-      cnt[b] = 0;
-      cnt[S.nbc + b] = (uint16_t)c0;
-      cnt[2 * S.nbc + b] = (uint16_t)(c0 + c1);
-      cnt[3 * S.nbc + b] = (uint16_t)(c0 + c1 + c2);
-      gbase[b] = p;
+    const uint32_t *grow = group_off + g * S.nbp;
+    const uint16_t *trow = tile_off + tile * S.nbp;
+    constexpr int Q = 2;
+    for (int b0 = tid; b0 < S.nb; b0 += Q * VS_THREADS) {
+      uint32_t p[Q];
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        const int b = b0 + q * VS_THREADS;
+        p[q] = b < S.nb ? bucket_off[b] + grow[b] + trow[b] : 0u;
+      }
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        const int b = b0 + q * VS_THREADS;
+        if (b < S.nb) {
+          uint32_t run = 0u;
+#pragma unroll
+          for (int w = 0; w < VS_WAVES; ++w) {
+            const uint32_t c = cnt[w * S.nbc + b];
+            cnt[w * S.nbc + b] = (uint16_t)run;
+            run += c;
+          }
+          gbase[b] = p[q];
+        }
+      }
     }
   }
   __syncthreads();
+  if (S.dbg == 5) { if (rk[S.dbg] == 12345u) rows[0] = 1u; return; }
+  const uint16_t *mine = cnt + wave * S.nbc;
   const uint32_t local_mask = (1u << S.lb) - 1u;
 #pragma unroll
   for (int j = 0; j < VS_ITERS; ++j) {
@@ -370,63 +429,207 @@ __global__ __launch_bounds__(VS_THREADS) void vs_scatter(const int64_t *__restri
   }
 }
 
+// ---- vs_bucket -------------------------------------------------------------------------------------
+// Cursor arrays in LDS, one per wave, indexed by local id.  The scan hands 16 consecutive ids to a
+// thread; the swizzles spread the runs of neighbouring threads over the banks.
+// 32-bit cursors (buckets of any size): word k -> vb_swz32(k).
+__device__ __forceinline__ uint32_t vb_swz32(uint32_t k) { return (k & ~15u) | ((k & 15u) ^ ((k >> 5) & 15u)); }
+// 16-bit cursors (buckets of at most VB_STAGED pairs), two to a word: word k / 2 -> vb_swz16w(k / 2).
+__device__ __forceinline__ uint32_t vb_swz16w(uint32_t w) { return (w & ~7u) | ((w & 7u) ^ ((w >> 5) & 7u)); }
+
+// Buckets of at most VB_STAGED pairs: the pairs are read once and stay in registers, the cursors are
+// 16 bits wide and the bucket's stretch of rowT is put together in LDS and stored line by line.
+// LDS: cur16[VB_WAVES][n_local] (as words), then stage[VB_STAGED].
 template <bool WANT_EDGES>
-__global__ __launch_bounds__(HC_WAVE) void vs_bucket(const uint2 *__restrict__ pairs,
-                                                      const uint32_t *__restrict__ bucket_off,
-                                                      const uint32_t *__restrict__ rows,
-                                                      int64_t *__restrict__ ptrT, int32_t *__restrict__ rowT,
-                                                      int32_t *__restrict__ edgeT, VsShape S) {
-  extern __shared__ uint32_t cur[];                      // one cursor per local id
+__device__ __forceinline__ void vb_small(const uint2 *__restrict__ mine, uint32_t n, uint32_t p0, int64_t b,
+                                         uint32_t *__restrict__ lds, uint32_t *__restrict__ s_wave,
+                                         const uint32_t *__restrict__ rows, int64_t *__restrict__ ptrT,
+                                         int32_t *__restrict__ rowT, int32_t *__restrict__ edgeT, const VsShape &S) {
+  const int tid = (int)threadIdx.x;
   const int lane = hc_lane();
-  const int64_t b = blockIdx.x;
-  const int n_local = 1 << S.lb;
-  const uint32_t p0 = bucket_off[b];
-  const uint32_t n = bucket_off[b + 1] - p0;
-  const uint2 *mine = pairs + p0;
-  for (int k = lane; k < n_local; k += HC_WAVE) cur[k] = 0u;
+  const int wave = tid >> 6;
+  const uint32_t n_local = 1u << S.lb;
+  const uint32_t words = (n_local + 1u) / 2u;             // cursor words per wave
+  uint32_t *stage = lds + VB_WAVES * words;
+  uint32_t *my = lds + (uint32_t)wave * words;
+  // the four waves own consecutive quarters of the bucket's pairs
+  const uint32_t quarter = ((n + VB_WAVES - 1) / VB_WAVES + HC_WAVE - 1) / HC_WAVE * HC_WAVE;
+  const uint32_t q_begin = (uint32_t)wave * quarter < n ? (uint32_t)wave * quarter : n;
+  const uint32_t q_len = q_begin + quarter < n ? quarter : n - q_begin;
+  uint2 pr[VB_ITERS];
+#pragma unroll
+  for (int j = 0; j < VB_ITERS; ++j) {
+    const uint32_t i = (uint32_t)j * HC_WAVE + lane;
+    pr[j] = i < q_len ? mine[q_begin + i] : make_uint2(0u, 0u);
+  }
+  for (uint32_t i = tid; i < VB_WAVES * words; i += VB_THREADS) lds[i] = 0u;
   __syncthreads();
-#pragma unroll 4
-  for (uint32_t i = lane; i < n; i += HC_WAVE) atomicAdd(&cur[mine[i].x], 1u);
-  __syncthreads();
-  // exclusive scan of the counts: the segment starts of this bucket's sources, i.e. its stretch of ptrT
-  uint32_t carry = 0u;
-  for (int k0 = 0; k0 < n_local; k0 += HC_WAVE) {
-    const int k = k0 + lane;
-    const uint32_t v = k < n_local ? cur[k] : 0u;
-    const uint32_t incl = vs_wave_incl_scan(v, lane);
-    const uint32_t excl = carry + incl - v;
-    const int64_t id = b * n_local + k;
-    if (k < n_local) {
-      cur[k] = excl;
-      if (id <= S.n_src) ptrT[id] = (int64_t)p0 + excl;
-    }
-    carry += (uint32_t)__builtin_amdgcn_readlane((int)incl, HC_WAVE - 1);
+#pragma unroll
+  for (int j = 0; j < VB_ITERS; ++j) {
+    const uint32_t i = (uint32_t)j * HC_WAVE + lane;
+    if (i < q_len) atomicAdd(&my[vb_swz16w(pr[j].x >> 1)], 1u << ((pr[j].x & 1u) * 16u));
   }
   __syncthreads();
-  // the pairs in order, four loads of 64 in flight: position = segment cursor + rank among equal ids
+  if (S.dbg == 1) { if (lds[lane] == 0xfffffff0u) rowT[0] = 1; return; }
+  // Counts -> cursors: local id k's segment starts at the exclusive sum over the ids below it (that is
+  // this bucket's stretch of ptrT), wave w's pairs of k follow those of the waves before it.
+  {
+    const uint32_t per = words >= (uint32_t)VB_THREADS ? words / VB_THREADS : 1u;   // words per thread
+    const uint32_t w0 = (uint32_t)tid * per;
+    uint32_t sum = 0u;
+    if (w0 < words)
+      for (uint32_t wd = w0; wd < w0 + per; ++wd) {
+        const uint32_t at = vb_swz16w(wd);
+#pragma unroll
+        for (int w = 0; w < VB_WAVES; ++w) {
+          const uint32_t v = lds[(uint32_t)w * words + at];
+          sum += (v & 0xffffu) + (v >> 16);
+        }
+      }
+    const uint32_t incl = vs_wave_incl_scan(sum, lane);
+    if (lane == HC_WAVE - 1) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t run = incl - sum;
+    for (int w = 0; w < wave; ++w) run += s_wave[w];
+    if (w0 < words)
+      for (uint32_t wd = w0; wd < w0 + per; ++wd) {
+        const uint32_t at = vb_swz16w(wd);
+        uint32_t v[VB_WAVES];
+#pragma unroll
+        for (int w = 0; w < VB_WAVES; ++w) v[w] = lds[(uint32_t)w * words + at];
+        uint32_t lo = run;                                 // cursors of the even id, wave by wave
+#pragma unroll
+        for (int w = 0; w < VB_WAVES; ++w) {
+          const uint32_t c = v[w] & 0xffffu;
+          v[w] = (v[w] & 0xffff0000u) | lo;
+          lo += c;
+        }
+        uint32_t hi = lo;                                  // then the odd id's
+#pragma unroll
+        for (int w = 0; w < VB_WAVES; ++w) {
+          const uint32_t c = v[w] >> 16;
+          v[w] = (v[w] & 0xffffu) | (hi << 16);
+          hi += c;
+        }
+        run = hi;
+#pragma unroll
+        for (int w = 0; w < VB_WAVES; ++w) lds[(uint32_t)w * words + at] = v[w];
+      }
+  }
+  __syncthreads();
+  for (uint32_t k = tid; k < n_local; k += VB_THREADS) {
+    const int64_t id = b * (int64_t)n_local + k;
+    const uint32_t v = lds[vb_swz16w(k >> 1)];            // wave 0's cursor = the segment's start
+    if (id <= S.n_src) ptrT[id] = (int64_t)p0 + ((v >> ((k & 1u) * 16u)) & 0xffffu);
+  }
+  __syncthreads();
+  if (S.dbg == 2) return;
+  // every wave ranks the pairs of its quarter in order, 64 at a time
+  const unsigned long long below = (1ull << lane) - 1ull;
+#pragma unroll
+  for (int j = 0; j < VB_ITERS; ++j) {
+    if ((uint32_t)j * HC_WAVE >= q_len) break;            // wave-uniform
+    const uint32_t i = (uint32_t)j * HC_WAVE + lane;
+    const bool live = i < q_len;
+    const uint32_t k = pr[j].x;
+    uint32_t before = 0u, same = 0u;
+    if (live) {
+      uint32_t *c = &my[vb_swz16w(k >> 1)];
+      const uint32_t sh = (k & 1u) * 16u;
+      const uint32_t v0 = *c;
+      atomicAdd(c, 1u << sh);
+      const uint32_t v1 = *c;
+      before = (v0 >> sh) & 0xffffu;
+      same = ((v1 >> sh) & 0xffffu) - before;
+    }
+    const uint32_t pos = before + vs_rank_among_equal(k, live, same, below);
+    if (live) stage[pos] = pr[j].y;
+  }
+  __syncthreads();
+  for (uint32_t i = tid; i < n; i += VB_THREADS) {
+    const uint32_t v = stage[i];
+    if (WANT_EDGES) {
+      edgeT[p0 + i] = (int32_t)v;
+      rowT[p0 + i] = (int32_t)rows[v];
+    } else {
+      rowT[p0 + i] = (int32_t)v;
+    }
+  }
+}
+
+// Buckets above VB_STAGED pairs (hub sources): 32-bit cursors, the pairs are read twice and the
+// results stored as they come.  LDS: cur[VB_WAVES][n_local].
+template <bool WANT_EDGES>
+__device__ __forceinline__ void vb_large(const uint2 *__restrict__ mine, uint32_t n, uint32_t p0, int64_t b,
+                                         uint32_t *__restrict__ cur, uint32_t *__restrict__ s_wave,
+                                         const uint32_t *__restrict__ rows, int64_t *__restrict__ ptrT,
+                                         int32_t *__restrict__ rowT, int32_t *__restrict__ edgeT, const VsShape &S) {
+  const int tid = (int)threadIdx.x;
+  const int lane = hc_lane();
+  const int wave = tid >> 6;
+  const uint32_t n_local = 1u << S.lb;
+  const uint32_t quarter = ((n + VB_WAVES - 1) / VB_WAVES + HC_WAVE - 1) / HC_WAVE * HC_WAVE;
+  const uint32_t q_begin = (uint32_t)wave * quarter < n ? (uint32_t)wave * quarter : n;
+  const uint32_t q_end = q_begin + quarter < n ? q_begin + quarter : n;
+  uint32_t *my = cur + (uint32_t)wave * n_local;
+  for (uint32_t i = tid; i < VB_WAVES * n_local; i += VB_THREADS) cur[i] = 0u;
+  __syncthreads();
+#pragma unroll 4
+  for (uint32_t i = q_begin + lane; i < q_end; i += HC_WAVE) atomicAdd(&my[vb_swz32(mine[i].x)], 1u);
+  __syncthreads();
+  {
+    const uint32_t per = n_local >= (uint32_t)VB_THREADS ? n_local / VB_THREADS : 1u;   // ids per thread
+    const uint32_t k0 = (uint32_t)tid * per;
+    uint32_t sum = 0u;
+    if (k0 < n_local)
+      for (uint32_t k = k0; k < k0 + per; ++k) {
+        const uint32_t at = vb_swz32(k);
+        sum += cur[at] + cur[n_local + at] + cur[2 * n_local + at] + cur[3 * n_local + at];
+      }
+    const uint32_t incl = vs_wave_incl_scan(sum, lane);
+    if (lane == HC_WAVE - 1) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t run = incl - sum;
+    for (int w = 0; w < wave; ++w) run += s_wave[w];
+    if (k0 < n_local)
+      for (uint32_t k = k0; k < k0 + per; ++k) {
+        const uint32_t at = vb_swz32(k);
+        const uint32_t c0 = cur[at], c1 = cur[n_local + at], c2 = cur[2 * n_local + at], c3 = cur[3 * n_local + at];
+        cur[at] = run;
+        cur[n_local + at] = run + c0;
+        cur[2 * n_local + at] = run + c0 + c1;
+        cur[3 * n_local + at] = run + c0 + c1 + c2;
+        run += c0 + c1 + c2 + c3;
+      }
+  }
+  __syncthreads();
+  for (uint32_t k = tid; k < n_local; k += VB_THREADS) {
+    const int64_t id = b * (int64_t)n_local + k;
+    if (id <= S.n_src) ptrT[id] = (int64_t)p0 + cur[vb_swz32(k)];    // wave 0's cursor = the segment's start
+  }
+  __syncthreads();
   const unsigned long long below = (1ull << lane) - 1ull;
   constexpr int DEPTH = 4;
-  for (uint32_t i0 = 0; i0 < n; i0 += DEPTH * HC_WAVE) {
+  for (uint32_t i0 = q_begin; i0 < q_end; i0 += DEPTH * HC_WAVE) {
     uint2 pr[DEPTH];
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       const uint32_t i = i0 + d * HC_WAVE + lane;
-      pr[d] = i < n ? mine[i] : make_uint2(0u, 0u);
+      pr[d] = i < q_end ? mine[i] : make_uint2(0u, 0u);
     }
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       const uint32_t i = i0 + d * HC_WAVE + lane;
-      const bool live = i < n;
-      const unsigned long long all = __ballot(live);
-      if (all == 0ull) break;                                       // wave-uniform
+      const bool live = i < q_end;
       const uint32_t k = pr[d].x;
-      const uint32_t k_first = (uint32_t)__builtin_amdgcn_readfirstlane((int)k);   // lane 0 is live
-      const bool uniform = __ballot(live && k != k_first) == 0ull;  // a hub's stretch: no matching needed
-      const unsigned long long peers = uniform ? all : vs_match(k, S.lb, all);
-      uint32_t pre = 0u;
-      if (live) pre = cur[k];
-      if (live && (peers >> lane) == 1ull) cur[k] = pre + (uint32_t)__popcll(peers);
-      const uint32_t pos = p0 + pre + (uint32_t)__popcll(peers & below);
+      uint32_t before = 0u, same = 0u;
+      if (live) {
+        uint32_t *c = &my[vb_swz32(k)];
+        before = *c;
+        atomicAdd(c, 1u);
+        same = *c - before;
+      }
+      const uint32_t pos = p0 + before + vs_rank_among_equal(k, live, same, below);
       if (live) {
         if (WANT_EDGES) {
           edgeT[pos] = (int32_t)pr[d].y;
@@ -439,6 +642,21 @@ __global__ __launch_bounds__(HC_WAVE) void vs_bucket(const uint2 *__restrict__ p
   }
 }
 
+template <bool WANT_EDGES>
+__global__ __launch_bounds__(VB_THREADS) void vs_bucket(const uint2 *__restrict__ pairs,
+                                                         const uint32_t *__restrict__ bucket_off,
+                                                         const uint32_t *__restrict__ rows,
+                                                         int64_t *__restrict__ ptrT, int32_t *__restrict__ rowT,
+                                                         int32_t *__restrict__ edgeT, VsShape S) {
+  extern __shared__ uint32_t vb_lds[];
+  __shared__ uint32_t s_wave[VB_WAVES];
+  const int64_t b = blockIdx.x;
+  const uint32_t p0 = bucket_off[b];
+  const uint32_t n = bucket_off[b + 1] - p0;               // block-uniform
+  if (n <= VB_STAGED) vb_small<WANT_EDGES>(pairs + p0, n, p0, b, vb_lds, s_wave, rows, ptrT, rowT, edgeT, S);
+  else vb_large<WANT_EDGES>(pairs + p0, n, p0, b, vb_lds, s_wave, rows, ptrT, rowT, edgeT, S);
+}
+
 struct VsLayout {
   size_t key32, tile_count, group_count, bucket_total, bucket_off, pairs, rows, bits, total;
 };
@@ -448,7 +666,10 @@ bool vs_shape(int64_t R, int64_t E, int64_t n_src, VsShape *S) {
   const int64_t ids = n_src + 1;
   int tb = 0;
   while (((int64_t)1 << tb) < ids) ++tb;
-  int lb = tb > 12 ? tb - 12 : 0;
+  // between 1024 and 2048 buckets where the ids allow it (enough blocks for vs_bucket, few enough counters
+  // per tile in vs_scatter); at most 12 local bits unless the buckets would be too many
+  int lb = tb > 11 ? tb - 11 : 0;
+  if (lb > 12) lb = 12;
   while (lb <= VS_MAX_LOCAL_BITS && ((ids + ((int64_t)1 << lb) - 1) >> lb) > VS_MAX_BUCKETS) ++lb;
   if (lb > VS_MAX_LOCAL_BITS) return false;
   S->R = R;
@@ -456,14 +677,24 @@ bool vs_shape(int64_t R, int64_t E, int64_t n_src, VsShape *S) {
   S->n_src = n_src;
   S->lb = lb;
   S->nb = (int)((ids + ((int64_t)1 << lb) - 1) >> lb);
-  int bb = 0;
-  while ((1 << bb) < S->nb) ++bb;
-  S->bbits = bb;
   S->nbp = (S->nb + 63) / 64 * 64;
   S->nbc = (S->nb + 1) / 2 * 2;
   S->ntiles = (E + VS_TILE - 1) / VS_TILE;
   S->ngroups = (S->ntiles + VS_GROUP - 1) / VS_GROUP;
+  const char *d = getenv("HISCACHE_VS_DBG");
+  S->dbg = d ? atoi(d) : 0;
   return true;
+}
+
+// Dynamic LDS of vs_scatter and vs_bucket.
+size_t vs_scatter_lds(const VsShape &S) {
+  return (size_t)S.nbc * sizeof(uint32_t) + (size_t)VS_WAVES * S.nbc * sizeof(uint16_t);
+}
+size_t vs_bucket_lds(const VsShape &S) {
+  const size_t n_local = (size_t)1 << S.lb;
+  const size_t small = VB_WAVES * ((n_local + 1) / 2) * sizeof(uint32_t) + (size_t)VB_STAGED * sizeof(uint32_t);
+  const size_t large = VB_WAVES * n_local * sizeof(uint32_t);
+  return small > large ? small : large;
 }
 
 VsLayout vs_layout(const VsShape &S) {
@@ -486,6 +717,22 @@ VsLayout vs_layout(const VsShape &S) {
   return L;
 }
 
+// A launch with more dynamic LDS than the default limit (64 KB) has to be allowed once per kernel; the
+// compute unit has 160 KB.  The largest size allowed so far is remembered per kernel (a benign race: two
+// threads may both ask).
+template <typename K>
+bool vs_allow_lds(K kernel, size_t bytes) {
+  static size_t allowed = 60 * 1024;
+  if (bytes <= allowed) return true;
+  if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          (int)bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  allowed = bytes;
+  return true;
+}
+
 }  // namespace
 
 bool vs_supported(int64_t E, int64_t n_src) {
@@ -500,8 +747,8 @@ size_t vs_workspace_bytes(int64_t E, int64_t n_src) {
 }
 
 int vs_launch(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row, const int64_t *hmap_src,
-              int64_t R, int64_t E, int64_t n_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT, char *ws,
-              size_t ws_bytes, hipStream_t st) {
+              const uint8_t *edge_drop, int64_t R, int64_t E, int64_t n_src, int64_t *ptrT, int32_t *rowT,
+              int32_t *edgeT, char *ws, size_t ws_bytes, hipStream_t st) {
   VsShape S;
   if (!vs_shape(R, E, n_src, &S)) return HC_EUNSUPPORTED;
   const VsLayout L = vs_layout(S);
@@ -522,26 +769,32 @@ int vs_launch(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row, c
     if (blocks > 0) vs_src_bits<<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(hmap_src, n_src, bits);
     src_bits = reinterpret_cast<const uint32_t *>(bits);
   }
+  const size_t lds = vs_scatter_lds(S), blds = vs_bucket_lds(S);
+  const bool lds_ok = edgeT != nullptr
+                          ? vs_allow_lds(&vs_scatter<false>, lds) && vs_allow_lds(&vs_bucket<true>, blds)
+                          : vs_allow_lds(&vs_scatter<true>, lds) && vs_allow_lds(&vs_bucket<false>, blds);
+  if (!lds_ok) return HC_ELAUNCH;
   const dim3 tgrid((unsigned)S.ntiles);
   if (hmap_row != nullptr)
-    vs_count<true><<<tgrid, dim3(VS_THREADS), 0, st>>>(ptr, idx, hmap_row, src_bits, key32, tile_count, S);
+    vs_count<true><<<tgrid, dim3(VS_THREADS), 0, st>>>(ptr, idx, hmap_row, src_bits, edge_drop, key32, tile_count, S);
   else
-    vs_count<false><<<tgrid, dim3(VS_THREADS), 0, st>>>(ptr, idx, hmap_row, src_bits, key32, tile_count, S);
+    vs_count<false><<<tgrid, dim3(VS_THREADS), 0, st>>>(ptr, idx, hmap_row, src_bits, edge_drop, key32, tile_count,
+                                                       S);
   vs_group_sum<<<dim3((unsigned)((S.nb + HC_BLOCK - 1) / HC_BLOCK), (unsigned)S.ngroups), dim3(HC_BLOCK), 0, st>>>(
       tile_count, group_count, S);
   vs_bucket_scan<<<dim3((unsigned)((S.nb + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK)), dim3(HC_BLOCK), 0, st>>>(
       group_count, bucket_total, S);
   vs_bucket_offsets<<<dim3(1), dim3(VS_OFF_THREADS), 0, st>>>(bucket_total, bucket_off, S);
-  const size_t lds = (size_t)S.nbc * sizeof(uint32_t) + (size_t)VS_WAVES * S.nbc * sizeof(uint16_t);
-  const size_t blds = ((size_t)1 << S.lb) * sizeof(uint32_t);
   if (edgeT != nullptr) {
     vs_scatter<false><<<tgrid, dim3(VS_THREADS), lds, st>>>(ptr, key32, tile_count, group_count, bucket_off, pairs,
                                                            rows, S);
-    vs_bucket<true><<<dim3((unsigned)S.nb), dim3(HC_WAVE), blds, st>>>(pairs, bucket_off, rows, ptrT, rowT, edgeT, S);
+    vs_bucket<true><<<dim3((unsigned)S.nb), dim3(VB_THREADS), blds, st>>>(pairs, bucket_off, rows, ptrT, rowT, edgeT,
+                                                                        S);
   } else {
     vs_scatter<true><<<tgrid, dim3(VS_THREADS), lds, st>>>(ptr, key32, tile_count, group_count, bucket_off, pairs,
                                                           rows, S);
-    vs_bucket<false><<<dim3((unsigned)S.nb), dim3(HC_WAVE), blds, st>>>(pairs, bucket_off, rows, ptrT, rowT, edgeT, S);
+    vs_bucket<false><<<dim3((unsigned)S.nb), dim3(VB_THREADS), blds, st>>>(pairs, bucket_off, rows, ptrT, rowT, edgeT,
+                                                                         S);
   }
   return hc_launch_status();
 }

@@ -108,10 +108,40 @@ def test_aggregation_and_admission_replay_like_eager(be):
         assert torch.equal(eager[4], eager[14])        # the history rows' gradient does not depend on the view
 
 
-def test_large_transposed_build_is_refused_on_a_capturing_stream(be):
-    """Above 2^20 edge slots the sort library would record memset nodes: the call returns an error on a
-    capturing stream, records nothing, and works again once the capture is over."""
+def test_large_transposed_build_is_captured_and_replayed(be):
+    """Above 2^20 edge slots the view comes from the library's own bucket sort, which is kernels only: the
+    call is recorded, and every replay (fresh edges between the replays) gives the eager result."""
     R, N, deg = 300_000, 50_000, 4
+    E = R * deg
+    assert E > 1 << 20
+    gen = torch.Generator(device=DEV).manual_seed(7)
+    ptr = torch.arange(R + 1, device=DEV, dtype=torch.int64) * deg
+    idx = torch.randint(0, N, (E,), device=DEV, generator=gen)
+    hsrc = torch.where(torch.rand(N, device=DEV, generator=gen) < 0.3, 1, -1).to(torch.int64)
+    be.build_transpose(ptr, idx, None, R, N, want_edges=False, history_map_src=hsrc)   # sizes the workspace pool
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            got = be.build_transpose(ptr, idx, None, R, N, want_edges=False, history_map_src=hsrc)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        idx.copy_(torch.randint(0, N, (E,), device=DEV, generator=gen))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = be.build_transpose(ptr, idx, None, R, N, want_edges=False, history_map_src=hsrc)
+        n_tr = int(eager[0][-1])
+        assert torch.equal(got[0], eager[0]), rep
+        assert torch.equal(got[1][:n_tr], eager[1][:n_tr]), rep
+
+
+def test_transposed_build_beyond_the_bucket_sort_is_refused_on_a_capturing_stream(be):
+    """More sources than the bucket sort takes (about 44 M) with more than 2^20 edge slots: the sort library
+    underneath would record memset nodes, so the call returns an error on a capturing stream, records nothing,
+    and works again once the capture is over."""
+    R, N, deg = 300_000, 46_000_000, 4
     E = R * deg
     assert E > 1 << 20
     gen = torch.Generator(device=DEV).manual_seed(7)
