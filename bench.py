@@ -232,8 +232,6 @@ def run_c2(args, row_mode=False):
                            torch.arange(N, device=dev), torch.full((N,), -1, device=dev))
     feat.requires_grad_(True)
     clk_f, clk_t, clk_b = KernelClock(), KernelClock(), KernelClock()
-    # per edge slot: did the forward read the table (what the autograd Function keeps for its backward)
-    edge_sub = None if row_mode else torch.empty(E, dtype=torch.uint8, device=dev)
 
     def step():
         # the same three launches the autograd Function issues, with a clock on each
@@ -242,11 +240,10 @@ def run_c2(args, row_mode=False):
             tr = clk_t(lambda: be.build_transpose(ptr, idx, hmap, R, N, want_edges=False))
             clk_b(lambda: be._aggr_bwd(ptr, idx, tr, g, hmap, None, feat, False, tuple(hbuf.shape), F, R, N))
         else:
-            out = clk_f(lambda: be._aggr_fwd(be.SUBST_SRC, ptr, idx, feat.detach(), hmap, hist, F, None, R,
-                                             edge_sub=edge_sub))
+            out = clk_f(lambda: be._aggr_fwd(be.SUBST_SRC, ptr, idx, feat.detach(), hmap, hist, F, None, R))
             # sources that were substituted by a table row get a zero gradient row (their feature row was
             # not read): their edges are left out of the view, as the autograd Function does
-            tr = clk_t(lambda: be.build_transpose(ptr, idx, None, R, N, want_edges=False, edge_drop=edge_sub))
+            tr = clk_t(lambda: be.build_transpose(ptr, idx, None, R, N, want_edges=False, history_map_src=hmap))
             clk_b(lambda: be._aggr_bwd(ptr, idx, tr, g, None, None, feat, False, None, 0, R, N))
         return out
 

@@ -77,7 +77,6 @@ struct FwdSrc {
   const void *htab;
   int64_t hsize;
   const uint32_t *bits;
-  uint8_t *edge_sub;      // nullable: edge_sub[e] = 1 when edge slot e read a table row, else 0
 };
 template <typename T, typename TH, int VEC, int CHUNKS, int UNROLL, bool STREAM, int WMODE>
 __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, const T *__restrict__ vin,
@@ -100,15 +99,10 @@ __device__ __forceinline__ void fwd_accumulate(const int64_t *__restrict__ idx, 
       my_addr = reinterpret_cast<int64_t>(vin + id * F);
       if (src.hmap != nullptr) {
         const bool maybe = src.bits == nullptr || ((src.bits[id >> 5] >> (id & 31)) & 1u) != 0u;
-        bool sub = false;
         if (maybe) {
           const int64_t slot = src.hmap[id];
-          if (slot != -1) {
-            my_addr = reinterpret_cast<int64_t>(htab + slot * src.hsize) | (MIXED ? 1 : 0);
-            sub = true;
-          }
+          if (slot != -1) my_addr = reinterpret_cast<int64_t>(htab + slot * src.hsize) | (MIXED ? 1 : 0);
         }
-        if (src.edge_sub != nullptr) src.edge_sub[base + lane] = sub ? 1 : 0;
       }
       if constexpr (WMODE == W_EDGE) my_w = ev[base + lane];
     }
@@ -296,9 +290,8 @@ template <typename T, typename TH, int VEC, int CHUNKS, int UNROLL, bool STREAM,
 __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const T *__restrict__ vin,
     const int64_t *__restrict__ hmap, const void *__restrict__ hbuf, int hist_dtype, int64_t hsize,
-    int src_mode, const uint32_t *__restrict__ src_bits, uint8_t *__restrict__ edge_sub,
-    const float *__restrict__ ev, int n_head, float *__restrict__ vout, int64_t R, int64_t long_thres,
-    FwdSched sched) {
+    int src_mode, const uint32_t *__restrict__ src_bits, const float *__restrict__ ev, int n_head,
+    float *__restrict__ vout, int64_t R, int64_t long_thres, FwdSched sched) {
   constexpr int F = HC_WAVE * VEC * CHUNKS;
   constexpr bool WEIGHTED = WMODE != W_NONE;
   // without heads the rows may be split: the split code is compiled for those modes only
@@ -308,7 +301,7 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_mean_fast(
   __shared__ int n_long_s;
   const int lane = hc_lane();
   const int wave = hc_wave_in_block();
-  const FwdSrc src{src_mode ? hmap : nullptr, hbuf, hsize, src_bits, edge_sub};
+  const FwdSrc src{src_mode ? hmap : nullptr, hbuf, hsize, src_bits};
   // every thread of the grid reads the same two words, so the decision is uniform
   const int n_listed = sched.head != nullptr ? sched.head->count : 0;
   const bool listed = sched.head != nullptr && n_listed <= sched.head->cap;
@@ -389,8 +382,8 @@ template <typename T, bool WEIGHTED>
 __global__ __launch_bounds__(HC_BLOCK) void fwd_generic(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const T *__restrict__ vin,
     const int64_t *__restrict__ hmap, const void *__restrict__ hbuf, int hist_dtype, int64_t hsize,
-    int src_mode, uint8_t *__restrict__ edge_sub, const float *__restrict__ ev, int64_t H,
-    float *__restrict__ vout, int64_t R, int64_t F) {
+    int src_mode, const float *__restrict__ ev, int64_t H, float *__restrict__ vout, int64_t R,
+    int64_t F) {
   constexpr int TILE_K = 4;
   const int lane = hc_lane();
   const int64_t vrow = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
@@ -433,7 +426,6 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_generic(
             my_addr = reinterpret_cast<int64_t>(static_cast<const char *>(hbuf) + slot * hsize * hesz);
             my_hist = same_type ? 0 : 1;
           }
-          if (edge_sub != nullptr && c0 == 0) edge_sub[base + lane] = slot != -1 ? 1 : 0;
         }
         if (WEIGHTED) my_w = ev[(base + lane) * H + head];
       }
@@ -527,8 +519,8 @@ __global__ __launch_bounds__(HC_BLOCK) void fwd_src_bits(const int64_t *__restri
 
 template <typename T, int VEC, int CHUNKS>
 int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const int64_t *hmap,
-                const void *hbuf, int hist_dtype, int64_t hsize, int src_mode, uint8_t *edge_sub, const float *ev,
-                int n_head, float *vout, int64_t R, int64_t n_src, FwdScratch ws, hipStream_t st) {
+                const void *hbuf, int hist_dtype, int64_t hsize, int src_mode, const float *ev, int n_head,
+                float *vout, int64_t R, int64_t n_src, FwdScratch ws, hipStream_t st) {
   constexpr int per = VEC * CHUNKS;
   constexpr int UNROLL = per >= 16 ? 4 : (per >= 4 ? 8 : 16);
   int64_t blocks = (R + FWD_ROWS_PER_BLOCK - 1) / FWD_ROWS_PER_BLOCK;
@@ -566,8 +558,8 @@ int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const i
   }
 #define HC_FWD_LAUNCH(TH, STREAM, WMODE)                                                                   \
   fwd_mean_fast<T, TH, VEC, CHUNKS, UNROLL, STREAM, WMODE><<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>( \
-      ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, src_bits, edge_sub, ev, n_head, \
-      vout, R, long_thres, sched)
+      ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype, hsize, src_mode, src_bits, ev, n_head, vout, R, \
+      long_thres, sched)
   if (ev != nullptr && n_head > 1) HC_FWD_LAUNCH(T, false, W_EDGE_HEAD);
   else if (ev != nullptr) HC_FWD_LAUNCH(T, false, W_EDGE);
   else if (src_mode && hmap != nullptr) {
@@ -584,14 +576,14 @@ int launch_fast(const int64_t *ptr, const int64_t *idx, const void *vin, const i
 template <typename T>
 int dispatch_fast(int64_t F, const int64_t *ptr, const int64_t *idx, const void *vin,
                   const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize, int src_mode,
-                  uint8_t *edge_sub, const float *ev, int n_head, float *vout, int64_t R, int64_t n_src,
-                  FwdScratch ws, hipStream_t st, bool *handled) {
+                  const float *ev, int n_head, float *vout, int64_t R, int64_t n_src, FwdScratch ws,
+                  hipStream_t st, bool *handled) {
   // F is the whole row (all heads); with several heads a lane's vector must not straddle two of them
   *handled = true;
 #define HC_FAST(V, C)                                                                              \
   if (F == 64 * (V) * (C) && (F / n_head) % (V) == 0)                                              \
-    return launch_fast<T, V, C>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_sub, ev, n_head, vout, R, \
-                                n_src, ws, st);
+    return launch_fast<T, V, C>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, ev, n_head, vout, R, n_src, \
+                                ws, st);
   constexpr int VMAX = 16 / (int)sizeof(T);
   if constexpr (VMAX == 8) {
     HC_FAST(8, 1) HC_FAST(8, 2) HC_FAST(8, 3) HC_FAST(8, 4)
@@ -607,17 +599,17 @@ int dispatch_fast(int64_t F, const int64_t *ptr, const int64_t *idx, const void 
 
 template <typename T>
 int launch_generic(const int64_t *ptr, const int64_t *idx, const void *vin, const int64_t *hmap,
-                   const void *hbuf, int hist_dtype, int64_t hsize, int src_mode, uint8_t *edge_sub,
-                   const float *ev, int64_t H, float *vout, int64_t R, int64_t F, hipStream_t st) {
+                   const void *hbuf, int hist_dtype, int64_t hsize, int src_mode, const float *ev,
+                   int64_t H, float *vout, int64_t R, int64_t F, hipStream_t st) {
   const int64_t blocks = (R * H + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
   if (!hc_grid_ok(blocks)) return HC_EUNSUPPORTED;
   dim3 g((unsigned)blocks), b(HC_BLOCK);
   if (ev)
     fwd_generic<T, true><<<g, b, 0, st>>>(ptr, idx, static_cast<const T *>(vin), hmap, hbuf, hist_dtype,
-                                          hsize, src_mode, edge_sub, ev, H, vout, R, F);
+                                          hsize, src_mode, ev, H, vout, R, F);
   else
     fwd_generic<T, false><<<g, b, 0, st>>>(ptr, idx, static_cast<const T *>(vin), hmap, hbuf,
-                                           hist_dtype, hsize, src_mode, edge_sub, ev, H, vout, R, F);
+                                           hist_dtype, hsize, src_mode, ev, H, vout, R, F);
   return hc_launch_status();
 }
 
@@ -647,11 +639,11 @@ extern "C" size_t hc_aggr_fwd_workspace_bytes(int mode, int64_t R, int64_t E, in
   return fwd_ws_layout(mode, R, E, n_src).total;
 }
 
-namespace {
-int aggr_fwd_impl(int mode, const int64_t *ptr, const int64_t *idx, const void *vin, int in_dtype,
-                  const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize, const float *edge_value,
-                  int64_t n_head, float *vout, uint8_t *edge_sub, int64_t R, int64_t F, int64_t n_src,
-                  void *workspace, size_t workspace_bytes, void *stream) {
+extern "C" int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, const void *vin,
+                           int in_dtype, const int64_t *hmap, const void *hbuf, int hist_dtype,
+                           int64_t hsize, const float *edge_value, int64_t n_head, float *vout,
+                           int64_t R, int64_t F, int64_t n_src, void *workspace,
+                           size_t workspace_bytes, void *stream) {
   const FwdScratch ws{workspace, workspace ? workspace_bytes : 0};
   HC_REQUIRE(R >= 0 && F > 0 && n_src >= 0 && n_head >= 1);
   if (R == 0) return HC_OK;
@@ -688,41 +680,22 @@ int aggr_fwd_impl(int mode, const int64_t *ptr, const int64_t *idx, const void *
     int rc;
     const int nh = (int)n_head;
     if (in_dtype == HC_F32)
-      rc = dispatch_fast<float>(Frow, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_sub, edge_value, nh, vout,
-                                R, n_src, ws, st, &handled);
+      rc = dispatch_fast<float>(Frow, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value, nh, vout, R,
+                                n_src, ws, st, &handled);
     else if (in_dtype == HC_F16)
-      rc = dispatch_fast<__half>(Frow, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_sub, edge_value, nh,
-                                 vout, R, n_src, ws, st, &handled);
+      rc = dispatch_fast<__half>(Frow, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value, nh, vout,
+                                 R, n_src, ws, st, &handled);
     else
       rc = dispatch_fast<__hip_bfloat16>(Frow, ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode,
-                                         edge_sub, edge_value, nh, vout, R, n_src, ws, st, &handled);
+                                         edge_value, nh, vout, R, n_src, ws, st, &handled);
     if (handled) return rc;
   }
   if (in_dtype == HC_F32)
-    return launch_generic<float>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_sub, edge_value,
+    return launch_generic<float>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value,
                                  n_head, vout, R, F, st);
   if (in_dtype == HC_F16)
-    return launch_generic<__half>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_sub, edge_value,
+    return launch_generic<__half>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_value,
                                   n_head, vout, R, F, st);
-  return launch_generic<__hip_bfloat16>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode, edge_sub,
+  return launch_generic<__hip_bfloat16>(ptr, idx, vin, hmap, hbuf, hist_dtype, hsize, src_mode,
                                         edge_value, n_head, vout, R, F, st);
-}
-}  // namespace
-
-extern "C" int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, const void *vin,
-                           int in_dtype, const int64_t *hmap, const void *hbuf, int hist_dtype,
-                           int64_t hsize, const float *edge_value, int64_t n_head, float *vout,
-                           int64_t R, int64_t F, int64_t n_src, void *workspace,
-                           size_t workspace_bytes, void *stream) {
-  return aggr_fwd_impl(mode, ptr, idx, vin, in_dtype, hmap, hbuf, hist_dtype, hsize, edge_value, n_head, vout,
-                       nullptr, R, F, n_src, workspace, workspace_bytes, stream);
-}
-
-extern "C" int hc_aggr_fwd_src_mask(const int64_t *ptr, const int64_t *idx, const void *vin, int in_dtype,
-                                    const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize,
-                                    float *vout, uint8_t *edge_sub, int64_t R, int64_t F, int64_t n_src,
-                                    void *workspace, size_t workspace_bytes, void *stream) {
-  HC_REQUIRE(hmap != nullptr && edge_sub != nullptr);
-  return aggr_fwd_impl(HC_SUBST_SRC, ptr, idx, vin, in_dtype, hmap, hbuf, hist_dtype, hsize, nullptr, 1, vout,
-                       edge_sub, R, F, n_src, workspace, workspace_bytes, stream);
 }

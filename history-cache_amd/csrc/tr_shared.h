@@ -46,8 +46,8 @@ __device__ __forceinline__ int64_t tr_row_of_wave(const int64_t *__restrict__ pt
 bool vs_supported(int64_t E, int64_t n_src);
 // Workspace of the bucket sort (0 when unsupported); 256-byte aligned base expected.
 size_t vs_workspace_bytes(int64_t E, int64_t n_src);
-// Enqueues the bucket sort.  hmap_row / hmap_src / edge_drop are nullable: rows with hmap_row[r] != -1,
-// sources with hmap_src[s] != -1 and edge slots with edge_drop[e] != 0 are left out.  Returns an hc_status.
+// Enqueues the bucket sort.  hmap_row / hmap_src are nullable: rows with hmap_row[r] != -1 and sources with
+// hmap_src[s] != -1 are left out.  Returns an hc_status.
 int vs_launch(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row, const int64_t *hmap_src,
-              const uint8_t *edge_drop, int64_t R, int64_t E, int64_t n_src, int64_t *ptrT, int32_t *rowT,
-              int32_t *edgeT, char *ws, size_t ws_bytes, hipStream_t st);
+              int64_t R, int64_t E, int64_t n_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT, char *ws,
+              size_t ws_bytes, hipStream_t st);

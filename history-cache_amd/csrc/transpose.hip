@@ -43,7 +43,6 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_expand_edges(const int64_t *__res
                                                              const int64_t *__restrict__ hmap_row,
                                                              const int64_t *__restrict__ hmap_src,
                                                              const uint32_t *__restrict__ src_bits,
-                                                             const uint8_t *__restrict__ edge_drop,
                                                              uint32_t *__restrict__ keys,
                                                              uint32_t *__restrict__ vals,
                                                              uint32_t *__restrict__ rows, int64_t R, int64_t E,
@@ -92,13 +91,6 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_expand_edges(const int64_t *__res
     for (int it = 0; it < TR_ITEMS; ++it) h[it] = live[it] ? hmap_row[row[it]] : -1;
 #pragma unroll
     for (int it = 0; it < TR_ITEMS; ++it) live[it] = live[it] && h[it] == -1;
-  }
-  if (edge_drop != nullptr) {  // edge slots the caller has flagged (a forward pass that substituted their sources)
-#pragma unroll
-    for (int it = 0; it < TR_ITEMS; ++it) {
-      const int64_t e = e0 + (int64_t)it * HC_BLOCK + threadIdx.x;
-      if (live[it] && edge_drop[e] != 0) live[it] = false;
-    }
   }
   int64_t src[TR_ITEMS];
 #pragma unroll
@@ -284,9 +276,8 @@ __device__ __forceinline__ int trs_load(const int *p) { return *p; }
 
 __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
     const int64_t *__restrict__ ptr, const int64_t *__restrict__ idx, const int64_t *__restrict__ hmap_row,
-    const int64_t *__restrict__ hmap_src, const uint8_t *__restrict__ edge_drop, uint32_t *__restrict__ keys,
-    int32_t *__restrict__ rows, int *__restrict__ count, TrSmallHeader *__restrict__ header,
-    int64_t *__restrict__ ptrT, TrDims dims) {
+    const int64_t *__restrict__ hmap_src, uint32_t *__restrict__ keys, int32_t *__restrict__ rows,
+    int *__restrict__ count, TrSmallHeader *__restrict__ header, int64_t *__restrict__ ptrT, TrDims dims) {
   __shared__ int64_t s_ptr[TR_LDS_ROWS];
   __shared__ int64_t s_range[2];
   __shared__ int s_wave[TRS_BLOCK / HC_WAVE];
@@ -329,7 +320,6 @@ __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
         live = row < R && ptr[row] <= e;
       }
       if (live && hmap_row != nullptr) live = hmap_row[row] == -1;
-      if (live && edge_drop != nullptr) live = edge_drop[e] == 0;
       int64_t src = live ? idx[e] : -1;
       if (src < 0 || src >= n_src) live = false;
       if (live && hmap_src != nullptr) live = hmap_src[src] == -1;
@@ -603,7 +593,7 @@ inline bool bucket_sorted(int64_t E, int64_t n_src) { return E > TR_BUCKET_SORT_
 // The four launches of the counting sort; dims.E / dims.n_src size the grids (upper bounds when the real
 // sizes are read on the device).
 int small_launch(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row, const int64_t *hmap_src,
-                 const uint8_t *edge_drop, const TrDims &dims, int64_t *ptrT, int32_t *rowT, int32_t *edgeT, char *w, const SmallLayout &S,
+                 const TrDims &dims, int64_t *ptrT, int32_t *rowT, int32_t *edgeT, char *w, const SmallLayout &S,
                  hipStream_t st) {
   TrSmallHeader *header = reinterpret_cast<TrSmallHeader *>(w);
   int *count = reinterpret_cast<int *>(w + S.count);
@@ -617,8 +607,8 @@ int small_launch(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row
   const int64_t pb = (E + HC_BLOCK - 1) / HC_BLOCK, ob = (n_src + TRS_ORDER_SOURCES - 1) / TRS_ORDER_SOURCES;
   if (!hc_grid_ok(cb) || !hc_grid_ok(eb) || !hc_grid_ok(pb) || !hc_grid_ok(ob)) return HC_EUNSUPPORTED;
   tr_small_clear<<<dim3((unsigned)cb), dim3(HC_BLOCK), 0, st>>>(reinterpret_cast<uint32_t *>(w), dims);
-  tr_small_count<<<dim3((unsigned)eb), dim3(TRS_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, edge_drop, keys, rows,
-                                                                 count, header, ptrT, dims);
+  tr_small_count<<<dim3((unsigned)eb), dim3(TRS_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, keys, rows, count,
+                                                                 header, ptrT, dims);
   tr_small_place<<<dim3((unsigned)pb), dim3(HC_BLOCK), 0, st>>>(keys, rows, count, tmp_row, tmp_edge, dims);
   if (n_src > 0)
     tr_small_order<<<dim3((unsigned)ob), dim3(HC_BLOCK), 0, st>>>(ptrT, tmp_row, tmp_edge, rowT, edgeT, dims);
@@ -693,10 +683,10 @@ extern "C" size_t hc_transpose_workspace_bytes(int64_t R, int64_t E, int64_t n_s
   return L.total;
 }
 
-namespace {
-int build_transpose_impl(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row, const int64_t *hmap_src,
-                         const uint8_t *edge_drop, int64_t R, int64_t E, int64_t n_src, int64_t *ptrT,
-                         int32_t *rowT, int32_t *edgeT, void *workspace, size_t workspace_bytes, void *stream) {
+extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row,
+                                  const int64_t *hmap_src, int64_t R, int64_t E, int64_t n_src, int64_t *ptrT,
+                                  int32_t *rowT, int32_t *edgeT, void *workspace, size_t workspace_bytes,
+                                  void *stream) {
   HC_REQUIRE(R >= 0 && E >= 0 && n_src >= 0 && ptrT);
   const int64_t lim = 0x7ffffffeLL;
   if (R > lim || E > lim || n_src > lim) return HC_EUNSUPPORTED;
@@ -714,12 +704,12 @@ int build_transpose_impl(const int64_t *ptr, const int64_t *idx, const int64_t *
     char *w = static_cast<char *>(workspace);
     if (reinterpret_cast<uintptr_t>(w) % 256 != 0) return HC_EWORKSPACE;
     const TrDims dims{R, E, n_src, nullptr, nullptr, nullptr};
-    return small_launch(ptr, idx, hmap_row, hmap_src, edge_drop, dims, ptrT, rowT, edgeT, w, S, st);
+    return small_launch(ptr, idx, hmap_row, hmap_src, dims, ptrT, rowT, edgeT, w, S, st);
   }
   if (bucket_sorted(E, n_src)) {
     char *w = static_cast<char *>(workspace);
     if (!workspace || reinterpret_cast<uintptr_t>(w) % 256 != 0) return HC_EWORKSPACE;
-    return vs_launch(ptr, idx, hmap_row, hmap_src, edge_drop, R, E, n_src, ptrT, rowT, edgeT, w, workspace_bytes, st);
+    return vs_launch(ptr, idx, hmap_row, hmap_src, R, E, n_src, ptrT, rowT, edgeT, w, workspace_bytes, st);
   }
   if (E > TR_SORT_MEMSET_EDGES) {
     // Above this size the sort library takes its one-sweep path, which clears its counters with
@@ -763,9 +753,9 @@ int build_transpose_impl(const int64_t *ptr, const int64_t *idx, const int64_t *
   const dim3 tgrid((unsigned)((E + tile - 1) / tile));
   if (want_edges) {
     if (items == 1)
-      tr_expand_edges<false, 1><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, src_bits, edge_drop, keys0, vals0, rows, R, E, n_src);
+      tr_expand_edges<false, 1><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, src_bits, keys0, vals0, rows, R, E, n_src);
     else
-      tr_expand_edges<false, TR_ITEMS_LARGE><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, src_bits, edge_drop, keys0,
+      tr_expand_edges<false, TR_ITEMS_LARGE><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, src_bits, keys0,
                                                                                vals0, rows, R, E, n_src);
     rocprim::double_buffer<uint32_t> dk(keys0, keys1), dv(vals0, vals1);
     if (rocprim::radix_sort_pairs<TrSortConfig>(temp, temp_bytes, dk, dv, (size_t)E, 0u, bits, st, false) != hipSuccess)
@@ -776,9 +766,9 @@ int build_transpose_impl(const int64_t *ptr, const int64_t *idx, const int64_t *
   } else {
     // value = destination row; dropped edge slots keep the fill value and sort behind the sentinel
     if (items == 1)
-      tr_expand_edges<true, 1><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, src_bits, edge_drop, keys0, vals0, nullptr, R, E, n_src);
+      tr_expand_edges<true, 1><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, src_bits, keys0, vals0, nullptr, R, E, n_src);
     else
-      tr_expand_edges<true, TR_ITEMS_LARGE><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, src_bits, edge_drop, keys0,
+      tr_expand_edges<true, TR_ITEMS_LARGE><<<tgrid, dim3(HC_BLOCK), 0, st>>>(ptr, idx, hmap_row, hmap_src, src_bits, keys0,
                                                                               vals0, nullptr, R, E, n_src);
     // rowT doubles as the sort's second value buffer; copy only if the result landed in the first
     uint32_t *rowT_u = reinterpret_cast<uint32_t *>(rowT);
@@ -796,24 +786,6 @@ int build_transpose_impl(const int64_t *ptr, const int64_t *idx, const int64_t *
     tr_finalize_ptr<<<dim3((unsigned)pblocks), dim3(HC_BLOCK), 0, st>>>(skeys, ptrT, E, n_src);
   }
   return hc_launch_status();
-}
-
-}  // namespace
-
-extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row,
-                                  const int64_t *hmap_src, int64_t R, int64_t E, int64_t n_src, int64_t *ptrT,
-                                  int32_t *rowT, int32_t *edgeT, void *workspace, size_t workspace_bytes,
-                                  void *stream) {
-  return build_transpose_impl(ptr, idx, hmap_row, hmap_src, nullptr, R, E, n_src, ptrT, rowT, edgeT, workspace,
-                              workspace_bytes, stream);
-}
-
-extern "C" int hc_build_transpose_edge_mask(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row,
-                                            const uint8_t *edge_drop, int64_t R, int64_t E, int64_t n_src,
-                                            int64_t *ptrT, int32_t *rowT, int32_t *edgeT, void *workspace,
-                                            size_t workspace_bytes, void *stream) {
-  return build_transpose_impl(ptr, idx, hmap_row, nullptr, edge_drop, R, E, n_src, ptrT, rowT, edgeT, workspace,
-                              workspace_bytes, stream);
 }
 
 // Limits of the variant with device-resident sizes: the counters are 32-bit and one block scans them.
@@ -837,6 +809,5 @@ extern "C" int hc_build_transpose_dev(const int64_t *ptr, const int64_t *idx, co
   char *w = static_cast<char *>(workspace);
   if (reinterpret_cast<uintptr_t>(w) % 256 != 0) return HC_EWORKSPACE;
   const TrDims dims{0, max_E, max_src, R_dev, E_dev, n_src_dev};
-  return small_launch(ptr, idx, nullptr, nullptr, nullptr, dims, ptrT, rowT, edgeT, w, S,
-                      static_cast<hipStream_t>(stream));
+  return small_launch(ptr, idx, nullptr, nullptr, dims, ptrT, rowT, edgeT, w, S, static_cast<hipStream_t>(stream));
 }

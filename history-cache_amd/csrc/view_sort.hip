@@ -26,8 +26,6 @@
 // by the number of memory requests rather than by bytes: the scattered 8-byte stores of vs_scatter
 // are one request per live slot, which is why there are two levels and not three, and why everything
 // else is staged so that its requests are whole lines.
-#include <cstdlib>
-
 #include "tr_shared.h"
 
 namespace {
@@ -100,7 +98,7 @@ __device__ __forceinline__ void vs_rows_setup(VsRowFinder &f, const int64_t *__r
                                               int64_t e0, int64_t a, int64_t b) {
   const int tid = (int)threadIdx.x;
   const int lane = hc_lane();
-  if (tid < 2 * HC_WAVE) {
+  if (tid < 2 * HC_WAVE) {                               // the first and the last row, by two waves side by side
     const int which = tid >> 6;
     const int64_t r = tr_row_of_wave(ptr, R, which == 0 ? a : b - 1, lane);
     if (lane == 0) {
@@ -175,7 +173,6 @@ struct VsShape {
   int nb;          // buckets: ids 0 .. n_src (ptrT has an entry for n_src too)
   int nbp;         // row pitch of the per-tile and per-group count matrices
   int nbc;         // pitch of a wave's 16-bit counters in vs_scatter's LDS (even)
-  int dbg;
 };
 
 template <bool ROWMAP>
@@ -183,7 +180,6 @@ __global__ __launch_bounds__(VS_THREADS) void vs_count(const int64_t *__restrict
                                                         const int64_t *__restrict__ idx,
                                                         const int64_t *__restrict__ hmap_row,
                                                         const uint32_t *__restrict__ src_bits,
-                                                        const uint8_t *__restrict__ edge_drop,
                                                         uint32_t *__restrict__ key32,
                                                         uint16_t *__restrict__ tile_count, VsShape S) {
   __shared__ uint32_t hist[VS_MAX_BUCKETS];
@@ -204,17 +200,6 @@ __global__ __launch_bounds__(VS_THREADS) void vs_count(const int64_t *__restrict
   for (int j = 0; j < VS_ITERS; ++j) {
     const int64_t e = base + (int64_t)j * HC_WAVE;
     src[j] = (e >= a && e < bnd) ? __builtin_nontemporal_load(idx + e) : -1;
-  }
-  if (edge_drop != nullptr) {
-    uint8_t d[VS_ITERS];
-#pragma unroll
-    for (int j = 0; j < VS_ITERS; ++j) {
-      const int64_t e = base + (int64_t)j * HC_WAVE;
-      d[j] = (e >= a && e < bnd) ? __builtin_nontemporal_load(edge_drop + e) : (uint8_t)0;
-    }
-#pragma unroll
-    for (int j = 0; j < VS_ITERS; ++j)
-      if (d[j] != 0) src[j] = -1;
   }
   if (ROWMAP && a < bnd) vs_rows_setup(rf, ptr, S.R, e0, a, bnd);   // block-uniform condition
   else __syncthreads();
@@ -283,12 +268,21 @@ __global__ __launch_bounds__(HC_BLOCK) void vs_bucket_scan(uint32_t *__restrict_
   const int b = (int)(blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block());
   if (b >= S.nb) return;
   uint32_t carry = 0u;
-  for (int64_t g0 = 0; g0 < S.ngroups; g0 += HC_WAVE) {
-    const int64_t g = g0 + lane;
-    const uint32_t v = g < S.ngroups ? group_count[g * S.nbp + b] : 0u;
-    const uint32_t incl = vs_wave_incl_scan(v, lane);
-    if (g < S.ngroups) group_count[g * S.nbp + b] = carry + incl - v;
-    carry += (uint32_t)__builtin_amdgcn_readlane((int)incl, HC_WAVE - 1);
+  constexpr int Q = 4;                                    // rounds of 64 groups whose loads are in flight together
+  for (int64_t g0 = 0; g0 < S.ngroups; g0 += Q * HC_WAVE) {
+    uint32_t v[Q];
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+      const int64_t g = g0 + q * HC_WAVE + lane;
+      v[q] = g < S.ngroups ? group_count[g * S.nbp + b] : 0u;
+    }
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+      const int64_t g = g0 + q * HC_WAVE + lane;
+      const uint32_t incl = vs_wave_incl_scan(v[q], lane);
+      if (g < S.ngroups) group_count[g * S.nbp + b] = carry + incl - v[q];
+      carry += (uint32_t)__builtin_amdgcn_readlane((int)incl, HC_WAVE - 1);
+    }
   }
   if (lane == 0) bucket_total[b] = carry;
 }
@@ -357,7 +351,6 @@ __global__ __launch_bounds__(VS_THREADS) void vs_scatter(const int64_t *__restri
   const int64_t bnd = e1 < last ? e1 : last;
   if (a < bnd) vs_rows_setup(rf, ptr, S.R, e0, a, bnd);   // block-uniform condition
   else __syncthreads();
-  if (S.dbg == 3) { if (key[S.dbg] == 12345u) rows[0] = 1u; return; }
   // Rank of every live slot among the slots of its bucket in this wave's eighth of the tile, in slot
   // order: the bucket's running count in front of these 64 slots plus the rank among them.
   uint32_t *mine32 = cnt32 + wave * (S.nbc / 2);
@@ -379,7 +372,6 @@ __global__ __launch_bounds__(VS_THREADS) void vs_scatter(const int64_t *__restri
     rk[j] = before + vs_rank_among_equal(b, live, same, below);
   }
   __syncthreads();
-  if (S.dbg == 4) { if (rk[S.dbg] == 12345u) rows[0] = 1u; return; }
   // the waves' counts become the eighths' offsets; base = the tile's first position in the bucket
   {
     const int64_t g = tile / VS_GROUP;
@@ -410,7 +402,6 @@ __global__ __launch_bounds__(VS_THREADS) void vs_scatter(const int64_t *__restri
     }
   }
   __syncthreads();
-  if (S.dbg == 5) { if (rk[S.dbg] == 12345u) rows[0] = 1u; return; }
   const uint16_t *mine = cnt + wave * S.nbc;
   const uint32_t local_mask = (1u << S.lb) - 1u;
 #pragma unroll
@@ -470,7 +461,6 @@ __device__ __forceinline__ void vb_small(const uint2 *__restrict__ mine, uint32_
     if (i < q_len) atomicAdd(&my[vb_swz16w(pr[j].x >> 1)], 1u << ((pr[j].x & 1u) * 16u));
   }
   __syncthreads();
-  if (S.dbg == 1) { if (lds[lane] == 0xfffffff0u) rowT[0] = 1; return; }
   // Counts -> cursors: local id k's segment starts at the exclusive sum over the ids below it (that is
   // this bucket's stretch of ptrT), wave w's pairs of k follow those of the waves before it.
   {
@@ -523,7 +513,6 @@ __device__ __forceinline__ void vb_small(const uint2 *__restrict__ mine, uint32_
     if (id <= S.n_src) ptrT[id] = (int64_t)p0 + ((v >> ((k & 1u) * 16u)) & 0xffffu);
   }
   __syncthreads();
-  if (S.dbg == 2) return;
   // every wave ranks the pairs of its quarter in order, 64 at a time
   const unsigned long long below = (1ull << lane) - 1ull;
 #pragma unroll
@@ -681,8 +670,6 @@ bool vs_shape(int64_t R, int64_t E, int64_t n_src, VsShape *S) {
   S->nbc = (S->nb + 1) / 2 * 2;
   S->ntiles = (E + VS_TILE - 1) / VS_TILE;
   S->ngroups = (S->ntiles + VS_GROUP - 1) / VS_GROUP;
-  const char *d = getenv("HISCACHE_VS_DBG");
-  S->dbg = d ? atoi(d) : 0;
   return true;
 }
 
@@ -747,8 +734,8 @@ size_t vs_workspace_bytes(int64_t E, int64_t n_src) {
 }
 
 int vs_launch(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row, const int64_t *hmap_src,
-              const uint8_t *edge_drop, int64_t R, int64_t E, int64_t n_src, int64_t *ptrT, int32_t *rowT,
-              int32_t *edgeT, char *ws, size_t ws_bytes, hipStream_t st) {
+              int64_t R, int64_t E, int64_t n_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT, char *ws,
+              size_t ws_bytes, hipStream_t st) {
   VsShape S;
   if (!vs_shape(R, E, n_src, &S)) return HC_EUNSUPPORTED;
   const VsLayout L = vs_layout(S);
@@ -776,10 +763,9 @@ int vs_launch(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row, c
   if (!lds_ok) return HC_ELAUNCH;
   const dim3 tgrid((unsigned)S.ntiles);
   if (hmap_row != nullptr)
-    vs_count<true><<<tgrid, dim3(VS_THREADS), 0, st>>>(ptr, idx, hmap_row, src_bits, edge_drop, key32, tile_count, S);
+    vs_count<true><<<tgrid, dim3(VS_THREADS), 0, st>>>(ptr, idx, hmap_row, src_bits, key32, tile_count, S);
   else
-    vs_count<false><<<tgrid, dim3(VS_THREADS), 0, st>>>(ptr, idx, hmap_row, src_bits, edge_drop, key32, tile_count,
-                                                       S);
+    vs_count<false><<<tgrid, dim3(VS_THREADS), 0, st>>>(ptr, idx, hmap_row, src_bits, key32, tile_count, S);
   vs_group_sum<<<dim3((unsigned)((S.nb + HC_BLOCK - 1) / HC_BLOCK), (unsigned)S.ngroups), dim3(HC_BLOCK), 0, st>>>(
       tile_count, group_count, S);
   vs_bucket_scan<<<dim3((unsigned)((S.nb + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK)), dim3(HC_BLOCK), 0, st>>>(

@@ -51,14 +51,10 @@ _SIGNATURES = {
     "hc_aggr_fwd_workspace_bytes": (_c_sz, [_c_int, _c_i64, _c_i64, _c_i64]),
     "hc_aggr_fwd": (_c_int, [_c_int, _c_p, _c_p, _c_p, _c_int, _c_p, _c_p, _c_int, _c_i64, _c_p, _c_i64,
                              _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]),
-    "hc_aggr_fwd_src_mask": (_c_int, [_c_p, _c_p, _c_p, _c_int, _c_p, _c_p, _c_int, _c_i64, _c_p, _c_p, _c_i64, _c_i64,
-                                      _c_i64, _c_p, _c_sz, _c_p]),
     "hc_aggr_fwd_long_row_edges": (_c_i64, [_c_i64, _c_int]),
     "hc_transpose_workspace_bytes": (_c_sz, [_c_i64, _c_i64, _c_i64]),
     "hc_build_transpose": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p,
                                     _c_sz, _c_p]),
-    "hc_build_transpose_edge_mask": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p,
-                                              _c_sz, _c_p]),
     "hc_transpose_dev_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
     "hc_build_transpose_dev": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_sz,
                                         _c_p]),
@@ -243,9 +239,7 @@ def check_csr(ptr, idx, num_node, n_src):
 
 
 # ----------------------------------------------------------------------------- raw launchers
-def _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, num_node, edge_sub=None):
-    """``edge_sub`` (per-source substitution only; uint8, one entry per edge slot of the first ``num_node`` rows):
-    the launch also notes, per edge slot, whether it read a row of the table (1) or of ``x`` (0)."""
+def _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, num_node):
     lib = load_library()
     _dev(ptr, "ptr", torch.int64)
     _dev(idx, "idx", torch.int64)
@@ -279,15 +273,6 @@ def _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, num_node, edge_s
     # scratch for the long-row list (large blocks only: the library reports 0 bytes otherwise)
     ws_bytes = int(lib.hc_aggr_fwd_workspace_bytes(mode, R, idx.numel(), n_src)) if n_head == 1 else 0
     ws = _workspace(ws_bytes, x.device) if ws_bytes > 0 else None
-    if edge_sub is not None:
-        if mode != SUBST_SRC or hmap is None or edge_value is not None:
-            raise ValueError("edge_sub goes with per-source substitution of a plain mean")
-        _dev(edge_sub, "edge_sub", torch.uint8)
-        rc = lib.hc_aggr_fwd_src_mask(_ptr(ptr), _ptr(idx), _ptr(x), _float_dtype(x, "input"), _ptr(hmap), _ptr(hbuf),
-                                      _float_dtype(hbuf, "history_buffer"), int(hsize), _ptr(out), _ptr(edge_sub),
-                                      R, F, n_src, _ptr(ws), ws_bytes, _stream())
-        _check(rc, "hc_aggr_fwd_src_mask")
-        return out
     rc = lib.hc_aggr_fwd(mode, _ptr(ptr), _ptr(idx), _ptr(x), _float_dtype(x, "input"),
                          _ptr(hmap), _ptr(hbuf), _float_dtype(hbuf, "history_buffer") if hmap is not None else 0,
                          int(hsize), _ptr(edge_value), n_head, _ptr(out), R, F, n_src, _ptr(ws), ws_bytes,
@@ -297,14 +282,13 @@ def _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, num_node, edge_s
 
 
 def build_transpose(ptr, idx, history_map_row, num_node, n_src, num_edge=None, want_edges=True,
-                    history_map_src=None, edge_drop=None):
+                    history_map_src=None):
     """Stable CSC view of the first ``num_node`` rows: returns (ptrT, rowT, edgeT).
 
     ``num_edge`` bounds the edge slots that are sorted (default: all of ``idx``).  With
     ``want_edges=False`` (enough for the mean aggregation) edgeT is None and the build is cheaper.
     Edges of rows flagged by ``history_map_row`` and edges whose source is flagged by
-    ``history_map_src`` (per-source substitution) are left out; ``edge_drop`` (uint8 per edge slot, what
-    ``_aggr_fwd(..., edge_sub=...)`` wrote) says the same per edge slot without another look at the map."""
+    ``history_map_src`` (per-source substitution) are left out."""
     lib = load_library()
     _dev(ptr, "ptr", torch.int64)
     _dev(idx, "idx", torch.int64)
@@ -325,16 +309,6 @@ def build_transpose(ptr, idx, history_map_row, num_node, n_src, num_edge=None, w
         raise ValueError("source_history_map is shorter than n_src")
     if hm is not None and hm.numel() < R:
         raise ValueError("history_map is shorter than num_node")
-    if edge_drop is not None:
-        if hs is not None:
-            raise ValueError("give source_history_map or edge_drop, not both")
-        _dev(edge_drop, "edge_drop", torch.uint8)
-        if edge_drop.numel() < E:
-            raise ValueError("edge_drop is shorter than the edge slots to sort")
-        rc = lib.hc_build_transpose_edge_mask(_ptr(ptr), _ptr(idx), _ptr(hm), _ptr(edge_drop), R, E, n_src,
-                                              _ptr(ptrT), _ptr(rowT), _ptr(edgeT), _ptr(ws), ws.numel(), _stream())
-        _check(rc, "hc_build_transpose_edge_mask")
-        return ptrT, rowT, edgeT
     rc = lib.hc_build_transpose(_ptr(ptr), _ptr(idx), _ptr(hm), _ptr(hs), R, E, n_src, _ptr(ptrT), _ptr(rowT),
                                 _ptr(edgeT), _ptr(ws), ws.numel(), _stream())
     _check(rc, "hc_build_transpose")
@@ -476,13 +450,7 @@ class _AggrHistory(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, ptr, idx, edge_value, hmap, hbuf, hsize, num_node, mode, num_edge=None, view=None):
         R = int(num_node) if num_node else ptr.numel() - 1
-        # Per-source substitution with a gradient wanted for x: the launch notes which edge slots read the
-        # table, so that backward's view leaves them out without looking every source up again.
-        ctx.edge_sub = None
-        if mode == SUBST_SRC and hmap is not None and edge_value is None and ctx.needs_input_grad[0]:
-            n_slots = idx.numel() if num_edge is None else min(int(num_edge), idx.numel())
-            ctx.edge_sub = torch.empty(max(n_slots, 1), dtype=torch.uint8, device=x.device)
-        out = _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, R, edge_sub=ctx.edge_sub)
+        out = _aggr_fwd(mode, ptr, idx, x, hmap, hbuf, hsize, edge_value, R)
         ctx.hc = (ptr, idx, hmap, hsize, R, mode, None if hbuf is None else tuple(hbuf.shape))
         # edge slots the first R rows can reach, when the caller knows it (a layer of a shared CSR owns a
         # prefix of idx): the transposed view then sorts that prefix only
@@ -537,10 +505,8 @@ class _AggrHistory(torch.autograd.Function):
         # read).  When the table needs no gradient those edges are left out of the view; when it does,
         # every source is summed and the rows of substituted sources are moved to the table's gradient.
         num_edge = ctx.num_edge
-        by_slot = ctx.edge_sub is not None and not want_table
         tr = build_transpose(ptr, idx, row_map, R, n_src, num_edge=num_edge, want_edges=ev is not None,
-                             history_map_src=None if (want_table or by_slot) else src_map,
-                             edge_drop=ctx.edge_sub if by_slot else None)
+                             history_map_src=None if want_table else src_map)
         grad_x, grad_h, edge_grad = _aggr_bwd(ptr, idx, tr, g, row_map, ev, x, want_eg, hshape, hsize, R,
                                               n_src, want_hist_grad=want_h)
         if want_table:

@@ -95,17 +95,6 @@ int hc_aggr_fwd(int mode, const int64_t *ptr, const int64_t *idx, const void *vi
                 const float *edge_value, int64_t n_head, float *vout, int64_t R, int64_t F,
                 int64_t n_src, void *workspace, size_t workspace_bytes, void *stream);
 
-/* hc_aggr_fwd_src_mask: hc_aggr_fwd in HC_SUBST_SRC mode (plain mean, hmap required) that also
- * notes, for every edge slot e in [ptr[0], ptr[R]), whether the launch read a row of the table
- * (edge_sub[e] = 1) or of vin (0); edge_sub has at least ptr[R] entries.  The answer costs the
- * forward one byte per edge and saves the backward's view (hc_build_transpose_edge_mask) a second
- * look-up of every source.  No reference counterpart: the reference substitutes per destination
- * row only (history_aggr.cu:21-25). */
-int hc_aggr_fwd_src_mask(const int64_t *ptr, const int64_t *idx, const void *vin, int in_dtype,
-                         const int64_t *hmap, const void *hbuf, int hist_dtype, int64_t hsize,
-                         float *vout, uint8_t *edge_sub, int64_t R, int64_t F, int64_t n_src,
-                         void *workspace, size_t workspace_bytes, void *stream);
-
 /* The long-row threshold T that hc_aggr_fwd applies to a mean aggregation with
  * rows of F elements of in_dtype; 0 when every row is summed strictly in CSR
  * order.  No reference counterpart (the reference sums every row with one
@@ -138,14 +127,6 @@ int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hm
                        const int64_t *hmap_src, int64_t R, int64_t E, int64_t n_src, int64_t *ptrT,
                        int32_t *rowT, int32_t *edgeT, void *workspace, size_t workspace_bytes,
                        void *stream);
-
-/* hc_build_transpose_edge_mask: hc_build_transpose with the dropped sources given per edge slot
- * (edge_drop[e] != 0: slot e is left out; E entries; what hc_aggr_fwd_src_mask wrote) instead of per
- * source.  Same outputs, same workspace. */
-int hc_build_transpose_edge_mask(const int64_t *ptr, const int64_t *idx, const int64_t *hmap_row,
-                                 const uint8_t *edge_drop, int64_t R, int64_t E, int64_t n_src,
-                                 int64_t *ptrT, int32_t *rowT, int32_t *edgeT, void *workspace,
-                                 size_t workspace_bytes, void *stream);
 
 /* hc_build_transpose_dev: the same view (no history maps: nothing is left out)
  * for a block whose sizes the host does not know yet -- a mini-batch that
