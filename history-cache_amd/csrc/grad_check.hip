@@ -984,6 +984,7 @@ __global__ __launch_bounds__(QT_BLOCK) void quantile_kernel(const float *__restr
   __shared__ QtShared sh;
   uint32_t rk[QT_REG];
   int nk = 0;
+  int nan_seen = 0;                    // torch.quantile answers NaN when any score is NaN: so does this kernel
   if constexpr (REG) {
 #pragma unroll
     for (int j = 0; j < QT_REG; ++j) {
@@ -992,8 +993,17 @@ __global__ __launch_bounds__(QT_BLOCK) void quantile_kernel(const float *__restr
       if (i < n) {
         rk[j] = qt_key(score[i]);
         nk = j + 1;
+        if (rk[j] == 0xffffffffu) nan_seen = 1;
       }
     }
+  } else {
+    for (int64_t i = threadIdx.x; i < n; i += QT_BLOCK)
+      if (score[i] != score[i]) nan_seen = 1;
+  }
+  nan_seen = __syncthreads_or(nan_seen);
+  if (nan_seen) {                      // block-uniform
+    if (threadIdx.x == 0) out[0] = __uint_as_float(0x7fc00000u);
+    return;
   }
   int64_t k_in_bin = 0;
   int n_equal = 0;

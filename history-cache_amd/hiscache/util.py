@@ -70,15 +70,19 @@ def quantile_threshold(score, rate):
         got = hiscache_backend.quantile_select(flat, lo, hi, w, one_minus_w)
         if got is not None:
             return got
-    srt = torch.sort(score.detach().reshape(-1).to(torch.float32)).values
+    flat = score.detach().reshape(-1).to(torch.float32)
+    srt = torch.sort(flat).values
     a = srt[lo:lo + 1]
     b = srt[hi:hi + 1]
     d = b - a
     if w < 0.5:
         m = d * w
-        return a + m
-    m = d * (1.0 - torch.tensor(w, dtype=torch.float32)).item()
-    return b - m
+        res = a + m
+    else:
+        m = d * (1.0 - torch.tensor(w, dtype=torch.float32)).item()
+        res = b - m
+    # torch.quantile answers NaN when any score is NaN (a sort would rank the NaN last and hide it)
+    return torch.where(torch.isnan(flat).any(), torch.full_like(res, float("nan")), res)
 
 
 def backward_on_this_thread(loss, **kwargs):

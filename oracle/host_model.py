@@ -21,6 +21,8 @@ def quantile_threshold(score, rate):
     operations; mathematically torch.quantile(score, rate), history_cache.py:211)."""
     s = np.sort(np.asarray(score, np.float32).reshape(-1))
     n = s.size
+    if np.isnan(s).any():            # torch.quantile answers NaN when any score is NaN (history_cache.py:211)
+        return np.float32("nan")
     pos = np.float32(np.float32(rate) * np.float32(n - 1))   # torch.quantile ranks in the data's dtype
     lo = min(int(np.floor(pos)), n - 1)
     hi = min(lo + 1, n - 1)

@@ -137,5 +137,93 @@ def main():
           [int(out[f"it{i}_header"]) for i in range(1, n_iter + 1)])
 
 
+# ---- the admission at the widths of the plumbing configuration -------------------------------------------
+# 100 000 nodes, 128-wide features and embeddings, about 10 000 one-hop rows per batch, rate 0.5, five
+# iterations with a staleness refresh.  The inputs are rebuilt from seeds by tests/helpers.py (exact_rows,
+# affine_ids); the fixture keeps the seeds and what the reference's update_history made of them: the record
+# mask, the reference's own scores and threshold (so that a test can count the rows at the knife edge should a
+# mask ever differ), the header, and digests of the maps and of the stored rows.
+WIDE_CASES = {
+    "": dict(N=100_000, Fin=128, H=128, n1=10_000, n_seed=1000, rate=0.5, staleness_thres=3, n_iter=5,
+             buffer_floats=128 * 24_000, seed=77),
+    # the hidden width of the papers100M- and mag240M-shaped configurations
+    "_h256": dict(N=100_000, Fin=128, H=256, n1=10_000, n_seed=1000, rate=0.5, staleness_thres=3, n_iter=5,
+                  buffer_floats=256 * 20_000, seed=78),
+}
+
+
+def wide_inputs(w, it):
+    """(sub_to_full[:n1], embedding rows, gradient rows) of iteration `it` (1-based)."""
+    from helpers import affine_ids, exact_rows
+    ids = affine_ids(w["N"], w["n1"], 7919 + 20 * it, 31 * it)       # overlaps the earlier batches in part
+    emb = exact_rows(w["seed"] + 100 * it, w["n1"], w["H"], octaves=1)
+    grad = exact_rows(w["seed"] + 100 * it + 1, w["n1"], w["H"])
+    return ids, emb, grad
+
+
+def digest(a):
+    import hashlib
+    return np.frombuffer(hashlib.sha256(np.ascontiguousarray(a).tobytes()).digest(), dtype=np.uint8).copy()
+
+
+def main_wide(suffix):
+    from helpers import exact_rows
+    HistoryCache = load_reference_class()
+    w = WIDE_CASES[suffix]
+    N, Fin, H = w["N"], w["Fin"], w["H"]
+    feats = torch.from_numpy(exact_rows(w["seed"], N, Fin, octaves=1))
+    hot = torch.from_numpy(((np.arange(N, dtype=np.int64) * 48271 + 11) % N).astype(np.int64))
+
+    c = HistoryCache.__new__(HistoryCache)
+    c.in_channels, c.hidden_channels, c.total_num_node = Fin, H, N
+    c.device = torch.device("cpu")
+    c.method, c.rate, c.staleness_thres, c.start_history = "grad", w["rate"], w["staleness_thres"], 0
+    c.feat_mode, c.distributed_store = "history_uvm", False
+    c.header, c.glb_iter, c.num_stored_history = 0, 0, 0
+    c.full2embed = torch.ones([2 * N + 1], dtype=torch.int64) * -1
+    c.buffer = torch.zeros(w["buffer_floats"])
+    c.embed2full = torch.ones(w["buffer_floats"] // H, dtype=torch.int64) * -1
+    n_feat = w["buffer_floats"] // Fin
+    cache_ids = hot[-n_feat:]
+    c.feat2full = cache_ids + N
+    c.full2embed[c.feat2full] = torch.arange(0, n_feat)
+    c.buffer.view(-1, Fin)[-n_feat:] = feats[cache_ids]
+
+    out = {k: np.asarray(v) for k, v in w.items()}
+    high = 0
+    for it in range(1, w["n_iter"] + 1):
+        ids, emb, grad = wide_inputs(w, it)
+        batch = types.SimpleNamespace(sub_to_full=torch.from_numpy(ids),
+                                      num_node_in_layer=torch.tensor([w["n_seed"], w["n1"]]))
+        # what lookup_and_load leaves behind for update_history (history_cache.py:307-310), seeds excluded as there
+        c.sub2embed = c.full2embed[batch.sub_to_full[: w["n1"]]]
+        pe = torch.from_numpy(emb.copy()).requires_grad_(True)
+        pe.grad = torch.from_numpy(grad.copy())
+        c.produced_embedding = pe
+        score = pe.grad.norm(dim=1)                                   # the reference's own expressions
+        thres = torch.quantile(score, w["rate"])                       # (history_cache.py:205, 211)
+        before = c.full2embed[batch.sub_to_full[: w["n1"]]].clone()
+        header_before = 0 if it % w["staleness_thres"] == 0 else c.header
+        c.update_history(batch, it)
+        after = c.full2embed[batch.sub_to_full[: w["n1"]]]
+        recorded = (after >= header_before) & (after < c.header) & (before == -1)
+        pre = f"it{it}_"
+        out[pre + "record_mask"] = np.packbits(recorded.numpy())
+        out[pre + "ref_score"] = score.numpy().copy()
+        out[pre + "ref_thres"] = np.float32(thres)
+        out[pre + "header"] = np.int64(c.header)
+        high = max(high, c.header)
+        out[pre + "full2embed_sha256"] = digest(c.full2embed.numpy())
+        out[pre + "embed2full_sha256"] = digest(c.embed2full.numpy())
+        out[pre + "buffer_front_sha256"] = digest(c.buffer.numpy()[: high * H])
+        out[pre + "rows_stored"] = np.int64(high)
+    path = os.path.join(HERE, "history_cache_golden_wide%s.npz" % suffix)
+    np.savez_compressed(path, **out)
+    print("wrote", path, "headers:", [int(out[f"it{i}_header"]) for i in range(1, w["n_iter"] + 1)],
+          "bytes:", os.path.getsize(path))
+
+
 if __name__ == "__main__":
     main()
+    for suffix in WIDE_CASES:
+        main_wide(suffix)

@@ -44,3 +44,41 @@ def power_law_graph(rng, num_nodes, degree_scale, alpha=2.0, max_degree=2000, po
     else:
         indices = rng.integers(0, num_nodes, size=E, dtype=np.int64)
     return indptr, indices.astype(np.int64)
+
+
+# ---- inputs that can be rebuilt bit for bit from a seed (fixtures then hold seeds and outputs only) --------
+_M64 = np.uint64(0xFFFFFFFFFFFFFFFF)
+
+
+def _splitmix64(x):
+    """The splitmix64 finaliser on uint64 arrays (wrap-around arithmetic, no floating point)."""
+    with np.errstate(over="ignore"):
+        z = (x + np.uint64(0x9E3779B97F4A7C15)) & _M64
+        z = ((z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)) & _M64
+        z = ((z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)) & _M64
+        return z ^ (z >> np.uint64(31))
+
+
+def exact_rows(seed, n, width, octaves=13):
+    """[n, width] float32 built from integer hashes and exactly representable operations only (no library
+    random stream, no transcendental function), so that any NumPy on any machine rebuilds the same bits:
+    entry = (sum of four 16-bit fields of a hash - 131070) / 65536, a bell-shaped value in (-2, 2), times a
+    per-row scale 2^-k * (1 + m/256) with k < octaves, which spreads the row norms over several octaves the
+    way gradient rows are spread."""
+    cell = np.arange(n * width, dtype=np.uint64).reshape(n, width)
+    with np.errstate(over="ignore"):
+        h = _splitmix64(cell * np.uint64(2) + np.uint64(seed) * np.uint64(0x100000001B3))
+        hr = _splitmix64(np.arange(n, dtype=np.uint64) * np.uint64(2) + np.uint64(1)
+                         + np.uint64(seed) * np.uint64(0x100000001B3))
+    f = [((h >> np.uint64(16 * q)) & np.uint64(0xFFFF)).astype(np.int64) for q in range(4)]
+    value = (f[0] + f[1] + f[2] + f[3] - 131070).astype(np.float64) / 65536.0
+    k = (hr % np.uint64(octaves)).astype(np.int64)
+    m = ((hr >> np.uint64(8)) & np.uint64(0xFF)).astype(np.float64)
+    scale = np.ldexp(1.0 + m / 256.0, -k)
+    return (value * scale[:, None]).astype(np.float32)
+
+
+def affine_ids(n_full, count, a, b):
+    """`count` distinct node ids (a * i + b) mod n_full; a must be coprime with n_full."""
+    assert np.gcd(a, n_full) == 1 and count <= n_full
+    return ((np.arange(count, dtype=np.int64) * a + b) % n_full).astype(np.int64)

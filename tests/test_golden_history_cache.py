@@ -76,3 +76,110 @@ def test_gpu_cache_reproduces_reference_vectors():
         assert cache.header == int(g[pre + "header"])
         front = g[pre + "buffer_front"]
         np.testing.assert_array_equal(cache.buffer.cpu().numpy()[: front.size], front)
+
+
+# ---- the admission at the plumbing configuration's widths (128-wide rows, 10 000 one-hop rows per batch) ----
+EXACT_ROWS_DIGEST = "7df0f62c50da8be0041fa1c1f53b8388f7e865cc1a8e791003906c644f65e219"
+WIDE = {h: os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "history_cache_golden_wide%s.npz" % sfx)
+        for h, sfx in ((128, ""), (256, "_h256"))}
+
+
+def wide_inputs(g, it):
+    from helpers import affine_ids, exact_rows
+    N, n1, H, seed = int(g["N"]), int(g["n1"]), int(g["H"]), int(g["seed"])
+    ids = affine_ids(N, n1, 7919 + 20 * it, 31 * it)
+    emb = exact_rows(seed + 100 * it, n1, H, octaves=1)
+    grad = exact_rows(seed + 100 * it + 1, n1, H)
+    return ids, emb, grad
+
+
+def sha256_of(t):
+    import hashlib
+    return np.frombuffer(hashlib.sha256(np.ascontiguousarray(t).tobytes()).digest(), dtype=np.uint8)
+
+
+def knife_edge_rows(score, thres):
+    """Rows whose score lies within 2 ulp of the threshold: the only rows whose side of `score < thres` can
+    depend on the order in which a row's squares were added."""
+    ulp = np.spacing(np.float32(abs(thres)))
+    return int((np.abs(score.astype(np.float64) - float(thres)) <= 2.0 * float(ulp)).sum())
+
+
+def check_wide_iteration(g, it, mask, score, header, full2embed, embed2full, buffer):
+    pre = f"it{it}_"
+    n1, H = int(g["n1"]), int(g["H"])
+    want_mask = np.unpackbits(g[pre + "record_mask"])[:n1].astype(bool)
+    differ = int((mask != want_mask).sum())
+    # should a mask ever differ, say how many rows sit at the knife edge of either side's threshold
+    edge = knife_edge_rows(g[pre + "ref_score"], g[pre + "ref_thres"]) + knife_edge_rows(score, g[pre + "ref_thres"])
+    assert differ == 0, f"iteration {it}: {differ} rows of the record mask differ; {edge} rows within 2 ulp of the threshold"
+    assert header == int(g[pre + "header"])
+    np.testing.assert_array_equal(sha256_of(full2embed), g[pre + "full2embed_sha256"])
+    np.testing.assert_array_equal(sha256_of(embed2full), g[pre + "embed2full_sha256"])
+    rows = int(g[pre + "rows_stored"])
+    np.testing.assert_array_equal(sha256_of(buffer[: rows * H]), g[pre + "buffer_front_sha256"])
+
+
+def test_exact_rows_are_rebuilt_bit_for_bit():
+    """The fixture's inputs come from integer hashes: a known digest pins them on any machine."""
+    from helpers import affine_ids, exact_rows
+    r = exact_rows(77, 300, 128)
+    assert r.dtype == np.float32 and np.isfinite(r).all() and (np.abs(r) < 4).all()
+    norms = np.linalg.norm(r.astype(np.float64), axis=1)
+    assert norms.max() / norms.min() > 500                   # rows spread over several octaves
+    assert sha256_of(r).tobytes().hex() == EXACT_ROWS_DIGEST
+    ids = affine_ids(100_000, 10_000, 7939, 31)
+    assert len(np.unique(ids)) == 10_000
+
+
+@pytest.mark.parametrize("hidden", [128, 256])
+def test_oracle_reproduces_reference_vectors_at_real_width(orc, hidden):
+    """oracle.host_model.update_history with the oracle's row scores (the kernel's lane order) against what the
+    reference's grad.norm(dim=1) + torch.quantile + masking recorded: masks, maps, header, stored rows."""
+    from helpers import exact_rows
+    from oracle import host_model
+    g = np.load(WIDE[hidden], allow_pickle=False)
+    N, Fin, H, n1 = int(g["N"]), int(g["Fin"]), int(g["H"]), int(g["n1"])
+    feats = torch.from_numpy(exact_rows(int(g["seed"]), N, Fin, octaves=1))
+    hot = ((np.arange(N, dtype=np.int64) * 48271 + 11) % N).astype(np.int64)
+    st = host_model.new_cache_state(N, Fin, H, int(g["buffer_floats"]), hot, feats)
+    for it in range(1, int(g["n_iter"]) + 1):
+        ids, emb, grad = wide_inputs(g, it)
+        sub_to_full = torch.from_numpy(ids)
+        sub2embed = st.full2embed[sub_to_full[:n1]]
+        score = orc.row_scores(grad)
+        mask, _ = host_model.update_history(st, sub_to_full, sub2embed, torch.from_numpy(emb), torch.from_numpy(score),
+                                            float(g["rate"]), int(g["staleness_thres"]), it)
+        check_wide_iteration(g, it, mask.numpy(), score, st.header, st.full2embed.numpy(), st.embed2full.numpy(),
+                             st.buffer.numpy())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("hidden", [128, 256])
+def test_gpu_cache_reproduces_reference_vectors_at_real_width(hidden):
+    """The GPU HistoryCache.update_history (hc_row_scores + hc_quantile_threshold + hc_cache_append) at 128- and
+    256-wide rows and 10 000 rows per batch against the reference's own admission, exactly."""
+    from helpers import exact_rows
+    from hiscache import HistoryCache, PinnedFeatureStore, make_config
+    dev = "cuda:0"
+    g = np.load(WIDE[hidden], allow_pickle=False)
+    N, Fin, H, n1 = int(g["N"]), int(g["Fin"]), int(g["H"]), int(g["n1"])
+    feats = torch.from_numpy(exact_rows(int(g["seed"]), N, Fin, octaves=1))
+    hot = ((np.arange(N, dtype=np.int64) * 48271 + 11) % N).astype(np.int64)
+    cfg = make_config(Fin, 5, H, 2, method="grad", rate=float(g["rate"]), staleness_thres=int(g["staleness_thres"]),
+                      device=dev)
+    cache = HistoryCache(PinnedFeatureStore(feats, device=dev), cfg, "history_uvm", total_num_node=N,
+                         buffer_bytes=int(g["buffer_floats"]) * 4, hot_ids=hot)
+    for it in range(1, int(g["n_iter"]) + 1):
+        ids, emb, grad = wide_inputs(g, it)
+        batch = SimpleNamespace(sub_to_full=torch.from_numpy(ids).to(dev),
+                                num_node_in_layer=torch.tensor([int(g["n_seed"]), n1]))
+        # what lookup_and_load leaves for update_history (reference history_cache.py:307-310)
+        cache.sub2embed = cache.full2embed[batch.sub_to_full[:n1]]
+        pe = torch.from_numpy(emb).to(dev).requires_grad_(True)
+        pe.grad = torch.from_numpy(grad).to(dev)
+        cache.produced_embedding = pe
+        cache.update_history(batch, it)
+        check_wide_iteration(g, it, cache.last_record_mask.cpu().numpy().astype(bool), cache.last_score.cpu().numpy(),
+                             cache.header, cache.full2embed.cpu().numpy(), cache.embed2full.cpu().numpy(),
+                             cache.buffer.cpu().numpy())

@@ -361,6 +361,20 @@ def test_quantile_threshold_matches_torch_quantile():
     assert worst <= 2, worst
 
 
+def test_quantile_threshold_is_nan_when_a_score_is_nan():
+    """torch.quantile answers NaN when any score is NaN (the reference then admits nothing,
+    hiscache/history_cache.py:211-215); the restatement and the package's host spelling do the same."""
+    from hiscache.util import quantile_threshold as pkg_quantile
+    from oracle import host_model
+    s = np.random.default_rng(3).standard_normal(500).astype(np.float32)
+    s[17] = np.nan
+    for rate in (0.0, 0.5, 1.0):
+        assert np.isnan(torch.quantile(torch.from_numpy(s), rate).numpy())
+        assert np.isnan(host_model.quantile_threshold(s, rate))
+        t = pkg_quantile(torch.from_numpy(s), rate)
+        assert np.isnan(t.numpy()[0]) and int((torch.from_numpy(s) < t).sum()) == 0
+
+
 def test_quantile_threshold_gives_torch_quantiles_admission_mask():
     """The reference thresholds with torch.quantile (hiscache/history_cache.py:211-215).  Over 1 200
     seeded batches at the 1-hop sizes of the plumbing and papers100M-shaped configurations (scores
