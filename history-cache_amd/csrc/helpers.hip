@@ -540,3 +540,76 @@ extern "C" int hc_ring_lookup(const int64_t *full2slot, int64_t n_full, const in
                                                          slot_out, rows_out, n);
   return hc_launch_status();
 }
+
+// ---------------------------------------------------------------------------------------
+// hc_load_mask: which rows of a batch must be read from the feature store, and the cache's
+// hit counters, in one launch (the reference spells the mask with three tensor operators and
+// prints the same counts from a debug branch, hiscache/history_cache.py:327-341).
+// ---------------------------------------------------------------------------------------
+namespace {
+constexpr int LM_COUNTERS = 8;
+
+__global__ __launch_bounds__(HC_BLOCK) void load_mask_kernel(const uint8_t *__restrict__ used,
+                                                              const int64_t *__restrict__ sub2feat,
+                                                              const int64_t *__restrict__ sub2embed,
+                                                              const uint8_t *__restrict__ prev_mask,
+                                                              int64_t n_all, int64_t n1, int64_t n_prev,
+                                                              uint8_t *__restrict__ hit_feat,
+                                                              uint8_t *__restrict__ load_mask,
+                                                              unsigned long long *__restrict__ counters) {
+  __shared__ unsigned int s_cnt[LM_COUNTERS];
+  if (threadIdx.x < LM_COUNTERS) s_cnt[threadIdx.x] = 0u;
+  __syncthreads();
+  const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
+  bool u = false, hit = false, load = false, emb = false, adm = false;
+  if (i < n_all) {
+    u = used[i] != 0;
+    hit = sub2feat != nullptr && sub2feat[i] != -1;
+    load = u && !hit;
+    if (hit_feat != nullptr) hit_feat[i] = hit ? 1 : 0;
+    if (load_mask != nullptr) load_mask[i] = load ? 1 : 0;
+  }
+  if (sub2embed != nullptr && i < n1) emb = sub2embed[i] != -1;
+  if (prev_mask != nullptr && i < n_prev) adm = prev_mask[i] != 0;
+  if (counters == nullptr) return;
+  const int lane = hc_lane();
+  const unsigned int c_pruned = (unsigned int)__popcll(__ballot(i < n_all && !u));
+  const unsigned int c_hit = (unsigned int)__popcll(__ballot(hit));
+  const unsigned int c_load = (unsigned int)__popcll(__ballot(load));
+  const unsigned int c_emb = (unsigned int)__popcll(__ballot(emb));
+  const unsigned int c_adm = (unsigned int)__popcll(__ballot(adm));
+  if (lane == 0) {
+    if (c_emb) atomicAdd(&s_cnt[3], c_emb);
+    if (c_pruned) atomicAdd(&s_cnt[4], c_pruned);
+    if (c_hit) atomicAdd(&s_cnt[5], c_hit);
+    if (c_load) atomicAdd(&s_cnt[6], c_load);
+    if (c_adm) atomicAdd(&s_cnt[7], c_adm);
+  }
+  __syncthreads();
+  if (threadIdx.x >= 3 && threadIdx.x < LM_COUNTERS && s_cnt[threadIdx.x] != 0u)
+    atomicAdd(&counters[threadIdx.x], (unsigned long long)s_cnt[threadIdx.x]);
+  if (blockIdx.x == 0 && threadIdx.x < 3) {
+    const unsigned long long add = threadIdx.x == 0 ? 1ull : (threadIdx.x == 1 ? (unsigned long long)n_all
+                                                                                : (unsigned long long)n1);
+    atomicAdd(&counters[threadIdx.x], add);
+  }
+}
+}  // namespace
+
+extern "C" int hc_load_mask(const uint8_t *used, const int64_t *sub2feat, const int64_t *sub2embed,
+                            const uint8_t *prev_mask, int64_t n_all, int64_t n1, int64_t n_prev,
+                            uint8_t *hit_feat, uint8_t *load_mask, int64_t *counters, void *stream) {
+  HC_REQUIRE(n_all >= 0 && n1 >= 0 && n_prev >= 0);
+  HC_REQUIRE(used != nullptr || n_all == 0);
+  HC_REQUIRE(sub2embed != nullptr || n1 == 0);
+  HC_REQUIRE(prev_mask != nullptr || n_prev == 0);
+  int64_t n = n_all > n1 ? n_all : n1;
+  if (n_prev > n) n = n_prev;
+  if (n == 0) n = 1;                               // the call is still counted
+  const int64_t b = (n + HC_BLOCK - 1) / HC_BLOCK;
+  if (!hc_grid_ok(b)) return HC_EUNSUPPORTED;
+  load_mask_kernel<<<dim3((unsigned)b), dim3(HC_BLOCK), 0, static_cast<hipStream_t>(stream)>>>(
+      used, sub2feat, sub2embed, prev_mask, n_all, n1, n_prev, hit_feat, load_mask,
+      reinterpret_cast<unsigned long long *>(counters));
+  return hc_launch_status();
+}

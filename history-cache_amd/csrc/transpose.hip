@@ -247,6 +247,7 @@ struct TrSmallHeader {
 struct TrDims {
   int64_t R, E, n_src;               // by value (or the upper bounds when the pointers are set)
   const int64_t *pR, *pE, *pS;       // nullable, all three or none
+  int32_t *overflow;                 // nullable: set to 1 when a size read on the device had to be clamped, else 0
 };
 __device__ __forceinline__ void tr_dims(const TrDims &d, int64_t &R, int64_t &E, int64_t &n_src) {
   R = d.R;
@@ -259,6 +260,12 @@ __device__ __forceinline__ void tr_dims(const TrDims &d, int64_t &R, int64_t &E,
     n_src = s < 0 ? 0 : (s < d.n_src ? s : d.n_src);
   }
 }
+// Did tr_dims clamp anything?  (A view of a truncated block is a valid view of the wrong block.)
+__device__ __forceinline__ bool tr_dims_clamped(const TrDims &d) {
+  if (d.pE == nullptr) return false;
+  const int64_t r = *d.pR, e = *d.pE, s = *d.pS;
+  return r < 0 || e < 0 || s < 0 || e > d.E || s > d.n_src;
+}
 
 // zero the ticket and the counters of sources [0, n_src] (rounded up to whole 16-byte groups)
 __global__ __launch_bounds__(HC_BLOCK) void tr_small_clear(uint32_t *__restrict__ p, TrDims dims) {
@@ -267,6 +274,7 @@ __global__ __launch_bounds__(HC_BLOCK) void tr_small_clear(uint32_t *__restrict_
   const int64_t n = (int64_t)(sizeof(TrSmallHeader) / sizeof(uint32_t)) + (n_src + 1 + 3) / 4 * 4;
   const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
   if (i < n) p[i] = 0u;
+  if (i == 0 && dims.overflow != nullptr) *dims.overflow = tr_dims_clamped(dims) ? 1 : 0;
 }
 
 // Read of a counter by the block that scans them.  The counters were only ever touched by atomics (which
@@ -703,7 +711,7 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
     if (!workspace || workspace_bytes < S.total) return HC_EWORKSPACE;
     char *w = static_cast<char *>(workspace);
     if (reinterpret_cast<uintptr_t>(w) % 256 != 0) return HC_EWORKSPACE;
-    const TrDims dims{R, E, n_src, nullptr, nullptr, nullptr};
+    const TrDims dims{R, E, n_src, nullptr, nullptr, nullptr, nullptr};
     return small_launch(ptr, idx, hmap_row, hmap_src, dims, ptrT, rowT, edgeT, w, S, st);
   }
   if (bucket_sorted(E, n_src)) {
@@ -800,7 +808,7 @@ extern "C" size_t hc_transpose_dev_workspace_bytes(int64_t max_E, int64_t max_sr
 extern "C" int hc_build_transpose_dev(const int64_t *ptr, const int64_t *idx, const int64_t *R_dev,
                                       const int64_t *E_dev, const int64_t *n_src_dev, int64_t max_E,
                                       int64_t max_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT,
-                                      void *workspace, size_t workspace_bytes, void *stream) {
+                                      int32_t *overflow, void *workspace, size_t workspace_bytes, void *stream) {
   HC_REQUIRE(ptr && idx && R_dev && E_dev && n_src_dev && ptrT && max_E >= 0 && max_src >= 0);
   HC_REQUIRE(rowT != nullptr || max_E == 0);
   if (max_E > TR_DEV_MAX_EDGES || max_src > TR_DEV_MAX_SOURCES) return HC_EUNSUPPORTED;
@@ -808,6 +816,6 @@ extern "C" int hc_build_transpose_dev(const int64_t *ptr, const int64_t *idx, co
   if (!workspace || workspace_bytes < S.total) return HC_EWORKSPACE;
   char *w = static_cast<char *>(workspace);
   if (reinterpret_cast<uintptr_t>(w) % 256 != 0) return HC_EWORKSPACE;
-  const TrDims dims{0, max_E, max_src, R_dev, E_dev, n_src_dev};
+  const TrDims dims{0, max_E, max_src, R_dev, E_dev, n_src_dev, overflow};
   return small_launch(ptr, idx, nullptr, nullptr, dims, ptrT, rowT, edgeT, w, S, static_cast<hipStream_t>(stream));
 }

@@ -47,6 +47,14 @@ class PinnedFeatureStore:
             return _be.cu_limited_stream(self.prefetch_cus, self.device)
         return torch.cuda.Stream(device=self.device)
 
+    def close(self):
+        """Release the read-ahead stream (a CU-limited stream is a driver object that lives until it is
+        destroyed; without this it goes at interpreter exit).  The store stays usable: the next ``prefetch``
+        makes a new stream."""
+        side, self._prefetch_side = self._prefetch_side, None
+        if side is not None and self.prefetch_cus > 0:
+            _be.release_cu_limited_stream(side)
+
     def get(self, ids):
         return _be.gather_rows(self.buffer, ids, out_dtype=self.out_dtype)
 

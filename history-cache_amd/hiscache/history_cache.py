@@ -57,6 +57,9 @@ class HistoryCache:
                                      device=self.device)
         self._header = torch.zeros(1, dtype=torch.int64, device=self.device)
         self._overflow = torch.zeros(1, dtype=torch.int64, device=self.device)
+        # what the lookups find (hiscache_backend.STAT_NAMES), counted on the device and read by stats() only
+        self._counters = torch.zeros(8, dtype=torch.int64, device=self.device)
+        self._uncounted_mask = None
         self._num_stored = torch.zeros(1, dtype=torch.int64, device=self.device)
         self.produced_embedding = None
         self.feat_mode = mode
@@ -183,6 +186,7 @@ class HistoryCache:
                                 self.hidden_channels, self.in_channels, self.full2embed,
                                 self.embed2full, self.feat2full, self._header, self._overflow)
         self.last_record_mask = mask
+        self._uncounted_mask = mask
         self.last_score = score
         self.produced_embedding = None
 
@@ -220,8 +224,9 @@ class HistoryCache:
         self.used_masks = _be.count_history_reconstruct(batch.ptr, batch.idx, self.sub2embed,
                                                         sub_to_full.shape[0], batch.y.shape[0],
                                                         num_layer)
-        hit_feat_mask = self.sub2feat != -1
-        load_mask = torch.logical_and(self.used_masks[0], ~hit_feat_mask)
+        # hit_feat = sub2feat != -1, load = used & ~hit_feat (reference :327-330) and the hit counters, one launch
+        hit_feat_mask, load_mask = _be.load_mask(self.used_masks[0], self.sub2feat, self.sub2embed,
+                                                 self._counted_mask(), self._counters)
         self.glb_iter += 1
         pre, exact = self._take_prefetched(batch, load_mask)
         if pre is not None and not exact:
@@ -283,13 +288,35 @@ class HistoryCache:
             return self.uvm.take(handle), False
         return self.uvm.take(handle, need), True
 
+    def _counted_mask(self):
+        """The last admission mask, once: the next lookup's launch adds its rows to the counters."""
+        m, self._uncounted_mask = self._uncounted_mask, None
+        return m
+
     def stats(self):
-        """Cache occupancy (synchronises)."""
+        """Cache occupancy, and what the lookups since construction (or ``reset_stats``) found: hit rates of the
+        embedding and the feature cache, rows pruned, rows and bytes read from the feature store, rows admitted
+        (the counts that the reference can log from its lookup, hiscache/history_cache.py:331-341).  The counters
+        live on the device and are read here only: this call synchronises, the lookups do not."""
         n = self.total_num_node
-        return {
+        c = dict(zip(_be.STAT_NAMES, (int(v) for v in self._counters.tolist())))
+        if self._uncounted_mask is not None:             # an update that no lookup has followed yet
+            c["rows_admitted"] += int(self._uncounted_mask.sum().item())
+        row_bytes = self.in_channels * self.uvm.buffer.element_size() if hasattr(self.uvm, "buffer") else 0
+        out = {
             "header": self.header,
             "overflow": self.overflow,
             "embed_cached": int((self.full2embed[:n] != -1).sum().item()),
             "feat_cached": int((self.full2embed[n:2 * n] != -1).sum().item()),
             "glb_iter": self.glb_iter,
         }
+        out.update(c)
+        out["embedding_hit_rate"] = c["embedding_hits"] / max(c["one_hop_nodes"], 1)
+        out["feature_hit_rate"] = c["feature_hits"] / max(c["nodes"], 1)
+        out["rows_not_loaded_rate"] = 1.0 - c["rows_loaded"] / max(c["nodes"], 1)    # the reference's "hit-rate"
+        out["bytes_from_feature_store"] = c["rows_loaded"] * row_bytes
+        return out
+
+    def reset_stats(self):
+        self._counters.zero_()
+        self._uncounted_mask = None

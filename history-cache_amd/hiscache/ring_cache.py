@@ -29,7 +29,7 @@ class RingHistoryCache:
 
     def __init__(self, uvm, total_num_node, in_channels, hidden_channels, capacity, num_layers,
                  table_dtype=torch.float16, rate=0.5, thres=None, age_limit=1 << 30, method="grad",
-                 device="cuda:0"):
+                 device="cuda:0", collect_stats=True):
         self.uvm = uvm
         self.total_num_node = int(total_num_node)
         self.in_channels = in_channels
@@ -53,6 +53,10 @@ class RingHistoryCache:
         self.cached_embedding = None
         self.used_masks = None
         self.last_record_mask = None
+        # what the lookups find (hiscache_backend.STAT_NAMES), counted on the device by one small launch per
+        # lookup and read by stats() only; collect_stats=False leaves the launch out
+        self._counters = torch.zeros(8, dtype=torch.int64, device=self.device) if collect_stats else None
+        self._uncounted_mask = None
 
     @property
     def header(self):
@@ -70,6 +74,9 @@ class RingHistoryCache:
             age_limit=self.age_limit)
         self.used_masks = _be.count_history_reconstruct(batch.ptr, batch.idx, self.sub2embed,
                                                         sub_to_full.shape[0], batch.y.shape[0], num_layer)
+        if self._counters is not None:
+            prev, self._uncounted_mask = self._uncounted_mask, None
+            _be.load_mask(self.used_masks[0], None, self.sub2embed, prev, self._counters)
         handle = getattr(batch, "prefetched_x", None)
         if handle is not None and handle.ids is sub_to_full:
             batch.prefetched_x = None
@@ -143,8 +150,27 @@ class RingHistoryCache:
                                      **common)
         emb.grad = None
         self.last_record_mask = mask
+        self._uncounted_mask = mask if self._counters is not None else None
         self.last_score = score
         self.produced_embedding = None
+
+    def stats(self):
+        """Table occupancy and what the lookups since construction found: embedding hit rate, rows pruned, rows
+        and bytes read from the feature store, rows admitted (the counts of the reference's lookup log,
+        /root/reference/hiscache/history_cache.py:331-341).  Synchronises; the lookups do not."""
+        out = {"header": self.header, "glb_iter": self.glb_iter,
+               "embed_cached": int((self.full2slot != -1).sum().item())}
+        if self._counters is None:
+            return out
+        c = dict(zip(_be.STAT_NAMES, (int(v) for v in self._counters.tolist())))
+        if self._uncounted_mask is not None:
+            c["rows_admitted"] += int(self._uncounted_mask.sum().item())
+        row_bytes = self.in_channels * self.uvm.buffer.element_size() if hasattr(self.uvm, "buffer") else 0
+        out.update(c)
+        out["embedding_hit_rate"] = c["embedding_hits"] / max(c["one_hop_nodes"], 1)
+        out["rows_not_loaded_rate"] = 1.0 - c["rows_loaded"] / max(c["nodes"], 1)
+        out["bytes_from_feature_store"] = c["rows_loaded"] * row_bytes
+        return out
 
     def preload(self, node_ids, rows=None):
         """Mark ``node_ids`` (unique int64 on the device) as cached in slots header.. (benchmark /

@@ -56,8 +56,8 @@ _SIGNATURES = {
     "hc_build_transpose": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p,
                                     _c_sz, _c_p]),
     "hc_transpose_dev_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
-    "hc_build_transpose_dev": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_sz,
-                                        _c_p]),
+    "hc_build_transpose_dev": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p,
+                                        _c_sz, _c_p]),
     "hc_aggr_bwd_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
     "hc_aggr_bwd_chunk_edges": (_c_i64, [_c_i64]),
     "hc_aggr_bwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_p,
@@ -66,6 +66,7 @@ _SIGNATURES = {
                                         _c_i64, _c_p, _c_sz, _c_p]),
     "hc_aggr_bwd_batch_view_typed": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_i64,
                                               _c_i64, _c_i64, _c_p]),
+    "hc_load_mask": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p]),
     "hc_count_history": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p]),
     "hc_row_scores": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_int, _c_p]),
     "hc_quantile_max_scores": (_c_i64, []),
@@ -824,7 +825,9 @@ _cu_stream_handles = []
 
 def _destroy_cu_streams():
     """At interpreter exit: wait for the device and give the CU-limited streams back while the HIP runtime is
-    still up (a stream of this kind left to the runtime's own teardown crashed a profiled run at exit)."""
+    still up (a stream of this kind left to the runtime's own teardown crashed a profiled run at exit: a
+    host-side crash in the process's teardown, after all results were out; no kernel was running).  Safe to
+    call any number of times: a handle is destroyed once."""
     if not _cu_stream_handles:
         return
     try:
@@ -833,7 +836,30 @@ def _destroy_cu_streams():
         pass
     lib = load_library()
     while _cu_stream_handles:
-        lib.hc_stream_destroy(_c_p(_cu_stream_handles.pop()))
+        handle = _cu_stream_handles.pop()
+        _forget_stream(handle)
+        lib.hc_stream_destroy(_c_p(handle))
+
+
+def _forget_stream(handle):
+    """Drop what this module keeps per stream (scratch buffer, epilogue ticket) for a stream that goes away."""
+    for table in (_ws_cache, _tickets):
+        for key in [k for k in table if k[1] == handle]:
+            del table[key]
+
+
+def release_cu_limited_stream(stream):
+    """Give a stream made by ``cu_limited_stream`` back before the interpreter exits: waits for its work,
+    destroys it and drops the scratch this module kept for it.  The torch wrapper must not be used afterwards.
+    Unknown or already released streams are ignored."""
+    handle = int(stream.cuda_stream)
+    if handle not in _cu_stream_handles:
+        return False
+    stream.synchronize()
+    _cu_stream_handles.remove(handle)
+    _forget_stream(handle)
+    load_library().hc_stream_destroy(_c_p(handle))
+    return True
 
 
 def cu_limited_stream(n_cus, device):
@@ -851,6 +877,46 @@ def cu_limited_stream(n_cus, device):
         atexit.register(_destroy_cu_streams)
     _cu_stream_handles.append(handle.value)
     return torch.cuda.ExternalStream(handle.value, device=device)
+
+
+STAT_NAMES = ("lookups", "nodes", "one_hop_nodes", "embedding_hits", "nodes_pruned", "feature_hits", "rows_loaded",
+              "rows_admitted")
+
+
+def load_mask(used, sub2feat=None, sub2embed=None, prev_mask=None, counters=None, want_masks=True):
+    """(hit_feat_mask, load_mask) of a batch -- ``load = used & ~(sub2feat != -1)``, the rows that have to come
+    from the feature store (/root/reference/hiscache/history_cache.py:327-330) -- in one launch that also adds the
+    batch's hit counts (and the rows admitted by ``prev_mask``) to ``counters`` (int64[8] on the device, order
+    ``STAT_NAMES``).  Without a feature cache (``sub2feat`` None) the load mask is ``used`` itself and only the
+    counters are touched: (None, used) is returned."""
+    lib = load_library()
+    _dev(used, "used")
+    if used.element_size() != 1:
+        raise ValueError("used must hold one byte per node")
+    n_all = used.numel()
+    n1 = 0 if sub2embed is None else _dev(sub2embed, "sub2embed", torch.int64).numel()
+    n_prev = 0
+    if prev_mask is not None:
+        _dev(prev_mask, "prev_mask")
+        if prev_mask.element_size() != 1:
+            raise ValueError("prev_mask must hold one byte per row")
+        n_prev = prev_mask.numel()
+    hit = load = None
+    if sub2feat is not None:
+        _dev(sub2feat, "sub2feat", torch.int64)
+        if sub2feat.numel() < n_all:
+            raise ValueError("sub2feat is shorter than used")
+        if want_masks:
+            hit = torch.empty(n_all, dtype=torch.bool, device=used.device)
+            load = torch.empty(n_all, dtype=torch.bool, device=used.device)
+    if counters is not None:
+        _dev(counters, "counters", torch.int64)
+        if counters.numel() < len(STAT_NAMES):
+            raise ValueError("counters must hold %d entries" % len(STAT_NAMES))
+    rc = lib.hc_load_mask(_ptr(used), _ptr(sub2feat), _ptr(sub2embed), _ptr(prev_mask), n_all, n1, n_prev,
+                          _ptr(hit), _ptr(load), _ptr(counters), _stream())
+    _check(rc, "hc_load_mask")
+    return hit, (load if sub2feat is not None else used)
 
 
 def fixup_rows(src, ids, need, have, out):
@@ -1147,10 +1213,13 @@ def sample_capacity(n_seed, fanout, num_nodes):
     return tuple(int(o.value) for o in out)
 
 
-def build_transpose_dev(ptr, idx, rows_dev, edges_dev, nodes_dev, max_edges, max_nodes, want_edges=False):
+def build_transpose_dev(ptr, idx, rows_dev, edges_dev, nodes_dev, max_edges, max_nodes, want_edges=False,
+                        overflow=None):
     """The transposed view of a block whose sizes are still on the device (one-element int64 views
     ``rows_dev``, ``edges_dev``, ``nodes_dev``, e.g. slices of the sampler's ``counts``): returns
-    (ptrT, rowT, edgeT) at the capacities ``max_nodes + 1`` / ``max_edges``; nothing is read back."""
+    (ptrT, rowT, edgeT) at the capacities ``max_nodes + 1`` / ``max_edges``; nothing is read back.
+    ``overflow`` (one int32 on the device, optional) is set to 1 when a size exceeded its capacity and the
+    view is that of the truncated block, else to 0."""
     lib = load_library()
     _dev(ptr, "ptr", torch.int64)
     _dev(idx, "idx", torch.int64)
@@ -1170,8 +1239,9 @@ def build_transpose_dev(ptr, idx, rows_dev, edges_dev, nodes_dev, max_edges, max
     edgeT = torch.empty(max(max_edges, 1), dtype=torch.int32, device=dev) if want_edges else None
     ws = _workspace(nbytes, dev)
     rc = lib.hc_build_transpose_dev(_ptr(ptr), _ptr(idx), _ptr(rows_dev), _ptr(edges_dev), _ptr(nodes_dev),
-                                    max_edges, max_nodes, _ptr(ptrT), _ptr(rowT), _ptr(edgeT), _ptr(ws),
-                                    ws.numel(), _stream())
+                                    max_edges, max_nodes, _ptr(ptrT), _ptr(rowT), _ptr(edgeT),
+                                    _ptr(None if overflow is None else _dev(overflow, "overflow", torch.int32)),
+                                    _ptr(ws), ws.numel(), _stream())
     _check(rc, "hc_build_transpose_dev")
     return ptrT, rowT, edgeT
 

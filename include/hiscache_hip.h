@@ -135,7 +135,13 @@ int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const int64_t *hm
  * max_E / max_src (the capacities of idx and of the node list, at most 2^24
  * each) size the launches, the workspace and the outputs: ptrT[max_src+1],
  * rowT[max_E], edgeT[max_E] (nullable).  Only ptrT[0..n_src] and the first
- * ptrT[n_src] entries of rowT/edgeT are written.  Four launches, kernels only
+ * ptrT[n_src] entries of rowT/edgeT are written.  Sizes beyond the capacities
+ * (*E_dev > max_E, *n_src_dev > max_src, or a negative size) are clamped, so
+ * that no access leaves idx or the outputs, and the view is then that of the
+ * truncated block (ptr must hold *R_dev + 1 offsets: the rows have no capacity
+ * argument): *overflow (one
+ * int32 in device memory, nullable) is set to 1 in that case and to 0
+ * otherwise, for the caller to check when it reads the sizes back.  Four launches, kernels only
  * (safe under stream capture), nothing is read back: this is how the sampler
  * emits the batch's transposed view together with the batch, so that backward
  * (hc_aggr_bwd_batch_view) builds none.  The loader of the reference hands over
@@ -145,7 +151,7 @@ size_t hc_transpose_dev_workspace_bytes(int64_t max_E, int64_t max_src);
 int hc_build_transpose_dev(const int64_t *ptr, const int64_t *idx, const int64_t *R_dev,
                            const int64_t *E_dev, const int64_t *n_src_dev, int64_t max_E,
                            int64_t max_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT,
-                           void *workspace, size_t workspace_bytes, void *stream);
+                           int32_t *overflow, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---------------------------------------------------------------- aggregation backward
  * Replaces AggrHistoryFunction::backward / AggrHistoryEdgeValueFunction::backward
@@ -504,6 +510,25 @@ int hc_fixup_rows(const void *src, int src_dtype, int64_t n_rows, const int64_t 
  * of lookup_and_load, hiscache/history_cache.py:310,315). */
 int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset, int64_t *out,
               int64_t n, void *stream);
+
+/* hc_load_mask: the rows of a batch that have to be read from the feature store,
+ * and the cache's hit counters, in one launch.  The reference spells the mask as
+ * load = used & ~(sub2feat != -1) with tensor operators
+ * (hiscache/history_cache.py:327-330) and can print the counts from a debug
+ * branch (:331-341); here they accumulate in device memory and are read only
+ * when the caller asks for them.
+ *   used[n_all]      bytes: row is still needed (used_masks[0] of hc_count_history)
+ *   sub2feat[n_all]  nullable: feature-cache slot per node, -1 = not cached
+ *   sub2embed[n1]    nullable: embedding slot per 1-hop node, -1 = not cached
+ *   prev_mask[n_prev] nullable: the admission mask of the previous update
+ *   hit_feat[n_all]  out, nullable: sub2feat[i] != -1
+ *   load_mask[n_all] out, nullable: used[i] && !hit_feat[i]
+ *   counters[8]      in/out, nullable, int64, += per call: [0] 1, [1] n_all, [2] n1,
+ *                    [3] embedding hits, [4] nodes pruned (!used), [5] feature-cache
+ *                    hits, [6] rows to load, [7] rows admitted by prev_mask. */
+int hc_load_mask(const uint8_t *used, const int64_t *sub2feat, const int64_t *sub2embed,
+                 const uint8_t *prev_mask, int64_t n_all, int64_t n1, int64_t n_prev,
+                 uint8_t *hit_feat, uint8_t *load_mask, int64_t *counters, void *stream);
 
 /* hc_ring_lookup: lookup of a ring table (full2slot / checkin / table as
  * hc_grad_check maintains them) for one batch, in one launch:

@@ -70,9 +70,9 @@ def test_argument_errors_are_status_codes():
     assert lib.hc_transpose_dev_workspace_bytes(big, 10) == 0 and lib.hc_transpose_dev_workspace_bytes(10, big) == 0
     need = lib.hc_transpose_dev_workspace_bytes(1000, 100)
     assert need >= 4 * 4 * 1000 + 4 * 101
-    assert lib.hc_build_transpose_dev(p, p, p, p, p, big, 10, p, p, null, p, 1 << 40, null) == 5
-    assert lib.hc_build_transpose_dev(p, p, p, p, p, 1000, 100, p, p, null, null, 0, null) == 4
-    assert lib.hc_build_transpose_dev(p, p, null, p, p, 1000, 100, p, p, null, p, need, null) == 1
+    assert lib.hc_build_transpose_dev(p, p, p, p, p, big, 10, p, p, null, null, p, 1 << 40, null) == 5
+    assert lib.hc_build_transpose_dev(p, p, p, p, p, 1000, 100, p, p, null, null, null, 0, null) == 4
+    assert lib.hc_build_transpose_dev(p, p, null, p, p, 1000, 100, p, p, null, null, p, need, null) == 1
     assert lib.hc_aggr_bwd_batch_view_typed(p, p, p, p, p, 8, 3, null, p, p, 4, 100, 4, null) == 5
     assert lib.hc_aggr_bwd_batch_view_typed(p, p, p, p, null, 8, 3, null, p, p, 4, 64, 4, null) == 1
     assert lib.hc_aggr_bwd_batch_view_typed(p, p, p, p, p, 8, 0, null, p, p, 4, 64, 4, null) == 1
@@ -253,3 +253,43 @@ def test_column_sums_by_matrix_vector_product():
     for n in (1, 7, 1024, 1025, 5000):
         g = torch.randn(n, 9, dtype=torch.float64)
         assert torch.allclose(hm._column_sums(g), g.sum(0), rtol=1e-12, atol=1e-12)
+
+
+def test_cu_limited_stream_teardown_is_idempotent(monkeypatch):
+    """The exit hook that gives CU-limited streams back destroys every handle once, drops the per-stream
+    scratch kept for it, survives a device that can no longer synchronise, and does nothing the second time;
+    releasing a stream by hand takes it off the hook's list."""
+    import hiscache_backend as be
+
+    destroyed = []
+
+    class Lib:
+        def hc_stream_destroy(self, handle):
+            destroyed.append(handle.value)
+            return 0
+
+    def no_device():
+        raise RuntimeError("no device")
+
+    monkeypatch.setattr(be, "load_library", lambda: Lib())
+    monkeypatch.setattr(be.torch.cuda, "synchronize", no_device)
+    monkeypatch.setattr(be, "_cu_stream_handles", [0x1000, 0x2000, 0x3000])
+    monkeypatch.setattr(be, "_ws_cache", {(0, 0x1000): "a", (0, 0x2000): "b", (0, 0): "default"})
+    monkeypatch.setattr(be, "_tickets", {(0, 0x2000): "t"})
+
+    class Stream:
+        cuda_stream = 0x2000
+        waited = 0
+
+        def synchronize(self):
+            Stream.waited += 1
+
+    assert be.release_cu_limited_stream(Stream()) is True
+    assert Stream.waited == 1 and destroyed == [0x2000]
+    assert be.release_cu_limited_stream(Stream()) is False          # already gone
+    assert (0, 0x2000) not in be._ws_cache and (0, 0x2000) not in be._tickets
+    be._destroy_cu_streams()
+    assert sorted(destroyed) == [0x1000, 0x2000, 0x3000] and be._cu_stream_handles == []
+    assert be._ws_cache == {(0, 0): "default"}
+    be._destroy_cu_streams()
+    assert len(destroyed) == 3

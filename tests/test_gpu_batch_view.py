@@ -153,13 +153,40 @@ def test_view_with_sizes_on_the_device(be, R, n_src, max_deg, hub_edges, slack):
     idx_cap = np.concatenate([idx, np.full(max_E - E, -7, np.int64)])     # capacity beyond the block: never read
     sizes = T(np.array([R, E, n_src], np.int64))
     want_ptrT, want_rowT, want_edgeT = _stable_view(ptr, idx, R, n_src)
+    flag = torch.full((1,), 7, dtype=torch.int32, device=DEV)
     for want_edges in (False, True):
         ptrT, rowT, edgeT = be.build_transpose_dev(T(ptr), T(idx_cap), sizes[0:1], sizes[1:2], sizes[2:3], max_E,
-                                                   max_src, want_edges=want_edges)
+                                                   max_src, want_edges=want_edges, overflow=flag)
         np.testing.assert_array_equal(ptrT[: n_src + 1].cpu().numpy(), want_ptrT)
         np.testing.assert_array_equal(rowT[:E].cpu().numpy(), want_rowT)
         if want_edges:
             np.testing.assert_array_equal(edgeT[:E].cpu().numpy(), want_edgeT)
+        assert int(flag) == 0
+
+
+def test_view_with_sizes_beyond_the_capacities_is_flagged(be):
+    """Sizes on the device that exceed what the launch was sized for are clamped (nothing is accessed out of
+    bounds) and the overflow word says so: the view is then that of the truncated block."""
+    rng = np.random.default_rng(5)
+    R, n_src, deg = 400, 300, 5
+    ptr = (np.arange(R + 1) * deg).astype(np.int64)
+    idx = rng.integers(0, n_src, size=R * deg, dtype=np.int64)
+    E = R * deg
+    flag = torch.zeros(1, dtype=torch.int32, device=DEV)
+    cut = 1200                                              # capacity for 1200 of the 2000 edge slots
+    sizes = T(np.array([R, E, n_src], np.int64))
+    ptrT, rowT, _ = be.build_transpose_dev(T(ptr), T(idx), sizes[0:1], sizes[1:2], sizes[2:3], cut, n_src,
+                                           overflow=flag)
+    assert int(flag) == 1
+    want_ptrT, want_rowT, _ = _stable_view(ptr[: cut // deg + 1], idx[:cut], cut // deg, n_src)
+    np.testing.assert_array_equal(ptrT.cpu().numpy(), want_ptrT)
+    np.testing.assert_array_equal(rowT[:cut].cpu().numpy(), want_rowT)
+    for bad in ([R, E, n_src + 50], [-1, E, n_src], [R, -3, n_src]):
+        flag.zero_()
+        be.build_transpose_dev(T(ptr), T(idx), *[T(np.array([v], np.int64)) for v in bad], E, n_src, overflow=flag)
+        assert int(flag) == 1, bad
+    be.build_transpose_dev(T(ptr), T(idx), sizes[0:1], sizes[1:2], sizes[2:3], E, n_src, overflow=flag)
+    assert int(flag) == 0
 
 
 @pytest.mark.parametrize("fanout,n_seed", [([5, 3], 64), ([15, 10, 5], 1200)])

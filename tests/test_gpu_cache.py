@@ -61,10 +61,19 @@ def test_lookup_update_cycles_match_model():
     from oracle import host_model
     rng, feats, cfg, cache, st = make_world(1)
     N, H = st.N, st.H
+    want = dict(lookups=0, nodes=0, one_hop_nodes=0, embedding_hits=0, nodes_pruned=0, feature_hits=0, rows_loaded=0,
+                rows_admitted=0)
     for it in range(1, 10):
         gpu, cpu = batch_pair(rng, N, 40, [6, 4, 3])
         cache.lookup_and_load(gpu, 3)
         ref = host_model.lookup_and_load(st, cpu, 3, feats)
+        want["lookups"] += 1
+        want["nodes"] += ref.sub2feat.numel()
+        want["one_hop_nodes"] += ref.sub2embed.numel()
+        want["embedding_hits"] += int((ref.sub2embed != -1).sum())
+        want["nodes_pruned"] += int((~ref.used_masks[0]).sum())
+        want["feature_hits"] += int((ref.sub2feat != -1).sum())
+        want["rows_loaded"] += int(ref.load_mask.sum())
         np.testing.assert_array_equal(cache.sub2embed.cpu().numpy(), ref.sub2embed.numpy())
         np.testing.assert_array_equal(cache.sub2feat.cpu().numpy(), ref.sub2feat.numpy())
         for a, b in zip(cache.used_masks, ref.used_masks):
@@ -84,6 +93,15 @@ def test_lookup_update_cycles_match_model():
         mask, _ = host_model.update_history(st, cpu.sub_to_full, ref.sub2embed, torch.from_numpy(emb), score,
                                             0.6, 4, it)
         np.testing.assert_array_equal(cache.last_record_mask.cpu().numpy(), mask.numpy())
+        want["rows_admitted"] += int(mask.sum())
+        if it in (4, 9):
+            # the counters of the lookups so far against the masks (the last admission has had no lookup behind it
+            # yet and is added by stats() itself)
+            got = cache.stats()
+            assert {k: got[k] for k in want} == want
+            assert got["embedding_hit_rate"] == want["embedding_hits"] / want["one_hop_nodes"]
+            assert got["feature_hit_rate"] == want["feature_hits"] / want["nodes"]
+            assert got["bytes_from_feature_store"] == want["rows_loaded"] * st.Fin * 4
         assert_state_equal(cache, st)
         n_emb = st.header
         np.testing.assert_array_equal(cache.buffer.view(-1, H)[:n_emb].cpu().numpy(),
@@ -534,6 +552,7 @@ def test_ring_cache_cycles_match_oracle():
         ref = dict(table=np.zeros((cap, H), np.uint16), f2s=np.full(N, -1, np.int64), s2f=np.full(cap, -1, np.int64),
                    checkin=np.full(cap, -1, np.int64), header=np.zeros(1, np.int64))
         n_stale = 0
+        stat = dict(admitted=0, hits=0, loaded=0, nodes=0)
         for it in range(1, 9):
             b = layered_batch(rng, N, 40, [6, 4, 3])
             batch = make_batch(b, rng.integers(0, 5, size=N), DEV)
@@ -548,6 +567,9 @@ def test_ring_cache_cycles_match_oracle():
             np.testing.assert_array_equal(cache.cached_embedding.cpu().numpy(), rows)
             used = orc.count_history_reconstruct(b["ptr"], b["idx"], slot, len(b["sub_to_full"]), 40, 3)
             np.testing.assert_array_equal(cache.used_masks[0].cpu().numpy(), used[0])
+            stat["hits"] += int((slot != -1).sum())
+            stat["loaded"] += int(used[0].sum())
+            stat["nodes"] += len(b["sub_to_full"])
             x_ref = feats[torch.from_numpy(b["sub_to_full"])].numpy() * used[0][:, None]
             np.testing.assert_array_equal(batch.x.cpu().numpy(), x_ref)
             emb = rng.standard_normal((n1, H)).astype(np.float32)
@@ -562,6 +584,7 @@ def test_ring_cache_cycles_match_oracle():
                                          ref["table"], orc.DT_F16, ref["f2s"], ref["s2f"], ref["checkin"],
                                          ref["header"], it)
             np.testing.assert_array_equal(cache.last_record_mask.cpu().numpy(), rmask)
+            stat["admitted"] += int(rmask.sum())
             np.testing.assert_array_equal(cache.full2slot.cpu().numpy(), ref["f2s"])
             np.testing.assert_array_equal(cache.slot2full.cpu().numpy(), ref["s2f"])
             np.testing.assert_array_equal(cache.checkin.cpu().numpy(), ref["checkin"])
@@ -570,6 +593,11 @@ def test_ring_cache_cycles_match_oracle():
             np.testing.assert_array_equal(cache.table.view(torch.int16).cpu().numpy().view(np.uint16)[live],
                                           ref["table"][live])
         assert (ref["s2f"] != -1).sum() > 0 and n_stale > 0
+        got = cache.stats()
+        assert got["lookups"] == 8 and got["embed_cached"] == int((ref["f2s"] != -1).sum())
+        assert got["rows_admitted"] == stat["admitted"] and got["embedding_hits"] == stat["hits"]
+        assert got["rows_loaded"] == stat["loaded"] and got["nodes_pruned"] == stat["nodes"] - stat["loaded"]
+        assert got["bytes_from_feature_store"] == stat["loaded"] * Fin * 4
 
 
 def test_ring_cache_refreshes_stale_entries_with_recomputed_values():
