@@ -41,7 +41,11 @@ HBM_PEAK_GBS = 8000.0
 AGE_LIMIT_ITERS = 100_000
 # the c3 / c5 training iterations that the default line reports beside the kernels' figures
 ITERATION_STEPS, ITERATION_WARMUP = 200, 20
-MEASURED_TRAFFIC = {"c2": 23.08e9, "c2row": 13.93e9, "c4": 3.48e9, "c3_batched": 51.94e9}
+# HBM bytes per launch by the counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 4 GiB copy), measured
+# with the library built from commit 6072fbd: profiles/aggr_c2_hbm_traffic.md, rows "C2 fwd_mean_fast" (c2),
+# "C4 gc_pass1 + gc_pass3_ring" (c4) and the three "batched layer" rows (c3_batched); c2row from the same
+# procedure over `--workload c2row` at commit 173ecbf (that kernel has not changed since).
+MEASURED_TRAFFIC = {"c2": 23.08e9, "c2row": 13.93e9, "c4": 3.49e9, "c3_batched": 51.97e9}
 
 
 def parse():
