@@ -1017,6 +1017,166 @@ __global__ __launch_bounds__(QT_BLOCK) void quantile_kernel(const float *__restr
   }
 }
 
+// ---- more scores than one block takes: the same select by the whole chip ------------------------
+// Four launches, one 8-bit digit each: every block replays the picks of the digits in front from the
+// histograms of the earlier launches (256 counters each, one wave), counts its share of the scores whose key
+// has that prefix in LDS and adds its 256 counts to the launch's histogram.  A lane keeps the count of the digit
+// it saw last in a register and touches LDS when the digit changes: the keys of gradient norms share their
+// leading digits, and a counter that every lane of a wave wants would serialise them.  A fifth launch finds
+// the smallest key above the selected one when the upper order statistic is another key, a sixth writes the
+// interpolation.  Workspace: QL_WORDS 32-bit words, cleared by a launch in front.
+constexpr int QL_BLOCK = 1024;
+constexpr int QL_MAX_BLOCKS = 256;    // every block ends with one atomic per counter: those on one address queue up
+constexpr int QL_NAN = 4 * 256;       // workspace word: number of NaN scores
+constexpr int QL_NEXT = 4 * 256 + 1;  // workspace word: smallest key above the selected one
+constexpr int QL_WORDS = 4 * 256 + 2;
+constexpr int64_t QL_FROM_N = 1 << 15;   // fewer scores go to the one block: its passes cost less than seven launches
+
+struct QlPick {
+  uint32_t prefix;    // the digits picked so far, in place
+  int64_t k;          // the rank among the keys with that prefix
+  uint32_t n_equal;   // how many keys have that prefix
+};
+
+// By one whole wave: the first `passes` digits of the key of rank k, from the launches' histograms.
+__device__ QlPick ql_replay(const uint32_t *__restrict__ hist, int passes, int64_t k, int lane) {
+  QlPick r{0u, k, 0u};
+  for (int p = 0; p < passes; ++p) {
+    const uint32_t *h = hist + p * 256;
+    const uint32_t c[4] = {h[4 * lane], h[4 * lane + 1], h[4 * lane + 2], h[4 * lane + 3]};
+    const long long mine = ((long long)c[0] + c[1]) + ((long long)c[2] + c[3]);
+    long long x = mine;
+#pragma unroll
+    for (int d = 1; d < HC_WAVE; d <<= 1) {
+      const long long y = __shfl_up(x, d, HC_WAVE);
+      if (lane >= d) x += y;
+    }
+    const unsigned long long reached = __ballot(x > (long long)r.k);
+    const int owner = reached != 0ull ? __builtin_ctzll(reached) : HC_WAVE - 1;
+    long long before = x - mine;
+    int b = 0;
+    for (; b < 3; ++b) {
+      if (before + (long long)c[b] > (long long)r.k) break;
+      before += c[b];
+    }
+    const int bin = __shfl(4 * lane + b, owner, HC_WAVE);
+    const long long front = __shfl(before, owner, HC_WAVE);
+    const uint32_t inside = (uint32_t)__shfl((int)c[b], owner, HC_WAVE);
+    r.prefix |= (uint32_t)bin << (24 - 8 * p);
+    r.k -= front;
+    r.n_equal = inside;
+  }
+  return r;
+}
+
+__global__ void ql_clear(uint32_t *__restrict__ ws) {
+  for (int i = threadIdx.x; i < QL_WORDS; i += blockDim.x) ws[i] = i == QL_NEXT ? 0xffffffffu : 0u;
+}
+
+// Calls f(key) for this thread's share of the scores.  VEC4 (score 16-byte aligned): four scores per load and
+// two loads in flight; the last n % 4 scores go to the first threads of block 0.
+template <bool VEC4, typename Fn>
+__device__ __forceinline__ void ql_for_each_key(const float *__restrict__ score, int64_t n, Fn f) {
+  const int64_t stride = (int64_t)gridDim.x * QL_BLOCK;
+  const int64_t t = (int64_t)blockIdx.x * QL_BLOCK + threadIdx.x;
+  if constexpr (VEC4) {
+    const float4 *__restrict__ s4 = reinterpret_cast<const float4 *>(score);
+    const int64_t n4 = n >> 2;
+    for (int64_t i = t; i < n4; i += 2 * stride) {
+      const float4 a = s4[i];
+      const bool two = i + stride < n4;
+      const float4 b = two ? s4[i + stride] : a;
+      f(qt_key(a.x)); f(qt_key(a.y)); f(qt_key(a.z)); f(qt_key(a.w));
+      if (two) { f(qt_key(b.x)); f(qt_key(b.y)); f(qt_key(b.z)); f(qt_key(b.w)); }
+    }
+    if (t < (n & 3)) f(qt_key(score[(n4 << 2) + t]));
+  } else {
+    for (int64_t i = t; i < n; i += stride) f(qt_key(score[i]));
+  }
+}
+
+template <int PASS, bool VEC4>
+__global__ __launch_bounds__(QL_BLOCK) void ql_pass(const float *__restrict__ score, int64_t n, int64_t k,
+                                                     uint32_t *__restrict__ ws) {
+  __shared__ uint32_t lh[256];
+  __shared__ uint32_t s_prefix;
+  if (threadIdx.x < HC_WAVE) {
+    const QlPick pk = ql_replay(ws, PASS, k, (int)threadIdx.x);
+    if (threadIdx.x == 0) s_prefix = pk.prefix;
+  }
+  if (threadIdx.x < 256) lh[threadIdx.x] = 0u;
+  __syncthreads();
+  const uint32_t prefix = s_prefix;
+  constexpr int shift = 24 - 8 * PASS;
+  constexpr uint32_t mask = PASS == 0 ? 0u : 0xffffffffu << (shift + 8);
+  uint32_t cur = 0u, cnt = 0u, nan = 0u;
+  ql_for_each_key<VEC4>(score, n, [&](uint32_t key) {
+    if (PASS == 0 && key == 0xffffffffu) ++nan;
+    if ((key & mask) == prefix) {
+      const uint32_t d = (key >> shift) & 0xffu;
+      if (d != cur) {
+        if (cnt) atomicAdd(&lh[cur], cnt);
+        cur = d;
+        cnt = 0u;
+      }
+      ++cnt;
+    }
+  });
+  if (cnt) atomicAdd(&lh[cur], cnt);
+  if (PASS == 0 && nan) atomicAdd(&ws[QL_NAN], nan);
+  __syncthreads();
+  if (threadIdx.x < 256) {
+    const uint32_t v = lh[threadIdx.x];
+    if (v) atomicAdd(&ws[PASS * 256 + threadIdx.x], v);
+  }
+}
+
+// The smallest key above the one of rank lo, when rank hi is not among the keys equal to it.
+template <bool VEC4>
+__global__ __launch_bounds__(QL_BLOCK) void ql_next(const float *__restrict__ score, int64_t n, int64_t lo,
+                                                     int64_t hi, uint32_t *__restrict__ ws) {
+  __shared__ uint32_t s_key, s_min;
+  __shared__ int s_need;
+  if (threadIdx.x < HC_WAVE) {
+    const QlPick pk = ql_replay(ws, 4, lo, (int)threadIdx.x);
+    if (threadIdx.x == 0) {
+      s_key = pk.prefix;
+      s_min = 0xffffffffu;
+      s_need = hi != lo && pk.k + 1 >= (int64_t)pk.n_equal;
+    }
+  }
+  __syncthreads();
+  if (!s_need) return;                  // block-uniform
+  const uint32_t key = s_key;
+  uint32_t m = 0xffffffffu;
+  ql_for_each_key<VEC4>(score, n, [&](uint32_t x) {
+    if (x > key && x < m) m = x;
+  });
+#pragma unroll
+  for (int d = HC_WAVE / 2; d > 0; d >>= 1) {
+    const uint32_t y = (uint32_t)__shfl_xor((int)m, d, HC_WAVE);
+    m = y < m ? y : m;
+  }
+  if (hc_lane() == 0 && m != 0xffffffffu) atomicMin(&s_min, m);
+  __syncthreads();
+  if (threadIdx.x == 0 && s_min != 0xffffffffu) atomicMin(&ws[QL_NEXT], s_min);
+}
+
+__global__ __launch_bounds__(HC_WAVE) void ql_final(int64_t lo, int64_t hi, float w, float one_minus_w,
+                                                     const uint32_t *__restrict__ ws, float *__restrict__ out) {
+  const QlPick pk = ql_replay(ws, 4, lo, (int)threadIdx.x);
+  if (threadIdx.x != 0) return;
+  if (ws[QL_NAN] != 0u) {
+    out[0] = __uint_as_float(0x7fc00000u);
+    return;
+  }
+  const uint32_t ka = pk.prefix;
+  const uint32_t kb = (hi != lo && pk.k + 1 >= (int64_t)pk.n_equal) ? ws[QL_NEXT] : ka;
+  const float a = qt_value(ka), b = qt_value(kb);
+  const float d = __fsub_rn(b, a);
+  out[0] = w < 0.5f ? __fadd_rn(a, __fmul_rn(d, w)) : __fsub_rn(b, __fmul_rn(d, one_minus_w));
+}
+
 }  // namespace
 
 extern "C" int64_t hc_quantile_max_scores(void) { return QT_MAX_N; }
@@ -1030,5 +1190,39 @@ extern "C" int hc_quantile_threshold(const float *score, int64_t n, int64_t lo, 
     quantile_kernel<true><<<dim3(1), dim3(QT_BLOCK), 0, st>>>(score, n, lo, hi, w, one_minus_w, out);
   else
     quantile_kernel<false><<<dim3(1), dim3(QT_BLOCK), 0, st>>>(score, n, lo, hi, w, one_minus_w, out);
+  return hc_launch_status();
+}
+
+extern "C" size_t hc_quantile_workspace_bytes(int64_t n) {
+  return n > QL_FROM_N ? (size_t)QL_WORDS * sizeof(uint32_t) : 0;
+}
+
+extern "C" int hc_quantile_threshold_ws(const float *score, int64_t n, int64_t lo, int64_t hi, float w,
+                                        float one_minus_w, float *out, void *workspace, size_t workspace_bytes,
+                                        void *stream) {
+  if (n <= QL_FROM_N) return hc_quantile_threshold(score, n, lo, hi, w, one_minus_w, out, stream);
+  HC_REQUIRE(score && out && lo >= 0 && hi >= lo && hi < n && hi <= lo + 1 && n <= (int64_t)0x7fffffff);
+  HC_REQUIRE(workspace && workspace_bytes >= hc_quantile_workspace_bytes(n) &&
+             (reinterpret_cast<uintptr_t>(workspace) & 3u) == 0);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint32_t *ws = static_cast<uint32_t *>(workspace);
+  int64_t blocks = (n + (int64_t)QL_BLOCK * 8 - 1) / ((int64_t)QL_BLOCK * 8);
+  if (blocks > QL_MAX_BLOCKS) blocks = QL_MAX_BLOCKS;
+  const dim3 grid((unsigned)blocks), block(QL_BLOCK);
+  ql_clear<<<dim3(1), dim3(256), 0, st>>>(ws);
+  if ((reinterpret_cast<uintptr_t>(score) & 15u) == 0) {
+    ql_pass<0, true><<<grid, block, 0, st>>>(score, n, lo, ws);
+    ql_pass<1, true><<<grid, block, 0, st>>>(score, n, lo, ws);
+    ql_pass<2, true><<<grid, block, 0, st>>>(score, n, lo, ws);
+    ql_pass<3, true><<<grid, block, 0, st>>>(score, n, lo, ws);
+    ql_next<true><<<grid, block, 0, st>>>(score, n, lo, hi, ws);
+  } else {
+    ql_pass<0, false><<<grid, block, 0, st>>>(score, n, lo, ws);
+    ql_pass<1, false><<<grid, block, 0, st>>>(score, n, lo, ws);
+    ql_pass<2, false><<<grid, block, 0, st>>>(score, n, lo, ws);
+    ql_pass<3, false><<<grid, block, 0, st>>>(score, n, lo, ws);
+    ql_next<false><<<grid, block, 0, st>>>(score, n, lo, hi, ws);
+  }
+  ql_final<<<dim3(1), dim3(HC_WAVE), 0, st>>>(lo, hi, w, one_minus_w, ws, out);
   return hc_launch_status();
 }

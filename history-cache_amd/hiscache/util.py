@@ -61,15 +61,14 @@ def quantile_threshold(score, rate):
     hi = min(lo + 1, n - 1)
     w = (pos - torch.tensor(float(lo), dtype=torch.float32)).item()
     if score.is_cuda:
-        # on the GPU: the two order statistics by a radix select and the interpolation, one launch
+        # on the GPU: the two order statistics by a radix select and the interpolation, no sort
         import hiscache_backend
         flat = score.detach().reshape(-1)
         if flat.dtype != torch.float32 or not flat.is_contiguous():
             flat = flat.to(torch.float32).contiguous()
         one_minus_w = (1.0 - torch.tensor(w, dtype=torch.float32)).item()
-        got = hiscache_backend.quantile_select(flat, lo, hi, w, one_minus_w)
-        if got is not None:
-            return got
+        return hiscache_backend.quantile_select(flat, lo, hi, w, one_minus_w)
+    # host tensors (the CPU tests' spelling of the same rule)
     flat = score.detach().reshape(-1).to(torch.float32)
     srt = torch.sort(flat).values
     a = srt[lo:lo + 1]

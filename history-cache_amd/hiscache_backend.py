@@ -71,6 +71,9 @@ _SIGNATURES = {
     "hc_row_scores": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_int, _c_p]),
     "hc_quantile_max_scores": (_c_i64, []),
     "hc_quantile_threshold": (_c_int, [_c_p, _c_i64, _c_i64, _c_i64, ctypes.c_float, ctypes.c_float, _c_p, _c_p]),
+    "hc_quantile_workspace_bytes": (_c_sz, [_c_i64]),
+    "hc_quantile_threshold_ws": (_c_int, [_c_p, _c_i64, _c_i64, _c_i64, ctypes.c_float, ctypes.c_float, _c_p, _c_p,
+                                          _c_sz, _c_p]),
     "hc_grad_check_workspace_bytes": (_c_sz, [_c_i64]),
     "hc_grad_check": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, ctypes.c_int32, _c_int,
                                _c_int, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_p,
@@ -659,24 +662,21 @@ def row_scores(grad, norm_kind=NORM_L2):
     return out
 
 
-_quantile_max = None
 
 
 def quantile_select(score, lo, hi, w, one_minus_w):
     """a + w*(b - a) (w < 0.5) or b - (b - a)*one_minus_w over the order statistics a, b of rank lo, hi of
-    ``score`` (fp32 on the GPU), every step rounded to fp32: one launch, no sort.  Returns a 1-element
-    tensor, or None when there are more scores than the kernel takes (the caller sorts instead)."""
-    global _quantile_max
+    ``score`` (fp32 on the GPU), every step rounded to fp32, by a radix select instead of a sort: one launch
+    by one block for the few thousand scores of a sampled batch, seven small launches over the whole chip for
+    more than 32 768.  Returns a 1-element tensor."""
     lib = load_library()
-    if _quantile_max is None:
-        _quantile_max = int(lib.hc_quantile_max_scores())
     score = _dev(score, "score", torch.float32)
     n = score.numel()
-    if n > _quantile_max:
-        return None
     out = torch.empty(1, dtype=torch.float32, device=score.device)
-    _check(lib.hc_quantile_threshold(_ptr(score), n, int(lo), int(hi), float(w), float(one_minus_w), _ptr(out),
-                                     _stream()), "hc_quantile_threshold")
+    nbytes = int(lib.hc_quantile_workspace_bytes(n))      # 0 when one block takes them all
+    ws = _workspace(nbytes, score.device)
+    _check(lib.hc_quantile_threshold_ws(_ptr(score), n, int(lo), int(hi), float(w), float(one_minus_w), _ptr(out),
+                                        _ptr(ws), ws.numel(), _stream()), "hc_quantile_threshold_ws")
     return out
 
 

@@ -263,11 +263,20 @@ int hc_row_scores(const float *grad, float *score, int64_t M, int64_t F, int nor
  * caller works out lo, hi and w from rate and n the way torch.quantile does
  * (pos = fp32(rate) * fp32(n - 1), lo = floor(pos), w = pos - lo).  One launch
  * (a radix select by one block); n <= hc_quantile_max_scores(), else
- * HC_EUNSUPPORTED (sort instead).  NaN scores rank behind +inf, as in a sort;
+ * HC_EUNSUPPORTED (hc_quantile_threshold_ws takes any size).  NaN scores rank behind +inf, as in a sort;
  * -0 ranks in front of +0. */
 int64_t hc_quantile_max_scores(void);
 int hc_quantile_threshold(const float *score, int64_t n, int64_t lo, int64_t hi, float w,
                           float one_minus_w, float *out, void *stream);
+/* The same threshold for any n < 2^31.  Up to 32 768 scores it is
+ * hc_quantile_threshold and needs no workspace; above, the select runs over the
+ * whole chip in seven small launches (a clear, one launch per 8-bit digit of the
+ * key, one for the upper order statistic, one for the interpolation) and needs
+ * hc_quantile_workspace_bytes(n) bytes, 4-byte aligned.  Same bits either way. */
+size_t hc_quantile_workspace_bytes(int64_t n);
+int hc_quantile_threshold_ws(const float *score, int64_t n, int64_t lo, int64_t hi, float w,
+                             float one_minus_w, float *out, void *workspace, size_t workspace_bytes,
+                             void *stream);
 
 /* hc_grad_check: the fused admission pass.  Replaces record_history
  * (grad_check.h:12-16, grad_check.cu:6-68) and the torch sequence of
