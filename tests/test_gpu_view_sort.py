@@ -89,3 +89,51 @@ def test_bucket_sorted_view_is_the_stable_sort(be, R, N, deg, empty, hub_row, po
                 np.testing.assert_array_equal(rowT.cpu().numpy()[:n], rows)
                 if want_edges:
                     np.testing.assert_array_equal(edgeT.cpu().numpy()[:n], order)
+
+
+def _even_ptr(R, E):
+    deg = np.full(R, E // R, np.int64)
+    deg[: E - (E // R) * R] += 1
+    ptr = np.zeros(R + 1, np.int64)
+    np.cumsum(deg, out=ptr[1:])
+    return ptr
+
+
+def _adversarial_blocks():
+    """(name, ptr, idx, N, row map, source map): blocks that put every edge into one bucket, leave none alive,
+    end exactly on a tile, consist of one row, repeat one id across a wave, or have as many sources as the
+    bucket sort takes (and one more, which goes to the library sort)."""
+    rng = np.random.default_rng(17)
+    R = 100_000
+    E = 8192 * 129                                         # a whole number of tiles of 8 192 edge slots
+    ptr = _even_ptr(R, E)
+    ar = np.arange(E, dtype=np.int64)
+    yield "one_source_takes_all", ptr, np.full(E, 7, np.int64), 1000, None, None
+    yield "a_single_source", ptr, np.zeros(E, np.int64), 1, None, None
+    yield "every_source_flagged", ptr, rng.integers(0, 50_000, size=E), 50_000, None, np.ones(50_000, np.int64)
+    yield "every_row_flagged", ptr, rng.integers(0, 50_000, size=E), 50_000, np.ones(R, np.int64), None
+    yield "one_row", np.array([0, E + 1], np.int64), rng.integers(0, 70_000, size=E + 1), 70_000, None, None
+    yield "one_id_per_wave", ptr, (ar // 64) % 3_000_000, 3_000_000, None, None
+    yield "two_ids_per_wave", ptr, (ar // 64) * 2 % 3_000_000 + (ar & 1), 3_000_000, None, None
+    yield "two_far_ids", ptr, (ar & 1) * 2_999_999, 3_000_000, None, None
+    yield "descending", ptr, 2_999_999 - (ar * 3_000_000) // E, 3_000_000, None, None
+    for N in (5376 * 8192 - 1, 5376 * 8192 + 1):
+        hs = np.where(rng.random(N) < 0.3, 1, -1).astype(np.int64)
+        yield "most_sources_%d" % N, ptr, rng.integers(0, N, size=E), N, np.where(rng.random(R) < 0.2, 3, -1), hs
+
+
+def test_bucket_sorted_view_on_adversarial_blocks(be):
+    for name, ptr, idx, N, hrow, hsrc in _adversarial_blocks():
+        R = len(ptr) - 1
+        idx = np.ascontiguousarray(idx, np.int64)
+        hrow = None if hrow is None else np.ascontiguousarray(hrow, np.int64)
+        want_ptrT, order, rows = stable_view(ptr, idx, R, N, len(idx), hrow, hsrc)
+        n = len(order)
+        for want_edges in (False, True):
+            ptrT, rowT, edgeT = be.build_transpose(T(ptr), T(idx), None if hrow is None else T(hrow), R, N,
+                                                   want_edges=want_edges,
+                                                   history_map_src=None if hsrc is None else T(hsrc))
+            np.testing.assert_array_equal(ptrT.cpu().numpy(), want_ptrT, err_msg=name)
+            np.testing.assert_array_equal(rowT.cpu().numpy()[:n], rows, err_msg=name)
+            if want_edges:
+                np.testing.assert_array_equal(edgeT.cpu().numpy()[:n], order, err_msg=name)
