@@ -226,3 +226,30 @@ def test_quantile_threshold_by_selection_equals_the_sort(n):
             ref = torch.quantile(torch.from_numpy(s32), rate).numpy()
             assert np.isnan(got[0]) and np.isnan(want[0]) and np.isnan(ref), f"n={n} rate={rate}"
             assert int((dev < torch.from_numpy(got).to(DEV)).sum()) == 0
+
+
+def test_quantile_entry_points_state_their_limits():
+    """The one-block entry point refuses more scores than hc_quantile_max_scores() with HC_EUNSUPPORTED and
+    launches nothing; the workspace variant refuses a workspace that is too small."""
+    import hiscache_backend as be
+    lib = be.load_library()
+    limit = int(lib.hc_quantile_max_scores())
+    assert limit == 1 << 17
+    score = torch.rand(limit + 1, device=DEV)
+    out = torch.full((1,), -7.0, device=DEV)
+    rc = lib.hc_quantile_threshold(be._ptr(score), limit + 1, 3, 4, 0.25, 0.75, be._ptr(out), be._stream())
+    assert rc == 5                                   # HC_EUNSUPPORTED
+    need = int(lib.hc_quantile_workspace_bytes(limit + 1))
+    assert need > 0 and int(lib.hc_quantile_workspace_bytes(1000)) == 0
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    rc = lib.hc_quantile_threshold_ws(be._ptr(score), limit + 1, 3, 4, 0.25, 0.75, be._ptr(out), be._ptr(ws), need - 1,
+                                      be._stream())
+    assert rc != 0
+    torch.cuda.synchronize()
+    assert float(out) == -7.0
+    rc = lib.hc_quantile_threshold_ws(be._ptr(score), limit + 1, 3, 4, 0.25, 0.75, be._ptr(out), be._ptr(ws), need,
+                                      be._stream())
+    assert rc == 0
+    srt = torch.sort(score).values
+    want = srt[3] + (srt[4] - srt[3]) * 0.25
+    assert float(out) == float(want)
