@@ -2,10 +2,11 @@
 
 TEST INFRASTRUCTURE ONLY (see hc_oracle.c).  Statement by statement it follows
 ``HistoryCache.update_history`` / ``lookup_and_load``
-(/root/reference/hiscache/history_cache.py:180-255, 275-356) and the eviction rules of
-``HistoryTable`` (/root/reference/hiscache/history_table.py:189-251), on CPU tensors, with the
+(/root/reference/hiscache/history_cache.py:180-255, 275-356) and the lookup and eviction rules of
+``HistoryTable`` (/root/reference/hiscache/history_table.py:94-125, 189-251), on CPU tensors, with the
 kernel calls replaced by the C oracle.  State lives in a plain object so tests can compare every
-tensor with the GPU implementation.
+tensor with the GPU implementation.  Pinned by vectors that the reference's own code produced
+(tests/golden: the cache's two entry points, the table's lookup and evictions).
 """
 import math
 from types import SimpleNamespace
@@ -117,6 +118,19 @@ def update_history(st, sub_to_full, sub2embed, produced_embedding, score, rate, 
     st.embed2full[st.header:st.header + num_to_record] = change_id
     st.header += num_to_record
     return record_mask, thres
+
+
+def table_lookup(full_to_history, history_buffer, sub_to_full, num_node, num_seed):
+    """history_table.py:100-125 for one layer: the slot of each of the first ``num_node`` sub-graph nodes
+    (-1 for the seeds and for nodes without an entry), the rows of the hits in node order, and the compact
+    ids [-1, 0, -1, 1, ...] that point into those rows."""
+    sub_to_history = full_to_history[sub_to_full[:num_node]].clone()
+    sub_to_history[:num_seed] = -1
+    mask = sub_to_history != -1
+    rows = history_buffer[sub_to_history[mask]]
+    compact = torch.full((num_node,), -1, dtype=torch.int64)
+    compact[mask] = torch.arange(int(mask.sum()))
+    return sub_to_history, rows, compact
 
 
 def evict_by_staleness(checkin, history_to_full, full_to_history, glb_iter, staleness_thres):

@@ -78,6 +78,21 @@ def exact_rows(seed, n, width, octaves=13):
     return (value * scale[:, None]).astype(np.float32)
 
 
+def exact_sum_rows(seed, n, width, octaves=9):
+    """[n, width] float32 whose row sums (of the values, of their magnitudes) are exact in fp32 in ANY order
+    of summation: entry = q * 2^-(10 + k) with an integer |q| <= 4096 from a hash and a per-row k < octaves,
+    so a row's partial sums are integers below 2^24 in units of 2^-(10 + k).  Scores built from such rows do
+    not depend on how a library folds a row."""
+    cell = np.arange(n * width, dtype=np.uint64).reshape(n, width)
+    with np.errstate(over="ignore"):
+        h = _splitmix64(cell * np.uint64(2) + np.uint64(seed) * np.uint64(0x100000001B3))
+        hr = _splitmix64(np.arange(n, dtype=np.uint64) * np.uint64(2) + np.uint64(1)
+                         + np.uint64(seed) * np.uint64(0x100000001B3))
+    q = (h & np.uint64(0x1FFF)).astype(np.int64) - 4096
+    k = (hr % np.uint64(octaves)).astype(np.int64)
+    return np.ldexp(q.astype(np.float64), -(10 + k)[:, None]).astype(np.float32)
+
+
 def affine_ids(n_full, count, a, b):
     """`count` distinct node ids (a * i + b) mod n_full; a must be coprime with n_full."""
     assert np.gcd(a, n_full) == 1 and count <= n_full
