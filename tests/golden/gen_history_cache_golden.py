@@ -4,7 +4,7 @@
 
 Run in the build container only (the reference tree is not available elsewhere):
 
-    python tests/golden/gen_history_cache_golden.py
+    python tests/golden/gen_history_cache_golden.py          (every fixture; `... fill` the constructor's only)
 
 The reference module's SOURCE TEXT is read from /root/reference, compiled and executed here (no
 importlib loader: a loader would prefer a ``__pycache__/*.pyc`` lying beside the source, and would
@@ -223,7 +223,72 @@ def main_wide(suffix):
           "bytes:", os.path.getsize(path))
 
 
+# ---- the constructor: allocate() and fill() -------------------------------------------------------------
+# HistoryCache.__init__ -> allocate() -> fill() (history_cache.py:12-62, 95-178) run as they are, on the CPU,
+# from dataset files written here (num_nodes.txt, sorted_indices.dat).  allocate() asks the CUDA runtime for the
+# free device memory; there is none here, so that one query answers 64 GiB for the duration of the call (the
+# limit in the configuration then decides the size, as in every run of the reference with a limit).  The buffer
+# that allocate() makes is uninitialised: only the rows that fill() writes are kept.
+FILL_CASES = {
+    "part": dict(N=1500, Fin=8, H=12, limit_gb=1e-5, seed=41),       # room for 336 feature rows of 1500
+    "all": dict(N=200, Fin=8, H=12, limit_gb=1e-5, seed=42),         # room for more rows than there are nodes
+    "wide": dict(N=3000, Fin=16, H=24, limit_gb=1e-4, seed=43),
+}
+
+
+def fill_inputs(c):
+    """(features, node ids sorted coldest to hottest) of a fill case, rebuilt from its seed."""
+    from helpers import exact_rows
+    feats = exact_rows(c["seed"], c["N"], c["Fin"], octaves=2)
+    hot = np.random.default_rng(c["seed"]).permutation(c["N"]).astype(np.int64)
+    return feats, hot
+
+
+def main_fill():
+    import tempfile
+    sys.path.insert(0, os.path.join(ROOT, "history-cache_amd"))
+    from hiscache.util import make_config
+    HistoryCache = load_reference_class()
+    out = {}
+    probe = torch.cuda.mem_get_info
+    torch.cuda.mem_get_info = lambda *a, **k: (64 << 30, 64 << 30)
+    try:
+        for name, c in FILL_CASES.items():
+            feats, hot = fill_inputs(c)
+            with tempfile.TemporaryDirectory() as root:
+                os.makedirs(os.path.join(root, "processed"))
+                with open(os.path.join(root, "processed", "num_nodes.txt"), "w") as f:
+                    f.write("%d\n" % c["N"])
+                hot.tofile(os.path.join(root, "processed", "sorted_indices.dat"))
+                cfg = make_config(c["Fin"], 5, c["H"], 2, method="grad", rate=0.5, staleness_thres=4,
+                                  limit=c["limit_gb"], device="cpu", path=root)
+                cache = HistoryCache(Store(torch.from_numpy(feats)), cfg, "history_uvm")
+            n_cached = min(cache.overall_feat_num, c["N"])
+            pre = name + "_"
+            out[pre + "hot"] = hot
+            out[pre + "max_buffer_byte"] = np.int64(cache.max_buffer_byte)
+            out[pre + "overall_feat_num"] = np.int64(cache.overall_feat_num)
+            out[pre + "overall_embed_num"] = np.int64(cache.overall_embed_num)
+            out[pre + "buffer_floats"] = np.int64(cache.buffer.shape[0])
+            out[pre + "feat2full"] = cache.feat2full.numpy().copy()
+            out[pre + "full2embed"] = cache.full2embed.numpy().copy()
+            out[pre + "embed2full"] = cache.embed2full.numpy().copy()
+            out[pre + "feature_rows"] = cache.buffer.view(-1, c["Fin"])[-n_cached:].numpy().copy()
+            out[pre + "header"] = np.int64(cache.header)
+            print(name, "buffer floats", cache.buffer.shape[0], "feature slots", cache.overall_feat_num,
+                  "cached", n_cached)
+    finally:
+        torch.cuda.mem_get_info = probe
+    path = os.path.join(HERE, "history_cache_fill_golden.npz")
+    np.savez_compressed(path, **out)
+    print("wrote", path, os.path.getsize(path), "bytes")
+
+
 if __name__ == "__main__":
-    main()
-    for suffix in WIDE_CASES:
-        main_wide(suffix)
+    if sys.argv[1:] == ["fill"]:
+        main_fill()
+    else:
+        main()
+        for suffix in WIDE_CASES:
+            main_wide(suffix)
+        main_fill()

@@ -183,3 +183,73 @@ def test_gpu_cache_reproduces_reference_vectors_at_real_width(hidden):
         check_wide_iteration(g, it, cache.last_record_mask.cpu().numpy().astype(bool), cache.last_score.cpu().numpy(),
                              cache.header, cache.full2embed.cpu().numpy(), cache.embed2full.cpu().numpy(),
                              cache.buffer.cpu().numpy())
+
+
+# ---- the constructor: allocate() and fill() as the reference ran them ---------------------------------------
+FILL = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "history_cache_fill_golden.npz")
+FILL_CASES = {                      # tests/golden/gen_history_cache_golden.py:FILL_CASES
+    "part": dict(N=1500, Fin=8, H=12, limit_gb=1e-5, seed=41),
+    "all": dict(N=200, Fin=8, H=12, limit_gb=1e-5, seed=42),
+    "wide": dict(N=3000, Fin=16, H=24, limit_gb=1e-4, seed=43),
+}
+
+
+def fill_inputs(c, g, name):
+    from helpers import exact_rows
+    feats = exact_rows(c["seed"], c["N"], c["Fin"], octaves=2)
+    hot = np.random.default_rng(c["seed"]).permutation(c["N"]).astype(np.int64)
+    np.testing.assert_array_equal(hot, g[name + "_hot"], err_msg="the case's inputs are not the fixture's")
+    return feats, hot
+
+
+def check_fill(name, g, N, Fin, buffer_floats, feat2full, full2embed, embed2full, buffer, header):
+    """The reference keeps only the cached block in feat2full; here it is slot-indexed with -1 in the empty
+    slots in front, so its tail is compared."""
+    pre = name + "_"
+    n_cached = len(g[pre + "feat2full"])
+    assert buffer_floats == int(g[pre + "buffer_floats"])
+    np.testing.assert_array_equal(feat2full[-n_cached:], g[pre + "feat2full"])
+    assert (feat2full[:-n_cached] == -1).all()
+    np.testing.assert_array_equal(full2embed, g[pre + "full2embed"])
+    np.testing.assert_array_equal(embed2full, g[pre + "embed2full"])
+    slots = buffer_floats // Fin
+    np.testing.assert_array_equal(buffer[: slots * Fin].reshape(slots, Fin)[-n_cached:], g[pre + "feature_rows"])
+    assert header == int(g[pre + "header"]) == 0
+
+
+@pytest.mark.parametrize("name", list(FILL_CASES))
+def test_oracle_reproduces_reference_constructor(name):
+    from oracle import host_model
+    g = np.load(FILL, allow_pickle=False)
+    c = FILL_CASES[name]
+    feats, hot = fill_inputs(c, g, name)
+    floats = int(g[name + "_buffer_floats"])
+    st = host_model.new_cache_state(c["N"], c["Fin"], c["H"], floats, hot, torch.from_numpy(feats))
+    assert floats // c["Fin"] == int(g[name + "_overall_feat_num"])
+    assert floats // c["H"] == int(g[name + "_overall_embed_num"])
+    check_fill(name, g, c["N"], c["Fin"], floats, st.feat2full.numpy(), st.full2embed.numpy(), st.embed2full.numpy(),
+               st.buffer.numpy(), st.header)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(FILL_CASES))
+def test_gpu_cache_reproduces_reference_constructor(name, tmp_path):
+    """HistoryCache.__init__ from dataset files (num_nodes.txt, sorted_indices.dat), sized by the
+    configuration's limit as the reference sizes it."""
+    from hiscache import HistoryCache, PinnedFeatureStore, make_config
+    dev = "cuda:0"
+    g = np.load(FILL, allow_pickle=False)
+    c = FILL_CASES[name]
+    feats, hot = fill_inputs(c, g, name)
+    os.makedirs(tmp_path / "processed")
+    (tmp_path / "processed" / "num_nodes.txt").write_text("%d\n" % c["N"])
+    hot.tofile(str(tmp_path / "processed" / "sorted_indices.dat"))
+    cfg = make_config(c["Fin"], 5, c["H"], 2, method="grad", rate=0.5, staleness_thres=4, limit=c["limit_gb"],
+                      device=dev, path=str(tmp_path))
+    cache = HistoryCache(PinnedFeatureStore(torch.from_numpy(feats), device=dev), cfg, "history_uvm")
+    assert cache.total_num_node == c["N"]
+    assert cache.max_buffer_byte == int(g[name + "_max_buffer_byte"])
+    assert cache.overall_feat_num == int(g[name + "_overall_feat_num"])
+    assert cache.overall_embed_num == int(g[name + "_overall_embed_num"])
+    check_fill(name, g, c["N"], c["Fin"], cache.buffer.numel(), cache.feat2full.cpu().numpy(),
+               cache.full2embed.cpu().numpy(), cache.embed2full.cpu().numpy(), cache.buffer.cpu().numpy(), cache.header)
