@@ -72,6 +72,9 @@ def parse():
     ap.add_argument("--sampler-replay", type=int, default=4,
                     help="c1 / c3 --with-sampler: slots of the device sampler whose launches are recorded in HIP graphs "
                          "and replayed, one launch per batch (0: every batch is launched kernel by kernel)")
+    ap.add_argument("--recorded", action="store_true",
+                    help="c1/c3: the iteration is recorded once per padded batch shape in a HIP graph and replayed "
+                         "(hiscache.RecordedIteration) instead of being enqueued operator by operator")
     ap.add_argument("--no-batch-view", action="store_true",
                     help="c3/c5: batches come without the transposed view of their CSR, so every layer's "
                          "backward builds one (the default: the loader emits it with the batch)")
@@ -765,7 +768,16 @@ def run_c3(args, with_batched=True):
     prefer_low_latency_gemm()                                            # what get_model() does by default
     model = HistorySAGE(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache).to(dev)
     model.train()
-    opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True)      # one multi-tensor launch per step
+    # one multi-tensor launch per step
+    opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True, capturable=bool(args.recorded))
+    recorded = None
+    if args.recorded:
+        # the pooled store shifts its folding at every read, which a replayed read cannot do: the rows are
+        # read ahead of time (outside the recording) and only corrected inside it
+        if not args.prefetch:
+            raise SystemExit("c3 --recorded goes with --prefetch")
+        from hiscache import RecordedIteration
+        recorded = RecordedIteration(model, cache, opt, L)
     class FoldedLabels:
         """Labels of a huge id space folded into a small table."""
         base = np.random.default_rng(3).integers(0, C, size=1 << 20)
@@ -827,7 +839,10 @@ def run_c3(args, with_batched=True):
         """The host-link read of the next batch (of the next --prefetch-depth batches), under the masks of the
         cache's present state (--prefetch-all: every row), runs beside this batch's forward and backward."""
         if sampled["sampler"] is None:
-            cache.prefetch(batches[state["it"] % n_pre], speculative=not args.prefetch_all)
+            for d in range(args.prefetch_depth):
+                nb = batches[(state["it"] + d) % n_pre]
+                if getattr(nb, "prefetched_x", None) is None:
+                    cache.prefetch(nb, speculative=not args.prefetch_all)
             return
         while len(sampled["ahead"]) < args.prefetch_depth:
             nxt = sampled_batch(state["it"] + len(sampled["ahead"]))
@@ -837,6 +852,10 @@ def run_c3(args, with_batched=True):
     def step():
         state["it"] += 1
         b = next_batch()
+        if recorded is not None:
+            start_prefetch()                                   # the next batch's rows, beside this replay
+            ev["load"](lambda: recorded(b, state["it"]))       # the whole iteration is one replay
+            return
         ev["load"](lambda: cache.lookup_and_load(b, L))
         if args.prefetch:
             start_prefetch()
@@ -872,7 +891,12 @@ def run_c3(args, with_batched=True):
         shape["edges"] = int(np.mean([x["idx"].size for x in samples]))
 
     batched = c3_batched_layer(args, samples) if with_batched else {"detail": None, "roofline": None}
+    rec_info = None
+    if recorded is not None:
+        rec_info = {"replays": recorded.replays, "unrecorded": recorded.unrecorded,
+                    "shapes": {str(k): v[:2] for k, v in recorded.shapes().items()}}
     return {
+        "recorded": rec_info,
         "metric": "papers100M-shaped iteration ms (1 GPU)", "value": sec * 1e3, "unit": "ms", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
@@ -1026,7 +1050,11 @@ def run_c1(args):
         table, model.table = model.table, None
         cpu_model = copy.deepcopy(model).cpu()
         model.table = table
-    opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True)
+    opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True, capturable=bool(args.recorded))
+    recorded = None
+    if args.recorded:
+        from hiscache import RecordedIteration
+        recorded = RecordedIteration(model, cache, opt, L)
     sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=1, device=dev, validate=False,
                               emit_view=not args.no_batch_view, replay_slots=args.sampler_replay)
     gen = torch.Generator(device=dev).manual_seed(1)
@@ -1043,6 +1071,9 @@ def run_c1(args):
             state["kept"].append(types.SimpleNamespace(ptr=b.ptr.clone(), idx=b.idx.clone(), y=b.y.clone(),
                                                        sub_to_full=b.sub_to_full.clone(),
                                                        num_node_in_layer=b.num_node_in_layer.clone()))
+        if recorded is not None:
+            ev["load"](lambda: recorded(b, state["it"]))      # the whole iteration is one replay
+            return
         ev["load"](lambda: cache.lookup_and_load(b, L))
         out = ev["forward"](lambda: model(b))
         loss = torch.nn.functional.nll_loss(out, b.y)
@@ -1073,6 +1104,9 @@ def run_c1(args):
         "ms_per_chunk_of_steps": chunk_figures(),
         "transposed_view": "built in backward" if args.no_batch_view else "emitted with the batch",
     }
+    if recorded is not None:
+        res["recorded"] = {"replays": recorded.replays, "unrecorded": recorded.unrecorded,
+                           "shapes": {str(k): v[:2] for k, v in recorded.shapes().items()}}
     if cpu_model is not None:
         # the same iteration with stock PyTorch CPU operators, over batches the GPU loop trained on
         from oracle import torch_cpu_path as tp

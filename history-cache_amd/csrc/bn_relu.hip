@@ -48,6 +48,15 @@ static bool bn_shape(int64_t n, int64_t C, BnShape *s) {
   return true;
 }
 
+// Rows that count: all n, or -- when the caller's matrix is padded to a fixed capacity and the number of rows
+// in use is only known on the device -- *n_dev, kept inside [1, n].  Rows behind it are neither counted nor
+// changed by a gradient: the forward writes zeros there, the backward a zero gradient.
+__device__ __forceinline__ int64_t bn_rows(int64_t n, const int64_t *__restrict__ n_dev) {
+  if (n_dev == nullptr) return n;
+  const int64_t m = *n_dev;
+  return m < 1 ? 1 : (m < n ? m : n);
+}
+
 // pre-activation; the same expression decides y > 0 in forward and in backward
 __device__ __forceinline__ float bn_pre(float x, float mean, float invstd, float g, float b) {
   return ((x - mean) * invstd) * g + b;
@@ -119,9 +128,10 @@ __global__ __launch_bounds__(BN_BLOCK) void bn_stats(
     const float *__restrict__ x, const float *__restrict__ bias, float *__restrict__ part,
     float *__restrict__ save_mean, float *__restrict__ save_invstd, float *__restrict__ running_mean,
     float *__restrict__ running_var, int64_t *__restrict__ batches_tracked, float momentum, float eps,
-    int64_t n, int C, BnShape sh, unsigned *__restrict__ ticket) {
+    int64_t n_cap, const int64_t *__restrict__ n_dev, int C, BnShape sh, unsigned *__restrict__ ticket) {
   __shared__ float4 s_red[2][BN_BLOCK];
   __shared__ int s_flag;
+  const int64_t n = bn_rows(n_cap, n_dev);
   const int G = sh.groups, P = sh.rows_per_pass;
   const int g = (int)threadIdx.x % G, p = (int)threadIdx.x / G;
   const int64_t lo = (int64_t)blockIdx.x * sh.slab_rows;
@@ -192,9 +202,13 @@ __global__ __launch_bounds__(BN_BLOCK) void bn_stats(
 __global__ __launch_bounds__(HC_BLOCK) void bn_apply(
     const float *__restrict__ x, const float *__restrict__ mean, const float *__restrict__ invstd,
     const float *__restrict__ gamma, const float *__restrict__ beta, float *__restrict__ y, int64_t n4,
-    int G) {
+    int G, int64_t n_cap, const int64_t *__restrict__ n_dev) {
   const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
   if (i >= n4) return;
+  if (n_dev != nullptr && i >= bn_rows(n_cap, n_dev) * G) {     // a padding row
+    *reinterpret_cast<float4 *>(y + 4 * i) = make_float4(0.f, 0.f, 0.f, 0.f);
+    return;
+  }
   const int c = (int)(i % G) * 4;
   const float4 v = bn_ld4(x + 4 * i), m = bn_ld4(mean + c), s = bn_ld4(invstd + c);
   const float4 ga = gamma ? bn_ld4(gamma + c) : make_float4(1.f, 1.f, 1.f, 1.f);
@@ -212,9 +226,11 @@ __global__ __launch_bounds__(BN_BLOCK) void bn_bwd_reduce(
     const float *__restrict__ dy, const float *__restrict__ x, const float *__restrict__ mean,
     const float *__restrict__ invstd, const float *__restrict__ gamma, const float *__restrict__ beta,
     float *__restrict__ part, float *__restrict__ dgamma, float *__restrict__ dbeta,
-    float *__restrict__ dbias, int64_t n, int C, BnShape sh, unsigned *__restrict__ ticket) {
+    float *__restrict__ dbias, int64_t n_cap, const int64_t *__restrict__ n_dev, int C, BnShape sh,
+    unsigned *__restrict__ ticket) {
   __shared__ float4 s_red[2][BN_BLOCK];
   __shared__ int s_flag;
+  const int64_t n = bn_rows(n_cap, n_dev);
   const int G = sh.groups, P = sh.rows_per_pass;
   const int g = (int)threadIdx.x % G, p = (int)threadIdx.x / G;
   const int64_t lo = (int64_t)blockIdx.x * sh.slab_rows;
@@ -277,9 +293,15 @@ __global__ __launch_bounds__(HC_BLOCK) void bn_bwd_apply(
     const float *__restrict__ dy, const float *__restrict__ x, const float *__restrict__ mean,
     const float *__restrict__ invstd, const float *__restrict__ gamma, const float *__restrict__ beta,
     const float *__restrict__ dgamma, const float *__restrict__ dbeta, float *__restrict__ dx, int64_t n4,
-    int G, float inv_n) {
+    int G, int64_t n_cap, const int64_t *__restrict__ n_dev) {
   const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
   if (i >= n4) return;
+  const int64_t n = bn_rows(n_cap, n_dev);
+  if (i >= n * G) {                                              // a padding row
+    *reinterpret_cast<float4 *>(dx + 4 * i) = make_float4(0.f, 0.f, 0.f, 0.f);
+    return;
+  }
+  const float inv_n = 1.0f / (float)n;
   const int c = (int)(i % G) * 4;
   const float4 v = bn_ld4(x + 4 * i), d = bn_ld4(dy + 4 * i);
   const float4 m = bn_ld4(mean + c), s = bn_ld4(invstd + c);
@@ -306,11 +328,11 @@ extern "C" size_t hc_bn_relu_workspace_bytes(int64_t n, int64_t C) {
   return hc_align_up((size_t)sh.slabs * 2 * (size_t)C * sizeof(float), 256);
 }
 
-extern "C" int hc_bn_relu_fwd(const float *x, const float *bias, const float *gamma, const float *beta,
-                              float *running_mean, float *running_var, int64_t *num_batches_tracked,
-                              float momentum, float eps, float *y, float *save_mean, float *save_invstd,
-                              int64_t n, int64_t C, void *workspace, size_t workspace_bytes, unsigned *ticket,
-                              void *stream) {
+extern "C" int hc_bn_relu_fwd_dev(const float *x, const float *bias, const float *gamma, const float *beta,
+                                  float *running_mean, float *running_var, int64_t *num_batches_tracked,
+                                  float momentum, float eps, float *y, float *save_mean, float *save_invstd,
+                                  int64_t n, int64_t C, const int64_t *n_dev, void *workspace,
+                                  size_t workspace_bytes, unsigned *ticket, void *stream) {
   HC_REQUIRE(x && y && save_mean && save_invstd && ticket);
   BnShape sh;
   if (!bn_shape(n, C, &sh)) return n >= 1 && C >= 1 ? HC_EUNSUPPORTED : HC_EINVAL;
@@ -322,16 +344,25 @@ extern "C" int hc_bn_relu_fwd(const float *x, const float *bias, const float *ga
   hipStream_t st = static_cast<hipStream_t>(stream);
   bn_stats<<<dim3((unsigned)sh.slabs), dim3(BN_BLOCK), 0, st>>>(
       x, bias, static_cast<float *>(workspace), save_mean, save_invstd, running_mean, running_var,
-      num_batches_tracked, momentum, eps, n, (int)C, sh, ticket);
+      num_batches_tracked, momentum, eps, n, n_dev, (int)C, sh, ticket);
   bn_apply<<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(x, save_mean, save_invstd, gamma, beta, y, n4,
-                                                              sh.groups);
+                                                              sh.groups, n, n_dev);
   return hc_launch_status();
 }
 
-extern "C" int hc_bn_relu_bwd(const float *dy, const float *x, const float *gamma, const float *beta,
-                              const float *save_mean, const float *save_invstd, float *dx, float *dgamma,
-                              float *dbeta, float *dbias, int64_t n, int64_t C, void *workspace,
-                              size_t workspace_bytes, unsigned *ticket, void *stream) {
+extern "C" int hc_bn_relu_fwd(const float *x, const float *bias, const float *gamma, const float *beta,
+                              float *running_mean, float *running_var, int64_t *num_batches_tracked,
+                              float momentum, float eps, float *y, float *save_mean, float *save_invstd,
+                              int64_t n, int64_t C, void *workspace, size_t workspace_bytes, unsigned *ticket,
+                              void *stream) {
+  return hc_bn_relu_fwd_dev(x, bias, gamma, beta, running_mean, running_var, num_batches_tracked, momentum, eps, y,
+                            save_mean, save_invstd, n, C, nullptr, workspace, workspace_bytes, ticket, stream);
+}
+
+extern "C" int hc_bn_relu_bwd_dev(const float *dy, const float *x, const float *gamma, const float *beta,
+                                  const float *save_mean, const float *save_invstd, float *dx, float *dgamma,
+                                  float *dbeta, float *dbias, int64_t n, int64_t C, const int64_t *n_dev,
+                                  void *workspace, size_t workspace_bytes, unsigned *ticket, void *stream) {
   HC_REQUIRE(dy && x && save_mean && save_invstd && dx && dgamma && dbeta && ticket);
   BnShape sh;
   if (!bn_shape(n, C, &sh)) return n >= 1 && C >= 1 ? HC_EUNSUPPORTED : HC_EINVAL;
@@ -342,9 +373,17 @@ extern "C" int hc_bn_relu_bwd(const float *dy, const float *x, const float *gamm
   if (!hc_grid_ok(blocks)) return HC_ELAUNCH;
   hipStream_t st = static_cast<hipStream_t>(stream);
   bn_bwd_reduce<<<dim3((unsigned)sh.slabs), dim3(BN_BLOCK), 0, st>>>(
-      dy, x, save_mean, save_invstd, gamma, beta, static_cast<float *>(workspace), dgamma, dbeta, dbias, n,
+      dy, x, save_mean, save_invstd, gamma, beta, static_cast<float *>(workspace), dgamma, dbeta, dbias, n, n_dev,
       (int)C, sh, ticket);
   bn_bwd_apply<<<dim3((unsigned)blocks), dim3(HC_BLOCK), 0, st>>>(
-      dy, x, save_mean, save_invstd, gamma, beta, dgamma, dbeta, dx, n4, sh.groups, 1.0f / (float)n);
+      dy, x, save_mean, save_invstd, gamma, beta, dgamma, dbeta, dx, n4, sh.groups, n, n_dev);
   return hc_launch_status();
+}
+
+extern "C" int hc_bn_relu_bwd(const float *dy, const float *x, const float *gamma, const float *beta,
+                              const float *save_mean, const float *save_invstd, float *dx, float *dgamma,
+                              float *dbeta, float *dbias, int64_t n, int64_t C, void *workspace,
+                              size_t workspace_bytes, unsigned *ticket, void *stream) {
+  return hc_bn_relu_bwd_dev(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, dbias, n, C, nullptr,
+                            workspace, workspace_bytes, ticket, stream);
 }

@@ -388,10 +388,13 @@ __global__ __launch_bounds__(HC_BLOCK) void gc_pass3_ring(
     const int64_t *__restrict__ chunk_prefix, const GcScalars *__restrict__ sc, const float *__restrict__ emb,
     const int64_t *__restrict__ sub_to_full, void *__restrict__ table, int table_dtype, int64_t capacity,
     int64_t *__restrict__ full2slot, int64_t *__restrict__ slot2full, int64_t *__restrict__ checkin,
-    int64_t *__restrict__ slot_out, int64_t *__restrict__ header, int64_t glb_iter, int64_t M, int64_t F,
-    int64_t n_tiles) {
+    int64_t *__restrict__ slot_out, int64_t *__restrict__ header, int64_t glb_iter_value,
+    const int64_t *__restrict__ glb_iter_dev, int64_t M, int64_t F, int64_t n_tiles) {
   const int lane = hc_lane();
   const int wave = hc_wave_in_block();
+  // the iteration number that admitted rows are stamped with: by value, or read from device memory by
+  // callers whose launches are recorded once and replayed
+  const int64_t glb_iter = glb_iter_dev != nullptr ? *glb_iter_dev : glb_iter_value;
   const int64_t tile0 = (int64_t)blockIdx.x * GC_TILE;
   const int64_t r = tile0 + lane;
   // everything that does not depend on anything else is requested first
@@ -625,14 +628,14 @@ extern "C" int hc_row_scores(const float *grad, float *score, int64_t M, int64_t
                              score, nullptr, M, F, static_cast<hipStream_t>(stream));
 }
 
-extern "C" int hc_grad_check(const float *grad, const float *score_in, const float *emb,
-                             const int64_t *slot, const int32_t *age, const uint8_t *used,
-                             const int64_t *sub_to_full, const float *thres, int32_t age_limit,
-                             int norm_kind, int cmp_kind, uint8_t *mask_out, float *score_out,
-                             int64_t *slot_out, void *table, int table_dtype, int64_t capacity,
-                             int64_t *full2slot, int64_t *slot2full, int64_t *checkin, int64_t *header,
-                             int64_t glb_iter, int64_t M, int64_t F, void *workspace,
-                             size_t workspace_bytes, void *stream) {
+namespace {
+int grad_check_launch(const float *grad, const float *score_in, const float *emb, const int64_t *slot,
+                      const int32_t *age, const uint8_t *used, const int64_t *sub_to_full, const float *thres,
+                      int32_t age_limit, int norm_kind, int cmp_kind, uint8_t *mask_out, float *score_out,
+                      int64_t *slot_out, void *table, int table_dtype, int64_t capacity, int64_t *full2slot,
+                      int64_t *slot2full, int64_t *checkin, int64_t *header, int64_t glb_iter,
+                      const int64_t *glb_iter_dev, int64_t M, int64_t F, void *workspace, size_t workspace_bytes,
+                      void *stream) {
   HC_REQUIRE(M >= 0 && F > 0 && capacity > 0);
   HC_REQUIRE(norm_kind == HC_NORM_L2 || norm_kind == HC_NORM_L1);
   HC_REQUIRE(cmp_kind == HC_CMP_LT || cmp_kind == HC_CMP_NOT_GT);
@@ -658,7 +661,7 @@ extern "C" int hc_grad_check(const float *grad, const float *score_in, const flo
     // two launches: every pass-3 block adds up the (at most 1 024) tile counts in front of it itself
     gc_pass3_ring<true><<<dim3((unsigned)tiles), dim3(HC_BLOCK), 0, st>>>(
         mask_out, tiles_buf, chunk_prefix, sc, emb, sub_to_full, table, table_dtype, capacity, full2slot, slot2full,
-        checkin, slot_out, header, glb_iter, M, F, tiles);
+        checkin, slot_out, header, glb_iter, glb_iter_dev, M, F, tiles);
     return hc_launch_status();
   }
   gc_pass2<<<dim3(1), dim3(GC_SCAN_THREADS), 0, st>>>(tiles_buf, tiles, chunk_prefix, sc, header, capacity, 1,
@@ -666,8 +669,36 @@ extern "C" int hc_grad_check(const float *grad, const float *score_in, const flo
   if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
   gc_pass3_ring<false><<<dim3((unsigned)tiles), dim3(HC_BLOCK), 0, st>>>(
       mask_out, tiles_buf, chunk_prefix, sc, emb, sub_to_full, table, table_dtype, capacity, full2slot, slot2full,
-      checkin, slot_out, header, glb_iter, M, F, tiles);
+      checkin, slot_out, header, glb_iter, glb_iter_dev, M, F, tiles);
   return hc_launch_status();
+}
+}  // namespace
+
+extern "C" int hc_grad_check(const float *grad, const float *score_in, const float *emb,
+                             const int64_t *slot, const int32_t *age, const uint8_t *used,
+                             const int64_t *sub_to_full, const float *thres, int32_t age_limit,
+                             int norm_kind, int cmp_kind, uint8_t *mask_out, float *score_out,
+                             int64_t *slot_out, void *table, int table_dtype, int64_t capacity,
+                             int64_t *full2slot, int64_t *slot2full, int64_t *checkin, int64_t *header,
+                             int64_t glb_iter, int64_t M, int64_t F, void *workspace,
+                             size_t workspace_bytes, void *stream) {
+  return grad_check_launch(grad, score_in, emb, slot, age, used, sub_to_full, thres, age_limit, norm_kind, cmp_kind,
+                           mask_out, score_out, slot_out, table, table_dtype, capacity, full2slot, slot2full, checkin,
+                           header, glb_iter, nullptr, M, F, workspace, workspace_bytes, stream);
+}
+
+extern "C" int hc_grad_check_dev(const float *grad, const float *score_in, const float *emb,
+                                 const int64_t *slot, const int32_t *age, const uint8_t *used,
+                                 const int64_t *sub_to_full, const float *thres, int32_t age_limit,
+                                 int norm_kind, int cmp_kind, uint8_t *mask_out, float *score_out,
+                                 int64_t *slot_out, void *table, int table_dtype, int64_t capacity,
+                                 int64_t *full2slot, int64_t *slot2full, int64_t *checkin, int64_t *header,
+                                 const int64_t *glb_iter_dev, int64_t M, int64_t F, void *workspace,
+                                 size_t workspace_bytes, void *stream) {
+  HC_REQUIRE(glb_iter_dev != nullptr);
+  return grad_check_launch(grad, score_in, emb, slot, age, used, sub_to_full, thres, age_limit, norm_kind, cmp_kind,
+                           mask_out, score_out, slot_out, table, table_dtype, capacity, full2slot, slot2full, checkin,
+                           header, 0, glb_iter_dev, M, F, workspace, workspace_bytes, stream);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -978,10 +1009,8 @@ __device__ uint32_t qt_next_above(const float *__restrict__ score, int64_t n, co
 // One block.  The order statistic of rank lo by four 8-bit passes; the one of rank hi = lo + 1 is the same key
 // when the rank stays among the keys equal to it, else the smallest key above it (one more pass).
 template <bool REG>
-__global__ __launch_bounds__(QT_BLOCK) void quantile_kernel(const float *__restrict__ score, int64_t n, int64_t lo,
-                                                             int64_t hi, float w, float one_minus_w,
-                                                             float *__restrict__ out) {
-  __shared__ QtShared sh;
+__device__ __forceinline__ void qt_block(const float *__restrict__ score, int64_t n, int64_t lo, int64_t hi, float w,
+                                         float one_minus_w, float *__restrict__ out, QtShared &sh) {
   uint32_t rk[QT_REG];
   int nk = 0;
   int nan_seen = 0;                    // torch.quantile answers NaN when any score is NaN: so does this kernel
@@ -1015,6 +1044,32 @@ __global__ __launch_bounds__(QT_BLOCK) void quantile_kernel(const float *__restr
     const float d = __fsub_rn(b, a);
     out[0] = w < 0.5f ? __fadd_rn(a, __fmul_rn(d, w)) : __fsub_rn(b, __fmul_rn(d, one_minus_w));
   }
+}
+
+template <bool REG>
+__global__ __launch_bounds__(QT_BLOCK) void quantile_kernel(const float *__restrict__ score, int64_t n, int64_t lo,
+                                                             int64_t hi, float w, float one_minus_w,
+                                                             float *__restrict__ out) {
+  __shared__ QtShared sh;
+  qt_block<REG>(score, n, lo, hi, w, one_minus_w, out, sh);
+}
+
+// The same with the number of scores read from device memory (kept inside [1, n_max]) and the rank worked
+// out here as the host works it out: pos = fp32(rate) * fp32(n - 1), lo = floor(pos), w = pos - lo, each
+// step rounded to fp32.
+template <bool REG>
+__global__ __launch_bounds__(QT_BLOCK) void quantile_kernel_dev(const float *__restrict__ score,
+                                                                 const int64_t *__restrict__ n_dev, int64_t n_max,
+                                                                 float rate, float *__restrict__ out) {
+  __shared__ QtShared sh;
+  int64_t n = *n_dev;
+  n = n < 1 ? 1 : (n < n_max ? n : n_max);
+  const float pos = __fmul_rn(rate, (float)(n - 1));
+  int64_t lo = (int64_t)floorf(pos);
+  lo = lo < 0 ? 0 : (lo < n - 1 ? lo : n - 1);
+  const int64_t hi = lo + 1 < n - 1 ? lo + 1 : n - 1;
+  const float w = __fsub_rn(pos, (float)lo);
+  qt_block<REG>(score, n, lo, hi, w, __fsub_rn(1.0f, w), out, sh);
 }
 
 // ---- more scores than one block takes: the same select by the whole chip ------------------------
@@ -1190,6 +1245,18 @@ extern "C" int hc_quantile_threshold(const float *score, int64_t n, int64_t lo, 
     quantile_kernel<true><<<dim3(1), dim3(QT_BLOCK), 0, st>>>(score, n, lo, hi, w, one_minus_w, out);
   else
     quantile_kernel<false><<<dim3(1), dim3(QT_BLOCK), 0, st>>>(score, n, lo, hi, w, one_minus_w, out);
+  return hc_launch_status();
+}
+
+extern "C" int hc_quantile_threshold_dev(const float *score, const int64_t *n_dev, int64_t n_max, float rate,
+                                         float *out, void *stream) {
+  HC_REQUIRE(score && n_dev && out && n_max >= 1 && rate >= 0.0f && rate <= 1.0f);
+  if (n_max > QT_MAX_N) return HC_EUNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (n_max <= (int64_t)QT_BLOCK * QT_REG)
+    quantile_kernel_dev<true><<<dim3(1), dim3(QT_BLOCK), 0, st>>>(score, n_dev, n_max, rate, out);
+  else
+    quantile_kernel_dev<false><<<dim3(1), dim3(QT_BLOCK), 0, st>>>(score, n_dev, n_max, rate, out);
   return hc_launch_status();
 }
 

@@ -196,13 +196,18 @@ __global__ __launch_bounds__(HC_BLOCK) void lookup_kernel(const int64_t *__restr
 template <typename TT>
 __global__ __launch_bounds__(HC_BLOCK) void ring_lookup_kernel(
     const int64_t *__restrict__ full2slot, int64_t n_full, const int64_t *__restrict__ ids,
-    const int64_t *__restrict__ checkin, int64_t now, int64_t age_limit, const TT *__restrict__ table,
-    int64_t capacity, int64_t F, int64_t *__restrict__ slot_out, float *__restrict__ rows_out, int64_t n) {
+    const int64_t *__restrict__ checkin, int64_t now_value, int64_t age_limit, const TT *__restrict__ table,
+    int64_t capacity, int64_t F, int64_t *__restrict__ slot_out, float *__restrict__ rows_out, int64_t n,
+    const int64_t *__restrict__ now_dev, const int64_t *__restrict__ n_valid_dev) {
   constexpr int V = 4;
   const int lane = hc_lane();
   const int64_t i = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
   if (i >= n) return;
-  const int64_t id = ids[i];
+  // callers whose launches are recorded once and replayed keep the iteration number and the number of ids
+  // in use in device memory: ids behind that number are padding and find nothing
+  const int64_t now = now_dev != nullptr ? *now_dev : now_value;
+  const bool padding = n_valid_dev != nullptr && i >= *n_valid_dev;
+  const int64_t id = padding ? -1 : ids[i];
   int64_t slot = (id >= 0 && id < n_full) ? full2slot[id] : -1;
   if (slot < 0 || slot >= capacity) slot = -1;
   if (slot >= 0 && checkin != nullptr && now - checkin[slot] >= age_limit) slot = -1;
@@ -224,6 +229,50 @@ __global__ __launch_bounds__(HC_BLOCK) void ring_lookup_kernel(
 }
 
 inline unsigned blocks_for(int64_t n) { return (unsigned)((n + HC_BLOCK - 1) / HC_BLOCK); }
+
+// Staging of a batch into arrays of fixed size: dst[i] = i < n_copy ? src[i] : fill for up to twelve arrays
+// of 8-, 4-, 2- or 1-byte elements (integers; rows of floats go through as their bit patterns with fill 0), and
+// a handful of 64-bit scalars (the batch's sizes, the iteration number) written to device memory, all in one
+// launch.
+constexpr int STAGE_MAX_ARRAYS = 12;
+constexpr int STAGE_MAX_SCALARS = 16;
+struct StagePlan {
+  const void *src[STAGE_MAX_ARRAYS];
+  void *dst[STAGE_MAX_ARRAYS];
+  int64_t n_copy[STAGE_MAX_ARRAYS];
+  int64_t n_total[STAGE_MAX_ARRAYS];
+  int64_t fill[STAGE_MAX_ARRAYS];
+  int elem[STAGE_MAX_ARRAYS];          // bytes per element: 8, 4, 2 or 1
+  int64_t *scalars_dst;
+  int64_t scalars[STAGE_MAX_SCALARS];
+  int n_scalars;
+};
+
+template <typename T>
+__device__ __forceinline__ void stage_one(const void *src_, void *dst_, int64_t m, int64_t n, int64_t fill) {
+  const T *__restrict__ src = static_cast<const T *>(src_);
+  T *__restrict__ dst = static_cast<T *>(dst_);
+  const int64_t stride = (int64_t)gridDim.x * HC_BLOCK;
+  for (int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x; i < n; i += stride) dst[i] = i < m ? src[i] : (T)fill;
+}
+
+__global__ __launch_bounds__(HC_BLOCK) void stage_kernel(StagePlan p) {
+  const int a = (int)blockIdx.y;
+  if (a == 0 && blockIdx.x == 0 && (int)threadIdx.x < p.n_scalars) p.scalars_dst[threadIdx.x] = p.scalars[threadIdx.x];
+  const int64_t n = p.n_total[a], m = p.n_copy[a];
+  switch (p.elem[a]) {                 // block-uniform
+    case 8: stage_one<int64_t>(p.src[a], p.dst[a], m, n, p.fill[a]); break;
+    case 4: stage_one<int32_t>(p.src[a], p.dst[a], m, n, p.fill[a]); break;
+    case 2: stage_one<int16_t>(p.src[a], p.dst[a], m, n, p.fill[a]); break;
+    case 1: stage_one<int8_t>(p.src[a], p.dst[a], m, n, p.fill[a]); break;
+    default: break;
+  }
+}
+
+inline unsigned blocks_for_stage(int64_t longest) {
+  int64_t bx = (longest + (int64_t)HC_BLOCK * 4 - 1) / ((int64_t)HC_BLOCK * 4);
+  return (unsigned)(bx > 2048 ? 2048 : (bx < 1 ? 1 : bx));
+}
 
 }  // namespace
 
@@ -515,10 +564,11 @@ extern "C" int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids
   return hc_launch_status();
 }
 
-extern "C" int hc_ring_lookup(const int64_t *full2slot, int64_t n_full, const int64_t *ids,
-                              const int64_t *checkin, int64_t now, int64_t age_limit, const void *table,
-                              int table_dtype, int64_t capacity, int64_t F, int64_t *slot_out,
-                              float *rows_out, int64_t n, void *stream) {
+namespace {
+int ring_lookup_launch(const int64_t *full2slot, int64_t n_full, const int64_t *ids, const int64_t *checkin,
+                       int64_t now, const int64_t *now_dev, const int64_t *n_valid_dev, int64_t age_limit,
+                       const void *table, int table_dtype, int64_t capacity, int64_t F, int64_t *slot_out,
+                       float *rows_out, int64_t n, void *stream) {
   HC_REQUIRE(n >= 0 && n_full >= 0 && capacity >= 0 && F > 0);
   if (table_dtype < HC_F32 || table_dtype > HC_BF16) return HC_EDTYPE;
   if (n == 0) return HC_OK;
@@ -530,14 +580,64 @@ extern "C" int hc_ring_lookup(const int64_t *full2slot, int64_t n_full, const in
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (table_dtype == HC_F32)
     ring_lookup_kernel<float><<<g, bl, 0, st>>>(full2slot, n_full, ids, checkin, now, age_limit,
-                                                static_cast<const float *>(table), capacity, F, slot_out, rows_out, n);
+                                                static_cast<const float *>(table), capacity, F, slot_out, rows_out, n,
+                                                now_dev, n_valid_dev);
   else if (table_dtype == HC_F16)
     ring_lookup_kernel<__half><<<g, bl, 0, st>>>(full2slot, n_full, ids, checkin, now, age_limit,
-                                                 static_cast<const __half *>(table), capacity, F, slot_out, rows_out, n);
+                                                 static_cast<const __half *>(table), capacity, F, slot_out, rows_out, n,
+                                                 now_dev, n_valid_dev);
   else
     ring_lookup_kernel<__hip_bfloat16><<<g, bl, 0, st>>>(full2slot, n_full, ids, checkin, now, age_limit,
                                                          static_cast<const __hip_bfloat16 *>(table), capacity, F,
-                                                         slot_out, rows_out, n);
+                                                         slot_out, rows_out, n, now_dev, n_valid_dev);
+  return hc_launch_status();
+}
+}  // namespace
+
+extern "C" int hc_ring_lookup(const int64_t *full2slot, int64_t n_full, const int64_t *ids,
+                              const int64_t *checkin, int64_t now, int64_t age_limit, const void *table,
+                              int table_dtype, int64_t capacity, int64_t F, int64_t *slot_out,
+                              float *rows_out, int64_t n, void *stream) {
+  return ring_lookup_launch(full2slot, n_full, ids, checkin, now, nullptr, nullptr, age_limit, table, table_dtype,
+                            capacity, F, slot_out, rows_out, n, stream);
+}
+
+extern "C" int hc_ring_lookup_dev(const int64_t *full2slot, int64_t n_full, const int64_t *ids,
+                                  const int64_t *checkin, const int64_t *now_dev, const int64_t *n_valid_dev,
+                                  int64_t age_limit, const void *table, int table_dtype, int64_t capacity,
+                                  int64_t F, int64_t *slot_out, float *rows_out, int64_t n, void *stream) {
+  HC_REQUIRE(now_dev != nullptr && n_valid_dev != nullptr);
+  return ring_lookup_launch(full2slot, n_full, ids, checkin, 0, now_dev, n_valid_dev, age_limit, table, table_dtype,
+                            capacity, F, slot_out, rows_out, n, stream);
+}
+
+extern "C" int hc_stage_arrays(const void *const *src, void *const *dst, const int64_t *n_copy,
+                               const int64_t *n_total, const int64_t *fill, const int *elem_bytes, int n_arrays,
+                               int64_t *scalars_dst, const int64_t *scalars, int n_scalars, void *stream) {
+  HC_REQUIRE(n_arrays >= 0 && n_arrays <= STAGE_MAX_ARRAYS && n_scalars >= 0 && n_scalars <= STAGE_MAX_SCALARS);
+  HC_REQUIRE(n_arrays == 0 || (src && dst && n_copy && n_total && fill && elem_bytes));
+  HC_REQUIRE(n_scalars == 0 || (scalars_dst && scalars));
+  if (n_arrays == 0 && n_scalars == 0) return HC_OK;
+  StagePlan p{};
+  int64_t longest = 1;
+  for (int a = 0; a < n_arrays; ++a) {
+    HC_REQUIRE(n_total[a] >= 0 && n_copy[a] >= 0 && n_copy[a] <= n_total[a]);
+    HC_REQUIRE(elem_bytes[a] == 8 || elem_bytes[a] == 4 || elem_bytes[a] == 2 || elem_bytes[a] == 1);
+    HC_REQUIRE(n_total[a] == 0 || dst[a] != nullptr);
+    HC_REQUIRE(n_copy[a] == 0 || src[a] != nullptr);
+    p.src[a] = src[a];
+    p.dst[a] = dst[a];
+    p.n_copy[a] = n_copy[a];
+    p.n_total[a] = n_total[a];
+    p.fill[a] = fill[a];
+    p.elem[a] = elem_bytes[a];
+    if (n_total[a] > longest) longest = n_total[a];
+  }
+  p.scalars_dst = scalars_dst;
+  p.n_scalars = n_scalars;
+  for (int k = 0; k < n_scalars; ++k) p.scalars[k] = scalars[k];
+  stage_kernel<<<dim3(blocks_for_stage(longest), (unsigned)(n_arrays > 0 ? n_arrays : 1)), dim3(HC_BLOCK), 0,
+                 static_cast<hipStream_t>(stream)>>>(p);
   return hc_launch_status();
 }
 

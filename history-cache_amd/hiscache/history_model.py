@@ -143,15 +143,18 @@ class _SageConvFunction(torch.autograd.Function):
         return g_x, g_wl, g_bl, g_wr, None, None, None, None, None, None, None, None, None
 
 
-def bn_relu(x, bn, bias=None, fused=True):
+def bn_relu(x, bn, bias=None, fused=True, n_dev=None):
     """``F.relu(bn(x + bias))`` (/root/reference/hiscache/history_model.py:139-140).  In training mode on
     the GPU this is one autograd node over the library's epilogue kernels (two launches forward, two
     backward, against eight and four operator by operator); ``bias`` then must NOT have been added to
     ``x`` yet.  Otherwise the torch operators run.  ``bn``'s running statistics and batch counter are
-    updated as ``torch.nn.BatchNorm1d.forward`` updates them."""
+    updated as ``torch.nn.BatchNorm1d.forward`` updates them.  ``n_dev`` (one int64 on the device; recorded
+    iterations over padded batches): the number of rows of ``x`` that are in use."""
     be = hiscache_backend
     if not (fused and bn.training and x.dim() == 2 and be.bn_relu_supported(x, x.shape[1])
             and x.shape[0] > 1):
+        if n_dev is not None:
+            raise ValueError("a row count on the device needs the fused epilogue (training mode, fp32 on the GPU)")
         if bias is not None:
             x = x + bias
         return F.relu(bn(x))
@@ -165,7 +168,7 @@ def bn_relu(x, bn, bias=None, fused=True):
         else:
             counter = bn.num_batches_tracked          # incremented by the statistics kernel
     return be.bias_bn_relu(x, bias, bn.weight, bn.bias, bn.running_mean if track else None,
-                           bn.running_var if track else None, momentum, bn.eps, counter)
+                           bn.running_var if track else None, momentum, bn.eps, counter, n_dev)
 
 
 class MySageConvHistory(torch.nn.Module):
@@ -251,6 +254,8 @@ class HistorySAGE(torch.nn.Module):
         none = torch.empty(0, device=x.device)
         nel = getattr(batch, "num_edge_in_layer", None)      # edges of the first num_node_in_layer[k] rows
         view = getattr(batch, "view", None)                  # shared transposed view, if the loader emitted it
+        # a batch padded to fixed sizes for a recorded iteration carries its real sizes on the device
+        dev = getattr(batch, "dev", None)
         for i, conv in enumerate(self.convs[:-1]):
             k = self.num_layers - 1 - i
             n = batch.num_node_in_layer[k]
@@ -265,7 +270,8 @@ class HistorySAGE(torch.nn.Module):
                 self.table.produced_embedding = his
             else:
                 x, his = conv(x, batch.ptr, batch.idx, none, none, 0, n, ne, add_bias=not defer, view=view)
-            x = bn_relu(x, self.bns[i], conv.lin_l.bias if defer else None, fused=self.fused_epilogue)
+            x = bn_relu(x, self.bns[i], conv.lin_l.bias if defer else None, fused=self.fused_epilogue,
+                        n_dev=None if dev is None else dev.nnl[k])
             x = F.dropout(x, p=self.dropout, training=self.training)
         x, his = self.convs[-1](x, batch.ptr, batch.idx, none, none, 0, batch.num_node_in_layer[0],
                                 None if nel is None else int(nel[0]), view=view)

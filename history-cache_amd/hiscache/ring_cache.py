@@ -67,16 +67,30 @@ class RingHistoryCache:
             num_layer = self.num_layers_all
         sub_to_full = batch.sub_to_full
         n1 = int(batch.num_node_in_layer[1])
-        self.glb_iter += 1
+        # A batch padded to fixed sizes for a recorded iteration (hiscache.RecordedIteration) carries its real
+        # sizes and the iteration number on the device: rows behind the real 1-hop nodes find nothing, and this
+        # object's own counter is kept by whoever replays the recording.
+        dev = getattr(batch, "dev", None)
+        if dev is None:
+            self.glb_iter += 1
         # slots (stale entries count as absent) and the cached rows of the hits, one launch
         self.sub2embed, self.cached_embedding = _be.ring_lookup(
-            self.full2slot, sub_to_full[:n1], self.table, checkin=self.checkin, now=self.glb_iter,
-            age_limit=self.age_limit)
+            self.full2slot, sub_to_full[:n1], self.table, checkin=self.checkin,
+            now=self.glb_iter if dev is None else dev.now, age_limit=self.age_limit,
+            n_valid=None if dev is None else dev.nnl[1])
         self.used_masks = _be.count_history_reconstruct(batch.ptr, batch.idx, self.sub2embed,
                                                         sub_to_full.shape[0], batch.y.shape[0], num_layer)
-        if self._counters is not None:
+        if self._counters is not None and dev is None:
             prev, self._uncounted_mask = self._uncounted_mask, None
             _be.load_mask(self.used_masks[0], None, self.sub2embed, prev, self._counters)
+        if dev is not None and getattr(dev, "prefetched", None) is not None:
+            # a padded batch whose rows were read ahead of time into fixed arrays (rows, the mask they were read
+            # under, the store's row ids): the rows that have become necessary since are read now, those that no
+            # longer are get cleared
+            pre = dev.prefetched
+            _be.fixup_rows(self.uvm.buffer, pre.src_ids, self.used_masks[0], pre.have, pre.rows)
+            batch.x = pre.rows
+            return None
         handle = getattr(batch, "prefetched_x", None)
         if handle is not None and handle.ids is sub_to_full:
             batch.prefetched_x = None
@@ -130,6 +144,14 @@ class RingHistoryCache:
         # rows with a slot were served from the table (stale entries were reported absent at lookup):
         # only rows that were computed in this iteration can be admitted, so no age is passed
         common = dict(checkin=self.checkin)
+        dev = getattr(batch, "dev", None)
+        if dev is not None:
+            # a padded batch: the rows behind the real 1-hop nodes are never admitted, the threshold is the
+            # quantile of the real rows' scores, and the iteration number comes from the device
+            if self.method != "grad" or emb.grad is None:
+                raise ValueError("recorded iterations admit by gradient")
+            common["used"] = dev.row_index[:n1] < dev.nnl[1]
+            glb_iter = dev.it
         if self.method == "grad" and emb.grad is not None:
             grad = emb.grad.contiguous()
             if self.thres is not None:
@@ -138,7 +160,8 @@ class RingHistoryCache:
                                              **common)
             else:
                 score = _be.row_scores(grad)
-                thres = quantile_threshold(score, self.rate)
+                thres = (quantile_threshold(score, self.rate) if dev is None
+                         else _be.quantile_select_dev(score, dev.nnl[1], self.rate))
                 mask, _ = _be.grad_check(None, emb.detach().contiguous(), slot, sub_to_full, thres, self.table,
                                          self.full2slot, self.slot2full, self._header, glb_iter, score=score,
                                          **common)
@@ -150,7 +173,7 @@ class RingHistoryCache:
                                      **common)
         emb.grad = None
         self.last_record_mask = mask
-        self._uncounted_mask = mask if self._counters is not None else None
+        self._uncounted_mask = mask if self._counters is not None and dev is None else None
         self.last_score = score
         self.produced_embedding = None
 

@@ -110,6 +110,17 @@ _SIGNATURES = {
                                 _c_p, _c_sz, _c_p, _c_p]),
     "hc_weight_grad_workspace_bytes": (_c_sz, [_c_i64, _c_i64, _c_i64, _c_int]),
     "hc_weight_grad": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_sz, _c_p]),
+    "hc_stage_arrays": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_p, _c_p, _c_int, _c_p]),
+    "hc_ring_lookup_dev": (_c_int, [_c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_i64, _c_i64, _c_p,
+                                    _c_p, _c_i64, _c_p]),
+    "hc_grad_check_dev": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, ctypes.c_int32, _c_int,
+                                   _c_int, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_p,
+                                   _c_p, _c_i64, _c_i64, _c_p, _c_sz, _c_p]),
+    "hc_quantile_threshold_dev": (_c_int, [_c_p, _c_p, _c_i64, ctypes.c_float, _c_p, _c_p]),
+    "hc_bn_relu_fwd_dev": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, ctypes.c_float, ctypes.c_float, _c_p,
+                                    _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_sz, _c_p, _c_p]),
+    "hc_bn_relu_bwd_dev": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64,
+                                    _c_p, _c_p, _c_sz, _c_p, _c_p]),
     "hc_typed_csr_workspace_bytes": (_c_sz, [_c_i64, _c_int]),
     "hc_edge_types_by_ranges": (_c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_p, _c_p, _c_i64, _c_i64, _c_p]),
     "hc_typed_csr": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_p,
@@ -680,6 +691,55 @@ def quantile_select(score, lo, hi, w, one_minus_w):
     return out
 
 
+def quantile_select_dev(score, n_dev, rate):
+    """``quantile_threshold(score[:n], rate)`` with n read from ``n_dev`` (one int64 on the device, kept inside
+    [1, len(score)]): the rank is worked out on the device as the host works it out, the same bits.  At most
+    hc_quantile_max_scores() scores.  For recorded iterations."""
+    lib = load_library()
+    score = _dev(score, "score", torch.float32)
+    _dev(n_dev, "n_dev", torch.int64)
+    out = torch.empty(1, dtype=torch.float32, device=score.device)
+    _check(lib.hc_quantile_threshold_dev(_ptr(score), _ptr(n_dev), score.numel(), float(rate), _ptr(out), _stream()),
+           "hc_quantile_threshold_dev")
+    return out
+
+
+def stage_arrays(arrays, scalars_dst=None, scalars=()):
+    """One launch that pads arrays into fixed-size ones and writes a few int64 scalars to device memory.
+    ``arrays``: up to 12 tuples (src, dst, n_copy, fill) of contiguous device tensors, src of dst's dtype
+    (elements of 8, 4, 2 or 1 bytes; they are moved as bit patterns): dst.view(-1)[i] = src.view(-1)[i] for
+    i < n_copy, ``fill`` (an integer; 0 for floating-point data) behind.  ``scalars`` (up to 16 Python ints) go
+    to ``scalars_dst[:len(scalars)]``."""
+    lib = load_library()
+    k = len(arrays)
+    if k > 12 or len(scalars) > 16:
+        raise ValueError("at most 12 arrays and 16 scalars per call")
+    P, I64 = ctypes.c_void_p * max(k, 1), ctypes.c_int64 * max(k, 1)
+    src, dst, n_copy, n_total, fill = P(), P(), I64(), I64(), I64()
+    elem = (ctypes.c_int * max(k, 1))()
+    for a, (s_, d_, n_, f_) in enumerate(arrays):
+        _dev(d_, "dst")
+        if d_.element_size() not in (8, 4, 2, 1) or not d_.is_contiguous():
+            raise ValueError("staged arrays are contiguous tensors of 8-, 4-, 2- or 1-byte elements")
+        n_ = int(n_)
+        if n_ < 0 or n_ > d_.numel():
+            raise ValueError("n_copy outside the destination")
+        if n_ > 0:
+            _dev(s_, "src", d_.dtype)
+            if s_.numel() < n_ or not s_.is_contiguous():
+                raise ValueError("source shorter than n_copy or not contiguous")
+            src[a] = s_.data_ptr()
+        dst[a], n_copy[a], n_total[a], fill[a] = d_.data_ptr(), n_, d_.numel(), int(f_)
+        elem[a] = d_.element_size()
+    vals = (ctypes.c_int64 * max(len(scalars), 1))(*[int(v) for v in scalars])
+    if scalars:
+        _dev(scalars_dst, "scalars_dst", torch.int64)
+        if scalars_dst.numel() < len(scalars):
+            raise ValueError("scalars_dst is too short")
+    _check(lib.hc_stage_arrays(src, dst, n_copy, n_total, fill, elem, k, _ptr(scalars_dst) if scalars else _c_p(None),
+                               vals, len(scalars), _stream()), "hc_stage_arrays")
+
+
 def grad_check(grad, emb, slot, sub_to_full, thres, table, full2slot, slot2full, header, glb_iter,
                age=None, age_limit=0, used=None, checkin=None, norm_kind=NORM_L2, cmp_kind=CMP_LT,
                score=None, want_slots=False, static_scratch=False):
@@ -730,12 +790,20 @@ def grad_check(grad, emb, slot, sub_to_full, thres, table, full2slot, slot2full,
     mask = torch.empty(M, dtype=torch.uint8, device=dev)
     score_out = torch.empty(M, dtype=torch.float32, device=dev)
     slot_out = torch.empty(M, dtype=torch.int64, device=dev) if want_slots else None
+    iter_on_device = isinstance(glb_iter, torch.Tensor)       # recorded iterations: one int64 on the device
+    if iter_on_device:
+        _dev(glb_iter, "glb_iter", torch.int64)
+        if static_scratch:
+            raise ValueError("glb_iter on the device goes with a workspace")
     args = (_ptr(grad), _ptr(score), _ptr(emb), _ptr(slot), _ptr(age), _ptr(used),
             _ptr(sub_to_full), _ptr(thres), int(age_limit), int(norm_kind), int(cmp_kind),
             _ptr(mask), _ptr(score_out), _ptr(slot_out), _ptr(table),
             _float_dtype(table, "table"), table.shape[0], _ptr(full2slot), _ptr(slot2full),
-            _ptr(checkin), _ptr(header), int(glb_iter), M, F)
-    if static_scratch:
+            _ptr(checkin), _ptr(header), _ptr(glb_iter) if iter_on_device else int(glb_iter), M, F)
+    if iter_on_device:
+        ws = _workspace(lib.hc_grad_check_workspace_bytes(M), dev)
+        _check(lib.hc_grad_check_dev(*args, _ptr(ws), ws.numel(), _stream()), "hc_grad_check_dev")
+    elif static_scratch:
         with torch.cuda.device(dev):
             _check(lib.hc_grad_check_static(*args, _stream()), "hc_grad_check_static")
     else:
@@ -955,10 +1023,11 @@ def lookup(map_tensor, ids, offset=0):
     return out
 
 
-def ring_lookup(full2slot, ids, table, checkin=None, now=0, age_limit=1 << 62, want_rows=True):
+def ring_lookup(full2slot, ids, table, checkin=None, now=0, age_limit=1 << 62, want_rows=True, n_valid=None):
     """Slots of ``ids`` in a ring table and the table rows of the hits, in one launch.  An entry with
     ``now - checkin[slot] >= age_limit`` counts as absent (-1).  Returns (slot[int64], rows[fp32] or
-    None); rows of absent ids are zero."""
+    None); rows of absent ids are zero.  For recorded iterations ``now`` may be a one-element int64 device
+    tensor, together with ``n_valid`` (the same): ids behind the first ``n_valid`` are padding and find nothing."""
     lib = load_library()
     _dev(full2slot, "full2slot", torch.int64)
     _dev(ids, "ids", torch.int64)
@@ -972,6 +1041,16 @@ def ring_lookup(full2slot, ids, table, checkin=None, now=0, age_limit=1 << 62, w
     n = ids.numel()
     slot = torch.empty(n, dtype=torch.int64, device=ids.device)
     rows = torch.empty((n, table.shape[1]), dtype=torch.float32, device=ids.device) if want_rows else None
+    if isinstance(now, torch.Tensor) or n_valid is not None:
+        if not isinstance(now, torch.Tensor) or n_valid is None:
+            raise ValueError("now and n_valid go together as one-element int64 device tensors")
+        _dev(now, "now", torch.int64)
+        _dev(n_valid, "n_valid", torch.int64)
+        rc = lib.hc_ring_lookup_dev(_ptr(full2slot), full2slot.numel(), _ptr(ids), _ptr(checkin), _ptr(now),
+                                    _ptr(n_valid), int(age_limit), _ptr(table), _float_dtype(table, "table"),
+                                    table.shape[0], table.shape[1], _ptr(slot), _ptr(rows), n, _stream())
+        _check(rc, "hc_ring_lookup_dev")
+        return slot, rows
     rc = lib.hc_ring_lookup(_ptr(full2slot), full2slot.numel(), _ptr(ids), _ptr(checkin), int(now), int(age_limit),
                             _ptr(table), _float_dtype(table, "table"), table.shape[0], table.shape[1], _ptr(slot),
                             _ptr(rows), n, _stream())
@@ -1079,40 +1158,41 @@ class _BiasBnRelu(torch.autograd.Function):
     bias; the running statistics are updated in place."""
 
     @staticmethod
-    def forward(ctx, x, bias, gamma, beta, running_mean, running_var, momentum, eps, batches_tracked=None):
+    def forward(ctx, x, bias, gamma, beta, running_mean, running_var, momentum, eps, batches_tracked=None,
+                n_dev=None):
         lib = load_library()
         n, C = x.shape
         y = torch.empty_like(x)
         stats = torch.empty((2, C), dtype=torch.float32, device=x.device)      # mean, 1/sqrt(var + eps)
         ws = _workspace(lib.hc_bn_relu_workspace_bytes(n, C), x.device)
         sp = stats.data_ptr()
-        _check(lib.hc_bn_relu_fwd(_ptr(x), _ptr(bias), _ptr(gamma), _ptr(beta), _ptr(running_mean),
-                                  _ptr(running_var), _ptr(batches_tracked), float(momentum), float(eps), _ptr(y),
-                                  _c_p(sp),
-                                  _c_p(sp + 4 * C), n, C, _ptr(ws), ws.numel(), _ptr(_ticket(x.device)),
-                                  _stream()), "hc_bn_relu_fwd")
+        _check(lib.hc_bn_relu_fwd_dev(_ptr(x), _ptr(bias), _ptr(gamma), _ptr(beta), _ptr(running_mean),
+                                      _ptr(running_var), _ptr(batches_tracked), float(momentum), float(eps), _ptr(y),
+                                      _c_p(sp), _c_p(sp + 4 * C), n, C, _ptr(n_dev), _ptr(ws), ws.numel(),
+                                      _ptr(_ticket(x.device)), _stream()), "hc_bn_relu_fwd")
         ctx.save_for_backward(x, stats, gamma if gamma is not None else x.new_empty(0),
                               beta if beta is not None else x.new_empty(0))
-        ctx.hc = (bias is not None, gamma is not None, beta is not None)
+        ctx.hc = (bias is not None, gamma is not None, beta is not None, n_dev)
         return y
 
     @staticmethod
     def backward(ctx, dy):
         lib = load_library()
         x, stats, gamma, beta = ctx.saved_tensors
-        has_bias, has_gamma, has_beta = ctx.hc
+        has_bias, has_gamma, has_beta, n_dev = ctx.hc
         dy = dy.contiguous()
         n, C = x.shape
         dx = torch.empty_like(x)
         grads = torch.empty((3, C), dtype=torch.float32, device=x.device)     # dgamma, dbeta, dbias
         ws = _workspace(lib.hc_bn_relu_workspace_bytes(n, C), x.device)
         sp, gp = stats.data_ptr(), grads.data_ptr()
-        _check(lib.hc_bn_relu_bwd(_ptr(dy), _ptr(x), _ptr(gamma if has_gamma else None),
-                                  _ptr(beta if has_beta else None), _c_p(sp), _c_p(sp + 4 * C), _ptr(dx),
-                                  _c_p(gp), _c_p(gp + 4 * C), _c_p(gp + 8 * C if has_bias else None), n, C,
-                                  _ptr(ws), ws.numel(), _ptr(_ticket(x.device)), _stream()), "hc_bn_relu_bwd")
+        _check(lib.hc_bn_relu_bwd_dev(_ptr(dy), _ptr(x), _ptr(gamma if has_gamma else None),
+                                      _ptr(beta if has_beta else None), _c_p(sp), _c_p(sp + 4 * C), _ptr(dx),
+                                      _c_p(gp), _c_p(gp + 4 * C), _c_p(gp + 8 * C if has_bias else None), n, C,
+                                      _ptr(n_dev), _ptr(ws), ws.numel(), _ptr(_ticket(x.device)), _stream()),
+               "hc_bn_relu_bwd")
         return (dx, grads[2] if has_bias else None, grads[0] if has_gamma else None,
-                grads[1] if has_beta else None, None, None, None, None, None)
+                grads[1] if has_beta else None, None, None, None, None, None, None)
 
 
 def weight_grad_supported(g, x):
@@ -1145,9 +1225,12 @@ def weight_grad(g, x0, x1=None):
     return (dw[0], dw[1]) if x1 is not None else dw[0]
 
 
-def bias_bn_relu(x, bias, gamma, beta, running_mean, running_var, momentum, eps, num_batches_tracked=None):
+def bias_bn_relu(x, bias, gamma, beta, running_mean, running_var, momentum, eps, num_batches_tracked=None,
+                 n_dev=None):
     """Training-mode ``relu(batch_norm(x + bias))``; x is [n, C] fp32 on the GPU, n >= 2.
-    ``num_batches_tracked`` (one int64 on the device, optional) is incremented by the call's first kernel."""
+    ``num_batches_tracked`` (one int64 on the device, optional) is incremented by the call's first kernel.
+    ``n_dev`` (one int64 on the device, optional; for recorded iterations): only the first ``n_dev`` rows are in
+    use; the others stay out of the statistics, get zeros in the output and a zero gradient."""
     _dev(x, "x")
     if x.dim() != 2:
         raise ValueError("x must be [n, C]")
@@ -1166,7 +1249,10 @@ def bias_bn_relu(x, bias, gamma, beta, running_mean, running_var, momentum, eps,
         _dev(num_batches_tracked, "num_batches_tracked", torch.int64)
         if num_batches_tracked.numel() != 1:
             raise ValueError("num_batches_tracked must hold one value")
-    return _BiasBnRelu.apply(x, bias, gamma, beta, running_mean, running_var, momentum, eps, num_batches_tracked)
+    if n_dev is not None:
+        _dev(n_dev, "n_dev", torch.int64)
+    return _BiasBnRelu.apply(x, bias, gamma, beta, running_mean, running_var, momentum, eps, num_batches_tracked,
+                             n_dev)
 
 
 def evict(checkin, slot2full, full2slot, stale_iter, sub2slot=None, score=None, thres=None):

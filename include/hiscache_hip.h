@@ -605,6 +605,65 @@ size_t hc_weight_grad_workspace_bytes(int64_t n, int64_t H, int64_t F, int n_ope
 int hc_weight_grad(const float *g, const float *x0, const float *x1, int64_t n, int64_t H, int64_t F,
                    float *dw0, float *dw1, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---------------------------------------------------------------- recorded iterations
+ * Entry points for callers that record the launches of one training iteration
+ * once (a HIP graph over arrays of a fixed, padded size) and replay them for
+ * every batch.  None of them has a counterpart in the reference, whose loop
+ * (hiscache/history_trainer.py:176-193) launches operator by operator.  What a
+ * replay cannot change -- a launch's arguments -- is read from device memory
+ * here: the number of rows in use and the iteration number.  Each is the entry
+ * point of the same name without the suffix in every other respect, the same
+ * kernels included.
+ *
+ * hc_stage_arrays: dst[a][i] = i < n_copy[a] ? src[a][i] : fill[a] for
+ * i in [0, n_total[a]) and up to 12 arrays of elements of 8, 4, 2 or 1 bytes
+ * (elem_bytes[a]; integers, or the bit patterns of floating-point rows with
+ * fill 0), and scalars_dst[k] = scalars[k] for up to 16 int64 values, in one
+ * launch: a batch's arrays padded into fixed-size ones (row offsets continued
+ * at the edge count, ids at -1) together with its sizes.  The argument arrays
+ * are host arrays, read before the call returns.
+ *
+ * hc_ring_lookup_dev: hc_ring_lookup with now = *now_dev and ids[i] for
+ * i >= *n_valid_dev taken as padding (slot -1, zero row).
+ *
+ * hc_grad_check_dev: hc_grad_check with glb_iter = *glb_iter_dev.  Padding rows
+ * are kept out with the `used` mask.
+ *
+ * hc_quantile_threshold_dev: hc_quantile_threshold over score[0, n) with
+ * n = *n_dev kept inside [1, n_max] and the rank worked out on the device as the
+ * host works it out for hc_quantile_threshold (pos = fp32(rate) * fp32(n - 1),
+ * lo = floor(pos), w = pos - lo): the same bits.  n_max <= hc_quantile_max_scores().
+ *
+ * hc_bn_relu_fwd_dev / hc_bn_relu_bwd_dev: hc_bn_relu_fwd / _bwd over a matrix
+ * of n rows of which the first *n_dev (kept inside [1, n]; n_dev NULL = all) are
+ * in use: only those enter the statistics and the column sums, y and dx of the
+ * others are zero.  The slab partition is that of n. */
+int hc_stage_arrays(const void *const *src, void *const *dst, const int64_t *n_copy, const int64_t *n_total,
+                    const int64_t *fill, const int *elem_bytes, int n_arrays, int64_t *scalars_dst,
+                    const int64_t *scalars, int n_scalars, void *stream);
+int hc_ring_lookup_dev(const int64_t *full2slot, int64_t n_full, const int64_t *ids, const int64_t *checkin,
+                       const int64_t *now_dev, const int64_t *n_valid_dev, int64_t age_limit,
+                       const void *table, int table_dtype, int64_t capacity, int64_t F, int64_t *slot_out,
+                       float *rows_out, int64_t n, void *stream);
+int hc_grad_check_dev(const float *grad, const float *score_in, const float *emb, const int64_t *slot,
+                      const int32_t *age, const uint8_t *used, const int64_t *sub_to_full,
+                      const float *thres, int32_t age_limit, int norm_kind, int cmp_kind,
+                      uint8_t *mask_out, float *score_out, int64_t *slot_out, void *table,
+                      int table_dtype, int64_t capacity, int64_t *full2slot, int64_t *slot2full,
+                      int64_t *checkin, int64_t *header, const int64_t *glb_iter_dev, int64_t M, int64_t F,
+                      void *workspace, size_t workspace_bytes, void *stream);
+int hc_quantile_threshold_dev(const float *score, const int64_t *n_dev, int64_t n_max, float rate, float *out,
+                              void *stream);
+int hc_bn_relu_fwd_dev(const float *x, const float *bias, const float *gamma, const float *beta,
+                       float *running_mean, float *running_var, int64_t *num_batches_tracked,
+                       float momentum, float eps, float *y, float *save_mean, float *save_invstd,
+                       int64_t n, int64_t C, const int64_t *n_dev, void *workspace, size_t workspace_bytes,
+                       unsigned *ticket, void *stream);
+int hc_bn_relu_bwd_dev(const float *dy, const float *x, const float *gamma, const float *beta,
+                       const float *save_mean, const float *save_invstd, float *dx, float *dgamma,
+                       float *dbeta, float *dbias, int64_t n, int64_t C, const int64_t *n_dev,
+                       void *workspace, size_t workspace_bytes, unsigned *ticket, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
