@@ -73,7 +73,7 @@ def parse():
                     help="c1 / c3 --with-sampler: slots of the device sampler whose launches are recorded in HIP graphs "
                          "and replayed, one launch per batch (0: every batch is launched kernel by kernel)")
     ap.add_argument("--recorded", action="store_true",
-                    help="c1/c3: the iteration is recorded once per padded batch shape in a HIP graph and replayed "
+                    help="c1/c3/c5: the iteration is recorded once per padded batch shape in a HIP graph and replayed "
                          "(hiscache.RecordedIteration) instead of being enqueued operator by operator")
     ap.add_argument("--no-batch-view", action="store_true",
                     help="c3/c5: batches come without the transposed view of their CSR, so every layer's "
@@ -772,10 +772,8 @@ def run_c3(args, with_batched=True):
     opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True, capturable=bool(args.recorded))
     recorded = None
     if args.recorded:
-        # the pooled store shifts its folding at every read, which a replayed read cannot do: the rows are
-        # read ahead of time (outside the recording) and only corrected inside it
-        if not args.prefetch:
-            raise SystemExit("c3 --recorded goes with --prefetch")
+        # (a read inside a recording keeps the pooled store's folding offset of the moment it was recorded; the
+        # batches differ, so the pool rows read still differ from replay to replay)
         from hiscache import RecordedIteration
         recorded = RecordedIteration(model, cache, opt, L)
     class FoldedLabels:
@@ -958,7 +956,12 @@ def run_c5(args):
     model = HistoryRGCN(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache, num_rel=K, dataset_name="rmag240m",
                         type_bounds=[n_paper, n_paper + n_author], pair_to_rel=pair_to_rel).to(dev)
     model.train()
-    opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True)      # one multi-tensor launch per step
+    # one multi-tensor launch per step
+    opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True, capturable=bool(args.recorded))
+    recorded = None
+    if args.recorded:
+        from hiscache import RecordedIteration
+        recorded = RecordedIteration(model, cache, opt, L)
 
     class FoldedLabels:
         base = np.random.default_rng(5).integers(0, C, size=1 << 20)
@@ -979,6 +982,11 @@ def run_c5(args):
     def step():
         b = batches[state["it"] % n_pre]
         state["it"] += 1
+        if recorded is not None:
+            if args.prefetch:
+                cache.prefetch(batches[state["it"] % n_pre], speculative=not args.prefetch_all)
+            ev["load"](lambda: recorded(b, state["it"]))       # the whole iteration is one replay
+            return
         ev["load"](lambda: cache.lookup_and_load(b, L))
         if args.prefetch:             # the next batch's host-link read runs under this batch's compute
             cache.prefetch(batches[state["it"] % n_pre], speculative=not args.prefetch_all)
@@ -1000,6 +1008,8 @@ def run_c5(args):
     shape = {k: int(np.mean([int(x["num_node_in_layer"][i]) for x in samples])) for i, k in enumerate(("n0", "n1", "n2"))}
     shape["edges"] = int(np.mean([x["idx"].size for x in samples]))
     return {
+        "recorded": None if recorded is None else {"replays": recorded.replays, "unrecorded": recorded.unrecorded,
+                                                   "shapes": {str(k): v[:2] for k, v in recorded.shapes().items()}},
         "metric": "mag240M-shaped RGCN iteration ms (1 GPU)", "value": sec * 1e3, "unit": "ms", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
@@ -1390,11 +1400,25 @@ def main():
             # became bound by the GPU; the mag240M-shaped loop is bound by the host and goes without)
             c3_args = argparse.Namespace(**vars(it_args))
             c3_args.prefetch = True
+            # *_recorded: the same loops with the iteration recorded once per padded batch shape in a HIP graph
+            # and replayed (hiscache.RecordedIteration): one staging launch and one replay per batch
+            r1_args = argparse.Namespace(**vars(it_args))
+            r1_args.recorded, r1_args.no_cpu_baseline = True, True
+            r3_args = argparse.Namespace(**vars(c3_args))
+            r3_args.recorded = True
+            rh_args = argparse.Namespace(**vars(hb_args))
+            rh_args.recorded = True
+            r5_args = argparse.Namespace(**vars(it_args))
+            r5_args.recorded, r5_args.prefetch = True, True      # once replayed, this loop too gains from the read-ahead
             runs = (("c1", it_args, lambda: run_c1(it_args)),
+                    ("c1_recorded", r1_args, lambda: run_c1(r1_args)),
                     ("c3", c3_args, lambda: run_c3(c3_args, with_batched=False)),
+                    ("c3_recorded", r3_args, lambda: run_c3(r3_args, with_batched=False)),
                     ("c5", it_args, lambda: run_c5(it_args)),
+                    ("c5_recorded", r5_args, lambda: run_c5(r5_args)),
                     ("c3_sampled", sm_args, lambda: run_c3(sm_args, with_batched=False)),
-                    ("c3_sampled_features_in_hbm", hb_args, lambda: run_c3(hb_args, with_batched=False)))
+                    ("c3_sampled_features_in_hbm", hb_args, lambda: run_c3(hb_args, with_batched=False)),
+                    ("c3_sampled_features_in_hbm_recorded", rh_args, lambda: run_c3(rh_args, with_batched=False)))
             for name, used_args, fn in runs:
                 gc.collect()
                 torch.cuda.empty_cache()
@@ -1405,6 +1429,8 @@ def main():
                     "feature_read_ahead": bool(used_args.prefetch),
                     "ms_per_chunk_of_steps": r.get("ms_per_chunk_of_steps"),
                     "phases_ms": r["phases_ms"], "phases_host_enqueue_ms": r["phases_host_enqueue_ms"]}
+                if r.get("recorded"):            # the whole iteration is the one phase called "load"
+                    res["iterations"][name]["recorded"] = r["recorded"]
                 if "cpu_baseline" in r:          # c1, the CPU-runnable configuration: the same iteration on the host
                     res["iterations"][name]["cpu_ms"] = r["cpu_baseline"]["value"]
                     res["iterations"][name]["cpu_cores"] = r["cpu_baseline"]["cores"]

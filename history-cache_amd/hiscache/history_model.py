@@ -549,6 +549,7 @@ class HistoryRGCN(torch.nn.Module):
         none = torch.empty(0, device=x.device)
         masks = self.table.used_masks
         view = getattr(batch, "view", None)                  # shared transposed view, if the loader emitted it
+        dev = getattr(batch, "dev", None)                    # a padded batch carries its real sizes on the device
         for i, conv in enumerate(self.convs[:-1]):
             n = batch.num_node_in_layer[L - 1 - i]
             et = etypes[: batch.num_edge_in_layer[L - 1 - i]]
@@ -561,7 +562,8 @@ class HistoryRGCN(torch.nn.Module):
                     self.table.produced_embedding.retain_grad()
             else:
                 x, his = conv(x, batch.ptr, batch.idx, et, None, none, none, um, 0, n, view=view)
-            x = bn_relu(x, self.bns[i], None, fused=self.fused_epilogue)
+            x = bn_relu(x, self.bns[i], None, fused=self.fused_epilogue,
+                        n_dev=None if dev is None else dev.nnl[L - 1 - i])
             x = F.dropout(x, p=self.dropout, training=self.training)
         um = masks[-2] if masks is not None else None
         x, his = self.convs[-1](x, batch.ptr, batch.idx, etypes[: batch.num_edge_in_layer[0]], None, none, none,

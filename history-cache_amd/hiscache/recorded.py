@@ -20,9 +20,9 @@ What stands in the way is that no two sampled batches have the same sizes, so:
   same padded iteration runs unrecorded, which also lets the GEMM library settle on its kernels outside a
   recording).
 
-The model must be a ``HistorySAGE`` in training mode with the fused epilogue, the cache a ``RingHistoryCache``
-that admits by gradient, the optimizer one whose step can be recorded (``capturable=True``).  The cache's
-hit counters are not kept for recorded iterations.
+The model is a ``HistorySAGE`` or a ``HistoryRGCN`` in training mode with the fused epilogue, the cache a
+``RingHistoryCache`` that admits by gradient, the optimizer one whose step can be recorded
+(``capturable=True``).  The cache's hit counters are not kept for recorded iterations.
 """
 import math
 from types import SimpleNamespace
@@ -36,7 +36,7 @@ from .util import backward_on_this_thread
 
 class _Record:
     __slots__ = ("caps", "e_cap", "batch", "scal", "graph", "loss", "uses", "ptr", "idx", "s2f", "y", "ptrT", "rowT",
-                 "x_pre", "have", "src_ids")
+                 "edgeT", "etype", "x_pre", "have", "src_ids")
 
 
 class RecordedIteration:
@@ -84,8 +84,9 @@ class RecordedIteration:
         return all(int(v) <= c for v, c in zip(nnl, caps)) and int(n_edges) <= e_cap
 
     # ------------------------------------------------------------------ records
-    def _new_record(self, j, has_view, handle):
+    def _new_record(self, j, view_kind, handle, etype):
         L, dev = self.L, self.device
+        has_view = view_kind > 0
         caps, e_cap = self._shape(j)
         r = _Record()
         r.caps, r.e_cap, r.graph, r.loss, r.uses = caps, e_cap, None, None, 0
@@ -96,6 +97,8 @@ class RecordedIteration:
         r.y = torch.zeros(caps[0], **i64)
         r.ptrT = torch.zeros(caps[L] + 1, **i64) if has_view else None
         r.rowT = torch.zeros(e_cap, dtype=torch.int32, device=dev) if has_view else None
+        r.edgeT = torch.zeros(e_cap, dtype=torch.int32, device=dev) if view_kind == 2 else None
+        r.etype = torch.zeros(e_cap, dtype=etype.dtype, device=dev) if etype is not None else None
         r.scal = torch.zeros(L + 4, **i64)             # nnl[0..L], edges, now, it
         r.x_pre = r.have = r.src_ids = None
         pre = None
@@ -104,9 +107,9 @@ class RecordedIteration:
             r.have = torch.zeros(caps[L], dtype=torch.uint8, device=dev)
             r.src_ids = torch.full((caps[L],), -1, **i64)
             pre = SimpleNamespace(rows=r.x_pre, have=r.have, src_ids=r.src_ids)
-        view = _be.BatchView(r.ptrT, r.rowT, None, caps[L - 1], caps[L], e_cap) if has_view else None
+        view = _be.BatchView(r.ptrT, r.rowT, r.edgeT, caps[L - 1], caps[L], e_cap) if has_view else None
         r.batch = SimpleNamespace(
-            ptr=r.ptr, idx=r.idx, sub_to_full=r.s2f, y=r.y, x=None, edge_type=None, typed_num_node_in_layer=None,
+            ptr=r.ptr, idx=r.idx, sub_to_full=r.s2f, y=r.y, x=None, edge_type=r.etype, typed_num_node_in_layer=None,
             num_node_in_layer=torch.tensor(caps, dtype=torch.int64), num_edge_in_layer=[e_cap] * L, view=view,
             dev=SimpleNamespace(nnl=[r.scal[k:k + 1] for k in range(L + 1)], edges=r.scal[L + 1:L + 2],
                                 now=r.scal[L + 2:L + 3], it=r.scal[L + 3:L + 4],
@@ -121,6 +124,10 @@ class RecordedIteration:
         if r.ptrT is not None:
             v = batch.view
             arrays += [(v.ptrT, r.ptrT, n_all + 1, n_edges), (v.rowT, r.rowT, n_edges, 0)]
+            if r.edgeT is not None:
+                arrays.append((v.edgeT, r.edgeT, n_edges, 0))
+        if r.etype is not None:
+            arrays.append((batch.edge_type, r.etype, n_edges, -1))
         if handle is not None:
             torch.cuda.current_stream(self.device).wait_event(handle.done)
             arrays += [(handle.rows.view(-1), r.x_pre.view(-1), n_all * r.x_pre.shape[1], 0),
@@ -160,10 +167,12 @@ class RecordedIteration:
             handle = None
         j = self._key_for(nnl, n_edges)
         self.cache.glb_iter += 1
-        key = None if j is None else (j, view is not None, handle is not None)
+        view_kind = 0 if view is None else (2 if view.edgeT is not None else 1)
+        etype = getattr(batch, "edge_type", None)
+        key = None if j is None else (j, view_kind, handle is not None, etype is not None)
         r = None if key is None else self._records.get(key)
         if r is None and key is not None and len(self._records) < self.max_records:
-            r = self._records[key] = self._new_record(j, view is not None, handle)
+            r = self._records[key] = self._new_record(j, view_kind, handle, etype)
         if r is None:
             # a shape outside the family, or more shapes than recordings are kept for: the ordinary iteration
             self.cache.glb_iter -= 1
@@ -185,6 +194,8 @@ class RecordedIteration:
         if r.graph is None:
             if self._capture_stream is None:
                 self._capture_stream = torch.cuda.Stream(device=self.device)    # default priority
+                with torch.cuda.stream(self._capture_stream):
+                    _be.prepare_stream(self.device)     # per-stream scratch words exist before anything is recorded
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=self._capture_stream):
                 r.loss = self._iteration(r.batch)
@@ -194,5 +205,6 @@ class RecordedIteration:
         return r.loss
 
     def shapes(self):
-        """The padded shapes in use: {(j, with view, with rows read ahead): ([n0 .. nL], edges, recorded?, uses)}."""
+        """The padded shapes in use: {(j, view kind 0/1/2 = none/rows/rows and edge slots, rows read ahead,
+        edge types given): ([n0 .. nL], edges, recorded?, uses)}."""
         return {k: (r.caps, r.e_cap, r.graph is not None, r.uses) for k, r in self._records.items()}

@@ -1148,6 +1148,12 @@ def _ticket(device):
     return t
 
 
+def prepare_stream(device):
+    """Create what this module keeps per stream (the epilogue kernels' ticket word) for torch's current stream
+    now, so that a recording on that stream allocates and clears nothing of the kind."""
+    _ticket(torch.device(device))
+
+
 def bn_relu_supported(x, channels):
     return x.is_cuda and x.dtype == torch.float32 and channels % 4 == 0 and 4 <= channels <= BN_RELU_MAX_CHANNELS
 

@@ -268,3 +268,66 @@ def test_batches_outside_the_recorded_family_take_the_ordinary_path():
         assert np.isfinite(float(loss))
     assert cache.glb_iter == it and rec.replays >= 2 and rec.unrecorded >= 3
     assert len(rec.shapes()) == 1
+
+
+def test_replayed_relational_iterations_equal_the_padded_ones():
+    """The relational model (5 relations from node-type ranges, fp16 features and table, the batch's view with edge
+    slots, rows read ahead): replayed and padded-but-unrecorded twins hold the same bits after every iteration."""
+    from helpers import power_law_graph
+    from hiscache import (HistoryRGCN, NeighborSampler, PinnedFeatureStore, RecordedIteration, RingHistoryCache,
+                          make_config, prefer_low_latency_gemm)
+    n_paper, n_author, n_inst = 20_000, 19_000, 1_000
+    N = n_paper + n_author + n_inst
+    Fin, H, C, K, L, n_seed, fanout = 64, 64, 9, 5, 2, 200, [10, 6]
+    rng = np.random.default_rng(12)
+    indptr, indices = power_law_graph(rng, N, 3.0, alpha=2.0, max_degree=300)
+    feats = torch.from_numpy(rng.standard_normal((N, Fin), dtype=np.float32).astype(np.float16))
+    labels = torch.from_numpy(rng.integers(0, C, size=N))
+    cached = torch.from_numpy(rng.permutation(N)[: N // 3].copy())
+    rows = torch.from_numpy((0.5 * rng.standard_normal((cached.numel(), H), dtype=np.float32)).astype(np.float16))
+    prefer_low_latency_gemm()
+
+    def world():
+        torch.manual_seed(21)
+        store = PinnedFeatureStore(feats, device=DEV, out_dtype=torch.float16)
+        cache = RingHistoryCache(store, N, Fin, H, capacity=N, num_layers=L, table_dtype=torch.float16, thres=0.05,
+                                 age_limit=4, device=DEV)
+        cache.preload(cached.to(DEV), rows.to(DEV))
+        cfg = make_config(Fin, C, H, L, device=DEV, model_type="rgcn", num_rel=K, name="rmag240m")
+        model = HistoryRGCN(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache, num_rel=K, dataset_name="rmag240m",
+                            type_bounds=[n_paper, n_paper + n_author],
+                            pair_to_rel=[[0, 1, 0], [2, 0, 3], [0, 4, 0]]).to(DEV)
+        model.train()
+        opt = torch.optim.Adam(model.parameters(), lr=1e-2, fused=True, capturable=True)
+        return cache, model, opt
+
+    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=12, device=DEV, emit_view=True,
+                              view_edges=True)
+    gen = torch.Generator(device=DEV).manual_seed(12)
+    seeds = [torch.randperm(n_paper, device=DEV, generator=gen)[:n_seed].contiguous() for _ in range(5)]
+    order = [0, 1, 2, 0, 3, 1, 4, 0, 2, 3]
+    twins = {}
+    for name, record in (("recorded", True), ("padded", False)):
+        cache, model, opt = world()
+        twins[name] = (cache, model, opt, RecordedIteration(model, cache, opt, L, step=1.02, round_to=64, record=record),
+                       [sampler.sample(seeds[k], rng_seed=500 + k) for k in order])
+    compute = torch.cuda.Stream()
+    compute.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(compute):
+        for i in range(len(order)):
+            losses = []
+            for name in ("recorded", "padded"):
+                cache, model, opt, runner, bs = twins[name]
+                if i + 1 < len(order):
+                    runner.prefetch(bs[i + 1])
+                losses.append(float(runner(bs[i], i + 1)))
+            assert losses[0] == losses[1] and np.isfinite(losses[0])
+            a, c = state_of(*twins["recorded"][:3]), state_of(*twins["padded"][:3])
+            same = [bool(torch.equal(x, y)) for x, y in zip(a, c)]
+            assert all(same), (i, same)
+            torch.zeros(1000, device=DEV).sum().item()           # eager work and a synchronisation in between
+    rec = twins["recorded"][3]
+    shapes = rec.shapes()
+    assert rec.replays >= len(order) // 2, shapes
+    assert all(k[1] == 2 and k[2] for k, v in shapes.items() if v[2])     # view with edge slots, rows read ahead
+    assert int((twins["recorded"][0].full2slot != -1).sum()) > cached.numel()   # rows were admitted
