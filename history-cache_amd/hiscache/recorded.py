@@ -69,6 +69,9 @@ class RecordedIteration:
         j = math.ceil(math.log(need) / math.log(self.step) - 1e-9) if need > 0 else 0
         while not self._holds(j, nnl, n_edges):        # rounding of the logarithm
             j += 1
+        # the rounding up of the rows may leave room one step below (and below that, while the shape still shrinks)
+        while self._shape(j - 1) != self._shape(j) and self._holds(j - 1, nnl, n_edges):
+            j -= 1
         return j
 
     def _shape(self, j):

@@ -293,3 +293,33 @@ def test_cu_limited_stream_teardown_is_idempotent(monkeypatch):
     assert be._ws_cache == {(0, 0): "default"}
     be._destroy_cu_streams()
     assert len(destroyed) == 3
+
+
+def test_recorded_iteration_shape_family():
+    """The padded shapes of hiscache.RecordedIteration: the smallest member of the family that holds the batch,
+    rows rounded up, a layer's rows a prefix of the next layer's; another number of seeds is not in the family."""
+    from types import SimpleNamespace
+
+    import torch
+
+    from hiscache import RecordedIteration
+    rec = RecordedIteration(None, SimpleNamespace(device=torch.device("cpu")), None, 3, step=1.125, round_to=256)
+    base = [1000, 5800, 25_800, 89_000]
+    assert rec._key_for(base, 88_000) == 0
+    caps, e_cap = rec._shape(0)
+    assert caps == [1000, 5888, 25_856, 89_088] and e_cap == 88_064
+    rng = np.random.default_rng(0)
+    for _ in range(300):
+        f = rng.uniform(0.6, 1.6, size=4)
+        nnl = [1000] + sorted(int(b * x) for b, x in zip(base[1:], f[:3]))
+        n_e = int(88_000 * f[3])
+        j = rec._key_for(nnl, n_e)
+        caps, e_cap = rec._shape(j)
+        assert all(a <= c for a, c in zip(nnl, caps)) and n_e <= e_cap
+        assert all(c % 256 == 0 for c in caps[1:]) and caps == sorted(caps)
+        assert not rec._holds(j - 1, nnl, n_e)                       # the smallest one
+    assert rec._key_for([999] + base[1:], 88_000) is None
+    # a hop that adds no node: the caps stay ordered
+    rec2 = RecordedIteration(None, SimpleNamespace(device=torch.device("cpu")), None, 2, round_to=64)
+    j = rec2._key_for([500, 500, 500], 0)
+    assert rec2._shape(j)[0] == [500, 512, 512]
