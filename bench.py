@@ -720,8 +720,8 @@ def pooled_store_class(pool_rows):
         def masked_get(self, ids, mask):
             return super().masked_get(self.fold(ids), mask)
 
-        def prefetch(self, ids, mask=None):
-            handle = super().prefetch(self.fold(ids), mask)
+        def prefetch(self, ids, mask=None, out=None):
+            handle = super().prefetch(self.fold(ids), mask, out=out)
             handle.ids = ids
             return handle
 
@@ -840,12 +840,18 @@ def run_c3(args, with_batched=True):
             for d in range(args.prefetch_depth):
                 nb = batches[(state["it"] + d) % n_pre]
                 if getattr(nb, "prefetched_x", None) is None:
-                    cache.prefetch(nb, speculative=not args.prefetch_all)
+                    read_ahead(nb)
             return
         while len(sampled["ahead"]) < args.prefetch_depth:
             nxt = sampled_batch(state["it"] + len(sampled["ahead"]))
-            cache.prefetch(nxt, speculative=not args.prefetch_all)
+            read_ahead(nxt)
             sampled["ahead"].append(nxt)
+
+    def read_ahead(nb):
+        if recorded is not None and not args.prefetch_all:
+            recorded.prefetch(nb)          # the rows go straight into the array that the batch's recording reads
+        else:
+            cache.prefetch(nb, speculative=not args.prefetch_all)
 
     def step():
         state["it"] += 1
@@ -984,7 +990,7 @@ def run_c5(args):
         state["it"] += 1
         if recorded is not None:
             if args.prefetch:
-                cache.prefetch(batches[state["it"] % n_pre], speculative=not args.prefetch_all)
+                recorded.prefetch(batches[state["it"] % n_pre])
             ev["load"](lambda: recorded(b, state["it"]))       # the whole iteration is one replay
             return
         ev["load"](lambda: cache.lookup_and_load(b, L))

@@ -79,18 +79,19 @@ class PinnedFeatureStore:
     def join(self, event):
         torch.cuda.current_stream(self.device).wait_event(event)
 
-    def prefetch(self, ids, mask=None):
+    def prefetch(self, ids, mask=None, out=None):
         """Start reading the rows of ``ids`` (all of them, or those flagged by ``mask``: the caller's guess
         of which will be needed) on a side stream (default priority) now, so that the host-link read
         overlaps whatever the caller queues next -- typically the previous batch's forward and
-        backward.  Returns a handle for ``take``; ``handle.mask`` is the mask that was read under."""
+        backward.  Returns a handle for ``take``; ``handle.mask`` is the mask that was read under.
+        ``out`` ([len(ids), F], optional): where the rows go instead of a new tensor."""
         cur = torch.cuda.current_stream(self.device)
         if self._prefetch_side is None:
             self._prefetch_side = self._make_prefetch_stream()
         side = self._prefetch_side
         side.wait_stream(cur)                      # the ids are produced on the current stream
         # enqueued on the side stream by name: switching torch's current stream and back costs the host 20 us
-        rows = _be.gather_rows(self.buffer, ids, mask=mask, out_dtype=self.out_dtype, stream=side)
+        rows = _be.gather_rows(self.buffer, ids, mask=mask, out=out, out_dtype=self.out_dtype, stream=side)
         done = torch.cuda.Event()
         done.record(side)
         rows.record_stream(side)

@@ -42,7 +42,7 @@ class _Record:
 class RecordedIteration:
 
     def __init__(self, model, cache, optimizer, num_layers, loss_fn=None, step=1.125, round_to=256,
-                 max_records=12, with_view=True, record=True):
+                 max_records=12, with_view=True, record=True, read_ahead_slots=2):
         self.model, self.cache, self.optimizer = model, cache, optimizer
         self.L = int(num_layers)
         self.loss_fn = loss_fn or torch.nn.functional.nll_loss
@@ -51,6 +51,11 @@ class RecordedIteration:
         self.max_records = int(max_records)
         self.with_view = bool(with_view)
         self.record = bool(record)        # False: the padded iterations run, but none is recorded (for comparison)
+        # rows read ahead go straight into a recording's own array; a shape then has this many recordings, used in
+        # turn, so that the read for a coming batch never writes what the replay in flight reads (read at most
+        # read_ahead_slots - 1 batches ahead)
+        self.read_ahead_slots = max(1, int(read_ahead_slots))
+        self._reads_started = 0
         self.device = cache.device
         self._base = None                 # sizes of the first batch: (n0, [n1 .. nL], E)
         self._records = {}
@@ -86,8 +91,17 @@ class RecordedIteration:
         caps, e_cap = self._shape(j)
         return all(int(v) <= c for v, c in zip(nnl, caps)) and int(n_edges) <= e_cap
 
+    def _describe(self, batch):
+        nnl = [int(v) for v in batch.num_node_in_layer]
+        n_edges = int(batch.idx.numel())
+        view = getattr(batch, "view", None) if self.with_view else None
+        if view is not None and (view.rows < nnl[self.L - 1] or view.n_src < nnl[self.L]):
+            view = None
+        view_kind = 0 if view is None else (2 if view.edgeT is not None else 1)
+        return nnl, n_edges, view_kind, getattr(batch, "edge_type", None)
+
     # ------------------------------------------------------------------ records
-    def _new_record(self, j, view_kind, handle, etype):
+    def _new_record(self, j, view_kind, pre_like, etype):
         L, dev = self.L, self.device
         has_view = view_kind > 0
         caps, e_cap = self._shape(j)
@@ -105,8 +119,8 @@ class RecordedIteration:
         r.scal = torch.zeros(L + 4, **i64)             # nnl[0..L], edges, now, it
         r.x_pre = r.have = r.src_ids = None
         pre = None
-        if handle is not None:                         # feature rows read ahead of time land here
-            r.x_pre = torch.zeros((caps[L], handle.rows.shape[1]), dtype=handle.rows.dtype, device=dev)
+        if pre_like is not None:                       # feature rows read ahead of time land here: (width, dtype)
+            r.x_pre = torch.zeros((caps[L], pre_like[0]), dtype=pre_like[1], device=dev)
             r.have = torch.zeros(caps[L], dtype=torch.uint8, device=dev)
             r.src_ids = torch.full((caps[L],), -1, **i64)
             pre = SimpleNamespace(rows=r.x_pre, have=r.have, src_ids=r.src_ids)
@@ -133,8 +147,12 @@ class RecordedIteration:
             arrays.append((batch.edge_type, r.etype, n_edges, -1))
         if handle is not None:
             torch.cuda.current_stream(self.device).wait_event(handle.done)
-            arrays += [(handle.rows.view(-1), r.x_pre.view(-1), n_all * r.x_pre.shape[1], 0),
-                       (handle.mask.view(torch.uint8), r.have, n_all, 0), (handle.src_ids, r.src_ids, n_all, -1)]
+            if handle.rows.data_ptr() == r.x_pre.data_ptr():       # read straight into this array: clear what lies behind
+                if n_all < r.x_pre.shape[0]:
+                    arrays.append((None, r.x_pre[n_all:].view(-1), 0, 0))
+            else:
+                arrays.append((handle.rows.view(-1), r.x_pre.view(-1), n_all * r.x_pre.shape[1], 0))
+            arrays += [(handle.mask.view(torch.uint8), r.have, n_all, 0), (handle.src_ids, r.src_ids, n_all, -1)]
             batch.prefetched_x = None
         _be.stage_arrays(arrays, r.scal, [int(v) for v in nnl] + [n_edges, int(now), int(it)])
 
@@ -142,7 +160,21 @@ class RecordedIteration:
         """Start the host-link read of ``batch``'s feature rows now, under the cache's present state, on the
         feature store's read-ahead stream: it then runs beside the iteration that is replayed next, and the
         iteration on ``batch`` reads only the rows that an admission has made necessary since."""
-        self.cache.prefetch(batch, speculative=True, num_layer=self.L)
+        out = None
+        store = self.cache.uvm
+        nnl, n_edges, view_kind, etype = self._describe(batch)
+        j = self._key_for(nnl, n_edges)
+        if j is not None and self.read_ahead_slots > 1 and hasattr(store, "out_dtype") and hasattr(store, "buffer"):
+            slot = self._reads_started % self.read_ahead_slots
+            self._reads_started += 1
+            key = (j, view_kind, slot, etype is not None)
+            r = self._records.get(key)
+            if r is None and len(self._records) < self.max_records:
+                r = self._records[key] = self._new_record(j, view_kind, (store.buffer.shape[1], store.out_dtype), etype)
+            if r is not None:
+                out = r.x_pre[: nnl[self.L]]
+                batch.recorded_key = key
+        self.cache.prefetch(batch, speculative=True, num_layer=self.L, out=out)
 
     def _iteration(self, b):
         self.cache.lookup_and_load(b, self.L)
@@ -159,23 +191,26 @@ class RecordedIteration:
         """Train on ``batch`` (as ``NeighborSampler`` or ``hiscache.synthetic.make_batch`` hand it over);
         ``glb_iter`` is the iteration number the admitted rows are stamped with.  Returns the loss (a device
         tensor that the next call with the same shape overwrites)."""
-        nnl = [int(v) for v in batch.num_node_in_layer]
-        n_edges = int(batch.idx.numel())
-        view = getattr(batch, "view", None) if self.with_view else None
-        if view is not None and (view.rows < nnl[self.L - 1] or view.n_src < nnl[self.L]):
-            view = None
+        nnl, n_edges, view_kind, etype = self._describe(batch)
         handle = getattr(batch, "prefetched_x", None)
         if handle is not None and (handle.ids is not batch.sub_to_full or handle.mask is None
                                    or handle.rows.element_size() not in (4, 2)):
             handle = None
         j = self._key_for(nnl, n_edges)
         self.cache.glb_iter += 1
-        view_kind = 0 if view is None else (2 if view.edgeT is not None else 1)
-        etype = getattr(batch, "edge_type", None)
-        key = None if j is None else (j, view_kind, handle is not None, etype is not None)
+        key = None
+        if j is not None:
+            # slot -1: no rows read ahead; -2: rows read ahead into a tensor of their own (copied in by the staging
+            # launch); 0, 1, ..: read straight into the array of that one of the shape's recordings
+            key = (j, view_kind, -1 if handle is None else -2, etype is not None)
+            own = getattr(batch, "recorded_key", None)
+            if handle is not None and own is not None and own[:2] == key[:2] and own in self._records \
+                    and self._records[own].x_pre.data_ptr() == handle.rows.data_ptr():
+                key = own
         r = None if key is None else self._records.get(key)
         if r is None and key is not None and len(self._records) < self.max_records:
-            r = self._records[key] = self._new_record(j, view_kind, handle, etype)
+            pre_like = None if handle is None else (handle.rows.shape[1], handle.rows.dtype)
+            r = self._records[key] = self._new_record(j, view_kind, pre_like, etype)
         if r is None:
             # a shape outside the family, or more shapes than recordings are kept for: the ordinary iteration
             self.cache.glb_iter -= 1
@@ -208,6 +243,7 @@ class RecordedIteration:
         return r.loss
 
     def shapes(self):
-        """The padded shapes in use: {(j, view kind 0/1/2 = none/rows/rows and edge slots, rows read ahead,
-        edge types given): ([n0 .. nL], edges, recorded?, uses)}."""
+        """The padded shapes in use: {(j, view kind 0/1/2 = none/rows/rows and edge slots, read-ahead slot (-1: no
+        rows read ahead, -2: copied in, 0..: read straight into that recording's array), edge types given):
+        ([n0 .. nL], edges, recorded?, uses)}."""
         return {k: (r.caps, r.e_cap, r.graph is not None, r.uses) for k, r in self._records.items()}

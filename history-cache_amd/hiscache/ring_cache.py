@@ -107,7 +107,7 @@ class RingHistoryCache:
         batch.x = self.uvm.masked_get(sub_to_full, self.used_masks[0])
         return None
 
-    def prefetch(self, batch, speculative=True, num_layer=None):
+    def prefetch(self, batch, speculative=True, num_layer=None, out=None):
         """Start the host-link read of ``batch``'s feature rows now, to overlap it with the work queued
         before that batch's ``lookup_and_load``.  ``speculative``: only the rows that the cache's PRESENT
         state makes necessary are read (a lookup and the used masks, as ``lookup_and_load`` computes
@@ -128,7 +128,8 @@ class RingHistoryCache:
                                   now=self.glb_iter + 1, age_limit=self.age_limit, want_rows=False)
         masks = _be.count_history_reconstruct(batch.ptr, batch.idx, slot, sub_to_full.shape[0],
                                               batch.y.shape[0], num_layer)
-        batch.prefetched_x = start(sub_to_full, masks[0])
+        # ``out`` (recorded iterations): the rows go straight into the array the recording reads them from
+        batch.prefetched_x = start(sub_to_full, masks[0]) if out is None else start(sub_to_full, masks[0], out=out)
 
     @torch.no_grad()
     def update_history(self, batch, glb_iter):

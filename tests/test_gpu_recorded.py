@@ -204,8 +204,8 @@ def test_replayed_iterations_equal_the_padded_ones(L, fanout, thres, read_ahead)
         return [sampler.sample(seeds[k], rng_seed=1000 + k) for k in order]
 
     worlds = {name: make_world(11, *args) for name in ("recorded", "padded", "plain")}
-    rec = RecordedIteration(*[worlds["recorded"][k] for k in (1, 0, 2)], L, step=1.02, round_to=64)
-    pad = RecordedIteration(*[worlds["padded"][k] for k in (1, 0, 2)], L, step=1.02, round_to=64, record=False)
+    rec = RecordedIteration(*[worlds["recorded"][k] for k in (1, 0, 2)], L, step=1.005, round_to=16)
+    pad = RecordedIteration(*[worlds["padded"][k] for k in (1, 0, 2)], L, step=1.005, round_to=16, record=False)
     cache_p, model_p, opt_p = worlds["plain"]
     sets = {name: batches() for name in worlds}
     for name in ("ptr", "idx", "sub_to_full"):
@@ -235,8 +235,8 @@ def test_replayed_iterations_equal_the_padded_ones(L, fanout, thres, read_ahead)
             losses["plain"].append(float(loss.detach()))
     torch.cuda.synchronize()
     shapes = rec.shapes()
-    assert rec.replays >= len(order) // 2 and sum(1 for v in shapes.values() if v[2]) >= 2, shapes
-    assert all(k[2] == read_ahead for k, v in shapes.items() if v[2])
+    assert rec.replays >= len(order) // 3 and sum(1 for v in shapes.values() if v[2]) >= 2, shapes
+    assert all((k[2] >= 0) == read_ahead for k, v in shapes.items() if v[2])      # rows read straight into place
     np.testing.assert_allclose(losses["recorded"], losses["plain"], rtol=2e-3)
     for p, q in zip(worlds["recorded"][1].parameters(), model_p.parameters()):
         assert float((p - q).detach().abs().max()) < 2e-2 * float(q.detach().abs().max())
@@ -309,7 +309,7 @@ def test_replayed_relational_iterations_equal_the_padded_ones():
     twins = {}
     for name, record in (("recorded", True), ("padded", False)):
         cache, model, opt = world()
-        twins[name] = (cache, model, opt, RecordedIteration(model, cache, opt, L, step=1.02, round_to=64, record=record),
+        twins[name] = (cache, model, opt, RecordedIteration(model, cache, opt, L, step=1.005, round_to=16, record=record),
                        [sampler.sample(seeds[k], rng_seed=500 + k) for k in order])
     compute = torch.cuda.Stream()
     compute.wait_stream(torch.cuda.current_stream())
@@ -328,6 +328,6 @@ def test_replayed_relational_iterations_equal_the_padded_ones():
             torch.zeros(1000, device=DEV).sum().item()           # eager work and a synchronisation in between
     rec = twins["recorded"][3]
     shapes = rec.shapes()
-    assert rec.replays >= len(order) // 2, shapes
-    assert all(k[1] == 2 and k[2] for k, v in shapes.items() if v[2])     # view with edge slots, rows read ahead
+    assert rec.replays >= len(order) // 3, shapes
+    assert all(k[1] == 2 and k[2] >= 0 for k, v in shapes.items() if v[2])     # view with edge slots, rows read ahead
     assert int((twins["recorded"][0].full2slot != -1).sum()) > cached.numel()   # rows were admitted
