@@ -42,7 +42,7 @@ class _Record:
 class RecordedIteration:
 
     def __init__(self, model, cache, optimizer, num_layers, loss_fn=None, step=1.125, round_to=256,
-                 max_records=12, with_view=True, record=True, read_ahead_slots=2):
+                 max_records=16, with_view=True, record=True, read_ahead_slots=2):
         self.model, self.cache, self.optimizer = model, cache, optimizer
         self.L = int(num_layers)
         self.loss_fn = loss_fn or torch.nn.functional.nll_loss
@@ -241,6 +241,10 @@ class RecordedIteration:
         r.graph.replay()
         self.replays += 1
         return r.loss
+
+    def clear(self):
+        """Drop every recording and its arrays (they are made again on demand)."""
+        self._records.clear()
 
     def shapes(self):
         """The padded shapes in use: {(j, view kind 0/1/2 = none/rows/rows and edge slots, read-ahead slot (-1: no
