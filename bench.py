@@ -289,8 +289,8 @@ def run_c2(args, row_mode=False):
     full_grad = None
     if not row_mode:
         # The same step when the history table wants its gradient too: no source is left out, the view holds all E
-        # edges and the backward gathers a gradient row for every one of them (the backward that BASELINE.md
-        # prices at E*F*4 + E*8 + (N+1)*8 + R*4 + N*F*4 bytes).  Timed with the forward beside it, so that the
+        # edges and the backward gathers a gradient row for every one of them (a backward of
+        # E*F*4 + E*8 + (N+1)*8 + R*4 + N*F*4 algorithmic bytes).  Timed with the forward beside it, so that the
         # three parts come from the same stretch of the run.
         ck_f, ck_t, ck_b = KernelClock(), KernelClock(), KernelClock()
 
