@@ -331,3 +331,33 @@ def test_replayed_relational_iterations_equal_the_padded_ones():
     assert rec.replays >= len(order) // 3, shapes
     assert all(k[1] == 2 and k[2] >= 0 for k, v in shapes.items() if v[2])     # view with edge slots, rows read ahead
     assert int((twins["recorded"][0].full2slot != -1).sum()) > cached.numel()   # rows were admitted
+
+
+def test_recorded_iterations_with_dropout_train():
+    """Dropout inside a recording draws from torch's graph-safe generator: the replays train (the loss falls over
+    repeated passes) and stay finite.  (Their random stream is not the eager one, so no twin is compared.)"""
+    from helpers import power_law_graph
+    from hiscache import (HistorySAGE, NeighborSampler, PinnedFeatureStore, RecordedIteration, RingHistoryCache,
+                          make_config, prefer_low_latency_gemm)
+    N, Fin, H, C, L = 20_000, 64, 64, 4, 2          # two layers: the cached rows have the input's width
+    rng = np.random.default_rng(4)
+    indptr, indices = power_law_graph(rng, N, 4.0, alpha=2.0, max_degree=200)
+    feats_np = rng.standard_normal((N, Fin)).astype(np.float32)
+    labels_np = (feats_np[:, :C].argmax(1)).astype(np.int64)            # learnable from a node's own features
+    prefer_low_latency_gemm()
+    torch.manual_seed(4)
+    cache = RingHistoryCache(PinnedFeatureStore(torch.from_numpy(feats_np), device=DEV), N, Fin, H, capacity=N,
+                             num_layers=L, table_dtype=torch.float32, rate=0.3, age_limit=2, device=DEV)
+    model = HistorySAGE(Fin, H, C, L, 0.3, "CSR_Layer", make_config(Fin, C, H, L, device=DEV, dropout=0.3), cache).to(DEV)
+    model.train()
+    opt = torch.optim.Adam(model.parameters(), lr=1e-2, fused=True, capturable=True)
+    sampler = NeighborSampler(indptr, indices, [6, 4], labels=torch.from_numpy(labels_np), seed=4, device=DEV,
+                              emit_view=True)
+    rec = RecordedIteration(model, cache, opt, L)
+    gen = torch.Generator(device=DEV).manual_seed(4)
+    losses = []
+    for it in range(1, 61):
+        seeds = torch.randperm(N, device=DEV, generator=gen)[:256].contiguous()
+        losses.append(float(rec(sampler.sample(seeds), it)))
+    assert all(np.isfinite(losses)) and rec.replays >= 50
+    assert np.mean(losses[-10:]) < 0.8 * np.mean(losses[:5]), (losses[:5], losses[-10:])
