@@ -159,11 +159,14 @@ class HistoryCache:
         and overwritten embedding slots are invalidated; maps and header advance."""
         if "history" not in self.feat_mode or self.staleness_thres == 0:
             return
-        if glb_iter < self.start_history:
-            return
-        if (glb_iter % self.staleness_thres) == 0:
-            torch.maximum(self._num_stored, self._header, out=self._num_stored)
-            self._header.zero_()
+        # A batch padded to fixed sizes for a recorded iteration (hiscache.RecordedIteration) carries its real
+        # sizes on the device; what depends on the iteration number on the HOST -- whether admission has started,
+        # the periodic restart of the write position -- is then done by ``before_update``, outside the recording.
+        dev = getattr(batch, "dev", None)
+        if dev is None:
+            if glb_iter < self.start_history:
+                return
+            self._restart_if_due(glb_iter)
         if self.produced_embedding is None:
             raise AssertionError("produced embedding is None")
         emb = self.produced_embedding
@@ -180,15 +183,38 @@ class HistoryCache:
         else:
             score = torch.randn([num_node], device=self.device)
         emb.grad = None
-        thres = quantile_threshold(score, self.rate)
+        if dev is None:
+            thres = quantile_threshold(score, self.rate)
+        else:
+            # the threshold is the quantile of the real rows' scores; a padding row never passes it
+            thres = _be.quantile_select_dev(score, dev.nnl[1], self.rate)
+            score = torch.where(dev.row_index[:num_node] < dev.nnl[1], score, torch.full_like(score, float("inf")))
         mask = _be.cache_append(score, thres, emb.detach().contiguous(), self.sub2embed,
                                 batch.sub_to_full[:num_node].contiguous(), self.buffer,
                                 self.hidden_channels, self.in_channels, self.full2embed,
                                 self.embed2full, self.feat2full, self._header, self._overflow)
         self.last_record_mask = mask
-        self._uncounted_mask = mask
+        self._uncounted_mask = mask if dev is None else None
         self.last_score = score
         self.produced_embedding = None
+
+    def _restart_if_due(self, glb_iter):
+        """Every ``staleness_thres`` iterations the write position goes back to the start of the buffer
+        (/root/reference/hiscache/history_cache.py:190-198)."""
+        if (glb_iter % self.staleness_thres) == 0:
+            torch.maximum(self._num_stored, self._header, out=self._num_stored)
+            self._header.zero_()
+
+    def before_update(self, glb_iter):
+        """For recorded iterations: the part of ``update_history`` that the host decides from the iteration number,
+        run in front of the replay (the lookup does not read the write position, so the order does not matter).
+        False when admission has not started yet at ``glb_iter``: that iteration is not one to replay."""
+        if "history" not in self.feat_mode or self.staleness_thres == 0:
+            return True
+        if glb_iter < self.start_history:
+            return False
+        self._restart_if_due(glb_iter)
+        return True
 
     # ------------------------------------------------------------------ lookup
     def lookup_and_load(self, batch, num_layer=None, feature_cache_only=False):
@@ -221,14 +247,30 @@ class HistoryCache:
         layer1_nodes = sub_to_full[:n1]
         self.sub2embed = _be.lookup(self.full2embed, layer1_nodes, 0)
         self.sub2feat = _be.lookup(self.full2embed, sub_to_full, self.total_num_node)
+        dev = getattr(batch, "dev", None)
+        if dev is not None:
+            # a padded batch (recorded iterations): the rows behind the real 1-hop nodes are real nodes of the next
+            # hop or padding, and count as not cached; so do the padding nodes for the feature cache
+            minus = torch.full_like(self.sub2embed[:1], -1)
+            self.sub2embed = torch.where(dev.row_index[:n1] < dev.nnl[1], self.sub2embed, minus)
+            self.sub2feat = torch.where(dev.row_index[: sub_to_full.shape[0]] < dev.nnl[-1], self.sub2feat, minus)
         self.used_masks = _be.count_history_reconstruct(batch.ptr, batch.idx, self.sub2embed,
                                                         sub_to_full.shape[0], batch.y.shape[0],
                                                         num_layer)
         # hit_feat = sub2feat != -1, load = used & ~hit_feat (reference :327-330) and the hit counters, one launch
+        # (the counters are not kept for recorded iterations)
         hit_feat_mask, load_mask = _be.load_mask(self.used_masks[0], self.sub2feat, self.sub2embed,
-                                                 self._counted_mask(), self._counters)
-        self.glb_iter += 1
-        pre, exact = self._take_prefetched(batch, load_mask)
+                                                 self._counted_mask() if dev is None else None,
+                                                 self._counters if dev is None else None)
+        if dev is None:
+            self.glb_iter += 1
+        if dev is not None and getattr(dev, "prefetched", None) is not None:
+            # rows read ahead of time into the recording's own arrays, under the masks of an earlier cache state
+            p = dev.prefetched
+            _be.fixup_rows(self.uvm.buffer, p.src_ids, load_mask, p.have, p.rows)
+            pre, exact = p.rows, True
+        else:
+            pre, exact = self._take_prefetched(batch, load_mask)
         if pre is not None and not exact:
             # every row was read ahead of time: keep what masked_get + the feature-cache merge would have
             # produced (needed rows and feature-cache hits), zero the rest
@@ -254,7 +296,7 @@ class HistoryCache:
         self.load_mask = load_mask
         return None
 
-    def prefetch(self, batch, speculative=True, num_layer=None):
+    def prefetch(self, batch, speculative=True, num_layer=None, out=None):
         """Start the host-link read of ``batch``'s feature rows now, to overlap it with the work queued
         before that batch's ``lookup_and_load``.  ``speculative``: the rows that the cache's PRESENT state
         makes necessary (slots, used masks and feature-cache hits as ``lookup_and_load`` computes them, one
@@ -275,7 +317,9 @@ class HistoryCache:
         sub2feat = _be.lookup(self.full2embed, sub_to_full, self.total_num_node)
         used = _be.count_history_reconstruct(batch.ptr, batch.idx, sub2embed, sub_to_full.shape[0],
                                              batch.y.shape[0], num_layer)
-        batch.prefetched_x = start(sub_to_full, torch.logical_and(used[0], sub2feat == -1))
+        mask = torch.logical_and(used[0], sub2feat == -1)
+        # ``out`` (recorded iterations): the rows go straight into the array the recording reads them from
+        batch.prefetched_x = start(sub_to_full, mask) if out is None else start(sub_to_full, mask, out=out)
 
     def _take_prefetched(self, batch, need):
         """(rows, exact): the rows of a read-ahead of this batch, or (None, False).  ``exact``: they were

@@ -21,7 +21,7 @@ What stands in the way is that no two sampled batches have the same sizes, so:
   recording).
 
 The model is a ``HistorySAGE`` or a ``HistoryRGCN`` in training mode with the fused epilogue, the cache a
-``RingHistoryCache`` that admits by gradient, the optimizer one whose step can be recorded
+``RingHistoryCache`` or a ``HistoryCache`` that admits by gradient, the optimizer one whose step can be recorded
 (``capturable=True``).  The cache's hit counters are not kept for recorded iterations.
 """
 import math
@@ -197,6 +197,11 @@ class RecordedIteration:
                                    or handle.rows.element_size() not in (4, 2)):
             handle = None
         j = self._key_for(nnl, n_edges)
+        # what a cache decides on the host from the iteration number (HistoryCache: has admission started, the
+        # periodic restart of its write position) happens here, in front of the replay
+        hook = getattr(self.cache, "before_update", None)
+        if hook is not None and not hook(glb_iter):
+            j = None
         self.cache.glb_iter += 1
         key = None
         if j is not None:

@@ -361,3 +361,68 @@ def test_recorded_iterations_with_dropout_train():
         losses.append(float(rec(sampler.sample(seeds), it)))
     assert all(np.isfinite(losses)) and rec.replays >= 50
     assert np.mean(losses[-10:]) < 0.8 * np.mean(losses[:5]), (losses[:5], losses[-10:])
+
+
+@pytest.mark.parametrize("read_ahead", [False, True])
+def test_replayed_iterations_with_the_flat_cache_equal_the_padded_ones(read_ahead):
+    """``HistoryCache`` (the reference's flat buffer with a feature cache in its tail, append-only admission, the
+    write position restarted every ``staleness_thres`` iterations): replayed and padded-but-unrecorded twins hold
+    the same bits after every iteration, the restart included."""
+    from helpers import power_law_graph
+    from hiscache import (HistoryCache, HistorySAGE, NeighborSampler, PinnedFeatureStore, RecordedIteration,
+                          make_config, prefer_low_latency_gemm)
+    N, Fin, H, C, L, n_seed, fanout = 30_000, 64, 64, 6, 3, 200, [6, 4, 3]
+    rng = np.random.default_rng(31)
+    indptr, indices = power_law_graph(rng, N, 4.0, alpha=2.0, max_degree=300)
+    feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32))
+    labels = torch.from_numpy(rng.integers(0, C, size=N))
+    hot = rng.permutation(N).astype(np.int64)
+    prefer_low_latency_gemm()
+
+    def world():
+        torch.manual_seed(17)
+        cfg = make_config(Fin, C, H, L, method="grad", rate=0.5, staleness_thres=4, device=DEV)
+        cache = HistoryCache(PinnedFeatureStore(feats, device=DEV), cfg, "history_uvm", total_num_node=N,
+                             buffer_bytes=6000 * 64 * 4, hot_ids=hot)
+        model = HistorySAGE(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache).to(DEV)
+        model.train()
+        opt = torch.optim.Adam(model.parameters(), lr=1e-2, fused=True, capturable=True)
+        return cache, model, opt
+
+    def state(cache, model, opt):
+        out = [p.detach().clone() for p in model.parameters()] + [b.clone() for b in model.buffers()]
+        out += [cache.buffer.clone(), cache.full2embed.clone(), cache.embed2full.clone(), cache._header.clone(),
+                cache._num_stored.clone()]
+        for st in opt.state.values():
+            out += [st["exp_avg"].clone(), st["exp_avg_sq"].clone()]
+        return out
+
+    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=31, device=DEV, emit_view=True)
+    gen = torch.Generator(device=DEV).manual_seed(31)
+    seeds = [torch.randperm(N, device=DEV, generator=gen)[:n_seed].contiguous() for _ in range(5)]
+    order = [0, 1, 2, 0, 3, 1, 4, 0, 2, 3, 1, 0]
+    twins = {}
+    for name, record in (("recorded", True), ("padded", False)):
+        cache, model, opt = world()
+        twins[name] = (cache, model, opt, RecordedIteration(model, cache, opt, L, step=1.005, round_to=16, record=record),
+                       [sampler.sample(seeds[k], rng_seed=700 + k) for k in order])
+    compute = torch.cuda.Stream()
+    compute.wait_stream(torch.cuda.current_stream())
+    admitted = []
+    with torch.cuda.stream(compute):
+        for i in range(len(order)):
+            losses = []
+            for name in ("recorded", "padded"):
+                cache, model, opt, runner, bs = twins[name]
+                if read_ahead and i + 1 < len(order):
+                    runner.prefetch(bs[i + 1])
+                losses.append(float(runner(bs[i], i + 1)))
+            assert losses[0] == losses[1] and np.isfinite(losses[0])
+            a, c = state(*twins["recorded"][:3]), state(*twins["padded"][:3])
+            same = [bool(torch.equal(x, y)) for x, y in zip(a, c)]
+            assert all(same), (i, same)
+            admitted.append(twins["recorded"][0].header)
+    rec = twins["recorded"][3]
+    assert rec.replays >= len(order) // 3, rec.shapes()
+    assert admitted[2] > 0 and admitted[3] < admitted[2]          # iteration 4 restarted the write position
+    assert twins["recorded"][0].glb_iter == len(order)
