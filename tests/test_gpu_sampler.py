@@ -148,6 +148,41 @@ def test_training_from_processed_files(tmp_path, in_device_memory):
     assert cache.header > 0
 
 
+def test_recorded_training_from_processed_files(tmp_path):
+    """The same pipeline with the sampler replayed from its slots and the iteration recorded and replayed
+    (hiscache.RecordedIteration): dataset directory -> store, sampler, HistoryCache from the files, get_model ->
+    thirty iterations; the loss falls on labels that a node's own features decide, rows are admitted."""
+    from hiscache import HistoryCache, ProcessedDataset, RecordedIteration, get_model, make_config, write_processed
+    rng = np.random.default_rng(231)
+    N, Fin, H, C, L = 6000, 32, 32, 4, 3
+    indptr, indices = simple_graph(rng, N, 10)
+    feats = rng.standard_normal((N, Fin)).astype(np.float32)
+    labels = feats[:, :C].argmax(1).astype(np.int64)
+    write_processed(tmp_path, indptr, indices, feats, hot_ids=rng.permutation(N), labels=labels,
+                    train_idx=rng.permutation(N)[:4500])
+    ds = ProcessedDataset(tmp_path, Fin)
+    store = ds.feature_store(device=DEV)
+    sampler = ds.sampler([4, 3, 2], device=DEV, seed=2, emit_view=True, replay_slots=3)
+    cfg = make_config(Fin, C, H, L, method="grad", rate=0.6, staleness_thres=5, device=DEV, path=str(tmp_path))
+    cache = HistoryCache(store, cfg, "history_uvm", buffer_bytes=1500 * int(np.lcm(Fin, H)) * 4)
+    torch.manual_seed(231)
+    model = get_model(cfg, cache).to(DEV).train()
+    opt = torch.optim.Adam(model.parameters(), lr=1e-2, fused=True, capturable=True)
+    step = RecordedIteration(model, cache, opt, L)
+    train = torch.from_numpy(ds.train_idx()).to(DEV)
+    pending = sampler.sample_async(train[:150])
+    losses, stored = [], 0
+    for it in range(1, 30):
+        batch = pending.get()
+        pending = sampler.sample_async(train[150 * it: 150 * (it + 1)])
+        losses.append(float(step(batch, it)))
+        stored = max(stored, cache.header)
+    pending.get()
+    assert all(np.isfinite(losses)) and step.replays >= 20, step.shapes()
+    assert np.mean(losses[-5:]) < 0.8 * np.mean(losses[:3]), losses
+    assert stored > 0 and cache.glb_iter == 29
+
+
 @pytest.mark.parametrize("view_edges", [False, True])
 def test_replayed_sampling_equals_the_launched_one(orc, view_edges):
     """NeighborSampler(replay_slots=K): the launches of a batch recorded once per slot in a HIP graph and
