@@ -98,6 +98,9 @@ __device__ __forceinline__ void bwd_accumulate(const int64_t *__restrict__ ptr, 
     if (lane < n) {
       my_row = bwd_live_row<MASKED>(rowT[base + lane], hmap, R);
       if (!MASKED || my_row >= 0) my_deg = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
+      // a row that the layer's own offsets leave empty (a batch padded for a recorded iteration keeps the rows
+      // behind a layer's real ones empty, while the batch's shared view still lists their edges) is stepped over
+      if (MASKED && my_row >= 0 && my_deg == 0.0f) my_row = -1;
     }
     // the staged edges that count, lowest position first (all of them without a mask)
     unsigned long long todo = MASKED ? __ballot(lane < n && my_row >= 0)
@@ -336,6 +339,8 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_mean_fast(
       if constexpr (WMODE == W_EDGE_HEAD) my_edge = edgeT[base + lane];
       else if constexpr (WMODE == W_EDGE) my_deg = ev[edgeT[base + lane]];   // the weight takes the divisor's place
       else if (!MASKED || my_row >= 0) my_deg = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
+      // a row that the layer's own offsets leave empty is stepped over (see bwd_accumulate)
+      if (MASKED && WMODE == W_NONE && my_row >= 0 && my_deg == 0.0f) my_row = -1;
     }
     // MASKED: only the live edges of the stage are visited (lowest position first), so that UNROLL rows are
     // in flight however many edges of other layers lie between them
@@ -435,7 +440,11 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_generic(
           my_row = -1;
         if (my_row < 0) my_s = 1.0f;
         else if (WEIGHTED) my_s = ev[(int64_t)edgeT[base + lane] * H + head];
-        else my_s = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
+        else {
+          my_s = (float)(int)(ptr[my_row + 1] - ptr[my_row]);
+          // a row that the layer's own offsets leave empty is stepped over (see bwd_accumulate)
+          if (mask_rows >= 0 && my_s == 0.0f) { my_row = -1; my_s = 1.0f; }
+        }
       }
       constexpr int GEN_UNROLL = 4;  // gradient rows in flight before the first add (order kept)
       for (int j = 0; j < n; j += GEN_UNROLL) {
@@ -818,10 +827,10 @@ __global__ __launch_bounds__(HC_BLOCK) void bwd_typed_batch_view(
       const int64_t e = edgeT[base + lane];
       if (row < R && e < E) {
         const int64_t rel = et[e];
-        if (rel >= 0 && rel < K) {
+        const int64_t d = ptr[row + 1] - ptr[row];      // 0: a row that the layer's own offsets leave empty
+        if (rel >= 0 && rel < K && d > 0) {
           my_group = row * K + rel;
-          const int64_t d = ptr[row + 1] - ptr[row];
-          my_w = 1.0f / (float)(d > 0 ? d : 1);
+          my_w = 1.0f / (float)d;
         }
       }
     }

@@ -230,11 +230,11 @@ __global__ __launch_bounds__(HC_BLOCK) void ring_lookup_kernel(
 
 inline unsigned blocks_for(int64_t n) { return (unsigned)((n + HC_BLOCK - 1) / HC_BLOCK); }
 
-// Staging of a batch into arrays of fixed size: dst[i] = i < n_copy ? src[i] : fill for up to twelve arrays
+// Staging of a batch into arrays of fixed size: dst[i] = i < n_copy ? src[i] : fill for up to sixteen arrays
 // of 8-, 4-, 2- or 1-byte elements (integers; rows of floats go through as their bit patterns with fill 0), and
 // a handful of 64-bit scalars (the batch's sizes, the iteration number) written to device memory, all in one
 // launch.
-constexpr int STAGE_MAX_ARRAYS = 12;
+constexpr int STAGE_MAX_ARRAYS = 16;
 constexpr int STAGE_MAX_SCALARS = 16;
 struct StagePlan {
   const void *src[STAGE_MAX_ARRAYS];

@@ -256,25 +256,28 @@ class HistorySAGE(torch.nn.Module):
         view = getattr(batch, "view", None)                  # shared transposed view, if the loader emitted it
         # a batch padded to fixed sizes for a recorded iteration carries its real sizes on the device
         dev = getattr(batch, "dev", None)
+        # ... and row offsets per layer, flat behind the layer's real rows (see hiscache.RecordedIteration)
+        ptrs = getattr(batch, "ptr_of_layer", None)
         for i, conv in enumerate(self.convs[:-1]):
             k = self.num_layers - 1 - i
             n = batch.num_node_in_layer[k]
             ne = None if nel is None else int(nel[k])
+            ptr = batch.ptr if ptrs is None else ptrs[k]
             # the bias of lin_l goes to the normalisation's kernels instead of a launch of its own
             defer = self.fused_epilogue and conv.fused and self.training and x.is_cuda
             if self.training and i == self.num_layers - 2:
                 # the layer whose output is one hop from the seeds uses (and produces) history
-                x, his = conv(x, batch.ptr, batch.idx, self.table.sub2embed,
+                x, his = conv(x, ptr, batch.idx, self.table.sub2embed,
                               self.table.cached_embedding, self.hidden_channels, n, ne, add_bias=not defer,
                               view=view)
                 self.table.produced_embedding = his
             else:
-                x, his = conv(x, batch.ptr, batch.idx, none, none, 0, n, ne, add_bias=not defer, view=view)
+                x, his = conv(x, ptr, batch.idx, none, none, 0, n, ne, add_bias=not defer, view=view)
             x = bn_relu(x, self.bns[i], conv.lin_l.bias if defer else None, fused=self.fused_epilogue,
                         n_dev=None if dev is None else dev.nnl[k])
             x = F.dropout(x, p=self.dropout, training=self.training)
-        x, his = self.convs[-1](x, batch.ptr, batch.idx, none, none, 0, batch.num_node_in_layer[0],
-                                None if nel is None else int(nel[0]), view=view)
+        x, his = self.convs[-1](x, batch.ptr if ptrs is None else ptrs[0], batch.idx, none, none, 0,
+                                batch.num_node_in_layer[0], None if nel is None else int(nel[0]), view=view)
         return x.log_softmax(dim=-1)
 
     def init_convs(self, **kwargs):
@@ -550,24 +553,27 @@ class HistoryRGCN(torch.nn.Module):
         masks = self.table.used_masks
         view = getattr(batch, "view", None)                  # shared transposed view, if the loader emitted it
         dev = getattr(batch, "dev", None)                    # a padded batch carries its real sizes on the device
+        ptrs = getattr(batch, "ptr_of_layer", None)          # ... and row offsets per layer (see HistorySAGE.forward)
         for i, conv in enumerate(self.convs[:-1]):
             n = batch.num_node_in_layer[L - 1 - i]
             et = etypes[: batch.num_edge_in_layer[L - 1 - i]]
             um = masks[i] if masks is not None else None
+            ptr = batch.ptr if ptrs is None else ptrs[L - 1 - i]
             if self.training and i == L - 2:
-                x, his = conv(x, batch.ptr, batch.idx, et, None, self.table.sub2embed,
+                x, his = conv(x, ptr, batch.idx, et, None, self.table.sub2embed,
                               self.table.cached_embedding, um, self.hidden_channels, n, view=view)
                 self.table.produced_embedding = his
                 if not getattr(his, "_hc_grad_sink", False):
                     self.table.produced_embedding.retain_grad()
             else:
-                x, his = conv(x, batch.ptr, batch.idx, et, None, none, none, um, 0, n, view=view)
+                x, his = conv(x, ptr, batch.idx, et, None, none, none, um, 0, n, view=view)
             x = bn_relu(x, self.bns[i], None, fused=self.fused_epilogue,
                         n_dev=None if dev is None else dev.nnl[L - 1 - i])
             x = F.dropout(x, p=self.dropout, training=self.training)
         um = masks[-2] if masks is not None else None
-        x, his = self.convs[-1](x, batch.ptr, batch.idx, etypes[: batch.num_edge_in_layer[0]], None, none, none,
-                                um, 0, batch.num_node_in_layer[0], view=view)
+        x, his = self.convs[-1](x, batch.ptr if ptrs is None else ptrs[0], batch.idx,
+                                etypes[: batch.num_edge_in_layer[0]], None, none, none, um, 0,
+                                batch.num_node_in_layer[0], view=view)
         return x.log_softmax(dim=-1)
 
     def reset_parameters(self):

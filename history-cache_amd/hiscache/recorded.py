@@ -8,8 +8,9 @@ What stands in the way is that no two sampled batches have the same sizes, so:
 
 * a batch is PADDED into arrays of fixed sizes (one ``hiscache_backend.stage_arrays`` launch): row offsets
   continued at the edge count, node ids at -1.  Padding rows have no edges, aggregate to zero, are never
-  referenced by a real row and receive no gradient.  A layer may then also compute real rows that it did
-  not need (the rows between its own count and the padded one belong to the next hop): nothing reads them;
+  referenced by a real row and receive no gradient.  Every layer gets row offsets of its own, flat behind its
+  real rows: the rows between a layer's count and the padded one are real rows of the next hop, whose sources
+  lie beyond the layer's input, and have to stay empty for that layer;
 * the sizes a result depends on are read from device memory, where the same launch writes them: the batch
   normalisation counts only the real rows and gives the others a zero output and a zero gradient, the ring
   lookup reports padding as absent, the admission threshold is the quantile of the real rows' scores,
@@ -36,7 +37,7 @@ from .util import backward_on_this_thread
 
 class _Record:
     __slots__ = ("caps", "e_cap", "batch", "scal", "graph", "loss", "uses", "ptr", "idx", "s2f", "y", "ptrT", "rowT",
-                 "edgeT", "etype", "x_pre", "have", "src_ids")
+                 "edgeT", "etype", "x_pre", "have", "src_ids", "ptrs")
 
 
 class RecordedIteration:
@@ -109,6 +110,11 @@ class RecordedIteration:
         r.caps, r.e_cap, r.graph, r.loss, r.uses = caps, e_cap, None, None, 0
         i64 = dict(dtype=torch.int64, device=dev)
         r.ptr = torch.zeros(caps[L - 1] + 1, **i64)
+        # Row offsets of every layer's own: those of the batch up to the layer's real rows, flat behind them.  The
+        # rows between a layer's real count and its padded count are real rows of the NEXT hop, whose sources lie
+        # beyond the layer's input: with the batch's own offsets the layer would aggregate them, reading behind
+        # its input.  (The last entry, the layer that covers every row of the batch, is the batch's array.)
+        r.ptrs = [torch.zeros(caps[k] + 1, **i64) for k in range(L - 1)] + [r.ptr]
         r.idx = torch.zeros(e_cap, **i64)
         r.s2f = torch.full((caps[L],), -1, **i64)
         r.y = torch.zeros(caps[0], **i64)
@@ -128,6 +134,7 @@ class RecordedIteration:
         r.batch = SimpleNamespace(
             ptr=r.ptr, idx=r.idx, sub_to_full=r.s2f, y=r.y, x=None, edge_type=r.etype, typed_num_node_in_layer=None,
             num_node_in_layer=torch.tensor(caps, dtype=torch.int64), num_edge_in_layer=[e_cap] * L, view=view,
+            ptr_of_layer=r.ptrs,
             dev=SimpleNamespace(nnl=[r.scal[k:k + 1] for k in range(L + 1)], edges=r.scal[L + 1:L + 2],
                                 now=r.scal[L + 2:L + 3], it=r.scal[L + 3:L + 4],
                                 row_index=torch.arange(caps[L], **i64), prefetched=pre))
@@ -138,6 +145,8 @@ class RecordedIteration:
         n_rows, n_all = int(nnl[L - 1]), int(nnl[L])
         arrays = [(batch.ptr, r.ptr, n_rows + 1, n_edges), (batch.idx, r.idx, n_edges, 0),
                   (batch.sub_to_full, r.s2f, n_all, -1), (batch.y, r.y, int(nnl[0]), 0)]
+        nel = batch.num_edge_in_layer                  # edges of the first nnl[k] rows
+        arrays += [(batch.ptr, r.ptrs[k], int(nnl[k]) + 1, int(nel[k])) for k in range(L - 1)]
         if r.ptrT is not None:
             v = batch.view
             arrays += [(v.ptrT, r.ptrT, n_all + 1, n_edges), (v.rowT, r.rowT, n_edges, 0)]

@@ -706,14 +706,14 @@ def quantile_select_dev(score, n_dev, rate):
 
 def stage_arrays(arrays, scalars_dst=None, scalars=()):
     """One launch that pads arrays into fixed-size ones and writes a few int64 scalars to device memory.
-    ``arrays``: up to 12 tuples (src, dst, n_copy, fill) of contiguous device tensors, src of dst's dtype
+    ``arrays``: up to 16 tuples (src, dst, n_copy, fill) of contiguous device tensors, src of dst's dtype
     (elements of 8, 4, 2 or 1 bytes; they are moved as bit patterns): dst.view(-1)[i] = src.view(-1)[i] for
     i < n_copy, ``fill`` (an integer; 0 for floating-point data) behind.  ``scalars`` (up to 16 Python ints) go
     to ``scalars_dst[:len(scalars)]``."""
     lib = load_library()
     k = len(arrays)
-    if k > 12 or len(scalars) > 16:
-        raise ValueError("at most 12 arrays and 16 scalars per call")
+    if k > 16 or len(scalars) > 16:
+        raise ValueError("at most 16 arrays and 16 scalars per call")
     P, I64 = ctypes.c_void_p * max(k, 1), ctypes.c_int64 * max(k, 1)
     src, dst, n_copy, n_total, fill = P(), P(), I64(), I64(), I64()
     elem = (ctypes.c_int * max(k, 1))()

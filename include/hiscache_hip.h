@@ -616,12 +616,15 @@ int hc_weight_grad(const float *g, const float *x0, const float *x1, int64_t n, 
  * kernels included.
  *
  * hc_stage_arrays: dst[a][i] = i < n_copy[a] ? src[a][i] : fill[a] for
- * i in [0, n_total[a]) and up to 12 arrays of elements of 8, 4, 2 or 1 bytes
+ * i in [0, n_total[a]) and up to 16 arrays of elements of 8, 4, 2 or 1 bytes
  * (elem_bytes[a]; integers, or the bit patterns of floating-point rows with
  * fill 0), and scalars_dst[k] = scalars[k] for up to 16 int64 values, in one
  * launch: a batch's arrays padded into fixed-size ones (row offsets continued
  * at the edge count, ids at -1) together with its sizes.  The argument arrays
- * are host arrays, read before the call returns.
+ * are host arrays, read before the call returns.  Every layer of a padded
+ * batch gets row offsets of its own, flat behind the layer's real rows: the
+ * rows between a layer's count and its padded count are real rows of the next
+ * hop, whose sources lie beyond the layer's input, and must stay empty.
  *
  * hc_ring_lookup_dev: hc_ring_lookup with now = *now_dev and ids[i] for
  * i >= *n_valid_dev taken as padding (slot -1, zero row).

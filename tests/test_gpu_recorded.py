@@ -426,3 +426,43 @@ def test_replayed_iterations_with_the_flat_cache_equal_the_padded_ones(read_ahea
     assert rec.replays >= len(order) // 3, rec.shapes()
     assert admitted[2] > 0 and admitted[3] < admitted[2]          # iteration 4 restarted the write position
     assert twins["recorded"][0].glb_iter == len(order)
+
+
+def test_padded_layers_aggregate_nothing_behind_their_real_rows():
+    """In a padded batch the rows between a layer's real count and its padded count are real rows of the next hop:
+    their sources lie behind the layer's input.  Every layer gets row offsets of its own that leave them empty, so
+    its aggregation output is zero there (it read nothing), whatever lies behind the input in memory."""
+    from helpers import power_law_graph
+    from hiscache import NeighborSampler, RecordedIteration, prefer_low_latency_gemm
+    N, Fin, H, C, L = 40_000, 64, 64, 5, 3
+    rng = np.random.default_rng(77)
+    indptr, indices = power_law_graph(rng, N, 4.0, alpha=2.0, max_degree=300)
+    feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32) + 3.0)     # no zero rows by chance
+    labels = torch.from_numpy(rng.integers(0, C, size=N))
+    cached = torch.from_numpy(rng.permutation(N)[: N // 4].copy())
+    rows = torch.from_numpy(rng.standard_normal((cached.numel(), H)).astype(np.float32) + 3.0)
+    prefer_low_latency_gemm()
+    cache, model, opt = make_world(5, 0.5, None, N, Fin, H, C, L, feats, cached, rows)
+    sampler = NeighborSampler(indptr, indices, [6, 4, 3], labels=labels, seed=77, device=DEV, emit_view=True)
+    rec = RecordedIteration(model, cache, opt, L, step=1.3, round_to=512, record=False)   # generous padding
+    gen = torch.Generator(device=DEV).manual_seed(77)
+    seen = []
+    hooks = [conv.register_forward_hook(lambda mod, args, out: seen.append(out[1].detach().clone()))
+             for conv in model.convs]
+    for it in (1, 2):
+        batch = sampler.sample(torch.randperm(N, device=DEV, generator=gen)[:250].contiguous())
+        nnl = [int(v) for v in batch.num_node_in_layer]
+        seen.clear()
+        loss = rec(batch, it)
+        assert np.isfinite(float(loss))
+        (caps, _, _, _), = rec.shapes().values()
+        assert caps[1] > nnl[1] and caps[2] > nnl[2]
+        for i, agg in enumerate(seen):                       # layer i produces the rows of hop L - 1 - i
+            k = L - 1 - i
+            assert agg.shape[0] == caps[k]
+            assert float(agg[nnl[k]:].abs().max() if caps[k] > nnl[k] else 0.0) == 0.0, (it, i)
+            assert float(agg[: nnl[k]].abs().sum()) > 0.0   # (while the real rows were aggregated)
+    for h in hooks:
+        h.remove()
+    for p in model.parameters():
+        assert torch.isfinite(p).all()
