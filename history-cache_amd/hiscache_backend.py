@@ -399,6 +399,17 @@ def build_batch_view(ptr, idx, num_node, n_src, num_edge=None, want_edges=False)
     return BatchView(ptrT, rowT, edgeT, R, n_src, E)
 
 
+def check_batch_view(view, n_src):
+    """Raise ValueError if the first ``n_src`` columns of a batch's transposed view are not valid: column offsets
+    must not decrease and must stay inside ``rowT``, rows inside [0, view.rows) (and edge slots, where the view
+    holds them, inside [0, view.num_edge))."""
+    if view.rowT.dtype != torch.int32:
+        raise ValueError("rowT must be int32")
+    check_csr(view.ptrT, view.rowT.to(torch.int64), n_src, view.rows)
+    if view.edgeT is not None:
+        check_csr(view.ptrT, view.edgeT.to(torch.int64), n_src, max(view.num_edge, 1))
+
+
 def _aggr_bwd_batch_view(ptr, view, g, hmap, hbuf_shape, hsize, num_node, n_src, want_hist_grad=True):
     """Gradient of the mean aggregation over the batch's shared view: (grad_input, grad_history or None)."""
     lib = load_library()
@@ -411,6 +422,8 @@ def _aggr_bwd_batch_view(ptr, view, g, hmap, hbuf_shape, hsize, num_node, n_src,
                          f"the layer has {R} / {n_src}")
     if g.shape[0] < R or (hmap is not None and hmap.numel() < R):
         raise ValueError("grad_output or history_map is shorter than num_node")
+    if CHECK_INPUTS:
+        check_batch_view(view, n_src)
     dev = g.device
     grad_x = torch.empty((n_src, F), dtype=torch.float32, device=dev)
     grad_h = None
@@ -448,6 +461,8 @@ def _aggr_bwd_typed_batch_view(ptr, view, edge_types, num_rel, used_mask, g, num
         used_mask = _dev(used_mask, "used_mask")
         if used_mask.element_size() != 1 or used_mask.numel() < n_src:
             raise ValueError("used_mask must hold one byte per source")
+    if CHECK_INPUTS:
+        check_batch_view(view, n_src)
     E = min(int(edge_types.numel()), view.num_edge)
     grad_x = torch.empty((int(n_src), F), dtype=torch.float32, device=g.device)
     rc = lib.hc_aggr_bwd_batch_view_typed(_ptr(ptr), _ptr(view.ptrT), _ptr(view.rowT), _ptr(view.edgeT),

@@ -466,3 +466,55 @@ def test_padded_layers_aggregate_nothing_behind_their_real_rows():
         h.remove()
     for p in model.parameters():
         assert torch.isfinite(p).all()
+
+
+@pytest.mark.parametrize("relational", [False, True])
+def test_padded_iterations_pass_the_device_side_input_checks(monkeypatch, relational):
+    """With the library's debugging switch on, every aggregation call of a padded iteration first has its row
+    offsets and neighbour ids checked on the device against the layer's input rows, and every backward over the
+    batch's view has the view's columns, rows and edge slots checked: a padded layer that reached behind its
+    input would be reported here instead of reading there."""
+    import hiscache_backend as be
+    from helpers import power_law_graph
+    from hiscache import (HistoryRGCN, NeighborSampler, PinnedFeatureStore, RecordedIteration, RingHistoryCache,
+                          make_config, prefer_low_latency_gemm)
+    N, Fin, H, C, L = 40_000, 64, 64, 5, 3
+    rng = np.random.default_rng(78)
+    indptr, indices = power_law_graph(rng, N, 4.0, alpha=2.0, max_degree=300)
+    feats = torch.from_numpy(rng.standard_normal((N, Fin)).astype(np.float32))
+    labels = torch.from_numpy(rng.integers(0, C, size=N))
+    cached = torch.from_numpy(rng.permutation(N)[: N // 4].copy())
+    rows = torch.from_numpy(rng.standard_normal((cached.numel(), H)).astype(np.float32))
+    prefer_low_latency_gemm()
+    if relational:
+        torch.manual_seed(6)
+        store = PinnedFeatureStore(feats, device=DEV)
+        cache = RingHistoryCache(store, N, Fin, H, capacity=N // 2, num_layers=L, table_dtype=torch.float32,
+                                 thres=0.05, age_limit=3, device=DEV)
+        cache.preload(cached.to(DEV), rows.to(DEV))
+        cfg = make_config(Fin, C, H, L, device=DEV, model_type="rgcn", num_rel=5, name="rmag240m")
+        model = HistoryRGCN(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache, num_rel=5, dataset_name="rmag240m",
+                            type_bounds=[N // 2, N - 1000], pair_to_rel=[[0, 1, 0], [2, 0, 3], [0, 4, 0]]).to(DEV)
+        model.train()
+        opt = torch.optim.Adam(model.parameters(), lr=1e-2, fused=True, capturable=True)
+    else:
+        cache, model, opt = make_world(6, 0.5, None, N, Fin, H, C, L, feats, cached, rows)
+    sampler = NeighborSampler(indptr, indices, [6, 4, 3], labels=labels, seed=78, device=DEV, emit_view=True,
+                              view_edges=relational)
+    rec = RecordedIteration(model, cache, opt, L, step=1.3, round_to=512, record=False)
+    gen = torch.Generator(device=DEV).manual_seed(78)
+    monkeypatch.setattr(be, "CHECK_INPUTS", True)
+    checked = []
+    real_check = be.check_csr
+    monkeypatch.setattr(be, "check_csr", lambda *a: (checked.append(a[2:]), real_check(*a))[1])
+    for it in (1, 2, 3):
+        batch = sampler.sample(torch.randperm(N // 2, device=DEV, generator=gen)[:250].contiguous())
+        assert np.isfinite(float(rec(batch, it)))
+    (caps, _, _, _), = rec.shapes().values()
+    # every layer's forward was checked against ITS input rows, every backward over the view against its sources
+    assert {(caps[k], caps[k + 1]) for k in range(L)} <= set(checked) or relational
+    assert len(checked) >= 3 * (2 * L - 1)            # (the first layer hands no gradient to the features)
+    # the check itself reports rows whose sources lie behind the input it is told of
+    b = rec._records[next(iter(rec._records))].batch
+    with pytest.raises(ValueError, match="neighbour ids outside"):
+        real_check(b.ptr, b.idx, caps[L - 1], caps[L - 1])
