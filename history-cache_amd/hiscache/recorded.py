@@ -240,9 +240,10 @@ class RecordedIteration:
             return loss.detach()
         self._stage(r, batch, nnl, n_edges, self.cache.glb_iter, glb_iter, handle)
         r.uses += 1
-        if r.uses == 1 or not self.record:
+        if r.uses == 1 or not self.record or _be.CHECK_INPUTS:
+            # the same padded iteration, unrecorded (always so under the library's input checks, which synchronise)
             self.unrecorded += 1
-            return self._iteration(r.batch)           # the same padded iteration, unrecorded
+            return self._iteration(r.batch)
         if r.graph is None:
             if self._capture_stream is None:
                 self._capture_stream = torch.cuda.Stream(device=self.device)    # default priority
