@@ -62,11 +62,14 @@ class ProcessedDataset:
     def train_idx(self):
         return self._array("train")
 
-    def feature_store(self, device="cuda:0", out_dtype=None, chunk_rows=1 << 20, in_device_memory=False):
+    def feature_store(self, device="cuda:0", out_dtype=None, chunk_rows=1 << 20, in_device_memory=False,
+                      hot_rows=0):
         """Pinned, GPU-mapped copy of ``node_features.dat``, read from disk in chunks (the file is
         never held twice in memory).  ``in_device_memory``: the matrix goes to the GPU's own memory
         instead (288 GB hold the papers100M matrix, 57 GB, beside its history table), and the store's
-        gathers read it there."""
+        gathers read it there.  ``hot_rows``: for a matrix that stays in host memory, copies of that many
+        rows, the last (hottest) entries of ``sorted_indices.dat``, are kept in device memory and served from
+        there (the reference's feature cache, history_cache.py:124-142)."""
         p = path.join(self.dir, "node_features.dat")
         want = self.num_nodes * self.feature_dim * self.feature_dtype.itemsize
         if os.path.getsize(p) != want:
@@ -85,7 +88,11 @@ class ProcessedDataset:
                 hi = min(self.num_nodes, lo + chunk_rows)
                 dst[lo:hi] = src[lo:hi]
         del src
-        return PinnedFeatureStore(buf, device=device, out_dtype=out_dtype or torch.float32)
+        store = PinnedFeatureStore(buf, device=device, out_dtype=out_dtype or torch.float32)
+        if hot_rows and not in_device_memory:
+            order = self.hot_ids()
+            store.set_hot_rows(torch.from_numpy(np.array(order[max(0, len(order) - int(hot_rows)):])))
+        return store
 
     def sampler(self, fanout, device="cuda:0", seed=0, emit_view=False, view_edges=False, replay_slots=0):
         """``emit_view``: every batch carries the transposed view of its CSR (``batch.view``), so that the

@@ -4,7 +4,11 @@ requested rows directly over the host link with a gather kernel.
 It offers the three members of ``cxgnndl.UVM`` that the cache uses -- ``buffer``, ``get(ids)``,
 ``masked_get(ids, mask)`` (call sites: /root/reference/hiscache/history_cache.py:161,283,301,345).
 ``masked_get`` returns zeros for rows whose mask is false: the caller adds cached features on top
-(history_cache.py:345-349)."""
+(history_cache.py:345-349).
+
+Two tiers: ``set_hot_rows(hot_ids)`` keeps copies of the most requested rows in device memory (the feature half
+of the reference's cache: hotness-ordered rows in GPU memory, history_cache.py:121-142); every read then takes
+those rows from there and only the others over the host link, with the same result."""
 import torch
 
 import hiscache_backend as _be
@@ -12,7 +16,7 @@ import hiscache_backend as _be
 
 class PinnedFeatureStore:
 
-    def __init__(self, features, device="cuda:0", out_dtype=torch.float32, prefetch_cus=0):
+    def __init__(self, features, device="cuda:0", out_dtype=torch.float32, prefetch_cus=0, hot_ids=None):
         # out_dtype: element type of the gathered rows (keep torch.float16 for fp16 feature files to
         # halve the traffic of the first aggregation layer)
         # prefetch_cus > 0: ``prefetch`` reads on a stream that is kept to that many compute units, so that
@@ -35,6 +39,50 @@ class PinnedFeatureStore:
         self._side = None
         self._done = None
         self._prefetch_side = None
+        self.hot_rows = None            # [n_hot, F] device copies of the most requested rows, or None
+        self.hot_slot = None            # int32 per node: its row in hot_rows, or -1
+        self.last_cold = None           # flags of the last tiered read: the rows that came over the host link
+        if hot_ids is not None:
+            self.set_hot_rows(hot_ids)
+
+    def set_hot_rows(self, hot_ids, rows=None, num_nodes=None, chunk_rows=1 << 22):
+        """Keep copies of the rows ``hot_ids`` (int64, no duplicates; the head of a hotness order such as
+        ``sorted_indices.dat``) in device memory.  ``rows``: the copies, if the caller has them already;
+        ``num_nodes``: size of the id space when it is not the number of rows of the host matrix."""
+        if self.buffer.is_cuda:
+            raise ValueError("the whole matrix is in device memory already")
+        hot_ids = torch.as_tensor(hot_ids, dtype=torch.int64).to(self.device).contiguous()
+        n_nodes = int(num_nodes if num_nodes is not None else self.buffer.shape[0])
+        k = hot_ids.numel()
+        if k and (int(hot_ids.min()) < 0 or int(hot_ids.max()) >= n_nodes):
+            raise ValueError("hot_ids outside the id space")
+        slot = torch.full((n_nodes,), -1, dtype=torch.int32, device=self.device)
+        slot[hot_ids] = torch.arange(k, dtype=torch.int32, device=self.device)
+        if rows is None:
+            rows = torch.empty((k, self.buffer.shape[1]), dtype=self.buffer.dtype, device=self.device)
+            for lo in range(0, k, chunk_rows):
+                hi = min(k, lo + chunk_rows)
+                _be.gather_rows(self.buffer, self._host_ids(hot_ids[lo:hi]), out=rows[lo:hi])
+        elif tuple(rows.shape) != (k, self.buffer.shape[1]) or not rows.is_cuda:
+            raise ValueError("rows must be a device tensor [len(hot_ids), F]")
+        self.hot_rows, self.hot_slot = rows.contiguous(), slot
+
+    def _host_ids(self, ids):
+        """Rows of the host matrix that hold the nodes ``ids`` (the ids themselves)."""
+        return ids
+
+    def _tiered(self, ids, mask, out, cold_stream):
+        """Both tiers' launches: the device tier on the current stream, the host tier on ``cold_stream``."""
+        rows, cold = _be.gather_rows_hot(self.hot_rows, self.hot_slot, ids, mask=mask, out=out, out_dtype=self.out_dtype)
+        src_ids = self._host_ids(ids)
+        if cold_stream is not None:
+            cold_stream.wait_stream(torch.cuda.current_stream(self.device))
+            cold.record_stream(cold_stream)
+            if src_ids is not ids:
+                src_ids.record_stream(cold_stream)
+        _be.gather_rows_flagged(self.buffer, src_ids, cold, rows, stream=cold_stream)
+        self.last_cold = cold
+        return rows, src_ids
 
     def _side_stream(self):
         if self._side is None:
@@ -50,16 +98,20 @@ class PinnedFeatureStore:
     def close(self):
         """Release the read-ahead stream (a CU-limited stream is a driver object that lives until it is
         destroyed; without this it goes at interpreter exit).  The store stays usable: the next ``prefetch``
-        makes a new stream."""
+        makes a new stream.  Call it only when every tensor that ``prefetch`` has handed out is gone: torch's
+        allocator marks a freed block on the streams that used it, and a destroyed stream cannot be marked
+        (the process would crash at that free)."""
         side, self._prefetch_side = self._prefetch_side, None
         if side is not None and self.prefetch_cus > 0:
             _be.release_cu_limited_stream(side)
 
     def get(self, ids):
-        return _be.gather_rows(self.buffer, ids, out_dtype=self.out_dtype)
+        return self.masked_get(ids, None)
 
     def masked_get(self, ids, mask):
-        return _be.gather_rows(self.buffer, ids, mask=mask, out_dtype=self.out_dtype)
+        if self.hot_rows is not None:
+            return self._tiered(ids, mask, None, None)[0]
+        return _be.gather_rows(self.buffer, self._host_ids(ids), mask=mask, out_dtype=self.out_dtype)
 
     def masked_get_async(self, ids, mask):
         """Start the gather on a side stream (default priority) that first waits for the work
@@ -69,7 +121,7 @@ class PinnedFeatureStore:
         side = self._side_stream()
         side.wait_stream(cur)
         with torch.cuda.stream(side):
-            out = _be.gather_rows(self.buffer, ids, mask=mask, out_dtype=self.out_dtype)
+            out = self.masked_get(ids, mask)
             self._done.record(side)
         out.record_stream(cur)
         ids.record_stream(side)          # the caller may drop its last reference before the read is done
@@ -89,16 +141,24 @@ class PinnedFeatureStore:
         if self._prefetch_side is None:
             self._prefetch_side = self._make_prefetch_stream()
         side = self._prefetch_side
-        side.wait_stream(cur)                      # the ids are produced on the current stream
-        # enqueued on the side stream by name: switching torch's current stream and back costs the host 20 us
-        rows = _be.gather_rows(self.buffer, ids, mask=mask, out=out, out_dtype=self.out_dtype, stream=side)
+        if self.hot_rows is not None:
+            # the rows with a device copy are taken here and now (a few microseconds at full width); only the
+            # others wait for the host link, on the side stream
+            rows, src_ids = self._tiered(ids, mask, out, side)
+        else:
+            src_ids = self._host_ids(ids)
+            side.wait_stream(cur)                  # the ids are produced on the current stream
+            # enqueued on the side stream by name: switching torch's current stream and back costs the host 20 us
+            rows = _be.gather_rows(self.buffer, src_ids, mask=mask, out=out, out_dtype=self.out_dtype, stream=side)
         done = torch.cuda.Event()
         done.record(side)
         rows.record_stream(side)
-        ids.record_stream(side)
+        src_ids.record_stream(side)
         if mask is not None:
             mask.record_stream(side)
-        return PrefetchedRows(ids, rows, done, mask)
+        handle = PrefetchedRows(ids, rows, done, mask)
+        handle.src_ids = src_ids
+        return handle
 
     def take(self, handle, need=None):
         """The rows of a ``prefetch``; the current stream waits for the read to finish.  ``need`` (the

@@ -90,6 +90,9 @@ _SIGNATURES = {
     "hc_gather_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_stream_create_cu_limited": (_c_int, [_c_int, _c_p]),
     "hc_stream_destroy": (_c_int, [_c_p]),
+    "hc_gather_rows_hot": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_p, _c_i64, _c_i64,
+                                    _c_p]),
+    "hc_gather_rows_flagged": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_fixup_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p]),
     "hc_ring_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_int, _c_i64, _c_i64, _c_p, _c_p,
@@ -900,6 +903,64 @@ def gather_rows(src, ids, mask=None, out=None, accumulate=False, out_dtype=torch
                             _ptr(out), _float_dtype(out, "out"), 1 if accumulate else 0, n, F,
                             _stream() if stream is None else _c_p(stream.cuda_stream))
     _check(rc, "hc_gather_rows")
+    return out
+
+
+def gather_rows_hot(hot, slot_map, ids, mask=None, out=None, out_dtype=torch.float32, cold=None, stream=None):
+    """The device-memory tier of a two-tier feature matrix: ``hot`` [n_hot, F] holds copies of the most
+    requested rows, ``slot_map`` (int32, one entry per node) a node's row in it or -1.  out[i] = hot row of
+    ids[i] where mask[i] and the node has one, 0 where not mask[i]; the other rows are left alone and flagged in
+    ``cold`` (uint8, one per id) for ``gather_rows_flagged``.  Returns (out, cold)."""
+    lib = load_library()
+    _dev(hot, "hot")
+    if hot.dim() != 2 or not hot.is_contiguous():
+        raise ValueError("hot must be a contiguous [n_hot, F] tensor")
+    _dev(slot_map, "slot_map", torch.int32)
+    _dev(ids, "ids", torch.int64)
+    n, F = ids.numel(), hot.shape[1]
+    if mask is not None:
+        _dev(mask, "mask")
+        if mask.dtype not in (torch.bool, torch.uint8) or mask.numel() < n:
+            raise ValueError("mask must be a bool tensor with one entry per id")
+    if out is None:
+        out = torch.empty((n, F), dtype=out_dtype, device=ids.device)
+    else:
+        _dev(out, "out")
+        if tuple(out.shape) != (n, F):
+            raise ValueError("out must be [len(ids), F]")
+    if cold is None:
+        cold = torch.empty(n, dtype=torch.uint8, device=ids.device)
+    else:
+        _dev(cold, "cold", torch.uint8)
+        if cold.numel() < n:
+            raise ValueError("cold must hold one byte per id")
+    rc = lib.hc_gather_rows_hot(_ptr(hot), _float_dtype(hot, "hot"), hot.shape[0], _ptr(slot_map), slot_map.numel(),
+                                _ptr(ids), _ptr(mask), _ptr(out), _float_dtype(out, "out"), _ptr(cold), n, F,
+                                _stream() if stream is None else _c_p(stream.cuda_stream))
+    _check(rc, "hc_gather_rows_hot")
+    return out, cold
+
+
+def gather_rows_flagged(src, ids, flag, out, stream=None):
+    """out[i] = src[ids[i]] for the rows with flag[i] (uint8), every other row of ``out`` is left as it is.
+    ``src`` may be a GPU tensor or a pinned host tensor (read zero-copy over the host link)."""
+    lib = load_library()
+    if not isinstance(src, torch.Tensor) or src.dim() != 2 or not src.is_contiguous():
+        raise ValueError("src must be a contiguous 2-D tensor")
+    if not src.is_cuda and not src.is_pinned():
+        raise RuntimeError("src must be on the GPU or in pinned host memory")
+    _dev(ids, "ids", torch.int64)
+    _dev(flag, "flag")
+    _dev(out, "out")
+    n, F = ids.numel(), src.shape[1]
+    if flag.dtype not in (torch.bool, torch.uint8) or flag.numel() < n:
+        raise ValueError("flag must hold one byte per id")
+    if tuple(out.shape) != (n, F):
+        raise ValueError("out must be [len(ids), F]")
+    rc = lib.hc_gather_rows_flagged(_ptr(src), _float_dtype(src, "src"), src.shape[0], _ptr(ids), _ptr(flag),
+                                    _ptr(out), _float_dtype(out, "out"), n, F,
+                                    _stream() if stream is None else _c_p(stream.cuda_stream))
+    _check(rc, "hc_gather_rows_flagged")
     return out
 
 

@@ -515,6 +515,33 @@ int hc_fixup_rows(const void *src, int src_dtype, int64_t n_rows, const int64_t 
                   const uint8_t *need, const uint8_t *have, void *dst, int dst_dtype, int64_t n,
                   int64_t F, void *stream);
 
+/* hc_gather_rows_hot / hc_gather_rows_flagged: a feature matrix in two tiers.
+ * The reference keeps the features of the most requested nodes in GPU memory
+ * beside the embeddings (hotness order from sorted_indices.dat,
+ * hiscache/history_cache.py:121-142) and merges them with the rows read
+ * through UVM (:345-350).  Here copies of the hot rows form a matrix
+ * hot[n_hot, F] in device memory, slot_map[n_map] (int32) holds a node's row in
+ * it or -1, and the whole matrix stays in pinned host memory.  A batch's rows
+ * come in two launches that write disjoint rows of dst[n, F]:
+ *   hc_gather_rows_hot: for every i, with take = (mask == NULL || mask[i]) and
+ *     ids[i] inside [0, n_map) (a negative id addresses from the end):
+ *     dst[i,:] = hot[slot_map[ids[i]],:] when taken and the slot lies in
+ *     [0, n_hot); dst[i,:] = 0 when not taken; otherwise the row is left alone
+ *     and cold[i] = 1 (cold[i] = 0 for the rows written here).  cold: n bytes.
+ *   hc_gather_rows_flagged: dst[i,:] = src[ids[i],:] for the rows with
+ *     flag[i] != 0 (cleared if ids[i] lies outside [0, n_rows)), other rows are
+ *     not touched.  src may be pinned, mapped host memory; ids may differ from
+ *     the first call's (a caller that stores the host matrix under other row
+ *     numbers).
+ * After both, dst equals hc_gather_rows(src, ..., ids, mask) when hot holds
+ * copies of src's rows. */
+int hc_gather_rows_hot(const void *hot, int hot_dtype, int64_t n_hot, const int32_t *slot_map,
+                       int64_t n_map, const int64_t *ids, const uint8_t *mask, void *dst, int dst_dtype,
+                       uint8_t *cold, int64_t n, int64_t F, void *stream);
+int hc_gather_rows_flagged(const void *src, int src_dtype, int64_t n_rows, const int64_t *ids,
+                           const uint8_t *flag, void *dst, int dst_dtype, int64_t n, int64_t F,
+                           void *stream);
+
 /* hc_lookup: out[i] = map[ids[i] + offset]  (int64 gather; the id translation
  * of lookup_and_load, hiscache/history_cache.py:310,315). */
 int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset, int64_t *out,
