@@ -59,6 +59,9 @@ def parse():
     ap.add_argument("--prefetch", action="store_true",
                     help="c3/c5: start each batch's host-link feature read one batch ahead, on a side stream, for "
                          "the rows that the cache's state at that moment makes necessary (fixed up at the lookup)")
+    ap.add_argument("--hot-fraction", type=float, default=0.0,
+                    help="c3 --with-sampler: copies of this share of the feature rows, the nodes with the most "
+                         "incoming edges, are kept in device memory; only the other rows cross the host link")
     ap.add_argument("--prefetch-cus", type=int, default=16,
                     help="with --prefetch: compute units the read-ahead's stream may use (0: an ordinary stream)")
     ap.add_argument("--prefetch-depth", type=int, default=1,
@@ -714,16 +717,8 @@ def pooled_store_class(pool_rows):
             self.reads += 1
             return (ids + self.reads * 1_000_003) % pool_rows
 
-        def get(self, ids):
-            return super().get(self.fold(ids))
-
-        def masked_get(self, ids, mask):
-            return super().masked_get(self.fold(ids), mask)
-
-        def prefetch(self, ids, mask=None, out=None):
-            handle = super().prefetch(self.fold(ids), mask, out=out)
-            handle.ids = ids
-            return handle
+        def _host_ids(self, ids):
+            return self.fold(ids)
 
     return PooledStore
 
@@ -804,6 +799,14 @@ def run_c3(args, with_batched=True):
         from hiscache import NeighborSampler
         indptr, indices = device_power_law_graph(N, 14.5, dev, gen)
         sampled["E_graph"] = indices.numel()
+        if args.hot_fraction > 0 and not args.features_in_hbm:
+            # hotness = incoming edges (what a pre-sampling pass of the reference's preprocessing counts)
+            k = min(N, int(N * args.hot_fraction))
+            counts = torch.bincount(indices, minlength=N)
+            hot_ids = torch.argsort(counts, descending=True)[:k].contiguous()
+            del counts
+            store.set_hot_rows(hot_ids, num_nodes=N)
+            del hot_ids
         sampled["sampler"] = NeighborSampler(indptr, indices, fanout, seed=3, device=dev, validate=False,
                                              emit_view=not args.no_batch_view,
                                              replay_slots=max(args.sampler_replay, args.prefetch_depth + 2)
@@ -915,6 +918,8 @@ def run_c3(args, with_batched=True):
         "feature_store": "device memory" if args.features_in_hbm else "pinned host memory, read zero-copy",
         "transposed_view": "built in backward" if args.no_batch_view else "emitted with the batch",
         "feature_rows_read_last_batch": int(cache.used_masks[0].sum()),
+        "feature_rows_in_device_memory": 0 if store.hot_rows is None else int(store.hot_rows.shape[0]),
+        "feature_rows_over_host_link_last_read": None if store.last_cold is None else int(store.last_cold.sum()),
         "cached_1hop_fraction_last_batch": float((cache.sub2embed != -1).float().mean()),
         "batched_history_layer": batched["detail"],
         "roofline": batched["roofline"],
@@ -1028,6 +1033,8 @@ def run_c5(args):
         "ms_per_chunk_of_steps": chunk_figures(),
         "transposed_view": "built in backward" if args.no_batch_view else "emitted with the batch",
         "feature_rows_read_last_batch": int(cache.used_masks[0].sum()),
+        "feature_rows_in_device_memory": 0 if store.hot_rows is None else int(store.hot_rows.shape[0]),
+        "feature_rows_over_host_link_last_read": None if store.last_cold is None else int(store.last_cold.sum()),
         "cached_1hop_fraction_last_batch": float((cache.sub2embed != -1).float().mean()),
     }
 

@@ -1,8 +1,8 @@
 // Two-tier feature rows: copies of the most requested rows of a feature matrix live in device memory, the
 // whole matrix stays in pinned host memory.  A batch's rows are fetched in two launches that write disjoint
 // rows of the same output:
-//   hc_gather_rows_hot      one wave per requested row, at full width: rows that have a device copy are
-//                           copied from it, rows that are not asked for are cleared, the others are flagged;
+//   hc_gather_rows_hot      at full width: rows that have a device copy are copied from it, rows that are not
+//                           asked for are cleared, the others are flagged;
 //   hc_gather_rows_flagged  the flagged rows, from the host matrix over the host link.  A wave examines 64
 //                           rows at a time (one flag and one id per lane), then walks the flagged ones two at
 //                           a time, so that a few hundred waves keep the link busy and no wave spends its
@@ -41,7 +41,17 @@ __device__ __forceinline__ void tier_copy_row(const TS *__restrict__ s, TD *__re
   }
 }
 
-template <typename TS, typename TD>
+// A wave serves HOT_ROWS consecutive requested rows: one lane per row reads the row's mask byte, id and slot (three
+// dependent reads for all rows at once instead of once per row), then the wave copies the rows HOT_INFLIGHT at a
+// time, every row's load issued before the first store.  With a wave per row the launch is a chain of four round
+// trips per 512-byte row and runs at a fraction of the memory rate.
+constexpr int HOT_ROWS = 16;
+constexpr int HOT_INFLIGHT = 4;
+constexpr int ROW_ZERO = 0, ROW_COPY = 1, ROW_SKIP = 2;
+
+// TIERED = false: the plain gather of a matrix in device memory (hot is the matrix, a node's row is its id, no row
+// is left to another launch).
+template <typename TS, typename TD, bool TIERED>
 __global__ __launch_bounds__(HC_BLOCK) void tier_hot_kernel(const TS *__restrict__ hot, int64_t n_hot,
                                                              const int32_t *__restrict__ slot_map, int64_t n_map,
                                                              const int64_t *__restrict__ ids,
@@ -49,22 +59,63 @@ __global__ __launch_bounds__(HC_BLOCK) void tier_hot_kernel(const TS *__restrict
                                                              TD *__restrict__ dst, uint8_t *__restrict__ cold,
                                                              int64_t n, int64_t F) {
   const int lane = hc_lane();
-  const int64_t i = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
-  if (i >= n) return;
-  bool take = mask == nullptr || mask[i] != 0;
-  int64_t id = 0;
-  if (take) {
-    id = ids[i];
-    if (id < 0) id += n_map;
-    if (id < 0 || id >= n_map) take = false;
+  const int64_t base = ((int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block()) * HOT_ROWS;
+  if (base >= n) return;
+  const int64_t i = base + lane;
+  int state = ROW_SKIP;
+  int64_t slot = 0;
+  if (lane < HOT_ROWS && i < n) {
+    bool take = mask == nullptr || mask[i] != 0;
+    int64_t id = 0;
+    if (take) {
+      id = ids[i];
+      if (id < 0) id += n_map;
+      if (id < 0 || id >= n_map) take = false;
+    }
+    if constexpr (TIERED) slot = take ? (int64_t)slot_map[id] : -1;
+    else slot = id;
+    const bool is_cold = TIERED && take && (slot < 0 || slot >= n_hot);
+    if constexpr (TIERED) cold[i] = is_cold ? 1 : 0;
+    state = is_cold ? ROW_SKIP : (take ? ROW_COPY : ROW_ZERO);     // a cold row is written by the other launch
   }
-  int64_t slot = -1;
-  if (take) slot = slot_map[id];
-  const bool is_cold = take && (slot < 0 || slot >= n_hot);
-  if (lane == 0) cold[i] = is_cold ? 1 : 0;
-  if (is_cold) return;                       // the other launch writes this row
-  const TS *s = take ? hot + slot * F : nullptr;
-  tier_copy_row<TS, TD>(s, dst + i * F, F, lane, tier_vec_ok(hot, dst, F));
+  const bool vec_ok = tier_vec_ok(hot, dst, F);
+#pragma unroll
+  for (int r0 = 0; r0 < HOT_ROWS; r0 += HOT_INFLIGHT) {
+    int st[HOT_INFLIGHT];
+    const TS *s[HOT_INFLIGHT];
+    bool any = false;
+#pragma unroll
+    for (int k = 0; k < HOT_INFLIGHT; ++k) {
+      st[k] = __builtin_amdgcn_readlane(state, r0 + k);
+      s[k] = hot + hc_readlane64(slot, r0 + k) * F;
+      any = any || st[k] != ROW_SKIP;
+    }
+    if (!any) continue;                                            // wave-uniform
+    TD *o = dst + (base + r0) * F;
+    if (vec_ok) {
+      for (int64_t c = (int64_t)lane * TV; c < F; c += HC_WAVE * TV) {
+        float v[HOT_INFLIGHT][TV];
+#pragma unroll
+        for (int k = 0; k < HOT_INFLIGHT; ++k) {
+#pragma unroll
+          for (int e = 0; e < TV; ++e) v[k][e] = 0.0f;
+          if (st[k] == ROW_COPY) hc_vec<TS, TV>::load(s[k] + c, v[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < HOT_INFLIGHT; ++k)
+          if (st[k] != ROW_SKIP) hc_vec<TD, TV>::store(o + k * F + c, v[k]);
+      }
+    } else {
+      for (int64_t c = lane; c < F; c += HC_WAVE) {
+        float v[HOT_INFLIGHT];
+#pragma unroll
+        for (int k = 0; k < HOT_INFLIGHT; ++k) v[k] = st[k] == ROW_COPY ? hc_to_f32<TS>(s[k][c]) : 0.0f;
+#pragma unroll
+        for (int k = 0; k < HOT_INFLIGHT; ++k)
+          if (st[k] != ROW_SKIP) o[k * F + c] = hc_from_f32<TD>(v[k]);
+      }
+    }
+  }
 }
 
 template <typename TS, typename TD>
@@ -120,20 +171,37 @@ __global__ __launch_bounds__(HC_BLOCK) void gather_flagged_kernel(const TS *__re
   }
 }
 
-template <typename TS>
+template <typename TS, bool TIERED>
 int launch_hot(const void *hot, int64_t n_hot, const int32_t *slot_map, int64_t n_map, const int64_t *ids,
                const uint8_t *mask, void *dst, int dst_dtype, uint8_t *cold, int64_t n, int64_t F, dim3 g,
                hipStream_t st) {
   const TS *h = static_cast<const TS *>(hot);
   const dim3 bl(HC_BLOCK);
   if (dst_dtype == HC_F32)
-    tier_hot_kernel<TS, float><<<g, bl, 0, st>>>(h, n_hot, slot_map, n_map, ids, mask, static_cast<float *>(dst), cold, n, F);
+    tier_hot_kernel<TS, float, TIERED><<<g, bl, 0, st>>>(h, n_hot, slot_map, n_map, ids, mask,
+                                                         static_cast<float *>(dst), cold, n, F);
   else if (dst_dtype == HC_F16)
-    tier_hot_kernel<TS, __half><<<g, bl, 0, st>>>(h, n_hot, slot_map, n_map, ids, mask, static_cast<__half *>(dst), cold, n, F);
+    tier_hot_kernel<TS, __half, TIERED><<<g, bl, 0, st>>>(h, n_hot, slot_map, n_map, ids, mask,
+                                                          static_cast<__half *>(dst), cold, n, F);
   else
-    tier_hot_kernel<TS, __hip_bfloat16><<<g, bl, 0, st>>>(h, n_hot, slot_map, n_map, ids, mask,
-                                                          static_cast<__hip_bfloat16 *>(dst), cold, n, F);
+    tier_hot_kernel<TS, __hip_bfloat16, TIERED><<<g, bl, 0, st>>>(h, n_hot, slot_map, n_map, ids, mask,
+                                                                  static_cast<__hip_bfloat16 *>(dst), cold, n, F);
   return hc_launch_status();
+}
+
+template <bool TIERED>
+int dispatch_hot(const void *hot, int hot_dtype, int64_t n_hot, const int32_t *slot_map, int64_t n_map,
+                 const int64_t *ids, const uint8_t *mask, void *dst, int dst_dtype, uint8_t *cold, int64_t n,
+                 int64_t F, hipStream_t st) {
+  const int64_t waves = (n + HOT_ROWS - 1) / HOT_ROWS;
+  const int64_t b = (waves + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  if (!hc_grid_ok(b)) return HC_EUNSUPPORTED;
+  const dim3 g((unsigned)b);
+  if (hot_dtype == HC_F32)
+    return launch_hot<float, TIERED>(hot, n_hot, slot_map, n_map, ids, mask, dst, dst_dtype, cold, n, F, g, st);
+  if (hot_dtype == HC_F16)
+    return launch_hot<__half, TIERED>(hot, n_hot, slot_map, n_map, ids, mask, dst, dst_dtype, cold, n, F, g, st);
+  return launch_hot<__hip_bfloat16, TIERED>(hot, n_hot, slot_map, n_map, ids, mask, dst, dst_dtype, cold, n, F, g, st);
 }
 
 template <typename TS>
@@ -162,13 +230,14 @@ extern "C" int hc_gather_rows_hot(const void *hot, int hot_dtype, int64_t n_hot,
   if (!dtype_ok(hot_dtype) || !dtype_ok(dst_dtype)) return HC_EDTYPE;
   if (n == 0) return HC_OK;
   HC_REQUIRE(ids && dst && cold && (slot_map || n_map == 0) && (hot || n_hot == 0));
-  const int64_t b = (n + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
-  if (!hc_grid_ok(b)) return HC_EUNSUPPORTED;
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 g((unsigned)b);
-  if (hot_dtype == HC_F32) return launch_hot<float>(hot, n_hot, slot_map, n_map, ids, mask, dst, dst_dtype, cold, n, F, g, st);
-  if (hot_dtype == HC_F16) return launch_hot<__half>(hot, n_hot, slot_map, n_map, ids, mask, dst, dst_dtype, cold, n, F, g, st);
-  return launch_hot<__hip_bfloat16>(hot, n_hot, slot_map, n_map, ids, mask, dst, dst_dtype, cold, n, F, g, st);
+  return dispatch_hot<true>(hot, hot_dtype, n_hot, slot_map, n_map, ids, mask, dst, dst_dtype, cold, n, F,
+                            static_cast<hipStream_t>(stream));
+}
+
+// The plain gather (hc_gather_rows without accumulation) of a matrix in device memory; arguments checked by the caller.
+int hc_gather_rows_device(const void *src, int src_dtype, int64_t n_rows, const int64_t *ids, const uint8_t *mask,
+                          void *dst, int dst_dtype, int64_t n, int64_t F, hipStream_t st) {
+  return dispatch_hot<false>(src, src_dtype, n_rows, nullptr, n_rows, ids, mask, dst, dst_dtype, nullptr, n, F, st);
 }
 
 extern "C" int hc_gather_rows_flagged(const void *src, int src_dtype, int64_t n_rows, const int64_t *ids,

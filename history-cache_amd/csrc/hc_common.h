@@ -27,6 +27,11 @@ static inline size_t hc_align_up(size_t v, size_t a) { return (v + a - 1) / a * 
 // 1024 threads are used by the scan kernel, so the bound is taken for those).
 static inline bool hc_grid_ok(int64_t blocks) { return blocks > 0 && blocks <= 0xffffffffLL / HC_BLOCK; }
 
+// feature_tiers.hip: the plain row gather of a matrix in device memory, several rows per wave
+// (hc_gather_rows hands such calls over; arguments are checked there).
+__attribute__((visibility("hidden"))) int hc_gather_rows_device(const void *src, int src_dtype, int64_t n_rows, const int64_t *ids, const uint8_t *mask,
+                          void *dst, int dst_dtype, int64_t n, int64_t F, hipStream_t st);
+
 #ifdef __HIPCC__
 
 __device__ __forceinline__ int hc_lane() { return (int)(threadIdx.x & (HC_WAVE - 1)); }

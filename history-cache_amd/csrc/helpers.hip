@@ -442,13 +442,21 @@ extern "C" int hc_gather_rows(const void *src, int src_dtype, int64_t n_rows, co
   // launch of one wave per row would park tens of thousands of waiting waves on the compute units,
   // in the way of whatever runs beside it on other streams.
   // (256 blocks = 1 024 waves read 56 - 57 GB/s, the same as 22 000 blocks).
+  // A table in device memory takes the launch that serves several rows per wave.
   constexpr int64_t HOST_GATHER_BLOCKS = 256;
-  if (b > HOST_GATHER_BLOCKS) {
+  constexpr int64_t CHUNKED_FROM_ROWS = 256;
+  if (b > HOST_GATHER_BLOCKS || (n >= CHUNKED_FROM_ROWS && !accumulate)) {
     hipPointerAttribute_t attr;
+    bool in_host_memory = false;
     if (hipPointerGetAttributes(&attr, src) == hipSuccess) {
-      if (attr.type == hipMemoryTypeHost) b = HOST_GATHER_BLOCKS;
+      in_host_memory = attr.type == hipMemoryTypeHost;
     } else {
       (void)hipGetLastError();   // an address the runtime does not know: treat it as device memory
+    }
+    if (in_host_memory) {
+      if (b > HOST_GATHER_BLOCKS) b = HOST_GATHER_BLOCKS;
+    } else if (n >= CHUNKED_FROM_ROWS && !accumulate) {
+      return hc_gather_rows_device(src, src_dtype, n_rows, ids, mask, dst, dst_dtype, n, F, st);
     }
   }
   dim3 g((unsigned)b), bl(HC_BLOCK);

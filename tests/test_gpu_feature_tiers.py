@@ -40,6 +40,8 @@ def test_two_launches_equal_the_plain_gather(src_dtype, out_dtype, N, F, n, hot_
     ids = torch.from_numpy(ids_np).to(DEV)
     mask = torch.from_numpy(rng.random(n) < 0.6).to(DEV) if masked else None
     want = be.gather_rows(src, ids, mask=mask, out_dtype=TORCH[out_dtype])
+    # (the same matrix in device memory is gathered several rows per wave: the same rows)
+    assert torch.equal(be.gather_rows(src.to(DEV), ids, mask=mask, out_dtype=TORCH[out_dtype]), want)
 
     out = torch.full((n, F), 7.0, dtype=TORCH[out_dtype], device=DEV)
     rows, cold = be.gather_rows_hot(hot, slot, ids, mask=mask, out=out)
