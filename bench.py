@@ -1423,6 +1423,12 @@ def main():
             rh_args.recorded = True
             r5_args = argparse.Namespace(**vars(it_args))
             r5_args.recorded, r5_args.prefetch = True, True      # once replayed, this loop too gains from the read-ahead
+            # c3_sampled_hot_rows: between the two placements -- the matrix in host memory, copies of the rows of the
+            # 30% of the nodes with the most incoming edges in device memory (17 GB); the others are read ahead
+            ht_args = argparse.Namespace(**vars(sm_args))
+            ht_args.hot_fraction = 0.3
+            rt_args = argparse.Namespace(**vars(ht_args))
+            rt_args.recorded = True
             runs = (("c1", it_args, lambda: run_c1(it_args)),
                     ("c1_recorded", r1_args, lambda: run_c1(r1_args)),
                     ("c3", c3_args, lambda: run_c3(c3_args, with_batched=False)),
@@ -1430,6 +1436,8 @@ def main():
                     ("c5", it_args, lambda: run_c5(it_args)),
                     ("c5_recorded", r5_args, lambda: run_c5(r5_args)),
                     ("c3_sampled", sm_args, lambda: run_c3(sm_args, with_batched=False)),
+                    ("c3_sampled_hot_rows", ht_args, lambda: run_c3(ht_args, with_batched=False)),
+                    ("c3_sampled_hot_rows_recorded", rt_args, lambda: run_c3(rt_args, with_batched=False)),
                     ("c3_sampled_features_in_hbm", hb_args, lambda: run_c3(hb_args, with_batched=False)),
                     ("c3_sampled_features_in_hbm_recorded", rh_args, lambda: run_c3(rh_args, with_batched=False)))
             for name, used_args, fn in runs:
@@ -1442,6 +1450,11 @@ def main():
                     "feature_read_ahead": bool(used_args.prefetch),
                     "ms_per_chunk_of_steps": r.get("ms_per_chunk_of_steps"),
                     "phases_ms": r["phases_ms"], "phases_host_enqueue_ms": r["phases_host_enqueue_ms"]}
+                if r.get("feature_rows_in_device_memory"):
+                    res["iterations"][name]["feature_rows"] = {
+                        "needed_last_batch": r["feature_rows_read_last_batch"],
+                        "over_host_link_last_read": r["feature_rows_over_host_link_last_read"],
+                        "copies_in_device_memory": r["feature_rows_in_device_memory"]}
                 if r.get("recorded"):            # the whole iteration is the one phase called "load"
                     res["iterations"][name]["recorded"] = r["recorded"]
                 if "cpu_baseline" in r:          # c1, the CPU-runnable configuration: the same iteration on the host

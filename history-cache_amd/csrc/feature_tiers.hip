@@ -118,10 +118,13 @@ __global__ __launch_bounds__(HC_BLOCK) void tier_hot_kernel(const TS *__restrict
   }
 }
 
-template <typename TS, typename TD>
+// FIXUP = true: rows that were gathered under a guess (have) brought to the exact answer (flag = need): the rows
+// where the two differ are the flagged ones, read if needed and cleared if not.
+template <typename TS, typename TD, bool FIXUP>
 __global__ __launch_bounds__(HC_BLOCK) void gather_flagged_kernel(const TS *__restrict__ src, int64_t n_rows,
                                                                    const int64_t *__restrict__ ids,
                                                                    const uint8_t *__restrict__ flag,
+                                                                   const uint8_t *__restrict__ have,
                                                                    TD *__restrict__ dst, int64_t n, int64_t F) {
   const int lane = hc_lane();
   const bool vec_ok = tier_vec_ok(src, dst, F);
@@ -131,8 +134,14 @@ __global__ __launch_bounds__(HC_BLOCK) void gather_flagged_kernel(const TS *__re
        chunk += stride) {
     const int64_t i = chunk * HC_WAVE + lane;
     bool flagged = i < n && flag[i] != 0;
+    bool read = flagged;
+    if constexpr (FIXUP) {
+      const bool hv = i < n && have[i] != 0;
+      read = flagged && !hv;                 // needed, not read yet
+      flagged = i < n && flagged != hv;      // (read, not needed any more: cleared)
+    }
     int64_t id = -1;
-    if (flagged) {
+    if (read) {
       id = ids[i];
       if (id < 0) id += n_rows;
       if (id < 0 || id >= n_rows) id = -1;   // a flagged row without a source row is cleared
@@ -204,19 +213,32 @@ int dispatch_hot(const void *hot, int hot_dtype, int64_t n_hot, const int32_t *s
   return launch_hot<__hip_bfloat16, TIERED>(hot, n_hot, slot_map, n_map, ids, mask, dst, dst_dtype, cold, n, F, g, st);
 }
 
-template <typename TS>
-int launch_flagged(const void *src, int64_t n_rows, const int64_t *ids, const uint8_t *flag, void *dst,
-                   int dst_dtype, int64_t n, int64_t F, dim3 g, hipStream_t st) {
+template <typename TS, bool FIXUP>
+int launch_flagged(const void *src, int64_t n_rows, const int64_t *ids, const uint8_t *flag, const uint8_t *have,
+                   void *dst, int dst_dtype, int64_t n, int64_t F, dim3 g, hipStream_t st) {
   const TS *s = static_cast<const TS *>(src);
   const dim3 bl(HC_BLOCK);
   if (dst_dtype == HC_F32)
-    gather_flagged_kernel<TS, float><<<g, bl, 0, st>>>(s, n_rows, ids, flag, static_cast<float *>(dst), n, F);
+    gather_flagged_kernel<TS, float, FIXUP><<<g, bl, 0, st>>>(s, n_rows, ids, flag, have, static_cast<float *>(dst), n, F);
   else if (dst_dtype == HC_F16)
-    gather_flagged_kernel<TS, __half><<<g, bl, 0, st>>>(s, n_rows, ids, flag, static_cast<__half *>(dst), n, F);
+    gather_flagged_kernel<TS, __half, FIXUP><<<g, bl, 0, st>>>(s, n_rows, ids, flag, have, static_cast<__half *>(dst), n, F);
   else
-    gather_flagged_kernel<TS, __hip_bfloat16><<<g, bl, 0, st>>>(s, n_rows, ids, flag,
-                                                                static_cast<__hip_bfloat16 *>(dst), n, F);
+    gather_flagged_kernel<TS, __hip_bfloat16, FIXUP><<<g, bl, 0, st>>>(s, n_rows, ids, flag, have,
+                                                                       static_cast<__hip_bfloat16 *>(dst), n, F);
   return hc_launch_status();
+}
+
+template <bool FIXUP>
+int dispatch_flagged(const void *src, int src_dtype, int64_t n_rows, const int64_t *ids, const uint8_t *flag,
+                     const uint8_t *have, void *dst, int dst_dtype, int64_t n, int64_t F, int64_t max_blocks,
+                     hipStream_t st) {
+  const int64_t chunks = (n + HC_WAVE - 1) / HC_WAVE;
+  int64_t b = (chunks + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
+  if (b > max_blocks) b = max_blocks;
+  const dim3 g((unsigned)b);
+  if (src_dtype == HC_F32) return launch_flagged<float, FIXUP>(src, n_rows, ids, flag, have, dst, dst_dtype, n, F, g, st);
+  if (src_dtype == HC_F16) return launch_flagged<__half, FIXUP>(src, n_rows, ids, flag, have, dst, dst_dtype, n, F, g, st);
+  return launch_flagged<__hip_bfloat16, FIXUP>(src, n_rows, ids, flag, have, dst, dst_dtype, n, F, g, st);
 }
 
 bool dtype_ok(int d) { return d >= HC_F32 && d <= HC_BF16; }
@@ -247,8 +269,6 @@ extern "C" int hc_gather_rows_flagged(const void *src, int src_dtype, int64_t n_
   if (!dtype_ok(src_dtype) || !dtype_ok(dst_dtype)) return HC_EDTYPE;
   if (n == 0) return HC_OK;
   HC_REQUIRE(ids && dst && flag && (src || n_rows == 0));
-  const int64_t chunks = (n + HC_WAVE - 1) / HC_WAVE;
-  int64_t b = (chunks + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
   // a matrix in host memory: a few hundred waves keep the link busy, more only stand in the way of the
   // kernels that run beside this one; a matrix in device memory: enough waves to fill the chip
   int64_t cap = 4096;
@@ -258,10 +278,12 @@ extern "C" int hc_gather_rows_flagged(const void *src, int src_dtype, int64_t n_
   } else {
     (void)hipGetLastError();
   }
-  if (b > cap) b = cap;
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 g((unsigned)b);
-  if (src_dtype == HC_F32) return launch_flagged<float>(src, n_rows, ids, flag, dst, dst_dtype, n, F, g, st);
-  if (src_dtype == HC_F16) return launch_flagged<__half>(src, n_rows, ids, flag, dst, dst_dtype, n, F, g, st);
-  return launch_flagged<__hip_bfloat16>(src, n_rows, ids, flag, dst, dst_dtype, n, F, g, st);
+  return dispatch_flagged<false>(src, src_dtype, n_rows, ids, flag, nullptr, dst, dst_dtype, n, F, cap,
+                                 static_cast<hipStream_t>(stream));
+}
+
+// hc_fixup_rows: the rows where need and have differ are few, whatever memory the matrix lies in.
+int hc_fixup_rows_chunked(const void *src, int src_dtype, int64_t n_rows, const int64_t *ids, const uint8_t *need,
+                          const uint8_t *have, void *dst, int dst_dtype, int64_t n, int64_t F, hipStream_t st) {
+  return dispatch_flagged<true>(src, src_dtype, n_rows, ids, need, have, dst, dst_dtype, n, F, 4096, st);
 }

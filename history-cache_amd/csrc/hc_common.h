@@ -32,6 +32,12 @@ static inline bool hc_grid_ok(int64_t blocks) { return blocks > 0 && blocks <= 0
 __attribute__((visibility("hidden"))) int hc_gather_rows_device(const void *src, int src_dtype, int64_t n_rows, const int64_t *ids, const uint8_t *mask,
                           void *dst, int dst_dtype, int64_t n, int64_t F, hipStream_t st);
 
+// feature_tiers.hip: hc_fixup_rows' launch (64 rows examined per wave, the few that differ read or cleared).
+__attribute__((visibility("hidden"))) int hc_fixup_rows_chunked(const void *src, int src_dtype, int64_t n_rows,
+                                                                const int64_t *ids, const uint8_t *need,
+                                                                const uint8_t *have, void *dst, int dst_dtype,
+                                                                int64_t n, int64_t F, hipStream_t st);
+
 #ifdef __HIPCC__
 
 __device__ __forceinline__ int hc_lane() { return (int)(threadIdx.x & (HC_WAVE - 1)); }

@@ -465,50 +465,6 @@ extern "C" int hc_gather_rows(const void *src, int src_dtype, int64_t n_rows, co
   return launch_gather<__hip_bfloat16>(src, n_rows, ids, mask, dst, dst_dtype, accumulate, n, F, g, bl, st);
 }
 
-namespace {
-
-// Rows that were gathered ahead of time under a guess of which are needed (have), brought to the exact
-// answer (need): a row that is needed but was not read is read now, a row that was read but is not needed
-// is cleared, every other row is left as it is.  Wave per row; the few rows that differ do the work.
-template <typename TS, typename TD>
-__global__ __launch_bounds__(HC_BLOCK) void fixup_rows_kernel(const TS *__restrict__ src, int64_t n_rows,
-                                                               const int64_t *__restrict__ ids,
-                                                               const uint8_t *__restrict__ need,
-                                                               const uint8_t *__restrict__ have,
-                                                               TD *__restrict__ dst, int64_t n, int64_t F) {
-  const int lane = hc_lane();
-  const int64_t i = (int64_t)blockIdx.x * HC_WAVES_PER_BLOCK + hc_wave_in_block();
-  if (i >= n) return;
-  const bool nd = need[i] != 0, hv = have[i] != 0;
-  if (nd == hv) return;
-  TD *__restrict__ o = dst + i * F;
-  bool take = nd;
-  int64_t id = 0;
-  if (take) {
-    id = ids[i];
-    if (id < 0) id += n_rows;
-    if (id < 0 || id >= n_rows) take = false;
-  }
-  const TS *__restrict__ s = src + id * F;
-  for (int64_t c = lane; c < F; c += HC_WAVE) o[c] = hc_from_f32<TD>(take ? hc_to_f32<TS>(s[c]) : 0.0f);
-}
-
-template <typename TS>
-int launch_fixup(const void *src, int64_t n_rows, const int64_t *ids, const uint8_t *need, const uint8_t *have,
-                 void *dst, int dst_dtype, int64_t n, int64_t F, dim3 g, dim3 bl, hipStream_t st) {
-  const TS *s = static_cast<const TS *>(src);
-  if (dst_dtype == HC_F32)
-    fixup_rows_kernel<TS, float><<<g, bl, 0, st>>>(s, n_rows, ids, need, have, static_cast<float *>(dst), n, F);
-  else if (dst_dtype == HC_F16)
-    fixup_rows_kernel<TS, __half><<<g, bl, 0, st>>>(s, n_rows, ids, need, have, static_cast<__half *>(dst), n, F);
-  else
-    fixup_rows_kernel<TS, __hip_bfloat16><<<g, bl, 0, st>>>(s, n_rows, ids, need, have,
-                                                            static_cast<__hip_bfloat16 *>(dst), n, F);
-  return hc_launch_status();
-}
-
-}  // namespace
-
 extern "C" int hc_stream_create_cu_limited(int n_cus, void **stream) {
   HC_REQUIRE(stream != nullptr && n_cus >= 1);
   *stream = nullptr;
@@ -552,13 +508,10 @@ extern "C" int hc_fixup_rows(const void *src, int src_dtype, int64_t n_rows, con
   if (src_dtype < HC_F32 || src_dtype > HC_BF16 || dst_dtype < HC_F32 || dst_dtype > HC_BF16) return HC_EDTYPE;
   if (n == 0) return HC_OK;
   HC_REQUIRE(ids && dst && need && have && (src || n_rows == 0));
-  const int64_t b = (n + HC_WAVES_PER_BLOCK - 1) / HC_WAVES_PER_BLOCK;
-  if (!hc_grid_ok(b)) return HC_EUNSUPPORTED;
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  dim3 g((unsigned)b), bl(HC_BLOCK);
-  if (src_dtype == HC_F32) return launch_fixup<float>(src, n_rows, ids, need, have, dst, dst_dtype, n, F, g, bl, st);
-  if (src_dtype == HC_F16) return launch_fixup<__half>(src, n_rows, ids, need, have, dst, dst_dtype, n, F, g, bl, st);
-  return launch_fixup<__hip_bfloat16>(src, n_rows, ids, need, have, dst, dst_dtype, n, F, g, bl, st);
+  // rows that were gathered ahead of time under a guess of which are needed (have), brought to the exact
+  // answer (need): the few rows that differ do the work
+  return hc_fixup_rows_chunked(src, src_dtype, n_rows, ids, need, have, dst, dst_dtype, n, F,
+                               static_cast<hipStream_t>(stream));
 }
 
 extern "C" int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset,
