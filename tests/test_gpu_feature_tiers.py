@@ -228,3 +228,63 @@ def test_training_on_a_tiered_store_equals_training_on_a_plain_one(recorded):
     assert cold_rows > 0
     if recorded:
         assert twins["tiered"][4].replays >= 3, twins["tiered"][4].shapes()
+
+
+def test_the_flat_cache_on_a_tiered_store_equals_the_flat_cache_on_a_plain_one():
+    """``HistoryCache`` (a feature cache of its own in the buffer's tail) over a store with hot rows: what its
+    feature cache does not hold comes through the store's two tiers; twins hold the same bits after every
+    iteration, with the next batch's rows read ahead."""
+    from helpers import power_law_graph
+    from hiscache import (HistoryCache, HistorySAGE, NeighborSampler, PinnedFeatureStore, backward_on_this_thread,
+                          make_config, prefer_low_latency_gemm)
+    N, Fin, H, C, L, n_seed, fanout = 30_000, 64, 64, 6, 3, 200, [6, 4, 3]
+    rng = np.random.default_rng(41)
+    indptr, indices = power_law_graph(rng, N, 4.0, alpha=2.0, max_degree=300)
+    feats = host_matrix(rng, N, Fin, "f32")
+    labels = torch.from_numpy(rng.integers(0, C, size=N))
+    hot = rng.permutation(N).astype(np.int64)                      # hottest last
+    prefer_low_latency_gemm()
+
+    def world(tiers):
+        torch.manual_seed(17)
+        cfg = make_config(Fin, C, H, L, method="grad", rate=0.5, staleness_thres=4, device=DEV)
+        # the store's device copies: the 9 000 hottest rows, of which the cache's own tail holds a part
+        store = PinnedFeatureStore(feats, device=DEV, prefetch_cus=16,
+                                   hot_ids=torch.from_numpy(hot[-9000:].copy()) if tiers else None)
+        cache = HistoryCache(store, cfg, "history_uvm", total_num_node=N, buffer_bytes=6000 * 64 * 4, hot_ids=hot)
+        model = HistorySAGE(Fin, H, C, L, 0.0, "CSR_Layer", cfg, cache).to(DEV)
+        model.train()
+        return store, cache, model, torch.optim.Adam(model.parameters(), lr=1e-2, fused=True)
+
+    sampler = NeighborSampler(indptr, indices, fanout, labels=labels, seed=41, device=DEV, emit_view=True)
+    gen = torch.Generator(device=DEV).manual_seed(41)
+    seeds = [torch.randperm(N, device=DEV, generator=gen)[:n_seed].contiguous() for _ in range(4)]
+    order = [0, 1, 2, 0, 3, 1, 2, 0]
+    twins = {name: world(name == "tiered") for name in ("tiered", "plain")}
+    sets = {name: [sampler.sample(seeds[k], rng_seed=900 + k) for k in order] for name in twins}
+    compute = torch.cuda.Stream()
+    compute.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(compute):
+        for i in range(len(order)):
+            xs, losses = [], []
+            for name in ("tiered", "plain"):
+                store, cache, model, opt = twins[name]
+                b = sets[name][i]
+                cache.lookup_and_load(b, L)
+                xs.append(b.x.clone())
+                if i + 1 < len(order):
+                    cache.prefetch(sets[name][i + 1], speculative=True, num_layer=L)
+                loss = torch.nn.functional.nll_loss(model(b), b.y)
+                opt.zero_grad(set_to_none=True)
+                backward_on_this_thread(loss)
+                opt.step()
+                cache.update_history(b, i + 1)
+                losses.append(float(loss.detach()))
+            assert torch.equal(xs[0], xs[1]), i
+            assert losses[0] == losses[1] and np.isfinite(losses[0])
+            a, c = twins["tiered"][1], twins["plain"][1]
+            assert torch.equal(a.buffer, c.buffer) and torch.equal(a.full2embed, c.full2embed)
+            for p, q in zip(twins["tiered"][2].parameters(), twins["plain"][2].parameters()):
+                assert torch.equal(p, q)
+    torch.cuda.synchronize()
+    assert twins["tiered"][0].last_cold is not None and int(twins["tiered"][0].last_cold.sum()) > 0
