@@ -621,25 +621,34 @@ __global__ __launch_bounds__(HC_BLOCK) void load_mask_kernel(const uint8_t *__re
   __shared__ unsigned int s_cnt[LM_COUNTERS];
   if (threadIdx.x < LM_COUNTERS) s_cnt[threadIdx.x] = 0u;
   __syncthreads();
-  const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
-  bool u = false, hit = false, load = false, emb = false, adm = false;
-  if (i < n_all) {
-    u = used[i] != 0;
-    hit = sub2feat != nullptr && sub2feat[i] != -1;
-    load = u && !hit;
-    if (hit_feat != nullptr) hit_feat[i] = hit ? 1 : 0;
-    if (load_mask != nullptr) load_mask[i] = load ? 1 : 0;
+  // A block walks the elements with the grid's stride and adds its counts to the totals once: every block's
+  // adds land on one cache line, where they are served one after the other (hundreds of blocks with one element
+  // per thread spent most of the kernel queueing there).
+  unsigned int c_pruned = 0u, c_hit = 0u, c_load = 0u, c_emb = 0u, c_adm = 0u;
+  int64_t n_max = n_all > n1 ? n_all : n1;
+  if (n_prev > n_max) n_max = n_prev;
+  const int64_t stride = (int64_t)gridDim.x * HC_BLOCK;
+  for (int64_t base = (int64_t)blockIdx.x * HC_BLOCK; base < n_max; base += stride) {   // block-uniform trip count
+    const int64_t i = base + threadIdx.x;
+    bool u = false, hit = false, load = false, emb = false, adm = false;
+    if (i < n_all) {
+      u = used[i] != 0;
+      hit = sub2feat != nullptr && sub2feat[i] != -1;
+      load = u && !hit;
+      if (hit_feat != nullptr) hit_feat[i] = hit ? 1 : 0;
+      if (load_mask != nullptr) load_mask[i] = load ? 1 : 0;
+    }
+    if (counters == nullptr) continue;
+    if (sub2embed != nullptr && i < n1) emb = sub2embed[i] != -1;
+    if (prev_mask != nullptr && i < n_prev) adm = prev_mask[i] != 0;
+    c_pruned += (unsigned int)__popcll(__ballot(i < n_all && !u));
+    c_hit += (unsigned int)__popcll(__ballot(hit));
+    c_load += (unsigned int)__popcll(__ballot(load));
+    c_emb += (unsigned int)__popcll(__ballot(emb));
+    c_adm += (unsigned int)__popcll(__ballot(adm));
   }
-  if (sub2embed != nullptr && i < n1) emb = sub2embed[i] != -1;
-  if (prev_mask != nullptr && i < n_prev) adm = prev_mask[i] != 0;
   if (counters == nullptr) return;
-  const int lane = hc_lane();
-  const unsigned int c_pruned = (unsigned int)__popcll(__ballot(i < n_all && !u));
-  const unsigned int c_hit = (unsigned int)__popcll(__ballot(hit));
-  const unsigned int c_load = (unsigned int)__popcll(__ballot(load));
-  const unsigned int c_emb = (unsigned int)__popcll(__ballot(emb));
-  const unsigned int c_adm = (unsigned int)__popcll(__ballot(adm));
-  if (lane == 0) {
+  if (hc_lane() == 0) {                      // the ballots gave every lane of a wave the wave's counts
     if (c_emb) atomicAdd(&s_cnt[3], c_emb);
     if (c_pruned) atomicAdd(&s_cnt[4], c_pruned);
     if (c_hit) atomicAdd(&s_cnt[5], c_hit);
@@ -667,8 +676,11 @@ extern "C" int hc_load_mask(const uint8_t *used, const int64_t *sub2feat, const 
   int64_t n = n_all > n1 ? n_all : n1;
   if (n_prev > n) n = n_prev;
   if (n == 0) n = 1;                               // the call is still counted
-  const int64_t b = (n + HC_BLOCK - 1) / HC_BLOCK;
+  int64_t b = (n + HC_BLOCK - 1) / HC_BLOCK;
   if (!hc_grid_ok(b)) return HC_EUNSUPPORTED;
+  // with counters: few blocks, each walking its share (one add per block and counter); without: a thread per element
+  const int64_t cap = counters != nullptr ? 128 : 4096;
+  if (b > cap) b = cap;
   load_mask_kernel<<<dim3((unsigned)b), dim3(HC_BLOCK), 0, static_cast<hipStream_t>(stream)>>>(
       used, sub2feat, sub2embed, prev_mask, n_all, n1, n_prev, hit_feat, load_mask,
       reinterpret_cast<unsigned long long *>(counters));
