@@ -6,7 +6,7 @@ Files and element types (raw little-endian arrays, no headers):
 ``node_features.dat`` ([num_nodes, feature_dim] float32, float16 for mag240m;
 history_cache.py:141-149), ``csr_ptr_undirected.dat`` / ``csr_idx_undirected.dat`` (int64 CSR;
 /root/reference/test/test_cache.py:19-25,43-49), ``split/time/train_idx.dat`` (int64;
-test/test_cache.py:54-56).  ``node_labels.dat`` (int64) is this package's name for the labels,
+test/test_cache.py:54-56) and, beside it, ``valid_idx.dat`` / ``test_idx.dat`` for the trainer's evaluation.  ``node_labels.dat`` (int64) is this package's name for the labels,
 which the reference takes from its external loader.
 """
 import os
@@ -24,6 +24,8 @@ _FILES = {
     "hot": ("sorted_indices.dat", np.int64),
     "labels": ("node_labels.dat", np.int64),
     "train": (path.join("split", "time", "train_idx.dat"), np.int64),
+    "valid": (path.join("split", "time", "valid_idx.dat"), np.int64),
+    "test": (path.join("split", "time", "test_idx.dat"), np.int64),
 }
 
 
@@ -61,6 +63,12 @@ class ProcessedDataset:
 
     def train_idx(self):
         return self._array("train")
+
+    def split_idx(self, split):
+        """Node ids of a split: "train", "valid" or "test" (``split/time/<split>_idx.dat``)."""
+        if split not in ("train", "valid", "test"):
+            raise KeyError(split)
+        return self._array(split)
 
     def feature_store(self, device="cuda:0", out_dtype=None, chunk_rows=1 << 20, in_device_memory=False,
                       hot_rows=0):
@@ -105,7 +113,8 @@ class ProcessedDataset:
                                emit_view=emit_view, view_edges=view_edges, replay_slots=replay_slots)
 
 
-def write_processed(root, indptr, indices, features, hot_ids=None, labels=None, train_idx=None):
+def write_processed(root, indptr, indices, features, hot_ids=None, labels=None, train_idx=None, valid_idx=None,
+                    test_idx=None):
     """Write a dataset in the layout above (for tests and for converting in-memory graphs)."""
     d = path.join(str(root), "processed")
     os.makedirs(path.join(d, "split", "time"), exist_ok=True)
@@ -118,7 +127,8 @@ def write_processed(root, indptr, indices, features, hot_ids=None, labels=None, 
     if feats.shape[0] != n:
         raise ValueError("features must have one row per node")
     feats.tofile(path.join(d, "node_features.dat"))
-    for key, arr in (("hot", hot_ids), ("labels", labels), ("train", train_idx)):
+    for key, arr in (("hot", hot_ids), ("labels", labels), ("train", train_idx), ("valid", valid_idx),
+                     ("test", test_idx)):
         if arr is not None:
             np.ascontiguousarray(arr, dtype=np.int64).tofile(path.join(d, _FILES[key][0]))
     return d

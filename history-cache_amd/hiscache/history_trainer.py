@@ -1,0 +1,165 @@
+"""HistoryTrainer: the loop around the path -- sample, ``lookup_and_load``, forward, loss, backward, optimizer,
+``update_history`` -- with the method names and attributes of the reference's trainer
+(/root/reference/hiscache/history_trainer.py:15-255: ``cxg_train_epoch`` :176-193, ``cxg_eval_epoch`` :195-227,
+``train`` :229-255).
+
+The reference takes its loader, its UVM store, optimizer, scheduler, loss and evaluator from two external packages
+(``cxgnndl.get_loader`` / ``cxgnndl.UVM``, ``cxgnncomp.get_optimizer`` ...).  Here they come from the dataset
+directory the configuration names (``ProcessedDataset``: graph, features, splits, hotness order), the device
+sampler (one batch ahead on its side stream, every batch with the transposed view of its CSR) and torch (Adam,
+NLL on the log-softmax the models return, accuracy).  What the hardware adds is opt-in: the feature matrix in
+device memory or its hottest rows there, and the iteration recorded per padded batch shape and replayed
+(``RecordedIteration``).
+"""
+import time
+
+import numpy as np
+import torch
+
+from .dataset import ProcessedDataset
+from .history_cache import HistoryCache
+from .history_model import get_model
+from .recorded import RecordedIteration
+from .util import backward_on_this_thread, log
+
+
+def _option(config, dotted, default):
+    node = config
+    for key in dotted.split("."):
+        if not hasattr(node, "get") or node.get(key) is None:
+            return default
+        node = node[key]
+    return node
+
+
+class HistoryTrainer:
+
+    def __init__(self, config, dataset=None, fanout=None, batch_size=None, lr=None, num_epochs=None, eval_begin=None,
+                 features_in_device_memory=False, hot_rows=0, cache_bytes=None, recorded=False, replay_slots=0,
+                 seed=0):
+        """``config``: the tree ``make_config`` builds (``dl.dataset.path`` names the dataset directory).  The
+        loader's settings are arguments, with the configuration's own keys as defaults where it has them
+        (``dl.sampler.train.batch_size`` / ``num_neighbors``, ``train.optimizer.lr``, ``train.train.num_epochs`` /
+        ``eval_begin``).  ``cache_bytes``: size of the cache's buffer (default: what the configuration's
+        ``history.limit`` and the free device memory give, as in the reference).  ``recorded``: train through
+        ``RecordedIteration`` (batches of ``batch_size`` seeds; the last, shorter batch of an epoch takes the
+        ordinary path)."""
+        self.config = config
+        self.device = torch.device(config.dl.device)
+        self.feat_mode = config.dl.loading.feat_mode
+        self.num_layers = int(config.train.model.num_layers)
+        self.batch_size = int(batch_size or _option(config, "dl.sampler.train.batch_size", 1000))
+        fanout = fanout or _option(config, "dl.sampler.train.num_neighbors", None)
+        if fanout is None or len(fanout) != self.num_layers:
+            raise ValueError("fanout: one neighbour count per layer")
+        self.num_epochs = int(num_epochs if num_epochs is not None else _option(config, "train.train.num_epochs", 1))
+        self.eval_begin = int(eval_begin if eval_begin is not None else _option(config, "train.train.eval_begin", 0))
+        self.dataset = dataset or ProcessedDataset(config.dl.dataset.path, config.dl.dataset.feature_dim)
+        ds = self.dataset
+        # the feature store (cxgnndl.UVM's role): pinned host memory read zero-copy, the hottest rows or the whole
+        # matrix in device memory on request
+        self.uvm = ds.feature_store(device=self.device, in_device_memory=features_in_device_memory,
+                                    hot_rows=hot_rows)
+        self.table = HistoryCache(uvm=self.uvm, config=config, mode=self.feat_mode, buffer_bytes=cache_bytes)
+        self.model = get_model(config, self.table).to(self.device)
+        self.recorded = bool(recorded)
+        self.optimizer = torch.optim.Adam(self.model.parameters(),
+                                          lr=float(lr or _option(config, "train.optimizer.lr", 1e-3)), fused=True,
+                                          capturable=self.recorded)
+        self.scheduler = None
+        self.loss_fn = torch.nn.functional.nll_loss
+        self.sampler = ds.sampler(list(fanout), device=self.device, seed=seed, emit_view=True,
+                                  replay_slots=replay_slots)
+        self.splits = {"train": torch.from_numpy(np.array(ds.train_idx())).to(self.device)}
+        for split, key in (("val", "valid"), ("test", "test")):
+            if ds.has(key):
+                self.splits[split] = torch.from_numpy(np.array(ds.split_idx(key))).to(self.device)
+        self._generator = torch.Generator(device=self.device).manual_seed(seed)
+        self._step = RecordedIteration(self.model, self.table, self.optimizer, self.num_layers,
+                                       loss_fn=self.loss_fn) if self.recorded else None
+        self.glb_iter = 0
+        self.val_metrics = []
+        self.test_metrics = []
+        self.best_metric = 0
+        self.metric = None
+        self.epoch_seconds = []
+
+    # ------------------------------------------------------------------ batches
+    def _batches(self, ids, shuffle):
+        """Batches of ``ids``, every one sampled on the sampler's side stream while the one before is in use."""
+        if shuffle:
+            ids = ids[torch.randperm(ids.numel(), device=self.device, generator=self._generator)]
+        chunks = [ids[lo:lo + self.batch_size].contiguous() for lo in range(0, ids.numel(), self.batch_size)]
+        if not chunks:
+            return
+        pending = self.sampler.sample_async(chunks[0])
+        for nxt in chunks[1:] + [None]:
+            batch = pending.get()
+            pending = self.sampler.sample_async(nxt) if nxt is not None else None
+            yield batch
+
+    @staticmethod
+    def evaluator(y_pred, y_true):
+        """Accuracy of the arg-max class (the evaluator of the node-classification datasets)."""
+        return (y_pred.argmax(dim=-1) == y_true).float().mean()
+
+    # ------------------------------------------------------------------ epochs
+    def cxg_train_epoch(self):
+        self.model.train()
+        tepoch = time.time()
+        num_layers = len(self.model.convs)
+        for batch in self._batches(self.splits["train"], shuffle=True):
+            if self._step is not None:
+                self._step(batch, self.glb_iter)
+            else:
+                self.optimizer.zero_grad(set_to_none=True)
+                self.table.lookup_and_load(batch, num_layers)
+                out = self.model(batch)
+                loss = self.loss_fn(out, batch.y)
+                backward_on_this_thread(loss)
+                self.optimizer.step()
+                self.table.update_history(batch, self.glb_iter)
+            if self.scheduler is not None:
+                self.scheduler.step()
+            self.glb_iter += 1
+        torch.cuda.synchronize(self.device)
+        self.epoch_seconds.append(time.time() - tepoch)
+        log.info(f"epoch time: {self.epoch_seconds[-1]}")
+
+    @torch.no_grad()
+    def cxg_eval_epoch(self, split="val"):
+        self.model.eval()
+        y_preds, y_trues, losses = [], [], []
+        tepoch = time.time()
+        num_layers = len(self.model.convs)
+        for batch in self._batches(self.splits[split], shuffle=False):
+            self.table.lookup_and_load(batch, num_layers, feature_cache_only=True)
+            out = self.model(batch)
+            losses.append(self.loss_fn(out, batch.y).detach())
+            y_preds.append(out.detach())
+            y_trues.append(batch.y.detach().clone())
+        torch.cuda.synchronize(self.device)
+        self.metric = self.evaluator(torch.cat(y_preds, dim=0), torch.cat(y_trues, dim=0)).item()
+        log.info(f"epoch time: {time.time() - tepoch}")
+        log.info(f"{split}-metric: {self.metric}")
+        if split == "val":
+            self.best_metric = max(self.best_metric, self.metric)
+            log.info(f"best-metric: {self.best_metric}")
+            self.val_metrics.append(self.metric)
+        else:
+            self.test_metrics.append(self.metric)
+
+    def train(self):
+        for epoch in range(self.num_epochs):
+            log.info(f"Epoch {epoch}/{self.num_epochs}")
+            self.cxg_train_epoch()
+            if epoch >= self.eval_begin:
+                if "val" in self.splits:
+                    self.cxg_eval_epoch(split="val")
+                if "test" in self.splits and "mag" not in str(self.config.dl.dataset.name).lower():
+                    self.cxg_eval_epoch(split="test")
+        if len(self.val_metrics) > 0:
+            val, test = np.array(self.val_metrics), np.array(self.test_metrics)
+            log.info(f"best-val-metrics: {val.max()} at epoch {val.argmax()}")
+            if len(test) == len(val):
+                log.info(f"best-test-metrics: {test.max()} valided test-metric {test[val.argmax()]}")

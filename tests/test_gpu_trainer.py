@@ -1,0 +1,63 @@
+"""``HistoryTrainer`` over a dataset directory: epochs of the ordinary and of the recorded loop, evaluation on the
+validation and test splits with the feature cache only, the bookkeeping the reference's trainer keeps."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def dataset(tmp_path, rng, N=6000, Fin=32, C=4):
+    from hiscache import write_processed
+    deg = 10
+    indptr = np.arange(0, (N + 1) * deg, deg, dtype=np.int64)
+    indices = rng.integers(0, N, size=N * deg).astype(np.int64)
+    feats = rng.standard_normal((N, Fin)).astype(np.float32)
+    labels = feats[:, :C].argmax(1).astype(np.int64)              # a node's own features decide its label
+    perm = rng.permutation(N)
+    write_processed(tmp_path, indptr, indices, feats, hot_ids=rng.permutation(N), labels=labels,
+                    train_idx=perm[:3700], valid_idx=perm[3700:4800], test_idx=perm[4800:])
+    return feats, labels
+
+
+@pytest.mark.parametrize("recorded,placement", [(False, "host"), (True, "host"), (True, "hot"), (False, "device")])
+def test_trainer_trains_and_evaluates(tmp_path, recorded, placement):
+    from hiscache import HistoryTrainer, make_config
+    rng = np.random.default_rng(77)
+    Fin, H, C, L = 32, 32, 4, 3
+    dataset(tmp_path, rng, Fin=Fin, C=C)
+    cfg = make_config(Fin, C, H, L, method="grad", rate=0.6, staleness_thres=5, device=DEV, path=str(tmp_path))
+    torch.manual_seed(7)
+    trainer = HistoryTrainer(cfg, fanout=[4, 3, 2], batch_size=200, lr=1e-2, num_epochs=3, eval_begin=1,
+                             features_in_device_memory=placement == "device",
+                             hot_rows=1500 if placement == "hot" else 0, cache_bytes=1500 * 32 * 4,
+                             recorded=recorded)
+    assert trainer.table.total_num_node == 6000 and set(trainer.splits) == {"train", "val", "test"}
+    assert (trainer.uvm.hot_rows is not None) == (placement == "hot")
+    trainer.train()
+    assert trainer.glb_iter == 3 * 19                              # 3 700 training nodes in batches of 200
+    assert len(trainer.val_metrics) == 2 and len(trainer.test_metrics) == 2 and len(trainer.epoch_seconds) == 3
+    assert trainer.best_metric == max(trainer.val_metrics)
+    assert trainer.val_metrics[-1] > 0.5 and trainer.test_metrics[-1] > 0.5    # four classes: chance is 0.25
+    assert trainer.table.header > 0                                 # rows were admitted
+    if recorded:
+        assert trainer._step.replays >= 30, trainer._step.shapes()  # (the nineteenth batch of an epoch is shorter)
+    assert not trainer.model.training                                # left in evaluation mode, as the reference leaves it
+
+
+def test_trainer_reads_its_settings_from_the_configuration(tmp_path):
+    from hiscache import Config, HistoryTrainer, make_config
+    rng = np.random.default_rng(78)
+    dataset(tmp_path, rng, N=2000)
+    cfg = make_config(32, 4, 32, 2, device=DEV, path=str(tmp_path))     # (two layers: hidden width = feature width)
+    cfg["dl"]["sampler"] = Config({"train": {"batch_size": 128, "num_neighbors": [3, 2]}})
+    cfg["train"]["train"] = Config({"num_epochs": 2, "eval_begin": 5})
+    cfg["train"]["optimizer"] = Config({"lr": 0.003})
+    trainer = HistoryTrainer(cfg, cache_bytes=400 * 32 * 4)
+    assert trainer.batch_size == 128 and trainer.num_epochs == 2 and trainer.eval_begin == 5
+    assert trainer.optimizer.param_groups[0]["lr"] == 0.003
+    trainer.train()
+    assert trainer.val_metrics == [] and len(trainer.epoch_seconds) == 2     # evaluation begins at epoch 5
+    with pytest.raises(ValueError):
+        HistoryTrainer(make_config(32, 4, 32, 2, device=DEV, path=str(tmp_path)), fanout=[3], cache_bytes=400 * 32 * 4)
