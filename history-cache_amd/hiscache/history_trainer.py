@@ -20,6 +20,7 @@ from .dataset import ProcessedDataset
 from .history_cache import HistoryCache
 from .history_model import get_model
 from .recorded import RecordedIteration
+from .ring_cache import RingHistoryCache
 from .util import backward_on_this_thread, log
 
 
@@ -35,13 +36,15 @@ def _option(config, dotted, default):
 class HistoryTrainer:
 
     def __init__(self, config, dataset=None, fanout=None, batch_size=None, lr=None, num_epochs=None, eval_begin=None,
-                 features_in_device_memory=False, hot_rows=0, cache_bytes=None, recorded=False, replay_slots=0,
-                 seed=0):
+                 features_in_device_memory=False, hot_rows=0, cache_bytes=None, ring_rows=0, recorded=False,
+                 replay_slots=0, seed=0):
         """``config``: the tree ``make_config`` builds (``dl.dataset.path`` names the dataset directory).  The
         loader's settings are arguments, with the configuration's own keys as defaults where it has them
         (``dl.sampler.train.batch_size`` / ``num_neighbors``, ``train.optimizer.lr``, ``train.train.num_epochs`` /
         ``eval_begin``).  ``cache_bytes``: size of the cache's buffer (default: what the configuration's
-        ``history.limit`` and the free device memory give, as in the reference).  ``recorded``: train through
+        ``history.limit`` and the free device memory give, as in the reference).  ``ring_rows`` > 0: the embeddings live in a
+        ``RingHistoryCache`` of that many fp16 rows instead (entries age out after ``history.staleness_thres``
+        iterations; no feature cache inside it: use ``hot_rows``).  ``recorded``: train through
         ``RecordedIteration`` (batches of ``batch_size`` seeds; the last, shorter batch of an epoch takes the
         ordinary path)."""
         self.config = config
@@ -60,7 +63,14 @@ class HistoryTrainer:
         # matrix in device memory on request
         self.uvm = ds.feature_store(device=self.device, in_device_memory=features_in_device_memory,
                                     hot_rows=hot_rows)
-        self.table = HistoryCache(uvm=self.uvm, config=config, mode=self.feat_mode, buffer_bytes=cache_bytes)
+        if ring_rows:
+            self.table = RingHistoryCache(self.uvm, ds.num_nodes, config.dl.dataset.feature_dim,
+                                          config.train.model.hidden_dim, capacity=int(ring_rows),
+                                          num_layers=self.num_layers, table_dtype=torch.float16,
+                                          rate=float(config.history.rate), method=config.history.method,
+                                          age_limit=int(config.history.staleness_thres), device=self.device)
+        else:
+            self.table = HistoryCache(uvm=self.uvm, config=config, mode=self.feat_mode, buffer_bytes=cache_bytes)
         self.model = get_model(config, self.table).to(self.device)
         self.recorded = bool(recorded)
         self.optimizer = torch.optim.Adam(self.model.parameters(),

@@ -62,10 +62,16 @@ class RingHistoryCache:
     def header(self):
         return int(self._header.item())
 
-    def lookup_and_load(self, batch, num_layer=None):
+    def lookup_and_load(self, batch, num_layer=None, feature_cache_only=False):
         if num_layer is None:
             num_layer = self.num_layers_all
         sub_to_full = batch.sub_to_full
+        if feature_cache_only:
+            # evaluation (/root/reference/hiscache/history_cache.py:276-288): every node's features, no embedding
+            # is looked up and the table's state is left alone
+            batch.x = self.uvm.get(sub_to_full)
+            self.sub2embed = self.cached_embedding = self.used_masks = None
+            return None
         n1 = int(batch.num_node_in_layer[1])
         # A batch padded to fixed sizes for a recorded iteration (hiscache.RecordedIteration) carries its real
         # sizes and the iteration number on the device: rows behind the real 1-hop nodes find nothing, and this

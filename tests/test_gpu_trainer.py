@@ -21,8 +21,10 @@ def dataset(tmp_path, rng, N=6000, Fin=32, C=4):
     return feats, labels
 
 
-@pytest.mark.parametrize("recorded,placement", [(False, "host"), (True, "host"), (True, "hot"), (False, "device")])
-def test_trainer_trains_and_evaluates(tmp_path, recorded, placement):
+@pytest.mark.parametrize("recorded,placement,ring", [(False, "host", False), (True, "host", False), (True, "hot", False),
+                                                     (False, "device", False), (False, "hot", True),
+                                                     (True, "host", True)])
+def test_trainer_trains_and_evaluates(tmp_path, recorded, placement, ring):
     from hiscache import HistoryTrainer, make_config
     rng = np.random.default_rng(77)
     Fin, H, C, L = 32, 32, 4, 3
@@ -32,7 +34,7 @@ def test_trainer_trains_and_evaluates(tmp_path, recorded, placement):
     trainer = HistoryTrainer(cfg, fanout=[4, 3, 2], batch_size=200, lr=1e-2, num_epochs=3, eval_begin=1,
                              features_in_device_memory=placement == "device",
                              hot_rows=1500 if placement == "hot" else 0, cache_bytes=1500 * 32 * 4,
-                             recorded=recorded)
+                             ring_rows=3000 if ring else 0, recorded=recorded)
     assert trainer.table.total_num_node == 6000 and set(trainer.splits) == {"train", "val", "test"}
     assert (trainer.uvm.hot_rows is not None) == (placement == "hot")
     trainer.train()
@@ -40,6 +42,7 @@ def test_trainer_trains_and_evaluates(tmp_path, recorded, placement):
     assert len(trainer.val_metrics) == 2 and len(trainer.test_metrics) == 2 and len(trainer.epoch_seconds) == 3
     assert trainer.best_metric == max(trainer.val_metrics)
     assert trainer.val_metrics[-1] > 0.5 and trainer.test_metrics[-1] > 0.5    # four classes: chance is 0.25
+    assert type(trainer.table).__name__ == ("RingHistoryCache" if ring else "HistoryCache")
     assert trainer.table.header > 0                                 # rows were admitted
     if recorded:
         assert trainer._step.replays >= 30, trainer._step.shapes()  # (the nineteenth batch of an epoch is shorter)
