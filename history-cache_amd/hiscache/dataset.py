@@ -71,13 +71,14 @@ class ProcessedDataset:
         return self._array(split)
 
     def feature_store(self, device="cuda:0", out_dtype=None, chunk_rows=1 << 20, in_device_memory=False,
-                      hot_rows=0):
+                      hot_rows=0, prefetch_cus=0):
         """Pinned, GPU-mapped copy of ``node_features.dat``, read from disk in chunks (the file is
         never held twice in memory).  ``in_device_memory``: the matrix goes to the GPU's own memory
         instead (288 GB hold the papers100M matrix, 57 GB, beside its history table), and the store's
         gathers read it there.  ``hot_rows``: for a matrix that stays in host memory, copies of that many
         rows, the last (hottest) entries of ``sorted_indices.dat``, are kept in device memory and served from
-        there (the reference's feature cache, history_cache.py:124-142)."""
+        there (the reference's feature cache, history_cache.py:124-142).  ``prefetch_cus``: see
+        ``PinnedFeatureStore`` (the stream of the read-ahead is kept to that many compute units)."""
         p = path.join(self.dir, "node_features.dat")
         want = self.num_nodes * self.feature_dim * self.feature_dtype.itemsize
         if os.path.getsize(p) != want:
@@ -96,7 +97,7 @@ class ProcessedDataset:
                 hi = min(self.num_nodes, lo + chunk_rows)
                 dst[lo:hi] = src[lo:hi]
         del src
-        store = PinnedFeatureStore(buf, device=device, out_dtype=out_dtype or torch.float32)
+        store = PinnedFeatureStore(buf, device=device, out_dtype=out_dtype or torch.float32, prefetch_cus=prefetch_cus)
         if hot_rows and not in_device_memory:
             order = self.hot_ids()
             store.set_hot_rows(torch.from_numpy(np.array(order[max(0, len(order) - int(hot_rows)):])))

@@ -37,7 +37,7 @@ class HistoryTrainer:
 
     def __init__(self, config, dataset=None, fanout=None, batch_size=None, lr=None, num_epochs=None, eval_begin=None,
                  features_in_device_memory=False, hot_rows=0, cache_bytes=None, ring_rows=0, recorded=False,
-                 replay_slots=0, seed=0):
+                 read_ahead=False, replay_slots=0, seed=0):
         """``config``: the tree ``make_config`` builds (``dl.dataset.path`` names the dataset directory).  The
         loader's settings are arguments, with the configuration's own keys as defaults where it has them
         (``dl.sampler.train.batch_size`` / ``num_neighbors``, ``train.optimizer.lr``, ``train.train.num_epochs`` /
@@ -46,7 +46,9 @@ class HistoryTrainer:
         ``RingHistoryCache`` of that many fp16 rows instead (entries age out after ``history.staleness_thres``
         iterations; no feature cache inside it: use ``hot_rows``).  ``recorded``: train through
         ``RecordedIteration`` (batches of ``batch_size`` seeds; the last, shorter batch of an epoch takes the
-        ordinary path)."""
+        ordinary path).  ``read_ahead``: the feature rows of the next batch are read over the host link beside
+        the current iteration (on a stream kept to 16 compute units; the epoch then runs on a stream of its
+        own), for a matrix that is not wholly in device memory."""
         self.config = config
         self.device = torch.device(config.dl.device)
         self.feat_mode = config.dl.loading.feat_mode
@@ -61,8 +63,10 @@ class HistoryTrainer:
         ds = self.dataset
         # the feature store (cxgnndl.UVM's role): pinned host memory read zero-copy, the hottest rows or the whole
         # matrix in device memory on request
+        self.read_ahead = bool(read_ahead) and not features_in_device_memory
         self.uvm = ds.feature_store(device=self.device, in_device_memory=features_in_device_memory,
-                                    hot_rows=hot_rows)
+                                    hot_rows=hot_rows, prefetch_cus=16 if self.read_ahead else 0)
+        self._compute = torch.cuda.Stream(device=self.device) if self.read_ahead else None   # default priority
         if ring_rows:
             self.table = RingHistoryCache(self.uvm, ds.num_nodes, config.dl.dataset.feature_dim,
                                           config.train.model.hidden_dim, capacity=int(ring_rows),
@@ -95,18 +99,35 @@ class HistoryTrainer:
         self.epoch_seconds = []
 
     # ------------------------------------------------------------------ batches
-    def _batches(self, ids, shuffle):
-        """Batches of ``ids``, every one sampled on the sampler's side stream while the one before is in use."""
+    def _batches(self, ids, shuffle, read_ahead=False):
+        """Batches of ``ids``, every one sampled on the sampler's side stream while the one before is in use;
+        with ``read_ahead`` a batch is handed out once the next one is drawn and its feature read is under way."""
         if shuffle:
             ids = ids[torch.randperm(ids.numel(), device=self.device, generator=self._generator)]
         chunks = [ids[lo:lo + self.batch_size].contiguous() for lo in range(0, ids.numel(), self.batch_size)]
         if not chunks:
             return
+        chunks.append(None)
         pending = self.sampler.sample_async(chunks[0])
-        for nxt in chunks[1:] + [None]:
-            batch = pending.get()
-            pending = self.sampler.sample_async(nxt) if nxt is not None else None
+        if not read_ahead:
+            for nxt in chunks[1:]:
+                batch = pending.get()
+                pending = self.sampler.sample_async(nxt) if nxt is not None else None
+                yield batch
+            return
+        batch = pending.get()
+        pending = self.sampler.sample_async(chunks[1]) if chunks[1] is not None else None
+        for k in range(1, len(chunks)):
+            nxt = None
+            if pending is not None:
+                nxt = pending.get()
+                pending = self.sampler.sample_async(chunks[k + 1]) if chunks[k + 1] is not None else None
+                if self._step is not None:
+                    self._step.prefetch(nxt)        # straight into the array the batch's recording reads
+                else:
+                    self.table.prefetch(nxt, speculative=True, num_layer=self.num_layers)
             yield batch
+            batch = nxt
 
     @staticmethod
     def evaluator(y_pred, y_true):
@@ -115,10 +136,19 @@ class HistoryTrainer:
 
     # ------------------------------------------------------------------ epochs
     def cxg_train_epoch(self):
+        if self._compute is None:
+            return self._train_epoch()
+        # the read-ahead runs beside the iteration only when the iteration is on a stream of its own
+        self._compute.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(self._compute):
+            self._train_epoch()
+        torch.cuda.current_stream(self.device).wait_stream(self._compute)
+
+    def _train_epoch(self):
         self.model.train()
         tepoch = time.time()
         num_layers = len(self.model.convs)
-        for batch in self._batches(self.splits["train"], shuffle=True):
+        for batch in self._batches(self.splits["train"], shuffle=True, read_ahead=self.read_ahead):
             if self._step is not None:
                 self._step(batch, self.glb_iter)
             else:

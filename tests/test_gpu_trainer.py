@@ -21,10 +21,11 @@ def dataset(tmp_path, rng, N=6000, Fin=32, C=4):
     return feats, labels
 
 
-@pytest.mark.parametrize("recorded,placement,ring", [(False, "host", False), (True, "host", False), (True, "hot", False),
-                                                     (False, "device", False), (False, "hot", True),
-                                                     (True, "host", True)])
-def test_trainer_trains_and_evaluates(tmp_path, recorded, placement, ring):
+@pytest.mark.parametrize("recorded,placement,ring,read_ahead",
+                         [(False, "host", False, False), (True, "host", False, False), (True, "hot", False, True),
+                          (False, "device", False, False), (False, "hot", True, True), (True, "host", True, True),
+                          (False, "host", False, True)])
+def test_trainer_trains_and_evaluates(tmp_path, recorded, placement, ring, read_ahead):
     from hiscache import HistoryTrainer, make_config
     rng = np.random.default_rng(77)
     Fin, H, C, L = 32, 32, 4, 3
@@ -34,7 +35,7 @@ def test_trainer_trains_and_evaluates(tmp_path, recorded, placement, ring):
     trainer = HistoryTrainer(cfg, fanout=[4, 3, 2], batch_size=200, lr=1e-2, num_epochs=3, eval_begin=1,
                              features_in_device_memory=placement == "device",
                              hot_rows=1500 if placement == "hot" else 0, cache_bytes=1500 * 32 * 4,
-                             ring_rows=3000 if ring else 0, recorded=recorded)
+                             ring_rows=3000 if ring else 0, recorded=recorded, read_ahead=read_ahead)
     assert trainer.table.total_num_node == 6000 and set(trainer.splits) == {"train", "val", "test"}
     assert (trainer.uvm.hot_rows is not None) == (placement == "hot")
     trainer.train()
@@ -45,6 +46,8 @@ def test_trainer_trains_and_evaluates(tmp_path, recorded, placement, ring):
     assert type(trainer.table).__name__ == ("RingHistoryCache" if ring else "HistoryCache")
     assert trainer.table.header > 0                                 # rows were admitted
     if recorded:
+        if read_ahead:                                              # rows read straight into the recordings' arrays
+            assert any(k[2] >= 0 and v[2] for k, v in trainer._step.shapes().items()), trainer._step.shapes()
         assert trainer._step.replays >= 30, trainer._step.shapes()  # (the nineteenth batch of an epoch is shorter)
     assert not trainer.model.training                                # left in evaluation mode, as the reference leaves it
 
