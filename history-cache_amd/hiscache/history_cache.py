@@ -14,7 +14,9 @@ Differences that a caller can see:
   * ``header`` lives on the device; reading the attribute synchronises;
   * rows that would be appended beyond the buffer are dropped and counted in ``overflow``
     (the reference raises a shape error there, history_cache.py:219-221);
-  * ``num_layer`` of ``lookup_and_load`` may be omitted (taken from the config).
+  * ``num_layer`` of ``lookup_and_load`` may be omitted (taken from the config);
+  * a ``feature_cache_only`` lookup clears ``used_masks`` (the reference leaves the last training batch's masks
+    in place, which its relational model then applies to the evaluation batch).
 """
 import math
 import time
@@ -232,6 +234,7 @@ class HistoryCache:
             _be.gather_rows(self.buffer.view(-1, self.in_channels), self.sub2feat, mask=hit, out=x,
                             accumulate=True)
             batch.x = x
+            self.used_masks = None          # nothing is pruned in evaluation: no masks of an earlier batch linger
             return None
 
         n1 = int(batch.num_node_in_layer[1])

@@ -550,7 +550,10 @@ class HistoryRGCN(torch.nn.Module):
         L = self.num_layers
         etypes = self.edge_types(batch)
         none = torch.empty(0, device=x.device)
-        masks = self.table.used_masks
+        # the used masks belong to the training lookup of this batch; an evaluation lookup
+        # (``feature_cache_only``) prunes nothing and computes none (the reference keeps reading the last
+        # training batch's masks there, /root/reference/hiscache/history_model.py:373-396)
+        masks = self.table.used_masks if self.training else None
         view = getattr(batch, "view", None)                  # shared transposed view, if the loader emitted it
         dev = getattr(batch, "dev", None)                    # a padded batch carries its real sizes on the device
         ptrs = getattr(batch, "ptr_of_layer", None)          # ... and row offsets per layer (see HistorySAGE.forward)

@@ -18,7 +18,7 @@ import torch
 
 from .dataset import ProcessedDataset
 from .history_cache import HistoryCache
-from .history_model import get_model
+from .history_model import HistoryRGCN, get_model
 from .recorded import RecordedIteration
 from .ring_cache import RingHistoryCache
 from .util import backward_on_this_thread, log
@@ -37,7 +37,7 @@ class HistoryTrainer:
 
     def __init__(self, config, dataset=None, fanout=None, batch_size=None, lr=None, num_epochs=None, eval_begin=None,
                  features_in_device_memory=False, hot_rows=0, cache_bytes=None, ring_rows=0, recorded=False,
-                 read_ahead=False, replay_slots=0, seed=0):
+                 read_ahead=False, replay_slots=0, seed=0, model_factory=None):
         """``config``: the tree ``make_config`` builds (``dl.dataset.path`` names the dataset directory).  The
         loader's settings are arguments, with the configuration's own keys as defaults where it has them
         (``dl.sampler.train.batch_size`` / ``num_neighbors``, ``train.optimizer.lr``, ``train.train.num_epochs`` /
@@ -48,7 +48,8 @@ class HistoryTrainer:
         ``RecordedIteration`` (batches of ``batch_size`` seeds; the last, shorter batch of an epoch takes the
         ordinary path).  ``read_ahead``: the feature rows of the next batch are read over the host link beside
         the current iteration (on a stream kept to 16 compute units; the epoch then runs on a stream of its
-        own), for a matrix that is not wholly in device memory."""
+        own), for a matrix that is not wholly in device memory.  ``model_factory(config, table)``: builds
+        the model instead of ``get_model`` (a relational model with its own node-type ranges, say)."""
         self.config = config
         self.device = torch.device(config.dl.device)
         self.feat_mode = config.dl.loading.feat_mode
@@ -75,15 +76,16 @@ class HistoryTrainer:
                                           age_limit=int(config.history.staleness_thres), device=self.device)
         else:
             self.table = HistoryCache(uvm=self.uvm, config=config, mode=self.feat_mode, buffer_bytes=cache_bytes)
-        self.model = get_model(config, self.table).to(self.device)
+        self.model = (model_factory or get_model)(config, self.table).to(self.device)
         self.recorded = bool(recorded)
         self.optimizer = torch.optim.Adam(self.model.parameters(),
                                           lr=float(lr or _option(config, "train.optimizer.lr", 1e-3)), fused=True,
                                           capturable=self.recorded)
         self.scheduler = None
         self.loss_fn = torch.nn.functional.nll_loss
+        # every batch comes with the transposed view of its CSR; the relational layer also reads the view's edge slots
         self.sampler = ds.sampler(list(fanout), device=self.device, seed=seed, emit_view=True,
-                                  replay_slots=replay_slots)
+                                  view_edges=isinstance(self.model, HistoryRGCN), replay_slots=replay_slots)
         self.splits = {"train": torch.from_numpy(np.array(ds.train_idx())).to(self.device)}
         for split, key in (("val", "valid"), ("test", "test")):
             if ds.has(key):

@@ -67,3 +67,31 @@ def test_trainer_reads_its_settings_from_the_configuration(tmp_path):
     assert trainer.val_metrics == [] and len(trainer.epoch_seconds) == 2     # evaluation begins at epoch 5
     with pytest.raises(ValueError):
         HistoryTrainer(make_config(32, 4, 32, 2, device=DEV, path=str(tmp_path)), fanout=[3], cache_bytes=400 * 32 * 4)
+
+
+@pytest.mark.parametrize("recorded", [False, True])
+def test_trainer_with_a_relational_model(tmp_path, recorded):
+    """A model factory in place of ``get_model``: the relational model with node-type ranges of this dataset (three
+    node types, five relations from the type pairs); the sampler then emits the view's edge slots too."""
+    from hiscache import HistoryRGCN, HistoryTrainer, make_config
+    rng = np.random.default_rng(79)
+    N, Fin, H, C, L, K = 6000, 32, 32, 4, 2, 5
+    dataset(tmp_path, rng, N=N, Fin=Fin, C=C)
+    cfg = make_config(Fin, C, H, L, method="grad", rate=0.6, staleness_thres=5, device=DEV, path=str(tmp_path),
+                      model_type="rgcn", num_rel=K, name="rmag240m")
+
+    def factory(config, table):
+        return HistoryRGCN(Fin, H, C, L, 0.0, "CSR_Layer", config, table, num_rel=K, dataset_name="rmag240m",
+                           type_bounds=[N // 2, N - 500], pair_to_rel=[[0, 1, 0], [2, 0, 3], [0, 4, 0]])
+
+    torch.manual_seed(8)
+    trainer = HistoryTrainer(cfg, fanout=[5, 4], batch_size=200, lr=1e-2, num_epochs=3, eval_begin=2,
+                             cache_bytes=1500 * 32 * 4, recorded=recorded, model_factory=factory)
+    assert trainer.sampler.view_edges
+    trainer.train()
+    assert len(trainer.val_metrics) == 1 and trainer.test_metrics == []      # (no test epoch for the mag datasets)
+    # (labels decided by a node's own features are out of reach of a model without a self term: only the run counts)
+    assert 0.0 <= trainer.val_metrics[0] <= 1.0 and trainer.table.header > 0
+    assert all(torch.isfinite(p).all() for p in trainer.model.parameters())
+    if recorded:
+        assert trainer._step.replays >= 30, trainer._step.shapes()
