@@ -14,13 +14,14 @@ from .history_model import (HistoryRGCN, HistorySAGE, MyRGCNConvHistory2, MySage
                             prefer_low_latency_gemm, typed_csr)
 from .history_table import HistoryTable
 from .history_trainer import HistoryTrainer
+from . import hotness
 from .recorded import RecordedIteration
 from .ring_cache import RingHistoryCache
 from .sampler import NeighborSampler
 from .util import Config, backward_on_this_thread, make_config, quantile_threshold
 
 __all__ = [
-    "HistoryCache", "HistoryTable", "HistoryTrainer", "RingHistoryCache", "RecordedIteration", "HistorySAGE", "HistoryRGCN", "MySageConvHistory", "MyRGCNConvHistory2", "typed_csr", "get_model", "prefer_low_latency_gemm",
+    "HistoryCache", "HistoryTable", "HistoryTrainer", "hotness", "RingHistoryCache", "RecordedIteration", "HistorySAGE", "HistoryRGCN", "MySageConvHistory", "MyRGCNConvHistory2", "typed_csr", "get_model", "prefer_low_latency_gemm",
     "PinnedFeatureStore", "NeighborSampler", "ProcessedDataset", "write_processed", "Config", "make_config", "quantile_threshold", "backward_on_this_thread",
     "count_history_reconstruct", "get_graph_structure_score", "record_history",
 ]
