@@ -42,6 +42,7 @@ class PinnedFeatureStore:
         self.hot_rows = None            # [n_hot, F] device copies of the most requested rows, or None
         self.hot_slot = None            # int32 per node: its row in hot_rows, or -1
         self.last_cold = None           # flags of the last tiered read: the rows that came over the host link
+        self._inflight = []             # (event, tensors) of reads that may still be running on the read-ahead stream
         if hot_ids is not None:
             self.set_hot_rows(hot_ids)
 
@@ -75,11 +76,8 @@ class PinnedFeatureStore:
         """Both tiers' launches: the device tier on the current stream, the host tier on ``cold_stream``."""
         rows, cold = _be.gather_rows_hot(self.hot_rows, self.hot_slot, ids, mask=mask, out=out, out_dtype=self.out_dtype)
         src_ids = self._host_ids(ids)
-        if cold_stream is not None:
+        if cold_stream is not None:           # (the caller keeps rows, ids and flags alive until that stream is done)
             cold_stream.wait_stream(torch.cuda.current_stream(self.device))
-            cold.record_stream(cold_stream)
-            if src_ids is not ids:
-                src_ids.record_stream(cold_stream)
         _be.gather_rows_flagged(self.buffer, src_ids, cold, rows, stream=cold_stream)
         self.last_cold = cold
         return rows, src_ids
@@ -98,12 +96,13 @@ class PinnedFeatureStore:
     def close(self):
         """Release the read-ahead stream (a CU-limited stream is a driver object that lives until it is
         destroyed; without this it goes at interpreter exit).  The store stays usable: the next ``prefetch``
-        makes a new stream.  Call it only when every tensor that ``prefetch`` has handed out is gone: torch's
-        allocator marks a freed block on the streams that used it, and a destroyed stream cannot be marked
-        (the process would crash at that free)."""
+        makes a new stream.  Reads in flight are waited for; tensors handed out earlier stay valid."""
         side, self._prefetch_side = self._prefetch_side, None
-        if side is not None and self.prefetch_cus > 0:
-            _be.release_cu_limited_stream(side)
+        if side is not None:
+            side.synchronize()
+            self._inflight.clear()
+            if self.prefetch_cus > 0:
+                _be.release_cu_limited_stream(side)
 
     def get(self, ids):
         return self.masked_get(ids, None)
@@ -152,10 +151,12 @@ class PinnedFeatureStore:
             rows = _be.gather_rows(self.buffer, src_ids, mask=mask, out=out, out_dtype=self.out_dtype, stream=side)
         done = torch.cuda.Event()
         done.record(side)
-        rows.record_stream(side)
-        src_ids.record_stream(side)
-        if mask is not None:
-            mask.record_stream(side)
+        # What the read touches stays referenced here until the read has finished, whatever becomes of the handle.
+        # (Marking the tensors as used by the side stream -- ``record_stream`` -- would do as well, but then torch's
+        # allocator touches that stream whenever one of them is freed, and a stream kept to a few compute units is
+        # destroyed by ``close()`` or at interpreter exit, possibly before the last of them.)
+        self._inflight = [entry for entry in self._inflight if not entry[0].query()]
+        self._inflight.append((done, (rows, ids, src_ids, mask, self.last_cold)))
         handle = PrefetchedRows(ids, rows, done, mask)
         handle.src_ids = src_ids
         return handle

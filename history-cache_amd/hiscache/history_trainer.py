@@ -84,6 +84,8 @@ class HistoryTrainer:
         self.scheduler = None
         self.loss_fn = torch.nn.functional.nll_loss
         # every batch comes with the transposed view of its CSR; the relational layer also reads the view's edge slots
+        if 0 < replay_slots < (3 if self.read_ahead else 2):
+            raise ValueError("replay_slots: at least as many as batches are alive at once (2, with the read-ahead 3)")
         self.sampler = ds.sampler(list(fanout), device=self.device, seed=seed, emit_view=True,
                                   view_edges=isinstance(self.model, HistoryRGCN), replay_slots=replay_slots)
         self.splits = {"train": torch.from_numpy(np.array(ds.train_idx())).to(self.device)}
@@ -99,6 +101,12 @@ class HistoryTrainer:
         self.best_metric = 0
         self.metric = None
         self.epoch_seconds = []
+
+    def close(self):
+        """Give the read-ahead stream back (it is made again on demand)."""
+        close = getattr(self.uvm, "close", None)
+        if close is not None:
+            close()
 
     # ------------------------------------------------------------------ batches
     def _batches(self, ids, shuffle, read_ahead=False):

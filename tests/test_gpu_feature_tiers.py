@@ -125,6 +125,14 @@ def test_store_reads_through_the_tiers_equal_the_plain_store(prefetch_cus):
             tiered.join(ev)
             assert torch.equal(rows_async, plain.masked_get(ids, need))
     torch.cuda.synchronize()
+    # the read-ahead stream goes while tensors that it filled are alive; they stay valid and are freed later
+    keep = rows.clone()
+    tiered.close()
+    assert torch.equal(rows, keep)
+    handle = tiered.prefetch(ids, guess)                           # (a new stream is made on demand)
+    assert torch.equal(tiered.take(handle, need), plain.masked_get(ids, need))
+    tiered.close()
+    del rows, handle, out, rows_async
     with pytest.raises(ValueError):
         PinnedFeatureStore(src.to(DEV), device=DEV, hot_ids=torch.arange(10))     # all of it is in device memory
     with pytest.raises(ValueError):

@@ -50,6 +50,7 @@ def test_trainer_trains_and_evaluates(tmp_path, recorded, placement, ring, read_
             assert any(k[2] >= 0 and v[2] for k, v in trainer._step.shapes().items()), trainer._step.shapes()
         assert trainer._step.replays >= 30, trainer._step.shapes()  # (the nineteenth batch of an epoch is shorter)
     assert not trainer.model.training                                # left in evaluation mode, as the reference leaves it
+    trainer.close()
 
 
 def test_trainer_reads_its_settings_from_the_configuration(tmp_path):
