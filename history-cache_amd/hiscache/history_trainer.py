@@ -37,7 +37,7 @@ class HistoryTrainer:
 
     def __init__(self, config, dataset=None, fanout=None, batch_size=None, lr=None, num_epochs=None, eval_begin=None,
                  features_in_device_memory=False, hot_rows=0, cache_bytes=None, ring_rows=0, recorded=False,
-                 read_ahead=False, replay_slots=0, seed=0, model_factory=None):
+                 read_ahead=False, replay_slots=4, seed=0, model_factory=None):
         """``config``: the tree ``make_config`` builds (``dl.dataset.path`` names the dataset directory).  The
         loader's settings are arguments, with the configuration's own keys as defaults where it has them
         (``dl.sampler.train.batch_size`` / ``num_neighbors``, ``train.optimizer.lr``, ``train.train.num_epochs`` /
@@ -48,7 +48,9 @@ class HistoryTrainer:
         ``RecordedIteration`` (batches of ``batch_size`` seeds; the last, shorter batch of an epoch takes the
         ordinary path).  ``read_ahead``: the feature rows of the next batch are read over the host link beside
         the current iteration (on a stream kept to 16 compute units; the epoch then runs on a stream of its
-        own), for a matrix that is not wholly in device memory.  ``model_factory(config, table)``: builds
+        own), for a matrix that is not wholly in device memory.  ``replay_slots``: the sampler's launches for a
+        batch are recorded once per slot and replayed (see ``NeighborSampler``; the trainer never holds more than
+        three batches, so four slots are safe; 0 switches it off).  ``model_factory(config, table)``: builds
         the model instead of ``get_model`` (a relational model with its own node-type ranges, say)."""
         self.config = config
         self.device = torch.device(config.dl.device)
