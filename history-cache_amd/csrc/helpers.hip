@@ -183,9 +183,13 @@ __global__ __launch_bounds__(HC_BLOCK) void lookup_kernel(const int64_t *__restr
                                                            int64_t map_len,
                                                            const int64_t *__restrict__ ids,
                                                            int64_t offset, int64_t *__restrict__ out,
-                                                           int64_t n) {
+                                                           int64_t n, const int64_t *__restrict__ n_valid_dev) {
   const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
   if (i >= n) return;
+  if (n_valid_dev != nullptr && i >= *n_valid_dev) {     // padding behind the entries in use finds nothing
+    out[i] = -1;
+    return;
+  }
   int64_t k = ids[i] + offset;
   if (k < 0) k += map_len;  // -1 addresses the last entry, as Python indexing does
   out[i] = (k >= 0 && k < map_len) ? map[k] : -1;
@@ -514,15 +518,28 @@ extern "C" int hc_fixup_rows(const void *src, int src_dtype, int64_t n_rows, con
                                static_cast<hipStream_t>(stream));
 }
 
-extern "C" int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset,
-                         int64_t *out, int64_t n, void *stream) {
+namespace {
+int lookup_launch(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset, const int64_t *n_valid_dev,
+                  int64_t *out, int64_t n, void *stream) {
   HC_REQUIRE(n >= 0 && map_len >= 0);
   if (n == 0) return HC_OK;
   HC_REQUIRE(map && ids && out);
   if (!hc_grid_ok((n + HC_BLOCK - 1) / HC_BLOCK)) return HC_EUNSUPPORTED;
   lookup_kernel<<<dim3(blocks_for(n)), dim3(HC_BLOCK), 0, static_cast<hipStream_t>(stream)>>>(
-      map, map_len, ids, offset, out, n);
+      map, map_len, ids, offset, out, n, n_valid_dev);
   return hc_launch_status();
+}
+}  // namespace
+
+extern "C" int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset,
+                         int64_t *out, int64_t n, void *stream) {
+  return lookup_launch(map, map_len, ids, offset, nullptr, out, n, stream);
+}
+
+extern "C" int hc_lookup_dev(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset,
+                             const int64_t *n_valid_dev, int64_t *out, int64_t n, void *stream) {
+  HC_REQUIRE(n_valid_dev != nullptr);
+  return lookup_launch(map, map_len, ids, offset, n_valid_dev, out, n, stream);
 }
 
 namespace {

@@ -248,15 +248,12 @@ class HistoryCache:
             return None
 
         layer1_nodes = sub_to_full[:n1]
-        self.sub2embed = _be.lookup(self.full2embed, layer1_nodes, 0)
-        self.sub2feat = _be.lookup(self.full2embed, sub_to_full, self.total_num_node)
         dev = getattr(batch, "dev", None)
-        if dev is not None:
-            # a padded batch (recorded iterations): the rows behind the real 1-hop nodes are real nodes of the next
-            # hop or padding, and count as not cached; so do the padding nodes for the feature cache
-            minus = torch.full_like(self.sub2embed[:1], -1)
-            self.sub2embed = torch.where(dev.row_index[:n1] < dev.nnl[1], self.sub2embed, minus)
-            self.sub2feat = torch.where(dev.row_index[: sub_to_full.shape[0]] < dev.nnl[-1], self.sub2feat, minus)
+        # a padded batch (recorded iterations): the rows behind the real 1-hop nodes are real nodes of the next
+        # hop or padding, and count as not cached; so do the padding nodes for the feature cache
+        self.sub2embed = _be.lookup(self.full2embed, layer1_nodes, 0, n_valid=None if dev is None else dev.nnl[1])
+        self.sub2feat = _be.lookup(self.full2embed, sub_to_full, self.total_num_node,
+                                   n_valid=None if dev is None else dev.nnl[-1])
         self.used_masks = _be.count_history_reconstruct(batch.ptr, batch.idx, self.sub2embed,
                                                         sub_to_full.shape[0], batch.y.shape[0],
                                                         num_layer)

@@ -95,6 +95,7 @@ _SIGNATURES = {
     "hc_gather_rows_flagged": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_fixup_rows": (_c_int, [_c_p, _c_int, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_i64, _c_p]),
     "hc_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p]),
+    "hc_lookup_dev": (_c_int, [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p]),
     "hc_ring_lookup": (_c_int, [_c_p, _c_i64, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_int, _c_i64, _c_i64, _c_p, _c_p,
                                 _c_i64, _c_p]),
     "hc_check_csr": (_c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_p]),
@@ -1087,12 +1088,19 @@ def fixup_rows(src, ids, need, have, out):
     return out
 
 
-def lookup(map_tensor, ids, offset=0):
-    """out[i] = map[ids[i] + offset] (int64 gather; negative positions index from the end)."""
+def lookup(map_tensor, ids, offset=0, n_valid=None):
+    """out[i] = map[ids[i] + offset] (int64 gather; negative positions index from the end).  ``n_valid`` (a
+    one-element int64 device tensor, for recorded iterations): entries at or behind it are padding and give -1."""
     lib = load_library()
     _dev(map_tensor, "map", torch.int64)
     _dev(ids, "ids", torch.int64)
     out = torch.empty(ids.numel(), dtype=torch.int64, device=ids.device)
+    if n_valid is not None:
+        _dev(n_valid, "n_valid", torch.int64)
+        rc = lib.hc_lookup_dev(_ptr(map_tensor), map_tensor.numel(), _ptr(ids), int(offset), _ptr(n_valid), _ptr(out),
+                               ids.numel(), _stream())
+        _check(rc, "hc_lookup_dev")
+        return out
     rc = lib.hc_lookup(_ptr(map_tensor), map_tensor.numel(), _ptr(ids), int(offset), _ptr(out), ids.numel(),
                        _stream())
     _check(rc, "hc_lookup")

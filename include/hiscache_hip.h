@@ -546,6 +546,11 @@ int hc_gather_rows_flagged(const void *src, int src_dtype, int64_t n_rows, const
  * of lookup_and_load, hiscache/history_cache.py:310,315). */
 int hc_lookup(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset, int64_t *out,
               int64_t n, void *stream);
+/* hc_lookup_dev: hc_lookup for a batch padded to a fixed size (recorded
+ * iterations): entries at or behind *n_valid_dev (one int64 in device memory)
+ * are padding and come out as -1. */
+int hc_lookup_dev(const int64_t *map, int64_t map_len, const int64_t *ids, int64_t offset,
+                  const int64_t *n_valid_dev, int64_t *out, int64_t n, void *stream);
 
 /* hc_load_mask: the rows of a batch that have to be read from the feature store,
  * and the cache's hit counters, in one launch.  The reference spells the mask as
