@@ -100,6 +100,20 @@ def test_quantile_with_the_count_on_the_device(n_max):
     assert torch.equal(be.quantile_select_dev(score, one(0), 0.5), quantile_threshold(score[:1], 0.5))
 
 
+def test_map_lookup_with_the_count_on_the_device():
+    import hiscache_backend as be
+    rng = np.random.default_rng(4)
+    table = T(rng.integers(-1, 1000, size=5000))
+    ids = T(np.concatenate([rng.integers(0, 2500, size=700), np.full(300, -1)]))       # padding ids are -1
+    for n_valid in (0, 1, 699, 700, 1000):
+        got = be.lookup(table, ids, 2500, n_valid=one(n_valid))
+        want = be.lookup(table, ids, 2500)
+        want[n_valid:] = -1
+        assert torch.equal(got, want)
+    with pytest.raises(ValueError):
+        be.lookup(table, ids, 0, n_valid=torch.tensor([5], dtype=torch.int32, device=DEV))
+
+
 def test_ring_lookup_and_admission_with_scalars_on_the_device(orc):
     """hc_ring_lookup_dev / hc_grad_check_dev against the by-value entry points on the same state."""
     import hiscache_backend as be
