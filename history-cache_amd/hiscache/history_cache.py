@@ -231,8 +231,8 @@ class HistoryCache:
             self.sub2feat = _be.lookup(self.full2embed, sub_to_full, self.total_num_node)
             hit = self.sub2feat != -1
             x = self.uvm.masked_get(sub_to_full, ~hit)
-            _be.gather_rows(self.buffer.view(-1, self.in_channels), self.sub2feat, mask=hit, out=x,
-                            accumulate=True)
+            # the feature cache's rows go where the store left zeros (the reference adds them on top, :285-287)
+            _be.gather_rows_flagged(self.buffer.view(-1, self.in_channels), self.sub2feat, hit, x)
             batch.x = x
             self.used_masks = None          # nothing is pruned in evaluation: no masks of an earlier batch linger
             return None
@@ -290,8 +290,9 @@ class HistoryCache:
         # are ignored by the aggregation
         self.cached_embedding = _be.gather_rows(self.buffer.view(-1, self.hidden_channels),
                                                 self.sub2embed)
-        _be.gather_rows(self.buffer.view(-1, self.in_channels), self.sub2feat, mask=hit_feat_mask,
-                        out=x, accumulate=True)
+        # the feature cache's rows go where the read left zeros (the reference adds them on top, :347-349): only
+        # the hit rows are touched
+        _be.gather_rows_flagged(self.buffer.view(-1, self.in_channels), self.sub2feat, hit_feat_mask, x)
         batch.x = x
         self.load_mask = load_mask
         return None
