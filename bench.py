@@ -81,7 +81,7 @@ def parse():
     ap.add_argument("--no-batch-view", action="store_true",
                     help="c3/c5: batches come without the transposed view of their CSR, so every layer's "
                          "backward builds one (the default: the loader emits it with the batch)")
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c2row", "c2w", "c4", "c3", "c3b", "c5", "sample", "layer", "copy"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c2row", "c2w", "c4", "c3", "c3b", "c5", "sample", "layer", "copy", "trainer"])
     ap.add_argument("--heads", type=int, default=1, help="c2w: heads of the weighted aggregation (divides 256)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--reps", type=int, default=8, help="c3b: measurements with freshly allocated tensors")
@@ -1281,6 +1281,56 @@ def device_power_law_graph(N, mean_degree, dev, gen, max_degree=100_000):
     return indptr, indices
 
 
+def run_trainer(args):
+    """Epochs of ``hiscache.HistoryTrainer`` over a dataset directory of the plumbing configuration's shape
+    (100 k nodes, degree 15, 128-dim fp32 features, 2-layer SAGE hidden 128, fanout [10, 5], batches of 1000 seeds,
+    the reference's flat ``HistoryCache`` with a 15 MB buffer): ms per iteration of the epochs behind the first.
+    --recorded, --prefetch (the read-ahead), --hot-fraction, --features-in-hbm and --sampler-replay choose the loop."""
+    import tempfile
+
+    import numpy as np
+    import torch
+
+    from hiscache import HistoryTrainer, make_config, write_processed
+
+    rng = np.random.default_rng(1)
+    N, Fin, H, C, L, deg, n_train, batch = 100_000, 128, 128, 10, 2, 15, 60_000, 1000
+    indptr = np.arange(0, (N + 1) * deg, deg, dtype=np.int64)
+    indices = rng.integers(0, N, size=N * deg).astype(np.int64)
+    feats = rng.standard_normal((N, Fin)).astype(np.float32)
+    labels = feats[:, :C].argmax(1).astype(np.int64)              # a node's own features decide its label
+    perm = rng.permutation(N)
+    epochs = max(2, min(args.steps, 6))
+    with tempfile.TemporaryDirectory() as root:
+        write_processed(root, indptr, indices, feats, hot_ids=np.argsort(np.bincount(indices, minlength=N), kind="stable"),
+                        labels=labels, train_idx=perm[:n_train], valid_idx=perm[n_train:n_train + 10_000])
+        cfg = make_config(Fin, C, H, L, method="grad", rate=0.5, staleness_thres=200, device="cuda:0", path=root)
+        trainer = HistoryTrainer(cfg, fanout=[10, 5], batch_size=batch, lr=1e-3, num_epochs=epochs, eval_begin=epochs - 1,
+                                 cache_bytes=30_000 * Fin * 4, recorded=args.recorded, read_ahead=args.prefetch,
+                                 hot_rows=int(N * args.hot_fraction), features_in_device_memory=args.features_in_hbm,
+                                 replay_slots=max(args.sampler_replay, 4) if args.sampler_replay else 0)
+        trainer.train()
+        iters = n_train // batch
+        per_epoch = [1e3 * s / iters for s in trainer.epoch_seconds]
+        ms = float(np.mean(per_epoch[1:]))
+        rec = trainer._step
+        res = {
+            "metric": "trainer iteration ms (1 GPU)", "value": ms, "unit": "ms", "n_gpus": 1, "steps": iters * (epochs - 1),
+            "warmup": iters, "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "HistoryTrainer on a dataset directory: %d nodes, degree %d, %d-dim fp32 features, "
+                                   "2-layer SAGE hidden %d, fanout [10,5], %d batches of %d seeds per epoch, flat "
+                                   "HistoryCache of %d rows" % (N, deg, Fin, H, iters, batch, 30_000)},
+            "ms_per_iteration_by_epoch": per_epoch, "val_metric": trainer.val_metrics,
+            "loop": {"recorded": bool(args.recorded), "read_ahead": bool(trainer.read_ahead),
+                     "hot_rows": int(N * args.hot_fraction), "features_in_device_memory": bool(args.features_in_hbm),
+                     "sampler_replay_slots": trainer.sampler.replay_slots},
+            "recorded": None if rec is None else {"replays": rec.replays, "unrecorded": rec.unrecorded},
+        }
+        trainer.close()
+    return res
+
+
 def run_sample(args):
     """Layered neighbour sampling on a papers100M-sized graph resident in HBM: time per batch when
     the caller waits for it, and what is left on the training thread when the next batch is
@@ -1482,6 +1532,8 @@ def main():
         res = run_c1(args)
     elif args.workload == "sample":
         res = run_sample(args)
+    elif args.workload == "trainer":
+        res = run_trainer(args)
     else:
         res = run_c3(args)
     print(json.dumps(res))
