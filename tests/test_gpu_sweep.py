@@ -304,3 +304,61 @@ def test_sweep_cache_policy_and_sampler(orc):
             case(orc, rng)
         except AssertionError as e:
             raise AssertionError("%s %d (seed %d): %s" % (case.__name__, i, s, str(e)[:600])) from None
+
+
+# ------------------------------------------------------------------------------ row gathers
+def row_gather_case(be, s):
+    """Masked row gathers of a matrix in device memory, in pinned host memory and in two tiers, and the fix-up of a
+    guessed gather, against NumPy indexing: the values are copies (or conversions of one element), so every bit
+    must agree."""
+    rng = np.random.default_rng(s)
+    F = int(rng.choice(WIDTHS[:31]))
+    src_dt, out_dt = [("f32", "f32"), ("f32", "f32"), ("f16", "f16"), ("f16", "f32"), ("bf16", "f32"),
+                      ("f32", "f16")][int(rng.integers(6))]
+    N = int(rng.choice([1, 2, 50, 777, 4000]))
+    n = int(rng.choice([1, 15, 16, 17, 63, 64, 65, 255, 256, 257, 1000, 3000]))
+    n = max(1, min(n, int(3e6 // F)))
+    src = torch.from_numpy(rng.standard_normal((N, F)).astype(np.float32)).to(TORCH_DT[src_dt])
+    host = torch.empty(src.shape, dtype=src.dtype, pin_memory=True)
+    host.copy_(src)
+    dev = src.to(DEV)
+    ids_np = rng.integers(-N, N, size=n)                             # negative ids address from the end
+    if n > 4:
+        ids_np[int(rng.integers(n))] = N + int(rng.integers(3))      # outside the matrix: a cleared row
+        ids_np[int(rng.integers(n))] = -N - 1 - int(rng.integers(3))
+    masked = rng.random() < 0.7
+    mask_np = rng.random(n) < rng.choice([0.0, 0.3, 0.9, 1.0]) if masked else np.ones(n, bool)
+    ids, mask = T(ids_np), (T(mask_np) if masked else None)
+    wrapped = np.where(ids_np < 0, ids_np + N, ids_np)
+    inside = (wrapped >= 0) & (wrapped < N)
+    take = inside & mask_np
+    want = src[torch.from_numpy(np.where(inside, wrapped, 0))].to(TORCH_DT[out_dt])
+    want[torch.from_numpy(~take)] = 0
+    for matrix in (dev, host):
+        got = be.gather_rows(matrix, ids, mask=mask, out_dtype=TORCH_DT[out_dt])
+        assert torch.equal(got.cpu(), want), ("gather", matrix.is_cuda)
+    # two tiers
+    k = int(N * rng.choice([0.0, 0.4, 1.0]))
+    hot_ids = T(rng.permutation(N)[:k].copy())
+    slot = torch.full((N,), -1, dtype=torch.int32, device=DEV)
+    slot[hot_ids] = torch.arange(k, dtype=torch.int32, device=DEV)
+    hot = dev[hot_ids].contiguous() if k else torch.empty((0, F), dtype=dev.dtype, device=DEV)
+    out = torch.full((n, F), 5.0, dtype=TORCH_DT[out_dt], device=DEV)
+    _, cold = be.gather_rows_hot(hot, slot, ids, mask=mask, out=out)
+    slot_np = slot.cpu().numpy()
+    eq(cold.cpu().numpy().astype(bool), take & (slot_np[np.where(inside, wrapped, 0)] < 0))
+    be.gather_rows_flagged(host, ids, cold, out)
+    assert torch.equal(out.cpu(), want), "tiers"
+    # a gather under a guess, brought to the exact mask
+    guess_np = rng.random(n) < 0.5
+    rows = be.gather_rows(host, ids, mask=T(guess_np), out_dtype=TORCH_DT[out_dt])
+    be.fixup_rows(host, ids, T(mask_np), T(guess_np), rows)
+    assert torch.equal(rows.cpu(), want), "fixup"
+
+
+def test_sweep_row_gathers(be):
+    for s in case_seeds(44, 400):
+        try:
+            row_gather_case(be, s)
+        except Exception as e:                     # name the case: its seed rebuilds the inputs
+            raise AssertionError(f"row gather case seed {s}: {e}") from e
