@@ -81,7 +81,7 @@ def parse():
     ap.add_argument("--no-batch-view", action="store_true",
                     help="c3/c5: batches come without the transposed view of their CSR, so every layer's "
                          "backward builds one (the default: the loader emits it with the batch)")
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c2row", "c2w", "c4", "c3", "c3b", "c5", "sample", "layer", "copy", "trainer"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c2row", "c2w", "c4", "c3", "c3b", "c5", "sample", "layer", "copy", "trainer", "dispatch"])
     ap.add_argument("--heads", type=int, default=1, help="c2w: heads of the weighted aggregation (divides 256)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--reps", type=int, default=8, help="c3b: measurements with freshly allocated tensors")
@@ -1281,6 +1281,78 @@ def device_power_law_graph(N, mean_degree, dev, gen, max_degree=100_000):
     return indptr, indices
 
 
+def run_dispatch(args):
+    """What a zero-copy host read costs the kernels that run beside it: a HIP graph of 60 one-element kernels
+    (nothing but their dispatch) replayed alone, beside a gather of 90 000 rows from pinned host memory on a stream
+    kept to 16 compute units, and beside the same gather from device memory on the same stream."""
+    import torch
+
+    import hiscache_backend as be
+
+    dev = "cuda:0"
+    N, F, n_rows, n_kernels = 4_000_000, 128, 90_000, 60
+    x = torch.zeros(1, device=dev)
+    capture = torch.cuda.Stream()
+    with torch.cuda.stream(capture):
+        for _ in range(3):
+            x.add_(1.0)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=capture):
+        for _ in range(n_kernels):
+            x.add_(1.0)
+    host = torch.empty((N, F), dtype=torch.float32, pin_memory=True)
+    host.normal_()
+    hbm = torch.randn((N, F), device=dev)
+    side = be.cu_limited_stream(args.prefetch_cus, torch.device(dev))
+    compute = torch.cuda.Stream()
+    gen = torch.Generator(device=dev).manual_seed(1)
+
+    def replay_us(beside):
+        ids = torch.randint(0, N, (n_rows,), device=dev, generator=gen)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        rows = None
+        if beside is not None:
+            side.wait_stream(torch.cuda.current_stream())
+            rows = be.gather_rows(beside, ids, stream=side)
+        with torch.cuda.stream(compute):
+            e0.record()
+            for _ in range(3):
+                graph.replay()
+            e1.record()
+        torch.cuda.synchronize()
+        del rows
+        return e0.elapsed_time(e1) / 3 * 1e3
+
+    def gather_us(matrix):
+        ids = torch.randint(0, N, (n_rows,), device=dev, generator=gen)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(side)
+        rows = be.gather_rows(matrix, ids, stream=side)
+        e1.record(side)
+        torch.cuda.synchronize()
+        del rows
+        return e0.elapsed_time(e1) * 1e3
+
+    reps = max(3, args.steps)
+    alone = min(replay_us(None) for _ in range(reps))
+    beside_host = min(replay_us(host) for _ in range(reps))
+    beside_hbm = min(replay_us(hbm) for _ in range(reps))
+    return {
+        "metric": "us per replay of a 60-kernel graph", "value": alone, "unit": "us", "n_gpus": 1, "steps": reps,
+        "warmup": 0, "ms_per_step": alone * 1e-3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "dispatch: %d one-element kernels in a HIP graph; beside them a gather of %d rows x %d "
+                               "fp32 on a stream kept to %d compute units" % (n_kernels, n_rows, F, args.prefetch_cus)},
+        "replay_us": {"alone": alone, "beside_host_gather": beside_host, "beside_device_memory_gather": beside_hbm},
+        "us_per_kernel": {"alone": alone / n_kernels, "beside_host_gather": beside_host / n_kernels,
+                          "beside_device_memory_gather": beside_hbm / n_kernels},
+        "gather_us": {"host": gather_us(host), "device_memory": gather_us(hbm)},
+    }
+
+
 def run_trainer(args):
     """Epochs of ``hiscache.HistoryTrainer`` over a dataset directory of the plumbing configuration's shape
     (100 k nodes, degree 15, 128-dim fp32 features, 2-layer SAGE hidden 128, fanout [10, 5], batches of 1000 seeds,
@@ -1534,6 +1606,8 @@ def main():
         res = run_sample(args)
     elif args.workload == "trainer":
         res = run_trainer(args)
+    elif args.workload == "dispatch":
+        res = run_dispatch(args)
     else:
         res = run_c3(args)
     print(json.dumps(res))
