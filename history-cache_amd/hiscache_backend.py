@@ -1010,13 +1010,17 @@ def release_cu_limited_stream(stream):
 def cu_limited_stream(n_cus, device):
     """A torch stream (default priority) whose kernels run on ``n_cus`` compute units only, spread over the
     chip: for work that waits on the host link beside compute (``PinnedFeatureStore.prefetch``).  The
-    stream lives until the interpreter exits."""
+    stream lives until the interpreter exits.  (The runtime has refused masks of 2 and of 4 units on an MI355X;
+    8 -- one per die -- and more work.)"""
     lib = load_library()
     device = torch.device(device)
     handle = ctypes.c_void_p()
     with torch.cuda.device(device):
-        _check(lib.hc_stream_create_cu_limited(int(n_cus), ctypes.cast(ctypes.pointer(handle), _c_p)),
-               "hc_stream_create_cu_limited")
+        rc = lib.hc_stream_create_cu_limited(int(n_cus), ctypes.cast(ctypes.pointer(handle), _c_p))
+        if rc == 3:                                  # HC_ELAUNCH: the runtime said no
+            raise RuntimeError(f"the runtime refused a stream kept to {int(n_cus)} compute units (masks of fewer than 8 "
+                               "units, one per die, have been refused on this GPU)")
+        _check(rc, "hc_stream_create_cu_limited")
     if not _cu_stream_handles:
         import atexit
         atexit.register(_destroy_cu_streams)
