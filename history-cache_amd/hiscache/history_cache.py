@@ -15,7 +15,8 @@ Differences that a caller can see:
   * rows that would be appended beyond the buffer are dropped and counted in ``overflow``
     (the reference raises a shape error there, history_cache.py:219-221);
   * ``num_layer`` of ``lookup_and_load`` may be omitted (taken from the config);
-  * a ``feature_cache_only`` lookup clears ``used_masks`` (the reference leaves the last training batch's masks
+  * a ``feature_cache_only`` lookup works in the modes without a cache too (all rows from the store), and
+    clears ``used_masks`` (the reference leaves the last training batch's masks
     in place, which its relational model then applies to the evaluation batch).
 """
 import math
@@ -227,6 +228,12 @@ class HistoryCache:
         if num_layer is None:
             num_layer = self.num_layers_all
         sub_to_full = batch.sub_to_full
+        if feature_cache_only and "history" not in self.feat_mode:
+            # no cache was allocated in this mode: every row comes from the store (the reference reads its
+            # missing buffer here, /root/reference/hiscache/history_cache.py:276-288)
+            batch.x = self.uvm.get(sub_to_full)
+            self.used_masks = None
+            return None
         if feature_cache_only:
             self.sub2feat = _be.lookup(self.full2embed, sub_to_full, self.total_num_node)
             hit = self.sub2feat != -1

@@ -199,7 +199,9 @@ class MySageConvHistory(torch.nn.Module):
         that follows (see ``bn_relu``).  ``view``: the batch's shared transposed view
         (``hiscache_backend.BatchView``), when the loader emitted one."""
         num_node = int(num_node)
-        use_hist = history_size > 0 and history_map is not None and history_map.numel() > 0
+        # (no rows to substitute from: the no-cache mode hands over a map of -1 and an empty buffer)
+        use_hist = (history_size > 0 and history_map is not None and history_map.numel() > 0
+                    and history_buffer is not None and history_buffer.numel() > 0)
         if self.fused and x.is_cuda and not (use_hist and history_buffer.requires_grad):
             sink = None
             if self.need_grad and self.training and history_size > 0:
@@ -465,7 +467,9 @@ class MyRGCNConvHistory2(torch.nn.Module):
         K = self.num_rel
         edge_types = edge_types.to(torch.int64).contiguous()
         self._count_of = edge_types
-        use_hist = history_size > 0 and history_map is not None and history_map.numel() > 0
+        # (no rows to substitute from: the no-cache mode hands over a map of -1 and an empty buffer)
+        use_hist = (history_size > 0 and history_map is not None and history_map.numel() > 0
+                    and history_buffer is not None and history_buffer.numel() > 0)
         if self.fused and x.is_cuda and not (use_hist and history_buffer.requires_grad):
             # the gradient that reaches the layer's output is handed to ``his.grad`` by the node's backward
             sink = _GradSink() if (self.need_grad and self.training and history_size > 0) else None

@@ -55,6 +55,10 @@ class HistoryTrainer:
         self.config = config
         self.device = torch.device(config.dl.device)
         self.feat_mode = config.dl.loading.feat_mode
+        self.recorded = bool(recorded)
+        if self.recorded and (config.history.method != "grad" or "history" not in self.feat_mode):
+            raise ValueError("recorded iterations need the embedding cache with admission by gradient "
+                             "(history.method = 'grad', a history_* feat_mode)")
         self.num_layers = int(config.train.model.num_layers)
         self.batch_size = int(batch_size or _option(config, "dl.sampler.train.batch_size", 1000))
         fanout = fanout or _option(config, "dl.sampler.train.num_neighbors", None)
@@ -79,7 +83,6 @@ class HistoryTrainer:
         else:
             self.table = HistoryCache(uvm=self.uvm, config=config, mode=self.feat_mode, buffer_bytes=cache_bytes)
         self.model = (model_factory or get_model)(config, self.table).to(self.device)
-        self.recorded = bool(recorded)
         self.optimizer = torch.optim.Adam(self.model.parameters(),
                                           lr=float(lr or _option(config, "train.optimizer.lr", 1e-3)), fused=True,
                                           capturable=self.recorded)
@@ -191,6 +194,9 @@ class HistoryTrainer:
             y_preds.append(out.detach())
             y_trues.append(batch.y.detach().clone())
         torch.cuda.synchronize(self.device)
+        if not y_preds:
+            log.info(f"{split}: no nodes")
+            return
         self.metric = self.evaluator(torch.cat(y_preds, dim=0), torch.cat(y_trues, dim=0)).item()
         log.info(f"epoch time: {time.time() - tepoch}")
         log.info(f"{split}-metric: {self.metric}")

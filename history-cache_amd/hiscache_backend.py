@@ -558,7 +558,9 @@ class _AggrHistory(torch.autograd.Function):
 
 
 def _norm_history(history_map, history_buffer, history_size):
-    if history_size == 0 or _empty(history_map):
+    # an empty buffer: no row can be substituted (the reference's no-cache mode hands over a map of -1 and an
+    # empty tensor, /root/reference/hiscache/history_cache.py:291-294, and its kernel then reads no history row)
+    if history_size == 0 or _empty(history_map) or _empty(history_buffer):
         return None, None, 0
     return history_map, history_buffer, int(history_size)
 

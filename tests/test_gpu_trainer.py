@@ -9,6 +9,7 @@ DEV = "cuda:0"
 
 
 def dataset(tmp_path, rng, N=6000, Fin=32, C=4):
+    """62% of the nodes train, 18% validate, 20% test."""
     from hiscache import write_processed
     deg = 10
     indptr = np.arange(0, (N + 1) * deg, deg, dtype=np.int64)
@@ -17,7 +18,7 @@ def dataset(tmp_path, rng, N=6000, Fin=32, C=4):
     labels = feats[:, :C].argmax(1).astype(np.int64)              # a node's own features decide its label
     perm = rng.permutation(N)
     write_processed(tmp_path, indptr, indices, feats, hot_ids=rng.permutation(N), labels=labels,
-                    train_idx=perm[:3700], valid_idx=perm[3700:4800], test_idx=perm[4800:])
+                    train_idx=perm[: N * 37 // 60], valid_idx=perm[N * 37 // 60: N * 4 // 5], test_idx=perm[N * 4 // 5:])
     return feats, labels
 
 
@@ -66,6 +67,9 @@ def test_trainer_reads_its_settings_from_the_configuration(tmp_path):
     assert trainer.optimizer.param_groups[0]["lr"] == 0.003
     trainer.train()
     assert trainer.val_metrics == [] and len(trainer.epoch_seconds) == 2     # evaluation begins at epoch 5
+    with pytest.raises(ValueError):          # a recording needs admission by gradient
+        HistoryTrainer(make_config(32, 4, 32, 2, method="random", device=DEV, path=str(tmp_path)), fanout=[3, 2],
+                       cache_bytes=400 * 32 * 4, recorded=True)
     with pytest.raises(ValueError):
         HistoryTrainer(make_config(32, 4, 32, 2, device=DEV, path=str(tmp_path)), fanout=[3], cache_bytes=400 * 32 * 4)
 
@@ -96,3 +100,17 @@ def test_trainer_with_a_relational_model(tmp_path, recorded):
     assert all(torch.isfinite(p).all() for p in trainer.model.parameters())
     if recorded:
         assert trainer._step.replays >= 30, trainer._step.shapes()
+
+
+def test_trainer_without_the_embedding_cache(tmp_path):
+    """``feat_mode = "uvm"``: features through the store, no embedding is cached or admitted
+    (/root/reference/hiscache/history_cache.py:290-304)."""
+    from hiscache import HistoryTrainer, make_config
+    rng = np.random.default_rng(80)
+    dataset(tmp_path, rng)
+    cfg = make_config(32, 4, 32, 3, device=DEV, path=str(tmp_path), feat_mode="uvm")
+    torch.manual_seed(3)
+    trainer = HistoryTrainer(cfg, fanout=[4, 3, 2], batch_size=200, lr=1e-2, num_epochs=3, eval_begin=2,
+                             cache_bytes=400 * 32 * 4)
+    trainer.train()
+    assert trainer.table.header == 0 and len(trainer.val_metrics) == 1 and trainer.val_metrics[0] > 0.4
