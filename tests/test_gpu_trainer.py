@@ -114,3 +114,18 @@ def test_trainer_without_the_embedding_cache(tmp_path):
                              cache_bytes=400 * 32 * 4)
     trainer.train()
     assert trainer.table.header == 0 and len(trainer.val_metrics) == 1 and trainer.val_metrics[0] > 0.4
+
+
+@pytest.mark.parametrize("method", ["random", "staleness"])
+def test_trainer_with_the_other_admission_policies(tmp_path, method):
+    """``history.method`` other than "grad": scores are drawn at random, no gradient of the embeddings is kept
+    (/root/reference/hiscache/history_cache.py:205-215)."""
+    from hiscache import HistoryTrainer, make_config
+    rng = np.random.default_rng(81)
+    dataset(tmp_path, rng)
+    cfg = make_config(32, 4, 32, 3, method=method, rate=0.5, staleness_thres=7, device=DEV, path=str(tmp_path))
+    torch.manual_seed(4)
+    trainer = HistoryTrainer(cfg, fanout=[4, 3, 2], batch_size=200, lr=1e-2, num_epochs=3, eval_begin=2,
+                             cache_bytes=1500 * 32 * 4)
+    trainer.train()
+    assert trainer.table.header > 0 and trainer.val_metrics[0] > 0.4
