@@ -3,6 +3,7 @@ argument checks return status codes (no kernel is launched here)."""
 import ctypes
 import os
 import re
+import types
 
 import numpy as np
 import pytest
@@ -323,3 +324,57 @@ def test_recorded_iteration_shape_family():
     rec2 = RecordedIteration(None, SimpleNamespace(device=torch.device("cpu")), None, 2, round_to=64)
     caps, e_cap = rec2._shape(rec2._key_for([500, 500, 500], 0))
     assert caps[0] == 500 and caps == sorted(caps) and all(c >= 500 for c in caps) and e_cap >= 0
+
+
+def test_trainer_hands_out_every_batch_once_and_reads_one_batch_ahead():
+    """The trainer's batch pipeline with stand-ins for the sampler and the recorded step (no GPU): every chunk of the
+    split becomes one batch, in order; a batch is sampled while the one before is in use; with the read-ahead the
+    feature read of batch k + 1 is started before batch k is handed out, and never for a batch twice."""
+    import torch
+    from hiscache.history_trainer import HistoryTrainer, _option
+    from hiscache import make_config
+
+    events = []
+
+    class Pending:
+        def __init__(self, seeds):
+            self.seeds = seeds
+
+        def get(self):
+            events.append(("got", int(self.seeds[0])))
+            return types.SimpleNamespace(seeds=self.seeds)
+
+    class Sampler:
+        def sample_async(self, seeds):
+            events.append(("sampling", int(seeds[0])))
+            return Pending(seeds)
+
+    class Step:
+        def prefetch(self, batch):
+            events.append(("read", int(batch.seeds[0])))
+
+    for n_ids, batch_size in ((10, 4), (4, 4), (1, 4), (0, 4), (23, 5)):
+        for read_ahead in (False, True):
+            t = object.__new__(HistoryTrainer)
+            t.device, t.batch_size, t.sampler, t._step, t.num_layers = torch.device("cpu"), batch_size, Sampler(), Step(), 2
+            events.clear()
+            ids = torch.arange(n_ids) * 10
+            firsts = []
+            for batch in t._batches(ids, shuffle=False, read_ahead=read_ahead):
+                events.append(("train", int(batch.seeds[0])))
+                firsts.append(int(batch.seeds[0]))
+            want = [int(ids[lo]) for lo in range(0, n_ids, batch_size)]
+            assert firsts == want
+            assert [e[1] for e in events if e[0] == "sampling"] == want          # every chunk sampled once, in order
+            for k, first in enumerate(want):
+                at = events.index(("train", first))
+                if k + 1 < len(want):                                            # the next batch is under way by then
+                    assert events.index(("sampling", want[k + 1])) < at
+                    if read_ahead:
+                        assert events.index(("read", want[k + 1])) < at
+            reads = [e[1] for e in events if e[0] == "read"]
+            assert reads == (want[1:] if read_ahead else [])
+
+    cfg = make_config(8, 2, 8, 2)
+    assert _option(cfg, "train.model.num_layers", 7) == 2
+    assert _option(cfg, "train.train.num_epochs", 7) == 7 and _option(cfg, "dl.sampler.train.batch_size", None) is None
