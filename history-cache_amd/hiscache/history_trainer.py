@@ -71,8 +71,11 @@ class HistoryTrainer:
         # the feature store (cxgnndl.UVM's role): pinned host memory read zero-copy, the hottest rows or the whole
         # matrix in device memory on request
         self.read_ahead = bool(read_ahead) and not features_in_device_memory
+        # (a matrix stored in fp16 -- the reference loads mag240M's that way, history_cache.py:148-149 -- stays fp16
+        # on its way into the first layer: half the bytes over the link)
         self.uvm = ds.feature_store(device=self.device, in_device_memory=features_in_device_memory,
-                                    hot_rows=hot_rows, prefetch_cus=16 if self.read_ahead else 0)
+                                    hot_rows=hot_rows, prefetch_cus=16 if self.read_ahead else 0,
+                                    out_dtype=torch.float16 if ds.feature_dtype == np.float16 else None)
         self._compute = torch.cuda.Stream(device=self.device) if self.read_ahead else None   # default priority
         if ring_rows:
             self.table = RingHistoryCache(self.uvm, ds.num_nodes, config.dl.dataset.feature_dim,

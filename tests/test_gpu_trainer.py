@@ -129,3 +129,26 @@ def test_trainer_with_the_other_admission_policies(tmp_path, method):
                              cache_bytes=1500 * 32 * 4)
     trainer.train()
     assert trainer.table.header > 0 and trainer.val_metrics[0] > 0.4
+
+
+@pytest.mark.parametrize("recorded", [False, True])
+def test_trainer_keeps_half_precision_features_in_half_precision(tmp_path, recorded):
+    from hiscache import HistoryTrainer, ProcessedDataset, make_config, write_processed
+    rng = np.random.default_rng(82)
+    N, Fin, C = 6000, 32, 4
+    indptr = np.arange(0, (N + 1) * 10, 10, dtype=np.int64)
+    indices = rng.integers(0, N, size=N * 10).astype(np.int64)
+    feats = rng.standard_normal((N, Fin)).astype(np.float16)
+    perm = rng.permutation(N)
+    write_processed(tmp_path, indptr, indices, feats, hot_ids=rng.permutation(N),
+                    labels=feats[:, :C].argmax(1).astype(np.int64), train_idx=perm[:3600], valid_idx=perm[3600:4800])
+    cfg = make_config(Fin, C, 32, 3, method="grad", rate=0.5, staleness_thres=7, device=DEV, path=str(tmp_path))
+    torch.manual_seed(5)
+    trainer = HistoryTrainer(cfg, dataset=ProcessedDataset(tmp_path, Fin, feature_dtype=np.float16), fanout=[4, 3, 2],
+                             batch_size=200, lr=1e-2, num_epochs=3, eval_begin=2, cache_bytes=1500 * 32 * 4,
+                             hot_rows=1000, read_ahead=True, recorded=recorded)
+    assert trainer.uvm.buffer.dtype == torch.float16 and trainer.uvm.out_dtype == torch.float16
+    assert trainer.uvm.hot_rows.dtype == torch.float16
+    trainer.train()
+    assert trainer.val_metrics[0] > 0.5 and trainer.table.header > 0
+    trainer.close()
