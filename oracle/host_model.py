@@ -83,6 +83,20 @@ def lookup_and_load(st, batch, num_layer, features):
                            used_masks=used_masks, load_mask=load_mask, x=x)
 
 
+def lookup_feature_cache_only(st, sub_to_full, features):
+    """history_cache.py:276-288, the evaluation lookup: feature-cache hits from the buffer's tail, every other
+    row from the host matrix.  Pinned by the reference's own run (history_cache_fill_golden.npz).
+    Returns (sub2feat, x)."""
+    sub2feat = st.full2embed[sub_to_full + st.N]
+    load_mask = sub2feat == -1
+    x = torch.zeros((sub_to_full.shape[0], st.Fin), dtype=torch.float32)
+    x[load_mask] = features[sub_to_full[load_mask]].to(torch.float32)
+    cached_feat = st.buffer.view(-1, st.Fin)[sub2feat]
+    cached_feat[load_mask] = 0
+    x += cached_feat
+    return sub2feat, x
+
+
 def update_history(st, sub_to_full, sub2embed, produced_embedding, score, rate, staleness_thres,
                    glb_iter):
     """history_cache.py:188-254 with the score given (the caller computes the row norms with the

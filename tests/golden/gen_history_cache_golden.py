@@ -244,6 +244,11 @@ def fill_inputs(c):
     return feats, hot
 
 
+def eval_ids(c):
+    """Node ids of a fill case's evaluation lookup, rebuilt from its seed (repeated ids included)."""
+    return np.random.default_rng(c["seed"] + 100).integers(0, c["N"], size=min(c["N"], 700)).astype(np.int64)
+
+
 def main_fill():
     import tempfile
     sys.path.insert(0, os.path.join(ROOT, "history-cache_amd"))
@@ -275,8 +280,16 @@ def main_fill():
             out[pre + "embed2full"] = cache.embed2full.numpy().copy()
             out[pre + "feature_rows"] = cache.buffer.view(-1, c["Fin"])[-n_cached:].numpy().copy()
             out[pre + "header"] = np.int64(cache.header)
+            # the evaluation lookup (history_cache.py:276-288) on the cache as fill() left it: nodes with and
+            # without a cached feature row, the store stand-in serving the others
+            ids = eval_ids(c)
+            batch = types.SimpleNamespace(sub_to_full=torch.from_numpy(ids), x=None)
+            cache.lookup_and_load(batch, 2, feature_cache_only=True)
+            out[pre + "eval_sub2feat"] = cache.sub2feat.numpy().copy()
+            out[pre + "eval_x"] = batch.x.numpy().copy()
             print(name, "buffer floats", cache.buffer.shape[0], "feature slots", cache.overall_feat_num,
-                  "cached", n_cached)
+                  "cached", n_cached, "evaluation lookup: rows from the cache",
+                  int((cache.sub2feat != -1).sum()), "of", len(ids))
     finally:
         torch.cuda.mem_get_info = probe
     path = os.path.join(HERE, "history_cache_fill_golden.npz")

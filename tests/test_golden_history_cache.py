@@ -202,6 +202,11 @@ def fill_inputs(c, g, name):
     return feats, hot
 
 
+def eval_ids(c):
+    """tests/golden/gen_history_cache_golden.py:eval_ids"""
+    return np.random.default_rng(c["seed"] + 100).integers(0, c["N"], size=min(c["N"], 700)).astype(np.int64)
+
+
 def check_fill(name, g, N, Fin, buffer_floats, feat2full, full2embed, embed2full, buffer, header):
     """The reference keeps only the cached block in feat2full; here it is slot-indexed with -1 in the empty
     slots in front, so its tail is compared."""
@@ -229,6 +234,10 @@ def test_oracle_reproduces_reference_constructor(name):
     assert floats // c["H"] == int(g[name + "_overall_embed_num"])
     check_fill(name, g, c["N"], c["Fin"], floats, st.feat2full.numpy(), st.full2embed.numpy(), st.embed2full.numpy(),
                st.buffer.numpy(), st.header)
+    # the reference's evaluation lookup (feature_cache_only=True) on the cache as its fill() left it
+    sub2feat, x = host_model.lookup_feature_cache_only(st, torch.from_numpy(eval_ids(c)), torch.from_numpy(feats))
+    np.testing.assert_array_equal(sub2feat.numpy(), g[name + "_eval_sub2feat"])
+    np.testing.assert_array_equal(x.numpy(), g[name + "_eval_x"])
 
 
 @pytest.mark.gpu
@@ -253,3 +262,10 @@ def test_gpu_cache_reproduces_reference_constructor(name, tmp_path):
     assert cache.overall_embed_num == int(g[name + "_overall_embed_num"])
     check_fill(name, g, c["N"], c["Fin"], cache.buffer.numel(), cache.feat2full.cpu().numpy(),
                cache.full2embed.cpu().numpy(), cache.embed2full.cpu().numpy(), cache.buffer.cpu().numpy(), cache.header)
+    # the evaluation lookup: the reference's own batch.x and feature slots for the same ids
+    from types import SimpleNamespace
+    batch = SimpleNamespace(sub_to_full=torch.from_numpy(eval_ids(c)).to(dev), x=None)
+    cache.lookup_and_load(batch, 2, feature_cache_only=True)
+    np.testing.assert_array_equal(cache.sub2feat.cpu().numpy(), g[name + "_eval_sub2feat"])
+    np.testing.assert_array_equal(batch.x.cpu().numpy(), g[name + "_eval_x"])
+    assert int((cache.sub2feat != -1).sum()) > 0 and cache.used_masks is None
