@@ -6,7 +6,8 @@ TEST INFRASTRUCTURE ONLY (see hc_oracle.c).  Statement by statement it follows
 ``HistoryTable`` (/root/reference/hiscache/history_table.py:94-125, 189-251), on CPU tensors, with the
 kernel calls replaced by the C oracle.  State lives in a plain object so tests can compare every
 tensor with the GPU implementation.  Pinned by vectors that the reference's own code produced
-(tests/golden: the cache's two entry points, the table's lookup and evictions).
+(tests/golden: the cache's two entry points, its constructor and its evaluation lookup, the table's lookup and
+evictions).
 """
 import math
 from types import SimpleNamespace
