@@ -152,3 +152,22 @@ def test_trainer_keeps_half_precision_features_in_half_precision(tmp_path, recor
     trainer.train()
     assert trainer.val_metrics[0] > 0.5 and trainer.table.header > 0
     trainer.close()
+
+
+def test_profiled_epoch_reports_the_phases(tmp_path):
+    """``dl.performance.prof``: ``train`` runs the profiled epoch, which sums the time of every phase as the
+    reference's does (load, forward, loss, backward, step, update, sample) and trains like the ordinary one."""
+    from hiscache import Config, HistoryTrainer, make_config
+    rng = np.random.default_rng(83)
+    dataset(tmp_path, rng)
+    cfg = make_config(32, 4, 32, 3, method="grad", rate=0.5, staleness_thres=7, device=DEV, path=str(tmp_path))
+    cfg["dl"]["performance"] = Config({"prof": True})
+    torch.manual_seed(6)
+    trainer = HistoryTrainer(cfg, fanout=[4, 3, 2], batch_size=200, lr=1e-2, num_epochs=2, eval_begin=1,
+                             cache_bytes=1500 * 32 * 4)
+    assert trainer.prof
+    trainer.train()
+    assert set(trainer.times) == {"load", "forward", "loss", "backward", "step", "update", "sample"}
+    assert all(v >= 0.0 for v in trainer.times.values()) and trainer.times["forward"] > 0 and trainer.times["backward"] > 0
+    assert sum(trainer.times.values()) < 2.0 * trainer.epoch_seconds[-1] + 0.1
+    assert trainer.glb_iter == 2 * 19 and trainer.val_metrics[0] > 0.5 and trainer.table.header > 0
