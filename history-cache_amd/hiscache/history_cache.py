@@ -345,6 +345,31 @@ class HistoryCache:
         m, self._uncounted_mask = self._uncounted_mask, None
         return m
 
+    _STATE = ("buffer", "full2embed", "embed2full", "feat2full", "_header", "_num_stored", "_overflow")
+
+    def state_dict(self):
+        """The cache's contents for a checkpoint (the reference saves none): copies of the buffer, the maps and the
+        write position, and the iteration counter."""
+        if "history" not in self.feat_mode:
+            return {"glb_iter": self.glb_iter}
+        out = {name.lstrip("_"): getattr(self, name).detach().clone() for name in self._STATE}
+        out["glb_iter"] = self.glb_iter
+        return out
+
+    def load_state_dict(self, state):
+        """Restore what ``state_dict`` saved into a cache of the same sizes."""
+        self.glb_iter = int(state["glb_iter"])
+        if "history" not in self.feat_mode:
+            return
+        for name in self._STATE:
+            src, dst = state[name.lstrip("_")], getattr(self, name)
+            if tuple(src.shape) != tuple(dst.shape) or src.dtype != dst.dtype:
+                raise ValueError(f"{name.lstrip('_')}: saved {tuple(src.shape)} {src.dtype}, "
+                                 f"this cache has {tuple(dst.shape)} {dst.dtype}")
+        for name in self._STATE:
+            getattr(self, name).copy_(state[name.lstrip("_")])
+        self.produced_embedding = self.sub2embed = self.sub2feat = self.cached_embedding = self.used_masks = None
+
     def stats(self):
         """Cache occupancy, and what the lookups since construction (or ``reset_stats``) found: hit rates of the
         embedding and the feature cache, rows pruned, rows and bytes read from the feature store, rows admitted

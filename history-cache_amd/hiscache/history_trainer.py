@@ -112,6 +112,28 @@ class HistoryTrainer:
         self.metric = None
         self.epoch_seconds = []
 
+    def state_dict(self):
+        """Model, optimizer, cache contents and the counters, for a checkpoint (the reference's trainer saves
+        none): ``torch.save(trainer.state_dict(), path)``."""
+        return {"model": self.model.state_dict(), "optimizer": self.optimizer.state_dict(),
+                "table": self.table.state_dict(), "glb_iter": self.glb_iter, "best_metric": self.best_metric,
+                "val_metrics": list(self.val_metrics), "test_metrics": list(self.test_metrics),
+                "generator": self._generator.get_state(), "sampler_batches": self.sampler.batches}
+
+    def load_state_dict(self, state):
+        """Resume from ``state_dict``'s result in a trainer built the same way (recordings are made again on
+        demand; the sampler continues its sequence of batch keys)."""
+        self.model.load_state_dict(state["model"])
+        self.optimizer.load_state_dict(state["optimizer"])
+        self.table.load_state_dict(state["table"])
+        self.glb_iter = int(state["glb_iter"])
+        self.best_metric = state["best_metric"]
+        self.val_metrics, self.test_metrics = list(state["val_metrics"]), list(state["test_metrics"])
+        self._generator.set_state(state["generator"].cpu())
+        self.sampler.batches = int(state["sampler_batches"])
+        if self._step is not None:
+            self._step.clear()
+
     def close(self):
         """Give the read-ahead stream back (it is made again on demand)."""
         close = getattr(self.uvm, "close", None)

@@ -184,6 +184,26 @@ class RingHistoryCache:
         self.last_score = score
         self.produced_embedding = None
 
+    _STATE = ("table", "full2slot", "slot2full", "checkin", "_header")
+
+    def state_dict(self):
+        """The table, its maps and write position and the iteration counter, copied, for a checkpoint."""
+        out = {name.lstrip("_"): getattr(self, name).detach().clone() for name in self._STATE}
+        out["glb_iter"] = self.glb_iter
+        return out
+
+    def load_state_dict(self, state):
+        """Restore what ``state_dict`` saved into a cache of the same sizes."""
+        for name in self._STATE:
+            src, dst = state[name.lstrip("_")], getattr(self, name)
+            if tuple(src.shape) != tuple(dst.shape) or src.dtype != dst.dtype:
+                raise ValueError(f"{name.lstrip('_')}: saved {tuple(src.shape)} {src.dtype}, "
+                                 f"this cache has {tuple(dst.shape)} {dst.dtype}")
+        for name in self._STATE:
+            getattr(self, name).copy_(state[name.lstrip("_")])
+        self.glb_iter = int(state["glb_iter"])
+        self.produced_embedding = self.sub2embed = self.cached_embedding = self.used_masks = None
+
     def stats(self):
         """Table occupancy and what the lookups since construction found: embedding hit rate, rows pruned, rows
         and bytes read from the feature store, rows admitted (the counts of the reference's lookup log,

@@ -171,3 +171,41 @@ def test_profiled_epoch_reports_the_phases(tmp_path):
     assert all(v >= 0.0 for v in trainer.times.values()) and trainer.times["forward"] > 0 and trainer.times["backward"] > 0
     assert sum(trainer.times.values()) < 2.0 * trainer.epoch_seconds[-1] + 0.1
     assert trainer.glb_iter == 2 * 19 and trainer.val_metrics[0] > 0.5 and trainer.table.header > 0
+
+
+@pytest.mark.parametrize("ring,recorded", [(False, False), (True, False), (False, True)])
+def test_checkpoint_and_resume_continue_the_same_run(tmp_path, ring, recorded):
+    """Two epochs in one go against one epoch, ``state_dict`` through ``torch.save`` / ``torch.load``, a fresh
+    trainer, ``load_state_dict`` and the second epoch: the same parameters, cache contents and counters, bit for
+    bit (the sampler's batch keys and the shuffling generator continue where they stopped)."""
+    from hiscache import HistoryTrainer, make_config
+    rng = np.random.default_rng(84)
+    dataset(tmp_path, rng)
+    cfg = make_config(32, 4, 32, 3, method="grad", rate=0.5, staleness_thres=7, device=DEV, path=str(tmp_path))
+
+    def build():
+        torch.manual_seed(9)
+        return HistoryTrainer(cfg, fanout=[4, 3, 2], batch_size=200, lr=1e-2, num_epochs=2, eval_begin=9,
+                              cache_bytes=1500 * 32 * 4, ring_rows=3000 if ring else 0, recorded=recorded, seed=3)
+
+    whole = build()
+    whole.cxg_train_epoch()
+    whole.cxg_train_epoch()
+    first = build()
+    first.cxg_train_epoch()
+    path = str(tmp_path / "checkpoint.pt")
+    torch.save(first.state_dict(), path)
+    resumed = build()
+    resumed.load_state_dict(torch.load(path, weights_only=True))
+    assert resumed.glb_iter == first.glb_iter == 19
+    resumed.cxg_train_epoch()
+    assert resumed.glb_iter == whole.glb_iter == 38
+    for p, q in zip(resumed.model.parameters(), whole.model.parameters()):
+        assert torch.equal(p, q)
+    a, b = resumed.table.state_dict(), whole.table.state_dict()
+    assert set(a) == set(b)
+    for k in a:
+        assert (torch.equal(a[k], b[k]) if isinstance(a[k], torch.Tensor) else a[k] == b[k]), k
+    other = HistoryTrainer(cfg, fanout=[4, 3, 2], batch_size=200, cache_bytes=700 * 32 * 4, ring_rows=1000 if ring else 0)
+    with pytest.raises(ValueError):
+        other.table.load_state_dict(first.table.state_dict())      # a cache of another size
