@@ -12,8 +12,11 @@
 //            leaves the first edge slot that mentions an unseen node in the node map
 //   flag     an edge owns its node when the map holds its own slot
 //   scan     owners before every slot -> new local ids in first-seen order
+//            (count and flag stay launches of their own: read through a functor inside the scans, their
+//            random reads of the graph and of the node map made a batch a third slower)
 //   relabel  idx <- local ids; owners append to sub_to_full
-//   commit   node map <- local ids of the new nodes; advance (lo, hi, edges)
+//   commit   node map <- local ids of the new nodes; its first thread writes the next hop's state
+//            (lo, hi, edges): every hop has a state of its own, so nothing it reads changes under it
 // perm_u is a keyed bijection of [0, deg): four Feistel rounds on the next even power of two with
 // cycle walking, so the picks of a row are distinct (sampling without replacement) at O(fanout)
 // work whatever the degree.  Everything is integer work with one well-defined result.
@@ -110,7 +113,6 @@ __global__ __launch_bounds__(HC_BLOCK) void sp_pick(const int64_t *__restrict__ 
                                                      const int64_t *__restrict__ sub_to_full,
                                                      const SpState *__restrict__ st, int64_t fanout,
                                                      int64_t num_nodes, int hop,
-                                                     const int32_t *__restrict__ cnt,
                                                      const int32_t *__restrict__ incl, int32_t *__restrict__ loc,
                                                      int64_t *__restrict__ ptr, int64_t *__restrict__ idx,
                                                      int64_t cap) {
@@ -120,8 +122,8 @@ __global__ __launch_bounds__(HC_BLOCK) void sp_pick(const int64_t *__restrict__ 
   if (i >= cap) return;
   const int64_t u = st->lo + i;
   if (u >= st->hi) return;
-  const int32_t c = cnt[i];
-  const int64_t begin = (int64_t)incl[i] - c;  // slot of the row's first pick inside this hop
+  const int64_t begin = i > 0 ? (int64_t)incl[i - 1] : 0;  // slot of the row's first pick inside this hop
+  const int32_t c = (int32_t)((int64_t)incl[i] - begin);
   const int64_t base = st->edges;
   if (sub == 0) ptr[u + 1] = base + incl[i];
   if (c == 0) return;
@@ -181,30 +183,26 @@ __global__ __launch_bounds__(HC_BLOCK) void sp_relabel(int64_t *__restrict__ idx
 }
 
 __global__ __launch_bounds__(HC_BLOCK) void sp_commit(const int64_t *__restrict__ sub_to_full,
-                                                       const SpState *__restrict__ st,
+                                                       const SpState *__restrict__ st, SpState *__restrict__ next,
                                                        const int32_t *__restrict__ incl, int64_t cap,
                                                        const int32_t *__restrict__ rank_incl,
-                                                       int32_t *__restrict__ loc, int64_t edge_cap) {
+                                                       int32_t *__restrict__ loc, int64_t *__restrict__ counts,
+                                                       int hop, int num_hops, int64_t edge_cap) {
   const int64_t i = (int64_t)blockIdx.x * HC_BLOCK + threadIdx.x;
   if (i >= edge_cap) return;
   const int64_t hop_edges = incl[cap - 1];
   const int64_t fresh = hop_edges > 0 ? rank_incl[hop_edges - 1] : 0;
+  if (i == 0) {  // the next hop's state (this hop's is read by the other threads and stays as it is)
+    next->lo = st->hi;
+    next->hi = st->hi + fresh;
+    next->edges = st->edges + hop_edges;
+    next->key = st->key;
+    counts[hop + 1] = st->hi + fresh;
+    counts[num_hops + 1 + hop] = st->edges + hop_edges;
+  }
   if (i >= fresh) return;
   const int64_t id = st->hi + i;
   loc[sub_to_full[id]] = (int32_t)id;
-}
-
-__global__ void sp_advance(SpState *__restrict__ st, const int32_t *__restrict__ incl, int64_t cap,
-                           const int32_t *__restrict__ rank_incl, int64_t *__restrict__ counts, int hop,
-                           int num_hops) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
-  const int64_t hop_edges = incl[cap - 1];
-  const int64_t fresh = hop_edges > 0 ? rank_incl[hop_edges - 1] : 0;
-  st->lo = st->hi;
-  st->hi += fresh;
-  st->edges += hop_edges;
-  counts[hop + 1] = st->hi;
-  counts[num_hops + 1 + hop] = st->edges;
 }
 
 __global__ __launch_bounds__(HC_BLOCK) void sp_reset(const int64_t *__restrict__ sub_to_full,
@@ -270,8 +268,8 @@ struct SpLayout {
 SpLayout sp_layout(const SpCaps &c) {
   SpLayout l{};
   size_t off = 0;
-  l.state = off;
-  off += 256;
+  l.state = off;                                   // one state per hop and the final one
+  off += hc_align_up(sizeof(SpState) * (HC_SAMPLE_MAX_HOPS + 1), 256);
   l.cnt = off;
   off += hc_align_up((size_t)(c.max_rows + 1) * 4, 256);
   l.incl = off;
@@ -336,7 +334,7 @@ int sample_layers_impl(const int64_t *indptr, const int64_t *indices, int64_t nu
     return HC_EUNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   char *w = static_cast<char *>(workspace);
-  SpState *st = reinterpret_cast<SpState *>(w + l.state);
+  SpState *states = reinterpret_cast<SpState *>(w + l.state);
   int32_t *cnt = reinterpret_cast<int32_t *>(w + l.cnt);
   int32_t *incl = reinterpret_cast<int32_t *>(w + l.incl);
   int32_t *flag = reinterpret_cast<int32_t *>(w + l.flag);
@@ -344,16 +342,17 @@ int sample_layers_impl(const int64_t *indptr, const int64_t *indices, int64_t nu
   void *scan_ws = w + l.scan;
   const dim3 bl(HC_BLOCK);
 
-  sp_init<<<dim3(sp_blocks(n_seed)), bl, 0, s>>>(seeds, n_seed, num_nodes, node_map, sub_to_full, ptr, counts, st,
+  sp_init<<<dim3(sp_blocks(n_seed)), bl, 0, s>>>(seeds, n_seed, num_nodes, node_map, sub_to_full, ptr, counts, states,
                                                  rng_seed, rng_seed_at);
   for (int k = 0; k < num_hops; ++k) {
     const int64_t cap = c.rows[k], ecap = c.edges[k];
+    const SpState *st = states + k;
     sp_count<<<dim3(sp_blocks(cap)), bl, 0, s>>>(indptr, sub_to_full, st, fanout[k], num_nodes, cnt, cap);
     size_t bytes = sp_scan_bytes(cap);
     if (rocprim::inclusive_scan(scan_ws, bytes, cnt, incl, (size_t)cap, rocprim::plus<int32_t>(), s) != hipSuccess)
       return HC_ELAUNCH;
     sp_pick<<<dim3(sp_blocks(cap * SP_GROUP)), bl, 0, s>>>(indptr, indices, sub_to_full, st, fanout[k], num_nodes,
-                                                          k, cnt, incl, node_map, ptr, idx, cap);
+                                                          k, incl, node_map, ptr, idx, cap);
     sp_flag<<<dim3(sp_blocks(ecap)), bl, 0, s>>>(idx, node_map, st, incl, cap, num_nodes, flag, ecap);
     bytes = sp_scan_bytes(ecap);
     if (rocprim::inclusive_scan(scan_ws, bytes, flag, rank, (size_t)ecap, rocprim::plus<int32_t>(), s) !=
@@ -361,10 +360,11 @@ int sample_layers_impl(const int64_t *indptr, const int64_t *indices, int64_t nu
       return HC_ELAUNCH;
     sp_relabel<<<dim3(sp_blocks(ecap)), bl, 0, s>>>(idx, node_map, st, incl, cap, num_nodes, rank, sub_to_full,
                                                    ecap);
-    sp_commit<<<dim3(sp_blocks(ecap)), bl, 0, s>>>(sub_to_full, st, incl, cap, rank, node_map, ecap);
-    sp_advance<<<dim3(1), dim3(HC_WAVE), 0, s>>>(st, incl, cap, rank, counts, k, num_hops);
+    sp_commit<<<dim3(sp_blocks(ecap)), bl, 0, s>>>(sub_to_full, st, states + k + 1, incl, cap, rank, node_map,
+                                                  counts, k, num_hops, ecap);
     if (hc_launch_status() != HC_OK) return HC_ELAUNCH;
   }
+  const SpState *st = states + num_hops;
   sp_reset<<<dim3(sp_blocks(c.total_nodes)), bl, 0, s>>>(sub_to_full, st, num_nodes, node_map, c.total_nodes);
   return hc_launch_status();
 }
