@@ -183,3 +183,50 @@ def test_ring_cache_at_the_full_table_size(orc, name):
         del ref_table
     del cache
     torch.cuda.empty_cache()
+
+
+def test_row_gathers_from_a_feature_matrix_of_the_full_size():
+    """The papers100M feature matrix at its real size in device memory (111 M x 128 fp32, 57 GB): rows whose contents
+    are a function of their number, read through ``hc_gather_rows`` (several rows per wave) and through the hot tier
+    (a 111 M-entry slot map, 50 M device copies whose slots run against the row order), the last row included --
+    byte offsets beyond 2^35."""
+    import hiscache_backend as be
+    N, F = 111_000_000, 128
+    need = N * F * 4 + 50_000_000 * F * 4 + N * 4 + (6 << 30)
+    free, _ = torch.cuda.mem_get_info()
+    if free < need:
+        pytest.skip("needs %.0f GB of device memory, %.0f GB are free" % (need / 1e9, free / 1e9))
+    col = torch.arange(F, device=DEV, dtype=torch.float32) / 256.0
+
+    def rows_of(ids):                                  # what row ``ids[i]`` of the matrix holds
+        return (ids % 99_991).to(torch.float32)[:, None] + (ids // 99_991 % 7).to(torch.float32)[:, None] * 0.5 + col
+
+    matrix = torch.empty((N, F), dtype=torch.float32, device=DEV)
+    step = 4_000_000
+    for lo in range(0, N, step):
+        hi = min(N, lo + step)
+        matrix[lo:hi] = rows_of(torch.arange(lo, hi, device=DEV))
+    gen = torch.Generator(device=DEV).manual_seed(7)
+    ids = torch.randint(0, N, (150_000,), device=DEV, generator=gen)
+    ids[0], ids[1], ids[2] = N - 1, 0, -1                                   # (-1 addresses the last row)
+    mask = torch.rand(150_000, device=DEV, generator=gen) < 0.9
+    want = rows_of(torch.where(ids < 0, ids + N, ids)) * mask[:, None]
+    assert torch.equal(be.gather_rows(matrix, ids, mask=mask), want)
+    # the hot tier: nodes [61 M, 111 M) have copies, in reverse order
+    n_hot = 50_000_000
+    slot = torch.full((N,), -1, dtype=torch.int32, device=DEV)
+    slot[N - n_hot:] = torch.arange(n_hot - 1, -1, -1, dtype=torch.int32, device=DEV)
+    hot = torch.empty((n_hot, F), dtype=torch.float32, device=DEV)
+    for lo in range(0, n_hot, step):
+        hi = min(n_hot, lo + step)
+        hot[lo:hi] = rows_of(N - 1 - torch.arange(lo, hi, device=DEV))
+    out = torch.full((150_000, F), -1.0, device=DEV)
+    _, cold = be.gather_rows_hot(hot, slot, ids, mask=mask, out=out)
+    wrapped = torch.where(ids < 0, ids + N, ids)
+    is_hot = wrapped >= N - n_hot
+    assert torch.equal(cold.bool(), mask & ~is_hot)
+    done = ~(mask & ~is_hot)
+    assert torch.equal(out[done], want[done]) and bool((out[~done] == -1.0).all())
+    be.gather_rows_flagged(matrix, ids, cold, out)                           # (the other tier, here device memory too)
+    assert torch.equal(out, want)
+    assert int(is_hot[mask].sum()) > 50_000 and int(cold.sum()) > 50_000
