@@ -58,6 +58,7 @@ class RecordedIteration:
         self.read_ahead_slots = max(1, int(read_ahead_slots))
         self._reads_started = 0
         self.device = cache.device
+        self._hub_edges = _be.bwd_chunk_edges(256) or (1 << 62)
         self._base = None                 # sizes of the first batch: (n0, [n1 .. nL], E)
         self._records = {}
         self._capture_stream = None
@@ -99,11 +100,15 @@ class RecordedIteration:
         if view is not None and (view.rows < nnl[self.L - 1] or view.n_src < nnl[self.L]):
             view = None
         view_kind = 0 if view is None else (2 if view.edgeT is not None else 1)
+        # a view known to hold no source above the backward's chunk length is recorded without the hub launches
+        if view is not None and view.max_in_degree is not None and view.max_in_degree <= self._hub_edges:
+            view_kind += 10
         return nnl, n_edges, view_kind, getattr(batch, "edge_type", None)
 
     # ------------------------------------------------------------------ records
     def _new_record(self, j, view_kind, pre_like, etype):
         L, dev = self.L, self.device
+        hubless, view_kind = view_kind >= 10, view_kind % 10
         has_view = view_kind > 0
         caps, e_cap = self._shape(j)
         r = _Record()
@@ -130,7 +135,8 @@ class RecordedIteration:
             r.have = torch.zeros(caps[L], dtype=torch.uint8, device=dev)
             r.src_ids = torch.full((caps[L],), -1, **i64)
             pre = SimpleNamespace(rows=r.x_pre, have=r.have, src_ids=r.src_ids)
-        view = _be.BatchView(r.ptrT, r.rowT, r.edgeT, caps[L - 1], caps[L], e_cap) if has_view else None
+        view = (_be.BatchView(r.ptrT, r.rowT, r.edgeT, caps[L - 1], caps[L], e_cap, 0 if hubless else None)
+                if has_view else None)
         r.batch = SimpleNamespace(
             ptr=r.ptr, idx=r.idx, sub_to_full=r.s2f, y=r.y, x=None, edge_type=r.etype, typed_num_node_in_layer=None,
             num_node_in_layer=torch.tensor(caps, dtype=torch.int64), num_edge_in_layer=[e_cap] * L, view=view,
@@ -262,7 +268,8 @@ class RecordedIteration:
         self._records.clear()
 
     def shapes(self):
-        """The padded shapes in use: {(j, view kind 0/1/2 = none/rows/rows and edge slots, read-ahead slot (-1: no
+        """The padded shapes in use: {(j, view kind 0/1/2 = none/rows/rows and edge slots -- +10 when the view is known
+        to hold no source above the backward's chunk length --, read-ahead slot (-1: no
         rows read ahead, -2: copied in, 0..: read straight into that recording's array), edge types given):
         ([n0 .. nL], edges, recorded?, uses)}."""
         return {k: (r.caps, r.e_cap, r.graph is not None, r.uses) for k, r in self._records.items()}

@@ -103,6 +103,9 @@ def make_batch(sample, labels, device, emit_view=False, view_edges=False):
         nnl = sample["num_node_in_layer"]
         batch.view = hiscache_backend.build_batch_view(batch.ptr, batch.idx, int(nnl[L - 1]), int(nnl[L]),
                                                        want_edges=view_edges)
+        # known here at no cost (the arrays are on the host): lets the backward leave its hub path out
+        idx = sample["idx"]
+        batch.view.max_in_degree = int(np.bincount(idx, minlength=1).max()) if len(idx) else 0
     return batch
 
 

@@ -377,11 +377,15 @@ class BatchView:
     ``rows`` rows.  A layer that owns the first R <= rows rows and the first n <= n_src sources uses a
     prefix of ``ptrT``; edges of other rows are stepped over in backward.  ``num_edge`` bounds the
     entries of ``rowT`` that hold edges."""
-    __slots__ = ("ptrT", "rowT", "edgeT", "rows", "n_src", "num_edge")
+    __slots__ = ("ptrT", "rowT", "edgeT", "rows", "n_src", "num_edge", "max_in_degree")
 
-    def __init__(self, ptrT, rowT, edgeT, rows, n_src, num_edge):
+    def __init__(self, ptrT, rowT, edgeT, rows, n_src, num_edge, max_in_degree=None):
         self.ptrT, self.rowT, self.edgeT = ptrT, rowT, edgeT
         self.rows, self.n_src, self.num_edge = int(rows), int(n_src), int(num_edge)
+        # the largest number of edges that one node of the batch has in the view, when whoever made the batch
+        # knows it (None: unknown).  A view without a source above the backward's chunk length needs neither
+        # the chunk sums nor the launch that combines them.
+        self.max_in_degree = None if max_in_degree is None else int(max_in_degree)
 
     def covers(self, num_node, n_src):
         return int(num_node) <= self.rows and int(n_src) <= self.n_src
@@ -435,7 +439,9 @@ def _aggr_bwd_batch_view(ptr, view, g, hmap, hbuf_shape, hsize, num_node, n_src,
         grad_h = torch.empty(hbuf_shape, dtype=torch.float32, device=dev)
         if grad_h.numel() != R * hsize:
             grad_h.zero_()
-    nbytes = lib.hc_aggr_bwd_workspace_bytes(view.num_edge, F)
+    chunk = bwd_chunk_edges(F)
+    hubless = view.max_in_degree is not None and (chunk == 0 or view.max_in_degree <= chunk)
+    nbytes = 0 if hubless else lib.hc_aggr_bwd_workspace_bytes(view.num_edge, F)
     ws = _workspace(nbytes, dev) if nbytes else None
     rc = lib.hc_aggr_bwd_batch_view(_ptr(ptr), _ptr(view.ptrT), _ptr(view.rowT), _ptr(g), _ptr(hmap),
                                     _ptr(grad_x), _ptr(grad_h), int(hsize), view.num_edge, R, F, int(n_src),

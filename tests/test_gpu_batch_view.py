@@ -96,15 +96,18 @@ def test_batch_view_equals_layer_view_without_hubs(be, orc, F):
         g = T(rng.standard_normal((R, F)).astype(np.float32))
         hmap = T(random_hmap(rng, R, 0.35))
         hbuf = T(rng.standard_normal((R, F)).astype(np.float32))
+        # (a view that knows it holds no hub: the backward then runs without its hub launches)
+        known = be.BatchView(view.ptrT, view.rowT, view.edgeT, view.rows, view.n_src, view.num_edge,
+                             max_in_degree=int(np.bincount(idx).max()))
         got = []
-        for v in (None, view):
+        for v in (None, view, known):
             xx = T(x).requires_grad_(True)
             hb = hbuf.clone().requires_grad_(True)
             out = be.aggr_forward_history(xx, tptr, tidx, hmap, hb, F, R, int(ptr[R]), v)
             out.backward(g)
             got.append((out.detach(), xx.grad, hb.grad))
-        for a, b in zip(*got):
-            assert torch.equal(a, b)
+        for a, b, c in zip(*got):
+            assert torch.equal(a, b) and torch.equal(a, c)
         ref, ref_h = orc.bwd_mean_row(ptr[:R + 1], idx, g.cpu().numpy(), hmap.cpu().numpy(), n_src,
                                       hbuf_shape=(R, F))
         np.testing.assert_array_equal(got[1][1].cpu().numpy(), ref)
