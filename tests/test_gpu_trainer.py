@@ -209,3 +209,24 @@ def test_checkpoint_and_resume_continue_the_same_run(tmp_path, ring, recorded):
     other = HistoryTrainer(cfg, fanout=[4, 3, 2], batch_size=200, cache_bytes=700 * 32 * 4, ring_rows=1000 if ring else 0)
     with pytest.raises(ValueError):
         other.table.load_state_dict(first.table.state_dict())      # a cache of another size
+
+
+@pytest.mark.parametrize("extra", [[], ["trainer.recorded=true", "trainer.read_ahead=true", "trainer.hot_rows=2000"]])
+def test_example_main_trains_from_its_configuration(tmp_path, extra):
+    """The example's entry (the role of /root/reference/example/main.py): YAML configuration, overrides, a dataset
+    written on request, ``HistoryTrainer(config).train()``."""
+    import importlib.util
+    import os
+    here = os.path.dirname(os.path.abspath(__file__))
+    spec = importlib.util.spec_from_file_location(
+        "hiscache_example_main", os.path.join(here, "..", "history-cache_amd", "example", "main.py"))
+    ex = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(ex)
+    trainer = ex.main(["--synthetic", "8000", f"dl.dataset.path={tmp_path}", "dl.dataset.feature_dim=32",
+                       "dl.dataset.num_classes=4", "train.model.hidden_dim=32", "dl.sampler.train.batch_size=400",
+                       "dl.sampler.train.num_neighbors=[4,3,2]", "train.optimizer.lr=0.01", "history.rate=0.6",
+                       "history.staleness_thres=5", "trainer.cache_megabytes=0.25", "train.train.num_epochs=3"] + extra)
+    assert trainer.glb_iter == 3 * 12                              # 4 800 training nodes in batches of 400
+    assert len(trainer.val_metrics) == 3 and trainer.val_metrics[-1] > 0.5 and trainer.test_metrics[-1] > 0.5
+    assert trainer.recorded == bool(extra) and (trainer.uvm.hot_rows is not None) == bool(extra)
+    assert os.path.exists(os.path.join(tmp_path, "processed", "sorted_indices.dat"))
