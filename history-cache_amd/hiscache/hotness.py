@@ -5,7 +5,8 @@ The feature cache of ``HistoryCache`` and the hot tier of ``PinnedFeatureStore``
 reference ranks nodes by one of three metrics, spelled out in /root/reference/test/test_cache.py: the degree
 (:18-24), how often a node turns up in the sampled batches of an epoch (:27-38), or a PageRank seeded at the
 training nodes (:41-77); ``get_cache_map`` (:128-143) takes the top of the ranking and ``test_cache`` (:146-161)
-measures the share of a batch's rows it serves.  The same functions here, on torch tensors (any device).
+measures the share of a batch's rows it serves; ``test_embedding_cache`` (:165-239) simulates embedding caches and
+counts the input rows they spare.  The same functions here, on torch tensors (any device).
 """
 import os
 from os import path
@@ -78,6 +79,56 @@ def feature_cache_hit_rate(cache_status, batches):
         visits += int(nodes.numel())
         hits += int(cache_status[nodes].sum())
     return (hits / visits if visits else 0.0), hits, visits
+
+
+def embedding_cache_hit_rate(batches, num_nodes, cache_layers=(1,), rate=0.9, staleness=200, expire=False,
+                             score_fn=None):
+    """Simulate embedding caches on a stream of batches and count the input rows they spare
+    (test_cache.py:165-239).  Layer k's cache holds nodes whose layer-k embedding is stored (k = 0: the seeds).
+    Per batch, top down: a layer-k row must be computed when it is needed and not cached; the neighbours of such
+    rows are needed in layer k+1 (:165-175, :201-208); an input row that is not needed is a hit (:211-213).
+    Then every layer of ``cache_layers`` admits its needed rows whose score lies under the ``rate`` quantile of
+    the layer's scores (:215-225; ``score_fn(n, device)``, default standard normal as there).
+    ``expire``: drop the entries admitted ``staleness`` iterations ago.  The reference writes that reset into a
+    temporary (:226-230), so its entries never expire: False reproduces it, True does what it means to.
+    Yields (hits, visits, entries held per layer) after every batch."""
+    status = {k: None for k in cache_layers}
+    admitted = {k: [] for k in cache_layers}
+    glb_iter = 0
+    for batch in batches:
+        glb_iter += 1
+        s2f, ptr, idx = batch.sub_to_full, batch.ptr, batch.idx
+        dev = s2f.device
+        nnl = [int(n) for n in batch.num_node_in_layer]
+        L = len(nnl) - 1
+        for k in status:
+            if status[k] is None:
+                status[k] = torch.zeros(int(num_nodes), dtype=torch.int64, device=dev)
+        needed = [torch.ones(nnl[0], dtype=torch.bool, device=dev)]
+        for k in range(L):
+            live = needed[k]
+            if k in status:
+                live = live & (status[k][s2f[:nnl[k]]] == 0)
+            deg = ptr[1:nnl[k] + 1] - ptr[:nnl[k]]
+            nxt = torch.zeros(nnl[k + 1], dtype=torch.bool, device=dev)
+            nxt[idx[:int(ptr[nnl[k]])][torch.repeat_interleave(live, deg)]] = True
+            needed.append(nxt)
+        visits = nnl[L]
+        hits = visits - int(needed[L].sum())
+        for k in sorted(status):
+            if k >= L:
+                continue
+            score = (score_fn or (lambda n, d: torch.randn(n, device=d)))(nnl[k], dev)
+            thres = torch.quantile(score, rate)
+            to_cache = s2f[:nnl[k]][(score < thres) & needed[k]]
+            admitted[k].append(to_cache)
+            status[k][to_cache] = glb_iter
+            if glb_iter >= staleness:
+                oldest = admitted[k].pop(0)
+                if expire:
+                    stale = oldest[glb_iter - status[k][oldest] >= staleness]
+                    status[k][stale] = 0
+        yield hits, visits, {k: int((status[k] != 0).sum()) for k in sorted(status)}
 
 
 def write_hotness_order(root, order):

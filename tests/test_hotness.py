@@ -1,5 +1,5 @@
 """Hotness orders (``hiscache.hotness``): the three metrics against brute force, the cached set's threshold rule, the
-file round trip; on the GPU the access counts of sampled batches and what the hottest rows buy a tiered store."""
+file round trip, the embedding-cache simulation against its loops; on the GPU the access counts of sampled batches and what the hottest rows buy a tiered store."""
 import numpy as np
 import pytest
 import torch
@@ -105,3 +105,91 @@ def test_access_counts_of_sampled_batches_and_what_the_hot_rows_serve():
     hot = torch.zeros(N, dtype=torch.bool, device=DEV)
     hot[hotness_order(metric)[-k:]] = True
     assert int(store.last_cold.sum()) == int((~hot[b.sub_to_full]).sum())
+    # the embedding-cache simulation on the device's batches and on host copies of them: the same counts
+    from types import SimpleNamespace
+    from hiscache.hotness import embedding_cache_hit_rate
+    table = torch.from_numpy(rng.standard_normal((len(batches), 4096)).astype(np.float32))
+
+    def scores():
+        it = iter(table)
+        return lambda n, d: next(it)[:n].to(d)
+    on_host = [SimpleNamespace(ptr=x.ptr.cpu(), idx=x.idx.cpu(), sub_to_full=x.sub_to_full.cpu(),
+                               num_node_in_layer=x.num_node_in_layer) for x in batches]
+    dev_run = list(embedding_cache_hit_rate(batches, N, rate=0.9, staleness=4, expire=True, score_fn=scores()))
+    assert dev_run == list(embedding_cache_hit_rate(on_host, N, rate=0.9, staleness=4, expire=True, score_fn=scores()))
+    assert dev_run[-1][0] > dev_run[0][0] and dev_run[-1][2][1] > 0
+
+
+def test_embedding_cache_simulation_against_loops():
+    """The simulation of /root/reference/test/test_cache.py:165-239 against its loops written out per row and per
+    edge, with scores from a table both sides read; entries that expire, and (as there) entries that never do."""
+    from types import SimpleNamespace
+    from hiscache.hotness import embedding_cache_hit_rate
+    rng = np.random.default_rng(5)
+    N, L = 400, 3
+    batches = []
+    for _ in range(12):
+        nnl = [10]
+        for _k in range(L):
+            nnl.append(nnl[-1] + int(rng.integers(5, 40)))
+        deg = rng.integers(0, 5, size=nnl[L - 1])
+        ptr = np.zeros(nnl[L - 1] + 1, np.int64)
+        ptr[1:] = np.cumsum(deg)
+        idx = np.zeros(ptr[-1], np.int64)
+        for k in range(L):                       # a row of layer k draws its neighbours among layer k+1's nodes
+            for r in range(nnl[k - 1] if k else 0, nnl[k]):
+                idx[ptr[r]:ptr[r + 1]] = rng.integers(0, nnl[k + 1], size=deg[r])
+        batches.append(SimpleNamespace(ptr=torch.from_numpy(ptr), idx=torch.from_numpy(idx),
+                                       sub_to_full=torch.from_numpy(rng.choice(N, size=nnl[L], replace=False)),
+                                       num_node_in_layer=torch.tensor(nnl)))
+    scores = torch.from_numpy(rng.standard_normal((len(batches) * L + 1, 200)).astype(np.float32))
+
+    def run_loops(cache_layers, staleness, expire):
+        status = {k: np.zeros(N, np.int64) for k in cache_layers}
+        admitted = {k: [] for k in cache_layers}
+        out, draw = [], 0
+        for it, b in enumerate(batches, start=1):
+            nnl = b.num_node_in_layer.tolist()
+            s2f, ptr, idx = b.sub_to_full.numpy(), b.ptr.numpy(), b.idx.numpy()
+            useful = [np.ones(nnl[0], bool)]
+            for k in range(L):
+                nxt = np.zeros(nnl[k + 1], bool)
+                for i in range(nnl[k]):
+                    cached = k in status and status[k][s2f[i]] != 0
+                    if useful[k][i] and not cached:
+                        for e in range(ptr[i], ptr[i + 1]):
+                            nxt[idx[e]] = True
+                useful.append(nxt)
+            hits = nnl[L] - int(useful[L].sum())
+            for k in sorted(status):
+                sc = scores[draw, :nnl[k]]
+                draw += 1
+                thres = float(torch.quantile(sc, 0.7))
+                ids = [int(s2f[i]) for i in range(nnl[k]) if float(sc[i]) < thres and useful[k][i]]
+                admitted[k].append(ids)
+                for v in ids:
+                    status[k][v] = it
+                if it >= staleness:
+                    for v in admitted[k].pop(0):
+                        if expire and it - status[k][v] >= staleness:
+                            status[k][v] = 0
+            out.append((hits, nnl[L], {k: int((status[k] != 0).sum()) for k in sorted(status)}))
+        return out
+
+    for cache_layers, staleness, expire in (((1,), 4, True), ((1,), 4, False), ((1, 2), 3, True), ((0, 1, 2), 200, False)):
+        draw = [0]
+
+        def score_fn(n, device):
+            draw[0] += 1
+            return scores[draw[0] - 1, :n].to(device)
+        got = list(embedding_cache_hit_rate(batches, N, cache_layers=cache_layers, rate=0.7, staleness=staleness,
+                                            expire=expire, score_fn=score_fn))
+        assert got == run_loops(cache_layers, staleness, expire), (cache_layers, staleness, expire)
+    # without a cache only the rows that no edge reaches are spared; the caches spare more
+    bare = list(embedding_cache_hit_rate(batches, N, cache_layers=()))
+    assert sum(h for h, _, _ in got) > sum(h for h, _, _ in bare) and bare[0][2] == {}
+    # the same batch twice with the seeds' layer cached: all seeds but the one with the largest score are held
+    # (the quantile 1.0 is that score and admission is strict), so the second pass needs one seed's rows only
+    twice = list(embedding_cache_hit_rate(batches[:1] * 2, N, cache_layers=(0,), rate=1.0,
+                                          score_fn=lambda n, d: torch.arange(n, dtype=torch.float32)))
+    assert twice[0][2] == {0: 9} and twice[1][0] > twice[0][0]
