@@ -1,7 +1,7 @@
 """HistoryTrainer: the loop around the path -- sample, ``lookup_and_load``, forward, loss, backward, optimizer,
 ``update_history`` -- with the method names and attributes of the reference's trainer
 (/root/reference/hiscache/history_trainer.py:15-255: ``cxg_train_epoch`` :176-193, ``cxg_eval_epoch`` :195-227,
-``train`` :229-255).
+``train`` :229-255, ``cxg_just_load`` :144-174, ``batch_to_file`` :134-141).
 
 The reference takes its loader, its UVM store, optimizer, scheduler, loss and evaluator from two external packages
 (``cxgnndl.get_loader`` / ``cxgnndl.UVM``, ``cxgnncomp.get_optimizer`` ...).  Here they come from the dataset
@@ -263,6 +263,37 @@ class HistoryTrainer:
                  + f" total-time: {sum(self.times.values())}")
 
     @torch.no_grad()
+    def cxg_just_load(self, num_epochs=3, rate=0.9, staleness=200, score_fn=None):
+        """The hit rate of historical embeddings without a model (/root/reference/hiscache/history_trainer.py:144-174):
+        over ``num_epochs`` epochs of sampled batches, the share of every batch's layer-1 nodes that a store
+        admitting the uncached nodes under the ``rate`` quantile of random scores, and holding an admission for
+        ``staleness`` batches, would already hold.  Returns one (hit rate, nodes held) per batch and advances
+        ``glb_iter`` as the reference does (which prints them and then leaves the process)."""
+        is_cached = torch.zeros(self.table.total_num_node, dtype=torch.int32, device=self.device)
+        admitted, out = [], []
+        for _ in range(int(num_epochs)):
+            for batch in self._batches(self.splits["train"], shuffle=True):
+                nodes = batch.sub_to_full[: int(batch.num_node_in_layer[1])]
+                held = is_cached[nodes] > 0
+                out.append((float(held.sum()) / max(nodes.numel(), 1), int((is_cached > 0).sum())))
+                log.info(f"history hitrate {out[-1][0]} {out[-1][1]}")
+                rand = score_fn(nodes.numel()) if score_fn is not None else torch.randn(
+                    nodes.numel(), device=self.device, generator=self._generator)
+                check_in = nodes[(rand < torch.quantile(rand, rate)) & ~held]
+                admitted.append(check_in)
+                if len(admitted) > staleness:
+                    is_cached[admitted.pop(0)] -= 1
+                is_cached[check_in] += 1
+                self.glb_iter += 1
+        return out
+
+    @staticmethod
+    def batch_to_file(batch, filename):
+        """The batch's CSR and layer sizes as a ``torch.save`` file (history_trainer.py:134-141, without leaving
+        the process)."""
+        torch.save({"ptr": batch.ptr.cpu(), "idx": batch.idx.cpu(),
+                    "num_node_in_layer": torch.as_tensor(batch.num_node_in_layer).cpu()}, filename)
+
     def cxg_eval_epoch(self, split="val"):
         self.model.eval()
         y_preds, y_trues, losses = [], [], []

@@ -230,3 +230,47 @@ def test_example_main_trains_from_its_configuration(tmp_path, extra):
     assert len(trainer.val_metrics) == 3 and trainer.val_metrics[-1] > 0.5 and trainer.test_metrics[-1] > 0.5
     assert trainer.recorded == bool(extra) and (trainer.uvm.hot_rows is not None) == bool(extra)
     assert os.path.exists(os.path.join(tmp_path, "processed", "sorted_indices.dat"))
+
+
+def test_just_load_hit_rates_and_batch_file(tmp_path):
+    """``cxg_just_load`` (/root/reference/hiscache/history_trainer.py:144-174) against a dictionary model run over the
+    same batches (a second trainer with the same seeds draws them again); ``batch_to_file`` round trip."""
+    from hiscache import HistoryTrainer, make_config
+    rng = np.random.default_rng(83)
+    dataset(tmp_path, rng, N=3000)
+    cfg = make_config(32, 4, 32, 2, device=DEV, path=str(tmp_path))
+
+    def build():
+        return HistoryTrainer(cfg, fanout=[4, 3], batch_size=150, cache_bytes=400 * 32 * 4, seed=3)
+
+    def score(n):                                         # a fixed pseudo-random order of the positions
+        return ((torch.arange(n, device=DEV) * 7919) % 1009).to(torch.float32)
+    a, b = build(), build()
+    got = a.cxg_just_load(num_epochs=2, rate=0.8, staleness=5, score_fn=score)
+    count, window, want = {}, [], []
+    for _ in range(2):
+        for batch in b._batches(b.splits["train"], shuffle=True):
+            nodes = batch.sub_to_full[: int(batch.num_node_in_layer[1])].tolist()
+            held = [count.get(v, 0) > 0 for v in nodes]
+            want.append((sum(held) / len(nodes), sum(1 for c in count.values() if c > 0)))
+            sc = score(len(nodes))
+            thres = float(torch.quantile(sc, 0.8))
+            new = [v for v, s, h in zip(nodes, sc.tolist(), held) if s < thres and not h]
+            window.append(new)
+            if len(window) > 5:
+                for v in window.pop(0):
+                    count[v] -= 1
+            for v in new:
+                count[v] = count.get(v, 0) + 1
+    assert len(got) == 2 * 13 and a.glb_iter == 26         # 1 850 training nodes in batches of 150
+    assert [g[1] for g in got] == [w[1] for w in want]
+    np.testing.assert_allclose([g[0] for g in got], [w[0] for w in want], rtol=1e-6)
+    assert got[0] == (0.0, 0) and max(g[0] for g in got) > 0.05
+    # with the default scores it runs from the trainer's generator
+    assert len(a.cxg_just_load(num_epochs=1)) == 13
+    batch = a.sampler.sample(a.splits["train"][:100].contiguous())
+    HistoryTrainer.batch_to_file(batch, tmp_path / "batch.pt")
+    back = torch.load(tmp_path / "batch.pt", weights_only=True)
+    assert torch.equal(back["ptr"], batch.ptr.cpu()) and torch.equal(back["idx"], batch.idx.cpu())
+    assert back["num_node_in_layer"].tolist() == batch.num_node_in_layer.tolist()
+    a.close(), b.close()
