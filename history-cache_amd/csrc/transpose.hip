@@ -248,6 +248,7 @@ struct TrDims {
   int64_t R, E, n_src;               // by value (or the upper bounds when the pointers are set)
   const int64_t *pR, *pE, *pS;       // nullable, all three or none
   int32_t *overflow;                 // nullable: set to 1 when a size read on the device had to be clamped, else 0
+  int64_t *max_count;                // nullable: receives the largest number of live edges of one source
 };
 __device__ __forceinline__ void tr_dims(const TrDims &d, int64_t &R, int64_t &E, int64_t &n_src) {
   R = d.R;
@@ -366,6 +367,7 @@ __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
   const int64_t n_entries = n_src + 1;                      // ptrT has n_src + 1 entries
   const int64_t padded = (n_entries + 3) / 4 * 4;           // the counter array is zero-padded to 256 bytes
   int carry = 0;
+  int longest = 0;                                          // the lane's largest counter
   for (int64_t base = 0; base < n_entries; base += TRS_SUPER) {
     const int64_t run0 = base + (int64_t)wave * WAVE_SPAN;
     int4 c[G];
@@ -373,6 +375,7 @@ __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
     for (int g = 0; g < G; ++g) {
       const int64_t i = run0 + ((int64_t)g * HC_WAVE + lane) * 4;
       c[g] = i < padded ? *reinterpret_cast<const int4 *>(count + i) : make_int4(0, 0, 0, 0);
+      longest = max(max(longest, max(c[g].x, c[g].y)), max(c[g].z, c[g].w));
     }
     int pre[G];                                             // entries of the run in front of the lane's four
     int run = 0;
@@ -418,6 +421,17 @@ __global__ __launch_bounds__(TRS_BLOCK) void tr_small_count(
           }
         }
       }
+    }
+  }
+  if (dims.max_count != nullptr) {                          // (kernel argument: the whole block takes the branch)
+#pragma unroll
+    for (int d = HC_WAVE / 2; d > 0; d >>= 1) longest = max(longest, __shfl_xor(longest, d, HC_WAVE));
+    if (lane == 0) s_wave[wave] = longest;                  // free since the last sweep's second barrier
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int m = 0;
+      for (int w = 0; w < NW; ++w) m = max(m, s_wave[w]);
+      *dims.max_count = m;
     }
   }
 }
@@ -711,7 +725,7 @@ extern "C" int hc_build_transpose(const int64_t *ptr, const int64_t *idx, const 
     if (!workspace || workspace_bytes < S.total) return HC_EWORKSPACE;
     char *w = static_cast<char *>(workspace);
     if (reinterpret_cast<uintptr_t>(w) % 256 != 0) return HC_EWORKSPACE;
-    const TrDims dims{R, E, n_src, nullptr, nullptr, nullptr, nullptr};
+    const TrDims dims{R, E, n_src, nullptr, nullptr, nullptr, nullptr, nullptr};
     return small_launch(ptr, idx, hmap_row, hmap_src, dims, ptrT, rowT, edgeT, w, S, st);
   }
   if (bucket_sorted(E, n_src)) {
@@ -809,6 +823,15 @@ extern "C" int hc_build_transpose_dev(const int64_t *ptr, const int64_t *idx, co
                                       const int64_t *E_dev, const int64_t *n_src_dev, int64_t max_E,
                                       int64_t max_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT,
                                       int32_t *overflow, void *workspace, size_t workspace_bytes, void *stream) {
+  return hc_build_transpose_dev_deg(ptr, idx, R_dev, E_dev, n_src_dev, max_E, max_src, ptrT, rowT, edgeT, overflow,
+                                    nullptr, workspace, workspace_bytes, stream);
+}
+
+extern "C" int hc_build_transpose_dev_deg(const int64_t *ptr, const int64_t *idx, const int64_t *R_dev,
+                                          const int64_t *E_dev, const int64_t *n_src_dev, int64_t max_E,
+                                          int64_t max_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT,
+                                          int32_t *overflow, int64_t *max_in_degree, void *workspace,
+                                          size_t workspace_bytes, void *stream) {
   HC_REQUIRE(ptr && idx && R_dev && E_dev && n_src_dev && ptrT && max_E >= 0 && max_src >= 0);
   HC_REQUIRE(rowT != nullptr || max_E == 0);
   if (max_E > TR_DEV_MAX_EDGES || max_src > TR_DEV_MAX_SOURCES) return HC_EUNSUPPORTED;
@@ -816,6 +839,6 @@ extern "C" int hc_build_transpose_dev(const int64_t *ptr, const int64_t *idx, co
   if (!workspace || workspace_bytes < S.total) return HC_EWORKSPACE;
   char *w = static_cast<char *>(workspace);
   if (reinterpret_cast<uintptr_t>(w) % 256 != 0) return HC_EWORKSPACE;
-  const TrDims dims{0, max_E, max_src, R_dev, E_dev, n_src_dev, overflow};
+  const TrDims dims{0, max_E, max_src, R_dev, E_dev, n_src_dev, overflow, max_in_degree};
   return small_launch(ptr, idx, nullptr, nullptr, dims, ptrT, rowT, edgeT, w, S, static_cast<hipStream_t>(stream));
 }

@@ -88,7 +88,7 @@ class NeighborSampler:
                 out = _be.sample_layers(self.indptr, self.indices, seeds, self.fanout, rng_seed, self.node_map,
                                         emit_view=self.emit_view, view_edges=self.view_edges)
             counts_host = self._host_pool.pop() if self._host_pool else torch.empty(
-                2 * len(self.fanout) + 1, dtype=torch.int64, pin_memory=True)
+                2 * len(self.fanout) + 2, dtype=torch.int64, pin_memory=True)
             counts_host.copy_(out[3], non_blocking=True)
             done = torch.cuda.Event()
             done.record(stream)
@@ -115,14 +115,14 @@ class NeighborSampler:
         L = len(self.fanout)
         c = counts_host.tolist()
         self._host_pool.append(counts_host)
-        nnl, nel = c[: L + 1], c[L + 1:]
+        nnl, nel = c[: L + 1], c[L + 1: 2 * L + 1]
         cur = torch.cuda.current_stream(self.device)
         view = None
         if self.emit_view:
             ptrT, rowT, edgeT = out[4], out[5], out[6]
             n_e = max(nel[-1], 1)
             view = _be.BatchView(ptrT[: nnl[L] + 1], rowT[:n_e], None if edgeT is None else edgeT[:n_e],
-                                 nnl[L - 1], nnl[L], nel[-1])
+                                 nnl[L - 1], nnl[L], nel[-1], max_in_degree=c[2 * L + 1])
         if stream != cur:
             # arrays of a replay slot belong to its graph and are never handed back to the allocator
             for t in ((seeds,) if pooled else (ptr, idx, s2f, seeds)) + (() if y is None else (y,)):

@@ -58,6 +58,8 @@ _SIGNATURES = {
     "hc_transpose_dev_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
     "hc_build_transpose_dev": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p,
                                         _c_sz, _c_p]),
+    "hc_build_transpose_dev_deg": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p,
+                                            _c_p, _c_sz, _c_p]),
     "hc_aggr_bwd_workspace_bytes": (_c_sz, [_c_i64, _c_i64]),
     "hc_aggr_bwd_chunk_edges": (_c_i64, [_c_i64]),
     "hc_aggr_bwd": (_c_int, [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_i64, _c_p,
@@ -1402,15 +1404,18 @@ def sample_capacity(n_seed, fanout, num_nodes):
 
 
 def build_transpose_dev(ptr, idx, rows_dev, edges_dev, nodes_dev, max_edges, max_nodes, want_edges=False,
-                        overflow=None):
+                        overflow=None, max_in_degree=None):
     """The transposed view of a block whose sizes are still on the device (one-element int64 views
     ``rows_dev``, ``edges_dev``, ``nodes_dev``, e.g. slices of the sampler's ``counts``): returns
     (ptrT, rowT, edgeT) at the capacities ``max_nodes + 1`` / ``max_edges``; nothing is read back.
     ``overflow`` (one int32 on the device, optional) is set to 1 when a size exceeded its capacity and the
-    view is that of the truncated block, else to 0."""
+    view is that of the truncated block, else to 0.  ``max_in_degree`` (a one-element int64 view on the device,
+    optional) receives the largest number of edges one source has in the view."""
     lib = load_library()
     _dev(ptr, "ptr", torch.int64)
     _dev(idx, "idx", torch.int64)
+    if max_in_degree is not None and _dev(max_in_degree, "max_in_degree", torch.int64).numel() < 1:
+        raise ValueError("max_in_degree is empty")
     for t, name in ((rows_dev, "rows_dev"), (edges_dev, "edges_dev"), (nodes_dev, "nodes_dev")):
         _dev(t, name, torch.int64)
         if t.numel() < 1:
@@ -1426,20 +1431,21 @@ def build_transpose_dev(ptr, idx, rows_dev, edges_dev, nodes_dev, max_edges, max
     rowT = torch.empty(max(max_edges, 1), dtype=torch.int32, device=dev)
     edgeT = torch.empty(max(max_edges, 1), dtype=torch.int32, device=dev) if want_edges else None
     ws = _workspace(nbytes, dev)
-    rc = lib.hc_build_transpose_dev(_ptr(ptr), _ptr(idx), _ptr(rows_dev), _ptr(edges_dev), _ptr(nodes_dev),
-                                    max_edges, max_nodes, _ptr(ptrT), _ptr(rowT), _ptr(edgeT),
-                                    _ptr(None if overflow is None else _dev(overflow, "overflow", torch.int32)),
-                                    _ptr(ws), ws.numel(), _stream())
-    _check(rc, "hc_build_transpose_dev")
+    rc = lib.hc_build_transpose_dev_deg(_ptr(ptr), _ptr(idx), _ptr(rows_dev), _ptr(edges_dev), _ptr(nodes_dev),
+                                        max_edges, max_nodes, _ptr(ptrT), _ptr(rowT), _ptr(edgeT),
+                                        _ptr(None if overflow is None else _dev(overflow, "overflow", torch.int32)),
+                                        _ptr(max_in_degree), _ptr(ws), ws.numel(), _stream())
+    _check(rc, "hc_build_transpose_dev_deg")
     return ptrT, rowT, edgeT
 
 
 def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map, emit_view=False, view_edges=False,
                   rng_seed_at=None):
     """Layered neighbour sampling without replacement.  Returns (ptr, idx, sub_to_full, counts) as
-    device tensors at their capacity; ``counts`` (int64[2L+1] on the device) holds the node count
+    device tensors at their capacity; ``counts`` (int64[2L+2] on the device) holds the node count
     within k hops for k = 0..L and then the cumulative edge count after every hop, so the caller
-    slices ptr[:counts[L-1]+1], idx[:counts[2L]], sub_to_full[:counts[L]] once it has read them.
+    slices ptr[:counts[L-1]+1], idx[:counts[2L]], sub_to_full[:counts[L]] once it has read them
+    (the last entry is written with ``emit_view`` only: the largest in-degree of a source in the view).
     ``seeds`` must be distinct valid node ids; ``node_map`` comes from ``sample_map`` and is left
     all-unseen again.  Stands where the reference's external loader does
     (/root/reference/hiscache/history_trainer.py:19,26).  ``emit_view=True`` appends (ptrT, rowT, edgeT):
@@ -1466,7 +1472,7 @@ def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map, emit_view=
     ptr = torch.empty(rows + 1, dtype=torch.int64, device=dev)
     idx = torch.empty(max(edges, 1), dtype=torch.int64, device=dev)
     s2f = torch.empty(max(nodes, 1), dtype=torch.int64, device=dev)
-    counts = torch.empty(2 * L + 1, dtype=torch.int64, device=dev)
+    counts = torch.empty(2 * L + 2, dtype=torch.int64, device=dev)     # (the last entry: see emit_view)
     ws_bytes = int(lib.hc_sample_workspace_bytes(n_seed, ctypes.cast(fan, _c_p), L, N))
     if ws_bytes == 0:
         raise ValueError("unsupported fanout / batch size")
@@ -1485,7 +1491,8 @@ def sample_layers(indptr, indices, seeds, fanout, rng_seed, node_map, emit_view=
     _check(rc, "hc_sample_layers")
     if emit_view:
         ptrT, rowT, edgeT = build_transpose_dev(ptr, idx, counts[L - 1:L], counts[2 * L:2 * L + 1],
-                                                counts[L:L + 1], edges, nodes, want_edges=view_edges)
+                                                counts[L:L + 1], edges, nodes, want_edges=view_edges,
+                                                max_in_degree=counts[2 * L + 1:])
         return ptr, idx, s2f, counts, ptrT, rowT, edgeT
     return ptr, idx, s2f, counts
 

@@ -152,6 +152,17 @@ int hc_build_transpose_dev(const int64_t *ptr, const int64_t *idx, const int64_t
                            const int64_t *E_dev, const int64_t *n_src_dev, int64_t max_E,
                            int64_t max_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT,
                            int32_t *overflow, void *workspace, size_t workspace_bytes, void *stream);
+/* hc_build_transpose_dev_deg: the same call with one more output, *max_in_degree
+ * (one int64 in device memory, nullable): the largest number of edges that one
+ * source has in the view, found by the block that scans the counters.  A caller
+ * that reads it back with the sizes knows whether the batch holds a source above
+ * hc_aggr_bwd_chunk_edges and may then call hc_aggr_bwd_batch_view without
+ * workspace, which runs it without its hub blocks and its second launch. */
+int hc_build_transpose_dev_deg(const int64_t *ptr, const int64_t *idx, const int64_t *R_dev,
+                               const int64_t *E_dev, const int64_t *n_src_dev, int64_t max_E,
+                               int64_t max_src, int64_t *ptrT, int32_t *rowT, int32_t *edgeT,
+                               int32_t *overflow, int64_t *max_in_degree, void *workspace,
+                               size_t workspace_bytes, void *stream);
 
 /* ---------------------------------------------------------------- aggregation backward
  * Replaces AggrHistoryFunction::backward / AggrHistoryEdgeValueFunction::backward

@@ -74,6 +74,7 @@ def test_argument_errors_are_status_codes():
     assert lib.hc_build_transpose_dev(p, p, p, p, p, big, 10, p, p, null, null, p, 1 << 40, null) == 5
     assert lib.hc_build_transpose_dev(p, p, p, p, p, 1000, 100, p, p, null, null, null, 0, null) == 4
     assert lib.hc_build_transpose_dev(p, p, null, p, p, 1000, 100, p, p, null, null, p, need, null) == 1
+    assert lib.hc_build_transpose_dev_deg(p, p, p, p, p, 1000, 100, p, p, null, null, null, null, 0, null) == 4
     assert lib.hc_aggr_bwd_batch_view_typed(p, p, p, p, p, 8, 3, null, p, p, 4, 100, 4, null) == 5
     assert lib.hc_aggr_bwd_batch_view_typed(p, p, p, p, null, 8, 3, null, p, p, 4, 64, 4, null) == 1
     assert lib.hc_aggr_bwd_batch_view_typed(p, p, p, p, p, 8, 0, null, p, p, 4, 64, 4, null) == 1

@@ -157,9 +157,14 @@ def test_view_with_sizes_on_the_device(be, R, n_src, max_deg, hub_edges, slack):
     sizes = T(np.array([R, E, n_src], np.int64))
     want_ptrT, want_rowT, want_edgeT = _stable_view(ptr, idx, R, n_src)
     flag = torch.full((1,), 7, dtype=torch.int32, device=DEV)
+    longest = torch.full((2,), -5, dtype=torch.int64, device=DEV)
     for want_edges in (False, True):
         ptrT, rowT, edgeT = be.build_transpose_dev(T(ptr), T(idx_cap), sizes[0:1], sizes[1:2], sizes[2:3], max_E,
-                                                   max_src, want_edges=want_edges, overflow=flag)
+                                                   max_src, want_edges=want_edges, overflow=flag,
+                                                   max_in_degree=longest[:1] if want_edges else None)
+        # the largest in-degree, on request (one word: the next one stays as it was)
+        assert longest.tolist() == ([int(np.bincount(idx, minlength=1).max()) if E else 0, -5] if want_edges
+                                    else [-5, -5])
         np.testing.assert_array_equal(ptrT[: n_src + 1].cpu().numpy(), want_ptrT)
         np.testing.assert_array_equal(rowT[:E].cpu().numpy(), want_rowT)
         if want_edges:
@@ -215,6 +220,7 @@ def test_sampler_emits_the_view_with_the_batch(be, orc, fanout, n_seed):
         R, n_all = int(b.num_node_in_layer[L - 1]), int(b.num_node_in_layer[L])
         v = b.view
         assert (v.rows, v.n_src, v.num_edge) == (R, n_all, b.idx.numel())
+        assert v.max_in_degree == int(torch.bincount(b.idx).max())     # read back with the batch's sizes
         want_ptrT, want_rowT, _ = _stable_view(b.ptr.cpu().numpy(), b.idx.cpu().numpy(), R, n_all)
         np.testing.assert_array_equal(v.ptrT.cpu().numpy(), want_ptrT)
         np.testing.assert_array_equal(v.rowT[: v.num_edge].cpu().numpy(), want_rowT)

@@ -343,7 +343,7 @@ def test_replayed_relational_iterations_equal_the_padded_ones():
     rec = twins["recorded"][3]
     shapes = rec.shapes()
     assert rec.replays >= len(order) // 3, shapes
-    assert all(k[1] == 2 and k[2] >= 0 for k, v in shapes.items() if v[2])     # view with edge slots, rows read ahead
+    assert all(k[1] % 10 == 2 and k[2] >= 0 for k, v in shapes.items() if v[2])     # view with edge slots, rows read ahead
     assert int((twins["recorded"][0].full2slot != -1).sum()) > cached.numel()   # rows were admitted
 
 
