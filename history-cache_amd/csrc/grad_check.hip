@@ -885,11 +885,12 @@ extern "C" int hc_evict(const int64_t *sub2slot, const float *score, const float
 // Admission threshold as a quantile of the scores: the two order statistics that
 // torch.quantile's linear interpolation reads (/root/reference/hiscache/history_cache.py:211,
 // history_table.py:173), found by a radix select instead of a sort, and the interpolation in
-// separately rounded fp32 steps.  One block; four 8-bit passes over keys that order like the
-// floats (sign flipped for non-negative values, all bits for negative ones) find the lower
-// statistic, one more pass the upper one where it is another key.  Up to 16 384 scores are
-// read once and kept in registers (a sampled batch's 1-hop nodes are a few thousand); up to
-// QT_MAX_N are read again in every pass.
+// separately rounded fp32 steps.  One block, over keys that order like the floats (sign flipped
+// for non-negative values, all bits for negative ones): the bits that all keys share are skipped,
+// 8-bit digit passes below them narrow the keys down to at most 128, which are ranked against
+// each other; that finds the lower statistic, one more pass the upper one where it is another
+// key.  Up to 16 384 scores are read once and kept in registers (a sampled batch's 1-hop nodes
+// are a few thousand); up to QT_MAX_N are read again in every pass.
 // ---------------------------------------------------------------------------------------
 namespace {
 
@@ -907,35 +908,99 @@ __device__ __forceinline__ float qt_value(uint32_t k) {
 
 constexpr int QT_WAVES = QT_BLOCK / HC_WAVE;
 constexpr int QT_REG = 16;   // keys a thread keeps in registers: up to QT_BLOCK * QT_REG scores are read once
+constexpr int QT_CAND = 128;   // this many keys or fewer are ranked against each other (m * m comparisons) instead of counted by digit
 
 struct QtShared {
   int hist[QT_WAVES][256];   // one histogram per wave: lanes of different waves never meet on a counter
   int total[256];
   int pick[3];               // the bin that holds the rank, the keys in front of it, the keys inside it
   uint32_t next;             // smallest key above the selected one
+  uint32_t range[2][QT_WAVES];   // the waves' smallest and largest keys
+  alignas(16) uint32_t cand[QT_CAND];    // the keys that are left, padded with 0xffffffff (no key: NaN ends the kernel earlier)
+  int n_cand;
+  uint32_t result[3];        // the selected key, the rank's position among the keys equal to it, their number
 };
+
+// f(key) for every key of the thread: from its registers (REG) or from `score`.
+template <bool REG, class F>
+__device__ __forceinline__ void qt_for_each(const float *__restrict__ score, int64_t n, const uint32_t (&rk)[QT_REG],
+                                            int nk, F f) {
+  if constexpr (REG) {
+#pragma unroll
+    for (int j = 0; j < QT_REG; ++j)
+      if (j < nk) f(rk[j]);
+  } else {
+    // eight loads issued together (a load per iteration would wait out the memory latency every time)
+    constexpr int U = 8;
+    for (int64_t base = threadIdx.x; base < n; base += (int64_t)QT_BLOCK * U) {
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t i = base + (int64_t)u * QT_BLOCK;
+        v[u] = score[i < n ? i : n - 1];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (base + (int64_t)u * QT_BLOCK < n) f(qt_key(v[u]));
+    }
+  }
+}
 
 // The key of rank k (0-based) among the n scores; every thread returns it.  REG: the keys sit in the
 // thread's registers (rk[0, nk)), otherwise they are read from `score` in every pass.  *k_in_bin and *n_equal
 // return the rank's position among the keys equal to the result and how many those are.
+// The smallest and the largest key fix the bits that all keys share (scores of one batch lie within a few
+// octaves: a pass over the leading byte would tell nothing apart); digit passes of up to 8 bits below them go on
+// only while more than QT_CAND keys are left, then the rest is ranked directly: a thread per key counts the
+// smaller and the equal ones.  Ten thousand scores take one digit pass instead of four.
 template <bool REG>
 __device__ uint32_t qt_select(const float *__restrict__ score, int64_t n, const uint32_t (&rk)[QT_REG], int nk,
                               int64_t k, QtShared &sh, int64_t *k_in_bin, int *n_equal) {
-  uint32_t prefix = 0u, mask = 0u;
   const int wave = (int)(threadIdx.x / HC_WAVE);
-  for (int shift = 24; shift >= 0; shift -= 8) {
+  const int lane = hc_lane();
+  uint32_t mn = 0xffffffffu, mx = 0u;
+  qt_for_each<REG>(score, n, rk, nk, [&](uint32_t key) {
+    mn = key < mn ? key : mn;
+    mx = key > mx ? key : mx;
+  });
+#pragma unroll
+  for (int d = HC_WAVE / 2; d > 0; d >>= 1) {
+    const uint32_t a = (uint32_t)__shfl_xor((int)mn, d, HC_WAVE), b = (uint32_t)__shfl_xor((int)mx, d, HC_WAVE);
+    mn = a < mn ? a : mn;
+    mx = b > mx ? b : mx;
+  }
+  if (lane == 0) {
+    sh.range[0][wave] = mn;
+    sh.range[1][wave] = mx;
+  }
+  if (threadIdx.x < QT_CAND) sh.cand[threadIdx.x] = 0xffffffffu;
+  if (threadIdx.x == 0) sh.n_cand = 0;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < QT_WAVES; ++w) {
+    const uint32_t a = sh.range[0][w], b = sh.range[1][w];
+    mn = a < mn ? a : mn;
+    mx = b > mx ? b : mx;
+  }
+  if (mn == mx) {                        // block-uniform: every score is the same
+    *k_in_bin = k;
+    *n_equal = (int)n;
+    return mn;
+  }
+  const int top = 31 - __clz((int)(mn ^ mx));              // the highest bit in which two keys differ
+  uint32_t mask = top == 31 ? 0u : ~((2u << top) - 1u);   // the bits above it are the same for all
+  uint32_t prefix = mn & mask;
+  int remaining = top + 1;                                 // undecided low bits
+  int64_t left = n;                                        // keys that agree with the prefix
+  while (remaining > 0 && left > QT_CAND) {                // block-uniform
+    const int bits = remaining < 8 ? remaining : 8;
+    const int shift = remaining - bits;
+    const uint32_t digit_mask = (1u << bits) - 1u;
     for (int b = threadIdx.x; b < QT_WAVES * 256; b += QT_BLOCK) (&sh.hist[0][0])[b] = 0;
     __syncthreads();
-    if constexpr (REG) {
-#pragma unroll
-      for (int j = 0; j < QT_REG; ++j)
-        if (j < nk && (rk[j] & mask) == prefix) atomicAdd(&sh.hist[wave][(rk[j] >> shift) & 0xffu], 1);
-    } else {
-      for (int64_t i = threadIdx.x; i < n; i += QT_BLOCK) {
-        const uint32_t key = qt_key(score[i]);
-        if ((key & mask) == prefix) atomicAdd(&sh.hist[wave][(key >> shift) & 0xffu], 1);
-      }
-    }
+    qt_for_each<REG>(score, n, rk, nk, [&](uint32_t key) {
+      if ((key & mask) == prefix) atomicAdd(&sh.hist[wave][(key >> shift) & digit_mask], 1);
+    });
     __syncthreads();
     if (threadIdx.x < 256) {
       int t = 0;
@@ -958,25 +1023,58 @@ __device__ uint32_t qt_select(const float *__restrict__ score, int64_t n, const 
       const unsigned long long reached = __ballot((int64_t)x > k);
       const int owner = reached != 0ull ? __builtin_ctzll(reached) : HC_WAVE - 1;
       if (l == owner) {
-        int before = x - mine, b = 0;
-        for (; b < 3; ++b) {
-          if ((int64_t)before + c[b] > k) break;
-          before += c[b];
-        }
+        // (indices known at compile time: an array indexed by a variable lives in scratch memory, and a kernel
+        // with scratch memory starts more slowly)
+        int before = x - mine, b = 0, inside = c[0];
+#pragma unroll
+        for (int t = 0; t < 3; ++t)
+          if (b == t && (int64_t)before + c[t] <= k) {
+            before += c[t];
+            b = t + 1;
+            inside = c[t + 1];
+          }
         sh.pick[0] = 4 * l + b;
         sh.pick[1] = before;           // at most n < 2^31
-        sh.pick[2] = c[b];
+        sh.pick[2] = inside;
       }
     }
     __syncthreads();
     prefix |= (uint32_t)sh.pick[0] << shift;
-    mask |= 0xffu << shift;
+    mask |= digit_mask << shift;
     k -= sh.pick[1];
-    *n_equal = sh.pick[2];
+    left = sh.pick[2];
+    remaining = shift;
     __syncthreads();
   }
-  *k_in_bin = k;
-  return prefix;
+  if (remaining == 0) {                  // every bit decided: the keys that are left are equal
+    *k_in_bin = k;
+    *n_equal = (int)left;
+    return prefix;
+  }
+  // at most QT_CAND keys left: side by side in LDS (in any order), every one ranked by its own thread
+  qt_for_each<REG>(score, n, rk, nk, [&](uint32_t key) {
+    if ((key & mask) == prefix) sh.cand[atomicAdd(&sh.n_cand, 1)] = key;
+  });
+  __syncthreads();
+  const int m = sh.n_cand;               // == left
+  if ((int)threadIdx.x < m) {
+    const uint32_t c = sh.cand[threadIdx.x];
+    int less = 0, equal = 0;
+    for (int j = 0; j < m; j += 4) {     // (the padding ranks above every key)
+      const uint4 x = *reinterpret_cast<const uint4 *>(&sh.cand[j]);
+      less += (int)(x.x < c) + (int)(x.y < c) + (int)(x.z < c) + (int)(x.w < c);
+      equal += (int)(x.x == c) + (int)(x.y == c) + (int)(x.z == c) + (int)(x.w == c);
+    }
+    if ((int64_t)less <= k && k < (int64_t)less + equal) {   // threads with equal keys write the same words
+      sh.result[0] = c;
+      sh.result[1] = (uint32_t)(k - less);
+      sh.result[2] = (uint32_t)equal;
+    }
+  }
+  __syncthreads();
+  *k_in_bin = (int64_t)sh.result[1];
+  *n_equal = (int)sh.result[2];
+  return sh.result[0];
 }
 
 // The smallest key above `key`; every thread returns it (0xffffffff when there is none).
@@ -986,16 +1084,9 @@ __device__ uint32_t qt_next_above(const float *__restrict__ score, int64_t n, co
   if (threadIdx.x == 0) sh.next = 0xffffffffu;
   __syncthreads();
   uint32_t m = 0xffffffffu;
-  if constexpr (REG) {
-#pragma unroll
-    for (int j = 0; j < QT_REG; ++j)
-      if (j < nk && rk[j] > key && rk[j] < m) m = rk[j];
-  } else {
-    for (int64_t i = threadIdx.x; i < n; i += QT_BLOCK) {
-      const uint32_t x = qt_key(score[i]);
-      if (x > key && x < m) m = x;
-    }
-  }
+  qt_for_each<REG>(score, n, rk, nk, [&](uint32_t x) {
+    if (x > key && x < m) m = x;
+  });
 #pragma unroll
   for (int d = HC_WAVE / 2; d > 0; d >>= 1) {
     const uint32_t y = (uint32_t)__shfl_xor((int)m, d, HC_WAVE);
@@ -1015,19 +1106,28 @@ __device__ __forceinline__ void qt_block(const float *__restrict__ score, int64_
   int nk = 0;
   int nan_seen = 0;                    // torch.quantile answers NaN when any score is NaN: so does this kernel
   if constexpr (REG) {
+    // every load issued before the first use (behind a bounds branch each would wait for the one in front:
+    // 0.5 us apiece); a load beyond the scores reads the last one again and is dropped
+    float v[QT_REG];
+#pragma unroll
+    for (int j = 0; j < QT_REG; ++j) {
+      const int64_t i = (int64_t)j * QT_BLOCK + threadIdx.x;
+      v[j] = score[i < n ? i : n - 1];
+    }
 #pragma unroll
     for (int j = 0; j < QT_REG; ++j) {
       const int64_t i = (int64_t)j * QT_BLOCK + threadIdx.x;
       rk[j] = 0u;
       if (i < n) {
-        rk[j] = qt_key(score[i]);
+        rk[j] = qt_key(v[j]);
         nk = j + 1;
         if (rk[j] == 0xffffffffu) nan_seen = 1;
       }
     }
   } else {
-    for (int64_t i = threadIdx.x; i < n; i += QT_BLOCK)
-      if (score[i] != score[i]) nan_seen = 1;
+    qt_for_each<false>(score, n, rk, 0, [&](uint32_t key) {
+      if (key == 0xffffffffu) nan_seen = 1;
+    });
   }
   nan_seen = __syncthreads_or(nan_seen);
   if (nan_seen) {                      // block-uniform
@@ -1047,7 +1147,7 @@ __device__ __forceinline__ void qt_block(const float *__restrict__ score, int64_
 }
 
 template <bool REG>
-__global__ __launch_bounds__(QT_BLOCK) void quantile_kernel(const float *__restrict__ score, int64_t n, int64_t lo,
+__global__ __launch_bounds__(QT_BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) void quantile_kernel(const float *__restrict__ score, int64_t n, int64_t lo,
                                                              int64_t hi, float w, float one_minus_w,
                                                              float *__restrict__ out) {
   __shared__ QtShared sh;
@@ -1058,7 +1158,7 @@ __global__ __launch_bounds__(QT_BLOCK) void quantile_kernel(const float *__restr
 // out here as the host works it out: pos = fp32(rate) * fp32(n - 1), lo = floor(pos), w = pos - lo, each
 // step rounded to fp32.
 template <bool REG>
-__global__ __launch_bounds__(QT_BLOCK) void quantile_kernel_dev(const float *__restrict__ score,
+__global__ __launch_bounds__(QT_BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) void quantile_kernel_dev(const float *__restrict__ score,
                                                                  const int64_t *__restrict__ n_dev, int64_t n_max,
                                                                  float rate, float *__restrict__ out) {
   __shared__ QtShared sh;
@@ -1110,13 +1210,17 @@ __device__ QlPick ql_replay(const uint32_t *__restrict__ hist, int passes, int64
     const int owner = reached != 0ull ? __builtin_ctzll(reached) : HC_WAVE - 1;
     long long before = x - mine;
     int b = 0;
-    for (; b < 3; ++b) {
-      if (before + (long long)c[b] > (long long)r.k) break;
-      before += c[b];
-    }
+    auto in_bin = c[0];                  // (indices known at compile time keep c out of scratch memory)
+#pragma unroll
+    for (int t = 0; t < 3; ++t)
+      if (b == t && before + (long long)c[t] <= (long long)r.k) {
+        before += c[t];
+        b = t + 1;
+        in_bin = c[t + 1];
+      }
     const int bin = __shfl(4 * lane + b, owner, HC_WAVE);
     const long long front = __shfl(before, owner, HC_WAVE);
-    const uint32_t inside = (uint32_t)__shfl((int)c[b], owner, HC_WAVE);
+    const uint32_t inside = (uint32_t)__shfl((int)in_bin, owner, HC_WAVE);
     r.prefix |= (uint32_t)bin << (24 - 8 * p);
     r.k -= front;
     r.n_equal = inside;

@@ -192,7 +192,7 @@ def test_small_helpers(be, orc):
     np.testing.assert_array_equal(be.lookup(T(m), T(ids), 3).cpu().numpy(), m[ids + 3])
 
 
-@pytest.mark.parametrize("n", [1, 2, 3, 257, 5800, 1 << 15, (1 << 15) + 1, 1 << 17, (1 << 17) + 3, 200_003, 2_000_000, 5_000_001])
+@pytest.mark.parametrize("n", [1, 2, 3, 257, 1024, 1025, 5800, 10_000, 1 << 14, (1 << 14) + 1, 1 << 15, (1 << 15) + 1, 1 << 17, (1 << 17) + 3, 200_003, 2_000_000, 5_000_001])
 def test_quantile_threshold_by_selection_equals_the_sort(n):
     """hc_quantile_threshold_ws (radix select of the two order statistics + the interpolation: one launch by one
     block up to 2^17 scores, the whole chip above) gives the bits of the sorted spelling -- which is
@@ -201,6 +201,11 @@ def test_quantile_threshold_by_selection_equals_the_sort(n):
     rng = np.random.default_rng(n)
     cases = [rng.standard_normal(n), np.abs(rng.standard_normal(n)) * np.exp(rng.normal(-3, 1.5, size=n)),
              rng.integers(0, 4, size=n).astype(np.float64), np.full(n, 0.25)]
+    # scores that share most of their bits: two neighbouring floats, and a range of 2^13 and of 2^5 neighbours
+    one = np.float32(1.0)
+    cases.append(np.where(rng.random(n) < 0.3, one, np.nextafter(one, np.float32(2))).astype(np.float32))
+    for span in (1 << 13, 1 << 5):
+        cases.append((one.view(np.uint32) + rng.integers(0, span, size=n).astype(np.uint32)).view(np.float32))
     if n > 3:
         wild = rng.standard_normal(n)
         wild[:2] = [np.inf, -np.inf]
