@@ -901,7 +901,8 @@ def run_c3(args, with_batched=True):
     if args.prefetch:
         # the read-ahead only runs beside the compute when the compute is on a stream of its own: the
         # default stream and the read's CU-limited stream wait for each other
-        compute = torch.cuda.Stream()
+        # of a few streams, the one that the reads slow down least (and on another hardware queue than the sampler's)
+        compute = store.quiet_stream(apart_from=[sampled["sampler"].stream()] if args.with_sampler else [])
         compute.wait_stream(torch.cuda.current_stream())
         torch.cuda.set_stream(compute)
     for _ in range(args.warmup):
@@ -1034,7 +1035,7 @@ def run_c5(args):
         ev["update"](lambda: cache.update_history(b, state["it"]))
 
     if args.prefetch:                 # see run_c3: the read-ahead needs the compute on a stream of its own
-        compute = torch.cuda.Stream()
+        compute = store.quiet_stream()
         compute.wait_stream(torch.cuda.current_stream())
         torch.cuda.set_stream(compute)
     for _ in range(args.warmup):

@@ -130,6 +130,46 @@ class PinnedFeatureStore:
     def join(self, event):
         torch.cuda.current_stream(self.device).wait_event(event)
 
+    def quiet_stream(self, candidates=4, rows=60_000, kernels=24, apart_from=()):
+        """A stream (default priority) for the work that runs beside ``prefetch``'s reads, chosen by measurement.
+        Which hardware queue a stream shares decides how much a host-link read on the read-ahead stream slows the
+        kernels that start beside it: about 2x on most queues, 5 - 30x on an unlucky one (a 0.9 ms iteration then
+        takes 2.2 ms), and a program cannot ask which it got.  So ``candidates`` streams are tried in turn: ``kernels``
+        small launches are timed on each while ``rows`` random rows are being read, and the one that finishes them
+        soonest is returned.  ``apart_from``: streams (the sampler's, say) whose hardware queue the result must not
+        share either.  A few milliseconds, once; without a read-ahead stream of limited width only ``apart_from``
+        is looked at."""
+        apart_from = [torch.cuda.current_stream(self.device)] + list(apart_from)
+        if self.prefetch_cus <= 0 or self.buffer.is_cuda:
+            return _be.stream_apart_from(apart_from, self.device)
+        if self._prefetch_side is None:
+            self._prefetch_side = self._make_prefetch_stream()
+        side, cur = self._prefetch_side, torch.cuda.current_stream(self.device)
+        n = int(self.buffer.shape[0])
+        rows = max(1, min(int(rows), n))
+        ids = torch.randint(0, n, (rows,), device=self.device)
+        out = torch.empty((rows, self.buffer.shape[1]), dtype=self.out_dtype, device=self.device)
+        small = torch.zeros(1 << 16, device=self.device)
+        best, best_ms = None, None
+        for _ in range(max(1, int(candidates))):
+            cand = _be.stream_apart_from(apart_from, self.device)
+            t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize(self.device)
+            cand.wait_stream(cur)
+            side.wait_stream(cur)
+            _be.gather_rows(self.buffer, self._host_ids(ids), out=out, stream=side)
+            with torch.cuda.stream(cand):
+                t0.record()
+                for _ in range(int(kernels)):
+                    small.add_(1.0)
+                t1.record()
+            torch.cuda.synchronize(self.device)
+            ms = t0.elapsed_time(t1)
+            if best_ms is None or ms < best_ms:
+                best, best_ms = cand, ms
+        self.quiet_stream_ms = best_ms
+        return best
+
     def prefetch(self, ids, mask=None, out=None):
         """Start reading the rows of ``ids`` (all of them, or those flagged by ``mask``: the caller's guess
         of which will be needed) on a side stream (default priority) now, so that the host-link read

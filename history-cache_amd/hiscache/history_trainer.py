@@ -76,7 +76,7 @@ class HistoryTrainer:
         self.uvm = ds.feature_store(device=self.device, in_device_memory=features_in_device_memory,
                                     hot_rows=hot_rows, prefetch_cus=16 if self.read_ahead else 0,
                                     out_dtype=torch.float16 if ds.feature_dtype == np.float16 else None)
-        self._compute = torch.cuda.Stream(device=self.device) if self.read_ahead else None   # default priority
+        self._compute = None
         if ring_rows:
             self.table = RingHistoryCache(self.uvm, ds.num_nodes, config.dl.dataset.feature_dim,
                                           config.train.model.hidden_dim, capacity=int(ring_rows),
@@ -96,6 +96,12 @@ class HistoryTrainer:
             raise ValueError("replay_slots: at least as many as batches are alive at once (2, with the read-ahead 3)")
         self.sampler = ds.sampler(list(fanout), device=self.device, seed=seed, emit_view=True,
                                   view_edges=isinstance(self.model, HistoryRGCN), replay_slots=replay_slots)
+        if self.read_ahead:
+            # the stream the epoch runs on beside the read-ahead: of a few, the one that the reads slow down least,
+            # and on another hardware queue than the sampler's
+            pick = getattr(self.uvm, "quiet_stream", None)
+            self._compute = (pick(apart_from=[self.sampler.stream()]) if pick is not None
+                             else torch.cuda.Stream(device=self.device))                     # default priority
         self.splits = {"train": torch.from_numpy(np.array(ds.train_idx())).to(self.device)}
         for split, key in (("val", "valid"), ("test", "test")):
             if ds.has(key):

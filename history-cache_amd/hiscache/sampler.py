@@ -75,9 +75,7 @@ class NeighborSampler:
         self.batches += 1
         cur = torch.cuda.current_stream(self.device)
         if stream is None:
-            if self._stream is None:
-                self._stream = torch.cuda.Stream(device=self.device)   # default priority
-            stream = self._stream
+            stream = self.stream()
         if stream != cur:
             stream.wait_stream(cur)                                    # seeds may have been produced there
         slot = self._replay_slot(seeds)
@@ -96,6 +94,13 @@ class NeighborSampler:
         if slot is not None:
             slot.done = done
         return _PendingBatch(self, out, counts_host, done, seeds, y, stream, pooled=slot is not None)
+
+    def stream(self):
+        """The sampler's side stream (default priority), made on first use: one that does not share a hardware
+        queue with the stream that is current then, or sampling ahead would take turns with the training on it."""
+        if self._stream is None:
+            self._stream = _be.stream_apart_from([torch.cuda.current_stream(self.device)], self.device)
+        return self._stream
 
     def _replay_slot(self, seeds):
         if not self.replay_slots:

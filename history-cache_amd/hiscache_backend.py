@@ -1003,6 +1003,43 @@ def _forget_stream(handle):
             del table[key]
 
 
+def streams_share_queue(a, b, device=None, chain=24):
+    """Do the torch streams ``a`` and ``b`` share a hardware queue?  Found by measurement: a chain of fills is queued
+    on ``b``, then one small launch on ``a``; on a queue of its own that launch is done long before the chain is.
+    The runtime hands its streams a few hardware queues (four by default) in the order of their first use, so two
+    streams that a program means to run side by side may turn out to take turns, and there is no call that tells."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    if a.cuda_stream == b.cuda_stream:
+        return True
+    big = torch.empty(1 << 24, device=device)                 # 64 MB: about 15 us per fill
+    small = torch.zeros(256, device=device)
+    torch.cuda.synchronize(device)
+    b0, b1, a1 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+    with torch.cuda.stream(b):
+        b0.record()
+        for _ in range(int(chain)):
+            big.fill_(1.0)
+        b1.record()
+    with torch.cuda.stream(a):
+        small.add_(1.0)
+        a1.record()
+    torch.cuda.synchronize(device)
+    return b0.elapsed_time(a1) >= 0.9 * b0.elapsed_time(b1)
+
+
+def stream_apart_from(others, device=None, candidates=8):
+    """A torch stream (default priority) that shares its hardware queue with none of ``others`` (see
+    ``streams_share_queue``): up to ``candidates`` new streams are tried, the last one is returned if none passes.
+    For the few long-lived streams of a training loop (the sampler's, the iteration's), made once."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    cand = None
+    for _ in range(max(1, int(candidates))):
+        cand = torch.cuda.Stream(device=device)
+        if not any(streams_share_queue(cand, o, device) for o in others):
+            break
+    return cand
+
+
 def release_cu_limited_stream(stream):
     """Give a stream made by ``cu_limited_stream`` back before the interpreter exits: waits for its work,
     destroys it and drops the scratch this module kept for it.  The torch wrapper must not be used afterwards.
