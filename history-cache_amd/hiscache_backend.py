@@ -1003,7 +1003,7 @@ def _forget_stream(handle):
             del table[key]
 
 
-def streams_share_queue(a, b, device=None, chain=24):
+def streams_share_queue(a, b, device=None, chain=16):
     """Do the torch streams ``a`` and ``b`` share a hardware queue?  Found by measurement: a chain of fills is queued
     on ``b``, then one small launch on ``a``; on a queue of its own that launch is done long before the chain is.
     The runtime hands its streams a few hardware queues (four by default) in the order of their first use, so two
@@ -1011,7 +1011,9 @@ def streams_share_queue(a, b, device=None, chain=24):
     device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
     if a.cuda_stream == b.cuda_stream:
         return True
-    big = torch.empty(1 << 24, device=device)                 # 64 MB: about 15 us per fill
+    # 256 MB: about 60 us per fill, a millisecond in all -- several times what the host needs to queue the chain,
+    # a tracer's overhead included (were the chain over before the small launch is queued, the answer would be "yes")
+    big = torch.empty(1 << 26, device=device)
     small = torch.zeros(256, device=device)
     torch.cuda.synchronize(device)
     b0, b1, a1 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
