@@ -325,7 +325,7 @@ class HistoryCache:
         sub2feat = _be.lookup(self.full2embed, sub_to_full, self.total_num_node)
         used = _be.count_history_reconstruct(batch.ptr, batch.idx, sub2embed, sub_to_full.shape[0],
                                              batch.y.shape[0], num_layer)
-        mask = torch.logical_and(used[0], sub2feat == -1)
+        _, mask = _be.load_mask(used[0], sub2feat)          # used & (sub2feat == -1), one launch
         # ``out`` (recorded iterations): the rows go straight into the array the recording reads them from
         batch.prefetched_x = start(sub_to_full, mask) if out is None else start(sub_to_full, mask, out=out)
 
