@@ -1584,6 +1584,12 @@ def main():
             r3_args.recorded = True
             rh_args = argparse.Namespace(**vars(hb_args))
             rh_args.recorded = True
+            # c3_features_in_hbm(_recorded): the configuration's own batches with the feature matrix in device memory
+            # beside the table (57 + 57 GB for papers100M: what 288 GB are for) -- no host link in the iteration
+            fh_args = argparse.Namespace(**vars(it_args))
+            fh_args.features_in_hbm = True
+            fr_args = argparse.Namespace(**vars(fh_args))
+            fr_args.recorded = True
             r5_args = argparse.Namespace(**vars(it_args))
             r5_args.recorded, r5_args.prefetch = True, True      # once replayed, this loop too gains from the read-ahead
             # c3_sampled_hot_rows: between the two placements -- the matrix in host memory, copies of the rows of the
@@ -1596,6 +1602,8 @@ def main():
                     ("c1_recorded", r1_args, lambda: run_c1(r1_args)),
                     ("c3", c3_args, lambda: run_c3(c3_args, with_batched=False)),
                     ("c3_recorded", r3_args, lambda: run_c3(r3_args, with_batched=False)),
+                    ("c3_features_in_hbm", fh_args, lambda: run_c3(fh_args, with_batched=False)),
+                    ("c3_features_in_hbm_recorded", fr_args, lambda: run_c3(fr_args, with_batched=False)),
                     ("c5", it_args, lambda: run_c5(it_args)),
                     ("c5_recorded", r5_args, lambda: run_c5(r5_args)),
                     ("c3_sampled", sm_args, lambda: run_c3(sm_args, with_batched=False)),
